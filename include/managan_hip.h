@@ -1,0 +1,182 @@
+/*
+ * managan_hip.h — C ABI of the MI355X (gfx950) implementation of the
+ * equivariant message-passing hot path: periodic cell-list neighbour search,
+ * fused Cartesian tensor products + per-irrep channel-mixing linears, and the
+ * edge->node segment sum.
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer unless the comment says "host";
+ *   - every tensor is dense row-major float32 (indices int32) unless stated;
+ *   - `stream` is a hipStream_t passed as void* (NULL = the null stream);
+ *   - every entry point returns an mg_status; nothing is thrown, nothing
+ *     terminates the process; mg_last_error() gives the text of the last
+ *     failure on the calling thread;
+ *   - no entry point allocates or frees device memory: callers own outputs and
+ *     pass workspaces whose sizes the *_workspace_bytes functions report;
+ *   - entry points only enqueue work on `stream`; they synchronise nothing.
+ *
+ * Each declaration names the reference interface it stands in for
+ * (file:line relative to the pb1729/learned-dynamics checkout).
+ */
+#ifndef MANAGAN_HIP_H
+#define MANAGAN_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void* mg_stream_t;
+
+enum mg_status {
+    MG_OK = 0,
+    MG_ERR_INVALID_ARGUMENT = 1, /* bad shape / size / null pointer / alignment */
+    MG_ERR_HIP = 2,              /* a HIP runtime call failed, see mg_last_error() */
+    MG_ERR_BOX_TOO_SMALL = 3,    /* "box dimension must be greater than 3*cutoff" */
+    MG_ERR_WORKSPACE = 4,        /* workspace smaller than *_workspace_bytes reports */
+    MG_ERR_UNSUPPORTED = 5       /* e.g. tensor rank > 2 */
+};
+
+const char* mg_status_string(int status);
+const char* mg_last_error(void);
+int mg_abi_version(void);
+
+/* ------------------------------------------------------------------------
+ * Stage A — periodic radius graph.
+ * Stands in for get_neighbours / get_edges
+ * (extensions/neighbour_grid/neighbour_grid.cpp:59-103,170-195) and the kernels
+ * assignParticlesToCells, createNeighbourListsKern, writeSrcDstKern
+ * (extensions/neighbour_grid/neighbour_grid_kern.cu:57-150,334-352).
+ * Two phases so the caller can size the edge arrays:
+ *   count: bins atoms, walks the 3x3x3 cell window, writes the CSR row_ptr
+ *          (batch*nodes+1, exclusive prefix), edge_counts (batch, inclusive
+ *          prefix per box, as the reference's edgeCounts) and stats[4] =
+ *          {E, max atoms in a cell, max degree, 0};
+ *   fill:  writes src[e] = b*nodes+i and dst[e] = b*nodes+j, rows ordered by
+ *          (b,i); order inside a row is deterministic.
+ * The reference's listmax / neighboursmax caps are not needed (exact-size CSR);
+ * callers that want the reference's overflow errors compare stats[1], stats[2]
+ * with their caps.
+ * ---------------------------------------------------------------------- */
+int mg_neighbour_ndiv(float cutoff, float box_x, float box_y, float box_z, int ndiv[3] /* host */);
+
+int mg_neighbour_workspace_bytes(int batch, int nodes, float cutoff,
+                                 float box_x, float box_y, float box_z, size_t* bytes /* host */);
+
+int mg_neighbour_count(const float* x /* (batch,nodes,3) */, int batch, int nodes, float cutoff,
+                       float box_x, float box_y, float box_z,
+                       void* workspace, size_t workspace_bytes,
+                       int* row_ptr /* batch*nodes+1 */, int* edge_counts /* batch */,
+                       int* stats /* 4 */, mg_stream_t stream);
+
+int mg_neighbour_fill(const void* workspace, size_t workspace_bytes, int batch, int nodes,
+                      float cutoff, float box_x, float box_y, float box_z,
+                      const int* row_ptr, int n_edges, int* src, int* dst, mg_stream_t stream);
+
+/* First step of the search on its own: wrapped positions (batch,nodes,3) and box-local
+ * linear cell ids (batch,nodes), as assignParticlesToCells computes them
+ * (extensions/neighbour_grid/neighbour_grid_kern.cu:75-82).  Diagnostic / test entry. */
+int mg_neighbour_wrap_cells(const float* x, int batch, int nodes, float cutoff,
+                            float box_x, float box_y, float box_z,
+                            float* wrapped, int* cell, mg_stream_t stream);
+
+/* CSR -> the reference's padded table (get_neighbours,
+ * extensions/neighbour_grid/neighbour_grid.cpp:59-103): neighbours
+ * (batch,nodes,neighboursmax) holds box-local indices, entries >= count are
+ * left untouched; counts (batch,nodes). */
+int mg_neighbour_pad(const int* row_ptr, const int* dst, int batch, int nodes, int neighboursmax,
+                     int* neighbours, int* counts, mg_stream_t stream);
+
+/* Padded gather / reduce (edges_read, edges_reduce:
+ * extensions/neighbour_grid/neighbour_grid.cpp:105-167; kernels
+ * neighbour_grid_kern.cu:226-306). */
+int mg_padded_edges_read(const int* counts, const int* neighbours, const float* x /* (batch,nodes,chan) */,
+                         int batch, int nodes, int neighboursmax, int chan,
+                         float* edge_data /* (batch,nodes,neighboursmax,chan) */, mg_stream_t stream);
+int mg_padded_edges_reduce(const int* counts, const float* edge_data, int batch, int nodes,
+                           int neighboursmax, int chan, float* out /* (batch,nodes,chan) */,
+                           mg_stream_t stream);
+
+/* r_ij[e] = boxwrap(box, x[dst[e]] - x[src[e]]) with floor-mod, fp32
+ * (managan/graph_layers.py:62-66 applied as in archs/meanflow_painn8.py:167-172)
+ * and, if shift != NULL, the periodic image rint(((x_j - x_i) - r_ij)/box) as int8 x3. */
+int mg_edge_vectors(const float* x /* (batch*nodes,3) */, const int* src, const int* dst, long n_edges,
+                    float box_x, float box_y, float box_z, float* r_ij /* (E,3) */,
+                    int8_t* shift /* (E,3) or NULL */, mg_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Stage C — gather to edges and sum edges -> nodes.
+ * Stand in for x_node[graph.dst] (managan/graph_layers.py:37-52) and
+ * torch_scatter.segment_coo(x_edge, graph.src, dim_size=batch*nodes)
+ * (managan/graph_layers.py:54-59).
+ * ---------------------------------------------------------------------- */
+/* row_ptr[r] = first e with index[e] >= r, r = 0..n_rows (index sorted ascending).
+ * index_is_int64 selects the element type of `index`. */
+int mg_segment_row_ptr(const void* index, int index_is_int64, long n_edges, int n_rows,
+                       int* row_ptr /* n_rows+1 */, mg_stream_t stream);
+/* out[r, :] = sum over e in [row_ptr[r], row_ptr[r+1]) of x_edge[e, :], in edge order. */
+int mg_segment_sum_csr(const float* x_edge /* (E,feat) */, const int* row_ptr, int n_rows, int feat,
+                       float* out /* (n_rows,feat) */, mg_stream_t stream);
+/* out[e, :] = x[index[e], :] */
+int mg_gather_rows(const float* x /* (n_rows,feat) */, const void* index, int index_is_int64,
+                   long n_edges, int n_rows, int feat, float* out /* (E,feat) */, mg_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Stage B — Cartesian tensor products (elementwise over rows x chan).
+ * Operand layouts (rows,chan), (rows,chan,3), (rows,chan,3,3).
+ * ---------------------------------------------------------------------- */
+/* bee_fwd_cuda (extensions/codegen_tensops/codegen_tensops.cpp:1519-1573, kernel
+ * codegen_tensops_kern.cu:3800-3875).  y: host array of 13 device pointers in the
+ * order 000,110,220,011,101,121,211,022,202,112,222,111,212. */
+int mg_bee_fwd(const float* l_0, const float* l_1, const float* l_2,
+               const float* r_0, const float* r_1, const float* r_2,
+               long rows, int chan, float* const y[13] /* host array */, mg_stream_t stream);
+/* bee_bwl_cuda / bee_bwr_cuda (codegen_tensops.cpp:1575-1769): gradient with respect to
+ * the left (resp. right) operands given the OTHER side's operands o_0,o_1,o_2 and the 13
+ * output gradients.  side = 0: o = r, outputs dl; side = 1: o = l, outputs dr. */
+int mg_bee_bwd(int side, const float* o_0, const float* o_1, const float* o_2,
+               const float* const dy[13] /* host array */, long rows, int chan,
+               float* d_0, float* d_1, float* d_2, mg_stream_t stream);
+/* cow_o0_fwd_cuda: products 000,110 (codegen_tensops.cpp:1771-1802). */
+int mg_cow_o0_fwd(const float* l_0, const float* l_1, const float* r_0, const float* r_1,
+                  long rows, int chan, float* y_000, float* y_110, mg_stream_t stream);
+/* cow_o1_fwd_cuda: products 011,101,111 (codegen_tensops.cpp:1868-1900). */
+int mg_cow_o1_fwd(const float* l_0, const float* l_1, const float* r_0, const float* r_1,
+                  long rows, int chan, float* y_011, float* y_101, float* y_111, mg_stream_t stream);
+/* cow_o0_bw{l,r}_cuda, cow_o1_bw{l,r}_cuda (codegen_tensops.cpp:1804-1866,1902-1978). */
+int mg_cow_o0_bwd(int side, const float* o_0, const float* o_1, const float* dy_000, const float* dy_110,
+                  long rows, int chan, float* d_0, float* d_1, mg_stream_t stream);
+int mg_cow_o1_bwd(int side, const float* o_0, const float* o_1, const float* dy_011, const float* dy_101,
+                  const float* dy_111, long rows, int chan, float* d_0, float* d_1, mg_stream_t stream);
+/* TensorProdBare.forward (managan/tensor_products.py:91-106) for one non-chiral
+ * (inds_l, inds_r, inds_o) with all ranks <= 2. */
+int mg_tensor_prod_bare(int inds_l, int inds_r, int inds_o, const float* x_l, const float* x_r,
+                        long rows, int chan, float* y, mg_stream_t stream);
+/* The three products the vector/scalar pair of one TensorProds stack needs in one pass:
+ * y_110 = v.v', y_011 = a v', y_112 = v (x) v' with v = left vector, v' = right vector,
+ * a = scalar (managan/tensor_products.py:91-121 applied three times). */
+int mg_tensor_prods_avd(const float* a, const float* v_l, const float* v_r, long rows, int chan,
+                        float* y_110, float* y_011, float* y_112, mg_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Stage B — per-irrep channel-mixing linear (dense contraction, MFMA).
+ * tensor_linear (extensions/tensor_ops/tensor_ops.cpp:31-93; kernel
+ * tensor_ops_kern.cu:6-42): y[r,o,t] = sum_i W[o,i] x[r,i,t], t < 3^inds;
+ * W is read with element strides (w_stride_o, w_stride_i) so a transposed view costs nothing.
+ * Optional fused epilogue (used for nn.Linear inside the MLPs, inds = 0):
+ *   y = act(y + bias[o]); act: 0 none, 1 SiLU, 2 LeakyReLU(0.1); bias may be NULL.
+ * accumulate != 0 adds into y instead of overwriting it.
+ * ---------------------------------------------------------------------- */
+int mg_tensor_linear(int inds, const float* W, long w_stride_o, long w_stride_i,
+                     const float* x, long rows, int dim_in, int dim_out,
+                     const float* bias, int act, int accumulate, float* y, mg_stream_t stream);
+/* dW[o,i] = sum_{r,t} dy[r,o,t] x[r,i,t]  (tensor_ops_kern.cu:45-71), dW dense (dim_out,dim_in). */
+int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows, int dim_in, int dim_out,
+                           float* dW, mg_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MANAGAN_HIP_H */

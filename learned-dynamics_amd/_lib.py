@@ -1,0 +1,92 @@
+"""ctypes binding of libmanagan_hip.so (the C ABI declared in include/managan_hip.h).
+
+The library is the only compute path: if it is missing the import fails with
+instructions to build it; there is no CPU or PyTorch fallback.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libmanagan_hip.so")
+
+c_float_p = ctypes.c_void_p   # device pointers travel as integers
+c_int_p = ctypes.c_void_p
+vp = ctypes.c_void_p
+i32 = ctypes.c_int
+i64 = ctypes.c_long
+f32 = ctypes.c_float
+PtrArray13 = ctypes.c_void_p * 13
+
+MG_OK = 0
+MG_ERR_INVALID_ARGUMENT = 1
+MG_ERR_HIP = 2
+MG_ERR_BOX_TOO_SMALL = 3
+MG_ERR_WORKSPACE = 4
+MG_ERR_UNSUPPORTED = 5
+
+_SIGNATURES = {
+    "mg_neighbour_ndiv": [f32, f32, f32, f32, ctypes.POINTER(i32 * 3)],
+    "mg_neighbour_workspace_bytes": [i32, i32, f32, f32, f32, f32, ctypes.POINTER(ctypes.c_size_t)],
+    "mg_neighbour_count": [vp, i32, i32, f32, f32, f32, f32, vp, ctypes.c_size_t, vp, vp, vp, vp],
+    "mg_neighbour_fill": [vp, ctypes.c_size_t, i32, i32, f32, f32, f32, f32, vp, i32, vp, vp, vp],
+    "mg_neighbour_wrap_cells": [vp, i32, i32, f32, f32, f32, f32, vp, vp, vp],
+    "mg_neighbour_pad": [vp, vp, i32, i32, i32, vp, vp, vp],
+    "mg_padded_edges_read": [vp, vp, vp, i32, i32, i32, i32, vp, vp],
+    "mg_padded_edges_reduce": [vp, vp, i32, i32, i32, i32, vp, vp],
+    "mg_edge_vectors": [vp, vp, vp, i64, f32, f32, f32, vp, vp, vp],
+    "mg_segment_row_ptr": [vp, i32, i64, i32, vp, vp],
+    "mg_segment_sum_csr": [vp, vp, i32, i32, vp, vp],
+    "mg_gather_rows": [vp, vp, i32, i64, i32, i32, vp, vp],
+    "mg_bee_fwd": [vp, vp, vp, vp, vp, vp, i64, i32, ctypes.POINTER(PtrArray13), vp],
+    "mg_bee_bwd": [i32, vp, vp, vp, ctypes.POINTER(PtrArray13), i64, i32, vp, vp, vp, vp],
+    "mg_cow_o0_fwd": [vp, vp, vp, vp, i64, i32, vp, vp, vp],
+    "mg_cow_o1_fwd": [vp, vp, vp, vp, i64, i32, vp, vp, vp, vp],
+    "mg_cow_o0_bwd": [i32, vp, vp, vp, vp, i64, i32, vp, vp, vp],
+    "mg_cow_o1_bwd": [i32, vp, vp, vp, vp, vp, i64, i32, vp, vp, vp],
+    "mg_tensor_prod_bare": [i32, i32, i32, vp, vp, i64, i32, vp, vp],
+    "mg_tensor_prods_avd": [vp, vp, vp, i64, i32, vp, vp, vp, vp],
+    "mg_tensor_linear": [i32, vp, i64, i64, vp, i64, i32, i32, vp, i32, i32, vp, vp],
+    "mg_tensor_linear_wgrad": [i32, vp, vp, i64, i32, i32, vp, vp],
+}
+
+_lib = None
+
+
+def load():
+    """Load the library once; raise if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            f"{LIB_PATH} is missing: build it with `python learned-dynamics_amd/build.py` "
+            "(hipcc, --offload-arch=gfx950). There is no fallback path.")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, argtypes in _SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.argtypes = argtypes
+        fn.restype = ctypes.c_int
+    lib.mg_status_string.restype = ctypes.c_char_p
+    lib.mg_status_string.argtypes = [ctypes.c_int]
+    lib.mg_last_error.restype = ctypes.c_char_p
+    lib.mg_last_error.argtypes = []
+    lib.mg_abi_version.restype = ctypes.c_int
+    lib.mg_abi_version.argtypes = []
+    _lib = lib
+    return lib
+
+
+def check(status):
+    """Turn a non-zero mg_status into the Python exception the reference would raise."""
+    if status == MG_OK:
+        return
+    lib = load()
+    text = lib.mg_last_error().decode(errors="replace")
+    if status == MG_ERR_BOX_TOO_SMALL:
+        raise RuntimeError("box dimension must be greater than 3*cutoff")
+    kind = lib.mg_status_string(status).decode()
+    raise RuntimeError(f"{kind}: {text}" if text else kind)
+
+
+def exported_symbols():
+    return sorted(_SIGNATURES) + ["mg_status_string", "mg_last_error", "mg_abi_version"]

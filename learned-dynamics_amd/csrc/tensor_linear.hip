@@ -1,0 +1,243 @@
+// Per-irrep channel-mixing linear on the matrix cores (fp32 MFMA, gfx950).
+//
+//   y[r, o, t] = act( sum_i W[o, i] x[r, i, t] + bias[o] ),   t < T = 3^inds
+//
+// GEMM view: M = the flattened (r, t) index, N = o, K = i.  x keeps its HBM
+// layout (r, i, t) all the way into LDS: for a k-slab [k0, k0+BK) the data of
+// one row r is one contiguous run of BK*T floats, so HBM is read with
+// unit-stride 16-byte accesses; the (r,t) <-> MFMA-row mapping is pure LDS
+// address arithmetic.  The LDS row stride RS is chosen with RS = T (mod 32), so
+// the 32 consecutive flattened rows a half-wave reads for one k land in 32
+// different banks.
+//
+// v_mfma_f32_32x32x2_f32 operand layout (wave64):
+//   A[m][k]: lane = m + 32k  (m < 32, k < 2)      B[k][n]: lane = n + 32k
+//   D[m][n]: n = lane % 32,  m = 8*(reg/4) + 4*(lane/32) + reg%4,  reg < 16
+#include "common.hpp"
+
+namespace mg {
+namespace {
+
+typedef float float16v __attribute__((ext_vector_type(16)));
+
+constexpr int kBK = 16;
+
+constexpr int lds_row_stride(int T) {
+    // smallest stride >= BK*T with stride % 32 == T % 32; for T == 1 any odd stride does
+    if (T == 1) return kBK + 1;
+    int s = kBK * T;
+    while (s % 32 != T % 32) s++;
+    return s;
+}
+
+__device__ __forceinline__ float activate(float v, int act) {
+    if (act == 1) return v / (1.0f + expf(-v));       // SiLU
+    if (act == 2) return v > 0.f ? v : 0.1f * v;      // LeakyReLU(0.1)
+    return v;
+}
+
+template <int T, int WAVES_M, int WAVES_N, int WM, int WN>
+struct Cfg {
+    static constexpr int NT = 64 * WAVES_M * WAVES_N;
+    static constexpr int BM = 32 * WAVES_M * WM;   // flattened (r,t) rows per workgroup
+    static constexpr int BN = 32 * WAVES_N * WN;
+    static constexpr int RB = BM / T;              // x rows per workgroup
+    static_assert(BM % T == 0, "tile must hold whole rows");
+    static constexpr int RS = lds_row_stride(T);
+    static constexpr int RSW = kBK + 1;
+    static constexpr int XV4 = RB * (kBK * T / 4);              // float4 loads per x tile
+    static constexpr int XV4_PER = (XV4 + NT - 1) / NT;
+    static constexpr int XS = RB * kBK * T;                     // scalar loads per x tile
+    static constexpr int XS_PER = (XS + NT - 1) / NT;
+    static constexpr int WS = BN * kBK;
+    static constexpr int WS_PER = (WS + NT - 1) / NT;
+};
+
+template <int T, int WAVES_M, int WAVES_N, int WM, int WN, bool XVEC>
+__global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
+linear_kernel(const float* __restrict__ W, long so, long si, const float* __restrict__ X, long R, int I, int O,
+              const float* __restrict__ bias, int act, int accumulate, float* __restrict__ Y) {
+    using C = Cfg<T, WAVES_M, WAVES_N, WM, WN>;
+    __shared__ float xs[C::RB * C::RS];
+    __shared__ float ws[C::BN * C::RSW];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave / WAVES_N, wave_n = wave % WAVES_N;
+    const long r0 = (long)blockIdx.x * C::RB;
+    const int n0 = blockIdx.y * C::BN;
+    const long row_floats = (long)I * T;
+
+    float16v acc[WM][WN];
+#pragma unroll
+    for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+        for (int ni = 0; ni < WN; ni++)
+#pragma unroll
+            for (int q = 0; q < 16; q++) acc[mi][ni][q] = 0.f;
+
+    // LDS read bases (without the k term)
+    int a_base[WM];
+#pragma unroll
+    for (int mi = 0; mi < WM; mi++) {
+        const int m = (wave_m * WM + mi) * 32 + (lane & 31);
+        a_base[mi] = (m / T) * C::RS + (m % T);
+    }
+    int b_base[WN];
+#pragma unroll
+    for (int ni = 0; ni < WN; ni++) b_base[ni] = ((wave_n * WN + ni) * 32 + (lane & 31)) * C::RSW;
+    const int khalf = lane >> 5;
+
+    // register staging of the next k-slab
+    // (the scalar x path is the fallback for odd sizes: it goes HBM -> LDS without staging)
+    float4 xv[XVEC ? C::XV4_PER : 1];
+    float wsc[C::WS_PER];
+
+    auto load_tile = [&](int k0) {
+        if constexpr (XVEC) {
+#pragma unroll
+            for (int j = 0; j < C::XV4_PER; j++) {
+                const int idx = tid + j * C::NT;
+                const int r = idx / (kBK * T / 4), c4 = idx % (kBK * T / 4);
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (idx < C::XV4 && r0 + r < R)
+                    v = *reinterpret_cast<const float4*>(X + (r0 + r) * row_floats + (long)k0 * T + c4 * 4);
+                xv[j] = v;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < C::WS_PER; j++) {
+            const int idx = tid + j * C::NT;
+            const int n = idx / kBK, k = idx % kBK;
+            float v = 0.f;
+            if (idx < C::WS && n0 + n < O && k0 + k < I) v = W[(long)(n0 + n) * so + (long)(k0 + k) * si];
+            wsc[j] = v;
+        }
+    };
+    auto store_tile = [&](int k0) {
+        if constexpr (XVEC) {
+#pragma unroll
+            for (int j = 0; j < C::XV4_PER; j++) {
+                const int idx = tid + j * C::NT;
+                if (idx < C::XV4) {
+                    const int r = idx / (kBK * T / 4), c4 = idx % (kBK * T / 4);
+                    float* p = xs + r * C::RS + c4 * 4;
+                    p[0] = xv[j].x; p[1] = xv[j].y; p[2] = xv[j].z; p[3] = xv[j].w;
+                }
+            }
+        } else {
+            const int valid = (I - k0 < kBK ? I - k0 : kBK) * T;
+            for (int idx = tid; idx < C::XS; idx += C::NT) {
+                const int r = idx / (kBK * T), c = idx % (kBK * T);
+                float v = 0.f;
+                if (r0 + r < R && c < valid) v = X[(r0 + r) * row_floats + (long)k0 * T + c];
+                xs[r * C::RS + c] = v;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < C::WS_PER; j++) {
+            const int idx = tid + j * C::NT;
+            if (idx < C::WS) ws[(idx / kBK) * C::RSW + idx % kBK] = wsc[j];
+        }
+    };
+
+    load_tile(0);
+    for (int k0 = 0; k0 < I; k0 += kBK) {
+        __syncthreads();          // everyone finished reading the previous slab
+        store_tile(k0);
+        __syncthreads();
+        if (k0 + kBK < I) load_tile(k0 + kBK);   // in flight during the MFMA loop
+#pragma unroll
+        for (int kk = 0; kk < kBK / 2; kk++) {
+            const int k = 2 * kk + khalf;
+            float a[WM], b[WN];
+#pragma unroll
+            for (int mi = 0; mi < WM; mi++) a[mi] = xs[a_base[mi] + k * T];
+#pragma unroll
+            for (int ni = 0; ni < WN; ni++) b[ni] = ws[b_base[ni] + k];
+#pragma unroll
+            for (int mi = 0; mi < WM; mi++)
+#pragma unroll
+                for (int ni = 0; ni < WN; ni++)
+                    acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[mi], b[ni], acc[mi][ni], 0, 0, 0);
+        }
+    }
+
+    // epilogue
+#pragma unroll
+    for (int ni = 0; ni < WN; ni++) {
+        const int n = n0 + (wave_n * WN + ni) * 32 + (lane & 31);
+        if (n >= O) continue;
+        const float bv = bias ? bias[n] : 0.f;
+#pragma unroll
+        for (int mi = 0; mi < WM; mi++) {
+#pragma unroll
+            for (int q = 0; q < 16; q++) {
+                const int m = (wave_m * WM + mi) * 32 + 8 * (q / 4) + 4 * khalf + (q % 4);
+                const long r = r0 + m / T;
+                if (r < R) {
+                    const long addr = (r * O + n) * T + (m % T);
+                    float v = acc[mi][ni][q] + bv;
+                    v = activate(v, act);
+                    if (accumulate) v += Y[addr];
+                    Y[addr] = v;
+                }
+            }
+        }
+    }
+}
+
+template <int T, int WAVES_M, int WAVES_N, int WM, int WN>
+int launch_cfg(const float* W, long so, long si, const float* X, long R, int I, int O, const float* bias, int act,
+               int accumulate, float* Y, hipStream_t st) {
+    using C = Cfg<T, WAVES_M, WAVES_N, WM, WN>;
+    const long gx = ceil_div(R, C::RB);
+    const long gy = ceil_div(O, C::BN);
+    MG_REQUIRE(gx <= 0x7fffffffL && gy <= 65535, "mg_tensor_linear: grid too large (rows=%ld dim_out=%d)", R, O);
+    const bool xvec = I > 0 && aligned16(X) && (I % kBK == 0) && (((long)I * T) % 4 == 0);
+    dim3 grid((unsigned)gx, (unsigned)gy), block(C::NT);
+    if (xvec)
+        hipLaunchKernelGGL((linear_kernel<T, WAVES_M, WAVES_N, WM, WN, true>), grid, block, 0, st, W, so, si, X, R, I,
+                           O, bias, act, accumulate, Y);
+    else
+        hipLaunchKernelGGL((linear_kernel<T, WAVES_M, WAVES_N, WM, WN, false>), grid, block, 0, st, W, so, si, X, R, I,
+                           O, bias, act, accumulate, Y);
+    return check_launch("mg_tensor_linear");
+}
+
+}  // namespace
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" {
+
+int mg_tensor_linear(int inds, const float* W, long w_stride_o, long w_stride_i, const float* x, long rows,
+                     int dim_in, int dim_out, const float* bias, int act, int accumulate, float* y,
+                     mg_stream_t stream) {
+    if (inds < 0 || inds > 2)
+        return fail(MG_ERR_UNSUPPORTED,
+                    "tensor_linear currently only supports a number of indices up to 2.");
+    MG_REQUIRE(rows >= 0 && dim_in >= 0 && dim_out >= 0, "mg_tensor_linear: negative size");
+    MG_REQUIRE(act >= 0 && act <= 2, "mg_tensor_linear: unknown activation %d", act);
+    if (rows == 0 || dim_out == 0) return MG_OK;
+    MG_REQUIRE(y != nullptr && (dim_in == 0 || (W != nullptr && x != nullptr)), "mg_tensor_linear: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const float* b = bias;
+    switch (inds) {
+        case 0:
+            if (dim_out <= 32) return launch_cfg<1, 4, 1, 2, 1>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
+            if (dim_out <= 64) return launch_cfg<1, 2, 2, 2, 1>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
+            return launch_cfg<1, 2, 2, 2, 2>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
+        case 1:
+            if (dim_out <= 32) return launch_cfg<3, 2, 1, 3, 1>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
+            if (dim_out <= 64) return launch_cfg<3, 2, 2, 3, 1>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
+            return launch_cfg<3, 2, 2, 3, 2>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
+        default:
+            if (dim_out <= 32) return launch_cfg<9, 3, 1, 3, 1>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
+            if (dim_out <= 64) return launch_cfg<9, 3, 1, 3, 2>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
+            return launch_cfg<9, 3, 2, 3, 2>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
+    }
+}
+
+}  // extern "C"

@@ -1,0 +1,103 @@
+"""Graph container and the gather / segment-sum / boxwrap helpers, mirroring
+managan/graph_layers.py of the reference (same names, arguments and error
+behaviour) on top of the HIP kernels.
+
+Differences that do not change results: the Graph also keeps the int32 index
+arrays and the CSR row_ptr the neighbour search produced, so gathers and
+segment sums run on them directly; rows are exact-size (the celllist_max /
+neighbours_max caps are only used to raise the reference's overflow errors).
+"""
+import torch
+
+from . import ops
+
+
+class Graph:
+    """Batch of graphs with the same number of nodes each; edges are stored flat
+    and index into a dimension of size batch*nodes.  src must be non-decreasing.
+    (managan/graph_layers.py:9-24)"""
+
+    def __init__(self, src, dst, edge_indices, batch, nodes, row_ptr=None):
+        self.src32 = src.to(torch.int32).contiguous()
+        self.dst32 = dst.to(torch.int32).contiguous()
+        self.src = src.to(torch.int64)
+        self.dst = dst.to(torch.int64)
+        self.edge_indices = edge_indices
+        self.batch = batch
+        self.nodes = nodes
+        self._row_ptr = row_ptr
+
+    @property
+    def row_ptr(self):
+        if self._row_ptr is None:
+            self._row_ptr = ops.segment_row_ptr(self.src32, self.batch * self.nodes)
+        return self._row_ptr
+
+    @staticmethod
+    def radius_graph(r0, box, pos, celllist_max=32, neighbours_max=64):
+        """Nodes are connected if they are within r0 of each other under periodic
+        boundary conditions given by box (3 floats).  pos: (batch, nodes, 3).
+        (managan/graph_layers.py:25-34)"""
+        batch, nodes, three = pos.shape
+        assert three == 3
+        assert torch.all(~torch.isnan(pos)), "some positions are NaN!"
+        src, dst, edge_indices, row_ptr = ops.get_edges(celllist_max, neighbours_max, r0, *box, pos,
+                                                        return_row_ptr=True)
+        ans = Graph(src, dst, edge_indices, batch, nodes, row_ptr=row_ptr)
+        setattr(ans, "box", box)
+        return ans
+
+
+def _flat_nodes(graph, x_node):
+    b, n, *rest = x_node.shape
+    assert b == graph.batch and n == graph.nodes
+    return x_node.reshape(graph.batch * graph.nodes, *rest).contiguous()
+
+
+def edges_read(graph: Graph, x_node: torch.Tensor):
+    """x_node: (batch, nodes, ...) -> (x_src, x_dst), each (edges, ...)."""
+    flat = _flat_nodes(graph, x_node)
+    return ops.gather_rows(flat, graph.src32), ops.gather_rows(flat, graph.dst32)
+
+
+def edges_read_dst(graph: Graph, x_node: torch.Tensor):
+    """x_node: (batch, nodes, ...) -> x_dst: (edges, ...)."""
+    return ops.gather_rows(_flat_nodes(graph, x_node), graph.dst32)
+
+
+def edges_reduce_src(graph: Graph, x_edge: torch.Tensor):
+    """Sum edge data onto the src node of each edge.  x_edge: (edges, ...)."""
+    ans = ops.segment_sum_csr(x_edge.contiguous(), graph.row_ptr, graph.batch * graph.nodes)
+    return ans.reshape(graph.batch, graph.nodes, *ans.shape[1:])
+
+
+def segment_sum(x_edge, index, dim_size):
+    """segment_coo(x_edge, index, dim_size=dim_size, reduce='sum') for a sorted index."""
+    row_ptr = ops.segment_row_ptr(index.contiguous(), dim_size)
+    return ops.segment_sum_csr(x_edge.contiguous(), row_ptr, dim_size)
+
+
+def boxwrap(box: torch.Tensor, delta_pos: torch.Tensor):
+    """Wrap a position difference to the shortest periodic image.  box: (3), delta_pos: (..., 3)."""
+    return (delta_pos + 0.5 * box) % box - 0.5 * box
+
+
+def edge_vectors(graph: Graph, pos: torch.Tensor, box, want_shift=False):
+    """r_ij = boxwrap(box, pos[dst] - pos[src]) in one kernel (what graph_setup computes with
+    two gathers and a wrap, archs/meanflow_painn8.py:167-172), optionally with the int8
+    periodic-image shift of every edge."""
+    flat = pos.reshape(graph.batch * graph.nodes, 3).contiguous()
+    return ops.edge_vectors(flat, graph.src32, graph.dst32, box, want_shift=want_shift)
+
+
+def graph_setup(r0, box, pos, neighbours_max=64, celllist_max=32):
+    graph = Graph.radius_graph(r0, box, pos, celllist_max=celllist_max, neighbours_max=neighbours_max)
+    return graph, edge_vectors(graph, pos, box)
+
+
+def expand_graph(graph: Graph, new_batch: int):
+    assert graph.batch == 1, "Graph to be expanded should have batch size 1"
+    offs = graph.nodes * torch.arange(new_batch, device=graph.src.device)[:, None]
+    src = (graph.src[None].expand(new_batch, -1) + offs).flatten()
+    dst = (graph.dst[None].expand(new_batch, -1) + offs).flatten()
+    return Graph(src, dst, None, new_batch, graph.nodes)

@@ -1,0 +1,456 @@
+"""Torch-facing operators over the C ABI.
+
+Each function validates its arguments the way the reference's C++ front ends
+do (device, contiguity, rank and per-axis size checks, same messages), allocates
+the outputs with torch, and enqueues the HIP kernels on the current torch
+stream through libmanagan_hip.so.  Nothing here computes on the CPU or with
+torch kernels: if the library is missing, importing this module fails.
+"""
+import ctypes
+import torch
+
+from . import _lib as L
+
+_lib = L.load()
+
+BEE_ORDER = ("000", "110", "220", "011", "101", "121", "211", "022", "202", "112", "222", "111", "212")
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _p(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
+
+
+def _check_input(t, name, dtype=torch.float32):
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+    if t.dtype != dtype:
+        raise RuntimeError(f"expected scalar type {str(dtype).replace('torch.', '').capitalize()} "
+                           f"but found {str(t.dtype).replace('torch.', '')} for {name}")
+
+
+# --------------------------------------------------------------------- stage A
+class NeighbourSearch:
+    """Result of the count phase; `fill()` writes the edges."""
+
+    def __init__(self, x, cutoff, box):
+        _check_input(x, "x")
+        if x.dim() != 3 or x.size(2) != 3:
+            raise RuntimeError("x must have shape (batch, nodes, 3)")
+        self.x = x
+        self.batch, self.nodes = int(x.size(0)), int(x.size(1))
+        self.cutoff = float(cutoff)
+        self.box = tuple(float(b) for b in box)
+        nbytes = ctypes.c_size_t(0)
+        L.check(_lib.mg_neighbour_workspace_bytes(self.batch, self.nodes, self.cutoff, *self.box,
+                                                  ctypes.byref(nbytes)))
+        dev = x.device
+        with torch.cuda.device(dev):
+            self.workspace = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
+            self.row_ptr = torch.empty(self.batch * self.nodes + 1, dtype=torch.int32, device=dev)
+            self.edge_counts = torch.empty(self.batch, dtype=torch.int32, device=dev)
+            self.stats = torch.empty(4, dtype=torch.int32, device=dev)
+            L.check(_lib.mg_neighbour_count(_p(x), self.batch, self.nodes, self.cutoff, *self.box,
+                                            _p(self.workspace), self.workspace.numel(), _p(self.row_ptr),
+                                            _p(self.edge_counts), _p(self.stats), _stream()))
+        self._host_stats = None
+
+    def host_stats(self):
+        """(E, max atoms per cell, max degree, overflow flag) — one device->host copy."""
+        if self._host_stats is None:
+            self._host_stats = tuple(int(v) for v in self.stats.tolist())
+            if self._host_stats[3]:
+                raise RuntimeError("edge count does not fit int32")
+        return self._host_stats
+
+    def fill(self, n_edges=None):
+        E = self.host_stats()[0] if n_edges is None else int(n_edges)
+        dev = self.x.device
+        with torch.cuda.device(dev):
+            src = torch.empty(E, dtype=torch.int32, device=dev)
+            dst = torch.empty(E, dtype=torch.int32, device=dev)
+            L.check(_lib.mg_neighbour_fill(_p(self.workspace), self.workspace.numel(), self.batch, self.nodes,
+                                           self.cutoff, *self.box, _p(self.row_ptr), E, _p(src), _p(dst),
+                                           _stream()))
+        return src, dst
+
+
+def _check_caps(search, listmax, neighboursmax):
+    """The reference's overflow errors, in the reference's order
+    (extensions/neighbour_grid/neighbour_grid_kern.cu:195-217)."""
+    _, max_cell, max_deg, _ = search.host_stats()
+    if max_cell > listmax:
+        raise RuntimeError("Cell list overflow occurred. Trying increasing listmax.")
+    if listmax not in (32, 64, 128, 256):
+        raise RuntimeError("expected listmax to be one of 32, 64, 128, 256. other values not supported!")
+    if max_deg > neighboursmax:
+        raise RuntimeError("Neighbour list overflow occurred. Try increasing neighboursmax.")
+
+
+def get_edges(listmax, neighboursmax, cutoff, box_x, box_y, box_z, x, return_row_ptr=False):
+    """(src int32[E], dst int32[E], edgeCounts int32[B]); extensions/neighbour_grid/neighbour_grid.cpp:170-195."""
+    search = NeighbourSearch(x, cutoff, (box_x, box_y, box_z))
+    _check_caps(search, listmax, neighboursmax)
+    src, dst = search.fill()
+    if return_row_ptr:
+        return src, dst, search.edge_counts, search.row_ptr
+    return src, dst, search.edge_counts
+
+
+def get_neighbours(listmax, neighboursmax, cutoff, box_x, box_y, box_z, x):
+    """(neighbours int32[B,N,neighboursmax], counts int32[B,N]); neighbour_grid.cpp:59-103."""
+    search = NeighbourSearch(x, cutoff, (box_x, box_y, box_z))
+    _check_caps(search, listmax, neighboursmax)
+    _, dst = search.fill()
+    B, N = search.batch, search.nodes
+    with torch.cuda.device(x.device):
+        neighbours = torch.empty(B, N, neighboursmax, dtype=torch.int32, device=x.device)
+        counts = torch.empty(B, N, dtype=torch.int32, device=x.device)
+        L.check(_lib.mg_neighbour_pad(_p(search.row_ptr), _p(dst), B, N, neighboursmax, _p(neighbours),
+                                      _p(counts), _stream()))
+    return neighbours, counts
+
+
+def wrap_cells(cutoff, box, x):
+    _check_input(x, "x")
+    B, N = int(x.size(0)), int(x.size(1))
+    with torch.cuda.device(x.device):
+        w = torch.empty_like(x)
+        cell = torch.empty(B, N, dtype=torch.int32, device=x.device)
+        L.check(_lib.mg_neighbour_wrap_cells(_p(x), B, N, float(cutoff), *[float(b) for b in box], _p(w),
+                                             _p(cell), _stream()))
+    return w, cell
+
+
+def padded_edges_read(counts, neighbours, x):
+    _check_input(counts, "neighbourCounts", torch.int32)
+    _check_input(neighbours, "neighbours", torch.int32)
+    _check_input(x, "x")
+    if counts.dim() != 2:
+        raise RuntimeError("neighbourCounts must have shape (batch, nodes)")
+    if neighbours.dim() != 3:
+        raise RuntimeError("neighbourCounts must have shape (batch, nodes, neighboursmax)")
+    if x.dim() != 3:
+        raise RuntimeError("x must have shape (batch, nodes, chan)")
+    B, N = counts.shape
+    if not (B == neighbours.size(0) == x.size(0)):
+        raise RuntimeError("batch dimension of all tensors must match")
+    if not (N == neighbours.size(1) == x.size(1)):
+        raise RuntimeError("node dimension of all tensors must match")
+    nmax, chan = int(neighbours.size(2)), int(x.size(2))
+    with torch.cuda.device(x.device):
+        out = torch.empty(B, N, nmax, chan, dtype=torch.float32, device=x.device)
+        L.check(_lib.mg_padded_edges_read(_p(counts), _p(neighbours), _p(x), B, N, nmax, chan, _p(out), _stream()))
+    return out
+
+
+def padded_edges_reduce(counts, neighbours, x):
+    _check_input(counts, "neighbourCounts", torch.int32)
+    _check_input(neighbours, "neighbours", torch.int32)
+    _check_input(x, "x")
+    if counts.dim() != 2:
+        raise RuntimeError("neighbourCounts must have shape (batch, nodes)")
+    if neighbours.dim() != 3:
+        raise RuntimeError("neighbours must have shape (batch, nodes, neighboursmax)")
+    if x.dim() != 4:
+        raise RuntimeError("x must have shape (batch, nodes, neighboursmax, chan)")
+    B, N = counts.shape
+    if not (B == neighbours.size(0) == x.size(0)):
+        raise RuntimeError("batch dimension of all tensors must match")
+    if not (N == neighbours.size(1) == x.size(1)):
+        raise RuntimeError("node dimension of all tensors must match")
+    nmax = int(neighbours.size(2))
+    if nmax != x.size(2):
+        raise RuntimeError("neighboursmax dimension must match between neighbours and x")
+    chan = int(x.size(3))
+    with torch.cuda.device(x.device):
+        out = torch.empty(B, N, chan, dtype=torch.float32, device=x.device)
+        L.check(_lib.mg_padded_edges_reduce(_p(counts), _p(x), B, N, nmax, chan, _p(out), _stream()))
+    return out
+
+
+def edge_vectors(pos, src, dst, box, want_shift=False):
+    """r_ij = boxwrap(box, pos[dst] - pos[src]) (E,3) and optionally the int8 image shift."""
+    _check_input(pos, "pos")
+    _check_input(src, "src", torch.int32)
+    _check_input(dst, "dst", torch.int32)
+    E = int(src.numel())
+    with torch.cuda.device(pos.device):
+        r = torch.empty(E, 3, dtype=torch.float32, device=pos.device)
+        shift = torch.empty(E, 3, dtype=torch.int8, device=pos.device) if want_shift else None
+        L.check(_lib.mg_edge_vectors(_p(pos), _p(src), _p(dst), E, *[float(b) for b in box], _p(r), _p(shift),
+                                     _stream()))
+    return (r, shift) if want_shift else r
+
+
+# --------------------------------------------------------------------- stage C
+def segment_row_ptr(index, n_rows):
+    if index.dtype not in (torch.int32, torch.int64):
+        raise RuntimeError("index must be int32 or int64")
+    _check_input(index, "index", index.dtype)
+    with torch.cuda.device(index.device):
+        row_ptr = torch.empty(n_rows + 1, dtype=torch.int32, device=index.device)
+        L.check(_lib.mg_segment_row_ptr(_p(index), int(index.dtype == torch.int64), int(index.numel()), int(n_rows),
+                                        _p(row_ptr), _stream()))
+    return row_ptr
+
+
+def segment_sum_csr(x_edge, row_ptr, n_rows):
+    """out[r] = sum of x_edge[row_ptr[r]:row_ptr[r+1]]; trailing dims kept."""
+    _check_input(x_edge, "x_edge")
+    _check_input(row_ptr, "row_ptr", torch.int32)
+    rest = tuple(x_edge.shape[1:])
+    feat = 1
+    for d in rest:
+        feat *= int(d)
+    with torch.cuda.device(x_edge.device):
+        out = torch.empty((n_rows,) + rest, dtype=torch.float32, device=x_edge.device)
+        L.check(_lib.mg_segment_sum_csr(_p(x_edge), _p(row_ptr), int(n_rows), feat, _p(out), _stream()))
+    return out
+
+
+def gather_rows(x, index):
+    """x[index] along dim 0 for a contiguous float32 x."""
+    _check_input(x, "x")
+    if index.dtype not in (torch.int32, torch.int64):
+        raise RuntimeError("index must be int32 or int64")
+    _check_input(index, "index", index.dtype)
+    rest = tuple(x.shape[1:])
+    feat = 1
+    for d in rest:
+        feat *= int(d)
+    E = int(index.numel())
+    with torch.cuda.device(x.device):
+        out = torch.empty((E,) + rest, dtype=torch.float32, device=x.device)
+        L.check(_lib.mg_gather_rows(_p(x), _p(index), int(index.dtype == torch.int64), E, int(x.size(0)), feat,
+                                    _p(out), _stream()))
+    return out
+
+
+# --------------------------------------------------------------------- stage B
+def _rows_chan(tensors_by_rank, names):
+    """Shape checks of the fused product ops: exactly (R,C), (R,C,3), (R,C,3,3), all R and C equal."""
+    rows = chan = None
+    for t, name, rank in zip(tensors_by_rank, names, (0, 1, 2) * 5):
+        _check_input(t, name)
+        if t.dim() != 2 + rank:
+            raise RuntimeError(f"{name} has wrong number of axes")
+        for ax in range(rank):
+            if t.size(2 + ax) != 3:
+                raise RuntimeError(f"{name} must have size 3 on tensor axes")
+        if rows is None:
+            rows, chan = int(t.size(0)), int(t.size(1))
+        if t.size(0) != rows:
+            raise RuntimeError(f"{name} batch size mismatch")
+        if t.size(1) != chan:
+            raise RuntimeError(f"{name} channel size mismatch")
+    return rows, chan
+
+
+def _shape(rows, chan, rank):
+    return (rows, chan) + (3,) * rank
+
+
+def bee_fwd(l_0, l_1, l_2, r_0, r_1, r_2):
+    rows, chan = _rows_chan((l_0, l_1, l_2), ("l_0", "l_1", "l_2"))
+    rows2, chan2 = _rows_chan((r_0, r_1, r_2), ("r_0", "r_1", "r_2"))
+    if rows2 != rows or chan2 != chan:
+        raise RuntimeError("left and right operands must agree on batch and channel sizes")
+    dev = l_0.device
+    with torch.cuda.device(dev):
+        ys = [torch.empty(_shape(rows, chan, int(lab[2])), dtype=torch.float32, device=dev) for lab in BEE_ORDER]
+        arr = L.PtrArray13(*[y.data_ptr() for y in ys])
+        L.check(_lib.mg_bee_fwd(_p(l_0), _p(l_1), _p(l_2), _p(r_0), _p(r_1), _p(r_2), rows, chan,
+                                ctypes.byref(arr), _stream()))
+    return ys
+
+
+def _bee_bwd(side, o_0, o_1, o_2, dys):
+    rows, chan = _rows_chan((o_0, o_1, o_2), ("x_0", "x_1", "x_2"))
+    if len(dys) != 13:
+        raise RuntimeError("expected 13 output gradients")
+    for dy, lab in zip(dys, BEE_ORDER):
+        _check_input(dy, f"dy_{lab}")
+        if tuple(dy.shape) != _shape(rows, chan, int(lab[2])):
+            raise RuntimeError(f"dy_{lab} has wrong shape")
+    dev = o_0.device
+    with torch.cuda.device(dev):
+        d = [torch.empty(_shape(rows, chan, k), dtype=torch.float32, device=dev) for k in range(3)]
+        arr = L.PtrArray13(*[dy.data_ptr() for dy in dys])
+        L.check(_lib.mg_bee_bwd(side, _p(o_0), _p(o_1), _p(o_2), ctypes.byref(arr), rows, chan, _p(d[0]),
+                                _p(d[1]), _p(d[2]), _stream()))
+    return d
+
+
+def bee_bwl(r_0, r_1, r_2, *dys):
+    return _bee_bwd(0, r_0, r_1, r_2, dys)
+
+
+def bee_bwr(l_0, l_1, l_2, *dys):
+    return _bee_bwd(1, l_0, l_1, l_2, dys)
+
+
+def _cow_inputs(l_0, l_1, r_0, r_1):
+    rows, chan = _rows_chan((l_0, l_1), ("l_0", "l_1"))
+    rows2, chan2 = _rows_chan((r_0, r_1), ("r_0", "r_1"))
+    if rows2 != rows or chan2 != chan:
+        raise RuntimeError("left and right operands must agree on batch and channel sizes")
+    return rows, chan
+
+
+def cow_o0_fwd(l_0, l_1, r_0, r_1):
+    rows, chan = _cow_inputs(l_0, l_1, r_0, r_1)
+    dev = l_0.device
+    with torch.cuda.device(dev):
+        y0 = torch.empty(rows, chan, dtype=torch.float32, device=dev)
+        y1 = torch.empty(rows, chan, dtype=torch.float32, device=dev)
+        L.check(_lib.mg_cow_o0_fwd(_p(l_0), _p(l_1), _p(r_0), _p(r_1), rows, chan, _p(y0), _p(y1), _stream()))
+    return [y0, y1]
+
+
+def cow_o1_fwd(l_0, l_1, r_0, r_1):
+    rows, chan = _cow_inputs(l_0, l_1, r_0, r_1)
+    dev = l_0.device
+    with torch.cuda.device(dev):
+        ys = [torch.empty(rows, chan, 3, dtype=torch.float32, device=dev) for _ in range(3)]
+        L.check(_lib.mg_cow_o1_fwd(_p(l_0), _p(l_1), _p(r_0), _p(r_1), rows, chan, _p(ys[0]), _p(ys[1]),
+                                   _p(ys[2]), _stream()))
+    return ys
+
+
+def _cow_bwd(which, side, o_0, o_1, dys):
+    rows, chan = _rows_chan((o_0, o_1), ("x_0", "x_1"))
+    ranks = (0, 0) if which == 0 else (1, 1, 1)
+    if len(dys) != len(ranks):
+        raise RuntimeError("wrong number of output gradients")
+    for k, (dy, rk) in enumerate(zip(dys, ranks)):
+        _check_input(dy, f"dy[{k}]")
+        if tuple(dy.shape) != _shape(rows, chan, rk):
+            raise RuntimeError(f"dy[{k}] has wrong shape")
+    dev = o_0.device
+    with torch.cuda.device(dev):
+        d0 = torch.empty(rows, chan, dtype=torch.float32, device=dev)
+        d1 = torch.empty(rows, chan, 3, dtype=torch.float32, device=dev)
+        if which == 0:
+            L.check(_lib.mg_cow_o0_bwd(side, _p(o_0), _p(o_1), _p(dys[0]), _p(dys[1]), rows, chan, _p(d0), _p(d1),
+                                       _stream()))
+        else:
+            L.check(_lib.mg_cow_o1_bwd(side, _p(o_0), _p(o_1), _p(dys[0]), _p(dys[1]), _p(dys[2]), rows, chan,
+                                       _p(d0), _p(d1), _stream()))
+    return [d0, d1]
+
+
+def cow_o0_bwl(r_0, r_1, *dys):
+    return _cow_bwd(0, 0, r_0, r_1, dys)
+
+
+def cow_o0_bwr(l_0, l_1, *dys):
+    return _cow_bwd(0, 1, l_0, l_1, dys)
+
+
+def cow_o1_bwl(r_0, r_1, *dys):
+    return _cow_bwd(1, 0, r_0, r_1, dys)
+
+
+def cow_o1_bwr(l_0, l_1, *dys):
+    return _cow_bwd(1, 1, l_0, l_1, dys)
+
+
+def tensor_prod_bare(inds_l, inds_r, inds_o, x_l, x_r):
+    """TensorProdBare.forward for operands (..., chan, (3,)^inds); leading dims must agree."""
+    _check_input(x_l, "x_l")
+    _check_input(x_r, "x_r")
+    lead_l = tuple(x_l.shape[:x_l.dim() - inds_l])
+    lead_r = tuple(x_r.shape[:x_r.dim() - inds_r])
+    if lead_l != lead_r:
+        raise RuntimeError(f"operands do not broadcast: {tuple(x_l.shape)} vs {tuple(x_r.shape)}")
+    if tuple(x_l.shape[x_l.dim() - inds_l:]) != (3,) * inds_l or tuple(x_r.shape[x_r.dim() - inds_r:]) != (3,) * inds_r:
+        raise RuntimeError("tensor axes must have size 3")
+    n = 1
+    for d in lead_l:
+        n *= int(d)
+    with torch.cuda.device(x_l.device):
+        y = torch.empty(lead_l + (3,) * inds_o, dtype=torch.float32, device=x_l.device)
+        L.check(_lib.mg_tensor_prod_bare(inds_l, inds_r, inds_o, _p(x_l), _p(x_r), n, 1, _p(y), _stream()))
+    return y
+
+
+def tensor_prods_avd(a, v_l, v_r):
+    """(v_l . v_r, a v_r, v_l (x) v_r) in one pass; a: (..., C), v: (..., C, 3)."""
+    for t, nm in ((a, "a"), (v_l, "v_l"), (v_r, "v_r")):
+        _check_input(t, nm)
+    if tuple(v_l.shape) != tuple(a.shape) + (3,) or tuple(v_r.shape) != tuple(v_l.shape):
+        raise RuntimeError("shape mismatch")
+    n = int(a.numel())
+    dev = a.device
+    with torch.cuda.device(dev):
+        y0 = torch.empty_like(a)
+        y1 = torch.empty_like(v_l)
+        y2 = torch.empty(tuple(v_l.shape) + (3,), dtype=torch.float32, device=dev)
+        L.check(_lib.mg_tensor_prods_avd(_p(a), _p(v_l), _p(v_r), n, 1, _p(y0), _p(y1), _p(y2), _stream()))
+    return y0, y1, y2
+
+
+ACT_NONE, ACT_SILU, ACT_LEAKY = 0, 1, 2
+
+
+def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=False):
+    """y[..., o, t] = act(sum_i W[o, i] x[..., i, t] + bias[o]); W may have any strides."""
+    if not W.is_cuda:
+        raise RuntimeError("W must be a CUDA tensor")
+    _check_input(x, "x")
+    if W.dtype != torch.float32:
+        raise RuntimeError("W must be float32")
+    if W.dim() != 2:
+        raise RuntimeError("expected W to be a matrix (2 dims)")
+    if inds > 2 or inds < 0:
+        raise RuntimeError("tensor_linear currently only supports a number of indices up to 2. "
+                           "go edit the code to add more (easy with copy/paste).")
+    dim_out, dim_in = int(W.size(0)), int(W.size(1))
+    batch_dims = x.dim() - (1 + inds)
+    if batch_dims < 0:
+        raise RuntimeError("x has too few dims")
+    if x.size(batch_dims) != dim_in:
+        raise RuntimeError("channel dim size mismatch for x")
+    for i in range(batch_dims + 1, batch_dims + inds + 1):
+        if x.size(i) != 3:
+            raise RuntimeError("expected tensor index dim to be 3d for input x")
+    rows = 1
+    for i in range(batch_dims):
+        rows *= int(x.size(i))
+    y_shape = list(x.shape)
+    y_shape[batch_dims] = dim_out
+    if bias is not None:
+        _check_input(bias, "bias")
+        if bias.numel() != dim_out:
+            raise RuntimeError("bias size mismatch")
+    with torch.cuda.device(x.device):
+        if out is None:
+            y = torch.empty(y_shape, dtype=torch.float32, device=x.device)
+        else:
+            _check_input(out, "out")
+            if list(out.shape) != y_shape:
+                raise RuntimeError("out has wrong shape")
+            y = out
+        L.check(_lib.mg_tensor_linear(inds, _p(W), int(W.stride(0)), int(W.stride(1)), _p(x), rows, dim_in, dim_out,
+                                      _p(bias), int(act), int(bool(accumulate)), _p(y), _stream()))
+    return y
+
+
+def tensor_linear_wgrad(inds, dy, x):
+    _check_input(dy, "dy")
+    _check_input(x, "x")
+    batch_dims = x.dim() - (1 + inds)
+    dim_in, dim_out = int(x.size(batch_dims)), int(dy.size(batch_dims))
+    rows = 1
+    for i in range(batch_dims):
+        rows *= int(x.size(i))
+    with torch.cuda.device(x.device):
+        dW = torch.empty(dim_out, dim_in, dtype=torch.float32, device=x.device)
+        L.check(_lib.mg_tensor_linear_wgrad(inds, _p(dy), _p(x), rows, dim_in, dim_out, _p(dW), _stream()))
+    return dW

@@ -1,0 +1,79 @@
+"""TensLinear / TensorProdBare / TensorProds and the small tensor norms,
+mirroring managan/tensor_products.py of the reference (same class names,
+constructor arguments and parameter names, so state dicts load unchanged) on
+top of the HIP kernels."""
+import torch
+import torch.nn as nn
+
+from . import ops
+
+
+class _TensorLinearFn(torch.autograd.Function):
+    """tensor_linear with gradients for W and x (extensions/tensor_ops/tensor_ops.cpp:31-169)."""
+
+    @staticmethod
+    def forward(ctx, inds, W, x):
+        ctx.inds = inds
+        ctx.save_for_backward(W, x)
+        return ops.tensor_linear_fwd(inds, W, x)
+
+    @staticmethod
+    def backward(ctx, dy):
+        W, x = ctx.saved_tensors
+        dy = dy.contiguous()
+        dW = dx = None
+        if ctx.needs_input_grad[1]:
+            dW = ops.tensor_linear_wgrad(ctx.inds, dy, x)
+        if ctx.needs_input_grad[2]:
+            dx = ops.tensor_linear_fwd(ctx.inds, W.t(), dy)   # strides of W are honoured: no copy
+        return None, dW, dx
+
+
+def tensor_linear(inds, W, x):
+    return _TensorLinearFn.apply(inds, W, x)
+
+
+class TensLinear(nn.Module):
+    """Linear layer for arbitrary tensor activations (managan/tensor_products.py:26-37)."""
+
+    def __init__(self, inds, dim_in, dim_out):
+        super().__init__()
+        self.W = nn.Parameter(torch.empty(dim_out, dim_in))
+        self.inds = inds
+        self.self_init()
+
+    def self_init(self):
+        _, fan_in = self.W.shape
+        nn.init.normal_(self.W, std=fan_in ** -0.5)
+
+    def forward(self, x):
+        return tensor_linear(self.inds, self.W, x.contiguous())
+
+
+class TensorProdBare(nn.Module):
+    """Tensor product with no linear maps around it (managan/tensor_products.py:91-106)."""
+
+    def __init__(self, inds_l, inds_r, inds_o):
+        super().__init__()
+        assert (inds_l + inds_r - inds_o) % 2 == 0, "parity mismatch"
+        contracts = (inds_l + inds_r - inds_o) // 2
+        assert 0 <= contracts <= min(inds_l, inds_r), \
+            f"{contracts} contractions is out of range for {inds_l}, {inds_r} index tensors"
+        self.inds = (inds_l, inds_r, inds_o)
+
+    def forward(self, x_l, x_r):
+        return ops.tensor_prod_bare(*self.inds, x_l.contiguous(), x_r.contiguous())
+
+
+class TensorProds(nn.Module):
+    """Tensor product sandwiched by linear maps (managan/tensor_products.py:109-121)."""
+
+    def __init__(self, inds_l: int, inds_r: int, inds_o: int, dim_l: int, dim_r: int, dim_o: int, rank: int):
+        super().__init__()
+        self.prod = TensorProdBare(inds_l, inds_r, inds_o)
+        self.lin_l = TensLinear(inds_l, dim_l, rank)
+        self.lin_r = TensLinear(inds_r, dim_r, rank)
+        self.lin_o = TensLinear(inds_o, rank, dim_o)
+
+    def forward(self, x_l, x_r):
+        return self.lin_o(self.prod(self.lin_l(x_l), self.lin_r(x_r)))

@@ -1,0 +1,87 @@
+"""MFMA tensor_linear against the oracle (plain matmul), rel 1e-5 / abs 1e-6
+scaled by the reduction length (fp32 accumulation order differs)."""
+import importlib
+
+import pytest
+import torch
+
+from oracle import products as OP
+
+pytestmark = pytest.mark.gpu
+
+
+def _check(y, ref, dim_in):
+    # accumulation-order noise grows like sqrt(K) * eps * |terms|
+    torch.testing.assert_close(y.cpu(), ref, rtol=1e-5, atol=1e-6 * max(1.0, dim_in ** 0.5))
+
+
+@pytest.mark.parametrize("inds", [0, 1, 2])
+@pytest.mark.parametrize("dims", [(64, 64), (117, 210), (16, 512), (128, 32), (8, 128), (20, 256), (1, 64), (64, 1)])
+def test_tensor_linear(ops, inds, dims):
+    dim_in, dim_out = dims
+    g = torch.Generator().manual_seed(100 + inds)
+    W = torch.randn(dim_out, dim_in, generator=g) * dim_in ** -0.5
+    x = torch.randn(10, 37, dim_in, *([3] * inds), generator=g)
+    y = ops.tensor_linear_fwd(inds, W.cuda(), x.cuda())
+    assert tuple(y.shape) == (10, 37, dim_out) + (3,) * inds
+    _check(y, OP.tensor_linear(inds, W, x), dim_in)
+
+
+@pytest.mark.parametrize("inds", [0, 1, 2])
+def test_tensor_linear_transposed_weight(ops, inds):
+    g = torch.Generator().manual_seed(7)
+    W = torch.randn(96, 48, generator=g)
+    x = torch.randn(50, 96, *([3] * inds), generator=g)
+    y = ops.tensor_linear_fwd(inds, W.cuda().t(), x.cuda())
+    _check(y, OP.tensor_linear(inds, W.t(), x), 96)
+
+
+def test_tensor_linear_large_rows(ops):
+    g = torch.Generator().manual_seed(8)
+    W = torch.randn(512, 512, generator=g) / 512 ** 0.5
+    x = torch.randn(3000, 512, generator=g)
+    b = torch.randn(512, generator=g)
+    y = ops.tensor_linear_fwd(0, W.cuda(), x.cuda(), bias=b.cuda(), act=ops.ACT_SILU)
+    ref = torch.nn.functional.silu(torch.nn.functional.linear(x, W, b))
+    _check(y, ref, 512)
+    y2 = ops.tensor_linear_fwd(0, W.cuda(), x.cuda(), bias=b.cuda(), act=ops.ACT_LEAKY)
+    _check(y2, torch.nn.functional.leaky_relu(torch.nn.functional.linear(x, W, b), 0.1), 512)
+
+
+def test_tensor_linear_accumulate(ops):
+    g = torch.Generator().manual_seed(9)
+    W = torch.randn(40, 24, generator=g)
+    x = torch.randn(33, 24, 3, generator=g)
+    base = torch.randn(33, 40, 3, generator=g)
+    out = base.cuda().clone()
+    ops.tensor_linear_fwd(1, W.cuda(), x.cuda(), out=out, accumulate=True)
+    _check(out, base + OP.tensor_linear(1, W, x), 24)
+
+
+def test_tensor_linear_empty_and_errors(ops):
+    W = torch.randn(8, 4).cuda()
+    y = ops.tensor_linear_fwd(1, W, torch.empty(0, 4, 3).cuda())
+    assert tuple(y.shape) == (0, 8, 3)
+    with pytest.raises(RuntimeError, match="channel dim size mismatch"):
+        ops.tensor_linear_fwd(0, W, torch.randn(3, 5).cuda())
+    with pytest.raises(RuntimeError, match="3d"):
+        ops.tensor_linear_fwd(1, W, torch.randn(3, 4, 2).cuda())
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ops.tensor_linear_fwd(0, W, torch.randn(4, 3).cuda().t())
+    with pytest.raises(RuntimeError, match="up to 2"):
+        ops.tensor_linear_fwd(3, W, torch.randn(2, 4, 3, 3, 3).cuda())
+
+
+@pytest.mark.parametrize("inds", [0, 1, 2])
+def test_tensor_linear_autograd(pkg, inds):
+    tp = importlib.import_module("learned-dynamics_amd.tensor_products")
+    g = torch.Generator().manual_seed(10)
+    W = torch.randn(70, 50, generator=g)
+    x = torch.randn(6, 21, 50, *([3] * inds), generator=g)
+    dy = torch.randn(6, 21, 70, *([3] * inds), generator=g)
+    Wr, xr = W.clone().requires_grad_(True), x.clone().requires_grad_(True)
+    OP.tensor_linear(inds, Wr, xr).backward(dy)
+    Wg, xg = W.cuda().requires_grad_(True), x.cuda().requires_grad_(True)
+    tp.tensor_linear(inds, Wg, xg).backward(dy.cuda())
+    torch.testing.assert_close(xg.grad.cpu(), xr.grad, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(Wg.grad.cpu(), Wr.grad, rtol=1e-5, atol=1e-4)

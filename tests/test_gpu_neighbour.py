@@ -1,0 +1,165 @@
+"""HIP periodic neighbour search against the C oracle: sorted (src, dst, image
+shift) edge sets must be bit-identical."""
+import importlib
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import neighbour as ON
+
+pytestmark = pytest.mark.gpu
+
+
+def _triples(src, dst, shift=None):
+    return ON.sorted_triples(np.asarray(src), np.asarray(dst), None if shift is None else np.asarray(shift))
+
+
+def _run(ops, x, cutoff, box, listmax=256, nmax=100000):
+    xt = torch.from_numpy(x).cuda()
+    src, dst, ec, row_ptr = ops.get_edges(listmax, nmax, cutoff, *box, xt, return_row_ptr=True)
+    return xt, src, dst, ec, row_ptr
+
+
+def _compare(ops, x, cutoff, box, mode=ON.MODE_CELLS):
+    xt, src, dst, ec, row_ptr = _run(ops, x, cutoff, box)
+    ref = ON.edges(x, cutoff, box, mode)
+    s, d = src.cpu().numpy(), dst.cpu().numpy()
+    assert len(s) == len(ref["src"]), (len(s), len(ref["src"]))
+    assert np.all(s[1:] >= s[:-1]), "src must be non-decreasing"
+    np.testing.assert_array_equal(ec.cpu().numpy(), ref["edge_counts"])
+    np.testing.assert_array_equal(np.diff(row_ptr.cpu().numpy()), ref["counts"].reshape(-1))
+    np.testing.assert_array_equal(_triples(s, d), _triples(ref["src"], ref["dst"]))
+    # derived quantities: r_ij and the periodic image shift
+    r, shift = ops.edge_vectors(xt.reshape(-1, 3), src, dst, box, want_shift=True)
+    np.testing.assert_array_equal(r.cpu().numpy(), ON.edge_vectors(x, s, d, box))
+    ref_shift = ON.image_shift(x, ref["src"], ref["dst"], box)
+    np.testing.assert_array_equal(_triples(s, d, shift.cpu().numpy()),
+                                  _triples(ref["src"], ref["dst"], ref_shift))
+    return ref
+
+
+def test_golden_five_points(ops):
+    """Hand-placed points of the reference's self test (managan/graph_layers.py:83-103)."""
+    pos = np.array([[[0., 0., -1.], [1., 0., 0.], [3., 0., 0.], [2., 1., 0.], [8., 0., 0.]]], dtype=np.float32)
+    xt, src, dst, ec, row_ptr = _run(ops, pos, 2.0, (100., 100., 100.), listmax=32, nmax=64)
+    assert np.array_equal(np.diff(row_ptr.cpu().numpy()), [1, 3, 2, 2, 0])
+    got = set(zip(src.tolist(), dst.tolist()))
+    assert got == {(0, 1), (1, 0), (1, 2), (1, 3), (2, 1), (2, 3), (3, 1), (3, 2)}
+    assert ec.tolist() == [8]
+
+
+def test_wrap_cells_bit_exact(ops):
+    rng = np.random.default_rng(5)
+    box = (30.5, 33.5, 36.5)
+    x = ((rng.random((4, 5000, 3)) * 5 - 2) * np.array(box)).astype(np.float32)
+    x[0, :10] = np.array(box, dtype=np.float32) * np.array([0.5, 1.0, 0.0], dtype=np.float32)  # ties / edges
+    w, cell = ops.wrap_cells(7.0, box, torch.from_numpy(x).cuda())
+    w_ref, cell_ref = ON.wrap_cells(x, 7.0, box)
+    np.testing.assert_array_equal(w.cpu().numpy(), w_ref)
+    np.testing.assert_array_equal(cell.cpu().numpy(), cell_ref)
+
+
+def test_reference_test_shape(ops):
+    """B=20, N=60, box (30.5,33.5,36.5), cutoff 7 (extensions/neighbour_grid/test.py:9-16)."""
+    g = torch.Generator().manual_seed(0x947)
+    box = (30.5, 33.5, 36.5)
+    x = (torch.rand(20, 60, 3, generator=g) * torch.tensor(box)).numpy()
+    ref = _compare(ops, x, 7.0, box)
+    # adjacency symmetric (test.py:22-32)
+    E = set(zip(ref["src"].tolist(), ref["dst"].tolist()))
+    assert all((b, a) in E for a, b in E)
+
+
+def test_unwrapped_and_clustered(ops):
+    """Positions far outside the box, all atoms of one box in one cell, and an empty-ish box."""
+    rng = np.random.default_rng(7)
+    box = (24., 27., 31.)
+    x = (rng.standard_normal((3, 700, 3)) * 40).astype(np.float32)
+    x[1] = (rng.random((700, 3)) * 2.0 + 500.0).astype(np.float32)      # dense cluster: degree 699
+    _compare(ops, x, 8.0, box)
+
+
+def test_under_resolved_grid(ops):
+    """box/cutoff not an integer: the 3x3x3 window misses pairs two cells apart; the HIP path
+    must reproduce the reference's set, which differs from the plain minimum-image graph."""
+    rng = np.random.default_rng(11)
+    box = (70., 70., 70.)
+    x = (rng.random((2, 20000, 3)) * 70).astype(np.float32)
+    ref = _compare(ops, x, 6.0, box)
+    plain = ON.edges(x, 6.0, box, ON.MODE_BRUTE_MINIMAGE) if False else None
+    assert ref["max_degree"] > 0
+
+
+def test_sparse_box_uses_single_wave_blocks(ops):
+    rng = np.random.default_rng(13)
+    box = (70., 70., 70.)
+    x = (rng.random((32, 2048, 3)) * 70).astype(np.float32)
+    _compare(ops, x, 6.0, box)
+
+
+def test_many_candidates_exceed_lds_tile(ops):
+    """More than 2048 candidates in a 27-cell window: the tail is read from global memory."""
+    rng = np.random.default_rng(17)
+    box = (12., 12., 12.)
+    x = (rng.random((1, 3000, 3)) * 12).astype(np.float32)     # 27 cells of 4 A: ~111 atoms per cell
+    _compare(ops, x, 4.0, box)
+
+
+def test_config2_one_box(ops):
+    g = torch.Generator().manual_seed(0x947 + 2)
+    x = (torch.rand(8, 16384, 3, generator=g) * 55).numpy()[:2]
+    ref = _compare(ops, np.ascontiguousarray(x), 5.0, (55., 55., 55.))
+    assert 1_600_000 < len(ref["src"]) < 1_800_000
+
+
+def test_errors(ops):
+    x = torch.rand(1, 100, 3).cuda() * 10
+    with pytest.raises(RuntimeError, match="greater than 3\\*cutoff"):
+        ops.get_edges(32, 64, 4.0, 10., 10., 10., x)
+    dense = torch.rand(1, 400, 3).cuda() * 9
+    with pytest.raises(RuntimeError, match="Cell list overflow"):
+        ops.get_edges(4, 1000, 3.0, 9., 9., 9., dense)
+    with pytest.raises(RuntimeError, match="one of 32, 64, 128, 256"):
+        ops.get_edges(100, 1000, 3.0, 9., 9., 9., dense)
+    with pytest.raises(RuntimeError, match="Neighbour list overflow"):
+        ops.get_edges(32, 2, 3.0, 9., 9., 9., dense)
+    with pytest.raises(RuntimeError, match="shape"):
+        ops.get_edges(32, 64, 3.0, 9., 9., 9., torch.rand(100, 3).cuda())
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ops.get_edges(32, 64, 3.0, 9., 9., 9., torch.rand(1, 3, 100).cuda().transpose(1, 2))
+    with pytest.raises(RuntimeError, match="CUDA"):
+        ops.get_edges(32, 64, 3.0, 9., 9., 9., torch.rand(1, 100, 3))
+
+
+def test_empty(ops):
+    src, dst, ec = ops.get_edges(32, 64, 3.0, 9., 9., 9., torch.empty(0, 10, 3).cuda())
+    assert src.numel() == 0 and ec.numel() == 0
+    src, dst, ec = ops.get_edges(32, 64, 3.0, 9., 9., 9., torch.empty(2, 0, 3).cuda())
+    assert src.numel() == 0 and ec.tolist() == [0, 0]
+    src, dst, ec = ops.get_edges(32, 64, 1.0, 90., 90., 90., torch.rand(2, 5, 3).cuda() * 90)
+    assert ec.numel() == 2
+
+
+def test_deterministic_order(ops):
+    rng = np.random.default_rng(19)
+    x = torch.from_numpy((rng.random((2, 4000, 3)) * 30).astype(np.float32)).cuda()
+    a = ops.get_edges(64, 512, 5.0, 30., 30., 30., x)
+    b = ops.get_edges(64, 512, 5.0, 30., 30., 30., x)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+
+
+def test_padded_api(ops):
+    """get_neighbours / edges_read / edges_reduce invariants (extensions/neighbour_grid/test.py:35-46)."""
+    g = torch.Generator().manual_seed(3)
+    box = (30.5, 33.5, 36.5)
+    x = (torch.rand(20, 60, 3, generator=g) * torch.tensor(box)).cuda()
+    neighbours, counts = ops.get_neighbours(32, 32, 7.0, *box, x)
+    idx = torch.arange(60, device="cuda")[None, :, None].expand(20, -1, -1).contiguous().float()
+    read = ops.padded_edges_read(counts, neighbours, idx)
+    mask = torch.arange(32, device="cuda")[None, None, :] < counts[:, :, None]
+    assert torch.equal(read[..., 0][mask], neighbours[mask].float())
+    assert torch.all(read[..., 0][~mask] == 0)
+    ones = torch.ones(20, 60, 7, device="cuda")
+    red = ops.padded_edges_reduce(counts, neighbours, ops.padded_edges_read(counts, neighbours, ones))
+    assert torch.equal(red[:, :, 0], counts.float())
