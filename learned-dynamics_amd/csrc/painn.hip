@@ -1,0 +1,242 @@
+// PaiNN message passing (edge side), fused gather-product-scatter over CSR rows.
+//
+// For edge e = (i <- j) with filter W(e) in R^{4n} (output of the radial MLP),
+// node activations A(j) in R^{4n}, node vectors v(j) in R^{n x 3} and unit-ish
+// direction u = r / sqrt(eps + |r|^2):
+//     P     = W(e) * A(j)                                  (elementwise, 4 blocks of n)
+//     m_v   = v(j) * P0 + (v(j) x u) * P1 + u (x) P2       (n x 3)
+//     m_a   = P3                                           (n)
+//     out_v(i) = res_v(i) + sum_j m_v,   out_a(i) = res_a(i) + sum_j m_a
+// Nothing per-edge is written to HBM: the only streamed operand is the filter
+// (16n bytes per edge); A(j) and v(j) are gathers of node-sized arrays that live
+// in L2 / Infinity Cache.  One wave owns (node, channel chunk); a lane owns four
+// consecutive channels and moves them with 16-byte accesses; when the chunk is
+// narrower than the wave the spare lanes take the next edges of the same node and
+// are folded with xor-shuffles.  Rows are summed in edge order: no atomics.
+#include "common.hpp"
+
+namespace mg {
+namespace {
+
+constexpr int kMaxChunks = 16;
+struct Chunks {
+    int n;
+    int start[kMaxChunks];   // first channel of the chunk
+    int lanes[kMaxChunks];   // lanes per edge, power of two <= 64
+};
+
+inline Chunks make_chunks(int units, int unit_width) {
+    Chunks c{};
+    int pos = 0;
+    while (units > 0 && c.n < kMaxChunks) {
+        int p = 64;
+        while (p > units) p >>= 1;
+        c.start[c.n] = pos * unit_width;
+        c.lanes[c.n] = p;
+        c.n++;
+        pos += p;
+        units -= p;
+    }
+    return c;
+}
+
+__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+__device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
+__device__ __forceinline__ float4 mul4(float4 a, float4 b) { return make_float4(a.x * b.x, a.y * b.y, a.z * b.z, a.w * b.w); }
+
+struct EdgeAcc {
+    float v[12];   // 4 channels x 3 components, channel-major (as in memory)
+    float a[4];
+    __device__ void zero() {
+#pragma unroll
+        for (int k = 0; k < 12; k++) v[k] = 0.f;
+#pragma unroll
+        for (int k = 0; k < 4; k++) a[k] = 0.f;
+    }
+};
+
+// accumulate one edge for 4 consecutive channels starting at c
+__device__ __forceinline__ void edge_term(EdgeAcc& acc, const float* __restrict__ filt_row,
+                                          const float* __restrict__ actv_row, const float* __restrict__ xv_row,
+                                          int n, int c, float ux, float uy, float uz) {
+    const float4 p0 = mul4(ld4(filt_row + c), ld4(actv_row + c));
+    const float4 p1 = mul4(ld4(filt_row + n + c), ld4(actv_row + n + c));
+    const float4 p2 = mul4(ld4(filt_row + 2 * n + c), ld4(actv_row + 2 * n + c));
+    const float4 p3 = mul4(ld4(filt_row + 3 * n + c), ld4(actv_row + 3 * n + c));
+    const float4 va = ld4(xv_row + 3 * c), vb = ld4(xv_row + 3 * c + 4), vc = ld4(xv_row + 3 * c + 8);
+    const float vv[12] = {va.x, va.y, va.z, va.w, vb.x, vb.y, vb.z, vb.w, vc.x, vc.y, vc.z, vc.w};
+    const float q0[4] = {p0.x, p0.y, p0.z, p0.w}, q1[4] = {p1.x, p1.y, p1.z, p1.w};
+    const float q2[4] = {p2.x, p2.y, p2.z, p2.w}, q3[4] = {p3.x, p3.y, p3.z, p3.w};
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const float x = vv[3 * k], y = vv[3 * k + 1], z = vv[3 * k + 2];
+        const float cx = y * uz - z * uy, cy = z * ux - x * uz, cz = x * uy - y * ux;   // v x u
+        acc.v[3 * k + 0] += x * q0[k] + cx * q1[k] + ux * q2[k];
+        acc.v[3 * k + 1] += y * q0[k] + cy * q1[k] + uy * q2[k];
+        acc.v[3 * k + 2] += z * q0[k] + cz * q1[k] + uz * q2[k];
+        acc.a[k] += q3[k];
+    }
+}
+
+__global__ void __launch_bounds__(256) painn_message_kernel(
+    const int* __restrict__ row_ptr, const int* __restrict__ dst, long n_nodes, const float* __restrict__ r_ij,
+    const float* __restrict__ filt, const float* __restrict__ actv, const float* __restrict__ x_v, int n,
+    float epsilon, const float* __restrict__ res_a, const float* __restrict__ res_v, float* __restrict__ out_a,
+    float* __restrict__ out_v, Chunks ch) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const long wave_global = ((long)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+    const long n_waves = ((long)gridDim.x * blockDim.x) / kWave;
+    const long items = n_nodes * ch.n;
+    const long row_f = 4L * n;
+    for (long item = wave_global; item < items; item += n_waves) {
+        const long node = item / ch.n;
+        const int ci = (int)(item - node * ch.n);
+        const int L = ch.lanes[ci];
+        const int c = ch.start[ci] + (lane & (L - 1)) * 4;
+        const int sub = lane / L, per_iter = kWave / L;
+        const long lo = row_ptr[node], hi = row_ptr[node + 1];
+        EdgeAcc acc;
+        acc.zero();
+        for (long e = lo + sub; e < hi; e += per_iter) {
+            const long j = dst[e];
+            const float rx = r_ij[3 * e], ry = r_ij[3 * e + 1], rz = r_ij[3 * e + 2];
+            const float inv = 1.0f / sqrtf(epsilon + (rx * rx + ry * ry + rz * rz));
+            edge_term(acc, filt + e * row_f, actv + j * row_f, x_v + j * 3L * n, n, c, rx * inv, ry * inv, rz * inv);
+        }
+        for (int d = L; d < kWave; d <<= 1) {
+#pragma unroll
+            for (int k = 0; k < 12; k++) acc.v[k] += __shfl_xor(acc.v[k], d);
+#pragma unroll
+            for (int k = 0; k < 4; k++) acc.a[k] += __shfl_xor(acc.a[k], d);
+        }
+        if (sub == 0) {
+            float* oa = out_a + node * n + c;
+            float* ov = out_v + (node * n + c) * 3;
+            if (res_a) {
+                const float4 r = ld4(res_a + node * n + c);
+                acc.a[0] += r.x; acc.a[1] += r.y; acc.a[2] += r.z; acc.a[3] += r.w;
+            }
+            if (res_v) {
+                const float* rv = res_v + (node * n + c) * 3;
+                const float4 ra = ld4(rv), rb = ld4(rv + 4), rc = ld4(rv + 8);
+                const float rr[12] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w, rc.x, rc.y, rc.z, rc.w};
+#pragma unroll
+                for (int k = 0; k < 12; k++) acc.v[k] += rr[k];
+            }
+            st4(oa, make_float4(acc.a[0], acc.a[1], acc.a[2], acc.a[3]));
+            st4(ov, make_float4(acc.v[0], acc.v[1], acc.v[2], acc.v[3]));
+            st4(ov + 4, make_float4(acc.v[4], acc.v[5], acc.v[6], acc.v[7]));
+            st4(ov + 8, make_float4(acc.v[8], acc.v[9], acc.v[10], acc.v[11]));
+        }
+    }
+}
+
+// fallback for channel counts that are not a multiple of 4 or unaligned operands:
+// one lane per channel, one wave per (node, 64-channel chunk)
+__global__ void __launch_bounds__(256) painn_message_scalar_kernel(
+    const int* __restrict__ row_ptr, const int* __restrict__ dst, long n_nodes, const float* __restrict__ r_ij,
+    const float* __restrict__ filt, const float* __restrict__ actv, const float* __restrict__ x_v, int n,
+    float epsilon, const float* __restrict__ res_a, const float* __restrict__ res_v, float* __restrict__ out_a,
+    float* __restrict__ out_v) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const long wave_global = ((long)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+    const long n_waves = ((long)gridDim.x * blockDim.x) / kWave;
+    const int chunks = (n + kWave - 1) / kWave;
+    const long items = n_nodes * chunks;
+    const long row_f = 4L * n;
+    for (long item = wave_global; item < items; item += n_waves) {
+        const long node = item / chunks;
+        const int c = (int)(item - node * chunks) * kWave + lane;
+        if (c >= n) continue;
+        float ax = 0.f, ay = 0.f, az = 0.f, aa = 0.f;
+        for (long e = row_ptr[node]; e < row_ptr[node + 1]; e++) {
+            const long j = dst[e];
+            const float rx = r_ij[3 * e], ry = r_ij[3 * e + 1], rz = r_ij[3 * e + 2];
+            const float inv = 1.0f / sqrtf(epsilon + (rx * rx + ry * ry + rz * rz));
+            const float ux = rx * inv, uy = ry * inv, uz = rz * inv;
+            const float* f = filt + e * row_f;
+            const float* a = actv + j * row_f;
+            const float p0 = f[c] * a[c], p1 = f[n + c] * a[n + c], p2 = f[2 * n + c] * a[2 * n + c];
+            const float p3 = f[3 * n + c] * a[3 * n + c];
+            const float* v = x_v + (j * n + c) * 3;
+            const float x = v[0], y = v[1], z = v[2];
+            ax += x * p0 + (y * uz - z * uy) * p1 + ux * p2;
+            ay += y * p0 + (z * ux - x * uz) * p1 + uy * p2;
+            az += z * p0 + (x * uy - y * ux) * p1 + uz * p2;
+            aa += p3;
+        }
+        const long o = node * n + c;
+        if (res_a) aa += res_a[o];
+        if (res_v) { ax += res_v[3 * o]; ay += res_v[3 * o + 1]; az += res_v[3 * o + 2]; }
+        out_a[o] = aa;
+        out_v[3 * o] = ax; out_v[3 * o + 1] = ay; out_v[3 * o + 2] = az;
+    }
+}
+
+// out[e, m] = cos(k_m d) for m < hn, sin(k_{m-hn} d) for hn <= m < n, k_m = (pi/rmax)(1 + m/2), hn = (n+1)/2
+__global__ void __launch_bounds__(256) radial_encode_painn_kernel(const float* __restrict__ r_ij, long E, int n,
+                                                                  float base, float* __restrict__ out) {
+    const long total = E * n;
+    const int hn = (n + 1) / 2;
+    for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (long)gridDim.x * blockDim.x) {
+        const long e = t / n;
+        const int m = (int)(t - e * n);
+        const float x = r_ij[3 * e], y = r_ij[3 * e + 1], z = r_ij[3 * e + 2];
+        const float d = sqrtf(x * x + y * y + z * z);
+        const int f = m < hn ? m : m - hn;
+        const float phase = (base * (float)(1 + f / 2)) * d;
+        out[t] = m < hn ? cosf(phase) : sinf(phase);
+    }
+}
+
+}  // namespace
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" {
+
+int mg_painn_radial_encode(const float* r_ij, long n_edges, int n, float rmax, float* out, mg_stream_t stream) {
+    MG_REQUIRE(n_edges >= 0 && n >= 0, "mg_painn_radial_encode: negative size");
+    MG_REQUIRE(rmax > 0.f, "mg_painn_radial_encode: rmax must be positive");
+    const long total = n_edges * n;
+    if (total == 0) return MG_OK;
+    MG_REQUIRE(r_ij && out, "mg_painn_radial_encode: null pointer");
+    const float base = (float)(3.14159265358979323846 / (double)rmax);
+    long blocks = ceil_div(total, 256);
+    if (blocks > 256L * 64) blocks = 256L * 64;
+    hipLaunchKernelGGL(radial_encode_painn_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, r_ij,
+                       n_edges, n, base, out);
+    return check_launch("mg_painn_radial_encode");
+}
+
+int mg_painn_message(const int* row_ptr, const int* dst, int n_nodes, long n_edges, const float* r_ij,
+                     const float* filt, const float* actv, const float* x_v, int n, float epsilon,
+                     const float* res_a, const float* res_v, float* out_a, float* out_v, mg_stream_t stream) {
+    MG_REQUIRE(n_nodes >= 0 && n_edges >= 0 && n >= 0, "mg_painn_message: negative size");
+    if (n_nodes == 0 || n == 0) return MG_OK;
+    MG_REQUIRE(row_ptr && out_a && out_v && actv && x_v, "mg_painn_message: null pointer");
+    MG_REQUIRE(n_edges == 0 || (dst && r_ij && filt), "mg_painn_message: null edge operand");
+    hipStream_t st = (hipStream_t)stream;
+    const bool vec = (n % 4 == 0) && aligned16(filt) && aligned16(actv) && aligned16(x_v) && aligned16(out_a) &&
+                     aligned16(out_v) && (!res_a || aligned16(res_a)) && (!res_v || aligned16(res_v));
+    if (vec) {
+        const Chunks ch = make_chunks(n / 4, 4);
+        int covered = 0;
+        for (int k = 0; k < ch.n; k++) covered += ch.lanes[k] * 4;
+        if (covered == n) {
+            long blocks = ceil_div((long)n_nodes * ch.n, 4);
+            if (blocks > 256L * 64) blocks = 256L * 64;
+            hipLaunchKernelGGL(painn_message_kernel, dim3((unsigned)blocks), dim3(256), 0, st, row_ptr, dst,
+                               (long)n_nodes, r_ij, filt, actv, x_v, n, epsilon, res_a, res_v, out_a, out_v, ch);
+            return check_launch("mg_painn_message");
+        }
+    }
+    long blocks = ceil_div((long)n_nodes * ceil_div(n, kWave), 4);
+    if (blocks > 256L * 64) blocks = 256L * 64;
+    hipLaunchKernelGGL(painn_message_scalar_kernel, dim3((unsigned)blocks), dim3(256), 0, st, row_ptr, dst,
+                       (long)n_nodes, r_ij, filt, actv, x_v, n, epsilon, res_a, res_v, out_a, out_v);
+    return check_launch("mg_painn_message");
+}
+
+}  // extern "C"

@@ -15,9 +15,14 @@ def _triples(src, dst, shift=None):
     return ON.sorted_triples(np.asarray(src), np.asarray(dst), None if shift is None else np.asarray(shift))
 
 
-def _run(ops, x, cutoff, box, listmax=256, nmax=100000):
+def _run(ops, x, cutoff, box, listmax=None, nmax=None):
     xt = torch.from_numpy(x).cuda()
-    src, dst, ec, row_ptr = ops.get_edges(listmax, nmax, cutoff, *box, xt, return_row_ptr=True)
+    if listmax is not None:
+        src, dst, ec, row_ptr = ops.get_edges(listmax, nmax, cutoff, *box, xt, return_row_ptr=True)
+    else:   # exact-size search without the reference's caps
+        search = ops.NeighbourSearch(xt, cutoff, box)
+        src, dst = search.fill()
+        ec, row_ptr = search.edge_counts, search.row_ptr
     return xt, src, dst, ec, row_ptr
 
 
@@ -87,7 +92,6 @@ def test_under_resolved_grid(ops):
     box = (70., 70., 70.)
     x = (rng.random((2, 20000, 3)) * 70).astype(np.float32)
     ref = _compare(ops, x, 6.0, box)
-    plain = ON.edges(x, 6.0, box, ON.MODE_BRUTE_MINIMAGE) if False else None
     assert ref["max_degree"] > 0
 
 
@@ -116,7 +120,7 @@ def test_config2_one_box(ops):
 def test_errors(ops):
     x = torch.rand(1, 100, 3).cuda() * 10
     with pytest.raises(RuntimeError, match="greater than 3\\*cutoff"):
-        ops.get_edges(32, 64, 4.0, 10., 10., 10., x)
+        ops.get_edges(32, 64, 5.5, 10., 10., 10., x)   # ceil(10/5.5) = 2 cells
     dense = torch.rand(1, 400, 3).cuda() * 9
     with pytest.raises(RuntimeError, match="Cell list overflow"):
         ops.get_edges(4, 1000, 3.0, 9., 9., 9., dense)
