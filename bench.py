@@ -1,0 +1,280 @@
+#!/usr/bin/env python3
+"""Benchmark of the equivariant message-passing hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload NAME] [--no-cpu]
+
+Prints ONE JSON line.  The default workload is BASELINE.json configs[2]: one
+PaiNN message-passing layer (Message + Update, n = 128, 16 radial functions) on
+16 polymer chains x 1024 beads in a periodic 80 A box with an 8 A cutoff; the
+metric is directed edges per second per layer.  A step is one forward pass of
+the layer with all inputs (positions, features, weights, edge list) resident in
+HBM.  Other workloads (reported under "other_workloads" and selectable with
+--workload): configs[1] neighbour search, configs[0] tensor-product trio.
+
+roofline: the kernel that dominates the step, timed on its own with HIP events
+on the launch stream: algorithmic FLOPs (or bytes) per launch / mean launch time.
+cpu_baseline: the CPU oracle (a port of the reference's math, not the
+reference's code) on a bounded sample of the same workload on the host cores.
+"""
+import argparse
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+PEAK_FP32_MFMA_TFLOPS = 157.3  # MI355X dense fp32 matrix
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="painn_layer",
+                    choices=["painn_layer", "neighbour", "products"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
+    ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
+    return ap.parse_args()
+
+
+def event_time(torch, fn, iters, warmup=2):
+    """Mean seconds per call, HIP events on the current (launch) stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(iters):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) * 1e-3 / iters
+
+
+def timed_steps(torch, fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+# ------------------------------------------------------------------ inputs
+def polymer_positions(torch, chains, beads, box, seed):
+    g = torch.Generator().manual_seed(seed)
+    steps = torch.randn(chains, beads, 3, generator=g)
+    steps = 3.8 * steps / steps.norm(dim=-1, keepdim=True)
+    origin = torch.rand(chains, 1, 3, generator=g) * box
+    return (steps.cumsum(1) + origin).reshape(1, chains * beads, 3).contiguous()
+
+
+def mlp_weights(mlp):
+    L = mlp.layers
+    return {"W1": L[0].weight.detach().cpu(), "b1": L[0].bias.detach().cpu(),
+            "W2": L[2].weight.detach().cpu(), "b2": L[2].bias.detach().cpu(),
+            "W3": L[4].weight.detach().cpu(), "b3": L[4].bias.detach().cpu()}
+
+
+# --------------------------------------------------------------- workloads
+def bench_painn_layer(torch, args):
+    ops = importlib.import_module("learned-dynamics_amd.ops")
+    painn = importlib.import_module("learned-dynamics_amd.painn")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    n, n_rbf, r0, box_len = 128, 16, 8.0, 80.0
+    box = (box_len,) * 3
+    seed = 0x947 + 3
+    torch.manual_seed(seed)
+    pos = polymer_positions(torch, 16, 1024, box_len, seed)
+    block = painn.Block(r0, n, n_rbf=n_rbf).cuda().eval()
+    g = torch.Generator().manual_seed(seed + 1)
+    x_a = torch.randn(1, 16384, n, generator=g)
+    x_v = torch.randn(1, 16384, n, 3, generator=g) / 3 ** 0.5
+    pos_d, x_a_d, x_v_d = pos.cuda(), x_a.cuda(), x_v.cuda()
+
+    with torch.no_grad():
+        graph, r_ij = gl.graph_setup(r0, box, pos_d, neighbours_max=512, celllist_max=128)
+        E, N = int(graph.src.numel()), 16384
+
+        def step():
+            return block((pos_d, graph, r_ij, None, None, x_a_d, x_v_d, box))
+
+        sec = timed_steps(torch, step, args.steps, args.warmup)
+
+        # --- dominant kernel: the 4n x 4n filter GEMM over E rows (fp32 MFMA)
+        h = torch.randn(E, 4 * n, device="cuda")
+        lin = block.message.mlp_dist.layers[2]
+        out = torch.empty(E, 4 * n, device="cuda")
+        t_gemm = event_time(torch, lambda: ops.tensor_linear_fwd(0, lin.weight, h, bias=lin.bias, act=ops.ACT_SILU,
+                                                                 out=out), 10)
+        flops = 2.0 * E * (4 * n) * (4 * n)
+        roofline = {"kernel": "linear_kernel<T=1,128x128> (filter MLP layer, E x 512 x 512)", "bound": "mfma",
+                    "achieved": flops / t_gemm / 1e12, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                    "frac": flops / t_gemm / 1e12 / PEAK_FP32_MFMA_TFLOPS, "traffic": None}
+        del h, out
+
+        # --- HBM-bound edge kernel: fused gather-product-scatter
+        filt = block.message.filters(r_ij)
+        actv = block.message.mlp_actv(x_a_d.reshape(N, n))
+        xv_flat, xa_flat = x_v_d.reshape(N, n, 3), x_a_d.reshape(N, n)
+        t_edge = event_time(torch, lambda: ops.painn_message(graph.row_ptr, graph.dst32, r_ij, filt, actv, xv_flat,
+                                                             0.1, xa_flat, xv_flat), 20)
+        edge_bytes = E * (16 * n + 4 + 12) + N * (16 * n + 16 * n)
+        roofline_hbm = {"kernel": "painn_message_kernel (fused gather-product-scatter)", "bound": "hbm",
+                        "achieved": edge_bytes / t_edge / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                        "frac": edge_bytes / t_edge / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                        "bytes_per_launch": edge_bytes, "ms": t_edge * 1e3}
+        t_graph = event_time(torch, lambda: gl.graph_setup(r0, box, pos_d, neighbours_max=512, celllist_max=128), 5)
+        breakdown = {"filter_gemm_512x512_ms": t_gemm * 1e3, "edge_kernel_ms": t_edge * 1e3,
+                     "graph_build_ms_not_in_step": t_graph * 1e3}
+        del filt, actv
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_painn_layer(torch, block, n, n_rbf, r0, box_len, seed)
+    result = {
+        "metric": "message-passing edges/sec per layer", "value": E / sec, "unit": "edges/s",
+        "ms_per_step": sec * 1e3, "dtype": "f32",
+        "config": {"workload": "BASELINE configs[2]: one PaiNN layer (Message + Update, residuals), 16 chains x 1024 "
+                               "beads, box 80 A, cutoff 8 A, n=128 scalar+128 vector channels, 16 radial functions",
+                   "edges": E, "atoms": N, "graph": "prebuilt (positions fixed); build time reported in breakdown"},
+        "roofline": roofline, "roofline_hbm": roofline_hbm, "breakdown": breakdown, "cpu_baseline": cpu,
+    }
+    return result
+
+
+def cpu_painn_layer(torch, block, n, n_rbf, r0, box_len, seed):
+    """Oracle (port of the reference math) on 2 of the 16 chains, host cores."""
+    from oracle import layers as OL
+    from oracle import neighbour as ON
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    box = (box_len,) * 3
+    pos = polymer_positions(torch, 2, 1024, box_len, seed)
+    Nc = pos.shape[1]
+    g = torch.Generator().manual_seed(seed + 2)
+    x_a = torch.randn(1, Nc, n, generator=g)
+    x_v = torch.randn(1, Nc, n, 3, generator=g) / 3 ** 0.5
+    ref = ON.edges(pos.numpy(), r0, box)
+    src, dst = torch.from_numpy(ref["src"]).long(), torch.from_numpy(ref["dst"]).long()
+    r_ij = torch.from_numpy(ON.edge_vectors(pos.numpy(), ref["src"], ref["dst"], box))
+    w_dist, w_actv = mlp_weights(block.message.mlp_dist), mlp_weights(block.message.mlp_actv)
+    w_upd = {"W_l": block.update.lin_l.W.detach().cpu(), "W_r": block.update.lin_r.W.detach().cpu(),
+             "W_v": block.update.lin_v.W.detach().cpu(), "mlp": mlp_weights(block.update.mlp),
+             "gn_gamma": block.update.gn.gamma.detach().cpu(), "gn_beta": block.update.gn.beta.detach().cpu()}
+
+    def layer():
+        da, dv = OL.painn_message(src, dst, 1, Nc, x_a, x_v, r_ij, w_dist, w_actv, r0, n, n_rbf)
+        xa, xv = x_a + da, x_v + dv
+        ua, uv = OL.painn_update(xa, xv, w_upd, n)
+        return xa + ua, xv + uv
+
+    with torch.no_grad():
+        layer()
+        times = []
+        t_all = time.perf_counter()
+        while len(times) < 3 or (time.perf_counter() - t_all < 10 and len(times) < 20):
+            t0 = time.perf_counter()
+            layer()
+            times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": len(src) / med, "unit": "edges/s", "cores": cores, "kind": "port",
+            "sample": f"2 of the 16 chains ({Nc} atoms, {len(src)} edges), same layer and weights, "
+                      f"median of {len(times)} runs, PyTorch CPU fp32"}
+
+
+def bench_neighbour(torch, args, with_cpu=True):
+    ops = importlib.import_module("learned-dynamics_amd.ops")
+    g = torch.Generator().manual_seed(0x947 + 2)
+    pos = (torch.rand(8, 16384, 3, generator=g) * 55).contiguous()
+    pos_d = pos.cuda()
+    box = (55., 55., 55.)
+
+    def step():
+        search = ops.NeighbourSearch(pos_d, 5.0, box)
+        return search.fill()     # includes the device->host copy of E, as get_edges does
+
+    src, _ = step()
+    E = int(src.numel())
+    sec = timed_steps(torch, step, args.steps, args.warmup)
+    alg_bytes = 12 * 8 * 16384 + 8 * E + 4 * 8
+    search = ops.NeighbourSearch(pos_d, 5.0, box)
+    t_fill = event_time(torch, lambda: search.fill(E), 10)
+    t_count = event_time(torch, lambda: ops.NeighbourSearch(pos_d, 5.0, box), 10)
+    out = {"metric": "neighbour search edges/sec", "value": E / sec, "unit": "edges/s", "ms_per_step": sec * 1e3,
+           "dtype": "f32+int32",
+           "config": {"workload": "BASELINE configs[1]: 8 boxes x 16384 atoms, box 55 A, cutoff 5 A", "edges": E},
+           "roofline": {"kernel": "whole search (bin, scan, place, order, pairs<count>, scan, pairs<fill>)",
+                        "bound": "hbm", "achieved": alg_bytes / sec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                        "frac": alg_bytes / sec / 1e9 / PEAK_HBM_GBS, "traffic": None},
+           "breakdown": {"count_phase_ms": t_count * 1e3, "fill_phase_ms": t_fill * 1e3}}
+    if with_cpu:
+        from oracle import neighbour as ON
+        one = pos[:1].numpy()
+        t0 = time.perf_counter()
+        ref = ON.edges(one, 5.0, box)
+        dt = time.perf_counter() - t0
+        out["cpu_baseline"] = {"value": len(ref["src"]) / dt, "unit": "edges/s", "cores": 1, "kind": "port",
+                               "sample": "1 of the 8 boxes, C cell list (oracle/neighbour_oracle.c), count+fill passes"}
+    return out
+
+
+def bench_products(torch, args):
+    ops = importlib.import_module("learned-dynamics_amd.ops")
+    out = {}
+    for rows in (4096, 262144):
+        g = torch.Generator().manual_seed(0x947 + 1)
+        x = torch.randn(rows, 64, generator=g).cuda()
+        v = torch.randn(rows, 64, 3, generator=g).cuda()
+        t = event_time(torch, lambda: ops.tensor_prods_avd(x, v, v), 50, warmup=5)
+        nbytes = rows * 64 * (4 + 12 + 4 + 12 + 36)
+        out[f"rows_{rows}"] = {"us": t * 1e6, "nodes_per_s": rows / t, "bytes": nbytes,
+                               "GB/s": nbytes / t / 1e9, "frac_of_hbm_peak": nbytes / t / 1e9 / PEAK_HBM_GBS}
+    return {"metric": "fused tensor-product trio (v.v, x v, v(x)v), BASELINE configs[0]", "unit": "nodes/s",
+            "value": out["rows_4096"]["nodes_per_s"], "detail": out,
+            "note": "includes allocation of the three outputs; 4096 rows (17.8 MB) is launch-latency bound"}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py: this build measures ONE GPU; independent boxes shard by batch with no communication, "
+              "so there is no multi-GPU figure to report (use --gpus 1).", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+
+    if args.workload == "painn_layer":
+        res = bench_painn_layer(torch, args)
+        if not args.no_extras:
+            small = argparse.Namespace(steps=10, warmup=3)
+            nb = bench_neighbour(torch, small, with_cpu=not args.no_cpu)
+            res["other_workloads"] = {"neighbour_search_configs[1]": nb, "tensor_products_configs[0]":
+                                      bench_products(torch, small)}
+    elif args.workload == "neighbour":
+        res = bench_neighbour(torch, args, with_cpu=not args.no_cpu)
+    else:
+        res = bench_products(torch, args)
+        res.setdefault("ms_per_step", res["detail"]["rows_4096"]["us"] * 1e-3)
+
+    line = {"metric": res.pop("metric"), "value": res.pop("value"), "unit": res.pop("unit"), "n_gpus": 1,
+            "steps": args.steps, "warmup": args.warmup, "ms_per_step": res.pop("ms_per_step"),
+            "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": res.pop("dtype", "f32"),
+            "data": "synthetic"}
+    line.update(res)
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -53,7 +53,7 @@ int mg_abi_version(void);
  *   count: bins atoms, walks the 3x3x3 cell window, writes the CSR row_ptr
  *          (batch*nodes+1, exclusive prefix), edge_counts (batch, inclusive
  *          prefix per box, as the reference's edgeCounts) and stats[4] =
- *          {E, max atoms in a cell, max degree, 0};
+ *          {E, max atoms in a cell, max degree, 1 if E overflowed int32};
  *   fill:  writes src[e] = b*nodes+i and dst[e] = b*nodes+j, rows ordered by
  *          (b,i); order inside a row is deterministic.
  * The reference's listmax / neighboursmax caps are not needed (exact-size CSR);
@@ -175,6 +175,25 @@ int mg_tensor_linear(int inds, const float* W, long w_stride_o, long w_stride_i,
 /* dW[o,i] = sum_{r,t} dy[r,o,t] x[r,i,t]  (tensor_ops_kern.cu:45-71), dW dense (dim_out,dim_in). */
 int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows, int dim_in, int dim_out,
                            float* dW, mg_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * PaiNN message passing (archs/meanflow_painn8.py:25-35,77-100).
+ * ---------------------------------------------------------------------- */
+/* radial_encode(r, n, rmax) (archs/meanflow_painn8.py:25-35): out (E,n) =
+ * [cos(k_m d)]_{m<hn} | [sin(k_m d)]_{m<n-hn}, k_m = (pi/rmax)(1 + m/2), hn = (n+1)/2, d = |r|. */
+int mg_painn_radial_encode(const float* r_ij /* (E,3) */, long n_edges, int n, float rmax,
+                           float* out /* (E,n) */, mg_stream_t stream);
+/* Message.forward after the two MLPs (archs/meanflow_painn8.py:91-100), fused over CSR rows:
+ *   P = filt[e] * actv[dst[e]];  u = r_ij[e] / sqrt(epsilon + |r_ij[e]|^2);  v = x_v[dst[e]]
+ *   out_v[i] = res_v[i] + sum_{e in row i} v*P[0:n] + (v x u)*P[n:2n] + u (x) P[2n:3n]
+ *   out_a[i] = res_a[i] + sum_{e in row i} P[3n:4n]
+ * filt (E,4n) is the radial MLP output per edge; actv (n_nodes,4n) is mlp_actv applied per
+ * NODE (a row-wise function commutes with the gather); res_a/res_v may be NULL. */
+int mg_painn_message(const int* row_ptr /* n_nodes+1 */, const int* dst /* E */, int n_nodes, long n_edges,
+                     const float* r_ij /* (E,3) */, const float* filt /* (E,4n) */,
+                     const float* actv /* (n_nodes,4n) */, const float* x_v /* (n_nodes,n,3) */,
+                     int n, float epsilon, const float* res_a, const float* res_v,
+                     float* out_a /* (n_nodes,n) */, float* out_v /* (n_nodes,n,3) */, mg_stream_t stream);
 
 #ifdef __cplusplus
 }

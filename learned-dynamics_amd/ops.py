@@ -454,3 +454,49 @@ def tensor_linear_wgrad(inds, dy, x):
         dW = torch.empty(dim_out, dim_in, dtype=torch.float32, device=x.device)
         L.check(_lib.mg_tensor_linear_wgrad(inds, _p(dy), _p(x), rows, dim_in, dim_out, _p(dW), _stream()))
     return dW
+
+
+# ----------------------------------------------------------------------- PaiNN
+def painn_radial_encode(r_ij, n, rmax):
+    """radial_encode of archs/meanflow_painn8.py:25-35: (E,3) -> (E,n)."""
+    _check_input(r_ij, "r_ij")
+    if r_ij.dim() != 2 or r_ij.size(1) != 3:
+        raise RuntimeError("r_ij must have shape (edges, 3)")
+    E = int(r_ij.size(0))
+    with torch.cuda.device(r_ij.device):
+        out = torch.empty(E, n, dtype=torch.float32, device=r_ij.device)
+        L.check(_lib.mg_painn_radial_encode(_p(r_ij), E, int(n), float(rmax), _p(out), _stream()))
+    return out
+
+
+def painn_message(row_ptr, dst, r_ij, filt, actv, x_v, epsilon, res_a=None, res_v=None):
+    """Fused gather-product-scatter of the PaiNN message (archs/meanflow_painn8.py:91-100).
+    filt (E,4n), actv (nodes,4n), x_v (nodes,n,3) -> out_a (nodes,n), out_v (nodes,n,3)."""
+    _check_input(row_ptr, "row_ptr", torch.int32)
+    _check_input(dst, "dst", torch.int32)
+    for t, nm in ((r_ij, "r_ij"), (filt, "filt"), (actv, "actv"), (x_v, "x_v")):
+        _check_input(t, nm)
+    n_nodes, n = int(x_v.size(0)), int(x_v.size(1))
+    E = int(dst.numel())
+    if tuple(x_v.shape) != (n_nodes, n, 3):
+        raise RuntimeError("x_v must have shape (nodes, n, 3)")
+    if tuple(actv.shape) != (n_nodes, 4 * n):
+        raise RuntimeError("actv must have shape (nodes, 4n)")
+    if tuple(filt.shape) != (E, 4 * n):
+        raise RuntimeError("filt must have shape (edges, 4n)")
+    if tuple(r_ij.shape) != (E, 3):
+        raise RuntimeError("r_ij must have shape (edges, 3)")
+    if row_ptr.numel() != n_nodes + 1:
+        raise RuntimeError("row_ptr must have nodes+1 entries")
+    for t, nm, shape in ((res_a, "res_a", (n_nodes, n)), (res_v, "res_v", (n_nodes, n, 3))):
+        if t is not None:
+            _check_input(t, nm)
+            if tuple(t.shape) != shape:
+                raise RuntimeError(f"{nm} has wrong shape")
+    dev = x_v.device
+    with torch.cuda.device(dev):
+        out_a = torch.empty(n_nodes, n, dtype=torch.float32, device=dev)
+        out_v = torch.empty(n_nodes, n, 3, dtype=torch.float32, device=dev)
+        L.check(_lib.mg_painn_message(_p(row_ptr), _p(dst), n_nodes, E, _p(r_ij), _p(filt), _p(actv), _p(x_v), n,
+                                      float(epsilon), _p(res_a), _p(res_v), _p(out_a), _p(out_v), _stream()))
+    return out_a, out_v

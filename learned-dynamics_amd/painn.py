@@ -1,0 +1,160 @@
+"""PaiNN message-passing blocks on the HIP kernels, mirroring the module names,
+constructor arguments and parameter names of archs/meanflow_painn8.py:25-125 of
+the reference (radial_encode, MLP, Message, Update, Block).
+
+Inference path.  Exact algebraic restructurings relative to the reference:
+  * mlp_actv is applied to the N node rows and gathered inside the edge kernel,
+    instead of being applied to the E gathered rows (a row-wise function
+    commutes with a gather);
+  * the gather of x_v, the cross product, the three scaled sums and both
+    segment sums run as ONE kernel over CSR rows; nothing of size E x n x 3 is
+    written to memory;
+  * the three TensLinear maps of Update that read x_v run as one GEMM with the
+    weights stacked.
+Message takes an optional n_rbf (number of radial functions); the default n
+reproduces the reference.
+"""
+import torch
+import torch.nn as nn
+
+from . import ops
+from .graph_layers import Graph, graph_setup
+from .tensor_products import TensLinear
+
+
+def radial_encode(r, n, rmax):
+    """r: (..., 3) -> (..., n)"""
+    lead = r.shape[:-1]
+    return ops.painn_radial_encode(r.reshape(-1, 3).contiguous(), n, rmax).reshape(*lead, n)
+
+
+def _linear(x, lin, act):
+    return ops.tensor_linear_fwd(0, lin.weight, x, bias=lin.bias, act=act)
+
+
+class MLP(nn.Module):
+    """Linear, SiLU, Linear, SiLU, Linear (archs/meanflow_painn8.py:38-51); bias and
+    activation are fused into the GEMM epilogue."""
+
+    def __init__(self, dim_in, dim_out):
+        super().__init__()
+        self.layers = nn.Sequential(
+            nn.Linear(dim_in, dim_out),
+            nn.SiLU(),
+            nn.Linear(dim_out, dim_out),
+            nn.SiLU(),
+            nn.Linear(dim_out, dim_out),
+        )
+
+    def forward(self, x_a):
+        lead = x_a.shape[:-1]
+        h = x_a.reshape(-1, x_a.shape[-1]).contiguous()
+        h = _linear(h, self.layers[0], ops.ACT_SILU)
+        h = _linear(h, self.layers[2], ops.ACT_SILU)
+        h = _linear(h, self.layers[4], ops.ACT_NONE)
+        return h.reshape(*lead, h.shape[-1])
+
+
+class ScalGroupNorm(nn.Module):
+    """Group norm over the nodes of a box and the channels of a group
+    (managan/layers_common.py:201-223)."""
+
+    def __init__(self, chan, groups, epsilon=1e-5):
+        super().__init__()
+        assert chan % groups == 0
+        self.chan, self.groups, self.epsilon = chan, groups, epsilon
+        self.gamma = nn.Parameter(torch.ones(chan))
+        self.beta = nn.Parameter(torch.zeros(chan))
+
+    def forward(self, x):
+        batch, nodes, chan = x.shape
+        x = x.reshape(batch, nodes, self.groups, -1)
+        mean = x.mean([1, 3], keepdim=True)
+        x_shift = x - mean
+        var = (x_shift ** 2).mean([1, 3], keepdim=True)
+        ans = x_shift / torch.sqrt(self.epsilon + var)
+        return self.beta + self.gamma * ans.reshape(batch, nodes, self.chan)
+
+
+class Update(nn.Module):
+    """archs/meanflow_painn8.py:53-75"""
+
+    def __init__(self, n):
+        super().__init__()
+        self.n = n
+        self.lin_l = TensLinear(1, n, n)
+        self.lin_r = TensLinear(1, n, n)
+        self.lin_v = TensLinear(1, n, n)
+        self.mlp = MLP(2 * n, 3 * n)
+        assert n % 4 == 0
+        self.gn = ScalGroupNorm(n, 4, epsilon=1.)
+
+    def forward(self, x_a, x_v):
+        n = self.n
+        W = torch.cat([self.lin_l.W, self.lin_r.W, self.lin_v.W], dim=0)        # (3n, n)
+        lrv = ops.tensor_linear_fwd(1, W, x_v.contiguous())                     # (B, N, 3n, 3)
+        x_v_l, x_v_r, x_v_v = lrv[..., :n, :], lrv[..., n:2 * n, :], lrv[..., 2 * n:, :]
+        inner_prod = (x_v_l * x_v_r).sum(-1)
+        y = self.mlp(torch.cat([x_a, torch.linalg.vector_norm(x_v_r, dim=-1)], dim=-1))
+        x_v = x_v_v * y[..., :n, None]
+        inner_prod = self.gn(inner_prod * y[..., n:2 * n])
+        x_a = inner_prod + y[..., 2 * n:]
+        x_v = x_v / torch.sqrt(1. + (x_v ** 2).sum(-1, keepdim=True))
+        return x_a, x_v
+
+
+class Message(nn.Module):
+    """archs/meanflow_painn8.py:77-100"""
+
+    def __init__(self, r0: float, n: int, n_rbf: int = None):
+        super().__init__()
+        self.r0 = r0
+        self.n = n
+        self.n_rbf = n if n_rbf is None else n_rbf
+        self.epsilon = 0.1
+        self.mlp_dist = MLP(self.n_rbf, 4 * n)
+        self.mlp_actv = MLP(n, 4 * n)
+
+    def filters(self, r_ij):
+        """(edges, 3) -> (edges, 4n): the per-edge filter, the one large per-edge tensor."""
+        return self.mlp_dist(ops.painn_radial_encode(r_ij, self.n_rbf, self.r0))
+
+    def forward(self, graph: Graph, x_a, x_v, r_ij, residual=False):
+        """x_a: (batch, atoms, n), x_v: (batch, atoms, n, 3), r_ij: (edges, 3).
+        Returns (dx_a, dx_v), or (x_a + dx_a, x_v + dx_v) with residual=True."""
+        B, N, n = x_a.shape
+        flat_a = x_a.reshape(B * N, n).contiguous()
+        flat_v = x_v.reshape(B * N, n, 3).contiguous()
+        filt = self.filters(r_ij.contiguous())
+        actv = self.mlp_actv(flat_a)
+        out_a, out_v = ops.painn_message(graph.row_ptr, graph.dst32, r_ij.contiguous(), filt, actv, flat_v,
+                                         self.epsilon, flat_a if residual else None, flat_v if residual else None)
+        return out_a.reshape(B, N, n), out_v.reshape(B, N, n, 3)
+
+
+class Block(nn.Module):
+    """archs/meanflow_painn8.py:102-125.  graph_bond may be None (no bond-graph message)."""
+
+    def __init__(self, r0: float, n: int, pos_mutable: bool = False, n_rbf: int = None):
+        super().__init__()
+        self.pos_mutable = pos_mutable
+        self.r0 = r0
+        self.message = Message(r0, n, n_rbf)
+        self.message_bond = Message(r0, n, n_rbf)
+        self.update = Update(n)
+        if self.pos_mutable:
+            self.lin_push_pos = TensLinear(1, n, 1)
+
+    def forward(self, tup):
+        pos, graph, r_ij, graph_bond, r_ij_bond, x_a, x_v, box = tup
+        if graph is None:
+            graph, r_ij = graph_setup(self.r0, box, pos)
+        if graph_bond is not None:
+            x_a, x_v = self.message_bond(graph_bond, x_a, x_v, r_ij_bond, residual=True)
+        x_a, x_v = self.message(graph, x_a, x_v, r_ij, residual=True)
+        dx_a, dx_v = self.update(x_a, x_v)
+        x_a, x_v = x_a + dx_a, x_v + dx_v
+        if self.pos_mutable:
+            pos = pos + self.lin_push_pos(x_v).squeeze(-2)
+            graph, r_ij = None, None
+        return pos, graph, r_ij, graph_bond, r_ij_bond, x_a, x_v, box
