@@ -41,6 +41,12 @@ inline Chunks make_chunks(int units, int unit_width) {
 }
 
 __device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+// streamed-once data: keep it from displacing the gathered node rows in L2
+typedef float float4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ float4 ld4_stream(const float* p) {
+    const float4v t = __builtin_nontemporal_load(reinterpret_cast<const float4v*>(p));
+    return make_float4(t.x, t.y, t.z, t.w);
+}
 __device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
 __device__ __forceinline__ float4 mul4(float4 a, float4 b) { return make_float4(a.x * b.x, a.y * b.y, a.z * b.z, a.w * b.w); }
 
@@ -55,40 +61,56 @@ struct EdgeAcc {
     }
 };
 
-// accumulate one edge for 4 consecutive channels starting at c
-__device__ __forceinline__ void edge_term(EdgeAcc& acc, const float* __restrict__ filt_row,
-                                          const float* __restrict__ actv_row, const float* __restrict__ xv_row,
-                                          int n, int c, float ux, float uy, float uz) {
-    const float4 p0 = mul4(ld4(filt_row + c), ld4(actv_row + c));
-    const float4 p1 = mul4(ld4(filt_row + n + c), ld4(actv_row + n + c));
-    const float4 p2 = mul4(ld4(filt_row + 2 * n + c), ld4(actv_row + 2 * n + c));
-    const float4 p3 = mul4(ld4(filt_row + 3 * n + c), ld4(actv_row + 3 * n + c));
-    const float4 va = ld4(xv_row + 3 * c), vb = ld4(xv_row + 3 * c + 4), vc = ld4(xv_row + 3 * c + 8);
-    const float vv[12] = {va.x, va.y, va.z, va.w, vb.x, vb.y, vb.z, vb.w, vc.x, vc.y, vc.z, vc.w};
-    const float q0[4] = {p0.x, p0.y, p0.z, p0.w}, q1[4] = {p1.x, p1.y, p1.z, p1.w};
-    const float q2[4] = {p2.x, p2.y, p2.z, p2.w}, q3[4] = {p3.x, p3.y, p3.z, p3.w};
+// operands of one edge for 4 consecutive channels starting at c
+struct EdgeLoads {
+    float4 f[4], a[4], v[3];
+    __device__ __forceinline__ void load(const float* __restrict__ filt_row, const float* __restrict__ actv_row,
+                                         const float* __restrict__ xv_row, int n, int c) {
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
-        const float x = vv[3 * k], y = vv[3 * k + 1], z = vv[3 * k + 2];
-        const float cx = y * uz - z * uy, cy = z * ux - x * uz, cz = x * uy - y * ux;   // v x u
-        acc.v[3 * k + 0] += x * q0[k] + cx * q1[k] + ux * q2[k];
-        acc.v[3 * k + 1] += y * q0[k] + cy * q1[k] + uy * q2[k];
-        acc.v[3 * k + 2] += z * q0[k] + cz * q1[k] + uz * q2[k];
-        acc.a[k] += q3[k];
+        for (int k = 0; k < 4; k++) {
+            f[k] = ld4_stream(filt_row + k * n + c);
+            a[k] = ld4(actv_row + k * n + c);
+        }
+#pragma unroll
+        for (int k = 0; k < 3; k++) v[k] = ld4(xv_row + 3 * c + 4 * k);
     }
-}
+    __device__ __forceinline__ void accumulate(EdgeAcc& acc, float ux, float uy, float uz) const {
+        const float4 p0 = mul4(f[0], a[0]), p1 = mul4(f[1], a[1]), p2 = mul4(f[2], a[2]), p3 = mul4(f[3], a[3]);
+        const float vv[12] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w,
+                              v[2].x, v[2].y, v[2].z, v[2].w};
+        const float q0[4] = {p0.x, p0.y, p0.z, p0.w}, q1[4] = {p1.x, p1.y, p1.z, p1.w};
+        const float q2[4] = {p2.x, p2.y, p2.z, p2.w}, q3[4] = {p3.x, p3.y, p3.z, p3.w};
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const float x = vv[3 * k], y = vv[3 * k + 1], z = vv[3 * k + 2];
+            const float cx = y * uz - z * uy, cy = z * ux - x * uz, cz = x * uy - y * ux;   // v x u
+            acc.v[3 * k + 0] += x * q0[k] + cx * q1[k] + ux * q2[k];
+            acc.v[3 * k + 1] += y * q0[k] + cy * q1[k] + uy * q2[k];
+            acc.v[3 * k + 2] += z * q0[k] + cz * q1[k] + uz * q2[k];
+            acc.a[k] += q3[k];
+        }
+    }
+};
 
-__global__ void __launch_bounds__(256) painn_message_kernel(
+// register budget of 5 waves per SIMD (102 VGPRs): room to keep a whole step's loads in flight
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 5))) painn_message_kernel(
     const int* __restrict__ row_ptr, const int* __restrict__ dst, long n_nodes, const float* __restrict__ r_ij,
     const float* __restrict__ filt, const float* __restrict__ actv, const float* __restrict__ x_v, int n,
     float epsilon, const float* __restrict__ res_a, const float* __restrict__ res_v, float* __restrict__ out_a,
     float* __restrict__ out_v, Chunks ch) {
     const int lane = threadIdx.x & (kWave - 1);
-    const long wave_global = ((long)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
-    const long n_waves = ((long)gridDim.x * blockDim.x) / kWave;
+    // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  Give every XCD
+    // one contiguous range of nodes: neighbouring nodes share most of their neighbours, so the
+    // gathers of actv / x_v rows are then served by that XCD's L2 instead of the fabric.
     const long items = n_nodes * ch.n;
+    const long per_xcd = (items + 7) / 8;
+    const int xcd = blockIdx.x & 7;
+    const long waves_per_xcd = (long)(gridDim.x >> 3) * (blockDim.x / kWave);
+    const long wave_local = (long)(blockIdx.x >> 3) * (blockDim.x / kWave) + threadIdx.x / kWave;
     const long row_f = 4L * n;
-    for (long item = wave_global; item < items; item += n_waves) {
+    for (long item_local = wave_local; item_local < per_xcd; item_local += waves_per_xcd) {
+        const long item = xcd * per_xcd + item_local;
+        if (item >= items) break;
         const long node = item / ch.n;
         const int ci = (int)(item - node * ch.n);
         const int L = ch.lanes[ci];
@@ -97,11 +119,22 @@ __global__ void __launch_bounds__(256) painn_message_kernel(
         const long lo = row_ptr[node], hi = row_ptr[node + 1];
         EdgeAcc acc;
         acc.zero();
-        for (long e = lo + sub; e < hi; e += per_iter) {
-            const long j = dst[e];
-            const float rx = r_ij[3 * e], ry = r_ij[3 * e + 1], rz = r_ij[3 * e + 2];
+        // The edge header (dst, r_ij) of the next step is fetched one step ahead of its use, so
+        // the eleven 16-byte operand loads of a step can all be issued at once.
+        long e = lo + sub;
+        long j = 0;
+        float rx = 0.f, ry = 0.f, rz = 0.f;
+        if (e < hi) { j = dst[e]; rx = r_ij[3 * e]; ry = r_ij[3 * e + 1]; rz = r_ij[3 * e + 2]; }
+        while (e < hi) {
+            EdgeLoads ld;
+            ld.load(filt + e * row_f, actv + j * row_f, x_v + j * 3L * n, n, c);
+            const long e_next = e + per_iter;
+            long j_next = 0;
+            float nx = 0.f, ny = 0.f, nz = 0.f;
+            if (e_next < hi) { j_next = dst[e_next]; nx = r_ij[3 * e_next]; ny = r_ij[3 * e_next + 1]; nz = r_ij[3 * e_next + 2]; }
             const float inv = 1.0f / sqrtf(epsilon + (rx * rx + ry * ry + rz * rz));
-            edge_term(acc, filt + e * row_f, actv + j * row_f, x_v + j * 3L * n, n, c, rx * inv, ry * inv, rz * inv);
+            ld.accumulate(acc, rx * inv, ry * inv, rz * inv);
+            e = e_next; j = j_next; rx = nx; ry = ny; rz = nz;
         }
         for (int d = L; d < kWave; d <<= 1) {
 #pragma unroll
@@ -226,7 +259,8 @@ int mg_painn_message(const int* row_ptr, const int* dst, int n_nodes, long n_edg
         for (int k = 0; k < ch.n; k++) covered += ch.lanes[k] * 4;
         if (covered == n) {
             long blocks = ceil_div((long)n_nodes * ch.n, 4);
-            if (blocks > 256L * 64) blocks = 256L * 64;
+            if (blocks > 256L * 32) blocks = 256L * 32;
+            blocks = ceil_div(blocks, 8) * 8;   // the XCD-aware item order needs a multiple of 8
             hipLaunchKernelGGL(painn_message_kernel, dim3((unsigned)blocks), dim3(256), 0, st, row_ptr, dst,
                                (long)n_nodes, r_ij, filt, actv, x_v, n, epsilon, res_a, res_v, out_a, out_v, ch);
             return check_launch("mg_painn_message");

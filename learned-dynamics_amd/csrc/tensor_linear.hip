@@ -205,6 +205,167 @@ int launch_cfg(const float* W, long so, long si, const float* X, long R, int I, 
     return check_launch("mg_tensor_linear");
 }
 
+
+// ---------------------------------------------------------------------------
+// T == 1 (plain rows x dim_in @ W^T): the MLP GEMMs that dominate a PaiNN layer.
+// 128x128 output tile, 4 waves (2x2, 64x64 each), BK = 32.
+//  * K order is permuted inside a slab: lanes 0-31 own k = 0..15 and lanes 32-63
+//    own k = 16..31 of the slab for BOTH operands, so MFMA step s multiplies
+//    A[m][16h+s] B[16h+s][n] (h = lane/32) and every lane fetches its 16 k values
+//    with four ds_read_b128 instead of 16 ds_read_b32.  Any pairing of k values
+//    into steps is a valid reordering of the K sum.
+//  * LDS rows are padded to 36 floats (9 quads, odd) so that b128 reads of 8
+//    consecutive rows and b128 writes of one row hit 32 distinct banks.
+//  * HBM side: a row of a slab is 128 B = one cache line, read by 8 lanes.
+//  * Workgroup ids are remapped so that the N-tiles of one M-tile run back to
+//    back on the SAME XCD (ids are dealt round-robin to the 8 XCDs, each with its
+//    own L2): x is then fetched from HBM once and re-read from that L2.
+constexpr int kBK1 = 32;
+constexpr int kRS1 = kBK1 + 4;
+
+template <bool WVEC>
+__global__ void __launch_bounds__(256)
+linear_rows_kernel(const float* __restrict__ W, long so, long si, const float* __restrict__ X, long R, int I, int O,
+                   const float* __restrict__ bias, int act, int accumulate, float* __restrict__ Y, int tiles_n,
+                   long tiles_total) {
+    __shared__ __attribute__((aligned(16))) float xs[128 * kRS1];
+    __shared__ __attribute__((aligned(16))) float ws[128 * kRS1];
+
+    // XCD-aware tile order
+    const long bid = blockIdx.x;
+    const long per_xcd = (tiles_total + 7) / 8;
+    const long logical = (bid % 8) * per_xcd + bid / 8;
+    if (logical >= tiles_total) return;
+    const long tile_m = logical / tiles_n;
+    const int tile_n = (int)(logical - tile_m * tiles_n);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+    const long r0 = tile_m * 128;
+    const int n0 = tile_n * 128;
+    const int khalf = lane >> 5;
+
+    float16v acc[2][2];
+#pragma unroll
+    for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+        for (int ni = 0; ni < 2; ni++)
+#pragma unroll
+            for (int q = 0; q < 16; q++) acc[mi][ni][q] = 0.f;
+
+    float4 xv[4], wv[4];
+    const int ld_r = tid >> 3, ld_c = (tid & 7) * 4;   // + 32 rows per j
+
+    auto load_tile = [&](int k0) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int r = ld_r + 32 * j;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (r0 + r < R) v = *reinterpret_cast<const float4*>(X + (r0 + r) * I + k0 + ld_c);
+            xv[j] = v;
+            float4 w = make_float4(0.f, 0.f, 0.f, 0.f);
+            const int n = n0 + r;
+            if (n < O) {
+                if constexpr (WVEC) {
+                    w = *reinterpret_cast<const float4*>(W + (long)n * so + k0 + ld_c);
+                } else {
+                    const float* wp = W + (long)n * so + (long)(k0 + ld_c) * si;
+                    w = make_float4(wp[0], wp[si], wp[2 * si], wp[3 * si]);
+                }
+            }
+            wv[j] = w;
+        }
+    };
+    auto store_tile = [&]() {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const int r = ld_r + 32 * j;
+            *reinterpret_cast<float4*>(xs + r * kRS1 + ld_c) = xv[j];
+            *reinterpret_cast<float4*>(ws + r * kRS1 + ld_c) = wv[j];
+        }
+    };
+
+    const float* a_ptr[2];
+    const float* b_ptr[2];
+#pragma unroll
+    for (int i = 0; i < 2; i++) {
+        a_ptr[i] = xs + ((wave_m * 2 + i) * 32 + (lane & 31)) * kRS1 + khalf * 16;
+        b_ptr[i] = ws + ((wave_n * 2 + i) * 32 + (lane & 31)) * kRS1 + khalf * 16;
+    }
+
+    load_tile(0);
+    for (int k0 = 0; k0 < I; k0 += kBK1) {
+        __syncthreads();
+        store_tile();
+        __syncthreads();
+        if (k0 + kBK1 < I) load_tile(k0 + kBK1);
+#pragma unroll
+        for (int half = 0; half < 2; half++) {
+            float4 a[2][2], b[2][2];
+#pragma unroll
+            for (int i = 0; i < 2; i++) {
+                a[i][0] = *reinterpret_cast<const float4*>(a_ptr[i] + half * 8);
+                a[i][1] = *reinterpret_cast<const float4*>(a_ptr[i] + half * 8 + 4);
+                b[i][0] = *reinterpret_cast<const float4*>(b_ptr[i] + half * 8);
+                b[i][1] = *reinterpret_cast<const float4*>(b_ptr[i] + half * 8 + 4);
+            }
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                float av[2], bv[2];
+#pragma unroll
+                for (int i = 0; i < 2; i++) {
+                    const float4 aa = a[i][s >> 2], bb = b[i][s >> 2];
+                    av[i] = (s & 3) == 0 ? aa.x : (s & 3) == 1 ? aa.y : (s & 3) == 2 ? aa.z : aa.w;
+                    bv[i] = (s & 3) == 0 ? bb.x : (s & 3) == 1 ? bb.y : (s & 3) == 2 ? bb.z : bb.w;
+                }
+#pragma unroll
+                for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+                    for (int ni = 0; ni < 2; ni++)
+                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x2f32(av[mi], bv[ni], acc[mi][ni], 0, 0, 0);
+            }
+        }
+    }
+
+#pragma unroll
+    for (int ni = 0; ni < 2; ni++) {
+        const int n = n0 + (wave_n * 2 + ni) * 32 + (lane & 31);
+        if (n >= O) continue;
+        const float bv = bias ? bias[n] : 0.f;
+#pragma unroll
+        for (int mi = 0; mi < 2; mi++) {
+#pragma unroll
+            for (int q = 0; q < 16; q++) {
+                const long r = r0 + (wave_m * 2 + mi) * 32 + 8 * (q / 4) + 4 * khalf + (q % 4);
+                if (r < R) {
+                    const long addr = r * O + n;
+                    float v = activate(acc[mi][ni][q] + bv, act);
+                    if (accumulate) v += Y[addr];
+                    Y[addr] = v;
+                }
+            }
+        }
+    }
+}
+
+int launch_rows(const float* W, long so, long si, const float* X, long R, int I, int O, const float* bias, int act,
+                int accumulate, float* Y, hipStream_t st) {
+    const long tiles_m = ceil_div(R, 128);
+    const int tiles_n = (int)ceil_div(O, 128);
+    const long total = tiles_m * tiles_n;
+    const long grid = ceil_div(total, 8) * 8;
+    MG_REQUIRE(grid <= 0x7fffffffL, "mg_tensor_linear: grid too large (rows=%ld dim_out=%d)", R, O);
+    const bool wvec = si == 1 && so % 4 == 0 && aligned16(W);
+    if (wvec)
+        hipLaunchKernelGGL(linear_rows_kernel<true>, dim3((unsigned)grid), dim3(256), 0, st, W, so, si, X, R, I, O, bias,
+                           act, accumulate, Y, tiles_n, total);
+    else
+        hipLaunchKernelGGL(linear_rows_kernel<false>, dim3((unsigned)grid), dim3(256), 0, st, W, so, si, X, R, I, O,
+                           bias, act, accumulate, Y, tiles_n, total);
+    return check_launch("mg_tensor_linear");
+}
+
 }  // namespace
 }  // namespace mg
 
@@ -226,6 +387,9 @@ int mg_tensor_linear(int inds, const float* W, long w_stride_o, long w_stride_i,
     const float* b = bias;
     switch (inds) {
         case 0:
+            // wide layers with 16-byte aligned rows of whole 32-wide k slabs take the tuned kernel
+            if (dim_out > 64 && dim_in % kBK1 == 0 && aligned16(x))
+                return launch_rows(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
             if (dim_out <= 32) return launch_cfg<1, 4, 1, 2, 1>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
             if (dim_out <= 64) return launch_cfg<1, 2, 2, 2, 1>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
             return launch_cfg<1, 2, 2, 2, 2>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
