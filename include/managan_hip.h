@@ -172,6 +172,14 @@ int mg_tensor_prods_avd(const float* a, const float* v_l, const float* v_r, long
 int mg_tensor_linear(int inds, const float* W, long w_stride_o, long w_stride_i,
                      const float* x, long rows, int dim_in, int dim_out,
                      const float* bias, int act, int accumulate, float* y, mg_stream_t stream);
+/* The same contraction with explicit memory layouts of x and y:
+ *   0 = (row, chan, comp), how the reference stores every tensor;
+ *   1 = (row, comp, chan), component-major: what the fused edge kernels gather from and
+ *       accumulate into, so that a wave's accesses are unit-stride. */
+int mg_tensor_linear_layout(int inds, const float* W, long w_stride_o, long w_stride_i,
+                            const float* x, long rows, int dim_in, int dim_out,
+                            const float* bias, int act, int accumulate,
+                            int x_layout, int y_layout, float* y, mg_stream_t stream);
 /* dW[o,i] = sum_{r,t} dy[r,o,t] x[r,i,t]  (tensor_ops_kern.cu:45-71), dW dense (dim_out,dim_in). */
 int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows, int dim_in, int dim_out,
                            float* dW, mg_stream_t stream);
@@ -194,6 +202,27 @@ int mg_painn_message(const int* row_ptr /* n_nodes+1 */, const int* dst /* E */,
                      const float* actv /* (n_nodes,4n) */, const float* x_v /* (n_nodes,n,3) */,
                      int n, float epsilon, const float* res_a, const float* res_v,
                      float* out_a /* (n_nodes,n) */, float* out_v /* (n_nodes,n,3) */, mg_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Rank-0/1/2 message passing with the 13 products (archs/diffuser_atoms15.py:227-253).
+ * ---------------------------------------------------------------------- */
+/* Per-edge geometry of Messages.forward (archs/diffuser_atoms15.py:239-240):
+ * enc (E,8) = radial_encode_8(r_ij, r0) (managan/jacobi_radenc.py:24-37), evaluated in fp64 and
+ * rounded to fp32; rhat (E,3) = tens_sigmoid(1, r_ij * 7 / r0) (managan/tensor_products.py:167-182). */
+int mg_bee_edge_geometry(const float* r_ij /* (E,3) */, long n_edges, float r0,
+                         float* enc /* (E,8) */, float* rhat /* (E,3) */, mg_stream_t stream);
+/* Messages.forward lines 241-247 and the edge sums of lines 250-252, fused over CSR rows.
+ * phi_a[e,c] = enc_b[c] + sum_m enc_W[c,m] enc[e,m]; phi_v, phi_d as in the reference;
+ * left operands La (N,chan), Lv (N,3,chan), Ld (N,9,chan) are L_k x_k in component-major layout.
+ *   P0 (E,3,chan)    = [y_000 | y_110 | y_220] per edge
+ *   S1 (N,3,5,chan)  = sum over the edges of each node of [y_011, y_101, y_121, y_211, y_111]
+ *   S2 (N,9,5,chan)  = ... of [y_022, y_202, y_112, y_222, y_212]
+ * node_order (N ints, or NULL) is the order in which rows are processed (e.g. cell order, for
+ * cache locality of the gathers); results do not depend on it. */
+int mg_bee_message(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
+                   const float* rhat, const float* enc, const float* La, const float* Lv, const float* Ld,
+                   int chan, const float* enc_W /* (chan,8) */, const float* enc_b /* (chan) */,
+                   float* P0, float* S1, float* S2, mg_stream_t stream);
 
 #ifdef __cplusplus
 }

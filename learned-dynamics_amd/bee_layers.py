@@ -1,0 +1,168 @@
+"""Rank-0/1/2 ("a/v/d") blocks built on the 13 Cartesian products, mirroring the
+module names, constructor arguments and parameter names of
+archs/diffuser_atoms15.py:29-110,227-253 of the reference (add_tens_prod_submodules,
+SelfTensProds, MLP, Messages) and TensGroupNorm of managan/tensor_products.py:215-232.
+
+Inference path.  Exact algebraic restructurings relative to the reference
+(they change only the order of fp32 additions):
+  * the ten bias-free output linears Y_lab of the vector and rank-2 products are
+    applied AFTER the sum over edges, on N rows instead of E rows, and the five
+    that feed one output run as one GEMM (weights concatenated along K);
+  * phi_a = lin_enc(radial_encode_8(r)) (K = 8) is recomputed inside the edge
+    kernel from the 8 encoded values; phi_v, phi_d, the gathered node features
+    and the 13 per-edge products are never written to memory, except the three
+    scalar products that feed the per-edge MLP;
+  * 0.1 * sum is applied once per node;  x + lin_direct(x) uses W_direct + I.
+radial_encode_8 is evaluated in fp64 (the reference's fp32 monomial evaluation is
+ill-conditioned: alternating coefficients up to ~1e5).
+"""
+import torch
+import torch.nn as nn
+
+from . import ops
+from .codegen_tensor_products import Bee
+from .graph_layers import Graph
+from .tensor_products import TensLinear
+
+LABELS_0 = ("000", "110", "220")
+LABELS_1 = ("011", "101", "121", "211", "111")
+LABELS_2 = ("022", "202", "112", "222", "212")
+
+
+def add_tens_prod_submodules(self, dim_a, dim_v, dim_d, chan):
+    for lab in ops.BEE_ORDER:
+        rank = int(lab[2])
+        setattr(self, f"Y_{lab}", TensLinear(rank, chan, (dim_a, dim_v, dim_d)[rank]))
+
+
+def apply_tens_prod_submodules(self, prods):
+    """prods: the 13 products in Bee order -> (y_0, y_1, y_2); one accumulating GEMM per product."""
+    outs = [None, None, None]
+    for lab, p in zip(ops.BEE_ORDER, prods):
+        rank = int(lab[2])
+        W = getattr(self, f"Y_{lab}").W
+        if outs[rank] is None:
+            outs[rank] = ops.tensor_linear_fwd(rank, W, p)
+        else:
+            ops.tensor_linear_fwd(rank, W, p, out=outs[rank], accumulate=True)
+    return tuple(outs)
+
+
+class TensGroupNorm(nn.Module):
+    """managan/tensor_products.py:215-232: x / sqrt(eps + mean over (nodes, group channels) of |x|^2), times gamma."""
+
+    def __init__(self, inds, chan, groups, epsilon=1e-5):
+        super().__init__()
+        assert chan % groups == 0
+        self.inds, self.chan, self.groups, self.epsilon = inds, chan, groups, epsilon
+        self.gamma = nn.Parameter(torch.ones(chan, *[1] * inds))
+
+    def forward(self, x):
+        batch, nodes = x.shape[:2]
+        xg = x.reshape(batch, nodes, self.groups, -1, 3 ** self.inds)
+        moment2 = (xg ** 2).sum(-1, keepdim=True).mean([1, 3], keepdim=True)
+        ans = xg / torch.sqrt(self.epsilon + moment2)
+        return self.gamma * ans.reshape(batch, nodes, self.chan, *[3] * self.inds)
+
+
+class SelfTensProds(nn.Module):
+    """archs/diffuser_atoms15.py:59-95"""
+
+    def __init__(self, dim_a, dim_v, dim_d, chan, groups=8):
+        super().__init__()
+        self.L0 = TensLinear(0, dim_a, chan)
+        self.R0 = TensLinear(0, dim_a, chan)
+        self.L1 = TensLinear(1, dim_v, chan)
+        self.R1 = TensLinear(1, dim_v, chan)
+        self.L2 = TensLinear(2, dim_d, chan)
+        self.R2 = TensLinear(2, dim_d, chan)
+        add_tens_prod_submodules(self, dim_a, dim_v, dim_d, chan)
+        self.gn_a = TensGroupNorm(0, dim_a, groups)
+        self.gn_v = TensGroupNorm(1, dim_v, groups)
+        self.gn_d = TensGroupNorm(2, dim_d, groups)
+
+    def forward(self, x_a, x_v, x_d):
+        *rest, dim_a = x_a.shape
+        dim_v, dim_d = x_v.shape[-2], x_d.shape[-3]
+        rows = 1
+        for d in rest:
+            rows *= d
+        x_a = x_a.reshape(rows, dim_a).contiguous()
+        x_v = x_v.reshape(rows, dim_v, 3).contiguous()
+        x_d = x_d.reshape(rows, dim_d, 3, 3).contiguous()
+        prods = Bee.apply(self.L0(x_a), self.L1(x_v), self.L2(x_d), self.R0(x_a), self.R1(x_v), self.R2(x_d))
+        y_a, y_v, y_d = apply_tens_prod_submodules(self, prods)
+        y_a = y_a.reshape(*rest, dim_a)
+        y_v = y_v.reshape(*rest, dim_v, 3)
+        y_d = y_d.reshape(*rest, dim_d, 3, 3)
+        return self.gn_a(y_a), self.gn_v(y_v), self.gn_d(y_d)
+
+
+class MLP(nn.Module):
+    """lin_direct(x) + [Linear(d,2d), LeakyReLU(.1), Linear(2d,2d), LeakyReLU(.1), Linear(2d,d)](x)
+    (archs/diffuser_atoms15.py:98-110)"""
+
+    def __init__(self, dim_a):
+        super().__init__()
+        self.lin_direct = nn.Linear(dim_a, dim_a, bias=False)
+        self.layers = nn.Sequential(
+            nn.Linear(dim_a, 2 * dim_a),
+            nn.LeakyReLU(0.1),
+            nn.Linear(2 * dim_a, 2 * dim_a),
+            nn.LeakyReLU(0.1),
+            nn.Linear(2 * dim_a, dim_a),
+        )
+
+    def forward(self, x, plus_identity=False):
+        """Returns mlp(x), or x + mlp(x) with plus_identity=True."""
+        lead = x.shape[:-1]
+        x2 = x.reshape(-1, x.shape[-1]).contiguous()
+        Wd = self.lin_direct.weight
+        if plus_identity:
+            Wd = Wd + torch.eye(Wd.shape[0], device=Wd.device, dtype=Wd.dtype)
+        out = ops.tensor_linear_fwd(0, Wd, x2)
+        L = self.layers
+        h = ops.tensor_linear_fwd(0, L[0].weight, x2, bias=L[0].bias, act=ops.ACT_LEAKY)
+        h = ops.tensor_linear_fwd(0, L[2].weight, h, bias=L[2].bias, act=ops.ACT_LEAKY)
+        ops.tensor_linear_fwd(0, L[4].weight, h, bias=L[4].bias, out=out, accumulate=True)
+        return out.reshape(*lead, out.shape[-1])
+
+
+class Messages(nn.Module):
+    """archs/diffuser_atoms15.py:227-253"""
+
+    def __init__(self, r0: float, dim_a: int, dim_v: int, dim_d: int, chan: int):
+        super().__init__()
+        self.r0 = r0
+        self.L0 = TensLinear(0, dim_a, chan)
+        self.L1 = TensLinear(1, dim_v, chan)
+        self.L2 = TensLinear(2, dim_d, chan)
+        add_tens_prod_submodules(self, dim_a, dim_v, dim_d, chan)
+        self.lin_enc = nn.Linear(8, chan)
+        self.mlp_a = MLP(dim_a)
+
+    def _cat_Y(self, labels, scale=None):
+        W = torch.cat([getattr(self, f"Y_{lab}").W for lab in labels], dim=1)
+        return W if scale is None else W * scale
+
+    def forward(self, graph: Graph, r_ij, x_a, x_v, x_d, node_order=None):
+        """x_a (batch, nodes, dim_a), x_v (..., dim_v, 3), x_d (..., dim_d, 3, 3), r_ij (edges, 3).
+        Returns 0.1 * sum over edges of the messages: (B_a, B_v, B_d) with the input shapes."""
+        B, N = x_a.shape[:2]
+        rows = B * N
+        C = ops.LAYOUT_COMP_CHAN
+        La = ops.tensor_linear_fwd(0, self.L0.W, x_a.reshape(rows, -1).contiguous())
+        Lv = ops.tensor_linear_fwd(1, self.L1.W, x_v.reshape(rows, -1, 3).contiguous(), y_layout=C)
+        Ld = ops.tensor_linear_fwd(2, self.L2.W, x_d.reshape(rows, -1, 3, 3).contiguous(), y_layout=C)
+        enc, rhat = ops.bee_edge_geometry(r_ij.contiguous(), self.r0)
+        P0, S1, S2 = ops.bee_message(graph.row_ptr, graph.dst32, rhat, enc, La, Lv, Ld, self.lin_enc.weight,
+                                     self.lin_enc.bias, node_order=node_order)
+        E, chan = P0.shape[0], P0.shape[2]
+        # scalar channel: per-edge linear + MLP, then the edge sum
+        psi_a = ops.tensor_linear_fwd(0, self._cat_Y(LABELS_0), P0.reshape(E, 3 * chan))
+        psi_a = self.mlp_a(psi_a, plus_identity=True)
+        B_a = ops.segment_sum_csr(psi_a, graph.row_ptr, rows).mul_(0.1)
+        # vector and rank-2 channels: output linears after the edge sum, on node rows
+        B_v = ops.tensor_linear_fwd(1, self._cat_Y(LABELS_1, 0.1), S1.reshape(rows, 3, 5 * chan), x_layout=C)
+        B_d = ops.tensor_linear_fwd(2, self._cat_Y(LABELS_2, 0.1), S2.reshape(rows, 9, 5 * chan), x_layout=C)
+        return (B_a.reshape(B, N, -1), B_v.reshape(B, N, -1, 3), B_d.reshape(B, N, -1, 3, 3))

@@ -1,0 +1,235 @@
+// Rank-0/1/2 ("a/v/d") message passing with the 13 Cartesian products, fused
+// over CSR rows.
+//
+// For edge e = (i <- j): phi_a = lin_enc(radial_encode_8(r_ij)) (chan),
+// rh = s / sqrt(1 + |s|^2) with s = r_ij * 7 / r0, phi_v = phi_a (x) rh,
+// phi_d = phi_a (x) rh (x) rh; left operands are the node features
+// l_k = (L_k x_k)[j]; the 13 products p_lab = prod_lab(l, phi) follow.
+// Because every right operand is phi_a[c] times a per-edge geometric factor, each
+// product is phi_a[c] * g_lab(l[c], rh): nothing of size E x chan x 3 x 3 exists.
+//
+// What leaves the kernel:
+//   P0 (E, 3, chan)      the three scalar products per edge (they feed a per-edge
+//                        MLP, which does not commute with the sum over edges)
+//   S1 (N, 3, 5, chan)   sum over the edges of node i of the five vector products
+//   S2 (N, 9, 5, chan)   ... of the five rank-2 products
+// The bias-free output linears Y_lab commute with the sum over edges, so they are
+// applied to S1/S2 on N rows afterwards; the (comp, label, chan) order makes
+// each of those one plain GEMM with K = 5*chan.
+//
+// Node features are read in component-major layout (node, comp, chan): the 13
+// gathers of a wave are 13 unit-stride 256-byte reads.  A lane owns one channel
+// and keeps its 60 running sums in registers; rows are summed in edge order.
+#include "common.hpp"
+
+namespace mg {
+namespace {
+
+struct Jacobi8 {
+    double a[8][9];   // coefficient of z^j in the i-th shifted Jacobi(1,0) polynomial
+};
+
+// binomial coefficients as doubles (exact for the sizes used here)
+double binom(int n, int k) {
+    if (k < 0 || k > n) return 0.0;
+    double r = 1.0;
+    for (int i = 1; i <= k; i++) r = r * (n - k + i) / i;
+    return r;
+}
+
+// P_n^{(1,0)}(2x-1) = sum_s C(n+1, n-s) C(n, s) (x-1)^s x^(n-s)
+Jacobi8 jacobi_table() {
+    Jacobi8 t{};
+    for (int n = 0; n < 8; n++)
+        for (int s = 0; s <= n; s++) {
+            const double w = binom(n + 1, n - s) * binom(n, s);
+            for (int k = 0; k <= s; k++)
+                t.a[n][k + n - s] += w * binom(s, k) * (((s - k) & 1) ? -1.0 : 1.0);
+        }
+    return t;
+}
+
+// enc (E,8): radial_encode_8; rhat (E,3): tens_sigmoid(1, r * 7 / r0).
+// The polynomial is evaluated in fp64: its monomial form has alternating
+// coefficients up to ~1e5, so an fp32 evaluation carries ~1e-3 of rounding noise.
+__global__ void __launch_bounds__(256) bee_geometry_kernel(const float* __restrict__ r_ij, long E, float r0,
+                                                           float scale, Jacobi8 jac, float* __restrict__ enc,
+                                                           float* __restrict__ rhat) {
+    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= E) return;
+    const float x = r_ij[3 * e], y = r_ij[3 * e + 1], z = r_ij[3 * e + 2];
+    const float d = sqrtf(x * x + y * y + z * z);
+    const float zz = d / r0;
+    const double zd = (double)zz;
+    const float cut = fmaxf(1.0f - zz, 0.0f);
+#pragma unroll
+    for (int i = 0; i < 8; i++) {
+        double acc = jac.a[i][8];
+#pragma unroll
+        for (int j = 7; j >= 0; j--) acc = acc * zd + jac.a[i][j];
+        enc[8 * e + i] = (float)(acc * (double)cut);
+    }
+    const float sx = x * scale, sy = y * scale, sz = z * scale;
+    const float inv = 1.0f / sqrtf(1.0f + (sx * sx + sy * sy + sz * sz));
+    rhat[3 * e] = sx * inv;
+    rhat[3 * e + 1] = sy * inv;
+    rhat[3 * e + 2] = sz * inv;
+}
+
+__device__ __forceinline__ void cross3(const float* a, const float* b, float* o) {
+    o[0] = a[1] * b[2] - a[2] * b[1];
+    o[1] = a[2] * b[0] - a[0] * b[2];
+    o[2] = a[0] * b[1] - a[1] * b[0];
+}
+
+__device__ __forceinline__ long uniform(long v) {
+    // the value is the same in every lane: keep it in scalar registers
+    const int lo = __builtin_amdgcn_readfirstlane((int)(v & 0xffffffffL));
+    const int hi = __builtin_amdgcn_readfirstlane((int)(v >> 32));
+    return ((long)hi << 32) | (unsigned)lo;
+}
+
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4)))
+bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst, const int* __restrict__ order,
+                   long n_nodes, const float* __restrict__ rhat, const float* __restrict__ enc,
+                   const float* __restrict__ La, const float* __restrict__ Lv, const float* __restrict__ Ld, int chan,
+                   const float* __restrict__ enc_W, const float* __restrict__ enc_b, float* __restrict__ P0,
+                   float* __restrict__ S1, float* __restrict__ S2) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int chunks = (chan + kWave - 1) / kWave;
+    const long items = n_nodes * chunks;
+    // contiguous ranges of the processing order per XCD (workgroup ids go round-robin over 8 XCDs)
+    const long per_xcd = (items + 7) / 8;
+    const int xcd = blockIdx.x & 7;
+    const long waves_per_xcd = (long)(gridDim.x >> 3) * (blockDim.x / kWave);
+    const long wave_local = (long)(blockIdx.x >> 3) * (blockDim.x / kWave) + threadIdx.x / kWave;
+
+    for (long item_local = wave_local; item_local < per_xcd; item_local += waves_per_xcd) {
+        const long item = uniform(xcd * per_xcd + item_local);
+        if (item >= items) break;
+        const long k_node = item / chunks;
+        const int c = (int)(item - k_node * chunks) * kWave + lane;
+        const bool active = c < chan;
+        const int cc = active ? c : chan - 1;   // inactive lanes shadow a valid channel, stores are masked
+        const long node = order ? (long)order[k_node] : k_node;
+        const long lo = row_ptr[node], hi = row_ptr[node + 1];
+
+        float w[8];
+#pragma unroll
+        for (int m = 0; m < 8; m++) w[m] = enc_W[cc * 8 + m];
+        const float bias = enc_b[cc];
+
+        float s1[15], s2[45];
+#pragma unroll
+        for (int k = 0; k < 15; k++) s1[k] = 0.f;
+#pragma unroll
+        for (int k = 0; k < 45; k++) s2[k] = 0.f;
+
+        for (long e = lo; e < hi; e++) {
+            const long j = dst[e];
+            float en[8], rh[3];
+#pragma unroll
+            for (int m = 0; m < 8; m++) en[m] = enc[8 * e + m];
+#pragma unroll
+            for (int t = 0; t < 3; t++) rh[t] = rhat[3 * e + t];
+            // gathers: 13 unit-stride rows
+            const float l0 = La[j * chan + cc];
+            float l1[3], l2[9];
+#pragma unroll
+            for (int t = 0; t < 3; t++) l1[t] = Lv[(j * 3 + t) * chan + cc];
+#pragma unroll
+            for (int k = 0; k < 9; k++) l2[k] = Ld[(j * 9 + k) * chan + cc];
+
+            float phi = bias;
+#pragma unroll
+            for (int m = 0; m < 8; m++) phi += w[m] * en[m];
+
+            // geometric pieces
+            float t_[3];   // L rh
+#pragma unroll
+            for (int x = 0; x < 3; x++) t_[x] = l2[3 * x] * rh[0] + l2[3 * x + 1] * rh[1] + l2[3 * x + 2] * rh[2];
+            const float dot1 = l1[0] * rh[0] + l1[1] * rh[1] + l1[2] * rh[2];          // l1 . rh
+            const float quad = t_[0] * rh[0] + t_[1] * rh[1] + t_[2] * rh[2];           // rh^T L rh
+            float cr[3];
+            cross3(l1, rh, cr);
+            const float pl0 = phi * l0;
+            const float pd1 = phi * dot1;
+
+            if (active) {
+                float* p = P0 + (e * 3) * chan + c;
+                p[0] = pl0;              // 000
+                p[chan] = pd1;           // 110
+                p[2 * chan] = phi * quad;  // 220
+            }
+            // vector sums, label order 011, 101, 121, 211, 111
+#pragma unroll
+            for (int x = 0; x < 3; x++) {
+                s1[x * 5 + 0] += pl0 * rh[x];
+                s1[x * 5 + 1] += phi * l1[x];
+                s1[x * 5 + 2] += pd1 * rh[x];
+                s1[x * 5 + 3] += phi * t_[x];
+                s1[x * 5 + 4] += phi * cr[x];
+            }
+            // rank-2 sums, label order 022, 202, 112, 222, 212 ; component xy -> 3x+y
+#pragma unroll
+            for (int x = 0; x < 3; x++) {
+                float rowx[3];
+                cross3(l2 + 3 * x, rh, rowx);   // L[x,:] x rh
+                const float pl1x = phi * l1[x];
+                const float ptx = phi * t_[x];
+#pragma unroll
+                for (int y = 0; y < 3; y++) {
+                    const int k = 3 * x + y;
+                    s2[k * 5 + 0] += pl0 * (rh[y] * rh[x]);
+                    s2[k * 5 + 1] += phi * l2[k];
+                    s2[k * 5 + 2] += pl1x * rh[y];
+                    s2[k * 5 + 3] += ptx * rh[y];
+                    s2[k * 5 + 4] += phi * rowx[y];
+                }
+            }
+        }
+        if (active) {
+#pragma unroll
+            for (int k = 0; k < 15; k++) S1[(node * 15 + k) * chan + c] = s1[k];
+#pragma unroll
+            for (int k = 0; k < 45; k++) S2[(node * 45 + k) * chan + c] = s2[k];
+        }
+    }
+}
+
+}  // namespace
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" {
+
+int mg_bee_edge_geometry(const float* r_ij, long n_edges, float r0, float* enc, float* rhat, mg_stream_t stream) {
+    MG_REQUIRE(n_edges >= 0, "mg_bee_edge_geometry: negative size");
+    MG_REQUIRE(r0 > 0.f, "mg_bee_edge_geometry: r0 must be positive");
+    if (n_edges == 0) return MG_OK;
+    MG_REQUIRE(r_ij && enc && rhat, "mg_bee_edge_geometry: null pointer");
+    static const Jacobi8 table = jacobi_table();
+    const float scale = (float)(7.0 / (double)r0);
+    hipLaunchKernelGGL(bee_geometry_kernel, dim3((unsigned)ceil_div(n_edges, 256)), dim3(256), 0, (hipStream_t)stream,
+                       r_ij, n_edges, r0, scale, table, enc, rhat);
+    return check_launch("mg_bee_edge_geometry");
+}
+
+int mg_bee_message(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
+                   const float* rhat, const float* enc, const float* La, const float* Lv, const float* Ld, int chan,
+                   const float* enc_W, const float* enc_b, float* P0, float* S1, float* S2, mg_stream_t stream) {
+    MG_REQUIRE(n_nodes >= 0 && n_edges >= 0 && chan >= 0, "mg_bee_message: negative size");
+    if (n_nodes == 0 || chan == 0) return MG_OK;
+    MG_REQUIRE(row_ptr && La && Lv && Ld && enc_W && enc_b && S1 && S2, "mg_bee_message: null pointer");
+    MG_REQUIRE(n_edges == 0 || (dst && rhat && enc && P0), "mg_bee_message: null edge operand");
+    const long items = (long)n_nodes * ceil_div(chan, kWave);
+    long blocks = ceil_div(items, 4);
+    if (blocks > 256L * 16) blocks = 256L * 16;
+    blocks = ceil_div(blocks, 8) * 8;
+    hipLaunchKernelGGL(bee_message_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, row_ptr, dst,
+                       node_order, (long)n_nodes, rhat, enc, La, Lv, Ld, chan, enc_W, enc_b, P0, S1, S2);
+    return check_launch("mg_bee_message");
+}
+
+}  // extern "C"

@@ -53,10 +53,10 @@ struct Cfg {
     static constexpr int WS_PER = (WS + NT - 1) / NT;
 };
 
-template <int T, int WAVES_M, int WAVES_N, int WM, int WN, bool XVEC>
+template <int T, int WAVES_M, int WAVES_N, int WM, int WN, bool XVEC, bool SOA_OUT>
 __global__ void __launch_bounds__(64 * WAVES_M * WAVES_N)
 linear_kernel(const float* __restrict__ W, long so, long si, const float* __restrict__ X, long R, int I, int O,
-              const float* __restrict__ bias, int act, int accumulate, float* __restrict__ Y) {
+              const float* __restrict__ bias, int act, int accumulate, float* __restrict__ Y, int out_T) {
     using C = Cfg<T, WAVES_M, WAVES_N, WM, WN>;
     __shared__ float xs[C::RB * C::RS];
     __shared__ float ws[C::BN * C::RSW];
@@ -176,7 +176,10 @@ linear_kernel(const float* __restrict__ W, long so, long si, const float* __rest
                 const int m = (wave_m * WM + mi) * 32 + 8 * (q / 4) + 4 * khalf + (q % 4);
                 const long r = r0 + m / T;
                 if (r < R) {
-                    const long addr = (r * O + n) * T + (m % T);
+                    // SOA_OUT: component-major output (row, comp, chan) instead of (row, chan, comp)
+                    // T == 1 with out_T > 1: rows are (row, comp) pairs, output stored (row, chan, comp)
+                    long addr = SOA_OUT ? (r * T + (m % T)) * O + n : (r * O + n) * T + (m % T);
+                    if (T == 1 && out_T > 1) addr = ((r / out_T) * O + n) * out_T + r % out_T;
                     float v = acc[mi][ni][q] + bv;
                     v = activate(v, act);
                     if (accumulate) v += Y[addr];
@@ -189,19 +192,25 @@ linear_kernel(const float* __restrict__ W, long so, long si, const float* __rest
 
 template <int T, int WAVES_M, int WAVES_N, int WM, int WN>
 int launch_cfg(const float* W, long so, long si, const float* X, long R, int I, int O, const float* bias, int act,
-               int accumulate, float* Y, hipStream_t st) {
+               int accumulate, float* Y, hipStream_t st, bool soa_out = false, int out_T = 1) {
     using C = Cfg<T, WAVES_M, WAVES_N, WM, WN>;
     const long gx = ceil_div(R, C::RB);
     const long gy = ceil_div(O, C::BN);
     MG_REQUIRE(gx <= 0x7fffffffL && gy <= 65535, "mg_tensor_linear: grid too large (rows=%ld dim_out=%d)", R, O);
     const bool xvec = I > 0 && aligned16(X) && (I % kBK == 0) && (((long)I * T) % 4 == 0);
     dim3 grid((unsigned)gx, (unsigned)gy), block(C::NT);
-    if (xvec)
-        hipLaunchKernelGGL((linear_kernel<T, WAVES_M, WAVES_N, WM, WN, true>), grid, block, 0, st, W, so, si, X, R, I,
-                           O, bias, act, accumulate, Y);
+    if (xvec && soa_out)
+        hipLaunchKernelGGL((linear_kernel<T, WAVES_M, WAVES_N, WM, WN, true, true>), grid, block, 0, st, W, so, si, X,
+                           R, I, O, bias, act, accumulate, Y, out_T);
+    else if (xvec)
+        hipLaunchKernelGGL((linear_kernel<T, WAVES_M, WAVES_N, WM, WN, true, false>), grid, block, 0, st, W, so, si, X,
+                           R, I, O, bias, act, accumulate, Y, out_T);
+    else if (soa_out)
+        hipLaunchKernelGGL((linear_kernel<T, WAVES_M, WAVES_N, WM, WN, false, true>), grid, block, 0, st, W, so, si, X,
+                           R, I, O, bias, act, accumulate, Y, out_T);
     else
-        hipLaunchKernelGGL((linear_kernel<T, WAVES_M, WAVES_N, WM, WN, false>), grid, block, 0, st, W, so, si, X, R, I,
-                           O, bias, act, accumulate, Y);
+        hipLaunchKernelGGL((linear_kernel<T, WAVES_M, WAVES_N, WM, WN, false, false>), grid, block, 0, st, W, so, si,
+                           X, R, I, O, bias, act, accumulate, Y, out_T);
     return check_launch("mg_tensor_linear");
 }
 
@@ -227,7 +236,7 @@ template <bool WVEC>
 __global__ void __launch_bounds__(256)
 linear_rows_kernel(const float* __restrict__ W, long so, long si, const float* __restrict__ X, long R, int I, int O,
                    const float* __restrict__ bias, int act, int accumulate, float* __restrict__ Y, int tiles_n,
-                   long tiles_total) {
+                   long tiles_total, int out_T) {
     __shared__ __attribute__((aligned(16))) float xs[128 * kRS1];
     __shared__ __attribute__((aligned(16))) float ws[128 * kRS1];
 
@@ -339,7 +348,8 @@ linear_rows_kernel(const float* __restrict__ W, long so, long si, const float* _
             for (int q = 0; q < 16; q++) {
                 const long r = r0 + (wave_m * 2 + mi) * 32 + 8 * (q / 4) + 4 * khalf + (q % 4);
                 if (r < R) {
-                    const long addr = r * O + n;
+                    // out_T > 1: the rows are (row, comp) pairs and the output is stored (row, chan, comp)
+                    const long addr = out_T == 1 ? r * O + n : ((r / out_T) * O + n) * out_T + r % out_T;
                     float v = activate(acc[mi][ni][q] + bv, act);
                     if (accumulate) v += Y[addr];
                     Y[addr] = v;
@@ -350,7 +360,7 @@ linear_rows_kernel(const float* __restrict__ W, long so, long si, const float* _
 }
 
 int launch_rows(const float* W, long so, long si, const float* X, long R, int I, int O, const float* bias, int act,
-                int accumulate, float* Y, hipStream_t st) {
+                int accumulate, float* Y, hipStream_t st, int out_T = 1) {
     const long tiles_m = ceil_div(R, 128);
     const int tiles_n = (int)ceil_div(O, 128);
     const long total = tiles_m * tiles_n;
@@ -359,10 +369,10 @@ int launch_rows(const float* W, long so, long si, const float* X, long R, int I,
     const bool wvec = si == 1 && so % 4 == 0 && aligned16(W);
     if (wvec)
         hipLaunchKernelGGL(linear_rows_kernel<true>, dim3((unsigned)grid), dim3(256), 0, st, W, so, si, X, R, I, O, bias,
-                           act, accumulate, Y, tiles_n, total);
+                           act, accumulate, Y, tiles_n, total, out_T);
     else
         hipLaunchKernelGGL(linear_rows_kernel<false>, dim3((unsigned)grid), dim3(256), 0, st, W, so, si, X, R, I, O,
-                           bias, act, accumulate, Y, tiles_n, total);
+                           bias, act, accumulate, Y, tiles_n, total, out_T);
     return check_launch("mg_tensor_linear");
 }
 
@@ -373,35 +383,48 @@ using namespace mg;
 
 extern "C" {
 
-int mg_tensor_linear(int inds, const float* W, long w_stride_o, long w_stride_i, const float* x, long rows,
-                     int dim_in, int dim_out, const float* bias, int act, int accumulate, float* y,
-                     mg_stream_t stream) {
+int mg_tensor_linear_layout(int inds, const float* W, long w_stride_o, long w_stride_i, const float* x, long rows,
+                            int dim_in, int dim_out, const float* bias, int act, int accumulate, int x_layout,
+                            int y_layout, float* y, mg_stream_t stream) {
     if (inds < 0 || inds > 2)
         return fail(MG_ERR_UNSUPPORTED,
                     "tensor_linear currently only supports a number of indices up to 2.");
     MG_REQUIRE(rows >= 0 && dim_in >= 0 && dim_out >= 0, "mg_tensor_linear: negative size");
     MG_REQUIRE(act >= 0 && act <= 2, "mg_tensor_linear: unknown activation %d", act);
+    MG_REQUIRE((x_layout == 0 || x_layout == 1) && (y_layout == 0 || y_layout == 1),
+               "mg_tensor_linear: layouts are 0 (row, chan, comp) or 1 (row, comp, chan)");
     if (rows == 0 || dim_out == 0) return MG_OK;
     MG_REQUIRE(y != nullptr && (dim_in == 0 || (W != nullptr && x != nullptr)), "mg_tensor_linear: null pointer");
     hipStream_t st = (hipStream_t)stream;
     const float* b = bias;
-    switch (inds) {
-        case 0:
-            // wide layers with 16-byte aligned rows of whole 32-wide k slabs take the tuned kernel
-            if (dim_out > 64 && dim_in % kBK1 == 0 && aligned16(x))
-                return launch_rows(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
-            if (dim_out <= 32) return launch_cfg<1, 4, 1, 2, 1>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
-            if (dim_out <= 64) return launch_cfg<1, 2, 2, 2, 1>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
-            return launch_cfg<1, 2, 2, 2, 2>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
-        case 1:
-            if (dim_out <= 32) return launch_cfg<3, 2, 1, 3, 1>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
-            if (dim_out <= 64) return launch_cfg<3, 2, 2, 3, 1>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
-            return launch_cfg<3, 2, 2, 3, 2>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
-        default:
-            if (dim_out <= 32) return launch_cfg<9, 3, 1, 3, 1>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
-            if (dim_out <= 64) return launch_cfg<9, 3, 1, 3, 2>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
-            return launch_cfg<9, 3, 2, 3, 2>(W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, b, act, accumulate, y, st);
+    const long so = w_stride_o, si = w_stride_i;
+    const int T = inds == 0 ? 1 : (inds == 1 ? 3 : 9);
+    if (inds == 0 || x_layout == 1) {
+        // component-major input: every (row, comp) pair is an independent row of a plain GEMM
+        const long R = rows * T;
+        const int out_T = (y_layout == 1) ? 1 : T;
+        if (dim_in % kBK1 == 0 && aligned16(x) && (dim_out > 64 || out_T > 1))
+            return launch_rows(W, so, si, x, R, dim_in, dim_out, b, act, accumulate, y, st, out_T);
+        if (dim_out <= 32) return launch_cfg<1, 4, 1, 2, 1>(W, so, si, x, R, dim_in, dim_out, b, act, accumulate, y, st, false, out_T);
+        if (dim_out <= 64) return launch_cfg<1, 2, 2, 2, 1>(W, so, si, x, R, dim_in, dim_out, b, act, accumulate, y, st, false, out_T);
+        return launch_cfg<1, 2, 2, 2, 2>(W, so, si, x, R, dim_in, dim_out, b, act, accumulate, y, st, false, out_T);
     }
+    const bool soa = y_layout == 1;
+    if (inds == 1) {
+        if (dim_out <= 32) return launch_cfg<3, 2, 1, 3, 1>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
+        if (dim_out <= 64) return launch_cfg<3, 2, 2, 3, 1>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
+        return launch_cfg<3, 2, 2, 3, 2>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
+    }
+    if (dim_out <= 32) return launch_cfg<9, 3, 1, 3, 1>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
+    if (dim_out <= 64) return launch_cfg<9, 3, 1, 3, 2>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
+    return launch_cfg<9, 3, 2, 3, 2>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
+}
+
+int mg_tensor_linear(int inds, const float* W, long w_stride_o, long w_stride_i, const float* x, long rows,
+                     int dim_in, int dim_out, const float* bias, int act, int accumulate, float* y,
+                     mg_stream_t stream) {
+    return mg_tensor_linear_layout(inds, W, w_stride_o, w_stride_i, x, rows, dim_in, dim_out, bias, act, accumulate, 0,
+                                   0, y, stream);
 }
 
 }  // extern "C"

@@ -399,8 +399,14 @@ def tensor_prods_avd(a, v_l, v_r):
 ACT_NONE, ACT_SILU, ACT_LEAKY = 0, 1, 2
 
 
-def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=False):
-    """y[..., o, t] = act(sum_i W[o, i] x[..., i, t] + bias[o]); W may have any strides."""
+LAYOUT_CHAN_COMP, LAYOUT_COMP_CHAN = 0, 1
+
+
+def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=False,
+                      x_layout=LAYOUT_CHAN_COMP, y_layout=LAYOUT_CHAN_COMP):
+    """y[..., o, t] = act(sum_i W[o, i] x[..., i, t] + bias[o]); W may have any strides.
+    Layout 0 stores a tensor as (..., chan, (3,)^inds) like the reference; layout 1 is
+    component-major (..., 3^inds, chan), the layout the fused edge kernels read and write."""
     if not W.is_cuda:
         raise RuntimeError("W must be a CUDA tensor")
     _check_input(x, "x")
@@ -412,19 +418,25 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
         raise RuntimeError("tensor_linear currently only supports a number of indices up to 2. "
                            "go edit the code to add more (easy with copy/paste).")
     dim_out, dim_in = int(W.size(0)), int(W.size(1))
-    batch_dims = x.dim() - (1 + inds)
-    if batch_dims < 0:
-        raise RuntimeError("x has too few dims")
-    if x.size(batch_dims) != dim_in:
-        raise RuntimeError("channel dim size mismatch for x")
-    for i in range(batch_dims + 1, batch_dims + inds + 1):
-        if x.size(i) != 3:
-            raise RuntimeError("expected tensor index dim to be 3d for input x")
+    T = 3 ** inds
+    if x_layout == LAYOUT_CHAN_COMP:
+        batch_dims = x.dim() - (1 + inds)
+        if batch_dims < 0:
+            raise RuntimeError("x has too few dims")
+        if x.size(batch_dims) != dim_in:
+            raise RuntimeError("channel dim size mismatch for x")
+        for i in range(batch_dims + 1, batch_dims + inds + 1):
+            if x.size(i) != 3:
+                raise RuntimeError("expected tensor index dim to be 3d for input x")
+    else:
+        batch_dims = x.dim() - 2
+        if batch_dims < 0 or x.size(-1) != dim_in or x.size(-2) != T:
+            raise RuntimeError("component-major x must have shape (..., 3^inds, dim_in)")
+    lead = [int(d) for d in x.shape[:batch_dims]]
     rows = 1
-    for i in range(batch_dims):
-        rows *= int(x.size(i))
-    y_shape = list(x.shape)
-    y_shape[batch_dims] = dim_out
+    for d in lead:
+        rows *= d
+    y_shape = lead + ([dim_out] + [3] * inds if y_layout == LAYOUT_CHAN_COMP else [T, dim_out])
     if bias is not None:
         _check_input(bias, "bias")
         if bias.numel() != dim_out:
@@ -437,8 +449,9 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
             if list(out.shape) != y_shape:
                 raise RuntimeError("out has wrong shape")
             y = out
-        L.check(_lib.mg_tensor_linear(inds, _p(W), int(W.stride(0)), int(W.stride(1)), _p(x), rows, dim_in, dim_out,
-                                      _p(bias), int(act), int(bool(accumulate)), _p(y), _stream()))
+        L.check(_lib.mg_tensor_linear_layout(inds, _p(W), int(W.stride(0)), int(W.stride(1)), _p(x), rows, dim_in,
+                                             dim_out, _p(bias), int(act), int(bool(accumulate)), int(x_layout),
+                                             int(y_layout), _p(y), _stream()))
     return y
 
 
@@ -500,3 +513,49 @@ def painn_message(row_ptr, dst, r_ij, filt, actv, x_v, epsilon, res_a=None, res_
         L.check(_lib.mg_painn_message(_p(row_ptr), _p(dst), n_nodes, E, _p(r_ij), _p(filt), _p(actv), _p(x_v), n,
                                       float(epsilon), _p(res_a), _p(res_v), _p(out_a), _p(out_v), _stream()))
     return out_a, out_v
+
+
+# ------------------------------------------------------- rank-0/1/2 messages
+def bee_edge_geometry(r_ij, r0):
+    """(E,3) -> enc (E,8) = radial_encode_8(r_ij, r0), rhat (E,3) = tens_sigmoid(1, r_ij*7/r0)."""
+    _check_input(r_ij, "r_ij")
+    if r_ij.dim() != 2 or r_ij.size(1) != 3:
+        raise RuntimeError("r_ij must have shape (edges, 3)")
+    E = int(r_ij.size(0))
+    with torch.cuda.device(r_ij.device):
+        enc = torch.empty(E, 8, dtype=torch.float32, device=r_ij.device)
+        rhat = torch.empty(E, 3, dtype=torch.float32, device=r_ij.device)
+        L.check(_lib.mg_bee_edge_geometry(_p(r_ij), E, float(r0), _p(enc), _p(rhat), _stream()))
+    return enc, rhat
+
+
+def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=None):
+    """Fused products + edge sums of the rank-0/1/2 message (see mg_bee_message).
+    La (N,chan), Lv (N,3,chan), Ld (N,9,chan) -> P0 (E,3,chan), S1 (N,3,5,chan), S2 (N,9,5,chan)."""
+    _check_input(row_ptr, "row_ptr", torch.int32)
+    _check_input(dst, "dst", torch.int32)
+    for t, nm in ((rhat, "rhat"), (enc, "enc"), (La, "La"), (Lv, "Lv"), (Ld, "Ld"), (enc_W, "enc_W"),
+                  (enc_b, "enc_b")):
+        _check_input(t, nm)
+    N, chan = int(La.size(0)), int(La.size(1))
+    E = int(dst.numel())
+    if tuple(Lv.shape) != (N, 3, chan) or tuple(Ld.shape) != (N, 9, chan):
+        raise RuntimeError("Lv / Ld must be component-major (nodes, 3, chan) / (nodes, 9, chan)")
+    if tuple(enc.shape) != (E, 8) or tuple(rhat.shape) != (E, 3):
+        raise RuntimeError("enc must be (edges, 8) and rhat (edges, 3)")
+    if tuple(enc_W.shape) != (chan, 8) or enc_b.numel() != chan:
+        raise RuntimeError("enc_W must be (chan, 8) and enc_b (chan)")
+    if row_ptr.numel() != N + 1:
+        raise RuntimeError("row_ptr must have nodes+1 entries")
+    if node_order is not None:
+        _check_input(node_order, "node_order", torch.int32)
+        if node_order.numel() != N:
+            raise RuntimeError("node_order must have one entry per node")
+    dev = La.device
+    with torch.cuda.device(dev):
+        P0 = torch.empty(E, 3, chan, dtype=torch.float32, device=dev)
+        S1 = torch.empty(N, 3, 5, chan, dtype=torch.float32, device=dev)
+        S2 = torch.empty(N, 9, 5, chan, dtype=torch.float32, device=dev)
+        L.check(_lib.mg_bee_message(_p(row_ptr), _p(dst), _p(node_order), N, E, _p(rhat), _p(enc), _p(La), _p(Lv),
+                                    _p(Ld), chan, _p(enc_W), _p(enc_b), _p(P0), _p(S1), _p(S2), _stream()))
+    return P0, S1, S2
