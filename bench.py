@@ -36,7 +36,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="painn_layer",
-                    choices=["painn_layer", "neighbour", "products"])
+                    choices=["painn_layer", "neighbour", "products", "denoiser"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
     return ap.parse_args()
@@ -243,6 +243,97 @@ def bench_products(torch, args):
             "note": "includes allocation of the three outputs; 4096 rows (17.8 MB) is launch-latency bound"}
 
 
+def chain_positions(torch, systems, atoms, box, seed, noise=1.0):
+    g = torch.Generator().manual_seed(seed)
+    steps = torch.randn(systems, atoms, 3, generator=g)
+    steps = 3.8 * steps / steps.norm(dim=-1, keepdim=True)
+    pos = steps.cumsum(1) + torch.rand(systems, 1, 3, generator=g) * box
+    return (pos + noise * torch.randn(systems, atoms, 3, generator=g)).contiguous()
+
+
+def bench_denoiser(torch, args, with_cpu=True):
+    """BASELINE configs[3]: 8-block rank-0/1/2 denoiser forward, 32 systems x 2048 atoms."""
+    den = importlib.import_module("learned-dynamics_amd.denoiser")
+    seed = 0x947 + 4
+    torch.manual_seed(seed)
+    B, N, box_len, r0 = 32, 2048, 70.0, 6.0
+    dims = dict(dim_a=256, dim_v=64, dim_d=16, chan=256, blocks=8)
+    box = (box_len,) * 3
+    x1 = chain_positions(torch, B, N, box_len, seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    x0 = x1 + torch.randn(B, N, 3, generator=g)
+    types = torch.randint(0, 20, (B, N), generator=g)
+    one_hot = torch.nn.functional.one_hot(types, 20).float()
+    s, t = torch.zeros(B), torch.rand(B, generator=g)
+    model = den.Denoiser(r0, **dims).cuda().eval()
+    dev = [v.cuda() for v in (s, t, x0, x1, one_hot)]
+
+    with torch.no_grad():
+        def step():
+            return model((dev[0], dev[1]), dev[2], dev[3], dev[4], box)
+        step()
+        sec = timed_steps(torch, step, args.steps, args.warmup)
+        gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+        graph, _ = gl.graph_setup(r0, box, dev[3], neighbours_max=256, celllist_max=64)
+        E = int(graph.src.numel())
+    out = {"metric": "denoiser forward atoms/sec", "value": B * N / sec, "unit": "atoms/s", "ms_per_step": sec * 1e3,
+           "dtype": "f32",
+           "config": {"workload": "BASELINE configs[3]: 8 x [Messages + SelfTensProds] rank-0/1/2 denoiser forward "
+                                  "(assembled from reference modules), 32 systems x 2048 atoms, box 70 A, cutoff 6 A, "
+                                  "256 scalar + 64 vector + 16 rank-2 channels, chan 256, graph rebuilt every forward",
+                      "edges": E, "atoms": B * N}}
+    if with_cpu:
+        out["cpu_baseline"] = cpu_denoiser_block(torch, model, x1[:1], r0, box, dims)
+    return out
+
+
+def cpu_denoiser_block(torch, model, x1, r0, box, dims):
+    """Oracle (fp32 PyTorch CPU port of the reference math): ONE block (Messages + SelfTensProds) on ONE of the
+    32 systems; the forward is 8 such blocks per system, so atoms/s = atoms / (8 * t_block)."""
+    from oracle import layers as OL
+    from oracle import neighbour as ON
+    from oracle import products as OP
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    N = x1.shape[1]
+    ref = ON.edges(x1.numpy(), r0, box)
+    src, dst = torch.from_numpy(ref["src"]).long(), torch.from_numpy(ref["dst"]).long()
+    r_ij = torch.from_numpy(ON.edge_vectors(x1.numpy(), ref["src"], ref["dst"], box))
+    msg, prod = model.messages[0], model.prods[0]
+    dd = lambda p: p.detach().cpu()
+    Lm = msg.mlp_a.layers
+    w = {"L0": dd(msg.L0.W), "L1": dd(msg.L1.W), "L2": dd(msg.L2.W),
+         "Y": {lab: dd(getattr(msg, f"Y_{lab}").W) for lab in OP.BEE_ORDER},
+         "enc_W": dd(msg.lin_enc.weight), "enc_b": dd(msg.lin_enc.bias),
+         "mlp_a": {"W_direct": dd(msg.mlp_a.lin_direct.weight), "W1": dd(Lm[0].weight), "b1": dd(Lm[0].bias),
+                   "W2": dd(Lm[2].weight), "b2": dd(Lm[2].bias), "W3": dd(Lm[4].weight), "b3": dd(Lm[4].bias)}}
+    ws = {k: dd(getattr(prod, k).W) for k in ("L0", "R0", "L1", "R1", "L2", "R2")}
+    ws["Y"] = {lab: dd(getattr(prod, f"Y_{lab}").W) for lab in OP.BEE_ORDER}
+    ws.update(gn_a=dd(prod.gn_a.gamma), gn_v=dd(prod.gn_v.gamma), gn_d=dd(prod.gn_d.gamma))
+    g = torch.Generator().manual_seed(1)
+    x_a = torch.randn(1, N, dims["dim_a"], generator=g)
+    x_v = torch.randn(1, N, dims["dim_v"], 3, generator=g)
+    x_d = torch.randn(1, N, dims["dim_d"], 3, 3, generator=g)
+
+    def block():
+        d = OL.bee_messages(src, dst, 1, N, r_ij, x_a, x_v, x_d, w, r0)
+        return OL.self_tens_prods(x_a + d[0], x_v + d[1], x_d + d[2], ws)
+
+    with torch.no_grad():
+        block()
+        times = []
+        t_all = time.perf_counter()
+        while len(times) < 3 or (time.perf_counter() - t_all < 10 and len(times) < 10):
+            t0 = time.perf_counter()
+            block()
+            times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": N / (dims["blocks"] * med), "unit": "atoms/s", "cores": cores, "kind": "port",
+            "sample": f"1 of 32 systems ({N} atoms, {len(src)} edges), 1 of 8 blocks timed (median of {len(times)}), "
+                      f"scaled by 8 blocks; PyTorch CPU fp32"}
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -260,10 +351,13 @@ def main():
         if not args.no_extras:
             small = argparse.Namespace(steps=10, warmup=3)
             nb = bench_neighbour(torch, small, with_cpu=not args.no_cpu)
-            res["other_workloads"] = {"neighbour_search_configs[1]": nb, "tensor_products_configs[0]":
-                                      bench_products(torch, small)}
+            dn = bench_denoiser(torch, argparse.Namespace(steps=3, warmup=1), with_cpu=not args.no_cpu)
+            res["other_workloads"] = {"denoiser_forward_configs[3]": dn, "neighbour_search_configs[1]": nb,
+                                      "tensor_products_configs[0]": bench_products(torch, small)}
     elif args.workload == "neighbour":
         res = bench_neighbour(torch, args, with_cpu=not args.no_cpu)
+    elif args.workload == "denoiser":
+        res = bench_denoiser(torch, args, with_cpu=not args.no_cpu)
     else:
         res = bench_products(torch, args)
         res.setdefault("ms_per_step", res["detail"]["rows_4096"]["us"] * 1e-3)

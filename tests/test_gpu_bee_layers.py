@@ -146,3 +146,44 @@ def test_state_dict_names_match_reference():
     names = set(bee.SelfTensProds(8, 8, 8, 8).state_dict().keys())
     for expect in ("L0.W", "R0.W", "L2.W", "R2.W", "Y_111.W", "gn_a.gamma", "gn_v.gamma", "gn_d.gamma"):
         assert expect in names, expect
+
+
+def test_denoiser_forward_matches_oracle_composition(pkg):
+    """Small instance of the configs[3] assembly, end to end against the float64 oracle."""
+    den = importlib.import_module("learned-dynamics_amd.denoiser")
+    torch.manual_seed(0x947 + 4)
+    dim_a, dim_v, dim_d, chan, blocks = 32, 16, 8, 32, 2
+    box, r0, B, N = (24., 24., 24.), 6.0, 2, 300
+    model = den.Denoiser(r0, dim_a, dim_v, dim_d, chan, blocks).cuda()
+    x1 = torch.rand(B, N, 3) * 24
+    x0 = x1 + torch.randn(B, N, 3)
+    one_hot = torch.nn.functional.one_hot(torch.randint(0, 20, (B, N)), 20).float()
+    s, t = torch.zeros(B), torch.rand(B)
+    with torch.no_grad():
+        v = model((s.cuda(), t.cuda()), x0.cuda(), x1.cuda(), one_hot.cuda(), box)
+    # oracle composition (float64)
+    dd = lambda p: p.detach().cpu().double()
+    ref = ON.edges(x1.numpy(), r0, box)
+    src, dst = torch.from_numpy(ref["src"]).long(), torch.from_numpy(ref["dst"]).long()
+    r_ij = torch.from_numpy(ON.edge_vectors(x1.numpy(), ref["src"], ref["dst"], box)).double()
+    x_a = torch.nn.functional.linear(one_hot.double(), dd(model.embed.weight), dd(model.embed.bias))
+    freqs = torch.exp(-torch.arange(32) / 31.0).double()
+    ph = torch.cat([t.double()[:, None] * freqs, (t - s).double()[:, None] * freqs], 1)
+    temb = torch.nn.functional.linear(torch.cat([torch.sin(ph), torch.cos(ph)], 1), dd(model.t_embed.lin1.weight),
+                                      dd(model.t_embed.lin1.bias))
+    x_a = x_a + temb[:, None]
+    x_v = OP.tensor_linear(1, dd(model.v_readin.W), (x1 - x0).double()[..., None, :])
+    x_d = torch.zeros(B, N, dim_d, 3, 3, dtype=torch.float64)
+    for msg, prod in zip(model.messages, model.prods):
+        w = {"L0": dd(msg.L0.W), "L1": dd(msg.L1.W), "L2": dd(msg.L2.W),
+             "Y": {lab: dd(getattr(msg, f"Y_{lab}").W) for lab in OP.BEE_ORDER},
+             "enc_W": dd(msg.lin_enc.weight), "enc_b": dd(msg.lin_enc.bias), "mlp_a": _mlp_leaky_weights(msg.mlp_a)}
+        d = OL.bee_messages(src, dst, B, N, r_ij, x_a, x_v, x_d, w, r0)
+        x_a, x_v, x_d = x_a + d[0], x_v + d[1], x_d + d[2]
+        ws = {k: dd(getattr(prod, k).W) for k in ("L0", "R0", "L1", "R1", "L2", "R2")}
+        ws["Y"] = {lab: dd(getattr(prod, f"Y_{lab}").W) for lab in OP.BEE_ORDER}
+        ws.update(gn_a=dd(prod.gn_a.gamma), gn_v=dd(prod.gn_v.gamma), gn_d=dd(prod.gn_d.gamma))
+        d = OL.self_tens_prods(x_a, x_v, x_d, ws)
+        x_a, x_v, x_d = x_a + d[0], x_v + d[1], x_d + d[2]
+    v_ref = (1. - (t - s).double()[:, None, None]) * OP.tensor_linear(1, dd(model.readout.W), x_v).squeeze(-2)
+    _close(v, v_ref, rtol=1e-4, atol_scale=2e-5)   # 2 blocks deep: fp32 rounding compounds through the group norms
