@@ -28,6 +28,7 @@ sys.path.insert(0, ROOT)
 
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 PEAK_FP32_MFMA_TFLOPS = 157.3  # MI355X dense fp32 matrix
+PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X dense bf16 matrix
 
 
 def parse():
@@ -39,6 +40,8 @@ def parse():
                     choices=["painn_layer", "neighbour", "products", "denoiser"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also run a plain 1 GiB device copy (yardstick for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     return ap.parse_args()
 
 
@@ -115,9 +118,20 @@ def bench_painn_layer(torch, args):
         t_gemm = event_time(torch, lambda: ops.tensor_linear_fwd(0, lin.weight, h, bias=lin.bias, act=ops.ACT_SILU,
                                                                  out=out), 10)
         flops = 2.0 * E * (4 * n) * (4 * n)
-        roofline = {"kernel": "linear_kernel<T=1,128x128> (filter MLP layer, E x 512 x 512)", "bound": "mfma",
-                    "achieved": flops / t_gemm / 1e12, "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                    "frac": flops / t_gemm / 1e12 / PEAK_FP32_MFMA_TFLOPS, "traffic": None}
+        split = ops.get_linear_mode() == ops.LINEAR_BF16X3
+        if split:
+            # operands split into 3 bf16 pieces, 6 bf16 MFMAs per fp32 product, fp32 accumulate
+            roofline = {"kernel": "linear_rows_bf16x3_pipelined_kernel (filter MLP layer, E x 512 x 512, bias+SiLU fused)",
+                        "bound": "mfma", "achieved": 6 * flops / t_gemm / 1e12, "peak": PEAK_BF16_MFMA_TFLOPS,
+                        "unit": "TFLOP/s", "frac": 6 * flops / t_gemm / 1e12 / PEAK_BF16_MFMA_TFLOPS, "traffic": None,
+                        "note": "achieved counts the executed bf16 MFMA FLOPs (6 per fp32 multiply-add pair); "
+                                "fp32-equivalent rate and its ratio to the fp32 MFMA peak are given alongside",
+                        "fp32_equivalent_tflops": flops / t_gemm / 1e12,
+                        "fp32_equivalent_over_fp32_mfma_peak": flops / t_gemm / 1e12 / PEAK_FP32_MFMA_TFLOPS}
+        else:
+            roofline = {"kernel": "linear_rows_kernel (fp32 MFMA, filter MLP layer, E x 512 x 512, bias+SiLU fused)",
+                        "bound": "mfma", "achieved": flops / t_gemm / 1e12, "peak": PEAK_FP32_MFMA_TFLOPS,
+                        "unit": "TFLOP/s", "frac": flops / t_gemm / 1e12 / PEAK_FP32_MFMA_TFLOPS, "traffic": None}
         del h, out
 
         # --- HBM-bound edge kernel: fused gather-product-scatter
@@ -346,6 +360,13 @@ def main():
         sys.exit(1)
     torch.cuda.set_device(0)
 
+    if args.calibrate_copy:
+        a = torch.empty(1 << 28, dtype=torch.float32, device="cuda")
+        b = torch.empty_like(a)
+        t_copy = event_time(torch, lambda: b.copy_(a), 5)
+        print(f"calibration copy: 1 GiB read + 1 GiB written in {t_copy * 1e3:.3f} ms "
+              f"({2 * a.numel() * 4 / t_copy / 1e9:.0f} GB/s)", file=sys.stderr)
+        del a, b
     if args.workload == "painn_layer":
         res = bench_painn_layer(torch, args)
         if not args.no_extras:

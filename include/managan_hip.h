@@ -180,6 +180,27 @@ int mg_tensor_linear_layout(int inds, const float* W, long w_stride_o, long w_st
                             const float* x, long rows, int dim_in, int dim_out,
                             const float* bias, int act, int accumulate,
                             int x_layout, int y_layout, float* y, mg_stream_t stream);
+/* Arithmetic used by the wide plain-row GEMMs (inds = 0 or component-major x, dim_in % 32 == 0):
+ *   0  fp32 MFMA (v_mfma_f32_32x32x2_f32);
+ *   1  operands split exactly into three bf16 pieces, six bf16 MFMAs per product, fp32
+ *      accumulation: same accuracy class as fp32 (dropped terms < 2^-24 |a||b|), ~2.7x the rate.
+ * Process-wide setting; no counterpart in the reference (its kernel is a plain fp32 dot product,
+ * extensions/tensor_ops/tensor_ops_kern.cu:6-42). */
+int mg_set_linear_mode(int mode);
+int mg_get_linear_mode(void);
+/* Pre-split weights for mode 1: W (dim_out, dim_in, any strides) -> three bf16 planes (hi, mid, lo),
+ * dim_out rounded up to 128 rows, in caller-owned memory of mg_linear_packed_weight_bytes bytes
+ * (16-byte aligned).  mg_tensor_linear_packed then computes, for plain rows x (rows, dim_in),
+ * y = act(x W^T + bias) with x split on the fly; out_comps = 1 writes y (rows, dim_out); out_comps =
+ * 3 or 9 treats the rows as (row, comp) pairs and writes y (rows/out_comps, dim_out, out_comps).
+ * dim_in % 32 == 0, x 16-byte aligned.  Same contraction as tensor_linear
+ * (extensions/tensor_ops/tensor_ops.cpp:31-93); the packing has no counterpart in the reference. */
+int mg_linear_packed_weight_bytes(int dim_in, int dim_out, size_t* bytes /* host */);
+int mg_linear_pack_weight(const float* W, long w_stride_o, long w_stride_i, int dim_in, int dim_out,
+                          void* packed, mg_stream_t stream);
+int mg_tensor_linear_packed(const void* packed_W, const float* x, long rows, int dim_in, int dim_out,
+                            const float* bias, int act, int accumulate, int out_comps, float* y,
+                            mg_stream_t stream);
 /* dW[o,i] = sum_{r,t} dy[r,o,t] x[r,i,t]  (tensor_ops_kern.cu:45-71), dW dense (dim_out,dim_in). */
 int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows, int dim_in, int dim_out,
                            float* dW, mg_stream_t stream);

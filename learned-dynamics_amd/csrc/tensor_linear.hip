@@ -14,9 +14,16 @@
 //   A[m][k]: lane = m + 32k  (m < 32, k < 2)      B[k][n]: lane = n + 32k
 //   D[m][n]: n = lane % 32,  m = 8*(reg/4) + 4*(lane/32) + reg%4,  reg < 16
 #include "common.hpp"
+#include <atomic>
 
 namespace mg {
+// defined in tensor_linear_bf16x3.hip
+int launch_rows_bf16x3(const float* W, long so, const float* X, long R, int I, int O, const float* bias, int act,
+                       int accumulate, float* Y, hipStream_t st, int out_T);
+
 namespace {
+
+std::atomic<int> g_linear_mode{1};   // 0: fp32 MFMA everywhere; 1 (default): bf16x3 split for the wide T=1 GEMMs
 
 typedef float float16v __attribute__((ext_vector_type(16)));
 
@@ -403,8 +410,11 @@ int mg_tensor_linear_layout(int inds, const float* W, long w_stride_o, long w_st
         // component-major input: every (row, comp) pair is an independent row of a plain GEMM
         const long R = rows * T;
         const int out_T = (y_layout == 1) ? 1 : T;
-        if (dim_in % kBK1 == 0 && aligned16(x) && (dim_out > 64 || out_T > 1))
+        if (dim_in % kBK1 == 0 && aligned16(x) && (dim_out > 64 || out_T > 1)) {
+            if (g_linear_mode.load() == 1 && si == 1 && so % 4 == 0 && aligned16(W) && dim_in >= 64 && R >= 1024)
+                return launch_rows_bf16x3(W, so, x, R, dim_in, dim_out, b, act, accumulate, y, st, out_T);
             return launch_rows(W, so, si, x, R, dim_in, dim_out, b, act, accumulate, y, st, out_T);
+        }
         if (dim_out <= 32) return launch_cfg<1, 4, 1, 2, 1>(W, so, si, x, R, dim_in, dim_out, b, act, accumulate, y, st, false, out_T);
         if (dim_out <= 64) return launch_cfg<1, 2, 2, 2, 1>(W, so, si, x, R, dim_in, dim_out, b, act, accumulate, y, st, false, out_T);
         return launch_cfg<1, 2, 2, 2, 2>(W, so, si, x, R, dim_in, dim_out, b, act, accumulate, y, st, false, out_T);
@@ -419,6 +429,14 @@ int mg_tensor_linear_layout(int inds, const float* W, long w_stride_o, long w_st
     if (dim_out <= 64) return launch_cfg<9, 3, 1, 3, 2>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
     return launch_cfg<9, 3, 2, 3, 2>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
 }
+
+int mg_set_linear_mode(int mode) {
+    MG_REQUIRE(mode == 0 || mode == 1, "mg_set_linear_mode: mode must be 0 (fp32 MFMA) or 1 (bf16x3 split)");
+    g_linear_mode.store(mode);
+    return MG_OK;
+}
+
+int mg_get_linear_mode(void) { return g_linear_mode.load(); }
 
 int mg_tensor_linear(int inds, const float* W, long w_stride_o, long w_stride_i, const float* x, long rows,
                      int dim_in, int dim_out, const float* bias, int act, int accumulate, float* y,

@@ -7,6 +7,8 @@ stream through libmanagan_hip.so.  Nothing here computes on the CPU or with
 torch kernels: if the library is missing, importing this module fails.
 """
 import ctypes
+import weakref
+
 import torch
 
 from . import _lib as L
@@ -397,6 +399,43 @@ def tensor_prods_avd(a, v_l, v_r):
 
 
 ACT_NONE, ACT_SILU, ACT_LEAKY = 0, 1, 2
+LINEAR_FP32_MFMA, LINEAR_BF16X3 = 0, 1
+
+
+def set_linear_mode(mode):
+    """0: fp32 MFMA; 1: bf16x3-split operands on the bf16 MFMA (fp32-class accuracy, faster)."""
+    L.check(_lib.mg_set_linear_mode(int(mode)))
+
+
+def get_linear_mode():
+    return int(_lib.mg_get_linear_mode())
+
+
+_packed_cache = {}
+
+
+def packed_weight(W):
+    """bf16x3 planes of W for mg_tensor_linear_packed.  Cached per tensor OBJECT (weak reference) and
+    version counter, so parameters are packed once and re-packed after an in-place update; a new
+    tensor that happens to reuse a freed address never hits a stale entry."""
+    key = id(W)
+    hit = _packed_cache.get(key)
+    if hit is not None and hit[0]() is W and hit[1] == W._version and hit[2] == (W.data_ptr(), tuple(W.stride())):
+        return hit[3]
+    dim_out, dim_in = int(W.size(0)), int(W.size(1))
+    nbytes = ctypes.c_size_t(0)
+    L.check(_lib.mg_linear_packed_weight_bytes(dim_in, dim_out, ctypes.byref(nbytes)))
+    with torch.cuda.device(W.device):
+        packed = torch.empty(nbytes.value, dtype=torch.uint8, device=W.device)
+        L.check(_lib.mg_linear_pack_weight(_p(W), int(W.stride(0)), int(W.stride(1)), dim_in, dim_out, _p(packed),
+                                           _stream()))
+    if len(_packed_cache) > 512:
+        for k in [k for k, v in _packed_cache.items() if v[0]() is None]:
+            del _packed_cache[k]
+        if len(_packed_cache) > 512:
+            _packed_cache.clear()
+    _packed_cache[key] = (weakref.ref(W), W._version, (W.data_ptr(), tuple(W.stride())), packed)
+    return packed
 
 
 LAYOUT_CHAN_COMP, LAYOUT_COMP_CHAN = 0, 1
@@ -449,9 +488,16 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
             if list(out.shape) != y_shape:
                 raise RuntimeError("out has wrong shape")
             y = out
-        L.check(_lib.mg_tensor_linear_layout(inds, _p(W), int(W.stride(0)), int(W.stride(1)), _p(x), rows, dim_in,
-                                             dim_out, _p(bias), int(act), int(bool(accumulate)), int(x_layout),
-                                             int(y_layout), _p(y), _stream()))
+        plain_rows = inds == 0 or x_layout == LAYOUT_COMP_CHAN
+        if (plain_rows and get_linear_mode() == LINEAR_BF16X3 and dim_in % 32 == 0 and dim_in >= 64
+                and dim_out >= 64 and rows * T >= 1024 and x.data_ptr() % 16 == 0):
+            out_comps = 1 if (inds == 0 or y_layout == LAYOUT_COMP_CHAN) else T
+            L.check(_lib.mg_tensor_linear_packed(_p(packed_weight(W)), _p(x), rows * T, dim_in, dim_out, _p(bias),
+                                                 int(act), int(bool(accumulate)), out_comps, _p(y), _stream()))
+        else:
+            L.check(_lib.mg_tensor_linear_layout(inds, _p(W), int(W.stride(0)), int(W.stride(1)), _p(x), rows,
+                                                 dim_in, dim_out, _p(bias), int(act), int(bool(accumulate)),
+                                                 int(x_layout), int(y_layout), _p(y), _stream()))
     return y
 
 

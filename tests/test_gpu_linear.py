@@ -85,3 +85,46 @@ def test_tensor_linear_autograd(pkg, inds):
     tp.tensor_linear(inds, Wg, xg).backward(dy.cuda())
     torch.testing.assert_close(xg.grad.cpu(), xr.grad, rtol=1e-5, atol=1e-5)
     torch.testing.assert_close(Wg.grad.cpu(), Wr.grad, rtol=1e-5, atol=1e-4)
+
+
+@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("shape", [(5000, 512, 512, 0), (3000, 96, 200, 0), (2000, 64, 128, 1), (1500, 160, 72, 2),
+                                   (1024, 64, 64, 0), (4096, 768, 256, 0)])
+def test_linear_modes_agree_with_float64(ops, mode, shape):
+    """fp32 MFMA (mode 0) and bf16x3-split MFMA (mode 1) against a float64 product: both must sit at
+    fp32 rounding level; the split path uses pre-packed weights and may transpose (row, comp) outputs."""
+    rows, dim_in, dim_out, inds = shape
+    T = 3 ** inds
+    g = torch.Generator().manual_seed(77)
+    W = torch.randn(dim_out, dim_in, generator=g) / dim_in ** 0.5
+    b = torch.randn(dim_out, generator=g)
+    x_cm = torch.randn(rows, T, dim_in, generator=g)                   # component-major rows
+    ref = (x_cm.double() @ W.double().t() + b.double())
+    ref = torch.nn.functional.silu(ref)                                # (rows, T, O)
+    ref_aos = ref.transpose(1, 2).reshape(rows, dim_out, *([3] * inds))
+    prev = ops.get_linear_mode()
+    try:
+        ops.set_linear_mode(mode)
+        C = ops.LAYOUT_COMP_CHAN
+        y = ops.tensor_linear_fwd(inds, W.cuda(), x_cm.cuda() if inds else x_cm[:, 0].contiguous().cuda(),
+                                  bias=b.cuda(), act=ops.ACT_SILU, x_layout=C if inds else 0)
+    finally:
+        ops.set_linear_mode(prev)
+    err = (y.cpu().double() - ref_aos).abs().max().item()
+    assert err < 2e-6 * max(1.0, dim_in ** 0.5), err
+    torch.testing.assert_close(y.cpu(), ref_aos.float(), rtol=1e-5, atol=1e-6 * dim_in ** 0.5)
+
+
+def test_packed_weight_cache_tracks_in_place_updates(ops):
+    prev = ops.get_linear_mode()
+    try:
+        ops.set_linear_mode(1)
+        W = torch.randn(128, 128, device="cuda")
+        x = torch.randn(2048, 128, device="cuda")
+        y1 = ops.tensor_linear_fwd(0, W, x)
+        with torch.no_grad():
+            W.mul_(2.0)
+        y2 = ops.tensor_linear_fwd(0, W, x)
+        torch.testing.assert_close(y2, 2 * y1, rtol=1e-5, atol=1e-5)
+    finally:
+        ops.set_linear_mode(prev)
