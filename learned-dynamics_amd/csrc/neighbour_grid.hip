@@ -28,7 +28,7 @@
 namespace mg {
 namespace {
 
-constexpr int kCandCapDense = 2048;   // candidates staged in LDS per home cell (32 KB), 4-wave workgroups
+constexpr int kCandCapDense = 1024;   // candidates staged in LDS per home cell (16 KB), 4-wave workgroups
 constexpr int kCandCapSparse = 256;   // sparse boxes: 1-wave workgroups, 4 KB
 constexpr int kScanThreads = 256;
 constexpr int kScanItems = 8;       // per thread
@@ -52,12 +52,14 @@ struct Workspace {
     int* cell_start;    // C + 1
     int* block_sums;    // scan scratch
     int* block_max;     // scan scratch
+    unsigned long long* masks;   // A x mask_words: hit bits of the count pass, reused by the fill pass
+    int mask_words;     // 64-candidate groups kept per atom (= LDS tile size / 64)
     size_t bytes;
 };
 
 inline size_t align_up(size_t v) { return (v + 255) & ~size_t(255); }
 
-Workspace carve(void* base, long A, long C) {
+Workspace carve(void* base, long A, long C, int mask_words) {
     Workspace w{};
     size_t off = 0;
     auto take = [&](size_t bytes) {
@@ -76,6 +78,8 @@ Workspace carve(void* base, long A, long C) {
     w.cell_start = static_cast<int*>(take(sizeof(int) * (C + 1)));
     w.block_sums = static_cast<int*>(take(sizeof(int) * scan_blocks));
     w.block_max = static_cast<int*>(take(sizeof(int) * scan_blocks));
+    w.masks = static_cast<unsigned long long*>(take(sizeof(unsigned long long) * A * mask_words));
+    w.mask_words = mask_words;
     w.bytes = off;
     return w;
 }
@@ -110,9 +114,8 @@ __device__ __forceinline__ int cell_coord(float w, float box, int ndiv) {
     return c < 0 ? 0 : c;   // only reachable with non-finite input
 }
 
-// remainder(a - b, box) for a, b in [0, box]
-__device__ __forceinline__ float min_image(float a, float b, float box, float half) {
-    float d = a - b;
+// remainder(d, box) for d = a - b with a, b in [0, box]
+__device__ __forceinline__ float wrap_delta(float d, float box, float half) {
     if (d > half) d -= box;
     else if (d < -half) d += box;
     return d;
@@ -121,8 +124,13 @@ __device__ __forceinline__ float min_image(float a, float b, float box, float ha
 // ------------------------------------------------------------------- kernels
 // Clearing is done by a kernel, not a memset node, so that the sequence behaves
 // the same when a caller records it into a HIP graph.
-__global__ void __launch_bounds__(256) zero_kernel(int* __restrict__ p, long n) {
-    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (long)gridDim.x * blockDim.x) p[i] = 0;
+__global__ void __launch_bounds__(256) zero3_kernel(int* __restrict__ a, long na, int* __restrict__ b, long nb,
+                                                    int* __restrict__ c, long nc) {
+    const long stride = (long)gridDim.x * blockDim.x;
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    for (long i = t; i < na; i += stride) a[i] = 0;
+    for (long i = t; i < nb; i += stride) b[i] = 0;
+    for (long i = t; i < nc; i += stride) c[i] = 0;
 }
 
 __global__ void __launch_bounds__(256) bin_kernel(const float* __restrict__ x, Grid g, Workspace w) {
@@ -247,9 +255,42 @@ __global__ void __launch_bounds__(kScanThreads) scan_top_kernel(int* block_sums,
     }
 }
 
+// whole scan in one workgroup (n small): out[0..n], optional total / max.  Each lane scans a
+// contiguous chunk serially, the chunk totals are scanned across the workgroup once.
+__global__ void __launch_bounds__(kScanThreads) scan_small_kernel(const int* __restrict__ in, int n,
+                                                                  int* __restrict__ out, int* out_total, int* out_max) {
+    __shared__ int lds[8];
+    const int chunk = (n + kScanThreads) / kScanThreads;          // covers indices 0..n
+    const int lo = threadIdx.x * chunk;
+    const int hi = lo + chunk < n ? lo + chunk : n;
+    int sum = 0, mx = 0;
+    for (int k = lo; k < hi; k++) {
+        const int v = in[k];
+        sum += v;
+        mx = v > mx ? v : mx;
+    }
+    int total;
+    int run = block_excl_scan(sum, &total, lds);
+    for (int k = lo; k < lo + chunk && k <= n; k++) {
+        out[k] = run;
+        if (k < n) run += in[k];
+    }
+    for (int d = kWave / 2; d > 0; d >>= 1) { int t = __shfl_xor(mx, d); mx = t > mx ? t : mx; }
+    if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = mx;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int mm = 0;
+        for (int k = 0; k < kScanThreads / kWave; k++) mm = lds[k] > mm ? lds[k] : mm;
+        if (out_total) *out_total = total;
+        if (out_max) *out_max = mm;
+    }
+}
+
+// nodes > 0: also edge_counts[b] = out[(b+1)*nodes] (inclusive prefix of edges per box)
 __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(const int* __restrict__ in, long n,
                                                                   const int* __restrict__ block_offsets,
-                                                                  int* __restrict__ out) {
+                                                                  int* __restrict__ out, int nodes,
+                                                                  int* __restrict__ edge_counts) {
     __shared__ int lds[8];
     const long base = (long)blockIdx.x * kScanTile + (long)threadIdx.x * kScanItems;
     int v[kScanItems];
@@ -263,22 +304,35 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(const int* __r
     int run = block_excl_scan(s, &total, lds) + block_offsets[blockIdx.x];
 #pragma unroll
     for (int k = 0; k < kScanItems; k++) {
-        if (base + k <= n) out[base + k] = run;   // index n receives the grand total
+        if (base + k <= n) {
+            out[base + k] = run;   // index n receives the grand total
+            if (nodes > 0 && base + k > 0) {
+                const unsigned idx = (unsigned)(base + k), q = idx / (unsigned)nodes;   // n < 2^31: 32-bit divide
+                if (q * (unsigned)nodes == idx) edge_counts[q - 1] = run;
+            }
+        }
         run += v[k];
     }
 }
 
-// edge_counts[b] = row_ptr[(b+1)*nodes]
-__global__ void edge_counts_kernel(const int* __restrict__ row_ptr, int batch, int nodes, int* edge_counts) {
-    const int b = blockIdx.x * blockDim.x + threadIdx.x;
-    if (b < batch) edge_counts[b] = row_ptr[(long)(b + 1) * nodes];
-}
 
-// One workgroup per home cell.  FILL = false: degrees.  FILL = true: src/dst.
+// One workgroup per home cell.  FILL = false: degrees (+ hit masks).  FILL = true: src/dst.
+//
+// The count pass keeps, per home atom, one 64-bit ballot per group of 64 window
+// candidates; the fill pass replays those masks and never touches the geometry
+// again (it stages only the candidates' atom ids).  Windows larger than the LDS
+// tile (kCandCap candidates) fall back to recomputing in the fill pass.
+//
+// Minimum image: in an axis where the home cell does not touch the periodic
+// boundary and there are at least 5 cells, |w_i - w_j| < 2/5 box < box/2 for every
+// window candidate, so remainder(w_i - w_j, box) is the plain difference and the
+// conditional +-box is skipped (same bits, 40 % fewer instructions per pair).
 template <bool FILL, int kCandCap>
 __global__ void __launch_bounds__(256) pairs_kernel(Grid g, Workspace w, const int* __restrict__ row_ptr,
                                                     int* __restrict__ src, int* __restrict__ dst) {
-    __shared__ float4 cand[kCandCap];
+    constexpr int kWords = kCandCap / kWave;
+    __shared__ float4 cand[FILL ? 1 : kCandCap];      // count pass: wrapped positions + atom id
+    __shared__ int cand_idx[FILL ? kCandCap : 1];     // fill pass: atom ids only
     __shared__ int range_start[27];
     __shared__ int range_prefix[28];
 
@@ -309,6 +363,7 @@ __global__ void __launch_bounds__(256) pairs_kernel(Grid g, Workspace w, const i
     }
     __syncthreads();
     const int M = range_prefix[27];
+    const bool masks_ok = M <= kCandCap;      // uniform: the count pass stored every ballot of this cell
 
     // candidate k of the concatenated window -> address in the cell-ordered array
     auto locate = [&](int k) {
@@ -321,44 +376,84 @@ __global__ void __launch_bounds__(256) pairs_kernel(Grid g, Workspace w, const i
     };
 
     const int staged = M < kCandCap ? M : kCandCap;
-    for (int k = threadIdx.x; k < staged; k += blockDim.x) cand[k] = w.sorted[locate(k)];
+    for (int k = threadIdx.x; k < staged; k += blockDim.x) {
+        const float4 v = w.sorted[locate(k)];
+        if (FILL) cand_idx[k] = __float_as_int(v.w);
+        else cand[k] = v;
+    }
     __syncthreads();
 
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave, nwaves = blockDim.x / kWave;
     const float hx = 0.5f * g.bx, hy = 0.5f * g.by, hz = 0.5f * g.bz;
+    const bool wrap_x = g.nx < 5 || cx == 0 || cx == g.nx - 1;
+    const bool wrap_y = g.ny < 5 || cy == 0 || cy == g.ny - 1;
+    const bool wrap_z = g.nz < 5 || cz == 0 || cz == g.nz - 1;
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
     const int node_base = b * g.nodes;
+
+    auto test_pair = [&](const float4& self, const float4& o) {
+        float dx = self.x - o.x, dy = self.y - o.y, dz = self.z - o.z;
+        if (wrap_x) dx = wrap_delta(dx, g.bx, hx);
+        if (wrap_y) dy = wrap_delta(dy, g.by, hy);
+        if (wrap_z) dz = wrap_delta(dz, g.bz, hz);
+        const float d2 = __fmaf_rn(dz, dz, __fmaf_rn(dy, dy, dx * dx));
+        return d2 <= g.r0sq;
+    };
 
     for (int h = wave; h < home_n; h += nwaves) {
         const float4 self = w.sorted[home_lo + h];
         const int self_idx = __float_as_int(self.w);
         const int row = node_base + self_idx;
+        unsigned long long* my_masks = w.masks + (long)row * kWords;
         int running = 0;
-        int out_base = 0;
-        if (FILL) out_base = row_ptr[row];
-        for (int k0 = 0; k0 < M; k0 += kWave) {
-            const int k = k0 + lane;
-            bool hit = false;
-            int other_idx = 0;
-            if (k < M) {
-                const float4 o = k < kCandCap ? cand[k] : w.sorted[locate(k)];
-                other_idx = __float_as_int(o.w);
-                const float dx = min_image(self.x, o.x, g.bx, hx);
-                const float dy = min_image(self.y, o.y, g.by, hy);
-                const float dz = min_image(self.z, o.z, g.bz, hz);
-                const float d2 = __fmaf_rn(dz, dz, __fmaf_rn(dy, dy, dx * dx));
-                hit = (other_idx != self_idx) && (d2 <= g.r0sq);
+        const int words = (M + kWave - 1) / kWave;     // <= kWords when masks_ok
+        if (!FILL) {
+            unsigned long long keep = 0;               // lane i keeps the ballot of candidate group i
+            for (int k0 = 0; k0 < M; k0 += kWave) {
+                const int k = k0 + lane;
+                bool hit = false;
+                if (k < M) {
+                    const float4 o = k < kCandCap ? cand[k] : w.sorted[locate(k)];
+                    hit = (__float_as_int(o.w) != self_idx) && test_pair(self, o);
+                }
+                const unsigned long long mask = __ballot(hit);
+                if (lane == k0 / kWave) keep = mask;
+                running += __popcll(mask);
             }
-            const unsigned long long mask = __ballot(hit);
-            if (FILL && hit) {
-                const int pos = out_base + running + __popcll(mask & lt_mask);
-                src[pos] = row;
-                dst[pos] = node_base + other_idx;
+            if (masks_ok && lane < words) my_masks[lane] = keep;   // one unit-stride store per atom
+            if (lane == 0) w.degree[row] = running;
+        } else {
+            const int out_base = row_ptr[row];
+            unsigned long long keep = 0;
+            if (masks_ok && lane < words) keep = my_masks[lane];
+            for (int k0 = 0; k0 < M; k0 += kWave) {
+                const int k = k0 + lane;
+                unsigned long long mask;
+                int other_idx = 0;
+                if (masks_ok) {
+                    const int it = k0 / kWave;
+                    const unsigned lo = __shfl((unsigned)(keep & 0xffffffffull), it);
+                    const unsigned hi = __shfl((unsigned)(keep >> 32), it);
+                    mask = ((unsigned long long)hi << 32) | lo;
+                    if (k < M) other_idx = cand_idx[k];
+                } else {
+                    bool hit = false;
+                    if (k < M) {
+                        const float4 o = w.sorted[locate(k)];
+                        other_idx = __float_as_int(o.w);
+                        hit = (other_idx != self_idx) && test_pair(self, o);
+                    }
+                    mask = __ballot(hit);
+                }
+                if ((mask >> lane) & 1ull) {
+                    const int pos = out_base + running + __popcll(mask & lt_mask);
+                    src[pos] = row;
+                    dst[pos] = node_base + other_idx;
+                }
+                running += __popcll(mask);
             }
-            running += __popcll(mask);
         }
-        if (!FILL && lane == 0) w.degree[row] = running;
     }
 }
 
@@ -447,14 +542,22 @@ __global__ void __launch_bounds__(256) edge_vectors_kernel(const float* __restri
 }
 
 int run_scan(const int* in, long n, int* out, Workspace& w, int* out_total, int* out_max, int* out_overflow,
-             hipStream_t st) {
+             hipStream_t st, int nodes = 0, int* edge_counts = nullptr) {
+    if (n <= 16384 && nodes == 0 && out_overflow == nullptr) {
+        hipLaunchKernelGGL(scan_small_kernel, dim3(1), dim3(kScanThreads), 0, st, in, (int)n, out, out_total, out_max);
+        return check_launch("neighbour scan");
+    }
     const int nblocks = (int)ceil_div(n + 1, kScanTile);
     hipLaunchKernelGGL(scan_sums_kernel, dim3(nblocks), dim3(kScanThreads), 0, st, in, n, w.block_sums, w.block_max);
     hipLaunchKernelGGL(scan_top_kernel, dim3(1), dim3(kScanThreads), 0, st, w.block_sums, w.block_max, nblocks,
                        out_total, out_max, out_overflow);
-    hipLaunchKernelGGL(scan_apply_kernel, dim3(nblocks), dim3(kScanThreads), 0, st, in, n, w.block_sums, out);
+    hipLaunchKernelGGL(scan_apply_kernel, dim3(nblocks), dim3(kScanThreads), 0, st, in, n, w.block_sums, out, nodes,
+                       edge_counts);
     return check_launch("neighbour scan");
 }
+
+int pairs_block_size(const Grid& g);
+int mask_words(const Grid& g) { return (pairs_block_size(g) == 64 ? kCandCapSparse : kCandCapDense) / kWave; }
 
 int pairs_block_size(const Grid& g) {
     // sparse boxes: one wave per cell is plenty
@@ -482,7 +585,7 @@ int mg_neighbour_workspace_bytes(int batch, int nodes, float cutoff, float box_x
     Grid g;
     if (int s = make_grid(cutoff, box_x, box_y, box_z, batch, nodes, &g)) return s;
     const long A = (long)batch * nodes, C = (long)batch * g.ncells;
-    *bytes = carve(nullptr, A, C).bytes + 256;
+    *bytes = carve(nullptr, A, C, mask_words(g)).bytes + 256;
     return MG_OK;
 }
 
@@ -495,20 +598,18 @@ int mg_neighbour_count(const float* x, int batch, int nodes, float cutoff, float
     MG_REQUIRE(batch == 0 || edge_counts, "mg_neighbour_count: edge_counts is null");
     const long A = (long)batch * nodes, C = (long)batch * g.ncells;
     void* base = reinterpret_cast<void*>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~uintptr_t(255));
-    Workspace w = carve(base, A, C);
+    Workspace w = carve(base, A, C, mask_words(g));
     if (w.bytes + 256 > workspace_bytes)
         return fail(MG_ERR_WORKSPACE, "mg_neighbour_count: workspace has %zu bytes, %zu needed", workspace_bytes,
                     w.bytes + 256);
     hipStream_t st = (hipStream_t)stream;
-    hipLaunchKernelGGL(zero_kernel, dim3(1), dim3(256), 0, st, stats, 4L);
-    hipLaunchKernelGGL(zero_kernel, dim3(1), dim3(256), 0, st, row_ptr, 1L);
     if (A == 0) {
-        if (batch > 0) hipLaunchKernelGGL(zero_kernel, dim3(1), dim3(256), 0, st, edge_counts, (long)batch);
+        hipLaunchKernelGGL(zero3_kernel, dim3(1), dim3(256), 0, st, stats, 4L, row_ptr, 1L, edge_counts, (long)batch);
         return check_launch("mg_neighbour_count");
     }
     MG_REQUIRE(x != nullptr, "mg_neighbour_count: x is null");
-    hipLaunchKernelGGL(zero_kernel, dim3((unsigned)(ceil_div(C, 256) < 1024 ? ceil_div(C, 256) : 1024)), dim3(256), 0,
-                       st, w.cell_count, C);
+    hipLaunchKernelGGL(zero3_kernel, dim3((unsigned)(ceil_div(C, 256) < 1024 ? ceil_div(C, 256) : 1024)), dim3(256), 0,
+                       st, stats, 4L, row_ptr, 1L, w.cell_count, C);
     const unsigned ablocks = (unsigned)ceil_div(A, 256);
     hipLaunchKernelGGL(bin_kernel, dim3(ablocks), dim3(256), 0, st, x, g, w);
     if (int s = run_scan(w.cell_count, C, w.cell_start, w, nullptr, stats + 1, nullptr, st)) return s;
@@ -520,9 +621,7 @@ int mg_neighbour_count(const float* x, int batch, int nodes, float cutoff, float
     else
         hipLaunchKernelGGL((pairs_kernel<false, kCandCapDense>), dim3((unsigned)C), dim3(256), 0, st, g, w,
                            (const int*)nullptr, (int*)nullptr, (int*)nullptr);
-    if (int s = run_scan(w.degree, A, row_ptr, w, stats + 0, stats + 2, stats + 3, st)) return s;
-    hipLaunchKernelGGL(edge_counts_kernel, dim3((unsigned)ceil_div(batch, 64)), dim3(64), 0, st, row_ptr, batch,
-                       nodes, edge_counts);
+    if (int s = run_scan(w.degree, A, row_ptr, w, stats + 0, stats + 2, stats + 3, st, nodes, edge_counts)) return s;
     return check_launch("mg_neighbour_count");
 }
 
@@ -536,7 +635,7 @@ int mg_neighbour_fill(const void* workspace, size_t workspace_bytes, int batch, 
     if (A == 0 || n_edges == 0) return MG_OK;
     MG_REQUIRE(workspace && row_ptr && src && dst, "mg_neighbour_fill: null pointer");
     void* base = reinterpret_cast<void*>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~uintptr_t(255));
-    Workspace w = carve(base, A, C);
+    Workspace w = carve(base, A, C, mask_words(g));
     if (w.bytes + 256 > workspace_bytes)
         return fail(MG_ERR_WORKSPACE, "mg_neighbour_fill: workspace has %zu bytes, %zu needed", workspace_bytes,
                     w.bytes + 256);

@@ -103,7 +103,8 @@ def test_sparse_box_uses_single_wave_blocks(ops):
 
 
 def test_many_candidates_exceed_lds_tile(ops):
-    """More than 2048 candidates in a 27-cell window: the tail is read from global memory."""
+    """More candidates in a 27-cell window than the LDS tile holds (1024): the tail is read from global
+    memory and the fill pass recomputes instead of replaying hit masks."""
     rng = np.random.default_rng(17)
     box = (12., 12., 12.)
     x = (rng.random((1, 3000, 3)) * 12).astype(np.float32)     # 27 cells of 4 A: ~111 atoms per cell
