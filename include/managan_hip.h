@@ -224,6 +224,41 @@ int mg_painn_message(const int* row_ptr /* n_nodes+1 */, const int* dst /* E */,
                      int n, float epsilon, const float* res_a, const float* res_v,
                      float* out_a /* (n_nodes,n) */, float* out_v /* (n_nodes,n,3) */, mg_stream_t stream);
 
+/* Update.forward (archs/meanflow_painn8.py:63-75), elementwise parts around its GEMMs.
+ * lrv (rows, 3n, 3) = [lin_l | lin_r | lin_v] applied to x_v (one stacked tensor_linear).
+ *   pre:  ip[r,c] = sum_x l[c,x] r[c,x];  cat[r] = [x_a[r] | |r[c]|]  (rows, 2n), the MLP input
+ *   vec:  v = lin_v(x_v) * y[:, 0:n];  out_v = res_v + v / sqrt(1 + |v|^2)   (y: (rows, 3n) MLP output)
+ * The scalar output is mg_group_norm(mode 1) of ip * y[:, n:2n] plus y[:, 2n:3n]. */
+int mg_painn_update_pre(const float* lrv, const float* x_a, long rows, int n, float* ip, float* cat,
+                        mg_stream_t stream);
+int mg_painn_update_vec(const float* lrv, const float* y, const float* res_v /* or NULL */, long rows, int n,
+                        float* out_v, mg_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * Norms, squash, remaining radial encodings (node- or edge-sized streaming kernels).
+ * ---------------------------------------------------------------------- */
+/* Group norms over the nodes of a box and the channels of a group.
+ *   mode 0  TensGroupNorm (managan/tensor_products.py:215-232):
+ *           out = gamma[c] * v / sqrt(eps + mean_{nodes, group chans}(sum_comp v^2))
+ *   mode 1  ScalGroupNorm (managan/layers_common.py:201-223), comps = 1:
+ *           out = beta[c] + gamma[c] * (v - mean) / sqrt(eps + var)
+ * v = x (* mul if mul != NULL); element (b, i, c, t) of x at x[((b*nodes + i)*x_stride + c)*comps + t]
+ * (x_stride = channels per row of the underlying buffer, so a channel slice needs no copy), same for
+ * mul / add with their strides; out (batch, nodes, chan, comps) dense; out += add, out += res when
+ * given.  scratch: mg_group_norm_scratch_bytes bytes of device memory (fp64 partial sums, folded in
+ * a fixed order: results are deterministic). */
+int mg_group_norm_scratch_bytes(int batch, int groups, size_t* bytes /* host */);
+int mg_group_norm(int mode, const float* x, long x_stride, const float* mul, long mul_stride,
+                  int batch, int nodes, int chan, int groups, int comps, float eps,
+                  const float* gamma, const float* beta, const float* add, long add_stride,
+                  const float* res, void* scratch, float* out, mg_stream_t stream);
+/* tens_sigmoid (managan/tensor_products.py:167-182): x / sqrt(1 + sum_comp x^2) per (row, chan). */
+int mg_tens_sigmoid(int inds, const float* x, long rows_times_chan, float* out, mg_stream_t stream);
+/* kind 1: sq_radial_encode(normed_sq_dist(r, rmax), n) (archs/diffuser_atoms14.py:32-48);
+ * kind 2: radial_encode_edge(r, n, rmax) (archs/diffuser_atoms5.py:25-30).  out (E, n). */
+int mg_radial_encode(int kind, const float* r_ij, long n_edges, int n, float rmax, float* out,
+                     mg_stream_t stream);
+
 /* ------------------------------------------------------------------------
  * Rank-0/1/2 message passing with the 13 products (archs/diffuser_atoms15.py:227-253).
  * ---------------------------------------------------------------------- */

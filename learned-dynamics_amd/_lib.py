@@ -55,6 +55,12 @@ _SIGNATURES = {
     "mg_tensor_linear_packed": [vp, vp, i64, i32, i32, vp, i32, i32, i32, vp, vp],
     "mg_set_linear_mode": [i32],
     "mg_get_linear_mode": [],
+    "mg_group_norm_scratch_bytes": [i32, i32, ctypes.POINTER(ctypes.c_size_t)],
+    "mg_group_norm": [i32, vp, i64, vp, i64, i32, i32, i32, i32, i32, f32, vp, vp, vp, i64, vp, vp, vp, vp],
+    "mg_tens_sigmoid": [i32, vp, i64, vp, vp],
+    "mg_painn_update_pre": [vp, vp, i64, i32, vp, vp, vp],
+    "mg_painn_update_vec": [vp, vp, vp, i64, i32, vp, vp],
+    "mg_radial_encode": [i32, vp, i64, i32, f32, vp, vp],
     "mg_painn_radial_encode": [vp, i64, i32, f32, vp, vp],
     "mg_painn_message": [vp, vp, i32, i64, vp, vp, vp, vp, i32, f32, vp, vp, vp, vp, vp],
 }

@@ -57,12 +57,10 @@ class TensGroupNorm(nn.Module):
         self.inds, self.chan, self.groups, self.epsilon = inds, chan, groups, epsilon
         self.gamma = nn.Parameter(torch.ones(chan, *[1] * inds))
 
-    def forward(self, x):
-        batch, nodes = x.shape[:2]
-        xg = x.reshape(batch, nodes, self.groups, -1, 3 ** self.inds)
-        moment2 = (xg ** 2).sum(-1, keepdim=True).mean([1, 3], keepdim=True)
-        ans = xg / torch.sqrt(self.epsilon + moment2)
-        return self.gamma * ans.reshape(batch, nodes, self.chan, *[3] * self.inds)
+    def forward(self, x, res=None):
+        """gamma * x / sqrt(eps + second moment of the group) (+ res)."""
+        return ops.group_norm(ops.GN_TENSOR, x.contiguous(), self.groups, self.gamma.reshape(-1).contiguous(), None,
+                              self.epsilon, res=res)
 
 
 class SelfTensProds(nn.Module):
@@ -81,7 +79,9 @@ class SelfTensProds(nn.Module):
         self.gn_v = TensGroupNorm(1, dim_v, groups)
         self.gn_d = TensGroupNorm(2, dim_d, groups)
 
-    def forward(self, x_a, x_v, x_d):
+    def forward(self, x_a, x_v, x_d, residual=False):
+        """Returns the three normalised product features, or x + them with residual=True."""
+        in_a, in_v, in_d = x_a, x_v, x_d
         *rest, dim_a = x_a.shape
         dim_v, dim_d = x_v.shape[-2], x_d.shape[-3]
         rows = 1
@@ -95,6 +95,9 @@ class SelfTensProds(nn.Module):
         y_a = y_a.reshape(*rest, dim_a)
         y_v = y_v.reshape(*rest, dim_v, 3)
         y_d = y_d.reshape(*rest, dim_d, 3, 3)
+        if residual:
+            return (self.gn_a(y_a, res=in_a.contiguous()), self.gn_v(y_v, res=in_v.contiguous()),
+                    self.gn_d(y_d, res=in_d.contiguous()))
         return self.gn_a(y_a), self.gn_v(y_v), self.gn_d(y_d)
 
 

@@ -1,0 +1,261 @@
+// Node-level pieces of the layers that call the hot path: group norms over the
+// atoms of a box, the tensor squash, the elementwise parts of the PaiNN update, and
+// the remaining radial encodings.  All HBM-bound streaming over node-sized (or, for
+// the encodings, edge-sized) arrays; the norms need one box-wide reduction each.
+//
+// Reductions are deterministic: workgroup partials in a caller-provided scratch
+// array (fp64), folded in a fixed order by the apply kernel.
+#include "common.hpp"
+
+namespace mg {
+namespace {
+
+constexpr int kChunks = 64;   // partial sums per (box, group)
+
+__device__ __forceinline__ double block_sum(double v, double* lds) {
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) v += __shfl_xor(v, d);
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    __syncthreads();
+    if (lane == 0) lds[wave] = v;
+    __syncthreads();
+    double t = 0.0;
+    for (int k = 0; k < (int)(blockDim.x / kWave); k++) t += lds[k];
+    return t;
+}
+
+// x element (box b, node i, channel c, comp t) at x[((b*N + i)*x_stride + c)*T + t]; optional elementwise
+// multiplier mul at the same index pattern with mul_stride.  partial[(b*G + g)*kChunks + chunk][0..1] =
+// (sum, sum of squares) over that chunk's nodes, the group's channels and all components.
+__global__ void __launch_bounds__(256) group_stats_kernel(const float* __restrict__ x, long x_stride,
+                                                          const float* __restrict__ mul, long mul_stride, int N,
+                                                          int chan, int groups, int T, double* __restrict__ partial) {
+    __shared__ double lds[8];
+    const int bg = blockIdx.x, chunk = blockIdx.y;
+    const int b = bg / groups, g = bg - b * groups;
+    const int cg = chan / groups;
+    const int per = (N + kChunks - 1) / kChunks;
+    const int n_lo = chunk * per, n_hi = n_lo + per < N ? n_lo + per : N;
+    const long row_elems = (long)cg * T;
+    double s = 0.0, ss = 0.0;
+    const long total = (long)(n_hi > n_lo ? n_hi - n_lo : 0) * row_elems;
+    for (long t = threadIdx.x; t < total; t += blockDim.x) {
+        const long i = n_lo + t / row_elems;
+        const long rem = t - (t / row_elems) * row_elems;      // (c_local, comp), comp fastest
+        const long c = g * cg + rem / T, comp = rem - (rem / T) * T;
+        float v = x[(((long)b * N + i) * x_stride + c) * T + comp];
+        if (mul) v *= mul[(((long)b * N + i) * mul_stride + c) * T + comp];
+        s += v;
+        ss += (double)v * v;
+    }
+    const double ts = block_sum(s, lds);
+    const double tss = block_sum(ss, lds);
+    if (threadIdx.x == 0) {
+        partial[((long)bg * kChunks + chunk) * 2] = ts;
+        partial[((long)bg * kChunks + chunk) * 2 + 1] = tss;
+    }
+}
+
+// fold the kChunks partials of every (box, group) in a fixed order: partial[bg*kChunks*2 + {0,1}] <- totals
+__global__ void group_finalize_kernel(double* __restrict__ partial, int n_bg) {
+    const int bg = blockIdx.x * blockDim.x + threadIdx.x;
+    if (bg >= n_bg) return;
+    double* p = partial + (long)bg * kChunks * 2;
+    double s = 0.0, ss = 0.0;
+    for (int k = 0; k < kChunks; k++) { s += p[2 * k]; ss += p[2 * k + 1]; }
+    p[0] = s;
+    p[1] = ss;
+}
+
+// mode 0 (TensGroupNorm): y = gamma[c] * v / sqrt(eps + mean(sum_comp v^2))
+// mode 1 (ScalGroupNorm, T = 1): y = beta[c] + gamma[c] * (v - mean) / sqrt(eps + var)
+// then y += add (optional, add_stride) and y += res (optional, same layout as out).
+__global__ void __launch_bounds__(256) group_apply_kernel(const float* __restrict__ x, long x_stride,
+                                                          const float* __restrict__ mul, long mul_stride,
+                                                          const double* __restrict__ partial, int B, int N, int chan,
+                                                          int groups, int T, int mode, float eps,
+                                                          const float* __restrict__ gamma, const float* __restrict__ beta,
+                                                          const float* __restrict__ add, long add_stride,
+                                                          const float* __restrict__ res, float* __restrict__ out) {
+    const long total = (long)B * N * chan * T;
+    const int cg = chan / groups;
+    for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (long)gridDim.x * blockDim.x) {
+        const long comp = t % T, c = (t / T) % chan, row = t / ((long)T * chan);
+        const int b = (int)(row / N), g = (int)(c / cg);
+        const double* p = partial + ((long)(b * groups + g) * kChunks) * 2;   // totals after the finalize kernel
+        const double s = p[0], ss = p[1];
+        float v = x[(row * x_stride + c) * T + comp];
+        if (mul) v *= mul[(row * mul_stride + c) * T + comp];
+        float y;
+        if (mode == 0) {
+            const double m2 = ss / ((double)N * cg);                      // mean over nodes and group channels
+            y = gamma[c] * (v / sqrtf(eps + (float)m2));
+        } else {
+            const double cnt = (double)N * cg;
+            const double mean = s / cnt;
+            double var = ss / cnt - mean * mean;
+            var = var > 0.0 ? var : 0.0;
+            y = beta[c] + gamma[c] * ((v - (float)mean) / sqrtf(eps + (float)var));
+        }
+        if (add) y += add[(row * add_stride + c) * T + comp];
+        if (res) y += res[t];
+        out[t] = y;
+    }
+}
+
+// x / sqrt(1 + sum_comp x^2) per (row, chan)
+__global__ void __launch_bounds__(256) tens_sigmoid_kernel(const float* __restrict__ x, long n, int T,
+                                                           float* __restrict__ out) {
+    for (long e = (long)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += (long)gridDim.x * blockDim.x) {
+        float v[9], q = 0.f;
+        for (int t = 0; t < T; t++) { v[t] = x[e * T + t]; q += v[t] * v[t]; }
+        const float inv = 1.0f / sqrtf(1.0f + q);
+        for (int t = 0; t < T; t++) out[e * T + t] = v[t] * inv;
+    }
+}
+
+// PaiNN Update, first elementwise stage: lrv (rows, 3n, 3) = [lin_l | lin_r | lin_v](x_v)
+//   ip[r,c] = sum_x l[c,x] r[c,x];  cat[r] = [x_a[r] | |r[c]|]   (rows, 2n)
+__global__ void __launch_bounds__(256) painn_update_pre_kernel(const float* __restrict__ lrv, const float* __restrict__ x_a,
+                                                               long rows, int n, float* __restrict__ ip,
+                                                               float* __restrict__ cat) {
+    const long total = rows * n;
+    for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (long)gridDim.x * blockDim.x) {
+        const long r = t / n;
+        const int c = (int)(t - r * n);
+        const float* l = lrv + (r * 3 * n + c) * 3;
+        const float* rr = lrv + (r * 3 * n + n + c) * 3;
+        ip[t] = l[0] * rr[0] + l[1] * rr[1] + l[2] * rr[2];
+        cat[r * 2 * n + c] = x_a[t];
+        cat[r * 2 * n + n + c] = sqrtf(rr[0] * rr[0] + rr[1] * rr[1] + rr[2] * rr[2]);
+    }
+}
+
+// PaiNN Update, vector output: v = lin_v(x_v) * y[0:n]; out = res_v + v / sqrt(1 + |v|^2)
+__global__ void __launch_bounds__(256) painn_update_vec_kernel(const float* __restrict__ lrv, const float* __restrict__ y,
+                                                               const float* __restrict__ res_v, long rows, int n,
+                                                               float* __restrict__ out_v) {
+    const long total = rows * n;
+    for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (long)gridDim.x * blockDim.x) {
+        const long r = t / n;
+        const int c = (int)(t - r * n);
+        const float* v = lrv + (r * 3 * n + 2 * n + c) * 3;
+        const float s = y[r * 3 * n + c];
+        const float a = v[0] * s, b = v[1] * s, d = v[2] * s;
+        const float inv = 1.0f / sqrtf(1.0f + (a * a + b * b + d * d));
+        float o0 = a * inv, o1 = b * inv, o2 = d * inv;
+        if (res_v) { o0 += res_v[3 * t]; o1 += res_v[3 * t + 1]; o2 += res_v[3 * t + 2]; }
+        out_v[3 * t] = o0; out_v[3 * t + 1] = o1; out_v[3 * t + 2] = o2;
+    }
+}
+
+// kinds: 1 sq_radial_encode of normed_sq_dist (archs/diffuser_atoms14.py:32-48)
+//        2 radial_encode_edge (archs/diffuser_atoms5.py:25-30)
+__global__ void __launch_bounds__(256) radial_encode_kernel(int kind, const float* __restrict__ r_ij, long E, int n,
+                                                            float rmax, float c0, float c1, float* __restrict__ out) {
+    const long total = E * n;
+    for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (long)gridDim.x * blockDim.x) {
+        const long e = t / n;
+        const int m = (int)(t - e * n);
+        const float x = r_ij[3 * e], y = r_ij[3 * e + 1], z = r_ij[3 * e + 2];
+        const float sq = x * x + y * y + z * z;
+        if (kind == 1) {
+            const float q = sq / (rmax * rmax);
+            const float h = sqrtf(1.0f + q);
+            const float coeff = c0 * expf(c1 * (float)m);        // (pi / sqrt 2) exp(n^-0.7 m)
+            out[t] = sinf(coeff * h) * (0.70710678118654752f - h);
+        } else {
+            const float q = sq / rmax;                             // divided by rmax, not rmax^2, as in the reference
+            const float cut = fmaxf(1.0f - q, 0.0f);
+            out[t] = cosf((c0 * (float)m) * sqrtf(q)) * cut;      // c0 = pi
+        }
+    }
+}
+
+long grid_for(long total) {
+    long b = ceil_div(total, 256);
+    return b > 256L * 32 ? 256L * 32 : (b < 1 ? 1 : b);
+}
+
+}  // namespace
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" {
+
+int mg_group_norm_scratch_bytes(int batch, int groups, size_t* bytes) {
+    MG_REQUIRE(bytes && batch >= 0 && groups >= 0, "mg_group_norm_scratch_bytes: bad argument");
+    *bytes = (size_t)batch * groups * kChunks * 2 * sizeof(double);
+    return MG_OK;
+}
+
+int mg_group_norm(int mode, const float* x, long x_stride, const float* mul, long mul_stride, int batch, int nodes,
+                  int chan, int groups, int comps, float eps, const float* gamma, const float* beta, const float* add,
+                  long add_stride, const float* res, void* scratch, float* out, mg_stream_t stream) {
+    MG_REQUIRE(mode == 0 || mode == 1, "mg_group_norm: mode must be 0 (tensor) or 1 (scalar)");
+    MG_REQUIRE(batch >= 0 && nodes >= 0 && chan >= 0 && groups > 0 && chan % groups == 0, "mg_group_norm: bad sizes");
+    MG_REQUIRE(comps == 1 || comps == 3 || comps == 9, "mg_group_norm: comps must be 1, 3 or 9");
+    MG_REQUIRE(mode == 0 || comps == 1, "mg_group_norm: the scalar norm takes comps == 1");
+    const long total = (long)batch * nodes * chan * comps;
+    if (total == 0) return MG_OK;
+    MG_REQUIRE(x && gamma && out && scratch && (mode == 0 || beta), "mg_group_norm: null pointer");
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(group_stats_kernel, dim3((unsigned)(batch * groups), kChunks), dim3(256), 0, st, x, x_stride, mul,
+                       mul_stride, nodes, chan, groups, comps, static_cast<double*>(scratch));
+    hipLaunchKernelGGL(group_finalize_kernel, dim3((unsigned)ceil_div((long)batch * groups, 64)), dim3(64), 0, st,
+                       static_cast<double*>(scratch), batch * groups);
+    hipLaunchKernelGGL(group_apply_kernel, dim3((unsigned)grid_for(total)), dim3(256), 0, st, x, x_stride, mul,
+                       mul_stride, static_cast<const double*>(scratch), batch, nodes, chan, groups, comps, mode, eps,
+                       gamma, beta, add, add_stride, res, out);
+    return check_launch("mg_group_norm");
+}
+
+int mg_tens_sigmoid(int inds, const float* x, long rows_times_chan, float* out, mg_stream_t stream) {
+    MG_REQUIRE(inds >= 0 && inds <= 2 && rows_times_chan >= 0, "mg_tens_sigmoid: bad argument");
+    if (rows_times_chan == 0) return MG_OK;
+    MG_REQUIRE(x && out, "mg_tens_sigmoid: null pointer");
+    const int T = inds == 0 ? 1 : (inds == 1 ? 3 : 9);
+    hipLaunchKernelGGL(tens_sigmoid_kernel, dim3((unsigned)grid_for(rows_times_chan)), dim3(256), 0,
+                       (hipStream_t)stream, x, rows_times_chan, T, out);
+    return check_launch("mg_tens_sigmoid");
+}
+
+int mg_painn_update_pre(const float* lrv, const float* x_a, long rows, int n, float* ip, float* cat,
+                        mg_stream_t stream) {
+    MG_REQUIRE(rows >= 0 && n >= 0, "mg_painn_update_pre: negative size");
+    if (rows * n == 0) return MG_OK;
+    MG_REQUIRE(lrv && x_a && ip && cat, "mg_painn_update_pre: null pointer");
+    hipLaunchKernelGGL(painn_update_pre_kernel, dim3((unsigned)grid_for(rows * n)), dim3(256), 0, (hipStream_t)stream,
+                       lrv, x_a, rows, n, ip, cat);
+    return check_launch("mg_painn_update_pre");
+}
+
+int mg_painn_update_vec(const float* lrv, const float* y, const float* res_v, long rows, int n, float* out_v,
+                        mg_stream_t stream) {
+    MG_REQUIRE(rows >= 0 && n >= 0, "mg_painn_update_vec: negative size");
+    if (rows * n == 0) return MG_OK;
+    MG_REQUIRE(lrv && y && out_v, "mg_painn_update_vec: null pointer");
+    hipLaunchKernelGGL(painn_update_vec_kernel, dim3((unsigned)grid_for(rows * n)), dim3(256), 0, (hipStream_t)stream,
+                       lrv, y, res_v, rows, n, out_v);
+    return check_launch("mg_painn_update_vec");
+}
+
+int mg_radial_encode(int kind, const float* r_ij, long n_edges, int n, float rmax, float* out, mg_stream_t stream) {
+    MG_REQUIRE(kind == 1 || kind == 2, "mg_radial_encode: kind must be 1 (sq_radial_encode) or 2 (radial_encode_edge)");
+    MG_REQUIRE(n_edges >= 0 && n >= 0 && rmax > 0.f, "mg_radial_encode: bad argument");
+    if (n_edges * n == 0) return MG_OK;
+    MG_REQUIRE(r_ij && out, "mg_radial_encode: null pointer");
+    float c0, c1 = 0.f;
+    if (kind == 1) {
+        c0 = (float)(3.14159265358979323846 * 0.70710678118654752440);
+        c1 = (float)pow((double)n, -0.7);
+    } else {
+        c0 = (float)3.14159265358979323846;
+    }
+    hipLaunchKernelGGL(radial_encode_kernel, dim3((unsigned)grid_for(n_edges * n)), dim3(256), 0, (hipStream_t)stream,
+                       kind, r_ij, n_edges, n, rmax, c0, c1, out);
+    return check_launch("mg_radial_encode");
+}
+
+}  // extern "C"

@@ -64,7 +64,6 @@ class Denoiser(nn.Module):
         for msg, prod in zip(self.messages, self.prods):
             d_a, d_v, d_d = msg(graph, r_ij, x_a, x_v, x_d, node_order=node_order)
             x_a, x_v, x_d = x_a + d_a, x_v + d_v, x_d + d_d
-            d_a, d_v, d_d = prod(x_a, x_v, x_d)
-            x_a, x_v, x_d = x_a + d_a, x_v + d_v, x_d + d_d
+            x_a, x_v, x_d = prod(x_a, x_v, x_d, residual=True)
         v_pred = self.readout(x_v).squeeze(-2)
         return (1. - (t - s)[:, None, None]) * v_pred

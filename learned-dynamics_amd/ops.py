@@ -605,3 +605,119 @@ def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=No
         L.check(_lib.mg_bee_message(_p(row_ptr), _p(dst), _p(node_order), N, E, _p(rhat), _p(enc), _p(La), _p(Lv),
                                     _p(Ld), chan, _p(enc_W), _p(enc_b), _p(P0), _p(S1), _p(S2), _stream()))
     return P0, S1, S2
+
+
+# ------------------------------------------------- norms, squash, update glue
+def _chan_view(t, name, lead_dims, chan, comps):
+    """t: (*lead, chan, comps...) possibly a channel slice of a wider contiguous buffer.
+    Returns the row stride in channels."""
+    if not t.is_cuda or t.dtype != torch.float32:
+        raise RuntimeError(f"{name} must be a float32 CUDA tensor")
+    t3 = t.reshape(-1, chan, comps) if t.is_contiguous() else t
+    if t.is_contiguous():
+        return chan
+    # accept (rows..., chan, comps) views whose only irregularity is a wider row
+    comp_dims = t.dim() - lead_dims - 1
+    strides, sizes = t.stride(), t.shape
+    inner = 1
+    for d in range(t.dim() - 1, lead_dims, -1):
+        if strides[d] != inner:
+            raise RuntimeError(f"{name}: unsupported memory layout")
+        inner *= sizes[d]
+    if strides[lead_dims] != comps:
+        raise RuntimeError(f"{name}: unsupported memory layout")
+    row_stride = strides[lead_dims - 1]
+    if row_stride % comps != 0:
+        raise RuntimeError(f"{name}: unsupported memory layout")
+    expect = row_stride
+    for d in range(lead_dims - 2, -1, -1):
+        expect *= sizes[d + 1]
+        if strides[d] != expect:
+            raise RuntimeError(f"{name}: unsupported memory layout")
+    return row_stride // comps
+
+
+GN_TENSOR, GN_SCALAR = 0, 1
+
+
+def group_norm(mode, x, groups, gamma, beta=None, eps=1e-5, mul=None, add=None, res=None):
+    """TensGroupNorm (mode 0) / ScalGroupNorm (mode 1) of v = x (* mul), plus optional add and res.
+    x: (batch, nodes, chan, (3,)^inds); x, mul and add may be channel slices of wider buffers."""
+    B, N, chan = int(x.shape[0]), int(x.shape[1]), int(x.shape[2])
+    comps = 1
+    for d in x.shape[3:]:
+        comps *= int(d)
+    xs = _chan_view(x, "x", 2, chan, comps)
+    ms = _chan_view(mul, "mul", 2, chan, comps) if mul is not None else 0
+    as_ = _chan_view(add, "add", 2, chan, comps) if add is not None else 0
+    _check_input(gamma, "gamma")
+    if beta is not None:
+        _check_input(beta, "beta")
+    if res is not None:
+        _check_input(res, "res")
+        if tuple(res.shape) != tuple(x.shape):
+            raise RuntimeError("res has wrong shape")
+    nbytes = ctypes.c_size_t(0)
+    L.check(_lib.mg_group_norm_scratch_bytes(B, int(groups), ctypes.byref(nbytes)))
+    with torch.cuda.device(x.device):
+        scratch = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=x.device)
+        out = torch.empty(tuple(x.shape), dtype=torch.float32, device=x.device)
+        L.check(_lib.mg_group_norm(int(mode), _p(x), xs, _p(mul), ms, B, N, chan, int(groups), comps, float(eps),
+                                   _p(gamma), _p(beta), _p(add), as_, _p(res), _p(scratch), _p(out), _stream()))
+    return out
+
+
+def tens_sigmoid(inds, x):
+    _check_input(x, "x")
+    T = 3 ** inds
+    with torch.cuda.device(x.device):
+        out = torch.empty_like(x)
+        L.check(_lib.mg_tens_sigmoid(int(inds), _p(x), int(x.numel()) // T, _p(out), _stream()))
+    return out
+
+
+def painn_update_pre(lrv, x_a):
+    """lrv (rows, 3n, 3), x_a (rows, n) -> ip (rows, n), cat (rows, 2n)."""
+    _check_input(lrv, "lrv")
+    _check_input(x_a, "x_a")
+    rows, n = int(x_a.shape[0]), int(x_a.shape[1])
+    if tuple(lrv.shape) != (rows, 3 * n, 3):
+        raise RuntimeError("lrv must have shape (rows, 3n, 3)")
+    with torch.cuda.device(x_a.device):
+        ip = torch.empty(rows, n, dtype=torch.float32, device=x_a.device)
+        cat = torch.empty(rows, 2 * n, dtype=torch.float32, device=x_a.device)
+        L.check(_lib.mg_painn_update_pre(_p(lrv), _p(x_a), rows, n, _p(ip), _p(cat), _stream()))
+    return ip, cat
+
+
+def painn_update_vec(lrv, y, res_v=None):
+    """v = lin_v(x_v) * y[:, :n]; returns res_v + v / sqrt(1 + |v|^2), shape (rows, n, 3)."""
+    _check_input(lrv, "lrv")
+    _check_input(y, "y")
+    rows, n = int(y.shape[0]), int(y.shape[1]) // 3
+    if tuple(lrv.shape) != (rows, 3 * n, 3):
+        raise RuntimeError("lrv must have shape (rows, 3n, 3)")
+    if res_v is not None:
+        _check_input(res_v, "res_v")
+    with torch.cuda.device(y.device):
+        out = torch.empty(rows, n, 3, dtype=torch.float32, device=y.device)
+        L.check(_lib.mg_painn_update_vec(_p(lrv), _p(y), _p(res_v), rows, n, _p(out), _stream()))
+    return out
+
+
+RADIAL_SQ, RADIAL_EDGE = 1, 2
+
+
+def radial_encode(kind, r_ij, n, rmax):
+    """kind 1: sq_radial_encode(normed_sq_dist(r, rmax), n); kind 2: radial_encode_edge(r, n, rmax)."""
+    _check_input(r_ij, "r_ij")
+    lead = tuple(r_ij.shape[:-1])
+    if r_ij.shape[-1] != 3:
+        raise RuntimeError("r_ij must have a last dimension of 3")
+    E = 1
+    for d in lead:
+        E *= int(d)
+    with torch.cuda.device(r_ij.device):
+        out = torch.empty(lead + (n,), dtype=torch.float32, device=r_ij.device)
+        L.check(_lib.mg_radial_encode(int(kind), _p(r_ij), E, int(n), float(rmax), _p(out), _stream()))
+    return out

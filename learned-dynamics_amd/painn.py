@@ -66,14 +66,10 @@ class ScalGroupNorm(nn.Module):
         self.gamma = nn.Parameter(torch.ones(chan))
         self.beta = nn.Parameter(torch.zeros(chan))
 
-    def forward(self, x):
-        batch, nodes, chan = x.shape
-        x = x.reshape(batch, nodes, self.groups, -1)
-        mean = x.mean([1, 3], keepdim=True)
-        x_shift = x - mean
-        var = (x_shift ** 2).mean([1, 3], keepdim=True)
-        ans = x_shift / torch.sqrt(self.epsilon + var)
-        return self.beta + self.gamma * ans.reshape(batch, nodes, self.chan)
+    def forward(self, x, mul=None, add=None, res=None):
+        """beta + gamma * norm(x * mul) + add + res (the extra operands are optional fusions)."""
+        return ops.group_norm(ops.GN_SCALAR, x, self.groups, self.gamma, self.beta, self.epsilon, mul=mul, add=add,
+                              res=res)
 
 
 class Update(nn.Module):
@@ -89,18 +85,22 @@ class Update(nn.Module):
         assert n % 4 == 0
         self.gn = ScalGroupNorm(n, 4, epsilon=1.)
 
-    def forward(self, x_a, x_v):
+    def forward(self, x_a, x_v, residual=False):
+        """Returns (dx_a, dx_v), or (x_a + dx_a, x_v + dx_v) with residual=True."""
         n = self.n
-        W = torch.cat([self.lin_l.W, self.lin_r.W, self.lin_v.W], dim=0)        # (3n, n)
-        lrv = ops.tensor_linear_fwd(1, W, x_v.contiguous())                     # (B, N, 3n, 3)
-        x_v_l, x_v_r, x_v_v = lrv[..., :n, :], lrv[..., n:2 * n, :], lrv[..., 2 * n:, :]
-        inner_prod = (x_v_l * x_v_r).sum(-1)
-        y = self.mlp(torch.cat([x_a, torch.linalg.vector_norm(x_v_r, dim=-1)], dim=-1))
-        x_v = x_v_v * y[..., :n, None]
-        inner_prod = self.gn(inner_prod * y[..., n:2 * n])
-        x_a = inner_prod + y[..., 2 * n:]
-        x_v = x_v / torch.sqrt(1. + (x_v ** 2).sum(-1, keepdim=True))
-        return x_a, x_v
+        B, N = x_a.shape[:2]
+        rows = B * N
+        flat_a = x_a.reshape(rows, n).contiguous()
+        flat_v = x_v.reshape(rows, n, 3).contiguous()
+        W = torch.cat([self.lin_l.W, self.lin_r.W, self.lin_v.W], dim=0)        # (3n, n): one GEMM for l, r, v
+        lrv = ops.tensor_linear_fwd(1, W, flat_v)                               # (rows, 3n, 3)
+        ip, cat = ops.painn_update_pre(lrv, flat_a)                             # l.r and [x_a | |r|]
+        y = self.mlp(cat)                                                       # (rows, 3n)
+        y3 = y.reshape(B, N, 3 * n)
+        out_a = self.gn(ip.reshape(B, N, n), mul=y3[..., n:2 * n], add=y3[..., 2 * n:],
+                        res=flat_a.reshape(B, N, n) if residual else None)
+        out_v = ops.painn_update_vec(lrv, y, flat_v if residual else None)
+        return out_a, out_v.reshape(B, N, n, 3)
 
 
 class Message(nn.Module):
@@ -152,8 +152,7 @@ class Block(nn.Module):
         if graph_bond is not None:
             x_a, x_v = self.message_bond(graph_bond, x_a, x_v, r_ij_bond, residual=True)
         x_a, x_v = self.message(graph, x_a, x_v, r_ij, residual=True)
-        dx_a, dx_v = self.update(x_a, x_v)
-        x_a, x_v = x_a + dx_a, x_v + dx_v
+        x_a, x_v = self.update(x_a, x_v, residual=True)
         if self.pos_mutable:
             pos = pos + self.lin_push_pos(x_v).squeeze(-2)
             graph, r_ij = None, None

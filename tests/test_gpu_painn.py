@@ -134,3 +134,47 @@ def test_state_dict_names_match_reference():
                    "update.lin_l.W", "update.lin_r.W", "update.lin_v.W", "update.mlp.layers.0.weight",
                    "update.gn.gamma", "update.gn.beta"):
         assert expect in names, expect
+
+
+def test_norm_and_squash_kernels(ops):
+    """ScalGroupNorm / TensGroupNorm / tens_sigmoid kernels against the oracle, including channel-slice
+    operands and the fused multiplier / add / residual."""
+    torch.manual_seed(21)
+    B, N, chan = 3, 70, 16
+    y = torch.randn(B, N, 3 * chan)
+    ip, res = torch.randn(B, N, chan), torch.randn(B, N, chan)
+    gamma, beta = torch.randn(chan), torch.randn(chan)
+    yc = y.cuda()
+    out = ops.group_norm(ops.GN_SCALAR, ip.cuda(), 4, gamma.cuda(), beta.cuda(), 1.0, mul=yc[..., chan:2 * chan],
+                         add=yc[..., 2 * chan:], res=res.cuda())
+    ref = OL.scal_group_norm(ip * y[..., chan:2 * chan], 4, gamma, beta, 1.0) + y[..., 2 * chan:] + res
+    _close(out, ref, atol_scale=2e-6)
+    for inds in (0, 1, 2):
+        x = torch.randn(B, N, chan, *([3] * inds)) * 2 + 0.3
+        g = torch.randn(chan, *([1] * inds))
+        out = ops.group_norm(ops.GN_TENSOR, x.cuda(), 8, g.reshape(-1).cuda(), None, 1e-5)
+        _close(out, OL.tens_group_norm(inds, x, 8, g), atol_scale=2e-6)
+        _close(ops.tens_sigmoid(inds, x.cuda()), OL.tens_sigmoid(inds, x), atol_scale=1e-6)
+
+
+@pytest.mark.parametrize("kind", [1, 2])
+def test_other_radial_encodings(ops, kind):
+    """sq_radial_encode (archs/diffuser_atoms14.py:32-48) and radial_encode_edge (archs/diffuser_atoms5.py:25-30),
+    restated here in float64 as the check."""
+    g = torch.Generator().manual_seed(3)
+    r = torch.randn(3000, 3, generator=g) * 3
+    n, rmax = 12, 7.0
+    out = ops.radial_encode(kind, r.cuda(), n, rmax)
+    rd = r.double()
+    if kind == 1:
+        q = (rd ** 2).sum(-1, keepdim=True) / rmax ** 2
+        coeffs = (torch.pi * 2 ** -0.5) * torch.exp(n ** -0.7 * torch.arange(0, n).double())
+        h = torch.sqrt(1 + q)
+        ref = torch.sin(coeffs * h) * (0.5 ** 0.5 - h)
+        tol = 4 * float((coeffs.max() * h.max())) * 2.0 ** -24 + 2e-6
+    else:
+        npi = torch.pi * torch.arange(0, n).double()
+        x_sq = (rd ** 2).sum(-1) / rmax
+        ref = torch.cos(npi * torch.sqrt(x_sq)[..., None]) * torch.relu(1. - x_sq)[..., None]
+        tol = 4 * float(npi.max() * torch.sqrt(x_sq).max()) * 2.0 ** -24 + 2e-6
+    torch.testing.assert_close(out.cpu().double(), ref, rtol=1e-5, atol=tol)
