@@ -31,6 +31,16 @@ PEAK_FP32_MFMA_TFLOPS = 157.3  # MI355X dense fp32 matrix
 PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X dense bf16 matrix
 
 
+def measured_traffic(kernel):
+    """HBM bytes per launch from the committed rocprofv3 --pmc summary (None if absent)."""
+    path = os.path.join(ROOT, "profiles", "painn_layer_configs2_traffic.json")
+    try:
+        with open(path) as f:
+            return json.load(f).get(kernel, {}).get("traffic_bytes")
+    except (OSError, ValueError):
+        return None
+
+
 def parse():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -123,7 +133,8 @@ def bench_painn_layer(torch, args):
             # operands split into 3 bf16 pieces, 6 bf16 MFMAs per fp32 product, fp32 accumulate
             roofline = {"kernel": "linear_rows_bf16x3_pipelined_kernel (filter MLP layer, E x 512 x 512, bias+SiLU fused)",
                         "bound": "mfma", "achieved": 6 * flops / t_gemm / 1e12, "peak": PEAK_BF16_MFMA_TFLOPS,
-                        "unit": "TFLOP/s", "frac": 6 * flops / t_gemm / 1e12 / PEAK_BF16_MFMA_TFLOPS, "traffic": None,
+                        "unit": "TFLOP/s", "frac": 6 * flops / t_gemm / 1e12 / PEAK_BF16_MFMA_TFLOPS,
+                        "traffic": measured_traffic("linear_rows_bf16x3_pipelined_kernel"),
                         "note": "achieved counts the executed bf16 MFMA FLOPs (6 per fp32 multiply-add pair); "
                                 "fp32-equivalent rate and its ratio to the fp32 MFMA peak are given alongside",
                         "fp32_equivalent_tflops": flops / t_gemm / 1e12,
@@ -143,7 +154,8 @@ def bench_painn_layer(torch, args):
         edge_bytes = E * (16 * n + 4 + 12) + N * (16 * n + 16 * n)
         roofline_hbm = {"kernel": "painn_message_kernel (fused gather-product-scatter)", "bound": "hbm",
                         "achieved": edge_bytes / t_edge / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                        "frac": edge_bytes / t_edge / 1e9 / PEAK_HBM_GBS, "traffic": None,
+                        "frac": edge_bytes / t_edge / 1e9 / PEAK_HBM_GBS,
+                        "traffic": measured_traffic("painn_message_kernel"),
                         "bytes_per_launch": edge_bytes, "ms": t_edge * 1e3}
         t_graph = event_time(torch, lambda: gl.graph_setup(r0, box, pos_d, neighbours_max=512, celllist_max=128), 5)
         breakdown = {"filter_gemm_512x512_ms": t_gemm * 1e3, "edge_kernel_ms": t_edge * 1e3,

@@ -38,7 +38,8 @@ constexpr int lds_row_stride(int T) {
 }
 
 __device__ __forceinline__ float activate(float v, int act) {
-    if (act == 1) return v / (1.0f + expf(-v));       // SiLU
+    // SiLU with the hardware exp2 / reciprocal (about 1 ulp each): far inside the fp32 tolerance
+    if (act == 1) return v * __frcp_rn(1.0f + __expf(-v));
     if (act == 2) return v > 0.f ? v : 0.1f * v;      // LeakyReLU(0.1)
     return v;
 }
