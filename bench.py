@@ -47,7 +47,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="painn_layer",
-                    choices=["painn_layer", "neighbour", "products", "denoiser"])
+                    choices=["painn_layer", "neighbour", "products", "denoiser", "stress"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -313,6 +313,46 @@ def bench_denoiser(torch, args, with_cpu=True):
     return out
 
 
+def bench_stress(torch, args):
+    """BASELINE configs[4] geometry and layer stack in fp32 storage: 65536 atoms uniform in a periodic cube at
+    0.1 atoms/A^3, cutoff 6 A, 4 x [Messages + SelfTensProds] with 128 channels per rank, neighbour rebuild inside
+    the step.  (The bf16-storage variant of that config is not built; this is the fp32 path at its size.)"""
+    bee = importlib.import_module("learned-dynamics_amd.bee_layers")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    seed = 0x947 + 5
+    torch.manual_seed(seed)
+    N, r0, C, layers = 65536, 6.0, 128, 4
+    L = (N / 0.1) ** (1.0 / 3.0)
+    box = (L, L, L)
+    g = torch.Generator().manual_seed(seed)
+    pos = (torch.rand(1, N, 3, generator=g) * L).cuda()
+    x_a = torch.randn(1, N, C, generator=g).cuda()
+    x_v = (torch.randn(1, N, C, 3, generator=g) / 3 ** 0.5).cuda()
+    x_d = (torch.randn(1, N, C, 3, 3, generator=g) / 3.0).cuda()
+    msgs = [bee.Messages(r0, C, C, C, C).cuda().eval() for _ in range(layers)]
+    prods = [bee.SelfTensProds(C, C, C, C).cuda().eval() for _ in range(layers)]
+    edges = [0]
+
+    with torch.no_grad():
+        def step():
+            graph, r_ij = gl.graph_setup(r0, box, pos, neighbours_max=256, celllist_max=64)
+            edges[0] = int(graph.src.numel())
+            a, v, d = x_a, x_v, x_d
+            for m, p in zip(msgs, prods):
+                da, dv, dd = m(graph, r_ij, a, v, d)
+                a, v, d = a + da, v + dv, d + dd
+                a, v, d = p(a, v, d, residual=True)
+            return a
+        step()
+        sec = timed_steps(torch, step, args.steps, args.warmup)
+    E = edges[0]
+    return {"metric": "message-passing edges/sec per layer", "value": E * layers / sec, "unit": "edges/s",
+            "ms_per_step": sec * 1e3, "dtype": "f32",
+            "config": {"workload": "BASELINE configs[4] in fp32 storage: 65536 atoms, density 0.1/A^3, cutoff 6 A, "
+                                   "4 x [Messages + SelfTensProds], 128 channels per rank, neighbour rebuild in the step",
+                       "edges": E, "atoms": N, "layers": layers, "atoms_per_s": N / sec}}
+
+
 def cpu_denoiser_block(torch, model, x1, r0, box, dims):
     """Oracle (fp32 PyTorch CPU port of the reference math): ONE block (Messages + SelfTensProds) on ONE of the
     32 systems; the forward is 8 such blocks per system, so atoms/s = atoms / (8 * t_block)."""
@@ -391,6 +431,8 @@ def main():
         res = bench_neighbour(torch, args, with_cpu=not args.no_cpu)
     elif args.workload == "denoiser":
         res = bench_denoiser(torch, args, with_cpu=not args.no_cpu)
+    elif args.workload == "stress":
+        res = bench_stress(torch, args)
     else:
         res = bench_products(torch, args)
         res.setdefault("ms_per_step", res["detail"]["rows_4096"]["us"] * 1e-3)

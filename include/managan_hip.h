@@ -75,6 +75,14 @@ int mg_neighbour_fill(const void* workspace, size_t workspace_bytes, int batch, 
                       float cutoff, float box_x, float box_y, float box_z,
                       const int* row_ptr, int n_edges, int* src, int* dst, mg_stream_t stream);
 
+/* After mg_neighbour_count on the same workspace: order[k] = global id (b*nodes + i) of the k-th atom in
+ * cell order (boxes, then cells x-major, then atom id).  Processing the rows of the fused edge kernels
+ * in this order keeps the gathered neighbours of consecutive rows close together in time (cache
+ * locality) when atom ids carry no spatial meaning.  No counterpart in the reference. */
+int mg_neighbour_cell_order(const void* workspace, size_t workspace_bytes, int batch, int nodes,
+                            float cutoff, float box_x, float box_y, float box_z,
+                            int* order /* batch*nodes */, mg_stream_t stream);
+
 /* First step of the search on its own: wrapped positions (batch,nodes,3) and box-local
  * linear cell ids (batch,nodes), as assignParticlesToCells computes them
  * (extensions/neighbour_grid/neighbour_grid_kern.cu:75-82).  Diagnostic / test entry. */

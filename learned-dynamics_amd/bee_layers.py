@@ -148,9 +148,13 @@ class Messages(nn.Module):
         W = torch.cat([getattr(self, f"Y_{lab}").W for lab in labels], dim=1)
         return W if scale is None else W * scale
 
-    def forward(self, graph: Graph, r_ij, x_a, x_v, x_d, node_order=None):
+    def forward(self, graph: Graph, r_ij, x_a, x_v, x_d, node_order="cell"):
         """x_a (batch, nodes, dim_a), x_v (..., dim_v, 3), x_d (..., dim_d, 3, 3), r_ij (edges, 3).
-        Returns 0.1 * sum over edges of the messages: (B_a, B_v, B_d) with the input shapes."""
+        Returns 0.1 * sum over edges of the messages: (B_a, B_v, B_d) with the input shapes.
+        node_order: row processing order of the edge kernel ("cell": the graph's cell order when it has
+        one, None: index order, or an int32 tensor); it does not change the results."""
+        if isinstance(node_order, str):
+            node_order = getattr(graph, "cell_order", None)
         B, N = x_a.shape[:2]
         rows = B * N
         C = ops.LAYOUT_COMP_CHAN

@@ -457,6 +457,14 @@ __global__ void __launch_bounds__(256) pairs_kernel(Grid g, Workspace w, const i
     }
 }
 
+// order[k] = global id of the k-th atom in cell order (cells x-major, atoms by id inside a cell)
+__global__ void __launch_bounds__(256) cell_order_kernel(Grid g, Workspace w, int* __restrict__ order) {
+    const long A = (long)g.batch * g.nodes;
+    const long k = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= A) return;
+    order[k] = (int)(k / g.nodes) * g.nodes + __float_as_int(w.sorted[k].w);
+}
+
 __global__ void __launch_bounds__(256) wrap_cells_kernel(const float* __restrict__ x, Grid g,
                                                          float* __restrict__ wrapped, int* __restrict__ cell) {
     const long A = (long)g.batch * g.nodes;
@@ -646,6 +654,23 @@ int mg_neighbour_fill(const void* workspace, size_t workspace_bytes, int batch, 
         hipLaunchKernelGGL((pairs_kernel<true, kCandCapDense>), dim3((unsigned)C), dim3(256), 0, (hipStream_t)stream,
                            g, w, row_ptr, src, dst);
     return check_launch("mg_neighbour_fill");
+}
+
+int mg_neighbour_cell_order(const void* workspace, size_t workspace_bytes, int batch, int nodes, float cutoff,
+                            float box_x, float box_y, float box_z, int* order, mg_stream_t stream) {
+    Grid g;
+    if (int s = make_grid(cutoff, box_x, box_y, box_z, batch, nodes, &g)) return s;
+    const long A = (long)batch * nodes, C = (long)batch * g.ncells;
+    if (A == 0) return MG_OK;
+    MG_REQUIRE(workspace && order, "mg_neighbour_cell_order: null pointer");
+    void* base = reinterpret_cast<void*>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~uintptr_t(255));
+    Workspace w = carve(base, A, C, mask_words(g));
+    if (w.bytes + 256 > workspace_bytes)
+        return fail(MG_ERR_WORKSPACE, "mg_neighbour_cell_order: workspace has %zu bytes, %zu needed", workspace_bytes,
+                    w.bytes + 256);
+    hipLaunchKernelGGL(cell_order_kernel, dim3((unsigned)ceil_div(A, 256)), dim3(256), 0, (hipStream_t)stream, g, w,
+                       order);
+    return check_launch("mg_neighbour_cell_order");
 }
 
 int mg_neighbour_wrap_cells(const float* x, int batch, int nodes, float cutoff, float box_x, float box_y,

@@ -50,7 +50,7 @@ class Denoiser(nn.Module):
         self.prods = nn.ModuleList([SelfTensProds(dim_a, dim_v, dim_d, chan) for _ in range(blocks)])
         self.readout = TensLinear(1, dim_v, 1)
 
-    def forward(self, st, x0, x1, one_hot, box, neighbours_max=256, celllist_max=64, node_order=None):
+    def forward(self, st, x0, x1, one_hot, box, neighbours_max=256, celllist_max=64, node_order="cell"):
         """st: ((batch), (batch)); x0, x1: (batch, atoms, 3); one_hot: (batch, atoms, types)."""
         s, t = st
         B, N = x1.shape[:2]

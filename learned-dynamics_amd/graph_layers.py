@@ -17,7 +17,7 @@ class Graph:
     and index into a dimension of size batch*nodes.  src must be non-decreasing.
     (managan/graph_layers.py:9-24)"""
 
-    def __init__(self, src, dst, edge_indices, batch, nodes, row_ptr=None):
+    def __init__(self, src, dst, edge_indices, batch, nodes, row_ptr=None, cell_order=None):
         self.src32 = src.to(torch.int32).contiguous()
         self.dst32 = dst.to(torch.int32).contiguous()
         self.src = src.to(torch.int64)
@@ -26,6 +26,7 @@ class Graph:
         self.batch = batch
         self.nodes = nodes
         self._row_ptr = row_ptr
+        self.cell_order = cell_order   # int32 atom ids in cell order, or None (radius graphs only)
 
     @property
     def row_ptr(self):
@@ -41,9 +42,9 @@ class Graph:
         batch, nodes, three = pos.shape
         assert three == 3
         assert torch.all(~torch.isnan(pos)), "some positions are NaN!"
-        src, dst, edge_indices, row_ptr = ops.get_edges(celllist_max, neighbours_max, r0, *box, pos,
-                                                        return_row_ptr=True)
-        ans = Graph(src, dst, edge_indices, batch, nodes, row_ptr=row_ptr)
+        src, dst, edge_indices, row_ptr, order = ops.get_edges(celllist_max, neighbours_max, r0, *box, pos,
+                                                               return_row_ptr=True, return_order=True)
+        ans = Graph(src, dst, edge_indices, batch, nodes, row_ptr=row_ptr, cell_order=order)
         setattr(ans, "box", box)
         return ans
 

@@ -82,6 +82,16 @@ class NeighbourSearch:
         return src, dst
 
 
+    def cell_order(self):
+        """int32 (batch*nodes): atom ids in cell order (a cache-friendly row order for the edge kernels)."""
+        dev = self.x.device
+        with torch.cuda.device(dev):
+            order = torch.empty(self.batch * self.nodes, dtype=torch.int32, device=dev)
+            L.check(_lib.mg_neighbour_cell_order(_p(self.workspace), self.workspace.numel(), self.batch, self.nodes,
+                                                 self.cutoff, *self.box, _p(order), _stream()))
+        return order
+
+
 def _check_caps(search, listmax, neighboursmax):
     """The reference's overflow errors, in the reference's order
     (extensions/neighbour_grid/neighbour_grid_kern.cu:195-217)."""
@@ -94,14 +104,17 @@ def _check_caps(search, listmax, neighboursmax):
         raise RuntimeError("Neighbour list overflow occurred. Try increasing neighboursmax.")
 
 
-def get_edges(listmax, neighboursmax, cutoff, box_x, box_y, box_z, x, return_row_ptr=False):
+def get_edges(listmax, neighboursmax, cutoff, box_x, box_y, box_z, x, return_row_ptr=False, return_order=False):
     """(src int32[E], dst int32[E], edgeCounts int32[B]); extensions/neighbour_grid/neighbour_grid.cpp:170-195."""
     search = NeighbourSearch(x, cutoff, (box_x, box_y, box_z))
     _check_caps(search, listmax, neighboursmax)
     src, dst = search.fill()
+    out = (src, dst, search.edge_counts)
     if return_row_ptr:
-        return src, dst, search.edge_counts, search.row_ptr
-    return src, dst, search.edge_counts
+        out = out + (search.row_ptr,)
+    if return_order:
+        out = out + (search.cell_order(),)
+    return out
 
 
 def get_neighbours(listmax, neighboursmax, cutoff, box_x, box_y, box_z, x):

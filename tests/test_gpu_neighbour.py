@@ -168,3 +168,18 @@ def test_padded_api(ops):
     ones = torch.ones(20, 60, 7, device="cuda")
     red = ops.padded_edges_reduce(counts, neighbours, ops.padded_edges_read(counts, neighbours, ones))
     assert torch.equal(red[:, :, 0], counts.float())
+
+
+def test_cell_order_is_a_permutation_sorted_by_cell(ops):
+    rng = np.random.default_rng(23)
+    box = (30., 30., 30.)
+    x = (rng.random((3, 2000, 3)) * 30).astype(np.float32)
+    search = ops.NeighbourSearch(torch.from_numpy(x).cuda(), 5.0, box)
+    order = search.cell_order().cpu().numpy()
+    assert np.array_equal(np.sort(order), np.arange(6000))
+    _, cell = ON.wrap_cells(x, 5.0, box)
+    flat_cell = cell.reshape(-1) + (np.arange(6000) // 2000) * 216          # 6^3 cells per box
+    keys = flat_cell[order]
+    assert np.all(np.diff(keys) >= 0)
+    same = np.diff(keys) == 0
+    assert np.all(np.diff(order)[same] > 0)                                   # atom id ascending inside a cell
