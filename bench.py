@@ -131,10 +131,10 @@ def bench_painn_layer(torch, args):
         split = ops.get_linear_mode() == ops.LINEAR_BF16X3
         if split:
             # operands split into 3 bf16 pieces, 6 bf16 MFMAs per fp32 product, fp32 accumulate
-            roofline = {"kernel": "linear_rows_bf16x3_pipelined_kernel (filter MLP layer, E x 512 x 512, bias+SiLU fused)",
+            roofline = {"kernel": "linear_rows_bf16x3_wide_kernel (filter MLP layer, E x 512 x 512, bias+SiLU fused)",
                         "bound": "mfma", "achieved": 6 * flops / t_gemm / 1e12, "peak": PEAK_BF16_MFMA_TFLOPS,
                         "unit": "TFLOP/s", "frac": 6 * flops / t_gemm / 1e12 / PEAK_BF16_MFMA_TFLOPS,
-                        "traffic": measured_traffic("linear_rows_bf16x3_pipelined_kernel"),
+                        "traffic": measured_traffic("linear_rows_bf16x3_wide_kernel"),
                         "note": "achieved counts the executed bf16 MFMA FLOPs (6 per fp32 multiply-add pair); "
                                 "fp32-equivalent rate and its ratio to the fp32 MFMA peak are given alongside",
                         "fp32_equivalent_tflops": flops / t_gemm / 1e12,

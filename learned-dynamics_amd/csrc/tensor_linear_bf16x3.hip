@@ -410,6 +410,174 @@ linear_rows_bf16x3_pipelined_kernel(const __bf16* __restrict__ Wp, const float* 
     else epilogue(std::false_type{});
 }
 
+
+// ---------------------------------------------------------------------------
+// Wide variant: 256x256 tile per workgroup, 8 waves (4x2) of 64x128, same K slab
+// and double buffering.  Per MFMA it needs 3/4 of the LDS reads and half of the
+// split/stage work and barriers of the 128x128 kernel; LDS 2 x 72 KB -> one
+// workgroup (two waves per SIMD) per CU.  Requires dim_out % 256 == 0.
+constexpr int kPlaneQ = 256 * kRowP;
+constexpr int kBufQ = 6 * kPlaneQ;
+
+__global__ void __launch_bounds__(512)
+linear_rows_bf16x3_wide_kernel(const __bf16* __restrict__ Wp, const float* __restrict__ X, long R, int I, int O,
+                               const float* __restrict__ bias, int act, int accumulate, float* __restrict__ Y,
+                               int tiles_n, long tiles_total, int out_T) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kBufQ];
+
+    const long bid = blockIdx.x;
+    const long per_xcd = (tiles_total + 7) / 8;
+    const long logical = (bid % 8) * per_xcd + bid / 8;
+    if (logical >= tiles_total) return;
+    const long tile_m = logical / tiles_n;
+    const int tile_n = (int)(logical - tile_m * tiles_n);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+    const long r0 = tile_m * 256;
+    const int n0 = tile_n * 256;
+    const int kgroup = lane >> 5;
+    const long plane_elems = (long)O * I;      // O is a multiple of 256 here
+
+    floatx16 acc[2][4];
+#pragma unroll
+    for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+        for (int ni = 0; ni < 4; ni++)
+#pragma unroll
+            for (int q = 0; q < 16; q++) acc[mi][ni][q] = 0.f;
+
+    // x tile of a slab: 256 rows x 16 floats = 1024 float4: thread -> rows (tid>>2) and (tid>>2)+128, k = (tid&3)*4
+    const int xr = tid >> 2, xc = (tid & 3) * 4;
+    // W tile: 3 planes x 256 rows x 32 B = 1536 pieces of 16 B: thread -> row (tid>>1), half (tid&1), every plane
+    const int wr = tid >> 1, wc = (tid & 1) * 8;
+    const int k_last = I - kBKp;
+
+    auto load_stage = [&](StageRegs& g, int k0) {
+        k0 = k0 < I ? k0 : k_last;
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const long r = r0 + xr + 128 * h;
+            g.x[h] = r < R ? *reinterpret_cast<const float4*>(X + r * I + k0 + xc) : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int p = 0; p < 3; p++)
+            g.w[p] = *reinterpret_cast<const bf16x8*>(Wp + p * plane_elems + (long)(n0 + wr) * I + k0 + wc);
+    };
+    auto store_stage = [&](const StageRegs& g, unsigned char* buf) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const Split4 sx = split(g.x[h]);
+            const int off = (xr + 128 * h) * kRowP + xc * 2;
+            *reinterpret_cast<bf16x4*>(buf + off) = sx.hi;
+            *reinterpret_cast<bf16x4*>(buf + kPlaneQ + off) = sx.mid;
+            *reinterpret_cast<bf16x4*>(buf + 2 * kPlaneQ + off) = sx.lo;
+        }
+#pragma unroll
+        for (int p = 0; p < 3; p++)
+            *reinterpret_cast<bf16x8*>(buf + (3 + p) * kPlaneQ + wr * kRowP + wc * 2) = g.w[p];
+    };
+
+    int a_off[2], b_off[4];
+#pragma unroll
+    for (int i = 0; i < 2; i++) a_off[i] = ((wave_m * 2 + i) * 32 + (lane & 31)) * kRowP + kgroup * 16;
+#pragma unroll
+    for (int i = 0; i < 4; i++) b_off[i] = 3 * kPlaneQ + ((wave_n * 4 + i) * 32 + (lane & 31)) * kRowP + kgroup * 16;
+
+    auto compute = [&](const unsigned char* buf) {
+        bf16x8 a[2][3];
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int p = 0; p < 3; p++) a[i][p] = *reinterpret_cast<const bf16x8*>(buf + p * kPlaneQ + a_off[i]);
+#pragma unroll
+        for (int nh = 0; nh < 2; nh++) {
+            bf16x8 b[2][3];
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int p = 0; p < 3; p++)
+                    b[i][p] = *reinterpret_cast<const bf16x8*>(buf + p * kPlaneQ + b_off[nh * 2 + i]);
+#pragma unroll
+            for (int t = 0; t < 6; t++) {
+                constexpr int pa[6] = {2, 0, 1, 1, 0, 0};   // lo*hi, hi*lo, mid*mid, mid*hi, hi*mid, hi*hi
+                constexpr int pb[6] = {0, 2, 1, 0, 1, 0};
+#pragma unroll
+                for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+                    for (int nj = 0; nj < 2; nj++)
+                        acc[mi][nh * 2 + nj] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mi][pa[t]], b[nj][pb[t]],
+                                                                                       acc[mi][nh * 2 + nj], 0, 0, 0);
+            }
+        }
+    };
+
+    unsigned char* buf0 = lds;
+    unsigned char* buf1 = lds + kBufQ;
+    // Waves w and w+4 share a SIMD.  The upper four stage the next slab before their
+    // MFMAs, the lower four after: while one wave of a SIMD splits and stores, the
+    // other keeps the matrix pipe busy.
+    const bool store_first = __builtin_amdgcn_readfirstlane(wave) >= 4;
+    StageRegs ga, gb;
+    load_stage(ga, 0);
+    load_stage(gb, kBKp);
+    store_stage(ga, buf0);
+    load_stage(ga, 2 * kBKp);
+    for (int k0 = 0; k0 < I; k0 += 2 * kBKp) {
+        __syncthreads();
+        if (store_first) {
+            store_stage(gb, buf1);
+            load_stage(gb, k0 + 3 * kBKp);
+        }
+        compute(buf0);
+        if (!store_first) {
+            store_stage(gb, buf1);
+            load_stage(gb, k0 + 3 * kBKp);
+        }
+        __syncthreads();
+        if (store_first) {
+            store_stage(ga, buf0);
+            load_stage(ga, k0 + 4 * kBKp);
+        }
+        compute(buf1);
+        if (!store_first) {
+            store_stage(ga, buf0);
+            load_stage(ga, k0 + 4 * kBKp);
+        }
+    }
+
+    auto epilogue = [&](auto plain) {
+        constexpr bool kPlain = decltype(plain)::value;
+#pragma unroll
+        for (int ni = 0; ni < 4; ni++) {
+            const int n = n0 + (wave_n * 4 + ni) * 32 + (lane & 31);
+            const float bv = bias ? bias[n] : 0.f;
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++) {
+#pragma unroll
+                for (int q = 0; q < 16; q++) {
+                    const long r = r0 + (wave_m * 2 + mi) * 32 + 8 * (q / 4) + 4 * kgroup + (q % 4);
+                    if (r < R) {
+                        long addr;
+                        if constexpr (kPlain) {
+                            addr = r * O + n;
+                        } else {
+                            const long row = r / out_T;
+                            addr = (row * O + n) * out_T + (r - row * out_T);
+                        }
+                        float v = activate(acc[mi][ni][q] + bv, act);
+                        if (accumulate) v += Y[addr];
+                        Y[addr] = v;
+                    }
+                }
+            }
+        }
+    };
+    if (out_T == 1) epilogue(std::true_type{});
+    else epilogue(std::false_type{});
+}
+
 }  // namespace
 
 // requires: dim_in % 32 == 0, x and W 16-byte aligned, W rows contiguous (stride_i == 1), so % 4 == 0
@@ -441,6 +609,17 @@ int pack_weight(const float* W, long so, long si, int I, int O, void* packed, hi
 
 int launch_rows_bf16x3_packed(const void* packed, const float* X, long R, int I, int O, const float* bias, int act,
                               int accumulate, float* Y, hipStream_t st, int out_T) {
+    if (O % 256 == 0 && ceil_div(R, 256) * (O / 256) >= 1024) {
+        const long tiles_m = ceil_div(R, 256);
+        const int tiles_n = O / 256;
+        const long total = tiles_m * tiles_n;
+        const long grid = ceil_div(total, 8) * 8;
+        MG_REQUIRE(grid <= 0x7fffffffL, "mg_tensor_linear_packed: grid too large (rows=%ld dim_out=%d)", R, O);
+        hipLaunchKernelGGL(linear_rows_bf16x3_wide_kernel, dim3((unsigned)grid), dim3(512), 0, st,
+                           static_cast<const __bf16*>(packed), X, R, I, O, bias, act, accumulate, Y, tiles_n, total,
+                           out_T);
+        return check_launch("mg_tensor_linear_packed");
+    }
     const long tiles_m = ceil_div(R, 128);
     const int tiles_n = (int)ceil_div(O, 128);
     const long total = tiles_m * tiles_n;

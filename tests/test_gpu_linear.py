@@ -89,7 +89,9 @@ def test_tensor_linear_autograd(pkg, inds):
 
 @pytest.mark.parametrize("mode", [0, 1])
 @pytest.mark.parametrize("shape", [(5000, 512, 512, 0), (3000, 96, 200, 0), (2000, 64, 128, 1), (1500, 160, 72, 2),
-                                   (1024, 64, 64, 0), (4096, 768, 256, 0)])
+                                   (1024, 64, 64, 0), (4096, 768, 256, 0),
+                                   # large enough for the 256x256-tile kernel (ragged last tile; transposed output)
+                                   (140001, 64, 512, 0), (90001, 32, 256, 1)])
 def test_linear_modes_agree_with_float64(ops, mode, shape):
     """fp32 MFMA (mode 0) and bf16x3-split MFMA (mode 1) against a float64 product: both must sit at
     fp32 rounding level; the split path uses pre-packed weights and may transpose (row, comp) outputs."""
