@@ -220,6 +220,13 @@ int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows,
  * [cos(k_m d)]_{m<hn} | [sin(k_m d)]_{m<n-hn}, k_m = (pi/rmax)(1 + m/2), hn = (n+1)/2, d = |r|. */
 int mg_painn_radial_encode(const float* r_ij /* (E,3) */, long n_edges, int n, float rmax,
                            float* out /* (E,n) */, mg_stream_t stream);
+/* First layer of Message.mlp_dist applied to the encoding without materialising it
+ * (archs/meanflow_painn8.py:25-35 feeding :38-51 at :92):
+ *   y[e,o] = act(bias[o] + sum_m W[o,m] radial_encode(r_ij[e], n, rmax)[m]),  y (E,dim_out).
+ * n <= 32; dim_out = 4 * 2^k <= 1024.  act as in mg_tensor_linear_layout. */
+int mg_painn_radial_linear(const float* r_ij /* (E,3) */, long n_edges, int n, float rmax, const float* W,
+                           long w_stride_o, long w_stride_i, const float* bias, int dim_out, int act,
+                           float* y, mg_stream_t stream);
 /* Message.forward after the two MLPs (archs/meanflow_painn8.py:91-100), fused over CSR rows:
  *   P = filt[e] * actv[dst[e]];  u = r_ij[e] / sqrt(epsilon + |r_ij[e]|^2);  v = x_v[dst[e]]
  *   out_v[i] = res_v[i] + sum_{e in row i} v*P[0:n] + (v x u)*P[n:2n] + u (x) P[2n:3n]

@@ -18,6 +18,13 @@
 namespace mg {
 namespace {
 
+__device__ __forceinline__ float activate_fast(float v, int act) {
+    // SiLU with the hardware exp2 / reciprocal (about 1 ulp each), as in the GEMM epilogues
+    if (act == 1) return v * __frcp_rn(1.0f + __expf(-v));
+    if (act == 2) return v > 0.f ? v : 0.1f * v;
+    return v;
+}
+
 constexpr int kMaxChunks = 16;
 struct Chunks {
     int n;
@@ -222,6 +229,78 @@ __global__ void __launch_bounds__(256) radial_encode_painn_kernel(const float* _
     }
 }
 
+// First layer of the radial MLP fused with the encoding:
+//   y[e, o] = act(b[o] + sum_m W[o, m] * enc[e, m]),  enc = radial_encode(r_ij[e])  (N_ENC >= n columns, zero padded)
+// The layer has K = n <= 32 and dim_out in the hundreds, so it is bound by writing y: a GEMM tile
+// machine buys nothing.  A workgroup takes 64 edges: their encodings go to LDS (one cos/sin per
+// entry), then every lane keeps the weights of four consecutive output channels in registers and
+// walks the 64 rows: the encoding row is an LDS broadcast, the output one 16-byte store per lane
+// (a wave writes 1 KB contiguous).
+template <int N_ENC>
+__global__ void __launch_bounds__(256) painn_radial_linear_kernel(const float* __restrict__ r_ij, long E, int n,
+                                                                  float base, const float* __restrict__ W, long so,
+                                                                  long si, const float* __restrict__ bias, int O,
+                                                                  int act, float* __restrict__ Y) {
+    constexpr int kRows = 64;
+    __shared__ __attribute__((aligned(16))) float enc[kRows * N_ENC];
+    const int tid = threadIdx.x;
+    const int groups = O / 4;               // lanes per output row; divides 256
+    const int g = tid % groups, sub = tid / groups;
+    const int rows_per_pass = 256 / groups;
+    const int hn = (n + 1) / 2;
+
+    float w[4][N_ENC], b[4];
+#pragma unroll
+    for (int c = 0; c < 4; c++) {
+        b[c] = bias ? bias[4 * g + c] : 0.f;
+#pragma unroll
+        for (int m = 0; m < N_ENC; m++) w[c][m] = m < n ? W[(long)(4 * g + c) * so + (long)m * si] : 0.f;
+    }
+
+    const long tiles = (E + kRows - 1) / kRows;
+    for (long tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+        const long e0 = tile * kRows;
+        __syncthreads();                    // the previous tile's rows are consumed
+#pragma unroll
+        for (int i = 0; i < kRows * N_ENC / 256; i++) {
+            const int idx = tid + 256 * i;
+            const int row = idx / N_ENC, m = idx % N_ENC;
+            const long e = e0 + row;
+            float v = 0.f;
+            if (e < E && m < n) {
+                const float x = r_ij[3 * e], y = r_ij[3 * e + 1], z = r_ij[3 * e + 2];
+                const float d = sqrtf(x * x + y * y + z * z);
+                const int f = m < hn ? m : m - hn;
+                const float phase = (base * (float)(1 + f / 2)) * d;
+                v = m < hn ? cosf(phase) : sinf(phase);
+            }
+            enc[idx] = v;
+        }
+        __syncthreads();
+        for (int row = sub; row < kRows; row += rows_per_pass) {
+            const long e = e0 + row;
+            if (e >= E) break;
+            float acc[4] = {b[0], b[1], b[2], b[3]};
+#pragma unroll
+            for (int m4 = 0; m4 < N_ENC / 4; m4++) {
+                const float4 ev = *reinterpret_cast<const float4*>(enc + row * N_ENC + 4 * m4);
+                const float evs[4] = {ev.x, ev.y, ev.z, ev.w};
+#pragma unroll
+                for (int k = 0; k < 4; k++)
+#pragma unroll
+                    for (int c = 0; c < 4; c++) acc[c] = fmaf(w[c][4 * m4 + k], evs[k], acc[c]);
+            }
+            typedef float floatx4 __attribute__((ext_vector_type(4)));
+            floatx4 out;
+            out.x = activate_fast(acc[0], act);
+            out.y = activate_fast(acc[1], act);
+            out.z = activate_fast(acc[2], act);
+            out.w = activate_fast(acc[3], act);
+            __builtin_nontemporal_store(out, reinterpret_cast<floatx4*>(Y + e * O + 4 * g));
+        }
+    }
+}
+
 }  // namespace
 }  // namespace mg
 
@@ -241,6 +320,29 @@ int mg_painn_radial_encode(const float* r_ij, long n_edges, int n, float rmax, f
     hipLaunchKernelGGL(radial_encode_painn_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, r_ij,
                        n_edges, n, base, out);
     return check_launch("mg_painn_radial_encode");
+}
+
+int mg_painn_radial_linear(const float* r_ij, long n_edges, int n, float rmax, const float* W, long w_stride_o,
+                           long w_stride_i, const float* bias, int dim_out, int act, float* y, mg_stream_t stream) {
+    MG_REQUIRE(n_edges >= 0 && n >= 0 && dim_out >= 0, "mg_painn_radial_linear: negative size");
+    MG_REQUIRE(rmax > 0.f, "mg_painn_radial_linear: rmax must be positive");
+    MG_REQUIRE(act >= 0 && act <= 2, "mg_painn_radial_linear: unknown activation %d", act);
+    MG_REQUIRE(n <= 32, "mg_painn_radial_linear: at most 32 radial functions (got %d)", n);
+    const int groups = dim_out / 4;
+    MG_REQUIRE(dim_out % 4 == 0 && groups >= 1 && groups <= 256 && 256 % groups == 0,
+               "mg_painn_radial_linear: dim_out must be 4 * a power of two, at most 1024 (got %d)", dim_out);
+    if (n_edges == 0) return MG_OK;
+    MG_REQUIRE(r_ij && W && y && aligned16(y), "mg_painn_radial_linear: null or unaligned pointer");
+    const float base = (float)(3.14159265358979323846 / (double)rmax);
+    long blocks = ceil_div(n_edges, 64);
+    if (blocks > 256L * 8) blocks = 256L * 8;
+    if (n <= 16)
+        hipLaunchKernelGGL(painn_radial_linear_kernel<16>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                           r_ij, n_edges, n, base, W, w_stride_o, w_stride_i, bias, dim_out, act, y);
+    else
+        hipLaunchKernelGGL(painn_radial_linear_kernel<32>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                           r_ij, n_edges, n, base, W, w_stride_o, w_stride_i, bias, dim_out, act, y);
+    return check_launch("mg_painn_radial_linear");
 }
 
 int mg_painn_message(const int* row_ptr, const int* dst, int n_nodes, long n_edges, const float* r_ij,

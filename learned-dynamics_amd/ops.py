@@ -541,6 +541,33 @@ def painn_radial_encode(r_ij, n, rmax):
     return out
 
 
+def painn_radial_linear_supported(n, dim_out):
+    """Shapes the fused encode + first-layer kernel takes."""
+    g = dim_out // 4
+    return n <= 32 and dim_out % 4 == 0 and 1 <= g <= 256 and 256 % g == 0
+
+
+def painn_radial_linear(r_ij, n, rmax, W, bias=None, act=ACT_NONE):
+    """act(bias + radial_encode(r_ij, n, rmax) @ W.T) without writing the encoding
+    (archs/meanflow_painn8.py:25-35 into the first layer of mlp_dist, :38-51)."""
+    _check_input(r_ij, "r_ij")
+    if r_ij.dim() != 2 or r_ij.size(1) != 3:
+        raise RuntimeError("r_ij must have shape (edges, 3)")
+    if W.dim() != 2 or W.size(1) != n:
+        raise RuntimeError("W must have shape (dim_out, n)")
+    if W.dtype != torch.float32 or not W.is_cuda:
+        raise RuntimeError("W must be a float32 CUDA tensor")
+    if bias is not None and (bias.dtype != torch.float32 or not bias.is_cuda or not bias.is_contiguous()
+                             or bias.numel() != W.size(0)):
+        raise RuntimeError("bias must be a contiguous float32 CUDA tensor of dim_out elements")
+    E, O = int(r_ij.size(0)), int(W.size(0))
+    with torch.cuda.device(r_ij.device):
+        y = torch.empty(E, O, dtype=torch.float32, device=r_ij.device)
+        L.check(_lib.mg_painn_radial_linear(_p(r_ij), E, int(n), float(rmax), _p(W), W.stride(0), W.stride(1),
+                                            _p(bias) if bias is not None else None, O, int(act), _p(y), _stream()))
+    return y
+
+
 def painn_message(row_ptr, dst, r_ij, filt, actv, x_v, epsilon, res_a=None, res_v=None):
     """Fused gather-product-scatter of the PaiNN message (archs/meanflow_painn8.py:91-100).
     filt (E,4n), actv (nodes,4n), x_v (nodes,n,3) -> out_a (nodes,n), out_v (nodes,n,3)."""

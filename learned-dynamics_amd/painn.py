@@ -50,9 +50,12 @@ class MLP(nn.Module):
         lead = x_a.shape[:-1]
         h = x_a.reshape(-1, x_a.shape[-1]).contiguous()
         h = _linear(h, self.layers[0], ops.ACT_SILU)
+        return self.after_first(h).reshape(*lead, -1)
+
+    def after_first(self, h):
+        """Layers 2 and 3 on the (rows, dim_out) output of the first layer + SiLU."""
         h = _linear(h, self.layers[2], ops.ACT_SILU)
-        h = _linear(h, self.layers[4], ops.ACT_NONE)
-        return h.reshape(*lead, h.shape[-1])
+        return _linear(h, self.layers[4], ops.ACT_NONE)
 
 
 class ScalGroupNorm(nn.Module):
@@ -117,6 +120,10 @@ class Message(nn.Module):
 
     def filters(self, r_ij):
         """(edges, 3) -> (edges, 4n): the per-edge filter, the one large per-edge tensor."""
+        first = self.mlp_dist.layers[0]
+        if ops.painn_radial_linear_supported(self.n_rbf, first.out_features):
+            h = ops.painn_radial_linear(r_ij, self.n_rbf, self.r0, first.weight, first.bias, ops.ACT_SILU)
+            return self.mlp_dist.after_first(h)
         return self.mlp_dist(ops.painn_radial_encode(r_ij, self.n_rbf, self.r0))
 
     def forward(self, graph: Graph, x_a, x_v, r_ij, residual=False):

@@ -47,6 +47,41 @@ def test_radial_encode(ops, n):
     torch.testing.assert_close(out.cpu(), ref, rtol=1e-5, atol=1e-6 + 4 * max_phase * 2.0 ** -24)
 
 
+@pytest.mark.parametrize("n,dim_out,act", [(16, 512, 1), (15, 64, 1), (7, 1024, 0), (32, 128, 2), (20, 4, 1)])
+def test_radial_linear_fused(ops, n, dim_out, act):
+    """Encoding + first linear layer in one kernel against the oracle's encoding followed by a
+    float64 product (K <= 32: the summation order cannot matter beyond a few ulp)."""
+    g = torch.Generator().manual_seed(n * 1000 + dim_out)
+    E = 4999                                           # ragged last tile of 64 rows
+    r = torch.randn(E, 3, generator=g) * 3
+    W = torch.randn(dim_out, n, generator=g) / n ** 0.5
+    b = torch.randn(dim_out, generator=g)
+    enc = OL.radial_encode_painn(r, n, 8.0).double()
+    pre = enc @ W.double().t() + b.double()
+    ref = {0: pre, 1: torch.nn.functional.silu(pre), 2: torch.where(pre > 0, pre, 0.1 * pre)}[act].float()
+    max_phase = (torch.pi / 8.0) * (1 + ((n + 1) // 2 - 1) // 2) * float(r.norm(dim=-1).max())
+    atol = 2e-6 + 4 * max_phase * 2.0 ** -24 * float(W.abs().sum(1).max())
+    y = ops.painn_radial_linear(r.cuda(), n, 8.0, W.cuda(), b.cuda(), act)
+    torch.testing.assert_close(y.cpu(), ref, rtol=1e-5, atol=atol)
+    # a weight given as a transposed view, no bias
+    Wt = W.t().contiguous().cuda().t()
+    y2 = ops.painn_radial_linear(r.cuda(), n, 8.0, Wt, None, act)
+    pre2 = enc @ W.double().t()
+    ref2 = {0: pre2, 1: torch.nn.functional.silu(pre2), 2: torch.where(pre2 > 0, pre2, 0.1 * pre2)}[act].float()
+    torch.testing.assert_close(y2.cpu(), ref2, rtol=1e-5, atol=atol)
+
+
+def test_radial_linear_fused_edge_cases(ops):
+    W = torch.randn(64, 16, device="cuda")
+    assert ops.painn_radial_linear(torch.empty(0, 3, device="cuda"), 16, 8.0, W).shape == (0, 64)
+    assert not ops.painn_radial_linear_supported(33, 64)
+    assert not ops.painn_radial_linear_supported(16, 48)
+    with pytest.raises(RuntimeError, match="at most 32 radial functions"):
+        ops.painn_radial_linear(torch.randn(10, 3, device="cuda"), 33, 8.0, torch.randn(64, 33, device="cuda"))
+    with pytest.raises(RuntimeError, match="dim_out must be"):
+        ops.painn_radial_linear(torch.randn(10, 3, device="cuda"), 16, 8.0, torch.randn(48, 16, device="cuda"))
+
+
 @pytest.mark.parametrize("n,with_res", [(128, True), (32, False), (4, True), (20, True), (6, False), (256, True), (192, False)])
 def test_fused_message_kernel(ops, n, with_res):
     torch.manual_seed(n)
