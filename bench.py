@@ -264,6 +264,21 @@ def bench_products(torch, args):
         nbytes = rows * 64 * (4 + 12 + 4 + 12 + 36)
         out[f"rows_{rows}"] = {"us": t * 1e6, "nodes_per_s": rows / t, "bytes": nbytes,
                                "GB/s": nbytes / t / 1e9, "frac_of_hbm_peak": nbytes / t / 1e9 / PEAK_HBM_GBS}
+    # the same three products as the reference module runs them: TensorProds(l, r, o) = lin_o(prod(lin_l, lin_r))
+    tp = importlib.import_module("learned-dynamics_amd.tensor_products")
+    torch.manual_seed(0x947 + 1)
+    mods = [tp.TensorProds(1, 1, 0, 64, 64, 64, 64).cuda(), tp.TensorProds(0, 1, 1, 64, 64, 64, 64).cuda(),
+            tp.TensorProds(1, 1, 2, 64, 64, 64, 64).cuda()]
+    for rows in (4096, 262144):
+        g = torch.Generator().manual_seed(0x947 + 1)
+        x = torch.randn(rows, 64, generator=g).cuda()
+        v = torch.randn(rows, 64, 3, generator=g).cuda()
+        with torch.no_grad():
+            t = event_time(torch, lambda: (mods[0](v, v), mods[1](x, v), mods[2](v, v)), 30, warmup=5)
+        flop = 2 * rows * 64 * 64 * ((3 + 3 + 1) + (1 + 3 + 3) + (3 + 3 + 9))
+        out[f"rows_{rows}"]["with_linears"] = {"us": t * 1e6, "GFLOP": flop / 1e9, "TFLOP/s": flop / t / 1e12,
+                                               "frac_of_fp32_mfma_peak": flop / t / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+                                               "launches": 12}
     return {"metric": "fused tensor-product trio (v.v, x v, v(x)v), BASELINE configs[0]", "unit": "nodes/s",
             "value": out["rows_4096"]["nodes_per_s"], "detail": out,
             "note": "includes allocation of the three outputs; 4096 rows (17.8 MB) is launch-latency bound"}
@@ -314,10 +329,12 @@ def bench_denoiser(torch, args, with_cpu=True):
 
 
 def bench_stress(torch, args):
-    """BASELINE configs[4] geometry and layer stack in fp32 storage: 65536 atoms uniform in a periodic cube at
-    0.1 atoms/A^3, cutoff 6 A, 4 x [Messages + SelfTensProds] with 128 channels per rank, neighbour rebuild inside
-    the step.  (The bf16-storage variant of that config is not built; this is the fp32 path at its size.)"""
+    """BASELINE configs[4]: 65536 atoms uniform in a periodic cube at 0.1 atoms/A^3, cutoff 6 A,
+    4 x [Messages + SelfTensProds] with 128 channels per rank, features stored as bf16 with fp32
+    accumulation, neighbour rebuild inside the step.  The fp32-storage path on the same problem is
+    timed beside it."""
     bee = importlib.import_module("learned-dynamics_amd.bee_layers")
+    b16 = importlib.import_module("learned-dynamics_amd.bee_layers_bf16")
     gl = importlib.import_module("learned-dynamics_amd.graph_layers")
     seed = 0x947 + 5
     torch.manual_seed(seed)
@@ -334,7 +351,7 @@ def bench_stress(torch, args):
     edges = [0]
 
     with torch.no_grad():
-        def step():
+        def step_f32():
             graph, r_ij = gl.graph_setup(r0, box, pos, neighbours_max=256, celllist_max=64)
             edges[0] = int(graph.src.numel())
             a, v, d = x_a, x_v, x_d
@@ -343,14 +360,26 @@ def bench_stress(torch, args):
                 a, v, d = a + da, v + dv, d + dd
                 a, v, d = p(a, v, d, residual=True)
             return a
-        step()
-        sec = timed_steps(torch, step, args.steps, args.warmup)
+
+        def step_bf16():
+            graph, r_ij = gl.graph_setup(r0, box, pos, neighbours_max=256, celllist_max=64)
+            edges[0] = int(graph.src.numel())
+            return b16.stack_forward(msgs, prods, graph, r_ij, x_a, x_v, x_d)
+
+        ref = step_f32()
+        out = step_bf16()[0]
+        rel = float((out - ref).abs().max() / ref.abs().max())
+        sec16 = timed_steps(torch, step_bf16, args.steps, args.warmup)
+        sec32 = timed_steps(torch, step_f32, args.steps, args.warmup)
     E = edges[0]
-    return {"metric": "message-passing edges/sec per layer", "value": E * layers / sec, "unit": "edges/s",
-            "ms_per_step": sec * 1e3, "dtype": "f32",
-            "config": {"workload": "BASELINE configs[4] in fp32 storage: 65536 atoms, density 0.1/A^3, cutoff 6 A, "
-                                   "4 x [Messages + SelfTensProds], 128 channels per rank, neighbour rebuild in the step",
-                       "edges": E, "atoms": N, "layers": layers, "atoms_per_s": N / sec}}
+    return {"metric": "message-passing edges/sec per layer", "value": E * layers / sec16, "unit": "edges/s",
+            "ms_per_step": sec16 * 1e3, "dtype": "bf16 storage, f32 accumulate",
+            "config": {"workload": "BASELINE configs[4]: 65536 atoms, density 0.1/A^3, cutoff 6 A, "
+                                   "4 x [Messages + SelfTensProds], 128 channels per rank, bf16 storage, "
+                                   "neighbour rebuild in the step",
+                       "edges": E, "atoms": N, "layers": layers, "atoms_per_s": N / sec16},
+            "max_abs_diff_vs_fp32_storage_over_scale": rel,
+            "fp32_storage": {"value": E * layers / sec32, "unit": "edges/s", "ms_per_step": sec32 * 1e3}}
 
 
 def cpu_denoiser_block(torch, model, x1, r0, box, dims):

@@ -295,6 +295,40 @@ int mg_bee_message(const int* row_ptr, const int* dst, const int* node_order, in
                    int chan, const float* enc_W /* (chan,8) */, const float* enc_b /* (chan) */,
                    float* P0, float* S1, float* S2, mg_stream_t stream);
 
+/* The 13 products of SelfTensProds.forward (archs/diffuser_atoms15.py:86-88; formulas of
+ * managan/codegen_tensor_products.py:235-249) on node rows in component-major layout:
+ * l0/r0 (N,chan), l1/r1 (N,3,chan), l2/r2 (N,9,chan) ->
+ * P0 (N,3,chan) [000,110,220], P1 (N,3,5,chan) [011,101,121,211,111], P2 (N,9,5,chan)
+ * [022,202,112,222,212]: the layout of S1/S2 above, so each rank's output linears are one GEMM. */
+int mg_bee_node_products(long n_nodes, int chan, const float* l0, const float* l1, const float* l2,
+                         const float* r0, const float* r1, const float* r2, float* P0, float* P1, float* P2,
+                         mg_stream_t stream);
+
+/* ------------------------------------------------------------------------
+ * bf16-storage configuration: feature tensors are bf16 in memory (void* below), every
+ * sum and product is fp32.  Same math and layouts as the fp32 entry points of the same name.
+ * ---------------------------------------------------------------------- */
+/* y = act(bias + x W^T): x bf16 (rows, dim_in), dim_in % 32 == 0; W = the buffer written by
+ * mg_linear_pack_weight (its hi and mid planes are used: 16 significand bits); y bf16
+ * (y_is_bf16 != 0) or fp32; out_comps / accumulate / act as mg_tensor_linear_packed
+ * (tensor_linear of extensions/tensor_ops/tensor_ops.cpp:31-93 on bf16 storage). */
+int mg_tensor_linear_bf16(const void* packed_W, const void* x, long rows, int dim_in, int dim_out,
+                          const float* bias, int act, int accumulate, int out_comps, int y_is_bf16, void* y,
+                          mg_stream_t stream);
+/* mg_bee_message with La, Lv, Ld, P0, S1, S2 stored as bf16 (enc, rhat, enc_W, enc_b fp32). */
+int mg_bee_message_bf16(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
+                        const float* rhat, const float* enc, const void* La, const void* Lv, const void* Ld,
+                        int chan, const float* enc_W, const float* enc_b, void* P0, void* S1, void* S2,
+                        mg_stream_t stream);
+/* mg_bee_node_products on bf16 storage. */
+int mg_bee_node_products_bf16(long n_nodes, int chan, const void* l0, const void* l1, const void* l2,
+                              const void* r0, const void* r1, const void* r2, void* P0, void* P1, void* P2,
+                              mg_stream_t stream);
+/* out[r,:] = scale * sum_{e in row r} x_edge[e,:]  (segment_coo at managan/graph_layers.py:54-59 on bf16
+ * storage, fp32 accumulation); feat % 4 == 0. */
+int mg_segment_sum_csr_bf16(const void* x_edge /* (E,feat) bf16 */, const int* row_ptr, int n_rows, int feat,
+                            float scale, void* out /* (n_rows,feat) bf16 */, mg_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

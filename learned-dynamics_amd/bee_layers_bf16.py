@@ -1,0 +1,118 @@
+"""bf16-storage forward of the rank-0/1/2 blocks (archs/diffuser_atoms15.py:59-110,227-253):
+the same modules and parameters as bee_layers.py (float32 weights, state dicts unchanged), with every
+feature tensor that lives in HBM stored as bfloat16 and every product and sum done in fp32.
+
+Storage layout: component-major, x_a (rows, dim_a), x_v (rows, 3, dim_v), x_d (rows, 9, dim_d) with
+rows = batch * nodes, so every linear map is one plain GEMM over (row, component) rows and the edge
+kernel's gathers are unit stride.  to_storage / from_storage convert from and to the reference's
+(batch, nodes, chan, 3, 3) float32 tensors at the ends of a stack.
+
+What is rounded to bf16: the node features between modules, L_k x_k, the per-edge scalar products
+and the hidden activations of the per-edge MLP, the per-node product sums.  Weights keep 16
+significand bits.  Group-norm statistics are taken in fp32.
+"""
+import torch
+
+from . import ops
+from .bee_layers import LABELS_0, LABELS_1, LABELS_2, Messages, SelfTensProds
+from .graph_layers import Graph
+
+
+def to_storage(x_a, x_v, x_d):
+    """(B,N,da), (B,N,dv,3), (B,N,dd,3,3) float32 -> (rows,da), (rows,3,dv), (rows,9,dd) bfloat16."""
+    B, N = x_a.shape[:2]
+    rows = B * N
+    return (x_a.reshape(rows, -1).to(torch.bfloat16).contiguous(),
+            x_v.reshape(rows, -1, 3).transpose(1, 2).to(torch.bfloat16).contiguous(),
+            x_d.reshape(rows, x_d.shape[2], 9).transpose(1, 2).to(torch.bfloat16).contiguous())
+
+
+def from_storage(s_a, s_v, s_d, batch):
+    """Inverse of to_storage (float32 result)."""
+    rows = s_a.shape[0]
+    N = rows // batch
+    return (s_a.float().reshape(batch, N, -1),
+            s_v.float().transpose(1, 2).reshape(batch, N, -1, 3).contiguous(),
+            s_d.float().transpose(1, 2).reshape(batch, N, -1, 3, 3).contiguous())
+
+
+def _lin(W, x, comps):
+    """x (rows, comps, dim_in) or (rows, dim_in) bf16 -> same leading shape with dim_out."""
+    rows = x.shape[0]
+    y = ops.tensor_linear_bf16(W, x.reshape(rows * comps, x.shape[-1]))
+    return y if comps == 1 else y.reshape(rows, comps, -1)
+
+
+def _cat_Y(mod, labels, scale=None):
+    W = torch.cat([getattr(mod, f"Y_{lab}").W for lab in labels], dim=1)
+    return W if scale is None else W * scale
+
+
+def mlp_forward(mlp, x, plus_identity=False):
+    """bee_layers.MLP on bf16 rows: lin_direct(x) [+ x] + layers(x)."""
+    Wd = mlp.lin_direct.weight
+    if plus_identity:
+        Wd = Wd + torch.eye(Wd.shape[0], device=Wd.device, dtype=Wd.dtype)
+    Ls = mlp.layers
+    h = ops.tensor_linear_bf16(Ls[0].weight, x, bias=Ls[0].bias, act=ops.ACT_LEAKY)
+    h = ops.tensor_linear_bf16(Ls[2].weight, h, bias=Ls[2].bias, act=ops.ACT_LEAKY)
+    out = ops.tensor_linear_bf16(Wd, x, out_dtype=torch.float32)
+    ops.tensor_linear_bf16(Ls[4].weight, h, bias=Ls[4].bias, out=out, accumulate=True)
+    return out.to(torch.bfloat16)
+
+
+def messages_forward(mod: Messages, graph: Graph, r_ij, s_a, s_v, s_d, node_order="cell"):
+    """Messages.forward (archs/diffuser_atoms15.py:238-253) on storage tensors; returns the three
+    0.1 * (sum over edges) increments in storage layout."""
+    if isinstance(node_order, str):
+        node_order = getattr(graph, "cell_order", None)
+    rows = s_a.shape[0]
+    La, Lv, Ld = _lin(mod.L0.W, s_a, 1), _lin(mod.L1.W, s_v, 3), _lin(mod.L2.W, s_d, 9)
+    enc, rhat = ops.bee_edge_geometry(r_ij.contiguous(), mod.r0)
+    P0, S1, S2 = ops.bee_message_bf16(graph.row_ptr, graph.dst32, rhat, enc, La, Lv, Ld, mod.lin_enc.weight,
+                                      mod.lin_enc.bias, node_order=node_order)
+    E, chan = P0.shape[0], P0.shape[2]
+    psi_a = ops.tensor_linear_bf16(_cat_Y(mod, LABELS_0), P0.reshape(E, 3 * chan))
+    psi_a = mlp_forward(mod.mlp_a, psi_a, plus_identity=True)
+    B_a = ops.segment_sum_csr_bf16(psi_a, graph.row_ptr, rows, 0.1)
+    B_v = _lin(_cat_Y(mod, LABELS_1, 0.1), S1.reshape(rows, 3, 5 * chan), 3)
+    B_d = _lin(_cat_Y(mod, LABELS_2, 0.1), S2.reshape(rows, 9, 5 * chan), 9)
+    return B_a, B_v, B_d
+
+
+def _tens_group_norm(gn, y, res, batch):
+    """TensGroupNorm (managan/tensor_products.py:215-232) on a component-major storage tensor
+    y (rows, T, dim) or (rows, dim): statistics in fp32 over (nodes, components, group channels)."""
+    rows = y.shape[0]
+    x = y.float().reshape(batch, rows // batch, -1, gn.groups, gn.chan // gn.groups)
+    m2 = (x * x).sum(2, keepdim=True).mean(dim=(1, 4), keepdim=True)
+    out = (x * torch.rsqrt(gn.epsilon + m2)).reshape(y.shape) * gn.gamma.reshape(-1)
+    if res is not None:
+        out = out + res.float()
+    return out.to(torch.bfloat16)
+
+
+def self_tens_prods_forward(mod: SelfTensProds, s_a, s_v, s_d, batch, residual=True):
+    """SelfTensProds.forward (archs/diffuser_atoms15.py:80-95) on storage tensors."""
+    rows = s_a.shape[0]
+    chan = mod.L0.W.shape[0]
+    P0, P1, P2 = ops.bee_node_products(_lin(mod.L0.W, s_a, 1), _lin(mod.L1.W, s_v, 3), _lin(mod.L2.W, s_d, 9),
+                                       _lin(mod.R0.W, s_a, 1), _lin(mod.R1.W, s_v, 3), _lin(mod.R2.W, s_d, 9))
+    y_a = _lin(_cat_Y(mod, LABELS_0), P0.reshape(rows, 3 * chan), 1)
+    y_v = _lin(_cat_Y(mod, LABELS_1), P1.reshape(rows, 3, 5 * chan), 3)
+    y_d = _lin(_cat_Y(mod, LABELS_2), P2.reshape(rows, 9, 5 * chan), 9)
+    return (_tens_group_norm(mod.gn_a, y_a, s_a if residual else None, batch),
+            _tens_group_norm(mod.gn_v, y_v, s_v if residual else None, batch),
+            _tens_group_norm(mod.gn_d, y_d, s_d if residual else None, batch))
+
+
+def stack_forward(messages, prods, graph, r_ij, x_a, x_v, x_d, node_order="cell"):
+    """blocks x [Messages (residual) -> SelfTensProds (residual)] with bf16 storage between and
+    inside the modules; float32 reference-layout tensors in and out."""
+    batch = x_a.shape[0]
+    s_a, s_v, s_d = to_storage(x_a, x_v, x_d)
+    for msg, prod in zip(messages, prods):
+        d_a, d_v, d_d = messages_forward(msg, graph, r_ij, s_a, s_v, s_d, node_order=node_order)
+        s_a, s_v, s_d = s_a + d_a, s_v + d_v, s_d + d_d
+        s_a, s_v, s_d = self_tens_prods_forward(prod, s_a, s_v, s_d, batch, residual=True)
+    return from_storage(s_a, s_v, s_d, batch)

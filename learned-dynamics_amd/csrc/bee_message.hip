@@ -89,12 +89,14 @@ __device__ __forceinline__ long uniform(long v) {
     return ((long)hi << 32) | (unsigned)lo;
 }
 
+// T: storage type of the node features and of the outputs (float, or __bf16 with fp32 arithmetic)
+template <typename T>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4)))
 bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst, const int* __restrict__ order,
                    long n_nodes, const float* __restrict__ rhat, const float* __restrict__ enc,
-                   const float* __restrict__ La, const float* __restrict__ Lv, const float* __restrict__ Ld, int chan,
-                   const float* __restrict__ enc_W, const float* __restrict__ enc_b, float* __restrict__ P0,
-                   float* __restrict__ S1, float* __restrict__ S2) {
+                   const T* __restrict__ La, const T* __restrict__ Lv, const T* __restrict__ Ld, int chan,
+                   const float* __restrict__ enc_W, const float* __restrict__ enc_b, T* __restrict__ P0,
+                   T* __restrict__ S1, T* __restrict__ S2) {
     const int lane = threadIdx.x & (kWave - 1);
     const int chunks = (chan + kWave - 1) / kWave;
     const long items = n_nodes * chunks;
@@ -133,12 +135,12 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
 #pragma unroll
             for (int t = 0; t < 3; t++) rh[t] = rhat[3 * e + t];
             // gathers: 13 unit-stride rows
-            const float l0 = La[j * chan + cc];
+            const float l0 = (float)La[j * chan + cc];
             float l1[3], l2[9];
 #pragma unroll
-            for (int t = 0; t < 3; t++) l1[t] = Lv[(j * 3 + t) * chan + cc];
+            for (int t = 0; t < 3; t++) l1[t] = (float)Lv[(j * 3 + t) * chan + cc];
 #pragma unroll
-            for (int k = 0; k < 9; k++) l2[k] = Ld[(j * 9 + k) * chan + cc];
+            for (int k = 0; k < 9; k++) l2[k] = (float)Ld[(j * 9 + k) * chan + cc];
 
             float phi = bias;
 #pragma unroll
@@ -156,10 +158,10 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
             const float pd1 = phi * dot1;
 
             if (active) {
-                float* p = P0 + (e * 3) * chan + c;
-                p[0] = pl0;              // 000
-                p[chan] = pd1;           // 110
-                p[2 * chan] = phi * quad;  // 220
+                T* p = P0 + (e * 3) * chan + c;
+                p[0] = (T)pl0;              // 000
+                p[chan] = (T)pd1;           // 110
+                p[2 * chan] = (T)(phi * quad);  // 220
             }
             // vector sums, label order 011, 101, 121, 211, 111
 #pragma unroll
@@ -190,9 +192,9 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
         }
         if (active) {
 #pragma unroll
-            for (int k = 0; k < 15; k++) S1[(node * 15 + k) * chan + c] = s1[k];
+            for (int k = 0; k < 15; k++) S1[(node * 15 + k) * chan + c] = (T)s1[k];
 #pragma unroll
-            for (int k = 0; k < 45; k++) S2[(node * 45 + k) * chan + c] = s2[k];
+            for (int k = 0; k < 45; k++) S2[(node * 45 + k) * chan + c] = (T)s2[k];
         }
     }
 }
@@ -201,6 +203,24 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
 }  // namespace mg
 
 using namespace mg;
+
+template <typename T>
+static int launch_bee_message(const char* what, const int* row_ptr, const int* dst, const int* node_order, int n_nodes,
+                              long n_edges, const float* rhat, const float* enc, const T* La, const T* Lv, const T* Ld,
+                              int chan, const float* enc_W, const float* enc_b, T* P0, T* S1, T* S2,
+                              mg_stream_t stream) {
+    MG_REQUIRE(n_nodes >= 0 && n_edges >= 0 && chan >= 0, "%s: negative size", what);
+    if (n_nodes == 0 || chan == 0) return MG_OK;
+    MG_REQUIRE(row_ptr && La && Lv && Ld && enc_W && enc_b && S1 && S2, "%s: null pointer", what);
+    MG_REQUIRE(n_edges == 0 || (dst && rhat && enc && P0), "%s: null edge operand", what);
+    const long items = (long)n_nodes * ceil_div(chan, kWave);
+    long blocks = ceil_div(items, 4);
+    if (blocks > 256L * 16) blocks = 256L * 16;
+    blocks = ceil_div(blocks, 8) * 8;
+    hipLaunchKernelGGL(bee_message_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, row_ptr, dst,
+                       node_order, (long)n_nodes, rhat, enc, La, Lv, Ld, chan, enc_W, enc_b, P0, S1, S2);
+    return check_launch(what);
+}
 
 extern "C" {
 
@@ -219,17 +239,17 @@ int mg_bee_edge_geometry(const float* r_ij, long n_edges, float r0, float* enc, 
 int mg_bee_message(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
                    const float* rhat, const float* enc, const float* La, const float* Lv, const float* Ld, int chan,
                    const float* enc_W, const float* enc_b, float* P0, float* S1, float* S2, mg_stream_t stream) {
-    MG_REQUIRE(n_nodes >= 0 && n_edges >= 0 && chan >= 0, "mg_bee_message: negative size");
-    if (n_nodes == 0 || chan == 0) return MG_OK;
-    MG_REQUIRE(row_ptr && La && Lv && Ld && enc_W && enc_b && S1 && S2, "mg_bee_message: null pointer");
-    MG_REQUIRE(n_edges == 0 || (dst && rhat && enc && P0), "mg_bee_message: null edge operand");
-    const long items = (long)n_nodes * ceil_div(chan, kWave);
-    long blocks = ceil_div(items, 4);
-    if (blocks > 256L * 16) blocks = 256L * 16;
-    blocks = ceil_div(blocks, 8) * 8;
-    hipLaunchKernelGGL(bee_message_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, row_ptr, dst,
-                       node_order, (long)n_nodes, rhat, enc, La, Lv, Ld, chan, enc_W, enc_b, P0, S1, S2);
-    return check_launch("mg_bee_message");
+    return launch_bee_message<float>("mg_bee_message", row_ptr, dst, node_order, n_nodes, n_edges, rhat, enc, La, Lv,
+                                     Ld, chan, enc_W, enc_b, P0, S1, S2, stream);
+}
+
+int mg_bee_message_bf16(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
+                        const float* rhat, const float* enc, const void* La, const void* Lv, const void* Ld, int chan,
+                        const float* enc_W, const float* enc_b, void* P0, void* S1, void* S2, mg_stream_t stream) {
+    return launch_bee_message<__bf16>("mg_bee_message_bf16", row_ptr, dst, node_order, n_nodes, n_edges, rhat, enc,
+                                      static_cast<const __bf16*>(La), static_cast<const __bf16*>(Lv),
+                                      static_cast<const __bf16*>(Ld), chan, enc_W, enc_b, static_cast<__bf16*>(P0),
+                                      static_cast<__bf16*>(S1), static_cast<__bf16*>(S2), stream);
 }
 
 }  // extern "C"

@@ -1,0 +1,109 @@
+// The 13 Cartesian products on node rows in component-major layout (node, comp, chan), for the
+// self-interaction block (archs/diffuser_atoms15.py:59-95) of the bf16-storage configuration.
+//
+// Inputs  l0/r0 (N, chan), l1/r1 (N, 3, chan), l2/r2 (N, 9, chan)
+// Outputs P0 (N, 3, chan)      labels 000, 110, 220
+//         P1 (N, 3, 5, chan)   labels 011, 101, 121, 211, 111 per vector component
+//         P2 (N, 9, 5, chan)   labels 022, 202, 112, 222, 212 per rank-2 component (xy -> 3x+y)
+// i.e. the layout the edge kernel uses for its per-node sums, so the output linears of a rank are
+// one GEMM with K = 3*chan or 5*chan.  A lane owns one (node, channel): every access of a wave is
+// unit stride.  Bound by HBM: 26 values in, 63 out per (node, channel).
+#include "common.hpp"
+
+namespace mg {
+namespace {
+
+template <typename T>
+__global__ void __launch_bounds__(256) node_products_kernel(long n_nodes, int chan, const T* __restrict__ l0,
+                                                            const T* __restrict__ l1, const T* __restrict__ l2,
+                                                            const T* __restrict__ r0, const T* __restrict__ r1,
+                                                            const T* __restrict__ r2, T* __restrict__ P0,
+                                                            T* __restrict__ P1, T* __restrict__ P2) {
+    const long total = n_nodes * chan;
+    for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (long)gridDim.x * blockDim.x) {
+        const long node = t / chan;
+        const int c = (int)(t - node * chan);
+        const float a = (float)l0[t], b = (float)r0[t];
+        float u[3], v[3], L[9], R[9];
+#pragma unroll
+        for (int x = 0; x < 3; x++) {
+            u[x] = (float)l1[(node * 3 + x) * chan + c];
+            v[x] = (float)r1[(node * 3 + x) * chan + c];
+        }
+#pragma unroll
+        for (int k = 0; k < 9; k++) {
+            L[k] = (float)l2[(node * 9 + k) * chan + c];
+            R[k] = (float)r2[(node * 9 + k) * chan + c];
+        }
+        float dot = 0.f, ddot = 0.f;
+#pragma unroll
+        for (int x = 0; x < 3; x++) dot += u[x] * v[x];
+#pragma unroll
+        for (int k = 0; k < 9; k++) ddot += L[k] * R[k];
+        T* p0 = P0 + (node * 3) * chan + c;
+        p0[0] = (T)(a * b);
+        p0[chan] = (T)dot;
+        p0[2 * chan] = (T)ddot;
+
+        const float cr[3] = {u[1] * v[2] - u[2] * v[1], u[2] * v[0] - u[0] * v[2], u[0] * v[1] - u[1] * v[0]};
+#pragma unroll
+        for (int x = 0; x < 3; x++) {
+            T* p1 = P1 + ((node * 3 + x) * 5) * chan + c;
+            p1[0] = (T)(a * v[x]);                                                      // 011
+            p1[chan] = (T)(u[x] * b);                                                   // 101
+            p1[2 * chan] = (T)(u[0] * R[3 * x] + u[1] * R[3 * x + 1] + u[2] * R[3 * x + 2]);   // 121: sum_k l_k r_{x k}
+            p1[3 * chan] = (T)(L[3 * x] * v[0] + L[3 * x + 1] * v[1] + L[3 * x + 2] * v[2]);   // 211
+            p1[4 * chan] = (T)cr[x];                                                    // 111
+        }
+#pragma unroll
+        for (int x = 0; x < 3; x++) {
+            // 212: row x of L crossed with v
+            const float rc[3] = {L[3 * x + 1] * v[2] - L[3 * x + 2] * v[1], L[3 * x + 2] * v[0] - L[3 * x] * v[2],
+                                 L[3 * x] * v[1] - L[3 * x + 1] * v[0]};
+#pragma unroll
+            for (int z = 0; z < 3; z++) {
+                const int k = 3 * x + z;
+                T* p2 = P2 + ((node * 9 + k) * 5) * chan + c;
+                p2[0] = (T)(a * R[k]);                                                  // 022
+                p2[chan] = (T)(L[k] * b);                                               // 202
+                p2[2 * chan] = (T)(u[x] * v[z]);                                        // 112
+                p2[3 * chan] = (T)(L[3 * x] * R[3 * z] + L[3 * x + 1] * R[3 * z + 1] + L[3 * x + 2] * R[3 * z + 2]);  // 222
+                p2[4 * chan] = (T)rc[z];                                                // 212
+            }
+        }
+    }
+}
+
+template <typename T>
+int launch(const char* what, long n_nodes, int chan, const void* l0, const void* l1, const void* l2, const void* r0,
+           const void* r1, const void* r2, void* P0, void* P1, void* P2, mg_stream_t stream) {
+    MG_REQUIRE(n_nodes >= 0 && chan >= 0, "%s: negative size", what);
+    if (n_nodes == 0 || chan == 0) return MG_OK;
+    MG_REQUIRE(l0 && l1 && l2 && r0 && r1 && r2 && P0 && P1 && P2, "%s: null pointer", what);
+    long blocks = ceil_div(n_nodes * chan, 256);
+    if (blocks > 256L * 32) blocks = 256L * 32;
+    hipLaunchKernelGGL(node_products_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, n_nodes,
+                       chan, static_cast<const T*>(l0), static_cast<const T*>(l1), static_cast<const T*>(l2),
+                       static_cast<const T*>(r0), static_cast<const T*>(r1), static_cast<const T*>(r2),
+                       static_cast<T*>(P0), static_cast<T*>(P1), static_cast<T*>(P2));
+    return check_launch(what);
+}
+
+}  // namespace
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" {
+
+int mg_bee_node_products(long n_nodes, int chan, const float* l0, const float* l1, const float* l2, const float* r0,
+                         const float* r1, const float* r2, float* P0, float* P1, float* P2, mg_stream_t stream) {
+    return launch<float>("mg_bee_node_products", n_nodes, chan, l0, l1, l2, r0, r1, r2, P0, P1, P2, stream);
+}
+
+int mg_bee_node_products_bf16(long n_nodes, int chan, const void* l0, const void* l1, const void* l2, const void* r0,
+                              const void* r1, const void* r2, void* P0, void* P1, void* P2, mg_stream_t stream) {
+    return launch<__bf16>("mg_bee_node_products_bf16", n_nodes, chan, l0, l1, l2, r0, r1, r2, P0, P1, P2, stream);
+}
+
+}  // extern "C"

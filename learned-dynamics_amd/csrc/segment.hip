@@ -94,6 +94,47 @@ __global__ void __launch_bounds__(256) segment_sum_kernel(const float* __restric
     }
 }
 
+// bf16 storage, fp32 accumulation: a lane owns 4 consecutive channels (8-byte loads), L lanes cover
+// one edge row, the other 64/L lane groups take further edges and are folded at the end.
+// out[row] = scale * sum over the row's edges.
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+
+__global__ void __launch_bounds__(256) segment_sum_bf16_kernel(const __bf16* __restrict__ x,
+                                                               const int* __restrict__ row_ptr, long n_rows, int feat,
+                                                               int L, int chunks, float scale,
+                                                               __bf16* __restrict__ out) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const long wave_global = ((long)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+    const long n_waves = ((long)gridDim.x * blockDim.x) / kWave;
+    const long items = n_rows * chunks;
+    const int sub = lane / L, per_iter = kWave / L;
+    for (long item = wave_global; item < items; item += n_waves) {
+        const long row = item / chunks;
+        const int c = (int)(item - row * chunks);
+        const int col = c * 256 + (lane & (L - 1)) * 4;
+        const bool active = col < feat;
+        const long lo = row_ptr[row], hi = row_ptr[row + 1];
+        float a[4] = {0.f, 0.f, 0.f, 0.f};
+        if (active) {
+            for (long e = lo + sub; e < hi; e += per_iter) {
+                const bf16x4 v = *reinterpret_cast<const bf16x4*>(x + e * feat + col);
+#pragma unroll
+                for (int k = 0; k < 4; k++) a[k] += (float)v[k];
+            }
+        }
+        for (int d = L; d < kWave; d <<= 1) {
+#pragma unroll
+            for (int k = 0; k < 4; k++) a[k] += __shfl_xor(a[k], d, kWave);
+        }
+        if (active && sub == 0) {
+            bf16x4 o;
+#pragma unroll
+            for (int k = 0; k < 4; k++) o[k] = (__bf16)(a[k] * scale);
+            *reinterpret_cast<bf16x4*>(out + row * feat + col) = o;
+        }
+    }
+}
+
 template <int VEC>
 __global__ void __launch_bounds__(256) gather_kernel(const float* __restrict__ x, const void* __restrict__ index,
                                                      int is64, long n_edges, long n_rows, int feat,
@@ -170,6 +211,26 @@ int mg_segment_sum_csr(const float* x_edge, const int* row_ptr, int n_rows, int 
         hipLaunchKernelGGL(segment_sum_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, x_edge,
                            row_ptr, (long)n_rows, feat, ch, out);
     return check_launch("mg_segment_sum_csr");
+}
+
+int mg_segment_sum_csr_bf16(const void* x_edge, const int* row_ptr, int n_rows, int feat, float scale, void* out,
+                            mg_stream_t stream) {
+    MG_REQUIRE(n_rows >= 0 && feat >= 0, "mg_segment_sum_csr_bf16: negative size");
+    if (n_rows == 0 || feat == 0) return MG_OK;
+    MG_REQUIRE(feat % 4 == 0, "mg_segment_sum_csr_bf16: feat must be a multiple of 4 (got %d)", feat);
+    MG_REQUIRE(row_ptr && out, "mg_segment_sum_csr_bf16: null pointer");
+    MG_REQUIRE((reinterpret_cast<uintptr_t>(x_edge) & 7u) == 0 && (reinterpret_cast<uintptr_t>(out) & 7u) == 0,
+               "mg_segment_sum_csr_bf16: pointers must be 8-byte aligned");
+    const int chunks = (int)ceil_div(feat, 256);
+    int L = 1;
+    while (L < 64 && L * 4 < (feat < 256 ? feat : 256)) L <<= 1;
+    const long items = (long)n_rows * chunks;
+    long blocks = ceil_div(items, 4);
+    if (blocks > 256L * 64) blocks = 256L * 64;
+    hipLaunchKernelGGL(segment_sum_bf16_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                       static_cast<const __bf16*>(x_edge), row_ptr, (long)n_rows, feat, L, chunks, scale,
+                       static_cast<__bf16*>(out));
+    return check_launch("mg_segment_sum_csr_bf16");
 }
 
 int mg_gather_rows(const float* x, const void* index, int index_is_int64, long n_edges, int n_rows, int feat,

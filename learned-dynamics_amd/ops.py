@@ -528,6 +528,110 @@ def tensor_linear_wgrad(inds, dy, x):
     return dW
 
 
+# ------------------------------------------------- bf16-storage configuration
+def _check_bf16(t, name):
+    if not t.is_cuda:
+        raise RuntimeError(f"{name} must be a CUDA tensor")
+    if t.dtype != torch.bfloat16:
+        raise RuntimeError(f"{name} must be bfloat16")
+    if not t.is_contiguous():
+        raise RuntimeError(f"{name} must be contiguous")
+
+
+def tensor_linear_bf16(W, x, bias=None, act=ACT_NONE, out=None, accumulate=False, out_comps=1,
+                       out_dtype=torch.bfloat16):
+    """y = act(bias + x W^T) on bf16 storage: x (rows, dim_in) bfloat16, W (dim_out, dim_in) float32
+    parameter (split once, 16 significand bits used), fp32 accumulation, y bfloat16 or float32.
+    out_comps = T > 1 treats consecutive groups of T rows as the components of one row and writes
+    y as (rows / T, dim_out, T)."""
+    _check_bf16(x, "x")
+    if W.dim() != 2 or W.dtype != torch.float32 or not W.is_cuda:
+        raise RuntimeError("W must be a float32 CUDA matrix")
+    if x.dim() != 2 or x.size(1) != W.size(1):
+        raise RuntimeError("x must have shape (rows, dim_in)")
+    rows, dim_in, dim_out = int(x.size(0)), int(W.size(1)), int(W.size(0))
+    if dim_in % 32:
+        raise RuntimeError("dim_in must be a multiple of 32 on the bf16 path")
+    if rows % out_comps:
+        raise RuntimeError("rows must be a multiple of out_comps")
+    if bias is not None and (bias.dtype != torch.float32 or not bias.is_contiguous() or bias.numel() != dim_out):
+        raise RuntimeError("bias must be a contiguous float32 tensor of dim_out elements")
+    shape = (rows, dim_out) if out_comps == 1 else (rows // out_comps, dim_out, out_comps)
+    with torch.cuda.device(x.device):
+        if out is None:
+            if accumulate:
+                raise RuntimeError("accumulate needs out")
+            out = torch.empty(shape, dtype=out_dtype, device=x.device)
+        elif tuple(out.shape) != shape or not out.is_contiguous() or out.dtype not in (torch.bfloat16, torch.float32):
+            raise RuntimeError("out has the wrong shape, dtype or layout")
+        L.check(_lib.mg_tensor_linear_bf16(_p(packed_weight(W)), _p(x), rows, dim_in, dim_out,
+                                           _p(bias) if bias is not None else None, int(act), int(bool(accumulate)),
+                                           int(out_comps), int(out.dtype == torch.bfloat16), _p(out), _stream()))
+    return out
+
+
+def bee_message_bf16(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=None):
+    """bee_message on bf16 storage: La (N,chan), Lv (N,3,chan), Ld (N,9,chan) bfloat16 ->
+    P0 (E,3,chan), S1 (N,3,5,chan), S2 (N,9,5,chan) bfloat16."""
+    for t, nm in ((La, "La"), (Lv, "Lv"), (Ld, "Ld")):
+        _check_bf16(t, nm)
+    for t, nm in ((rhat, "rhat"), (enc, "enc"), (enc_W, "enc_W"), (enc_b, "enc_b")):
+        _check_input(t, nm)
+    N, chan = int(La.size(0)), int(La.size(1))
+    E = int(dst.numel())
+    if tuple(Lv.shape) != (N, 3, chan) or tuple(Ld.shape) != (N, 9, chan):
+        raise RuntimeError("Lv, Ld must be (nodes, 3, chan), (nodes, 9, chan)")
+    if tuple(rhat.shape) != (E, 3) or tuple(enc.shape) != (E, 8) or tuple(enc_W.shape) != (chan, 8):
+        raise RuntimeError("rhat (E,3), enc (E,8), enc_W (chan,8) expected")
+    if row_ptr.dtype != torch.int32 or dst.dtype != torch.int32 or row_ptr.numel() != N + 1:
+        raise RuntimeError("row_ptr (nodes+1) and dst must be int32")
+    if node_order is not None and (node_order.dtype != torch.int32 or node_order.numel() != N):
+        raise RuntimeError("node_order must be int32 with one entry per node")
+    with torch.cuda.device(La.device):
+        P0 = torch.empty(E, 3, chan, dtype=torch.bfloat16, device=La.device)
+        S1 = torch.empty(N, 3, 5, chan, dtype=torch.bfloat16, device=La.device)
+        S2 = torch.empty(N, 9, 5, chan, dtype=torch.bfloat16, device=La.device)
+        L.check(_lib.mg_bee_message_bf16(_p(row_ptr), _p(dst), _p(node_order) if node_order is not None else None,
+                                         N, E, _p(rhat), _p(enc), _p(La), _p(Lv), _p(Ld), chan, _p(enc_W),
+                                         _p(enc_b), _p(P0), _p(S1), _p(S2), _stream()))
+    return P0, S1, S2
+
+
+def bee_node_products(l0, l1, l2, r0, r1, r2):
+    """The 13 products on node rows in component-major layout (float32 or bfloat16 storage):
+    l0/r0 (N,chan), l1/r1 (N,3,chan), l2/r2 (N,9,chan) -> P0 (N,3,chan), P1 (N,3,5,chan), P2 (N,9,5,chan)."""
+    bf = l0.dtype == torch.bfloat16
+    for t, nm in ((l0, "l0"), (l1, "l1"), (l2, "l2"), (r0, "r0"), (r1, "r1"), (r2, "r2")):
+        (_check_bf16 if bf else _check_input)(t, nm)
+    N, chan = int(l0.size(0)), int(l0.size(1))
+    for t, comps in ((l0, None), (r0, None), (l1, 3), (r1, 3), (l2, 9), (r2, 9)):
+        want = (N, chan) if comps is None else (N, comps, chan)
+        if tuple(t.shape) != want:
+            raise RuntimeError("operands must be (nodes, chan), (nodes, 3, chan), (nodes, 9, chan)")
+    with torch.cuda.device(l0.device):
+        P0 = torch.empty(N, 3, chan, dtype=l0.dtype, device=l0.device)
+        P1 = torch.empty(N, 3, 5, chan, dtype=l0.dtype, device=l0.device)
+        P2 = torch.empty(N, 9, 5, chan, dtype=l0.dtype, device=l0.device)
+        fn = _lib.mg_bee_node_products_bf16 if bf else _lib.mg_bee_node_products
+        L.check(fn(N, chan, _p(l0), _p(l1), _p(l2), _p(r0), _p(r1), _p(r2), _p(P0), _p(P1), _p(P2), _stream()))
+    return P0, P1, P2
+
+
+def segment_sum_csr_bf16(x_edge, row_ptr, n_rows, scale=1.0):
+    """scale * (sum of the bfloat16 edge rows of each CSR row), fp32 accumulation, bfloat16 result."""
+    _check_bf16(x_edge, "x_edge")
+    if x_edge.dim() != 2 or x_edge.size(1) % 4:
+        raise RuntimeError("x_edge must be (edges, feat) with feat a multiple of 4")
+    if row_ptr.dtype != torch.int32 or row_ptr.numel() != n_rows + 1:
+        raise RuntimeError("row_ptr must be int32 with n_rows + 1 entries")
+    feat = int(x_edge.size(1))
+    with torch.cuda.device(x_edge.device):
+        out = torch.empty(n_rows, feat, dtype=torch.bfloat16, device=x_edge.device)
+        L.check(_lib.mg_segment_sum_csr_bf16(_p(x_edge), _p(row_ptr), int(n_rows), feat, float(scale), _p(out),
+                                             _stream()))
+    return out
+
+
 # ----------------------------------------------------------------------- PaiNN
 def painn_radial_encode(r_ij, n, rmax):
     """radial_encode of archs/meanflow_painn8.py:25-35: (E,3) -> (E,n)."""
