@@ -125,11 +125,29 @@ def bench_painn_layer(torch, args):
         h = torch.randn(E, 4 * n, device="cuda")
         lin = block.message.mlp_dist.layers[2]
         out = torch.empty(E, 4 * n, device="cuda")
-        t_gemm = event_time(torch, lambda: ops.tensor_linear_fwd(0, lin.weight, h, bias=lin.bias, act=ops.ACT_SILU,
-                                                                 out=out), 10)
+        mode = ops.get_linear_mode()
+        if mode == ops.LINEAR_F16X2:
+            # as the layer runs it: row bounds carried over from the previous layer's weight norms
+            bound = ops.linear_out_bound(block.message.mlp_dist.layers[0].weight, block.message.mlp_dist.layers[0].bias,
+                                         None)
+            t_gemm = event_time(torch, lambda: ops.tensor_linear_f16x2(lin.weight, h, bound, bias=lin.bias,
+                                                                       act=ops.ACT_SILU, out=out), 10)
+        else:
+            t_gemm = event_time(torch, lambda: ops.tensor_linear_fwd(0, lin.weight, h, bias=lin.bias, act=ops.ACT_SILU,
+                                                                     out=out), 10)
         flops = 2.0 * E * (4 * n) * (4 * n)
-        split = ops.get_linear_mode() == ops.LINEAR_BF16X3
-        if split:
+        split = mode == ops.LINEAR_BF16X3
+        if mode == ops.LINEAR_F16X2:
+            # operands split into 2 fp16 pieces, 3 fp16 MFMAs per fp32 product, fp32 accumulate
+            roofline = {"kernel": "linear_rows_f16x2_kernel<4,4> (filter MLP layer, E x 512 x 512, bias+SiLU fused)",
+                        "bound": "mfma", "achieved": 3 * flops / t_gemm / 1e12, "peak": PEAK_BF16_MFMA_TFLOPS,
+                        "unit": "TFLOP/s", "frac": 3 * flops / t_gemm / 1e12 / PEAK_BF16_MFMA_TFLOPS,
+                        "traffic": measured_traffic("linear_rows_f16x2_kernel"),
+                        "note": "achieved counts the executed fp16 MFMA FLOPs (3 per fp32 multiply-add pair) against "
+                                "the fp16 dense peak; fp32-equivalent rate and its ratio to the fp32 MFMA peak alongside",
+                        "fp32_equivalent_tflops": flops / t_gemm / 1e12,
+                        "fp32_equivalent_over_fp32_mfma_peak": flops / t_gemm / 1e12 / PEAK_FP32_MFMA_TFLOPS}
+        elif split:
             # operands split into 3 bf16 pieces, 6 bf16 MFMAs per fp32 product, fp32 accumulate
             roofline = {"kernel": "linear_rows_bf16x3_wide_kernel (filter MLP layer, E x 512 x 512, bias+SiLU fused)",
                         "bound": "mfma", "achieved": 6 * flops / t_gemm / 1e12, "peak": PEAK_BF16_MFMA_TFLOPS,

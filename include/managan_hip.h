@@ -191,7 +191,9 @@ int mg_tensor_linear_layout(int inds, const float* W, long w_stride_o, long w_st
 /* Arithmetic used by the wide plain-row GEMMs (inds = 0 or component-major x, dim_in % 32 == 0):
  *   0  fp32 MFMA (v_mfma_f32_32x32x2_f32);
  *   1  operands split exactly into three bf16 pieces, six bf16 MFMAs per product, fp32
- *      accumulation: same accuracy class as fp32 (dropped terms < 2^-24 |a||b|), ~2.7x the rate.
+ *      accumulation: same accuracy class as fp32 (dropped terms < 2^-24 |a||b|), ~2.7x the rate;
+ *   2  as 1 for callers of mg_tensor_linear*; the host side additionally routes wide plain-row
+ *      layers through mg_tensor_linear_f16x2 (below).
  * Process-wide setting; no counterpart in the reference (its kernel is a plain fp32 dot product,
  * extensions/tensor_ops/tensor_ops_kern.cu:6-42). */
 int mg_set_linear_mode(int mode);
@@ -209,6 +211,27 @@ int mg_linear_pack_weight(const float* W, long w_stride_o, long w_stride_i, int 
 int mg_tensor_linear_packed(const void* packed_W, const float* x, long rows, int dim_in, int dim_out,
                             const float* bias, int act, int accumulate, int out_comps, float* y,
                             mg_stream_t stream);
+/* Mode 2: two-piece fp16 split with per-row power-of-two scales, three fp16 MFMAs per product,
+ * fp32 accumulation (a few fp32 ulps per product; half the matrix work of mode 1).
+ * mg_linear_f16x2_pack_weight: W -> hi / lo fp16 planes (dim_out rounded up to 256 rows) followed by
+ * one fp32 inverse scale per row, in caller-owned memory of mg_linear_f16x2_packed_weight_bytes bytes.
+ * mg_tensor_linear_f16x2: y = act(x W^T + bias) for plain rows x (rows, dim_in), dim_in % 32 == 0;
+ * x_rowmax[r * x_rowmax_stride + p], p < x_rowmax_parts, holds upper bounds of max_i |x[r,i]| (the
+ * largest part is used; any bound within a factor 2^14 of the true maximum keeps full accuracy;
+ * stride 0 = one bound for all rows): the y_rowmax output of the call that produced x,
+ * mg_row_absmax(x) (one part), or a bound the caller derives from the producing layer's weights.  y_rowmax, if not NULL,
+ * receives (rows, mg_tensor_linear_f16x2_rowmax_parts(rows, dim_out)) partial row maxima of |y|
+ * (out_comps must be 1).  out_comps / accumulate / act as in mg_tensor_linear_packed.
+ * Same contraction as tensor_linear (extensions/tensor_ops/tensor_ops.cpp:31-93); packing, scales
+ * and row maxima have no counterpart in the reference. */
+int mg_linear_f16x2_packed_weight_bytes(int dim_in, int dim_out, size_t* bytes /* host */);
+int mg_linear_f16x2_pack_weight(const float* W, long w_stride_o, long w_stride_i, int dim_in, int dim_out,
+                                void* packed, mg_stream_t stream);
+int mg_row_absmax(const float* x, long rows, int dim, float* out /* (rows) */, mg_stream_t stream);
+int mg_tensor_linear_f16x2_rowmax_parts(long rows, int dim_out);   /* returns the count, not a status */
+int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts,
+                           long x_rowmax_stride, long rows, int dim_in, int dim_out, const float* bias, int act, int accumulate,
+                           int out_comps, float* y, float* y_rowmax, mg_stream_t stream);
 /* dW[o,i] = sum_{r,t} dy[r,o,t] x[r,i,t]  (tensor_ops_kern.cu:45-71), dW dense (dim_out,dim_in). */
 int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows, int dim_in, int dim_out,
                            float* dW, mg_stream_t stream);

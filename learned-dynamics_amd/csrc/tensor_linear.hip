@@ -23,7 +23,7 @@ int launch_rows_bf16x3(const float* W, long so, const float* X, long R, int I, i
 
 namespace {
 
-std::atomic<int> g_linear_mode{1};   // 0: fp32 MFMA everywhere; 1 (default): bf16x3 split for the wide T=1 GEMMs
+std::atomic<int> g_linear_mode{2};   // 0: fp32 MFMA everywhere; 1: bf16x3 split for the wide T=1 GEMMs; 2 (default): host side uses the f16x2 entry point where it can, bf16x3 here
 
 typedef float float16v __attribute__((ext_vector_type(16)));
 
@@ -412,7 +412,7 @@ int mg_tensor_linear_layout(int inds, const float* W, long w_stride_o, long w_st
         const long R = rows * T;
         const int out_T = (y_layout == 1) ? 1 : T;
         if (dim_in % kBK1 == 0 && aligned16(x) && (dim_out > 64 || out_T > 1)) {
-            if (g_linear_mode.load() == 1 && si == 1 && so % 4 == 0 && aligned16(W) && dim_in >= 64 && R >= 1024)
+            if (g_linear_mode.load() >= 1 && si == 1 && so % 4 == 0 && aligned16(W) && dim_in >= 64 && R >= 1024)
                 return launch_rows_bf16x3(W, so, x, R, dim_in, dim_out, b, act, accumulate, y, st, out_T);
             return launch_rows(W, so, si, x, R, dim_in, dim_out, b, act, accumulate, y, st, out_T);
         }
@@ -432,7 +432,7 @@ int mg_tensor_linear_layout(int inds, const float* W, long w_stride_o, long w_st
 }
 
 int mg_set_linear_mode(int mode) {
-    MG_REQUIRE(mode == 0 || mode == 1, "mg_set_linear_mode: mode must be 0 (fp32 MFMA) or 1 (bf16x3 split)");
+    MG_REQUIRE(mode >= 0 && mode <= 2, "mg_set_linear_mode: mode must be 0 (fp32 MFMA), 1 (bf16x3 split) or 2 (f16x2 split)");
     g_linear_mode.store(mode);
     return MG_OK;
 }

@@ -1,0 +1,419 @@
+// fp32-class GEMM on the fp16 matrix cores with two-piece operand splitting ("f16x2").
+//
+// Every fp32 operand is scaled by a per-row power of two (exact) and split into two fp16
+// pieces, v = hi + lo with hi = RNE16(v) and lo = RNE16(v - hi): 11 + 11 significand bits, so
+// |v - hi - lo| <= 2^-22 |v|.  A product is assembled from three piece products
+//     a*b ~= a_lo*b_hi + a_hi*b_lo + a_hi*b_hi            (dropped: a_lo*b_lo <= 2^-22 |a||b|)
+// accumulated in fp32 by v_mfma_f32_32x32x16_f16: half the matrix work of a three-piece bf16
+// split, at an error of a few fp32 ulps per product (the rounding of an fp32 dot product of
+// length K is of the same size).  The power-of-two scales put the largest element of an x row
+// (a W row) into [2^14, 2^15), which removes fp16's narrow exponent range from the picture:
+// an element e of a row with scaled maximum M carries an error of max(2^-22 |e|, 2^-25), i.e.
+// the result is normwise as accurate as the fp32 dot product whenever M >= 1, and the scales
+// are undone exactly in the epilogue.  The row maxima of x come from the kernel that produced
+// x (this kernel's own epilogue can emit them for its output) or from row_absmax_kernel.
+//
+// Tile TM x TN per workgroup = (64 WM) x (64 NI), waves WM x 2, wave tile 64 x (32 NI), K slab
+// 16, LDS double buffered with one barrier per slab; the staging of slab k+1 (global fp32 ->
+// scale, split -> LDS planes) sits in the instruction stream of slab k's MFMAs, and the two
+// waves of a SIMD stage at opposite ends of the slab period.
+// v_mfma_f32_32x32x16_f16 layout: A[m][k]: lane = m + 32*(k/8), 8 consecutive k per lane;
+// B[k][n] likewise; D[m][n]: n = lane%32, m = 8*(q/4) + 4*(lane/32) + q%4 for register q.
+#include "common.hpp"
+#include <type_traits>
+
+namespace mg {
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
+typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
+
+constexpr int kBK = 16;
+constexpr int kRow = 48;   // bytes per LDS row of one plane: 16 fp16 + pad (3 quads: conflict free for b128 reads)
+
+__device__ __forceinline__ float activate(float v, int act) {
+    if (act == 1) return v * __frcp_rn(1.0f + __expf(-v));
+    if (act == 2) return v > 0.f ? v : 0.1f * v;
+    return v;
+}
+
+// power of two s with amax * s in [2^14, 2^15); *inv = 1/s.  amax >= 0; zero, tiny, inf and nan give
+// a finite in-range scale (the products then follow fp16/fp32 arithmetic on their own)
+__device__ __forceinline__ float pow2_scale(float amax, float* inv) {
+    int e = (int)(__float_as_uint(amax) >> 23) & 0xff;
+    int se = 268 - e;                   // 127 + 14 - (e - 127)
+    if (e == 255) se = 127;
+    se = se < 1 ? 1 : (se > 253 ? 253 : se);
+    *inv = __uint_as_float((unsigned)(254 - se) << 23);
+    return __uint_as_float((unsigned)se << 23);
+}
+
+struct HalfSplit4 {
+    halfx4 hi, lo;
+};
+
+__device__ __forceinline__ HalfSplit4 split(float4 v, float s) {
+    HalfSplit4 r;
+    const float in[4] = {v.x * s, v.y * s, v.z * s, v.w * s};
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        const _Float16 h = (_Float16)in[k];
+        r.hi[k] = h;
+        r.lo[k] = (_Float16)(in[k] - (float)h);
+    }
+    return r;
+}
+
+// one wave per output row: row maximum -> scale -> hi / lo planes (O_pad rows, zero filled) + 1/scale per row
+__global__ void __launch_bounds__(256) pack_weight_f16x2_kernel(const float* __restrict__ W, long so, long si, int I,
+                                                                int O, int O_pad, _Float16* __restrict__ planes,
+                                                                float* __restrict__ inv_scale) {
+    const int lane = threadIdx.x & 63;
+    const long total = (long)O_pad * I;
+    for (long o = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6; o < O_pad; o += ((long)gridDim.x * blockDim.x) >> 6) {
+        float amax = 0.f;
+        if (o < O)
+            for (int i = lane; i < I; i += 64) amax = fmaxf(amax, fabsf(W[o * so + (long)i * si]));
+        for (int d = 1; d < 64; d <<= 1) amax = fmaxf(amax, __shfl_xor(amax, d));
+        float inv;
+        const float s = pow2_scale(amax, &inv);
+        for (int i = lane; i < I; i += 64) {
+            const float v = o < O ? W[o * so + (long)i * si] * s : 0.f;
+            const _Float16 h = (_Float16)v;
+            planes[o * I + i] = h;
+            planes[total + o * I + i] = (_Float16)(v - (float)h);
+        }
+        if (lane == 0) inv_scale[o] = inv;
+    }
+}
+
+// out[r] = max_i |x[r, i]|; a wave per row, 16-byte loads when the row length allows
+__global__ void __launch_bounds__(256) row_absmax_kernel(const float* __restrict__ x, long R, int I,
+                                                         float* __restrict__ out) {
+    const int lane = threadIdx.x & 63;
+    const long wave = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const long n_waves = ((long)gridDim.x * blockDim.x) >> 6;
+    for (long r = wave; r < R; r += n_waves) {
+        const float* row = x + r * I;
+        float m = 0.f;
+        if ((I & 3) == 0) {
+            for (int i = lane * 4; i < I; i += 256) {
+                const float4 v = *reinterpret_cast<const float4*>(row + i);
+                m = fmaxf(fmaxf(m, fmaxf(fabsf(v.x), fabsf(v.y))), fmaxf(fabsf(v.z), fabsf(v.w)));
+            }
+        } else {
+            for (int i = lane; i < I; i += 64) m = fmaxf(m, fabsf(row[i]));
+        }
+        for (int d = 1; d < 64; d <<= 1) m = fmaxf(m, __shfl_xor(m, d));
+        if (lane == 0) out[r] = m;
+    }
+}
+
+struct StageRegs {
+    float4 x[2];       // 2 rows x 4 consecutive k (fp32)
+    halfx8 w[2];       // one 16-byte piece of each W plane
+};
+
+template <int WM, int NI>
+__global__ void __launch_bounds__(128 * WM)
+linear_rows_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restrict__ w_inv, const float* __restrict__ X,
+                         const float* __restrict__ xmax, int xmax_parts, long xmax_stride, long R, int I, int O, int O_pad,
+                         const float* __restrict__ bias, int act, int accumulate, float* __restrict__ Y,
+                         float* __restrict__ ymax, int tiles_n, long tiles_total, int out_T) {
+    static_assert(WM == NI, "the W staging assumes one 16-byte piece per plane and thread");
+    constexpr int TM = 64 * WM, TN = 64 * NI;
+    constexpr int kPlaneX = TM * kRow, kPlaneW = TN * kRow;
+    constexpr int kBuf = 2 * kPlaneX + 2 * kPlaneW;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kBuf];
+    __shared__ float inv_sx[TM];
+
+    const long bid = blockIdx.x;
+    const long per_xcd = (tiles_total + 7) / 8;
+    const long logical = (bid % 8) * per_xcd + bid / 8;
+    if (logical >= tiles_total) return;
+    const long tile_m = logical / tiles_n;
+    const int tile_n = (int)(logical - tile_m * tiles_n);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int wave_m = wave >> 1, wave_n = wave & 1;
+    const long r0 = tile_m * TM;
+    const int n0 = tile_n * TN;
+    const int kgroup = lane >> 5;
+    const long plane_elems = (long)O_pad * I;
+
+    floatx16 acc[2][NI];
+#pragma unroll
+    for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+        for (int ni = 0; ni < NI; ni++)
+#pragma unroll
+            for (int q = 0; q < 16; q++) acc[mi][ni][q] = 0.f;
+
+    // x tile of a slab: TM rows x 16 floats: thread -> rows (tid>>2) and (tid>>2) + TM/2, k = (tid&3)*4
+    const int xr = tid >> 2, xc = (tid & 3) * 4;
+    // W tile: 2 planes x TN rows x 32 B: thread -> row (tid>>1), half (tid&1), both planes
+    const int wr = tid >> 1, wc = (tid & 1) * 8;
+    const int k_last = I - kBK;
+
+    float sx[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const long r = r0 + xr + (TM / 2) * h;
+        float amax = 0.f;
+        if (r < R)
+            for (int p = 0; p < xmax_parts; p++) amax = fmaxf(amax, xmax[r * xmax_stride + p]);
+        float inv;
+        sx[h] = pow2_scale(amax, &inv);
+        if ((tid & 3) == 0) inv_sx[xr + (TM / 2) * h] = inv;
+    }
+
+    // Rows past the end of x are clamped to the last row instead of being predicated: their
+    // accumulators are never written, and a loop body without branches lets every load stay in
+    // flight until the slab that needs it (a conditional load forces a full drain of the queue).
+    const float* xrow[2];
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const long r = r0 + xr + (TM / 2) * h;
+        xrow[h] = X + (r < R ? r : R - 1) * I + xc;
+    }
+    const _Float16* wrow = Wp + (long)(n0 + wr) * I + wc;
+    auto load_stage = [&](StageRegs& g, int k0) {
+        k0 = k0 < I ? k0 : k_last;                   // clamped: the surplus loads of the last trips are never used
+#pragma unroll
+        for (int h = 0; h < 2; h++) g.x[h] = *reinterpret_cast<const float4*>(xrow[h] + k0);
+#pragma unroll
+        for (int p = 0; p < 2; p++) g.w[p] = *reinterpret_cast<const halfx8*>(wrow + p * plane_elems + k0);
+    };
+    auto store_stage = [&](const StageRegs& g, unsigned char* buf) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const HalfSplit4 s = split(g.x[h], sx[h]);
+            const int off = (xr + (TM / 2) * h) * kRow + xc * 2;
+            *reinterpret_cast<halfx4*>(buf + off) = s.hi;
+            *reinterpret_cast<halfx4*>(buf + kPlaneX + off) = s.lo;
+        }
+#pragma unroll
+        for (int p = 0; p < 2; p++)
+            *reinterpret_cast<halfx8*>(buf + 2 * kPlaneX + p * kPlaneW + wr * kRow + wc * 2) = g.w[p];
+    };
+
+    int a_off[2], b_off[NI];
+#pragma unroll
+    for (int i = 0; i < 2; i++) a_off[i] = ((wave_m * 2 + i) * 32 + (lane & 31)) * kRow + kgroup * 16;
+#pragma unroll
+    for (int i = 0; i < NI; i++) b_off[i] = 2 * kPlaneX + ((wave_n * NI + i) * 32 + (lane & 31)) * kRow + kgroup * 16;
+
+    auto compute = [&](const unsigned char* buf) {
+        halfx8 a[2][2];
+#pragma unroll
+        for (int i = 0; i < 2; i++)
+#pragma unroll
+            for (int p = 0; p < 2; p++) a[i][p] = *reinterpret_cast<const halfx8*>(buf + p * kPlaneX + a_off[i]);
+#pragma unroll
+        for (int nh = 0; nh < NI / 2; nh++) {
+            halfx8 b[2][2];
+#pragma unroll
+            for (int i = 0; i < 2; i++)
+#pragma unroll
+                for (int p = 0; p < 2; p++)
+                    b[i][p] = *reinterpret_cast<const halfx8*>(buf + p * kPlaneW + b_off[nh * 2 + i]);
+            // small terms first; each round goes over the four independent accumulators
+#pragma unroll
+            for (int t = 0; t < 3; t++) {
+                constexpr int pa[3] = {1, 0, 0};   // lo*hi, hi*lo, hi*hi
+                constexpr int pb[3] = {0, 1, 0};
+#pragma unroll
+                for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+                    for (int nj = 0; nj < 2; nj++)
+                        acc[mi][nh * 2 + nj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi][pa[t]], b[nj][pb[t]],
+                                                                                      acc[mi][nh * 2 + nj], 0, 0, 0);
+            }
+        }
+    };
+
+    unsigned char* buf0 = lds;
+    unsigned char* buf1 = lds + kBuf;
+    // Waves w and w + 4 (w + 2 in the four-wave shape) share a SIMD.  The upper half stages the
+    // next slab before its MFMAs, the lower half after: while one wave of a SIMD splits and
+    // stores, the other keeps the matrix pipe busy.
+    const bool store_first = __builtin_amdgcn_readfirstlane(wave) >= WM;
+    StageRegs ga, gb;
+    load_stage(ga, 0);
+    load_stage(gb, kBK);
+    store_stage(ga, buf0);
+    load_stage(ga, 2 * kBK);
+    // I is a multiple of 32: slabs are handled in pairs (even slab in buf0, odd slab in buf1).
+    // One branch-free loop per staging position.
+    auto main_loop = [&](auto first) {
+        constexpr bool kFirst = decltype(first)::value;
+        for (int k0 = 0; k0 < I; k0 += 2 * kBK) {
+            __syncthreads();
+            if constexpr (kFirst) {
+                store_stage(gb, buf1);
+                load_stage(gb, k0 + 3 * kBK);
+            }
+            compute(buf0);
+            if constexpr (!kFirst) {
+                store_stage(gb, buf1);
+                load_stage(gb, k0 + 3 * kBK);
+            }
+            __syncthreads();
+            if constexpr (kFirst) {
+                store_stage(ga, buf0);
+                load_stage(ga, k0 + 4 * kBK);
+            }
+            compute(buf1);
+            if constexpr (!kFirst) {
+                store_stage(ga, buf0);
+                load_stage(ga, k0 + 4 * kBK);
+            }
+        }
+    };
+    if (store_first) main_loop(std::true_type{});
+    else main_loop(std::false_type{});
+
+    auto epilogue = [&](auto plain) {
+        constexpr bool kPlain = decltype(plain)::value;
+        float rmax[2][16];
+#pragma unroll
+        for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+            for (int q = 0; q < 16; q++) rmax[mi][q] = 0.f;
+#pragma unroll
+        for (int ni = 0; ni < NI; ni++) {
+            const int n = n0 + (wave_n * NI + ni) * 32 + (lane & 31);
+            if (n >= O) continue;
+            const float bv = bias ? bias[n] : 0.f;
+            const float iw = w_inv[n];
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++) {
+#pragma unroll
+                for (int q = 0; q < 16; q++) {
+                    const int rl = (wave_m * 2 + mi) * 32 + 8 * (q / 4) + 4 * kgroup + (q % 4);
+                    const long r = r0 + rl;
+                    if (r < R) {
+                        long addr;
+                        if constexpr (kPlain) {
+                            addr = r * O + n;
+                        } else {   // rows are (row, comp) pairs, output stored (row, chan, comp)
+                            const long row = r / out_T;
+                            addr = (row * O + n) * out_T + (r - row * out_T);
+                        }
+                        float v = activate(acc[mi][ni][q] * inv_sx[rl] * iw + bv, act);
+                        if (accumulate) v += Y[addr];
+                        Y[addr] = v;
+                        rmax[mi][q] = fmaxf(rmax[mi][q], fabsf(v));
+                    }
+                }
+            }
+        }
+        if (ymax) {
+            const int parts = tiles_n * 2;
+            const int part = tile_n * 2 + wave_n;
+#pragma unroll
+            for (int mi = 0; mi < 2; mi++)
+#pragma unroll
+                for (int q = 0; q < 16; q++) {
+                    float m = rmax[mi][q];
+#pragma unroll
+                    for (int d = 1; d < 32; d <<= 1) m = fmaxf(m, __shfl_xor(m, d));
+                    const long r = r0 + (wave_m * 2 + mi) * 32 + 8 * (q / 4) + 4 * kgroup + (q % 4);
+                    if ((lane & 31) == 0 && r < R) ymax[r * parts + part] = m;
+                }
+        }
+    };
+    if (out_T == 1) epilogue(std::true_type{});
+    else epilogue(std::false_type{});
+}
+
+inline int o_pad_of(int dim_out) { return (dim_out + 255) / 256 * 256; }
+inline bool use_wide(long R, int O) { return ceil_div(R, 256) * ceil_div(O, 256) >= 512; }
+
+}  // namespace
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" {
+
+int mg_linear_f16x2_packed_weight_bytes(int dim_in, int dim_out, size_t* bytes) {
+    MG_REQUIRE(bytes != nullptr && dim_in >= 0 && dim_out >= 0, "mg_linear_f16x2_packed_weight_bytes: bad argument");
+    const size_t o_pad = (size_t)o_pad_of(dim_out);
+    *bytes = 2 * o_pad * (size_t)dim_in * sizeof(_Float16) + o_pad * sizeof(float);
+    return MG_OK;
+}
+
+int mg_linear_f16x2_pack_weight(const float* W, long w_stride_o, long w_stride_i, int dim_in, int dim_out,
+                                void* packed, mg_stream_t stream) {
+    MG_REQUIRE(dim_in >= 0 && dim_out >= 0, "mg_linear_f16x2_pack_weight: negative size");
+    if (dim_in == 0 || dim_out == 0) return MG_OK;
+    MG_REQUIRE(W && packed && aligned16(packed), "mg_linear_f16x2_pack_weight: null or unaligned pointer");
+    MG_REQUIRE(dim_in % 8 == 0, "mg_linear_f16x2_pack_weight: dim_in must be a multiple of 8");
+    const int O_pad = o_pad_of(dim_out);
+    _Float16* planes = static_cast<_Float16*>(packed);
+    float* inv = reinterpret_cast<float*>(planes + 2L * O_pad * dim_in);
+    hipLaunchKernelGGL(pack_weight_f16x2_kernel, dim3((unsigned)ceil_div(O_pad, 4)), dim3(256), 0, (hipStream_t)stream,
+                       W, w_stride_o, w_stride_i, dim_in, dim_out, O_pad, planes, inv);
+    return check_launch("mg_linear_f16x2_pack_weight");
+}
+
+int mg_row_absmax(const float* x, long rows, int dim, float* out, mg_stream_t stream) {
+    MG_REQUIRE(rows >= 0 && dim >= 0, "mg_row_absmax: negative size");
+    if (rows == 0) return MG_OK;
+    MG_REQUIRE(out && (x || dim == 0), "mg_row_absmax: null pointer");
+    MG_REQUIRE(dim % 4 != 0 || aligned16(x), "mg_row_absmax: x must be 16-byte aligned");
+    long blocks = ceil_div(rows, 4);
+    if (blocks > 256L * 32) blocks = 256L * 32;
+    hipLaunchKernelGGL(row_absmax_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, x, rows, dim, out);
+    return check_launch("mg_row_absmax");
+}
+
+int mg_tensor_linear_f16x2_rowmax_parts(long rows, int dim_out) {
+    return use_wide(rows, dim_out) ? 2 * (int)ceil_div(dim_out, 256) : 2 * (int)ceil_div(dim_out, 128);
+}
+
+int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts, long x_rowmax_stride,
+                           long rows,
+                           int dim_in, int dim_out, const float* bias, int act, int accumulate, int out_comps,
+                           float* y, float* y_rowmax, mg_stream_t stream) {
+    MG_REQUIRE(rows >= 0 && dim_in > 0 && dim_out >= 0, "mg_tensor_linear_f16x2: bad size");
+    MG_REQUIRE(dim_in % 32 == 0, "mg_tensor_linear_f16x2: dim_in must be a multiple of 32");
+    MG_REQUIRE(act >= 0 && act <= 2, "mg_tensor_linear_f16x2: unknown activation %d", act);
+    MG_REQUIRE(out_comps == 1 || out_comps == 3 || out_comps == 9, "mg_tensor_linear_f16x2: out_comps must be 1, 3 or 9");
+    MG_REQUIRE(x_rowmax_parts >= 1 && x_rowmax_parts <= 64, "mg_tensor_linear_f16x2: x_rowmax_parts must be in 1..64");
+    MG_REQUIRE(x_rowmax_stride == 0 || x_rowmax_stride >= x_rowmax_parts,
+               "mg_tensor_linear_f16x2: x_rowmax_stride must be 0 (one bound for all rows) or >= x_rowmax_parts");
+    MG_REQUIRE(y_rowmax == nullptr || out_comps == 1, "mg_tensor_linear_f16x2: y_rowmax needs out_comps == 1");
+    if (rows == 0 || dim_out == 0) return MG_OK;
+    MG_REQUIRE(packed_W && x && y && x_rowmax && aligned16(x) && aligned16(packed_W),
+               "mg_tensor_linear_f16x2: null or unaligned pointer");
+    const int O_pad = o_pad_of(dim_out);
+    const _Float16* planes = static_cast<const _Float16*>(packed_W);
+    const float* w_inv = reinterpret_cast<const float*>(planes + 2L * O_pad * dim_in);
+    hipStream_t st = (hipStream_t)stream;
+    if (use_wide(rows, dim_out)) {
+        const long tiles_m = ceil_div(rows, 256);
+        const int tiles_n = (int)ceil_div(dim_out, 256);
+        const long total = tiles_m * tiles_n;
+        const long grid = ceil_div(total, 8) * 8;
+        MG_REQUIRE(grid <= 0x7fffffffL, "mg_tensor_linear_f16x2: grid too large (rows=%ld dim_out=%d)", rows, dim_out);
+        hipLaunchKernelGGL((linear_rows_f16x2_kernel<4, 4>), dim3((unsigned)grid), dim3(512), 0, st, planes, w_inv, x,
+                           x_rowmax, x_rowmax_parts, x_rowmax_stride, rows, dim_in, dim_out, O_pad, bias, act, accumulate, y, y_rowmax,
+                           tiles_n, total, out_comps);
+    } else {
+        const long tiles_m = ceil_div(rows, 128);
+        const int tiles_n = (int)ceil_div(dim_out, 128);
+        const long total = tiles_m * tiles_n;
+        const long grid = ceil_div(total, 8) * 8;
+        MG_REQUIRE(grid <= 0x7fffffffL, "mg_tensor_linear_f16x2: grid too large (rows=%ld dim_out=%d)", rows, dim_out);
+        hipLaunchKernelGGL((linear_rows_f16x2_kernel<2, 2>), dim3((unsigned)grid), dim3(256), 0, st, planes, w_inv, x,
+                           x_rowmax, x_rowmax_parts, x_rowmax_stride, rows, dim_in, dim_out, O_pad, bias, act, accumulate, y, y_rowmax,
+                           tiles_n, total, out_comps);
+    }
+    return check_launch("mg_tensor_linear_f16x2");
+}
+
+}  // extern "C"

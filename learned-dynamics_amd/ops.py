@@ -412,11 +412,13 @@ def tensor_prods_avd(a, v_l, v_r):
 
 
 ACT_NONE, ACT_SILU, ACT_LEAKY = 0, 1, 2
-LINEAR_FP32_MFMA, LINEAR_BF16X3 = 0, 1
+LINEAR_FP32_MFMA, LINEAR_BF16X3, LINEAR_F16X2 = 0, 1, 2
 
 
 def set_linear_mode(mode):
-    """0: fp32 MFMA; 1: bf16x3-split operands on the bf16 MFMA (fp32-class accuracy, faster)."""
+    """0: fp32 MFMA; 1: bf16x3-split operands on the bf16 MFMA (fp32-class accuracy, faster);
+    2 (default): two-piece fp16 split with per-row scales where the layer shape allows (a few fp32
+    ulps per product, half the matrix work of mode 1), mode 1 elsewhere."""
     L.check(_lib.mg_set_linear_mode(int(mode)))
 
 
@@ -427,21 +429,22 @@ def get_linear_mode():
 _packed_cache = {}
 
 
-def packed_weight(W):
-    """bf16x3 planes of W for mg_tensor_linear_packed.  Cached per tensor OBJECT (weak reference) and
-    version counter, so parameters are packed once and re-packed after an in-place update; a new
-    tensor that happens to reuse a freed address never hits a stale entry."""
-    key = id(W)
+def _packed(W, kind):
+    """Pre-split planes of W for the packed GEMM entry points.  Cached per tensor OBJECT (weak
+    reference) and version counter, so parameters are packed once and re-packed after an in-place
+    update; a new tensor that happens to reuse a freed address never hits a stale entry."""
+    key = (id(W), kind)
     hit = _packed_cache.get(key)
     if hit is not None and hit[0]() is W and hit[1] == W._version and hit[2] == (W.data_ptr(), tuple(W.stride())):
         return hit[3]
     dim_out, dim_in = int(W.size(0)), int(W.size(1))
     nbytes = ctypes.c_size_t(0)
-    L.check(_lib.mg_linear_packed_weight_bytes(dim_in, dim_out, ctypes.byref(nbytes)))
+    size_fn, pack_fn = ((_lib.mg_linear_packed_weight_bytes, _lib.mg_linear_pack_weight) if kind == "bf16x3" else
+                        (_lib.mg_linear_f16x2_packed_weight_bytes, _lib.mg_linear_f16x2_pack_weight))
+    L.check(size_fn(dim_in, dim_out, ctypes.byref(nbytes)))
     with torch.cuda.device(W.device):
         packed = torch.empty(nbytes.value, dtype=torch.uint8, device=W.device)
-        L.check(_lib.mg_linear_pack_weight(_p(W), int(W.stride(0)), int(W.stride(1)), dim_in, dim_out, _p(packed),
-                                           _stream()))
+        L.check(pack_fn(_p(W), int(W.stride(0)), int(W.stride(1)), dim_in, dim_out, _p(packed), _stream()))
     if len(_packed_cache) > 512:
         for k in [k for k, v in _packed_cache.items() if v[0]() is None]:
             del _packed_cache[k]
@@ -449,6 +452,120 @@ def packed_weight(W):
             _packed_cache.clear()
     _packed_cache[key] = (weakref.ref(W), W._version, (W.data_ptr(), tuple(W.stride())), packed)
     return packed
+
+
+def packed_weight(W):
+    """bf16x3 planes of W for mg_tensor_linear_packed."""
+    return _packed(W, "bf16x3")
+
+
+def packed_weight_f16x2(W):
+    """fp16 hi/lo planes + per-row inverse scales of W for mg_tensor_linear_f16x2."""
+    return _packed(W, "f16x2")
+
+
+def row_absmax(x):
+    """(rows, dim) -> (rows, 1): max_i |x[r, i]|, the row bounds mg_tensor_linear_f16x2 scales by."""
+    _check_input(x, "x")
+    if x.dim() != 2:
+        raise RuntimeError("x must have two dims")
+    with torch.cuda.device(x.device):
+        out = torch.empty(x.size(0), 1, dtype=torch.float32, device=x.device)
+        L.check(_lib.mg_row_absmax(_p(x), int(x.size(0)), int(x.size(1)), _p(out), _stream()))
+    return out
+
+
+_bound_cache = {}
+
+
+def linear_in_unit_bound(device):
+    """(1, 1) bound for inputs whose entries are at most 1 in magnitude (sines, cosines, one-hots)."""
+    key = ("unit", str(device))
+    hit = _bound_cache.get(key)
+    if hit is None:
+        hit = _bound_cache[key] = torch.ones(1, 1, dtype=torch.float32, device=device)
+    return hit
+
+
+def linear_out_bound(W, bias, in_bound):
+    """Upper bound of |act(x W^T + bias)| per row, given upper bounds in_bound ((rows, 1) or (1, 1);
+    None: entries of x are at most 1 in magnitude) of |x| per row, for any act with |act(z)| <= |z|
+    (identity, SiLU, LeakyReLU):  |y[r, o]| <= in_bound[r] * max_o sum_i |W[o, i]| + max_o |bias[o]|.
+    The two weight norms are cached per parameter object and version (device tensors; no host
+    synchronisation).  These bounds feed mg_tensor_linear_f16x2, whose accuracy does not depend on
+    how tight they are as long as they stay within a factor 2^14 of the true row maxima."""
+    if in_bound is None:
+        in_bound = linear_in_unit_bound(W.device)
+    key = ("norms", id(W), id(bias))
+    hit = _bound_cache.get(key)
+    if (hit is None or hit[0]() is not W or hit[1] != W._version
+            or (bias is not None and (hit[2]() is not bias or hit[3] != bias._version))):
+        with torch.no_grad():
+            l1 = W.detach().abs().sum(dim=1).amax().reshape(1, 1)
+            bmax = bias.detach().abs().amax().reshape(1, 1) if bias is not None else torch.zeros_like(l1)
+        hit = (weakref.ref(W), W._version, weakref.ref(bias) if bias is not None else None,
+               bias._version if bias is not None else 0, l1, bmax, {})
+        if len(_bound_cache) > 1024:
+            _bound_cache.clear()
+        _bound_cache[key] = hit
+    l1, bmax, per_input = hit[4], hit[5], hit[6]
+    if in_bound.numel() == 1:
+        # a constant input bound (cached tensor object) gives a constant output bound: computed once
+        memo = per_input.get(id(in_bound))
+        if memo is not None and memo[0]() is in_bound:
+            return memo[1]
+        out = torch.addcmul(bmax, in_bound.reshape(1, 1), l1)
+        if len(per_input) > 16:
+            per_input.clear()
+        per_input[id(in_bound)] = (weakref.ref(in_bound), out)
+        return out
+    return torch.addcmul(bmax, in_bound.reshape(-1, 1), l1)
+
+
+def f16x2_supported(rows, dim_in, dim_out, x):
+    return dim_in % 32 == 0 and dim_in >= 64 and dim_out >= 64 and rows >= 1024 and x.data_ptr() % 16 == 0
+
+
+def tensor_linear_f16x2(W, x, x_rowmax=None, bias=None, act=ACT_NONE, out=None, accumulate=False, out_comps=1,
+                        want_rowmax=False):
+    """y = act(x W^T + bias) for plain rows x (rows, dim_in) through the two-piece fp16 split.
+    x_rowmax (rows, parts), or (1, parts) for one bound shared by all rows: upper bounds of the
+    row maxima of |x| (None: computed here).  Returns y, or (y, y_rowmax) with want_rowmax=True."""
+    _check_input(x, "x")
+    if x.dim() != 2 or W.dim() != 2 or x.size(1) != W.size(1):
+        raise RuntimeError("expected x (rows, dim_in) and W (dim_out, dim_in)")
+    rows, dim_in, dim_out = int(x.size(0)), int(W.size(1)), int(W.size(0))
+    if x_rowmax is None:
+        x_rowmax = row_absmax(x)
+    _check_input(x_rowmax, "x_rowmax")
+    if x_rowmax.dim() != 2 or x_rowmax.size(0) not in (1, rows):
+        raise RuntimeError("x_rowmax must be (rows, parts) or (1, parts)")
+    rowmax_stride = int(x_rowmax.size(1)) if x_rowmax.size(0) == rows and rows > 1 else 0
+    if bias is not None:
+        _check_input(bias, "bias")
+        if bias.numel() != dim_out:
+            raise RuntimeError("bias size mismatch")
+    if rows % out_comps != 0:
+        raise RuntimeError("rows must be a multiple of out_comps")
+    y_shape = [rows, dim_out] if out_comps == 1 else [rows // out_comps, dim_out, out_comps]
+    with torch.cuda.device(x.device):
+        if out is None:
+            y = torch.empty(y_shape, dtype=torch.float32, device=x.device)
+        else:
+            _check_input(out, "out")
+            if out.numel() != rows * dim_out:
+                raise RuntimeError("out has wrong size")
+            y = out
+        ymax = None
+        if want_rowmax:
+            if out_comps != 1:
+                raise RuntimeError("row maxima are only produced for out_comps == 1")
+            parts = int(_lib.mg_tensor_linear_f16x2_rowmax_parts(rows, dim_out))
+            ymax = torch.empty(rows, parts, dtype=torch.float32, device=x.device)
+        L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(W)), _p(x), _p(x_rowmax), int(x_rowmax.size(1)),
+                                            rowmax_stride, rows, dim_in, dim_out, _p(bias), int(act), int(bool(accumulate)),
+                                            int(out_comps), _p(y), _p(ymax), _stream()))
+    return (y, ymax) if want_rowmax else y
 
 
 LAYOUT_CHAN_COMP, LAYOUT_COMP_CHAN = 0, 1
@@ -502,9 +619,16 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
                 raise RuntimeError("out has wrong shape")
             y = out
         plain_rows = inds == 0 or x_layout == LAYOUT_COMP_CHAN
-        if (plain_rows and get_linear_mode() == LINEAR_BF16X3 and dim_in % 32 == 0 and dim_in >= 64
-                and dim_out >= 64 and rows * T >= 1024 and x.data_ptr() % 16 == 0):
-            out_comps = 1 if (inds == 0 or y_layout == LAYOUT_COMP_CHAN) else T
+        mode = get_linear_mode()
+        wide = (plain_rows and dim_in % 32 == 0 and dim_in >= 64 and dim_out >= 64 and rows * T >= 1024
+                and x.data_ptr() % 16 == 0)
+        out_comps = 1 if (inds == 0 or y_layout == LAYOUT_COMP_CHAN) else T
+        if wide and mode == LINEAR_F16X2:
+            x2 = x.reshape(rows * T, dim_in)
+            L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(W)), _p(x2), _p(row_absmax(x2)), 1, 1, rows * T,
+                                                dim_in, dim_out, _p(bias), int(act), int(bool(accumulate)),
+                                                out_comps, _p(y), None, _stream()))
+        elif wide and mode == LINEAR_BF16X3:
             L.check(_lib.mg_tensor_linear_packed(_p(packed_weight(W)), _p(x), rows * T, dim_in, dim_out, _p(bias),
                                                  int(act), int(bool(accumulate)), out_comps, _p(y), _stream()))
         else:

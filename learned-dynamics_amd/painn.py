@@ -28,13 +28,24 @@ def radial_encode(r, n, rmax):
     return ops.painn_radial_encode(r.reshape(-1, 3).contiguous(), n, rmax).reshape(*lead, n)
 
 
-def _linear(x, lin, act):
-    return ops.tensor_linear_fwd(0, lin.weight, x, bias=lin.bias, act=act)
+def _linear(x, lin, act, bound=None):
+    """One nn.Linear with fused bias and activation.  bound: upper bounds of the row maxima of |x|
+    ((rows, 1) or (1, 1)) if the caller knows them.  Returns (y, bound of the rows of |y| or None)."""
+    rows = x.shape[0]
+    if ops.get_linear_mode() == ops.LINEAR_F16X2 and ops.f16x2_supported(rows, lin.in_features, lin.out_features, x):
+        if bound is None:
+            bound = ops.row_absmax(x)
+        y = ops.tensor_linear_f16x2(lin.weight, x, bound, bias=lin.bias, act=act)
+    else:
+        y = ops.tensor_linear_fwd(0, lin.weight, x, bias=lin.bias, act=act)
+    return y, (ops.linear_out_bound(lin.weight, lin.bias, bound) if bound is not None else None)
 
 
 class MLP(nn.Module):
     """Linear, SiLU, Linear, SiLU, Linear (archs/meanflow_painn8.py:38-51); bias and
-    activation are fused into the GEMM epilogue."""
+    activation are fused into the GEMM epilogue.  The wide layers run on the split-fp16 matrix
+    path; the row bounds it scales by are carried from layer to layer through the weight norms
+    (|SiLU(z)| <= |z|), so only the first layer ever looks at the data for them."""
 
     def __init__(self, dim_in, dim_out):
         super().__init__()
@@ -46,16 +57,16 @@ class MLP(nn.Module):
             nn.Linear(dim_out, dim_out),
         )
 
-    def forward(self, x_a):
+    def forward(self, x_a, bound=None):
         lead = x_a.shape[:-1]
         h = x_a.reshape(-1, x_a.shape[-1]).contiguous()
-        h = _linear(h, self.layers[0], ops.ACT_SILU)
-        return self.after_first(h).reshape(*lead, -1)
+        h, bound = _linear(h, self.layers[0], ops.ACT_SILU, bound)
+        return self.after_first(h, bound).reshape(*lead, -1)
 
-    def after_first(self, h):
+    def after_first(self, h, bound=None):
         """Layers 2 and 3 on the (rows, dim_out) output of the first layer + SiLU."""
-        h = _linear(h, self.layers[2], ops.ACT_SILU)
-        return _linear(h, self.layers[4], ops.ACT_NONE)
+        h, bound = _linear(h, self.layers[2], ops.ACT_SILU, bound)
+        return _linear(h, self.layers[4], ops.ACT_NONE, bound)[0]
 
 
 class ScalGroupNorm(nn.Module):
@@ -123,8 +134,9 @@ class Message(nn.Module):
         first = self.mlp_dist.layers[0]
         if ops.painn_radial_linear_supported(self.n_rbf, first.out_features):
             h = ops.painn_radial_linear(r_ij, self.n_rbf, self.r0, first.weight, first.bias, ops.ACT_SILU)
-            return self.mlp_dist.after_first(h)
-        return self.mlp_dist(ops.painn_radial_encode(r_ij, self.n_rbf, self.r0))
+            # the encoding is cosines and sines: entries at most 1
+            return self.mlp_dist.after_first(h, ops.linear_out_bound(first.weight, first.bias, None))
+        return self.mlp_dist(ops.painn_radial_encode(r_ij, self.n_rbf, self.r0), ops.linear_in_unit_bound(r_ij.device))
 
     def forward(self, graph: Graph, x_a, x_v, r_ij, residual=False):
         """x_a: (batch, atoms, n), x_v: (batch, atoms, n, 3), r_ij: (edges, 3).
