@@ -220,7 +220,7 @@ int mg_tensor_linear_packed(const void* packed_W, const float* x, long rows, int
  * largest part is used; any bound within a factor 2^14 of the true maximum keeps full accuracy;
  * stride 0 = one bound for all rows): the y_rowmax output of the call that produced x,
  * mg_row_absmax(x) (one part), or a bound the caller derives from the producing layer's weights.  y_rowmax, if not NULL,
- * receives (rows, mg_tensor_linear_f16x2_rowmax_parts(rows, dim_out)) partial row maxima of |y|
+ * receives (rows, mg_tensor_linear_f16x2_rowmax_parts(rows, dim_in, dim_out)) partial row maxima of |y|
  * (out_comps must be 1).  out_comps / accumulate / act as in mg_tensor_linear_packed.
  * Same contraction as tensor_linear (extensions/tensor_ops/tensor_ops.cpp:31-93); packing, scales
  * and row maxima have no counterpart in the reference. */
@@ -228,7 +228,7 @@ int mg_linear_f16x2_packed_weight_bytes(int dim_in, int dim_out, size_t* bytes /
 int mg_linear_f16x2_pack_weight(const float* W, long w_stride_o, long w_stride_i, int dim_in, int dim_out,
                                 void* packed, mg_stream_t stream);
 int mg_row_absmax(const float* x, long rows, int dim, float* out /* (rows) */, mg_stream_t stream);
-int mg_tensor_linear_f16x2_rowmax_parts(long rows, int dim_out);   /* returns the count, not a status */
+int mg_tensor_linear_f16x2_rowmax_parts(long rows, int dim_in, int dim_out);   /* returns the count, not a status */
 int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts,
                            long x_rowmax_stride, long rows, int dim_in, int dim_out, const float* bias, int act, int accumulate,
                            int out_comps, float* y, float* y_rowmax, mg_stream_t stream);

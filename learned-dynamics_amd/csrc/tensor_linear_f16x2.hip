@@ -49,6 +49,14 @@ __device__ __forceinline__ float pow2_scale(float amax, float* inv) {
     return __uint_as_float((unsigned)se << 23);
 }
 
+template <int ACT>
+__device__ __forceinline__ float activate_c(float v) {
+    // SiLU through the hardware exp2 and reciprocal (about 1 ulp each): far inside the fp32 tolerance
+    if constexpr (ACT == 1) return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
+    if constexpr (ACT == 2) return v > 0.f ? v : 0.1f * v;
+    return v;
+}
+
 struct HalfSplit4 {
     halfx4 hi, lo;
 };
@@ -329,8 +337,234 @@ linear_rows_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restric
     else epilogue(std::false_type{});
 }
 
+// ---------------------------------------------------------------------------
+// Row-streaming variant for large problems: tile 256 x 256, eight waves, wave w owns rows
+// [32 w, 32 w + 32) of the tile and ALL 256 columns.
+//   * x never touches LDS: a lane loads the 16 consecutive floats of ITS row that it will feed to
+//     the matrix core (lane = row + 32 g holds k = 32 c + 16 g .. + 16 of chunk c: 64 contiguous
+//     bytes, four 16-byte loads), two chunks ahead, and splits them in registers.  Every row is
+//     loaded and split exactly once per tile, nothing about x is tied to a barrier, and the LDS
+//     carries only W.
+//   * W planes (already fp16) go global -> registers -> LDS, double buffered, K chunk 32 (rows of
+//     64 B padded to 80 B: conflict free for 16-byte reads), one barrier per chunk.
+//   * the k order inside a chunk is a permutation (MFMA step s takes k = 16 g + 8 s .. + 8 from
+//     lane group g); W is read from LDS with the same permutation, so the products pair up.
+constexpr int kCK = 32;                     // k per chunk (two MFMA steps)
+constexpr int kRowW = 80;                   // bytes per LDS row of one W plane
+constexpr int kPlaneWQ = 256 * kRowW;
+constexpr int kBufWQ = 2 * kPlaneWQ;
+
+__global__ void __launch_bounds__(512)
+linear_rows_f16x2_stream_kernel(const _Float16* __restrict__ Wp, const float* __restrict__ w_inv,
+                                const float* __restrict__ X, const float* __restrict__ xmax, int xmax_parts,
+                                long xmax_stride, long R, int I, int O, int O_pad, const float* __restrict__ bias,
+                                int act, int accumulate, float* __restrict__ Y, float* __restrict__ ymax, int tiles_n,
+                                long tiles_total, int out_T) {
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kBufWQ];
+    __shared__ float inv_sx[256];
+
+    const long bid = blockIdx.x;
+    const long per_xcd = (tiles_total + 7) / 8;
+    const long logical = (bid % 8) * per_xcd + bid / 8;
+    if (logical >= tiles_total) return;
+    const long tile_m = logical / tiles_n;
+    const int tile_n = (int)(logical - tile_m * tiles_n);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int m = lane & 31, g = lane >> 5;
+    const long r0 = tile_m * 256;
+    const int n0 = tile_n * 256;
+    const long plane_elems = (long)O_pad * I;
+
+    floatx16 acc[8];
+#pragma unroll
+    for (int ni = 0; ni < 8; ni++)
+#pragma unroll
+        for (int q = 0; q < 16; q++) acc[ni][q] = 0.f;
+
+    // this lane's row of x (clamped past the end: those accumulators are never written)
+    const long my_row = r0 + wave * 32 + m;
+    const long ld_row = my_row < R ? my_row : R - 1;
+    const float* xrow = X + ld_row * I + 16 * g;
+    float sx;
+    {
+        float amax = 0.f;
+        for (int p = 0; p < xmax_parts; p++) amax = fmaxf(amax, xmax[ld_row * xmax_stride + p]);
+        float inv;
+        sx = pow2_scale(amax, &inv);
+        if (g == 0) inv_sx[wave * 32 + m] = inv;
+    }
+    // W staging: 2 planes x 256 rows x 64 B per chunk = 2048 pieces of 16 B, four per thread
+    const _Float16* wsrc[4];
+    int wdst[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const int q = tid + 512 * j;
+        const int plane = q >> 10, row = (q & 1023) >> 2, piece = q & 3;
+        wsrc[j] = Wp + plane * plane_elems + (long)(n0 + row) * I + 8 * piece;
+        wdst[j] = plane * kPlaneWQ + row * kRowW + piece * 16;
+    }
+    const int k_last = I - kCK;
+
+    struct ARegs { float4 v[4]; };
+    struct WRegs { halfx8 v[4]; };
+    auto load_a = [&](ARegs& a, int k0) {
+        k0 = k0 < I ? k0 : k_last;
+#pragma unroll
+        for (int j = 0; j < 4; j++) a.v[j] = *reinterpret_cast<const float4*>(xrow + k0 + 4 * j);
+    };
+    auto load_w = [&](WRegs& w, int k0) {
+        k0 = k0 < I ? k0 : k_last;
+#pragma unroll
+        for (int j = 0; j < 4; j++) w.v[j] = *reinterpret_cast<const halfx8*>(wsrc[j] + k0);
+    };
+    auto store_w = [&](const WRegs& w, unsigned char* buf) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) *reinterpret_cast<halfx8*>(buf + wdst[j]) = w.v[j];
+    };
+    const int b_off = m * kRowW + 32 * g;
+    auto compute = [&](const ARegs& a, const unsigned char* buf) {
+        halfx8 ah[2], al[2];
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const HalfSplit4 p0 = split(a.v[2 * s], sx), p1 = split(a.v[2 * s + 1], sx);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                ah[s][i] = p0.hi[i]; ah[s][4 + i] = p1.hi[i];
+                al[s][i] = p0.lo[i]; al[s][4 + i] = p1.lo[i];
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 2; s++)
+#pragma unroll
+            for (int ni = 0; ni < 8; ni++) {
+                const halfx8 bh = *reinterpret_cast<const halfx8*>(buf + b_off + ni * 32 * kRowW + 16 * s);
+                const halfx8 bl = *reinterpret_cast<const halfx8*>(buf + kPlaneWQ + b_off + ni * 32 * kRowW + 16 * s);
+                acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[s], bh, acc[ni], 0, 0, 0);
+                acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[s], bl, acc[ni], 0, 0, 0);
+                acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[s], bh, acc[ni], 0, 0, 0);
+            }
+    };
+
+    unsigned char* buf0 = lds;
+    unsigned char* buf1 = lds + kBufWQ;
+    ARegs a0, a1;
+    WRegs w;
+    load_w(w, 0);
+    load_a(a0, 0);
+    store_w(w, buf0);
+    load_w(w, kCK);
+    load_a(a1, kCK);
+    __syncthreads();
+    // I is a multiple of 64 here: chunks in pairs (even chunk: a0 / buf0, odd chunk: a1 / buf1)
+    for (int k0 = 0; k0 < I; k0 += 2 * kCK) {
+        // W (L2 resident, needed one chunk later) is requested before x (HBM, needed two chunks
+        // later): loads return in order, so the wait for W never includes the youngest x loads
+        compute(a0, buf0);
+        store_w(w, buf1);
+        __builtin_amdgcn_sched_barrier(0);     // keep this issue order: the compiler would hoist the loads
+        load_w(w, k0 + 2 * kCK);
+        __builtin_amdgcn_sched_barrier(0);
+        load_a(a0, k0 + 2 * kCK);
+        __syncthreads();
+        compute(a1, buf1);
+        store_w(w, buf0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(w, k0 + 3 * kCK);
+        __builtin_amdgcn_sched_barrier(0);
+        load_a(a1, k0 + 3 * kCK);
+        __syncthreads();
+    }
+
+    // Fast path (plain rows, full tile of columns, no accumulate): one row pointer, row scale and
+    // bounds check per accumulator row, column offsets as immediates, activation chosen at compile
+    // time.  The epilogue runs once per tile with nothing to overlap it, so its instruction count
+    // is what matters.
+    auto epilogue_fast = [&](auto act_tag) {
+        constexpr int kAct = decltype(act_tag)::value;
+        float bv[8], iw[8];
+#pragma unroll
+        for (int ni = 0; ni < 8; ni++) {
+            bv[ni] = bias ? bias[n0 + ni * 32 + m] : 0.f;
+            iw[ni] = w_inv[n0 + ni * 32 + m];
+        }
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+            const int rl = wave * 32 + 8 * (q / 4) + 4 * g + (q % 4);
+            const long r = r0 + rl;
+            if (r < R) {
+                float* yrow = Y + r * O + n0 + m;
+                const float isx = inv_sx[rl];
+                float mx = 0.f;
+#pragma unroll
+                for (int ni = 0; ni < 8; ni++) {
+                    const float v = activate_c<kAct>(acc[ni][q] * isx * iw[ni] + bv[ni]);
+                    yrow[ni * 32] = v;
+                    mx = fmaxf(mx, fabsf(v));
+                }
+                if (ymax) {
+#pragma unroll
+                    for (int d = 1; d < 32; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+                    if (m == 0) ymax[r * tiles_n + tile_n] = mx;
+                }
+            }
+        }
+    };
+    if (out_T == 1 && !accumulate && n0 + 256 <= O) {
+        if (act == 1) epilogue_fast(std::integral_constant<int, 1>{});
+        else if (act == 2) epilogue_fast(std::integral_constant<int, 2>{});
+        else epilogue_fast(std::integral_constant<int, 0>{});
+        return;
+    }
+
+    auto epilogue = [&](auto plain) {
+        constexpr bool kPlain = decltype(plain)::value;
+        float rmax[16];
+#pragma unroll
+        for (int q = 0; q < 16; q++) rmax[q] = 0.f;
+#pragma unroll
+        for (int ni = 0; ni < 8; ni++) {
+            const int n = n0 + ni * 32 + m;
+            if (n >= O) continue;
+            const float bv = bias ? bias[n] : 0.f;
+            const float iw = w_inv[n];
+#pragma unroll
+            for (int q = 0; q < 16; q++) {
+                const int rl = wave * 32 + 8 * (q / 4) + 4 * g + (q % 4);
+                const long r = r0 + rl;
+                if (r < R) {
+                    long addr;
+                    if constexpr (kPlain) {
+                        addr = r * O + n;
+                    } else {   // rows are (row, comp) pairs, output stored (row, chan, comp)
+                        const long row = r / out_T;
+                        addr = (row * O + n) * out_T + (r - row * out_T);
+                    }
+                    float v = activate(acc[ni][q] * inv_sx[rl] * iw + bv, act);
+                    if (accumulate) v += Y[addr];
+                    Y[addr] = v;
+                    rmax[q] = fmaxf(rmax[q], fabsf(v));
+                }
+            }
+        }
+        if (ymax) {
+#pragma unroll
+            for (int q = 0; q < 16; q++) {
+                float mx = rmax[q];
+#pragma unroll
+                for (int d = 1; d < 32; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+                const long r = r0 + wave * 32 + 8 * (q / 4) + 4 * g + (q % 4);
+                if (m == 0 && r < R) ymax[r * tiles_n + tile_n] = mx;
+            }
+        }
+    };
+    if (out_T == 1) epilogue(std::true_type{});
+    else epilogue(std::false_type{});
+}
+
 inline int o_pad_of(int dim_out) { return (dim_out + 255) / 256 * 256; }
-inline bool use_wide(long R, int O) { return ceil_div(R, 256) * ceil_div(O, 256) >= 512; }
+inline bool use_wide(long R, int I, int O) { return I % 64 == 0 && ceil_div(R, 256) * ceil_div(O, 256) >= 512; }
 
 }  // namespace
 }  // namespace mg
@@ -371,8 +605,8 @@ int mg_row_absmax(const float* x, long rows, int dim, float* out, mg_stream_t st
     return check_launch("mg_row_absmax");
 }
 
-int mg_tensor_linear_f16x2_rowmax_parts(long rows, int dim_out) {
-    return use_wide(rows, dim_out) ? 2 * (int)ceil_div(dim_out, 256) : 2 * (int)ceil_div(dim_out, 128);
+int mg_tensor_linear_f16x2_rowmax_parts(long rows, int dim_in, int dim_out) {
+    return use_wide(rows, dim_in, dim_out) ? (int)ceil_div(dim_out, 256) : 2 * (int)ceil_div(dim_out, 128);
 }
 
 int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts, long x_rowmax_stride,
@@ -394,13 +628,13 @@ int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_
     const _Float16* planes = static_cast<const _Float16*>(packed_W);
     const float* w_inv = reinterpret_cast<const float*>(planes + 2L * O_pad * dim_in);
     hipStream_t st = (hipStream_t)stream;
-    if (use_wide(rows, dim_out)) {
+    if (use_wide(rows, dim_in, dim_out)) {
         const long tiles_m = ceil_div(rows, 256);
         const int tiles_n = (int)ceil_div(dim_out, 256);
         const long total = tiles_m * tiles_n;
         const long grid = ceil_div(total, 8) * 8;
         MG_REQUIRE(grid <= 0x7fffffffL, "mg_tensor_linear_f16x2: grid too large (rows=%ld dim_out=%d)", rows, dim_out);
-        hipLaunchKernelGGL((linear_rows_f16x2_kernel<4, 4>), dim3((unsigned)grid), dim3(512), 0, st, planes, w_inv, x,
+        hipLaunchKernelGGL(linear_rows_f16x2_stream_kernel, dim3((unsigned)grid), dim3(512), 0, st, planes, w_inv, x,
                            x_rowmax, x_rowmax_parts, x_rowmax_stride, rows, dim_in, dim_out, O_pad, bias, act, accumulate, y, y_rowmax,
                            tiles_n, total, out_comps);
     } else {

@@ -560,7 +560,7 @@ def tensor_linear_f16x2(W, x, x_rowmax=None, bias=None, act=ACT_NONE, out=None, 
         if want_rowmax:
             if out_comps != 1:
                 raise RuntimeError("row maxima are only produced for out_comps == 1")
-            parts = int(_lib.mg_tensor_linear_f16x2_rowmax_parts(rows, dim_out))
+            parts = int(_lib.mg_tensor_linear_f16x2_rowmax_parts(rows, dim_in, dim_out))
             ymax = torch.empty(rows, parts, dtype=torch.float32, device=x.device)
         L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(W)), _p(x), _p(x_rowmax), int(x_rowmax.size(1)),
                                             rowmax_stride, rows, dim_in, dim_out, _p(bias), int(act), int(bool(accumulate)),
