@@ -216,9 +216,10 @@ int mg_tensor_linear_packed(const void* packed_W, const float* x, long rows, int
  * mg_linear_f16x2_pack_weight: W -> hi / lo fp16 planes (dim_out rounded up to 256 rows) followed by
  * one fp32 inverse scale per row, in caller-owned memory of mg_linear_f16x2_packed_weight_bytes bytes.
  * mg_tensor_linear_f16x2: y = act(x W^T + bias) for plain rows x (rows, dim_in), dim_in % 32 == 0;
- * x_rowmax[r * x_rowmax_stride + p], p < x_rowmax_parts, holds upper bounds of max_i |x[r,i]| (the
- * largest part is used; any bound within a factor 2^14 of the true maximum keeps full accuracy;
- * stride 0 = one bound for all rows): the y_rowmax output of the call that produced x,
+ * x_rowmax[(r / x_rows_per_bound) * x_rowmax_stride + p], p < x_rowmax_parts, holds upper bounds of
+ * max_i |x[r,i]| (the largest part is used; any bound within a factor 2^14 of the true maximum keeps
+ * full accuracy; stride 0 = one bound for all rows; x_rows_per_bound = 3 or 9 when the rows are the
+ * components of a node that carries one bound): the y_rowmax output of the call that produced x,
  * mg_row_absmax(x) (one part), or a bound the caller derives from the producing layer's weights.  y_rowmax, if not NULL,
  * receives (rows, mg_tensor_linear_f16x2_rowmax_parts(rows, dim_in, dim_out)) partial row maxima of |y|
  * (out_comps must be 1).  out_comps / accumulate / act as in mg_tensor_linear_packed.
@@ -230,7 +231,7 @@ int mg_linear_f16x2_pack_weight(const float* W, long w_stride_o, long w_stride_i
 int mg_row_absmax(const float* x, long rows, int dim, float* out /* (rows) */, mg_stream_t stream);
 int mg_tensor_linear_f16x2_rowmax_parts(long rows, int dim_in, int dim_out);   /* returns the count, not a status */
 int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts,
-                           long x_rowmax_stride, long rows, int dim_in, int dim_out, const float* bias, int act, int accumulate,
+                           long x_rowmax_stride, long x_rows_per_bound, long rows, int dim_in, int dim_out, const float* bias, int act, int accumulate,
                            int out_comps, float* y, float* y_rowmax, mg_stream_t stream);
 /* dW[o,i] = sum_{r,t} dy[r,o,t] x[r,i,t]  (tensor_ops_kern.cu:45-71), dW dense (dim_out,dim_in). */
 int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows, int dim_in, int dim_out,

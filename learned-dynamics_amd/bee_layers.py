@@ -48,6 +48,42 @@ def apply_tens_prod_submodules(self, prods):
     return tuple(outs)
 
 
+def _derived(module, key, params, make):
+    """A tensor computed from parameters (a concatenation, a scaled copy), cached on the module until
+    one of the parameters changes (object or version), so that pre-split weight planes and norms
+    keyed on the tensor object stay valid from one forward to the next."""
+    cache = module.__dict__.setdefault("_derived_cache", {})
+    stamp = tuple((id(p), p._version, p.data_ptr()) for p in params)
+    hit = cache.get(key)
+    if hit is None or hit[0] != stamp:
+        with torch.no_grad():
+            hit = cache[key] = (stamp, make())
+    return hit[1]
+
+
+def _cat_Y(module, labels, scale=None):
+    """[Y_lab.W for lab in labels] concatenated along K (optionally scaled): one GEMM per output rank."""
+    params = tuple(getattr(module, f"Y_{lab}").W for lab in labels)
+
+    def make():
+        W = torch.cat(params, dim=1)
+        return W if scale is None else W * scale
+    return _derived(module, ("cat_Y", labels, scale), params, make)
+
+
+def _linear(x, W, bias, act, bound, out=None, accumulate=False):
+    """Plain-row linear with fused bias / activation.  With the split-fp16 matrix path active and
+    a row bound of |x| at hand, the bound is used (no pass over x) and the bound of the output rows
+    is returned with y; otherwise (y, None)."""
+    rows, dim_in, dim_out = x.shape[0], W.shape[1], W.shape[0]
+    if (bound is not None and ops.get_linear_mode() == ops.LINEAR_F16X2
+            and ops.f16x2_supported(rows, dim_in, dim_out, x)):
+        y = ops.tensor_linear_f16x2(W, x, bound, bias=bias, act=act, out=out, accumulate=accumulate)
+    else:
+        y = ops.tensor_linear_fwd(0, W, x, bias=bias, act=act, out=out, accumulate=accumulate)
+    return y, (ops.linear_out_bound(W, bias, bound) if bound is not None and not accumulate else None)
+
+
 class TensGroupNorm(nn.Module):
     """managan/tensor_products.py:215-232: x / sqrt(eps + mean over (nodes, group channels) of |x|^2), times gamma."""
 
@@ -90,8 +126,18 @@ class SelfTensProds(nn.Module):
         x_a = x_a.reshape(rows, dim_a).contiguous()
         x_v = x_v.reshape(rows, dim_v, 3).contiguous()
         x_d = x_d.reshape(rows, dim_d, 3, 3).contiguous()
-        prods = Bee.apply(self.L0(x_a), self.L1(x_v), self.L2(x_d), self.R0(x_a), self.R1(x_v), self.R2(x_d))
-        y_a, y_v, y_d = apply_tens_prod_submodules(self, prods)
+        # L_k x_k and R_k x_k are written component-major; the 13 products then land as
+        # (row, comp, label, chan), so the 13 output linears are three GEMMs with K = 3 chan,
+        # 5 chan, 5 chan instead of thirteen accumulating ones
+        C = ops.LAYOUT_COMP_CHAN
+        chan = self.L0.W.shape[0]
+        ops_in = [ops.tensor_linear_fwd(k, lin.W, x, y_layout=C if k else ops.LAYOUT_CHAN_COMP)
+                  for side in ((self.L0, self.L1, self.L2), (self.R0, self.R1, self.R2))
+                  for k, (lin, x) in enumerate(zip(side, (x_a, x_v, x_d)))]
+        P0, P1, P2 = ops.bee_node_products(*ops_in)
+        y_a = ops.tensor_linear_fwd(0, _cat_Y(self, LABELS_0), P0.reshape(rows, 3 * chan))
+        y_v = ops.tensor_linear_fwd(1, _cat_Y(self, LABELS_1), P1.reshape(rows, 3, 5 * chan), x_layout=C)
+        y_d = ops.tensor_linear_fwd(2, _cat_Y(self, LABELS_2), P2.reshape(rows, 9, 5 * chan), x_layout=C)
         y_a = y_a.reshape(*rest, dim_a)
         y_v = y_v.reshape(*rest, dim_v, 3)
         y_d = y_d.reshape(*rest, dim_d, 3, 3)
@@ -116,18 +162,22 @@ class MLP(nn.Module):
             nn.Linear(2 * dim_a, dim_a),
         )
 
-    def forward(self, x, plus_identity=False):
-        """Returns mlp(x), or x + mlp(x) with plus_identity=True."""
+    def forward(self, x, plus_identity=False, bound=None):
+        """Returns mlp(x), or x + mlp(x) with plus_identity=True.  bound: upper bounds of the row
+        maxima of |x| ((rows, 1) or (1, 1)) if the caller has them."""
         lead = x.shape[:-1]
         x2 = x.reshape(-1, x.shape[-1]).contiguous()
         Wd = self.lin_direct.weight
         if plus_identity:
-            Wd = Wd + torch.eye(Wd.shape[0], device=Wd.device, dtype=Wd.dtype)
-        out = ops.tensor_linear_fwd(0, Wd, x2)
+            Wd = _derived(self, "direct_plus_identity", (Wd,),
+                          lambda: Wd + torch.eye(Wd.shape[0], device=Wd.device, dtype=Wd.dtype))
         L = self.layers
-        h = ops.tensor_linear_fwd(0, L[0].weight, x2, bias=L[0].bias, act=ops.ACT_LEAKY)
-        h = ops.tensor_linear_fwd(0, L[2].weight, h, bias=L[2].bias, act=ops.ACT_LEAKY)
-        ops.tensor_linear_fwd(0, L[4].weight, h, bias=L[4].bias, out=out, accumulate=True)
+        if bound is None and ops.get_linear_mode() == ops.LINEAR_F16X2:
+            bound = ops.row_absmax(x2)
+        out, _ = _linear(x2, Wd, None, ops.ACT_NONE, bound)
+        h, b1 = _linear(x2, L[0].weight, L[0].bias, ops.ACT_LEAKY, bound)
+        h, b2 = _linear(h, L[2].weight, L[2].bias, ops.ACT_LEAKY, b1)
+        _linear(h, L[4].weight, L[4].bias, ops.ACT_NONE, b2, out=out, accumulate=True)
         return out.reshape(*lead, out.shape[-1])
 
 
@@ -145,8 +195,7 @@ class Messages(nn.Module):
         self.mlp_a = MLP(dim_a)
 
     def _cat_Y(self, labels, scale=None):
-        W = torch.cat([getattr(self, f"Y_{lab}").W for lab in labels], dim=1)
-        return W if scale is None else W * scale
+        return _cat_Y(self, labels, scale)
 
     def forward(self, graph: Graph, r_ij, x_a, x_v, x_d, node_order="cell"):
         """x_a (batch, nodes, dim_a), x_v (..., dim_v, 3), x_d (..., dim_d, 3, 3), r_ij (edges, 3).
@@ -166,8 +215,10 @@ class Messages(nn.Module):
                                      self.lin_enc.bias, node_order=node_order)
         E, chan = P0.shape[0], P0.shape[2]
         # scalar channel: per-edge linear + MLP, then the edge sum
-        psi_a = ops.tensor_linear_fwd(0, self._cat_Y(LABELS_0), P0.reshape(E, 3 * chan))
-        psi_a = self.mlp_a(psi_a, plus_identity=True)
+        P0 = P0.reshape(E, 3 * chan)
+        bound = ops.row_absmax(P0) if ops.get_linear_mode() == ops.LINEAR_F16X2 else None
+        psi_a, bound = _linear(P0, self._cat_Y(LABELS_0), None, ops.ACT_NONE, bound)
+        psi_a = self.mlp_a(psi_a, plus_identity=True, bound=bound)
         B_a = ops.segment_sum_csr(psi_a, graph.row_ptr, rows).mul_(0.1)
         # vector and rank-2 channels: output linears after the edge sum, on node rows
         B_v = ops.tensor_linear_fwd(1, self._cat_Y(LABELS_1, 0.1), S1.reshape(rows, 3, 5 * chan), x_layout=C)

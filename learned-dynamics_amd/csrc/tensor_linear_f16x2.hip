@@ -13,10 +13,24 @@
 // are undone exactly in the epilogue.  The row maxima of x come from the kernel that produced
 // x (this kernel's own epilogue can emit them for its output) or from row_absmax_kernel.
 //
-// Tile TM x TN per workgroup = (64 WM) x (64 NI), waves WM x 2, wave tile 64 x (32 NI), K slab
-// 16, LDS double buffered with one barrier per slab; the staging of slab k+1 (global fp32 ->
-// scale, split -> LDS planes) sits in the instruction stream of slab k's MFMAs, and the two
-// waves of a SIMD stage at opposite ends of the slab period.
+// Kernel shape (row streaming): a workgroup of WAVES waves owns a tile of 32 WAVES rows x 32 NI
+// columns; wave w owns rows [32 w, 32 w + 32) of the tile and ALL its columns.
+//   * x never touches LDS: a lane loads the 16 consecutive floats of ITS row that it will feed to
+//     the matrix core (lane = row + 32 g holds k = 32 c + 16 g .. + 16 of chunk c: 64 contiguous
+//     bytes, four 16-byte loads), two chunks ahead, and splits them in registers.  Every row is
+//     loaded and split exactly once per tile, nothing about x is tied to a barrier, and the LDS
+//     carries only W.
+//   * W planes (already fp16) go global -> registers -> LDS, double buffered, K chunk 32 (rows of
+//     64 B padded to 80 B: conflict free for 16-byte reads), one barrier per chunk.
+//   * the k order inside a chunk is a permutation (MFMA step s takes k = 16 g + 8 s .. + 8 from
+//     lane group g); W is read from LDS with the same permutation, so the products pair up.
+//   * loads are never predicated (rows past the end are clamped to the last row, whose
+//     accumulators are simply not written): a loop body without branches lets every load stay in
+//     flight until the chunk that needs it.  W (L2 resident, needed one chunk later) is requested
+//     before x (HBM, needed two chunks later), because loads return in order.
+//   * the epilogue runs once per tile with nothing to overlap it, so its instruction count is
+//     what matters: one row pointer, row scale and bounds check per accumulator row, column
+//     offsets as immediates, activation and accumulate chosen at compile time.
 // v_mfma_f32_32x32x16_f16 layout: A[m][k]: lane = m + 32*(k/8), 8 consecutive k per lane;
 // B[k][n] likewise; D[m][n]: n = lane%32, m = 8*(q/4) + 4*(lane/32) + q%4 for register q.
 #include "common.hpp"
@@ -29,8 +43,6 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
 typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
 
-constexpr int kBK = 16;
-constexpr int kRow = 48;   // bytes per LDS row of one plane: 16 fp16 + pad (3 quads: conflict free for b128 reads)
 
 __device__ __forceinline__ float activate(float v, int act) {
     if (act == 1) return v * __frcp_rn(1.0f + __expf(-v));
@@ -118,22 +130,20 @@ __global__ void __launch_bounds__(256) row_absmax_kernel(const float* __restrict
     }
 }
 
-struct StageRegs {
-    float4 x[2];       // 2 rows x 4 consecutive k (fp32)
-    halfx8 w[2];       // one 16-byte piece of each W plane
-};
+constexpr int kCK = 32;                     // k per chunk (two MFMA steps)
+constexpr int kRowW = 80;                   // bytes per LDS row of one W plane (64 + 16 pad)
 
-template <int WM, int NI>
-__global__ void __launch_bounds__(128 * WM)
+template <int WAVES, int NI>
+__global__ void __launch_bounds__(64 * WAVES)
 linear_rows_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restrict__ w_inv, const float* __restrict__ X,
-                         const float* __restrict__ xmax, int xmax_parts, long xmax_stride, long R, int I, int O, int O_pad,
-                         const float* __restrict__ bias, int act, int accumulate, float* __restrict__ Y,
-                         float* __restrict__ ymax, int tiles_n, long tiles_total, int out_T) {
-    static_assert(WM == NI, "the W staging assumes one 16-byte piece per plane and thread");
-    constexpr int TM = 64 * WM, TN = 64 * NI;
-    constexpr int kPlaneX = TM * kRow, kPlaneW = TN * kRow;
-    constexpr int kBuf = 2 * kPlaneX + 2 * kPlaneW;
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kBuf];
+                         const float* __restrict__ xmax, int xmax_parts, long xmax_stride, long xmax_div, long R, int I,
+                         int O, int O_pad, const float* __restrict__ bias, int act, int accumulate,
+                         float* __restrict__ Y, float* __restrict__ ymax, int tiles_n, long tiles_total, int out_T) {
+    constexpr int TM = 32 * WAVES, TN = 32 * NI, THREADS = 64 * WAVES;
+    constexpr int kPlaneW = TN * kRowW, kBufW = 2 * kPlaneW;
+    constexpr int kPieces = 8 * TN;                          // 16-byte pieces of W per chunk (2 planes x TN rows x 4)
+    constexpr int kPer = (kPieces + THREADS - 1) / THREADS;  // per thread
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kBufW];
     __shared__ float inv_sx[TM];
 
     const long bid = blockIdx.x;
@@ -145,241 +155,14 @@ linear_rows_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restric
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int wave_m = wave >> 1, wave_n = wave & 1;
+    const int m = lane & 31, g = lane >> 5;
     const long r0 = tile_m * TM;
     const int n0 = tile_n * TN;
-    const int kgroup = lane >> 5;
     const long plane_elems = (long)O_pad * I;
 
-    floatx16 acc[2][NI];
+    floatx16 acc[NI];
 #pragma unroll
-    for (int mi = 0; mi < 2; mi++)
-#pragma unroll
-        for (int ni = 0; ni < NI; ni++)
-#pragma unroll
-            for (int q = 0; q < 16; q++) acc[mi][ni][q] = 0.f;
-
-    // x tile of a slab: TM rows x 16 floats: thread -> rows (tid>>2) and (tid>>2) + TM/2, k = (tid&3)*4
-    const int xr = tid >> 2, xc = (tid & 3) * 4;
-    // W tile: 2 planes x TN rows x 32 B: thread -> row (tid>>1), half (tid&1), both planes
-    const int wr = tid >> 1, wc = (tid & 1) * 8;
-    const int k_last = I - kBK;
-
-    float sx[2];
-#pragma unroll
-    for (int h = 0; h < 2; h++) {
-        const long r = r0 + xr + (TM / 2) * h;
-        float amax = 0.f;
-        if (r < R)
-            for (int p = 0; p < xmax_parts; p++) amax = fmaxf(amax, xmax[r * xmax_stride + p]);
-        float inv;
-        sx[h] = pow2_scale(amax, &inv);
-        if ((tid & 3) == 0) inv_sx[xr + (TM / 2) * h] = inv;
-    }
-
-    // Rows past the end of x are clamped to the last row instead of being predicated: their
-    // accumulators are never written, and a loop body without branches lets every load stay in
-    // flight until the slab that needs it (a conditional load forces a full drain of the queue).
-    const float* xrow[2];
-#pragma unroll
-    for (int h = 0; h < 2; h++) {
-        const long r = r0 + xr + (TM / 2) * h;
-        xrow[h] = X + (r < R ? r : R - 1) * I + xc;
-    }
-    const _Float16* wrow = Wp + (long)(n0 + wr) * I + wc;
-    auto load_stage = [&](StageRegs& g, int k0) {
-        k0 = k0 < I ? k0 : k_last;                   // clamped: the surplus loads of the last trips are never used
-#pragma unroll
-        for (int h = 0; h < 2; h++) g.x[h] = *reinterpret_cast<const float4*>(xrow[h] + k0);
-#pragma unroll
-        for (int p = 0; p < 2; p++) g.w[p] = *reinterpret_cast<const halfx8*>(wrow + p * plane_elems + k0);
-    };
-    auto store_stage = [&](const StageRegs& g, unsigned char* buf) {
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const HalfSplit4 s = split(g.x[h], sx[h]);
-            const int off = (xr + (TM / 2) * h) * kRow + xc * 2;
-            *reinterpret_cast<halfx4*>(buf + off) = s.hi;
-            *reinterpret_cast<halfx4*>(buf + kPlaneX + off) = s.lo;
-        }
-#pragma unroll
-        for (int p = 0; p < 2; p++)
-            *reinterpret_cast<halfx8*>(buf + 2 * kPlaneX + p * kPlaneW + wr * kRow + wc * 2) = g.w[p];
-    };
-
-    int a_off[2], b_off[NI];
-#pragma unroll
-    for (int i = 0; i < 2; i++) a_off[i] = ((wave_m * 2 + i) * 32 + (lane & 31)) * kRow + kgroup * 16;
-#pragma unroll
-    for (int i = 0; i < NI; i++) b_off[i] = 2 * kPlaneX + ((wave_n * NI + i) * 32 + (lane & 31)) * kRow + kgroup * 16;
-
-    auto compute = [&](const unsigned char* buf) {
-        halfx8 a[2][2];
-#pragma unroll
-        for (int i = 0; i < 2; i++)
-#pragma unroll
-            for (int p = 0; p < 2; p++) a[i][p] = *reinterpret_cast<const halfx8*>(buf + p * kPlaneX + a_off[i]);
-#pragma unroll
-        for (int nh = 0; nh < NI / 2; nh++) {
-            halfx8 b[2][2];
-#pragma unroll
-            for (int i = 0; i < 2; i++)
-#pragma unroll
-                for (int p = 0; p < 2; p++)
-                    b[i][p] = *reinterpret_cast<const halfx8*>(buf + p * kPlaneW + b_off[nh * 2 + i]);
-            // small terms first; each round goes over the four independent accumulators
-#pragma unroll
-            for (int t = 0; t < 3; t++) {
-                constexpr int pa[3] = {1, 0, 0};   // lo*hi, hi*lo, hi*hi
-                constexpr int pb[3] = {0, 1, 0};
-#pragma unroll
-                for (int mi = 0; mi < 2; mi++)
-#pragma unroll
-                    for (int nj = 0; nj < 2; nj++)
-                        acc[mi][nh * 2 + nj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(a[mi][pa[t]], b[nj][pb[t]],
-                                                                                      acc[mi][nh * 2 + nj], 0, 0, 0);
-            }
-        }
-    };
-
-    unsigned char* buf0 = lds;
-    unsigned char* buf1 = lds + kBuf;
-    // Waves w and w + 4 (w + 2 in the four-wave shape) share a SIMD.  The upper half stages the
-    // next slab before its MFMAs, the lower half after: while one wave of a SIMD splits and
-    // stores, the other keeps the matrix pipe busy.
-    const bool store_first = __builtin_amdgcn_readfirstlane(wave) >= WM;
-    StageRegs ga, gb;
-    load_stage(ga, 0);
-    load_stage(gb, kBK);
-    store_stage(ga, buf0);
-    load_stage(ga, 2 * kBK);
-    // I is a multiple of 32: slabs are handled in pairs (even slab in buf0, odd slab in buf1).
-    // One branch-free loop per staging position.
-    auto main_loop = [&](auto first) {
-        constexpr bool kFirst = decltype(first)::value;
-        for (int k0 = 0; k0 < I; k0 += 2 * kBK) {
-            __syncthreads();
-            if constexpr (kFirst) {
-                store_stage(gb, buf1);
-                load_stage(gb, k0 + 3 * kBK);
-            }
-            compute(buf0);
-            if constexpr (!kFirst) {
-                store_stage(gb, buf1);
-                load_stage(gb, k0 + 3 * kBK);
-            }
-            __syncthreads();
-            if constexpr (kFirst) {
-                store_stage(ga, buf0);
-                load_stage(ga, k0 + 4 * kBK);
-            }
-            compute(buf1);
-            if constexpr (!kFirst) {
-                store_stage(ga, buf0);
-                load_stage(ga, k0 + 4 * kBK);
-            }
-        }
-    };
-    if (store_first) main_loop(std::true_type{});
-    else main_loop(std::false_type{});
-
-    auto epilogue = [&](auto plain) {
-        constexpr bool kPlain = decltype(plain)::value;
-        float rmax[2][16];
-#pragma unroll
-        for (int mi = 0; mi < 2; mi++)
-#pragma unroll
-            for (int q = 0; q < 16; q++) rmax[mi][q] = 0.f;
-#pragma unroll
-        for (int ni = 0; ni < NI; ni++) {
-            const int n = n0 + (wave_n * NI + ni) * 32 + (lane & 31);
-            if (n >= O) continue;
-            const float bv = bias ? bias[n] : 0.f;
-            const float iw = w_inv[n];
-#pragma unroll
-            for (int mi = 0; mi < 2; mi++) {
-#pragma unroll
-                for (int q = 0; q < 16; q++) {
-                    const int rl = (wave_m * 2 + mi) * 32 + 8 * (q / 4) + 4 * kgroup + (q % 4);
-                    const long r = r0 + rl;
-                    if (r < R) {
-                        long addr;
-                        if constexpr (kPlain) {
-                            addr = r * O + n;
-                        } else {   // rows are (row, comp) pairs, output stored (row, chan, comp)
-                            const long row = r / out_T;
-                            addr = (row * O + n) * out_T + (r - row * out_T);
-                        }
-                        float v = activate(acc[mi][ni][q] * inv_sx[rl] * iw + bv, act);
-                        if (accumulate) v += Y[addr];
-                        Y[addr] = v;
-                        rmax[mi][q] = fmaxf(rmax[mi][q], fabsf(v));
-                    }
-                }
-            }
-        }
-        if (ymax) {
-            const int parts = tiles_n * 2;
-            const int part = tile_n * 2 + wave_n;
-#pragma unroll
-            for (int mi = 0; mi < 2; mi++)
-#pragma unroll
-                for (int q = 0; q < 16; q++) {
-                    float m = rmax[mi][q];
-#pragma unroll
-                    for (int d = 1; d < 32; d <<= 1) m = fmaxf(m, __shfl_xor(m, d));
-                    const long r = r0 + (wave_m * 2 + mi) * 32 + 8 * (q / 4) + 4 * kgroup + (q % 4);
-                    if ((lane & 31) == 0 && r < R) ymax[r * parts + part] = m;
-                }
-        }
-    };
-    if (out_T == 1) epilogue(std::true_type{});
-    else epilogue(std::false_type{});
-}
-
-// ---------------------------------------------------------------------------
-// Row-streaming variant for large problems: tile 256 x 256, eight waves, wave w owns rows
-// [32 w, 32 w + 32) of the tile and ALL 256 columns.
-//   * x never touches LDS: a lane loads the 16 consecutive floats of ITS row that it will feed to
-//     the matrix core (lane = row + 32 g holds k = 32 c + 16 g .. + 16 of chunk c: 64 contiguous
-//     bytes, four 16-byte loads), two chunks ahead, and splits them in registers.  Every row is
-//     loaded and split exactly once per tile, nothing about x is tied to a barrier, and the LDS
-//     carries only W.
-//   * W planes (already fp16) go global -> registers -> LDS, double buffered, K chunk 32 (rows of
-//     64 B padded to 80 B: conflict free for 16-byte reads), one barrier per chunk.
-//   * the k order inside a chunk is a permutation (MFMA step s takes k = 16 g + 8 s .. + 8 from
-//     lane group g); W is read from LDS with the same permutation, so the products pair up.
-constexpr int kCK = 32;                     // k per chunk (two MFMA steps)
-constexpr int kRowW = 80;                   // bytes per LDS row of one W plane
-constexpr int kPlaneWQ = 256 * kRowW;
-constexpr int kBufWQ = 2 * kPlaneWQ;
-
-__global__ void __launch_bounds__(512)
-linear_rows_f16x2_stream_kernel(const _Float16* __restrict__ Wp, const float* __restrict__ w_inv,
-                                const float* __restrict__ X, const float* __restrict__ xmax, int xmax_parts,
-                                long xmax_stride, long R, int I, int O, int O_pad, const float* __restrict__ bias,
-                                int act, int accumulate, float* __restrict__ Y, float* __restrict__ ymax, int tiles_n,
-                                long tiles_total, int out_T) {
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kBufWQ];
-    __shared__ float inv_sx[256];
-
-    const long bid = blockIdx.x;
-    const long per_xcd = (tiles_total + 7) / 8;
-    const long logical = (bid % 8) * per_xcd + bid / 8;
-    if (logical >= tiles_total) return;
-    const long tile_m = logical / tiles_n;
-    const int tile_n = (int)(logical - tile_m * tiles_n);
-
-    const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int m = lane & 31, g = lane >> 5;
-    const long r0 = tile_m * 256;
-    const int n0 = tile_n * 256;
-    const long plane_elems = (long)O_pad * I;
-
-    floatx16 acc[8];
-#pragma unroll
-    for (int ni = 0; ni < 8; ni++)
+    for (int ni = 0; ni < NI; ni++)
 #pragma unroll
         for (int q = 0; q < 16; q++) acc[ni][q] = 0.f;
 
@@ -390,45 +173,46 @@ linear_rows_f16x2_stream_kernel(const _Float16* __restrict__ Wp, const float* __
     float sx;
     {
         float amax = 0.f;
-        for (int p = 0; p < xmax_parts; p++) amax = fmaxf(amax, xmax[ld_row * xmax_stride + p]);
+        const float* xm = xmax + (ld_row / xmax_div) * xmax_stride;
+        for (int p = 0; p < xmax_parts; p++) amax = fmaxf(amax, xm[p]);
         float inv;
         sx = pow2_scale(amax, &inv);
         if (g == 0) inv_sx[wave * 32 + m] = inv;
     }
-    // W staging: 2 planes x 256 rows x 64 B per chunk = 2048 pieces of 16 B, four per thread
-    const _Float16* wsrc[4];
-    int wdst[4];
+    const _Float16* wsrc[kPer];
+    int wdst[kPer];
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const int q = tid + 512 * j;
-        const int plane = q >> 10, row = (q & 1023) >> 2, piece = q & 3;
+    for (int j = 0; j < kPer; j++) {
+        int q = tid + THREADS * j;
+        if (q >= kPieces) q = kPieces - 1;                    // surplus threads repeat the last piece
+        const int plane = q / (4 * TN), row = (q % (4 * TN)) >> 2, piece = q & 3;
         wsrc[j] = Wp + plane * plane_elems + (long)(n0 + row) * I + 8 * piece;
-        wdst[j] = plane * kPlaneWQ + row * kRowW + piece * 16;
+        wdst[j] = plane * kPlaneW + row * kRowW + piece * 16;
     }
     const int k_last = I - kCK;
 
     struct ARegs { float4 v[4]; };
-    struct WRegs { halfx8 v[4]; };
+    struct WRegs { halfx8 v[kPer]; };
     auto load_a = [&](ARegs& a, int k0) {
-        k0 = k0 < I ? k0 : k_last;
+        k0 = k0 < I ? k0 : k_last;                            // surplus loads of the last trips are never used
 #pragma unroll
         for (int j = 0; j < 4; j++) a.v[j] = *reinterpret_cast<const float4*>(xrow + k0 + 4 * j);
     };
     auto load_w = [&](WRegs& w, int k0) {
         k0 = k0 < I ? k0 : k_last;
 #pragma unroll
-        for (int j = 0; j < 4; j++) w.v[j] = *reinterpret_cast<const halfx8*>(wsrc[j] + k0);
+        for (int j = 0; j < kPer; j++) w.v[j] = *reinterpret_cast<const halfx8*>(wsrc[j] + k0);
     };
     auto store_w = [&](const WRegs& w, unsigned char* buf) {
 #pragma unroll
-        for (int j = 0; j < 4; j++) *reinterpret_cast<halfx8*>(buf + wdst[j]) = w.v[j];
+        for (int j = 0; j < kPer; j++) *reinterpret_cast<halfx8*>(buf + wdst[j]) = w.v[j];
     };
     const int b_off = m * kRowW + 32 * g;
-    auto compute = [&](const ARegs& a, const unsigned char* buf) {
+    auto compute = [&](const ARegs& a, const unsigned char* buf, float scale) {
         halfx8 ah[2], al[2];
 #pragma unroll
         for (int s = 0; s < 2; s++) {
-            const HalfSplit4 p0 = split(a.v[2 * s], sx), p1 = split(a.v[2 * s + 1], sx);
+            const HalfSplit4 p0 = split(a.v[2 * s], scale), p1 = split(a.v[2 * s + 1], scale);
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 ah[s][i] = p0.hi[i]; ah[s][4 + i] = p1.hi[i];
@@ -438,9 +222,10 @@ linear_rows_f16x2_stream_kernel(const _Float16* __restrict__ Wp, const float* __
 #pragma unroll
         for (int s = 0; s < 2; s++)
 #pragma unroll
-            for (int ni = 0; ni < 8; ni++) {
+            for (int ni = 0; ni < NI; ni++) {
                 const halfx8 bh = *reinterpret_cast<const halfx8*>(buf + b_off + ni * 32 * kRowW + 16 * s);
-                const halfx8 bl = *reinterpret_cast<const halfx8*>(buf + kPlaneWQ + b_off + ni * 32 * kRowW + 16 * s);
+                const halfx8 bl = *reinterpret_cast<const halfx8*>(buf + kPlaneW + b_off + ni * 32 * kRowW + 16 * s);
+                // small terms first
                 acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[s], bh, acc[ni], 0, 0, 0);
                 acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[s], bl, acc[ni], 0, 0, 0);
                 acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[s], bh, acc[ni], 0, 0, 0);
@@ -448,7 +233,7 @@ linear_rows_f16x2_stream_kernel(const _Float16* __restrict__ Wp, const float* __
     };
 
     unsigned char* buf0 = lds;
-    unsigned char* buf1 = lds + kBufWQ;
+    unsigned char* buf1 = lds + kBufW;
     ARegs a0, a1;
     WRegs w;
     load_w(w, 0);
@@ -457,18 +242,18 @@ linear_rows_f16x2_stream_kernel(const _Float16* __restrict__ Wp, const float* __
     load_w(w, kCK);
     load_a(a1, kCK);
     __syncthreads();
-    // I is a multiple of 64 here: chunks in pairs (even chunk: a0 / buf0, odd chunk: a1 / buf1)
+    // chunks in pairs (even chunk: a0 / buf0, odd chunk: a1 / buf1); with an odd chunk count the
+    // surplus chunk (a clamped reload of the last one) is scaled by zero instead of being branched
+    // around, which keeps the loop body straight-line
     for (int k0 = 0; k0 < I; k0 += 2 * kCK) {
-        // W (L2 resident, needed one chunk later) is requested before x (HBM, needed two chunks
-        // later): loads return in order, so the wait for W never includes the youngest x loads
-        compute(a0, buf0);
+        compute(a0, buf0, sx);
         store_w(w, buf1);
         __builtin_amdgcn_sched_barrier(0);     // keep this issue order: the compiler would hoist the loads
         load_w(w, k0 + 2 * kCK);
         __builtin_amdgcn_sched_barrier(0);
         load_a(a0, k0 + 2 * kCK);
         __syncthreads();
-        compute(a1, buf1);
+        compute(a1, buf1, k0 + kCK < I ? sx : 0.f);
         store_w(w, buf0);
         __builtin_amdgcn_sched_barrier(0);
         load_w(w, k0 + 3 * kCK);
@@ -477,15 +262,14 @@ linear_rows_f16x2_stream_kernel(const _Float16* __restrict__ Wp, const float* __
         __syncthreads();
     }
 
-    // Fast path (plain rows, full tile of columns, no accumulate): one row pointer, row scale and
-    // bounds check per accumulator row, column offsets as immediates, activation chosen at compile
-    // time.  The epilogue runs once per tile with nothing to overlap it, so its instruction count
-    // is what matters.
-    auto epilogue_fast = [&](auto act_tag) {
+    const bool full_cols = n0 + TN <= O;
+    // ---- fast path, plain rows: y (rows, O)
+    auto epilogue_rows = [&](auto act_tag, auto acc_tag) {
         constexpr int kAct = decltype(act_tag)::value;
-        float bv[8], iw[8];
+        constexpr bool kAccumulate = decltype(acc_tag)::value;
+        float bv[NI], iw[NI];
 #pragma unroll
-        for (int ni = 0; ni < 8; ni++) {
+        for (int ni = 0; ni < NI; ni++) {
             bv[ni] = bias ? bias[n0 + ni * 32 + m] : 0.f;
             iw[ni] = w_inv[n0 + ni * 32 + m];
         }
@@ -498,8 +282,9 @@ linear_rows_f16x2_stream_kernel(const _Float16* __restrict__ Wp, const float* __
                 const float isx = inv_sx[rl];
                 float mx = 0.f;
 #pragma unroll
-                for (int ni = 0; ni < 8; ni++) {
-                    const float v = activate_c<kAct>(acc[ni][q] * isx * iw[ni] + bv[ni]);
+                for (int ni = 0; ni < NI; ni++) {
+                    float v = activate_c<kAct>(acc[ni][q] * isx * iw[ni] + bv[ni]);
+                    if constexpr (kAccumulate) v += yrow[ni * 32];
                     yrow[ni * 32] = v;
                     mx = fmaxf(mx, fabsf(v));
                 }
@@ -511,60 +296,108 @@ linear_rows_f16x2_stream_kernel(const _Float16* __restrict__ Wp, const float* __
             }
         }
     };
-    if (out_T == 1 && !accumulate && n0 + 256 <= O) {
-        if (act == 1) epilogue_fast(std::integral_constant<int, 1>{});
-        else if (act == 2) epilogue_fast(std::integral_constant<int, 2>{});
-        else epilogue_fast(std::integral_constant<int, 0>{});
-        return;
-    }
-
-    auto epilogue = [&](auto plain) {
-        constexpr bool kPlain = decltype(plain)::value;
-        float rmax[16];
+    // ---- fast path, rows are (row, comp) pairs and y is stored (row, chan, comp): no bias, no activation
+    auto epilogue_comps = [&](auto t_tag) {
+        constexpr int T = decltype(t_tag)::value;
+        float iw[NI];
 #pragma unroll
-        for (int q = 0; q < 16; q++) rmax[q] = 0.f;
+        for (int ni = 0; ni < NI; ni++) iw[ni] = w_inv[n0 + ni * 32 + m];
 #pragma unroll
-        for (int ni = 0; ni < 8; ni++) {
-            const int n = n0 + ni * 32 + m;
-            if (n >= O) continue;
-            const float bv = bias ? bias[n] : 0.f;
-            const float iw = w_inv[n];
+        for (int q = 0; q < 16; q++) {
+            const int rl = wave * 32 + 8 * (q / 4) + 4 * g + (q % 4);
+            const long r = r0 + rl;
+            if (r < R) {
+                const long row = r / T;
+                float* yp = Y + (row * O + n0 + m) * T + (r - row * T);
+                const float isx = inv_sx[rl];
 #pragma unroll
-            for (int q = 0; q < 16; q++) {
-                const int rl = wave * 32 + 8 * (q / 4) + 4 * g + (q % 4);
-                const long r = r0 + rl;
-                if (r < R) {
-                    long addr;
-                    if constexpr (kPlain) {
-                        addr = r * O + n;
-                    } else {   // rows are (row, comp) pairs, output stored (row, chan, comp)
-                        const long row = r / out_T;
-                        addr = (row * O + n) * out_T + (r - row * out_T);
-                    }
-                    float v = activate(acc[ni][q] * inv_sx[rl] * iw + bv, act);
-                    if (accumulate) v += Y[addr];
-                    Y[addr] = v;
-                    rmax[q] = fmaxf(rmax[q], fabsf(v));
+                for (int ni = 0; ni < NI; ni++) {
+                    float v = acc[ni][q] * isx * iw[ni];
+                    if (accumulate) v += yp[ni * 32 * T];
+                    yp[ni * 32 * T] = v;
                 }
             }
         }
-        if (ymax) {
+    };
+    if (full_cols && out_T == 1) {
+        if (accumulate) {
+            if (act == 1) epilogue_rows(std::integral_constant<int, 1>{}, std::true_type{});
+            else if (act == 2) epilogue_rows(std::integral_constant<int, 2>{}, std::true_type{});
+            else epilogue_rows(std::integral_constant<int, 0>{}, std::true_type{});
+        } else {
+            if (act == 1) epilogue_rows(std::integral_constant<int, 1>{}, std::false_type{});
+            else if (act == 2) epilogue_rows(std::integral_constant<int, 2>{}, std::false_type{});
+            else epilogue_rows(std::integral_constant<int, 0>{}, std::false_type{});
+        }
+        return;
+    }
+    if (full_cols && act == 0 && bias == nullptr && out_T == 3) { epilogue_comps(std::integral_constant<int, 3>{}); return; }
+    if (full_cols && act == 0 && bias == nullptr && out_T == 9) { epilogue_comps(std::integral_constant<int, 9>{}); return; }
+
+    // ---- general path: partial column tiles, or components with bias / activation
+    float rmax[16];
 #pragma unroll
-            for (int q = 0; q < 16; q++) {
-                float mx = rmax[q];
+    for (int q = 0; q < 16; q++) rmax[q] = 0.f;
 #pragma unroll
-                for (int d = 1; d < 32; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
-                const long r = r0 + wave * 32 + 8 * (q / 4) + 4 * g + (q % 4);
-                if (m == 0 && r < R) ymax[r * tiles_n + tile_n] = mx;
+    for (int ni = 0; ni < NI; ni++) {
+        const int n = n0 + ni * 32 + m;
+        if (n >= O) continue;
+        const float bv = bias ? bias[n] : 0.f;
+        const float iw = w_inv[n];
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+            const int rl = wave * 32 + 8 * (q / 4) + 4 * g + (q % 4);
+            const long r = r0 + rl;
+            if (r < R) {
+                const long row = r / out_T;
+                const long addr = (row * O + n) * out_T + (r - row * out_T);
+                float v = activate(acc[ni][q] * inv_sx[rl] * iw + bv, act);
+                if (accumulate) v += Y[addr];
+                Y[addr] = v;
+                rmax[q] = fmaxf(rmax[q], fabsf(v));
             }
         }
-    };
-    if (out_T == 1) epilogue(std::true_type{});
-    else epilogue(std::false_type{});
+    }
+    if (ymax) {
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+            float mx = rmax[q];
+#pragma unroll
+            for (int d = 1; d < 32; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+            const long r = r0 + wave * 32 + 8 * (q / 4) + 4 * g + (q % 4);
+            if (m == 0 && r < R) ymax[r * tiles_n + tile_n] = mx;
+        }
+    }
 }
 
 inline int o_pad_of(int dim_out) { return (dim_out + 255) / 256 * 256; }
-inline bool use_wide(long R, int I, int O) { return I % 64 == 0 && ceil_div(R, 256) * ceil_div(O, 256) >= 512; }
+
+struct Shape {
+    int ni;      // 32-column blocks per tile
+    int waves;   // waves per workgroup (32 rows each)
+};
+inline Shape choose_shape(long R, int O) {
+    Shape s;
+    s.ni = O <= 32 ? 1 : (O <= 64 ? 2 : (O <= 128 ? 4 : 8));
+    const long tiles = ceil_div(R, 256) * ceil_div(O, 32 * s.ni);
+    s.waves = tiles >= 512 ? 8 : 4;
+    return s;
+}
+
+template <int WAVES, int NI>
+int launch(const _Float16* planes, const float* w_inv, const float* x, const float* xmax, int parts, long stride,
+           long div, long rows, int I, int O, int O_pad, const float* bias, int act, int accumulate, float* y,
+           float* ymax, int out_T, hipStream_t st) {
+    const long tiles_m = ceil_div(rows, 32 * WAVES);
+    const int tiles_n = (int)ceil_div(O, 32 * NI);
+    const long total = tiles_m * tiles_n;
+    const long grid = ceil_div(total, 8) * 8;
+    MG_REQUIRE(grid <= 0x7fffffffL, "mg_tensor_linear_f16x2: grid too large (rows=%ld dim_out=%d)", rows, O);
+    hipLaunchKernelGGL((linear_rows_f16x2_kernel<WAVES, NI>), dim3((unsigned)grid), dim3(64 * WAVES), 0, st, planes,
+                       w_inv, x, xmax, parts, stride, div, rows, I, O, O_pad, bias, act, accumulate, y, ymax, tiles_n,
+                       total, out_T);
+    return check_launch("mg_tensor_linear_f16x2");
+}
 
 }  // namespace
 }  // namespace mg
@@ -606,13 +439,14 @@ int mg_row_absmax(const float* x, long rows, int dim, float* out, mg_stream_t st
 }
 
 int mg_tensor_linear_f16x2_rowmax_parts(long rows, int dim_in, int dim_out) {
-    return use_wide(rows, dim_in, dim_out) ? (int)ceil_div(dim_out, 256) : 2 * (int)ceil_div(dim_out, 128);
+    (void)dim_in;
+    return (int)ceil_div(dim_out, 32 * choose_shape(rows, dim_out).ni);
 }
 
-int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts, long x_rowmax_stride,
-                           long rows,
-                           int dim_in, int dim_out, const float* bias, int act, int accumulate, int out_comps,
-                           float* y, float* y_rowmax, mg_stream_t stream) {
+int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts,
+                           long x_rowmax_stride, long x_rows_per_bound, long rows, int dim_in, int dim_out,
+                           const float* bias, int act, int accumulate, int out_comps, float* y, float* y_rowmax,
+                           mg_stream_t stream) {
     MG_REQUIRE(rows >= 0 && dim_in > 0 && dim_out >= 0, "mg_tensor_linear_f16x2: bad size");
     MG_REQUIRE(dim_in % 32 == 0, "mg_tensor_linear_f16x2: dim_in must be a multiple of 32");
     MG_REQUIRE(act >= 0 && act <= 2, "mg_tensor_linear_f16x2: unknown activation %d", act);
@@ -620,6 +454,7 @@ int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_
     MG_REQUIRE(x_rowmax_parts >= 1 && x_rowmax_parts <= 64, "mg_tensor_linear_f16x2: x_rowmax_parts must be in 1..64");
     MG_REQUIRE(x_rowmax_stride == 0 || x_rowmax_stride >= x_rowmax_parts,
                "mg_tensor_linear_f16x2: x_rowmax_stride must be 0 (one bound for all rows) or >= x_rowmax_parts");
+    MG_REQUIRE(x_rows_per_bound >= 1, "mg_tensor_linear_f16x2: x_rows_per_bound must be positive");
     MG_REQUIRE(y_rowmax == nullptr || out_comps == 1, "mg_tensor_linear_f16x2: y_rowmax needs out_comps == 1");
     if (rows == 0 || dim_out == 0) return MG_OK;
     MG_REQUIRE(packed_W && x && y && x_rowmax && aligned16(x) && aligned16(packed_W),
@@ -628,26 +463,21 @@ int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_
     const _Float16* planes = static_cast<const _Float16*>(packed_W);
     const float* w_inv = reinterpret_cast<const float*>(planes + 2L * O_pad * dim_in);
     hipStream_t st = (hipStream_t)stream;
-    if (use_wide(rows, dim_in, dim_out)) {
-        const long tiles_m = ceil_div(rows, 256);
-        const int tiles_n = (int)ceil_div(dim_out, 256);
-        const long total = tiles_m * tiles_n;
-        const long grid = ceil_div(total, 8) * 8;
-        MG_REQUIRE(grid <= 0x7fffffffL, "mg_tensor_linear_f16x2: grid too large (rows=%ld dim_out=%d)", rows, dim_out);
-        hipLaunchKernelGGL(linear_rows_f16x2_stream_kernel, dim3((unsigned)grid), dim3(512), 0, st, planes, w_inv, x,
-                           x_rowmax, x_rowmax_parts, x_rowmax_stride, rows, dim_in, dim_out, O_pad, bias, act, accumulate, y, y_rowmax,
-                           tiles_n, total, out_comps);
-    } else {
-        const long tiles_m = ceil_div(rows, 128);
-        const int tiles_n = (int)ceil_div(dim_out, 128);
-        const long total = tiles_m * tiles_n;
-        const long grid = ceil_div(total, 8) * 8;
-        MG_REQUIRE(grid <= 0x7fffffffL, "mg_tensor_linear_f16x2: grid too large (rows=%ld dim_out=%d)", rows, dim_out);
-        hipLaunchKernelGGL((linear_rows_f16x2_kernel<2, 2>), dim3((unsigned)grid), dim3(256), 0, st, planes, w_inv, x,
-                           x_rowmax, x_rowmax_parts, x_rowmax_stride, rows, dim_in, dim_out, O_pad, bias, act, accumulate, y, y_rowmax,
-                           tiles_n, total, out_comps);
+    const Shape sh = choose_shape(rows, dim_out);
+#define MG_F16X2_LAUNCH(WV, N)                                                                                       \
+    return launch<WV, N>(planes, w_inv, x, x_rowmax, x_rowmax_parts, x_rowmax_stride, x_rows_per_bound, rows, dim_in, \
+                         dim_out, O_pad, bias, act, accumulate, y, y_rowmax, out_comps, st)
+    if (sh.waves == 8) {
+        if (sh.ni == 1) MG_F16X2_LAUNCH(8, 1);
+        if (sh.ni == 2) MG_F16X2_LAUNCH(8, 2);
+        if (sh.ni == 4) MG_F16X2_LAUNCH(8, 4);
+        MG_F16X2_LAUNCH(8, 8);
     }
-    return check_launch("mg_tensor_linear_f16x2");
+    if (sh.ni == 1) MG_F16X2_LAUNCH(4, 1);
+    if (sh.ni == 2) MG_F16X2_LAUNCH(4, 2);
+    if (sh.ni == 4) MG_F16X2_LAUNCH(4, 4);
+    MG_F16X2_LAUNCH(4, 8);
+#undef MG_F16X2_LAUNCH
 }
 
 }  // extern "C"

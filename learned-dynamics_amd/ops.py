@@ -523,11 +523,11 @@ def linear_out_bound(W, bias, in_bound):
 
 
 def f16x2_supported(rows, dim_in, dim_out, x):
-    return dim_in % 32 == 0 and dim_in >= 64 and dim_out >= 64 and rows >= 1024 and x.data_ptr() % 16 == 0
+    return dim_in % 32 == 0 and dim_in >= 64 and dim_out >= 8 and rows >= 1024 and x.data_ptr() % 16 == 0
 
 
 def tensor_linear_f16x2(W, x, x_rowmax=None, bias=None, act=ACT_NONE, out=None, accumulate=False, out_comps=1,
-                        want_rowmax=False):
+                        want_rowmax=False, rows_per_bound=1):
     """y = act(x W^T + bias) for plain rows x (rows, dim_in) through the two-piece fp16 split.
     x_rowmax (rows, parts), or (1, parts) for one bound shared by all rows: upper bounds of the
     row maxima of |x| (None: computed here).  Returns y, or (y, y_rowmax) with want_rowmax=True."""
@@ -538,9 +538,9 @@ def tensor_linear_f16x2(W, x, x_rowmax=None, bias=None, act=ACT_NONE, out=None, 
     if x_rowmax is None:
         x_rowmax = row_absmax(x)
     _check_input(x_rowmax, "x_rowmax")
-    if x_rowmax.dim() != 2 or x_rowmax.size(0) not in (1, rows):
-        raise RuntimeError("x_rowmax must be (rows, parts) or (1, parts)")
-    rowmax_stride = int(x_rowmax.size(1)) if x_rowmax.size(0) == rows and rows > 1 else 0
+    if x_rowmax.dim() != 2 or (x_rowmax.size(0) != 1 and x_rowmax.size(0) * rows_per_bound != rows):
+        raise RuntimeError("x_rowmax must be (rows / rows_per_bound, parts) or (1, parts)")
+    rowmax_stride = int(x_rowmax.size(1)) if x_rowmax.size(0) > 1 or rows == rows_per_bound else 0
     if bias is not None:
         _check_input(bias, "bias")
         if bias.numel() != dim_out:
@@ -563,7 +563,7 @@ def tensor_linear_f16x2(W, x, x_rowmax=None, bias=None, act=ACT_NONE, out=None, 
             parts = int(_lib.mg_tensor_linear_f16x2_rowmax_parts(rows, dim_in, dim_out))
             ymax = torch.empty(rows, parts, dtype=torch.float32, device=x.device)
         L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(W)), _p(x), _p(x_rowmax), int(x_rowmax.size(1)),
-                                            rowmax_stride, rows, dim_in, dim_out, _p(bias), int(act), int(bool(accumulate)),
+                                            rowmax_stride, int(rows_per_bound), rows, dim_in, dim_out, _p(bias), int(act), int(bool(accumulate)),
                                             int(out_comps), _p(y), _p(ymax), _stream()))
     return (y, ymax) if want_rowmax else y
 
@@ -623,9 +623,9 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
         wide = (plain_rows and dim_in % 32 == 0 and dim_in >= 64 and dim_out >= 64 and rows * T >= 1024
                 and x.data_ptr() % 16 == 0)
         out_comps = 1 if (inds == 0 or y_layout == LAYOUT_COMP_CHAN) else T
-        if wide and mode == LINEAR_F16X2:
+        if (plain_rows and mode == LINEAR_F16X2 and f16x2_supported(rows * T, dim_in, dim_out, x)):
             x2 = x.reshape(rows * T, dim_in)
-            L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(W)), _p(x2), _p(row_absmax(x2)), 1, 1, rows * T,
+            L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(W)), _p(x2), _p(row_absmax(x2)), 1, 1, 1, rows * T,
                                                 dim_in, dim_out, _p(bias), int(act), int(bool(accumulate)),
                                                 out_comps, _p(y), None, _stream()))
         elif wide and mode == LINEAR_BF16X3:
