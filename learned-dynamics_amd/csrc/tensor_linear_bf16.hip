@@ -8,10 +8,20 @@
 // so the only rounding beyond fp32 accumulation is the bf16 storage of the activations themselves.
 // These layers are bound by HBM traffic (2 bytes per element in and out), not by the MFMAs.
 //
-// Tile 128x128 per workgroup, 4 waves (2x2) of 64x64, K slab 32, LDS double buffer
-// (2 x 30 KB -> two workgroups per CU), one barrier per slab.  Tiles go HBM -> registers -> LDS
-// as 16-byte pieces; LDS rows are 80 bytes (5 quads, odd: ds_read_b128 of 8 consecutive rows
-// covers all banks).  v_mfma_f32_32x32x16_bf16: A[m][k] lane = m + 32*(k/8), 8 k per lane.
+// Row-streaming shape: a workgroup of WAVES waves owns 32 WAVES rows x 32 NI columns; wave w owns
+// rows [32 w, 32 w + 32) and all columns of the tile.
+//   * x never touches LDS: lane = row + 32 g loads the 16 consecutive bf16 of ITS row that it
+//     feeds to the matrix core (k = 32 c + 16 g .. + 16 of chunk c, two 16-byte loads that ARE
+//     the MFMA operands), two chunks ahead.  No load is predicated (rows past the end are
+//     clamped and never written), so loads stay in flight across the loop.
+//   * the two W planes go global -> registers -> LDS, double buffered, chunk of 32 k (80-byte rows:
+//     conflict free for 16-byte reads), one barrier per chunk; W is requested before x because
+//     loads return in order and W (L2 resident) is needed first.
+//   * W is the FIRST matrix operand and x the second, so a lane ends up with its own row of x and
+//     four consecutive output channels per accumulator quad: the epilogue writes 8-byte (bf16) or
+//     16-byte (fp32) vectors, one row pointer and one bounds check per lane.
+// v_mfma_f32_32x32x16_bf16: A[i][k]: lane = i + 32*(k/8), 8 k per lane; B[k][j] likewise;
+// D[i][j]: j = lane%32, i = 8*(q/4) + 4*(lane/32) + q%4 for register q.
 #include "common.hpp"
 #include <type_traits>
 
@@ -19,30 +29,41 @@ namespace mg {
 namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef float floatx4 __attribute__((ext_vector_type(4)));
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
-constexpr int kBK = 32;
-constexpr int kRowB = 80;
-constexpr int kPlane = 128 * kRowB;
-constexpr int kBuf = 3 * kPlane;            // x, W hi, W mid
+constexpr int kCK = 32;      // k per chunk (two MFMA steps)
+constexpr int kRowW = 80;    // bytes per LDS row of one W plane (64 + 16 pad)
 
-__device__ __forceinline__ float activate(float v, int act) {
-    if (act == 1) return v * __frcp_rn(1.0f + __expf(-v));
-    if (act == 2) return v > 0.f ? v : 0.1f * v;
+template <int ACT>
+__device__ __forceinline__ float activate_c(float v) {
+    // SiLU through the hardware exp2 and reciprocal (about 1 ulp each)
+    if constexpr (ACT == 1) return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
+    if constexpr (ACT == 2) return v > 0.f ? v : 0.1f * v;
     return v;
 }
 
-struct Stage {
-    bf16x8 x[2];
-    bf16x8 w[2][2];
-};
+__device__ __forceinline__ floatx4 load4(const float* p) { return *reinterpret_cast<const floatx4*>(p); }
+__device__ __forceinline__ floatx4 load4(const __bf16* p) {
+    const bf16x4 t = *reinterpret_cast<const bf16x4*>(p);
+    return floatx4{(float)t[0], (float)t[1], (float)t[2], (float)t[3]};
+}
+__device__ __forceinline__ void store4(float* p, floatx4 v) { *reinterpret_cast<floatx4*>(p) = v; }
+__device__ __forceinline__ void store4(__bf16* p, floatx4 v) {
+    *reinterpret_cast<bf16x4*>(p) = bf16x4{(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
+}
 
-template <typename YT>
-__global__ void __launch_bounds__(256)
-linear_rows_bf16_kernel(const __bf16* __restrict__ Wp, long plane_elems, const __bf16* __restrict__ X, long R, int I,
-                        int O, const float* __restrict__ bias, int act, int accumulate, YT* __restrict__ Y,
-                        int tiles_n, long tiles_total, int out_T) {
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kBuf];
+template <int WAVES, int NI, typename YT>
+__global__ void __launch_bounds__(64 * WAVES)
+linear_rows_bf16_kernel(const __bf16* __restrict__ Wp, long plane_elems, int w_rows, const __bf16* __restrict__ X,
+                        long R, int I, int O, const float* __restrict__ bias, int act, int accumulate,
+                        YT* __restrict__ Y, int tiles_n, long tiles_total, int out_T) {
+    constexpr int TM = 32 * WAVES, TN = 32 * NI, THREADS = 64 * WAVES;
+    constexpr int kPlaneW = TN * kRowW, kBufW = 2 * kPlaneW;
+    constexpr int kPieces = 8 * TN;                          // 16-byte pieces of W per chunk (2 planes x TN rows x 4)
+    constexpr int kPer = (kPieces + THREADS - 1) / THREADS;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kBufW];
 
     const long bid = blockIdx.x;
     const long per_xcd = (tiles_total + 7) / 8;
@@ -53,121 +74,177 @@ linear_rows_bf16_kernel(const __bf16* __restrict__ Wp, long plane_elems, const _
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
-    const int wave_m = wave >> 1, wave_n = wave & 1;
-    const long r0 = tile_m * 128;
-    const int n0 = tile_n * 128;
-    const int kgroup = lane >> 5;
+    const int m = lane & 31, g = lane >> 5;
+    const long r0 = tile_m * TM;
+    const int n0 = tile_n * TN;
 
-    floatx16 acc[2][2];
+    floatx16 acc[NI];
 #pragma unroll
-    for (int mi = 0; mi < 2; mi++)
+    for (int ni = 0; ni < NI; ni++)
 #pragma unroll
-        for (int ni = 0; ni < 2; ni++)
-#pragma unroll
-            for (int q = 0; q < 16; q++) acc[mi][ni][q] = 0.f;
+        for (int q = 0; q < 16; q++) acc[ni][q] = 0.f;
 
-    // a 128 x 32 bf16 tile is 512 pieces of 16 bytes: thread -> rows (tid>>2) and (tid>>2)+64, piece tid&3
-    const int sr = tid >> 2, sc = (tid & 3) * 8;
-    const int k_last = I - kBK;
-    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
-
-    auto load_stage = [&](Stage& g, int k0) {
-        k0 = k0 < I ? k0 : k_last;                     // surplus loads of the last trips are never used
+    const long my_row = r0 + wave * 32 + m;
+    const long ld_row = my_row < R ? my_row : R - 1;       // clamped: such rows are never written
+    const __bf16* xrow = X + ld_row * I + 16 * g;
+    const __bf16* wsrc[kPer];
+    int wdst[kPer];
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const long r = r0 + sr + 64 * h;
-            g.x[h] = r < R ? *reinterpret_cast<const bf16x8*>(X + r * I + k0 + sc) : zero;
-#pragma unroll
-            for (int p = 0; p < 2; p++)
-                g.w[p][h] = *reinterpret_cast<const bf16x8*>(Wp + p * plane_elems + (long)(n0 + sr + 64 * h) * I + k0 + sc);
-        }
-    };
-    auto store_stage = [&](const Stage& g, unsigned char* buf) {
-#pragma unroll
-        for (int h = 0; h < 2; h++) {
-            const int off = (sr + 64 * h) * kRowB + sc * 2;
-            *reinterpret_cast<bf16x8*>(buf + off) = g.x[h];
-            *reinterpret_cast<bf16x8*>(buf + kPlane + off) = g.w[0][h];
-            *reinterpret_cast<bf16x8*>(buf + 2 * kPlane + off) = g.w[1][h];
-        }
-    };
-
-    int a_off[2], b_off[2];
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        a_off[i] = ((wave_m * 2 + i) * 32 + (lane & 31)) * kRowB + kgroup * 16;
-        b_off[i] = kPlane + ((wave_n * 2 + i) * 32 + (lane & 31)) * kRowB + kgroup * 16;
+    for (int j = 0; j < kPer; j++) {
+        int q = tid + THREADS * j;
+        if (q >= kPieces) q = kPieces - 1;                   // surplus threads repeat the last piece
+        const int plane = q / (4 * TN), row = (q % (4 * TN)) >> 2, piece = q & 3;
+        int wrow = n0 + row;
+        if (wrow >= w_rows) wrow = w_rows - 1;               // columns past dim_out are never written
+        wsrc[j] = Wp + plane * plane_elems + (long)wrow * I + 8 * piece;
+        wdst[j] = plane * kPlaneW + row * kRowW + piece * 16;
     }
-    auto compute = [&](const unsigned char* buf) {
+    const int k_last = I - kCK;
+
+    struct ARegs { bf16x8 v[2]; };
+    struct WRegs { bf16x8 v[kPer]; };
+    auto load_a = [&](ARegs& a, int k0) {
+        k0 = k0 < I ? k0 : k_last;                           // surplus loads of the last trips are never used
+#pragma unroll
+        for (int s = 0; s < 2; s++) a.v[s] = *reinterpret_cast<const bf16x8*>(xrow + k0 + 8 * s);
+    };
+    auto load_w = [&](WRegs& w, int k0) {
+        k0 = k0 < I ? k0 : k_last;
+#pragma unroll
+        for (int j = 0; j < kPer; j++) w.v[j] = *reinterpret_cast<const bf16x8*>(wsrc[j] + k0);
+    };
+    auto store_w = [&](const WRegs& w, unsigned char* buf) {
+#pragma unroll
+        for (int j = 0; j < kPer; j++) *reinterpret_cast<bf16x8*>(buf + wdst[j]) = w.v[j];
+    };
+    const int b_off = m * kRowW + 32 * g;
+    const bf16x8 zero = {0, 0, 0, 0, 0, 0, 0, 0};
+    auto compute = [&](const ARegs& a, const unsigned char* buf, bool live) {
 #pragma unroll
         for (int s = 0; s < 2; s++) {
-            bf16x8 a[2], b[2][2];
+            const bf16x8 xs = live ? a.v[s] : zero;          // a surplus odd chunk contributes nothing
 #pragma unroll
-            for (int i = 0; i < 2; i++) {
-                a[i] = *reinterpret_cast<const bf16x8*>(buf + a_off[i] + s * 32);
-#pragma unroll
-                for (int p = 0; p < 2; p++) b[i][p] = *reinterpret_cast<const bf16x8*>(buf + p * kPlane + b_off[i] + s * 32);
+            for (int ni = 0; ni < NI; ni++) {
+                const bf16x8 wh = *reinterpret_cast<const bf16x8*>(buf + b_off + ni * 32 * kRowW + 16 * s);
+                const bf16x8 wm = *reinterpret_cast<const bf16x8*>(buf + kPlaneW + b_off + ni * 32 * kRowW + 16 * s);
+                acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wm, xs, acc[ni], 0, 0, 0);   // small term first
+                acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wh, xs, acc[ni], 0, 0, 0);
             }
-#pragma unroll
-            for (int p = 1; p >= 0; p--)     // small terms first
-#pragma unroll
-                for (int mi = 0; mi < 2; mi++)
-#pragma unroll
-                    for (int ni = 0; ni < 2; ni++)
-                        acc[mi][ni] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a[mi], b[ni][p], acc[mi][ni], 0, 0, 0);
         }
     };
 
     unsigned char* buf0 = lds;
-    unsigned char* buf1 = lds + kBuf;
-    Stage ga, gb;
-    load_stage(ga, 0);
-    load_stage(gb, kBK);
-    store_stage(ga, buf0);
-    load_stage(ga, 2 * kBK);
-    // slabs in pairs (even slab in buf0, odd slab in buf1); an odd slab count runs one surplus slab
-    // on clamped (valid) addresses whose products are discarded by the k0 < I test
-    for (int k0 = 0; k0 < I; k0 += 2 * kBK) {
+    unsigned char* buf1 = lds + kBufW;
+    ARegs a0, a1;
+    WRegs w;
+    load_w(w, 0);
+    load_a(a0, 0);
+    store_w(w, buf0);
+    load_w(w, kCK);
+    load_a(a1, kCK);
+    __syncthreads();
+    for (int k0 = 0; k0 < I; k0 += 2 * kCK) {
+        compute(a0, buf0, true);
+        store_w(w, buf1);
+        __builtin_amdgcn_sched_barrier(0);     // keep this issue order: the compiler would hoist the loads
+        load_w(w, k0 + 2 * kCK);
+        __builtin_amdgcn_sched_barrier(0);
+        load_a(a0, k0 + 2 * kCK);
         __syncthreads();
-        compute(buf0);
-        store_stage(gb, buf1);
-        load_stage(gb, k0 + 3 * kBK);
+        compute(a1, buf1, k0 + kCK < I);
+        store_w(w, buf0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(w, k0 + 3 * kCK);
+        __builtin_amdgcn_sched_barrier(0);
+        load_a(a1, k0 + 3 * kCK);
         __syncthreads();
-        if (k0 + kBK < I) compute(buf1);
-        store_stage(ga, buf0);
-        load_stage(ga, k0 + 4 * kBK);
     }
 
-    auto epilogue = [&](auto plain) {
-        constexpr bool kPlain = decltype(plain)::value;
+    // lane (m, g) holds row my_row and, for accumulator quad qq of block ni, the four channels
+    // n0 + 32 ni + 8 qq + 4 g .. + 4
+    if (my_row >= R) return;
+    if (out_T == 1 && n0 + TN <= O && (O & 3) == 0) {
+        YT* yrow = Y + my_row * O + n0 + 4 * g;
+        const float* brow = bias ? bias + n0 + 4 * g : nullptr;
+        auto epilogue = [&](auto act_tag) {
+            constexpr int kAct = decltype(act_tag)::value;
 #pragma unroll
-        for (int ni = 0; ni < 2; ni++) {
-            const int n = n0 + (wave_n * 2 + ni) * 32 + (lane & 31);
-            if (n >= O) continue;
-            const float bv = bias ? bias[n] : 0.f;
+            for (int ni = 0; ni < NI; ni++)
 #pragma unroll
-            for (int mi = 0; mi < 2; mi++) {
+                for (int qq = 0; qq < 4; qq++) {
+                    const int c = 32 * ni + 8 * qq;
+                    floatx4 v = {acc[ni][4 * qq], acc[ni][4 * qq + 1], acc[ni][4 * qq + 2], acc[ni][4 * qq + 3]};
+                    if (brow) v += load4(brow + c);
 #pragma unroll
-                for (int q = 0; q < 16; q++) {
-                    const long r = r0 + (wave_m * 2 + mi) * 32 + 8 * (q / 4) + 4 * kgroup + (q % 4);
-                    if (r < R) {
-                        long addr;
-                        if constexpr (kPlain) {
-                            addr = r * O + n;
-                        } else {
-                            const long row = r / out_T;
-                            addr = (row * O + n) * out_T + (r - row * out_T);
-                        }
-                        float v = activate(acc[mi][ni][q] + bv, act);
-                        if (accumulate) v += (float)Y[addr];
-                        Y[addr] = (YT)v;
-                    }
+                    for (int i = 0; i < 4; i++) v[i] = activate_c<kAct>(v[i]);
+                    if (accumulate) v += load4(yrow + c);
+                    store4(yrow + c, v);
                 }
+        };
+        if (act == 1) epilogue(std::integral_constant<int, 1>{});
+        else if (act == 2) epilogue(std::integral_constant<int, 2>{});
+        else epilogue(std::integral_constant<int, 0>{});
+        return;
+    }
+    // general path: partial column tiles, or rows that are (row, comp) pairs with y stored (row, chan, comp)
+    const long row = my_row / out_T;
+    const long comp = my_row - row * out_T;
+#pragma unroll
+    for (int ni = 0; ni < NI; ni++)
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+            const int n = n0 + 32 * ni + 8 * (q / 4) + 4 * g + (q % 4);
+            if (n < O) {
+                const long addr = (row * O + n) * out_T + comp;
+                float v = acc[ni][q] + (bias ? bias[n] : 0.f);
+                v = act == 1 ? activate_c<1>(v) : (act == 2 ? activate_c<2>(v) : v);
+                if (accumulate) v += (float)Y[addr];
+                Y[addr] = (YT)v;
             }
         }
-    };
-    if (out_T == 1) epilogue(std::true_type{});
-    else epilogue(std::false_type{});
+}
+
+struct Shape {
+    int ni, waves;
+};
+inline Shape choose_shape(long R, int O) {
+    Shape s;
+    s.ni = O <= 32 ? 1 : (O <= 64 ? 2 : (O <= 128 ? 4 : 8));
+    const long tiles = ceil_div(R, 256) * ceil_div(O, 32 * s.ni);
+    s.waves = tiles >= 512 ? 8 : 4;
+    return s;
+}
+
+template <int WAVES, int NI, typename YT>
+int launch(const __bf16* Wp, long plane_elems, int w_rows, const __bf16* x, long rows, int I, int O, const float* bias,
+           int act, int accumulate, YT* y, int out_T, hipStream_t st) {
+    const long tiles_m = ceil_div(rows, 32 * WAVES);
+    const int tiles_n = (int)ceil_div(O, 32 * NI);
+    const long total = tiles_m * tiles_n;
+    const long grid = ceil_div(total, 8) * 8;
+    MG_REQUIRE(grid <= 0x7fffffffL, "mg_tensor_linear_bf16: grid too large (rows=%ld dim_out=%d)", rows, O);
+    hipLaunchKernelGGL((linear_rows_bf16_kernel<WAVES, NI, YT>), dim3((unsigned)grid), dim3(64 * WAVES), 0, st, Wp,
+                       plane_elems, w_rows, x, rows, I, O, bias, act, accumulate, y, tiles_n, total, out_T);
+    return check_launch("mg_tensor_linear_bf16");
+}
+
+template <typename YT>
+int dispatch(const __bf16* Wp, long plane_elems, int w_rows, const __bf16* x, long rows, int I, int O,
+             const float* bias, int act, int accumulate, YT* y, int out_T, hipStream_t st) {
+    const Shape sh = choose_shape(rows, O);
+#define MG_BF16_LAUNCH(WV, N) \
+    return launch<WV, N, YT>(Wp, plane_elems, w_rows, x, rows, I, O, bias, act, accumulate, y, out_T, st)
+    if (sh.waves == 8) {
+        if (sh.ni == 1) MG_BF16_LAUNCH(8, 1);
+        if (sh.ni == 2) MG_BF16_LAUNCH(8, 2);
+        if (sh.ni == 4) MG_BF16_LAUNCH(8, 4);
+        MG_BF16_LAUNCH(8, 8);
+    }
+    if (sh.ni == 1) MG_BF16_LAUNCH(4, 1);
+    if (sh.ni == 2) MG_BF16_LAUNCH(4, 2);
+    if (sh.ni == 4) MG_BF16_LAUNCH(4, 4);
+    MG_BF16_LAUNCH(4, 8);
+#undef MG_BF16_LAUNCH
 }
 
 }  // namespace
@@ -184,23 +261,17 @@ int mg_tensor_linear_bf16(const void* packed_W, const void* x, long rows, int di
     MG_REQUIRE(act >= 0 && act <= 2, "mg_tensor_linear_bf16: unknown activation %d", act);
     MG_REQUIRE(out_comps == 1 || out_comps == 3 || out_comps == 9, "mg_tensor_linear_bf16: out_comps must be 1, 3 or 9");
     if (rows == 0 || dim_out == 0) return MG_OK;
-    MG_REQUIRE(packed_W && x && y && aligned16(x) && aligned16(packed_W), "mg_tensor_linear_bf16: null or unaligned pointer");
-    const long tiles_m = ceil_div(rows, 128);
-    const int tiles_n = (int)ceil_div(dim_out, 128);
-    const long total = tiles_m * tiles_n;
-    const long grid = ceil_div(total, 8) * 8;
-    MG_REQUIRE(grid <= 0x7fffffffL, "mg_tensor_linear_bf16: grid too large (rows=%ld dim_out=%d)", rows, dim_out);
-    const long plane_elems = (long)tiles_n * 128 * dim_in;
+    MG_REQUIRE(packed_W && x && y && aligned16(x) && aligned16(packed_W) && aligned16(y),
+               "mg_tensor_linear_bf16: null or unaligned pointer");
+    MG_REQUIRE(bias == nullptr || aligned16(bias), "mg_tensor_linear_bf16: bias must be 16-byte aligned");
+    const int w_rows = (int)ceil_div(dim_out, 128) * 128;       // rows per plane in the packed format
+    const long plane_elems = (long)w_rows * dim_in;
     hipStream_t st = (hipStream_t)stream;
     if (y_is_bf16)
-        hipLaunchKernelGGL(linear_rows_bf16_kernel<__bf16>, dim3((unsigned)grid), dim3(256), 0, st,
-                           static_cast<const __bf16*>(packed_W), plane_elems, static_cast<const __bf16*>(x), rows, dim_in,
-                           dim_out, bias, act, accumulate, static_cast<__bf16*>(y), tiles_n, total, out_comps);
-    else
-        hipLaunchKernelGGL(linear_rows_bf16_kernel<float>, dim3((unsigned)grid), dim3(256), 0, st,
-                           static_cast<const __bf16*>(packed_W), plane_elems, static_cast<const __bf16*>(x), rows, dim_in,
-                           dim_out, bias, act, accumulate, static_cast<float*>(y), tiles_n, total, out_comps);
-    return check_launch("mg_tensor_linear_bf16");
+        return dispatch<__bf16>(static_cast<const __bf16*>(packed_W), plane_elems, w_rows, static_cast<const __bf16*>(x),
+                                rows, dim_in, dim_out, bias, act, accumulate, static_cast<__bf16*>(y), out_comps, st);
+    return dispatch<float>(static_cast<const __bf16*>(packed_W), plane_elems, w_rows, static_cast<const __bf16*>(x), rows,
+                           dim_in, dim_out, bias, act, accumulate, static_cast<float*>(y), out_comps, st);
 }
 
 }  // extern "C"
