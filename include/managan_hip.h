@@ -238,6 +238,20 @@ int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows,
                            float* dW, mg_stream_t stream);
 
 /* ------------------------------------------------------------------------
+ * Ant16 (managan/codegen_tensor_products.py:19-34; ant16_o0_cuda / ant16_o1_cuda / ant16_o2_cuda /
+ * ant16_oc_cuda, extensions/codegen_tensops/codegen_tensops.cpp:610-667,823-890,1072-1140,1327-1390):
+ *   y[b,o,:] (+)= sum_t sum_{i<dim_l, j<dim_r} P_t[o,i,j] * (left_t[b,i,:] (x) x_r[b,j,:])
+ * over n_terms <= 4 product types that share the output rank rank_o.  labels[t] indexes the order
+ * 000 110 220 011 101 121 211 022 202 112 222 111 212; P_t (dim_o, dim_l, dim_r) and
+ * left_t (rows, dim_l, (3,)^rank_l) dense; x_k (rows, dim_k, (3,)^k); y (rows, dim_o, (3,)^rank_o).
+ * labels, P and left are HOST arrays of n_terms entries (device pointers inside).  accumulate != 0
+ * adds into y.  One call per reference function (o0: 000 110 220; o1: 011 101 121 211;
+ * o2: 022 202 112 222; oc: 111 into y_1c and 212 into y_2c as two calls). */
+int mg_ant16_fwd(int rank_o, int n_terms, const int* labels, const float* const* P, const float* const* left,
+                 const float* x_0, const float* x_1, const float* x_2, long rows, int dim_0, int dim_1, int dim_2,
+                 int dim_l, int accumulate, float* y, mg_stream_t stream);
+
+/* ------------------------------------------------------------------------
  * PaiNN message passing (archs/meanflow_painn8.py:25-35,77-100).
  * ---------------------------------------------------------------------- */
 /* radial_encode(r, n, rmax) (archs/meanflow_painn8.py:25-35): out (E,n) =

@@ -376,6 +376,90 @@ def cow_o1_bwr(l_0, l_1, *dys):
     return _cow_bwd(1, 1, l_0, l_1, dys)
 
 
+# ---------------------------------------------------------------- Ant16
+def _ant16_check(x_0, x_1, x_2, pairs):
+    """Shape checks of ant16_o*_cuda (extensions/codegen_tensops/codegen_tensops.cpp:610-660), same messages."""
+    for t, nm in ((x_0, "x_0"), (x_1, "x_1"), (x_2, "x_2")):
+        if t is not None:
+            _check_input(t, nm)
+    batch = None
+    dims = [None, None, None]
+    for k, (t, nm) in enumerate(((x_0, "x_0"), (x_1, "x_1"), (x_2, "x_2"))):
+        if t is None:
+            continue
+        if t.dim() != 2 + k:
+            raise RuntimeError(f"{nm} has wrong number of axes")
+        if batch is None:
+            batch = int(t.size(0))
+        elif t.size(0) != batch:
+            raise RuntimeError(f"{nm}: expected axis 0 to have size batch")
+        dims[k] = int(t.size(1))
+        for ax in range(2, 2 + k):
+            if t.size(ax) != 3:
+                raise RuntimeError(f"{nm}: expected axis {ax} to have size 3")
+    dim_l = None
+    for lab, P, left in pairs:
+        _check_input(P, f"P_{lab}")
+        _check_input(left, f"left_{lab}")
+        rl, rr, ro = int(lab[0]), int(lab[1]), int(lab[2])
+        if P.dim() != 3:
+            raise RuntimeError(f"P_{lab} has wrong number of axes")
+        if P.size(0) != dims[ro]:
+            raise RuntimeError(f"P_{lab}: expected axis 0 to have size dim_{ro}")
+        if dim_l is None:
+            dim_l = int(P.size(1))
+        elif P.size(1) != dim_l:
+            raise RuntimeError(f"P_{lab}: expected axis 1 to have size dim_l")
+        if P.size(2) != dims[rr]:
+            raise RuntimeError(f"P_{lab}: expected axis 2 to have size dim_{rr}")
+        if left.dim() != 2 + rl:
+            raise RuntimeError(f"left_{lab} has wrong number of axes")
+        if left.size(0) != batch:
+            raise RuntimeError(f"left_{lab}: expected axis 0 to have size batch")
+        if left.size(1) != dim_l:
+            raise RuntimeError(f"left_{lab}: expected axis 1 to have size dim_l")
+        for ax in range(2, 2 + rl):
+            if left.size(ax) != 3:
+                raise RuntimeError(f"left_{lab}: expected axis {ax} to have size 3")
+    return batch, dims, dim_l
+
+
+def _ant16(rank_o, x_0, x_1, x_2, pairs):
+    """y (rows, dim_o, (3,)^rank_o) = sum over the given (label, P, left) of the Ant16 contraction."""
+    batch, dims, dim_l = _ant16_check(x_0, x_1, x_2, pairs)
+    dev = pairs[0][1].device
+    n = len(pairs)
+    labels = (ctypes.c_int * n)(*[BEE_ORDER.index(lab) for lab, _, _ in pairs])
+    Ps = (ctypes.c_void_p * n)(*[P.data_ptr() for _, P, _ in pairs])
+    lefts = (ctypes.c_void_p * n)(*[left.data_ptr() for _, _, left in pairs])
+    with torch.cuda.device(dev):
+        y = torch.empty(_shape(batch, dims[rank_o], rank_o), dtype=torch.float32, device=dev)
+        if batch > 0:
+            L.check(_lib.mg_ant16_fwd(rank_o, n, labels, Ps, lefts, _p(x_0), _p(x_1), _p(x_2), batch,
+                                      dims[0] or 0, dims[1] or 0, dims[2] or 0, dim_l, 0, _p(y), _stream()))
+    return y
+
+
+def ant16_o0(x_0, x_1, x_2, P_000, left_000, P_110, left_110, P_220, left_220):
+    return [_ant16(0, x_0, x_1, x_2, [("000", P_000, left_000), ("110", P_110, left_110), ("220", P_220, left_220)])]
+
+
+def ant16_o1(x_0, x_1, x_2, P_011, left_011, P_101, left_101, P_121, left_121, P_211, left_211):
+    return [_ant16(1, x_0, x_1, x_2, [("011", P_011, left_011), ("101", P_101, left_101), ("121", P_121, left_121),
+                                      ("211", P_211, left_211)])]
+
+
+def ant16_o2(x_0, x_1, x_2, P_022, left_022, P_202, left_202, P_112, left_112, P_222, left_222):
+    return [_ant16(2, x_0, x_1, x_2, [("022", P_022, left_022), ("202", P_202, left_202), ("112", P_112, left_112),
+                                      ("222", P_222, left_222)])]
+
+
+def ant16_oc(x_1, x_2, P_111, left_111, P_212, left_212):
+    """The two chiral products: (y_1c, y_2c).  x_2 only fixes dim_2 (rank-2 output channels)."""
+    return [_ant16(1, None, x_1, x_2, [("111", P_111, left_111)]),
+            _ant16(2, None, x_1, x_2, [("212", P_212, left_212)])]
+
+
 def tensor_prod_bare(inds_l, inds_r, inds_o, x_l, x_r):
     """TensorProdBare.forward for operands (..., chan, (3,)^inds); leading dims must agree."""
     _check_input(x_l, "x_l")

@@ -1,6 +1,7 @@
 """Drop-in for the reference's `codegen_tensops_cuda` extension
 (extensions/codegen_tensops/codegen_tensops.cpp:1980-2011).  The Bee and Cow
-families are implemented; the legacy Ant16 family raises NotImplementedError."""
+families and the Ant16 forward functions run on the HIP kernels; the Ant16 backward functions
+(training of the legacy architectures) raise NotImplementedError."""
 import importlib
 
 _ops = importlib.import_module("learned-dynamics_amd.ops")
@@ -23,13 +24,18 @@ def set_kern_attributes():
 
 def _ant16_unavailable(name):
     def fn(*args, **kwargs):
-        raise NotImplementedError(f"{name}: the Ant16 kernel family is not implemented")
+        raise NotImplementedError(f"{name}: only the forward functions of the Ant16 family are implemented")
     fn.__name__ = name
     return fn
 
 
+ant16_o0_cuda = _ops.ant16_o0
+ant16_o1_cuda = _ops.ant16_o1
+ant16_o2_cuda = _ops.ant16_o2
+ant16_oc_cuda = _ops.ant16_oc
+
 for _o in ("o0", "o1", "o2", "oc"):
-    for _suffix in ("", "_backward", "_backleft", "_wtsback"):
+    for _suffix in ("_backward", "_backleft", "_wtsback"):
         _name = f"ant16_{_o}{_suffix}_cuda"
         globals()[_name] = _ant16_unavailable(_name)
 for _suffix in ("", "_backward", "_backleft", "_wtsback"):

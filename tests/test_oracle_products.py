@@ -147,6 +147,31 @@ def test_ant16_reduces_to_bee_for_diagonal_weights():
     assert torch.allclose(y2, prods["022"] + prods["202"] + prods["112"] + prods["222"] + prods["212"])
 
 
+def test_ant16_against_explicit_loops():
+    """P[o, l, r] pairs channel l of `left` with channel r of x (and not the other way round): explicit
+    loops over (b, o, l, r) around the single-channel products, on sizes where every axis differs."""
+    g = torch.Generator().manual_seed(21)
+    batch, dims, dl = 2, (3, 4, 2), 5
+    x = [torch.randn(batch, dims[k], *([3] * k), generator=g, dtype=torch.float64) for k in range(3)]
+    P = {lab: torch.randn(dims[int(lab[2])], dl, dims[int(lab[1])], generator=g, dtype=torch.float64)
+         for lab in OP.BEE_ORDER}
+    left = {lab: torch.randn(batch, dl, *([3] * int(lab[0])), generator=g, dtype=torch.float64)
+            for lab in OP.BEE_ORDER}
+    ys = OP.ant16(x[0], x[1], x[2], P, left)
+    want = [torch.zeros_like(y) for y in ys]
+    for lab in OP.BEE_ORDER:
+        rl, rr, ro = int(lab[0]), int(lab[1]), int(lab[2])
+        for b in range(batch):
+            for o in range(dims[ro]):
+                for l in range(dl):
+                    for r in range(dims[rr]):
+                        # product() takes (rows, chan, ...) operands: one row, one channel
+                        prod = OP.product(lab, left[lab][b:b + 1, l:l + 1], x[rr][b:b + 1, r:r + 1])[0, 0]
+                        want[ro][b, o] += P[lab][o, l, r] * prod
+    for y, w in zip(ys, want):
+        assert torch.allclose(y, w)
+
+
 def test_backward_helper_matches_finite_differences():
     (l0, l1, l2), (r0, r1, r2) = _ops(seed=13, rows=2, chan=2)
     g = torch.Generator().manual_seed(14)
