@@ -87,14 +87,15 @@ def test_tensor_linear_autograd(pkg, inds):
     torch.testing.assert_close(Wg.grad.cpu(), Wr.grad, rtol=1e-5, atol=1e-4)
 
 
-@pytest.mark.parametrize("mode", [0, 1])
+@pytest.mark.parametrize("mode", [0, 1, 2])
 @pytest.mark.parametrize("shape", [(5000, 512, 512, 0), (3000, 96, 200, 0), (2000, 64, 128, 1), (1500, 160, 72, 2),
                                    (1024, 64, 64, 0), (4096, 768, 256, 0),
                                    # large enough for the 256x256-tile kernel (ragged last tile; transposed output)
                                    (140001, 64, 512, 0), (90001, 32, 256, 1)])
 def test_linear_modes_agree_with_float64(ops, mode, shape):
-    """fp32 MFMA (mode 0) and bf16x3-split MFMA (mode 1) against a float64 product: both must sit at
-    fp32 rounding level; the split path uses pre-packed weights and may transpose (row, comp) outputs."""
+    """fp32 MFMA (mode 0), bf16x3-split MFMA (mode 1) and two-piece fp16 split (mode 2) against a float64
+    product: all must sit at fp32 rounding level; the split paths use pre-packed weights and may
+    transpose (row, comp) outputs."""
     rows, dim_in, dim_out, inds = shape
     T = 3 ** inds
     g = torch.Generator().manual_seed(77)
@@ -115,6 +116,83 @@ def test_linear_modes_agree_with_float64(ops, mode, shape):
     err = (y.cpu().double() - ref_aos).abs().max().item()
     assert err < 2e-6 * max(1.0, dim_in ** 0.5), err
     torch.testing.assert_close(y.cpu(), ref_aos.float(), rtol=1e-5, atol=1e-6 * dim_in ** 0.5)
+
+
+@pytest.mark.parametrize("shape", [(70000, 512, 512, 1), (3001, 256, 192, 0), (1500, 96, 16, 2), (2048, 1280, 64, 0),
+                                   (1024, 64, 8, 0), (40000, 160, 130, 1), (140001, 64, 256, 2)])
+def test_linear_f16x2_rows_of_very_different_size(ops, shape):
+    """mg_tensor_linear_f16x2 through the C ABI.  Rows spanning twelve orders of magnitude: the per-row
+    power-of-two scales keep the error relative to EACH row's own scale at fp32 rounding level (a single
+    scale for the tensor would not); weight rows of different size likewise.  Also: accumulate, the row
+    maxima the epilogue emits, and their use as the next call's bounds."""
+    rows, dim_in, dim_out, act = shape
+    g = torch.Generator().manual_seed(rows + dim_out)
+    W = torch.randn(dim_out, dim_in, generator=g) / dim_in ** 0.5
+    W[::3] *= 1e-4
+    W[1::5] *= 300.0
+    b = torch.randn(dim_out, generator=g) * 1e-3
+    x = torch.randn(rows, dim_in, generator=g)
+    x *= 10.0 ** torch.randint(-6, 7, (rows, 1), generator=g).float()
+    pre = x.double() @ W.double().t() + b.double()
+    ref = {0: pre, 1: torch.nn.functional.silu(pre), 2: torch.where(pre > 0, pre, 0.1 * pre)}[act]
+    # error budget per entry: fp32-level rounding of a length-K dot product whose terms are bounded by
+    # |x row| * |W row|, plus rel 2e-6 of the result (rounding, hardware exp2 / reciprocal in SiLU)
+    budget = (x.abs().amax(1, keepdim=True).double() * W.abs().amax(1).double() * 4e-7 * dim_in ** 0.5
+              + 2e-6 * ref.abs() + 1e-30)
+    y, ymax = ops.tensor_linear_f16x2(W.cuda(), x.cuda(), bias=b.cuda(), act=act, want_rowmax=True)
+    assert bool(((y.cpu().double() - ref).abs() <= budget).all())
+    assert torch.equal(ymax.amax(dim=1), y.abs().amax(dim=1))
+    # explicit bounds: exact maxima, and a loose shared bound (accuracy must not depend on tightness)
+    y2 = ops.tensor_linear_f16x2(W.cuda(), x.cuda(), ops.row_absmax(x.cuda()) * 100.0, bias=b.cuda(), act=act)
+    assert bool(((y2.cpu().double() - ref).abs() <= budget).all())
+    # accumulate into an existing result, bounds taken from the previous call's emitted maxima
+    W2 = torch.randn(dim_in, dim_out, generator=g) / dim_out ** 0.5
+    if dim_out % 32 == 0 and dim_out >= 64:
+        base = torch.randn(rows, dim_in, generator=g)
+        out = base.cuda().clone()
+        ops.tensor_linear_f16x2(W2.cuda(), y, ymax, out=out, accumulate=True)
+        ref2 = base.double() + y.cpu().double() @ W2.double().t()
+        budget2 = (y.cpu().abs().amax(1, keepdim=True).double() * W2.abs().amax(1).double() * 4e-7 * dim_out ** 0.5
+                   + 2e-6 * ref2.abs() + 4e-7 * base.abs().double() + 1e-30)
+        assert bool(((out.cpu().double() - ref2).abs() <= budget2).all())
+
+
+def test_linear_f16x2_component_outputs_and_node_bounds(ops):
+    """Rows that are (node, comp) pairs with one bound per node, output stored (node, chan, comp)."""
+    g = torch.Generator().manual_seed(4)
+    nodes, T, dim_in, dim_out = 700, 9, 320, 16
+    W = torch.randn(dim_out, dim_in, generator=g) / dim_in ** 0.5
+    x = torch.randn(nodes, T, dim_in, generator=g)
+    bound = x.abs().amax(dim=(1, 2)).reshape(nodes, 1)
+    y = ops.tensor_linear_f16x2(W.cuda(), x.reshape(nodes * T, dim_in).cuda(), bound.cuda(), out_comps=T,
+                                rows_per_bound=T)
+    ref = (x.double() @ W.double().t()).transpose(1, 2)
+    assert y.shape == (nodes, dim_out, T)
+    torch.testing.assert_close(y.cpu().double(), ref, rtol=1e-5, atol=2e-6 * dim_in ** 0.5)
+    base = torch.randn(nodes, dim_out, T, generator=g)
+    out = base.cuda().clone()
+    ops.tensor_linear_f16x2(W.cuda(), x.reshape(nodes * T, dim_in).cuda(), bound.cuda(), out=out, accumulate=True,
+                            out_comps=T, rows_per_bound=T)
+    torch.testing.assert_close(out.cpu().double(), base.double() + ref, rtol=1e-5, atol=2e-6 * dim_in ** 0.5)
+
+
+def test_linear_out_bound_is_an_upper_bound(ops):
+    g = torch.Generator().manual_seed(5)
+    W = torch.randn(96, 64, generator=g).cuda()
+    b = torch.randn(96, generator=g).cuda()
+    x = torch.randn(500, 64, generator=g).cuda() * 3
+    xb = ops.row_absmax(x)
+    assert torch.equal(xb[:, 0], x.abs().amax(1))
+    yb = ops.linear_out_bound(W, b, xb)
+    y = torch.nn.functional.silu(torch.nn.functional.linear(x, W, b))
+    assert bool((y.abs().amax(1, keepdim=True) <= yb).all())
+    unit = ops.linear_out_bound(W, b, None)                      # inputs bounded by 1
+    y1 = torch.nn.functional.linear(torch.rand(100, 64, device="cuda") * 2 - 1, W, b)
+    assert unit.shape == (1, 1) and bool((y1.abs().amax() <= unit).all())
+    assert ops.linear_out_bound(W, b, None) is unit                # cached per parameter version
+    with torch.no_grad():
+        W.mul_(2.0)
+    assert float(ops.linear_out_bound(W, b, None)) > float(unit)  # recomputed after an in-place update
 
 
 def test_packed_weight_cache_tracks_in_place_updates(ops):
