@@ -168,13 +168,16 @@ def bench_painn_layer(torch, args):
         actv = block.message.mlp_actv(x_a_d.reshape(N, n))
         xv_flat, xa_flat = x_v_d.reshape(N, n, 3), x_a_d.reshape(N, n)
         t_edge = event_time(torch, lambda: ops.painn_message(graph.row_ptr, graph.dst32, r_ij, filt, actv, xv_flat,
-                                                             0.1, xa_flat, xv_flat), 20)
+                                                             0.1, xa_flat, xv_flat, node_order=graph.cell_order), 20)
+        t_edge_index_order = event_time(torch, lambda: ops.painn_message(graph.row_ptr, graph.dst32, r_ij, filt, actv,
+                                                                         xv_flat, 0.1, xa_flat, xv_flat), 20)
         edge_bytes = E * (16 * n + 4 + 12) + N * (16 * n + 16 * n)
         roofline_hbm = {"kernel": "painn_message_kernel (fused gather-product-scatter)", "bound": "hbm",
                         "achieved": edge_bytes / t_edge / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                         "frac": edge_bytes / t_edge / 1e9 / PEAK_HBM_GBS,
                         "traffic": measured_traffic("painn_message_kernel"),
-                        "bytes_per_launch": edge_bytes, "ms": t_edge * 1e3}
+                        "bytes_per_launch": edge_bytes, "ms": t_edge * 1e3,
+                        "ms_rows_in_index_order": t_edge_index_order * 1e3}
         t_graph = event_time(torch, lambda: gl.graph_setup(r0, box, pos_d, neighbours_max=512, celllist_max=128), 5)
         breakdown = {"filter_gemm_512x512_ms": t_gemm * 1e3, "edge_kernel_ms": t_edge * 1e3,
                      "graph_build_ms_not_in_step": t_graph * 1e3}

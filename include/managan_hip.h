@@ -270,8 +270,11 @@ int mg_painn_radial_linear(const float* r_ij /* (E,3) */, long n_edges, int n, f
  *   out_v[i] = res_v[i] + sum_{e in row i} v*P[0:n] + (v x u)*P[n:2n] + u (x) P[2n:3n]
  *   out_a[i] = res_a[i] + sum_{e in row i} P[3n:4n]
  * filt (E,4n) is the radial MLP output per edge; actv (n_nodes,4n) is mlp_actv applied per
- * NODE (a row-wise function commutes with the gather); res_a/res_v may be NULL. */
-int mg_painn_message(const int* row_ptr /* n_nodes+1 */, const int* dst /* E */, int n_nodes, long n_edges,
+ * NODE (a row-wise function commutes with the gather); res_a/res_v may be NULL.
+ * node_order (n_nodes ints, or NULL) is the order in which rows are processed (e.g. the cell order
+ * of the neighbour search, for cache locality of the gathers); results do not depend on it. */
+int mg_painn_message(const int* row_ptr /* n_nodes+1 */, const int* dst /* E */, const int* node_order,
+                     int n_nodes, long n_edges,
                      const float* r_ij /* (E,3) */, const float* filt /* (E,4n) */,
                      const float* actv /* (n_nodes,4n) */, const float* x_v /* (n_nodes,n,3) */,
                      int n, float epsilon, const float* res_a, const float* res_v,
@@ -331,7 +334,10 @@ int mg_bee_edge_geometry(const float* r_ij /* (E,3) */, long n_edges, float r0,
 int mg_bee_message(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
                    const float* rhat, const float* enc, const float* La, const float* Lv, const float* Ld,
                    int chan, const float* enc_W /* (chan,8) */, const float* enc_b /* (chan) */,
-                   float* P0, float* S1, float* S2, mg_stream_t stream);
+                   float* P0, float* S1, float* S2, float* node_max, mg_stream_t stream);
+/* node_max (above and below; may be NULL): (N, ceil(chan/64)) partial maxima of |S1|, |S2| (of |P0|,
+ * |P1|, |P2| below) per node, which mg_tensor_linear_f16x2 accepts as row bounds of those tensors
+ * (x_rows_per_bound = 3 or 9); no counterpart in the reference. */
 
 /* The 13 products of SelfTensProds.forward (archs/diffuser_atoms15.py:86-88; formulas of
  * managan/codegen_tensor_products.py:235-249) on node rows in component-major layout:
@@ -340,7 +346,7 @@ int mg_bee_message(const int* row_ptr, const int* dst, const int* node_order, in
  * [022,202,112,222,212]: the layout of S1/S2 above, so each rank's output linears are one GEMM. */
 int mg_bee_node_products(long n_nodes, int chan, const float* l0, const float* l1, const float* l2,
                          const float* r0, const float* r1, const float* r2, float* P0, float* P1, float* P2,
-                         mg_stream_t stream);
+                         float* node_max /* needs chan % 64 == 0 */, mg_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * bf16-storage configuration: feature tensors are bf16 in memory (void* below), every

@@ -50,7 +50,7 @@ _SIGNATURES = {
     "mg_tensor_linear_wgrad": [i32, vp, vp, i64, i32, i32, vp, vp],
     "mg_tensor_linear_layout": [i32, vp, i64, i64, vp, i64, i32, i32, vp, i32, i32, i32, i32, vp, vp],
     "mg_bee_edge_geometry": [vp, i64, f32, vp, vp, vp],
-    "mg_bee_message": [vp, vp, vp, i32, i64, vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, vp, vp],
+    "mg_bee_message": [vp, vp, vp, i32, i64, vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, vp, vp, vp],
     "mg_linear_packed_weight_bytes": [i32, i32, ctypes.POINTER(ctypes.c_size_t)],
     "mg_linear_pack_weight": [vp, i64, i64, i32, i32, vp, vp],
     "mg_tensor_linear_packed": [vp, vp, i64, i32, i32, vp, i32, i32, i32, vp, vp],
@@ -69,14 +69,14 @@ _SIGNATURES = {
     "mg_painn_update_pre": [vp, vp, i64, i32, vp, vp, vp],
     "mg_painn_update_vec": [vp, vp, vp, i64, i32, vp, vp],
     "mg_radial_encode": [i32, vp, i64, i32, f32, vp, vp],
-    "mg_bee_node_products": [i64, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp],
+    "mg_bee_node_products": [i64, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp],
     "mg_bee_node_products_bf16": [i64, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp],
     "mg_tensor_linear_bf16": [vp, vp, i64, i32, i32, vp, i32, i32, i32, i32, vp, vp],
     "mg_bee_message_bf16": [vp, vp, vp, i32, i64, vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, vp, vp],
     "mg_segment_sum_csr_bf16": [vp, vp, i32, i32, f32, vp, vp],
     "mg_painn_radial_encode": [vp, i64, i32, f32, vp, vp],
     "mg_painn_radial_linear": [vp, i64, i32, f32, vp, i64, i64, vp, i32, i32, vp, vp],
-    "mg_painn_message": [vp, vp, i32, i64, vp, vp, vp, vp, i32, f32, vp, vp, vp, vp, vp],
+    "mg_painn_message": [vp, vp, vp, i32, i64, vp, vp, vp, vp, i32, f32, vp, vp, vp, vp, vp],
 }
 
 _lib = None

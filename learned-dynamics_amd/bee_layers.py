@@ -134,10 +134,13 @@ class SelfTensProds(nn.Module):
         ops_in = [ops.tensor_linear_fwd(k, lin.W, x, y_layout=C if k else ops.LAYOUT_CHAN_COMP)
                   for side in ((self.L0, self.L1, self.L2), (self.R0, self.R1, self.R2))
                   for k, (lin, x) in enumerate(zip(side, (x_a, x_v, x_d)))]
-        P0, P1, P2 = ops.bee_node_products(*ops_in)
-        y_a = ops.tensor_linear_fwd(0, _cat_Y(self, LABELS_0), P0.reshape(rows, 3 * chan))
-        y_v = ops.tensor_linear_fwd(1, _cat_Y(self, LABELS_1), P1.reshape(rows, 3, 5 * chan), x_layout=C)
-        y_d = ops.tensor_linear_fwd(2, _cat_Y(self, LABELS_2), P2.reshape(rows, 9, 5 * chan), x_layout=C)
+        P0, P1, P2, nmax = ops.bee_node_products(*ops_in, want_node_max=True)
+        # nmax: per-node maxima of the products, the row bounds of the three GEMMs
+        y_a = ops.tensor_linear_fwd(0, _cat_Y(self, LABELS_0), P0.reshape(rows, 3 * chan), row_bound=nmax)
+        y_v = ops.tensor_linear_fwd(1, _cat_Y(self, LABELS_1), P1.reshape(rows, 3, 5 * chan), x_layout=C,
+                                    row_bound=nmax, rows_per_bound=3)
+        y_d = ops.tensor_linear_fwd(2, _cat_Y(self, LABELS_2), P2.reshape(rows, 9, 5 * chan), x_layout=C,
+                                    row_bound=nmax, rows_per_bound=9)
         y_a = y_a.reshape(*rest, dim_a)
         y_v = y_v.reshape(*rest, dim_v, 3)
         y_d = y_d.reshape(*rest, dim_d, 3, 3)
@@ -211,8 +214,8 @@ class Messages(nn.Module):
         Lv = ops.tensor_linear_fwd(1, self.L1.W, x_v.reshape(rows, -1, 3).contiguous(), y_layout=C)
         Ld = ops.tensor_linear_fwd(2, self.L2.W, x_d.reshape(rows, -1, 3, 3).contiguous(), y_layout=C)
         enc, rhat = ops.bee_edge_geometry(r_ij.contiguous(), self.r0)
-        P0, S1, S2 = ops.bee_message(graph.row_ptr, graph.dst32, rhat, enc, La, Lv, Ld, self.lin_enc.weight,
-                                     self.lin_enc.bias, node_order=node_order)
+        P0, S1, S2, nmax = ops.bee_message(graph.row_ptr, graph.dst32, rhat, enc, La, Lv, Ld, self.lin_enc.weight,
+                                           self.lin_enc.bias, node_order=node_order, want_node_max=True)
         E, chan = P0.shape[0], P0.shape[2]
         # scalar channel: per-edge linear + MLP, then the edge sum
         P0 = P0.reshape(E, 3 * chan)
@@ -221,6 +224,8 @@ class Messages(nn.Module):
         psi_a = self.mlp_a(psi_a, plus_identity=True, bound=bound)
         B_a = ops.segment_sum_csr(psi_a, graph.row_ptr, rows).mul_(0.1)
         # vector and rank-2 channels: output linears after the edge sum, on node rows
-        B_v = ops.tensor_linear_fwd(1, self._cat_Y(LABELS_1, 0.1), S1.reshape(rows, 3, 5 * chan), x_layout=C)
-        B_d = ops.tensor_linear_fwd(2, self._cat_Y(LABELS_2, 0.1), S2.reshape(rows, 9, 5 * chan), x_layout=C)
+        B_v = ops.tensor_linear_fwd(1, self._cat_Y(LABELS_1, 0.1), S1.reshape(rows, 3, 5 * chan), x_layout=C,
+                                    row_bound=nmax, rows_per_bound=3)
+        B_d = ops.tensor_linear_fwd(2, self._cat_Y(LABELS_2, 0.1), S2.reshape(rows, 9, 5 * chan), x_layout=C,
+                                    row_bound=nmax, rows_per_bound=9)
         return (B_a.reshape(B, N, -1), B_v.reshape(B, N, -1, 3), B_d.reshape(B, N, -1, 3, 3))

@@ -18,7 +18,8 @@ __global__ void __launch_bounds__(256) node_products_kernel(long n_nodes, int ch
                                                             const T* __restrict__ l1, const T* __restrict__ l2,
                                                             const T* __restrict__ r0, const T* __restrict__ r1,
                                                             const T* __restrict__ r2, T* __restrict__ P0,
-                                                            T* __restrict__ P1, T* __restrict__ P2) {
+                                                            T* __restrict__ P1, T* __restrict__ P2,
+                                                            float* __restrict__ node_max) {
     const long total = n_nodes * chan;
     for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (long)gridDim.x * blockDim.x) {
         const long node = t / chan;
@@ -44,6 +45,7 @@ __global__ void __launch_bounds__(256) node_products_kernel(long n_nodes, int ch
         p0[0] = (T)(a * b);
         p0[chan] = (T)dot;
         p0[2 * chan] = (T)ddot;
+        float mx = fmaxf(fabsf(a * b), fmaxf(fabsf(dot), fabsf(ddot)));
 
         const float cr[3] = {u[1] * v[2] - u[2] * v[1], u[2] * v[0] - u[0] * v[2], u[0] * v[1] - u[1] * v[0]};
 #pragma unroll
@@ -54,6 +56,9 @@ __global__ void __launch_bounds__(256) node_products_kernel(long n_nodes, int ch
             p1[2 * chan] = (T)(u[0] * R[3 * x] + u[1] * R[3 * x + 1] + u[2] * R[3 * x + 2]);   // 121: sum_k l_k r_{x k}
             p1[3 * chan] = (T)(L[3 * x] * v[0] + L[3 * x + 1] * v[1] + L[3 * x + 2] * v[2]);   // 211
             p1[4 * chan] = (T)cr[x];                                                    // 111
+            mx = fmaxf(mx, fmaxf(fmaxf(fabsf(a * v[x]), fabsf(u[x] * b)), fabsf(cr[x])));
+            mx = fmaxf(mx, fabsf(u[0] * R[3 * x] + u[1] * R[3 * x + 1] + u[2] * R[3 * x + 2]));
+            mx = fmaxf(mx, fabsf(L[3 * x] * v[0] + L[3 * x + 1] * v[1] + L[3 * x + 2] * v[2]));
         }
 #pragma unroll
         for (int x = 0; x < 3; x++) {
@@ -69,15 +74,24 @@ __global__ void __launch_bounds__(256) node_products_kernel(long n_nodes, int ch
                 p2[2 * chan] = (T)(u[x] * v[z]);                                        // 112
                 p2[3 * chan] = (T)(L[3 * x] * R[3 * z] + L[3 * x + 1] * R[3 * z + 1] + L[3 * x + 2] * R[3 * z + 2]);  // 222
                 p2[4 * chan] = (T)rc[z];                                                // 212
+                mx = fmaxf(mx, fmaxf(fmaxf(fabsf(a * R[k]), fabsf(L[k] * b)), fmaxf(fabsf(u[x] * v[z]), fabsf(rc[z]))));
+                mx = fmaxf(mx, fabsf(L[3 * x] * R[3 * z] + L[3 * x + 1] * R[3 * z + 1] + L[3 * x + 2] * R[3 * z + 2]));
             }
+        }
+        if (node_max) {
+            // chan is a multiple of 64 here, so a wave lies inside one node: one partial maximum
+            // per (node, 64-channel chunk), a row bound for the GEMMs that read P0 / P1 / P2
+            for (int d = 1; d < kWave; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+            if ((threadIdx.x & (kWave - 1)) == 0) node_max[node * (chan / kWave) + c / kWave] = mx;
         }
     }
 }
 
 template <typename T>
 int launch(const char* what, long n_nodes, int chan, const void* l0, const void* l1, const void* l2, const void* r0,
-           const void* r1, const void* r2, void* P0, void* P1, void* P2, mg_stream_t stream) {
+           const void* r1, const void* r2, void* P0, void* P1, void* P2, float* node_max, mg_stream_t stream) {
     MG_REQUIRE(n_nodes >= 0 && chan >= 0, "%s: negative size", what);
+    MG_REQUIRE(node_max == nullptr || chan % kWave == 0, "%s: node_max needs chan to be a multiple of 64", what);
     if (n_nodes == 0 || chan == 0) return MG_OK;
     MG_REQUIRE(l0 && l1 && l2 && r0 && r1 && r2 && P0 && P1 && P2, "%s: null pointer", what);
     long blocks = ceil_div(n_nodes * chan, 256);
@@ -85,7 +99,7 @@ int launch(const char* what, long n_nodes, int chan, const void* l0, const void*
     hipLaunchKernelGGL(node_products_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, n_nodes,
                        chan, static_cast<const T*>(l0), static_cast<const T*>(l1), static_cast<const T*>(l2),
                        static_cast<const T*>(r0), static_cast<const T*>(r1), static_cast<const T*>(r2),
-                       static_cast<T*>(P0), static_cast<T*>(P1), static_cast<T*>(P2));
+                       static_cast<T*>(P0), static_cast<T*>(P1), static_cast<T*>(P2), node_max);
     return check_launch(what);
 }
 
@@ -97,13 +111,14 @@ using namespace mg;
 extern "C" {
 
 int mg_bee_node_products(long n_nodes, int chan, const float* l0, const float* l1, const float* l2, const float* r0,
-                         const float* r1, const float* r2, float* P0, float* P1, float* P2, mg_stream_t stream) {
-    return launch<float>("mg_bee_node_products", n_nodes, chan, l0, l1, l2, r0, r1, r2, P0, P1, P2, stream);
+                         const float* r1, const float* r2, float* P0, float* P1, float* P2, float* node_max,
+                         mg_stream_t stream) {
+    return launch<float>("mg_bee_node_products", n_nodes, chan, l0, l1, l2, r0, r1, r2, P0, P1, P2, node_max, stream);
 }
 
 int mg_bee_node_products_bf16(long n_nodes, int chan, const void* l0, const void* l1, const void* l2, const void* r0,
                               const void* r1, const void* r2, void* P0, void* P1, void* P2, mg_stream_t stream) {
-    return launch<__bf16>("mg_bee_node_products_bf16", n_nodes, chan, l0, l1, l2, r0, r1, r2, P0, P1, P2, stream);
+    return launch<__bf16>("mg_bee_node_products_bf16", n_nodes, chan, l0, l1, l2, r0, r1, r2, P0, P1, P2, nullptr, stream);
 }
 
 }  // extern "C"

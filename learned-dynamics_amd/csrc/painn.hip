@@ -101,7 +101,8 @@ struct EdgeLoads {
 
 // register budget of 5 waves per SIMD (102 VGPRs): room to keep a whole step's loads in flight
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 5))) painn_message_kernel(
-    const int* __restrict__ row_ptr, const int* __restrict__ dst, long n_nodes, const float* __restrict__ r_ij,
+    const int* __restrict__ row_ptr, const int* __restrict__ dst, const int* __restrict__ node_order, long n_nodes,
+    const float* __restrict__ r_ij,
     const float* __restrict__ filt, const float* __restrict__ actv, const float* __restrict__ x_v, int n,
     float epsilon, const float* __restrict__ res_a, const float* __restrict__ res_v, float* __restrict__ out_a,
     float* __restrict__ out_v, Chunks ch) {
@@ -118,8 +119,10 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 5))
     for (long item_local = wave_local; item_local < per_xcd; item_local += waves_per_xcd) {
         const long item = xcd * per_xcd + item_local;
         if (item >= items) break;
-        const long node = item / ch.n;
-        const int ci = (int)(item - node * ch.n);
+        const long slot = item / ch.n;
+        const int ci = (int)(item - slot * ch.n);
+        // optional processing order (results do not depend on it)
+        const long node = node_order ? node_order[slot] : slot;
         const int L = ch.lanes[ci];
         const int c = ch.start[ci] + (lane & (L - 1)) * 4;
         const int sub = lane / L, per_iter = kWave / L;
@@ -345,7 +348,8 @@ int mg_painn_radial_linear(const float* r_ij, long n_edges, int n, float rmax, c
     return check_launch("mg_painn_radial_linear");
 }
 
-int mg_painn_message(const int* row_ptr, const int* dst, int n_nodes, long n_edges, const float* r_ij,
+int mg_painn_message(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
+                     const float* r_ij,
                      const float* filt, const float* actv, const float* x_v, int n, float epsilon,
                      const float* res_a, const float* res_v, float* out_a, float* out_v, mg_stream_t stream) {
     MG_REQUIRE(n_nodes >= 0 && n_edges >= 0 && n >= 0, "mg_painn_message: negative size");
@@ -364,7 +368,7 @@ int mg_painn_message(const int* row_ptr, const int* dst, int n_nodes, long n_edg
             if (blocks > 256L * 32) blocks = 256L * 32;
             blocks = ceil_div(blocks, 8) * 8;   // the XCD-aware item order needs a multiple of 8
             hipLaunchKernelGGL(painn_message_kernel, dim3((unsigned)blocks), dim3(256), 0, st, row_ptr, dst,
-                               (long)n_nodes, r_ij, filt, actv, x_v, n, epsilon, res_a, res_v, out_a, out_v, ch);
+                               node_order, (long)n_nodes, r_ij, filt, actv, x_v, n, epsilon, res_a, res_v, out_a, out_v, ch);
             return check_launch("mg_painn_message");
         }
     }

@@ -656,10 +656,12 @@ LAYOUT_CHAN_COMP, LAYOUT_COMP_CHAN = 0, 1
 
 
 def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=False,
-                      x_layout=LAYOUT_CHAN_COMP, y_layout=LAYOUT_CHAN_COMP):
+                      x_layout=LAYOUT_CHAN_COMP, y_layout=LAYOUT_CHAN_COMP, row_bound=None, rows_per_bound=1):
     """y[..., o, t] = act(sum_i W[o, i] x[..., i, t] + bias[o]); W may have any strides.
     Layout 0 stores a tensor as (..., chan, (3,)^inds) like the reference; layout 1 is
-    component-major (..., 3^inds, chan), the layout the fused edge kernels read and write."""
+    component-major (..., 3^inds, chan), the layout the fused edge kernels read and write.
+    row_bound ((rows of the GEMM) / rows_per_bound, parts): upper bounds of the row maxima of |x| from
+    the kernel that produced x, used by the split-fp16 matrix path instead of a pass over x."""
     if not W.is_cuda:
         raise RuntimeError("W must be a CUDA tensor")
     _check_input(x, "x")
@@ -709,7 +711,13 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
         out_comps = 1 if (inds == 0 or y_layout == LAYOUT_COMP_CHAN) else T
         if (plain_rows and mode == LINEAR_F16X2 and f16x2_supported(rows * T, dim_in, dim_out, x)):
             x2 = x.reshape(rows * T, dim_in)
-            L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(W)), _p(x2), _p(row_absmax(x2)), 1, 1, 1, rows * T,
+            if row_bound is None:
+                row_bound, rows_per_bound = row_absmax(x2), 1
+            elif row_bound.dim() != 2 or row_bound.size(0) * rows_per_bound != rows * T:
+                raise RuntimeError("row_bound must be (rows / rows_per_bound, parts)")
+            L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(W)), _p(x2), _p(row_bound),
+                                                int(row_bound.size(1)), int(row_bound.size(1)), int(rows_per_bound),
+                                                rows * T,
                                                 dim_in, dim_out, _p(bias), int(act), int(bool(accumulate)),
                                                 out_comps, _p(y), None, _stream()))
         elif wide and mode == LINEAR_BF16X3:
@@ -805,9 +813,11 @@ def bee_message_bf16(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_ord
     return P0, S1, S2
 
 
-def bee_node_products(l0, l1, l2, r0, r1, r2):
+def bee_node_products(l0, l1, l2, r0, r1, r2, want_node_max=False):
     """The 13 products on node rows in component-major layout (float32 or bfloat16 storage):
-    l0/r0 (N,chan), l1/r1 (N,3,chan), l2/r2 (N,9,chan) -> P0 (N,3,chan), P1 (N,3,5,chan), P2 (N,9,5,chan)."""
+    l0/r0 (N,chan), l1/r1 (N,3,chan), l2/r2 (N,9,chan) -> P0 (N,3,chan), P1 (N,3,5,chan), P2 (N,9,5,chan)
+    (+ node_max (N, chan/64): partial maxima of all products per node, float32 operands with
+    chan % 64 == 0 only; None otherwise)."""
     bf = l0.dtype == torch.bfloat16
     for t, nm in ((l0, "l0"), (l1, "l1"), (l2, "l2"), (r0, "r0"), (r1, "r1"), (r2, "r2")):
         (_check_bf16 if bf else _check_input)(t, nm)
@@ -820,9 +830,16 @@ def bee_node_products(l0, l1, l2, r0, r1, r2):
         P0 = torch.empty(N, 3, chan, dtype=l0.dtype, device=l0.device)
         P1 = torch.empty(N, 3, 5, chan, dtype=l0.dtype, device=l0.device)
         P2 = torch.empty(N, 9, 5, chan, dtype=l0.dtype, device=l0.device)
-        fn = _lib.mg_bee_node_products_bf16 if bf else _lib.mg_bee_node_products
-        L.check(fn(N, chan, _p(l0), _p(l1), _p(l2), _p(r0), _p(r1), _p(r2), _p(P0), _p(P1), _p(P2), _stream()))
-    return P0, P1, P2
+        node_max = None
+        if bf:
+            L.check(_lib.mg_bee_node_products_bf16(N, chan, _p(l0), _p(l1), _p(l2), _p(r0), _p(r1), _p(r2), _p(P0),
+                                                   _p(P1), _p(P2), _stream()))
+        else:
+            if want_node_max and chan % 64 == 0:
+                node_max = torch.empty(N, chan // 64, dtype=torch.float32, device=l0.device)
+            L.check(_lib.mg_bee_node_products(N, chan, _p(l0), _p(l1), _p(l2), _p(r0), _p(r1), _p(r2), _p(P0), _p(P1),
+                                              _p(P2), _p(node_max), _stream()))
+    return (P0, P1, P2, node_max) if want_node_max else (P0, P1, P2)
 
 
 def segment_sum_csr_bf16(x_edge, row_ptr, n_rows, scale=1.0):
@@ -880,9 +897,10 @@ def painn_radial_linear(r_ij, n, rmax, W, bias=None, act=ACT_NONE):
     return y
 
 
-def painn_message(row_ptr, dst, r_ij, filt, actv, x_v, epsilon, res_a=None, res_v=None):
+def painn_message(row_ptr, dst, r_ij, filt, actv, x_v, epsilon, res_a=None, res_v=None, node_order=None):
     """Fused gather-product-scatter of the PaiNN message (archs/meanflow_painn8.py:91-100).
-    filt (E,4n), actv (nodes,4n), x_v (nodes,n,3) -> out_a (nodes,n), out_v (nodes,n,3)."""
+    filt (E,4n), actv (nodes,4n), x_v (nodes,n,3) -> out_a (nodes,n), out_v (nodes,n,3).
+    node_order (int32, nodes): processing order of the rows (does not change the results)."""
     _check_input(row_ptr, "row_ptr", torch.int32)
     _check_input(dst, "dst", torch.int32)
     for t, nm in ((r_ij, "r_ij"), (filt, "filt"), (actv, "actv"), (x_v, "x_v")):
@@ -904,11 +922,15 @@ def painn_message(row_ptr, dst, r_ij, filt, actv, x_v, epsilon, res_a=None, res_
             _check_input(t, nm)
             if tuple(t.shape) != shape:
                 raise RuntimeError(f"{nm} has wrong shape")
+    if node_order is not None:
+        _check_input(node_order, "node_order", torch.int32)
+        if node_order.numel() != n_nodes:
+            raise RuntimeError("node_order must have one entry per node")
     dev = x_v.device
     with torch.cuda.device(dev):
         out_a = torch.empty(n_nodes, n, dtype=torch.float32, device=dev)
         out_v = torch.empty(n_nodes, n, 3, dtype=torch.float32, device=dev)
-        L.check(_lib.mg_painn_message(_p(row_ptr), _p(dst), n_nodes, E, _p(r_ij), _p(filt), _p(actv), _p(x_v), n,
+        L.check(_lib.mg_painn_message(_p(row_ptr), _p(dst), _p(node_order), n_nodes, E, _p(r_ij), _p(filt), _p(actv), _p(x_v), n,
                                       float(epsilon), _p(res_a), _p(res_v), _p(out_a), _p(out_v), _stream()))
     return out_a, out_v
 
@@ -927,9 +949,10 @@ def bee_edge_geometry(r_ij, r0):
     return enc, rhat
 
 
-def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=None):
+def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=None, want_node_max=False):
     """Fused products + edge sums of the rank-0/1/2 message (see mg_bee_message).
-    La (N,chan), Lv (N,3,chan), Ld (N,9,chan) -> P0 (E,3,chan), S1 (N,3,5,chan), S2 (N,9,5,chan)."""
+    La (N,chan), Lv (N,3,chan), Ld (N,9,chan) -> P0 (E,3,chan), S1 (N,3,5,chan), S2 (N,9,5,chan)
+    (+ node_max (N, ceil(chan/64)): partial maxima of |S1|, |S2| per node, with want_node_max)."""
     _check_input(row_ptr, "row_ptr", torch.int32)
     _check_input(dst, "dst", torch.int32)
     for t, nm in ((rhat, "rhat"), (enc, "enc"), (La, "La"), (Lv, "Lv"), (Ld, "Ld"), (enc_W, "enc_W"),
@@ -954,9 +977,11 @@ def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=No
         P0 = torch.empty(E, 3, chan, dtype=torch.float32, device=dev)
         S1 = torch.empty(N, 3, 5, chan, dtype=torch.float32, device=dev)
         S2 = torch.empty(N, 9, 5, chan, dtype=torch.float32, device=dev)
+        node_max = torch.empty(N, (chan + 63) // 64, dtype=torch.float32, device=dev) if want_node_max else None
         L.check(_lib.mg_bee_message(_p(row_ptr), _p(dst), _p(node_order), N, E, _p(rhat), _p(enc), _p(La), _p(Lv),
-                                    _p(Ld), chan, _p(enc_W), _p(enc_b), _p(P0), _p(S1), _p(S2), _stream()))
-    return P0, S1, S2
+                                    _p(Ld), chan, _p(enc_W), _p(enc_b), _p(P0), _p(S1), _p(S2), _p(node_max),
+                                    _stream()))
+    return (P0, S1, S2, node_max) if want_node_max else (P0, S1, S2)
 
 
 # ------------------------------------------------- norms, squash, update glue

@@ -64,8 +64,11 @@ def test_bee_message_kernel(ops, chan):
     Ld_cm = Ld.reshape(N, chan, 9).transpose(1, 2).contiguous()
     order = torch.randperm(N).int().cuda()
     for node_order in (None, order):
-        P0, S1, S2 = ops.bee_message(row_ptr, dst.int().cuda(), rhat, enc, La.cuda(), Lv_cm.cuda(), Ld_cm.cuda(),
-                                     encW.cuda(), encb.cuda(), node_order=node_order)
+        P0, S1, S2, nmax = ops.bee_message(row_ptr, dst.int().cuda(), rhat, enc, La.cuda(), Lv_cm.cuda(), Ld_cm.cuda(),
+                                           encW.cuda(), encb.cuda(), node_order=node_order, want_node_max=True)
+        # the emitted per-node maxima are exactly the maxima of what was written
+        assert nmax.shape == (N, (chan + 63) // 64)
+        assert torch.equal(nmax.amax(1), torch.maximum(S1.abs().amax(dim=(1, 2, 3)), S2.abs().amax(dim=(1, 2, 3))))
         # oracle on the device's own enc / rhat (they are checked separately)
         phi_a = torch.nn.functional.linear(enc.cpu(), encW, encb)
         rh = rhat.cpu()
@@ -80,6 +83,19 @@ def test_bee_message_kernel(ops, chan):
         for k, lab in enumerate(("022", "202", "112", "222", "212")):
             ref = torch.zeros(N, chan, 3, 3).index_add_(0, src, prods[lab]).reshape(N, chan, 9)
             _close(S2[:, :, k], ref.transpose(1, 2), atol_scale=4e-6)
+
+
+def test_node_products_emit_node_maxima(ops):
+    g = torch.Generator().manual_seed(3)
+    N, chan = 50, 128
+    t = [torch.randn(N, *([c] if c > 1 else []), chan, generator=g).cuda() for c in (1, 3, 9, 1, 3, 9)]
+    P0, P1, P2, nmax = ops.bee_node_products(*t, want_node_max=True)
+    assert nmax.shape == (N, 2)
+    want = torch.stack([P0.abs().amax(dim=(1, 2)), P1.abs().amax(dim=(1, 2, 3)), P2.abs().amax(dim=(1, 2, 3))]).amax(0)
+    assert torch.equal(nmax.amax(1), want)
+    # channel counts that a wave straddles: no maxima (the caller falls back to a pass over the rows)
+    t = [torch.randn(N, *([c] if c > 1 else []), 40, generator=g).cuda() for c in (1, 3, 9, 1, 3, 9)]
+    assert ops.bee_node_products(*t, want_node_max=True)[3] is None
 
 
 def _mlp_leaky_weights(m):
