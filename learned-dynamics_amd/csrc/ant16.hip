@@ -145,6 +145,10 @@ ant16_kernel(Terms terms, const float* __restrict__ x_0, const float* __restrict
     }
 }
 
+__global__ void __launch_bounds__(256) fill_zero_kernel(float* __restrict__ y, long n) {
+    for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (long)gridDim.x * blockDim.x) y[t] = 0.f;
+}
+
 }  // namespace
 }  // namespace mg
 
@@ -190,7 +194,13 @@ int mg_ant16_fwd(int rank_o, int n_terms, const int* labels, const float* const*
     const dim3 grid((unsigned)ceil_div(rows, BPT), (unsigned)ceil_div(dim_o, 128));
     MG_REQUIRE(ceil_div(rows, BPT) <= 0x7fffffffL, "mg_ant16_fwd: too many rows");
     if (terms.n == 0) {
-        if (!accumulate) MG_HIP(hipMemsetAsync(y, 0, (size_t)rows * dim_o * CO * sizeof(float), st));
+        if (!accumulate) {   // a kernel, not a memset node: callers may capture this launch into a graph
+            const long total = rows * dim_o * CO;
+            long blocks = ceil_div(total, 256);
+            if (blocks > 4096) blocks = 4096;
+            hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)blocks), dim3(256), 0, st, y, total);
+            return check_launch("mg_ant16_fwd");
+        }
         return MG_OK;
     }
 #define MG_ANT16_LAUNCH(R)                                                                                          \
