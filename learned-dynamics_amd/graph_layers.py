@@ -6,6 +6,10 @@ Differences that do not change results: the Graph also keeps the int32 index
 arrays and the CSR row_ptr the neighbour search produced, so gathers and
 segment sums run on them directly; rows are exact-size (the celllist_max /
 neighbours_max caps are only used to raise the reference's overflow errors).
+
+Gathers and segment sums are differentiable (each is the other's adjoint, and the
+adjoints are expressed with the same two autograd functions, so second derivatives
+as taken by torch.autograd.functional.jvp(create_graph=True) work too).
 """
 import torch
 
@@ -27,6 +31,20 @@ class Graph:
         self.nodes = nodes
         self._row_ptr = row_ptr
         self.cell_order = cell_order   # int32 atom ids in cell order, or None (radius graphs only)
+        self._by_src = None
+        self._by_dst = None
+
+    @property
+    def by_src(self):
+        if self._by_src is None:
+            self._by_src = _SortedIndex(self.src32, self.batch * self.nodes, row_ptr=self.row_ptr, is_sorted=True)
+        return self._by_src
+
+    @property
+    def by_dst(self):
+        if self._by_dst is None:
+            self._by_dst = _SortedIndex(self.dst32, self.batch * self.nodes)
+        return self._by_dst
 
     @property
     def row_ptr(self):
@@ -49,6 +67,67 @@ class Graph:
         return ans
 
 
+class _SortedIndex:
+    """An index along dim 0 together with what its adjoint needs: the permutation that sorts it
+    and the CSR row pointer of the sorted index.  For a sorted index the permutation is None."""
+
+    def __init__(self, index32, n_rows, row_ptr=None, is_sorted=False):
+        self.index = index32
+        self.n_rows = n_rows
+        self._row_ptr = row_ptr
+        self._perm = None
+        self.is_sorted = is_sorted
+
+    @property
+    def perm(self):
+        if self.is_sorted:
+            return None
+        if self._perm is None:
+            # stable sort by destination: index plumbing, done once per graph and only when a
+            # gradient through a gather-by-dst is asked for
+            self._perm = torch.sort(self.index.long(), stable=True).indices.to(torch.int32).contiguous()
+        return self._perm
+
+    @property
+    def row_ptr(self):
+        if self._row_ptr is None:
+            idx = self.index if self.is_sorted else ops.gather_rows(
+                self.index.to(torch.float32).reshape(-1, 1), self.perm).reshape(-1).to(torch.int32)
+            self._row_ptr = ops.segment_row_ptr(idx.contiguous(), self.n_rows)
+        return self._row_ptr
+
+
+class _Gather(torch.autograd.Function):
+    """x[index] along dim 0; adjoint: sum of the gradient rows that share an index
+    (edges_read / edges_read_dst of managan/graph_layers.py:37-52 rely on torch indexing for this)."""
+
+    @staticmethod
+    def forward(ctx, x, sidx):
+        ctx.sidx = sidx
+        return ops.gather_rows(x.contiguous(), sidx.index)
+
+    @staticmethod
+    def backward(ctx, dy):
+        return _ScatterSum.apply(dy, ctx.sidx), None
+
+
+class _ScatterSum(torch.autograd.Function):
+    """out[r] = sum of the rows e with index[e] = r; adjoint: a gather
+    (torch_scatter.segment_coo at managan/graph_layers.py:54-59 for a sorted index)."""
+
+    @staticmethod
+    def forward(ctx, x_edge, sidx):
+        ctx.sidx = sidx
+        x_edge = x_edge.contiguous()
+        if not sidx.is_sorted:
+            x_edge = ops.gather_rows(x_edge, sidx.perm)       # rows in index order
+        return ops.segment_sum_csr(x_edge, sidx.row_ptr, sidx.n_rows)
+
+    @staticmethod
+    def backward(ctx, dy):
+        return _Gather.apply(dy, ctx.sidx), None
+
+
 def _flat_nodes(graph, x_node):
     b, n, *rest = x_node.shape
     assert b == graph.batch and n == graph.nodes
@@ -58,24 +137,26 @@ def _flat_nodes(graph, x_node):
 def edges_read(graph: Graph, x_node: torch.Tensor):
     """x_node: (batch, nodes, ...) -> (x_src, x_dst), each (edges, ...)."""
     flat = _flat_nodes(graph, x_node)
-    return ops.gather_rows(flat, graph.src32), ops.gather_rows(flat, graph.dst32)
+    return _Gather.apply(flat, graph.by_src), _Gather.apply(flat, graph.by_dst)
 
 
 def edges_read_dst(graph: Graph, x_node: torch.Tensor):
     """x_node: (batch, nodes, ...) -> x_dst: (edges, ...)."""
-    return ops.gather_rows(_flat_nodes(graph, x_node), graph.dst32)
+    return _Gather.apply(_flat_nodes(graph, x_node), graph.by_dst)
 
 
 def edges_reduce_src(graph: Graph, x_edge: torch.Tensor):
     """Sum edge data onto the src node of each edge.  x_edge: (edges, ...)."""
-    ans = ops.segment_sum_csr(x_edge.contiguous(), graph.row_ptr, graph.batch * graph.nodes)
+    ans = _ScatterSum.apply(x_edge, graph.by_src)
     return ans.reshape(graph.batch, graph.nodes, *ans.shape[1:])
 
 
 def segment_sum(x_edge, index, dim_size):
     """segment_coo(x_edge, index, dim_size=dim_size, reduce='sum') for a sorted index."""
-    row_ptr = ops.segment_row_ptr(index.contiguous(), dim_size)
-    return ops.segment_sum_csr(x_edge.contiguous(), row_ptr, dim_size)
+    index = index.contiguous()
+    sidx = _SortedIndex(index if index.dtype == torch.int32 else index.to(torch.int32), dim_size,
+                        row_ptr=ops.segment_row_ptr(index, dim_size), is_sorted=True)
+    return _ScatterSum.apply(x_edge, sidx)
 
 
 def boxwrap(box: torch.Tensor, delta_pos: torch.Tensor):

@@ -91,3 +91,50 @@ def test_torch_scatter_shim(pkg):
     out = segment_coo(x, idx, dim_size=50)
     ref = torch.zeros(50, 16, 3).index_add_(0, idx.cpu(), x.cpu())
     torch.testing.assert_close(out.cpu(), ref, rtol=1e-5, atol=1e-5)
+
+
+def test_gather_and_segment_sum_are_differentiable(pkg):
+    """edges_read / edges_read_dst / edges_reduce_src against torch indexing and index_add_ under
+    autograd, including a second derivative (the meanflow loss differentiates a jvp:
+    archs/meanflow_painn8.py:274-282)."""
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    g = torch.Generator().manual_seed(11)
+    B, N, E, C = 2, 40, 700, 6
+    src = torch.sort(torch.randint(0, B * N, (E,), generator=g)).values
+    dst = torch.randint(0, B * N, (E,), generator=g)
+    graph = gl.Graph(src.cuda(), dst.cuda(), None, B, N)
+    x = torch.randn(B, N, C, 3, generator=g)
+    w_e = torch.randn(E, C, 3, generator=g)
+
+    def model(x_node, gather_src_dst, reduce):
+        xs, xd = gather_src_dst(x_node)
+        m = xs * xd * w_e.to(x_node.device) + xd ** 3          # nonlinear in the gathered rows
+        return (reduce(m) ** 2).sum()
+
+    def ref_gather(x_node):
+        flat = x_node.reshape(B * N, C, 3)
+        return flat[src], flat[dst]
+
+    def ref_reduce(m):
+        return torch.zeros(B * N, C, 3, dtype=m.dtype).index_add_(0, src, m).reshape(B, N, C, 3)
+
+    xr = x.clone().requires_grad_(True)
+    loss_r = model(xr, ref_gather, ref_reduce)
+    (gr,) = torch.autograd.grad(loss_r, xr, create_graph=True)
+    (ggr,) = torch.autograd.grad((gr ** 2).sum(), xr)
+
+    xg = x.cuda().requires_grad_(True)
+    loss_g = model(xg, lambda t: gl.edges_read(graph, t), lambda m: gl.edges_reduce_src(graph, m))
+    (gg,) = torch.autograd.grad(loss_g, xg, create_graph=True)
+    (ggg,) = torch.autograd.grad((gg ** 2).sum(), xg)
+    torch.testing.assert_close(loss_g.cpu(), loss_r, rtol=1e-5, atol=1e-5)
+    torch.testing.assert_close(gg.detach().cpu(), gr.detach(), rtol=1e-4, atol=1e-4 * float(gr.detach().abs().max()))
+    torch.testing.assert_close(ggg.cpu(), ggr, rtol=1e-4, atol=1e-4 * float(ggr.abs().max()))
+    # the torch_scatter shim carries the same autograd
+    pkg.install_shims()
+    import torch_scatter
+    e = torch.randn(E, 5, generator=g).cuda().requires_grad_(True)
+    out = torch_scatter.segment_coo(e, src.cuda(), dim_size=B * N, reduce="sum")
+    out.square().sum().backward()
+    ref_e = torch.zeros(B * N, 5).index_add_(0, src, e.detach().cpu())
+    torch.testing.assert_close(e.grad.cpu(), 2 * ref_e[src], rtol=1e-5, atol=1e-5)
