@@ -334,10 +334,11 @@ int mg_bee_edge_geometry(const float* r_ij /* (E,3) */, long n_edges, float r0,
 int mg_bee_message(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
                    const float* rhat, const float* enc, const float* La, const float* Lv, const float* Ld,
                    int chan, const float* enc_W /* (chan,8) */, const float* enc_b /* (chan) */,
-                   float* P0, float* S1, float* S2, float* node_max, mg_stream_t stream);
+                   float* P0, float* S1, float* S2, float* node_max, float* edge_max, mg_stream_t stream);
 /* node_max (above and below; may be NULL): (N, ceil(chan/64)) partial maxima of |S1|, |S2| (of |P0|,
  * |P1|, |P2| below) per node, which mg_tensor_linear_f16x2 accepts as row bounds of those tensors
- * (x_rows_per_bound = 3 or 9); no counterpart in the reference. */
+ * (x_rows_per_bound = 3 or 9); edge_max (may be NULL): (E, ceil(chan/64)) partial maxima of the rows
+ * of P0; no counterpart in the reference. */
 
 /* The 13 products of SelfTensProds.forward (archs/diffuser_atoms15.py:86-88; formulas of
  * managan/codegen_tensor_products.py:235-249) on node rows in component-major layout:

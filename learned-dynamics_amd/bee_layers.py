@@ -214,12 +214,12 @@ class Messages(nn.Module):
         Lv = ops.tensor_linear_fwd(1, self.L1.W, x_v.reshape(rows, -1, 3).contiguous(), y_layout=C)
         Ld = ops.tensor_linear_fwd(2, self.L2.W, x_d.reshape(rows, -1, 3, 3).contiguous(), y_layout=C)
         enc, rhat = ops.bee_edge_geometry(r_ij.contiguous(), self.r0)
-        P0, S1, S2, nmax = ops.bee_message(graph.row_ptr, graph.dst32, rhat, enc, La, Lv, Ld, self.lin_enc.weight,
+        P0, S1, S2, nmax, emax = ops.bee_message(graph.row_ptr, graph.dst32, rhat, enc, La, Lv, Ld, self.lin_enc.weight,
                                            self.lin_enc.bias, node_order=node_order, want_node_max=True)
         E, chan = P0.shape[0], P0.shape[2]
         # scalar channel: per-edge linear + MLP, then the edge sum
         P0 = P0.reshape(E, 3 * chan)
-        bound = ops.row_absmax(P0) if ops.get_linear_mode() == ops.LINEAR_F16X2 else None
+        bound = emax if ops.get_linear_mode() == ops.LINEAR_F16X2 else None     # row maxima of P0 from the edge kernel
         psi_a, bound = _linear(P0, self._cat_Y(LABELS_0), None, ops.ACT_NONE, bound)
         psi_a = self.mlp_a(psi_a, plus_identity=True, bound=bound)
         B_a = ops.segment_sum_csr(psi_a, graph.row_ptr, rows).mul_(0.1)

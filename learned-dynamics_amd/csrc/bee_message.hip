@@ -96,7 +96,8 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
                    long n_nodes, const float* __restrict__ rhat, const float* __restrict__ enc,
                    const T* __restrict__ La, const T* __restrict__ Lv, const T* __restrict__ Ld, int chan,
                    const float* __restrict__ enc_W, const float* __restrict__ enc_b, T* __restrict__ P0,
-                   T* __restrict__ S1, T* __restrict__ S2, float* __restrict__ node_max) {
+                   T* __restrict__ S1, T* __restrict__ S2, float* __restrict__ node_max,
+                   float* __restrict__ edge_max) {
     const int lane = threadIdx.x & (kWave - 1);
     const int chunks = (chan + kWave - 1) / kWave;
     const long items = n_nodes * chunks;
@@ -163,6 +164,12 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
                 p[chan] = (T)pd1;           // 110
                 p[2 * chan] = (T)(phi * quad);  // 220
             }
+            if (edge_max) {
+                // largest |P0| entry of this (edge, 64-channel chunk): a row bound for the per-edge GEMM
+                float mx = fmaxf(fmaxf(fabsf(pl0), fabsf(pd1)), fabsf(phi * quad));
+                for (int d = 1; d < kWave; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+                if (lane == 0) edge_max[e * chunks + (item - k_node * chunks)] = mx;
+            }
             // vector sums, label order 011, 101, 121, 211, 111
 #pragma unroll
             for (int x = 0; x < 3; x++) {
@@ -218,7 +225,7 @@ template <typename T>
 static int launch_bee_message(const char* what, const int* row_ptr, const int* dst, const int* node_order, int n_nodes,
                               long n_edges, const float* rhat, const float* enc, const T* La, const T* Lv, const T* Ld,
                               int chan, const float* enc_W, const float* enc_b, T* P0, T* S1, T* S2,
-                              float* node_max, mg_stream_t stream) {
+                              float* node_max, float* edge_max, mg_stream_t stream) {
     MG_REQUIRE(n_nodes >= 0 && n_edges >= 0 && chan >= 0, "%s: negative size", what);
     if (n_nodes == 0 || chan == 0) return MG_OK;
     MG_REQUIRE(row_ptr && La && Lv && Ld && enc_W && enc_b && S1 && S2, "%s: null pointer", what);
@@ -228,7 +235,7 @@ static int launch_bee_message(const char* what, const int* row_ptr, const int* d
     if (blocks > 256L * 16) blocks = 256L * 16;
     blocks = ceil_div(blocks, 8) * 8;
     hipLaunchKernelGGL(bee_message_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, row_ptr, dst,
-                       node_order, (long)n_nodes, rhat, enc, La, Lv, Ld, chan, enc_W, enc_b, P0, S1, S2, node_max);
+                       node_order, (long)n_nodes, rhat, enc, La, Lv, Ld, chan, enc_W, enc_b, P0, S1, S2, node_max, edge_max);
     return check_launch(what);
 }
 
@@ -249,9 +256,9 @@ int mg_bee_edge_geometry(const float* r_ij, long n_edges, float r0, float* enc, 
 int mg_bee_message(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
                    const float* rhat, const float* enc, const float* La, const float* Lv, const float* Ld, int chan,
                    const float* enc_W, const float* enc_b, float* P0, float* S1, float* S2, float* node_max,
-                   mg_stream_t stream) {
+                   float* edge_max, mg_stream_t stream) {
     return launch_bee_message<float>("mg_bee_message", row_ptr, dst, node_order, n_nodes, n_edges, rhat, enc, La, Lv,
-                                     Ld, chan, enc_W, enc_b, P0, S1, S2, node_max, stream);
+                                     Ld, chan, enc_W, enc_b, P0, S1, S2, node_max, edge_max, stream);
 }
 
 int mg_bee_message_bf16(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
@@ -260,7 +267,7 @@ int mg_bee_message_bf16(const int* row_ptr, const int* dst, const int* node_orde
     return launch_bee_message<__bf16>("mg_bee_message_bf16", row_ptr, dst, node_order, n_nodes, n_edges, rhat, enc,
                                       static_cast<const __bf16*>(La), static_cast<const __bf16*>(Lv),
                                       static_cast<const __bf16*>(Ld), chan, enc_W, enc_b, static_cast<__bf16*>(P0),
-                                      static_cast<__bf16*>(S1), static_cast<__bf16*>(S2), nullptr, stream);
+                                      static_cast<__bf16*>(S1), static_cast<__bf16*>(S2), nullptr, nullptr, stream);
 }
 
 }  // extern "C"

@@ -603,6 +603,8 @@ def linear_out_bound(W, bias, in_bound):
             per_input.clear()
         per_input[id(in_bound)] = (weakref.ref(in_bound), out)
         return out
+    if in_bound.dim() == 2 and in_bound.size(1) > 1:           # partial maxima per row: the largest counts
+        in_bound = in_bound.amax(dim=1, keepdim=True)
     return torch.addcmul(bmax, in_bound.reshape(-1, 1), l1)
 
 
@@ -952,7 +954,8 @@ def bee_edge_geometry(r_ij, r0):
 def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=None, want_node_max=False):
     """Fused products + edge sums of the rank-0/1/2 message (see mg_bee_message).
     La (N,chan), Lv (N,3,chan), Ld (N,9,chan) -> P0 (E,3,chan), S1 (N,3,5,chan), S2 (N,9,5,chan)
-    (+ node_max (N, ceil(chan/64)): partial maxima of |S1|, |S2| per node, with want_node_max)."""
+    (+ node_max (N, ceil(chan/64)) and edge_max (E, ceil(chan/64)): partial maxima of |S1|, |S2| per node
+    and of |P0| per edge, with want_node_max)."""
     _check_input(row_ptr, "row_ptr", torch.int32)
     _check_input(dst, "dst", torch.int32)
     for t, nm in ((rhat, "rhat"), (enc, "enc"), (La, "La"), (Lv, "Lv"), (Ld, "Ld"), (enc_W, "enc_W"),
@@ -978,10 +981,11 @@ def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=No
         S1 = torch.empty(N, 3, 5, chan, dtype=torch.float32, device=dev)
         S2 = torch.empty(N, 9, 5, chan, dtype=torch.float32, device=dev)
         node_max = torch.empty(N, (chan + 63) // 64, dtype=torch.float32, device=dev) if want_node_max else None
+        edge_max = torch.empty(E, (chan + 63) // 64, dtype=torch.float32, device=dev) if want_node_max else None
         L.check(_lib.mg_bee_message(_p(row_ptr), _p(dst), _p(node_order), N, E, _p(rhat), _p(enc), _p(La), _p(Lv),
                                     _p(Ld), chan, _p(enc_W), _p(enc_b), _p(P0), _p(S1), _p(S2), _p(node_max),
-                                    _stream()))
-    return (P0, S1, S2, node_max) if want_node_max else (P0, S1, S2)
+                                    _p(edge_max), _stream()))
+    return (P0, S1, S2, node_max, edge_max) if want_node_max else (P0, S1, S2)
 
 
 # ------------------------------------------------- norms, squash, update glue

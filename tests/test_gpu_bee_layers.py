@@ -64,11 +64,12 @@ def test_bee_message_kernel(ops, chan):
     Ld_cm = Ld.reshape(N, chan, 9).transpose(1, 2).contiguous()
     order = torch.randperm(N).int().cuda()
     for node_order in (None, order):
-        P0, S1, S2, nmax = ops.bee_message(row_ptr, dst.int().cuda(), rhat, enc, La.cuda(), Lv_cm.cuda(), Ld_cm.cuda(),
+        P0, S1, S2, nmax, emax = ops.bee_message(row_ptr, dst.int().cuda(), rhat, enc, La.cuda(), Lv_cm.cuda(), Ld_cm.cuda(),
                                            encW.cuda(), encb.cuda(), node_order=node_order, want_node_max=True)
         # the emitted per-node maxima are exactly the maxima of what was written
         assert nmax.shape == (N, (chan + 63) // 64)
         assert torch.equal(nmax.amax(1), torch.maximum(S1.abs().amax(dim=(1, 2, 3)), S2.abs().amax(dim=(1, 2, 3))))
+        assert emax.shape == (E, (chan + 63) // 64) and torch.equal(emax.amax(1), P0.abs().amax(dim=(1, 2)))
         # oracle on the device's own enc / rhat (they are checked separately)
         phi_a = torch.nn.functional.linear(enc.cpu(), encW, encb)
         rh = rhat.cpu()
