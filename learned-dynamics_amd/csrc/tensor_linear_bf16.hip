@@ -162,6 +162,60 @@ linear_rows_bf16_kernel(const __bf16* __restrict__ Wp, long plane_elems, int w_r
 
     // lane (m, g) holds row my_row and, for accumulator quad qq of block ni, the four channels
     // n0 + 32 ni + 8 qq + 4 g .. + 4
+    //
+    // bf16 output, full tile: the rows are first transposed through the wave's own slice of the
+    // (now idle) W buffers, so that the stores to HBM are 16 bytes per lane and whole 64..256-byte
+    // row segments per instruction instead of 8-byte pieces scattered over 32 rows (the output is
+    // half of this kernel's traffic).  A wave touches only its own slice and its LDS operations
+    // execute in order, so no barrier is needed.
+    constexpr int kRegion = 2 * kBufW / WAVES;                              // bytes of LDS per wave
+    constexpr int kColsFit = (kRegion - 512) / 64;                          // 32 rows x (2 cols + 16) bytes
+    constexpr int kPassCols = kColsFit >= 128 ? 128 : (kColsFit >= 64 ? 64 : (kColsFit >= 32 ? 32 : 0));
+    if constexpr (std::is_same<YT, __bf16>::value && kPassCols > 0) {
+        if (out_T == 1 && n0 + TN <= O && (O & 7) == 0 && !accumulate) {
+            constexpr int kCols = kPassCols < TN ? kPassCols : TN;          // columns per pass
+            constexpr int kRowBytes = 2 * kCols + 16;
+            constexpr int kPieces = 32 * kCols / 8;                         // 16-byte pieces per pass
+            unsigned char* slice = lds + wave * kRegion;
+            const float* brow = bias ? bias + n0 + 4 * g : nullptr;
+            auto epilogue = [&](auto act_tag) {
+                constexpr int kAct = decltype(act_tag)::value;
+#pragma unroll
+                for (int pass = 0; pass < TN / kCols; pass++) {
+#pragma unroll
+                    for (int nl = 0; nl < kCols / 32; nl++) {
+                        const int ni = pass * (kCols / 32) + nl;
+#pragma unroll
+                        for (int qq = 0; qq < 4; qq++) {
+                            floatx4 v = {acc[ni][4 * qq], acc[ni][4 * qq + 1], acc[ni][4 * qq + 2], acc[ni][4 * qq + 3]};
+                            if (brow) v += load4(brow + 32 * ni + 8 * qq);
+#pragma unroll
+                            for (int i = 0; i < 4; i++) v[i] = activate_c<kAct>(v[i]);
+                            store4(reinterpret_cast<__bf16*>(slice + m * kRowBytes) + 32 * nl + 8 * qq + 4 * g, v);
+                        }
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                    for (int it = 0; it < (kPieces + 63) / 64; it++) {
+                        const int piece = it * 64 + lane;
+                        const int row = piece / (kCols / 8), c8 = piece % (kCols / 8);
+                        const long r = r0 + wave * 32 + row;
+                        if (piece < kPieces && r < R) {
+                            const bf16x8 t = *reinterpret_cast<const bf16x8*>(slice + row * kRowBytes + c8 * 16);
+                            *reinterpret_cast<bf16x8*>(Y + r * O + n0 + pass * kCols + c8 * 8) = t;
+                        }
+                    }
+                    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                    __builtin_amdgcn_wave_barrier();
+                }
+            };
+            if (act == 1) epilogue(std::integral_constant<int, 1>{});
+            else if (act == 2) epilogue(std::integral_constant<int, 2>{});
+            else epilogue(std::integral_constant<int, 0>{});
+            return;
+        }
+    }
     if (my_row >= R) return;
     if (out_T == 1 && n0 + TN <= O && (O & 3) == 0) {
         YT* yrow = Y + my_row * O + n0 + 4 * g;
