@@ -90,7 +90,8 @@ __device__ __forceinline__ long uniform(long v) {
 }
 
 // T: storage type of the node features and of the outputs (float, or __bf16 with fp32 arithmetic)
-template <typename T>
+// PIPE: keep one edge of operands in flight ahead of the one being consumed (pays on long rows)
+template <typename T, bool PIPE>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4)))
 bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst, const int* __restrict__ order,
                    long n_nodes, const float* __restrict__ rhat, const float* __restrict__ enc,
@@ -128,21 +129,53 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
 #pragma unroll
         for (int k = 0; k < 45; k++) s2[k] = 0.f;
 
+        // Software pipeline: the 13 gathered rows, the encoding and the direction of edge e + 1 are
+        // requested before edge e is consumed (the gathers are L2 / fabric latency, and a wave has
+        // nothing else to do while it waits), and dst of edge e + 2 one step earlier still.  The
+        // look-ahead indices are clamped to the row, so no load is predicated.
+        struct EdgeOps {
+            T l0, l1[3], l2[9];
+            float en[8], rh[3];
+        };
+        auto fetch = [&](EdgeOps& o, long e, long j) {
+            o.l0 = La[j * chan + cc];
+#pragma unroll
+            for (int t = 0; t < 3; t++) o.l1[t] = Lv[(j * 3 + t) * chan + cc];
+#pragma unroll
+            for (int k = 0; k < 9; k++) o.l2[k] = Ld[(j * 9 + k) * chan + cc];
+#pragma unroll
+            for (int m = 0; m < 8; m++) o.en[m] = enc[8 * e + m];
+#pragma unroll
+            for (int t = 0; t < 3; t++) o.rh[t] = rhat[3 * e + t];
+        };
+        const long last = hi - 1;
+        EdgeOps nxt;
+        long j_next = 0;
+        if (PIPE && lo < hi) {
+            fetch(nxt, lo, dst[lo]);
+            j_next = dst[lo + 1 < hi ? lo + 1 : last];
+        }
         for (long e = lo; e < hi; e++) {
-            const long j = dst[e];
+            EdgeOps cur;
+            if constexpr (PIPE) {
+                cur = nxt;
+                const long e1 = e + 1 < hi ? e + 1 : last;
+                fetch(nxt, e1, j_next);
+                j_next = dst[e + 2 < hi ? e + 2 : last];
+            } else {
+                fetch(cur, e, dst[e]);
+            }
             float en[8], rh[3];
 #pragma unroll
-            for (int m = 0; m < 8; m++) en[m] = enc[8 * e + m];
+            for (int m = 0; m < 8; m++) en[m] = cur.en[m];
 #pragma unroll
-            for (int t = 0; t < 3; t++) rh[t] = rhat[3 * e + t];
-            // gathers: 13 unit-stride rows
-            const float l0 = (float)La[j * chan + cc];
+            for (int t = 0; t < 3; t++) rh[t] = cur.rh[t];
+            const float l0 = (float)cur.l0;
             float l1[3], l2[9];
 #pragma unroll
-            for (int t = 0; t < 3; t++) l1[t] = (float)Lv[(j * 3 + t) * chan + cc];
+            for (int t = 0; t < 3; t++) l1[t] = (float)cur.l1[t];
 #pragma unroll
-            for (int k = 0; k < 9; k++) l2[k] = (float)Ld[(j * 9 + k) * chan + cc];
-
+            for (int k = 0; k < 9; k++) l2[k] = (float)cur.l2[k];
             float phi = bias;
 #pragma unroll
             for (int m = 0; m < 8; m++) phi += w[m] * en[m];
@@ -234,8 +267,15 @@ static int launch_bee_message(const char* what, const int* row_ptr, const int* d
     long blocks = ceil_div(items, 4);
     if (blocks > 256L * 16) blocks = 256L * 16;
     blocks = ceil_div(blocks, 8) * 8;
-    hipLaunchKernelGGL(bee_message_kernel<T>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, row_ptr, dst,
-                       node_order, (long)n_nodes, rhat, enc, La, Lv, Ld, chan, enc_W, enc_b, P0, S1, S2, node_max, edge_max);
+    // rows of a few edges do not repay the pipeline's start-up (one extra set of loads per row)
+    if (n_edges >= 32L * n_nodes)
+        hipLaunchKernelGGL((bee_message_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                           row_ptr, dst, node_order, (long)n_nodes, rhat, enc, La, Lv, Ld, chan, enc_W, enc_b, P0, S1, S2,
+                           node_max, edge_max);
+    else
+        hipLaunchKernelGGL((bee_message_kernel<T, false>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
+                           row_ptr, dst, node_order, (long)n_nodes, rhat, enc, La, Lv, Ld, chan, enc_W, enc_b, P0, S1, S2,
+                           node_max, edge_max);
     return check_launch(what);
 }
 

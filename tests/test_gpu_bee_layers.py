@@ -48,10 +48,11 @@ def test_linear_layouts(ops, lin_layout):
     torch.testing.assert_close(y.cpu(), ref_cm, rtol=1e-5, atol=1e-5)
 
 
-@pytest.mark.parametrize("chan", [64, 8, 100])
-def test_bee_message_kernel(ops, chan):
+@pytest.mark.parametrize("chan,E", [(64, 3000), (8, 3000), (100, 3000), (64, 9000), (40, 7000)])
+def test_bee_message_kernel(ops, chan, E):
+    """E / N below and above 32: the kernel pipelines its gathers only on long rows."""
     torch.manual_seed(chan)
-    N, E = 200, 3000
+    N = 200
     src = torch.sort(torch.randint(0, N, (E,))).values
     src[src == 5] = 6
     dst = torch.randint(0, N, (E,))
