@@ -8,7 +8,9 @@
 // from a few LDS reads right before the fp32 matrix instruction (v_mfma_f32_32x32x2_f32: exact
 // fp32 products), and P is read in place.  A workgroup owns the rows of one tile (32, 10 or 3 rows
 // for output rank 0, 1, 2: 32 = rows x components, rounded down to whole rows) and up to four
-// 32-channel column blocks (one per wave); operands of the tile are staged in LDS per product type.
+// 32-channel column blocks; its four waves split the contraction over the left channels, so an
+// A value is built once and meets every column block; operands of the tile are staged in LDS per
+// product type and the partial accumulators are summed through LDS.
 // Every product component is a short signed dot product  sum_t l[lb + t ls] * r[rb + t rs]  whose
 // offsets depend only on the lane's output component, so one generic inner loop serves all 13 types.
 #include "common.hpp"
@@ -63,6 +65,8 @@ __device__ __forceinline__ Dot dot_of(int label, int c) {
     }
 }
 
+constexpr int kMaxNT = 4;   // 32-channel column blocks per workgroup (dim_o <= 128 per grid row)
+
 template <int RANK_O>
 __global__ void __launch_bounds__(256)
 ant16_kernel(Terms terms, const float* __restrict__ x_0, const float* __restrict__ x_1, const float* __restrict__ x_2,
@@ -74,17 +78,20 @@ ant16_kernel(Terms terms, const float* __restrict__ x_0, const float* __restrict
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int m = lane & 31, kk = lane >> 5;
     const long b0 = (long)blockIdx.x * BPT;
-    const int o0 = (blockIdx.y * 4 + wave) * 32;
-    const bool wave_active = o0 < dim_o;
+    const int o_base = blockIdx.y * (32 * kMaxNT);
+    const int nt = (dim_o - o_base + 31) / 32 < kMaxNT ? (dim_o - o_base + 31) / 32 : kMaxNT;   // column blocks here
     // this lane's A row: (row b0 + bl, component co)
     const int bl = m / CO, co = m - bl * CO;
     const bool row_ok = bl < BPT && b0 + bl < rows;
-    int o_ld = o0 + m;                                   // this lane's B column (clamped for loads)
-    if (o_ld >= dim_o) o_ld = dim_o - 1;
 
-    floatx16 acc;
+    // The four waves share the tile's rows and all its column blocks and split the contraction:
+    // wave w takes the left channels i = w, w + 4, ...; an A value is built once and meets every
+    // column block; the partial accumulators are summed through LDS at the end.
+    floatx16 acc[kMaxNT];
 #pragma unroll
-    for (int q = 0; q < 16; q++) acc[q] = 0.f;
+    for (int t = 0; t < kMaxNT; t++)
+#pragma unroll
+        for (int q = 0; q < 16; q++) acc[t][q] = 0.f;
 
     for (int ti = 0; ti < terms.n; ti++) {
         const int label = terms.t[ti].label;
@@ -105,42 +112,76 @@ ant16_kernel(Terms terms, const float* __restrict__ x_0, const float* __restrict
             xs[t] = b0 + b < rows ? xr[(b0 + b) * xrow + (t - b * xrow)] : 0.f;
         }
         __syncthreads();
-        if (!wave_active) continue;
         const Dot d = dot_of(label, co);
         const float* lrow_p = ls + (row_ok ? bl : 0) * lrow + d.lb;
         const float* xrow_p = xs + (row_ok ? bl : 0) * xrow + d.rb;
-        const float* Pl = terms.t[ti].P + (long)o_ld * dim_l * dim_r;
-        for (int i = 0; i < dim_l; i++) {
+        // this lane's B columns (clamped for loads; columns past dim_o are never written)
+        const float* Pn[kMaxNT];
+#pragma unroll
+        for (int t = 0; t < kMaxNT; t++) {
+            int o = o_base + t * 32 + m;
+            if (o >= dim_o) o = dim_o - 1;
+            Pn[t] = terms.t[ti].P + (long)o * dim_l * dim_r;
+        }
+        for (int i = wave; i < dim_l; i += 4) {
             float lv[9];
 #pragma unroll
             for (int t = 0; t < 9; t++) lv[t] = t < d.nt ? lrow_p[i * CL + t * d.ls] : 0.f;
             if (d.cross) lv[1] = -lv[1];
-            const float* Pi = Pl + (long)i * dim_r;
-            for (int j0 = 0; j0 < dim_r; j0 += 2) {
-                const int j = j0 + kk;
-                const bool j_ok = j < dim_r;
-                const int jc = j_ok ? j : dim_r - 1;
-                const float* rp = xrow_p + jc * CR;
-                float a = 0.f;
+            // four K-steps per trip: all B values are requested before the first is consumed, so
+            // the load latency is paid once per trip instead of once per matrix instruction
+            for (int j0 = 0; j0 < dim_r; j0 += 8) {
+                float bval[4][kMaxNT], aval[4];
 #pragma unroll
-                for (int t = 0; t < 9; t++)
-                    if (t < d.nt) a = fmaf(lv[t], rp[t * d.rs], a);
-                a = (row_ok && j_ok) ? a : 0.f;
-                const float bval = j_ok ? Pi[jc] : 0.f;
-                acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a, bval, acc, 0, 0, 0);
+                for (int u = 0; u < 4; u++) {
+                    const int j = j0 + 2 * u + kk;
+                    const bool j_ok = j < dim_r;
+                    const int jc = j_ok ? j : dim_r - 1;
+                    const long poff = (long)i * dim_r + jc;
+#pragma unroll
+                    for (int t = 0; t < kMaxNT; t++) bval[u][t] = (t < nt && j_ok) ? Pn[t][poff] : 0.f;
+                    const float* rp = xrow_p + jc * CR;
+                    float a = 0.f;
+#pragma unroll
+                    for (int t = 0; t < 9; t++)
+                        if (t < d.nt) a = fmaf(lv[t], rp[t * d.rs], a);
+                    aval[u] = (row_ok && j_ok) ? a : 0.f;
+                }
+#pragma unroll
+                for (int u = 0; u < 4; u++)
+#pragma unroll
+                    for (int t = 0; t < kMaxNT; t++)
+                        if (t < nt) acc[t] = __builtin_amdgcn_mfma_f32_32x32x2f32(aval[u], bval[u][t], acc[t], 0, 0, 0);
             }
         }
     }
-    if (!wave_active) return;
-    const int o = o0 + m;
-    if (o >= dim_o) return;
+    // sum the four partial tiles: waves 1..3 park theirs in LDS (64 floats per (block, register): no conflicts)
+    __syncthreads();
+    float* red = smem;                                   // [3][kMaxNT][16][64]
+    if (wave > 0) {
 #pragma unroll
-    for (int q = 0; q < 16; q++) {
-        const int mr = 8 * (q / 4) + 4 * kk + (q % 4);     // accumulator row -> (row, component)
-        const int b = mr / CO, c = mr - b * CO;
-        if (b < BPT && b0 + b < rows) {
-            float* p = y + ((b0 + b) * dim_o + o) * CO + c;
-            *p = accumulate ? *p + acc[q] : acc[q];
+        for (int t = 0; t < kMaxNT; t++)
+            if (t < nt)
+#pragma unroll
+                for (int q = 0; q < 16; q++) red[(((wave - 1) * kMaxNT + t) * 16 + q) * 64 + lane] = acc[t][q];
+    }
+    __syncthreads();
+    if (wave > 0) return;
+#pragma unroll
+    for (int t = 0; t < kMaxNT; t++) {
+        if (t >= nt) break;
+        const int o = o_base + t * 32 + m;
+#pragma unroll
+        for (int q = 0; q < 16; q++) {
+            float v = acc[t][q];
+#pragma unroll
+            for (int w = 0; w < 3; w++) v += red[((w * kMaxNT + t) * 16 + q) * 64 + lane];
+            const int mr = 8 * (q / 4) + 4 * kk + (q % 4);     // accumulator row -> (row, component)
+            const int b = mr / CO, c = mr - b * CO;
+            if (o < dim_o && b < BPT && b0 + b < rows) {
+                float* p = y + ((b0 + b) * dim_o + o) * CO + c;
+                *p = accumulate ? *p + v : v;
+            }
         }
     }
 }
@@ -187,6 +228,7 @@ int mg_ant16_fwd(int rank_o, int n_terms, const int* labels, const float* const*
         const size_t need = (size_t)BPT * ((size_t)dim_l * CL + (size_t)dim_r * CR);
         if (need > lds_floats) lds_floats = need;
     }
+    if (lds_floats < 3 * kMaxNT * 16 * 64) lds_floats = 3 * kMaxNT * 16 * 64;   // the final reduction reuses the tiles' space
     const size_t lds_bytes = lds_floats * sizeof(float);
     MG_REQUIRE(lds_bytes <= 160 * 1024, "mg_ant16_fwd: a tile of operands needs %zu bytes of LDS (limit 163840): "
                "channel counts too wide", lds_bytes);
