@@ -34,31 +34,16 @@
 // v_mfma_f32_32x32x16_f16 layout: A[m][k]: lane = m + 32*(k/8), 8 consecutive k per lane;
 // B[k][n] likewise; D[m][n]: n = lane%32, m = 8*(q/4) + 4*(lane/32) + q%4 for register q.
 #include "common.hpp"
+#include "f16x2.hpp"
 #include <type_traits>
 
 namespace mg {
 namespace {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-typedef _Float16 halfx8 __attribute__((ext_vector_type(8)));
-typedef _Float16 halfx4 __attribute__((ext_vector_type(4)));
-
-
 __device__ __forceinline__ float activate(float v, int act) {
     if (act == 1) return v * __frcp_rn(1.0f + __expf(-v));
     if (act == 2) return v > 0.f ? v : 0.1f * v;
     return v;
-}
-
-// power of two s with amax * s in [2^14, 2^15); *inv = 1/s.  amax >= 0; zero, tiny, inf and nan give
-// a finite in-range scale (the products then follow fp16/fp32 arithmetic on their own)
-__device__ __forceinline__ float pow2_scale(float amax, float* inv) {
-    int e = (int)(__float_as_uint(amax) >> 23) & 0xff;
-    int se = 268 - e;                   // 127 + 14 - (e - 127)
-    if (e == 255) se = 127;
-    se = se < 1 ? 1 : (se > 253 ? 253 : se);
-    *inv = __uint_as_float((unsigned)(254 - se) << 23);
-    return __uint_as_float((unsigned)se << 23);
 }
 
 template <int ACT>
@@ -67,22 +52,6 @@ __device__ __forceinline__ float activate_c(float v) {
     if constexpr (ACT == 1) return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
     if constexpr (ACT == 2) return v > 0.f ? v : 0.1f * v;
     return v;
-}
-
-struct HalfSplit4 {
-    halfx4 hi, lo;
-};
-
-__device__ __forceinline__ HalfSplit4 split(float4 v, float s) {
-    HalfSplit4 r;
-    const float in[4] = {v.x * s, v.y * s, v.z * s, v.w * s};
-#pragma unroll
-    for (int k = 0; k < 4; k++) {
-        const _Float16 h = (_Float16)in[k];
-        r.hi[k] = h;
-        r.lo[k] = (_Float16)(in[k] - (float)h);
-    }
-    return r;
 }
 
 // one wave per output row: row maximum -> scale -> hi / lo planes (O_pad rows, zero filled) + 1/scale per row
@@ -130,8 +99,6 @@ __global__ void __launch_bounds__(256) row_absmax_kernel(const float* __restrict
     }
 }
 
-constexpr int kCK = 32;                     // k per chunk (two MFMA steps)
-constexpr int kRowW = 80;                   // bytes per LDS row of one W plane (64 + 16 pad)
 
 template <int WAVES, int NI>
 __global__ void __launch_bounds__(64 * WAVES)
