@@ -280,6 +280,24 @@ int mg_painn_message(const int* row_ptr /* n_nodes+1 */, const int* dst /* E */,
                      int n, float epsilon, const float* res_a, const float* res_v,
                      float* out_a /* (n_nodes,n) */, float* out_v /* (n_nodes,n,3) */, mg_stream_t stream);
 
+/* mg_painn_message with the LAST layer of the radial MLP folded in (archs/meanflow_painn8.py:38-51 at :92,
+ * then :93-100): filt[e] = bias3 + W3 h[e] is produced on the matrix cores (split-fp16 arithmetic, as
+ * mg_tensor_linear_f16x2) and consumed in the same kernel, so the (E,4n) filter is never stored.
+ *   h (E,hidden): the MLP's second layer output (after its SiLU); h_rowmax: upper bounds of max_k |h[e,k]| as for
+ *   mg_tensor_linear_f16x2 (h_rowmax_parts values per row, row stride h_rowmax_stride floats, 0 = one shared row).
+ *   packed_W3: mg_linear_f16x2_pack_weight of W3 with its 4n rows PERMUTED to (c / 64, k, c % 64) for filter
+ *   column k n + c (k = 0..3), i.e. packed row 256 (c / 64) + 64 k + c % 64; bias3 (4n) in the same order.
+ *   src (E): the receiving node of every edge (sorted ascending; row_ptr is its CSR form).
+ *   workspace: mg_painn_filter_message_workspace_bytes(n_edges, n) bytes, 16-byte aligned (partial sums).
+ * n % 64 == 0, hidden % 32 == 0 and >= 64.  Sums run in edge order within blocks of 32 edges and then in
+ * block order: deterministic, and equal to mg_painn_message up to fp32 summation order. */
+int mg_painn_filter_message_workspace_bytes(long n_edges, int n, size_t* bytes);
+int mg_painn_filter_message(const void* packed_W3, const float* bias3, const float* h, const float* h_rowmax,
+                            int h_rowmax_parts, long h_rowmax_stride, int hidden, const int* row_ptr,
+                            const int* src, const int* dst, const float* r_ij, const float* actv, const float* x_v,
+                            long n_nodes, long n_edges, int n, float epsilon, const float* res_a,
+                            const float* res_v, void* workspace, float* out_a, float* out_v, mg_stream_t stream);
+
 /* Update.forward (archs/meanflow_painn8.py:63-75), elementwise parts around its GEMMs.
  * lrv (rows, 3n, 3) = [lin_l | lin_r | lin_v] applied to x_v (one stacked tensor_linear).
  *   pre:  ip[r,c] = sum_x l[c,x] r[c,x];  cat[r] = [x_a[r] | |r[c]|]  (rows, 2n), the MLP input

@@ -20,7 +20,7 @@ namespace {
 
 __device__ __forceinline__ float activate_fast(float v, int act) {
     // SiLU with the hardware exp2 / reciprocal (about 1 ulp each), as in the GEMM epilogues
-    if (act == 1) return v * __frcp_rn(1.0f + __expf(-v));
+    if (act == 1) return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
     if (act == 2) return v > 0.f ? v : 0.1f * v;
     return v;
 }

@@ -1,0 +1,389 @@
+// PaiNN message with the last layer of the filter MLP folded in: the per-edge filter
+//     W(e) = h(e) W3^T + b3            (h: (edges, hidden) output of the MLP's second layer, W3: (4n, hidden))
+// is produced tile by tile on the matrix cores and consumed in the same kernel by
+//     P = W(e) * A(j),  m_v = v(j) P0 + (v(j) x u) P1 + u (x) P2,  m_a = P3,   out(i) = res(i) + sum_e m(e)
+// (archs/meanflow_painn8.py:77-100), so the (edges, 4n) filter never exists in memory.
+//
+// * The GEMM is the split-fp16 row-streaming kernel (three MFMAs per product, fp32 accumulate,
+//   per-row power-of-two scales) with the operands swapped: W is the FIRST matrix operand, so an
+//   accumulator register holds one EDGE (lane % 32) and four consecutive filter columns.  A lane
+//   then owns its edge's neighbour index and direction, and gathers A(j) / v(j) as 16-byte pieces.
+// * The rows of W3 are packed in the order (channel block of 64, k = 0..3, channel in block): one
+//   256-column tile holds all four filter blocks of 64 channels, i.e. everything the message of
+//   those channels needs.
+// * Edges are sorted by receiving node.  A wave reduces its 32 edges through its slice of LDS
+//   (free once the main loop is over): lanes take one output column each and walk the 32 rows,
+//   flushing at the row boundaries of the graph.  A run of edges that starts at the first row of
+//   the wave's block goes to partial slot A of the block, a run that starts later and ends at the
+//   block's last row to slot B, a run strictly inside the block is a whole node and is written
+//   directly (plus the residual).  A second small kernel adds the slots of every node in block
+//   order: fixed summation order, no atomics.
+#include "common.hpp"
+#include "f16x2.hpp"
+
+namespace mg {
+namespace {
+
+constexpr int kFW = 8;                       // waves per workgroup
+constexpr int kFTM = 32 * kFW;               // edges per tile
+constexpr int kFTN = 256;                    // filter columns per tile: 4 blocks x 64 channels
+constexpr int kFNI = kFTN / 32;
+
+__device__ __forceinline__ float4 ldf4(const float* p) { return *reinterpret_cast<const float4*>(p); }
+
+__global__ void __launch_bounds__(64 * kFW)
+painn_filter_message_kernel(const _Float16* __restrict__ Wp, const float* __restrict__ w_inv,
+                            const float* __restrict__ bias, const float* __restrict__ X,
+                            const float* __restrict__ xmax, int xmax_parts, long xmax_stride, long R, int I,
+                            const int* __restrict__ src, const int* __restrict__ dst, const float* __restrict__ r_ij,
+                            const float* __restrict__ actv, const float* __restrict__ x_v, int n, float epsilon,
+                            const float* __restrict__ res_a, const float* __restrict__ res_v,
+                            float* __restrict__ slots, long n_blocks, float* __restrict__ out_a,
+                            float* __restrict__ out_v, int tiles_n, long tiles_total) {
+    constexpr int THREADS = 64 * kFW;
+    constexpr int kPlaneW = kFTN * kRowW, kBufW = 2 * kPlaneW;
+    constexpr int kPieces = 8 * kFTN;
+    constexpr int kPer = kPieces / THREADS;                  // 4
+    constexpr int kSlice = 2 * kBufW / kFW / 4;              // floats of LDS per wave after the main loop
+    constexpr int kRed = 68;                                 // floats per row of a slice: 64 + 4 (spreads the 16-byte writes over the banks)
+    static_assert(kSlice >= 32 * kRed, "a reduction pass needs 32 rows x 64 columns per wave");
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kBufW];
+    __shared__ __attribute__((aligned(16))) float wb[2 * kFTN];   // the tile's 1 / weight scale, then its bias
+
+    const long bid = blockIdx.x;
+    const long per_xcd = (tiles_total + 7) / 8;
+    const long logical = (bid % 8) * per_xcd + bid / 8;
+    if (logical >= tiles_total) return;
+    const long tile_m = logical / tiles_n;
+    const int tile_n = (int)(logical - tile_m * tiles_n);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int m = lane & 31, g = lane >> 5;
+    const long r0 = tile_m * kFTM;
+    const int n0 = tile_n * kFTN;
+    const long plane_elems = (long)tiles_n * kFTN * I;
+
+    floatx16 acc[kFNI];
+#pragma unroll
+    for (int ni = 0; ni < kFNI; ni++)
+#pragma unroll
+        for (int q = 0; q < 16; q++) acc[ni][q] = 0.f;
+
+    const long block = r0 / 32 + wave;                       // this wave's block of 32 edges
+    const long my_row = block * 32 + m;
+    const long ld_row = my_row < R ? my_row : R - 1;
+    const float* xrow = X + ld_row * I + 16 * g;
+    float sx, isx;
+    {
+        float amax = 0.f;
+        const float* xm = xmax + ld_row * xmax_stride;
+        for (int p = 0; p < xmax_parts; p++) amax = fmaxf(amax, xm[p]);
+        sx = pow2_scale(amax, &isx);
+    }
+    // the edge this lane owns in the epilogue
+    const int my_src = src[ld_row];
+    const long my_j = dst[ld_row];
+    float ux = r_ij[3 * ld_row], uy = r_ij[3 * ld_row + 1], uz = r_ij[3 * ld_row + 2];
+
+    const _Float16* wsrc[kPer];
+    int wdst[kPer];
+#pragma unroll
+    for (int j = 0; j < kPer; j++) {
+        const int q = tid + THREADS * j;
+        const int plane = q / (4 * kFTN), row = (q % (4 * kFTN)) >> 2, piece = q & 3;
+        wsrc[j] = Wp + plane * plane_elems + (long)(n0 + row) * I + 8 * piece;
+        wdst[j] = plane * kPlaneW + row * kRowW + piece * 16;
+    }
+    if (tid < kFTN) {
+        wb[tid] = w_inv[n0 + tid];
+        wb[kFTN + tid] = bias[n0 + tid];
+    }
+    const int k_last = I - kCK;
+
+    struct ARegs { float4 v[4]; };
+    struct WRegs { halfx8 v[kPer]; };
+    auto load_a = [&](ARegs& a, int k0) {
+        k0 = k0 < I ? k0 : k_last;
+#pragma unroll
+        for (int j = 0; j < 4; j++) a.v[j] = *reinterpret_cast<const float4*>(xrow + k0 + 4 * j);
+    };
+    auto load_w = [&](WRegs& w, int k0) {
+        k0 = k0 < I ? k0 : k_last;
+#pragma unroll
+        for (int j = 0; j < kPer; j++) w.v[j] = *reinterpret_cast<const halfx8*>(wsrc[j] + k0);
+    };
+    auto store_w = [&](const WRegs& w, unsigned char* buf) {
+#pragma unroll
+        for (int j = 0; j < kPer; j++) *reinterpret_cast<halfx8*>(buf + wdst[j]) = w.v[j];
+    };
+    const int b_off = m * kRowW + 32 * g;
+    auto compute = [&](const ARegs& a, const unsigned char* buf, float scale) {
+        halfx8 ah[2], al[2];
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const HalfSplit4 p0 = split(a.v[2 * s], scale), p1 = split(a.v[2 * s + 1], scale);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                ah[s][i] = p0.hi[i]; ah[s][4 + i] = p1.hi[i];
+                al[s][i] = p0.lo[i]; al[s][4 + i] = p1.lo[i];
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 2; s++)
+#pragma unroll
+            for (int ni = 0; ni < kFNI; ni++) {
+                const halfx8 bh = *reinterpret_cast<const halfx8*>(buf + b_off + ni * 32 * kRowW + 16 * s);
+                const halfx8 bl = *reinterpret_cast<const halfx8*>(buf + kPlaneW + b_off + ni * 32 * kRowW + 16 * s);
+                // W first: D[i][j] with i the filter column in the block and j the edge
+                acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bh, al[s], acc[ni], 0, 0, 0);
+                acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bl, ah[s], acc[ni], 0, 0, 0);
+                acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(bh, ah[s], acc[ni], 0, 0, 0);
+            }
+    };
+
+    unsigned char* buf0 = lds;
+    unsigned char* buf1 = lds + kBufW;
+    ARegs a0, a1;
+    WRegs w;
+    load_w(w, 0);
+    load_a(a0, 0);
+    store_w(w, buf0);
+    load_w(w, kCK);
+    load_a(a1, kCK);
+    __syncthreads();
+    for (int k0 = 0; k0 < I; k0 += 2 * kCK) {
+        compute(a0, buf0, sx);
+        store_w(w, buf1);
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(w, k0 + 2 * kCK);
+        __builtin_amdgcn_sched_barrier(0);
+        load_a(a0, k0 + 2 * kCK);
+        __syncthreads();
+        compute(a1, buf1, k0 + kCK < I ? sx : 0.f);
+        store_w(w, buf0);
+        __builtin_amdgcn_sched_barrier(0);
+        load_w(w, k0 + 3 * kCK);
+        __builtin_amdgcn_sched_barrier(0);
+        load_a(a1, k0 + 3 * kCK);
+        __syncthreads();
+    }
+    // every wave is past its last read of the W buffers: LDS is now eight private slices
+
+    const bool valid = my_row < R;
+    {
+        const float inv = 1.0f / sqrtf(epsilon + (ux * ux + uy * uy + uz * uz));
+        ux *= inv; uy *= inv; uz *= inv;
+    }
+    // runs of equal receiving node among the wave's rows: bit r set = row r starts a run
+    const long rows_left = R - block * 32;
+    const int nv = rows_left >= 32 ? 32 : (rows_left > 0 ? (int)rows_left : 0);
+    const int prev_src = __shfl_up(my_src, 1);
+    const unsigned starts = (unsigned)__ballot(g == 0 && (m == 0 || my_src != prev_src));
+    const int runs = __popc(starts);
+    const int second = runs >= 2 ? __ffs(starts & ~1u) - 1 : 32;      // first row of the second run
+    float* slice = reinterpret_cast<float*>(lds) + wave * kSlice;
+    const int cb = 64 * tile_n;                               // first channel of this tile
+    const long row4n = 4L * n;
+    const float* arow = actv + my_j * row4n;
+    const float* vrow = x_v + my_j * 3L * n;
+    float* slot_a = slots + block * row4n;
+    float* slot_b = slots + (n_blocks + block) * row4n;
+    const float keep = valid ? 1.f : 0.f;                     // rows past the end add nothing
+
+    // gathered operands of one group: 4 consecutive channels, all four filter blocks
+    struct Gather { float4 a[4], v[3]; };
+    auto gather = [&](Gather& t, int gidx) {
+        const int c = cb + 32 * (gidx >> 2) + 8 * (gidx & 3) + 4 * g;
+#pragma unroll
+        for (int k = 0; k < 4; k++) t.a[k] = ldf4(arow + k * n + c);
+#pragma unroll
+        for (int k = 0; k < 3; k++) t.v[k] = ldf4(vrow + 3 * c + 4 * k);
+    };
+    auto flush = [&](float sum, int run_start, int r, long off_v, long off_a, bool is_v) {
+        // the run [run_start, r] of this wave's rows is complete; the same branch for every lane
+        const long off_slot = is_v ? off_v : 3L * n + off_a;
+        if (run_start == 0) {
+            slot_a[off_slot] = sum;
+        } else if (r == 31) {
+            slot_b[off_slot] = sum;
+        } else {
+            const long node = __shfl(my_src, r);
+            if (is_v) {
+                const long at = node * 3L * n + off_v;
+                out_v[at] = (res_v ? res_v[at] : 0.f) + sum;
+            } else {
+                const long at = node * n + off_a;
+                out_a[at] = (res_a ? res_a[at] : 0.f) + sum;
+            }
+        }
+    };
+
+    Gather cur, nxt;
+    gather(cur, 0);
+#pragma unroll
+    for (int gidx = 0; gidx < 8; gidx++) {
+        // the next group's gathers fly during this group's arithmetic and the reduction
+        gather(nxt, gidx < 7 ? gidx + 1 : 7);
+        __builtin_amdgcn_sched_barrier(0);
+        const int h = gidx >> 2, qq = gidx & 3, gi = gidx & 1;
+        const int cl = 32 * h + 8 * qq + 4 * g;               // channel in the tile's block of 64
+        float4 p[4];
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const float4 iw = *reinterpret_cast<const float4*>(wb + 64 * k + cl);
+            const float4 bv = *reinterpret_cast<const float4*>(wb + 256 + 64 * k + cl);
+            const float4 a = cur.a[k];
+            const floatx16& t = acc[2 * k + h];
+            p[k].x = (t[4 * qq + 0] * isx * iw.x + bv.x) * a.x;
+            p[k].y = (t[4 * qq + 1] * isx * iw.y + bv.y) * a.y;
+            p[k].z = (t[4 * qq + 2] * isx * iw.z + bv.z) * a.z;
+            p[k].w = (t[4 * qq + 3] * isx * iw.w + bv.w) * a.w;
+        }
+        const float4 v0 = cur.v[0], v1 = cur.v[1], v2 = cur.v[2];
+        const float vv[12] = {v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w, v2.x, v2.y, v2.z, v2.w};
+        const float q0[4] = {p[0].x, p[0].y, p[0].z, p[0].w}, q1[4] = {p[1].x, p[1].y, p[1].z, p[1].w};
+        const float q2[4] = {p[2].x, p[2].y, p[2].z, p[2].w};
+        float o[12];
+#pragma unroll
+        for (int t = 0; t < 4; t++) {
+            const float x = vv[3 * t], y = vv[3 * t + 1], z = vv[3 * t + 2];
+            const float cx = y * uz - z * uy, cy = z * ux - x * uz, cz = x * uy - y * ux;   // v x u
+            o[3 * t + 0] = x * q0[t] + cx * q1[t] + ux * q2[t];
+            o[3 * t + 1] = y * q0[t] + cy * q1[t] + uy * q2[t];
+            o[3 * t + 2] = z * q0[t] + cz * q1[t] + uz * q2[t];
+        }
+        // row m of the slice: 64 floats = [g][gi][12 of m_v, 4 of m_a]
+        float* wr = slice + m * kRed + g * 32 + gi * 16;
+        *reinterpret_cast<float4*>(wr) = make_float4(o[0] * keep, o[1] * keep, o[2] * keep, o[3] * keep);
+        *reinterpret_cast<float4*>(wr + 4) = make_float4(o[4] * keep, o[5] * keep, o[6] * keep, o[7] * keep);
+        *reinterpret_cast<float4*>(wr + 8) = make_float4(o[8] * keep, o[9] * keep, o[10] * keep, o[11] * keep);
+        *reinterpret_cast<float4*>(wr + 12) = make_float4(p[3].x * keep, p[3].y * keep, p[3].z * keep, p[3].w * keep);
+        cur = nxt;
+        if (gi == 0) continue;
+        // ---- two groups are in the slice: reduce its 64 columns over the rows
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        // lane = output column: which element of the node's outputs it is
+        const int cg = lane >> 5, cgi = (lane >> 4) & 1, k16 = lane & 15;
+        const int cch = cb + 32 * h + 8 * ((qq & 2) + cgi) + 4 * cg;
+        const bool is_v = k16 < 12;
+        const long off_v = 3L * cch + k16;                    // in the (n, 3) vector part
+        const long off_a = cch + (k16 - 12);                  // in the (n) scalar part
+        if (nv > 0) {
+            if (runs <= 2) {
+                // the usual case: all rows in flight at once, one or two sums, no branches in the loop
+                float val[32];
+#pragma unroll
+                for (int r = 0; r < 32; r++) val[r] = slice[r * kRed + lane];
+                float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+                for (int r = 0; r < 32; r++) {
+                    s0 += r < second ? val[r] : 0.f;
+                    s1 += r < second ? 0.f : val[r];
+                }
+                flush(s0, 0, second - 1, off_v, off_a, is_v);
+                if (runs == 2) flush(s1, second, nv - 1, off_v, off_a, is_v);
+            } else {
+                float sum = 0.f;
+                int run_start = 0;
+                for (int r = 0; r < nv; r++) {
+                    sum += slice[r * kRed + lane];
+                    if ((r == nv - 1) || ((starts >> (r + 1)) & 1u)) {
+                        flush(sum, run_start, r, off_v, off_a, is_v);
+                        sum = 0.f;
+                        run_start = r + 1;
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
+// out(node) = res(node) + the partial sums of the blocks its edges lie in, in block order.  Nodes whose
+// edges lie strictly inside one block were written by the kernel above and are skipped; nodes without
+// edges get the residual.  One thread per four consecutive floats of the node's 4n outputs.
+__global__ void __launch_bounds__(256)
+painn_message_finish_kernel(const int* __restrict__ row_ptr, long n_nodes, long n_blocks, int n,
+                            const float* __restrict__ slots, const float* __restrict__ res_a,
+                            const float* __restrict__ res_v, float* __restrict__ out_a, float* __restrict__ out_v) {
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= n_nodes * n) return;
+    const long node = idx / n;
+    const int x = (int)(idx - node * n) * 4;                  // offset in the node's [3n of v | n of a]
+    const long lo = row_ptr[node], hi = row_ptr[node + 1];
+    const bool is_v = x < 3 * n;
+    const float* res = is_v ? res_v : res_a;
+    float* out = is_v ? out_v + node * 3L * n + x : out_a + node * (long)n + (x - 3 * n);
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (res) s = ldf4(is_v ? res + node * 3L * n + x : res + node * (long)n + (x - 3 * n));
+    if (hi > lo) {
+        const long b_lo = lo / 32, b_hi = (hi - 1) / 32;
+        if (b_lo == b_hi && lo > 32 * b_lo && hi - 1 < 32 * b_lo + 31) return;   // written directly
+        const long row4n = 4L * n;
+        for (long b = b_lo; b <= b_hi; b++) {
+            const float* slot = 32 * b >= lo ? slots + b * row4n : slots + (n_blocks + b) * row4n;
+            const float4 t = ldf4(slot + x);
+            s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+        }
+    }
+    *reinterpret_cast<float4*>(out) = s;
+}
+
+}  // namespace
+}  // namespace mg
+
+using namespace mg;
+
+extern "C" {
+
+int mg_painn_filter_message_workspace_bytes(long n_edges, int n, size_t* bytes) {
+    MG_REQUIRE(bytes != nullptr && n_edges >= 0 && n >= 0, "mg_painn_filter_message_workspace_bytes: bad argument");
+    // slots A and B of every block of 32 edges, 4n floats each (never zero bytes: callers allocate it)
+    *bytes = (size_t)(2L * (ceil_div(n_edges, 32) + 1) * 4L * n) * sizeof(float);
+    return MG_OK;
+}
+
+int mg_painn_filter_message(const void* packed_W3, const float* bias3, const float* h, const float* h_rowmax,
+                            int h_rowmax_parts, long h_rowmax_stride, int hidden, const int* row_ptr,
+                            const int* src, const int* dst, const float* r_ij, const float* actv, const float* x_v,
+                            long n_nodes, long n_edges, int n, float epsilon, const float* res_a,
+                            const float* res_v, void* workspace, float* out_a, float* out_v, mg_stream_t stream) {
+    MG_REQUIRE(n >= 64 && n % 64 == 0, "mg_painn_filter_message: n must be a multiple of 64 (got %d)", n);
+    MG_REQUIRE(hidden >= 64 && hidden % 32 == 0, "mg_painn_filter_message: hidden must be a multiple of 32, at least 64 (got %d)", hidden);
+    MG_REQUIRE(n_nodes >= 0 && n_edges >= 0, "mg_painn_filter_message: negative size");
+    MG_REQUIRE(n_edges < (1L << 31) && n_nodes < (1L << 31), "mg_painn_filter_message: int32 indices");
+    MG_REQUIRE(h_rowmax_parts >= 1 && h_rowmax_parts <= 64, "mg_painn_filter_message: 1..64 bound parts");
+    if (n_nodes == 0) return MG_OK;
+    MG_REQUIRE(packed_W3 && bias3 && row_ptr && actv && x_v && out_a && out_v, "mg_painn_filter_message: null operand");
+    MG_REQUIRE(aligned16(packed_W3) && aligned16(bias3) && aligned16(actv) && aligned16(x_v) && aligned16(out_a) &&
+                   aligned16(out_v) && (!res_a || aligned16(res_a)) && (!res_v || aligned16(res_v)),
+               "mg_painn_filter_message: operands must be 16-byte aligned");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const long n_blocks = ceil_div(n_edges, 32);
+    if (n_edges > 0) {
+        MG_REQUIRE(h && h_rowmax && src && dst && r_ij && workspace, "mg_painn_filter_message: null edge operand");
+        MG_REQUIRE(aligned16(h) && aligned16(workspace), "mg_painn_filter_message: h and workspace must be 16-byte aligned");
+        const int tiles_n = n / 64;
+        const long tiles_total = ceil_div(n_edges, kFTM) * tiles_n;
+        const long O_pad = (long)tiles_n * kFTN;                       // = 4n: already a multiple of 256
+        const _Float16* planes = static_cast<const _Float16*>(packed_W3);
+        const float* w_inv = reinterpret_cast<const float*>(planes + 2 * O_pad * hidden);
+        const long grid = 8 * ceil_div(tiles_total, 8);
+        MG_REQUIRE(grid < (1L << 31), "mg_painn_filter_message: too many tiles");
+        painn_filter_message_kernel<<<dim3((unsigned)grid), dim3(64 * kFW), 0, s>>>(
+            planes, w_inv, bias3, h, h_rowmax, h_rowmax_parts, h_rowmax_stride, n_edges, hidden, src, dst, r_ij, actv,
+            x_v, n, epsilon, res_a, res_v, static_cast<float*>(workspace), n_blocks, out_a, out_v, tiles_n, tiles_total);
+        if (int st = check_launch("painn_filter_message_kernel")) return st;
+    }
+    const long threads = n_nodes * n;
+    painn_message_finish_kernel<<<dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, s>>>(
+        row_ptr, n_nodes, n_blocks, n, static_cast<const float*>(workspace), res_a, res_v, out_a, out_v);
+    return check_launch("painn_message_finish_kernel");
+}
+
+}  // extern "C"

@@ -33,7 +33,7 @@ constexpr int kPlane = 128 * kRowB;       // bytes per plane
 
 __device__ __forceinline__ float activate(float v, int act) {
     // SiLU with the hardware exp2 / reciprocal (about 1 ulp each): far inside the fp32 tolerance
-    if (act == 1) return v * __frcp_rn(1.0f + __expf(-v));
+    if (act == 1) return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
     if (act == 2) return v > 0.f ? v : 0.1f * v;
     return v;
 }

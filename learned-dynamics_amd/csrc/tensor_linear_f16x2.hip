@@ -41,7 +41,7 @@ namespace mg {
 namespace {
 
 __device__ __forceinline__ float activate(float v, int act) {
-    if (act == 1) return v * __frcp_rn(1.0f + __expf(-v));
+    if (act == 1) return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
     if (act == 2) return v > 0.f ? v : 0.1f * v;
     return v;
 }

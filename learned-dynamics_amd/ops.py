@@ -937,6 +937,66 @@ def painn_message(row_ptr, dst, r_ij, filt, actv, x_v, epsilon, res_a=None, res_
     return out_a, out_v
 
 
+def painn_filter_message_supported(n, hidden, n_edges):
+    """The fused filter + message kernel: channel blocks of 64, a hidden width the matrix path tiles, and
+    enough edges to fill the chip with 256-edge tiles."""
+    return (get_linear_mode() == LINEAR_F16X2 and n % 64 == 0 and hidden % 32 == 0 and hidden >= 64
+            and n_edges >= 1024)
+
+
+def painn_filter_permutation(n, device):
+    """Order of the 4n filter columns in the fused kernel's packed weight: (channel block of 64, k, channel
+    in block).  perm[p] is the filter column k n + c that packed row p holds."""
+    c = torch.arange(n, device=device)
+    k = torch.arange(4, device=device)
+    col = (k[None, :, None] * n + (c.reshape(n // 64, 1, 64)))     # (blocks, 4, 64)
+    return col.reshape(-1)
+
+
+def painn_filter_message(W3_perm, bias3_perm, h, h_bound, row_ptr, src, dst, r_ij, actv, x_v, epsilon,
+                         res_a=None, res_v=None):
+    """painn_message(filt = h @ W3.T + bias3, ...) without storing filt.  W3_perm / bias3_perm: W3 / bias3 with
+    rows in painn_filter_permutation order; h (edges, hidden); h_bound (edges, parts) or (1, parts): upper
+    bounds of the row maxima of |h|."""
+    for t, nm in ((W3_perm, "W3_perm"), (bias3_perm, "bias3_perm"), (h, "h"), (h_bound, "h_bound"), (r_ij, "r_ij"),
+                  (actv, "actv"), (x_v, "x_v")):
+        _check_input(t, nm)
+    for t, nm in ((row_ptr, "row_ptr"), (src, "src"), (dst, "dst")):
+        _check_input(t, nm, torch.int32)
+    n_nodes, n = int(x_v.size(0)), int(x_v.size(1))
+    E, hidden = int(h.size(0)), int(h.size(1))
+    if tuple(x_v.shape) != (n_nodes, n, 3):
+        raise RuntimeError("x_v must have shape (nodes, n, 3)")
+    if tuple(actv.shape) != (n_nodes, 4 * n):
+        raise RuntimeError("actv must have shape (nodes, 4n)")
+    if tuple(W3_perm.shape) != (4 * n, hidden) or tuple(bias3_perm.shape) != (4 * n,):
+        raise RuntimeError("W3_perm must have shape (4n, hidden) and bias3_perm (4n,)")
+    if tuple(r_ij.shape) != (E, 3) or src.numel() != E or dst.numel() != E:
+        raise RuntimeError("r_ij, src and dst must have one row per edge")
+    if row_ptr.numel() != n_nodes + 1:
+        raise RuntimeError("row_ptr must have nodes+1 entries")
+    if h_bound.dim() != 2 or h_bound.size(0) not in (1, E) or not 1 <= h_bound.size(1) <= 64:
+        raise RuntimeError("h_bound must be (edges, parts) or (1, parts) with 1..64 parts")
+    for t, nm, shape in ((res_a, "res_a", (n_nodes, n)), (res_v, "res_v", (n_nodes, n, 3))):
+        if t is not None:
+            _check_input(t, nm)
+            if tuple(t.shape) != shape:
+                raise RuntimeError(f"{nm} has wrong shape")
+    dev = x_v.device
+    nbytes = ctypes.c_size_t(0)
+    L.check(_lib.mg_painn_filter_message_workspace_bytes(E, n, ctypes.byref(nbytes)))
+    with torch.cuda.device(dev):
+        out_a = torch.empty(n_nodes, n, dtype=torch.float32, device=dev)
+        out_v = torch.empty(n_nodes, n, 3, dtype=torch.float32, device=dev)
+        work = torch.empty(nbytes.value // 4, dtype=torch.float32, device=dev)
+        stride = 0 if h_bound.size(0) == 1 else int(h_bound.size(1))
+        L.check(_lib.mg_painn_filter_message(
+            _p(packed_weight_f16x2(W3_perm)), _p(bias3_perm), _p(h), _p(h_bound), int(h_bound.size(1)), stride,
+            hidden, _p(row_ptr), _p(src), _p(dst), _p(r_ij), _p(actv), _p(x_v), n_nodes, E, n, float(epsilon),
+            _p(res_a), _p(res_v), _p(work), _p(out_a), _p(out_v), _stream()))
+    return out_a, out_v
+
+
 # ------------------------------------------------------- rank-0/1/2 messages
 def bee_edge_geometry(r_ij, r0):
     """(E,3) -> enc (E,8) = radial_encode_8(r_ij, r0), rhat (E,3) = tens_sigmoid(1, r_ij*7/r0)."""

@@ -129,14 +129,30 @@ class Message(nn.Module):
         self.mlp_dist = MLP(self.n_rbf, 4 * n)
         self.mlp_actv = MLP(n, 4 * n)
 
-    def filters(self, r_ij):
-        """(edges, 3) -> (edges, 4n): the per-edge filter, the one large per-edge tensor."""
+    def _hidden(self, r_ij):
+        """Radial encoding + first layer + SiLU of the filter MLP: (edges, 4n) and the bound of its rows."""
         first = self.mlp_dist.layers[0]
         if ops.painn_radial_linear_supported(self.n_rbf, first.out_features):
             h = ops.painn_radial_linear(r_ij, self.n_rbf, self.r0, first.weight, first.bias, ops.ACT_SILU)
             # the encoding is cosines and sines: entries at most 1
-            return self.mlp_dist.after_first(h, ops.linear_out_bound(first.weight, first.bias, None))
-        return self.mlp_dist(ops.painn_radial_encode(r_ij, self.n_rbf, self.r0), ops.linear_in_unit_bound(r_ij.device))
+            return h, ops.linear_out_bound(first.weight, first.bias, None)
+        return _linear(ops.painn_radial_encode(r_ij, self.n_rbf, self.r0), first, ops.ACT_SILU,
+                       ops.linear_in_unit_bound(r_ij.device))
+
+    def filters(self, r_ij):
+        """(edges, 3) -> (edges, 4n): the per-edge filter, the one large per-edge tensor."""
+        return self.mlp_dist.after_first(*self._hidden(r_ij))
+
+    def _permuted_last(self):
+        """Last layer of the filter MLP with its rows in the column order of the fused kernel."""
+        last = self.mlp_dist.layers[4]
+        cache = self.__dict__.setdefault("_perm_cache", {})
+        stamp = tuple((id(p), p._version, p.data_ptr()) for p in (last.weight, last.bias))
+        if cache.get("stamp") != stamp:
+            with torch.no_grad():
+                perm = ops.painn_filter_permutation(self.n, last.weight.device)
+                cache.update(stamp=stamp, W=last.weight[perm].contiguous(), b=last.bias[perm].contiguous())
+        return cache["W"], cache["b"]
 
     def forward(self, graph: Graph, x_a, x_v, r_ij, residual=False):
         """x_a: (batch, atoms, n), x_v: (batch, atoms, n, 3), r_ij: (edges, 3).
@@ -144,10 +160,20 @@ class Message(nn.Module):
         B, N, n = x_a.shape
         flat_a = x_a.reshape(B * N, n).contiguous()
         flat_v = x_v.reshape(B * N, n, 3).contiguous()
-        filt = self.filters(r_ij.contiguous())
+        r_ij = r_ij.contiguous()
         actv = self.mlp_actv(flat_a)
-        out_a, out_v = ops.painn_message(graph.row_ptr, graph.dst32, r_ij.contiguous(), filt, actv, flat_v,
-                                         self.epsilon, flat_a if residual else None, flat_v if residual else None)
+        res_a, res_v = (flat_a, flat_v) if residual else (None, None)
+        if ops.painn_filter_message_supported(n, 4 * n, r_ij.shape[0]):
+            # the filter's last layer runs inside the edge kernel: the (edges, 4n) filter is never stored
+            h, bound = self._hidden(r_ij)
+            h, bound = _linear(h, self.mlp_dist.layers[2], ops.ACT_SILU, bound)
+            W3, b3 = self._permuted_last()
+            out_a, out_v = ops.painn_filter_message(W3, b3, h, bound, graph.row_ptr, graph.src32, graph.dst32, r_ij,
+                                                    actv, flat_v, self.epsilon, res_a, res_v)
+            return out_a.reshape(B, N, n), out_v.reshape(B, N, n, 3)
+        filt = self.filters(r_ij)
+        out_a, out_v = ops.painn_message(graph.row_ptr, graph.dst32, r_ij, filt, actv, flat_v,
+                                         self.epsilon, res_a, res_v)
         return out_a.reshape(B, N, n), out_v.reshape(B, N, n, 3)
 
 

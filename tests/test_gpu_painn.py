@@ -108,6 +108,71 @@ def test_fused_message_kernel(ops, n, with_res):
     _close(out_v, ref_v, atol_scale=2e-6)
 
 
+def _degrees(kind, N, g):
+    """Row lengths that exercise every way a node's edges can sit in the kernel's blocks of 32 edges."""
+    if kind == "long":          # rows span several blocks
+        return torch.randint(40, 140, (N,), generator=g)
+    if kind == "short":         # many whole rows inside one block, empty rows between them
+        return torch.randint(0, 9, (N,), generator=g)
+    if kind == "aligned":       # rows that start and end exactly on block boundaries, and one-edge rows
+        return torch.tensor([32, 64, 1, 31, 32, 0, 0, 96, 33, 31] * (N // 10))
+    return torch.cat([torch.randint(0, 5, (N // 2,), generator=g), torch.randint(20, 300, (N - N // 2,), generator=g)])[
+        torch.randperm(N, generator=g)]
+
+
+@pytest.mark.parametrize("n,hidden,kind,with_res", [(128, 512, "long", True), (64, 256, "short", False),
+                                                    (128, 96, "aligned", True), (192, 128, "mixed", True),
+                                                    (64, 64, "mixed", False)])
+def test_filter_message_fused_with_last_linear(ops, n, hidden, kind, with_res):
+    """filt = h W3^T + b3 produced inside the edge kernel against the two-kernel path fed with the same
+    split-fp16 product, and against plain fp64 arithmetic."""
+    g = torch.Generator().manual_seed(n + hidden)
+    N = 400
+    deg = _degrees(kind, N, g)
+    src = torch.repeat_interleave(torch.arange(N), deg)
+    E = int(src.numel())
+    dst = torch.randint(0, N, (E,), generator=g)
+    r = torch.randn(E, 3, generator=g) * 3
+    h = torch.randn(E, hidden, generator=g) * torch.rand(E, 1, generator=g) * 4
+    W3 = torch.randn(4 * n, hidden, generator=g) / hidden ** 0.5
+    b3 = torch.randn(4 * n, generator=g)
+    actv = torch.randn(N, 4 * n, generator=g)
+    x_a, x_v = torch.randn(N, n, generator=g), torch.randn(N, n, 3, generator=g)
+    dev = lambda t: t.cuda()
+    row_ptr = ops.segment_row_ptr(dev(src.int()), N)
+    perm = ops.painn_filter_permutation(n, "cuda")
+    assert torch.equal(torch.sort(perm).values, torch.arange(4 * n, device="cuda"))
+    W3p, b3p = dev(W3)[perm].contiguous(), dev(b3)[perm].contiguous()
+    bound = ops.row_absmax(dev(h))
+    res = (dev(x_a), dev(x_v)) if with_res else (None, None)
+    out_a, out_v = ops.painn_filter_message(W3p, b3p, dev(h), bound, row_ptr, dev(src.int()), dev(dst.int()), dev(r),
+                                            dev(actv), dev(x_v), 0.1, *res)
+    # the same numbers through the stored filter
+    filt = ops.tensor_linear_f16x2(dev(W3), dev(h), bound, bias=dev(b3))
+    two_a, two_v = ops.painn_message(row_ptr, dev(dst.int()), dev(r), filt, dev(actv), dev(x_v), 0.1, *res)
+    _close(out_a, two_a.cpu(), atol_scale=2e-6)
+    _close(out_v, two_v.cpu(), atol_scale=2e-6)
+    # and plain arithmetic
+    d = lambda t: t.double()
+    p = (d(h) @ d(W3).T + d(b3)) * d(actv)[dst]
+    u = d(r) / torch.sqrt(0.1 + (d(r) ** 2).sum(-1, keepdim=True))
+    v = d(x_v)[dst]
+    m_v = v * p[:, :n, None] + torch.linalg.cross(v, u[:, None].expand_as(v)) * p[:, n:2 * n, None] \
+        + u[:, None] * p[:, 2 * n:3 * n, None]
+    ref_v = torch.zeros(N, n, 3, dtype=torch.float64).index_add_(0, src, m_v)
+    ref_a = torch.zeros(N, n, dtype=torch.float64).index_add_(0, src, p[:, 3 * n:])
+    if with_res:
+        ref_v, ref_a = ref_v + x_v, ref_a + x_a
+    _close(out_a, ref_a.float(), atol_scale=3e-6)
+    _close(out_v, ref_v.float(), atol_scale=3e-6)
+    # a shared bound for all rows (one row of parts) is accepted as well
+    shared = bound.amax().reshape(1, 1)
+    sh_a, sh_v = ops.painn_filter_message(W3p, b3p, dev(h), shared, row_ptr, dev(src.int()), dev(dst.int()), dev(r),
+                                          dev(actv), dev(x_v), 0.1, *res)
+    _close(sh_a, ref_a.float(), atol_scale=3e-6)
+    _close(sh_v, ref_v.float(), atol_scale=3e-6)
+
+
 @pytest.mark.parametrize("n,n_rbf", [(32, None), (128, 16)])
 def test_message_module(pkg, n, n_rbf):
     painn = importlib.import_module("learned-dynamics_amd.painn")
