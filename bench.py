@@ -181,7 +181,34 @@ def bench_painn_layer(torch, args):
         t_graph = event_time(torch, lambda: gl.graph_setup(r0, box, pos_d, neighbours_max=512, celllist_max=128), 5)
         breakdown = {"filter_gemm_512x512_ms": t_gemm * 1e3, "edge_kernel_ms": t_edge * 1e3,
                      "graph_build_ms_not_in_step": t_graph * 1e3}
-        del filt, actv
+        del filt
+        if ops.painn_filter_message_supported(n, 4 * n, E):
+            # as the layer runs it: the filter MLP's last layer inside the edge kernel (the largest kernel of
+            # the step); the stand-alone GEMM above is the MLP's middle layer, the second largest
+            msg = block.message
+            h1, b1 = msg._hidden(r_ij)
+            h2, b2 = painn._linear(h1, msg.mlp_dist.layers[2], ops.ACT_SILU, b1)
+            W3, b3 = msg._permuted_last()
+            del h1
+            t_fused = event_time(torch, lambda: ops.painn_filter_message(
+                W3, b3, h2, b2, graph.row_ptr, graph.src32, graph.dst32, r_ij, actv, xv_flat, 0.1, xa_flat, xv_flat), 10)
+            del h2
+            breakdown["filter_last_layer_plus_edge_kernel_ms"] = t_fused * 1e3
+            roofline_gemm = roofline
+            roofline = {"kernel": "painn_filter_message_kernel (E x 512 x 512 split-fp16 GEMM whose epilogue gathers, "
+                                  "multiplies and row-sums the messages) + painn_message_finish_kernel (about 1 % of the time)",
+                        "bound": "mfma", "achieved": 3 * flops / t_fused / 1e12, "peak": PEAK_BF16_MFMA_TFLOPS,
+                        "unit": "TFLOP/s", "frac": 3 * flops / t_fused / 1e12 / PEAK_BF16_MFMA_TFLOPS,
+                        "traffic": measured_traffic("painn_filter_message_kernel"),
+                        "note": "achieved counts the executed fp16 MFMA FLOPs of the GEMM part (3 per fp32 multiply-add "
+                                "pair) against the fp16 dense peak; the message arithmetic and gathers in the epilogue "
+                                "count as overhead",
+                        "fp32_equivalent_tflops": flops / t_fused / 1e12,
+                        "second_kernel": roofline_gemm}
+            roofline_hbm["note"] = ("the stand-alone edge kernel (filter read from memory); this workload runs the fused "
+                                    "kernel above instead, the stand-alone one serves channel counts that are not a "
+                                    "multiple of 64 and the other GEMM modes")
+        del actv
 
     cpu = None
     if not args.no_cpu:
