@@ -1,8 +1,10 @@
 """Ant16 / Bee / Cow0 / Cow1 autograd functions, mirroring
 managan/codegen_tensor_products.py:19-101 of the reference on top of the HIP
-kernels (Bee, Cow: forward and both backward passes; Ant16: forward)."""
+kernels (Bee, Cow: forward and both backward passes; Ant16: forward kernel, backward as
+device-side contractions)."""
 import torch
 
+from . import ant16_backward as a16
 from . import ops
 
 
@@ -10,15 +12,22 @@ def _c(ts):
     return [t.contiguous() for t in ts]
 
 
+_ANT16_LABELS = ("000", "110", "220", "011", "101", "121", "211", "111", "022", "202", "112", "222", "212")
+
+
 class Ant16(torch.autograd.Function):
-    """managan/codegen_tensor_products.py:19-61.  Forward only: the legacy architectures that use it
-    run inference here; differentiating through it raises."""
+    """managan/codegen_tensor_products.py:19-61.  Arguments after x_0, x_1, x_2 are (P, left) pairs in
+    the order 000 110 220 011 101 121 211 111 022 202 112 222 212; gradients come back in that order."""
 
     @staticmethod
     def forward(ctx, x_0, x_1, x_2,
                 P_000, left_000, P_110, left_110, P_220, left_220,
                 P_011, left_011, P_101, left_101, P_121, left_121, P_211, left_211, P_111, left_111,
                 P_022, left_022, P_202, left_202, P_112, left_112, P_222, left_222, P_212, left_212):
+        ctx.save_for_backward(x_0, x_1, x_2,
+                              P_000, left_000, P_110, left_110, P_220, left_220,
+                              P_011, left_011, P_101, left_101, P_121, left_121, P_211, left_211, P_111, left_111,
+                              P_022, left_022, P_202, left_202, P_112, left_112, P_222, left_222, P_212, left_212)
         y_0, = ops.ant16_o0(x_0, x_1, x_2, P_000, left_000, P_110, left_110, P_220, left_220)
         y_1, = ops.ant16_o1(x_0, x_1, x_2, P_011, left_011, P_101, left_101, P_121, left_121, P_211, left_211)
         y_2, = ops.ant16_o2(x_0, x_1, x_2, P_022, left_022, P_202, left_202, P_112, left_112, P_222, left_222)
@@ -26,8 +35,22 @@ class Ant16(torch.autograd.Function):
         return y_0, y_1 + y_1c, y_2 + y_2c
 
     @staticmethod
-    def backward(ctx, *dys):
-        raise NotImplementedError("Ant16: backward is not implemented (inference only)")
+    def backward(ctx, dy_0, dy_1, dy_2):
+        xs = ctx.saved_tensors[:3]
+        pairs = ctx.saved_tensors[3:]
+        dys = (dy_0, dy_1, dy_2)
+        dxs = [None, None, None]
+        grads = []
+        for k, lab in enumerate(_ANT16_LABELS):
+            P, left = pairs[2 * k], pairs[2 * k + 1]
+            dy, x, r = dys[int(lab[2])], xs[int(lab[1])], int(lab[1])
+            needs = ctx.needs_input_grad
+            if needs[r]:
+                d = a16.grad_x(lab, dy, P, left)
+                dxs[r] = d if dxs[r] is None else dxs[r] + d
+            grads.append(a16.grad_P(lab, dy, left, x) if needs[3 + 2 * k] else None)
+            grads.append(a16.grad_left(lab, dy, P, x) if needs[4 + 2 * k] else None)
+        return (*dxs, *grads)
 
 
 class Bee(torch.autograd.Function):

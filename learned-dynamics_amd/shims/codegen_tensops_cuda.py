@@ -1,10 +1,11 @@
 """Drop-in for the reference's `codegen_tensops_cuda` extension
 (extensions/codegen_tensops/codegen_tensops.cpp:1980-2011).  The Bee and Cow
 families and the Ant16 forward functions run on the HIP kernels; the Ant16 backward functions
-(training of the legacy architectures) raise NotImplementedError."""
+(training of the legacy architectures) are device-side contractions through the GEMM library."""
 import importlib
 
 _ops = importlib.import_module("learned-dynamics_amd.ops")
+_a16 = importlib.import_module("learned-dynamics_amd.ant16_backward")
 
 bee_fwd_cuda = _ops.bee_fwd
 bee_bwl_cuda = _ops.bee_bwl
@@ -22,9 +23,9 @@ def set_kern_attributes():
     return None
 
 
-def _ant16_unavailable(name):
+def _unavailable(name):
     def fn(*args, **kwargs):
-        raise NotImplementedError(f"{name}: only the forward functions of the Ant16 family are implemented")
+        raise NotImplementedError(f"{name}: the reference's worked example kernel is not part of this library")
     fn.__name__ = name
     return fn
 
@@ -34,10 +35,23 @@ ant16_o1_cuda = _ops.ant16_o1
 ant16_o2_cuda = _ops.ant16_o2
 ant16_oc_cuda = _ops.ant16_oc
 
-for _o in ("o0", "o1", "o2", "oc"):
-    for _suffix in ("_backward", "_backleft", "_wtsback"):
+
+def _checked(name, fn):
+    def wrapper(*tensors):
+        for k, t in enumerate(tensors):
+            _ops._check_input(t, f"{name} argument {k}")
+        return fn(*tensors)
+    wrapper.__name__ = name
+    return wrapper
+
+
+for _o in ("o0", "o1", "o2"):
+    for _suffix, _fn in (("_backward", _a16.backward), ("_backleft", _a16.backleft), ("_wtsback", _a16.wtsback)):
         _name = f"ant16_{_o}{_suffix}_cuda"
-        globals()[_name] = _ant16_unavailable(_name)
+        globals()[_name] = _checked(_name, (lambda f, o: lambda *a: f(o, *a))(_fn, _o))
+ant16_oc_backward_cuda = _checked("ant16_oc_backward_cuda", _a16.oc_backward)
+ant16_oc_backleft_cuda = _checked("ant16_oc_backleft_cuda", _a16.oc_backleft)
+ant16_oc_wtsback_cuda = _checked("ant16_oc_wtsback_cuda", _a16.oc_wtsback)
 for _suffix in ("", "_backward", "_backleft", "_wtsback"):
     _name = f"fused_tensor_prods_example{_suffix}_cuda"
-    globals()[_name] = _ant16_unavailable(_name)
+    globals()[_name] = _unavailable(_name)

@@ -67,3 +67,74 @@ def test_ant16_shim_functions_and_errors(ops):
     y0, = ops.ant16_o0(e[0], e[1], e[2], d(P["000"]), d(left["000"][:0]), d(P["110"]), d(left["110"][:0]),
                        d(P["220"]), d(left["220"][:0]))
     assert y0.shape == (0, 32)
+
+
+def _oracle_grads(x, P, left, cot):
+    """Gradients of sum_k <y_k, cot_k> by autograd through the float64 oracle."""
+    xd = [t.double().requires_grad_() for t in x]
+    Pd = {k: v.double().requires_grad_() for k, v in P.items()}
+    ld = {k: v.double().requires_grad_() for k, v in left.items()}
+    ys = OP.ant16(*xd, Pd, ld)
+    sum((y * c.double()).sum() for y, c in zip(ys, cot)).backward()
+    return [t.grad for t in xd], {k: v.grad for k, v in Pd.items()}, {k: v.grad for k, v in ld.items()}
+
+
+@pytest.mark.parametrize("shape", [(10, 64, 48, 32, 16), (23, 24, 40, 16, 8)])
+def test_ant16_backward_matches_autograd_of_oracle(shape):
+    """All 29 gradients of the Ant16 function (managan/codegen_tensor_products.py:35-61)."""
+    cg = importlib.import_module("learned-dynamics_amd.codegen_tensor_products")
+    batch, d0, d1, d2, dl = shape
+    x, P, left = _inputs(batch, d0, d1, d2, dl, seed=sum(shape) + 1)
+    g = torch.Generator().manual_seed(3)
+    cot = [torch.randn(batch, (d0, d1, d2)[k], *([3] * k), generator=g) for k in range(3)]
+    args = [t.requires_grad_() for t in _args(x, P, left, "cuda")]
+    ys = cg.Ant16.apply(*args)
+    sum((y * c.cuda()).sum() for y, c in zip(ys, cot)).backward()
+    rx, rP, rl = _oracle_grads(x, P, left, cot)
+    order = ("000", "110", "220", "011", "101", "121", "211", "111", "022", "202", "112", "222", "212")
+    refs = list(rx)
+    for lab in order:
+        refs += [rP[lab], rl[lab]]
+    for a, r in zip(args, refs):
+        assert a.grad is not None and a.grad.shape == r.shape
+        torch.testing.assert_close(a.grad.cpu().double(), r, rtol=1e-5, atol=4e-6 * float(r.abs().max()))
+
+
+def test_ant16_backward_shim_families():
+    """ant16_o*_backward / _backleft / _wtsback_cuda with the reference's argument orders
+    (extensions/codegen_tensops/codegen_tensops.cpp:1981-2000)."""
+    importlib.import_module("learned-dynamics_amd").install_shims()
+    shim = importlib.import_module("codegen_tensops_cuda")
+    batch, d0, d1, d2, dl = 9, 16, 24, 8, 8
+    x, P, left = _inputs(batch, d0, d1, d2, dl, seed=77)
+    g = torch.Generator().manual_seed(4)
+    cot = [torch.randn(batch, (d0, d1, d2)[k], *([3] * k), generator=g) for k in range(3)]
+    d = lambda t: t.cuda()
+    close = lambda a, r: torch.testing.assert_close(a.cpu().double(), r, rtol=1e-5, atol=4e-6 * float(r.abs().max()) + 1e-12)
+    fams = {"o0": (0, ("000", "110", "220")), "o1": (1, ("011", "101", "121", "211")), "o2": (2, ("022", "202", "112", "222"))}
+    for fam, (ro, labs) in fams.items():
+        # the family alone: zero cotangents for the other ranks, other product types switched off
+        only = [cot[k] if k == ro else torch.zeros_like(cot[k]) for k in range(3)]
+        Pz = {k: (v if k in labs else torch.zeros_like(v)) for k, v in P.items()}
+        rx, rP, rl = _oracle_grads(x, Pz, left, only)
+        pl = [t for lab in labs for t in (d(P[lab]), d(left[lab]))]
+        dx = getattr(shim, f"ant16_{fam}_backward_cuda")(d(cot[ro]), *pl)
+        for k in range(3):
+            close(dx[k], rx[k])
+        dl_ = getattr(shim, f"ant16_{fam}_backleft_cuda")(d(x[0]), d(x[1]), d(x[2]), d(cot[ro]), *[d(P[lab]) for lab in labs])
+        dP = getattr(shim, f"ant16_{fam}_wtsback_cuda")(d(x[0]), d(x[1]), d(x[2]), d(cot[ro]), *[d(left[lab]) for lab in labs])
+        for k, lab in enumerate(labs):
+            close(dl_[k], rl[lab])
+            close(dP[k], rP[lab])
+    # chiral pair
+    only = [torch.zeros_like(cot[0]), cot[1], cot[2]]
+    Pz = {k: (v if k in ("111", "212") else torch.zeros_like(v)) for k, v in P.items()}
+    rx, rP, rl = _oracle_grads(x, Pz, left, only)
+    dx1, dx2 = shim.ant16_oc_backward_cuda(d(cot[1]), d(cot[2]), d(P["111"]), d(left["111"]), d(P["212"]), d(left["212"]))
+    close(dx1, rx[1])
+    assert dx2.shape == (batch, d2, 3, 3) and not bool(dx2.any())
+    dl111, dl212 = shim.ant16_oc_backleft_cuda(d(x[1]), d(x[2]), d(cot[1]), d(cot[2]), d(P["111"]), d(P["212"]))
+    dP111, dP212 = shim.ant16_oc_wtsback_cuda(d(x[1]), d(x[2]), d(cot[1]), d(cot[2]), d(left["111"]), d(left["212"]))
+    close(dl111, rl["111"]); close(dl212, rl["212"]); close(dP111, rP["111"]); close(dP212, rP["212"])
+    with pytest.raises(RuntimeError):
+        shim.ant16_o0_backward_cuda(cot[0], *pl[:6])          # host tensor

@@ -191,3 +191,27 @@ def test_backward_helper_matches_finite_differences():
             ls_m = [l0, l1, l2]; ls_m[k] = tm.reshape(t.shape)
             fd = (loss(ls_p, (r0, r1, r2)) - loss(ls_m, (r0, r1, r2))) / (2 * h)
             assert abs(fd - dl[k].reshape(-1)[j]) < 1e-6
+
+
+def test_ant16_backward_contractions_against_autograd():
+    """The host-side contractions behind the Ant16 backward functions (a pure torch module, so it runs
+    here in float64 on the CPU) against autograd through the oracle's forward: every product type,
+    every operand, on sizes where all axes differ."""
+    import importlib
+    a16 = importlib.import_module("learned-dynamics_amd.ant16_backward")
+    g = torch.Generator().manual_seed(33)
+    batch, dims, dl = 3, (4, 5, 2), 6
+    x = [torch.randn(batch, dims[k], *([3] * k), generator=g, dtype=torch.float64, requires_grad=True) for k in range(3)]
+    for lab in OP.BEE_ORDER:
+        rl, rr, ro = (int(c) for c in lab)
+        P = torch.randn(dims[ro], dl, dims[rr], generator=g, dtype=torch.float64, requires_grad=True)
+        left = torch.randn(batch, dl, *([3] * rl), generator=g, dtype=torch.float64, requires_grad=True)
+        zeros_P = {k: torch.zeros(dims[int(k[2])], dl, dims[int(k[1])], dtype=torch.float64) for k in OP.BEE_ORDER}
+        zeros_l = {k: torch.zeros(batch, dl, *([3] * int(k[0])), dtype=torch.float64) for k in OP.BEE_ORDER}
+        zeros_P[lab], zeros_l[lab] = P, left
+        y = OP.ant16(x[0], x[1], x[2], zeros_P, zeros_l)[ro]
+        dy = torch.randn(y.shape, generator=g, dtype=torch.float64)
+        gx, gP, gl = torch.autograd.grad((y * dy).sum(), (x[rr], P, left))
+        assert torch.allclose(a16.grad_x(lab, dy, P, left), gx, atol=1e-12)
+        assert torch.allclose(a16.grad_P(lab, dy, left, x[rr]), gP, atol=1e-12)
+        assert torch.allclose(a16.grad_left(lab, dy, P, x[rr]), gl, atol=1e-12)
