@@ -365,12 +365,28 @@ def bench_denoiser(torch, args, with_cpu=True):
         gl = importlib.import_module("learned-dynamics_amd.graph_layers")
         graph, _ = gl.graph_setup(r0, box, dev[3], neighbours_max=256, celllist_max=64)
         E = int(graph.src.numel())
+        # one system (2048 atoms): a forward pass is ~600 launches of a few microseconds each, so the host
+        # sets the pace; the same layers replayed from a captured HIP graph (neighbour search outside)
+        ro = importlib.import_module("learned-dynamics_amd.rollout")
+        one = [v[:1].contiguous() for v in dev]
+        g1, _ = gl.graph_setup(r0, box, one[3], neighbours_max=256, celllist_max=64)
+
+        def layers(s_, t_, x0_, x1_):
+            return model.forward_on_graph((s_, t_), x0_, x1_, one[4], g1, gl.edge_vectors(g1, x1_, box))
+        t_eager = event_time(torch, lambda: layers(*one[:4]), 10)
+        captured = ro.GraphedCall(layers, *one[:4])
+        t_graph = event_time(torch, lambda: captured(*one[:4]), 10)
+        single = {"atoms": N, "edges": int(g1.src.numel()), "layers_eager_ms": t_eager * 1e3,
+                  "layers_hip_graph_replay_ms": t_graph * 1e3,
+                  "note": "8 blocks on a prebuilt neighbour graph, one system; the replay includes the copies "
+                          "into the capture's static inputs"}
     out = {"metric": "denoiser forward atoms/sec", "value": B * N / sec, "unit": "atoms/s", "ms_per_step": sec * 1e3,
            "dtype": "f32",
            "config": {"workload": "BASELINE configs[3]: 8 x [Messages + SelfTensProds] rank-0/1/2 denoiser forward "
                                   "(assembled from reference modules), 32 systems x 2048 atoms, box 70 A, cutoff 6 A, "
                                   "256 scalar + 64 vector + 16 rank-2 channels, chan 256, graph rebuilt every forward",
-                      "edges": E, "atoms": B * N}}
+                      "edges": E, "atoms": B * N},
+           "single_system": single}
     if with_cpu:
         out["cpu_baseline"] = cpu_denoiser_block(torch, model, x1[:1], r0, box, dims)
     return out

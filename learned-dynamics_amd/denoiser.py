@@ -52,11 +52,16 @@ class Denoiser(nn.Module):
 
     def forward(self, st, x0, x1, one_hot, box, neighbours_max=256, celllist_max=64, node_order="cell"):
         """st: ((batch), (batch)); x0, x1: (batch, atoms, 3); one_hot: (batch, atoms, types)."""
+        graph, r_ij = graph_setup(self.r0, box, x1.contiguous(), neighbours_max=neighbours_max,
+                                  celllist_max=celllist_max)
+        return self.forward_on_graph(st, x0, x1, one_hot, graph, r_ij, node_order=node_order)
+
+    def forward_on_graph(self, st, x0, x1, one_hot, graph, r_ij, node_order="cell"):
+        """The forward pass after the neighbour search: no host synchronisation, fixed launch sequence
+        for a given edge count (what a captured HIP graph replays)."""
         s, t = st
         B, N = x1.shape[:2]
         dim_a, dim_v, dim_d = self.dims
-        graph, r_ij = graph_setup(self.r0, box, x1.contiguous(), neighbours_max=neighbours_max,
-                                  celllist_max=celllist_max)
         x_a = ops.tensor_linear_fwd(0, self.embed.weight, one_hot.contiguous(), bias=self.embed.bias)
         x_a = x_a + self.t_embed(st)[:, None]
         x_v = self.v_readin((x1 - x0)[..., None, :].contiguous())

@@ -1,0 +1,107 @@
+"""Callers of the hot path (learned-dynamics_amd/rollout.py): the one-call meanflow sampler
+(archs/meanflow_painn8.py:302-310), the reverse-diffusion loop (archs/diffuser_atoms15.py:536-555),
+the rollout loop (managan/predictor.py:164-176), and HIP-graph capture of the layers on a prebuilt
+neighbour graph: every replay must equal the eager result, with eager work and synchronisations
+between the replays."""
+import importlib
+import math
+
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+
+def _chain(systems, atoms, box, seed):
+    g = torch.Generator().manual_seed(seed)
+    steps = torch.randn(systems, atoms, 3, generator=g)
+    steps = 3.8 * steps / steps.norm(dim=-1, keepdim=True)
+    return (steps.cumsum(1) + torch.rand(systems, 1, 3, generator=g) * box).cuda()
+
+
+def test_schedule_and_diffusion_loop_closed_forms(pkg):
+    ro = importlib.import_module("learned-dynamics_amd.rollout")
+    t = torch.tensor([0.0, 0.5, 1.0])
+    sig = ro.nodecay_cosine_schedule(t, 20.0)
+    assert abs(float(sig[0]) - 20.0) < 1e-4 and abs(float(sig[2])) < 1e-6       # sigma_max at t = 0, 0 at t = 1
+    assert abs(float(sig[1]) - math.cos(math.pi / 4) / math.sqrt(1 / 400 + 0.5)) < 1e-6
+    # a network that knows the answer: x1_pred = target, epsilon_pred = (noised - target) / sigma.  Then the
+    # combined epsilon is exact, and with the fresh noise switched off (generator producing the same draw is
+    # not needed: the last step has sigma_next = 0) the chain ends at the target up to the remaining noise
+    x_0 = torch.zeros(2, 5, 3, device="cuda")
+    target = torch.randn(2, 5, 3, device="cuda", generator=torch.Generator("cuda").manual_seed(1))
+    sigma_max, zeta = 5.0, 0.3
+
+    def dn(t, x0, noised):
+        s = ro.nodecay_cosine_schedule(t, sigma_max)[:, None, None]
+        return (noised - target) / s, target
+    out = ro.diffusion_generate(dn, x_0, sigma_max, zeta, steps=12, generator=torch.Generator("cuda").manual_seed(2))
+    # after the last step sigma = 0: every bit of noise has been removed by exact predictions
+    torch.testing.assert_close(out, target, rtol=0, atol=1e-4)
+
+
+def test_meanflow_generate_and_rollout(pkg):
+    ro = importlib.import_module("learned-dynamics_amd.rollout")
+    den = importlib.import_module("learned-dynamics_amd.denoiser")
+    torch.manual_seed(0x947)
+    B, N, L_box, r0 = 2, 256, 40.0, 6.0
+    box = (L_box,) * 3
+    model = den.Denoiser(r0, dim_a=64, dim_v=32, dim_d=16, chan=64, blocks=2).cuda().eval()
+    one_hot = torch.nn.functional.one_hot(torch.randint(0, 20, (B, N)), 20).float().cuda()
+    x = _chain(B, N, L_box, 5)
+    dn = lambda st, x0, z1: model(st, x0, z1, one_hot, box)
+    gen = torch.Generator("cuda").manual_seed(7)
+    with torch.no_grad():
+        nxt = ro.meanflow_generate(dn, x, 0.5, generator=gen)
+        # the same draw by hand
+        gen2 = torch.Generator("cuda").manual_seed(7)
+        z1 = x + 0.5 * torch.randn(x.shape, device="cuda", generator=gen2)
+        ref = z1 - model((torch.zeros(B).cuda(), torch.ones(B).cuda()), x, z1, one_hot, box)
+    torch.testing.assert_close(nxt, ref, rtol=0, atol=0)
+    # rollout: each frame feeds the next, the state is left at the last frame
+    state = x.clone()
+    gen3 = torch.Generator("cuda").manual_seed(9)
+    traj = ro.rollout(lambda s: ro.meanflow_generate(dn, s, 0.5, generator=gen3), 3, state)
+    assert traj.shape == (3, B, N, 3) and torch.equal(traj[-1], state)
+    gen4 = torch.Generator("cuda").manual_seed(9)
+    with torch.no_grad():
+        step0 = ro.meanflow_generate(dn, x, 0.5, generator=gen4)
+        step1 = ro.meanflow_generate(dn, step0, 0.5, generator=gen4)
+    torch.testing.assert_close(traj[0], step0, rtol=0, atol=0)
+    torch.testing.assert_close(traj[1], step1, rtol=0, atol=0)
+    assert ro.rollout(lambda s: s + 1.0, 2, torch.zeros(3, device="cuda"), ret=False) is None
+
+
+def test_captured_forward_replays_equal_eager(pkg):
+    ro = importlib.import_module("learned-dynamics_amd.rollout")
+    den = importlib.import_module("learned-dynamics_amd.denoiser")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    torch.manual_seed(0x947 + 1)
+    B, N, L_box, r0 = 1, 512, 40.0, 6.0
+    box = (L_box,) * 3
+    model = den.Denoiser(r0, dim_a=64, dim_v=32, dim_d=16, chan=64, blocks=2).cuda().eval()
+    one_hot = torch.nn.functional.one_hot(torch.randint(0, 20, (B, N)), 20).float().cuda()
+    x1 = _chain(B, N, L_box, 11)
+    s, t = torch.zeros(B).cuda(), torch.ones(B).cuda()
+    with torch.no_grad():
+        graph, _ = gl.graph_setup(r0, box, x1, neighbours_max=256, celllist_max=64)
+
+    def layers(s, t, x0, x1):
+        # the topology is fixed; edge vectors follow the positions inside the captured region
+        r_ij = gl.edge_vectors(graph, x1, box)
+        return model.forward_on_graph((s, t), x0, x1, one_hot, graph, r_ij)
+
+    captured = ro.GraphedCall(layers, s, t, x1, x1)
+    g = torch.Generator("cuda").manual_seed(3)
+    for k in range(4):
+        # small moves keep every pair on the same side of the cutoff's edge list (the topology is reused)
+        x0 = x1 + 0.01 * torch.randn(x1.shape, device="cuda", generator=g)
+        tt = torch.rand(B, device="cuda", generator=g)
+        with torch.no_grad():
+            eager = layers(s, tt, x0, x1)
+        torch.cuda.synchronize()
+        out = captured(s, tt, x0, x1).clone()
+        torch.cuda.synchronize()
+        torch.testing.assert_close(out, eager, rtol=0, atol=0)
+    with pytest.raises(RuntimeError, match="shapes"):
+        captured(s, t, x1[:, :10], x1)
