@@ -21,6 +21,7 @@
 // gathers of a wave are 13 unit-stride 256-byte reads.  A lane owns one channel
 // and keeps its 60 running sums in registers; rows are summed in edge order.
 #include "common.hpp"
+#include <type_traits>
 
 namespace mg {
 namespace {
@@ -82,6 +83,23 @@ __device__ __forceinline__ void cross3(const float* a, const float* b, float* o)
     o[2] = a[0] * b[1] - a[1] * b[0];
 }
 
+// max over the wave of non-negative values, valid in lane 63: six cross-lane VALU moves (shifts within
+// rows of 16 lanes, then row broadcasts), no LDS traffic
+__device__ __forceinline__ float wave_max_nonneg_last_lane(float v) {
+    auto step = [](float x, auto ctrl, auto row_mask) {
+        const int moved = __builtin_amdgcn_update_dpp(0, __float_as_int(x), decltype(ctrl)::value,
+                                                      decltype(row_mask)::value, 0xf, false);
+        return fmaxf(x, __int_as_float(moved));
+    };
+    v = step(v, std::integral_constant<int, 0x111>{}, std::integral_constant<int, 0xf>{});   // row_shr:1
+    v = step(v, std::integral_constant<int, 0x112>{}, std::integral_constant<int, 0xf>{});   // row_shr:2
+    v = step(v, std::integral_constant<int, 0x114>{}, std::integral_constant<int, 0xf>{});   // row_shr:4
+    v = step(v, std::integral_constant<int, 0x118>{}, std::integral_constant<int, 0xf>{});   // row_shr:8
+    v = step(v, std::integral_constant<int, 0x142>{}, std::integral_constant<int, 0xa>{});   // row_bcast:15
+    v = step(v, std::integral_constant<int, 0x143>{}, std::integral_constant<int, 0xc>{});   // row_bcast:31
+    return v;
+}
+
 __device__ __forceinline__ long uniform(long v) {
     // the value is the same in every lane: keep it in scalar registers
     const int lo = __builtin_amdgcn_readfirstlane((int)(v & 0xffffffffL));
@@ -137,12 +155,16 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
             T l0, l1[3], l2[9];
             float en[8], rh[3];
         };
+        const unsigned lane_off = (unsigned)cc;   // rows are addressed as (uniform base) + 32-bit lane offset
         auto fetch = [&](EdgeOps& o, long e, long j) {
-            o.l0 = La[j * chan + cc];
+            const T* a = La + j * chan;
+            const T* v = Lv + j * 3 * chan;
+            const T* d = Ld + j * 9 * chan;
+            o.l0 = a[lane_off];
 #pragma unroll
-            for (int t = 0; t < 3; t++) o.l1[t] = Lv[(j * 3 + t) * chan + cc];
+            for (int t = 0; t < 3; t++) o.l1[t] = (v + t * chan)[lane_off];
 #pragma unroll
-            for (int k = 0; k < 9; k++) o.l2[k] = Ld[(j * 9 + k) * chan + cc];
+            for (int k = 0; k < 9; k++) o.l2[k] = (d + k * chan)[lane_off];
 #pragma unroll
             for (int m = 0; m < 8; m++) o.en[m] = enc[8 * e + m];
 #pragma unroll
@@ -192,16 +214,16 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
             const float pd1 = phi * dot1;
 
             if (active) {
-                T* p = P0 + (e * 3) * chan + c;
-                p[0] = (T)pl0;              // 000
-                p[chan] = (T)pd1;           // 110
-                p[2 * chan] = (T)(phi * quad);  // 220
+                T* p = P0 + (e * 3) * chan;
+                p[lane_off] = (T)pl0;                       // 000
+                (p + chan)[lane_off] = (T)pd1;              // 110
+                (p + 2 * chan)[lane_off] = (T)(phi * quad); // 220
             }
             if (edge_max) {
                 // largest |P0| entry of this (edge, 64-channel chunk): a row bound for the per-edge GEMM
                 float mx = fmaxf(fmaxf(fabsf(pl0), fabsf(pd1)), fabsf(phi * quad));
-                for (int d = 1; d < kWave; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
-                if (lane == 0) edge_max[e * chunks + (item - k_node * chunks)] = mx;
+                mx = wave_max_nonneg_last_lane(active ? mx : 0.f);
+                if (lane == kWave - 1) edge_max[e * chunks + (item - k_node * chunks)] = mx;
             }
             // vector sums, label order 011, 101, 121, 211, 111
 #pragma unroll
@@ -231,10 +253,12 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
             }
         }
         if (active) {
+            T* o1 = S1 + node * 15 * chan;
+            T* o2 = S2 + node * 45 * chan;
 #pragma unroll
-            for (int k = 0; k < 15; k++) S1[(node * 15 + k) * chan + c] = (T)s1[k];
+            for (int k = 0; k < 15; k++) (o1 + k * chan)[lane_off] = (T)s1[k];
 #pragma unroll
-            for (int k = 0; k < 45; k++) S2[(node * 45 + k) * chan + c] = (T)s2[k];
+            for (int k = 0; k < 45; k++) (o2 + k * chan)[lane_off] = (T)s2[k];
         }
         if (node_max) {
             // largest |sum| of this (node, 64-channel chunk): a row bound for the GEMMs that read S1 / S2
@@ -243,8 +267,8 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
             for (int k = 0; k < 15; k++) mx = fmaxf(mx, fabsf(s1[k]));
 #pragma unroll
             for (int k = 0; k < 45; k++) mx = fmaxf(mx, fabsf(s2[k]));
-            for (int d = 1; d < kWave; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
-            if (lane == 0) node_max[node * chunks + (item - k_node * chunks)] = mx;
+            mx = wave_max_nonneg_last_lane(active ? mx : 0.f);
+            if (lane == kWave - 1) node_max[node * chunks + (item - k_node * chunks)] = mx;
         }
     }
 }
