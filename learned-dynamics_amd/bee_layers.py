@@ -184,6 +184,31 @@ class MLP(nn.Module):
         return out.reshape(*lead, out.shape[-1])
 
 
+    def summed_over_rows(self, x, row_ptr, n_out, plus_identity=False, bound=None, scale=1.0):
+        """scale * (sum over the rows of each CSR segment of forward(x, plus_identity)), x (rows, d) ->
+        (n_out, d).  Only the first two layers are nonlinear: the direct linear and the last layer commute
+        with the sum, so they run on the n_out summed rows instead of on every row:
+            sum_e mlp(x_e) = (W_direct [+ I]) sum_e x_e + W_last sum_e h_e + (rows in the segment) b_last
+        with h = act(W_2 act(W_1 x + b_1) + b_2)."""
+        Wd = self.lin_direct.weight
+        if plus_identity:
+            Wd = _derived(self, "direct_plus_identity", (Wd,),
+                          lambda: Wd + torch.eye(Wd.shape[0], device=Wd.device, dtype=Wd.dtype))
+        L = self.layers
+        if bound is None and ops.get_linear_mode() == ops.LINEAR_F16X2:
+            bound = ops.row_absmax(x)
+        h, b1 = _linear(x, L[0].weight, L[0].bias, ops.ACT_LEAKY, bound)
+        h, _ = _linear(h, L[2].weight, L[2].bias, ops.ACT_LEAKY, b1)
+        s_x = ops.segment_sum_csr(x, row_ptr, n_out)
+        s_h = ops.segment_sum_csr(h, row_ptr, n_out)
+        del h
+        out = ops.tensor_linear_fwd(0, Wd, s_x)
+        ops.tensor_linear_fwd(0, L[4].weight, s_h, out=out, accumulate=True)
+        count = (row_ptr[1:] - row_ptr[:-1]).to(out.dtype)[:, None]
+        out = torch.addcmul(out, count, L[4].bias[None, :])
+        return out.mul_(scale) if scale != 1.0 else out
+
+
 class Messages(nn.Module):
     """archs/diffuser_atoms15.py:227-253"""
 
@@ -221,8 +246,7 @@ class Messages(nn.Module):
         P0 = P0.reshape(E, 3 * chan)
         bound = emax if ops.get_linear_mode() == ops.LINEAR_F16X2 else None     # row maxima of P0 from the edge kernel
         psi_a, bound = _linear(P0, self._cat_Y(LABELS_0), None, ops.ACT_NONE, bound)
-        psi_a = self.mlp_a(psi_a, plus_identity=True, bound=bound)
-        B_a = ops.segment_sum_csr(psi_a, graph.row_ptr, rows).mul_(0.1)
+        B_a = self.mlp_a.summed_over_rows(psi_a, graph.row_ptr, rows, plus_identity=True, bound=bound, scale=0.1)
         # vector and rank-2 channels: output linears after the edge sum, on node rows
         B_v = ops.tensor_linear_fwd(1, self._cat_Y(LABELS_1, 0.1), S1.reshape(rows, 3, 5 * chan), x_layout=C,
                                     row_bound=nmax, rows_per_bound=3)

@@ -61,6 +61,25 @@ def mlp_forward(mlp, x, plus_identity=False):
     return out.to(torch.bfloat16)
 
 
+def mlp_summed_over_rows(mlp, x, row_ptr, n_out, plus_identity=False, scale=1.0):
+    """scale * (sum over each CSR segment of mlp_forward(mlp, x, plus_identity)) as bf16 (n_out, d).  The
+    direct linear and the last layer are linear in their inputs, so they are applied to the summed rows
+    (bee_layers.MLP.summed_over_rows); the sums themselves are stored in bf16 like every other feature."""
+    Wd = mlp.lin_direct.weight
+    if plus_identity:
+        Wd = Wd + torch.eye(Wd.shape[0], device=Wd.device, dtype=Wd.dtype)
+    Ls = mlp.layers
+    h = ops.tensor_linear_bf16(Ls[0].weight, x, bias=Ls[0].bias, act=ops.ACT_LEAKY)
+    h = ops.tensor_linear_bf16(Ls[2].weight, h, bias=Ls[2].bias, act=ops.ACT_LEAKY)
+    s_x = ops.segment_sum_csr_bf16(x, row_ptr, n_out)
+    s_h = ops.segment_sum_csr_bf16(h, row_ptr, n_out)
+    del h
+    out = ops.tensor_linear_bf16(Wd, s_x, out_dtype=torch.float32)
+    ops.tensor_linear_bf16(Ls[4].weight, s_h, out=out, accumulate=True)
+    count = (row_ptr[1:] - row_ptr[:-1]).to(out.dtype)[:, None]
+    return torch.addcmul(out, count, Ls[4].bias[None, :]).mul_(scale).to(torch.bfloat16)
+
+
 def messages_forward(mod: Messages, graph: Graph, r_ij, s_a, s_v, s_d, node_order="cell"):
     """Messages.forward (archs/diffuser_atoms15.py:238-253) on storage tensors; returns the three
     0.1 * (sum over edges) increments in storage layout."""
@@ -73,8 +92,7 @@ def messages_forward(mod: Messages, graph: Graph, r_ij, s_a, s_v, s_d, node_orde
                                       mod.lin_enc.bias, node_order=node_order)
     E, chan = P0.shape[0], P0.shape[2]
     psi_a = ops.tensor_linear_bf16(_cat_Y(mod, LABELS_0), P0.reshape(E, 3 * chan))
-    psi_a = mlp_forward(mod.mlp_a, psi_a, plus_identity=True)
-    B_a = ops.segment_sum_csr_bf16(psi_a, graph.row_ptr, rows, 0.1)
+    B_a = mlp_summed_over_rows(mod.mlp_a, psi_a, graph.row_ptr, rows, plus_identity=True, scale=0.1)
     B_v = _lin(_cat_Y(mod, LABELS_1, 0.1), S1.reshape(rows, 3, 5 * chan), 3)
     B_d = _lin(_cat_Y(mod, LABELS_2, 0.1), S2.reshape(rows, 9, 5 * chan), 9)
     return B_a, B_v, B_d

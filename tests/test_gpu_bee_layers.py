@@ -205,3 +205,40 @@ def test_denoiser_forward_matches_oracle_composition(pkg):
         x_a, x_v, x_d = x_a + d[0], x_v + d[1], x_d + d[2]
     v_ref = (1. - (t - s).double()[:, None, None]) * OP.tensor_linear(1, dd(model.readout.W), x_v).squeeze(-2)
     _close(v, v_ref, rtol=1e-4, atol_scale=2e-5)   # 2 blocks deep: fp32 rounding compounds through the group norms
+
+
+@pytest.mark.parametrize("plus_identity", [False, True])
+def test_mlp_summed_over_rows_equals_sum_of_rows(pkg, plus_identity):
+    """MLP.summed_over_rows applies the direct linear and the last layer after the segment sum: the result
+    must equal the segment sum of the per-row MLP (archs/diffuser_atoms15.py:98-110, 244-246) up to the
+    order of fp32 additions, also for empty segments and with the bias of the last layer counted once per
+    row of the segment."""
+    bee = importlib.import_module("learned-dynamics_amd.bee_layers")
+    ops = importlib.import_module("learned-dynamics_amd.ops")
+    torch.manual_seed(5)
+    d, N = 64, 300
+    mlp = bee.MLP(d).cuda()
+    with torch.no_grad():
+        mlp.layers[4].bias.normal_()                      # make the bias term visible
+    deg = torch.randint(0, 40, (N,))
+    deg[::7] = 0
+    src = torch.repeat_interleave(torch.arange(N), deg)
+    E = int(src.numel())
+    x = torch.randn(E, d).cuda()
+    row_ptr = ops.segment_row_ptr(src.int().cuda(), N)
+    with torch.no_grad():
+        got = mlp.summed_over_rows(x, row_ptr, N, plus_identity=plus_identity, scale=0.1)
+        per_row = mlp(x, plus_identity=plus_identity)
+        # float64 reference of the same thing from plain torch modules
+        xd = x.double().cpu()
+        L = mlp.layers
+        f = torch.nn.functional
+        h = f.leaky_relu(f.linear(xd, L[0].weight.double().cpu(), L[0].bias.double().cpu()), 0.1)
+        h = f.leaky_relu(f.linear(h, L[2].weight.double().cpu(), L[2].bias.double().cpu()), 0.1)
+        y = f.linear(h, L[4].weight.double().cpu(), L[4].bias.double().cpu()) + f.linear(xd, mlp.lin_direct.weight.double().cpu())
+        if plus_identity:
+            y = y + xd
+        ref = 0.1 * torch.zeros(N, d, dtype=torch.float64).index_add_(0, src, y)
+    torch.testing.assert_close(per_row.cpu().double(), y, rtol=1e-5, atol=2e-6 * float(y.abs().max()))
+    torch.testing.assert_close(got.cpu().double(), ref, rtol=1e-5, atol=3e-6 * float(ref.abs().max()))
+    assert not bool(got[deg.cuda() == 0].any())
