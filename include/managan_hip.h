@@ -298,6 +298,21 @@ int mg_painn_filter_message(const void* packed_W3, const float* bias3, const flo
                             long n_nodes, long n_edges, int n, float epsilon, const float* res_a,
                             const float* res_v, void* workspace, float* out_a, float* out_v, mg_stream_t stream);
 
+/* A per-edge nn.Linear followed by the sum over the edges of each node, in one kernel: the pattern
+ * `edges_reduce_src(graph, mlp(...))` of archs/diffuser_atoms15.py:244-246 (managan/graph_layers.py:54-59) for a
+ * layer of the MLP whose output is only needed summed.
+ *   out[s] = scale * sum_{rows r with seg[r] == s} act(bias + W x[r]),   out (n_out, dim_out)
+ * x (rows, dim_in) with rows sorted by seg (ascending; row_ptr is the CSR form of seg, n_out + 1 entries);
+ * packed_W / x_rowmax as for mg_tensor_linear_f16x2 (bounds per row, stride 0 = one shared row of parts);
+ * y (rows, dim_out) also receives the per-row values when it is not NULL.  dim_out % 256 == 0, dim_in % 32 == 0
+ * and >= 64.  workspace: mg_tensor_linear_f16x2_rowsum_workspace_bytes(rows, dim_out) bytes, 16-byte aligned.
+ * Sums run in row order within blocks of 32 rows, then in block order (no atomics). */
+int mg_tensor_linear_f16x2_rowsum_workspace_bytes(long rows, int dim_out, size_t* bytes);
+int mg_tensor_linear_f16x2_rowsum(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts,
+                                  long x_rowmax_stride, long rows, int dim_in, int dim_out, const float* bias, int act,
+                                  const int* row_ptr, const int* seg, long n_out, float scale, void* workspace,
+                                  float* y, float* out, mg_stream_t stream);
+
 /* Update.forward (archs/meanflow_painn8.py:63-75), elementwise parts around its GEMMs.
  * lrv (rows, 3n, 3) = [lin_l | lin_r | lin_v] applied to x_v (one stacked tensor_linear).
  *   pre:  ip[r,c] = sum_x l[c,x] r[c,x];  cat[r] = [x_a[r] | |r[c]|]  (rows, 2n), the MLP input

@@ -184,12 +184,14 @@ class MLP(nn.Module):
         return out.reshape(*lead, out.shape[-1])
 
 
-    def summed_over_rows(self, x, row_ptr, n_out, plus_identity=False, bound=None, scale=1.0):
+    def summed_over_rows(self, x, row_ptr, n_out, plus_identity=False, bound=None, scale=1.0, seg=None, s_x=None):
         """scale * (sum over the rows of each CSR segment of forward(x, plus_identity)), x (rows, d) ->
         (n_out, d).  Only the first two layers are nonlinear: the direct linear and the last layer commute
         with the sum, so they run on the n_out summed rows instead of on every row:
             sum_e mlp(x_e) = (W_direct [+ I]) sum_e x_e + W_last sum_e h_e + (rows in the segment) b_last
-        with h = act(W_2 act(W_1 x + b_1) + b_2)."""
+        with h = act(W_2 act(W_1 x + b_1) + b_2).  seg (rows,) int32: the segment of every row; with it the
+        second layer sums its output rows in its own epilogue and h is never stored.  s_x: sum_e x_e if the
+        caller already has it."""
         Wd = self.lin_direct.weight
         if plus_identity:
             Wd = _derived(self, "direct_plus_identity", (Wd,),
@@ -198,10 +200,16 @@ class MLP(nn.Module):
         if bound is None and ops.get_linear_mode() == ops.LINEAR_F16X2:
             bound = ops.row_absmax(x)
         h, b1 = _linear(x, L[0].weight, L[0].bias, ops.ACT_LEAKY, bound)
-        h, _ = _linear(h, L[2].weight, L[2].bias, ops.ACT_LEAKY, b1)
-        s_x = ops.segment_sum_csr(x, row_ptr, n_out)
-        s_h = ops.segment_sum_csr(h, row_ptr, n_out)
+        if (seg is not None and b1 is not None
+                and ops.f16x2_rowsum_supported(h.shape[0], L[2].in_features, L[2].out_features, h)):
+            s_h, _ = ops.tensor_linear_f16x2_rowsum(L[2].weight, h, b1, row_ptr, seg, n_out, bias=L[2].bias,
+                                                    act=ops.ACT_LEAKY)
+        else:
+            h, _ = _linear(h, L[2].weight, L[2].bias, ops.ACT_LEAKY, b1)
+            s_h = ops.segment_sum_csr(h, row_ptr, n_out)
         del h
+        if s_x is None:
+            s_x = ops.segment_sum_csr(x, row_ptr, n_out)
         out = ops.tensor_linear_fwd(0, Wd, s_x)
         ops.tensor_linear_fwd(0, L[4].weight, s_h, out=out, accumulate=True)
         count = (row_ptr[1:] - row_ptr[:-1]).to(out.dtype)[:, None]
@@ -245,8 +253,16 @@ class Messages(nn.Module):
         # scalar channel: per-edge linear + MLP, then the edge sum
         P0 = P0.reshape(E, 3 * chan)
         bound = emax if ops.get_linear_mode() == ops.LINEAR_F16X2 else None     # row maxima of P0 from the edge kernel
-        psi_a, bound = _linear(P0, self._cat_Y(LABELS_0), None, ops.ACT_NONE, bound)
-        B_a = self.mlp_a.summed_over_rows(psi_a, graph.row_ptr, rows, plus_identity=True, bound=bound, scale=0.1)
+        Y0 = self._cat_Y(LABELS_0)
+        if bound is not None and ops.f16x2_rowsum_supported(E, 3 * chan, Y0.shape[0], P0):
+            # psi_a and its sum over the edges of each node from one kernel
+            s_psi, psi_a = ops.tensor_linear_f16x2_rowsum(Y0, P0, bound, graph.row_ptr, graph.src32, rows, want_rows=True)
+            bound = ops.linear_out_bound(Y0, None, bound)
+        else:
+            psi_a, bound = _linear(P0, Y0, None, ops.ACT_NONE, bound)
+            s_psi = None
+        B_a = self.mlp_a.summed_over_rows(psi_a, graph.row_ptr, rows, plus_identity=True, bound=bound, scale=0.1,
+                                          seg=graph.src32, s_x=s_psi)
         # vector and rank-2 channels: output linears after the edge sum, on node rows
         B_v = ops.tensor_linear_fwd(1, self._cat_Y(LABELS_1, 0.1), S1.reshape(rows, 3, 5 * chan), x_layout=C,
                                     row_bound=nmax, rows_per_bound=3)

@@ -31,61 +31,31 @@ constexpr int kFNI = kFTN / 32;
 
 __device__ __forceinline__ float4 ldf4(const float* p) { return *reinterpret_cast<const float4*>(p); }
 
-__global__ void __launch_bounds__(64 * kFW)
-painn_filter_message_kernel(const _Float16* __restrict__ Wp, const float* __restrict__ w_inv,
-                            const float* __restrict__ bias, const float* __restrict__ X,
-                            const float* __restrict__ xmax, int xmax_parts, long xmax_stride, long R, int I,
-                            const int* __restrict__ src, const int* __restrict__ dst, const float* __restrict__ r_ij,
-                            const float* __restrict__ actv, const float* __restrict__ x_v, int n, float epsilon,
-                            const float* __restrict__ res_a, const float* __restrict__ res_v,
-                            float* __restrict__ slots, long n_blocks, float* __restrict__ out_a,
-                            float* __restrict__ out_v, int tiles_n, long tiles_total) {
-    constexpr int THREADS = 64 * kFW;
-    constexpr int kPlaneW = kFTN * kRowW, kBufW = 2 * kPlaneW;
-    constexpr int kPieces = 8 * kFTN;
-    constexpr int kPer = kPieces / THREADS;                  // 4
-    constexpr int kSlice = 2 * kBufW / kFW / 4;              // floats of LDS per wave after the main loop
-    constexpr int kRed = 68;                                 // floats per row of a slice: 64 + 4 (spreads the 16-byte writes over the banks)
-    static_assert(kSlice >= 32 * kRed, "a reduction pass needs 32 rows x 64 columns per wave");
-    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kBufW];
-    __shared__ __attribute__((aligned(16))) float wb[2 * kFTN];   // the tile's 1 / weight scale, then its bias
+template <int ACT>
+__device__ __forceinline__ float activate_c(float v) {
+    // 1: SiLU through the hardware exp2 and reciprocal (about 1 ulp each); 2: LeakyReLU(0.1)
+    if constexpr (ACT == 1) return v * __builtin_amdgcn_rcpf(1.0f + __expf(-v));
+    if constexpr (ACT == 2) return v > 0.f ? v : 0.1f * v;
+    return v;
+}
 
-    const long bid = blockIdx.x;
-    const long per_xcd = (tiles_total + 7) / 8;
-    const long logical = (bid % 8) * per_xcd + bid / 8;
-    if (logical >= tiles_total) return;
-    const long tile_m = logical / tiles_n;
-    const int tile_n = (int)(logical - tile_m * tiles_n);
+constexpr int kFThreads = 64 * kFW;
+constexpr int kFPlaneW = kFTN * kRowW, kFBufW = 2 * kFPlaneW;   // bytes of one W plane / of both planes of a chunk
+constexpr int kFSlice = 2 * kFBufW / kFW / 4;                    // floats of LDS per wave once the main loop is over
+constexpr int kFRed = 68;                                        // floats per row of a slice: 64 + 4 (spreads 16-byte writes over the banks)
+static_assert(kFSlice >= 32 * kFRed, "a reduction pass needs 32 rows x 64 columns per wave");
 
+// acc[ni][q] += sum_k W[n0 + 32 ni + i][k] x[row][k] for the wave's 32 rows (row = lane % 32) and the tile's 256
+// columns, i = 8 (q / 4) + 4 (lane / 32) + q % 4: the split-fp16 row-streaming main loop with W as the first
+// matrix operand.  xrow: this lane's row of x, offset by 16 (lane / 32); lds: 2 * kFBufW bytes; all waves of
+// the workgroup call it together, and the W buffers are free again when it returns.
+__device__ __forceinline__ void wfirst_gemm_tile(floatx16 (&acc)[kFNI], const _Float16* __restrict__ Wp,
+                                                 long plane_elems, int n0, const float* __restrict__ xrow, int I,
+                                                 float sx, unsigned char* lds) {
+    constexpr int THREADS = kFThreads, kPlaneW = kFPlaneW, kBufW = kFBufW;
+    constexpr int kPer = 8 * kFTN / THREADS;                 // 16-byte pieces of W per thread and chunk
     const int tid = threadIdx.x;
-    const int lane = tid & 63, wave = tid >> 6;
-    const int m = lane & 31, g = lane >> 5;
-    const long r0 = tile_m * kFTM;
-    const int n0 = tile_n * kFTN;
-    const long plane_elems = (long)tiles_n * kFTN * I;
-
-    floatx16 acc[kFNI];
-#pragma unroll
-    for (int ni = 0; ni < kFNI; ni++)
-#pragma unroll
-        for (int q = 0; q < 16; q++) acc[ni][q] = 0.f;
-
-    const long block = r0 / 32 + wave;                       // this wave's block of 32 edges
-    const long my_row = block * 32 + m;
-    const long ld_row = my_row < R ? my_row : R - 1;
-    const float* xrow = X + ld_row * I + 16 * g;
-    float sx, isx;
-    {
-        float amax = 0.f;
-        const float* xm = xmax + ld_row * xmax_stride;
-        for (int p = 0; p < xmax_parts; p++) amax = fmaxf(amax, xm[p]);
-        sx = pow2_scale(amax, &isx);
-    }
-    // the edge this lane owns in the epilogue
-    const int my_src = src[ld_row];
-    const long my_j = dst[ld_row];
-    float ux = r_ij[3 * ld_row], uy = r_ij[3 * ld_row + 1], uz = r_ij[3 * ld_row + 2];
-
+    const int m = tid & 31, g = (tid >> 5) & 1;
     const _Float16* wsrc[kPer];
     int wdst[kPer];
 #pragma unroll
@@ -94,10 +64,6 @@ painn_filter_message_kernel(const _Float16* __restrict__ Wp, const float* __rest
         const int plane = q / (4 * kFTN), row = (q % (4 * kFTN)) >> 2, piece = q & 3;
         wsrc[j] = Wp + plane * plane_elems + (long)(n0 + row) * I + 8 * piece;
         wdst[j] = plane * kPlaneW + row * kRowW + piece * 16;
-    }
-    if (tid < kFTN) {
-        wb[tid] = w_inv[n0 + tid];
-        wb[kFTN + tid] = bias[n0 + tid];
     }
     const int k_last = I - kCK;
 
@@ -168,6 +134,62 @@ painn_filter_message_kernel(const _Float16* __restrict__ Wp, const float* __rest
         load_a(a1, k0 + 3 * kCK);
         __syncthreads();
     }
+}
+
+__global__ void __launch_bounds__(64 * kFW)
+painn_filter_message_kernel(const _Float16* __restrict__ Wp, const float* __restrict__ w_inv,
+                            const float* __restrict__ bias, const float* __restrict__ X,
+                            const float* __restrict__ xmax, int xmax_parts, long xmax_stride, long R, int I,
+                            const int* __restrict__ src, const int* __restrict__ dst, const float* __restrict__ r_ij,
+                            const float* __restrict__ actv, const float* __restrict__ x_v, int n, float epsilon,
+                            const float* __restrict__ res_a, const float* __restrict__ res_v,
+                            float* __restrict__ slots, long n_blocks, float* __restrict__ out_a,
+                            float* __restrict__ out_v, int tiles_n, long tiles_total) {
+    constexpr int kSlice = kFSlice, kRed = kFRed;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kFBufW];
+    __shared__ __attribute__((aligned(16))) float wb[2 * kFTN];   // the tile's 1 / weight scale, then its bias
+
+    const long bid = blockIdx.x;
+    const long per_xcd = (tiles_total + 7) / 8;
+    const long logical = (bid % 8) * per_xcd + bid / 8;
+    if (logical >= tiles_total) return;
+    const long tile_m = logical / tiles_n;
+    const int tile_n = (int)(logical - tile_m * tiles_n);
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int m = lane & 31, g = lane >> 5;
+    const long r0 = tile_m * kFTM;
+    const int n0 = tile_n * kFTN;
+    const long plane_elems = (long)tiles_n * kFTN * I;
+
+    floatx16 acc[kFNI];
+#pragma unroll
+    for (int ni = 0; ni < kFNI; ni++)
+#pragma unroll
+        for (int q = 0; q < 16; q++) acc[ni][q] = 0.f;
+
+    const long block = r0 / 32 + wave;                       // this wave's block of 32 edges
+    const long my_row = block * 32 + m;
+    const long ld_row = my_row < R ? my_row : R - 1;
+    const float* xrow = X + ld_row * I + 16 * g;
+    float sx, isx;
+    {
+        float amax = 0.f;
+        const float* xm = xmax + ld_row * xmax_stride;
+        for (int p = 0; p < xmax_parts; p++) amax = fmaxf(amax, xm[p]);
+        sx = pow2_scale(amax, &isx);
+    }
+    // the edge this lane owns in the epilogue
+    const int my_src = src[ld_row];
+    const long my_j = dst[ld_row];
+    float ux = r_ij[3 * ld_row], uy = r_ij[3 * ld_row + 1], uz = r_ij[3 * ld_row + 2];
+
+    if (tid < kFTN) {
+        wb[tid] = w_inv[n0 + tid];
+        wb[kFTN + tid] = bias[n0 + tid];
+    }
+    wfirst_gemm_tile(acc, Wp, plane_elems, n0, xrow, I, sx, lds);
     // every wave is past its last read of the W buffers: LDS is now eight private slices
 
     const bool valid = my_row < R;
@@ -304,6 +326,162 @@ painn_filter_message_kernel(const _Float16* __restrict__ Wp, const float* __rest
     }
 }
 
+// y = act(x W^T + bias) for rows sorted by segment (seg[row] ascending), reduced over the rows of each segment
+// in the epilogue: out[s] = scale * sum_{rows of s} y[row].  Same tile, same slots A / B per block of 32 rows
+// and same finishing pass as the message kernel above; y itself is written only when STORE_Y is set
+// (coalesced, from the LDS slice the reduction reads anyway).
+template <int ACT, bool STORE_Y>
+__global__ void __launch_bounds__(64 * kFW)
+linear_rowsum_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restrict__ w_inv,
+                           const float* __restrict__ bias, const float* __restrict__ X,
+                           const float* __restrict__ xmax, int xmax_parts, long xmax_stride, long R, int I, int O,
+                           const int* __restrict__ seg, float* __restrict__ slots, long n_blocks, float scale,
+                           float* __restrict__ Y, float* __restrict__ out, int tiles_n, long tiles_total) {
+    constexpr int kSlice = kFSlice, kRed = kFRed;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kFBufW];
+    __shared__ __attribute__((aligned(16))) float wb[2 * kFTN];   // the tile's 1 / weight scale, then its bias
+
+    const long bid = blockIdx.x;
+    const long per_xcd = (tiles_total + 7) / 8;
+    const long logical = (bid % 8) * per_xcd + bid / 8;
+    if (logical >= tiles_total) return;
+    const long tile_m = logical / tiles_n;
+    const int tile_n = (int)(logical - tile_m * tiles_n);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int m = lane & 31, g = lane >> 5;
+    const int n0 = tile_n * kFTN;
+    const long plane_elems = (long)O * I;
+
+    floatx16 acc[kFNI];
+#pragma unroll
+    for (int ni = 0; ni < kFNI; ni++)
+#pragma unroll
+        for (int q = 0; q < 16; q++) acc[ni][q] = 0.f;
+
+    const long block = tile_m * kFW + wave;                  // this wave's block of 32 rows
+    const long my_row = block * 32 + m;
+    const long ld_row = my_row < R ? my_row : R - 1;
+    const float* xrow = X + ld_row * I + 16 * g;
+    float sx, isx;
+    {
+        float amax = 0.f;
+        const float* xm = xmax + ld_row * xmax_stride;
+        for (int p = 0; p < xmax_parts; p++) amax = fmaxf(amax, xm[p]);
+        sx = pow2_scale(amax, &isx);
+    }
+    const int my_seg = seg[ld_row];
+    if (tid < kFTN) {
+        wb[tid] = w_inv[n0 + tid];
+        wb[kFTN + tid] = bias ? bias[n0 + tid] : 0.f;
+    }
+    wfirst_gemm_tile(acc, Wp, plane_elems, n0, xrow, I, sx, lds);
+
+    const float keep = my_row < R ? 1.f : 0.f;               // rows past the end add nothing
+    const long rows_left = R - block * 32;
+    const int nv = rows_left >= 32 ? 32 : (rows_left > 0 ? (int)rows_left : 0);
+    const int prev_seg = __shfl_up(my_seg, 1);
+    const unsigned starts = (unsigned)__ballot(g == 0 && (m == 0 || my_seg != prev_seg));
+    const int runs = __popc(starts);
+    const int second = runs >= 2 ? __ffs(starts & ~1u) - 1 : 32;
+    float* slice = reinterpret_cast<float*>(lds) + wave * kSlice;
+    float* slot_a = slots + block * O;
+    float* slot_b = slots + (n_blocks + block) * O;
+
+#pragma unroll
+    for (int pass = 0; pass < 4; pass++) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int ni = 2 * pass + h;
+#pragma unroll
+            for (int qq = 0; qq < 4; qq++) {
+                const int cl = 32 * ni + 8 * qq + 4 * g;      // column in the tile
+                const float4 iw = *reinterpret_cast<const float4*>(wb + cl);
+                const float4 bv = *reinterpret_cast<const float4*>(wb + kFTN + cl);
+                float4 v;
+                v.x = keep * activate_c<ACT>(acc[ni][4 * qq + 0] * isx * iw.x + bv.x);
+                v.y = keep * activate_c<ACT>(acc[ni][4 * qq + 1] * isx * iw.y + bv.y);
+                v.z = keep * activate_c<ACT>(acc[ni][4 * qq + 2] * isx * iw.z + bv.z);
+                v.w = keep * activate_c<ACT>(acc[ni][4 * qq + 3] * isx * iw.w + bv.w);
+                *reinterpret_cast<float4*>(slice + m * kRed + 32 * h + 8 * qq + 4 * g) = v;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int col = n0 + 64 * pass + lane;                // lane = output column of this pass
+        auto flush = [&](float sum, int run_start, int r) {
+            if (run_start == 0) {
+                slot_a[col] = sum;
+            } else if (r == 31) {
+                slot_b[col] = sum;
+            } else {
+                const long s_id = __shfl(my_seg, r);          // a whole segment inside the block
+                out[s_id * O + col] = scale * sum;
+            }
+        };
+        if (nv > 0) {
+            float val[32];
+#pragma unroll
+            for (int r = 0; r < 32; r++) val[r] = slice[r * kRed + lane];
+            if constexpr (STORE_Y) {
+                float* yp = Y + block * 32 * O + col;
+#pragma unroll
+                for (int r = 0; r < 32; r++)
+                    if (r < nv) yp[(long)r * O] = val[r];
+            }
+            if (runs <= 2) {
+                float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+                for (int r = 0; r < 32; r++) {
+                    s0 += r < second ? val[r] : 0.f;
+                    s1 += r < second ? 0.f : val[r];
+                }
+                flush(s0, 0, second - 1);
+                if (runs == 2) flush(s1, second, nv - 1);
+            } else {
+                float sum = 0.f;
+                int run_start = 0;
+                for (int r = 0; r < nv; r++) {
+                    sum += slice[r * kRed + lane];
+                    if ((r == nv - 1) || ((starts >> (r + 1)) & 1u)) {
+                        flush(sum, run_start, r);
+                        sum = 0.f;
+                        run_start = r + 1;
+                    }
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
+// out[s] = scale * (slots of the blocks the rows of segment s lie in, in block order); segments strictly inside
+// one block were written by the kernel above, empty segments get zero.  One thread per four columns.
+__global__ void __launch_bounds__(256)
+rowsum_finish_kernel(const int* __restrict__ row_ptr, long n_out, long n_blocks, int O, const float* __restrict__ slots,
+                     float scale, float* __restrict__ out) {
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const int quads = O / 4;
+    if (idx >= n_out * quads) return;
+    const long s_id = idx / quads;
+    const int x = (int)(idx - s_id * quads) * 4;
+    const long lo = row_ptr[s_id], hi = row_ptr[s_id + 1];
+    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (hi > lo) {
+        const long b_lo = lo / 32, b_hi = (hi - 1) / 32;
+        if (b_lo == b_hi && lo > 32 * b_lo && hi - 1 < 32 * b_lo + 31) return;   // written directly
+        for (long b = b_lo; b <= b_hi; b++) {
+            const float* slot = 32 * b >= lo ? slots + b * O : slots + (n_blocks + b) * O;
+            const float4 t = ldf4(slot + x);
+            s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
+        }
+    }
+    *reinterpret_cast<float4*>(out + s_id * O + x) = make_float4(scale * s.x, scale * s.y, scale * s.z, scale * s.w);
+}
+
 // out(node) = res(node) + the partial sums of the blocks its edges lie in, in block order.  Nodes whose
 // edges lie strictly inside one block were written by the kernel above and are skipped; nodes without
 // edges get the residual.  One thread per four consecutive floats of the node's 4n outputs.
@@ -384,6 +562,58 @@ int mg_painn_filter_message(const void* packed_W3, const float* bias3, const flo
     painn_message_finish_kernel<<<dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, s>>>(
         row_ptr, n_nodes, n_blocks, n, static_cast<const float*>(workspace), res_a, res_v, out_a, out_v);
     return check_launch("painn_message_finish_kernel");
+}
+
+int mg_tensor_linear_f16x2_rowsum_workspace_bytes(long rows, int dim_out, size_t* bytes) {
+    MG_REQUIRE(bytes != nullptr && rows >= 0 && dim_out >= 0, "mg_tensor_linear_f16x2_rowsum_workspace_bytes: bad argument");
+    *bytes = (size_t)(2L * (ceil_div(rows, 32) + 1) * dim_out) * sizeof(float);
+    return MG_OK;
+}
+
+int mg_tensor_linear_f16x2_rowsum(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts,
+                                  long x_rowmax_stride, long rows, int dim_in, int dim_out, const float* bias, int act,
+                                  const int* row_ptr, const int* seg, long n_out, float scale, void* workspace,
+                                  float* y, float* out, mg_stream_t stream) {
+    MG_REQUIRE(dim_out >= 256 && dim_out % 256 == 0, "mg_tensor_linear_f16x2_rowsum: dim_out must be a multiple of 256 (got %d)", dim_out);
+    MG_REQUIRE(dim_in >= 64 && dim_in % 32 == 0, "mg_tensor_linear_f16x2_rowsum: dim_in must be a multiple of 32, at least 64 (got %d)", dim_in);
+    MG_REQUIRE(rows >= 0 && n_out >= 0 && rows < (1L << 31) && n_out < (1L << 31), "mg_tensor_linear_f16x2_rowsum: bad size");
+    MG_REQUIRE(act >= 0 && act <= 2, "mg_tensor_linear_f16x2_rowsum: unknown activation %d", act);
+    MG_REQUIRE(x_rowmax_parts >= 1 && x_rowmax_parts <= 64, "mg_tensor_linear_f16x2_rowsum: 1..64 bound parts");
+    if (n_out == 0) return MG_OK;
+    MG_REQUIRE(packed_W && row_ptr && out && aligned16(packed_W) && aligned16(out) && (!bias || aligned16(bias)),
+               "mg_tensor_linear_f16x2_rowsum: null or unaligned operand");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const long n_blocks = ceil_div(rows, 32);
+    if (rows > 0) {
+        MG_REQUIRE(x && x_rowmax && seg && workspace && aligned16(x) && aligned16(workspace) && (!y || aligned16(y)),
+                   "mg_tensor_linear_f16x2_rowsum: null or unaligned row operand");
+        const int tiles_n = dim_out / kFTN;
+        const long tiles_total = ceil_div(rows, kFTM) * tiles_n;
+        const _Float16* planes = static_cast<const _Float16*>(packed_W);
+        const float* w_inv = reinterpret_cast<const float*>(planes + 2L * dim_out * dim_in);
+        const long grid = 8 * ceil_div(tiles_total, 8);
+        MG_REQUIRE(grid < (1L << 31), "mg_tensor_linear_f16x2_rowsum: too many tiles");
+        float* slots = static_cast<float*>(workspace);
+#define MG_ROWSUM_LAUNCH(A, S)                                                                                       \
+    linear_rowsum_f16x2_kernel<A, S><<<dim3((unsigned)grid), dim3(64 * kFW), 0, s>>>(                                \
+        planes, w_inv, bias, x, x_rowmax, x_rowmax_parts, x_rowmax_stride, rows, dim_in, dim_out, seg, slots, n_blocks, \
+        scale, y, out, tiles_n, tiles_total)
+        if (y) {
+            if (act == 1) MG_ROWSUM_LAUNCH(1, true);
+            else if (act == 2) MG_ROWSUM_LAUNCH(2, true);
+            else MG_ROWSUM_LAUNCH(0, true);
+        } else {
+            if (act == 1) MG_ROWSUM_LAUNCH(1, false);
+            else if (act == 2) MG_ROWSUM_LAUNCH(2, false);
+            else MG_ROWSUM_LAUNCH(0, false);
+        }
+#undef MG_ROWSUM_LAUNCH
+        if (int st = check_launch("linear_rowsum_f16x2_kernel")) return st;
+    }
+    const long threads = n_out * (dim_out / 4);
+    rowsum_finish_kernel<<<dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, s>>>(
+        row_ptr, n_out, n_blocks, dim_out, static_cast<const float*>(workspace), scale, out);
+    return check_launch("rowsum_finish_kernel");
 }
 
 }  // extern "C"

@@ -937,6 +937,45 @@ def painn_message(row_ptr, dst, r_ij, filt, actv, x_v, epsilon, res_a=None, res_
     return out_a, out_v
 
 
+def f16x2_rowsum_supported(rows, dim_in, dim_out, x):
+    """The GEMM whose epilogue sums the rows of each segment: 256-column tiles, and enough rows to fill the chip."""
+    return (get_linear_mode() == LINEAR_F16X2 and dim_out % 256 == 0 and dim_in % 32 == 0 and dim_in >= 64
+            and rows >= 4096 and x.data_ptr() % 16 == 0)
+
+
+def tensor_linear_f16x2_rowsum(W, x, x_bound, row_ptr, seg, n_out, bias=None, act=ACT_NONE, scale=1.0, want_rows=False):
+    """(out, y): out[s] = scale * sum over the rows r of segment s of act(bias + W x[r]) (n_out, dim_out); y is the
+    per-row result (rows, dim_out) when want_rows is set, else None.  Rows are sorted by segment: seg (rows,) int32
+    ascending, row_ptr its CSR form.  x_bound: (rows, parts) or (1, parts) upper bounds of the row maxima of |x|."""
+    for t, nm in ((W, "W"), (x, "x"), (x_bound, "x_bound")):
+        _check_input(t, nm)
+    for t, nm in ((row_ptr, "row_ptr"), (seg, "seg")):
+        _check_input(t, nm, torch.int32)
+    if x.dim() != 2 or W.dim() != 2 or x.size(1) != W.size(1):
+        raise RuntimeError("x must have shape (rows, dim_in) and W (dim_out, dim_in)")
+    rows, dim_in, dim_out = int(x.size(0)), int(W.size(1)), int(W.size(0))
+    if seg.numel() != rows or row_ptr.numel() != n_out + 1:
+        raise RuntimeError("seg must have one entry per row and row_ptr n_out + 1 entries")
+    if x_bound.dim() != 2 or x_bound.size(0) not in (1, rows) or not 1 <= x_bound.size(1) <= 64:
+        raise RuntimeError("x_bound must be (rows, parts) or (1, parts) with 1..64 parts")
+    if bias is not None:
+        _check_input(bias, "bias")
+        if bias.numel() != dim_out:
+            raise RuntimeError("bias must have dim_out elements")
+    dev = x.device
+    nbytes = ctypes.c_size_t(0)
+    L.check(_lib.mg_tensor_linear_f16x2_rowsum_workspace_bytes(rows, dim_out, ctypes.byref(nbytes)))
+    with torch.cuda.device(dev):
+        out = torch.empty(n_out, dim_out, dtype=torch.float32, device=dev)
+        y = torch.empty(rows, dim_out, dtype=torch.float32, device=dev) if want_rows else None
+        work = torch.empty(nbytes.value // 4, dtype=torch.float32, device=dev)
+        stride = 0 if x_bound.size(0) == 1 else int(x_bound.size(1))
+        L.check(_lib.mg_tensor_linear_f16x2_rowsum(
+            _p(packed_weight_f16x2(W)), _p(x), _p(x_bound), int(x_bound.size(1)), stride, rows, dim_in, dim_out,
+            _p(bias), int(act), _p(row_ptr), _p(seg), int(n_out), float(scale), _p(work), _p(y), _p(out), _stream()))
+    return out, y
+
+
 def painn_filter_message_supported(n, hidden, n_edges):
     """The fused filter + message kernel: channel blocks of 64, a hidden width the matrix path tiles, and
     enough edges to fill the chip with 256-edge tiles."""

@@ -208,3 +208,46 @@ def test_packed_weight_cache_tracks_in_place_updates(ops):
         torch.testing.assert_close(y2, 2 * y1, rtol=1e-5, atol=1e-5)
     finally:
         ops.set_linear_mode(prev)
+
+
+def _segment_lengths(kind, n, g):
+    if kind == "long":
+        return torch.randint(40, 140, (n,), generator=g)
+    if kind == "short":
+        return torch.randint(0, 9, (n,), generator=g)
+    if kind == "aligned":
+        return torch.tensor([32, 64, 1, 31, 32, 0, 0, 96, 33, 31] * (n // 10))
+    return torch.cat([torch.randint(0, 5, (n // 2,), generator=g), torch.randint(20, 300, (n - n // 2,), generator=g)])[
+        torch.randperm(n, generator=g)]
+
+
+@pytest.mark.parametrize("dim_in,dim_out,act,kind,want_rows", [(512, 512, 2, "long", False), (96, 256, 0, "short", True),
+                                                               (256, 256, 1, "aligned", True), (64, 768, 2, "mixed", False)])
+def test_linear_with_row_sums_in_the_epilogue(ops, dim_in, dim_out, act, kind, want_rows):
+    """out[s] = scale * sum over the rows of segment s of act(x W^T + b), against the plain GEMM followed by
+    the segment sum, and against float64; segments placed in every way relative to the kernel's 32-row blocks."""
+    g = torch.Generator().manual_seed(dim_in + dim_out)
+    n_seg = 300
+    lengths = _segment_lengths(kind, n_seg, g)
+    seg = torch.repeat_interleave(torch.arange(n_seg), lengths)
+    rows = int(seg.numel())
+    x = (torch.randn(rows, dim_in, generator=g) * (torch.rand(rows, 1, generator=g) * 3)).cuda()
+    W = (torch.randn(dim_out, dim_in, generator=g) / dim_in ** 0.5).cuda()
+    b = torch.randn(dim_out, generator=g).cuda()
+    row_ptr = ops.segment_row_ptr(seg.int().cuda(), n_seg)
+    bound = ops.row_absmax(x)
+    out, y = ops.tensor_linear_f16x2_rowsum(W, x, bound, row_ptr, seg.int().cuda(), n_seg, bias=b, act=act, scale=0.5,
+                                            want_rows=want_rows)
+    y_ref = ops.tensor_linear_f16x2(W, x, bound, bias=b, act=act)
+    if want_rows:
+        assert torch.equal(y, y_ref)          # the same accumulators through another epilogue
+    else:
+        assert y is None
+    two_step = 0.5 * ops.segment_sum_csr(y_ref, row_ptr, n_seg)
+    z = x.double().cpu() @ W.double().cpu().T + b.double().cpu()
+    z = torch.nn.functional.silu(z) if act == 1 else (torch.nn.functional.leaky_relu(z, 0.1) if act == 2 else z)
+    ref = 0.5 * torch.zeros(n_seg, dim_out, dtype=torch.float64).index_add_(0, seg, z)
+    scale = float(ref.abs().max())
+    torch.testing.assert_close(out, two_step, rtol=1e-5, atol=2e-6 * scale)
+    torch.testing.assert_close(out.cpu().double(), ref, rtol=1e-5, atol=3e-6 * scale)
+    assert not bool(out[(lengths == 0).cuda()].any())
