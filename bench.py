@@ -340,6 +340,26 @@ def chain_positions(torch, systems, atoms, box, seed, noise=1.0):
     return (pos + noise * torch.randn(systems, atoms, 3, generator=g)).contiguous()
 
 
+def single_system_latency(torch, model, dev, box, r0, atoms):
+    """One system of the denoiser workload: the 8 blocks on a prebuilt neighbour graph, run eagerly and replayed
+    from a captured HIP graph (the neighbour search stays outside the capture)."""
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    ro = importlib.import_module("learned-dynamics_amd.rollout")
+    with torch.no_grad():
+        one = [v[:1].contiguous() for v in dev]
+        g1, _ = gl.graph_setup(r0, box, one[3], neighbours_max=256, celllist_max=64)
+
+        def layers(s_, t_, x0_, x1_):
+            return model.forward_on_graph((s_, t_), x0_, x1_, one[4], g1, gl.edge_vectors(g1, x1_, box))
+        t_eager = event_time(torch, lambda: layers(*one[:4]), 10)
+        captured = ro.GraphedCall(layers, *one[:4])
+        t_graph = event_time(torch, lambda: captured(*one[:4]), 10)
+    return {"atoms": atoms, "edges": int(g1.src.numel()), "layers_eager_ms": t_eager * 1e3,
+            "layers_hip_graph_replay_ms": t_graph * 1e3,
+            "note": "8 blocks on a prebuilt neighbour graph, one system; the replay includes the copies into the "
+                    "capture's static inputs"}
+
+
 def bench_denoiser(torch, args, with_cpu=True):
     """BASELINE configs[3]: 8-block rank-0/1/2 denoiser forward, 32 systems x 2048 atoms."""
     den = importlib.import_module("learned-dynamics_amd.denoiser")
@@ -365,21 +385,7 @@ def bench_denoiser(torch, args, with_cpu=True):
         gl = importlib.import_module("learned-dynamics_amd.graph_layers")
         graph, _ = gl.graph_setup(r0, box, dev[3], neighbours_max=256, celllist_max=64)
         E = int(graph.src.numel())
-        # one system (2048 atoms): a forward pass is ~600 launches of a few microseconds each, so the host
-        # sets the pace; the same layers replayed from a captured HIP graph (neighbour search outside)
-        ro = importlib.import_module("learned-dynamics_amd.rollout")
-        one = [v[:1].contiguous() for v in dev]
-        g1, _ = gl.graph_setup(r0, box, one[3], neighbours_max=256, celllist_max=64)
-
-        def layers(s_, t_, x0_, x1_):
-            return model.forward_on_graph((s_, t_), x0_, x1_, one[4], g1, gl.edge_vectors(g1, x1_, box))
-        t_eager = event_time(torch, lambda: layers(*one[:4]), 10)
-        captured = ro.GraphedCall(layers, *one[:4])
-        t_graph = event_time(torch, lambda: captured(*one[:4]), 10)
-        single = {"atoms": N, "edges": int(g1.src.numel()), "layers_eager_ms": t_eager * 1e3,
-                  "layers_hip_graph_replay_ms": t_graph * 1e3,
-                  "note": "8 blocks on a prebuilt neighbour graph, one system; the replay includes the copies "
-                          "into the capture's static inputs"}
+    single = None if args.no_extras else single_system_latency(torch, model, dev, box, r0, N)
     out = {"metric": "denoiser forward atoms/sec", "value": B * N / sec, "unit": "atoms/s", "ms_per_step": sec * 1e3,
            "dtype": "f32",
            "config": {"workload": "BASELINE configs[3]: 8 x [Messages + SelfTensProds] rank-0/1/2 denoiser forward "

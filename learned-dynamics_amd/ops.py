@@ -538,6 +538,25 @@ def _packed(W, kind):
     return packed
 
 
+_padded_cache = {}
+
+
+def _zero_padded_columns(W, k_pad):
+    """W (dim_out, dim_in) with zero columns appended up to k_pad; cached per parameter object and version."""
+    if int(W.size(1)) == k_pad:
+        return W
+    key = (id(W), k_pad)
+    hit = _padded_cache.get(key)
+    if hit is not None and hit[0]() is W and hit[1] == W._version and hit[2] == W.data_ptr():
+        return hit[3]
+    with torch.no_grad():
+        Wp = torch.nn.functional.pad(W.detach(), (0, k_pad - int(W.size(1)))).contiguous()
+    if len(_padded_cache) > 256:
+        _padded_cache.clear()
+    _padded_cache[key] = (weakref.ref(W), W._version, W.data_ptr(), Wp)
+    return Wp
+
+
 def packed_weight(W):
     """bf16x3 planes of W for mg_tensor_linear_packed."""
     return _packed(W, "bf16x3")
@@ -711,7 +730,20 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
         wide = (plain_rows and dim_in % 32 == 0 and dim_in >= 64 and dim_out >= 64 and rows * T >= 1024
                 and x.data_ptr() % 16 == 0)
         out_comps = 1 if (inds == 0 or y_layout == LAYOUT_COMP_CHAN) else T
-        if (plain_rows and mode == LINEAR_F16X2 and f16x2_supported(rows * T, dim_in, dim_out, x)):
+        if (mode == LINEAR_F16X2 and inds > 0 and x_layout == LAYOUT_CHAN_COMP and y_layout == LAYOUT_COMP_CHAN
+                and rows * T >= 65536 and dim_out >= 64 and row_bound is None):
+            # (row, chan, comp) -> (row, comp, chan) rows (K zero-padded to a multiple of 32), then the plain-row
+            # matrix path: its component-major output is written at the full store rate, which the generic
+            # kernel's layout mapping is not
+            k_pad = (dim_in + 31) // 32 * 32
+            xt = x.reshape(rows, dim_in, T).transpose(1, 2)
+            xt = torch.nn.functional.pad(xt, (0, k_pad - dim_in)) if k_pad != dim_in else xt.contiguous()
+            x2 = xt.reshape(rows * T, k_pad)
+            Wp = _zero_padded_columns(W, k_pad)
+            L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(Wp)), _p(x2), _p(row_absmax(x2)), 1, 1, 1,
+                                                rows * T, k_pad, dim_out, _p(bias), int(act), int(bool(accumulate)),
+                                                1, _p(y), None, _stream()))
+        elif (plain_rows and mode == LINEAR_F16X2 and f16x2_supported(rows * T, dim_in, dim_out, x)):
             x2 = x.reshape(rows * T, dim_in)
             if row_bound is None:
                 row_bound, rows_per_bound = row_absmax(x2), 1

@@ -251,3 +251,24 @@ def test_linear_with_row_sums_in_the_epilogue(ops, dim_in, dim_out, act, kind, w
     torch.testing.assert_close(out, two_step, rtol=1e-5, atol=2e-6 * scale)
     torch.testing.assert_close(out.cpu().double(), ref, rtol=1e-5, atol=3e-6 * scale)
     assert not bool(out[(lengths == 0).cuda()].any())
+
+
+@pytest.mark.parametrize("inds,rows,dim_in,dim_out", [(2, 8000, 16, 64), (1, 22000, 40, 96), (1, 30000, 64, 256)])
+def test_component_major_output_from_reference_layout_at_many_rows(ops, inds, rows, dim_in, dim_out):
+    """x in the reference layout (rows, chan, 3..), y component-major (rows, 3^inds, chan_out): at many rows
+    the dispatcher transposes x and uses the plain-row matrix path (K zero-padded to a multiple of 32).
+    Against the einsum of extensions/tensor_ops/test.py:9-15 in float64, with accumulate."""
+    T = 3 ** inds
+    assert rows * T >= 65536
+    g = torch.Generator().manual_seed(rows)
+    x = torch.randn(rows, dim_in, *([3] * inds), generator=g).cuda()
+    W = (torch.randn(dim_out, dim_in, generator=g) / dim_in ** 0.5).cuda()
+    y = ops.tensor_linear_fwd(inds, W, x, y_layout=ops.LAYOUT_COMP_CHAN)
+    ref = torch.einsum("oi,bit->bto", W.double().cpu(), x.double().cpu().reshape(rows, dim_in, T))
+    assert y.shape == (rows, T, dim_out)
+    torch.testing.assert_close(y.cpu().double(), ref, rtol=1e-5, atol=2e-6 * float(ref.abs().max()))
+    y2 = ops.tensor_linear_fwd(inds, W, x, y_layout=ops.LAYOUT_COMP_CHAN, out=y.clone(), accumulate=True)
+    torch.testing.assert_close(y2.cpu().double(), 2 * ref, rtol=1e-5, atol=4e-6 * float(ref.abs().max()))
+    # the same numbers as the generic kernel gives at fewer rows (first rows only)
+    small = ops.tensor_linear_fwd(inds, W, x[:500].contiguous(), y_layout=ops.LAYOUT_COMP_CHAN)
+    torch.testing.assert_close(y[:500], small, rtol=1e-5, atol=2e-6 * float(ref.abs().max()))
