@@ -385,7 +385,7 @@ def bench_denoiser(torch, args, with_cpu=True):
         gl = importlib.import_module("learned-dynamics_amd.graph_layers")
         graph, _ = gl.graph_setup(r0, box, dev[3], neighbours_max=256, celllist_max=64)
         E = int(graph.src.numel())
-    single = None if args.no_extras else single_system_latency(torch, model, dev, box, r0, N)
+    single = None if getattr(args, "no_extras", False) else single_system_latency(torch, model, dev, box, r0, N)
     out = {"metric": "denoiser forward atoms/sec", "value": B * N / sec, "unit": "atoms/s", "ms_per_step": sec * 1e3,
            "dtype": "f32",
            "config": {"workload": "BASELINE configs[3]: 8 x [Messages + SelfTensProds] rank-0/1/2 denoiser forward "
