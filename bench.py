@@ -139,7 +139,7 @@ def bench_painn_layer(torch, args):
         split = mode == ops.LINEAR_BF16X3
         if mode == ops.LINEAR_F16X2:
             # operands split into 2 fp16 pieces, 3 fp16 MFMAs per fp32 product, fp32 accumulate
-            roofline = {"kernel": "linear_rows_f16x2_kernel<4,4> (filter MLP layer, E x 512 x 512, bias+SiLU fused)",
+            roofline = {"kernel": "linear_rows_f16x2_kernel<8 waves, 256 columns> (filter MLP layer, E x 512 x 512, bias+SiLU fused)",
                         "bound": "mfma", "achieved": 3 * flops / t_gemm / 1e12, "peak": PEAK_BF16_MFMA_TFLOPS,
                         "unit": "TFLOP/s", "frac": 3 * flops / t_gemm / 1e12 / PEAK_BF16_MFMA_TFLOPS,
                         "traffic": measured_traffic("linear_rows_f16x2_kernel"),

@@ -1,3 +1,7 @@
+// Two kernels that end a per-edge GEMM with a sum over the edges of each node, so that the per-edge
+// result is never stored: the PaiNN message (below) and a plain linear layer whose rows are only
+// needed summed per segment (linear_rowsum_f16x2_kernel, further down).
+//
 // PaiNN message with the last layer of the filter MLP folded in: the per-edge filter
 //     W(e) = h(e) W3^T + b3            (h: (edges, hidden) output of the MLP's second layer, W3: (4n, hidden))
 // is produced tile by tile on the matrix cores and consumed in the same kernel by
