@@ -340,6 +340,42 @@ def chain_positions(torch, systems, atoms, box, seed, noise=1.0):
     return (pos + noise * torch.randn(systems, atoms, 3, generator=g)).contiguous()
 
 
+def edge_kernel_roofline(torch, msg, graph, r_ij, rows, bf16=False):
+    """The fused rank-0/1/2 edge kernel of one Messages layer timed alone (HIP events): algorithmic bytes =
+    per edge 3 chan outputs + indices, encoding and direction; per node 13 chan inputs read once and 60 chan
+    sums written (4 bytes each, 2 with bf16 storage)."""
+    ops = importlib.import_module("learned-dynamics_amd.ops")
+    chan = int(msg.lin_enc.weight.shape[0])
+    dev = r_ij.device
+    dt = torch.bfloat16 if bf16 else torch.float32
+    g = torch.Generator(device="cuda").manual_seed(1)
+    La = torch.randn(rows, chan, device=dev, generator=g).to(dt)
+    Lv = torch.randn(rows, 3, chan, device=dev, generator=g).to(dt)
+    Ld = torch.randn(rows, 9, chan, device=dev, generator=g).to(dt)
+    enc, rhat = ops.bee_edge_geometry(r_ij.contiguous(), msg.r0)
+    order = getattr(graph, "cell_order", None)
+    if bf16:
+        fn = lambda: ops.bee_message_bf16(graph.row_ptr, graph.dst32, rhat, enc, La, Lv, Ld, msg.lin_enc.weight,
+                                          msg.lin_enc.bias, node_order=order)
+    else:
+        fn = lambda: ops.bee_message(graph.row_ptr, graph.dst32, rhat, enc, La, Lv, Ld, msg.lin_enc.weight,
+                                     msg.lin_enc.bias, node_order=order, want_node_max=True)
+    t = event_time(torch, fn, 10)
+    E = int(graph.src.numel())
+    w = 2 if bf16 else 4
+    nbytes = E * (3 * chan * w + 4 + 32 + 12) + rows * (13 + 60) * chan * w
+    return {"kernel": "bee_message_kernel (gathers, 13 products, edge sums; one Messages layer)", "bound": "hbm",
+            "achieved": nbytes / t / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": nbytes / t / 1e9 / PEAK_HBM_GBS,
+            "traffic": None, "bytes_per_launch": nbytes, "ms": t * 1e3,
+            # the 13 products are 167 flop per (edge, channel), the 60 running sums another 60
+            "fp32_vector_tflops": E * chan * 227 / t / 1e12,
+            "fp32_vector_frac_of_peak": E * chan * 227 / t / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+            "note": "gathered node rows are served by L2 and counted once per node; with ~90 edges per node "
+                    "(configs[4]) the kernel is bound by its fp32 vector arithmetic (packed fp32 instructions "
+                    "are compiled out, which halves the vector peak), with ~16 (configs[3]) by L2 gather latency "
+                    "and its 7 GB of outputs"}
+
+
 def single_system_latency(torch, model, dev, box, r0, atoms):
     """One system of the denoiser workload: the 8 blocks on a prebuilt neighbour graph, run eagerly and replayed
     from a captured HIP graph (the neighbour search stays outside the capture)."""
@@ -385,6 +421,7 @@ def bench_denoiser(torch, args, with_cpu=True):
         gl = importlib.import_module("learned-dynamics_amd.graph_layers")
         graph, _ = gl.graph_setup(r0, box, dev[3], neighbours_max=256, celllist_max=64)
         E = int(graph.src.numel())
+        edge_roof = edge_kernel_roofline(torch, model.messages[0], graph, gl.edge_vectors(graph, dev[3], box), B * N)
     single = None if getattr(args, "no_extras", False) else single_system_latency(torch, model, dev, box, r0, N)
     out = {"metric": "denoiser forward atoms/sec", "value": B * N / sec, "unit": "atoms/s", "ms_per_step": sec * 1e3,
            "dtype": "f32",
@@ -392,7 +429,7 @@ def bench_denoiser(torch, args, with_cpu=True):
                                   "(assembled from reference modules), 32 systems x 2048 atoms, box 70 A, cutoff 6 A, "
                                   "256 scalar + 64 vector + 16 rank-2 channels, chan 256, graph rebuilt every forward",
                       "edges": E, "atoms": B * N},
-           "single_system": single}
+           "roofline_hbm": edge_roof, "single_system": single}
     if with_cpu:
         out["cpu_baseline"] = cpu_denoiser_block(torch, model, x1[:1], r0, box, dims)
     return out
@@ -441,6 +478,8 @@ def bench_stress(torch, args):
         rel = float((out - ref).abs().max() / ref.abs().max())
         sec16 = timed_steps(torch, step_bf16, args.steps, args.warmup)
         sec32 = timed_steps(torch, step_f32, args.steps, args.warmup)
+        graph, r_ij = gl.graph_setup(r0, box, pos, neighbours_max=256, celllist_max=64)
+        edge_roof = edge_kernel_roofline(torch, msgs[0], graph, r_ij, N, bf16=True)
     E = edges[0]
     return {"metric": "message-passing edges/sec per layer", "value": E * layers / sec16, "unit": "edges/s",
             "ms_per_step": sec16 * 1e3, "dtype": "bf16 storage, f32 accumulate",
@@ -448,7 +487,7 @@ def bench_stress(torch, args):
                                    "4 x [Messages + SelfTensProds], 128 channels per rank, bf16 storage, "
                                    "neighbour rebuild in the step",
                        "edges": E, "atoms": N, "layers": layers, "atoms_per_s": N / sec16},
-            "max_abs_diff_vs_fp32_storage_over_scale": rel,
+            "roofline_hbm": edge_roof, "max_abs_diff_vs_fp32_storage_over_scale": rel,
             "fp32_storage": {"value": E * layers / sec32, "unit": "edges/s", "ms_per_step": sec32 * 1e3}}
 
 
