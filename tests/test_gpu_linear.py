@@ -272,3 +272,21 @@ def test_component_major_output_from_reference_layout_at_many_rows(ops, inds, ro
     # the same numbers as the generic kernel gives at fewer rows (first rows only)
     small = ops.tensor_linear_fwd(inds, W, x[:500].contiguous(), y_layout=ops.LAYOUT_COMP_CHAN)
     torch.testing.assert_close(y[:500], small, rtol=1e-5, atol=2e-6 * float(ref.abs().max()))
+
+
+def test_linear_with_row_sums_edge_cases(ops):
+    W = torch.randn(256, 64).cuda()
+    row_ptr = torch.zeros(11, dtype=torch.int32, device="cuda")
+    seg = torch.empty(0, dtype=torch.int32, device="cuda")
+    out, y = ops.tensor_linear_f16x2_rowsum(W, torch.empty(0, 64, device="cuda"), torch.ones(1, 1, device="cuda"), row_ptr, seg,
+                                            10, want_rows=True)
+    assert out.shape == (10, 256) and not bool(out.any()) and y.shape == (0, 256)
+    # one segment holding every row, fewer rows than a tile
+    x = torch.randn(77, 64).cuda()
+    seg = torch.zeros(77, dtype=torch.int32, device="cuda")
+    row_ptr = torch.tensor([0, 77], dtype=torch.int32, device="cuda")
+    out, _ = ops.tensor_linear_f16x2_rowsum(W, x, ops.row_absmax(x), row_ptr, seg, 1)
+    ref = (x.double() @ W.double().T).sum(0, keepdim=True)
+    torch.testing.assert_close(out.double(), ref, rtol=1e-5, atol=3e-6 * float(ref.abs().max()))
+    with pytest.raises(RuntimeError, match="multiple of 256"):
+        ops.tensor_linear_f16x2_rowsum(W[:128].contiguous(), x, ops.row_absmax(x), row_ptr, seg, 1)

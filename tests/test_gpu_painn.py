@@ -278,3 +278,21 @@ def test_other_radial_encodings(ops, kind):
         ref = torch.cos(npi * torch.sqrt(x_sq)[..., None]) * torch.relu(1. - x_sq)[..., None]
         tol = 4 * float(npi.max() * torch.sqrt(x_sq).max()) * 2.0 ** -24 + 2e-6
     torch.testing.assert_close(out.cpu().double(), ref, rtol=1e-5, atol=tol)
+
+
+def test_filter_message_without_edges_returns_the_residual(ops):
+    """No edges at all: every node gets its residual (or zero), nothing else is touched."""
+    n, hidden, N = 64, 128, 50
+    g = torch.Generator().manual_seed(3)
+    W3, b3 = torch.randn(4 * n, hidden, generator=g).cuda(), torch.randn(4 * n, generator=g).cuda()
+    actv, x_a, x_v = torch.randn(N, 4 * n).cuda(), torch.randn(N, n).cuda(), torch.randn(N, n, 3).cuda()
+    empty_i = torch.empty(0, dtype=torch.int32, device="cuda")
+    row_ptr = torch.zeros(N + 1, dtype=torch.int32, device="cuda")
+    h, bound, r = torch.empty(0, hidden, device="cuda"), torch.ones(1, 1, device="cuda"), torch.empty(0, 3, device="cuda")
+    out_a, out_v = ops.painn_filter_message(W3, b3, h, bound, row_ptr, empty_i, empty_i, r, actv, x_v, 0.1, x_a, x_v)
+    assert torch.equal(out_a, x_a) and torch.equal(out_v, x_v)
+    out_a, out_v = ops.painn_filter_message(W3, b3, h, bound, row_ptr, empty_i, empty_i, r, actv, x_v, 0.1)
+    assert not bool(out_a.any()) and not bool(out_v.any())
+    with pytest.raises(RuntimeError, match="multiple of 64"):
+        ops.painn_filter_message(W3[:4 * 48], b3[:4 * 48], h, bound, row_ptr, empty_i, empty_i, r, actv[:, :4 * 48].contiguous(),
+                                 x_v[:, :48].contiguous(), 0.1)
