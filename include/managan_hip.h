@@ -298,6 +298,19 @@ int mg_painn_filter_message(const void* packed_W3, const float* bias3, const flo
                             long n_nodes, long n_edges, int n, float epsilon, const float* res_a,
                             const float* res_v, void* workspace, float* out_a, float* out_v, mg_stream_t stream);
 
+/* SelfTensProds.forward after its six input linears (archs/diffuser_atoms15.py:82-94), one output rank per call:
+ *   y[node, o, comp] = sum over the product types `lab` of output rank rank_o, channels c of
+ *                      Y[o, (lab, c)] * p_lab(l, r)[node, comp, c]
+ * with the product types in the order 000 110 220 (rank 0), 011 101 121 211 111 (rank 1), 022 202 112 222 212
+ * (rank 2) (managan/codegen_tensor_products.py:235-249), so Y = [Y_lab ...] concatenated along its input axis,
+ * packed with mg_linear_f16x2_pack_weight (dim_out x n_types*chan).  The products are built in registers and
+ * never stored.  l_k, r_k: component-major (nodes, 3^k, chan); node_bound (nodes): an upper bound of every
+ * |product component| of the node (e.g. 9 max|l| max|r|; any bound within 2^14 of the largest keeps fp32
+ * accuracy); y: (nodes, dim_out, 3^rank_o), the reference's layout.  chan % 32 == 0. */
+int mg_bee_products_linear(int rank_o, const float* l_0, const float* l_1, const float* l_2, const float* r_0,
+                           const float* r_1, const float* r_2, const float* node_bound, long n_nodes, int chan,
+                           const void* packed_W, int dim_out, float* y, mg_stream_t stream);
+
 /* A per-edge nn.Linear followed by the sum over the edges of each node, in one kernel: the pattern
  * `edges_reduce_src(graph, mlp(...))` of archs/diffuser_atoms15.py:244-246 (managan/graph_layers.py:54-59) for a
  * layer of the MLP whose output is only needed summed.

@@ -131,16 +131,30 @@ class SelfTensProds(nn.Module):
         # 5 chan, 5 chan instead of thirteen accumulating ones
         C = ops.LAYOUT_COMP_CHAN
         chan = self.L0.W.shape[0]
-        ops_in = [ops.tensor_linear_fwd(k, lin.W, x, y_layout=C if k else ops.LAYOUT_CHAN_COMP)
-                  for side in ((self.L0, self.L1, self.L2), (self.R0, self.R1, self.R2))
-                  for k, (lin, x) in enumerate(zip(side, (x_a, x_v, x_d)))]
-        P0, P1, P2, nmax = ops.bee_node_products(*ops_in, want_node_max=True)
-        # nmax: per-node maxima of the products, the row bounds of the three GEMMs
-        y_a = ops.tensor_linear_fwd(0, _cat_Y(self, LABELS_0), P0.reshape(rows, 3 * chan), row_bound=nmax)
-        y_v = ops.tensor_linear_fwd(1, _cat_Y(self, LABELS_1), P1.reshape(rows, 3, 5 * chan), x_layout=C,
-                                    row_bound=nmax, rows_per_bound=3)
-        y_d = ops.tensor_linear_fwd(2, _cat_Y(self, LABELS_2), P2.reshape(rows, 9, 5 * chan), x_layout=C,
-                                    row_bound=nmax, rows_per_bound=9)
+        pairs = [ops.tensor_linear_fwd(k, lin.W, x, y_layout=C if k else ops.LAYOUT_CHAN_COMP, want_rowmax=True)
+                 for side in ((self.L0, self.L1, self.L2), (self.R0, self.R1, self.R2))
+                 for k, (lin, x) in enumerate(zip(side, (x_a, x_v, x_d)))]
+        ops_in = [p[0] for p in pairs]
+        if ops.bee_products_linear_supported(rows, chan):
+            # products and output linears in one kernel per output rank: the 13 products are never stored.
+            # Its row scales need a bound of the products per node: 9 max|l| max|r| (at most 9 terms per
+            # component), from the row maxima the six GEMMs above emit
+            def node_max(side):
+                cols = [(m if m is not None else ops.row_absmax(t.reshape(rows, -1))).reshape(rows, -1)
+                        for t, m in side]
+                return torch.cat(cols, dim=1).amax(dim=1)
+            bound = 9.0 * node_max(pairs[:3]) * node_max(pairs[3:])
+            y_a = ops.bee_products_linear(0, _cat_Y(self, LABELS_0), *ops_in, bound)
+            y_v = ops.bee_products_linear(1, _cat_Y(self, LABELS_1), *ops_in, bound)
+            y_d = ops.bee_products_linear(2, _cat_Y(self, LABELS_2), *ops_in, bound)
+        else:
+            P0, P1, P2, nmax = ops.bee_node_products(*ops_in, want_node_max=True)
+            # nmax: per-node maxima of the products, the row bounds of the three GEMMs
+            y_a = ops.tensor_linear_fwd(0, _cat_Y(self, LABELS_0), P0.reshape(rows, 3 * chan), row_bound=nmax)
+            y_v = ops.tensor_linear_fwd(1, _cat_Y(self, LABELS_1), P1.reshape(rows, 3, 5 * chan), x_layout=C,
+                                        row_bound=nmax, rows_per_bound=3)
+            y_d = ops.tensor_linear_fwd(2, _cat_Y(self, LABELS_2), P2.reshape(rows, 9, 5 * chan), x_layout=C,
+                                        row_bound=nmax, rows_per_bound=9)
         y_a = y_a.reshape(*rest, dim_a)
         y_v = y_v.reshape(*rest, dim_v, 3)
         y_d = y_d.reshape(*rest, dim_d, 3, 3)

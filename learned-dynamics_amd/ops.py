@@ -677,12 +677,15 @@ LAYOUT_CHAN_COMP, LAYOUT_COMP_CHAN = 0, 1
 
 
 def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=False,
-                      x_layout=LAYOUT_CHAN_COMP, y_layout=LAYOUT_CHAN_COMP, row_bound=None, rows_per_bound=1):
+                      x_layout=LAYOUT_CHAN_COMP, y_layout=LAYOUT_CHAN_COMP, row_bound=None, rows_per_bound=1,
+                      want_rowmax=False):
     """y[..., o, t] = act(sum_i W[o, i] x[..., i, t] + bias[o]); W may have any strides.
     Layout 0 stores a tensor as (..., chan, (3,)^inds) like the reference; layout 1 is
     component-major (..., 3^inds, chan), the layout the fused edge kernels read and write.
     row_bound ((rows of the GEMM) / rows_per_bound, parts): upper bounds of the row maxima of |x| from
-    the kernel that produced x, used by the split-fp16 matrix path instead of a pass over x."""
+    the kernel that produced x, used by the split-fp16 matrix path instead of a pass over x.
+    want_rowmax: return (y, rowmax) with rowmax ((GEMM rows), parts) partial row maxima of |y| when the kernel
+    that ran can emit them (plain-row output through the split-fp16 path), else (y, None)."""
     if not W.is_cuda:
         raise RuntimeError("W must be a CUDA tensor")
     _check_input(x, "x")
@@ -730,6 +733,13 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
         wide = (plain_rows and dim_in % 32 == 0 and dim_in >= 64 and dim_out >= 64 and rows * T >= 1024
                 and x.data_ptr() % 16 == 0)
         out_comps = 1 if (inds == 0 or y_layout == LAYOUT_COMP_CHAN) else T
+        ymax = None
+
+        def rowmax_buffer(k_in):
+            if not (want_rowmax and out_comps == 1 and not accumulate):
+                return None
+            parts = int(_lib.mg_tensor_linear_f16x2_rowmax_parts(rows * T, k_in, dim_out))
+            return torch.empty(rows * T, parts, dtype=torch.float32, device=x.device)
         if (mode == LINEAR_F16X2 and inds > 0 and x_layout == LAYOUT_CHAN_COMP and y_layout == LAYOUT_COMP_CHAN
                 and rows * T >= 65536 and dim_out >= 64 and row_bound is None):
             # (row, chan, comp) -> (row, comp, chan) rows (K zero-padded to a multiple of 32), then the plain-row
@@ -740,20 +750,22 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
             xt = torch.nn.functional.pad(xt, (0, k_pad - dim_in)) if k_pad != dim_in else xt.contiguous()
             x2 = xt.reshape(rows * T, k_pad)
             Wp = _zero_padded_columns(W, k_pad)
+            ymax = rowmax_buffer(k_pad)
             L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(Wp)), _p(x2), _p(row_absmax(x2)), 1, 1, 1,
                                                 rows * T, k_pad, dim_out, _p(bias), int(act), int(bool(accumulate)),
-                                                1, _p(y), None, _stream()))
+                                                1, _p(y), _p(ymax), _stream()))
         elif (plain_rows and mode == LINEAR_F16X2 and f16x2_supported(rows * T, dim_in, dim_out, x)):
             x2 = x.reshape(rows * T, dim_in)
             if row_bound is None:
                 row_bound, rows_per_bound = row_absmax(x2), 1
             elif row_bound.dim() != 2 or row_bound.size(0) * rows_per_bound != rows * T:
                 raise RuntimeError("row_bound must be (rows / rows_per_bound, parts)")
+            ymax = rowmax_buffer(dim_in)
             L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(W)), _p(x2), _p(row_bound),
                                                 int(row_bound.size(1)), int(row_bound.size(1)), int(rows_per_bound),
                                                 rows * T,
                                                 dim_in, dim_out, _p(bias), int(act), int(bool(accumulate)),
-                                                out_comps, _p(y), None, _stream()))
+                                                out_comps, _p(y), _p(ymax), _stream()))
         elif wide and mode == LINEAR_BF16X3:
             L.check(_lib.mg_tensor_linear_packed(_p(packed_weight(W)), _p(x), rows * T, dim_in, dim_out, _p(bias),
                                                  int(act), int(bool(accumulate)), out_comps, _p(y), _stream()))
@@ -761,7 +773,7 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
             L.check(_lib.mg_tensor_linear_layout(inds, _p(W), int(W.stride(0)), int(W.stride(1)), _p(x), rows,
                                                  dim_in, dim_out, _p(bias), int(act), int(bool(accumulate)),
                                                  int(x_layout), int(y_layout), _p(y), _stream()))
-    return y
+    return (y, ymax) if want_rowmax else y
 
 
 def tensor_linear_wgrad(inds, dy, x):
@@ -967,6 +979,34 @@ def painn_message(row_ptr, dst, r_ij, filt, actv, x_v, epsilon, res_a=None, res_
         L.check(_lib.mg_painn_message(_p(row_ptr), _p(dst), _p(node_order), n_nodes, E, _p(r_ij), _p(filt), _p(actv), _p(x_v), n,
                                       float(epsilon), _p(res_a), _p(res_v), _p(out_a), _p(out_v), _stream()))
     return out_a, out_v
+
+
+def bee_products_linear_supported(n_nodes, chan):
+    return get_linear_mode() == LINEAR_F16X2 and chan % 32 == 0 and chan >= 32 and n_nodes >= 1024
+
+
+def bee_products_linear(rank_o, W, l0, l1, l2, r0, r1, r2, node_bound):
+    """y (nodes, dim_out, (3,)^rank_o) = sum over the product types of output rank rank_o of Y_lab p_lab(l, r), with
+    W = [Y_lab ...] concatenated along the input axis in the order 000 110 220 / 011 101 121 211 111 /
+    022 202 112 222 212.  l_k, r_k component-major (nodes, 3^k, chan) ((nodes, chan) for k = 0); node_bound (nodes,):
+    upper bound of every |product component| of the node."""
+    for t, nm in ((W, "W"), (l0, "l0"), (l1, "l1"), (l2, "l2"), (r0, "r0"), (r1, "r1"), (r2, "r2"), (node_bound, "node_bound")):
+        _check_input(t, nm)
+    N, chan = int(l0.size(0)), int(l0.size(1))
+    for t, comps in ((l0, None), (r0, None), (l1, 3), (r1, 3), (l2, 9), (r2, 9)):
+        if tuple(t.shape) != ((N, chan) if comps is None else (N, comps, chan)):
+            raise RuntimeError("operands must be (nodes, chan), (nodes, 3, chan), (nodes, 9, chan)")
+    n_types = 3 if rank_o == 0 else 5
+    if W.dim() != 2 or int(W.size(1)) != n_types * chan:
+        raise RuntimeError(f"W must be (dim_out, {n_types} * chan)")
+    if node_bound.numel() != N:
+        raise RuntimeError("node_bound must have one entry per node")
+    dim_out = int(W.size(0))
+    with torch.cuda.device(l0.device):
+        y = torch.empty((N, dim_out) + (3,) * rank_o, dtype=torch.float32, device=l0.device)
+        L.check(_lib.mg_bee_products_linear(int(rank_o), _p(l0), _p(l1), _p(l2), _p(r0), _p(r1), _p(r2), _p(node_bound),
+                                            N, chan, _p(packed_weight_f16x2(W)), dim_out, _p(y), _stream()))
+    return y
 
 
 def f16x2_rowsum_supported(rows, dim_in, dim_out, x):

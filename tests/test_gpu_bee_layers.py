@@ -242,3 +242,67 @@ def test_mlp_summed_over_rows_equals_sum_of_rows(pkg, plus_identity):
     torch.testing.assert_close(per_row.cpu().double(), y, rtol=1e-5, atol=2e-6 * float(y.abs().max()))
     torch.testing.assert_close(got.cpu().double(), ref, rtol=1e-5, atol=3e-6 * float(ref.abs().max()))
     assert not bool(got[deg.cuda() == 0].any())
+
+
+@pytest.mark.parametrize("chan,dims,N", [(64, (48, 40, 16), 1500), (32, (256, 64, 16), 1100), (96, (32, 100, 8), 1300)])
+def test_products_and_output_linears_in_one_kernel(pkg, chan, dims, N):
+    """mg_bee_products_linear (13 products built in registers + the concatenated Y linears) against the
+    stored-products path (node_products_kernel + one GEMM per rank) and against float64 einsums of the
+    oracle's products; operands with rows of very different size."""
+    ops = importlib.import_module("learned-dynamics_amd.ops")
+    g = torch.Generator().manual_seed(chan + N)
+    size = torch.rand(N, 1, generator=g) * 3 + 0.01
+    l = [torch.randn(N, chan, generator=g) * size, torch.randn(N, 3, chan, generator=g) * size[:, None],
+         torch.randn(N, 9, chan, generator=g) * size[:, None]]
+    r = [torch.randn(N, chan, generator=g), torch.randn(N, 3, chan, generator=g), torch.randn(N, 9, chan, generator=g)]
+    dev = [t.cuda() for t in l + r]
+    lmax = torch.cat([t.reshape(N, -1) for t in l], 1).abs().amax(1)
+    rmax = torch.cat([t.reshape(N, -1) for t in r], 1).abs().amax(1)
+    bound = (9.0 * lmax * rmax).cuda()
+    P0, P1, P2, nmax = ops.bee_node_products(*dev, want_node_max=True)
+    # the oracle's products in the reference layout (rows, chan, 3..)
+    to_ref = lambda t, k: t if k == 0 else t.reshape(N, 3 ** k, chan).transpose(1, 2).reshape(N, chan, *([3] * k))
+    prods = dict(zip(OP.BEE_ORDER, OP.bee(*[to_ref(t.double(), k) for k, t in enumerate(l)],
+                                          *[to_ref(t.double(), k) for k, t in enumerate(r)])))
+    groups = (("000", "110", "220"), ("011", "101", "121", "211", "111"), ("022", "202", "112", "222", "212"))
+    for rank, (labs, P, dim_out) in enumerate(zip(groups, (P0, P1, P2), dims)):
+        W = (torch.randn(dim_out, len(labs) * chan, generator=g) / (len(labs) * chan) ** 0.5).cuda()
+        y = ops.bee_products_linear(rank, W, *dev, bound)
+        T = 3 ** rank
+        assert y.shape == (N, dim_out) + (3,) * rank
+        if rank == 0:
+            stored = ops.tensor_linear_fwd(0, W, P.reshape(N, 3 * chan))
+        else:
+            stored = ops.tensor_linear_fwd(rank, W, P.reshape(N, T, len(labs) * chan), x_layout=ops.LAYOUT_COMP_CHAN)
+        ref = sum(torch.einsum("oc,nc...->no...", W[:, k * chan:(k + 1) * chan].double().cpu(), prods[lab])
+                  for k, lab in enumerate(labs))
+        scale = float(ref.abs().max())
+        torch.testing.assert_close(y, stored, rtol=1e-5, atol=3e-6 * scale)
+        torch.testing.assert_close(y.cpu().double(), ref, rtol=1e-5, atol=3e-6 * scale)
+        # rows of small nodes keep their relative accuracy (per-node scales)
+        small = (size[:, 0] < 0.1)
+        if bool(small.any()):
+            rs = ref[small]
+            torch.testing.assert_close(y.cpu().double()[small], rs, rtol=1e-5, atol=3e-6 * float(rs.abs().max()))
+
+
+def test_self_tens_prods_module_fused_path(pkg):
+    """SelfTensProds at a size that takes the products + linears kernel (chan % 32 == 0, >= 1024 nodes)."""
+    bee = importlib.import_module("learned-dynamics_amd.bee_layers")
+    torch.manual_seed(8)
+    dim_a, dim_v, dim_d, chan = 64, 32, 16, 64
+    mod = bee.SelfTensProds(dim_a, dim_v, dim_d, chan).cuda()
+    with torch.no_grad():
+        for gn in (mod.gn_a, mod.gn_v, mod.gn_d):
+            gn.gamma.copy_(torch.randn_like(gn.gamma))
+    x_a, x_v, x_d = torch.randn(2, 700, dim_a), torch.randn(2, 700, dim_v, 3), torch.randn(2, 700, dim_d, 3, 3)
+    with torch.no_grad():
+        y_a, y_v, y_d = mod(x_a.cuda(), x_v.cuda(), x_d.cuda(), residual=True)
+    dd = lambda t: t.detach().cpu()
+    w = {k: dd(getattr(mod, k).W) for k in ("L0", "R0", "L1", "R1", "L2", "R2")}
+    w["Y"] = {lab: dd(getattr(mod, f"Y_{lab}").W) for lab in OP.BEE_ORDER}
+    w.update(gn_a=dd(mod.gn_a.gamma), gn_v=dd(mod.gn_v.gamma), gn_d=dd(mod.gn_d.gamma))
+    ra, rv, rd = OL.self_tens_prods(x_a, x_v, x_d, w)
+    _close(y_a, x_a + ra, atol_scale=5e-6)
+    _close(y_v, x_v + rv, atol_scale=5e-6)
+    _close(y_d, x_d + rd, atol_scale=5e-6)
