@@ -306,10 +306,12 @@ int mg_painn_filter_message(const void* packed_W3, const float* bias3, const flo
  * packed with mg_linear_f16x2_pack_weight (dim_out x n_types*chan).  The products are built in registers and
  * never stored.  l_k, r_k: component-major (nodes, 3^k, chan); node_bound (nodes): an upper bound of every
  * |product component| of the node (e.g. 9 max|l| max|r|; any bound within 2^14 of the largest keeps fp32
- * accuracy); y: (nodes, dim_out, 3^rank_o), the reference's layout.  chan % 32 == 0. */
+ * accuracy); y: (nodes, dim_out, 3^rank_o), the reference's layout.  chan % 32 == 0.
+ * k_order 0: the columns of Y are ordered (type, channel) as above.  k_order 1 (rank_o == 2, dim_out <= 64):
+ * (channel / 32, type, channel % 32); the kernel then stages the operands of 32 channels in LDS for all types. */
 int mg_bee_products_linear(int rank_o, const float* l_0, const float* l_1, const float* l_2, const float* r_0,
                            const float* r_1, const float* r_2, const float* node_bound, long n_nodes, int chan,
-                           const void* packed_W, int dim_out, float* y, mg_stream_t stream);
+                           const void* packed_W, int k_order, int dim_out, float* y, mg_stream_t stream);
 
 /* A per-edge nn.Linear followed by the sum over the edges of each node, in one kernel: the pattern
  * `edges_reduce_src(graph, mlp(...))` of archs/diffuser_atoms15.py:244-246 (managan/graph_layers.py:54-59) for a

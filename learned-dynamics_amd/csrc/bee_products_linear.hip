@@ -221,6 +221,202 @@ products_linear_kernel(const _Float16* __restrict__ Wp, const float* __restrict_
     }
 }
 
+// Rank-2 output (nine GEMM rows per node): the 13 + 13 component rows of the tile's nodes are staged in LDS once
+// per block of 32 channels and serve all five product types and all nine components from there; reading the
+// operands through L1 instead costs one cache lookup per lane and 16 bytes, which bounded the kernel above.
+// K is ordered (channel block of 32, product type, channel in block); the caller packs W with its columns in
+// that order.
+template <int NI>
+__global__ void __launch_bounds__(256)
+products_linear_staged_kernel(const _Float16* __restrict__ Wp, const float* __restrict__ w_inv, Operands ops,
+                              const float* __restrict__ node_bound, long n_nodes, int chan, int O, int O_pad,
+                              float* __restrict__ Y, int tiles_n, long tiles_total) {
+    constexpr int T = 9, WAVES = 4, TM = 32 * WAVES, TN = 32 * NI, THREADS = 64 * WAVES;
+    constexpr int NN = TM / T + 2;                           // nodes a tile of TM rows can touch
+    constexpr int kRowF = 36;                                // floats per staged row: 32 channels + 4 (bank spread)
+    constexpr int kPlaneW = TN * kRowW, kBufW = 2 * kPlaneW;
+    constexpr int kPieces = 8 * TN;
+    constexpr int kPer = (kPieces + THREADS - 1) / THREADS;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kBufW];
+    __shared__ __attribute__((aligned(16))) float stage[26 * NN * kRowF];
+    __shared__ float inv_sx[TM];
+
+    const long bid = blockIdx.x;
+    const long per_xcd = (tiles_total + 7) / 8;
+    const long logical = (bid % 8) * per_xcd + bid / 8;
+    if (logical >= tiles_total) return;
+    const long tile_m = logical / tiles_n;
+    const int tile_n = (int)(logical - tile_m * tiles_n);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int m = lane & 31, g = lane >> 5;
+    const long R = n_nodes * T;
+    const int NL = ops.n_labels;
+    const int I = NL * chan;
+    const long r0 = tile_m * TM;
+    const int n0 = tile_n * TN;
+    const long plane_elems = (long)O_pad * I;
+    const long node_lo = r0 / T;
+
+    floatx16 acc[NI];
+#pragma unroll
+    for (int ni = 0; ni < NI; ni++)
+#pragma unroll
+        for (int q = 0; q < 16; q++) acc[ni][q] = 0.f;
+
+    const long my_row = r0 + wave * 32 + m;
+    const long ld_row = my_row < R ? my_row : R - 1;
+    const long node = ld_row / T;
+    const int co = (int)(ld_row - node * T);
+    const int nl = (int)(node - node_lo);                    // 0 .. NN-1
+    float sx;
+    {
+        float inv;
+        sx = pow2_scale(node_bound[node], &inv);
+        if (g == 0) inv_sx[wave * 32 + m] = inv;
+    }
+    const _Float16* wsrc[kPer];
+    int wdst[kPer];
+#pragma unroll
+    for (int j = 0; j < kPer; j++) {
+        int q = tid + THREADS * j;
+        if (q >= kPieces) q = kPieces - 1;
+        const int plane = q / (4 * TN), row = (q % (4 * TN)) >> 2, piece = q & 3;
+        wsrc[j] = Wp + plane * plane_elems + (long)(n0 + row) * I + 8 * piece;
+        wdst[j] = plane * kPlaneW + row * kRowW + piece * 16;
+    }
+    const int k_last = I - kCK;
+    struct ARegs { float4 v[4]; };
+    struct WRegs { halfx8 v[kPer]; };
+
+    // staged row index: 0 l_0, 1..3 l_1, 4..12 l_2, 13 r_0, 14..16 r_1, 17..25 r_2
+    constexpr int kStagePieces = 26 * NN * 8, kStagePer = (kStagePieces + THREADS - 1) / THREADS;
+    auto stage_block = [&](int cb) {
+        // all loads of the block are requested before the first LDS store: one round trip, not kStagePer.
+        // (Requesting the next block a whole block early, to hide that round trip too, measured slower: the
+        // weight loads of every chunk then queue behind it.)
+        float4 v[kStagePer];
+        int dst[kStagePer];
+#pragma unroll
+        for (int u = 0; u < kStagePer; u++) {
+            int idx = tid + THREADS * u;
+            idx = idx < kStagePieces ? idx : kStagePieces - 1;       // surplus threads repeat the last piece
+            const int rr = idx / (NN * 8), rem = idx - rr * (NN * 8);
+            const int nd = rem >> 3, piece = rem & 7;
+            long ng = node_lo + nd;
+            ng = ng < n_nodes ? ng : n_nodes - 1;
+            const int side = rr >= 13, k = side ? rr - 13 : rr;      // k: 0, 1..3, 4..12
+            const int rank = k == 0 ? 0 : (k < 4 ? 1 : 2);
+            const int comp = k == 0 ? 0 : (k < 4 ? k - 1 : k - 4);
+            const int C = rank == 0 ? 1 : (rank == 1 ? 3 : 9);
+            const float* base = side ? ops.r[rank] : ops.l[rank];
+            v[u] = *reinterpret_cast<const float4*>(base + (ng * C + comp) * chan + cb * 32 + 4 * piece);
+            dst[u] = (rr * NN + nd) * kRowF + 4 * piece;
+        }
+#pragma unroll
+        for (int u = 0; u < kStagePer; u++) *reinterpret_cast<float4*>(stage + dst[u]) = v[u];
+    };
+    auto build_a = [&](ARegs& a, int li) {
+        const int label = ops.labels[li];
+        const int rl = kPRankL[label], rr = kPRankR[label];
+        const SignedDot d = signed_dot(label, co);
+        const int lrow = (rl == 0 ? 0 : (rl == 1 ? 1 : 4)) + d.lb;
+        const int rrow = 13 + (rr == 0 ? 0 : (rr == 1 ? 1 : 4)) + d.rb;
+        const float* lp = stage + (lrow * NN + nl) * kRowF + 16 * g;
+        const float* rp = stage + (rrow * NN + nl) * kRowF + 16 * g;
+        const int lstep = d.ls * NN * kRowF, rstep = d.rs * NN * kRowF;
+#pragma unroll
+        for (int j = 0; j < 4; j++) a.v[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        for (int t = 0; t < d.nt; t++) {                  // trip count fixed by the product type: uniform
+            const float sgn = (d.cross && t == 1) ? -1.f : 1.f;
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float4 x = *reinterpret_cast<const float4*>(lp + t * lstep + 4 * j);
+                const float4 y = *reinterpret_cast<const float4*>(rp + t * rstep + 4 * j);
+                a.v[j].x += sgn * x.x * y.x;
+                a.v[j].y += sgn * x.y * y.y;
+                a.v[j].z += sgn * x.z * y.z;
+                a.v[j].w += sgn * x.w * y.w;
+            }
+        }
+    };
+    auto load_w = [&](WRegs& w, int k0) {
+        k0 = k0 < I ? k0 : k_last;
+#pragma unroll
+        for (int j = 0; j < kPer; j++) w.v[j] = *reinterpret_cast<const halfx8*>(wsrc[j] + k0);
+    };
+    auto store_w = [&](const WRegs& w, unsigned char* buf) {
+#pragma unroll
+        for (int j = 0; j < kPer; j++) *reinterpret_cast<halfx8*>(buf + wdst[j]) = w.v[j];
+    };
+    const int b_off = m * kRowW + 32 * g;
+    auto compute = [&](const ARegs& a, const unsigned char* buf) {
+        halfx8 ah[2], al[2];
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            const HalfSplit4 p0 = split(a.v[2 * s], sx), p1 = split(a.v[2 * s + 1], sx);
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                ah[s][i] = p0.hi[i]; ah[s][4 + i] = p1.hi[i];
+                al[s][i] = p0.lo[i]; al[s][4 + i] = p1.lo[i];
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 2; s++)
+#pragma unroll
+            for (int ni = 0; ni < NI; ni++) {
+                const halfx8 bh = *reinterpret_cast<const halfx8*>(buf + b_off + ni * 32 * kRowW + 16 * s);
+                const halfx8 bl = *reinterpret_cast<const halfx8*>(buf + kPlaneW + b_off + ni * 32 * kRowW + 16 * s);
+                acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[s], bh, acc[ni], 0, 0, 0);
+                acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[s], bl, acc[ni], 0, 0, 0);
+                acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[s], bh, acc[ni], 0, 0, 0);
+            }
+    };
+
+    WRegs w;
+    load_w(w, 0);
+    stage_block(0);
+    store_w(w, lds);
+    load_w(w, kCK);
+    __syncthreads();
+    const int n_chunks = I / kCK;
+    int li = 0, cb = 0;
+    for (int ch = 0; ch < n_chunks; ch++) {
+        ARegs a;
+        build_a(a, li);
+        compute(a, lds + (ch & 1) * kBufW);
+        store_w(w, lds + ((ch + 1) & 1) * kBufW);         // chunk ch + 1 (a clamped reload past the end, never used)
+        load_w(w, (ch + 2) * kCK);
+        if (++li == NL) {
+            li = 0;
+            cb++;
+            __syncthreads();                               // every wave has built its last operand of this block
+            if (ch + 1 < n_chunks) stage_block(cb);
+        }
+        __syncthreads();
+    }
+
+    float iw[NI];
+#pragma unroll
+    for (int ni = 0; ni < NI; ni++) {
+        const int n = n0 + ni * 32 + m;
+        iw[ni] = n < O ? w_inv[n] : 0.f;
+    }
+#pragma unroll
+    for (int q = 0; q < 16; q++) {
+        const int rl = wave * 32 + 8 * (q / 4) + 4 * g + (q % 4);
+        const long r = r0 + rl;
+        if (r < R) {
+            const long nd = r / T;
+            float* yp = Y + (nd * O + n0 + m) * T + (r - nd * T);
+            const float isx = inv_sx[rl];
+#pragma unroll
+            for (int ni = 0; ni < NI; ni++)
+                if (n0 + ni * 32 + m < O) yp[ni * 32 * T] = acc[ni][q] * isx * iw[ni];
+        }
+    }
+}
+
 template <int WAVES, int NI, int T>
 int launch(const _Float16* planes, const float* w_inv, const Operands& ops, const float* bound, long n_nodes, int chan,
            int O, int O_pad, float* y, hipStream_t st) {
@@ -252,7 +448,9 @@ extern "C" {
 
 int mg_bee_products_linear(int rank_o, const float* l_0, const float* l_1, const float* l_2, const float* r_0,
                            const float* r_1, const float* r_2, const float* node_bound, long n_nodes, int chan,
-                           const void* packed_W, int dim_out, float* y, mg_stream_t stream) {
+                           const void* packed_W, int k_order, int dim_out, float* y, mg_stream_t stream) {
+    MG_REQUIRE(k_order == 0 || (k_order == 1 && rank_o == 2 && dim_out <= 64),
+               "mg_bee_products_linear: k_order 1 (channel blocks outermost) is for rank_o == 2 with dim_out <= 64");
     MG_REQUIRE(rank_o >= 0 && rank_o <= 2, "mg_bee_products_linear: rank_o must be 0, 1 or 2");
     MG_REQUIRE(chan >= 32 && chan % 32 == 0, "mg_bee_products_linear: chan must be a multiple of 32 (got %d)", chan);
     MG_REQUIRE(n_nodes >= 0 && dim_out >= 0, "mg_bee_products_linear: negative size");
@@ -272,6 +470,21 @@ int mg_bee_products_linear(int rank_o, const float* l_0, const float* l_1, const
     const _Float16* planes = static_cast<const _Float16*>(packed_W);
     const float* w_inv = reinterpret_cast<const float*>(planes + 2L * O_pad * dim_in);
     hipStream_t st = (hipStream_t)stream;
+    if (k_order == 1) {
+        const long tiles_m = ceil_div(n_nodes * 9, 128);
+        const int ni = dim_out <= 32 ? 1 : 2;
+        const int tiles_n = (int)ceil_div(dim_out, 32 * ni);
+        const long total = tiles_m * tiles_n;
+        const long grid = ceil_div(total, 8) * 8;
+        MG_REQUIRE(grid <= 0x7fffffffL, "mg_bee_products_linear: grid too large");
+        if (ni == 1)
+            hipLaunchKernelGGL((products_linear_staged_kernel<1>), dim3((unsigned)grid), dim3(256), 0, st, planes, w_inv,
+                               ops, node_bound, n_nodes, chan, dim_out, O_pad, y, tiles_n, total);
+        else
+            hipLaunchKernelGGL((products_linear_staged_kernel<2>), dim3((unsigned)grid), dim3(256), 0, st, planes, w_inv,
+                               ops, node_bound, n_nodes, chan, dim_out, O_pad, y, tiles_n, total);
+        return check_launch("mg_bee_products_linear");
+    }
     if (rank_o == 0) return dispatch<1>(planes, w_inv, ops, node_bound, n_nodes, chan, dim_out, O_pad, y, st);
     if (rank_o == 1) return dispatch<3>(planes, w_inv, ops, node_bound, n_nodes, chan, dim_out, O_pad, y, st);
     return dispatch<9>(planes, w_inv, ops, node_bound, n_nodes, chan, dim_out, O_pad, y, st);

@@ -1002,11 +1002,33 @@ def bee_products_linear(rank_o, W, l0, l1, l2, r0, r1, r2, node_bound):
     if node_bound.numel() != N:
         raise RuntimeError("node_bound must have one entry per node")
     dim_out = int(W.size(0))
+    k_order = 1 if (rank_o == 2 and dim_out <= 64) else 0
+    if k_order:
+        W = _channel_block_major_columns(W, n_types, chan)
     with torch.cuda.device(l0.device):
         y = torch.empty((N, dim_out) + (3,) * rank_o, dtype=torch.float32, device=l0.device)
         L.check(_lib.mg_bee_products_linear(int(rank_o), _p(l0), _p(l1), _p(l2), _p(r0), _p(r1), _p(r2), _p(node_bound),
-                                            N, chan, _p(packed_weight_f16x2(W)), dim_out, _p(y), _stream()))
+                                            N, chan, _p(packed_weight_f16x2(W)), k_order, dim_out, _p(y), _stream()))
     return y
+
+
+_reordered_cache = {}
+
+
+def _channel_block_major_columns(W, n_types, chan):
+    """W (dim_out, n_types * chan) with its columns reordered from (type, channel) to (channel block of 32, type,
+    channel in block); cached per tensor object and version."""
+    key = (id(W), n_types, chan)
+    hit = _reordered_cache.get(key)
+    if hit is not None and hit[0]() is W and hit[1] == W._version and hit[2] == W.data_ptr():
+        return hit[3]
+    with torch.no_grad():
+        Wr = (W.detach().reshape(W.shape[0], n_types, chan // 32, 32).permute(0, 2, 1, 3)
+              .reshape(W.shape[0], n_types * chan).contiguous())
+    if len(_reordered_cache) > 256:
+        _reordered_cache.clear()
+    _reordered_cache[key] = (weakref.ref(W), W._version, W.data_ptr(), Wr)
+    return Wr
 
 
 def f16x2_rowsum_supported(rows, dim_in, dim_out, x):
