@@ -298,6 +298,14 @@ int mg_painn_filter_message(const void* packed_W3, const float* bias3, const flo
                             long n_nodes, long n_edges, int n, float epsilon, const float* res_a,
                             const float* res_v, void* workspace, float* out_a, float* out_v, mg_stream_t stream);
 
+/* mg_tensor_linear_f16x2_rowsum on bf16 storage: x (rows, dim_in) and the optional y (rows, dim_out) bfloat16,
+ * packed_W as for mg_tensor_linear_bf16, out (n_out, dim_out) float32 = scale * sum over the rows of each segment
+ * of the bfloat16-rounded act(bias + W x[r]) (the values y holds), accumulated in fp32.  dim_out % 128 == 0. */
+int mg_tensor_linear_bf16_rowsum_workspace_bytes(long rows, int dim_out, size_t* bytes);
+int mg_tensor_linear_bf16_rowsum(const void* packed_W, const void* x, long rows, int dim_in, int dim_out,
+                                 const float* bias, int act, const int* row_ptr, const int* seg, long n_out, float scale,
+                                 void* workspace, void* y, float* out, mg_stream_t stream);
+
 /* SelfTensProds.forward after its six input linears (archs/diffuser_atoms15.py:82-94), one output rank per call:
  *   y[node, o, comp] = sum over the product types `lab` of output rank rank_o, channels c of
  *                      Y[o, (lab, c)] * p_lab(l, r)[node, comp, c]

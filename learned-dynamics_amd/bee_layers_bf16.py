@@ -61,19 +61,26 @@ def mlp_forward(mlp, x, plus_identity=False):
     return out.to(torch.bfloat16)
 
 
-def mlp_summed_over_rows(mlp, x, row_ptr, n_out, plus_identity=False, scale=1.0):
+def mlp_summed_over_rows(mlp, x, row_ptr, n_out, plus_identity=False, scale=1.0, seg=None, s_x=None):
     """scale * (sum over each CSR segment of mlp_forward(mlp, x, plus_identity)) as bf16 (n_out, d).  The
     direct linear and the last layer are linear in their inputs, so they are applied to the summed rows
-    (bee_layers.MLP.summed_over_rows); the sums themselves are stored in bf16 like every other feature."""
+    (bee_layers.MLP.summed_over_rows).  With seg (the segment of every row) the second layer sums its
+    bf16-rounded output rows in its own epilogue and never stores them; s_x: the sums of x if the caller has
+    them.  Sums are accumulated in fp32 and stored in bf16 like every other feature."""
     Wd = mlp.lin_direct.weight
     if plus_identity:
         Wd = Wd + torch.eye(Wd.shape[0], device=Wd.device, dtype=Wd.dtype)
     Ls = mlp.layers
     h = ops.tensor_linear_bf16(Ls[0].weight, x, bias=Ls[0].bias, act=ops.ACT_LEAKY)
-    h = ops.tensor_linear_bf16(Ls[2].weight, h, bias=Ls[2].bias, act=ops.ACT_LEAKY)
-    s_x = ops.segment_sum_csr_bf16(x, row_ptr, n_out)
-    s_h = ops.segment_sum_csr_bf16(h, row_ptr, n_out)
+    if seg is not None and ops.bf16_rowsum_supported(h.shape[0], Ls[2].in_features, Ls[2].out_features):
+        s_h, _ = ops.tensor_linear_bf16_rowsum(Ls[2].weight, h, row_ptr, seg, n_out, bias=Ls[2].bias, act=ops.ACT_LEAKY)
+        s_h = s_h.to(torch.bfloat16)
+    else:
+        h = ops.tensor_linear_bf16(Ls[2].weight, h, bias=Ls[2].bias, act=ops.ACT_LEAKY)
+        s_h = ops.segment_sum_csr_bf16(h, row_ptr, n_out)
     del h
+    if s_x is None:
+        s_x = ops.segment_sum_csr_bf16(x, row_ptr, n_out)
     out = ops.tensor_linear_bf16(Wd, s_x, out_dtype=torch.float32)
     ops.tensor_linear_bf16(Ls[4].weight, s_h, out=out, accumulate=True)
     count = (row_ptr[1:] - row_ptr[:-1]).to(out.dtype)[:, None]
@@ -91,8 +98,15 @@ def messages_forward(mod: Messages, graph: Graph, r_ij, s_a, s_v, s_d, node_orde
     P0, S1, S2 = ops.bee_message_bf16(graph.row_ptr, graph.dst32, rhat, enc, La, Lv, Ld, mod.lin_enc.weight,
                                       mod.lin_enc.bias, node_order=node_order)
     E, chan = P0.shape[0], P0.shape[2]
-    psi_a = ops.tensor_linear_bf16(_cat_Y(mod, LABELS_0), P0.reshape(E, 3 * chan))
-    B_a = mlp_summed_over_rows(mod.mlp_a, psi_a, graph.row_ptr, rows, plus_identity=True, scale=0.1)
+    Y0 = _cat_Y(mod, LABELS_0)
+    if ops.bf16_rowsum_supported(E, 3 * chan, Y0.shape[0]):
+        s_psi, psi_a = ops.tensor_linear_bf16_rowsum(Y0, P0.reshape(E, 3 * chan), graph.row_ptr, graph.src32, rows,
+                                                     want_rows=True)
+        s_psi = s_psi.to(torch.bfloat16)
+    else:
+        psi_a, s_psi = ops.tensor_linear_bf16(Y0, P0.reshape(E, 3 * chan)), None
+    B_a = mlp_summed_over_rows(mod.mlp_a, psi_a, graph.row_ptr, rows, plus_identity=True, scale=0.1,
+                               seg=graph.src32, s_x=s_psi)
     B_v = _lin(_cat_Y(mod, LABELS_1, 0.1), S1.reshape(rows, 3, 5 * chan), 3)
     B_d = _lin(_cat_Y(mod, LABELS_2, 0.1), S2.reshape(rows, 9, 5 * chan), 9)
     return B_a, B_v, B_d

@@ -24,6 +24,7 @@
 //   order: fixed summation order, no atomics.
 #include "common.hpp"
 #include "f16x2.hpp"
+#include "rowsum_finish.hpp"
 
 namespace mg {
 namespace {
@@ -460,30 +461,6 @@ linear_rowsum_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restr
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
     }
-}
-
-// out[s] = scale * (slots of the blocks the rows of segment s lie in, in block order); segments strictly inside
-// one block were written by the kernel above, empty segments get zero.  One thread per four columns.
-__global__ void __launch_bounds__(256)
-rowsum_finish_kernel(const int* __restrict__ row_ptr, long n_out, long n_blocks, int O, const float* __restrict__ slots,
-                     float scale, float* __restrict__ out) {
-    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    const int quads = O / 4;
-    if (idx >= n_out * quads) return;
-    const long s_id = idx / quads;
-    const int x = (int)(idx - s_id * quads) * 4;
-    const long lo = row_ptr[s_id], hi = row_ptr[s_id + 1];
-    float4 s = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (hi > lo) {
-        const long b_lo = lo / 32, b_hi = (hi - 1) / 32;
-        if (b_lo == b_hi && lo > 32 * b_lo && hi - 1 < 32 * b_lo + 31) return;   // written directly
-        for (long b = b_lo; b <= b_hi; b++) {
-            const float* slot = 32 * b >= lo ? slots + b * O : slots + (n_blocks + b) * O;
-            const float4 t = ldf4(slot + x);
-            s.x += t.x; s.y += t.y; s.z += t.z; s.w += t.w;
-        }
-    }
-    *reinterpret_cast<float4*>(out + s_id * O + x) = make_float4(scale * s.x, scale * s.y, scale * s.z, scale * s.w);
 }
 
 // out(node) = res(node) + the partial sums of the blocks its edges lie in, in block order.  Nodes whose

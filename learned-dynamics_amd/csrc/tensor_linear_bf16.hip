@@ -23,6 +23,7 @@
 // v_mfma_f32_32x32x16_bf16: A[i][k]: lane = i + 32*(k/8), 8 k per lane; B[k][j] likewise;
 // D[i][j]: j = lane%32, i = 8*(q/4) + 4*(lane/32) + q%4 for register q.
 #include "common.hpp"
+#include "rowsum_finish.hpp"
 #include <type_traits>
 
 namespace mg {
@@ -54,11 +55,22 @@ __device__ __forceinline__ void store4(__bf16* p, floatx4 v) {
     *reinterpret_cast<bf16x4*>(p) = bf16x4{(__bf16)v[0], (__bf16)v[1], (__bf16)v[2], (__bf16)v[3]};
 }
 
-template <int WAVES, int NI, typename YT>
+// Sum of the output rows per segment in the epilogue (rows sorted by segment): seg[row] ascending, two partial
+// slots per block of 32 rows, runs inside a block written to `out` directly, as in the fp32 kernels that do this.
+struct RowSum {
+    const int* seg;
+    float* slots;
+    long n_blocks;
+    float* out;      // (segments, O) float32
+    float scale;
+    int store_y;     // also write the rows themselves
+};
+
+template <int WAVES, int NI, typename YT, bool ROWSUM = false>
 __global__ void __launch_bounds__(64 * WAVES)
 linear_rows_bf16_kernel(const __bf16* __restrict__ Wp, long plane_elems, int w_rows, const __bf16* __restrict__ X,
                         long R, int I, int O, const float* __restrict__ bias, int act, int accumulate,
-                        YT* __restrict__ Y, int tiles_n, long tiles_total, int out_T) {
+                        YT* __restrict__ Y, int tiles_n, long tiles_total, int out_T, RowSum rs = RowSum{}) {
     constexpr int TM = 32 * WAVES, TN = 32 * NI, THREADS = 64 * WAVES;
     constexpr int kPlaneW = TN * kRowW, kBufW = 2 * kPlaneW;
     constexpr int kPieces = 8 * TN;                          // 16-byte pieces of W per chunk (2 planes x TN rows x 4)
@@ -172,8 +184,22 @@ linear_rows_bf16_kernel(const __bf16* __restrict__ Wp, long plane_elems, int w_r
     constexpr int kColsFit = (kRegion - 512) / 64;                          // 32 rows x (2 cols + 16) bytes
     constexpr int kPassCols = kColsFit >= 128 ? 128 : (kColsFit >= 64 ? 64 : (kColsFit >= 32 ? 32 : 0));
     if constexpr (std::is_same<YT, __bf16>::value && kPassCols > 0) {
-        if (out_T == 1 && n0 + TN <= O && (O & 7) == 0 && !accumulate) {
+        if (ROWSUM || (out_T == 1 && n0 + TN <= O && (O & 7) == 0 && !accumulate)) {
             constexpr int kCols = kPassCols < TN ? kPassCols : TN;          // columns per pass
+            static_assert(!ROWSUM || kCols % 64 == 0, "the row sums take whole groups of 64 columns per pass");
+            // ROWSUM: runs of equal segment among the wave's rows (bit r set = row r starts a run)
+            const long block = r0 / 32 + wave;
+            int my_seg = 0, nv = 0, runs = 1, second = 32;
+            unsigned starts = 1u;
+            if constexpr (ROWSUM) {
+                my_seg = rs.seg[ld_row];
+                const long rows_left = R - block * 32;
+                nv = rows_left >= 32 ? 32 : (rows_left > 0 ? (int)rows_left : 0);
+                const int prev_seg = __shfl_up(my_seg, 1);
+                starts = (unsigned)__ballot(g == 0 && (m == 0 || my_seg != prev_seg));
+                runs = __popc(starts);
+                second = runs >= 2 ? __ffs(starts & ~1u) - 1 : 32;
+            }
             constexpr int kRowBytes = 2 * kCols + 16;
             constexpr int kPieces = 32 * kCols / 8;                         // 16-byte pieces per pass
             unsigned char* slice = lds + wave * kRegion;
@@ -191,19 +217,70 @@ linear_rows_bf16_kernel(const __bf16* __restrict__ Wp, long plane_elems, int w_r
                             if (brow) v += load4(brow + 32 * ni + 8 * qq);
 #pragma unroll
                             for (int i = 0; i < 4; i++) v[i] = activate_c<kAct>(v[i]);
+                            if constexpr (ROWSUM) {
+                                if (my_row >= R) v = floatx4{0.f, 0.f, 0.f, 0.f};      // rows past the end add nothing
+                            }
                             store4(reinterpret_cast<__bf16*>(slice + m * kRowBytes) + 32 * nl + 8 * qq + 4 * g, v);
                         }
                     }
                     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                     __builtin_amdgcn_wave_barrier();
+                    if (!ROWSUM || rs.store_y) {
 #pragma unroll
-                    for (int it = 0; it < (kPieces + 63) / 64; it++) {
-                        const int piece = it * 64 + lane;
-                        const int row = piece / (kCols / 8), c8 = piece % (kCols / 8);
-                        const long r = r0 + wave * 32 + row;
-                        if (piece < kPieces && r < R) {
-                            const bf16x8 t = *reinterpret_cast<const bf16x8*>(slice + row * kRowBytes + c8 * 16);
-                            *reinterpret_cast<bf16x8*>(Y + r * O + n0 + pass * kCols + c8 * 8) = t;
+                        for (int it = 0; it < (kPieces + 63) / 64; it++) {
+                            const int piece = it * 64 + lane;
+                            const int row = piece / (kCols / 8), c8 = piece % (kCols / 8);
+                            const long r = r0 + wave * 32 + row;
+                            if (piece < kPieces && r < R) {
+                                const bf16x8 t = *reinterpret_cast<const bf16x8*>(slice + row * kRowBytes + c8 * 16);
+                                *reinterpret_cast<bf16x8*>(Y + r * O + n0 + pass * kCols + c8 * 8) = t;
+                            }
+                        }
+                    }
+                    if constexpr (ROWSUM) {
+                        // lanes take one column (two with 128-column passes) and add the bf16 values of the rows
+                        // in fp32, split at the run boundaries
+                        if (nv > 0) {
+#pragma unroll
+                            for (int cc = 0; cc < (kCols + 63) / 64; cc++) {
+                                const int cl = cc * 64 + lane;                       // column in this pass
+                                if (cl < kCols) {
+                                    const int col = n0 + pass * kCols + cl;
+                                    const __bf16* colp = reinterpret_cast<const __bf16*>(slice) + cl;
+                                    auto flush = [&](float sum, int run_start, int r) {
+                                        if (run_start == 0) {
+                                            rs.slots[block * O + col] = sum;
+                                        } else if (r == 31) {
+                                            rs.slots[(rs.n_blocks + block) * O + col] = sum;
+                                        } else {
+                                            const long s_id = __shfl(my_seg, r);
+                                            rs.out[s_id * O + col] = rs.scale * sum;
+                                        }
+                                    };
+                                    if (runs <= 2) {
+                                        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+                                        for (int r = 0; r < 32; r++) {
+                                            const float val = (float)colp[r * (kRowBytes / 2)];
+                                            s0 += r < second ? val : 0.f;
+                                            s1 += r < second ? 0.f : val;
+                                        }
+                                        flush(s0, 0, second - 1);
+                                        if (runs == 2) flush(s1, second, nv - 1);
+                                    } else {
+                                        float sum = 0.f;
+                                        int run_start = 0;
+                                        for (int r = 0; r < nv; r++) {
+                                            sum += (float)colp[r * (kRowBytes / 2)];
+                                            if ((r == nv - 1) || ((starts >> (r + 1)) & 1u)) {
+                                                flush(sum, run_start, r);
+                                                sum = 0.f;
+                                                run_start = r + 1;
+                                            }
+                                        }
+                                    }
+                                }
+                            }
                         }
                     }
                     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -301,12 +378,62 @@ int dispatch(const __bf16* Wp, long plane_elems, int w_rows, const __bf16* x, lo
 #undef MG_BF16_LAUNCH
 }
 
+template <int NI>
+int launch_rowsum(const __bf16* Wp, long plane_elems, int w_rows, const __bf16* x, long rows, int I, int O,
+                  const float* bias, int act, __bf16* y, const RowSum& rs, hipStream_t st) {
+    const long tiles_m = ceil_div(rows, 256);
+    const int tiles_n = O / (32 * NI);
+    const long total = tiles_m * tiles_n;
+    const long grid = ceil_div(total, 8) * 8;
+    MG_REQUIRE(grid <= 0x7fffffffL, "mg_tensor_linear_bf16_rowsum: grid too large");
+    hipLaunchKernelGGL((linear_rows_bf16_kernel<8, NI, __bf16, true>), dim3((unsigned)grid), dim3(512), 0, st, Wp,
+                       plane_elems, w_rows, x, rows, I, O, bias, act, 0, y, tiles_n, total, 1, rs);
+    return check_launch("mg_tensor_linear_bf16_rowsum");
+}
+
 }  // namespace
 }  // namespace mg
 
 using namespace mg;
 
 extern "C" {
+
+int mg_tensor_linear_bf16_rowsum_workspace_bytes(long rows, int dim_out, size_t* bytes) {
+    MG_REQUIRE(bytes != nullptr && rows >= 0 && dim_out >= 0, "mg_tensor_linear_bf16_rowsum_workspace_bytes: bad argument");
+    *bytes = (size_t)(2L * (ceil_div(rows, 32) + 1) * dim_out) * sizeof(float);
+    return MG_OK;
+}
+
+int mg_tensor_linear_bf16_rowsum(const void* packed_W, const void* x, long rows, int dim_in, int dim_out,
+                                 const float* bias, int act, const int* row_ptr, const int* seg, long n_out, float scale,
+                                 void* workspace, void* y, float* out, mg_stream_t stream) {
+    MG_REQUIRE(dim_out >= 128 && dim_out % 128 == 0, "mg_tensor_linear_bf16_rowsum: dim_out must be a multiple of 128 (got %d)", dim_out);
+    MG_REQUIRE(dim_in > 0 && dim_in % 32 == 0, "mg_tensor_linear_bf16_rowsum: dim_in must be a multiple of 32 (got %d)", dim_in);
+    MG_REQUIRE(rows >= 0 && n_out >= 0 && rows < (1L << 31) && n_out < (1L << 31), "mg_tensor_linear_bf16_rowsum: bad size");
+    MG_REQUIRE(act >= 0 && act <= 2, "mg_tensor_linear_bf16_rowsum: unknown activation %d", act);
+    if (n_out == 0) return MG_OK;
+    MG_REQUIRE(packed_W && row_ptr && out && aligned16(packed_W) && aligned16(out) && (!bias || aligned16(bias)),
+               "mg_tensor_linear_bf16_rowsum: null or unaligned operand");
+    hipStream_t st = (hipStream_t)stream;
+    const long n_blocks = ceil_div(rows, 32);
+    if (rows > 0) {
+        MG_REQUIRE(x && seg && workspace && aligned16(x) && aligned16(workspace) && (!y || aligned16(y)),
+                   "mg_tensor_linear_bf16_rowsum: null or unaligned row operand");
+        const int w_rows = (int)ceil_div(dim_out, 128) * 128;
+        const long plane_elems = (long)w_rows * dim_in;
+        RowSum rs{seg, static_cast<float*>(workspace), n_blocks, out, scale, y != nullptr};
+        const int st_code = dim_out % 256 == 0
+            ? launch_rowsum<8>(static_cast<const __bf16*>(packed_W), plane_elems, w_rows, static_cast<const __bf16*>(x),
+                               rows, dim_in, dim_out, bias, act, static_cast<__bf16*>(y), rs, st)
+            : launch_rowsum<4>(static_cast<const __bf16*>(packed_W), plane_elems, w_rows, static_cast<const __bf16*>(x),
+                               rows, dim_in, dim_out, bias, act, static_cast<__bf16*>(y), rs, st);
+        if (st_code) return st_code;
+    }
+    const long threads = n_out * (dim_out / 4);
+    rowsum_finish_kernel<<<dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, st>>>(
+        row_ptr, n_out, n_blocks, dim_out, static_cast<const float*>(workspace), scale, out);
+    return check_launch("rowsum_finish_kernel");
+}
 
 int mg_tensor_linear_bf16(const void* packed_W, const void* x, long rows, int dim_in, int dim_out, const float* bias,
                           int act, int accumulate, int out_comps, int y_is_bf16, void* y, mg_stream_t stream) {

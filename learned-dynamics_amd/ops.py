@@ -888,6 +888,37 @@ def bee_node_products(l0, l1, l2, r0, r1, r2, want_node_max=False):
     return (P0, P1, P2, node_max) if want_node_max else (P0, P1, P2)
 
 
+def bf16_rowsum_supported(rows, dim_in, dim_out):
+    return dim_out % 128 == 0 and dim_in % 32 == 0 and rows >= 4096
+
+
+def tensor_linear_bf16_rowsum(W, x, row_ptr, seg, n_out, bias=None, act=ACT_NONE, scale=1.0, want_rows=False):
+    """(out, y): out (n_out, dim_out) float32 = scale * sum over the rows of each segment of the bfloat16-rounded
+    act(bias + W x[r]); y (rows, dim_out) bfloat16 with want_rows, else None.  x (rows, dim_in) bfloat16 sorted by
+    segment: seg (rows,) int32 ascending, row_ptr its CSR form."""
+    _check_bf16(x, "x")
+    _check_input(W, "W")
+    for t, nm in ((row_ptr, "row_ptr"), (seg, "seg")):
+        _check_input(t, nm, torch.int32)
+    if x.dim() != 2 or W.dim() != 2 or x.size(1) != W.size(1):
+        raise RuntimeError("x must have shape (rows, dim_in) and W (dim_out, dim_in)")
+    rows, dim_in, dim_out = int(x.size(0)), int(W.size(1)), int(W.size(0))
+    if seg.numel() != rows or row_ptr.numel() != n_out + 1:
+        raise RuntimeError("seg must have one entry per row and row_ptr n_out + 1 entries")
+    if bias is not None and (bias.dtype != torch.float32 or not bias.is_contiguous() or bias.numel() != dim_out):
+        raise RuntimeError("bias must be a contiguous float32 tensor of dim_out elements")
+    nbytes = ctypes.c_size_t(0)
+    L.check(_lib.mg_tensor_linear_bf16_rowsum_workspace_bytes(rows, dim_out, ctypes.byref(nbytes)))
+    with torch.cuda.device(x.device):
+        out = torch.empty(n_out, dim_out, dtype=torch.float32, device=x.device)
+        y = torch.empty(rows, dim_out, dtype=torch.bfloat16, device=x.device) if want_rows else None
+        work = torch.empty(nbytes.value // 4, dtype=torch.float32, device=x.device)
+        L.check(_lib.mg_tensor_linear_bf16_rowsum(_p(packed_weight(W)), _p(x), rows, dim_in, dim_out, _p(bias), int(act),
+                                                  _p(row_ptr), _p(seg), int(n_out), float(scale), _p(work), _p(y),
+                                                  _p(out), _stream()))
+    return out, y
+
+
 def segment_sum_csr_bf16(x_edge, row_ptr, n_rows, scale=1.0):
     """scale * (sum of the bfloat16 edge rows of each CSR row), fp32 accumulation, bfloat16 result."""
     _check_bf16(x_edge, "x_edge")

@@ -180,3 +180,38 @@ def test_stack_bf16_against_fp32_oracle(pkg):
         err = (out.cpu().double() - ref).abs()
         assert float(err.max()) <= 1e-2 * scale, (float(err.max()), scale)
         assert float(err.pow(2).mean().sqrt()) <= 1e-2 * float(ref.pow(2).mean().sqrt())
+
+
+@pytest.mark.parametrize("dim_in,dim_out,act,kind,want_rows", [(256, 256, 2, "long", False), (384, 128, 0, "short", True),
+                                                               (64, 384, 1, "aligned", True), (128, 512, 2, "mixed", False)])
+def test_linear_bf16_with_row_sums_in_the_epilogue(ops, dim_in, dim_out, act, kind, want_rows):
+    """out[s] = scale * sum over the rows of segment s of the bf16-rounded act(x W^T + b): exactly the fp32 sum
+    of what mg_tensor_linear_bf16 writes (order of additions aside), for segments placed in every way relative
+    to the kernel's 32-row blocks."""
+    g = torch.Generator().manual_seed(dim_in + dim_out)
+    n_seg = 300
+    if kind == "long":
+        lengths = torch.randint(40, 140, (n_seg,), generator=g)
+    elif kind == "short":
+        lengths = torch.randint(0, 9, (n_seg,), generator=g)
+    elif kind == "aligned":
+        lengths = torch.tensor([32, 64, 1, 31, 32, 0, 0, 96, 33, 31] * (n_seg // 10))
+    else:
+        lengths = torch.cat([torch.randint(0, 5, (n_seg // 2,), generator=g),
+                             torch.randint(20, 300, (n_seg - n_seg // 2,), generator=g)])[torch.randperm(n_seg, generator=g)]
+    seg = torch.repeat_interleave(torch.arange(n_seg), lengths)
+    rows = int(seg.numel())
+    x = torch.randn(rows, dim_in, generator=g).cuda().to(torch.bfloat16)
+    W = (torch.randn(dim_out, dim_in, generator=g) / dim_in ** 0.5).cuda()
+    b = torch.randn(dim_out, generator=g).cuda()
+    row_ptr = ops.segment_row_ptr(seg.int().cuda(), n_seg)
+    out, y = ops.tensor_linear_bf16_rowsum(W, x, row_ptr, seg.int().cuda(), n_seg, bias=b, act=act, scale=0.5,
+                                           want_rows=want_rows)
+    y_ref = ops.tensor_linear_bf16(W, x, bias=b, act=act)
+    if want_rows:
+        assert torch.equal(y, y_ref)
+    else:
+        assert y is None
+    ref = 0.5 * torch.zeros(n_seg, dim_out, dtype=torch.float64).index_add_(0, seg, y_ref.double().cpu())
+    torch.testing.assert_close(out.cpu().double(), ref, rtol=1e-5, atol=2e-6 * float(ref.abs().max()))
+    assert not bool(out[(lengths == 0).cuda()].any())
