@@ -306,6 +306,13 @@ int mg_tensor_linear_bf16_rowsum(const void* packed_W, const void* x, long rows,
                                  const float* bias, int act, const int* row_ptr, const int* seg, long n_out, float scale,
                                  void* workspace, void* y, float* out, mg_stream_t stream);
 
+/* x (rows, dim, comps) in the reference's tensor layout (managan/tensor_products.py:17-24: channel, then the 3^k
+ * components) -> xt (rows * comps, dim_pad): one plain GEMM row per (row, component) with the channels zero-padded
+ * to dim_pad (a power of two, 32..256), and rowmax (rows * comps): max |xt| per output row.  What
+ * mg_tensor_linear_f16x2 needs to apply a TensLinear to many rows with component-major output. */
+int mg_components_to_rows(const float* x, long rows, int dim, int comps, int dim_pad, float* xt, float* rowmax,
+                          mg_stream_t stream);
+
 /* SelfTensProds.forward after its six input linears (archs/diffuser_atoms15.py:82-94), one output rank per call:
  *   y[node, o, comp] = sum over the product types `lab` of output rank rank_o, channels c of
  *                      Y[o, (lab, c)] * p_lab(l, r)[node, comp, c]

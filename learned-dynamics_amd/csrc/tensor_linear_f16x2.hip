@@ -100,6 +100,28 @@ __global__ void __launch_bounds__(256) row_absmax_kernel(const float* __restrict
 }
 
 
+// x (rows, K, T) in the reference's tensor layout (channel, then components) -> xt (rows * T, K_pad): one plain
+// GEMM row per (row, component), channels zero-padded to K_pad, and the maximum of |xt| per output row.
+// A thread writes four consecutive channels of one output row; the K_pad / 4 threads of a row are neighbours.
+__global__ void __launch_bounds__(256) components_to_rows_kernel(const float* __restrict__ x, long rows, int K, int T,
+                                                                 int K_pad, float* __restrict__ xt,
+                                                                 float* __restrict__ rowmax) {
+    const int per_row = K_pad / 4;                            // 8, 16, ...: a power of two <= 64
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long out_row = idx / per_row;
+    const int k0 = (int)(idx - out_row * per_row) * 4;
+    const bool live = out_row < rows * T;
+    const long r = live ? out_row / T : 0;
+    const int t = live ? (int)(out_row - r * T) : 0;
+    float v[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) v[j] = (live && k0 + j < K) ? x[(r * K + k0 + j) * T + t] : 0.f;
+    if (live) *reinterpret_cast<float4*>(xt + out_row * K_pad + k0) = make_float4(v[0], v[1], v[2], v[3]);
+    float mx = fmaxf(fmaxf(fabsf(v[0]), fabsf(v[1])), fmaxf(fabsf(v[2]), fabsf(v[3])));
+    for (int d = 1; d < per_row; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+    if (live && k0 == 0) rowmax[out_row] = mx;
+}
+
 template <int WAVES, int NI>
 __global__ void __launch_bounds__(64 * WAVES)
 linear_rows_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restrict__ w_inv, const float* __restrict__ X,
@@ -403,6 +425,19 @@ int mg_row_absmax(const float* x, long rows, int dim, float* out, mg_stream_t st
     if (blocks > 256L * 32) blocks = 256L * 32;
     hipLaunchKernelGGL(row_absmax_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, x, rows, dim, out);
     return check_launch("mg_row_absmax");
+}
+
+int mg_components_to_rows(const float* x, long rows, int dim, int comps, int dim_pad, float* xt, float* rowmax,
+                          mg_stream_t stream) {
+    MG_REQUIRE(rows >= 0 && dim > 0 && comps > 0, "mg_components_to_rows: bad size");
+    MG_REQUIRE(dim_pad >= dim && dim_pad % 32 == 0 && dim_pad <= 256 && (dim_pad & (dim_pad - 1)) == 0,
+               "mg_components_to_rows: dim_pad must be a power of two in 32..256, at least dim (got %d for %d)", dim_pad, dim);
+    if (rows == 0) return MG_OK;
+    MG_REQUIRE(x && xt && rowmax && aligned16(xt), "mg_components_to_rows: null or unaligned pointer");
+    const long threads = rows * comps * (dim_pad / 4);
+    hipLaunchKernelGGL(components_to_rows_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
+                       (hipStream_t)stream, x, rows, dim, comps, dim_pad, xt, rowmax);
+    return check_launch("mg_components_to_rows");
 }
 
 int mg_tensor_linear_f16x2_rowmax_parts(long rows, int dim_in, int dim_out) {

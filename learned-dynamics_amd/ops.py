@@ -746,12 +746,19 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
             # matrix path: its component-major output is written at the full store rate, which the generic
             # kernel's layout mapping is not
             k_pad = (dim_in + 31) // 32 * 32
-            xt = x.reshape(rows, dim_in, T).transpose(1, 2)
-            xt = torch.nn.functional.pad(xt, (0, k_pad - dim_in)) if k_pad != dim_in else xt.contiguous()
-            x2 = xt.reshape(rows * T, k_pad)
+            if k_pad <= 256 and k_pad & (k_pad - 1) == 0:
+                # transposition, padding and the row maxima in one pass
+                x2 = torch.empty(rows * T, k_pad, dtype=torch.float32, device=x.device)
+                x2max = torch.empty(rows * T, 1, dtype=torch.float32, device=x.device)
+                L.check(_lib.mg_components_to_rows(_p(x), rows, dim_in, T, k_pad, _p(x2), _p(x2max), _stream()))
+            else:
+                xt = x.reshape(rows, dim_in, T).transpose(1, 2)
+                xt = torch.nn.functional.pad(xt, (0, k_pad - dim_in)) if k_pad != dim_in else xt.contiguous()
+                x2 = xt.reshape(rows * T, k_pad)
+                x2max = row_absmax(x2)
             Wp = _zero_padded_columns(W, k_pad)
             ymax = rowmax_buffer(k_pad)
-            L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(Wp)), _p(x2), _p(row_absmax(x2)), 1, 1, 1,
+            L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(Wp)), _p(x2), _p(x2max), 1, 1, 1,
                                                 rows * T, k_pad, dim_out, _p(bias), int(act), int(bool(accumulate)),
                                                 1, _p(y), _p(ymax), _stream()))
         elif (plain_rows and mode == LINEAR_F16X2 and f16x2_supported(rows * T, dim_in, dim_out, x)):

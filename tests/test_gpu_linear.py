@@ -253,7 +253,7 @@ def test_linear_with_row_sums_in_the_epilogue(ops, dim_in, dim_out, act, kind, w
     assert not bool(out[(lengths == 0).cuda()].any())
 
 
-@pytest.mark.parametrize("inds,rows,dim_in,dim_out", [(2, 8000, 16, 64), (1, 22000, 40, 96), (1, 30000, 64, 256)])
+@pytest.mark.parametrize("inds,rows,dim_in,dim_out", [(2, 8000, 16, 64), (1, 22000, 40, 96), (1, 30000, 64, 256), (1, 25000, 70, 64)])
 def test_component_major_output_from_reference_layout_at_many_rows(ops, inds, rows, dim_in, dim_out):
     """x in the reference layout (rows, chan, 3..), y component-major (rows, 3^inds, chan_out): at many rows
     the dispatcher transposes x and uses the plain-row matrix path (K zero-padded to a multiple of 32).
