@@ -280,6 +280,17 @@ int mg_painn_message(const int* row_ptr /* n_nodes+1 */, const int* dst /* E */,
                      int n, float epsilon, const float* res_a, const float* res_v,
                      float* out_a /* (n_nodes,n) */, float* out_v /* (n_nodes,n,3) */, mg_stream_t stream);
 
+/* The first two layers of the radial MLP from the edge vectors (archs/meanflow_painn8.py:25-35 feeding :38-51):
+ *   y[e] = SiLU(b2 + W2 SiLU(b1 + W1 radial_encode(r_ij[e], 16, rmax))),   y (E, hidden)
+ * in one kernel; the first layer's output is produced chunk by chunk on the matrix cores and never stored.
+ * 16 radial functions; hidden = 256 or 512.  W1 (hidden, 16) float32 with the given strides; packed_W2:
+ * mg_linear_f16x2_pack_weight of W2 (hidden, hidden) with its INPUT channels permuted inside every group of 32:
+ * position 16 g + p (g = 0, 1; p = 0..15) holds channel 8 (p / 4) + 4 g + p % 4.  h1_bound (1 float, device): an
+ * upper bound of |SiLU(b1 + W1 enc)| (e.g. max_o sum_i |W1[o,i]| + max |b1|: the encodings are at most 1). */
+int mg_painn_filter_hidden(const float* r_ij, long n_edges, float rmax, const float* W1, long w1_stride_o,
+                           long w1_stride_i, const float* b1, const void* packed_W2, const float* b2, int hidden,
+                           const float* h1_bound, float* y, mg_stream_t stream);
+
 /* mg_painn_message with the LAST layer of the radial MLP folded in (archs/meanflow_painn8.py:38-51 at :92,
  * then :93-100): filt[e] = bias3 + W3 h[e] is produced on the matrix cores (split-fp16 arithmetic, as
  * mg_tensor_linear_f16x2) and consumed in the same kernel, so the (E,4n) filter is never stored.

@@ -50,12 +50,26 @@ constexpr int kFSlice = 2 * kFBufW / kFW / 4;                    // floats of LD
 constexpr int kFRed = 68;                                        // floats per row of a slice: 64 + 4 (spreads 16-byte writes over the banks)
 static_assert(kFSlice >= 32 * kFRed, "a reduction pass needs 32 rows x 64 columns per wave");
 
+// Source of the second operand: the 16 values x[row][k0 + 16 g ..] of this lane's row for chunk k0, from memory
+struct RowFromMemory {
+    static constexpr bool kAhead = true;      // requested two chunks before use (HBM latency)
+    const float* xrow;       // this lane's row of x, offset by 16 (lane / 32)
+    int I;
+    __device__ __forceinline__ void operator()(float4 (&v)[4], int k0) const {
+        k0 = k0 < I ? k0 : I - kCK;                       // surplus requests of the last trips are never used
+#pragma unroll
+        for (int j = 0; j < 4; j++) v[j] = *reinterpret_cast<const float4*>(xrow + k0 + 4 * j);
+    }
+};
+
 // acc[ni][q] += sum_k W[n0 + 32 ni + i][k] x[row][k] for the wave's 32 rows (row = lane % 32) and the tile's 256
 // columns, i = 8 (q / 4) + 4 (lane / 32) + q % 4: the split-fp16 row-streaming main loop with W as the first
-// matrix operand.  xrow: this lane's row of x, offset by 16 (lane / 32); lds: 2 * kFBufW bytes; all waves of
-// the workgroup call it together, and the W buffers are free again when it returns.
+// matrix operand.  a_src(v, k0) delivers the lane's 16 values of x for chunk k0 (two chunks ahead of their use);
+// lds: 2 * kFBufW bytes; all waves of the workgroup call it together, and the W buffers are free again when it
+// returns.
+template <typename ASrc>
 __device__ __forceinline__ void wfirst_gemm_tile(floatx16 (&acc)[kFNI], const _Float16* __restrict__ Wp,
-                                                 long plane_elems, int n0, const float* __restrict__ xrow, int I,
+                                                 long plane_elems, int n0, const ASrc& a_src, int I,
                                                  float sx, unsigned char* lds) {
     constexpr int THREADS = kFThreads, kPlaneW = kFPlaneW, kBufW = kFBufW;
     constexpr int kPer = 8 * kFTN / THREADS;                 // 16-byte pieces of W per thread and chunk
@@ -74,11 +88,7 @@ __device__ __forceinline__ void wfirst_gemm_tile(floatx16 (&acc)[kFNI], const _F
 
     struct ARegs { float4 v[4]; };
     struct WRegs { halfx8 v[kPer]; };
-    auto load_a = [&](ARegs& a, int k0) {
-        k0 = k0 < I ? k0 : k_last;
-#pragma unroll
-        for (int j = 0; j < 4; j++) a.v[j] = *reinterpret_cast<const float4*>(xrow + k0 + 4 * j);
-    };
+    auto load_a = [&](ARegs& a, int k0) { a_src(a.v, k0); };
     auto load_w = [&](WRegs& w, int k0) {
         k0 = k0 < I ? k0 : k_last;
 #pragma unroll
@@ -115,29 +125,51 @@ __device__ __forceinline__ void wfirst_gemm_tile(floatx16 (&acc)[kFNI], const _F
 
     unsigned char* buf0 = lds;
     unsigned char* buf1 = lds + kBufW;
-    ARegs a0, a1;
     WRegs w;
-    load_w(w, 0);
-    load_a(a0, 0);
-    store_w(w, buf0);
-    load_w(w, kCK);
-    load_a(a1, kCK);
-    __syncthreads();
-    for (int k0 = 0; k0 < I; k0 += 2 * kCK) {
-        compute(a0, buf0, sx);
-        store_w(w, buf1);
-        __builtin_amdgcn_sched_barrier(0);
-        load_w(w, k0 + 2 * kCK);
-        __builtin_amdgcn_sched_barrier(0);
-        load_a(a0, k0 + 2 * kCK);
-        __syncthreads();
-        compute(a1, buf1, k0 + kCK < I ? sx : 0.f);
+    if constexpr (ASrc::kAhead) {
+        ARegs a0, a1;
+        load_w(w, 0);
+        load_a(a0, 0);
         store_w(w, buf0);
-        __builtin_amdgcn_sched_barrier(0);
-        load_w(w, k0 + 3 * kCK);
-        __builtin_amdgcn_sched_barrier(0);
-        load_a(a1, k0 + 3 * kCK);
+        load_w(w, kCK);
+        load_a(a1, kCK);
         __syncthreads();
+        for (int k0 = 0; k0 < I; k0 += 2 * kCK) {
+            compute(a0, buf0, sx);
+            store_w(w, buf1);
+            __builtin_amdgcn_sched_barrier(0);
+            load_w(w, k0 + 2 * kCK);
+            __builtin_amdgcn_sched_barrier(0);
+            load_a(a0, k0 + 2 * kCK);
+            __syncthreads();
+            compute(a1, buf1, k0 + kCK < I ? sx : 0.f);
+            store_w(w, buf0);
+            __builtin_amdgcn_sched_barrier(0);
+            load_w(w, k0 + 3 * kCK);
+            __builtin_amdgcn_sched_barrier(0);
+            load_a(a1, k0 + 3 * kCK);
+            __syncthreads();
+        }
+    } else {
+        ARegs a;
+        load_w(w, 0);
+        store_w(w, buf0);
+        load_w(w, kCK);
+        __syncthreads();
+        for (int k0 = 0; k0 < I; k0 += 2 * kCK) {
+            load_a(a, k0);
+            compute(a, buf0, sx);
+            store_w(w, buf1);
+            __builtin_amdgcn_sched_barrier(0);
+            load_w(w, k0 + 2 * kCK);
+            __syncthreads();
+            load_a(a, k0 + kCK);
+            compute(a, buf1, k0 + kCK < I ? sx : 0.f);
+            store_w(w, buf0);
+            __builtin_amdgcn_sched_barrier(0);
+            load_w(w, k0 + 3 * kCK);
+            __syncthreads();
+        }
     }
 }
 
@@ -194,7 +226,7 @@ painn_filter_message_kernel(const _Float16* __restrict__ Wp, const float* __rest
         wb[tid] = w_inv[n0 + tid];
         wb[kFTN + tid] = bias[n0 + tid];
     }
-    wfirst_gemm_tile(acc, Wp, plane_elems, n0, xrow, I, sx, lds);
+    wfirst_gemm_tile(acc, Wp, plane_elems, n0, RowFromMemory{xrow, I}, I, sx, lds);
     // every wave is past its last read of the W buffers: LDS is now eight private slices
 
     const bool valid = my_row < R;
@@ -380,7 +412,7 @@ linear_rowsum_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restr
         wb[tid] = w_inv[n0 + tid];
         wb[kFTN + tid] = bias ? bias[n0 + tid] : 0.f;
     }
-    wfirst_gemm_tile(acc, Wp, plane_elems, n0, xrow, I, sx, lds);
+    wfirst_gemm_tile(acc, Wp, plane_elems, n0, RowFromMemory{xrow, I}, I, sx, lds);
 
     const float keep = my_row < R ? 1.f : 0.f;               // rows past the end add nothing
     const long rows_left = R - block * 32;
@@ -457,6 +489,166 @@ linear_rowsum_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restr
                 }
             }
         }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// First two layers of the PaiNN filter MLP from the edge vectors (archs/meanflow_painn8.py:25-35 feeding
+// :38-51): y = SiLU(W2 SiLU(W1 enc(|r|) + b1) + b2), y (edges, hidden), with the first layer's output never
+// stored.  The first layer has K = 16, exactly one matrix-core step: for every 32-column chunk of its output
+// the generator below runs three split-fp16 MFMAs (W1 block x encodings) and lands the chunk in registers in
+// the accumulator layout, which IS the operand layout the second layer's main loop wants (lane = edge, 16 of
+// the chunk's 32 channels per lane half) up to a fixed permutation of the channels inside a chunk; the caller
+// packs W2 with its input channels in that order (position 16 g + p of a chunk holds channel
+// 8 (p / 4) + 4 g + p % 4).
+constexpr int kHidMax = 512;
+
+struct HiddenFromDistance {
+    static constexpr bool kAhead = false;     // built right before use: LDS and matrix-core latency only
+    const _Float16* w1h;     // LDS: W1 (hidden, 16) hi / lo halves, each row scaled by a power of two
+    const _Float16* w1l;
+    const float* w1inv;      // LDS: 1 / (row scale * 2^14)
+    const float* b1;         // LDS
+    halfx8 eh, el;           // this lane's 8 encodings k = 8 g .. 8 g + 7, times 2^14, as hi + lo
+    int I, m, g;
+    __device__ __forceinline__ void operator()(float4 (&v)[4], int k0) const {
+        k0 = k0 < I ? k0 : I - kCK;
+        const halfx8 ah = *reinterpret_cast<const halfx8*>(w1h + (k0 + m) * 16 + 8 * g);
+        const halfx8 al = *reinterpret_cast<const halfx8*>(w1l + (k0 + m) * 16 + 8 * g);
+        floatx16 d;
+#pragma unroll
+        for (int q = 0; q < 16; q++) d[q] = 0.f;
+        d = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, el, d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, eh, d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, eh, d, 0, 0, 0);
+#pragma unroll
+        for (int qq = 0; qq < 4; qq++) {
+            const float4 iw = *reinterpret_cast<const float4*>(w1inv + k0 + 8 * qq + 4 * g);
+            const float4 bv = *reinterpret_cast<const float4*>(b1 + k0 + 8 * qq + 4 * g);
+            v[qq].x = activate_c<1>(d[4 * qq + 0] * iw.x + bv.x);
+            v[qq].y = activate_c<1>(d[4 * qq + 1] * iw.y + bv.y);
+            v[qq].z = activate_c<1>(d[4 * qq + 2] * iw.z + bv.z);
+            v[qq].w = activate_c<1>(d[4 * qq + 3] * iw.w + bv.w);
+        }
+    }
+};
+
+__global__ void __launch_bounds__(64 * kFW)
+painn_filter_hidden_kernel(const _Float16* __restrict__ Wp, const float* __restrict__ w_inv,
+                           const float* __restrict__ bias2, const float* __restrict__ r_ij, long R, float base,
+                           const float* __restrict__ W1, long so, long si, const float* __restrict__ b1g, int hidden,
+                           const float* __restrict__ h1_bound, float* __restrict__ Y, int tiles_n, long tiles_total) {
+    constexpr int kSlice = kFSlice, kRed = kFRed;
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kFBufW];
+    __shared__ __attribute__((aligned(16))) float wb[2 * kFTN];
+    __shared__ __attribute__((aligned(16))) _Float16 w1h[kHidMax * 16];
+    __shared__ __attribute__((aligned(16))) _Float16 w1l[kHidMax * 16];
+    __shared__ __attribute__((aligned(16))) float w1inv[kHidMax];
+    __shared__ __attribute__((aligned(16))) float b1s[kHidMax];
+
+    const long bid = blockIdx.x;
+    const long per_xcd = (tiles_total + 7) / 8;
+    const long logical = (bid % 8) * per_xcd + bid / 8;
+    if (logical >= tiles_total) return;
+    const long tile_m = logical / tiles_n;
+    const int tile_n = (int)(logical - tile_m * tiles_n);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int m = lane & 31, g = lane >> 5;
+    const int n0 = tile_n * kFTN;
+    const int I = hidden, O = hidden;
+    const long plane_elems = (long)O * I;
+
+    // first-layer weights: one row per thread, split into fp16 hi + lo under a per-row power-of-two scale
+    for (int t = tid; t < hidden; t += kFThreads) {
+        float wrow[16];
+        float amax = 0.f;
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            wrow[k] = W1[t * so + k * si];
+            amax = fmaxf(amax, fabsf(wrow[k]));
+        }
+        float inv;
+        const float sc = pow2_scale(amax, &inv);
+#pragma unroll
+        for (int k = 0; k < 16; k++) {
+            const float sv = wrow[k] * sc;
+            const _Float16 h = (_Float16)sv;
+            w1h[t * 16 + k] = h;
+            w1l[t * 16 + k] = (_Float16)(sv - (float)h);
+        }
+        w1inv[t] = inv * (1.0f / 16384.0f);                  // the encodings are scaled by 2^14
+        b1s[t] = b1g ? b1g[t] : 0.f;
+    }
+    if (tid < kFTN) {
+        wb[tid] = w_inv[n0 + tid];
+        wb[kFTN + tid] = bias2 ? bias2[n0 + tid] : 0.f;
+    }
+
+    floatx16 acc[kFNI];
+#pragma unroll
+    for (int ni = 0; ni < kFNI; ni++)
+#pragma unroll
+        for (int q = 0; q < 16; q++) acc[ni][q] = 0.f;
+
+    const long block = tile_m * kFW + wave;
+    const long my_row = block * 32 + m;
+    const long ld_row = my_row < R ? my_row : R - 1;
+    float sx, isx;
+    sx = pow2_scale(h1_bound[0], &isx);
+
+    // the lane's half of the 16 radial encodings of its edge (archs/meanflow_painn8.py:25-35 with n = 16:
+    // entries 0..7 are cos, 8..15 sin of (pi / rmax) (1 + f / 2) d, f = entry % 8)
+    HiddenFromDistance gen;
+    {
+        const float x = r_ij[3 * ld_row], y = r_ij[3 * ld_row + 1], z = r_ij[3 * ld_row + 2];
+        const float dist = sqrtf(x * x + y * y + z * z);
+#pragma unroll
+        for (int i = 0; i < 8; i++) {
+            const float phase = (base * (float)(1 + i / 2)) * dist;
+            const float e = (g == 0 ? cosf(phase) : sinf(phase)) * 16384.0f;
+            const _Float16 h = (_Float16)e;
+            gen.eh[i] = h;
+            gen.el[i] = (_Float16)(e - (float)h);
+        }
+    }
+    gen.w1h = w1h; gen.w1l = w1l; gen.w1inv = w1inv; gen.b1 = b1s; gen.I = I; gen.m = m; gen.g = g;
+    __syncthreads();                                         // the first-layer tables are in LDS
+    wfirst_gemm_tile(acc, Wp, plane_elems, n0, gen, I, sx, lds);
+
+    // y = SiLU(acc / scales + b2), written through the wave's LDS slice so that every store instruction covers
+    // whole 256-byte row segments
+    float* slice = reinterpret_cast<float*>(lds) + wave * kSlice;
+    const long rows_left = R - block * 32;
+    const int nv = rows_left >= 32 ? 32 : (rows_left > 0 ? (int)rows_left : 0);
+#pragma unroll
+    for (int pass = 0; pass < 4; pass++) {
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const int ni = 2 * pass + h;
+#pragma unroll
+            for (int qq = 0; qq < 4; qq++) {
+                const int cl = 32 * ni + 8 * qq + 4 * g;
+                const float4 iw = *reinterpret_cast<const float4*>(wb + cl);
+                const float4 bv = *reinterpret_cast<const float4*>(wb + kFTN + cl);
+                float4 v;
+                v.x = activate_c<1>(acc[ni][4 * qq + 0] * isx * iw.x + bv.x);
+                v.y = activate_c<1>(acc[ni][4 * qq + 1] * isx * iw.y + bv.y);
+                v.z = activate_c<1>(acc[ni][4 * qq + 2] * isx * iw.z + bv.z);
+                v.w = activate_c<1>(acc[ni][4 * qq + 3] * isx * iw.w + bv.w);
+                *reinterpret_cast<float4*>(slice + m * kRed + 32 * h + 8 * qq + 4 * g) = v;
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        float* yp = Y + block * 32 * O + n0 + 64 * pass + lane;
+#pragma unroll
+        for (int r = 0; r < 32; r++)
+            if (r < nv) yp[(long)r * O] = slice[r * kRed + lane];
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
@@ -595,6 +787,29 @@ int mg_tensor_linear_f16x2_rowsum(const void* packed_W, const float* x, const fl
     rowsum_finish_kernel<<<dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, s>>>(
         row_ptr, n_out, n_blocks, dim_out, static_cast<const float*>(workspace), scale, out);
     return check_launch("rowsum_finish_kernel");
+}
+
+int mg_painn_filter_hidden(const float* r_ij, long n_edges, float rmax, const float* W1, long w1_stride_o,
+                           long w1_stride_i, const float* b1, const void* packed_W2, const float* b2, int hidden,
+                           const float* h1_bound, float* y, mg_stream_t stream) {
+    MG_REQUIRE(hidden >= 256 && hidden % 256 == 0 && hidden <= kHidMax,
+               "mg_painn_filter_hidden: hidden must be 256 or 512 (got %d)", hidden);
+    MG_REQUIRE(n_edges >= 0 && n_edges < (1L << 31), "mg_painn_filter_hidden: bad size");
+    MG_REQUIRE(rmax > 0.f, "mg_painn_filter_hidden: rmax must be positive");
+    if (n_edges == 0) return MG_OK;
+    MG_REQUIRE(r_ij && W1 && packed_W2 && h1_bound && y && aligned16(packed_W2) && aligned16(y),
+               "mg_painn_filter_hidden: null or unaligned pointer");
+    const int tiles_n = hidden / kFTN;
+    const long tiles_total = ceil_div(n_edges, kFTM) * tiles_n;
+    const _Float16* planes = static_cast<const _Float16*>(packed_W2);
+    const float* w_inv = reinterpret_cast<const float*>(planes + 2L * hidden * hidden);
+    const long grid = 8 * ceil_div(tiles_total, 8);
+    MG_REQUIRE(grid < (1L << 31), "mg_painn_filter_hidden: too many tiles");
+    const float base = (float)(3.14159265358979323846 / (double)rmax);
+    painn_filter_hidden_kernel<<<dim3((unsigned)grid), dim3(64 * kFW), 0, static_cast<hipStream_t>(stream)>>>(
+        planes, w_inv, b2, r_ij, n_edges, base, W1, w1_stride_o, w1_stride_i, b1, hidden, h1_bound, y, tiles_n,
+        tiles_total);
+    return check_launch("painn_filter_hidden_kernel");
 }
 
 }  // extern "C"

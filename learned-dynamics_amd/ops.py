@@ -1108,6 +1108,56 @@ def tensor_linear_f16x2_rowsum(W, x, x_bound, row_ptr, seg, n_out, bias=None, ac
     return out, y
 
 
+def painn_filter_hidden_supported(n_rbf, hidden, n_edges):
+    """First two filter layers in one kernel: 16 radial functions, hidden width 256 or 512."""
+    return get_linear_mode() == LINEAR_F16X2 and n_rbf == 16 and hidden in (256, 512) and n_edges >= 1024
+
+
+_chunk_perm_cache = {}
+
+
+def _operand_order_columns(W):
+    """W (dim_out, dim_in) with the input channels of every group of 32 reordered to the accumulator order of the
+    matrix core (position 16 g + p holds channel 8 (p / 4) + 4 g + p % 4); cached per tensor object and version."""
+    key = id(W)
+    hit = _chunk_perm_cache.get(key)
+    if hit is not None and hit[0]() is W and hit[1] == W._version and hit[2] == W.data_ptr():
+        return hit[3]
+    pos = torch.arange(32, device=W.device)
+    g, p = pos // 16, pos % 16
+    src = 8 * (p // 4) + 4 * g + p % 4
+    cols = (torch.arange(0, W.shape[1], 32, device=W.device)[:, None] + src[None, :]).reshape(-1)
+    with torch.no_grad():
+        Wr = W.detach()[:, cols].contiguous()
+    if len(_chunk_perm_cache) > 256:
+        _chunk_perm_cache.clear()
+    _chunk_perm_cache[key] = (weakref.ref(W), W._version, W.data_ptr(), Wr)
+    return Wr
+
+
+def painn_filter_hidden(r_ij, rmax, W1, b1, W2, b2, h1_bound):
+    """SiLU(b2 + W2 SiLU(b1 + W1 radial_encode(r_ij, 16, rmax))) (edges, hidden) without storing the first layer's
+    output.  h1_bound: (1, 1) upper bound of the first layer's output (linear_out_bound(W1, b1, None))."""
+    for t, nm in ((r_ij, "r_ij"), (W2, "W2"), (b2, "b2"), (h1_bound, "h1_bound")):
+        _check_input(t, nm)
+    if not W1.is_cuda or W1.dtype != torch.float32 or W1.dim() != 2 or W1.size(1) != 16:
+        raise RuntimeError("W1 must be a float32 CUDA matrix (hidden, 16)")
+    hidden = int(W1.size(0))
+    if tuple(W2.shape) != (hidden, hidden) or b2.numel() != hidden or (b1 is not None and b1.numel() != hidden):
+        raise RuntimeError("W2 must be (hidden, hidden), b1 and b2 (hidden,)")
+    if r_ij.dim() != 2 or r_ij.size(1) != 3:
+        raise RuntimeError("r_ij must have shape (edges, 3)")
+    if b1 is not None:
+        _check_input(b1, "b1")
+    E = int(r_ij.size(0))
+    with torch.cuda.device(r_ij.device):
+        y = torch.empty(E, hidden, dtype=torch.float32, device=r_ij.device)
+        L.check(_lib.mg_painn_filter_hidden(_p(r_ij), E, float(rmax), _p(W1), int(W1.stride(0)), int(W1.stride(1)),
+                                            _p(b1), _p(packed_weight_f16x2(_operand_order_columns(W2))), _p(b2), hidden,
+                                            _p(h1_bound), _p(y), _stream()))
+    return y
+
+
 def painn_filter_message_supported(n, hidden, n_edges):
     """The fused filter + message kernel: channel blocks of 64, a hidden width the matrix path tiles, and
     enough edges to fill the chip with 256-edge tiles."""

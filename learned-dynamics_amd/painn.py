@@ -165,8 +165,15 @@ class Message(nn.Module):
         res_a, res_v = (flat_a, flat_v) if residual else (None, None)
         if ops.painn_filter_message_supported(n, 4 * n, r_ij.shape[0]):
             # the filter's last layer runs inside the edge kernel: the (edges, 4n) filter is never stored
-            h, bound = self._hidden(r_ij)
-            h, bound = _linear(h, self.mlp_dist.layers[2], ops.ACT_SILU, bound)
+            first, second = self.mlp_dist.layers[0], self.mlp_dist.layers[2]
+            if ops.painn_filter_hidden_supported(self.n_rbf, second.out_features, r_ij.shape[0]):
+                # encoding, first and second layer in one kernel: the first layer's output is never stored
+                b1 = ops.linear_out_bound(first.weight, first.bias, None)
+                h = ops.painn_filter_hidden(r_ij, self.r0, first.weight, first.bias, second.weight, second.bias, b1)
+                bound = ops.linear_out_bound(second.weight, second.bias, b1)
+            else:
+                h, bound = self._hidden(r_ij)
+                h, bound = _linear(h, second, ops.ACT_SILU, bound)
             W3, b3 = self._permuted_last()
             out_a, out_v = ops.painn_filter_message(W3, b3, h, bound, graph.row_ptr, graph.src32, graph.dst32, r_ij,
                                                     actv, flat_v, self.epsilon, res_a, res_v)

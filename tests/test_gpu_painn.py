@@ -296,3 +296,25 @@ def test_filter_message_without_edges_returns_the_residual(ops):
     with pytest.raises(RuntimeError, match="multiple of 64"):
         ops.painn_filter_message(W3[:4 * 48], b3[:4 * 48], h, bound, row_ptr, empty_i, empty_i, r, actv[:, :4 * 48].contiguous(),
                                  x_v[:, :48].contiguous(), 0.1)
+
+
+@pytest.mark.parametrize("hidden,E", [(512, 3000), (256, 1500), (512, 257)])
+def test_first_two_filter_layers_from_edge_vectors(ops, hidden, E):
+    """mg_painn_filter_hidden against the two separate kernels (fused encode + first layer, then the GEMM) and
+    against float64 arithmetic on the oracle's encoding."""
+    g = torch.Generator().manual_seed(hidden + E)
+    r = (torch.randn(E, 3, generator=g) * 3).cuda()
+    W1 = (torch.randn(hidden, 16, generator=g) / 4).cuda()
+    b1 = torch.randn(hidden, generator=g).cuda()
+    W2 = (torch.randn(hidden, hidden, generator=g) / hidden ** 0.5).cuda()
+    b2 = torch.randn(hidden, generator=g).cuda()
+    bound1 = ops.linear_out_bound(W1, b1, None)
+    y = ops.painn_filter_hidden(r, 8.0, W1, b1, W2, b2, bound1)
+    h1 = ops.painn_radial_linear(r, 16, 8.0, W1, b1, ops.ACT_SILU)
+    two = ops.tensor_linear_f16x2(W2, h1, bound1, bias=b2, act=ops.ACT_SILU)
+    enc = OL.radial_encode_painn(r.cpu().double(), 16, 8.0)
+    f = torch.nn.functional
+    ref = f.silu(f.linear(f.silu(f.linear(enc, W1.double().cpu(), b1.double().cpu())), W2.double().cpu(), b2.double().cpu()))
+    scale = float(ref.abs().max())
+    torch.testing.assert_close(y, two, rtol=1e-5, atol=3e-6 * scale)
+    torch.testing.assert_close(y.cpu().double(), ref, rtol=1e-5, atol=4e-6 * scale)
