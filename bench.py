@@ -186,10 +186,28 @@ def bench_painn_layer(torch, args):
             # as the layer runs it: the filter MLP's last layer inside the edge kernel (the largest kernel of
             # the step); the stand-alone GEMM above is the MLP's middle layer, the second largest
             msg = block.message
-            h1, b1 = msg._hidden(r_ij)
-            h2, b2 = painn._linear(h1, msg.mlp_dist.layers[2], ops.ACT_SILU, b1)
+            first, second = msg.mlp_dist.layers[0], msg.mlp_dist.layers[2]
+            b1 = ops.linear_out_bound(first.weight, first.bias, None)
+            if ops.painn_filter_hidden_supported(n_rbf, 4 * n, E):
+                # encoding + first + second layer of the filter MLP in one kernel (the second largest kernel)
+                hidden_fn = lambda: ops.painn_filter_hidden(r_ij, r0, first.weight, first.bias, second.weight,
+                                                            second.bias, b1)
+                t_hidden = event_time(torch, hidden_fn, 10)
+                h2, b2 = hidden_fn(), ops.linear_out_bound(second.weight, second.bias, b1)
+                breakdown["filter_encode_plus_two_layers_ms"] = t_hidden * 1e3
+                hidden_flops = 3 * (flops + 2.0 * E * 16 * 4 * n)
+                roofline = {"kernel": "painn_filter_hidden_kernel (radial encoding, E x 16 x 512 and E x 512 x 512 "
+                                      "split-fp16 GEMMs, bias + SiLU; the first layer's output stays in registers)",
+                            "bound": "mfma", "achieved": hidden_flops / t_hidden / 1e12, "peak": PEAK_BF16_MFMA_TFLOPS,
+                            "unit": "TFLOP/s", "frac": hidden_flops / t_hidden / 1e12 / PEAK_BF16_MFMA_TFLOPS,
+                            "traffic": measured_traffic("painn_filter_hidden_kernel"),
+                            "fp32_equivalent_tflops": hidden_flops / 3 / t_hidden / 1e12,
+                            "stand_alone_gemm_for_comparison": roofline}
+            else:
+                h1, _ = msg._hidden(r_ij)
+                h2, b2 = painn._linear(h1, second, ops.ACT_SILU, b1)
+                del h1
             W3, b3 = msg._permuted_last()
-            del h1
             t_fused = event_time(torch, lambda: ops.painn_filter_message(
                 W3, b3, h2, b2, graph.row_ptr, graph.src32, graph.dst32, r_ij, actv, xv_flat, 0.1, xa_flat, xv_flat), 10)
             del h2
