@@ -317,6 +317,22 @@ int mg_tensor_linear_bf16_rowsum(const void* packed_W, const void* x, long rows,
                                  const float* bias, int act, const int* row_ptr, const int* seg, long n_out, float scale,
                                  void* workspace, void* y, float* out, mg_stream_t stream);
 
+/* The per-edge part of the scalar messages on bf16 storage (archs/diffuser_atoms15.py:98-110 MLP.forward applied
+ * at :244-246 to psi_a = Y P0) reduced to the two sums over edges that the layers after the sum need:
+ *   psi = Y x (rows, 128);  h1 = act(b1 + W1 psi) (rows, 256);  h2 = act(b2 + W2 h1) (rows, 256)
+ *   sum_psi (n_out, 128) float32 = sum over the rows of each segment of bfloat16(psi)
+ *   sum_h2  (n_out, 256) float32 = sum over the rows of each segment of bfloat16(h2)
+ * with every intermediate rounded to bfloat16 exactly where mg_tensor_linear_bf16 rounds it when it stores, so
+ * the result equals three mg_tensor_linear_bf16[_rowsum] calls up to fp32 summation order; no per-row tensor is
+ * written.  x (rows, dim_in) bfloat16, dim_in % 32 == 0; packed_Y, packed_W1, packed_W2 as for
+ * mg_tensor_linear_bf16, where the INPUT channels of W1 and W2 are permuted inside every group of 32 so that
+ * position 16 g + p holds channel 8 (p / 4) + 4 g + p % 4 (g = 0, 1; p = 0..15).  seg, row_ptr as for
+ * mg_tensor_linear_bf16_rowsum. */
+int mg_mlp_chain_bf16_workspace_bytes(long rows, size_t* bytes);
+int mg_mlp_chain_bf16(const void* x, long rows, int dim_in, const void* packed_Y, const void* packed_W1,
+                      const float* b1, const void* packed_W2, const float* b2, int act, const int* row_ptr,
+                      const int* seg, long n_out, void* workspace, float* sum_psi, float* sum_h2, mg_stream_t stream);
+
 /* x (rows, dim, comps) in the reference's tensor layout (managan/tensor_products.py:17-24: channel, then the 3^k
  * components) -> xt (rows * comps, dim_pad): one plain GEMM row per (row, component) with the channels zero-padded
  * to dim_pad (a power of two, 32..256), and rowmax (rows * comps): max |xt| per output row.  What

@@ -61,15 +61,25 @@ def mlp_forward(mlp, x, plus_identity=False):
     return out.to(torch.bfloat16)
 
 
+def _mlp_after_sums(mlp, s_x, s_h, row_ptr, plus_identity, scale):
+    """(W_direct [+ 1]) s_x + W_last s_h + count * b_last, scaled, as bf16: the linear tail of the MLP applied to
+    the sums over rows of its input and of its last hidden layer."""
+    Wd = mlp.lin_direct.weight
+    if plus_identity:
+        Wd = Wd + torch.eye(Wd.shape[0], device=Wd.device, dtype=Wd.dtype)
+    last = mlp.layers[4]
+    out = ops.tensor_linear_bf16(Wd, s_x, out_dtype=torch.float32)
+    ops.tensor_linear_bf16(last.weight, s_h, out=out, accumulate=True)
+    count = (row_ptr[1:] - row_ptr[:-1]).to(out.dtype)[:, None]
+    return torch.addcmul(out, count, last.bias[None, :]).mul_(scale).to(torch.bfloat16)
+
+
 def mlp_summed_over_rows(mlp, x, row_ptr, n_out, plus_identity=False, scale=1.0, seg=None, s_x=None):
     """scale * (sum over each CSR segment of mlp_forward(mlp, x, plus_identity)) as bf16 (n_out, d).  The
     direct linear and the last layer are linear in their inputs, so they are applied to the summed rows
     (bee_layers.MLP.summed_over_rows).  With seg (the segment of every row) the second layer sums its
     bf16-rounded output rows in its own epilogue and never stores them; s_x: the sums of x if the caller has
     them.  Sums are accumulated in fp32 and stored in bf16 like every other feature."""
-    Wd = mlp.lin_direct.weight
-    if plus_identity:
-        Wd = Wd + torch.eye(Wd.shape[0], device=Wd.device, dtype=Wd.dtype)
     Ls = mlp.layers
     h = ops.tensor_linear_bf16(Ls[0].weight, x, bias=Ls[0].bias, act=ops.ACT_LEAKY)
     if seg is not None and ops.bf16_rowsum_supported(h.shape[0], Ls[2].in_features, Ls[2].out_features):
@@ -81,13 +91,10 @@ def mlp_summed_over_rows(mlp, x, row_ptr, n_out, plus_identity=False, scale=1.0,
     del h
     if s_x is None:
         s_x = ops.segment_sum_csr_bf16(x, row_ptr, n_out)
-    out = ops.tensor_linear_bf16(Wd, s_x, out_dtype=torch.float32)
-    ops.tensor_linear_bf16(Ls[4].weight, s_h, out=out, accumulate=True)
-    count = (row_ptr[1:] - row_ptr[:-1]).to(out.dtype)[:, None]
-    return torch.addcmul(out, count, Ls[4].bias[None, :]).mul_(scale).to(torch.bfloat16)
+    return _mlp_after_sums(mlp, s_x, s_h, row_ptr, plus_identity, scale)
 
 
-def messages_forward(mod: Messages, graph: Graph, r_ij, s_a, s_v, s_d, node_order="cell"):
+def messages_forward(mod: Messages, graph: Graph, r_ij, s_a, s_v, s_d, node_order="cell", chain=True):
     """Messages.forward (archs/diffuser_atoms15.py:238-253) on storage tensors; returns the three
     0.1 * (sum over edges) increments in storage layout."""
     if isinstance(node_order, str):
@@ -99,14 +106,22 @@ def messages_forward(mod: Messages, graph: Graph, r_ij, s_a, s_v, s_d, node_orde
                                       mod.lin_enc.bias, node_order=node_order)
     E, chan = P0.shape[0], P0.shape[2]
     Y0 = _cat_Y(mod, LABELS_0)
-    if ops.bf16_rowsum_supported(E, 3 * chan, Y0.shape[0]):
-        s_psi, psi_a = ops.tensor_linear_bf16_rowsum(Y0, P0.reshape(E, 3 * chan), graph.row_ptr, graph.src32, rows,
-                                                     want_rows=True)
-        s_psi = s_psi.to(torch.bfloat16)
+    Ls = mod.mlp_a.layers
+    if chain and ops.mlp_chain_bf16_supported(E, 3 * chan, Y0.shape[0], Ls[0].out_features) \
+            and Ls[2].out_features == Ls[0].out_features:
+        # psi_a and both hidden layers stay in registers; only their sums over the edges of a node are written
+        s_psi, s_h = ops.mlp_chain_bf16(Y0, P0.reshape(E, 3 * chan), Ls[0].weight, Ls[0].bias, Ls[2].weight,
+                                        Ls[2].bias, graph.row_ptr, graph.src32, rows)
+        B_a = _mlp_after_sums(mod.mlp_a, s_psi.to(torch.bfloat16), s_h.to(torch.bfloat16), graph.row_ptr, True, 0.1)
     else:
-        psi_a, s_psi = ops.tensor_linear_bf16(Y0, P0.reshape(E, 3 * chan)), None
-    B_a = mlp_summed_over_rows(mod.mlp_a, psi_a, graph.row_ptr, rows, plus_identity=True, scale=0.1,
-                               seg=graph.src32, s_x=s_psi)
+        if ops.bf16_rowsum_supported(E, 3 * chan, Y0.shape[0]):
+            s_psi, psi_a = ops.tensor_linear_bf16_rowsum(Y0, P0.reshape(E, 3 * chan), graph.row_ptr, graph.src32,
+                                                         rows, want_rows=True)
+            s_psi = s_psi.to(torch.bfloat16)
+        else:
+            psi_a, s_psi = ops.tensor_linear_bf16(Y0, P0.reshape(E, 3 * chan)), None
+        B_a = mlp_summed_over_rows(mod.mlp_a, psi_a, graph.row_ptr, rows, plus_identity=True, scale=0.1,
+                                   seg=graph.src32, s_x=s_psi)
     B_v = _lin(_cat_Y(mod, LABELS_1, 0.1), S1.reshape(rows, 3, 5 * chan), 3)
     B_d = _lin(_cat_Y(mod, LABELS_2, 0.1), S2.reshape(rows, 9, 5 * chan), 9)
     return B_a, B_v, B_d

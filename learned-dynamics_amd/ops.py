@@ -926,6 +926,39 @@ def tensor_linear_bf16_rowsum(W, x, row_ptr, seg, n_out, bias=None, act=ACT_NONE
     return out, y
 
 
+def mlp_chain_bf16_supported(rows, dim_in, dim_psi, hidden):
+    return dim_psi == 128 and hidden == 256 and dim_in % 32 == 0 and rows >= 4096
+
+
+def mlp_chain_bf16(Y, x, W1, b1, W2, b2, row_ptr, seg, n_out, act=ACT_LEAKY):
+    """(sum_psi (n_out, 128), sum_h2 (n_out, 256)) float32: the sums over the rows of each segment of the
+    bfloat16-rounded psi = Y x and h2 = act(b2 + W2 act(b1 + W1 psi)), every layer rounded to bfloat16 as
+    tensor_linear_bf16 stores it, in one kernel that writes no per-row tensor.  x (rows, dim_in) bfloat16 sorted
+    by segment (seg ascending, row_ptr its CSR form); Y (128, dim_in), W1 (256, 128), W2 (256, 256) float32."""
+    _check_bf16(x, "x")
+    for t, nm in ((Y, "Y"), (W1, "W1"), (W2, "W2"), (b1, "b1"), (b2, "b2")):
+        _check_input(t, nm)
+    for t, nm in ((row_ptr, "row_ptr"), (seg, "seg")):
+        _check_input(t, nm, torch.int32)
+    rows, dim_in = int(x.size(0)), int(x.size(1))
+    if (x.dim() != 2 or tuple(Y.shape) != (128, dim_in) or tuple(W1.shape) != (256, 128) or tuple(W2.shape) != (256, 256)
+            or b1.numel() != 256 or b2.numel() != 256 or dim_in % 32):
+        raise RuntimeError("mlp_chain_bf16: x (rows, dim_in), Y (128, dim_in), W1 (256, 128), W2 (256, 256) expected")
+    if seg.numel() != rows or row_ptr.numel() != n_out + 1:
+        raise RuntimeError("seg must have one entry per row and row_ptr n_out + 1 entries")
+    nbytes = ctypes.c_size_t(0)
+    L.check(_lib.mg_mlp_chain_bf16_workspace_bytes(rows, ctypes.byref(nbytes)))
+    with torch.cuda.device(x.device):
+        s_psi = torch.empty(n_out, 128, dtype=torch.float32, device=x.device)
+        s_h = torch.empty(n_out, 256, dtype=torch.float32, device=x.device)
+        work = torch.empty(nbytes.value // 4, dtype=torch.float32, device=x.device)
+        L.check(_lib.mg_mlp_chain_bf16(_p(x), rows, dim_in, _p(packed_weight(Y)),
+                                       _p(packed_weight(_operand_order_columns(W1))), _p(b1),
+                                       _p(packed_weight(_operand_order_columns(W2))), _p(b2), int(act), _p(row_ptr),
+                                       _p(seg), int(n_out), _p(work), _p(s_psi), _p(s_h), _stream()))
+    return s_psi, s_h
+
+
 def segment_sum_csr_bf16(x_edge, row_ptr, n_rows, scale=1.0):
     """scale * (sum of the bfloat16 edge rows of each CSR row), fp32 accumulation, bfloat16 result."""
     _check_bf16(x_edge, "x_edge")

@@ -215,3 +215,69 @@ def test_linear_bf16_with_row_sums_in_the_epilogue(ops, dim_in, dim_out, act, ki
     ref = 0.5 * torch.zeros(n_seg, dim_out, dtype=torch.float64).index_add_(0, seg, y_ref.double().cpu())
     torch.testing.assert_close(out.cpu().double(), ref, rtol=1e-5, atol=2e-6 * float(ref.abs().max()))
     assert not bool(out[(lengths == 0).cuda()].any())
+
+
+@pytest.mark.parametrize("kind,dim_in", [("mixed", 384), ("short", 384), ("tiny", 96), ("aligned", 32)])
+def test_scalar_message_chain_in_one_kernel(ops, kind, dim_in):
+    """mg_mlp_chain_bf16 against the three separate kernels it replaces: the sums over segments of the bf16-rounded
+    psi = Y x and h2 = leaky(W2 leaky(W1 psi + b1) + b2).  psi is computed in the same order as by the plain
+    kernel, so its sums agree to fp32 summation order.  The two later layers multiply in a permuted order of the
+    input channels, so a few bf16 roundings of h1 and h2 fall the other way (one unit in the last place, 2^-8
+    relative): the sums of h2 are compared with an allowance of two such units of the largest element, and no
+    more than 5 % of them may differ beyond fp32 summation order at all."""
+    g = torch.Generator().manual_seed(11 + dim_in)
+    n_seg = 300
+    if kind == "mixed":
+        lengths = torch.cat([torch.randint(0, 5, (n_seg // 2,), generator=g),
+                             torch.randint(20, 300, (n_seg - n_seg // 2,), generator=g)])[torch.randperm(n_seg, generator=g)]
+    elif kind == "short":
+        lengths = torch.randint(0, 9, (n_seg,), generator=g)
+    elif kind == "tiny":
+        n_seg = 4
+        lengths = torch.tensor([30, 0, 6, 1])
+    else:
+        lengths = torch.tensor([32, 64, 1, 31, 32, 0, 0, 96, 33, 31] * (n_seg // 10))
+    seg = torch.repeat_interleave(torch.arange(n_seg), lengths)
+    rows = int(seg.numel())
+    x = torch.randn(rows, dim_in, generator=g).cuda().to(torch.bfloat16)
+    Y = (torch.randn(128, dim_in, generator=g) / dim_in ** 0.5).cuda()
+    W1 = (torch.randn(256, 128, generator=g) / 128 ** 0.5).cuda()
+    W2 = (torch.randn(256, 256, generator=g) / 256 ** 0.5).cuda()
+    b1, b2 = torch.randn(256, generator=g).cuda(), torch.randn(256, generator=g).cuda()
+    segc = seg.int().cuda()
+    row_ptr = ops.segment_row_ptr(segc, n_seg)
+    s_psi, s_h = ops.mlp_chain_bf16(Y, x, W1, b1, W2, b2, row_ptr, segc, n_seg)
+    psi = ops.tensor_linear_bf16(Y, x)
+    h2 = ops.tensor_linear_bf16(W2, ops.tensor_linear_bf16(W1, psi, bias=b1, act=ops.ACT_LEAKY), bias=b2,
+                                act=ops.ACT_LEAKY)
+    ref_psi = torch.zeros(n_seg, 128, dtype=torch.float64).index_add_(0, seg, psi.double().cpu())
+    ref_h = torch.zeros(n_seg, 256, dtype=torch.float64).index_add_(0, seg, h2.double().cpu())
+    torch.testing.assert_close(s_psi.cpu().double(), ref_psi, rtol=1e-5, atol=2e-6 * float(ref_psi.abs().max()))
+    err = (s_h.cpu().double() - ref_h).abs()
+    ulp = 2.0 ** -8 * float(h2.float().abs().max())
+    assert float(err.max()) <= 2 * ulp + 1e-5 * float(ref_h.abs().max())
+    assert float((err > 1e-5 * ref_h.abs().clamp_min(1.0)).double().mean()) < 0.05
+    empty = (lengths == 0).cuda()
+    assert not bool(s_psi[empty].any()) and not bool(s_h[empty].any())
+
+
+def test_messages_bf16_chain_equals_separate_kernels(pkg, ops):
+    """messages_forward with the one-kernel scalar chain against the same call with the separate kernels."""
+    bl = importlib.import_module("learned-dynamics_amd.bee_layers")
+    b16 = importlib.import_module("learned-dynamics_amd.bee_layers_bf16")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    torch.manual_seed(3)
+    N, chan, r0 = 4096, 128, 5.0
+    side = (N / 0.1) ** (1 / 3)
+    pos = (torch.rand(1, N, 3) * side).cuda()
+    mod = bl.Messages(r0, chan, chan, chan, chan).cuda()
+    x_a, x_v, x_d = torch.randn(1, N, chan).cuda(), torch.randn(1, N, chan, 3).cuda(), torch.randn(1, N, chan, 3, 3).cuda()
+    with torch.no_grad():
+        graph, r_ij = gl.graph_setup(r0, (side, side, side), pos, neighbours_max=256, celllist_max=64)
+        s = b16.to_storage(x_a, x_v, x_d)
+        out_chain = b16.messages_forward(mod, graph, r_ij, *s, chain=True)
+        out_sep = b16.messages_forward(mod, graph, r_ij, *s, chain=False)
+    assert graph.src.numel() >= 4096                          # the chain kernel is the one that ran
+    assert torch.equal(out_chain[1], out_sep[1]) and torch.equal(out_chain[2], out_sep[2])
+    a, b = out_chain[0].float(), out_sep[0].float()
+    assert float((a - b).abs().max()) <= 2.0 ** -6 * float(b.abs().max())
