@@ -1,0 +1,126 @@
+"""Dataset chunk files and checkpoint dicts in the reference's on-disk formats (managan/statefiles.py:16-42,
+managan/config.py:125-137): CPU only."""
+import importlib
+import io
+import os
+import pickle
+import struct
+
+import numpy as np
+import pytest
+import torch
+
+sf = importlib.import_module("learned-dynamics_amd.statefiles")
+
+
+def _chunk_bytes(metadata, shape, x):
+    """A chunk assembled by hand from the format's description: `!III` lengths, pickle, pickle, .npy."""
+    payload = io.BytesIO()
+    np.save(payload, x, allow_pickle=False)
+    subs = [pickle.dumps(metadata), pickle.dumps(shape), payload.getvalue()]
+    return struct.pack("!III", *map(len, subs)) + b"".join(subs)
+
+
+def test_reads_a_hand_assembled_chunk():
+    x = np.arange(2 * 3 * 5 * 3, dtype=np.float32).reshape(2, 3, 5, 3)          # (L, batch, atoms, 3)
+    meta = {"poly_len": 5, "space_dim": 3, "k": 1.0}                              # managan/sims.py:164-224
+    st = sf.read_state_from_file(io.BytesIO(_chunk_bytes(meta, (5, 3), x)), device="cpu")
+    assert st.shape == (5, 3) and st.size == (2, 3) and st.metadata == meta
+    assert torch.equal(st.x, torch.from_numpy(x))
+    assert st[1].size == (3,) and torch.equal(st[1].x, torch.from_numpy(x[1]))
+
+
+def test_writer_produces_the_documented_layout_and_round_trips():
+    x = torch.randn(4, 2, 7, 3)
+    buf = io.BytesIO()
+    sf.save_state_to_file(buf, sf.TrajectoryState((7, 3), x, {"poly_len": 7, "space_dim": 3}))
+    raw = buf.getvalue()
+    n0, n1, n2 = struct.unpack("!III", raw[:12])
+    assert len(raw) == 12 + n0 + n1 + n2
+    assert pickle.loads(raw[12:12 + n0]) == {"poly_len": 7, "space_dim": 3}     # our own bytes: plain pickle is fine
+    assert pickle.loads(raw[12 + n0:12 + n0 + n1]) == (7, 3)
+    assert np.array_equal(np.load(io.BytesIO(raw[12 + n0 + n1:]), allow_pickle=False), x.numpy())
+    assert raw == _chunk_bytes({"poly_len": 7, "space_dim": 3}, (7, 3), x.numpy())
+    back = sf.read_state_from_file(io.BytesIO(raw), device="cpu")
+    assert back.shape == (7, 3) and back.size == (4, 2) and torch.equal(back.x, x)
+
+
+class _Boom:
+    def __reduce__(self):
+        return (os.system, ("echo executed > /tmp/statefile_pickle_ran",))
+
+
+class _Meta:
+    def __init__(self):
+        self.seq, self.box = "GYDPETGTWG", (30.0, 30.0, 30.0)
+
+
+def test_pickled_objects_are_never_instantiated(tmp_path):
+    """A metadata pickle naming a callable is decoded into an inert record; nothing is imported or called."""
+    marker = "/tmp/statefile_pickle_ran"
+    if os.path.exists(marker):
+        os.remove(marker)
+    x = np.zeros((1, 1, 2, 3), np.float32)
+    st = sf.read_state_from_file(io.BytesIO(_chunk_bytes({"evil": _Boom()}, (2, 3), x)), device="cpu")
+    assert not os.path.exists(marker)
+    rec = st.metadata["evil"]
+    assert isinstance(rec, sf.OpaqueObject) and rec.name == "system" and rec.args == ("echo executed > /tmp/statefile_pickle_ran",)
+    st = sf.read_state_from_file(io.BytesIO(_chunk_bytes(_Meta(), (2, 3), x)), device="cpu")
+    rec = st.metadata
+    assert isinstance(rec, sf.OpaqueObject) and rec.name == "_Meta" and not isinstance(rec, _Meta)
+    assert rec.state == {"seq": "GYDPETGTWG", "box": (30.0, 30.0, 30.0)}
+
+
+@pytest.mark.parametrize("damage", ["short_header", "truncated", "bad_shape", "bad_npy", "shape_mismatch"])
+def test_malformed_chunks_raise_dataset_error(damage):
+    x = np.zeros((2, 4, 3), np.float32)
+    raw = _chunk_bytes({}, (4, 3), x)
+    if damage == "short_header":
+        raw = raw[:7]
+    elif damage == "truncated":
+        raw = raw[:-5]
+    elif damage == "bad_shape":
+        raw = _chunk_bytes({}, "4x3", x)
+    elif damage == "bad_npy":
+        subs = [pickle.dumps({}), pickle.dumps((4, 3)), b"not an npy file"]
+        raw = struct.pack("!III", *map(len, subs)) + b"".join(subs)
+    else:
+        raw = _chunk_bytes({}, (5, 3), x)
+    with pytest.raises(sf.DatasetError):
+        sf.read_state_from_file(io.BytesIO(raw), device="cpu")
+
+
+def test_checkpoint_states_load_into_mirrored_modules_by_name(tmp_path):
+    """A checkpoint dict as managan/config.py:125-137 writes it, whose "dn" state dict carries the parameter names
+    of archs/meanflow_painn8.py:63-125 (`blocks.<i>.message.mlp_dist.layers.0.weight`, `...update.lin_l.W`, ...)."""
+    painn = importlib.import_module("learned-dynamics_amd.painn")
+    torch.manual_seed(0)
+    trained = [painn.Block(8.0, 32, pos_mutable=(i == 1)) for i in range(2)]
+    dn = {}
+    for i, blk in enumerate(trained):
+        for k, v in blk.state_dict().items():
+            dn[f"blocks.{i}.{k}"] = v.clone()
+    dn["embed.weight"] = torch.randn(4, 32)
+    path = tmp_path / "model.pt"
+    torch.save({"args": ["repel5:l64_t3", "meanflow_painn8"], "kwargs": {"r_cut": 8.0, "dim": 32}, "states": {"dn": dn}}, path)
+    ckpt = sf.load_checkpoint(path)
+    assert ckpt["args"][1] == "meanflow_painn8" and ckpt["kwargs"]["dim"] == 32
+    fresh = painn.Block(8.0, 32, pos_mutable=True)
+    sf.load_module_states(fresh, ckpt["states"]["dn"], "blocks.1")
+    for k, v in trained[1].state_dict().items():
+        assert torch.equal(fresh.state_dict()[k], v)
+    with pytest.raises(RuntimeError):                       # block 0 has no lin_push_pos: strict loading says so
+        sf.load_module_states(painn.Block(8.0, 32, pos_mutable=True), ckpt["states"]["dn"], "blocks.0")
+    with pytest.raises(KeyError):
+        sf.load_module_states(fresh, ckpt["states"]["dn"], "blocks.7")
+    assert set(sf.states_under(dn, "blocks.0.update")) == {k[len("update."):] for k in trained[0].state_dict() if k.startswith("update.")}
+
+
+def test_checkpoint_with_pickled_objects_is_refused(tmp_path):
+    path = tmp_path / "bad.pt"
+    torch.save({"args": [_Meta()], "kwargs": {}, "states": {}}, path)
+    with pytest.raises(Exception):
+        sf.load_checkpoint(path)
+    torch.save([1, 2, 3], path)
+    with pytest.raises(sf.DatasetError):
+        sf.load_checkpoint(path)
