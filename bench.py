@@ -47,7 +47,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="painn_layer",
-                    choices=["painn_layer", "neighbour", "products", "denoiser", "stress"])
+                    choices=["painn_layer", "neighbour", "products", "denoiser", "stress", "polymer"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
     ap.add_argument("--calibrate-copy", action="store_true",
@@ -350,6 +350,43 @@ def bench_products(torch, args):
             "note": "includes allocation of the three outputs; 4096 rows (17.8 MB) is launch-latency bound"}
 
 
+def bench_polymer(torch, args, with_cpu=True):
+    """The chain generator that feeds the models (polymer_sim(SimId.REPEL5, ...), the reference's own test shape
+    extensions/polymer_sims_cuda/test.py:9-17 scaled up to fill the GPU: one workgroup per chain)."""
+    ops = importlib.import_module("learned-dynamics_amd.ops")
+    out = {}
+    for batch, n, nsteps in ((32, 200, 100), (4096, 64, 100), (2048, 200, 100)):
+        g = torch.Generator().manual_seed(0x947 + 6)
+        steps = torch.randn(batch, n, 3, generator=g)
+        x = (0.8 * steps / steps.norm(dim=-1, keepdim=True)).cumsum(1).cuda()
+        v = torch.zeros(batch, n, 3).cuda()
+        drag = torch.ones(n).cuda()
+        t = event_time(torch, lambda: ops.repel5_sim(x, v, drag, 1.0, 0.01, nsteps, 7), 5, warmup=2)
+        pairs = batch * n * max(n - 3, 0) * (nsteps + 1)
+        out[f"batch{batch}_n{n}"] = {"ms": t * 1e3, "bead_steps_per_s": batch * n * nsteps / t,
+                                     "pair_forces_per_s": pairs / t, "fp32_vector_tflops": pairs * 19 / t / 1e12,
+                                     "frac_of_fp32_vector_peak": pairs * 19 / t / 1e12 / (PEAK_FP32_MFMA_TFLOPS / 2)}
+    res = {"metric": "chain generator bead-steps/sec (repel5, 100 steps per call)", "unit": "bead-steps/s",
+           "value": out["batch2048_n200"]["bead_steps_per_s"], "ms_per_step": out["batch2048_n200"]["ms"],
+           "detail": out,
+           "note": "19 flop per pair force (3 sub, 5 for |d|^2 + eps, 3 mul for the 6th power, 1 division counted as 1, "
+                   "6 for the scaled accumulate); the peak is the fp32 vector rate without packed instructions; "
+                   "32 chains occupy 32 of 256 CUs, which is all the parallelism the reference's test shape has"}
+    if with_cpu:
+        import numpy as np
+        OPY = importlib.import_module("oracle.polymer")
+        batch, n, nsteps = 8, 200, 10
+        rng = np.random.default_rng(0)
+        x0 = np.cumsum(rng.normal(size=(batch, n, 3)) * 0.46, axis=1).astype(np.float32)
+        normals = OPY.philox_normals(7, batch, n, 0, nsteps + 1)
+        t0 = time.perf_counter()
+        OPY.repel5_sim(x0, np.zeros_like(x0), np.ones(n, np.float32), 1.0, 0.01, nsteps, normals)
+        dt = time.perf_counter() - t0
+        res["cpu_baseline"] = {"value": batch * n * nsteps / dt, "unit": "bead-steps/s", "cores": 1, "kind": "port",
+                               "sample": f"{batch} chains x {n} beads x {nsteps} steps, numpy oracle"}
+    return res
+
+
 def chain_positions(torch, systems, atoms, box, seed, noise=1.0):
     g = torch.Generator().manual_seed(seed)
     steps = torch.randn(systems, atoms, 3, generator=g)
@@ -589,6 +626,8 @@ def main():
         res = bench_denoiser(torch, args, with_cpu=not args.no_cpu)
     elif args.workload == "stress":
         res = bench_stress(torch, args)
+    elif args.workload == "polymer":
+        res = bench_polymer(torch, args, with_cpu=not args.no_cpu)
     else:
         res = bench_products(torch, args)
         res.setdefault("ms_per_step", res["detail"]["rows_4096"]["us"] * 1e-3)

@@ -333,6 +333,18 @@ int mg_mlp_chain_bf16(const void* x, long rows, int dim_in, const void* packed_Y
                       const float* b1, const void* packed_W2, const float* b2, int act, const int* row_ptr,
                       const int* seg, long n_out, void* workspace, float* sum_psi, float* sum_h2, mg_stream_t stream);
 
+/* repel5_sim (extensions/polymer_sims_cuda/polymer_sims_kern.cu:145-164, bound as polymer_sim(SimId.REPEL5, ...) in
+ * polymer_sims.cpp:17-47): Langevin dynamics of batch_size chains of n beads, x and v (batch_size, n, 3) float32
+ * updated in place, drag (n).  Per call: half velocity update, max(nsteps, 1) position updates with full velocity
+ * updates between them, half velocity update.  Forces: harmonic bonds (K 20, r0 0.8) to the chain neighbours and
+ * 20 d / (|d|^2 + 0.2)^6 from every bead that is not a cyclic neighbour.  One workgroup per chain, n <= 2048; unlike
+ * the reference's 256-thread blocks, every force is computed from the positions of one step.  The normals of bead
+ * b = chain * n + i at velocity update first_kick + s are Box-Muller transforms of Philox4x32-10(counter (b,
+ * first_kick + s, 0, 0), key seed): a call with first_kick advanced by max(nsteps, 1) + 1 continues the stream
+ * (the reference reseeds XORWOW from the wall clock on every call). */
+int mg_repel5_sim(float* x, float* v, const float* drag, float T, float dt, int nsteps, int batch_size, int n,
+                  unsigned long long seed, unsigned int first_kick, mg_stream_t stream);
+
 /* x (rows, dim, comps) in the reference's tensor layout (managan/tensor_products.py:17-24: channel, then the 3^k
  * components) -> xt (rows * comps, dim_pad): one plain GEMM row per (row, component) with the channels zero-padded
  * to dim_pad (a power of two, 32..256), and rowmax (rows * comps): max |xt| per output row.  What

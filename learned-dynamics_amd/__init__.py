@@ -24,7 +24,7 @@ _SHIMS = os.path.join(os.path.dirname(os.path.abspath(__file__)), "shims")
 
 
 def install_shims():
-    """Make `import neighbour_grid_cuda`, `tensor_ops_cuda`, `codegen_tensops_cuda`
+    """Make `import neighbour_grid_cuda`, `tensor_ops_cuda`, `codegen_tensops_cuda`, `polymer_sims_cuda`
     and `torch_scatter` resolve to this package's HIP implementations."""
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
     for path in (root, _SHIMS):

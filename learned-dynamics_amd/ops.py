@@ -1416,3 +1416,24 @@ def radial_encode(kind, r_ij, n, rmax):
         out = torch.empty(lead + (n,), dtype=torch.float32, device=r_ij.device)
         L.check(_lib.mg_radial_encode(int(kind), _p(r_ij), E, int(n), float(rmax), _p(out), _stream()))
     return out
+
+
+# ------------------------------------------------------------------ data generator
+def repel5_sim(x, v, drag, T, dt, nsteps, seed, first_kick=0):
+    """Langevin dynamics of bead chains in place (polymer_sim(SimId.REPEL5, ...) of
+    extensions/polymer_sims_cuda/polymer_sims.cpp:17-47): x, v (batch, n, 3), drag (n).  seed, first_kick: the
+    noise of velocity update first_kick + s of bead b is a pure function of (seed, b, first_kick + s)."""
+    for t, nm in ((x, "x"), (v, "v"), (drag, "drag")):
+        _check_input(t, nm)
+    if x.dim() != 3 or v.dim() != 3 or drag.dim() != 1:
+        raise RuntimeError("Input tensors must have correct dimensions")
+    if x.size(0) != v.size(0):
+        raise RuntimeError("Batch sizes must match")
+    if x.size(1) != v.size(1) or x.size(1) != drag.size(0):
+        raise RuntimeError("Number of particles must match")
+    if x.size(2) != 3 or v.size(2) != 3:
+        raise RuntimeError("Position and velocity must be 3D")
+    with torch.cuda.device(x.device):
+        L.check(_lib.mg_repel5_sim(_p(x), _p(v), _p(drag), float(T), float(dt), int(nsteps), int(x.size(0)),
+                                   int(x.size(1)), int(seed) & 0xFFFFFFFFFFFFFFFF, int(first_kick), _stream()))
+
