@@ -265,6 +265,17 @@ int mg_painn_radial_encode(const float* r_ij /* (E,3) */, long n_edges, int n, f
 int mg_painn_radial_linear(const float* r_ij /* (E,3) */, long n_edges, int n, float rmax, const float* W,
                            long w_stride_o, long w_stride_i, const float* bias, int dim_out, int act,
                            float* y, mg_stream_t stream);
+/* mg_painn_message with the filter taken from a table instead of one row per edge.  The radial MLP of
+ * Message.forward (archs/meanflow_painn8.py:92) sees an edge only through d = |r_ij|, and its input
+ * radial_encode(r, n, rmax) (:25-35) consists of cos / sin (k pi d / rmax) with integer k, so the filter is a smooth
+ * function of d with period 2 rmax.  table (table_rows, 4n): that function at d = k * period / table_rows, k = 0 ..
+ * table_rows - 1 (table_rows a power of two, period = 2 rmax); every edge interpolates its filter between the four
+ * rows around d (4-point Lagrange, indices wrapped), error <= 0.0234 (period / table_rows)^4 max |d^4 filter / dd^4|.
+ * Everything else as mg_painn_message. */
+int mg_painn_table_message(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
+                           const float* r_ij, const float* table, int table_rows, float period, const float* actv,
+                           const float* x_v, int n, float epsilon, const float* res_a, const float* res_v, float* out_a,
+                           float* out_v, mg_stream_t stream);
 /* Message.forward after the two MLPs (archs/meanflow_painn8.py:91-100), fused over CSR rows:
  *   P = filt[e] * actv[dst[e]];  u = r_ij[e] / sqrt(epsilon + |r_ij[e]|^2);  v = x_v[dst[e]]
  *   out_v[i] = res_v[i] + sum_{e in row i} v*P[0:n] + (v x u)*P[n:2n] + u (x) P[2n:3n]

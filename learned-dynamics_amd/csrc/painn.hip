@@ -81,6 +81,28 @@ struct EdgeLoads {
 #pragma unroll
         for (int k = 0; k < 3; k++) v[k] = ld4(xv_row + 3 * c + 4 * k);
     }
+    // the filter from a periodic table of its values at d = k h (k = 0 .. mask): 4-point Lagrange interpolation
+    // between the rows i - 1 .. i + 2 with weights w (error at most 0.0234 h^4 max |fourth derivative|)
+    __device__ __forceinline__ void load_table(const float* __restrict__ tab, int i, int mask, const float (&w)[4],
+                                               const float* __restrict__ actv_row, const float* __restrict__ xv_row,
+                                               int n, int c) {
+        const long row_f = 4L * n;
+        const float* r0 = tab + (long)((i - 1) & mask) * row_f + c;
+        const float* r1 = tab + (long)(i & mask) * row_f + c;
+        const float* r2 = tab + (long)((i + 1) & mask) * row_f + c;
+        const float* r3 = tab + (long)((i + 2) & mask) * row_f + c;
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            const float4 t0 = ld4(r0 + k * n), t1 = ld4(r1 + k * n), t2 = ld4(r2 + k * n), t3 = ld4(r3 + k * n);
+            f[k] = make_float4(w[0] * t0.x + w[1] * t1.x + w[2] * t2.x + w[3] * t3.x,
+                               w[0] * t0.y + w[1] * t1.y + w[2] * t2.y + w[3] * t3.y,
+                               w[0] * t0.z + w[1] * t1.z + w[2] * t2.z + w[3] * t3.z,
+                               w[0] * t0.w + w[1] * t1.w + w[2] * t2.w + w[3] * t3.w);
+            a[k] = ld4(actv_row + k * n + c);
+        }
+#pragma unroll
+        for (int k = 0; k < 3; k++) v[k] = ld4(xv_row + 3 * c + 4 * k);
+    }
     __device__ __forceinline__ void accumulate(EdgeAcc& acc, float ux, float uy, float uz) const {
         const float4 p0 = mul4(f[0], a[0]), p1 = mul4(f[1], a[1]), p2 = mul4(f[2], a[2]), p3 = mul4(f[3], a[3]);
         const float vv[12] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w,
@@ -100,12 +122,15 @@ struct EdgeLoads {
 };
 
 // register budget of 5 waves per SIMD (102 VGPRs): room to keep a whole step's loads in flight
-__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 5))) painn_message_kernel(
+// TABLE: `filt` is a table of the filter over one period of the distance (rows d = k / inv_h, k = 0 .. tab_mask)
+// instead of one row per edge
+template <bool TABLE>
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TABLE ? 3 : 4, TABLE ? 4 : 5))) painn_message_kernel(
     const int* __restrict__ row_ptr, const int* __restrict__ dst, const int* __restrict__ node_order, long n_nodes,
     const float* __restrict__ r_ij,
     const float* __restrict__ filt, const float* __restrict__ actv, const float* __restrict__ x_v, int n,
     float epsilon, const float* __restrict__ res_a, const float* __restrict__ res_v, float* __restrict__ out_a,
-    float* __restrict__ out_v, Chunks ch) {
+    float* __restrict__ out_v, Chunks ch, int tab_mask, float inv_h) {
     const int lane = threadIdx.x & (kWave - 1);
     // Workgroup ids are dealt round-robin to the 8 XCDs, each with its own L2.  Give every XCD
     // one contiguous range of nodes: neighbouring nodes share most of their neighbours, so the
@@ -137,12 +162,23 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 5))
         if (e < hi) { j = dst[e]; rx = r_ij[3 * e]; ry = r_ij[3 * e + 1]; rz = r_ij[3 * e + 2]; }
         while (e < hi) {
             EdgeLoads ld;
-            ld.load(filt + e * row_f, actv + j * row_f, x_v + j * 3L * n, n, c);
+            const float r2 = rx * rx + ry * ry + rz * rz;
+            if constexpr (TABLE) {
+                const float u = sqrtf(r2) * inv_h;
+                const float fl = floorf(u);
+                const float t = u - fl;
+                const float tp = t + 1.0f, tm = t - 1.0f, tq = t - 2.0f;
+                const float w[4] = {-(1.0f / 6.0f) * t * tm * tq, 0.5f * tp * tm * tq, -0.5f * tp * t * tq,
+                                    (1.0f / 6.0f) * tp * t * tm};
+                ld.load_table(filt, (int)fl, tab_mask, w, actv + j * row_f, x_v + j * 3L * n, n, c);
+            } else {
+                ld.load(filt + e * row_f, actv + j * row_f, x_v + j * 3L * n, n, c);
+            }
             const long e_next = e + per_iter;
             long j_next = 0;
             float nx = 0.f, ny = 0.f, nz = 0.f;
             if (e_next < hi) { j_next = dst[e_next]; nx = r_ij[3 * e_next]; ny = r_ij[3 * e_next + 1]; nz = r_ij[3 * e_next + 2]; }
-            const float inv = 1.0f / sqrtf(epsilon + (rx * rx + ry * ry + rz * rz));
+            const float inv = 1.0f / sqrtf(epsilon + r2);
             ld.accumulate(acc, rx * inv, ry * inv, rz * inv);
             e = e_next; j = j_next; rx = nx; ry = ny; rz = nz;
         }
@@ -367,8 +403,9 @@ int mg_painn_message(const int* row_ptr, const int* dst, const int* node_order, 
             long blocks = ceil_div((long)n_nodes * ch.n, 4);
             if (blocks > 256L * 32) blocks = 256L * 32;
             blocks = ceil_div(blocks, 8) * 8;   // the XCD-aware item order needs a multiple of 8
-            hipLaunchKernelGGL(painn_message_kernel, dim3((unsigned)blocks), dim3(256), 0, st, row_ptr, dst,
-                               node_order, (long)n_nodes, r_ij, filt, actv, x_v, n, epsilon, res_a, res_v, out_a, out_v, ch);
+            hipLaunchKernelGGL(painn_message_kernel<false>, dim3((unsigned)blocks), dim3(256), 0, st, row_ptr, dst,
+                               node_order, (long)n_nodes, r_ij, filt, actv, x_v, n, epsilon, res_a, res_v, out_a, out_v, ch,
+                               0, 0.f);
             return check_launch("mg_painn_message");
         }
     }
@@ -377,6 +414,33 @@ int mg_painn_message(const int* row_ptr, const int* dst, const int* node_order, 
     hipLaunchKernelGGL(painn_message_scalar_kernel, dim3((unsigned)blocks), dim3(256), 0, st, row_ptr, dst,
                        (long)n_nodes, r_ij, filt, actv, x_v, n, epsilon, res_a, res_v, out_a, out_v);
     return check_launch("mg_painn_message");
+}
+
+int mg_painn_table_message(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
+                           const float* r_ij, const float* table, int table_rows, float period, const float* actv,
+                           const float* x_v, int n, float epsilon, const float* res_a, const float* res_v, float* out_a,
+                           float* out_v, mg_stream_t stream) {
+    MG_REQUIRE(n_nodes >= 0 && n_edges >= 0 && n >= 0, "mg_painn_table_message: negative size");
+    if (n_nodes == 0 || n == 0) return MG_OK;
+    MG_REQUIRE(row_ptr && out_a && out_v && actv && x_v && table, "mg_painn_table_message: null pointer");
+    MG_REQUIRE(n_edges == 0 || (dst && r_ij), "mg_painn_table_message: null edge operand");
+    MG_REQUIRE(table_rows >= 4 && (table_rows & (table_rows - 1)) == 0,
+               "mg_painn_table_message: table_rows must be a power of two >= 4 (got %d)", table_rows);
+    MG_REQUIRE(period > 0.f, "mg_painn_table_message: period must be positive");
+    MG_REQUIRE(n % 4 == 0 && aligned16(table) && aligned16(actv) && aligned16(x_v) && aligned16(out_a) && aligned16(out_v) &&
+                   (!res_a || aligned16(res_a)) && (!res_v || aligned16(res_v)),
+               "mg_painn_table_message: n must be a multiple of 4 and the operands 16-byte aligned");
+    const Chunks ch = make_chunks(n / 4, 4);
+    int covered = 0;
+    for (int k = 0; k < ch.n; k++) covered += ch.lanes[k] * 4;
+    MG_REQUIRE(covered == n, "mg_painn_table_message: unsupported channel count %d", n);
+    long blocks = ceil_div((long)n_nodes * ch.n, 4);
+    if (blocks > 256L * 32) blocks = 256L * 32;
+    blocks = ceil_div(blocks, 8) * 8;
+    hipLaunchKernelGGL(painn_message_kernel<true>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, row_ptr, dst,
+                       node_order, (long)n_nodes, r_ij, table, actv, x_v, n, epsilon, res_a, res_v, out_a, out_v, ch,
+                       table_rows - 1, (float)table_rows / period);
+    return check_launch("mg_painn_table_message");
 }
 
 }  // extern "C"

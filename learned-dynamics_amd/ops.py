@@ -1052,6 +1052,44 @@ def painn_message(row_ptr, dst, r_ij, filt, actv, x_v, epsilon, res_a=None, res_
     return out_a, out_v
 
 
+def painn_table_message(row_ptr, dst, r_ij, table, period, actv, x_v, epsilon, res_a=None, res_v=None, node_order=None):
+    """painn_message with the per-edge filter interpolated from `table` (rows, 4n): the filter as a function of
+    the edge length at d = k * period / rows (rows a power of two; the function has period `period`)."""
+    _check_input(row_ptr, "row_ptr", torch.int32)
+    _check_input(dst, "dst", torch.int32)
+    for t, nm in ((r_ij, "r_ij"), (table, "table"), (actv, "actv"), (x_v, "x_v")):
+        _check_input(t, nm)
+    n_nodes, n = int(x_v.size(0)), int(x_v.size(1))
+    E = int(dst.numel())
+    if tuple(x_v.shape) != (n_nodes, n, 3):
+        raise RuntimeError("x_v must have shape (nodes, n, 3)")
+    if tuple(actv.shape) != (n_nodes, 4 * n):
+        raise RuntimeError("actv must have shape (nodes, 4n)")
+    if table.dim() != 2 or table.size(1) != 4 * n:
+        raise RuntimeError("table must have shape (rows, 4n)")
+    if tuple(r_ij.shape) != (E, 3):
+        raise RuntimeError("r_ij must have shape (edges, 3)")
+    if row_ptr.numel() != n_nodes + 1:
+        raise RuntimeError("row_ptr must have nodes+1 entries")
+    for t, nm, shape in ((res_a, "res_a", (n_nodes, n)), (res_v, "res_v", (n_nodes, n, 3))):
+        if t is not None:
+            _check_input(t, nm)
+            if tuple(t.shape) != shape:
+                raise RuntimeError(f"{nm} has wrong shape")
+    if node_order is not None:
+        _check_input(node_order, "node_order", torch.int32)
+        if node_order.numel() != n_nodes:
+            raise RuntimeError("node_order must have one entry per node")
+    dev = x_v.device
+    with torch.cuda.device(dev):
+        out_a = torch.empty(n_nodes, n, dtype=torch.float32, device=dev)
+        out_v = torch.empty(n_nodes, n, 3, dtype=torch.float32, device=dev)
+        L.check(_lib.mg_painn_table_message(_p(row_ptr), _p(dst), _p(node_order), n_nodes, E, _p(r_ij), _p(table),
+                                            int(table.size(0)), float(period), _p(actv), _p(x_v), n, float(epsilon),
+                                            _p(res_a), _p(res_v), _p(out_a), _p(out_v), _stream()))
+    return out_a, out_v
+
+
 def bee_products_linear_supported(n_nodes, chan):
     return get_linear_mode() == LINEAR_F16X2 and chan % 32 == 0 and chan >= 32 and n_nodes >= 1024
 

@@ -14,6 +14,8 @@ Inference path.  Exact algebraic restructurings relative to the reference:
 Message takes an optional n_rbf (number of radial functions); the default n
 reproduces the reference.
 """
+import math
+
 import torch
 import torch.nn as nn
 
@@ -154,6 +156,53 @@ class Message(nn.Module):
                 cache.update(stamp=stamp, W=last.weight[perm].contiguous(), b=last.bias[perm].contiguous())
         return cache["W"], cache["b"]
 
+    # The filter sees an edge only through its length d, and radial_encode is made of cos / sin (k pi d / r0) with
+    # integer k: the filter is a smooth function of d with period 2 r0.  It is evaluated on a grid over one period
+    # (a few thousand rows through the same kernels as the exact path) and every edge interpolates between the four
+    # grid rows around its d.  The grid is accepted per set of weights by comparing the interpolation with the exact
+    # filter at the grid's midpoints, where the 4-point Lagrange error is largest.
+    TABLE_ROWS = (2048, 4096, 8192)
+    TABLE_TOL = 3e-6            # of max |filter|: the level of the split-fp16 GEMMs that evaluate the filter itself
+    use_table = True
+
+    def _grid_encoding(self, rows, shift, device):
+        """radial_encode at the lengths (k + shift) 2 r0 / rows, k = 0 .. rows - 1: (rows, n_rbf).  The lengths are
+        known exactly, so the phases are formed in float64 and only the encodings are rounded to float32."""
+        cache = self.__dict__.setdefault("_grid_cache", {})
+        key = (rows, shift, str(device))
+        if key not in cache:
+            n = self.n_rbf
+            hn = (n + 1) // 2
+            d = (torch.arange(rows, dtype=torch.float64) + shift) * (2.0 * self.r0 / rows)
+            phase = (math.pi / self.r0) * (1 + torch.arange(hn) // 2).to(torch.float64)[None, :] * d[:, None]
+            enc = torch.cat([torch.cos(phase), torch.sin(phase[:, :n - hn])], dim=-1)
+            cache[key] = enc.to(torch.float32).to(device).contiguous()
+        return cache[key]
+
+    def filter_table(self, rows, shift=0.0):
+        """The filter at d = (k + shift) 2 r0 / rows, k = 0 .. rows - 1: (rows, 4n)."""
+        enc = self._grid_encoding(rows, shift, self.mlp_dist.layers[0].weight.device)
+        return self.mlp_dist(enc, ops.linear_in_unit_bound(enc.device))
+
+    def table_rows(self):
+        """Rows of the grid whose interpolation error is below TABLE_TOL for the current weights, or 0 if none of
+        TABLE_ROWS is fine enough (then the filter is evaluated per edge).  Decided once per set of weights."""
+        params = list(self.mlp_dist.parameters())
+        stamp = tuple((id(p), p._version, p.data_ptr()) for p in params)
+        cache = self.__dict__.setdefault("_table_cache", {})
+        if cache.get("stamp") != stamp:
+            chosen = 0
+            with torch.no_grad():
+                for rows in self.TABLE_ROWS:
+                    tab = self.filter_table(rows)
+                    mid = self.filter_table(rows, 0.5)
+                    interp = (9.0 / 16.0) * (tab + tab.roll(-1, 0)) - (1.0 / 16.0) * (tab.roll(1, 0) + tab.roll(-2, 0))
+                    if float((interp - mid).abs().max()) <= self.TABLE_TOL * float(tab.abs().max()):
+                        chosen = rows
+                        break
+            cache.update(stamp=stamp, rows=chosen)
+        return cache["rows"]
+
     def forward(self, graph: Graph, x_a, x_v, r_ij, residual=False):
         """x_a: (batch, atoms, n), x_v: (batch, atoms, n, 3), r_ij: (edges, 3).
         Returns (dx_a, dx_v), or (x_a + dx_a, x_v + dx_v) with residual=True."""
@@ -163,6 +212,13 @@ class Message(nn.Module):
         r_ij = r_ij.contiguous()
         actv = self.mlp_actv(flat_a)
         res_a, res_v = (flat_a, flat_v) if residual else (None, None)
+        if self.use_table and n % 4 == 0 and r_ij.shape[0] >= 4 * self.TABLE_ROWS[0]:
+            rows = self.table_rows()
+            if rows and r_ij.shape[0] >= 4 * rows:
+                # the grid is re-evaluated in every call (a few thousand rows): nothing of a forward is cached
+                out_a, out_v = ops.painn_table_message(graph.row_ptr, graph.dst32, r_ij, self.filter_table(rows),
+                                                       2.0 * self.r0, actv, flat_v, self.epsilon, res_a, res_v)
+                return out_a.reshape(B, N, n), out_v.reshape(B, N, n, 3)
         if ops.painn_filter_message_supported(n, 4 * n, r_ij.shape[0]):
             # the filter's last layer runs inside the edge kernel: the (edges, 4n) filter is never stored
             first, second = self.mlp_dist.layers[0], self.mlp_dist.layers[2]
