@@ -318,3 +318,84 @@ def test_first_two_filter_layers_from_edge_vectors(ops, hidden, E):
     scale = float(ref.abs().max())
     torch.testing.assert_close(y, two, rtol=1e-5, atol=3e-6 * scale)
     torch.testing.assert_close(y.cpu().double(), ref, rtol=1e-5, atol=4e-6 * scale)
+
+
+@pytest.mark.parametrize("n,rows", [(128, 256), (32, 512), (20, 256)])
+def test_table_message_kernel_interpolates_a_known_periodic_filter(ops, n, rows):
+    """mg_painn_table_message with a table of an analytic filter, cos(m pi d / r0 + phase) per column with m <= 3,
+    against mg_painn_message fed with that filter evaluated per edge in float64.  Edge lengths run from 0 to beyond
+    two periods, so the wrap of the row index and the interval [rows - 1, rows) are covered.  4-point Lagrange error
+    bound: 0.0234 h^4 (3 pi / r0)^4 = 7e-7 at h = 2 r0 / 256, r0 = 4."""
+    g = torch.Generator().manual_seed(n + rows)
+    r0, N = 4.0, 300
+    deg = torch.randint(0, 40, (N,), generator=g)
+    src = torch.repeat_interleave(torch.arange(N), deg)
+    E = int(src.numel())
+    dst = torch.randint(0, N, (E,), generator=g)
+    length = torch.rand(E, generator=g).double() * 4.5 * r0
+    length[:4] = torch.tensor([0.0, 2 * r0, 2 * r0 * (1 - 1e-7), 2 * r0 * (rows - 0.5) / rows])
+    direction = torch.randn(E, 3, generator=g).double()
+    r = (direction / direction.norm(dim=-1, keepdim=True) * length[:, None]).float()
+    m = torch.randint(0, 4, (4 * n,), generator=g).double()
+    phase = torch.rand(4 * n, generator=g).double() * 6.28
+    amp = torch.randn(4 * n, generator=g).double()
+    f = lambda d: amp * torch.cos(m * (torch.pi / r0) * d[:, None] + phase)
+    table = f(torch.arange(rows).double() * (2 * r0 / rows)).float()
+    filt = f(r.double().norm(dim=-1)).float()                # at the float32 edge vectors the kernel sees
+    actv = torch.randn(N, 4 * n, generator=g)
+    x_a, x_v = torch.randn(N, n, generator=g), torch.randn(N, n, 3, generator=g)
+    dev = lambda t: t.cuda()
+    row_ptr = ops.segment_row_ptr(dev(src.int()), N)
+    got_a, got_v = ops.painn_table_message(row_ptr, dev(dst.int()), dev(r), dev(table), 2 * r0, dev(actv), dev(x_v), 0.1,
+                                           dev(x_a), dev(x_v))
+    ref_a, ref_v = ops.painn_message(row_ptr, dev(dst.int()), dev(r), dev(filt), dev(actv), dev(x_v), 0.1, dev(x_a), dev(x_v))
+    _close(got_a, ref_a.cpu(), atol_scale=3e-6)
+    _close(got_v, ref_v.cpu(), atol_scale=3e-6)
+    with pytest.raises(RuntimeError, match="power of two"):
+        ops.painn_table_message(row_ptr, dev(dst.int()), dev(r), dev(table[:rows - 1].contiguous()), 2 * r0, dev(actv),
+                                dev(x_v), 0.1)
+
+
+@pytest.mark.parametrize("n_rbf", [16, None])
+def test_message_with_filter_table_equals_filter_mlp_per_edge(pkg, n_rbf):
+    """Message.forward through the grid of the filter against the same module evaluating the filter MLP on every
+    edge, on edge vectors of any length (the filter has period 2 r0 in the length)."""
+    painn = importlib.import_module("learned-dynamics_amd.painn")
+    torch.manual_seed(7)
+    n, N, r0 = 64, 512, 6.0
+    msg = painn.Message(r0, n, n_rbf).cuda()
+    g = torch.Generator().manual_seed(8)
+    deg = torch.randint(20, 60, (N,), generator=g)
+    src = torch.repeat_interleave(torch.arange(N), deg)
+    E = int(src.numel())
+    dst = torch.randint(0, N, (E,), generator=g)
+    r = torch.randn(E, 3, generator=g) * torch.rand(E, 1, generator=g) * 2.5 * r0
+    r[0] = 0.0
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    graph = gl.Graph(src.cuda(), dst.cuda(), None, 1, N)
+    x_a, x_v = torch.randn(1, N, n).cuda(), torch.randn(1, N, n, 3).cuda()
+    with torch.no_grad():
+        rows = msg.table_rows()
+        assert rows in msg.TABLE_ROWS and E >= 4 * rows
+        a1, v1 = msg(graph, x_a, x_v, r.cuda(), residual=True)
+        msg.use_table = False
+        a0, v0 = msg(graph, x_a, x_v, r.cuda(), residual=True)
+    assert float(r.norm(dim=-1).max()) > 2 * r0
+    _close(a1, a0.cpu(), atol_scale=3e-6)
+    _close(v1, v0.cpu(), atol_scale=3e-6)
+
+
+def test_filter_table_is_rejected_when_the_filter_is_too_rough(pkg):
+    """With first-layer weights scaled up the filter varies faster than any of the grids resolves: the midpoint
+    check refuses them and the module evaluates the MLP per edge; a change of the weights is noticed."""
+    painn = importlib.import_module("learned-dynamics_amd.painn")
+    torch.manual_seed(9)
+    msg = painn.Message(6.0, 32, 32).cuda()
+    with torch.no_grad():
+        assert msg.table_rows() in msg.TABLE_ROWS
+        msg.mlp_dist.layers[0].weight.mul_(300.0)
+        msg.mlp_dist.layers[2].weight.mul_(30.0)
+        assert msg.table_rows() == 0
+        msg.mlp_dist.layers[0].weight.mul_(1 / 300.0)
+        msg.mlp_dist.layers[2].weight.mul_(1 / 30.0)
+        assert msg.table_rows() in msg.TABLE_ROWS
