@@ -104,7 +104,11 @@ struct EdgeLoads {
         for (int k = 0; k < 3; k++) v[k] = ld4(xv_row + 3 * c + 4 * k);
     }
     __device__ __forceinline__ void accumulate(EdgeAcc& acc, float ux, float uy, float uz) const {
-        const float4 p0 = mul4(f[0], a[0]), p1 = mul4(f[1], a[1]), p2 = mul4(f[2], a[2]), p3 = mul4(f[3], a[3]);
+        accumulate_products(acc, mul4(f[0], a[0]), mul4(f[1], a[1]), mul4(f[2], a[2]), mul4(f[3], a[3]), ux, uy, uz);
+    }
+    // p0 .. p3: filter x activation of the four blocks for this lane's 4 channels
+    __device__ __forceinline__ void accumulate_products(EdgeAcc& acc, float4 p0, float4 p1, float4 p2, float4 p3, float ux,
+                                                        float uy, float uz) const {
         const float vv[12] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w,
                               v[2].x, v[2].y, v[2].z, v[2].w};
         const float q0[4] = {p0.x, p0.y, p0.z, p0.w}, q1[4] = {p1.x, p1.y, p1.z, p1.w};
@@ -203,6 +207,116 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TABLE 
                 for (int k = 0; k < 12; k++) acc.v[k] += rr[k];
             }
             st4(oa, make_float4(acc.a[0], acc.a[1], acc.a[2], acc.a[3]));
+            st4(ov, make_float4(acc.v[0], acc.v[1], acc.v[2], acc.v[3]));
+            st4(ov + 4, make_float4(acc.v[4], acc.v[5], acc.v[6], acc.v[7]));
+            st4(ov + 8, make_float4(acc.v[8], acc.v[9], acc.v[10], acc.v[11]));
+        }
+    }
+}
+
+// The table variant with the grid in LDS.  A workgroup owns one slice of 16 channels (its 4 x 16 filter columns of
+// every grid row: rows x 64 floats, at most 512 rows) and walks over nodes; the 4 lanes of an edge hold 4 channels
+// each, so a wave takes 16 edges of its node per step and only the node rows (actv, x_v) come through the vector
+// caches: 3.5 KB per edge instead of 11.5 KB.  actv is expected slice-major, (node, n / 16, 4, 16), so that a
+// slice's 64 values are two whole cache lines; x_v (node, n, 3) already has a slice's 48 values contiguous.
+// Bank conflicts: the 4 lanes of an edge read 64 contiguous bytes of a random grid row, so which banks an edge hits
+// must not depend on its row.  LDS rows are exactly 64 floats and edge slot s reads the blocks in the order
+// (q + s) % 4, q = 0..3: neighbouring edge slots are always in different 16-bank groups.  actv is gathered in the
+// same rotated order and the four products are rotated back in registers (two conditional swaps).
+constexpr int kSliceChan = 16, kSliceCols = 4 * kSliceChan, kSliceRowF = kSliceCols, kSliceMaxRows = 512;
+
+__global__ void __launch_bounds__(1024) painn_table_message_lds_kernel(
+    const int* __restrict__ row_ptr, const int* __restrict__ dst, long n_nodes, const float* __restrict__ r_ij,
+    const float* __restrict__ table, int tab_rows, float inv_h, const float* __restrict__ actv_s,
+    const float* __restrict__ x_v, int n, float epsilon, const float* __restrict__ res_a,
+    const float* __restrict__ res_v, float* __restrict__ out_a, float* __restrict__ out_v) {
+    extern __shared__ float tab[];                            // tab_rows x kSliceRowF
+    const int n_slices = n / kSliceChan;
+    const int slice = blockIdx.x % n_slices;
+    const int group = blockIdx.x / n_slices, groups = gridDim.x / n_slices;
+    for (int q = threadIdx.x; q < tab_rows * (kSliceCols / 4); q += blockDim.x) {
+        const int row = q / (kSliceCols / 4), piece = q % (kSliceCols / 4), k = piece / 4, c4 = piece % 4;
+        st4(tab + row * kSliceRowF + 4 * piece, ld4(table + (long)row * 4 * n + k * n + slice * kSliceChan + 4 * c4));
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave, waves = blockDim.x / kWave;
+    const int l4 = lane & 3, sub = lane >> 2;                 // 4 channels of edge `sub` of the step
+    constexpr int kPerIter = kWave / 4;
+    const int mask = tab_rows - 1;
+    for (long node = (long)group * waves + wave; node < n_nodes; node += (long)groups * waves) {
+        const long lo = row_ptr[node], hi = row_ptr[node + 1];
+        EdgeAcc acc;
+        acc.zero();
+        long e = lo + sub;
+        long j = 0;
+        float rx = 0.f, ry = 0.f, rz = 0.f;
+        if (e < hi) { j = dst[e]; rx = r_ij[3 * e]; ry = r_ij[3 * e + 1]; rz = r_ij[3 * e + 2]; }
+        while (e < hi) {
+            EdgeLoads ld;
+            const float* a_row = actv_s + (j * n_slices + slice) * kSliceCols + 4 * l4;
+            const float* v_row = x_v + (j * n + slice * kSliceChan + 4 * l4) * 3;
+#pragma unroll
+            for (int q = 0; q < 4; q++) ld.a[q] = ld4(a_row + ((q + sub) & 3) * kSliceChan);
+#pragma unroll
+            for (int k = 0; k < 3; k++) ld.v[k] = ld4(v_row + 4 * k);
+            const long e_next = e + kPerIter;
+            long j_next = 0;
+            float nx = 0.f, ny = 0.f, nz = 0.f;
+            if (e_next < hi) { j_next = dst[e_next]; nx = r_ij[3 * e_next]; ny = r_ij[3 * e_next + 1]; nz = r_ij[3 * e_next + 2]; }
+            const float r2 = rx * rx + ry * ry + rz * rz;
+            const float u = sqrtf(r2) * inv_h;
+            const float fl = floorf(u);
+            const float t = u - fl;
+            const float tp = t + 1.0f, tm = t - 1.0f, tq = t - 2.0f;
+            const float w0 = -(1.0f / 6.0f) * t * tm * tq, w1 = 0.5f * tp * tm * tq, w2 = -0.5f * tp * t * tq,
+                        w3 = (1.0f / 6.0f) * tp * t * tm;
+            const int i = (int)fl;
+            const float* p0 = tab + ((i - 1) & mask) * kSliceRowF + 4 * l4;
+            const float* p1 = tab + (i & mask) * kSliceRowF + 4 * l4;
+            const float* p2 = tab + ((i + 1) & mask) * kSliceRowF + 4 * l4;
+            const float* p3 = tab + ((i + 2) & mask) * kSliceRowF + 4 * l4;
+            float4 pr[4];                                     // pr[q]: product of block (q + sub) % 4
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const int off = ((q + sub) & 3) * kSliceChan;
+                const float4 t0 = ld4(p0 + off), t1 = ld4(p1 + off), t2 = ld4(p2 + off), t3 = ld4(p3 + off);
+                const float4 fq = make_float4(w0 * t0.x + w1 * t1.x + w2 * t2.x + w3 * t3.x, w0 * t0.y + w1 * t1.y + w2 * t2.y + w3 * t3.y,
+                                              w0 * t0.z + w1 * t1.z + w2 * t2.z + w3 * t3.z, w0 * t0.w + w1 * t1.w + w2 * t2.w + w3 * t3.w);
+                pr[q] = mul4(fq, ld.a[q]);
+            }
+            // block k sits in pr[(k - sub) % 4]: rotate by sub's low bit, then by its second bit
+            const bool s1 = sub & 1, s2 = sub & 2;
+            auto sel = [](bool c, float4 x, float4 y) { return make_float4(c ? x.x : y.x, c ? x.y : y.y, c ? x.z : y.z, c ? x.w : y.w); };
+            float4 tr[4], bk[4];
+#pragma unroll
+            for (int k = 0; k < 4; k++) tr[k] = sel(s1, pr[(k + 3) & 3], pr[k]);
+#pragma unroll
+            for (int k = 0; k < 4; k++) bk[k] = sel(s2, tr[(k + 2) & 3], tr[k]);
+            const float inv = 1.0f / sqrtf(epsilon + r2);
+            ld.accumulate_products(acc, bk[0], bk[1], bk[2], bk[3], rx * inv, ry * inv, rz * inv);
+            e = e_next; j = j_next; rx = nx; ry = ny; rz = nz;
+        }
+        for (int d = 4; d < kWave; d <<= 1) {
+#pragma unroll
+            for (int k = 0; k < 12; k++) acc.v[k] += __shfl_xor(acc.v[k], d);
+#pragma unroll
+            for (int k = 0; k < 4; k++) acc.a[k] += __shfl_xor(acc.a[k], d);
+        }
+        if (sub == 0) {
+            const long o = node * n + slice * kSliceChan + 4 * l4;
+            if (res_a) {
+                const float4 r = ld4(res_a + o);
+                acc.a[0] += r.x; acc.a[1] += r.y; acc.a[2] += r.z; acc.a[3] += r.w;
+            }
+            if (res_v) {
+                const float* rv = res_v + o * 3;
+                const float4 ra = ld4(rv), rb = ld4(rv + 4), rc = ld4(rv + 8);
+                const float rr[12] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w, rc.x, rc.y, rc.z, rc.w};
+#pragma unroll
+                for (int k = 0; k < 12; k++) acc.v[k] += rr[k];
+            }
+            st4(out_a + o, make_float4(acc.a[0], acc.a[1], acc.a[2], acc.a[3]));
+            float* ov = out_v + o * 3;
             st4(ov, make_float4(acc.v[0], acc.v[1], acc.v[2], acc.v[3]));
             st4(ov + 4, make_float4(acc.v[4], acc.v[5], acc.v[6], acc.v[7]));
             st4(ov + 8, make_float4(acc.v[8], acc.v[9], acc.v[10], acc.v[11]));
@@ -441,6 +555,34 @@ int mg_painn_table_message(const int* row_ptr, const int* dst, const int* node_o
                        node_order, (long)n_nodes, r_ij, table, actv, x_v, n, epsilon, res_a, res_v, out_a, out_v, ch,
                        table_rows - 1, (float)table_rows / period);
     return check_launch("mg_painn_table_message");
+}
+
+int mg_painn_table_message_sliced(const int* row_ptr, const int* dst, int n_nodes, long n_edges, const float* r_ij,
+                                  const float* table, int table_rows, float period, const float* actv_sliced,
+                                  const float* x_v, int n, float epsilon, const float* res_a, const float* res_v,
+                                  float* out_a, float* out_v, mg_stream_t stream) {
+    MG_REQUIRE(n_nodes >= 0 && n_edges >= 0 && n >= 0, "mg_painn_table_message_sliced: negative size");
+    if (n_nodes == 0 || n == 0) return MG_OK;
+    MG_REQUIRE(row_ptr && out_a && out_v && actv_sliced && x_v && table, "mg_painn_table_message_sliced: null pointer");
+    MG_REQUIRE(n_edges == 0 || (dst && r_ij), "mg_painn_table_message_sliced: null edge operand");
+    MG_REQUIRE(table_rows >= 4 && table_rows <= kSliceMaxRows && (table_rows & (table_rows - 1)) == 0,
+               "mg_painn_table_message_sliced: table_rows must be a power of two in 4..%d (got %d)", kSliceMaxRows, table_rows);
+    MG_REQUIRE(period > 0.f, "mg_painn_table_message_sliced: period must be positive");
+    MG_REQUIRE(n % kSliceChan == 0 && aligned16(table) && aligned16(actv_sliced) && aligned16(x_v) && aligned16(out_a) &&
+                   aligned16(out_v) && (!res_a || aligned16(res_a)) && (!res_v || aligned16(res_v)),
+               "mg_painn_table_message_sliced: n must be a multiple of %d and the operands 16-byte aligned", kSliceChan);
+    const int n_slices = n / kSliceChan;
+    const size_t lds_bytes = (size_t)table_rows * kSliceRowF * sizeof(float);
+    // more than 64 KB of dynamic LDS has to be asked for (per device, so on every call)
+    MG_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(painn_table_message_lds_kernel),
+                               hipFuncAttributeMaxDynamicSharedMemorySize, kSliceMaxRows * kSliceRowF * (int)sizeof(float)));
+    long groups = ceil_div(256, n_slices);                    // one workgroup per CU
+    const long max_groups = ceil_div(n_nodes, 16);
+    if (groups > max_groups) groups = max_groups;
+    hipLaunchKernelGGL(painn_table_message_lds_kernel, dim3((unsigned)(groups * n_slices)), dim3(1024), lds_bytes,
+                       (hipStream_t)stream, row_ptr, dst, (long)n_nodes, r_ij, table, table_rows, (float)table_rows / period,
+                       actv_sliced, x_v, n, epsilon, res_a, res_v, out_a, out_v);
+    return check_launch("mg_painn_table_message_sliced");
 }
 
 }  // extern "C"

@@ -628,7 +628,7 @@ def linear_out_bound(W, bias, in_bound):
 
 
 def f16x2_supported(rows, dim_in, dim_out, x):
-    return dim_in % 32 == 0 and dim_in >= 64 and dim_out >= 8 and rows >= 1024 and x.data_ptr() % 16 == 0
+    return dim_in % 32 == 0 and dim_in >= 64 and dim_out >= 8 and rows >= 256 and x.data_ptr() % 16 == 0
 
 
 def tensor_linear_f16x2(W, x, x_rowmax=None, bias=None, act=ACT_NONE, out=None, accumulate=False, out_comps=1,
@@ -1087,6 +1087,51 @@ def painn_table_message(row_ptr, dst, r_ij, table, period, actv, x_v, epsilon, r
         L.check(_lib.mg_painn_table_message(_p(row_ptr), _p(dst), _p(node_order), n_nodes, E, _p(r_ij), _p(table),
                                             int(table.size(0)), float(period), _p(actv), _p(x_v), n, float(epsilon),
                                             _p(res_a), _p(res_v), _p(out_a), _p(out_v), _stream()))
+    return out_a, out_v
+
+
+PAINN_SLICE = 16              # channels per slice of painn_table_message_sliced
+PAINN_SLICED_MAX_ROWS = 512   # table rows that fit in LDS beside a slice's 64 columns
+
+
+def painn_slice_permutation(n, device):
+    """Column order of actv for painn_table_message_sliced: position (s, k, c) of (n / 16, 4, 16) holds column
+    k n + 16 s + c."""
+    s, k, c = torch.meshgrid(torch.arange(n // PAINN_SLICE), torch.arange(4), torch.arange(PAINN_SLICE), indexing="ij")
+    return (k * n + PAINN_SLICE * s + c).reshape(-1).to(device)
+
+
+def painn_table_message_sliced(row_ptr, dst, r_ij, table, period, actv_sliced, x_v, epsilon, res_a=None, res_v=None):
+    """painn_table_message with the table held in LDS (at most 512 rows, n a multiple of 16) and actv given with its
+    columns in the order of painn_slice_permutation."""
+    _check_input(row_ptr, "row_ptr", torch.int32)
+    _check_input(dst, "dst", torch.int32)
+    for t, nm in ((r_ij, "r_ij"), (table, "table"), (actv_sliced, "actv_sliced"), (x_v, "x_v")):
+        _check_input(t, nm)
+    n_nodes, n = int(x_v.size(0)), int(x_v.size(1))
+    E = int(dst.numel())
+    if tuple(x_v.shape) != (n_nodes, n, 3):
+        raise RuntimeError("x_v must have shape (nodes, n, 3)")
+    if tuple(actv_sliced.shape) != (n_nodes, 4 * n):
+        raise RuntimeError("actv_sliced must have shape (nodes, 4n)")
+    if table.dim() != 2 or table.size(1) != 4 * n:
+        raise RuntimeError("table must have shape (rows, 4n)")
+    if tuple(r_ij.shape) != (E, 3):
+        raise RuntimeError("r_ij must have shape (edges, 3)")
+    if row_ptr.numel() != n_nodes + 1:
+        raise RuntimeError("row_ptr must have nodes+1 entries")
+    for t, nm, shape in ((res_a, "res_a", (n_nodes, n)), (res_v, "res_v", (n_nodes, n, 3))):
+        if t is not None:
+            _check_input(t, nm)
+            if tuple(t.shape) != shape:
+                raise RuntimeError(f"{nm} has wrong shape")
+    dev = x_v.device
+    with torch.cuda.device(dev):
+        out_a = torch.empty(n_nodes, n, dtype=torch.float32, device=dev)
+        out_v = torch.empty(n_nodes, n, 3, dtype=torch.float32, device=dev)
+        L.check(_lib.mg_painn_table_message_sliced(_p(row_ptr), _p(dst), n_nodes, E, _p(r_ij), _p(table),
+                                                   int(table.size(0)), float(period), _p(actv_sliced), _p(x_v), n,
+                                                   float(epsilon), _p(res_a), _p(res_v), _p(out_a), _p(out_v), _stream()))
     return out_a, out_v
 
 

@@ -65,6 +65,11 @@ class MLP(nn.Module):
         h, bound = _linear(h, self.layers[0], ops.ACT_SILU, bound)
         return self.after_first(h, bound).reshape(*lead, -1)
 
+    def hidden(self, x, bound=None):
+        """The (rows, dim_out) input of the last layer and the bound of its rows."""
+        h, bound = _linear(x, self.layers[0], ops.ACT_SILU, bound)
+        return _linear(h, self.layers[2], ops.ACT_SILU, bound)
+
     def after_first(self, h, bound=None):
         """Layers 2 and 3 on the (rows, dim_out) output of the first layer + SiLU."""
         h, bound = _linear(h, self.layers[2], ops.ACT_SILU, bound)
@@ -145,6 +150,22 @@ class Message(nn.Module):
         """(edges, 3) -> (edges, 4n): the per-edge filter, the one large per-edge tensor."""
         return self.mlp_dist.after_first(*self._hidden(r_ij))
 
+    use_sliced = True
+
+    def _sliced_actv_last(self):
+        """Last layer of mlp_actv with its rows in the slice-major column order of painn_table_message_sliced."""
+        last = self.mlp_actv.layers[4]
+        cache = self.__dict__.setdefault("_slice_cache", {})
+        stamp = tuple((id(p), p._version, p.data_ptr()) for p in (last.weight, last.bias))
+        if cache.get("stamp") != stamp:
+            with torch.no_grad():
+                perm = ops.painn_slice_permutation(self.n, last.weight.device)
+                lin = nn.Linear(last.in_features, last.out_features, device=last.weight.device)
+                lin.weight.copy_(last.weight[perm])
+                lin.bias.copy_(last.bias[perm])
+            cache.update(stamp=stamp, lin=lin)
+        return cache["lin"]
+
     def _permuted_last(self):
         """Last layer of the filter MLP with its rows in the column order of the fused kernel."""
         last = self.mlp_dist.layers[4]
@@ -161,7 +182,7 @@ class Message(nn.Module):
     # (a few thousand rows through the same kernels as the exact path) and every edge interpolates between the four
     # grid rows around its d.  The grid is accepted per set of weights by comparing the interpolation with the exact
     # filter at the grid's midpoints, where the 4-point Lagrange error is largest.
-    TABLE_ROWS = (2048, 4096, 8192)
+    TABLE_ROWS = (512, 2048, 4096, 8192)      # 512 rows fit in LDS beside a slice of 16 channels
     TABLE_TOL = 3e-6            # of max |filter|: the level of the split-fp16 GEMMs that evaluate the filter itself
     use_table = True
 
@@ -210,15 +231,25 @@ class Message(nn.Module):
         flat_a = x_a.reshape(B * N, n).contiguous()
         flat_v = x_v.reshape(B * N, n, 3).contiguous()
         r_ij = r_ij.contiguous()
-        actv = self.mlp_actv(flat_a)
         res_a, res_v = (flat_a, flat_v) if residual else (None, None)
+        actv = None
         if self.use_table and n % 4 == 0 and r_ij.shape[0] >= 4 * self.TABLE_ROWS[0]:
             rows = self.table_rows()
+            if rows and rows <= ops.PAINN_SLICED_MAX_ROWS and n % ops.PAINN_SLICE == 0 and self.use_sliced:
+                # the grid fits in LDS: actv comes out of its MLP with the columns regrouped slice by slice
+                h_a, b_a = self.mlp_actv.hidden(flat_a)
+                actv_s = _linear(h_a, self._sliced_actv_last(), ops.ACT_NONE, b_a)[0]
+                out_a, out_v = ops.painn_table_message_sliced(graph.row_ptr, graph.dst32, r_ij, self.filter_table(rows),
+                                                              2.0 * self.r0, actv_s, flat_v, self.epsilon, res_a, res_v)
+                return out_a.reshape(B, N, n), out_v.reshape(B, N, n, 3)
+            actv = self.mlp_actv(flat_a)
             if rows and r_ij.shape[0] >= 4 * rows:
                 # the grid is re-evaluated in every call (a few thousand rows): nothing of a forward is cached
                 out_a, out_v = ops.painn_table_message(graph.row_ptr, graph.dst32, r_ij, self.filter_table(rows),
                                                        2.0 * self.r0, actv, flat_v, self.epsilon, res_a, res_v)
                 return out_a.reshape(B, N, n), out_v.reshape(B, N, n, 3)
+        if actv is None:
+            actv = self.mlp_actv(flat_a)
         if ops.painn_filter_message_supported(n, 4 * n, r_ij.shape[0]):
             # the filter's last layer runs inside the edge kernel: the (edges, 4n) filter is never stored
             first, second = self.mlp_dist.layers[0], self.mlp_dist.layers[2]
