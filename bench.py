@@ -233,30 +233,52 @@ def bench_painn_layer(torch, args):
             # kernel; the two GEMM kernels above are the path taken when the grid is rejected for a set of weights
             table = msg.filter_table(rows)
             t_build = event_time(torch, lambda: msg.filter_table(rows), 20)
-            t_table = event_time(torch, lambda: ops.painn_table_message(graph.row_ptr, graph.dst32, r_ij, table, 2 * r0,
-                                                                        actv, xv_flat, 0.1, xa_flat, xv_flat), 20)
+            sliced = msg.use_sliced and rows <= ops.PAINN_SLICED_MAX_ROWS and n % ops.PAINN_SLICE == 0
+            if sliced:
+                actv_s = actv[:, ops.painn_slice_permutation(n, "cuda")].contiguous()
+                t_table = event_time(torch, lambda: ops.painn_table_message_sliced(
+                    graph.row_ptr, graph.dst32, r_ij, table, 2 * r0, actv_s, xv_flat, 0.1, xa_flat, xv_flat), 20)
+                msg.use_sliced = False
+                sec_cached_grid = timed_steps(torch, step, max(3, args.steps // 4), 2)
+                msg.use_sliced = True
+                breakdown["layer_ms_with_the_grid_read_through_the_caches"] = sec_cached_grid * 1e3
+            else:
+                t_table = event_time(torch, lambda: ops.painn_table_message(
+                    graph.row_ptr, graph.dst32, r_ij, table, 2 * r0, actv, xv_flat, 0.1, xa_flat, xv_flat), 20)
             msg.use_table = False
             sec_exact = timed_steps(torch, step, max(3, args.steps // 4), 2)
             msg.use_table = True
             hbm_bytes = E * 16 + N * (16 * n + 12 * n) + 2 * N * 16 * n + rows * 16 * n
-            cache_bytes = E * (4 * 16 * n + 16 * n + 12 * n + 16)
+            gather_bytes = E * (16 * n + 12 * n + 16)
+            grid_bytes = E * 4 * 16 * n
+            cache_bytes = gather_bytes + (0 if sliced else grid_bytes)
             l1_fill_peak = 256 * 64 * 2.4                     # GB/s: 256 CUs x 64 B per clock x 2.4 GHz
+            flop = E * n * (4 * 4 * 2 + 4 + 9 + 18 + 1)       # interpolation, products, cross product, accumulation
             breakdown["filter_grid_evaluation_ms"] = t_build * 1e3
             breakdown["table_edge_kernel_ms"] = t_table * 1e3
             breakdown["layer_ms_with_filter_mlp_per_edge"] = sec_exact * 1e3
-            roofline = {"kernel": "painn_message_kernel<table> (per edge: 4 grid rows of the filter interpolated, node "
-                                  "rows gathered, products, sums over the edges of a node)",
-                        "bound": "hbm", "achieved": hbm_bytes / t_table / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                        "frac": hbm_bytes / t_table / 1e9 / PEAK_HBM_GBS,
-                        "traffic": measured_traffic("painn_message_kernel<true>"),
+            kernel = ("painn_table_message_lds_kernel (a workgroup keeps 16 channels of the %d-row filter grid in LDS; per "
+                      "edge: 4 grid rows interpolated, node rows gathered, products, sums over the edges of a node)" % rows
+                      if sliced else
+                      "painn_message_kernel<table> (per edge: 4 rows of the %d-row filter grid interpolated, node rows "
+                      "gathered, products, sums over the edges of a node)" % rows)
+            roofline = {"kernel": kernel, "bound": "hbm", "achieved": hbm_bytes / t_table / 1e9, "peak": PEAK_HBM_GBS,
+                        "unit": "GB/s", "frac": hbm_bytes / t_table / 1e9 / PEAK_HBM_GBS,
+                        "traffic": measured_traffic("painn_table_message_lds_kernel" if sliced else "painn_message_kernel<true>"),
                         "bytes_per_launch": hbm_bytes, "ms": t_table * 1e3,
                         "cache_to_cu": {"bytes_per_launch": cache_bytes, "achieved": cache_bytes / t_table / 1e9,
                                         "peak": l1_fill_peak, "unit": "GB/s",
                                         "frac": cache_bytes / t_table / 1e9 / l1_fill_peak},
-                        "note": "the kernel's operands are the 4 MB grid and node-sized arrays, all cache resident: its "
-                                "algorithmic HBM bytes are 20x fewer than the streamed-filter kernel's (roofline_hbm) at "
-                                "the same duration, so the HBM fraction is small by construction; what bounds it is the "
-                                "11.5 KB per edge that move from L2 to the CUs (cache_to_cu, against 64 B per clock per CU)",
+                        "lds_reads": {"bytes_per_launch": grid_bytes if sliced else 0,
+                                      "achieved": (grid_bytes if sliced else 0) / t_table / 1e9, "unit": "GB/s"},
+                        "fp32_vector": {"flop_per_launch": flop, "achieved": flop / t_table / 1e12, "unit": "TFLOP/s",
+                                        "peak": PEAK_FP32_MFMA_TFLOPS / 2,
+                                        "frac": flop / t_table / 1e12 / (PEAK_FP32_MFMA_TFLOPS / 2)},
+                        "note": "every operand of the kernel is cache resident (node-sized arrays and the filter grid), "
+                                "so its algorithmic HBM bytes are 20x fewer than those of the kernel that streams a "
+                                "stored filter (roofline_hbm) and the HBM fraction is small by construction; what "
+                                "bounds it is vector arithmetic (fp32_vector, without packed instructions) and the "
+                                "gathers of node rows from L2 (cache_to_cu, against 64 B per clock per CU)",
                         "filter_mlp_per_edge_path": roofline}
         del actv
 

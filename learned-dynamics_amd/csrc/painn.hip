@@ -219,11 +219,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TABLE 
 // each, so a wave takes 16 edges of its node per step and only the node rows (actv, x_v) come through the vector
 // caches: 3.5 KB per edge instead of 11.5 KB.  actv is expected slice-major, (node, n / 16, 4, 16), so that a
 // slice's 64 values are two whole cache lines; x_v (node, n, 3) already has a slice's 48 values contiguous.
-// Bank conflicts: the 4 lanes of an edge read 64 contiguous bytes of a random grid row, so which banks an edge hits
-// must not depend on its row.  LDS rows are exactly 64 floats and edge slot s reads the blocks in the order
-// (q + s) % 4, q = 0..3: neighbouring edge slots are always in different 16-bank groups.  actv is gathered in the
-// same rotated order and the four products are rotated back in registers (two conditional swaps).
-constexpr int kSliceChan = 16, kSliceCols = 4 * kSliceChan, kSliceRowF = kSliceCols, kSliceMaxRows = 512;
+// LDS rows are padded to 68 floats so that the rows different edges read start in different banks.
+constexpr int kSliceChan = 16, kSliceCols = 4 * kSliceChan, kSliceRowF = kSliceCols + 4, kSliceMaxRows = 512;
 
 __global__ void __launch_bounds__(1024) painn_table_message_lds_kernel(
     const int* __restrict__ row_ptr, const int* __restrict__ dst, long n_nodes, const float* __restrict__ r_ij,
@@ -243,26 +240,34 @@ __global__ void __launch_bounds__(1024) painn_table_message_lds_kernel(
     const int l4 = lane & 3, sub = lane >> 2;                 // 4 channels of edge `sub` of the step
     constexpr int kPerIter = kWave / 4;
     const int mask = tab_rows - 1;
+    // 32-bit element offsets (the host checks that they fit) and running pointers keep the address arithmetic,
+    // a third of the loop's vector instructions otherwise, short
+    const unsigned a_stride = (unsigned)n_slices * kSliceCols, v_stride = 3u * (unsigned)n;
+    const float* a_base = actv_s + slice * kSliceCols + 4 * l4;
+    const float* v_base = x_v + (slice * kSliceChan + 4 * l4) * 3;
+    const float* tab_l = tab + 4 * l4;
     for (long node = (long)group * waves + wave; node < n_nodes; node += (long)groups * waves) {
-        const long lo = row_ptr[node], hi = row_ptr[node + 1];
+        const int lo = row_ptr[node], hi = row_ptr[node + 1];
         EdgeAcc acc;
         acc.zero();
-        long e = lo + sub;
-        long j = 0;
+        int e = lo + sub;
+        const int* dp = dst + e;
+        const float* rp = r_ij + 3L * e;
+        unsigned j = 0;
         float rx = 0.f, ry = 0.f, rz = 0.f;
-        if (e < hi) { j = dst[e]; rx = r_ij[3 * e]; ry = r_ij[3 * e + 1]; rz = r_ij[3 * e + 2]; }
+        if (e < hi) { j = (unsigned)*dp; rx = rp[0]; ry = rp[1]; rz = rp[2]; }
         while (e < hi) {
             EdgeLoads ld;
-            const float* a_row = actv_s + (j * n_slices + slice) * kSliceCols + 4 * l4;
-            const float* v_row = x_v + (j * n + slice * kSliceChan + 4 * l4) * 3;
+            const float* a_row = a_base + j * a_stride;
+            const float* v_row = v_base + j * v_stride;
 #pragma unroll
-            for (int q = 0; q < 4; q++) ld.a[q] = ld4(a_row + ((q + sub) & 3) * kSliceChan);
+            for (int k = 0; k < 4; k++) ld.a[k] = ld4(a_row + k * kSliceChan);
 #pragma unroll
             for (int k = 0; k < 3; k++) ld.v[k] = ld4(v_row + 4 * k);
-            const long e_next = e + kPerIter;
-            long j_next = 0;
+            e += kPerIter; dp += kPerIter; rp += 3 * kPerIter;
+            unsigned j_next = 0;
             float nx = 0.f, ny = 0.f, nz = 0.f;
-            if (e_next < hi) { j_next = dst[e_next]; nx = r_ij[3 * e_next]; ny = r_ij[3 * e_next + 1]; nz = r_ij[3 * e_next + 2]; }
+            if (e < hi) { j_next = (unsigned)*dp; nx = rp[0]; ny = rp[1]; nz = rp[2]; }
             const float r2 = rx * rx + ry * ry + rz * rz;
             const float u = sqrtf(r2) * inv_h;
             const float fl = floorf(u);
@@ -271,30 +276,20 @@ __global__ void __launch_bounds__(1024) painn_table_message_lds_kernel(
             const float w0 = -(1.0f / 6.0f) * t * tm * tq, w1 = 0.5f * tp * tm * tq, w2 = -0.5f * tp * t * tq,
                         w3 = (1.0f / 6.0f) * tp * t * tm;
             const int i = (int)fl;
-            const float* p0 = tab + ((i - 1) & mask) * kSliceRowF + 4 * l4;
-            const float* p1 = tab + (i & mask) * kSliceRowF + 4 * l4;
-            const float* p2 = tab + ((i + 1) & mask) * kSliceRowF + 4 * l4;
-            const float* p3 = tab + ((i + 2) & mask) * kSliceRowF + 4 * l4;
-            float4 pr[4];                                     // pr[q]: product of block (q + sub) % 4
+            const float* p0 = tab_l + ((i - 1) & mask) * kSliceRowF;
+            const float* p1 = tab_l + (i & mask) * kSliceRowF;
+            const float* p2 = tab_l + ((i + 1) & mask) * kSliceRowF;
+            const float* p3 = tab_l + ((i + 2) & mask) * kSliceRowF;
 #pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const int off = ((q + sub) & 3) * kSliceChan;
-                const float4 t0 = ld4(p0 + off), t1 = ld4(p1 + off), t2 = ld4(p2 + off), t3 = ld4(p3 + off);
-                const float4 fq = make_float4(w0 * t0.x + w1 * t1.x + w2 * t2.x + w3 * t3.x, w0 * t0.y + w1 * t1.y + w2 * t2.y + w3 * t3.y,
-                                              w0 * t0.z + w1 * t1.z + w2 * t2.z + w3 * t3.z, w0 * t0.w + w1 * t1.w + w2 * t2.w + w3 * t3.w);
-                pr[q] = mul4(fq, ld.a[q]);
+            for (int k = 0; k < 4; k++) {
+                const float4 t0 = ld4(p0 + k * kSliceChan), t1 = ld4(p1 + k * kSliceChan), t2 = ld4(p2 + k * kSliceChan),
+                             t3 = ld4(p3 + k * kSliceChan);
+                ld.f[k] = make_float4(w0 * t0.x + w1 * t1.x + w2 * t2.x + w3 * t3.x, w0 * t0.y + w1 * t1.y + w2 * t2.y + w3 * t3.y,
+                                      w0 * t0.z + w1 * t1.z + w2 * t2.z + w3 * t3.z, w0 * t0.w + w1 * t1.w + w2 * t2.w + w3 * t3.w);
             }
-            // block k sits in pr[(k - sub) % 4]: rotate by sub's low bit, then by its second bit
-            const bool s1 = sub & 1, s2 = sub & 2;
-            auto sel = [](bool c, float4 x, float4 y) { return make_float4(c ? x.x : y.x, c ? x.y : y.y, c ? x.z : y.z, c ? x.w : y.w); };
-            float4 tr[4], bk[4];
-#pragma unroll
-            for (int k = 0; k < 4; k++) tr[k] = sel(s1, pr[(k + 3) & 3], pr[k]);
-#pragma unroll
-            for (int k = 0; k < 4; k++) bk[k] = sel(s2, tr[(k + 2) & 3], tr[k]);
-            const float inv = 1.0f / sqrtf(epsilon + r2);
-            ld.accumulate_products(acc, bk[0], bk[1], bk[2], bk[3], rx * inv, ry * inv, rz * inv);
-            e = e_next; j = j_next; rx = nx; ry = ny; rz = nz;
+            const float inv = __builtin_amdgcn_rsqf(epsilon + r2);
+            ld.accumulate(acc, rx * inv, ry * inv, rz * inv);
+            j = j_next; rx = nx; ry = ny; rz = nz;
         }
         for (int d = 4; d < kWave; d <<= 1) {
 #pragma unroll
@@ -571,6 +566,7 @@ int mg_painn_table_message_sliced(const int* row_ptr, const int* dst, int n_node
     MG_REQUIRE(n % kSliceChan == 0 && aligned16(table) && aligned16(actv_sliced) && aligned16(x_v) && aligned16(out_a) &&
                    aligned16(out_v) && (!res_a || aligned16(res_a)) && (!res_v || aligned16(res_v)),
                "mg_painn_table_message_sliced: n must be a multiple of %d and the operands 16-byte aligned", kSliceChan);
+    MG_REQUIRE((long)n_nodes * 4 * n < (1L << 32), "mg_painn_table_message_sliced: n_nodes * 4 n must be below 2^32");
     const int n_slices = n / kSliceChan;
     const size_t lds_bytes = (size_t)table_rows * kSliceRowF * sizeof(float);
     // more than 64 KB of dynamic LDS has to be asked for (per device, so on every call)

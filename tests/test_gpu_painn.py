@@ -354,6 +354,21 @@ def test_table_message_kernel_interpolates_a_known_periodic_filter(ops, n, rows)
     with pytest.raises(RuntimeError, match="power of two"):
         ops.painn_table_message(row_ptr, dev(dst.int()), dev(r), dev(table[:rows - 1].contiguous()), 2 * r0, dev(actv),
                                 dev(x_v), 0.1)
+    if n % ops.PAINN_SLICE == 0:
+        # the variant that keeps the table in LDS, fed with actv in slice-major column order
+        perm = ops.painn_slice_permutation(n, "cuda")
+        assert torch.equal(torch.sort(perm).values, torch.arange(4 * n, device="cuda"))
+        sl_a, sl_v = ops.painn_table_message_sliced(row_ptr, dev(dst.int()), dev(r), dev(table), 2 * r0,
+                                                    dev(actv)[:, perm].contiguous(), dev(x_v), 0.1, dev(x_a), dev(x_v))
+        _close(sl_a, ref_a.cpu(), atol_scale=3e-6)
+        _close(sl_v, ref_v.cpu(), atol_scale=3e-6)
+        no_a, no_v = ops.painn_table_message_sliced(row_ptr, dev(dst.int()), dev(r), dev(table), 2 * r0,
+                                                    dev(actv)[:, perm].contiguous(), dev(x_v), 0.1)
+        _close(no_a, (ref_a - dev(x_a)).cpu(), atol_scale=3e-6)
+        _close(no_v, (ref_v - dev(x_v)).cpu(), atol_scale=3e-6)
+        with pytest.raises(RuntimeError, match="power of two in 4..512"):
+            ops.painn_table_message_sliced(row_ptr, dev(dst.int()), dev(r), dev(table.repeat(4, 1)), 2 * r0,
+                                           dev(actv), dev(x_v), 0.1)
 
 
 @pytest.mark.parametrize("n_rbf", [16, None])
@@ -377,12 +392,15 @@ def test_message_with_filter_table_equals_filter_mlp_per_edge(pkg, n_rbf):
     with torch.no_grad():
         rows = msg.table_rows()
         assert rows in msg.TABLE_ROWS and E >= 4 * rows
-        a1, v1 = msg(graph, x_a, x_v, r.cuda(), residual=True)
+        a1, v1 = msg(graph, x_a, x_v, r.cuda(), residual=True)       # grid in LDS when 512 rows are enough
+        msg.use_sliced = False
+        a2, v2 = msg(graph, x_a, x_v, r.cuda(), residual=True)       # grid read through the caches
         msg.use_table = False
         a0, v0 = msg(graph, x_a, x_v, r.cuda(), residual=True)
     assert float(r.norm(dim=-1).max()) > 2 * r0
-    _close(a1, a0.cpu(), atol_scale=3e-6)
-    _close(v1, v0.cpu(), atol_scale=3e-6)
+    for a, v in ((a1, v1), (a2, v2)):
+        _close(a, a0.cpu(), atol_scale=3e-6)
+        _close(v, v0.cpu(), atol_scale=3e-6)
 
 
 def test_filter_table_is_rejected_when_the_filter_is_too_rough(pkg):
