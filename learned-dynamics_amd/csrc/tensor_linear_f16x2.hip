@@ -368,9 +368,9 @@ struct Shape {
 inline Shape choose_shape(long R, int O) {
     Shape s;
     s.ni = O <= 32 ? 1 : (O <= 64 ? 2 : (O <= 128 ? 4 : 8));
-    // few rows: narrower column tiles until the 256 CUs have a workgroup each (at most 64 column tiles: the
+    // few rows: narrower column tiles until the 256 CUs have two workgroups each (at most 64 column tiles: the
     // row maxima are emitted per column tile)
-    while (s.ni > 1 && ceil_div(R, 128) * ceil_div(O, 32 * s.ni) < 256 && ceil_div(O, 16 * s.ni) <= 64) s.ni >>= 1;
+    while (s.ni > 1 && ceil_div(R, 128) * ceil_div(O, 32 * s.ni) < 512 && ceil_div(O, 16 * s.ni) <= 64) s.ni >>= 1;
     const long tiles = ceil_div(R, 256) * ceil_div(O, 32 * s.ni);
     s.waves = tiles >= 512 ? 8 : 4;
     return s;
