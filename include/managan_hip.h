@@ -352,6 +352,13 @@ int mg_mlp_chain_bf16(const void* x, long rows, int dim_in, const void* packed_Y
                       const float* b1, const void* packed_W2, const float* b2, int act, const int* row_ptr,
                       const int* seg, long n_out, void* workspace, float* sum_psi, float* sum_h2, mg_stream_t stream);
 
+/* The three edge sums of DisplacementTensors.forward (archs/diffuser_atoms15.py:218-224) over CSR rows: with
+ * u = s r / sqrt(1 + |s r|^2), s = scale (7 / r0 in the reference, tens_sigmoid of managan/tensor_products.py:167-182),
+ *   out_a[i,c] = sum_e phi[e,c];  out_v[i,c,x] = sum_e phi[e,c] u_x;  out_d[i,c,x,y] = sum_e phi[e,c] u_x u_y
+ * phi (E, chan) is the radial MLP's output per edge; the per-edge tensors phi (x) u, phi (x) u (x) u are never stored. */
+int mg_displacement_sums(const int* row_ptr, long n_nodes, long n_edges, const float* r_ij, const float* phi, int chan,
+                         float scale, float* out_a, float* out_v, float* out_d, mg_stream_t stream);
+
 /* repel5_sim (extensions/polymer_sims_cuda/polymer_sims_kern.cu:145-164, bound as polymer_sim(SimId.REPEL5, ...) in
  * polymer_sims.cpp:17-47): Langevin dynamics of batch_size chains of n beads, x and v (batch_size, n, 3) float32
  * updated in place, drag (n).  Per call: half velocity update, max(nsteps, 1) position updates with full velocity

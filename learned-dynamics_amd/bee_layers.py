@@ -231,6 +231,32 @@ class MLP(nn.Module):
         return out.mul_(scale) if scale != 1.0 else out
 
 
+class DisplacementTensors(nn.Module):
+    """archs/diffuser_atoms15.py:206-225: ACE-like embedding of the neighbourhood.  The radial MLP runs per edge
+    through the matrix path; its output times the squashed direction and its outer square is summed per node
+    inside one kernel (ops.displacement_sums), so the (edges, dim_a, 3) and (edges, dim_a, 3, 3) tensors the
+    reference builds for its scatter sums are never stored."""
+
+    def __init__(self, r0: float, dim_a: int, dim_v: int, dim_d: int):
+        super().__init__()
+        self.r0 = r0
+        self.mlp_radial = nn.Sequential(nn.Linear(8, dim_a), MLP(dim_a))
+        self.readout_v = TensLinear(1, dim_a, dim_v)
+        self.readout_d = TensLinear(2, dim_a, dim_d)
+
+    def forward(self, graph: Graph, r_ij):
+        """r_ij (edges, 3) -> A_a (batch, nodes, dim_a), A_v (batch, nodes, dim_v, 3), A_d (batch, nodes, dim_d, 3, 3)."""
+        r_ij = r_ij.contiguous()
+        enc, _ = ops.bee_edge_geometry(r_ij, self.r0)                            # radial_encode_8: (edges, 8)
+        first = self.mlp_radial[0]
+        x = ops.tensor_linear_fwd(0, first.weight, enc, bias=first.bias)
+        rad = self.mlp_radial[1](x)                                              # (edges, dim_a)
+        A_a, A_v, A_d = ops.displacement_sums(graph.row_ptr, r_ij, rad, 7.0 / self.r0)
+        B, N = graph.batch, graph.nodes
+        return (A_a.reshape(B, N, -1), self.readout_v(A_v.reshape(B, N, -1, 3)),
+                self.readout_d(A_d.reshape(B, N, -1, 3, 3)))
+
+
 class Messages(nn.Module):
     """archs/diffuser_atoms15.py:227-253"""
 

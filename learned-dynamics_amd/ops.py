@@ -1501,6 +1501,26 @@ def radial_encode(kind, r_ij, n, rmax):
     return out
 
 
+def displacement_sums(row_ptr, r_ij, phi, scale):
+    """(A_a (N, C), A_v (N, C, 3), A_d (N, C, 3, 3)): sums over the edges of each CSR row of phi, phi (x) u and
+    phi (x) u (x) u with u = tens_sigmoid(1, scale * r_ij) (archs/diffuser_atoms15.py:218-224)."""
+    _check_input(row_ptr, "row_ptr", torch.int32)
+    _check_input(r_ij, "r_ij")
+    _check_input(phi, "phi")
+    E = int(r_ij.size(0))
+    if tuple(r_ij.shape) != (E, 3) or phi.dim() != 2 or phi.size(0) != E:
+        raise RuntimeError("r_ij (edges, 3) and phi (edges, chan) expected")
+    n_nodes, C = int(row_ptr.numel()) - 1, int(phi.size(1))
+    dev = phi.device
+    with torch.cuda.device(dev):
+        out_a = torch.empty(n_nodes, C, dtype=torch.float32, device=dev)
+        out_v = torch.empty(n_nodes, C, 3, dtype=torch.float32, device=dev)
+        out_d = torch.empty(n_nodes, C, 3, 3, dtype=torch.float32, device=dev)
+        L.check(_lib.mg_displacement_sums(_p(row_ptr), n_nodes, E, _p(r_ij), _p(phi), C, float(scale), _p(out_a),
+                                          _p(out_v), _p(out_d), _stream()))
+    return out_a, out_v, out_d
+
+
 # ------------------------------------------------------------------ data generator
 def repel5_sim(x, v, drag, T, dt, nsteps, seed, first_kick=0):
     """Langevin dynamics of bead chains in place (polymer_sim(SimId.REPEL5, ...) of

@@ -16,6 +16,7 @@ Follows (relative to the reference checkout):
   archs/diffuser_atoms15.py:29-57          the 13 Y_* linears and their sums
   archs/diffuser_atoms15.py:59-95          SelfTensProds
   archs/diffuser_atoms15.py:98-110         MLP with direct path and LeakyReLU(0.1)
+  archs/diffuser_atoms15.py:206-225        DisplacementTensors
   archs/diffuser_atoms15.py:227-253        Messages (Bee)
 """
 import math
@@ -181,6 +182,19 @@ def bee_messages(src, dst, batch, nodes, r_ij, x_a, x_v, x_d, w, r0):
     return (0.1 * edges_reduce_src(src, psi_a, batch, nodes),
             0.1 * edges_reduce_src(src, psi_v, batch, nodes),
             0.1 * edges_reduce_src(src, psi_d, batch, nodes))
+
+
+def displacement_tensors(src, batch, nodes, r_ij, w, r0):
+    """DisplacementTensors.forward (archs/diffuser_atoms15.py:216-225).  w: lin_W (dim_a, 8), lin_b (dim_a),
+    mlp (dict for mlp_leaky, dim_a -> dim_a), readout_v (dim_v, dim_a), readout_d (dim_d, dim_a)."""
+    rad = mlp_leaky(F.linear(radial_encode_8(r_ij, r0), w["lin_W"], w["lin_b"]), w["mlp"])     # (E, dim_a)
+    u = tens_sigmoid(1, r_ij * (7.0 / r0))
+    phi_v = rad[..., None] * u[..., None, :]
+    phi_d = rad[..., None, None] * u[..., None, None, :] * u[..., None, :, None]
+    A_a = edges_reduce_src(src, rad, batch, nodes)
+    A_v = edges_reduce_src(src, phi_v, batch, nodes)
+    A_d = edges_reduce_src(src, phi_d, batch, nodes)
+    return A_a, P.tensor_linear(1, w["readout_v"], A_v), P.tensor_linear(2, w["readout_d"], A_d)
 
 
 def self_tens_prods(x_a, x_v, x_d, w, groups=8):

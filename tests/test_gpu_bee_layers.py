@@ -306,3 +306,59 @@ def test_self_tens_prods_module_fused_path(pkg):
     _close(y_a, x_a + ra, atol_scale=5e-6)
     _close(y_v, x_v + rv, atol_scale=5e-6)
     _close(y_d, x_d + rd, atol_scale=5e-6)
+
+
+@pytest.mark.parametrize("chan,kind", [(64, "mixed"), (100, "short"), (7, "mixed"), (256, "long")])
+def test_displacement_sums_kernel(ops, chan, kind):
+    """mg_displacement_sums against float64 index_add of the per-edge tensors the reference materialises
+    (archs/diffuser_atoms15.py:218-224), with empty rows, channel counts that are not a multiple of 64 and
+    rows much longer than a wave."""
+    g = torch.Generator().manual_seed(chan)
+    N = 200
+    deg = {"mixed": torch.randint(0, 40, (N,), generator=g), "short": torch.randint(0, 3, (N,), generator=g),
+           "long": torch.randint(100, 300, (N,), generator=g)}[kind]
+    src = torch.repeat_interleave(torch.arange(N), deg)
+    E = int(src.numel())
+    r = torch.randn(E, 3, generator=g) * 3
+    phi = torch.randn(E, chan, generator=g)
+    row_ptr = ops.segment_row_ptr(src.int().cuda(), N)
+    s = 7.0 / 6.0
+    A_a, A_v, A_d = ops.displacement_sums(row_ptr, r.cuda(), phi.cuda(), s)
+    u = OL.tens_sigmoid(1, r.double() * s)
+    p = phi.double()
+    ref_a = torch.zeros(N, chan, dtype=torch.float64).index_add_(0, src, p)
+    ref_v = torch.zeros(N, chan, 3, dtype=torch.float64).index_add_(0, src, p[..., None] * u[:, None, :])
+    ref_d = torch.zeros(N, chan, 3, 3, dtype=torch.float64).index_add_(
+        0, src, p[..., None, None] * u[:, None, :, None] * u[:, None, None, :])
+    _close(A_a, ref_a.float(), atol_scale=2e-6)
+    _close(A_v, ref_v.float(), atol_scale=2e-6)
+    _close(A_d, ref_d.float(), atol_scale=2e-6)
+    assert not bool(A_a[(deg == 0).cuda()].any()) and not bool(A_d[(deg == 0).cuda()].any())
+
+
+@pytest.mark.parametrize("dims", [(64, 32, 16), (128, 64, 16), (20, 12, 5)])
+def test_displacement_tensors_module(pkg, dims):
+    """DisplacementTensors.forward against the oracle's restatement of archs/diffuser_atoms15.py:206-225."""
+    bee = importlib.import_module("learned-dynamics_amd.bee_layers")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    dim_a, dim_v, dim_d = dims
+    torch.manual_seed(0x947 + 14)
+    box, r0 = (30., 30., 30.), 6.0
+    pos = torch.rand(2, 500, 3) * 30
+    mod = bee.DisplacementTensors(r0, dim_a, dim_v, dim_d).cuda()
+    assert sorted(mod.state_dict()) == sorted(
+        ["mlp_radial.0.weight", "mlp_radial.0.bias", "mlp_radial.1.lin_direct.weight"]
+        + [f"mlp_radial.1.layers.{i}.{p}" for i in (0, 2, 4) for p in ("weight", "bias")] + ["readout_v.W", "readout_d.W"])
+    with torch.no_grad():
+        graph, r_ij = gl.graph_setup(r0, box, pos.cuda(), neighbours_max=256, celllist_max=64)
+        A_a, A_v, A_d = mod(graph, r_ij)
+    assert A_a.shape == (2, 500, dim_a) and A_v.shape == (2, 500, dim_v, 3) and A_d.shape == (2, 500, dim_d, 3, 3)
+    src, dst = graph.src.cpu(), graph.dst.cpu()
+    r_ref = torch.from_numpy(ON.edge_vectors(pos.numpy(), src.numpy(), dst.numpy(), box))
+    dd = lambda t: t.detach().cpu().double()
+    w = {"lin_W": dd(mod.mlp_radial[0].weight), "lin_b": dd(mod.mlp_radial[0].bias),
+         "mlp": _mlp_leaky_weights(mod.mlp_radial[1]), "readout_v": dd(mod.readout_v.W), "readout_d": dd(mod.readout_d.W)}
+    ra, rv, rd = OL.displacement_tensors(src, 2, 500, r_ref.double(), w, r0)
+    _close(A_a, ra, atol_scale=5e-6)
+    _close(A_v, rv, atol_scale=5e-6)
+    _close(A_d, rd, atol_scale=5e-6)

@@ -205,3 +205,48 @@ def test_bee_messages_reduces_to_scalar_message_when_vectors_vanish():
     u = ((x_a[0] @ w["L0"].T)[dst] * phi) @ Y["000"].T
     expect = torch.zeros(N, dim_a, dtype=torch.float64).index_add_(0, src, u + OL.mlp_leaky(u, w["mlp_a"]))
     assert torch.allclose(B_a[0], 0.1 * expect)
+
+
+def test_displacement_tensors_closed_form_and_equivariance():
+    """One edge per node along a known direction: A_a = phi, A_v = phi u, A_d = phi u u^T with
+    u = s r / sqrt(1 + |s r|^2), s = 7 / r0, written out by hand; identity read-outs.  Then a ring graph under the
+    reference's rotation: rank-k outputs rotate as rank-k tensors, and the sums are explicit loops over edges."""
+    g = torch.Generator().manual_seed(8)
+    dim_a, dim_v, dim_d, N, r0 = 5, 5, 5, 6, 6.0
+    rn = lambda *s: torch.randn(*s, generator=g, dtype=torch.float64) * 0.5
+    w = {"lin_W": rn(dim_a, 8), "lin_b": rn(dim_a), "mlp": _rand_mlp(dim_a, dim_a, g, leaky=True),
+         "readout_v": torch.eye(dim_a, dtype=torch.float64), "readout_d": torch.eye(dim_a, dtype=torch.float64)}
+    src = torch.arange(N)
+    r_ij = torch.zeros(N, 3, dtype=torch.float64)
+    r_ij[:, 0] = torch.linspace(0.5, 5.5, N)                 # along x
+    A_a, A_v, A_d = OL.displacement_tensors(src, 1, N, r_ij, w, r0)
+    z = r_ij[:, 0] / r0
+    enc = OL.radial_encode_8(r_ij, r0)
+    assert torch.allclose(enc[:, 0], 1 - z) and torch.allclose(enc[:, 1], (3 * z - 1) * (1 - z))   # P0 = 1, P1 = 3z - 1
+    phi = OL.mlp_leaky(enc @ w["lin_W"].T + w["lin_b"], w["mlp"])
+    s = 7.0 / r0
+    ux = s * r_ij[:, 0] / torch.sqrt(1 + (s * r_ij[:, 0]) ** 2)
+    assert torch.allclose(A_a[0], phi)
+    assert torch.allclose(A_v[0, :, :, 0], phi * ux[:, None]) and not bool(A_v[0, :, :, 1:].any())
+    assert torch.allclose(A_d[0, :, :, 0, 0], phi * (ux ** 2)[:, None])
+    assert not bool(A_d[0, :, :, 1:, :].any()) and not bool(A_d[0, :, :, :, 1:].any())
+    # ring graph: explicit loops, read-outs mixing channels, rotation
+    w["readout_v"], w["readout_d"] = rn(3, dim_a), rn(2, dim_a)
+    src, dst = _ring_graph(N)
+    pos = rn(N, 3) * 4
+    r_ij = pos[dst] - pos[src]
+    out = OL.displacement_tensors(src, 1, N, r_ij, w, r0)
+    phi = OL.mlp_leaky(OL.radial_encode_8(r_ij, r0) @ w["lin_W"].T + w["lin_b"], w["mlp"])
+    u = OL.tens_sigmoid(1, r_ij * s)
+    A_v = torch.zeros(N, dim_a, 3, dtype=torch.float64)
+    A_d = torch.zeros(N, dim_a, 3, 3, dtype=torch.float64)
+    for e in range(2 * N):
+        for c in range(dim_a):
+            A_v[src[e], c] += phi[e, c] * u[e]
+            A_d[src[e], c] += phi[e, c] * torch.outer(u[e], u[e])
+    assert torch.allclose(out[1][0], torch.einsum("oc,ncx->nox", w["readout_v"], A_v))
+    assert torch.allclose(out[2][0], torch.einsum("oc,ncxy->noxy", w["readout_d"], A_d))
+    out_r = OL.displacement_tensors(src, 1, N, r_ij @ ROT, w, r0)
+    for k in range(3):
+        assert torch.allclose(out_r[k], _rot(out[k], k), atol=1e-10)
+
