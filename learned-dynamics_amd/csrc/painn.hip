@@ -117,9 +117,11 @@ struct EdgeLoads {
         for (int k = 0; k < 4; k++) {
             const float x = vv[3 * k], y = vv[3 * k + 1], z = vv[3 * k + 2];
             const float cx = y * uz - z * uy, cy = z * ux - x * uz, cz = x * uy - y * ux;   // v x u
-            acc.v[3 * k + 0] += x * q0[k] + cx * q1[k] + ux * q2[k];
-            acc.v[3 * k + 1] += y * q0[k] + cy * q1[k] + uy * q2[k];
-            acc.v[3 * k + 2] += z * q0[k] + cz * q1[k] + uz * q2[k];
+            // three fused multiply-adds straight into the running sum (a separate add per component would be
+            // a twentieth of the loop's vector instructions)
+            acc.v[3 * k + 0] = fmaf(ux, q2[k], fmaf(cx, q1[k], fmaf(x, q0[k], acc.v[3 * k + 0])));
+            acc.v[3 * k + 1] = fmaf(uy, q2[k], fmaf(cy, q1[k], fmaf(y, q0[k], acc.v[3 * k + 1])));
+            acc.v[3 * k + 2] = fmaf(uz, q2[k], fmaf(cz, q1[k], fmaf(z, q0[k], acc.v[3 * k + 2])));
             acc.a[k] += q3[k];
         }
     }

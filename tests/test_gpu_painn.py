@@ -403,6 +403,20 @@ def test_message_with_filter_table_equals_filter_mlp_per_edge(pkg, n_rbf):
         _close(v, v0.cpu(), atol_scale=3e-6)
 
 
+def test_table_message_kernels_without_edges_return_the_residual(ops):
+    n, N, rows = 32, 40, 64
+    g = torch.Generator().manual_seed(1)
+    row_ptr = torch.zeros(N + 1, dtype=torch.int32, device="cuda")
+    e_i, e_f = torch.zeros(0, dtype=torch.int32, device="cuda"), torch.zeros(0, 3, device="cuda")
+    table, actv = torch.randn(rows, 4 * n, generator=g).cuda(), torch.randn(N, 4 * n, generator=g).cuda()
+    x_a, x_v = torch.randn(N, n, generator=g).cuda(), torch.randn(N, n, 3, generator=g).cuda()
+    for fn in (ops.painn_table_message, ops.painn_table_message_sliced):
+        a, v = fn(row_ptr, e_i, e_f, table, 8.0, actv, x_v, 0.1, x_a, x_v)
+        assert torch.equal(a, x_a) and torch.equal(v, x_v)
+        a, v = fn(row_ptr, e_i, e_f, table, 8.0, actv, x_v, 0.1)
+        assert not bool(a.any()) and not bool(v.any())
+
+
 def test_filter_table_is_rejected_when_the_filter_is_too_rough(pkg):
     """With first-layer weights scaled up the filter varies faster than any of the grids resolves: the midpoint
     check refuses them and the module evaluates the MLP per edge; a change of the weights is noticed."""
