@@ -113,7 +113,13 @@ class Update(nn.Module):
         rows = B * N
         flat_a = x_a.reshape(rows, n).contiguous()
         flat_v = x_v.reshape(rows, n, 3).contiguous()
-        W = torch.cat([self.lin_l.W, self.lin_r.W, self.lin_v.W], dim=0)        # (3n, n): one GEMM for l, r, v
+        params = (self.lin_l.W, self.lin_r.W, self.lin_v.W)
+        cache = self.__dict__.setdefault("_lrv_cache", {})
+        stamp = tuple((id(p), p._version, p.data_ptr()) for p in params)
+        if cache.get("stamp") != stamp:                                         # (3n, n): one GEMM for l, r, v; kept
+            with torch.no_grad():                                               # while the weights are unchanged, so
+                cache.update(stamp=stamp, W=torch.cat(params, dim=0))           # its packed planes stay valid too
+        W = cache["W"]
         lrv = ops.tensor_linear_fwd(1, W, flat_v)                               # (rows, 3n, 3)
         ip, cat = ops.painn_update_pre(lrv, flat_a)                             # l.r and [x_a | |r|]
         y = self.mlp(cat)                                                       # (rows, 3n)
