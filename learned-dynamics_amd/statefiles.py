@@ -158,3 +158,109 @@ def load_module_states(module: torch.nn.Module, state_dict, prefix: str = "", st
     if not sub:
         raise KeyError(f"no entries below {prefix!r} in the state dict")
     return module.load_state_dict(sub, strict=strict)
+
+
+# ------------------------------------------------------------------ dataset directories
+def save_predictor_params_to_file(file, box, shape, name):
+    """`predictor_params.pickle` of a dataset directory (managan/statefiles.py:44-50): box, item shape and the
+    predictor's name."""
+    pickle.dump({"box": box, "shape": tuple(shape), "name": name}, file)
+
+
+def read_predictor_params_from_file(file):
+    """managan/statefiles.py:52-54, decoded without instantiating anything."""
+    params = _inert_loads(file.read())
+    if not isinstance(params, dict) or "box" not in params or "shape" not in params:
+        raise DatasetError('predictor parameters must be a dict with "box" and "shape"')
+    return params
+
+
+class DatasetState:
+    """One chunk file as a trajectory with a cursor (managan/statefiles.py:57-74): `x` is frame `t` of the first
+    `batch` saved trajectories."""
+
+    def __init__(self, fnm, batch=1, device=None):
+        with open(fnm, "rb") as f:
+            self.traj = read_state_from_file(f, device)
+        if len(self.traj.size) < 2:
+            raise DatasetError("a dataset chunk holds (time, batch, ...) trajectories")
+        self.L, saved_batch, *rest = self.traj.size
+        if batch > saved_batch:
+            raise DatasetError(f"requested batch {batch} cannot exceed saved batch {saved_batch}")
+        self.size = (batch,) + tuple(rest)
+        self.shape = self.traj.shape
+        self.batch = batch
+        self.t = 0
+
+    @property
+    def x(self):
+        return self.traj.x[self.t, :self.batch]
+
+    @property
+    def metadata(self):
+        return self.traj.metadata
+
+    def to_model_predictor_state(self):
+        return TrajectoryState(self.shape, self.x.clone(), self.metadata)
+
+
+class DatasetPredictor:
+    """Walks the `.bin` chunks of a dataset directory in shuffled order (managan/statefiles.py:76-113).  rng: a
+    `random.Random` for the shuffle (the reference uses the global one)."""
+
+    def __init__(self, dataset_dir, stride=1, repeat=False, rng=None, device=None):
+        import os
+        import random
+        self.dataset_dir, self.stride, self.repeat, self.device = dataset_dir, stride, repeat, device
+        self._rng = rng if rng is not None else random
+        with open(os.path.join(dataset_dir, "predictor_params.pickle"), "rb") as f:
+            params = read_predictor_params_from_file(f)
+        self._box, self._shape = params["box"], params["shape"]
+        self.file_list = sorted(fnm for fnm in os.listdir(dataset_dir) if fnm.endswith(".bin"))
+        self._rng.shuffle(self.file_list)
+        self.file_index = 0
+
+    def get_box(self):
+        return self._box
+
+    def shape(self):
+        return self._shape
+
+    def sample_q(self, batch):
+        import os
+        if self.file_index >= len(self.file_list):
+            if not self.repeat:
+                raise DatasetError("out of files in dataset!")
+            self._rng.shuffle(self.file_list)
+            self.file_index = 0
+        ans = DatasetState(os.path.join(self.dataset_dir, self.file_list[self.file_index]), batch, self.device)
+        self.file_index += 1
+        return ans
+
+    def predict(self, L, state, ret=True):
+        """Advance the cursor by L strides; returns frames t + stride, ..., t + L stride of the first `batch`
+        trajectories, shape (L, batch, ...)."""
+        if not isinstance(state, DatasetState):
+            raise DatasetError("DatasetPredictor can only handle DatasetState's")
+        if not L * self.stride < state.L - state.t:
+            raise DatasetError(f"DatasetPredictor tried to predict {self.stride}*{L} steps, but only "
+                               f"{state.L - state.t - 1} data remains")
+        t_old = state.t
+        state.t += L * self.stride
+        if ret:
+            return state.traj.x[t_old + self.stride:state.t + 1:self.stride, :state.batch]
+
+
+def get_dataset_predictor(spec):
+    return DatasetPredictor(spec)
+
+
+def get_strided_dataset_predictor(spec):
+    """"<stride>?<directory>" (managan/statefiles.py:118-121)."""
+    stride, dataset_dir = spec.split("?")
+    return DatasetPredictor(dataset_dir, stride=int(stride))
+
+
+def get_repeated_dataset_predictor(spec):
+    stride, dataset_dir = spec.split("?")
+    return DatasetPredictor(dataset_dir, stride=int(stride), repeat=True)

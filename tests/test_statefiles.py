@@ -124,3 +124,46 @@ def test_checkpoint_with_pickled_objects_is_refused(tmp_path):
     torch.save([1, 2, 3], path)
     with pytest.raises(sf.DatasetError):
         sf.load_checkpoint(path)
+
+
+def test_dataset_directory_walk(tmp_path):
+    """predictor_params.pickle + .bin chunks as the reference lays a dataset out (managan/statefiles.py:76-113):
+    every chunk is visited once per epoch, `predict` returns strided frames and moves the cursor, and running out
+    of frames or files raises."""
+    import random
+    d = tmp_path / "ds"
+    d.mkdir()
+    with open(d / "predictor_params.pickle", "wb") as f:
+        sf.save_predictor_params_to_file(f, (30.0, 30.0, 30.0), (5, 3), "repel5_l5_t1")
+    chunks = {}
+    for i in range(3):
+        x = torch.arange(9 * 4 * 5 * 3, dtype=torch.float32).reshape(9, 4, 5, 3) + 1000 * i
+        chunks[float(x[0, 0, 0, 0])] = x
+        with open(d / f"{i}.bin", "wb") as f:
+            sf.save_state_to_file(f, sf.TrajectoryState((5, 3), x, {"poly_len": 5, "space_dim": 3}))
+    (d / "notes.txt").write_text("ignored")
+    pred = sf.DatasetPredictor(str(d), stride=2, rng=random.Random(0), device="cpu")
+    assert pred.get_box() == (30.0, 30.0, 30.0) and pred.shape() == (5, 3) and len(pred.file_list) == 3
+    seen = set()
+    for _ in range(3):
+        st = pred.sample_q(2)
+        x = chunks[float(st.x[0, 0, 0])]
+        seen.add(float(st.x[0, 0, 0]))
+        assert st.size == (2, ) and st.shape == (5, 3) and st.L == 9 and st.metadata == {"poly_len": 5, "space_dim": 3}
+        out = pred.predict(3, st)
+        assert torch.equal(out, x[2:7:2, :2]) and st.t == 6 and torch.equal(st.x, x[6, :2])
+        assert torch.equal(st.to_model_predictor_state().x, x[6, :2])
+        assert pred.predict(1, st, ret=False) is None and st.t == 8
+        with pytest.raises(sf.DatasetError, match="data remains"):
+            pred.predict(1, st)
+    assert len(seen) == 3
+    with pytest.raises(sf.DatasetError, match="out of files"):
+        pred.sample_q(2)
+    with pytest.raises(sf.DatasetError, match="cannot exceed saved batch"):
+        sf.DatasetState(str(d / "0.bin"), batch=5, device="cpu")
+    rep = sf.get_repeated_dataset_predictor(f"3?{d}")
+    rep.device = "cpu"
+    assert rep.stride == 3 and rep.repeat
+    for _ in range(7):
+        rep.sample_q(1)                                          # goes round again instead of raising
+    assert sf.get_strided_dataset_predictor(f"2?{d}").stride == 2
