@@ -371,7 +371,7 @@ inline Shape choose_shape(long R, int O) {
     // column tiles that divide O: a partly filled tile takes the slow, bounds-checked epilogue (O = 384 with
     // 256-column tiles ran 4 times slower than with 128-column tiles)
     if (O % 32 == 0)
-        while (s.ni > 1 && O % (32 * s.ni) != 0) s.ni >>= 1;
+        while (s.ni > 1 && O % (32 * s.ni) != 0 && ceil_div(O, 16 * s.ni) <= 64) s.ni >>= 1;
     // few rows: narrower column tiles until the 256 CUs have two workgroups each (at most 64 column tiles: the
     // row maxima are emitted per column tile)
     while (s.ni > 1 && ceil_div(R, 128) * ceil_div(O, 32 * s.ni) < 512 && ceil_div(O, 16 * s.ni) <= 64) s.ni >>= 1;

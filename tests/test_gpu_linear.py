@@ -119,7 +119,10 @@ def test_linear_modes_agree_with_float64(ops, mode, shape):
 
 
 @pytest.mark.parametrize("shape", [(70000, 512, 512, 1), (3001, 256, 192, 0), (1500, 96, 16, 2), (2048, 1280, 64, 0),
-                                   (1024, 64, 8, 0), (40000, 160, 130, 1), (140001, 64, 256, 2)])
+                                   (1024, 64, 8, 0), (40000, 160, 130, 1), (140001, 64, 256, 2),
+                                   # column tiles chosen to divide the width and narrowed for few rows
+                                   (49152, 128, 384, 1), (16384, 256, 384, 0), (512, 512, 512, 1), (300, 64, 96, 2),
+                                   (700, 64, 2080, 0), (2048, 64, 1056, 0)])
 def test_linear_f16x2_rows_of_very_different_size(ops, shape):
     """mg_tensor_linear_f16x2 through the C ABI.  Rows spanning twelve orders of magnitude: the per-row
     power-of-two scales keep the error relative to EACH row's own scale at fp32 rounding level (a single
