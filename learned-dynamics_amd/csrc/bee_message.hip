@@ -107,6 +107,20 @@ __device__ __forceinline__ long uniform(long v) {
     return ((long)hi << 32) | (unsigned)lo;
 }
 
+// Gathers of node rows go through buffer loads: the row's byte offset is uniform (scalar offset operand), the lane's
+// channel offset a constant vector register, so a gather needs no vector address arithmetic at all (with global
+// loads every one of the 13 gathers of an edge built its own 64-bit per-lane address: a tenth of the loop).
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t node_rows(const void* base, long bytes) {
+    const unsigned n = bytes > 0xffffffffL ? 0xffffffffu : (unsigned)bytes;
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(base), 0, (int)n, 0x00020000);
+}
+__device__ __forceinline__ float gather_row(__amdgpu_buffer_rsrc_t r, unsigned lane_bytes, unsigned row_bytes, float) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)lane_bytes, (int)row_bytes, 0));
+}
+__device__ __forceinline__ __bf16 gather_row(__amdgpu_buffer_rsrc_t r, unsigned lane_bytes, unsigned row_bytes, __bf16) {
+    return __builtin_bit_cast(__bf16, __builtin_amdgcn_raw_buffer_load_b16(r, (int)lane_bytes, (int)row_bytes, 0));
+}
+
 // T: storage type of the node features and of the outputs (float, or __bf16 with fp32 arithmetic)
 // PIPE: keep one edge of operands in flight ahead of the one being consumed (pays on long rows)
 template <typename T, bool PIPE>
@@ -120,6 +134,8 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
     const int lane = threadIdx.x & (kWave - 1);
     const int chunks = (chan + kWave - 1) / kWave;
     const long items = n_nodes * chunks;
+    const long a_bytes = n_nodes * chan * (long)sizeof(T);
+    const __amdgpu_buffer_rsrc_t rs_a = node_rows(La, a_bytes), rs_v = node_rows(Lv, 3 * a_bytes), rs_d = node_rows(Ld, 9 * a_bytes);
     // contiguous ranges of the processing order per XCD (workgroup ids go round-robin over 8 XCDs)
     const long per_xcd = (items + 7) / 8;
     const int xcd = blockIdx.x & 7;
@@ -156,15 +172,15 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
             float en[8], rh[3];
         };
         const unsigned lane_off = (unsigned)cc;   // rows are addressed as (uniform base) + 32-bit lane offset
+        const unsigned lane_bytes = lane_off * (unsigned)sizeof(T);
+        const unsigned row_bytes = (unsigned)chan * (unsigned)sizeof(T);
         auto fetch = [&](EdgeOps& o, long e, long j) {
-            const T* a = La + j * chan;
-            const T* v = Lv + j * 3 * chan;
-            const T* d = Ld + j * 9 * chan;
-            o.l0 = a[lane_off];
+            const unsigned jr = (unsigned)__builtin_amdgcn_readfirstlane((int)j) * row_bytes;   // byte offset of La[j]
+            o.l0 = gather_row(rs_a, lane_bytes, jr, T{});
 #pragma unroll
-            for (int t = 0; t < 3; t++) o.l1[t] = (v + t * chan)[lane_off];
+            for (int t = 0; t < 3; t++) o.l1[t] = gather_row(rs_v, lane_bytes, 3u * jr + (unsigned)t * row_bytes, T{});
 #pragma unroll
-            for (int k = 0; k < 9; k++) o.l2[k] = (d + k * chan)[lane_off];
+            for (int k = 0; k < 9; k++) o.l2[k] = gather_row(rs_d, lane_bytes, 9u * jr + (unsigned)k * row_bytes, T{});
 #pragma unroll
             for (int m = 0; m < 8; m++) o.en[m] = enc[8 * e + m];
 #pragma unroll
@@ -287,6 +303,8 @@ static int launch_bee_message(const char* what, const int* row_ptr, const int* d
     if (n_nodes == 0 || chan == 0) return MG_OK;
     MG_REQUIRE(row_ptr && La && Lv && Ld && enc_W && enc_b && S1 && S2, "%s: null pointer", what);
     MG_REQUIRE(n_edges == 0 || (dst && rhat && enc && P0), "%s: null edge operand", what);
+    MG_REQUIRE((long)n_nodes * 9 * chan * (long)sizeof(T) < (1L << 32),
+               "%s: the rank-2 node rows must stay below 4 GiB (32-bit row offsets)", what);
     const long items = (long)n_nodes * ceil_div(chan, kWave);
     long blocks = ceil_div(items, 4);
     if (blocks > 256L * 16) blocks = 256L * 16;
