@@ -51,7 +51,8 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-comparisons", action="store_true",
-                    help="painn_layer: skip the stand-alone timings of the kernels the layer no longer runs")
+                    help="painn_layer: skip the stand-alone timings of the kernels the layer no longer runs; "
+                         "stress: skip the timing of the fp32-storage stack")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also run a plain 1 GiB device copy (yardstick for rocprofv3 FETCH_SIZE/WRITE_SIZE)")
     return ap.parse_args()
@@ -594,7 +595,7 @@ def bench_stress(torch, args):
         out = step_bf16()[0]
         rel = float((out - ref).abs().max() / ref.abs().max())
         sec16 = timed_steps(torch, step_bf16, args.steps, args.warmup)
-        sec32 = timed_steps(torch, step_f32, args.steps, args.warmup)
+        sec32 = None if getattr(args, "no_comparisons", False) else timed_steps(torch, step_f32, args.steps, args.warmup)
         graph, r_ij = gl.graph_setup(r0, box, pos, neighbours_max=256, celllist_max=64)
         edge_roof = edge_kernel_roofline(torch, msgs[0], graph, r_ij, N, bf16=True)
     E = edges[0]
@@ -605,7 +606,8 @@ def bench_stress(torch, args):
                                    "neighbour rebuild in the step",
                        "edges": E, "atoms": N, "layers": layers, "atoms_per_s": N / sec16},
             "roofline_hbm": edge_roof, "max_abs_diff_vs_fp32_storage_over_scale": rel,
-            "fp32_storage": {"value": E * layers / sec32, "unit": "edges/s", "ms_per_step": sec32 * 1e3}}
+            "fp32_storage": None if sec32 is None else {"value": E * layers / sec32, "unit": "edges/s",
+                                                        "ms_per_step": sec32 * 1e3}}
 
 
 def cpu_denoiser_block(torch, model, x1, r0, box, dims):

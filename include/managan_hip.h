@@ -502,6 +502,15 @@ int mg_bee_node_products_bf16(long n_nodes, int chan, const void* l0, const void
 int mg_segment_sum_csr_bf16(const void* x_edge /* (E,feat) bf16 */, const int* row_ptr, int n_rows, int feat,
                             float scale, void* out /* (n_rows,feat) bf16 */, mg_stream_t stream);
 
+/* TensGroupNorm (managan/tensor_products.py:215-232) on bf16 storage, component-major: y, res (optional), out
+ * (batch * nodes, comps, chan) bfloat16,
+ *   out = gamma[c] * y / sqrt(eps + mean over (nodes, channels of the group) of sum_comps y^2) (+ res).
+ * chan % 8 == 0, comps * chan <= 4608.  scratch: mg_tens_group_norm_bf16_scratch_bytes(batch, groups) bytes,
+ * 8-byte aligned.  Statistics are summed in a fixed order. */
+int mg_tens_group_norm_bf16_scratch_bytes(int batch, int groups, size_t* bytes);
+int mg_tens_group_norm_bf16(const void* y, const void* res, int batch, int nodes, int comps, int chan, int groups, float eps,
+                            const float* gamma, void* scratch, void* out, mg_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

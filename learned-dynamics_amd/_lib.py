@@ -85,6 +85,8 @@ _SIGNATURES = {
     "mg_mlp_chain_bf16": [vp, i64, i32, vp, vp, vp, vp, vp, i32, vp, vp, i64, vp, vp, vp, vp],
     "mg_repel5_sim": [vp, vp, vp, f32, f32, i32, i32, i32, ctypes.c_uint64, ctypes.c_uint32, vp],
     "mg_displacement_sums": [vp, i64, i64, vp, vp, i32, f32, vp, vp, vp, vp],
+    "mg_tens_group_norm_bf16_scratch_bytes": [i32, i32, ctypes.POINTER(ctypes.c_size_t)],
+    "mg_tens_group_norm_bf16": [vp, vp, i32, i32, i32, i32, i32, f32, vp, vp, vp, vp],
     "mg_components_to_rows": [vp, i64, i32, i32, i32, vp, vp, vp],
     "mg_bee_products_linear": [i32, vp, vp, vp, vp, vp, vp, vp, i64, i32, vp, i32, i32, vp, vp],
     "mg_tensor_linear_f16x2_rowsum_workspace_bytes": [i64, i32, ctypes.POINTER(ctypes.c_size_t)],

@@ -14,7 +14,7 @@ significand bits.  Group-norm statistics are taken in fp32.
 import torch
 
 from . import ops
-from .bee_layers import LABELS_0, LABELS_1, LABELS_2, Messages, SelfTensProds
+from .bee_layers import LABELS_0, LABELS_1, LABELS_2, Messages, SelfTensProds, _derived
 from .graph_layers import Graph
 
 
@@ -44,15 +44,23 @@ def _lin(W, x, comps):
 
 
 def _cat_Y(mod, labels, scale=None):
-    W = torch.cat([getattr(mod, f"Y_{lab}").W for lab in labels], dim=1)
-    return W if scale is None else W * scale
+    """[Y_lab.W for lab in labels] concatenated along K (optionally scaled), kept while the weights are unchanged so
+    that its packed planes stay valid from one forward to the next."""
+    params = tuple(getattr(mod, f"Y_{lab}").W for lab in labels)
+
+    def make():
+        W = torch.cat(params, dim=1)
+        return W if scale is None else W * scale
+    return _derived(mod, ("cat_Y_bf16", labels, scale), params, make)
 
 
 def mlp_forward(mlp, x, plus_identity=False):
     """bee_layers.MLP on bf16 rows: lin_direct(x) [+ x] + layers(x)."""
     Wd = mlp.lin_direct.weight
     if plus_identity:
-        Wd = Wd + torch.eye(Wd.shape[0], device=Wd.device, dtype=Wd.dtype)
+        W0 = Wd
+        Wd = _derived(mlp, "direct_plus_identity", (W0,),
+                      lambda: W0 + torch.eye(W0.shape[0], device=W0.device, dtype=W0.dtype))
     Ls = mlp.layers
     h = ops.tensor_linear_bf16(Ls[0].weight, x, bias=Ls[0].bias, act=ops.ACT_LEAKY)
     h = ops.tensor_linear_bf16(Ls[2].weight, h, bias=Ls[2].bias, act=ops.ACT_LEAKY)
@@ -66,7 +74,9 @@ def _mlp_after_sums(mlp, s_x, s_h, row_ptr, plus_identity, scale):
     the sums over rows of its input and of its last hidden layer."""
     Wd = mlp.lin_direct.weight
     if plus_identity:
-        Wd = Wd + torch.eye(Wd.shape[0], device=Wd.device, dtype=Wd.dtype)
+        W0 = Wd
+        Wd = _derived(mlp, "direct_plus_identity", (W0,),
+                      lambda: W0 + torch.eye(W0.shape[0], device=W0.device, dtype=W0.dtype))
     last = mlp.layers[4]
     out = ops.tensor_linear_bf16(Wd, s_x, out_dtype=torch.float32)
     ops.tensor_linear_bf16(last.weight, s_h, out=out, accumulate=True)
@@ -127,10 +137,17 @@ def messages_forward(mod: Messages, graph: Graph, r_ij, s_a, s_v, s_d, node_orde
     return B_a, B_v, B_d
 
 
+def _flat_gamma(gn):
+    return _derived(gn, "flat_gamma", (gn.gamma,), lambda: gn.gamma.detach().reshape(-1).contiguous())
+
+
 def _tens_group_norm(gn, y, res, batch):
     """TensGroupNorm (managan/tensor_products.py:215-232) on a component-major storage tensor
     y (rows, T, dim) or (rows, dim): statistics in fp32 over (nodes, components, group channels)."""
     rows = y.shape[0]
+    comps = 1 if y.dim() == 2 else y.shape[1]
+    if ops.tens_group_norm_bf16_supported(comps, gn.chan):
+        return ops.tens_group_norm_bf16(y, batch, gn.groups, _flat_gamma(gn), gn.epsilon, res)
     x = y.float().reshape(batch, rows // batch, -1, gn.groups, gn.chan // gn.groups)
     m2 = (x * x).sum(2, keepdim=True).mean(dim=(1, 4), keepdim=True)
     out = (x * torch.rsqrt(gn.epsilon + m2)).reshape(y.shape) * gn.gamma.reshape(-1)

@@ -961,6 +961,33 @@ def mlp_chain_bf16(Y, x, W1, b1, W2, b2, row_ptr, seg, n_out, act=ACT_LEAKY):
     return s_psi, s_h
 
 
+def tens_group_norm_bf16_supported(comps, chan):
+    return chan % 8 == 0 and comps * chan <= 4608
+
+
+def tens_group_norm_bf16(y, batch, groups, gamma, eps, res=None):
+    """TensGroupNorm on a component-major bf16 storage tensor y (batch * nodes, comps, chan) or (batch * nodes, chan):
+    gamma * y / sqrt(eps + second moment of the group over nodes, components and the group's channels) (+ res)."""
+    _check_bf16(y, "y")
+    _check_input(gamma, "gamma")
+    if res is not None:
+        _check_bf16(res, "res")
+        if res.shape != y.shape:
+            raise RuntimeError("res must have the shape of y")
+    rows, chan = int(y.size(0)), int(y.size(-1))
+    comps = 1 if y.dim() == 2 else int(y.size(1))
+    if rows % batch or gamma.numel() != chan:
+        raise RuntimeError("rows must be a multiple of batch and gamma must have chan entries")
+    nbytes = ctypes.c_size_t(0)
+    L.check(_lib.mg_tens_group_norm_bf16_scratch_bytes(int(batch), int(groups), ctypes.byref(nbytes)))
+    with torch.cuda.device(y.device):
+        out = torch.empty_like(y)
+        scratch = torch.empty((nbytes.value + 7) // 8, dtype=torch.float64, device=y.device)
+        L.check(_lib.mg_tens_group_norm_bf16(_p(y), _p(res), int(batch), rows // batch, comps, chan, int(groups), float(eps),
+                                             _p(gamma), _p(scratch), _p(out), _stream()))
+    return out
+
+
 def segment_sum_csr_bf16(x_edge, row_ptr, n_rows, scale=1.0):
     """scale * (sum of the bfloat16 edge rows of each CSR row), fp32 accumulation, bfloat16 result."""
     _check_bf16(x_edge, "x_edge")

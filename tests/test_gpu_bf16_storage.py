@@ -281,3 +281,33 @@ def test_messages_bf16_chain_equals_separate_kernels(pkg, ops):
     assert torch.equal(out_chain[1], out_sep[1]) and torch.equal(out_chain[2], out_sep[2])
     a, b = out_chain[0].float(), out_sep[0].float()
     assert float((a - b).abs().max()) <= 2.0 ** -6 * float(b.abs().max())
+
+
+@pytest.mark.parametrize("comps,chan,groups,with_res", [(1, 128, 8, True), (3, 128, 8, True), (9, 128, 8, False),
+                                                        (9, 64, 4, True), (3, 24, 8, True), (9, 512, 8, True)])
+def test_tens_group_norm_bf16(ops, comps, chan, groups, with_res):
+    """mg_tens_group_norm_bf16 against TensGroupNorm's formula (managan/tensor_products.py:215-232) in float64 on the
+    same bf16 inputs: the result is the exact value rounded to bf16, up to one unit in the last place where the fp32
+    scale falls on the other side of a rounding boundary."""
+    g = torch.Generator().manual_seed(comps * chan + groups)
+    batch, nodes, eps = 2, 777, 1e-5
+    shape = (batch * nodes, chan) if comps == 1 else (batch * nodes, comps, chan)
+    y = (torch.randn(shape, generator=g) * torch.rand(1, generator=g) * 3).to(torch.bfloat16)
+    y[nodes:] *= 0.25                                        # the two boxes have different statistics
+    res = torch.randn(shape, generator=g).to(torch.bfloat16) if with_res else None
+    gamma = torch.randn(chan, generator=g)
+    out = ops.tens_group_norm_bf16(y.cuda(), batch, groups, gamma.cuda(), eps, res.cuda() if with_res else None)
+    x = y.double().reshape(batch, nodes, comps, groups, chan // groups)
+    m2 = (x * x).sum(2, keepdim=True).mean(dim=(1, 4), keepdim=True)
+    ref = (x / torch.sqrt(eps + m2)).reshape(y.shape) * gamma.double()
+    fp32_noise = 3e-7 * ref.abs()                            # of the fp32 value that is rounded to bfloat16
+    if with_res:
+        fp32_noise = 3e-7 * (ref.abs() + res.double().abs())  # the sum may cancel
+        ref = ref + res.double()
+    assert out.dtype == torch.bfloat16 and out.shape == y.shape
+    err = (out.cpu().double() - ref).abs()
+    half_ulp = 2.0 ** (torch.floor(torch.log2(ref.abs().clamp_min(1e-30))) - 8)      # of bfloat16 at the exact value
+    assert bool((err <= 2.02 * half_ulp + fp32_noise).all())
+    assert float((err > 1.001 * half_ulp + fp32_noise).double().mean()) < 0.01       # almost always correctly rounded
+    with pytest.raises(RuntimeError, match="multiple of 8"):
+        ops.tens_group_norm_bf16(torch.zeros(4, 12, dtype=torch.bfloat16, device="cuda"), 1, 4, torch.ones(12, device="cuda"), eps)
