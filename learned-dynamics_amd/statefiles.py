@@ -12,7 +12,9 @@ numbers, strings and bytes only and turns every other object into an inert `Opaq
 read with `torch.load(weights_only=True)`.
 """
 import io
+import os
 import pickle
+import random
 import struct
 from dataclasses import dataclass, field
 from typing import Any, Optional, Tuple
@@ -209,8 +211,6 @@ class DatasetPredictor:
     `random.Random` for the shuffle (the reference uses the global one)."""
 
     def __init__(self, dataset_dir, stride=1, repeat=False, rng=None, device=None):
-        import os
-        import random
         self.dataset_dir, self.stride, self.repeat, self.device = dataset_dir, stride, repeat, device
         self._rng = rng if rng is not None else random
         with open(os.path.join(dataset_dir, "predictor_params.pickle"), "rb") as f:
@@ -227,7 +227,6 @@ class DatasetPredictor:
         return self._shape
 
     def sample_q(self, batch):
-        import os
         if self.file_index >= len(self.file_list):
             if not self.repeat:
                 raise DatasetError("out of files in dataset!")
