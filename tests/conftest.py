@@ -1,4 +1,5 @@
 import importlib
+import json
 import os
 import sys
 
@@ -7,6 +8,13 @@ import pytest
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
+
+
+def load_golden(key):
+    """One section of tests/golden/reference_vectors.json: the numeric vectors the reference's own self tests hold
+    for this path, kept as data."""
+    with open(os.path.join(ROOT, "tests", "golden", "reference_vectors.json")) as f:
+        return json.load(f)[key]
 
 
 def pytest_configure(config):

@@ -6,6 +6,7 @@ import numpy as np
 import pytest
 import torch
 
+from conftest import load_golden
 from oracle import neighbour as ON
 
 pytestmark = pytest.mark.gpu
@@ -46,12 +47,13 @@ def _compare(ops, x, cutoff, box, mode=ON.MODE_CELLS):
 
 def test_golden_five_points(ops):
     """Hand-placed points of the reference's self test (managan/graph_layers.py:83-103)."""
-    pos = np.array([[[0., 0., -1.], [1., 0., 0.], [3., 0., 0.], [2., 1., 0.], [8., 0., 0.]]], dtype=np.float32)
-    xt, src, dst, ec, row_ptr = _run(ops, pos, 2.0, (100., 100., 100.), listmax=32, nmax=64)
-    assert np.array_equal(np.diff(row_ptr.cpu().numpy()), [1, 3, 2, 2, 0])
+    five = load_golden("graph_layers_five_points")
+    pos = np.array(five["positions"], dtype=np.float32)
+    xt, src, dst, ec, row_ptr = _run(ops, pos, five["radius"], tuple(five["box"]), listmax=32, nmax=64)
+    assert np.array_equal(np.diff(row_ptr.cpu().numpy()), five["degrees"][0])
     got = set(zip(src.tolist(), dst.tolist()))
-    assert got == {(0, 1), (1, 0), (1, 2), (1, 3), (2, 1), (2, 3), (3, 1), (3, 2)}
-    assert ec.tolist() == [8]
+    assert got == {tuple(e) for e in five["edges"]}
+    assert ec.tolist() == [len(five["edges"])]
 
 
 def test_wrap_cells_bit_exact(ops):

@@ -5,6 +5,7 @@ import numpy as np
 import pytest
 import torch
 
+from conftest import load_golden
 from oracle import layers as OL
 
 pytestmark = pytest.mark.gpu
@@ -64,23 +65,23 @@ def test_graph_layers_golden(pkg):
     """The reference's self test (managan/graph_layers.py:80-122): degrees, the sum-of-products
     matrix 'calculated on paper', and the wrap bound."""
     gl = importlib.import_module("learned-dynamics_amd.graph_layers")
-    positions = torch.tensor([[[0., 0., -1.], [1., 0., 0.], [3., 0., 0.], [2., 1., 0.], [8., 0., 0.]]], device="cuda")
-    graph = gl.Graph.radius_graph(2., (100., 100., 100.), positions)
+    five = load_golden("graph_layers_five_points")
+    box = tuple(five["box"])
+    positions = torch.tensor(five["positions"], device="cuda")
+    graph = gl.Graph.radius_graph(five["radius"], box, positions)
     assert torch.all(graph.src[1:] >= graph.src[:-1])
     assert graph.src.dtype == torch.int64 and graph.dst.dtype == torch.int64
     ones = torch.ones_like(graph.dst, dtype=torch.float)
     degrees = gl.edges_reduce_src(graph, ones)
-    assert torch.allclose(degrees, torch.tensor([[1., 3., 2., 2., 0.]], device="cuda"))
+    assert torch.allclose(degrees, torch.tensor(five["degrees"], device="cuda", dtype=torch.float))
     x = torch.arange(5, device="cuda").to(torch.float).repeat(4).reshape(1, 5, 4)
     s, d = gl.edges_read(graph, x)
     sumprod = gl.edges_reduce_src(graph, s * d)
-    expected = torch.tensor([[0., 0., 2., 6.], [20., 0., 6., 8.], [18., 12., 0., 2.], [14., 12., 4., 0.],
-                             [0., 0., 0., 0.]], device="cuda")[None]
-    assert torch.allclose(sumprod, expected)
+    assert torch.allclose(sumprod, torch.tensor(five["sum_of_products"], device="cuda"))
     pos_src, pos_dst = gl.edges_read(graph, positions)
-    delta = gl.boxwrap(torch.tensor((100., 100., 100.), device="cuda"), pos_dst - pos_src)
-    assert torch.all((delta ** 2).sum(-1) < 2.001 ** 2)
-    assert torch.equal(delta, gl.edge_vectors(graph, positions, (100., 100., 100.)))
+    delta = gl.boxwrap(torch.tensor(box, device="cuda"), pos_dst - pos_src)
+    assert torch.all((delta ** 2).sum(-1) < five["wrapped_length_bound"] ** 2)
+    assert torch.equal(delta, gl.edge_vectors(graph, positions, box))
 
 
 def test_torch_scatter_shim(pkg):

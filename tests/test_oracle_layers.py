@@ -7,12 +7,11 @@ import numpy as np
 import pytest
 import torch
 
+from conftest import load_golden
 from oracle import layers as OL
 from oracle import products as OP
 
-ROT = torch.tensor([[-0.2590, -0.5228, 0.8121],
-                    [0.6468, -0.7184, -0.2562],
-                    [0.7174, 0.4589, 0.5242]], dtype=torch.float64)   # managan/symmetries.py:54-57
+ROT = torch.tensor(load_golden("symmetry_checks")["rotation"], dtype=torch.float64)   # managan/symmetries.py:54-57
 Q, _ = torch.linalg.qr(ROT)
 ROT = Q * torch.sign(torch.linalg.det(Q))            # exact rotation next to the printed one
 

@@ -7,40 +7,41 @@ import ctypes
 import numpy as np
 import pytest
 
+from conftest import load_golden
 from oracle import neighbour as ON
+
+FIVE = load_golden("graph_layers_five_points")      # managan/graph_layers.py:83-122
 
 
 def test_golden_five_points():
     # managan/graph_layers.py:83-103: r0=2, box 100 connects (0,1) and (1,2,3)
-    pos = np.array([[[0., 0., -1.], [1., 0., 0.], [3., 0., 0.], [2., 1., 0.], [8., 0., 0.]]], dtype=np.float32)
+    pos = np.array(FIVE["positions"], dtype=np.float32)
+    box = tuple(FIVE["box"])
     for mode in (ON.MODE_CELLS, ON.MODE_BRUTE_WINDOW, ON.MODE_BRUTE_MINIMAGE):
-        r = ON.edges(pos, 2.0, (100., 100., 100.), mode)
-        assert r["counts"].tolist() == [[1, 3, 2, 2, 0]]
-        assert set(zip(r["src"].tolist(), r["dst"].tolist())) == {
-            (0, 1), (1, 0), (1, 2), (1, 3), (2, 1), (2, 3), (3, 1), (3, 2)}
-        assert r["edge_counts"].tolist() == [8]
-    src, dst, ec = ON.get_edges(32, 64, 2.0, 100., 100., 100., pos)
+        r = ON.edges(pos, FIVE["radius"], box, mode)
+        assert r["counts"].tolist() == FIVE["degrees"]
+        assert set(zip(r["src"].tolist(), r["dst"].tolist())) == {tuple(e) for e in FIVE["edges"]}
+        assert r["edge_counts"].tolist() == [len(FIVE["edges"])]
+    src, dst, ec = ON.get_edges(32, 64, FIVE["radius"], *box, pos)
     assert np.all(src[1:] >= src[:-1])
     # boxwrap bound of the same self test (graph_layers.py:120-122)
-    d = ON.edge_vectors(pos, src, dst, (100., 100., 100.))
-    assert np.all((d ** 2).sum(-1) < 2.001 ** 2)
+    d = ON.edge_vectors(pos, src, dst, box)
+    assert np.all((d ** 2).sum(-1) < FIVE["wrapped_length_bound"] ** 2)
 
 
 def test_golden_sumprod_through_oracle_scatter():
     """graph_layers.py:106-117: sum_j x_i x_j 'calculated on paper'."""
     import torch
     from oracle import layers as OL
-    pos = np.array([[[0., 0., -1.], [1., 0., 0.], [3., 0., 0.], [2., 1., 0.], [8., 0., 0.]]], dtype=np.float32)
-    src, dst, _ = ON.get_edges(32, 64, 2.0, 100., 100., 100., pos)
+    pos = np.array(FIVE["positions"], dtype=np.float32)
+    src, dst, _ = ON.get_edges(32, 64, FIVE["radius"], *FIVE["box"], pos)
     src_t, dst_t = torch.from_numpy(src).long(), torch.from_numpy(dst).long()
     x = torch.arange(5).float().repeat(4).reshape(1, 5, 4)
     flat = x.reshape(5, 4)
     sumprod = OL.edges_reduce_src(src_t, flat[src_t] * OL.edges_read_dst(dst_t, x, 1, 5), 1, 5)
-    expected = torch.tensor([[0., 0., 2., 6.], [20., 0., 6., 8.], [18., 12., 0., 2.], [14., 12., 4., 0.],
-                             [0., 0., 0., 0.]])[None]
-    assert torch.equal(sumprod, expected)
+    assert torch.equal(sumprod, torch.tensor(FIVE["sum_of_products"]))
     deg = OL.edges_reduce_src(src_t, torch.ones(len(src)), 1, 5)
-    assert deg.tolist() == [[1., 3., 2., 2., 0.]]
+    assert deg.tolist() == FIVE["degrees"]
 
 
 def test_reference_invariants_on_its_test_shape():

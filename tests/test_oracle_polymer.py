@@ -4,6 +4,7 @@ noise generator against published known-answer vectors.  CPU only."""
 import numpy as np
 import pytest
 
+from conftest import load_golden
 from oracle import polymer as OPY
 
 
@@ -92,14 +93,9 @@ def test_energy_is_conserved_without_drag_and_time_reverses():
 def test_philox_known_answers():
     """Known-answer vectors of Philox4x32-10 from the reference implementation of Salmon et al. (Random123
     kat_vectors: counter, key -> output)."""
-    kat = [
-        ((0x00000000, 0x00000000, 0x00000000, 0x00000000), (0x00000000, 0x00000000),
-         (0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8)),
-        ((0xffffffff, 0xffffffff, 0xffffffff, 0xffffffff), (0xffffffff, 0xffffffff),
-         (0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd)),
-        ((0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344), (0xa4093822, 0x299f31d0),
-         (0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1)),
-    ]
+    kat = [tuple(tuple(int(w, 16) for w in v[k]) for k in ("counter", "key", "output"))
+           for v in load_golden("philox4x32_10")["vectors"]]
+    assert len(kat) == 3
     for counter, key, want in kat:
         got = OPY.philox4x32_10(np.array(counter, dtype=np.uint32), np.array(key, dtype=np.uint32))
         assert tuple(int(g) for g in got) == want

@@ -7,11 +7,10 @@ import itertools
 import pytest
 import torch
 
+from conftest import load_golden
 from oracle import products as OP
 
-ROT = torch.tensor([[-0.2590, -0.5228, 0.8121],
-                    [0.6468, -0.7184, -0.2562],
-                    [0.7174, 0.4589, 0.5242]], dtype=torch.float64)
+ROT = torch.tensor(load_golden("symmetry_checks")["rotation"], dtype=torch.float64)
 
 
 def _rand(rows, chan, rank, seed, dtype=torch.float64):
