@@ -487,7 +487,8 @@ def edge_kernel_roofline(torch, msg, graph, r_ij, rows, bf16=False):
             "traffic": None, "bytes_per_launch": nbytes, "ms": t * 1e3,
             # the 13 products are 167 flop per (edge, channel), the 60 running sums another 60
             "fp32_vector_tflops": E * chan * 227 / t / 1e12,
-            "fp32_vector_frac_of_peak": E * chan * 227 / t / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+            # the vector rate without packed fp32 instructions (compiled out here) is half the published 157.3 TFLOP/s
+            "fp32_vector_frac_of_peak": E * chan * 227 / t / 1e12 / (PEAK_FP32_MFMA_TFLOPS / 2),
             "note": "gathered node rows are served by L2 and counted once per node; with ~90 edges per node "
                     "(configs[4]) the kernel is bound by its fp32 vector arithmetic (packed fp32 instructions "
                     "are compiled out, which halves the vector peak), with ~16 (configs[3]) by L2 gather latency "
