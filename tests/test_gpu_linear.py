@@ -293,3 +293,34 @@ def test_linear_with_row_sums_edge_cases(ops):
     torch.testing.assert_close(out.double(), ref, rtol=1e-5, atol=3e-6 * float(ref.abs().max()))
     with pytest.raises(RuntimeError, match="multiple of 256"):
         ops.tensor_linear_f16x2_rowsum(W[:128].contiguous(), x, ops.row_absmax(x), row_ptr, seg, 1)
+
+
+@pytest.mark.parametrize("inds", [0, 1, 2])
+def test_plain_entry_point_through_ctypes(pkg, inds):
+    """mg_tensor_linear called as a foreign caller would (raw pointers, element strides of W, the current stream):
+    the transposed view of W, bias + SiLU for inds = 0, accumulation into y, and zero rows."""
+    import ctypes
+    L = importlib.import_module("learned-dynamics_amd._lib")
+    lib = L.load()
+    g = torch.Generator().manual_seed(40 + inds)
+    Wt = torch.randn(48, 96, generator=g)                      # stored (dim_in, dim_out): W = Wt.t()
+    x = torch.randn(33, 48, *([3] * inds), generator=g)
+    bias = torch.randn(96, generator=g) if inds == 0 else None
+    y0 = torch.randn(33, 96, *([3] * inds), generator=g)
+    Wd, xd, yd = Wt.cuda(), x.cuda(), y0.cuda()
+    bd = bias.cuda() if bias is not None else None
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    act = 1 if inds == 0 else 0
+    L.check(lib.mg_tensor_linear(inds, Wd.data_ptr(), Wd.stride(1), Wd.stride(0), xd.data_ptr(), 33, 48, 96,
+                                 bd.data_ptr() if bd is not None else None, act, 0, yd.data_ptr(), st))
+    ref = OP.tensor_linear(inds, Wt.t(), x)
+    if inds == 0:
+        ref = torch.nn.functional.silu(ref + bias)
+    _check(yd, ref, 48)
+    L.check(lib.mg_tensor_linear(inds, Wd.data_ptr(), Wd.stride(1), Wd.stride(0), xd.data_ptr(), 33, 48, 96,
+                                 None, 0, 1, yd.data_ptr(), st))
+    _check(yd, ref + OP.tensor_linear(inds, Wt.t(), x), 48)
+    before = yd.clone()
+    L.check(lib.mg_tensor_linear(inds, Wd.data_ptr(), Wd.stride(1), Wd.stride(0), xd.data_ptr(), 0, 48, 96,
+                                 None, 0, 0, yd.data_ptr(), st))
+    assert torch.equal(yd, before)
