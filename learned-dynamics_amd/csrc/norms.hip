@@ -27,6 +27,8 @@ __device__ __forceinline__ double block_sum(double v, double* lds) {
 // x element (box b, node i, channel c, comp t) at x[((b*N + i)*x_stride + c)*T + t]; optional elementwise
 // multiplier mul at the same index pattern with mul_stride.  partial[(b*G + g)*kChunks + chunk][0..1] =
 // (sum, sum of squares) over that chunk's nodes, the group's channels and all components.
+// A group's channels and components of one node are cg*T consecutive floats, so an element is addressed by its
+// node and its offset in that run; both advance by constants from one trip to the next (no division per element).
 __global__ void __launch_bounds__(256) group_stats_kernel(const float* __restrict__ x, long x_stride,
                                                           const float* __restrict__ mul, long mul_stride, int N,
                                                           int chan, int groups, int T, double* __restrict__ partial) {
@@ -36,17 +38,22 @@ __global__ void __launch_bounds__(256) group_stats_kernel(const float* __restric
     const int cg = chan / groups;
     const int per = (N + kChunks - 1) / kChunks;
     const int n_lo = chunk * per, n_hi = n_lo + per < N ? n_lo + per : N;
-    const long row_elems = (long)cg * T;
+    const int run = cg * T;
+    const int step_i = (int)blockDim.x / run, step_r = (int)blockDim.x % run;
+    int i = n_lo + (int)threadIdx.x / run, r = (int)threadIdx.x % run;
+    const float* xg = x + (long)g * cg * T;
+    const float* mul_g = mul ? mul + (long)g * cg * T : nullptr;
+    const long x_row = x_stride * T, m_row = mul_stride * T;
     double s = 0.0, ss = 0.0;
-    const long total = (long)(n_hi > n_lo ? n_hi - n_lo : 0) * row_elems;
-    for (long t = threadIdx.x; t < total; t += blockDim.x) {
-        const long i = n_lo + t / row_elems;
-        const long rem = t - (t / row_elems) * row_elems;      // (c_local, comp), comp fastest
-        const long c = g * cg + rem / T, comp = rem - (rem / T) * T;
-        float v = x[(((long)b * N + i) * x_stride + c) * T + comp];
-        if (mul) v *= mul[(((long)b * N + i) * mul_stride + c) * T + comp];
+    while (i < n_hi) {
+        const long row = (long)b * N + i;
+        float v = xg[row * x_row + r];
+        if (mul_g) v *= mul_g[row * m_row + r];
         s += v;
         ss += (double)v * v;
+        i += step_i;
+        r += step_r;
+        if (r >= run) { r -= run; i++; }
     }
     const double ts = block_sum(s, lds);
     const double tss = block_sum(ss, lds);
@@ -56,8 +63,10 @@ __global__ void __launch_bounds__(256) group_stats_kernel(const float* __restric
     }
 }
 
-// fold the kChunks partials of every (box, group) in a fixed order: partial[bg*kChunks*2 + {0,1}] <- totals
-__global__ void group_finalize_kernel(double* __restrict__ partial, int n_bg) {
+// fold the kChunks partials of every (box, group) in a fixed order and derive what the apply kernel uses:
+// partial[bg*kChunks*2 + {0,1}] <- totals, + 2 <- the mean that is subtracted (0 for the tensor norm),
+// + 3 <- the denominator sqrt(eps + variance or mean square); both rounded to float as the apply kernel takes them
+__global__ void group_finalize_kernel(double* __restrict__ partial, int n_bg, double count, int mode, float eps) {
     const int bg = blockIdx.x * blockDim.x + threadIdx.x;
     if (bg >= n_bg) return;
     double* p = partial + (long)bg * kChunks * 2;
@@ -65,41 +74,48 @@ __global__ void group_finalize_kernel(double* __restrict__ partial, int n_bg) {
     for (int k = 0; k < kChunks; k++) { s += p[2 * k]; ss += p[2 * k + 1]; }
     p[0] = s;
     p[1] = ss;
+    if (mode == 0) {
+        p[2] = 0.0;
+        p[3] = (double)sqrtf(eps + (float)(ss / count));          // mean over nodes, group channels of sum_comp v^2
+    } else {
+        const double mean = s / count;
+        double var = ss / count - mean * mean;
+        var = var > 0.0 ? var : 0.0;
+        p[2] = (double)(float)mean;
+        p[3] = (double)sqrtf(eps + (float)var);
+    }
 }
 
 // mode 0 (TensGroupNorm): y = gamma[c] * v / sqrt(eps + mean(sum_comp v^2))
 // mode 1 (ScalGroupNorm, T = 1): y = beta[c] + gamma[c] * (v - mean) / sqrt(eps + var)
 // then y += add (optional, add_stride) and y += res (optional, same layout as out).
+// A thread keeps one (channel, component) position k = c*T + comp of the rows of box blockIdx.z and walks over
+// nodes: channel, group, gamma, beta and the group's statistics are fixed per thread, consecutive threads touch
+// consecutive floats.
 __global__ void __launch_bounds__(256) group_apply_kernel(const float* __restrict__ x, long x_stride,
                                                           const float* __restrict__ mul, long mul_stride,
-                                                          const double* __restrict__ partial, int B, int N, int chan,
-                                                          int groups, int T, int mode, float eps,
+                                                          const double* __restrict__ partial, int N, int chan,
+                                                          int groups, int T, int mode,
                                                           const float* __restrict__ gamma, const float* __restrict__ beta,
                                                           const float* __restrict__ add, long add_stride,
                                                           const float* __restrict__ res, float* __restrict__ out) {
-    const long total = (long)B * N * chan * T;
-    const int cg = chan / groups;
-    for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (long)gridDim.x * blockDim.x) {
-        const long comp = t % T, c = (t / T) % chan, row = t / ((long)T * chan);
-        const int b = (int)(row / N), g = (int)(c / cg);
-        const double* p = partial + ((long)(b * groups + g) * kChunks) * 2;   // totals after the finalize kernel
-        const double s = p[0], ss = p[1];
-        float v = x[(row * x_stride + c) * T + comp];
-        if (mul) v *= mul[(row * mul_stride + c) * T + comp];
-        float y;
-        if (mode == 0) {
-            const double m2 = ss / ((double)N * cg);                      // mean over nodes and group channels
-            y = gamma[c] * (v / sqrtf(eps + (float)m2));
-        } else {
-            const double cnt = (double)N * cg;
-            const double mean = s / cnt;
-            double var = ss / cnt - mean * mean;
-            var = var > 0.0 ? var : 0.0;
-            y = beta[c] + gamma[c] * ((v - (float)mean) / sqrtf(eps + (float)var));
-        }
-        if (add) y += add[(row * add_stride + c) * T + comp];
-        if (res) y += res[t];
-        out[t] = y;
+    const int k = blockIdx.x * blockDim.x + threadIdx.x;
+    const int CT = chan * T;
+    if (k >= CT) return;
+    const int b = blockIdx.z;
+    const int c = k / T, g = c / (chan / groups);
+    const double* p = partial + ((long)(b * groups + g) * kChunks) * 2;
+    const float mean = (float)p[2], denom = (float)p[3];
+    const float ga = gamma[c], be = mode == 0 ? 0.f : beta[c];
+    const long x_row = x_stride * T, m_row = mul_stride * T, a_row = add_stride * T;
+    for (int i = blockIdx.y; i < N; i += gridDim.y) {
+        const long row = (long)b * N + i;
+        float v = x[row * x_row + k];
+        if (mul) v *= mul[row * m_row + k];
+        float y = mode == 0 ? ga * (v / denom) : be + ga * ((v - mean) / denom);
+        if (add) y += add[row * a_row + k];
+        if (res) y += res[row * CT + k];
+        out[row * CT + k] = y;
     }
 }
 
@@ -200,13 +216,19 @@ int mg_group_norm(int mode, const float* x, long x_stride, const float* mul, lon
     const long total = (long)batch * nodes * chan * comps;
     if (total == 0) return MG_OK;
     MG_REQUIRE(x && gamma && out && scratch && (mode == 0 || beta), "mg_group_norm: null pointer");
+    MG_REQUIRE(batch <= 65535 && (long)chan * comps <= 0x7fffffffL, "mg_group_norm: more than 65535 boxes");
     hipStream_t st = (hipStream_t)stream;
     hipLaunchKernelGGL(group_stats_kernel, dim3((unsigned)(batch * groups), kChunks), dim3(256), 0, st, x, x_stride, mul,
                        mul_stride, nodes, chan, groups, comps, static_cast<double*>(scratch));
     hipLaunchKernelGGL(group_finalize_kernel, dim3((unsigned)ceil_div((long)batch * groups, 64)), dim3(64), 0, st,
-                       static_cast<double*>(scratch), batch * groups);
-    hipLaunchKernelGGL(group_apply_kernel, dim3((unsigned)grid_for(total)), dim3(256), 0, st, x, x_stride, mul,
-                       mul_stride, static_cast<const double*>(scratch), batch, nodes, chan, groups, comps, mode, eps,
+                       static_cast<double*>(scratch), batch * groups, (double)nodes * (chan / groups), mode, eps);
+    const int CT = chan * comps;
+    const int threads = CT >= 256 ? 256 : (int)ceil_div(CT, kWave) * kWave;
+    const long kx = ceil_div(CT, threads);
+    long ny = ceil_div(8192L, kx * batch);                      // about 8192 workgroups, each thread a few nodes
+    ny = ny > nodes ? nodes : (ny < 1 ? 1 : ny);
+    hipLaunchKernelGGL(group_apply_kernel, dim3((unsigned)kx, (unsigned)ny, (unsigned)batch), dim3(threads), 0, st, x,
+                       x_stride, mul, mul_stride, static_cast<const double*>(scratch), nodes, chan, groups, comps, mode,
                        gamma, beta, add, add_stride, res, out);
     return check_launch("mg_group_norm");
 }
