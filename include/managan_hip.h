@@ -409,13 +409,14 @@ int mg_tensor_linear_f16x2_rowsum(const void* packed_W, const float* x, const fl
                                   float* y, float* out, mg_stream_t stream);
 
 /* Update.forward (archs/meanflow_painn8.py:63-75), elementwise parts around its GEMMs.
- * lrv (rows, 3n, 3) = [lin_l | lin_r | lin_v] applied to x_v (one stacked tensor_linear).
+ * lrv = [lin_l | lin_r | lin_v] applied to x_v (one stacked tensor_linear), stored (rows, 3n, 3) as the reference
+ * stores tensors (lrv_comp_major = 0) or component-major (rows, 3, 3n) (lrv_comp_major = 1).
  *   pre:  ip[r,c] = sum_x l[c,x] r[c,x];  cat[r] = [x_a[r] | |r[c]|]  (rows, 2n), the MLP input
- *   vec:  v = lin_v(x_v) * y[:, 0:n];  out_v = res_v + v / sqrt(1 + |v|^2)   (y: (rows, 3n) MLP output)
+ *   vec:  v = lin_v(x_v) * y[:, 0:n];  out_v (rows, n, 3) = res_v + v / sqrt(1 + |v|^2)   (y: (rows, 3n) MLP output)
  * The scalar output is mg_group_norm(mode 1) of ip * y[:, n:2n] plus y[:, 2n:3n]. */
-int mg_painn_update_pre(const float* lrv, const float* x_a, long rows, int n, float* ip, float* cat,
+int mg_painn_update_pre(const float* lrv, int lrv_comp_major, const float* x_a, long rows, int n, float* ip, float* cat,
                         mg_stream_t stream);
-int mg_painn_update_vec(const float* lrv, const float* y, const float* res_v /* or NULL */, long rows, int n,
+int mg_painn_update_vec(const float* lrv, int lrv_comp_major, const float* y, const float* res_v /* or NULL */, long rows, int n,
                         float* out_v, mg_stream_t stream);
 
 /* ------------------------------------------------------------------------

@@ -130,39 +130,47 @@ __global__ void __launch_bounds__(256) tens_sigmoid_kernel(const float* __restri
     }
 }
 
-// PaiNN Update, first elementwise stage: lrv (rows, 3n, 3) = [lin_l | lin_r | lin_v](x_v)
+// PaiNN Update, first elementwise stage: lrv = [lin_l | lin_r | lin_v](x_v), stored (rows, 3n, 3) or, COMP_MAJOR,
+// (rows, 3, 3n) (what the GEMM stores at full rate, and what a wave reads here with unit stride)
 //   ip[r,c] = sum_x l[c,x] r[c,x];  cat[r] = [x_a[r] | |r[c]|]   (rows, 2n)
-__global__ void __launch_bounds__(256) painn_update_pre_kernel(const float* __restrict__ lrv, const float* __restrict__ x_a,
-                                                               long rows, int n, float* __restrict__ ip,
-                                                               float* __restrict__ cat) {
-    const long total = rows * n;
-    for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (long)gridDim.x * blockDim.x) {
-        const long r = t / n;
-        const int c = (int)(t - r * n);
-        const float* l = lrv + (r * 3 * n + c) * 3;
-        const float* rr = lrv + (r * 3 * n + n + c) * 3;
-        ip[t] = l[0] * rr[0] + l[1] * rr[1] + l[2] * rr[2];
-        cat[r * 2 * n + c] = x_a[t];
-        cat[r * 2 * n + n + c] = sqrtf(rr[0] * rr[0] + rr[1] * rr[1] + rr[2] * rr[2]);
-    }
+// One workgroup row per node row: blockIdx.x = r, the channel from blockIdx.y and the thread.
+template <bool COMP_MAJOR>
+__device__ __forceinline__ float lrv_at(const float* __restrict__ row, int n, int j, int x) {
+    return COMP_MAJOR ? row[x * 3 * n + j] : row[j * 3 + x];
 }
 
-// PaiNN Update, vector output: v = lin_v(x_v) * y[0:n]; out = res_v + v / sqrt(1 + |v|^2)
+template <bool COMP_MAJOR>
+__global__ void __launch_bounds__(256) painn_update_pre_kernel(const float* __restrict__ lrv, const float* __restrict__ x_a,
+                                                               int n, float* __restrict__ ip, float* __restrict__ cat) {
+    const long r = blockIdx.x;
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= n) return;
+    const float* row = lrv + r * 9 * n;
+    float l[3], rr[3];
+#pragma unroll
+    for (int x = 0; x < 3; x++) { l[x] = lrv_at<COMP_MAJOR>(row, n, c, x); rr[x] = lrv_at<COMP_MAJOR>(row, n, n + c, x); }
+    ip[r * n + c] = l[0] * rr[0] + l[1] * rr[1] + l[2] * rr[2];
+    cat[r * 2 * n + c] = x_a[r * n + c];
+    cat[r * 2 * n + n + c] = sqrtf(rr[0] * rr[0] + rr[1] * rr[1] + rr[2] * rr[2]);
+}
+
+// PaiNN Update, vector output: v = lin_v(x_v) * y[0:n]; out = res_v + v / sqrt(1 + |v|^2), out (rows, n, 3)
+template <bool COMP_MAJOR>
 __global__ void __launch_bounds__(256) painn_update_vec_kernel(const float* __restrict__ lrv, const float* __restrict__ y,
-                                                               const float* __restrict__ res_v, long rows, int n,
+                                                               const float* __restrict__ res_v, int n,
                                                                float* __restrict__ out_v) {
-    const long total = rows * n;
-    for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < total; t += (long)gridDim.x * blockDim.x) {
-        const long r = t / n;
-        const int c = (int)(t - r * n);
-        const float* v = lrv + (r * 3 * n + 2 * n + c) * 3;
-        const float s = y[r * 3 * n + c];
-        const float a = v[0] * s, b = v[1] * s, d = v[2] * s;
-        const float inv = 1.0f / sqrtf(1.0f + (a * a + b * b + d * d));
-        float o0 = a * inv, o1 = b * inv, o2 = d * inv;
-        if (res_v) { o0 += res_v[3 * t]; o1 += res_v[3 * t + 1]; o2 += res_v[3 * t + 2]; }
-        out_v[3 * t] = o0; out_v[3 * t + 1] = o1; out_v[3 * t + 2] = o2;
-    }
+    const long r = blockIdx.x;
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= n) return;
+    const float* row = lrv + r * 9 * n;
+    const float s = y[r * 3 * n + c];
+    const float a = lrv_at<COMP_MAJOR>(row, n, 2 * n + c, 0) * s, b = lrv_at<COMP_MAJOR>(row, n, 2 * n + c, 1) * s,
+                d = lrv_at<COMP_MAJOR>(row, n, 2 * n + c, 2) * s;
+    const float inv = 1.0f / sqrtf(1.0f + (a * a + b * b + d * d));
+    float o0 = a * inv, o1 = b * inv, o2 = d * inv;
+    const long t = r * n + c;
+    if (res_v) { o0 += res_v[3 * t]; o1 += res_v[3 * t + 1]; o2 += res_v[3 * t + 2]; }
+    out_v[3 * t] = o0; out_v[3 * t + 1] = o1; out_v[3 * t + 2] = o2;
 }
 
 // kinds: 1 sq_radial_encode of normed_sq_dist (archs/diffuser_atoms14.py:32-48)
@@ -243,23 +251,33 @@ int mg_tens_sigmoid(int inds, const float* x, long rows_times_chan, float* out, 
     return check_launch("mg_tens_sigmoid");
 }
 
-int mg_painn_update_pre(const float* lrv, const float* x_a, long rows, int n, float* ip, float* cat,
+int mg_painn_update_pre(const float* lrv, int lrv_comp_major, const float* x_a, long rows, int n, float* ip, float* cat,
                         mg_stream_t stream) {
     MG_REQUIRE(rows >= 0 && n >= 0, "mg_painn_update_pre: negative size");
     if (rows * n == 0) return MG_OK;
     MG_REQUIRE(lrv && x_a && ip && cat, "mg_painn_update_pre: null pointer");
-    hipLaunchKernelGGL(painn_update_pre_kernel, dim3((unsigned)grid_for(rows * n)), dim3(256), 0, (hipStream_t)stream,
-                       lrv, x_a, rows, n, ip, cat);
+    MG_REQUIRE(rows <= 0x7fffffffL, "mg_painn_update_pre: more than 2^31 - 1 rows");
+    const int threads = n >= 256 ? 256 : (int)ceil_div(n, kWave) * kWave;
+    const dim3 grid((unsigned)rows, (unsigned)ceil_div(n, threads));
+    if (lrv_comp_major)
+        hipLaunchKernelGGL(painn_update_pre_kernel<true>, grid, dim3(threads), 0, (hipStream_t)stream, lrv, x_a, n, ip, cat);
+    else
+        hipLaunchKernelGGL(painn_update_pre_kernel<false>, grid, dim3(threads), 0, (hipStream_t)stream, lrv, x_a, n, ip, cat);
     return check_launch("mg_painn_update_pre");
 }
 
-int mg_painn_update_vec(const float* lrv, const float* y, const float* res_v, long rows, int n, float* out_v,
-                        mg_stream_t stream) {
+int mg_painn_update_vec(const float* lrv, int lrv_comp_major, const float* y, const float* res_v, long rows, int n,
+                        float* out_v, mg_stream_t stream) {
     MG_REQUIRE(rows >= 0 && n >= 0, "mg_painn_update_vec: negative size");
     if (rows * n == 0) return MG_OK;
     MG_REQUIRE(lrv && y && out_v, "mg_painn_update_vec: null pointer");
-    hipLaunchKernelGGL(painn_update_vec_kernel, dim3((unsigned)grid_for(rows * n)), dim3(256), 0, (hipStream_t)stream,
-                       lrv, y, res_v, rows, n, out_v);
+    MG_REQUIRE(rows <= 0x7fffffffL, "mg_painn_update_vec: more than 2^31 - 1 rows");
+    const int threads = n >= 256 ? 256 : (int)ceil_div(n, kWave) * kWave;
+    const dim3 grid((unsigned)rows, (unsigned)ceil_div(n, threads));
+    if (lrv_comp_major)
+        hipLaunchKernelGGL(painn_update_vec_kernel<true>, grid, dim3(threads), 0, (hipStream_t)stream, lrv, y, res_v, n, out_v);
+    else
+        hipLaunchKernelGGL(painn_update_vec_kernel<false>, grid, dim3(threads), 0, (hipStream_t)stream, lrv, y, res_v, n, out_v);
     return check_launch("mg_painn_update_vec");
 }
 

@@ -1483,17 +1483,25 @@ def tens_sigmoid(inds, x):
     return out
 
 
+def _lrv_layout(lrv, rows, n):
+    """1 for component-major (rows, 3, 3n), 0 for the reference's (rows, 3n, 3)."""
+    if tuple(lrv.shape) == (rows, 3 * n, 3):
+        return 0
+    if tuple(lrv.shape) == (rows, 3, 3 * n):
+        return 1
+    raise RuntimeError("lrv must have shape (rows, 3n, 3) or, component-major, (rows, 3, 3n)")
+
+
 def painn_update_pre(lrv, x_a):
-    """lrv (rows, 3n, 3), x_a (rows, n) -> ip (rows, n), cat (rows, 2n)."""
+    """lrv (rows, 3n, 3) or component-major (rows, 3, 3n), x_a (rows, n) -> ip (rows, n), cat (rows, 2n)."""
     _check_input(lrv, "lrv")
     _check_input(x_a, "x_a")
     rows, n = int(x_a.shape[0]), int(x_a.shape[1])
-    if tuple(lrv.shape) != (rows, 3 * n, 3):
-        raise RuntimeError("lrv must have shape (rows, 3n, 3)")
+    layout = _lrv_layout(lrv, rows, n)
     with torch.cuda.device(x_a.device):
         ip = torch.empty(rows, n, dtype=torch.float32, device=x_a.device)
         cat = torch.empty(rows, 2 * n, dtype=torch.float32, device=x_a.device)
-        L.check(_lib.mg_painn_update_pre(_p(lrv), _p(x_a), rows, n, _p(ip), _p(cat), _stream()))
+        L.check(_lib.mg_painn_update_pre(_p(lrv), layout, _p(x_a), rows, n, _p(ip), _p(cat), _stream()))
     return ip, cat
 
 
@@ -1502,13 +1510,12 @@ def painn_update_vec(lrv, y, res_v=None):
     _check_input(lrv, "lrv")
     _check_input(y, "y")
     rows, n = int(y.shape[0]), int(y.shape[1]) // 3
-    if tuple(lrv.shape) != (rows, 3 * n, 3):
-        raise RuntimeError("lrv must have shape (rows, 3n, 3)")
+    layout = _lrv_layout(lrv, rows, n)
     if res_v is not None:
         _check_input(res_v, "res_v")
     with torch.cuda.device(y.device):
         out = torch.empty(rows, n, 3, dtype=torch.float32, device=y.device)
-        L.check(_lib.mg_painn_update_vec(_p(lrv), _p(y), _p(res_v), rows, n, _p(out), _stream()))
+        L.check(_lib.mg_painn_update_vec(_p(lrv), layout, _p(y), _p(res_v), rows, n, _p(out), _stream()))
     return out
 
 

@@ -120,7 +120,8 @@ class Update(nn.Module):
             with torch.no_grad():                                               # while the weights are unchanged, so
                 cache.update(stamp=stamp, W=torch.cat(params, dim=0))           # its packed planes stay valid too
         W = cache["W"]
-        lrv = ops.tensor_linear_fwd(1, W, flat_v)                               # (rows, 3n, 3)
+        # component-major (rows, 3, 3n): the GEMM stores whole rows, the two kernels below read with unit stride
+        lrv = ops.tensor_linear_fwd(1, W, flat_v, y_layout=ops.LAYOUT_COMP_CHAN)
         ip, cat = ops.painn_update_pre(lrv, flat_a)                             # l.r and [x_a | |r|]
         y = self.mlp(cat)                                                       # (rows, 3n)
         y3 = y.reshape(B, N, 3 * n)

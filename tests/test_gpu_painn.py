@@ -431,3 +431,30 @@ def test_filter_table_is_rejected_when_the_filter_is_too_rough(pkg):
         msg.mlp_dist.layers[0].weight.mul_(1 / 300.0)
         msg.mlp_dist.layers[2].weight.mul_(1 / 30.0)
         assert msg.table_rows() in msg.TABLE_ROWS
+
+
+@pytest.mark.parametrize("rows,n", [(37, 20), (5, 300), (0, 8)])
+def test_update_elementwise_kernels_in_both_layouts(ops, rows, n):
+    """The two elementwise stages of Update.forward (archs/meanflow_painn8.py:63-75) against their formulas, with
+    lrv in the reference's (rows, 3n, 3) layout and component-major (rows, 3, 3n): same bits either way."""
+    g = torch.Generator().manual_seed(11)
+    lrv = torch.randn(rows, 3 * n, 3, generator=g)
+    x_a, y = torch.randn(rows, n, generator=g), torch.randn(rows, 3 * n, generator=g)
+    res = torch.randn(rows, n, 3, generator=g)
+    l, r, v = lrv[:, :n], lrv[:, n:2 * n], lrv[:, 2 * n:]
+    want_ip = (l.double() * r.double()).sum(-1)
+    want_cat = torch.cat([x_a.double(), r.double().norm(dim=-1)], dim=-1)
+    vs = v.double() * y[:, :n, None].double()
+    want_v = res.double() + vs / torch.sqrt(1.0 + (vs ** 2).sum(-1, keepdim=True))
+    outs = []
+    for lay in (lrv.cuda(), lrv.permute(0, 2, 1).contiguous().cuda()):
+        ip, cat = ops.painn_update_pre(lay, x_a.cuda())
+        out_v = ops.painn_update_vec(lay, y.cuda(), res.cuda())
+        torch.testing.assert_close(ip.cpu().double(), want_ip, rtol=1e-5, atol=1e-5)
+        torch.testing.assert_close(cat.cpu().double(), want_cat, rtol=1e-5, atol=1e-6)
+        torch.testing.assert_close(out_v.cpu().double(), want_v, rtol=1e-5, atol=1e-6)
+        outs.append((ip, cat, out_v))
+    for a, b in zip(*outs):
+        assert torch.equal(a, b)
+    with pytest.raises(RuntimeError, match="lrv must have shape"):
+        ops.painn_update_pre(torch.zeros(rows, 3 * n + 1, 3, device="cuda"), x_a.cuda())
