@@ -12,9 +12,6 @@ namespace {
 
 constexpr int kChunks = 64;   // partial sums per (box, group)
 
-__device__ __forceinline__ float4 ld4(const float* p) { return *reinterpret_cast<const float4*>(p); }
-__device__ __forceinline__ void st4(float* p, float4 v) { *reinterpret_cast<float4*>(p) = v; }
-
 __device__ __forceinline__ double block_sum(double v, double* lds) {
 #pragma unroll
     for (int d = kWave / 2; d > 0; d >>= 1) v += __shfl_xor(v, d);
@@ -142,10 +139,6 @@ __device__ __forceinline__ float lrv_at(const float* __restrict__ row, int n, in
     return COMP_MAJOR ? row[x * 3 * n + j] : row[j * 3 + x];
 }
 
-__device__ __forceinline__ float dot3(float a0, float a1, float a2, float b0, float b1, float b2) {
-    return fmaf(a2, b2, fmaf(a1, b1, a0 * b0));               // one fixed order for every variant of these kernels
-}
-
 template <bool COMP_MAJOR>
 __global__ void __launch_bounds__(256) painn_update_pre_kernel(const float* __restrict__ lrv, const float* __restrict__ x_a,
                                                                int n, float* __restrict__ ip, float* __restrict__ cat) {
@@ -156,38 +149,9 @@ __global__ void __launch_bounds__(256) painn_update_pre_kernel(const float* __re
     float l[3], rr[3];
 #pragma unroll
     for (int x = 0; x < 3; x++) { l[x] = lrv_at<COMP_MAJOR>(row, n, c, x); rr[x] = lrv_at<COMP_MAJOR>(row, n, n + c, x); }
-    ip[r * n + c] = dot3(l[0], l[1], l[2], rr[0], rr[1], rr[2]);
+    ip[r * n + c] = l[0] * rr[0] + l[1] * rr[1] + l[2] * rr[2];
     cat[r * 2 * n + c] = x_a[r * n + c];
-    cat[r * 2 * n + n + c] = sqrtf(dot3(rr[0], rr[1], rr[2], rr[0], rr[1], rr[2]));
-}
-
-// the same on component-major lrv with n % 4 == 0: a thread takes 4 channels of a row with 16-byte accesses
-__global__ void __launch_bounds__(256) painn_update_pre4_kernel(const float* __restrict__ lrv, const float* __restrict__ x_a,
-                                                                long rows, int n, float* __restrict__ ip,
-                                                                float* __restrict__ cat) {
-    const int n4 = n / 4;
-    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= rows * n4) return;
-    const long r = t / n4;
-    const int c = (int)(t - r * n4) * 4;
-    const float* row = lrv + r * 9 * n;
-    float4 l[3], q[3];
-#pragma unroll
-    for (int x = 0; x < 3; x++) { l[x] = ld4(row + x * 3 * n + c); q[x] = ld4(row + x * 3 * n + n + c); }
-    st4(ip + r * n + c, make_float4(dot3(l[0].x, l[1].x, l[2].x, q[0].x, q[1].x, q[2].x),
-                                    dot3(l[0].y, l[1].y, l[2].y, q[0].y, q[1].y, q[2].y),
-                                    dot3(l[0].z, l[1].z, l[2].z, q[0].z, q[1].z, q[2].z),
-                                    dot3(l[0].w, l[1].w, l[2].w, q[0].w, q[1].w, q[2].w)));
-    st4(cat + r * 2 * n + c, ld4(x_a + r * n + c));
-    st4(cat + r * 2 * n + n + c, make_float4(sqrtf(dot3(q[0].x, q[1].x, q[2].x, q[0].x, q[1].x, q[2].x)),
-                                             sqrtf(dot3(q[0].y, q[1].y, q[2].y, q[0].y, q[1].y, q[2].y)),
-                                             sqrtf(dot3(q[0].z, q[1].z, q[2].z, q[0].z, q[1].z, q[2].z)),
-                                             sqrtf(dot3(q[0].w, q[1].w, q[2].w, q[0].w, q[1].w, q[2].w))));
-}
-
-__device__ __forceinline__ void squash3(float a, float b, float d, float* o) {
-    const float inv = 1.0f / sqrtf(1.0f + dot3(a, b, d, a, b, d));
-    o[0] = a * inv; o[1] = b * inv; o[2] = d * inv;
+    cat[r * 2 * n + n + c] = sqrtf(rr[0] * rr[0] + rr[1] * rr[1] + rr[2] * rr[2]);
 }
 
 // PaiNN Update, vector output: v = lin_v(x_v) * y[0:n]; out = res_v + v / sqrt(1 + |v|^2), out (rows, n, 3)
@@ -200,40 +164,13 @@ __global__ void __launch_bounds__(256) painn_update_vec_kernel(const float* __re
     if (c >= n) return;
     const float* row = lrv + r * 9 * n;
     const float s = y[r * 3 * n + c];
-    float o[3];
-    squash3(lrv_at<COMP_MAJOR>(row, n, 2 * n + c, 0) * s, lrv_at<COMP_MAJOR>(row, n, 2 * n + c, 1) * s,
-            lrv_at<COMP_MAJOR>(row, n, 2 * n + c, 2) * s, o);
+    const float a = lrv_at<COMP_MAJOR>(row, n, 2 * n + c, 0) * s, b = lrv_at<COMP_MAJOR>(row, n, 2 * n + c, 1) * s,
+                d = lrv_at<COMP_MAJOR>(row, n, 2 * n + c, 2) * s;
+    const float inv = 1.0f / sqrtf(1.0f + (a * a + b * b + d * d));
+    float o0 = a * inv, o1 = b * inv, o2 = d * inv;
     const long t = r * n + c;
-    if (res_v) { o[0] += res_v[3 * t]; o[1] += res_v[3 * t + 1]; o[2] += res_v[3 * t + 2]; }
-    out_v[3 * t] = o[0]; out_v[3 * t + 1] = o[1]; out_v[3 * t + 2] = o[2];
-}
-
-__global__ void __launch_bounds__(256) painn_update_vec4_kernel(const float* __restrict__ lrv, const float* __restrict__ y,
-                                                                const float* __restrict__ res_v, long rows, int n,
-                                                                float* __restrict__ out_v) {
-    const int n4 = n / 4;
-    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (t >= rows * n4) return;
-    const long r = t / n4;
-    const int c = (int)(t - r * n4) * 4;
-    const float* row = lrv + r * 9 * n + 2 * n + c;
-    const float4 s = ld4(y + r * 3 * n + c);
-    const float4 v0 = ld4(row), v1 = ld4(row + 3 * n), v2 = ld4(row + 6 * n);
-    float o[12];                                              // 4 channels x 3 components, the order of out_v
-    squash3(v0.x * s.x, v1.x * s.x, v2.x * s.x, o);
-    squash3(v0.y * s.y, v1.y * s.y, v2.y * s.y, o + 3);
-    squash3(v0.z * s.z, v1.z * s.z, v2.z * s.z, o + 6);
-    squash3(v0.w * s.w, v1.w * s.w, v2.w * s.w, o + 9);
-    const long base = (r * n + c) * 3;
-    if (res_v) {
-        const float4 a = ld4(res_v + base), b = ld4(res_v + base + 4), d = ld4(res_v + base + 8);
-        const float rr[12] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w, d.x, d.y, d.z, d.w};
-#pragma unroll
-        for (int k = 0; k < 12; k++) o[k] += rr[k];
-    }
-    st4(out_v + base, make_float4(o[0], o[1], o[2], o[3]));
-    st4(out_v + base + 4, make_float4(o[4], o[5], o[6], o[7]));
-    st4(out_v + base + 8, make_float4(o[8], o[9], o[10], o[11]));
+    if (res_v) { o0 += res_v[3 * t]; o1 += res_v[3 * t + 1]; o2 += res_v[3 * t + 2]; }
+    out_v[3 * t] = o0; out_v[3 * t + 1] = o1; out_v[3 * t + 2] = o2;
 }
 
 // kinds: 1 sq_radial_encode of normed_sq_dist (archs/diffuser_atoms14.py:32-48)
@@ -319,14 +256,10 @@ int mg_painn_update_pre(const float* lrv, int lrv_comp_major, const float* x_a, 
     MG_REQUIRE(rows >= 0 && n >= 0, "mg_painn_update_pre: negative size");
     if (rows * n == 0) return MG_OK;
     MG_REQUIRE(lrv && x_a && ip && cat, "mg_painn_update_pre: null pointer");
-    MG_REQUIRE(rows <= 0x7fffffffL && rows * n < (1L << 38), "mg_painn_update_pre: too many rows");
+    MG_REQUIRE(rows <= 0x7fffffffL, "mg_painn_update_pre: more than 2^31 - 1 rows");
     const int threads = n >= 256 ? 256 : (int)ceil_div(n, kWave) * kWave;
     const dim3 grid((unsigned)rows, (unsigned)ceil_div(n, threads));
-    const auto aligned = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
-    if (lrv_comp_major && n % 4 == 0 && aligned(lrv) && aligned(x_a) && aligned(ip) && aligned(cat))
-        hipLaunchKernelGGL(painn_update_pre4_kernel, dim3((unsigned)ceil_div(rows * (n / 4), 256L)), dim3(256), 0,
-                           (hipStream_t)stream, lrv, x_a, rows, n, ip, cat);
-    else if (lrv_comp_major)
+    if (lrv_comp_major)
         hipLaunchKernelGGL(painn_update_pre_kernel<true>, grid, dim3(threads), 0, (hipStream_t)stream, lrv, x_a, n, ip, cat);
     else
         hipLaunchKernelGGL(painn_update_pre_kernel<false>, grid, dim3(threads), 0, (hipStream_t)stream, lrv, x_a, n, ip, cat);
@@ -338,14 +271,10 @@ int mg_painn_update_vec(const float* lrv, int lrv_comp_major, const float* y, co
     MG_REQUIRE(rows >= 0 && n >= 0, "mg_painn_update_vec: negative size");
     if (rows * n == 0) return MG_OK;
     MG_REQUIRE(lrv && y && out_v, "mg_painn_update_vec: null pointer");
-    MG_REQUIRE(rows <= 0x7fffffffL && rows * n < (1L << 38), "mg_painn_update_vec: too many rows");
+    MG_REQUIRE(rows <= 0x7fffffffL, "mg_painn_update_vec: more than 2^31 - 1 rows");
     const int threads = n >= 256 ? 256 : (int)ceil_div(n, kWave) * kWave;
     const dim3 grid((unsigned)rows, (unsigned)ceil_div(n, threads));
-    const auto aligned = [](const void* q) { return reinterpret_cast<uintptr_t>(q) % 16 == 0; };
-    if (lrv_comp_major && n % 4 == 0 && aligned(lrv) && aligned(y) && aligned(res_v) && aligned(out_v))
-        hipLaunchKernelGGL(painn_update_vec4_kernel, dim3((unsigned)ceil_div(rows * (n / 4), 256L)), dim3(256), 0,
-                           (hipStream_t)stream, lrv, y, res_v, rows, n, out_v);
-    else if (lrv_comp_major)
+    if (lrv_comp_major)
         hipLaunchKernelGGL(painn_update_vec_kernel<true>, grid, dim3(threads), 0, (hipStream_t)stream, lrv, y, res_v, n, out_v);
     else
         hipLaunchKernelGGL(painn_update_vec_kernel<false>, grid, dim3(threads), 0, (hipStream_t)stream, lrv, y, res_v, n, out_v);
