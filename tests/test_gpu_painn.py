@@ -433,7 +433,7 @@ def test_filter_table_is_rejected_when_the_filter_is_too_rough(pkg):
         assert msg.table_rows() in msg.TABLE_ROWS
 
 
-@pytest.mark.parametrize("rows,n", [(37, 20), (5, 300), (0, 8)])
+@pytest.mark.parametrize("rows,n", [(37, 20), (5, 300), (7, 10), (0, 8)])
 def test_update_elementwise_kernels_in_both_layouts(ops, rows, n):
     """The two elementwise stages of Update.forward (archs/meanflow_painn8.py:63-75) against their formulas, with
     lrv in the reference's (rows, 3n, 3) layout and component-major (rows, 3, 3n): same bits either way."""
