@@ -55,7 +55,13 @@ int mg_abi_version(void);
  *          prefix per box, as the reference's edgeCounts) and stats[4] =
  *          {E, max atoms in a cell, max degree, 1 if E overflowed int32};
  *   fill:  writes src[e] = b*nodes+i and dst[e] = b*nodes+j, rows ordered by
- *          (b,i); order inside a row is deterministic.
+ *          (b,i); order inside a row is deterministic.  n_edges is the CAPACITY of
+ *          src and dst in edges: an edge whose position row_ptr[row] + k is not
+ *          below n_edges is dropped (nothing is ever written past the arrays).  A
+ *          caller that sized the arrays without reading stats[0] back (no host
+ *          synchronisation, e.g. under stream capture) compares stats[0] with its
+ *          capacity afterwards: the first min(stats[0], n_edges) entries are the
+ *          complete rows, in order, that fit.
  * The reference's listmax / neighboursmax caps are not needed (exact-size CSR);
  * callers that want the reference's overflow errors compare stats[1], stats[2]
  * with their caps.

@@ -323,13 +323,20 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(const int* __r
 // again (it stages only the candidates' atom ids).  Windows larger than the LDS
 // tile (kCandCap candidates) fall back to recomputing in the fill pass.
 //
-// Minimum image: in an axis where the home cell does not touch the periodic
-// boundary and there are at least 5 cells, |w_i - w_j| < 2/5 box < box/2 for every
-// window candidate, so remainder(w_i - w_j, box) is the plain difference and the
-// conditional +-box is skipped (same bits, 40 % fewer instructions per pair).
+// Minimum image: a wrapped coordinate lies in [0, box] with BOTH ends possible
+// (remainderf(x - box/2, box) + box/2 gives exactly box for x = box, -box, 3 box, ...
+// and for x within half an ulp below box), and such an atom sits in cell 0 because
+// the cell index is taken modulo ndiv.  So cell 0 holds coordinates near 0 and
+// coordinates equal (or within rounding of) box; every other cell c holds
+// coordinates within rounding of [c, c+1) box/ndiv.  In an axis with at least 5
+// cells whose window (home - 1 .. home + 1) contains neither cell 0 nor, from the
+// other side, wraps around the box (home cell 2 .. ndiv-2), |w_i - w_j| < 2/5 box
+// < box/2 for every window candidate, remainder(w_i - w_j, box) is the plain
+// difference and the conditional +-box is skipped (same bits, 40 % fewer
+// instructions per pair).  Home cell 1 keeps the wrap: its window contains cell 0.
 template <bool FILL, int kCandCap>
 __global__ void __launch_bounds__(256) pairs_kernel(Grid g, Workspace w, const int* __restrict__ row_ptr,
-                                                    int* __restrict__ src, int* __restrict__ dst) {
+                                                    int* __restrict__ src, int* __restrict__ dst, int capacity) {
     constexpr int kWords = kCandCap / kWave;
     __shared__ float4 cand[FILL ? 1 : kCandCap];      // count pass: wrapped positions + atom id
     __shared__ int cand_idx[FILL ? kCandCap : 1];     // fill pass: atom ids only
@@ -386,9 +393,9 @@ __global__ void __launch_bounds__(256) pairs_kernel(Grid g, Workspace w, const i
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave, nwaves = blockDim.x / kWave;
     const float hx = 0.5f * g.bx, hy = 0.5f * g.by, hz = 0.5f * g.bz;
-    const bool wrap_x = g.nx < 5 || cx == 0 || cx == g.nx - 1;
-    const bool wrap_y = g.ny < 5 || cy == 0 || cy == g.ny - 1;
-    const bool wrap_z = g.nz < 5 || cz == 0 || cz == g.nz - 1;
+    const bool wrap_x = g.nx < 5 || cx <= 1 || cx == g.nx - 1;
+    const bool wrap_y = g.ny < 5 || cy <= 1 || cy == g.ny - 1;
+    const bool wrap_z = g.nz < 5 || cz <= 1 || cz == g.nz - 1;
     const unsigned long long lt_mask = (1ull << lane) - 1ull;
     const int node_base = b * g.nodes;
 
@@ -448,8 +455,10 @@ __global__ void __launch_bounds__(256) pairs_kernel(Grid g, Workspace w, const i
                 }
                 if ((mask >> lane) & 1ull) {
                     const int pos = out_base + running + __popcll(mask & lt_mask);
-                    src[pos] = row;
-                    dst[pos] = node_base + other_idx;
+                    if (pos < capacity) {      // src / dst hold `capacity` edges: the rest is dropped, never written
+                        src[pos] = row;
+                        dst[pos] = node_base + other_idx;
+                    }
                 }
                 running += __popcll(mask);
             }
@@ -625,10 +634,10 @@ int mg_neighbour_count(const float* x, int batch, int nodes, float cutoff, float
     hipLaunchKernelGGL(order_kernel, dim3(ablocks), dim3(256), 0, st, g, w);
     if (pairs_block_size(g) == 64)
         hipLaunchKernelGGL((pairs_kernel<false, kCandCapSparse>), dim3((unsigned)C), dim3(64), 0, st, g, w,
-                           (const int*)nullptr, (int*)nullptr, (int*)nullptr);
+                           (const int*)nullptr, (int*)nullptr, (int*)nullptr, 0);
     else
         hipLaunchKernelGGL((pairs_kernel<false, kCandCapDense>), dim3((unsigned)C), dim3(256), 0, st, g, w,
-                           (const int*)nullptr, (int*)nullptr, (int*)nullptr);
+                           (const int*)nullptr, (int*)nullptr, (int*)nullptr, 0);
     if (int s = run_scan(w.degree, A, row_ptr, w, stats + 0, stats + 2, stats + 3, st, nodes, edge_counts)) return s;
     return check_launch("mg_neighbour_count");
 }
@@ -649,10 +658,10 @@ int mg_neighbour_fill(const void* workspace, size_t workspace_bytes, int batch, 
                     w.bytes + 256);
     if (pairs_block_size(g) == 64)
         hipLaunchKernelGGL((pairs_kernel<true, kCandCapSparse>), dim3((unsigned)C), dim3(64), 0, (hipStream_t)stream,
-                           g, w, row_ptr, src, dst);
+                           g, w, row_ptr, src, dst, n_edges);
     else
         hipLaunchKernelGGL((pairs_kernel<true, kCandCapDense>), dim3((unsigned)C), dim3(256), 0, (hipStream_t)stream,
-                           g, w, row_ptr, src, dst);
+                           g, w, row_ptr, src, dst, n_edges);
     return check_launch("mg_neighbour_fill");
 }
 

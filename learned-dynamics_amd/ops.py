@@ -71,14 +71,26 @@ class NeighbourSearch:
         return self._host_stats
 
     def fill(self, n_edges=None):
+        """src, dst of exactly E edges (E read back from the device unless the caller passes the capacity to use:
+        edges beyond a capacity below E are dropped, never written)."""
         E = self.host_stats()[0] if n_edges is None else int(n_edges)
         dev = self.x.device
         with torch.cuda.device(dev):
             src = torch.empty(E, dtype=torch.int32, device=dev)
             dst = torch.empty(E, dtype=torch.int32, device=dev)
+        return self.fill_into(src, dst)
+
+    def fill_into(self, src, dst):
+        """Write the edges into caller-owned int32 arrays whose common length is the capacity; no host
+        synchronisation.  `stats[0]` (device) holds the true edge count for the caller to compare."""
+        _check_input(src, "src", torch.int32)
+        _check_input(dst, "dst", torch.int32)
+        if src.numel() != dst.numel():
+            raise RuntimeError("src and dst must have the same length")
+        with torch.cuda.device(self.x.device):
             L.check(_lib.mg_neighbour_fill(_p(self.workspace), self.workspace.numel(), self.batch, self.nodes,
-                                           self.cutoff, *self.box, _p(self.row_ptr), E, _p(src), _p(dst),
-                                           _stream()))
+                                           self.cutoff, *self.box, _p(self.row_ptr), int(src.numel()), _p(src),
+                                           _p(dst), _stream()))
         return src, dst
 
 

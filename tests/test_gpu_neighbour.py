@@ -67,6 +67,37 @@ def test_wrap_cells_bit_exact(ops):
     np.testing.assert_array_equal(cell.cpu().numpy(), cell_ref)
 
 
+@pytest.mark.parametrize("box,cutoff", __import__("neighbour_cases").FACE_BOXES)
+def test_atoms_on_the_box_faces(ops, box, cutoff):
+    """Wrapped coordinate exactly `box` (x = box, -box, 3 box, nextafter(box, 0)): the atom is filed in cell 0 and its
+    partners in cell 1 are reached only through the minimum image (neighbour_grid_kern.cu:39-48,75-80,124-139).  Cells
+    narrower than the cutoff (70/6, 86.861/6) and exact cells (55/5), all three axes, then a random box with 5 % of
+    the coordinates snapped to such values."""
+    import neighbour_cases as NC
+    for axis in range(3):
+        ref = _compare(ops, NC.hand_placed_line(box, cutoff, axis), cutoff, box)
+        E = set(zip(ref["src"].tolist(), ref["dst"].tolist()))
+        assert all((j, i) in E for i, j in E)
+    _compare(ops, NC.snapped_random(box, 6000, 3, seed=29), cutoff, box)
+    _compare(ops, NC.snapped_random(box, 300, 2, seed=31), cutoff, box)      # sparse: one-wave workgroups
+
+
+def test_fill_capacity_is_never_exceeded(ops):
+    """src / dst shorter than the edge count: nothing is written past them and the leading rows are intact."""
+    rng = np.random.default_rng(37)
+    x = torch.from_numpy((rng.random((2, 3000, 3)) * 30).astype(np.float32)).cuda()
+    search = ops.NeighbourSearch(x, 5.0, (30., 30., 30.))
+    E = search.host_stats()[0]
+    full_src, full_dst = search.fill()
+    cap = E // 2
+    guard = 4096
+    src = torch.full((cap + guard,), -7, dtype=torch.int32, device="cuda")
+    dst = torch.full((cap + guard,), -7, dtype=torch.int32, device="cuda")
+    search.fill_into(src[:cap], dst[:cap])
+    assert torch.equal(src[:cap], full_src[:cap]) and torch.equal(dst[:cap], full_dst[:cap])
+    assert torch.all(src[cap:] == -7) and torch.all(dst[cap:] == -7)
+
+
 def test_reference_test_shape(ops):
     """B=20, N=60, box (30.5,33.5,36.5), cutoff 7 (extensions/neighbour_grid/test.py:9-16)."""
     g = torch.Generator().manual_seed(0x947)

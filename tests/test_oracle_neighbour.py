@@ -147,3 +147,44 @@ def test_image_shift_reconstructs_displacement():
     flat = x.reshape(-1, 3).astype(np.float64)
     recon = flat[r["dst"]] - flat[r["src"]] - shift * np.array(box)
     assert np.all(np.sqrt((recon ** 2).sum(-1)) <= 5.0 + 1e-3)
+
+
+# ---- atoms exactly on the periodic faces (wrapped coordinate == box, filed in cell 0) ---------------------
+def test_two_atoms_across_the_face_are_neighbours():
+    """box 70, cutoff 6 (12 cells of 5.83): x = 70.0 wraps to exactly 70.0 and is filed in cell 0; its partner at
+    x = 5.9 sits in cell 1, 5.9 away through the face.  The reference applies the minimum image to every pair
+    (neighbour_grid_kern.cu:44-48,135), so both directions are listed."""
+    import neighbour_cases as NC
+    for axis in range(3):
+        x = np.zeros((1, 2, 3), dtype=np.float32)
+        x[0, 0, axis], x[0, 1, axis] = 5.9, 70.0
+        w, cell = ON.wrap_cells(x, 6.0, (70., 70., 70.))
+        assert w[0, 1, axis] == np.float32(70.0) and cell[0, 1] == 0 and cell[0, 0] != 0
+        for mode in (ON.MODE_CELLS, ON.MODE_BRUTE_WINDOW, ON.MODE_BRUTE_MINIMAGE):
+            r = ON.edges(x, 6.0, (70., 70., 70.), mode)
+            assert set(zip(r["src"].tolist(), r["dst"].tolist())) == {(0, 1), (1, 0)}
+    assert NC.face_values(70.)[0] == np.float32(70.)
+
+
+@pytest.mark.parametrize("box,cutoff", __import__("neighbour_cases").FACE_BOXES)
+def test_face_atoms_cell_walk_equals_brute_force(box, cutoff):
+    import neighbour_cases as NC
+    for axis in range(3):
+        x = NC.hand_placed_line(box, cutoff, axis)
+        w, cell = ON.wrap_cells(x, cutoff, box)
+        nd, _ = ON.ndiv(cutoff, box)
+        a = ON.edges(x, cutoff, box, ON.MODE_CELLS)
+        b = ON.edges(x, cutoff, box, ON.MODE_BRUTE_WINDOW)
+        np.testing.assert_array_equal(ON.sorted_triples(a["src"], a["dst"]), ON.sorted_triples(b["src"], b["dst"]))
+        # the case the test exists for is present: an edge from an atom whose axis cell is 1 to an atom whose wrapped
+        # coordinate is exactly `box`
+        stride = [nd[1] * nd[2], nd[2], 1][axis]
+        axis_cell = (cell[0] // stride) % nd[axis]
+        on_face = w[0, :, axis] == np.float32(box[axis])
+        assert np.any((axis_cell[a["src"]] == 1) & on_face[a["dst"]])
+        E = set(zip(a["src"].tolist(), a["dst"].tolist()))
+        assert all((j, i) in E for i, j in E)
+    x = NC.snapped_random(box, 1500, 2, seed=3)
+    a = ON.edges(x, cutoff, box, ON.MODE_CELLS)
+    b = ON.edges(x, cutoff, box, ON.MODE_BRUTE_WINDOW)
+    np.testing.assert_array_equal(ON.sorted_triples(a["src"], a["dst"]), ON.sorted_triples(b["src"], b["dst"]))
