@@ -166,9 +166,12 @@ def apply_Y(prods, Y):
     return tuple(out)
 
 
-def bee_messages(src, dst, batch, nodes, r_ij, x_a, x_v, x_d, w, r0):
-    """w: L0,L1,L2, Y (dict), enc_W (chan,8), enc_b (chan), mlp_a (dict)."""
-    enc = F.linear(radial_encode_8(r_ij, r0), w["enc_W"], w["enc_b"])      # (E, chan)
+def bee_messages(src, dst, batch, nodes, r_ij, x_a, x_v, x_d, w, r0, radial_dtype=None):
+    """w: L0,L1,L2, Y (dict), enc_W (chan,8), enc_b (chan), mlp_a (dict).  radial_dtype: evaluate radial_encode_8 in
+    that dtype and round once (its fp32 monomial form carries ~1e-3 of rounding noise of its own, which would
+    otherwise dominate every fp32 evaluation of this function)."""
+    enc8 = radial_encode_8(r_ij, r0) if radial_dtype is None else radial_encode_8(r_ij.to(radial_dtype), r0).to(r_ij.dtype)
+    enc = F.linear(enc8, w["enc_W"], w["enc_b"])      # (E, chan)
     rh = tens_sigmoid(1, r_ij * (7.0 / r0))
     phi_a = enc
     phi_v = enc[..., None] * rh[..., None, :]
@@ -184,10 +187,12 @@ def bee_messages(src, dst, batch, nodes, r_ij, x_a, x_v, x_d, w, r0):
             0.1 * edges_reduce_src(src, psi_d, batch, nodes))
 
 
-def displacement_tensors(src, batch, nodes, r_ij, w, r0):
+def displacement_tensors(src, batch, nodes, r_ij, w, r0, radial_dtype=None):
     """DisplacementTensors.forward (archs/diffuser_atoms15.py:216-225).  w: lin_W (dim_a, 8), lin_b (dim_a),
-    mlp (dict for mlp_leaky, dim_a -> dim_a), readout_v (dim_v, dim_a), readout_d (dim_d, dim_a)."""
-    rad = mlp_leaky(F.linear(radial_encode_8(r_ij, r0), w["lin_W"], w["lin_b"]), w["mlp"])     # (E, dim_a)
+    mlp (dict for mlp_leaky, dim_a -> dim_a), readout_v (dim_v, dim_a), readout_d (dim_d, dim_a).
+    radial_dtype: as in bee_messages."""
+    enc8 = radial_encode_8(r_ij, r0) if radial_dtype is None else radial_encode_8(r_ij.to(radial_dtype), r0).to(r_ij.dtype)
+    rad = mlp_leaky(F.linear(enc8, w["lin_W"], w["lin_b"]), w["mlp"])     # (E, dim_a)
     u = tens_sigmoid(1, r_ij * (7.0 / r0))
     phi_v = rad[..., None] * u[..., None, :]
     phi_d = rad[..., None, None] * u[..., None, None, :] * u[..., None, :, None]

@@ -10,8 +10,15 @@ import torch
 from oracle import layers as OL
 from oracle import neighbour as ON
 from oracle import products as OP
+from parity import assert_parity
 
 pytestmark = pytest.mark.gpu
+
+
+def _to(tree, dtype):
+    if isinstance(tree, dict):
+        return {k: _to(v, dtype) for k, v in tree.items()}
+    return tree.to(dtype)
 
 
 def _close(a, ref, rtol=1e-5, atol_scale=2e-6):
@@ -128,10 +135,12 @@ def test_messages_module(pkg, dims):
     w = {"L0": dd(msg.L0.W), "L1": dd(msg.L1.W), "L2": dd(msg.L2.W),
          "Y": {lab: dd(getattr(msg, f"Y_{lab}").W) for lab in OP.BEE_ORDER},
          "enc_W": dd(msg.lin_enc.weight), "enc_b": dd(msg.lin_enc.bias), "mlp_a": _mlp_leaky_weights(msg.mlp_a)}
-    ra, rv, rd = OL.bee_messages(src, dst, 2, 500, r_ref.double(), x_a.double(), x_v.double(), x_d.double(), w, r0)
-    _close(B_a, ra, atol_scale=5e-6)
-    _close(B_v, rv, atol_scale=5e-6)
-    _close(B_d, rd, atol_scale=5e-6)
+    r64 = OL.bee_messages(src, dst, 2, 500, r_ref.double(), x_a.double(), x_v.double(), x_d.double(), w, r0)
+    # the fp32 evaluation of the same math (radial polynomial rounded once from float64, as the kernel does: the
+    # reference's fp32 monomial form is ill-conditioned, see tests/test_oracle_layers.py)
+    r32 = OL.bee_messages(src, dst, 2, 500, r_ref, x_a, x_v, x_d, _to(w, torch.float32), r0, radial_dtype=torch.float64)
+    for k, (got, name) in enumerate(zip((B_a, B_v, B_d), "avd")):
+        assert_parity(got, r32[k], r64[k], f"Messages {dims} B_{name}")
 
 
 def test_self_tens_prods_module(pkg):
@@ -149,10 +158,10 @@ def test_self_tens_prods_module(pkg):
     w = {k: dd(getattr(mod, k).W) for k in ("L0", "R0", "L1", "R1", "L2", "R2")}
     w["Y"] = {lab: dd(getattr(mod, f"Y_{lab}").W) for lab in OP.BEE_ORDER}
     w.update(gn_a=dd(mod.gn_a.gamma), gn_v=dd(mod.gn_v.gamma), gn_d=dd(mod.gn_d.gamma))
-    ra, rv, rd = OL.self_tens_prods(x_a, x_v, x_d, w)
-    _close(y_a, ra, atol_scale=5e-6)
-    _close(y_v, rv, atol_scale=5e-6)
-    _close(y_d, rd, atol_scale=5e-6)
+    r32 = OL.self_tens_prods(x_a, x_v, x_d, w)
+    r64 = OL.self_tens_prods(x_a.double(), x_v.double(), x_d.double(), _to(w, torch.float64))
+    for k, (got, name) in enumerate(zip((y_a, y_v, y_d), "avd")):
+        assert_parity(got, r32[k], r64[k], f"SelfTensProds y_{name}")
 
 
 def test_state_dict_names_match_reference():
@@ -164,6 +173,38 @@ def test_state_dict_names_match_reference():
     names = set(bee.SelfTensProds(8, 8, 8, 8).state_dict().keys())
     for expect in ("L0.W", "R0.W", "L2.W", "R2.W", "Y_111.W", "gn_a.gamma", "gn_v.gamma", "gn_d.gamma"):
         assert expect in names, expect
+
+
+def denoiser_oracle(model, s, t, x0, x1, one_hot, box, r0, dtype):
+    """The Denoiser assembly (embed + time embed + read-in, blocks of Messages + SelfTensProds with residuals,
+    read-out with the meanflow factor) composed from the oracle's functions in `dtype`; the graph is the oracle's."""
+    B, N = x1.shape[:2]
+    dim_d = model.prods[0].L2.W.shape[1]
+    dd = lambda p: p.detach().cpu().to(dtype)
+    ref = ON.edges(x1.numpy(), r0, box)
+    src, dst = torch.from_numpy(ref["src"]).long(), torch.from_numpy(ref["dst"]).long()
+    r_ij = torch.from_numpy(ON.edge_vectors(x1.numpy(), ref["src"], ref["dst"], box)).to(dtype)
+    x_a = torch.nn.functional.linear(one_hot.to(dtype), dd(model.embed.weight), dd(model.embed.bias))
+    freqs = torch.exp(-torch.arange(32) / 31.0).to(dtype)
+    ph = torch.cat([t.to(dtype)[:, None] * freqs, (t - s).to(dtype)[:, None] * freqs], 1)
+    temb = torch.nn.functional.linear(torch.cat([torch.sin(ph), torch.cos(ph)], 1), dd(model.t_embed.lin1.weight),
+                                      dd(model.t_embed.lin1.bias))
+    x_a = x_a + temb[:, None]
+    x_v = OP.tensor_linear(1, dd(model.v_readin.W), (x1 - x0).to(dtype)[..., None, :])
+    x_d = torch.zeros(B, N, dim_d, 3, 3, dtype=dtype)
+    for msg, prod in zip(model.messages, model.prods):
+        w = {"L0": dd(msg.L0.W), "L1": dd(msg.L1.W), "L2": dd(msg.L2.W),
+             "Y": {lab: dd(getattr(msg, f"Y_{lab}").W) for lab in OP.BEE_ORDER},
+             "enc_W": dd(msg.lin_enc.weight), "enc_b": dd(msg.lin_enc.bias),
+             "mlp_a": _to(_mlp_leaky_weights(msg.mlp_a), dtype)}
+        d = OL.bee_messages(src, dst, B, N, r_ij, x_a, x_v, x_d, w, r0, radial_dtype=torch.float64)
+        x_a, x_v, x_d = x_a + d[0], x_v + d[1], x_d + d[2]
+        ws = {k: dd(getattr(prod, k).W) for k in ("L0", "R0", "L1", "R1", "L2", "R2")}
+        ws["Y"] = {lab: dd(getattr(prod, f"Y_{lab}").W) for lab in OP.BEE_ORDER}
+        ws.update(gn_a=dd(prod.gn_a.gamma), gn_v=dd(prod.gn_v.gamma), gn_d=dd(prod.gn_d.gamma))
+        d = OL.self_tens_prods(x_a, x_v, x_d, ws)
+        x_a, x_v, x_d = x_a + d[0], x_v + d[1], x_d + d[2]
+    return (1. - (t - s).to(dtype)[:, None, None]) * OP.tensor_linear(1, dd(model.readout.W), x_v).squeeze(-2)
 
 
 def test_denoiser_forward_matches_oracle_composition(pkg):
@@ -179,32 +220,9 @@ def test_denoiser_forward_matches_oracle_composition(pkg):
     s, t = torch.zeros(B), torch.rand(B)
     with torch.no_grad():
         v = model((s.cuda(), t.cuda()), x0.cuda(), x1.cuda(), one_hot.cuda(), box)
-    # oracle composition (float64)
-    dd = lambda p: p.detach().cpu().double()
-    ref = ON.edges(x1.numpy(), r0, box)
-    src, dst = torch.from_numpy(ref["src"]).long(), torch.from_numpy(ref["dst"]).long()
-    r_ij = torch.from_numpy(ON.edge_vectors(x1.numpy(), ref["src"], ref["dst"], box)).double()
-    x_a = torch.nn.functional.linear(one_hot.double(), dd(model.embed.weight), dd(model.embed.bias))
-    freqs = torch.exp(-torch.arange(32) / 31.0).double()
-    ph = torch.cat([t.double()[:, None] * freqs, (t - s).double()[:, None] * freqs], 1)
-    temb = torch.nn.functional.linear(torch.cat([torch.sin(ph), torch.cos(ph)], 1), dd(model.t_embed.lin1.weight),
-                                      dd(model.t_embed.lin1.bias))
-    x_a = x_a + temb[:, None]
-    x_v = OP.tensor_linear(1, dd(model.v_readin.W), (x1 - x0).double()[..., None, :])
-    x_d = torch.zeros(B, N, dim_d, 3, 3, dtype=torch.float64)
-    for msg, prod in zip(model.messages, model.prods):
-        w = {"L0": dd(msg.L0.W), "L1": dd(msg.L1.W), "L2": dd(msg.L2.W),
-             "Y": {lab: dd(getattr(msg, f"Y_{lab}").W) for lab in OP.BEE_ORDER},
-             "enc_W": dd(msg.lin_enc.weight), "enc_b": dd(msg.lin_enc.bias), "mlp_a": _mlp_leaky_weights(msg.mlp_a)}
-        d = OL.bee_messages(src, dst, B, N, r_ij, x_a, x_v, x_d, w, r0)
-        x_a, x_v, x_d = x_a + d[0], x_v + d[1], x_d + d[2]
-        ws = {k: dd(getattr(prod, k).W) for k in ("L0", "R0", "L1", "R1", "L2", "R2")}
-        ws["Y"] = {lab: dd(getattr(prod, f"Y_{lab}").W) for lab in OP.BEE_ORDER}
-        ws.update(gn_a=dd(prod.gn_a.gamma), gn_v=dd(prod.gn_v.gamma), gn_d=dd(prod.gn_d.gamma))
-        d = OL.self_tens_prods(x_a, x_v, x_d, ws)
-        x_a, x_v, x_d = x_a + d[0], x_v + d[1], x_d + d[2]
-    v_ref = (1. - (t - s).double()[:, None, None]) * OP.tensor_linear(1, dd(model.readout.W), x_v).squeeze(-2)
-    _close(v, v_ref, rtol=1e-4, atol_scale=2e-5)   # 2 blocks deep: fp32 rounding compounds through the group norms
+    v32 = denoiser_oracle(model, s, t, x0, x1, one_hot, box, r0, torch.float32)
+    v64 = denoiser_oracle(model, s, t, x0, x1, one_hot, box, r0, torch.float64)
+    assert_parity(v, v32, v64, "2-block denoiser v")
 
 
 @pytest.mark.parametrize("plus_identity", [False, True])
@@ -302,10 +320,10 @@ def test_self_tens_prods_module_fused_path(pkg):
     w = {k: dd(getattr(mod, k).W) for k in ("L0", "R0", "L1", "R1", "L2", "R2")}
     w["Y"] = {lab: dd(getattr(mod, f"Y_{lab}").W) for lab in OP.BEE_ORDER}
     w.update(gn_a=dd(mod.gn_a.gamma), gn_v=dd(mod.gn_v.gamma), gn_d=dd(mod.gn_d.gamma))
-    ra, rv, rd = OL.self_tens_prods(x_a, x_v, x_d, w)
-    _close(y_a, x_a + ra, atol_scale=5e-6)
-    _close(y_v, x_v + rv, atol_scale=5e-6)
-    _close(y_d, x_d + rd, atol_scale=5e-6)
+    r32 = OL.self_tens_prods(x_a, x_v, x_d, w)
+    r64 = OL.self_tens_prods(x_a.double(), x_v.double(), x_d.double(), _to(w, torch.float64))
+    for k, (got, x, name) in enumerate(zip((y_a, y_v, y_d), (x_a, x_v, x_d), "avd")):
+        assert_parity(got, x + r32[k], x.double() + r64[k], f"SelfTensProds (products + linears kernel) y_{name}")
 
 
 @pytest.mark.parametrize("chan,kind", [(64, "mixed"), (100, "short"), (7, "mixed"), (256, "long")])
@@ -358,7 +376,7 @@ def test_displacement_tensors_module(pkg, dims):
     dd = lambda t: t.detach().cpu().double()
     w = {"lin_W": dd(mod.mlp_radial[0].weight), "lin_b": dd(mod.mlp_radial[0].bias),
          "mlp": _mlp_leaky_weights(mod.mlp_radial[1]), "readout_v": dd(mod.readout_v.W), "readout_d": dd(mod.readout_d.W)}
-    ra, rv, rd = OL.displacement_tensors(src, 2, 500, r_ref.double(), w, r0)
-    _close(A_a, ra, atol_scale=5e-6)
-    _close(A_v, rv, atol_scale=5e-6)
-    _close(A_d, rd, atol_scale=5e-6)
+    r64 = OL.displacement_tensors(src, 2, 500, r_ref.double(), w, r0)
+    r32 = OL.displacement_tensors(src, 2, 500, r_ref, _to(w, torch.float32), r0, radial_dtype=torch.float64)
+    for k, (got, name) in enumerate(zip((A_a, A_v, A_d), "avd")):
+        assert_parity(got, r32[k], r64[k], f"DisplacementTensors {dims} A_{name}")

@@ -6,8 +6,13 @@ exact in fp32 (a quarter turn maps the cubic periodic box onto itself and only p
 coordinates), and the stated tolerance between the bf16-storage and the fp32-storage stacks."""
 import importlib
 
+import numpy as np
 import pytest
 import torch
+
+from oracle import layers as OL
+from oracle import neighbour as ON
+from parity import assert_parity
 
 pytestmark = pytest.mark.gpu
 
@@ -106,6 +111,79 @@ def test_configs2_painn_layer_is_equivariant_at_full_size(pkg):
     with torch.no_grad():
         out_t = run(pos + torch.tensor([8.0, -16.0, 24.0], device="cuda"), x_v)
     torch.testing.assert_close(out_t[5], a, rtol=1e-5, atol=2e-5 * float(a.abs().max()))
+
+
+def test_configs2_message_filter_grid_against_per_edge_mlp_and_oracle_at_full_size(pkg):
+    """The PaiNN Message of configs[2] (16 chains x 1024 beads, box 80, cutoff 8, n = 128, 16 radial functions) at
+    full size: the path that interpolates the filter from its grid against the path that evaluates the filter MLP
+    on every edge (both HIP), and 64 sampled nodes of both against the oracle's Message
+    (archs/meanflow_painn8.py:85-100) evaluated in float32 and float64 on exactly those nodes' edges."""
+    painn = importlib.import_module("learned-dynamics_amd.painn")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    n, r0, L, N = 128, 8.0, 80.0, 16384
+    box = (L, L, L)
+    torch.manual_seed(SEED + 3)
+    msg = painn.Message(r0, n, 16).cuda().eval()
+    pos = _polymer(16, 1024, L, SEED + 3)
+    g = torch.Generator().manual_seed(SEED + 4)
+    x_a = torch.randn(1, N, n, generator=g)
+    x_v = torch.randn(1, N, n, 3, generator=g) / 3 ** 0.5
+    with torch.no_grad():
+        graph, r_ij = gl.graph_setup(r0, box, pos.cuda(), neighbours_max=512, celllist_max=128)
+        assert msg.table_rows() == 512
+        ta, tv = msg(graph, x_a.cuda(), x_v.cuda(), r_ij)              # filter from the grid held in LDS
+        msg.use_table = False
+        ea, ev = msg(graph, x_a.cuda(), x_v.cuda(), r_ij)              # filter MLP on every edge
+    E = int(graph.src.numel())
+    assert 1_300_000 < E < 1_800_000
+    # oracle on the rows of 64 sampled nodes
+    sample = torch.randint(0, N, (64,), generator=g).sort().values.unique()
+    row_ptr = graph.row_ptr.cpu().long()
+    pick = torch.cat([torch.arange(int(row_ptr[i]), int(row_ptr[i + 1])) for i in sample.tolist()])
+    src, dst = graph.src.cpu()[pick], graph.dst.cpu()[pick]
+    r_ref = torch.from_numpy(ON.edge_vectors(pos.numpy(), src.numpy(), dst.numpy(), box))
+    assert torch.equal(r_ij.cpu()[pick], r_ref)
+    mlp_w = lambda m, dt: {k: getattr(m.layers[i], a).detach().cpu().to(dt) for k, i, a in
+                           (("W1", 0, "weight"), ("b1", 0, "bias"), ("W2", 2, "weight"), ("b2", 2, "bias"),
+                            ("W3", 4, "weight"), ("b3", 4, "bias"))}
+    refs = {}
+    for dt in (torch.float32, torch.float64):
+        ra, rv = OL.painn_message(src, dst, 1, N, x_a.to(dt), x_v.to(dt), r_ref.to(dt), mlp_w(msg.mlp_dist, dt),
+                                  mlp_w(msg.mlp_actv, dt), r0, n, 16)
+        refs[dt] = (ra[0, sample], rv[0, sample])
+    for name, (a, v) in (("filter grid", (ta, tv)), ("filter MLP per edge", (ea, ev))):
+        assert_parity(a[0, sample.cuda()], refs[torch.float32][0], refs[torch.float64][0], f"configs[2] Message, {name}, dx_a")
+        assert_parity(v[0, sample.cuda()], refs[torch.float32][1], refs[torch.float64][1], f"configs[2] Message, {name}, dx_v")
+    # the two HIP paths against each other on every node: the interpolation error bound of the grid (3e-6 of
+    # max |filter|, accepted per set of weights) times the sum over a row's edges, on top of the usual tolerance
+    torch.testing.assert_close(ta, ea, rtol=1e-5, atol=1e-6 + 4e-6 * float(ea.abs().max()))
+    torch.testing.assert_close(tv, ev, rtol=1e-5, atol=1e-6 + 4e-6 * float(ev.abs().max()))
+
+
+def test_configs3_one_system_of_the_full_batch_against_the_oracle(pkg):
+    """configs[3] at full size (32 systems x 2048 atoms, 8 blocks, 256 / 64 / 16 channels, chan 256): the forward of
+    the whole batch on the GPU, and the first system of it against the oracle's composition in float32 and float64
+    (systems are independent graphs and the group norms take their statistics per system)."""
+    den = importlib.import_module("learned-dynamics_amd.denoiser")
+    from test_gpu_bee_layers import denoiser_oracle
+    B, N, L, r0 = 32, 2048, 70.0, 6.0
+    box = (L, L, L)
+    torch.manual_seed(SEED + 4)
+    model = den.Denoiser(r0, dim_a=256, dim_v=64, dim_d=16, chan=256, blocks=8).cuda().eval()
+    g = torch.Generator().manual_seed(SEED + 4)
+    steps = torch.randn(B, N, 3, generator=g)
+    steps = 3.8 * steps / steps.norm(dim=-1, keepdim=True)
+    x1 = steps.cumsum(1) + torch.rand(B, 1, 3, generator=g) * L + torch.randn(B, N, 3, generator=g)
+    x0 = x1 + torch.randn(B, N, 3, generator=g)
+    one_hot = torch.nn.functional.one_hot(torch.randint(0, 20, (B, N), generator=g), 20).float()
+    s, t = torch.zeros(B), torch.rand(B, generator=g)
+    with torch.no_grad():
+        v = model((s.cuda(), t.cuda()), x0.cuda(), x1.cuda(), one_hot.cuda(), box)
+    first = lambda x: x[:1].contiguous()
+    args = (first(s), first(t), first(x0), first(x1), first(one_hot), box, r0)
+    v32 = denoiser_oracle(model, *args, torch.float32)
+    v64 = denoiser_oracle(model, *args, torch.float64)
+    assert_parity(v[:1], v32, v64, "configs[3] denoiser, system 0 of 32")
 
 
 def test_configs3_denoiser_is_equivariant_at_full_size(pkg):

@@ -11,8 +11,16 @@ import torch
 
 from oracle import layers as OL
 from oracle import neighbour as ON
+from parity import assert_parity
 
 pytestmark = pytest.mark.gpu
+
+
+def _to(tree, dtype):
+    """Weights (nested dicts of tensors) in another float dtype."""
+    if isinstance(tree, dict):
+        return {k: _to(v, dtype) for k, v in tree.items()}
+    return tree.to(dtype)
 
 
 def _close(a, ref, rtol=1e-5, atol_scale=1e-6):
@@ -192,10 +200,12 @@ def test_message_module(pkg, n, n_rbf):
     src, dst = graph.src.cpu(), graph.dst.cpu()
     r_ref = torch.from_numpy(ON.edge_vectors(pos.numpy(), src.numpy(), dst.numpy(), box))
     assert torch.equal(r_ij.cpu(), r_ref)
-    ra, rv = OL.painn_message(src, dst, 1, 1024, x_a, x_v, r_ref, _mlp_weights(msg.mlp_dist),
-                              _mlp_weights(msg.mlp_actv), 8.0, n, n_rbf)
-    _close(dx_a, ra, atol_scale=3e-6)
-    _close(dx_v, rv, atol_scale=3e-6)
+    wd, wa = _mlp_weights(msg.mlp_dist), _mlp_weights(msg.mlp_actv)
+    ra, rv = OL.painn_message(src, dst, 1, 1024, x_a, x_v, r_ref, wd, wa, 8.0, n, n_rbf)
+    D = torch.float64
+    ra64, rv64 = OL.painn_message(src, dst, 1, 1024, x_a.to(D), x_v.to(D), r_ref.to(D), _to(wd, D), _to(wa, D), 8.0, n, n_rbf)
+    assert_parity(dx_a, ra, ra64, f"painn Message n={n} dx_a")
+    assert_parity(dx_v, rv, rv64, f"painn Message n={n} dx_v")
 
 
 def test_update_and_block(pkg):
@@ -221,8 +231,13 @@ def test_update_and_block(pkg):
          "W_v": blk.update.lin_v.W.detach().cpu(), "mlp": _mlp_weights(blk.update.mlp),
          "gn_gamma": blk.update.gn.gamma.detach().cpu(), "gn_beta": blk.update.gn.beta.detach().cpu()}
     ua, uv = OL.painn_update(xa, xv, w, n)
-    _close(out[5], xa + ua, atol_scale=5e-6)
-    _close(out[6], xv + uv, atol_scale=5e-6)
+    D = torch.float64
+    da64, dv64 = OL.painn_message(src, dst, 2, 256, x_a.to(D), x_v.to(D), r_ref.to(D), _to(_mlp_weights(blk.message.mlp_dist), D),
+                                  _to(_mlp_weights(blk.message.mlp_actv), D), 8.0, n, 16)
+    xa64, xv64 = x_a.to(D) + da64, x_v.to(D) + dv64
+    ua64, uv64 = OL.painn_update(xa64, xv64, _to(w, D), n)
+    assert_parity(out[5], xa + ua, xa64 + ua64, "painn Block x_a")
+    assert_parity(out[6], xv + uv, xv64 + uv64, "painn Block x_v")
 
 
 def test_state_dict_names_match_reference():
