@@ -81,6 +81,15 @@ int mg_neighbour_fill(const void* workspace, size_t workspace_bytes, int batch, 
                       float cutoff, float box_x, float box_y, float box_z,
                       const int* row_ptr, int n_edges, int* src, int* dst, mg_stream_t stream);
 
+/* Both phases in one call for a caller that sizes src / dst itself (`capacity` edges each) and does not want to read
+ * the edge count back in between: get_edges (extensions/neighbour_grid/neighbour_grid.cpp:170-195) without its
+ * device->host copies.  Edges beyond the capacity are dropped as in mg_neighbour_fill; stats[0] holds the true count.
+ * Nothing in it synchronises or allocates, so the call can be recorded into a HIP graph. */
+int mg_neighbour_edges(const float* x /* (batch,nodes,3) */, int batch, int nodes, float cutoff,
+                       float box_x, float box_y, float box_z, void* workspace, size_t workspace_bytes,
+                       int* row_ptr /* batch*nodes+1 */, int* edge_counts /* batch */, int* stats /* 4 */,
+                       int capacity, int* src /* capacity */, int* dst /* capacity */, mg_stream_t stream);
+
 /* After mg_neighbour_count on the same workspace: order[k] = global id (b*nodes + i) of the k-th atom in
  * cell order (boxes, then cells x-major, then atom id).  Processing the rows of the fused edge kernels
  * in this order keeps the gathered neighbours of consecutive rows close together in time (cache

@@ -29,6 +29,7 @@ _SIGNATURES = {
     "mg_neighbour_workspace_bytes": [i32, i32, f32, f32, f32, f32, ctypes.POINTER(ctypes.c_size_t)],
     "mg_neighbour_count": [vp, i32, i32, f32, f32, f32, f32, vp, ctypes.c_size_t, vp, vp, vp, vp],
     "mg_neighbour_fill": [vp, ctypes.c_size_t, i32, i32, f32, f32, f32, f32, vp, i32, vp, vp, vp],
+    "mg_neighbour_edges": [vp, i32, i32, f32, f32, f32, f32, vp, ctypes.c_size_t, vp, vp, vp, i32, vp, vp, vp],
     "mg_neighbour_cell_order": [vp, ctypes.c_size_t, i32, i32, f32, f32, f32, f32, vp, vp],
     "mg_neighbour_wrap_cells": [vp, i32, i32, f32, f32, f32, f32, vp, vp, vp],
     "mg_neighbour_pad": [vp, vp, i32, i32, i32, vp, vp, vp],

@@ -665,6 +665,18 @@ int mg_neighbour_fill(const void* workspace, size_t workspace_bytes, int batch, 
     return check_launch("mg_neighbour_fill");
 }
 
+int mg_neighbour_edges(const float* x, int batch, int nodes, float cutoff, float box_x, float box_y, float box_z,
+                       void* workspace, size_t workspace_bytes, int* row_ptr, int* edge_counts, int* stats,
+                       int capacity, int* src, int* dst, mg_stream_t stream) {
+    MG_REQUIRE(capacity >= 0, "mg_neighbour_edges: negative capacity");
+    MG_REQUIRE(capacity == 0 || (src && dst), "mg_neighbour_edges: src / dst is null");
+    if (int s = mg_neighbour_count(x, batch, nodes, cutoff, box_x, box_y, box_z, workspace, workspace_bytes, row_ptr,
+                                   edge_counts, stats, stream))
+        return s;
+    return mg_neighbour_fill(workspace, workspace_bytes, batch, nodes, cutoff, box_x, box_y, box_z, row_ptr, capacity,
+                             src, dst, stream);
+}
+
 int mg_neighbour_cell_order(const void* workspace, size_t workspace_bytes, int batch, int nodes, float cutoff,
                             float box_x, float box_y, float box_z, int* order, mg_stream_t stream) {
     Grid g;

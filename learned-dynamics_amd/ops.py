@@ -104,6 +104,33 @@ class NeighbourSearch:
         return order
 
 
+def neighbour_edges(x, cutoff, box, capacity, out=None):
+    """Radius graph into arrays of `capacity` edges without reading the edge count back: one enqueue, no host
+    synchronisation (recordable into a HIP graph once `out` holds the buffers of an earlier call).
+    Returns dict(src, dst, row_ptr, edge_counts, stats, workspace); stats[0] (device) is the true edge count, edges
+    beyond the capacity are dropped."""
+    _check_input(x, "x")
+    if x.dim() != 3 or x.size(2) != 3:
+        raise RuntimeError("x must have shape (batch, nodes, 3)")
+    B, N = int(x.size(0)), int(x.size(1))
+    box = tuple(float(b) for b in box)
+    dev = x.device
+    with torch.cuda.device(dev):
+        if out is None:
+            nbytes = ctypes.c_size_t(0)
+            L.check(_lib.mg_neighbour_workspace_bytes(B, N, float(cutoff), *box, ctypes.byref(nbytes)))
+            out = dict(workspace=torch.empty(nbytes.value, dtype=torch.uint8, device=dev),
+                       row_ptr=torch.empty(B * N + 1, dtype=torch.int32, device=dev),
+                       edge_counts=torch.empty(B, dtype=torch.int32, device=dev),
+                       stats=torch.empty(4, dtype=torch.int32, device=dev),
+                       src=torch.empty(int(capacity), dtype=torch.int32, device=dev),
+                       dst=torch.empty(int(capacity), dtype=torch.int32, device=dev))
+        L.check(_lib.mg_neighbour_edges(_p(x), B, N, float(cutoff), *box, _p(out["workspace"]), out["workspace"].numel(),
+                                        _p(out["row_ptr"]), _p(out["edge_counts"]), _p(out["stats"]),
+                                        int(out["src"].numel()), _p(out["src"]), _p(out["dst"]), _stream()))
+    return out
+
+
 def _check_caps(search, listmax, neighboursmax):
     """The reference's overflow errors, in the reference's order
     (extensions/neighbour_grid/neighbour_grid_kern.cu:195-217)."""

@@ -98,6 +98,30 @@ def test_fill_capacity_is_never_exceeded(ops):
     assert torch.all(src[cap:] == -7) and torch.all(dst[cap:] == -7)
 
 
+def test_one_call_search_into_caller_sized_arrays(ops):
+    """mg_neighbour_edges: count + fill in one enqueue; with enough capacity the result is the two-phase result, with
+    less the leading edges; buffers can be reused for another set of positions."""
+    rng = np.random.default_rng(41)
+    box = (30., 30., 30.)
+    x = torch.from_numpy((rng.random((2, 3000, 3)) * 30).astype(np.float32)).cuda()
+    search = ops.NeighbourSearch(x, 5.0, box)
+    E = search.host_stats()[0]
+    src, dst = search.fill()
+    out = ops.neighbour_edges(x, 5.0, box, E + 100)
+    assert out["stats"].tolist() == list(search.host_stats())
+    assert torch.equal(out["src"][:E], src) and torch.equal(out["dst"][:E], dst)
+    assert torch.equal(out["row_ptr"], search.row_ptr) and torch.equal(out["edge_counts"], search.edge_counts)
+    x2 = torch.from_numpy((rng.random((2, 3000, 3)) * 30).astype(np.float32)).cuda()
+    ops.neighbour_edges(x2, 5.0, box, None, out=out)
+    s2 = ops.NeighbourSearch(x2, 5.0, box)
+    E2 = s2.host_stats()[0]
+    src2, dst2 = s2.fill()
+    n = min(E2, E + 100)
+    assert int(out["stats"][0]) == E2 and torch.equal(out["src"][:n], src2[:n]) and torch.equal(out["dst"][:n], dst2[:n])
+    small = ops.neighbour_edges(x, 5.0, box, E // 3)
+    assert int(small["stats"][0]) == E and torch.equal(small["src"], src[:E // 3]) and torch.equal(small["dst"], dst[:E // 3])
+
+
 def test_reference_test_shape(ops):
     """B=20, N=60, box (30.5,33.5,36.5), cutoff 7 (extensions/neighbour_grid/test.py:9-16)."""
     g = torch.Generator().manual_seed(0x947)
