@@ -90,6 +90,19 @@ int mg_neighbour_edges(const float* x /* (batch,nodes,3) */, int batch, int node
                        int* row_ptr /* batch*nodes+1 */, int* edge_counts /* batch */, int* stats /* 4 */,
                        int capacity, int* src /* capacity */, int* dst /* capacity */, mg_stream_t stream);
 
+/* mg_neighbour_edges without a workspace argument, for callers that cannot allocate one (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid allocation).  No counterpart in the reference.  The workspace
+ * is a 32 MiB buffer built into the library (one per GPU, held until the process ends); a search that needs more
+ * (about 176 bytes per atom: more than roughly 180 000 atoms over all boxes) is refused with MG_ERR_WORKSPACE and
+ * a message.  The call allocates and frees nothing and synchronises nothing; inputs and outputs are the caller's.
+ * All calls on one GPU share the buffer: calls that overlap in time on the same GPU (two streams, two threads)
+ * race, calls ordered on one stream do not.  The first call on a device looks the buffer's address up
+ * (hipGetSymbolAddress): make that call outside stream capture. */
+int mg_neighbour_edges_static(const float* x /* (batch,nodes,3) */, int batch, int nodes, float cutoff,
+                              float box_x, float box_y, float box_z,
+                              int* row_ptr /* batch*nodes+1 */, int* edge_counts /* batch */, int* stats /* 4 */,
+                              int capacity, int* src /* capacity */, int* dst /* capacity */, mg_stream_t stream);
+
 /* After mg_neighbour_count on the same workspace: order[k] = global id (b*nodes + i) of the k-th atom in
  * cell order (boxes, then cells x-major, then atom id).  Processing the rows of the fused edge kernels
  * in this order keeps the gathered neighbours of consecutive rows close together in time (cache

@@ -30,6 +30,7 @@ _SIGNATURES = {
     "mg_neighbour_count": [vp, i32, i32, f32, f32, f32, f32, vp, ctypes.c_size_t, vp, vp, vp, vp],
     "mg_neighbour_fill": [vp, ctypes.c_size_t, i32, i32, f32, f32, f32, f32, vp, i32, vp, vp, vp],
     "mg_neighbour_edges": [vp, i32, i32, f32, f32, f32, f32, vp, ctypes.c_size_t, vp, vp, vp, i32, vp, vp, vp],
+    "mg_neighbour_edges_static": [vp, i32, i32, f32, f32, f32, f32, vp, vp, vp, i32, vp, vp, vp],
     "mg_neighbour_cell_order": [vp, ctypes.c_size_t, i32, i32, f32, f32, f32, f32, vp, vp],
     "mg_neighbour_wrap_cells": [vp, i32, i32, f32, f32, f32, f32, vp, vp, vp],
     "mg_neighbour_pad": [vp, vp, i32, i32, i32, vp, vp, vp],

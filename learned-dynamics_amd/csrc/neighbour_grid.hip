@@ -24,9 +24,35 @@
 //   when box/cutoff is not an integer the cells are narrower than the cutoff and
 //   pairs two cells apart are not listed.
 #include "common.hpp"
+#include <mutex>
 
 namespace mg {
 namespace {
+
+// Built-in workspace of mg_neighbour_edges_static, for callers that cannot allocate one.  One copy per GPU, held
+// from the moment the library is loaded until the process ends.  Host code never passes `scratch` itself anywhere:
+// the name is a host-side handle, the device address comes from hipGetSymbolAddress (scratch_of_current_device).
+constexpr size_t kScratchBytes = size_t(32) << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+constexpr int kMaxDevices = 64;
+void* g_scratch_ptr[kMaxDevices] = {nullptr};
+std::mutex g_scratch_mutex;
+
+// Device address of this GPU's copy of `scratch`; looked up once per device, with that device current.
+int scratch_of_current_device(void** out) {
+    int dev = -1;
+    MG_HIP(hipGetDevice(&dev));
+    MG_REQUIRE(dev >= 0 && dev < kMaxDevices, "device index %d out of range", dev);
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void* p = nullptr;
+        MG_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+        MG_REQUIRE(p != nullptr, "hipGetSymbolAddress returned a null address for the built-in workspace");
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return MG_OK;
+}
 
 constexpr int kCandCapDense = 1024;   // candidates staged in LDS per home cell (16 KB), 4-wave workgroups
 constexpr int kCandCapSparse = 256;   // sparse boxes: 1-wave workgroups, 4 KB
@@ -675,6 +701,24 @@ int mg_neighbour_edges(const float* x, int batch, int nodes, float cutoff, float
         return s;
     return mg_neighbour_fill(workspace, workspace_bytes, batch, nodes, cutoff, box_x, box_y, box_z, row_ptr, capacity,
                              src, dst, stream);
+}
+
+int mg_neighbour_edges_static(const float* x, int batch, int nodes, float cutoff, float box_x, float box_y,
+                              float box_z, int* row_ptr, int* edge_counts, int* stats, int capacity, int* src,
+                              int* dst, mg_stream_t stream) {
+    size_t need = 0;
+    if (int s = mg_neighbour_workspace_bytes(batch, nodes, cutoff, box_x, box_y, box_z, &need)) return s;
+    if (need > kScratchBytes)
+        return fail(MG_ERR_WORKSPACE,
+                    "mg_neighbour_edges_static: this search needs %zu bytes of workspace, the built-in one holds %zu "
+                    "(about %ld atoms in total); use mg_neighbour_edges with a workspace of your own",
+                    need, kScratchBytes, (long)(kScratchBytes / 180));
+    void* ws = nullptr;
+    if (int s = scratch_of_current_device(&ws)) return s;
+    // every array of the workspace that must start at zero (the cell histogram) is cleared by a kernel inside
+    // mg_neighbour_count; everything else is written before it is read, so what the previous call left is harmless
+    return mg_neighbour_edges(x, batch, nodes, cutoff, box_x, box_y, box_z, ws, kScratchBytes, row_ptr, edge_counts,
+                              stats, capacity, src, dst, stream);
 }
 
 int mg_neighbour_cell_order(const void* workspace, size_t workspace_bytes, int batch, int nodes, float cutoff,
