@@ -271,32 +271,38 @@ def bench_painn_layer(torch, args):
                       if sliced else
                       "painn_message_kernel<table> (per edge: 4 rows of the %d-row filter grid interpolated, node rows "
                       "gathered, products, sums over the edges of a node)" % rows)
-            roofline = {"kernel": kernel, "bound": "hbm", "achieved": hbm_bytes / t_table / 1e9, "peak": PEAK_HBM_GBS,
-                        "unit": "GB/s", "frac": hbm_bytes / t_table / 1e9 / PEAK_HBM_GBS,
+            roofline = {"kernel": kernel, "bound": "fp32_vector", "achieved": flop / t_table / 1e12,
+                        "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": flop / t_table / 1e12 / PEAK_FP32_MFMA_TFLOPS,
                         "traffic": measured_traffic("painn_table_message_lds_kernel" if sliced else "painn_message_kernel<true>"),
-                        "bytes_per_launch": hbm_bytes, "ms": t_table * 1e3,
+                        "flop_per_launch": flop, "ms": t_table * 1e3,
+                        "peak_note": "157.3 TFLOP/s is the published fp32 vector peak and needs packed fp32 instructions, "
+                                     "which are compiled out here; 78.65 TFLOP/s is reachable without them",
+                        "hbm": {"bytes_per_launch": hbm_bytes, "achieved": hbm_bytes / t_table / 1e9, "peak": PEAK_HBM_GBS,
+                                "unit": "GB/s", "frac": hbm_bytes / t_table / 1e9 / PEAK_HBM_GBS},
                         "cache_to_cu": {"bytes_per_launch": cache_bytes, "achieved": cache_bytes / t_table / 1e9,
                                         "peak": l1_fill_peak, "unit": "GB/s",
                                         "frac": cache_bytes / t_table / 1e9 / l1_fill_peak},
                         "lds_reads": {"bytes_per_launch": grid_bytes if sliced else 0,
                                       "achieved": (grid_bytes if sliced else 0) / t_table / 1e9, "unit": "GB/s"},
-                        "fp32_vector": {"flop_per_launch": flop, "achieved": flop / t_table / 1e12, "unit": "TFLOP/s",
-                                        "peak": PEAK_FP32_MFMA_TFLOPS / 2,
-                                        "frac": flop / t_table / 1e12 / (PEAK_FP32_MFMA_TFLOPS / 2)},
-                        "note": "every operand of the kernel is cache resident (node-sized arrays and the filter grid), "
-                                "so its algorithmic HBM bytes are 20x fewer than those of the kernel that streams a "
-                                "stored filter (roofline_hbm) and the HBM fraction is small by construction; what "
-                                "bounds it is vector arithmetic (fp32_vector, without packed instructions) and the "
-                                "gathers of node rows from L2 (cache_to_cu, against 64 B per clock per CU)",
+                        "note": "every operand of the kernel is cache resident (node-sized arrays and the filter grid): "
+                                "the kernel is bound by vector arithmetic and by the gathers of node rows from L2 "
+                                "(cache_to_cu, against 64 B per clock per CU), not by HBM (hbm)",
                         "filter_mlp_per_edge_path": roofline}
         del actv
 
     cpu = None
     if not args.no_cpu:
         cpu = cpu_painn_layer(torch, block, n, n_rbf, r0, box_len, seed)
+    per_edge_ms = breakdown.get("layer_ms_with_filter_mlp_per_edge")
     result = {
         "metric": "message-passing edges/sec per layer", "value": E / sec, "unit": "edges/s",
-        "ms_per_step": sec * 1e3, "dtype": "f32",
+        "ms_per_step": sec * 1e3,
+        "dtype": "f32 storage and accumulation; products of the wide linears as split-fp16 MFMA (2 x 11 significand bits)",
+        "value_note": "the filter MLP of the layer is evaluated on a 512-point grid over the edge length and "
+                      "interpolated per edge (accepted per set of weights at 3e-6 of max |filter|); "
+                      "value_filter_mlp_per_edge is the same layer with the MLP evaluated on every edge",
+        "value_filter_mlp_per_edge": None if per_edge_ms is None else E / (per_edge_ms * 1e-3),
+        "ms_per_step_filter_mlp_per_edge": per_edge_ms,
         "config": {"workload": "BASELINE configs[2]: one PaiNN layer (Message + Update, residuals), 16 chains x 1024 "
                                "beads, box 80 A, cutoff 8 A, n=128 scalar+128 vector channels, 16 radial functions",
                    "edges": E, "atoms": N, "graph": "prebuilt (positions fixed); build time reported in breakdown"},
@@ -481,18 +487,21 @@ def edge_kernel_roofline(torch, msg, graph, r_ij, rows, bf16=False):
     t = event_time(torch, fn, 10)
     E = int(graph.src.numel())
     w = 2 if bf16 else 4
-    nbytes = E * (3 * chan * w + 4 + 32 + 12) + rows * (13 + 60) * chan * w
+    # algorithmic bytes: the 13 node components read once and the 63 per-channel product sums written once per node,
+    # plus index and edge vector per edge.  The three scalar products the kernel also stores per edge (the input of the
+    # per-edge MLP) are not compulsory traffic and are listed on their own.
+    nbytes = rows * (13 + 63) * chan * w + E * 16
+    p0_bytes = E * 3 * chan * w
     return {"kernel": "bee_message_kernel (gathers, 13 products, edge sums; one Messages layer)", "bound": "hbm",
             "achieved": nbytes / t / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": nbytes / t / 1e9 / PEAK_HBM_GBS,
             "traffic": None, "bytes_per_launch": nbytes, "ms": t * 1e3,
+            "per_edge_scalar_products_stored_bytes": p0_bytes,
+            "frac_counting_the_stored_scalar_products": (nbytes + p0_bytes) / t / 1e9 / PEAK_HBM_GBS,
             # the 13 products are 167 flop per (edge, channel), the 60 running sums another 60
             "fp32_vector_tflops": E * chan * 227 / t / 1e12,
-            # the vector rate without packed fp32 instructions (compiled out here) is half the published 157.3 TFLOP/s
-            "fp32_vector_frac_of_peak": E * chan * 227 / t / 1e12 / (PEAK_FP32_MFMA_TFLOPS / 2),
-            "note": "gathered node rows are served by L2 and counted once per node; with ~90 edges per node "
-                    "(configs[4]) the kernel is bound by its fp32 vector arithmetic (packed fp32 instructions "
-                    "are compiled out, which halves the vector peak), with ~16 (configs[3]) by L2 gather latency "
-                    "and its 7 GB of outputs"}
+            "fp32_vector_frac_of_peak": E * chan * 227 / t / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+            "note": "gathered node rows are served by L2 and counted once per node; the fp32 vector peak is the "
+                    "published 157.3 TFLOP/s, which needs packed fp32 instructions (compiled out here: 78.65 reachable)"}
 
 
 def single_system_latency(torch, model, dev, box, r0, atoms):
@@ -548,13 +557,13 @@ def bench_denoiser(torch, args, with_cpu=True):
                                   "(assembled from reference modules), 32 systems x 2048 atoms, box 70 A, cutoff 6 A, "
                                   "256 scalar + 64 vector + 16 rank-2 channels, chan 256, graph rebuilt every forward",
                       "edges": E, "atoms": B * N},
-           "roofline_hbm": edge_roof, "single_system": single}
+           "roofline": edge_roof, "single_system": single}
     if with_cpu:
         out["cpu_baseline"] = cpu_denoiser_block(torch, model, x1[:1], r0, box, dims)
     return out
 
 
-def bench_stress(torch, args):
+def bench_stress(torch, args, with_cpu=True):
     """BASELINE configs[4]: 65536 atoms uniform in a periodic cube at 0.1 atoms/A^3, cutoff 6 A,
     4 x [Messages + SelfTensProds] with 128 channels per rank, features stored as bf16 with fp32
     accumulation, neighbour rebuild inside the step.  The fp32-storage path on the same problem is
@@ -600,15 +609,73 @@ def bench_stress(torch, args):
         graph, r_ij = gl.graph_setup(r0, box, pos, neighbours_max=256, celllist_max=64)
         edge_roof = edge_kernel_roofline(torch, msgs[0], graph, r_ij, N, bf16=True)
     E = edges[0]
+    cpu = cpu_stress_layer(torch, msgs[0], prods[0], r0, C, seed) if with_cpu else None
     return {"metric": "message-passing edges/sec per layer", "value": E * layers / sec16, "unit": "edges/s",
+            "roofline": edge_roof, "cpu_baseline": cpu,
             "ms_per_step": sec16 * 1e3, "dtype": "bf16 storage, f32 accumulate",
             "config": {"workload": "BASELINE configs[4]: 65536 atoms, density 0.1/A^3, cutoff 6 A, "
                                    "4 x [Messages + SelfTensProds], 128 channels per rank, bf16 storage, "
                                    "neighbour rebuild in the step",
                        "edges": E, "atoms": N, "layers": layers, "atoms_per_s": N / sec16},
-            "roofline_hbm": edge_roof, "max_abs_diff_vs_fp32_storage_over_scale": rel,
+            "max_abs_diff_vs_fp32_storage_over_scale": rel,
             "fp32_storage": None if sec32 is None else {"value": E * layers / sec32, "unit": "edges/s",
                                                         "ms_per_step": sec32 * 1e3}}
+
+
+def _bee_weights(msg, prod):
+    """Weights of one Messages + SelfTensProds pair as the oracle takes them."""
+    from oracle import products as OP
+    dd = lambda p: p.detach().cpu()
+    Lm = msg.mlp_a.layers
+    w = {"L0": dd(msg.L0.W), "L1": dd(msg.L1.W), "L2": dd(msg.L2.W),
+         "Y": {lab: dd(getattr(msg, f"Y_{lab}").W) for lab in OP.BEE_ORDER},
+         "enc_W": dd(msg.lin_enc.weight), "enc_b": dd(msg.lin_enc.bias),
+         "mlp_a": {"W_direct": dd(msg.mlp_a.lin_direct.weight), "W1": dd(Lm[0].weight), "b1": dd(Lm[0].bias),
+                   "W2": dd(Lm[2].weight), "b2": dd(Lm[2].bias), "W3": dd(Lm[4].weight), "b3": dd(Lm[4].bias)}}
+    ws = {k: dd(getattr(prod, k).W) for k in ("L0", "R0", "L1", "R1", "L2", "R2")}
+    ws["Y"] = {lab: dd(getattr(prod, f"Y_{lab}").W) for lab in OP.BEE_ORDER}
+    ws.update(gn_a=dd(prod.gn_a.gamma), gn_v=dd(prod.gn_v.gamma), gn_d=dd(prod.gn_d.gamma))
+    return w, ws
+
+
+def cpu_stress_layer(torch, msg, prod, r0, C, seed):
+    """Oracle (fp32 PyTorch CPU port of the reference math): ONE layer (Messages + SelfTensProds, 128 channels per
+    rank) on 1024 atoms at the density of configs[4] (1/64 of its atoms; the per-edge rank-2 tensors of the
+    reference formulation, 13 of size edges x 128 x 9, do not fit the host for more)."""
+    from oracle import layers as OL
+    from oracle import neighbour as ON
+    cores = min(os.cpu_count() or 1, 16)
+    torch.set_num_threads(cores)
+    N = 1024
+    L = (N / 0.1) ** (1.0 / 3.0)
+    box = (L, L, L)
+    g = torch.Generator().manual_seed(seed + 7)
+    pos = (torch.rand(1, N, 3, generator=g) * L).contiguous()
+    ref = ON.edges(pos.numpy(), r0, box)
+    src, dst = torch.from_numpy(ref["src"]).long(), torch.from_numpy(ref["dst"]).long()
+    r_ij = torch.from_numpy(ON.edge_vectors(pos.numpy(), ref["src"], ref["dst"], box))
+    w, ws = _bee_weights(msg, prod)
+    x_a = torch.randn(1, N, C, generator=g)
+    x_v = torch.randn(1, N, C, 3, generator=g) / 3 ** 0.5
+    x_d = torch.randn(1, N, C, 3, 3, generator=g) / 3.0
+
+    def layer():
+        d = OL.bee_messages(src, dst, 1, N, r_ij, x_a, x_v, x_d, w, r0)
+        return OL.self_tens_prods(x_a + d[0], x_v + d[1], x_d + d[2], ws)
+
+    with torch.no_grad():
+        layer()
+        times = []
+        t_all = time.perf_counter()
+        while len(times) < 3 or (time.perf_counter() - t_all < 10 and len(times) < 10):
+            t0 = time.perf_counter()
+            layer()
+            times.append(time.perf_counter() - t0)
+    times.sort()
+    med = times[len(times) // 2]
+    return {"value": len(src) / med, "unit": "edges/s", "cores": cores, "kind": "port",
+            "sample": f"{N} atoms at 0.1 / A^3 ({len(src)} edges; 1/64 of the atoms), one of the 4 layers, fp32 storage, "
+                      f"median of {len(times)} runs, PyTorch CPU fp32; neighbour search not included"}
 
 
 def cpu_denoiser_block(torch, model, x1, r0, box, dims):
@@ -680,17 +747,19 @@ def main():
     if args.workload == "painn_layer":
         res = bench_painn_layer(torch, args)
         if not args.no_extras:
-            small = argparse.Namespace(steps=10, warmup=3)
+            small = argparse.Namespace(steps=20, warmup=10)
             nb = bench_neighbour(torch, small, with_cpu=not args.no_cpu)
-            dn = bench_denoiser(torch, argparse.Namespace(steps=3, warmup=1), with_cpu=not args.no_cpu)
+            dn = bench_denoiser(torch, argparse.Namespace(steps=20, warmup=5), with_cpu=not args.no_cpu)
+            st = bench_stress(torch, argparse.Namespace(steps=20, warmup=5, no_comparisons=False), with_cpu=not args.no_cpu)
             res["other_workloads"] = {"denoiser_forward_configs[3]": dn, "neighbour_search_configs[1]": nb,
-                                      "tensor_products_configs[0]": bench_products(torch, small)}
+                                      "tensor_products_configs[0]": bench_products(torch, small),
+                                      "stress_configs[4]": st}
     elif args.workload == "neighbour":
         res = bench_neighbour(torch, args, with_cpu=not args.no_cpu)
     elif args.workload == "denoiser":
         res = bench_denoiser(torch, args, with_cpu=not args.no_cpu)
     elif args.workload == "stress":
-        res = bench_stress(torch, args)
+        res = bench_stress(torch, args, with_cpu=not args.no_cpu)
     elif args.workload == "polymer":
         res = bench_polymer(torch, args, with_cpu=not args.no_cpu)
     else:
