@@ -306,11 +306,17 @@ int mg_painn_table_message(const int* row_ptr, const int* dst, const int* node_o
                            float* out_v, mg_stream_t stream);
 /* mg_painn_table_message with the table in LDS: table_rows <= 512, n % 16 == 0.  A workgroup keeps the filter columns of
  * one slice of 16 channels for every table row in LDS, so only node rows are gathered through the caches.
+ * What an edge contributes apart from its node rows (its first table row, the four interpolation weights, the
+ * direction r / sqrt(epsilon + |r|^2)) is written once per edge by mg_painn_edge_records into `records` (n_edges x 8
+ * floats, 16-byte aligned) and read by every slice.
  * actv_sliced (n_nodes, n / 16, 4, 16): actv with its columns regrouped slice by slice, element (s, k, c) = column
- * k n + 16 s + c of mg_painn_message's actv.  Same results as mg_painn_table_message up to fp32 summation order. */
-int mg_painn_table_message_sliced(const int* row_ptr, const int* dst, int n_nodes, long n_edges, const float* r_ij,
-                                  const float* table, int table_rows, float period, const float* actv_sliced,
-                                  const float* x_v, int n, float epsilon, const float* res_a, const float* res_v,
+ * k n + 16 s + c of mg_painn_message's actv.  node_order as in mg_painn_message.  Same results as
+ * mg_painn_table_message up to fp32 summation order. */
+int mg_painn_edge_records(const float* r_ij /* (E,3) */, long n_edges, int table_rows, float period, float epsilon,
+                          float* records /* (E,8) */, mg_stream_t stream);
+int mg_painn_table_message_sliced(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
+                                  const float* records, const float* table, int table_rows, const float* actv_sliced,
+                                  const float* x_v, int n, const float* res_a, const float* res_v,
                                   float* out_a, float* out_v, mg_stream_t stream);
 /* Message.forward after the two MLPs (archs/meanflow_painn8.py:91-100), fused over CSR rows:
  *   P = filt[e] * actv[dst[e]];  u = r_ij[e] / sqrt(epsilon + |r_ij[e]|^2);  v = x_v[dst[e]]

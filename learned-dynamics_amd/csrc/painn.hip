@@ -221,103 +221,146 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(TABLE 
 // each, so a wave takes 16 edges of its node per step and only the node rows (actv, x_v) come through the vector
 // caches: 3.5 KB per edge instead of 11.5 KB.  actv is expected slice-major, (node, n / 16, 4, 16), so that a
 // slice's 64 values are two whole cache lines; x_v (node, n, 3) already has a slice's 48 values contiguous.
+//
+// What an edge contributes besides its node rows depends on the edge alone, not on the channel: the first of its four
+// grid rows, the four interpolation weights and the direction.  A pass over the edges writes them once as a 32-byte
+// record (painn_edge_records_kernel); the 8 slices x 4 lanes that work on an edge read the record instead of
+// repeating the square root, floor, weight polynomials and reciprocal square root (a fifth of the loop's vector
+// instructions before).  The grid in LDS carries three extra rows (copies of rows 0..2) behind the last one, so the
+// four rows of an edge are always consecutive: one address per edge, the rest are immediates.
 // LDS rows are padded to 68 floats so that the rows different edges read start in different banks.
 constexpr int kSliceChan = 16, kSliceCols = 4 * kSliceChan, kSliceRowF = kSliceCols + 4, kSliceMaxRows = 512;
+constexpr int kSliceExtraRows = 3;
+
+// rec[2e] = (float offset of the first grid row in LDS as int bits, w0, w1, w2), rec[2e+1] = (w3, ux, uy, uz):
+// grid rows i-1 .. i+2 with i = floor(|r| / h), 4-point Lagrange weights at t = |r| / h - i, u = r / sqrt(eps + |r|^2)
+__global__ void __launch_bounds__(256) painn_edge_records_kernel(const float* __restrict__ r_ij, long E, int mask,
+                                                                 float inv_h, float epsilon, float4* __restrict__ rec) {
+    const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (e >= E) return;
+    const float rx = r_ij[3 * e], ry = r_ij[3 * e + 1], rz = r_ij[3 * e + 2];
+    const float r2 = rx * rx + ry * ry + rz * rz;
+    const float u = sqrtf(r2) * inv_h;
+    const float fl = floorf(u);
+    const float t = u - fl;
+    const float tp = t + 1.0f, tm = t - 1.0f, tq = t - 2.0f;
+    const float w0 = -(1.0f / 6.0f) * t * tm * tq, w1 = 0.5f * tp * tm * tq, w2 = -0.5f * tp * t * tq,
+                w3 = (1.0f / 6.0f) * tp * t * tm;
+    const int first = ((int)fl - 1) & mask;                   // 0 .. rows - 1; rows first .. first + 3 exist in LDS
+    const float inv = 1.0f / sqrtf(epsilon + r2);
+    rec[2 * e] = make_float4(__int_as_float(first * kSliceRowF), w0, w1, w2);
+    rec[2 * e + 1] = make_float4(w3, rx * inv, ry * inv, rz * inv);
+}
+
+// Sum of 16 per-lane values over the 16 lanes that share (lane & 3), leaving value s of the 16 in the lane with
+// (lane >> 2) == s: each step pairs the registers, exchanges the halves two lanes do not keep and adds, so the whole
+// reduction is 15 additions instead of 16 x 4.  Lane halves (xor 32) and odd / even rows of 16 lanes (xor 16) are
+// exchanged by the swap instructions, lanes 8 and 4 apart by LDS-crossbar swizzles.
+__device__ __forceinline__ void swap_add32(float& a, const float b) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    a = __uint_as_float(r[0]) + __uint_as_float(r[1]);        // lanes 0..31: a over both halves; 32..63: b
+}
+__device__ __forceinline__ void swap_add16(float& a, const float b) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    a = __uint_as_float(r[0]) + __uint_as_float(r[1]);        // even rows of 16 lanes: a; odd rows: b
+}
+template <int XOR>
+__device__ __forceinline__ void swizzle_add(float& a, const float b, bool upper) {
+    const float keep = upper ? b : a, send = upper ? a : b;
+    constexpr int pattern = (XOR << 10) | 0x1f;               // lane' = lane ^ XOR inside each group of 32
+    a = keep + __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(send), pattern));
+}
 
 __global__ void __launch_bounds__(1024) painn_table_message_lds_kernel(
-    const int* __restrict__ row_ptr, const int* __restrict__ dst, long n_nodes, const float* __restrict__ r_ij,
-    const float* __restrict__ table, int tab_rows, float inv_h, const float* __restrict__ actv_s,
-    const float* __restrict__ x_v, int n, float epsilon, const float* __restrict__ res_a,
-    const float* __restrict__ res_v, float* __restrict__ out_a, float* __restrict__ out_v) {
-    extern __shared__ float tab[];                            // tab_rows x kSliceRowF
+    const int* __restrict__ row_ptr, const int* __restrict__ dst, const int* __restrict__ node_order, long n_nodes,
+    const float4* __restrict__ rec, const float* __restrict__ table, int tab_rows, const float* __restrict__ actv_s,
+    const float* __restrict__ x_v, int n, const float* __restrict__ res_a, const float* __restrict__ res_v,
+    float* __restrict__ out_a, float* __restrict__ out_v) {
+    extern __shared__ float tab[];                            // (tab_rows + 3) x kSliceRowF
     const int n_slices = n / kSliceChan;
+    // consecutive workgroup ids go to consecutive XCDs: with 8 slices every XCD works on one slice, and its L2 only
+    // ever holds that slice's columns of the node rows
     const int slice = blockIdx.x % n_slices;
     const int group = blockIdx.x / n_slices, groups = gridDim.x / n_slices;
-    for (int q = threadIdx.x; q < tab_rows * (kSliceCols / 4); q += blockDim.x) {
+    for (int q = threadIdx.x; q < (tab_rows + kSliceExtraRows) * (kSliceCols / 4); q += blockDim.x) {
         const int row = q / (kSliceCols / 4), piece = q % (kSliceCols / 4), k = piece / 4, c4 = piece % 4;
-        st4(tab + row * kSliceRowF + 4 * piece, ld4(table + (long)row * 4 * n + k * n + slice * kSliceChan + 4 * c4));
+        st4(tab + row * kSliceRowF + 4 * piece,
+            ld4(table + (long)(row & (tab_rows - 1)) * 4 * n + k * n + slice * kSliceChan + 4 * c4));
     }
     __syncthreads();
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave, waves = blockDim.x / kWave;
     const int l4 = lane & 3, sub = lane >> 2;                 // 4 channels of edge `sub` of the step
     constexpr int kPerIter = kWave / 4;
-    const int mask = tab_rows - 1;
-    // 32-bit element offsets (the host checks that they fit) and running pointers keep the address arithmetic,
-    // a third of the loop's vector instructions otherwise, short
+    // 32-bit element offsets (the host checks that they fit) keep the address arithmetic short
     const unsigned a_stride = (unsigned)n_slices * kSliceCols, v_stride = 3u * (unsigned)n;
     const float* a_base = actv_s + slice * kSliceCols + 4 * l4;
     const float* v_base = x_v + (slice * kSliceChan + 4 * l4) * 3;
     const float* tab_l = tab + 4 * l4;
-    for (long node = (long)group * waves + wave; node < n_nodes; node += (long)groups * waves) {
+    // after the reduction a lane holds ONE of its channel quad's 16 sums: the vector sums 0..11 (channel-major, as in
+    // memory), then the 4 scalar sums
+    const bool is_a = sub >= 12;
+    const long o_lane = slice * kSliceChan + 4 * l4;
+    for (long slot = (long)group * waves + wave; slot < n_nodes; slot += (long)groups * waves) {
+        const long node = node_order ? node_order[slot] : slot;
         const int lo = row_ptr[node], hi = row_ptr[node + 1];
-        EdgeAcc acc;
-        acc.zero();
+        float acc[16];
+#pragma unroll
+        for (int k = 0; k < 16; k++) acc[k] = 0.f;
         int e = lo + sub;
-        const int* dp = dst + e;
-        const float* rp = r_ij + 3L * e;
         unsigned j = 0;
-        float rx = 0.f, ry = 0.f, rz = 0.f;
-        if (e < hi) { j = (unsigned)*dp; rx = rp[0]; ry = rp[1]; rz = rp[2]; }
+        float4 ra = make_float4(0.f, 0.f, 0.f, 0.f), rb = ra;
+        if (e < hi) { j = (unsigned)dst[e]; ra = rec[2 * (long)e]; rb = rec[2 * (long)e + 1]; }
         while (e < hi) {
-            EdgeLoads ld;
             const float* a_row = a_base + j * a_stride;
             const float* v_row = v_base + j * v_stride;
+            float4 a[4], v[3];
 #pragma unroll
-            for (int k = 0; k < 4; k++) ld.a[k] = ld4(a_row + k * kSliceChan);
+            for (int k = 0; k < 4; k++) a[k] = ld4(a_row + k * kSliceChan);
 #pragma unroll
-            for (int k = 0; k < 3; k++) ld.v[k] = ld4(v_row + 4 * k);
-            e += kPerIter; dp += kPerIter; rp += 3 * kPerIter;
+            for (int k = 0; k < 3; k++) v[k] = ld4(v_row + 4 * k);
+            e += kPerIter;
             unsigned j_next = 0;
-            float nx = 0.f, ny = 0.f, nz = 0.f;
-            if (e < hi) { j_next = (unsigned)*dp; nx = rp[0]; ny = rp[1]; nz = rp[2]; }
-            const float r2 = rx * rx + ry * ry + rz * rz;
-            const float u = sqrtf(r2) * inv_h;
-            const float fl = floorf(u);
-            const float t = u - fl;
-            const float tp = t + 1.0f, tm = t - 1.0f, tq = t - 2.0f;
-            const float w0 = -(1.0f / 6.0f) * t * tm * tq, w1 = 0.5f * tp * tm * tq, w2 = -0.5f * tp * t * tq,
-                        w3 = (1.0f / 6.0f) * tp * t * tm;
-            const int i = (int)fl;
-            const float* p0 = tab_l + ((i - 1) & mask) * kSliceRowF;
-            const float* p1 = tab_l + (i & mask) * kSliceRowF;
-            const float* p2 = tab_l + ((i + 1) & mask) * kSliceRowF;
-            const float* p3 = tab_l + ((i + 2) & mask) * kSliceRowF;
+            float4 na = ra, nb = rb;
+            if (e < hi) { j_next = (unsigned)dst[e]; na = rec[2 * (long)e]; nb = rec[2 * (long)e + 1]; }
+            const float* tp = tab_l + __float_as_int(ra.x);
+            const float w0 = ra.y, w1 = ra.z, w2 = ra.w, w3 = rb.x, ux = rb.y, uy = rb.z, uz = rb.w;
+            float p[4][4];                                    // filter x activation: block k, channel c
 #pragma unroll
             for (int k = 0; k < 4; k++) {
-                const float4 t0 = ld4(p0 + k * kSliceChan), t1 = ld4(p1 + k * kSliceChan), t2 = ld4(p2 + k * kSliceChan),
-                             t3 = ld4(p3 + k * kSliceChan);
-                ld.f[k] = make_float4(w0 * t0.x + w1 * t1.x + w2 * t2.x + w3 * t3.x, w0 * t0.y + w1 * t1.y + w2 * t2.y + w3 * t3.y,
-                                      w0 * t0.z + w1 * t1.z + w2 * t2.z + w3 * t3.z, w0 * t0.w + w1 * t1.w + w2 * t2.w + w3 * t3.w);
+                const float4 t0 = ld4(tp + k * kSliceChan), t1 = ld4(tp + kSliceRowF + k * kSliceChan),
+                             t2 = ld4(tp + 2 * kSliceRowF + k * kSliceChan), t3 = ld4(tp + 3 * kSliceRowF + k * kSliceChan);
+                p[k][0] = (w0 * t0.x + w1 * t1.x + w2 * t2.x + w3 * t3.x) * a[k].x;
+                p[k][1] = (w0 * t0.y + w1 * t1.y + w2 * t2.y + w3 * t3.y) * a[k].y;
+                p[k][2] = (w0 * t0.z + w1 * t1.z + w2 * t2.z + w3 * t3.z) * a[k].z;
+                p[k][3] = (w0 * t0.w + w1 * t1.w + w2 * t2.w + w3 * t3.w) * a[k].w;
             }
-            const float inv = __builtin_amdgcn_rsqf(epsilon + r2);
-            ld.accumulate(acc, rx * inv, ry * inv, rz * inv);
-            j = j_next; rx = nx; ry = ny; rz = nz;
-        }
-        for (int d = 4; d < kWave; d <<= 1) {
+            const float vv[12] = {v[0].x, v[0].y, v[0].z, v[0].w, v[1].x, v[1].y, v[1].z, v[1].w,
+                                  v[2].x, v[2].y, v[2].z, v[2].w};
 #pragma unroll
-            for (int k = 0; k < 12; k++) acc.v[k] += __shfl_xor(acc.v[k], d);
-#pragma unroll
-            for (int k = 0; k < 4; k++) acc.a[k] += __shfl_xor(acc.a[k], d);
-        }
-        if (sub == 0) {
-            const long o = node * n + slice * kSliceChan + 4 * l4;
-            if (res_a) {
-                const float4 r = ld4(res_a + o);
-                acc.a[0] += r.x; acc.a[1] += r.y; acc.a[2] += r.z; acc.a[3] += r.w;
+            for (int c = 0; c < 4; c++) {
+                const float x = vv[3 * c], y = vv[3 * c + 1], z = vv[3 * c + 2];
+                const float cx = y * uz - z * uy, cy = z * ux - x * uz, cz = x * uy - y * ux;   // v x u
+                acc[3 * c + 0] = fmaf(ux, p[2][c], fmaf(cx, p[1][c], fmaf(x, p[0][c], acc[3 * c + 0])));
+                acc[3 * c + 1] = fmaf(uy, p[2][c], fmaf(cy, p[1][c], fmaf(y, p[0][c], acc[3 * c + 1])));
+                acc[3 * c + 2] = fmaf(uz, p[2][c], fmaf(cz, p[1][c], fmaf(z, p[0][c], acc[3 * c + 2])));
+                acc[12 + c] += p[3][c];
             }
-            if (res_v) {
-                const float* rv = res_v + o * 3;
-                const float4 ra = ld4(rv), rb = ld4(rv + 4), rc = ld4(rv + 8);
-                const float rr[12] = {ra.x, ra.y, ra.z, ra.w, rb.x, rb.y, rb.z, rb.w, rc.x, rc.y, rc.z, rc.w};
-#pragma unroll
-                for (int k = 0; k < 12; k++) acc.v[k] += rr[k];
-            }
-            st4(out_a + o, make_float4(acc.a[0], acc.a[1], acc.a[2], acc.a[3]));
-            float* ov = out_v + o * 3;
-            st4(ov, make_float4(acc.v[0], acc.v[1], acc.v[2], acc.v[3]));
-            st4(ov + 4, make_float4(acc.v[4], acc.v[5], acc.v[6], acc.v[7]));
-            st4(ov + 8, make_float4(acc.v[8], acc.v[9], acc.v[10], acc.v[11]));
+            j = j_next; ra = na; rb = nb;
         }
+        // 16 sums over the 16 edge slots of the wave: value index sub = bit2 + 2 bit3 + 4 bit4 + 8 bit5 of the lane id
+#pragma unroll
+        for (int k = 0; k < 8; k++) swap_add32(acc[k], acc[k + 8]);          // registers 0..7: value k + 8 bit5
+#pragma unroll
+        for (int k = 0; k < 4; k++) swap_add16(acc[k], acc[k + 4]);          // registers 0..3: value k + 4 bit4 + 8 bit5
+#pragma unroll
+        for (int k = 0; k < 2; k++) swizzle_add<8>(acc[k], acc[k + 2], (lane & 8) != 0);
+        swizzle_add<4>(acc[0], acc[1], (lane & 4) != 0);
+        const long o = node * n + o_lane;
+        float sum = acc[0];
+        float* outp = is_a ? out_a + o + (sub - 12) : out_v + o * 3 + sub;
+        const float* resp = is_a ? (res_a ? res_a + o + (sub - 12) : nullptr) : (res_v ? res_v + o * 3 + sub : nullptr);
+        if (resp) sum += *resp;
+        *outp = sum;
     }
 }
 
@@ -554,32 +597,49 @@ int mg_painn_table_message(const int* row_ptr, const int* dst, const int* node_o
     return check_launch("mg_painn_table_message");
 }
 
-int mg_painn_table_message_sliced(const int* row_ptr, const int* dst, int n_nodes, long n_edges, const float* r_ij,
-                                  const float* table, int table_rows, float period, const float* actv_sliced,
-                                  const float* x_v, int n, float epsilon, const float* res_a, const float* res_v,
-                                  float* out_a, float* out_v, mg_stream_t stream) {
+int mg_painn_edge_records(const float* r_ij, long n_edges, int table_rows, float period, float epsilon,
+                           float* records, mg_stream_t stream) {
+    MG_REQUIRE(n_edges >= 0, "mg_painn_edge_records: negative size");
+    if (n_edges == 0) return MG_OK;
+    MG_REQUIRE(r_ij && records && aligned16(records), "mg_painn_edge_records: null or unaligned pointer");
+    MG_REQUIRE(table_rows >= 4 && table_rows <= kSliceMaxRows && (table_rows & (table_rows - 1)) == 0,
+               "mg_painn_edge_records: table_rows must be a power of two in 4..%d (got %d)", kSliceMaxRows, table_rows);
+    MG_REQUIRE(period > 0.f, "mg_painn_edge_records: period must be positive");
+    hipLaunchKernelGGL(painn_edge_records_kernel, dim3((unsigned)ceil_div(n_edges, 256)), dim3(256), 0,
+                       (hipStream_t)stream, r_ij, n_edges, table_rows - 1, (float)table_rows / period, epsilon,
+                       reinterpret_cast<float4*>(records));
+    return check_launch("mg_painn_edge_records");
+}
+
+int mg_painn_table_message_sliced(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
+                                  const float* records, const float* table, int table_rows, const float* actv_sliced,
+                                  const float* x_v, int n, const float* res_a, const float* res_v, float* out_a,
+                                  float* out_v, mg_stream_t stream) {
     MG_REQUIRE(n_nodes >= 0 && n_edges >= 0 && n >= 0, "mg_painn_table_message_sliced: negative size");
     if (n_nodes == 0 || n == 0) return MG_OK;
     MG_REQUIRE(row_ptr && out_a && out_v && actv_sliced && x_v && table, "mg_painn_table_message_sliced: null pointer");
-    MG_REQUIRE(n_edges == 0 || (dst && r_ij), "mg_painn_table_message_sliced: null edge operand");
+    MG_REQUIRE(n_edges == 0 || (dst && records), "mg_painn_table_message_sliced: null edge operand");
     MG_REQUIRE(table_rows >= 4 && table_rows <= kSliceMaxRows && (table_rows & (table_rows - 1)) == 0,
                "mg_painn_table_message_sliced: table_rows must be a power of two in 4..%d (got %d)", kSliceMaxRows, table_rows);
-    MG_REQUIRE(period > 0.f, "mg_painn_table_message_sliced: period must be positive");
     MG_REQUIRE(n % kSliceChan == 0 && aligned16(table) && aligned16(actv_sliced) && aligned16(x_v) && aligned16(out_a) &&
-                   aligned16(out_v) && (!res_a || aligned16(res_a)) && (!res_v || aligned16(res_v)),
+                   aligned16(out_v) && (!res_a || aligned16(res_a)) && (!res_v || aligned16(res_v)) &&
+                   (!records || aligned16(records)),
                "mg_painn_table_message_sliced: n must be a multiple of %d and the operands 16-byte aligned", kSliceChan);
     MG_REQUIRE((long)n_nodes * 4 * n < (1L << 32), "mg_painn_table_message_sliced: n_nodes * 4 n must be below 2^32");
+    MG_REQUIRE(n_edges < (1L << 31), "mg_painn_table_message_sliced: n_edges must be below 2^31");
     const int n_slices = n / kSliceChan;
-    const size_t lds_bytes = (size_t)table_rows * kSliceRowF * sizeof(float);
+    const size_t lds_bytes = (size_t)(table_rows + kSliceExtraRows) * kSliceRowF * sizeof(float);
     // more than 64 KB of dynamic LDS has to be asked for (per device, so on every call)
     MG_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(painn_table_message_lds_kernel),
-                               hipFuncAttributeMaxDynamicSharedMemorySize, kSliceMaxRows * kSliceRowF * (int)sizeof(float)));
+                               hipFuncAttributeMaxDynamicSharedMemorySize,
+                               (kSliceMaxRows + kSliceExtraRows) * kSliceRowF * (int)sizeof(float)));
     long groups = ceil_div(256, n_slices);                    // one workgroup per CU
     const long max_groups = ceil_div(n_nodes, 16);
     if (groups > max_groups) groups = max_groups;
     hipLaunchKernelGGL(painn_table_message_lds_kernel, dim3((unsigned)(groups * n_slices)), dim3(1024), lds_bytes,
-                       (hipStream_t)stream, row_ptr, dst, (long)n_nodes, r_ij, table, table_rows, (float)table_rows / period,
-                       actv_sliced, x_v, n, epsilon, res_a, res_v, out_a, out_v);
+                       (hipStream_t)stream, row_ptr, dst, node_order, (long)n_nodes,
+                       reinterpret_cast<const float4*>(records), table, table_rows, actv_sliced, x_v, n, res_a, res_v,
+                       out_a, out_v);
     return check_launch("mg_painn_table_message_sliced");
 }
 

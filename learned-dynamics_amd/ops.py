@@ -1169,9 +1169,24 @@ def painn_slice_permutation(n, device):
     return (k * n + PAINN_SLICE * s + c).reshape(-1).to(device)
 
 
-def painn_table_message_sliced(row_ptr, dst, r_ij, table, period, actv_sliced, x_v, epsilon, res_a=None, res_v=None):
+def painn_edge_records(r_ij, table_rows, period, epsilon):
+    """(edges, 8): per edge the first of its four grid rows, the interpolation weights and the direction, for
+    painn_table_message_sliced."""
+    _check_input(r_ij, "r_ij")
+    E = int(r_ij.size(0))
+    if tuple(r_ij.shape) != (E, 3):
+        raise RuntimeError("r_ij must have shape (edges, 3)")
+    with torch.cuda.device(r_ij.device):
+        rec = torch.empty(E, 8, dtype=torch.float32, device=r_ij.device)
+        L.check(_lib.mg_painn_edge_records(_p(r_ij), E, int(table_rows), float(period), float(epsilon), _p(rec), _stream()))
+    return rec
+
+
+def painn_table_message_sliced(row_ptr, dst, r_ij, table, period, actv_sliced, x_v, epsilon, res_a=None, res_v=None,
+                               node_order=None, records=None):
     """painn_table_message with the table held in LDS (at most 512 rows, n a multiple of 16) and actv given with its
-    columns in the order of painn_slice_permutation."""
+    columns in the order of painn_slice_permutation.  records: painn_edge_records(r_ij, rows, period, epsilon) if the
+    caller keeps them (they depend on the edges, not on the features)."""
     _check_input(row_ptr, "row_ptr", torch.int32)
     _check_input(dst, "dst", torch.int32)
     for t, nm in ((r_ij, "r_ij"), (table, "table"), (actv_sliced, "actv_sliced"), (x_v, "x_v")):
@@ -1193,13 +1208,26 @@ def painn_table_message_sliced(row_ptr, dst, r_ij, table, period, actv_sliced, x
             _check_input(t, nm)
             if tuple(t.shape) != shape:
                 raise RuntimeError(f"{nm} has wrong shape")
+    if node_order is not None:
+        _check_input(node_order, "node_order", torch.int32)
+        if node_order.numel() != n_nodes:
+            raise RuntimeError("node_order must have one entry per node")
+    rows = int(table.size(0))
+    if rows < 4 or rows > PAINN_SLICED_MAX_ROWS or rows & (rows - 1):
+        raise RuntimeError(f"table rows must be a power of two in 4..{PAINN_SLICED_MAX_ROWS} (got {rows})")
+    if records is None:
+        records = painn_edge_records(r_ij, rows, period, epsilon)
+    else:
+        _check_input(records, "records")
+        if tuple(records.shape) != (E, 8):
+            raise RuntimeError("records must have shape (edges, 8)")
     dev = x_v.device
     with torch.cuda.device(dev):
         out_a = torch.empty(n_nodes, n, dtype=torch.float32, device=dev)
         out_v = torch.empty(n_nodes, n, 3, dtype=torch.float32, device=dev)
-        L.check(_lib.mg_painn_table_message_sliced(_p(row_ptr), _p(dst), n_nodes, E, _p(r_ij), _p(table),
-                                                   int(table.size(0)), float(period), _p(actv_sliced), _p(x_v), n,
-                                                   float(epsilon), _p(res_a), _p(res_v), _p(out_a), _p(out_v), _stream()))
+        L.check(_lib.mg_painn_table_message_sliced(_p(row_ptr), _p(dst), _p(node_order), n_nodes, E, _p(records),
+                                                   _p(table), rows, _p(actv_sliced), _p(x_v), n, _p(res_a), _p(res_v),
+                                                   _p(out_a), _p(out_v), _stream()))
     return out_a, out_v
 
 

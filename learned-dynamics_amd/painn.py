@@ -158,6 +158,7 @@ class Message(nn.Module):
         return self.mlp_dist.after_first(*self._hidden(r_ij))
 
     use_sliced = True
+    use_cell_order = True
 
     def _sliced_actv_last(self):
         """Last layer of mlp_actv with its rows in the slice-major column order of painn_table_message_sliced."""
@@ -246,8 +247,11 @@ class Message(nn.Module):
                 # the grid fits in LDS: actv comes out of its MLP with the columns regrouped slice by slice
                 h_a, b_a = self.mlp_actv.hidden(flat_a)
                 actv_s = _linear(h_a, self._sliced_actv_last(), ops.ACT_NONE, b_a)[0]
+                # rows in cell order when the graph has one: consecutive rows then gather the same neighbours
+                order = getattr(graph, "cell_order", None) if self.use_cell_order else None
                 out_a, out_v = ops.painn_table_message_sliced(graph.row_ptr, graph.dst32, r_ij, self.filter_table(rows),
-                                                              2.0 * self.r0, actv_s, flat_v, self.epsilon, res_a, res_v)
+                                                              2.0 * self.r0, actv_s, flat_v, self.epsilon, res_a, res_v,
+                                                              node_order=order)
                 return out_a.reshape(B, N, n), out_v.reshape(B, N, n, 3)
             actv = self.mlp_actv(flat_a)
             if rows and r_ij.shape[0] >= 4 * rows:

@@ -381,6 +381,13 @@ def test_table_message_kernel_interpolates_a_known_periodic_filter(ops, n, rows)
                                                     dev(actv)[:, perm].contiguous(), dev(x_v), 0.1)
         _close(no_a, (ref_a - dev(x_a)).cpu(), atol_scale=3e-6)
         _close(no_v, (ref_v - dev(x_v)).cpu(), atol_scale=3e-6)
+        # rows processed in another order, records passed in by the caller: same bits
+        order = torch.randperm(N, generator=g).int().cuda()
+        records = ops.painn_edge_records(dev(r), rows, 2 * r0, 0.1)
+        or_a, or_v = ops.painn_table_message_sliced(row_ptr, dev(dst.int()), dev(r), dev(table), 2 * r0,
+                                                    dev(actv)[:, perm].contiguous(), dev(x_v), 0.1, dev(x_a), dev(x_v),
+                                                    node_order=order, records=records)
+        assert torch.equal(or_a, sl_a) and torch.equal(or_v, sl_v)
         with pytest.raises(RuntimeError, match="power of two in 4..512"):
             ops.painn_table_message_sliced(row_ptr, dev(dst.int()), dev(r), dev(table.repeat(4, 1)), 2 * r0,
                                            dev(actv), dev(x_v), 0.1)
