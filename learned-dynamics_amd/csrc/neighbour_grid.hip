@@ -1,30 +1,32 @@
 // Periodic cell-list radius graph for gfx950.
 //
 // Pipeline (all on the caller's stream, no allocation, no host sync):
-//   bin      wrap each atom into the box, cell id, histogram of cell sizes
-//   scan     exclusive prefix of the histogram -> cell_start
-//   place    atoms into cell order (slot from the histogram atomics)
-//   order    rank atoms inside their cell by index so the cell-ordered array,
-//            and with it every output row, is deterministic
-//   pairs<0> one workgroup per home cell: the 27 window cells are staged in LDS
+//   bin      wrap each atom into the box, cell id
+//   sort     one workgroup per box: counting sort by cell in LDS (histogram, scan,
+//            placement, rank by atom id inside the cell, so that the cell-ordered
+//            array, and with it every output row, is deterministic) -> cell_start.
+//            Boxes of more than 16384 atoms or 4096 cells take four kernels instead
+//            (histogram with global atomics, scan, place, order)
+//   count    one workgroup per home cell: the 27 window cells are staged in LDS
 //            once, each wave takes home atoms and sweeps the staged candidates
-//            64 at a time, counting hits with ballot/popcount -> degree
+//            64 at a time, counting hits with ballot/popcount -> degree, hit masks
 //   scan     degrees -> CSR row_ptr (+ per-box edge counts, statistics)
-//   pairs<1> same sweep, hits compacted with ballot + prefix popcount and written
-//            at row_ptr[i] + running offset (exact-size rows, no atomics per edge)
+//   fill     replays the hit masks, compacts a row's hits in LDS and writes them
+//            at row_ptr[i] (exact-size rows, no atomics per edge)
 //
 // fp32 recipe (this file is compiled with -ffp-contract=off):
 //   w    = remainderf(x - box/2, box) + box/2                 (IEEE remainder)
 //   cell = (int)(((float)ndiv * w) / box) % ndiv              (correctly rounded divide)
-//   d    = remainder(w_i - w_j, box) per axis, evaluated as one conditional
-//          +-box (|w_i - w_j| <= box, so the quotient is -1, 0 or 1 and the
-//          result is exact; ties at +-box/2 keep their sign like round-to-even)
+//   d    = remainder(w_i - w_j, box) per axis, evaluated as fma(-rint(t / box), box, t)
+//          (|w_i - w_j| <= box, so the multiple is -1, 0 or 1 and the result is exact;
+//          see count_kernel for why quotients within rounding of 1/2 do not matter)
 //   d2   = fma(dz,dz, fma(dy,dy, dx*dx)) <= cutoff*cutoff, i != j
 //   only the periodic 3x3x3 cell window is searched, with ndiv = ceil(box/cutoff):
 //   when box/cutoff is not an integer the cells are narrower than the cutoff and
 //   pairs two cells apart are not listed.
 #include "common.hpp"
 #include <mutex>
+#include <type_traits>
 
 namespace mg {
 namespace {
@@ -76,8 +78,11 @@ struct Workspace {
     int* degree;        // A
     int* cell_count;    // C
     int* cell_start;    // C + 1
-    int* block_sums;    // scan scratch
+    int* block_sums;    // scan scratch (cell histogram)
     int* block_max;     // scan scratch
+    int* deg_sums;      // sums / maxima of the degrees per tile of kScanTile rows
+    int* deg_max;
+    int* box_max;       // batch: largest cell occupancy of each box (per-box sort)
     unsigned long long* masks;   // A x mask_words: hit bits of the count pass, reused by the fill pass
     int mask_words;     // 64-candidate groups kept per atom (= LDS tile size / 64)
     size_t bytes;
@@ -104,6 +109,9 @@ Workspace carve(void* base, long A, long C, int mask_words) {
     w.cell_start = static_cast<int*>(take(sizeof(int) * (C + 1)));
     w.block_sums = static_cast<int*>(take(sizeof(int) * scan_blocks));
     w.block_max = static_cast<int*>(take(sizeof(int) * scan_blocks));
+    w.deg_sums = static_cast<int*>(take(sizeof(int) * scan_blocks));
+    w.deg_max = static_cast<int*>(take(sizeof(int) * scan_blocks));
+    w.box_max = static_cast<int*>(take(sizeof(int) * (A > 0 ? A : 1)));   // (batch <= A)
     w.masks = static_cast<unsigned long long*>(take(sizeof(unsigned long long) * A * mask_words));
     w.mask_words = mask_words;
     w.bytes = off;
@@ -120,6 +128,8 @@ int make_grid(float cutoff, float bx, float by, float bz, int batch, int nodes, 
     const long ncells = (long)nd[0] * nd[1] * nd[2];
     MG_REQUIRE(ncells * (batch > 0 ? batch : 1) < 0x7fffffffL, "too many cells (%ld per box)", ncells);
     MG_REQUIRE((long)batch * nodes < 0x7fffffffL, "batch*nodes does not fit int32");
+    MG_REQUIRE((long)nd[0] * (batch > 0 ? batch : 1) <= 65535 && nd[1] <= 65535,
+               "batch * cells along x (%ld) and cells along y (%d) must not exceed 65535", (long)nd[0] * batch, nd[1]);
     g->nx = nd[0]; g->ny = nd[1]; g->nz = nd[2]; g->ncells = (int)ncells;
     g->bx = bx; g->by = by; g->bz = bz;
     g->r0sq = cutoff * cutoff;
@@ -140,11 +150,13 @@ __device__ __forceinline__ int cell_coord(float w, float box, int ndiv) {
     return c < 0 ? 0 : c;   // only reachable with non-finite input
 }
 
-// remainder(d, box) for d = a - b with a, b in [0, box]
-__device__ __forceinline__ float wrap_delta(float d, float box, float half) {
-    if (d > half) d -= box;
-    else if (d < -half) d += box;
-    return d;
+__device__ __forceinline__ int wave_incl_scan(int v, int lane) {
+#pragma unroll
+    for (int d = 1; d < kWave; d <<= 1) {
+        int t = __shfl_up(v, d);
+        if (lane >= d) v += t;
+    }
+    return v;
 }
 
 // ------------------------------------------------------------------- kernels
@@ -159,6 +171,8 @@ __global__ void __launch_bounds__(256) zero3_kernel(int* __restrict__ a, long na
     for (long i = t; i < nc; i += stride) c[i] = 0;
 }
 
+// HIST: also the histogram of cell sizes and each atom's slot in its cell (boxes too large for the per-box sort)
+template <bool HIST>
 __global__ void __launch_bounds__(256) bin_kernel(const float* __restrict__ x, Grid g, Workspace w) {
     const long A = (long)g.batch * g.nodes;
     const long a = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -174,7 +188,94 @@ __global__ void __launch_bounds__(256) bin_kernel(const float* __restrict__ x, G
     const int cell = ((b * g.nx + cx) * g.ny + cy) * g.nz + cz;
     w.wrapped[a] = make_float4(wx, wy, wz, __int_as_float(i));
     w.cell_of[a] = cell;
-    w.slot[a] = atomicAdd(&w.cell_count[cell], 1);
+    if (HIST) w.slot[a] = atomicAdd(&w.cell_count[cell], 1);
+}
+
+// Counting sort of one box by cell, entirely in LDS: histogram (LDS atomics), scan, placement, rank by atom id
+// inside the cell.  One workgroup per box; replaces the histogram / scan / place / order kernels for boxes of at
+// most kSortNodes atoms and kSortCells cells.  Writes cell_start (global positions), sorted, box_max[b].
+constexpr int kSortThreads = 1024, kSortNodes = 16384, kSortCells = 4096;   // 2^14 atoms: 14 key bits
+__global__ void __launch_bounds__(kSortThreads) sort_box_kernel(Grid g, Workspace w) {
+    constexpr int kPer = kSortNodes / kSortThreads, kCellsPer = kSortCells / kSortThreads;
+    __shared__ int start[kSortCells + 1];     // cell sizes, then exclusive starts (start[ncells] = nodes)
+    // keys (cell << 14 | atom) in cell order: a key of a later cell compares greater than any key of this cell, so the
+    // rank loop may read past the end of its cell without a bounds check (the array ends in 8 keys of INT_MAX)
+    __shared__ int placed[kSortNodes + 8];
+    __shared__ int wave_sum[kSortThreads / kWave], wave_max[kSortThreads / kWave];
+    const int b = blockIdx.x, tid = threadIdx.x;
+    const int lane = tid & (kWave - 1), wave = tid / kWave;
+    const long base = (long)b * g.nodes;
+    const int cell_base = b * g.ncells;
+    for (int c = tid; c <= g.ncells; c += kSortThreads) start[c] = 0;
+    __syncthreads();
+    int cl[kPer], sl[kPer];
+#pragma unroll
+    for (int j = 0; j < kPer; j++) {
+        const int i = tid + kSortThreads * j;
+        cl[j] = 0; sl[j] = 0;
+        if (i < g.nodes) {
+            cl[j] = w.cell_of[base + i] - cell_base;
+            sl[j] = atomicAdd(&start[cl[j]], 1);
+        }
+    }
+    __syncthreads();
+    // exclusive scan of the cell sizes: a thread owns kCellsPer consecutive cells
+    int cnt[kCellsPer], sum = 0, mx = 0;
+#pragma unroll
+    for (int k = 0; k < kCellsPer; k++) {
+        const int c = tid * kCellsPer + k;
+        cnt[k] = c < g.ncells ? start[c] : 0;
+        sum += cnt[k];
+        mx = cnt[k] > mx ? cnt[k] : mx;
+    }
+    const int incl = wave_incl_scan(sum, lane);
+    for (int d = kWave / 2; d > 0; d >>= 1) { const int t = __shfl_xor(mx, d); mx = t > mx ? t : mx; }
+    if (lane == kWave - 1) wave_sum[wave] = incl;
+    if (lane == 0) wave_max[wave] = mx;
+    __syncthreads();
+    int run = incl - sum;
+    for (int k = 0; k < wave; k++) run += wave_sum[k];
+#pragma unroll
+    for (int k = 0; k < kCellsPer; k++) {
+        const int c = tid * kCellsPer + k;
+        if (c < g.ncells) {
+            start[c] = run;
+            w.cell_start[cell_base + c] = (int)base + run;
+        }
+        run += cnt[k];
+    }
+    if (tid == 0) {
+        start[g.ncells] = g.nodes;
+        int m = 0;
+        for (int k = 0; k < kSortThreads / kWave; k++) m = wave_max[k] > m ? wave_max[k] : m;
+        w.box_max[b] = m;
+        if (b == g.batch - 1) w.cell_start[(long)g.batch * g.ncells] = g.batch * g.nodes;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kPer; j++) {
+        const int i = tid + kSortThreads * j;
+        if (i < g.nodes) placed[start[cl[j]] + sl[j]] = (cl[j] << 14) | i;
+    }
+    if (tid < 8) placed[g.nodes + tid] = 0x7fffffff;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < kPer; j++) {
+        const int i = tid + kSortThreads * j;
+        if (i < g.nodes) {
+            const int lo = start[cl[j]], hi = start[cl[j] + 1];
+            const int key = (cl[j] << 14) | i;
+            int rank = 0;
+            for (int q0 = lo; q0 < hi; q0 += 8) {          // 8 independent LDS reads per trip, one wait
+                int v[8];
+#pragma unroll
+                for (int u = 0; u < 8; u++) v[u] = placed[q0 + u];
+#pragma unroll
+                for (int u = 0; u < 8; u++) rank += v[u] < key ? 1 : 0;
+            }
+            w.sorted[base + lo + rank] = w.wrapped[base + i];
+        }
+    }
 }
 
 __global__ void __launch_bounds__(256) place_kernel(Grid g, Workspace w) {
@@ -197,15 +298,7 @@ __global__ void __launch_bounds__(256) order_kernel(Grid g, Workspace w) {
     w.sorted[lo + rank] = w.wrapped[a];
 }
 
-// --- three-kernel exclusive scan of n ints: out[0..n] (out[n] = total) -------
-__device__ __forceinline__ int wave_incl_scan(int v, int lane) {
-#pragma unroll
-    for (int d = 1; d < kWave; d <<= 1) {
-        int t = __shfl_up(v, d);
-        if (lane >= d) v += t;
-    }
-    return v;
-}
+// --- two-kernel exclusive scan of n ints: out[0..n] (out[n] = total) -------
 
 // block-wide exclusive scan of one value per thread (256 threads); returns the
 // exclusive prefix and leaves the block total in *total
@@ -251,42 +344,13 @@ __global__ void __launch_bounds__(kScanThreads) scan_sums_kernel(const int* __re
     }
 }
 
-// single workgroup: block_sums -> exclusive offsets in place; total and max out
-__global__ void __launch_bounds__(kScanThreads) scan_top_kernel(int* block_sums, const int* block_max,
-                                                                int nblocks, int* out_total /* may be null */,
-                                                                int* out_max /* may be null */,
-                                                                int* out_overflow /* may be null */) {
-    __shared__ int lds[8];
-    long long carry = 0;
-    int mx = 0;
-    for (int base = 0; base < nblocks; base += kScanThreads) {
-        const int k = base + threadIdx.x;
-        const int v = k < nblocks ? block_sums[k] : 0;
-        const int m = k < nblocks ? block_max[k] : 0;
-        mx = m > mx ? m : mx;
-        int total;
-        const int ex = block_excl_scan(v, &total, lds);
-        if (k < nblocks) block_sums[k] = (int)(carry + ex);
-        carry += total;
-    }
-    for (int d = kWave / 2; d > 0; d >>= 1) { int t = __shfl_xor(mx, d); mx = t > mx ? t : mx; }
-    if ((threadIdx.x & (kWave - 1)) == 0) lds[threadIdx.x / kWave] = mx;
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int mm = 0;
-        for (int k = 0; k < kScanThreads / kWave; k++) mm = lds[k] > mm ? lds[k] : mm;
-        if (out_total) *out_total = carry > 0x7fffffffLL ? 0x7fffffff : (int)carry;
-        if (out_max) *out_max = mm;
-        if (out_overflow) *out_overflow = carry > 0x7fffffffLL ? 1 : 0;
-    }
-}
-
 // whole scan in one workgroup (n small): out[0..n], optional total / max.  Each lane scans a
 // contiguous chunk serially, the chunk totals are scanned across the workgroup once.
-__global__ void __launch_bounds__(kScanThreads) scan_small_kernel(const int* __restrict__ in, int n,
-                                                                  int* __restrict__ out, int* out_total, int* out_max) {
-    __shared__ int lds[8];
-    const int chunk = (n + kScanThreads) / kScanThreads;          // covers indices 0..n
+constexpr int kScanSmallThreads = 1024;
+__global__ void __launch_bounds__(kScanSmallThreads) scan_small_kernel(const int* __restrict__ in, int n,
+                                                                       int* __restrict__ out, int* out_total, int* out_max) {
+    __shared__ int lds[16];
+    const int chunk = (n + kScanSmallThreads) / kScanSmallThreads;          // covers indices 0..n
     const int lo = threadIdx.x * chunk;
     const int hi = lo + chunk < n ? lo + chunk : n;
     int sum = 0, mx = 0;
@@ -306,18 +370,66 @@ __global__ void __launch_bounds__(kScanThreads) scan_small_kernel(const int* __r
     __syncthreads();
     if (threadIdx.x == 0) {
         int mm = 0;
-        for (int k = 0; k < kScanThreads / kWave; k++) mm = lds[k] > mm ? lds[k] : mm;
+        for (int k = 0; k < kScanSmallThreads / kWave; k++) mm = lds[k] > mm ? lds[k] : mm;
         if (out_total) *out_total = total;
         if (out_max) *out_max = mm;
     }
 }
 
 // nodes > 0: also edge_counts[b] = out[(b+1)*nodes] (inclusive prefix of edges per box)
+// Every workgroup adds up the sums of the workgroups before it (at most a few thousand values: one strided pass)
+// instead of waiting for a third kernel to scan them; workgroup 0 also reduces all of them to the totals.
 __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(const int* __restrict__ in, long n,
-                                                                  const int* __restrict__ block_offsets,
+                                                                  const int* __restrict__ block_sums,
+                                                                  const int* __restrict__ block_max, int nblocks,
                                                                   int* __restrict__ out, int nodes,
-                                                                  int* __restrict__ edge_counts) {
+                                                                  int* __restrict__ edge_counts, int* out_total,
+                                                                  int* out_max, int* out_overflow,
+                                                                  const int* __restrict__ box_max, int n_box,
+                                                                  int* out_box_max) {
     __shared__ int lds[8];
+    __shared__ long long before_lds[kScanThreads / kWave];
+    __shared__ int max_lds[kScanThreads / kWave];
+    long long before = 0, all = 0;
+    int mx = 0;
+    const bool totals = blockIdx.x == 0;
+    const int upto = totals ? nblocks : (int)blockIdx.x;
+    for (int k = threadIdx.x; k < upto; k += kScanThreads) {
+        const int v = block_sums[k];
+        all += v;
+        if (k < (int)blockIdx.x) before += v;
+        if (totals) { const int m = block_max[k]; mx = m > mx ? m : mx; }
+    }
+    for (int d = kWave / 2; d > 0; d >>= 1) {
+        before += __shfl_xor(before, d);
+        all += __shfl_xor(all, d);
+        const int t = __shfl_xor(mx, d);
+        mx = t > mx ? t : mx;
+    }
+    if ((threadIdx.x & (kWave - 1)) == 0) {
+        before_lds[threadIdx.x / kWave] = totals ? all : before;
+        max_lds[threadIdx.x / kWave] = mx;
+    }
+    __syncthreads();
+    long long sum_w = 0;
+    int max_w = 0;
+    for (int k = 0; k < kScanThreads / kWave; k++) {
+        sum_w += before_lds[k];
+        max_w = max_lds[k] > max_w ? max_lds[k] : max_w;
+    }
+    const int block_offset = totals ? 0 : (int)sum_w;         // (an overflowing total is flagged by workgroup 0)
+    if (totals && box_max != nullptr && threadIdx.x < kWave) {
+        // largest cell occupancy over the boxes (the per-box sort leaves one value per box)
+        int m = 0;
+        for (int k = threadIdx.x; k < n_box; k += kWave) m = box_max[k] > m ? box_max[k] : m;
+        for (int d = kWave / 2; d > 0; d >>= 1) { const int t = __shfl_xor(m, d); m = t > m ? t : m; }
+        if (threadIdx.x == 0) *out_box_max = m;
+    }
+    if (totals && threadIdx.x == 0) {
+        if (out_total) *out_total = sum_w > 0x7fffffffLL ? 0x7fffffff : (int)sum_w;
+        if (out_max) *out_max = max_w;
+        if (out_overflow) *out_overflow = sum_w > 0x7fffffffLL ? 1 : 0;
+    }
     const long base = (long)blockIdx.x * kScanTile + (long)threadIdx.x * kScanItems;
     int v[kScanItems];
     int s = 0;
@@ -327,7 +439,7 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(const int* __r
         s += v[k];
     }
     int total;
-    int run = block_excl_scan(s, &total, lds) + block_offsets[blockIdx.x];
+    int run = block_excl_scan(s, &total, lds) + block_offset;
 #pragma unroll
     for (int k = 0; k < kScanItems; k++) {
         if (base + k <= n) {
@@ -342,152 +454,275 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(const int* __r
 }
 
 
-// One workgroup per home cell.  FILL = false: degrees (+ hit masks).  FILL = true: src/dst.
+// One workgroup per home cell, two passes.  The count pass stages the 27 window cells in LDS once
+// (wrapped positions + atom ids), each wave takes home atoms and sweeps the staged candidates 64 at a
+// time; it keeps, per home atom, one 64-bit ballot per group of 64 candidates.  The fill pass replays
+// those masks and never touches the geometry again (it stages only the candidates' atom ids).
+// Windows larger than the LDS tile (kCandCap candidates) take a slow path that reads the tail from
+// global memory and recomputes the geometry in the fill pass.
 //
-// The count pass keeps, per home atom, one 64-bit ballot per group of 64 window
-// candidates; the fill pass replays those masks and never touches the geometry
-// again (it stages only the candidates' atom ids).  Windows larger than the LDS
-// tile (kCandCap candidates) fall back to recomputing in the fill pass.
-//
-// Minimum image: a wrapped coordinate lies in [0, box] with BOTH ends possible
-// (remainderf(x - box/2, box) + box/2 gives exactly box for x = box, -box, 3 box, ...
-// and for x within half an ulp below box), and such an atom sits in cell 0 because
-// the cell index is taken modulo ndiv.  So cell 0 holds coordinates near 0 and
-// coordinates equal (or within rounding of) box; every other cell c holds
-// coordinates within rounding of [c, c+1) box/ndiv.  In an axis with at least 5
-// cells whose window (home - 1 .. home + 1) contains neither cell 0 nor, from the
-// other side, wraps around the box (home cell 2 .. ndiv-2), |w_i - w_j| < 2/5 box
-// < box/2 for every window candidate, remainder(w_i - w_j, box) is the plain
-// difference and the conditional +-box is skipped (same bits, 40 % fewer
-// instructions per pair).  Home cell 1 keeps the wrap: its window contains cell 0.
-template <bool FILL, int kCandCap>
-__global__ void __launch_bounds__(256) pairs_kernel(Grid g, Workspace w, const int* __restrict__ row_ptr,
-                                                    int* __restrict__ src, int* __restrict__ dst, int capacity) {
+// The hot loops are straight-line code:
+//   * the tile is padded to a multiple of 64 with candidates at +infinity (their distance test fails),
+//     so no lane checks whether its candidate exists;
+//   * the home atom is itself a candidate (the centre cell is part of the window, its place there is
+//     known) and passes the distance test: its bit is cleared once after the sweep instead of
+//     comparing ids on every pair;
+//   * minimum image without compares: remainder(t, box) = t - rint(t / box) box, evaluated as
+//     fma(-rint(t * (1 / box)), box, t).  For |t| <= box the multiple is -1, 0 or 1 and the fma is
+//     exact, so the result is the IEEE remainder bit for bit unless t / box is within rounding of
+//     +-1/2, where the other representative may be chosen; there |result| is about box / 2, which
+//     exceeds the cutoff (the grid has at least 3 cells per axis, so box > 2 cutoff): such a pair is
+//     listed by neither choice.
+//   * a wrapped coordinate lies in [0, box] with BOTH ends possible (remainderf(x - box/2, box) +
+//     box/2 gives exactly box for x = box, -box, 3 box, ... and for x within half an ulp below box),
+//     and such an atom sits in cell 0 because the cell index is taken modulo ndiv.  Only a home cell
+//     whose window holds neither cell 0 nor cell ndiv - 1 on any axis (coordinates 2 .. ndiv - 3,
+//     ndiv >= 5) skips the minimum image altogether: there |w_i - w_j| < 2/5 box.
+//   * the fill pass compacts the hits of a row into a per-wave LDS buffer with mbcnt prefix counts and
+//     writes them as whole runs, a few full-width stores per row instead of a dozen partial ones.
+constexpr int kRowBuf = 256;              // fill pass: hits buffered per wave before they are written (ints)
+
+struct Window {
+    int M;            // candidates in the 27 cells
+    int self_base;    // the home cell's atoms are candidates self_base .. self_base + home_n - 1
+    int home_lo, home_n;
+};
+
+// First wave: lane t < 27 looks cell t of the window up, a shuffle scan gives the prefix of the lengths.
+// Returns false (uniformly) when the home cell is empty.
+__device__ __forceinline__ bool window_ranges(const Grid& g, const Workspace& w, int b, int cx, int cy, int cz,
+                                              int* range_start, int* range_prefix, Window* win) {
+    if (threadIdx.x < kWave) {
+        const int lane = threadIdx.x;
+        const int t = lane < 27 ? lane : 26;
+        const int dx = t / 9 - 1, dy = (t / 3) % 3 - 1, dz = t % 3 - 1;      // divisions by constants: multiplies
+        int nx = cx + dx, ny = cy + dy, nz = cz + dz;                        // periodic neighbours without a division
+        nx = nx < 0 ? nx + g.nx : (nx >= g.nx ? nx - g.nx : nx);
+        ny = ny < 0 ? ny + g.ny : (ny >= g.ny ? ny - g.ny : ny);
+        nz = nz < 0 ? nz + g.nz : (nz >= g.nz ? nz - g.nz : nz);
+        const int nc = ((b * g.nx + nx) * g.ny + ny) * g.nz + nz;
+        const int start = w.cell_start[nc];
+        const int len = lane < 27 ? w.cell_start[nc + 1] - start : 0;
+        int incl = len;
+#pragma unroll
+        for (int d = 1; d < 32; d <<= 1) {
+            const int up = __shfl_up(incl, d);
+            if (lane >= d) incl += up;
+        }
+        if (lane < 27) {
+            range_start[lane] = start;
+            range_prefix[lane + 1] = incl;
+        }
+        if (lane == 0) range_prefix[0] = 0;
+    }
+    __syncthreads();
+    win->M = range_prefix[27];
+    win->self_base = range_prefix[13];
+    win->home_lo = range_start[13];
+    win->home_n = range_prefix[14] - range_prefix[13];
+    return win->home_n > 0;
+}
+
+// candidate k of the concatenated window -> address in the cell-ordered array
+__device__ __forceinline__ int locate(const int* range_start, const int* range_prefix, int k) {
+    int lo = 0, hi = 26;   // last range with prefix <= k
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (range_prefix[mid] <= k) lo = mid; else hi = mid - 1;
+    }
+    return range_start[lo] + (k - range_prefix[lo]);
+}
+
+// WRAP: bit 0 / 1 / 2 = apply the minimum image along x / y / z
+template <int WRAP>
+__device__ __forceinline__ bool within_cutoff(const float4& self, const float4& o, const Grid& g, float ibx, float iby,
+                                              float ibz) {
+    float dx = self.x - o.x, dy = self.y - o.y, dz = self.z - o.z;
+    if (WRAP & 1) dx = __fmaf_rn(-rintf(dx * ibx), g.bx, dx);
+    if (WRAP & 2) dy = __fmaf_rn(-rintf(dy * iby), g.by, dy);
+    if (WRAP & 4) dz = __fmaf_rn(-rintf(dz * ibz), g.bz, dz);
+    const float d2 = __fmaf_rn(dz, dz, __fmaf_rn(dy, dy, dx * dx));
+    return d2 <= g.r0sq;
+}
+
+template <int kCandCap>
+__global__ void __launch_bounds__(256) count_kernel(Grid g, Workspace w) {
     constexpr int kWords = kCandCap / kWave;
-    __shared__ float4 cand[FILL ? 1 : kCandCap];      // count pass: wrapped positions + atom id
-    __shared__ int cand_idx[FILL ? kCandCap : 1];     // fill pass: atom ids only
+    __shared__ float4 cand[kCandCap];
     __shared__ int range_start[27];
     __shared__ int range_prefix[28];
 
-    const int cell = blockIdx.x;              // global cell id
-    const int home_lo = w.cell_start[cell];
-    const int home_n = w.cell_start[cell + 1] - home_lo;
-    if (home_n == 0) return;                  // uniform over the workgroup
-
-    const int b = cell / g.ncells;
-    const int c = cell - b * g.ncells;
-    const int cx = c / (g.ny * g.nz), cy = (c / g.nz) % g.ny, cz = c % g.nz;
-
-    if (threadIdx.x < 27) {
-        const int t = threadIdx.x;
-        const int dx = t / 9 - 1, dy = (t / 3) % 3 - 1, dz = t % 3 - 1;
-        const int nx = (cx + dx + g.nx) % g.nx;
-        const int ny = (cy + dy + g.ny) % g.ny;
-        const int nz = (cz + dz + g.nz) % g.nz;
-        const int nc = ((b * g.nx + nx) * g.ny + ny) * g.nz + nz;
-        range_start[t] = w.cell_start[nc];
-        range_prefix[t + 1] = w.cell_start[nc + 1] - w.cell_start[nc];
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int acc = 0;
-        range_prefix[0] = 0;
-        for (int t = 0; t < 27; t++) { acc += range_prefix[t + 1]; range_prefix[t + 1] = acc; }
-    }
-    __syncthreads();
-    const int M = range_prefix[27];
-    const bool masks_ok = M <= kCandCap;      // uniform: the count pass stored every ballot of this cell
-
-    // candidate k of the concatenated window -> address in the cell-ordered array
-    auto locate = [&](int k) {
-        int lo = 0, hi = 26;   // last range with prefix <= k
-        while (lo < hi) {
-            const int mid = (lo + hi + 1) >> 1;
-            if (range_prefix[mid] <= k) lo = mid; else hi = mid - 1;
-        }
-        return range_start[lo] + (k - range_prefix[lo]);
-    };
-
-    const int staged = M < kCandCap ? M : kCandCap;
-    for (int k = threadIdx.x; k < staged; k += blockDim.x) {
-        const float4 v = w.sorted[locate(k)];
-        if (FILL) cand_idx[k] = __float_as_int(v.w);
-        else cand[k] = v;
-    }
-    __syncthreads();
-
+    // grid (nz, ny, nx * batch): the cell coordinates come from the workgroup id without a division chain
+    const int cz = blockIdx.x, cy = blockIdx.y;
+    const int b = blockIdx.z / g.nx, cx = blockIdx.z - b * g.nx;
+    Window win;
+    if (!window_ranges(g, w, b, cx, cy, cz, range_start, range_prefix, &win)) return;   // uniform
+    const int M = win.M;
     const int lane = threadIdx.x & (kWave - 1);
     const int wave = threadIdx.x / kWave, nwaves = blockDim.x / kWave;
-    const float hx = 0.5f * g.bx, hy = 0.5f * g.by, hz = 0.5f * g.bz;
-    const bool wrap_x = g.nx < 5 || cx <= 1 || cx == g.nx - 1;
-    const bool wrap_y = g.ny < 5 || cy <= 1 || cy == g.ny - 1;
-    const bool wrap_z = g.nz < 5 || cz <= 1 || cz == g.nz - 1;
-    const unsigned long long lt_mask = (1ull << lane) - 1ull;
+
+    const int staged = M < kCandCap ? M : kCandCap;
+    const int padded = (staged + kWave - 1) & ~(kWave - 1);        // <= kCandCap (a multiple of 64)
+    const float inf = __int_as_float(0x7f800000);
+    for (int k = threadIdx.x; k < padded; k += blockDim.x)
+        cand[k] = k < staged ? w.sorted[locate(range_start, range_prefix, k)] : make_float4(inf, inf, inf, __int_as_float(-1));
+    __syncthreads();
+
+    // an axis needs the minimum image unless the window stays clear of cells 0 and ndiv - 1 (see above)
+    const int wrap = ((g.nx < 5 || cx < 2 || cx > g.nx - 3) ? 1 : 0) | ((g.ny < 5 || cy < 2 || cy > g.ny - 3) ? 2 : 0) |
+                     ((g.nz < 5 || cz < 2 || cz > g.nz - 3) ? 4 : 0);
+    const float ibx = 1.0f / g.bx, iby = 1.0f / g.by, ibz = 1.0f / g.bz;
     const int node_base = b * g.nodes;
 
-    auto test_pair = [&](const float4& self, const float4& o) {
-        float dx = self.x - o.x, dy = self.y - o.y, dz = self.z - o.z;
-        if (wrap_x) dx = wrap_delta(dx, g.bx, hx);
-        if (wrap_y) dy = wrap_delta(dy, g.by, hy);
-        if (wrap_z) dz = wrap_delta(dz, g.bz, hz);
-        const float d2 = __fmaf_rn(dz, dz, __fmaf_rn(dy, dy, dx * dx));
-        return d2 <= g.r0sq;
-    };
-
-    for (int h = wave; h < home_n; h += nwaves) {
-        const float4 self = w.sorted[home_lo + h];
-        const int self_idx = __float_as_int(self.w);
-        const int row = node_base + self_idx;
-        unsigned long long* my_masks = w.masks + (long)row * kWords;
+    for (int h = wave; h < win.home_n; h += nwaves) {
+        const int k_self = win.self_base + h;
+        float4 self;
+        if (k_self < kCandCap) self = cand[k_self];
+        else self = w.sorted[win.home_lo + h];
+        const int row = node_base + __float_as_int(self.w);
         int running = 0;
-        const int words = (M + kWave - 1) / kWave;     // <= kWords when masks_ok
-        if (!FILL) {
-            unsigned long long keep = 0;               // lane i keeps the ballot of candidate group i
-            for (int k0 = 0; k0 < M; k0 += kWave) {
-                const int k = k0 + lane;
-                bool hit = false;
-                if (k < M) {
-                    const float4 o = k < kCandCap ? cand[k] : w.sorted[locate(k)];
-                    hit = (__float_as_int(o.w) != self_idx) && test_pair(self, o);
-                }
-                const unsigned long long mask = __ballot(hit);
+        unsigned long long keep = 0;                   // lane i keeps the ballot of candidate group i
+        auto sweep = [&](auto wrap_tag) {
+            constexpr int kWrap = decltype(wrap_tag)::value;
+            for (int k0 = 0; k0 < padded; k0 += kWave) {
+                const unsigned long long mask = __ballot(within_cutoff<kWrap>(self, cand[k0 + lane], g, ibx, iby, ibz));
                 if (lane == k0 / kWave) keep = mask;
                 running += __popcll(mask);
             }
-            if (masks_ok && lane < words) my_masks[lane] = keep;   // one unit-stride store per atom
-            if (lane == 0) w.degree[row] = running;
+        };
+        switch (wrap) {                                // uniform over the workgroup
+            case 0: sweep(std::integral_constant<int, 0>{}); break;
+            case 1: sweep(std::integral_constant<int, 1>{}); break;
+            case 2: sweep(std::integral_constant<int, 2>{}); break;
+            case 3: sweep(std::integral_constant<int, 3>{}); break;
+            case 4: sweep(std::integral_constant<int, 4>{}); break;
+            case 5: sweep(std::integral_constant<int, 5>{}); break;
+            case 6: sweep(std::integral_constant<int, 6>{}); break;
+            default: sweep(std::integral_constant<int, 7>{}); break;
+        }
+        if (k_self < kCandCap) {
+            // the atom found itself: take its bit out of the kept ballot and of the count
+            const int g_self = k_self / kWave;
+            const unsigned long long bit = 1ull << (k_self & (kWave - 1));
+            const int found = lane == g_self ? (int)((keep & bit) != 0ull) : 0;
+            if (lane == g_self) keep &= ~bit;
+            running -= __shfl(found, g_self);
+        }
+        // candidates beyond the tile: from global memory, ids compared
+        for (int k0 = kCandCap; k0 < M; k0 += kWave) {
+            const int k = k0 + lane;
+            bool hit = false;
+            if (k < M) {
+                const float4 o = w.sorted[locate(range_start, range_prefix, k)];
+                hit = k != k_self && within_cutoff<7>(self, o, g, ibx, iby, ibz);
+            }
+            running += __popcll(__ballot(hit));
+        }
+        // masks are kept by position in the cell-ordered array: the home atoms of a cell write one contiguous block
+        if (M <= kCandCap && lane < padded / kWave) w.masks[(long)(win.home_lo + h) * kWords + lane] = keep;
+        if (lane == 0) w.degree[row] = running;
+    }
+}
+
+template <int kCandCap>
+__global__ void __launch_bounds__(256) fill_kernel(Grid g, Workspace w, const int* __restrict__ row_ptr,
+                                                   int* __restrict__ src, int* __restrict__ dst, int capacity) {
+    constexpr int kWords = kCandCap / kWave;
+    constexpr int kMaxWaves = 4;
+    __shared__ int cand_idx[kCandCap];
+    __shared__ int row_buf[kMaxWaves * kRowBuf];
+    __shared__ int range_start[27];
+    __shared__ int range_prefix[28];
+
+    // grid (nz, ny, nx * batch): the cell coordinates come from the workgroup id without a division chain
+    const int cz = blockIdx.x, cy = blockIdx.y;
+    const int b = blockIdx.z / g.nx, cx = blockIdx.z - b * g.nx;
+    Window win;
+    if (!window_ranges(g, w, b, cx, cy, cz, range_start, range_prefix, &win)) return;
+    const int M = win.M;
+    const int lane = threadIdx.x & (kWave - 1);
+    const int wave = threadIdx.x / kWave, nwaves = blockDim.x / kWave;
+    const int staged = M < kCandCap ? M : kCandCap;
+    const int padded = (staged + kWave - 1) & ~(kWave - 1);
+    for (int k = threadIdx.x; k < padded; k += blockDim.x)
+        cand_idx[k] = k < staged ? __float_as_int(w.sorted[locate(range_start, range_prefix, k)].w) : 0;
+    __syncthreads();
+
+    const int node_base = b * g.nodes;
+    const float ibx = 1.0f / g.bx, iby = 1.0f / g.by, ibz = 1.0f / g.bz;
+    int* buf = row_buf + wave * kRowBuf;
+
+    // leave the buffered hits of row `row` at out_pos .. out_pos + cnt - 1 (edges beyond the capacity are dropped)
+    auto flush = [&](int row, int out_pos, int cnt) {
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        for (int i = lane; i < cnt; i += kWave) {
+            const int pos = out_pos + i;
+            if (pos < capacity) {
+                src[pos] = row;
+                dst[pos] = buf[i];
+            }
+        }
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    // the fast path keeps one home atom's row start and masks in flight while the previous atom's hits are written
+    int next_row = 0, next_pos = 0;
+    unsigned long long next_keep = 0;
+    auto fetch = [&](int h) {
+        next_row = node_base + cand_idx[win.self_base + h];
+        next_pos = row_ptr[next_row];
+        next_keep = lane < padded / kWave ? w.masks[(long)(win.home_lo + h) * kWords + lane] : 0ull;
+    };
+    if (M <= kCandCap && wave < win.home_n) fetch(wave);
+    for (int h = wave; h < win.home_n; h += nwaves) {
+        const int k_self = win.self_base + h;
+        if (M <= kCandCap) {
+            const int row = next_row;
+            int out_pos = next_pos;
+            int cnt = 0;
+            const unsigned long long keep = next_keep;
+            if (h + nwaves < win.home_n) fetch(h + nwaves);
+            const unsigned keep_lo = (unsigned)(keep & 0xffffffffull), keep_hi = (unsigned)(keep >> 32);
+            for (int k0 = 0; k0 < padded; k0 += kWave) {
+                const int it = k0 / kWave;
+                const unsigned lo = __builtin_amdgcn_readlane(keep_lo, it), hi = __builtin_amdgcn_readlane(keep_hi, it);
+                const unsigned below = __builtin_amdgcn_mbcnt_hi(hi, __builtin_amdgcn_mbcnt_lo(lo, 0u));   // hits in lower lanes
+                const unsigned mine = lane < 32 ? (lo >> lane) & 1u : (hi >> (lane - 32)) & 1u;
+                if (mine) buf[cnt + below] = node_base + cand_idx[k0 + lane];
+                cnt += __popc(lo) + __popc(hi);
+                if (cnt > kRowBuf - kWave) {             // uniform: the next group might not fit
+                    flush(row, out_pos, cnt);
+                    out_pos += cnt;
+                    cnt = 0;
+                }
+            }
+            flush(row, out_pos, cnt);
         } else {
-            const int out_base = row_ptr[row];
-            unsigned long long keep = 0;
-            if (masks_ok && lane < words) keep = my_masks[lane];
+            // window larger than the tile: no masks were kept, recompute (ids compared, candidates from global memory)
+            const float4 self = w.sorted[win.home_lo + h];
+            const int row = node_base + __float_as_int(self.w);
+            int out_pos = row_ptr[row];
+            int cnt = 0;
             for (int k0 = 0; k0 < M; k0 += kWave) {
                 const int k = k0 + lane;
-                unsigned long long mask;
+                bool hit = false;
                 int other_idx = 0;
-                if (masks_ok) {
-                    const int it = k0 / kWave;
-                    const unsigned lo = __shfl((unsigned)(keep & 0xffffffffull), it);
-                    const unsigned hi = __shfl((unsigned)(keep >> 32), it);
-                    mask = ((unsigned long long)hi << 32) | lo;
-                    if (k < M) other_idx = cand_idx[k];
-                } else {
-                    bool hit = false;
-                    if (k < M) {
-                        const float4 o = w.sorted[locate(k)];
-                        other_idx = __float_as_int(o.w);
-                        hit = (other_idx != self_idx) && test_pair(self, o);
-                    }
-                    mask = __ballot(hit);
+                if (k < M) {
+                    const float4 o = w.sorted[locate(range_start, range_prefix, k)];
+                    other_idx = __float_as_int(o.w);
+                    hit = k != k_self && within_cutoff<7>(self, o, g, ibx, iby, ibz);
                 }
-                if ((mask >> lane) & 1ull) {
-                    const int pos = out_base + running + __popcll(mask & lt_mask);
-                    if (pos < capacity) {      // src / dst hold `capacity` edges: the rest is dropped, never written
-                        src[pos] = row;
-                        dst[pos] = node_base + other_idx;
-                    }
+                const unsigned long long mask = __ballot(hit);
+                if (hit) buf[cnt + __popcll(mask & ((1ull << lane) - 1ull))] = node_base + other_idx;
+                cnt += __popcll(mask);
+                if (cnt > kRowBuf - kWave) {
+                    flush(row, out_pos, cnt);
+                    out_pos += cnt;
+                    cnt = 0;
                 }
-                running += __popcll(mask);
             }
+            flush(row, out_pos, cnt);
         }
     }
 }
@@ -587,19 +822,20 @@ __global__ void __launch_bounds__(256) edge_vectors_kernel(const float* __restri
 int run_scan(const int* in, long n, int* out, Workspace& w, int* out_total, int* out_max, int* out_overflow,
              hipStream_t st, int nodes = 0, int* edge_counts = nullptr) {
     if (n <= 16384 && nodes == 0 && out_overflow == nullptr) {
-        hipLaunchKernelGGL(scan_small_kernel, dim3(1), dim3(kScanThreads), 0, st, in, (int)n, out, out_total, out_max);
+        hipLaunchKernelGGL(scan_small_kernel, dim3(1), dim3(kScanSmallThreads), 0, st, in, (int)n, out, out_total, out_max);
         return check_launch("neighbour scan");
     }
     const int nblocks = (int)ceil_div(n + 1, kScanTile);
     hipLaunchKernelGGL(scan_sums_kernel, dim3(nblocks), dim3(kScanThreads), 0, st, in, n, w.block_sums, w.block_max);
-    hipLaunchKernelGGL(scan_top_kernel, dim3(1), dim3(kScanThreads), 0, st, w.block_sums, w.block_max, nblocks,
-                       out_total, out_max, out_overflow);
-    hipLaunchKernelGGL(scan_apply_kernel, dim3(nblocks), dim3(kScanThreads), 0, st, in, n, w.block_sums, out, nodes,
-                       edge_counts);
+    hipLaunchKernelGGL(scan_apply_kernel, dim3(nblocks), dim3(kScanThreads), 0, st, in, n, w.block_sums, w.block_max,
+                       nblocks, out, nodes, edge_counts, out_total, out_max, out_overflow, (const int*)nullptr, 0,
+                       (int*)nullptr);
     return check_launch("neighbour scan");
 }
 
 int pairs_block_size(const Grid& g);
+// one workgroup per cell, laid out so that the kernels read the cell coordinates off the workgroup id
+dim3 cell_grid(const Grid& g) { return dim3((unsigned)g.nz, (unsigned)g.ny, (unsigned)(g.nx * g.batch)); }
 int mask_words(const Grid& g) { return (pairs_block_size(g) == 64 ? kCandCapSparse : kCandCapDense) / kWave; }
 
 int pairs_block_size(const Grid& g) {
@@ -651,20 +887,30 @@ int mg_neighbour_count(const float* x, int batch, int nodes, float cutoff, float
         return check_launch("mg_neighbour_count");
     }
     MG_REQUIRE(x != nullptr, "mg_neighbour_count: x is null");
-    hipLaunchKernelGGL(zero3_kernel, dim3((unsigned)(ceil_div(C, 256) < 1024 ? ceil_div(C, 256) : 1024)), dim3(256), 0,
-                       st, stats, 4L, row_ptr, 1L, w.cell_count, C);
     const unsigned ablocks = (unsigned)ceil_div(A, 256);
-    hipLaunchKernelGGL(bin_kernel, dim3(ablocks), dim3(256), 0, st, x, g, w);
-    if (int s = run_scan(w.cell_count, C, w.cell_start, w, nullptr, stats + 1, nullptr, st)) return s;
-    hipLaunchKernelGGL(place_kernel, dim3(ablocks), dim3(256), 0, st, g, w);
-    hipLaunchKernelGGL(order_kernel, dim3(ablocks), dim3(256), 0, st, g, w);
+    const int deg_tiles = (int)ceil_div(A + 1, kScanTile);
+    const bool per_box_sort = nodes <= kSortNodes && g.ncells <= kSortCells;
+    if (per_box_sort) {
+        // six launches in all: bin, per-box sort, count, two for the scan of the degrees, fill
+        hipLaunchKernelGGL(bin_kernel<false>, dim3(ablocks), dim3(256), 0, st, x, g, w);
+        hipLaunchKernelGGL(sort_box_kernel, dim3((unsigned)batch), dim3(kSortThreads), 0, st, g, w);
+    } else {
+        hipLaunchKernelGGL(zero3_kernel, dim3((unsigned)(ceil_div(C, 256) < 1024 ? ceil_div(C, 256) : 1024)), dim3(256),
+                           0, st, stats, 4L, row_ptr, 1L, w.cell_count, C);
+        hipLaunchKernelGGL(bin_kernel<true>, dim3(ablocks), dim3(256), 0, st, x, g, w);
+        if (int s = run_scan(w.cell_count, C, w.cell_start, w, nullptr, stats + 1, nullptr, st)) return s;
+        hipLaunchKernelGGL(place_kernel, dim3(ablocks), dim3(256), 0, st, g, w);
+        hipLaunchKernelGGL(order_kernel, dim3(ablocks), dim3(256), 0, st, g, w);
+    }
     if (pairs_block_size(g) == 64)
-        hipLaunchKernelGGL((pairs_kernel<false, kCandCapSparse>), dim3((unsigned)C), dim3(64), 0, st, g, w,
-                           (const int*)nullptr, (int*)nullptr, (int*)nullptr, 0);
+        hipLaunchKernelGGL((count_kernel<kCandCapSparse>), cell_grid(g), dim3(64), 0, st, g, w);
     else
-        hipLaunchKernelGGL((pairs_kernel<false, kCandCapDense>), dim3((unsigned)C), dim3(256), 0, st, g, w,
-                           (const int*)nullptr, (int*)nullptr, (int*)nullptr, 0);
-    if (int s = run_scan(w.degree, A, row_ptr, w, stats + 0, stats + 2, stats + 3, st, nodes, edge_counts)) return s;
+        hipLaunchKernelGGL((count_kernel<kCandCapDense>), cell_grid(g), dim3(256), 0, st, g, w);
+    hipLaunchKernelGGL(scan_sums_kernel, dim3((unsigned)deg_tiles), dim3(kScanThreads), 0, st, (const int*)w.degree, A,
+                       w.deg_sums, w.deg_max);
+    hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)deg_tiles), dim3(kScanThreads), 0, st, (const int*)w.degree, A,
+                       (const int*)w.deg_sums, (const int*)w.deg_max, deg_tiles, row_ptr, nodes, edge_counts, stats + 0,
+                       stats + 2, stats + 3, per_box_sort ? (const int*)w.box_max : (const int*)nullptr, batch, stats + 1);
     return check_launch("mg_neighbour_count");
 }
 
@@ -683,10 +929,10 @@ int mg_neighbour_fill(const void* workspace, size_t workspace_bytes, int batch, 
         return fail(MG_ERR_WORKSPACE, "mg_neighbour_fill: workspace has %zu bytes, %zu needed", workspace_bytes,
                     w.bytes + 256);
     if (pairs_block_size(g) == 64)
-        hipLaunchKernelGGL((pairs_kernel<true, kCandCapSparse>), dim3((unsigned)C), dim3(64), 0, (hipStream_t)stream,
+        hipLaunchKernelGGL((fill_kernel<kCandCapSparse>), cell_grid(g), dim3(64), 0, (hipStream_t)stream,
                            g, w, row_ptr, src, dst, n_edges);
     else
-        hipLaunchKernelGGL((pairs_kernel<true, kCandCapDense>), dim3((unsigned)C), dim3(256), 0, (hipStream_t)stream,
+        hipLaunchKernelGGL((fill_kernel<kCandCapDense>), cell_grid(g), dim3(256), 0, (hipStream_t)stream,
                            g, w, row_ptr, src, dst, n_edges);
     return check_launch("mg_neighbour_fill");
 }

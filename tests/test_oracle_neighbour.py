@@ -104,6 +104,36 @@ def test_under_resolved_grid_drops_pairs_two_cells_apart():
         assert np.all((ds == 0) | (ds == 1) | (ds == 11))
 
 
+def test_rint_fma_minimum_image_equals_remainderf_wherever_a_pair_can_be_listed():
+    """The HIP kernels evaluate remainder(t, box) for t = a - b, a, b in [0, box], as fma(-rint(t * (1 / box)), box, t).
+    The multiple is -1, 0 or 1 and the fma is exact, so the value equals libm's remainderf bit for bit, except that
+    for t / box within rounding of +-1/2 the other representative (t + box instead of t, ...) may be chosen.  There the
+    magnitude of either representative is about box / 2 > cutoff (at least 3 cells per axis), so no listed pair can
+    be affected: the test demands exact equality everywhere else and |value| > 0.49 box where the two differ."""
+    L = ON.lib()
+    rng = np.random.default_rng(5)
+    rem = np.vectorize(lambda a, b: L.nbr_oracle_remainderf(a, b), otypes=[np.float32])
+    for box in (np.float32(55.0), np.float32(30.5), np.float32(86.861), np.float32(7.3), np.float32(70.0)):
+        half = np.float32(0.5) * box
+        a = (rng.random(200000).astype(np.float32) * box).astype(np.float32)
+        b = (rng.random(200000).astype(np.float32) * box).astype(np.float32)
+        a[:8] = [box, 0, half, box, half, 0, np.nextafter(half, box), np.nextafter(half, np.float32(0))]
+        b[:8] = [0, box, 0, half, box, half, 0, 0]
+        # and many operands right around the tie
+        a[8:5000] = (half + (rng.random(4992) - 0.5) * 1e-5 * float(box)).astype(np.float32)
+        b[8:5000] = 0
+        t = (a - b).astype(np.float32)
+        inv = (np.float32(1.0) / box).astype(np.float32)
+        r = np.rint((t * inv).astype(np.float32)).astype(np.float32)
+        assert set(np.unique(r)) <= {-1.0, 0.0, 1.0}
+        got = (t.astype(np.float64) - r.astype(np.float64) * float(box)).astype(np.float32)       # the fma: exact, rounded once
+        assert np.array_equal(got.astype(np.float64), t.astype(np.float64) - r.astype(np.float64) * float(box))   # nothing to round
+        ref = rem(t, np.full_like(t, box))
+        differ = (got * got).view(np.uint32) != (ref * ref).view(np.uint32)
+        assert np.all(np.abs(got[differ]) > 0.49 * box) and np.all(np.abs(ref[differ]) > 0.49 * box)
+        assert differ.sum() < 5000
+
+
 def test_branch_wrap_equals_remainderf():
     """d = a - b with a, b in [0, box]; one conditional +-box must equal remainderf(d, box)."""
     L = ON.lib()
