@@ -91,8 +91,8 @@ class _SortedIndex:
     @property
     def row_ptr(self):
         if self._row_ptr is None:
-            idx = self.index if self.is_sorted else ops.gather_rows(
-                self.index.to(torch.float32).reshape(-1, 1), self.perm).reshape(-1).to(torch.int32)
+            # integer gather (a float32 detour would round node ids above 2^24)
+            idx = self.index if self.is_sorted else self.index[self.perm.long()]
             self._row_ptr = ops.segment_row_ptr(idx.contiguous(), self.n_rows)
         return self._row_ptr
 
@@ -174,6 +174,24 @@ def edge_vectors(graph: Graph, pos: torch.Tensor, box, want_shift=False):
 
 def graph_setup(r0, box, pos, neighbours_max=64, celllist_max=32):
     graph = Graph.radius_graph(r0, box, pos, celllist_max=celllist_max, neighbours_max=neighbours_max)
+    return graph, edge_vectors(graph, pos, box)
+
+
+def graph_setup_capacity(r0, box, pos, capacity, buffers=None):
+    """graph_setup without the device->host copy of the edge count: the edge arrays hold `capacity` edges, of which
+    the first E (graph.stats[0], on the device) are the graph; row_ptr is exact.  Nothing in it synchronises, so the
+    call can be recorded into a HIP graph together with the layers (pass the `buffers` of an earlier call,
+    graph.buffers, so that a replay writes into the same memory).  Entries of src / dst past E are valid but
+    meaningless node indices: only kernels that walk the edges through row_ptr may be used on such a graph
+    (graph.padded is True); per-edge tensors such as r_ij have `capacity` rows."""
+    out = ops.neighbour_edges(pos.contiguous(), r0, box, capacity, out=buffers)
+    batch, nodes = int(pos.shape[0]), int(pos.shape[1])
+    graph = Graph(out["src"], out["dst"], out["edge_counts"], batch, nodes, row_ptr=out["row_ptr"],
+                  cell_order=out["order"])
+    graph.box = box
+    graph.padded = True
+    graph.stats = out["stats"]
+    graph.buffers = out
     return graph, edge_vectors(graph, pos, box)
 
 

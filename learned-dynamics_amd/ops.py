@@ -107,8 +107,8 @@ class NeighbourSearch:
 def neighbour_edges(x, cutoff, box, capacity, out=None):
     """Radius graph into arrays of `capacity` edges without reading the edge count back: one enqueue, no host
     synchronisation (recordable into a HIP graph once `out` holds the buffers of an earlier call).
-    Returns dict(src, dst, row_ptr, edge_counts, stats, workspace); stats[0] (device) is the true edge count, edges
-    beyond the capacity are dropped."""
+    Returns dict(src, dst, row_ptr, edge_counts, stats, workspace, order); stats[0] (device) is the true edge count,
+    edges beyond the capacity are dropped; order is the cell order of the atoms."""
     _check_input(x, "x")
     if x.dim() != 3 or x.size(2) != 3:
         raise RuntimeError("x must have shape (batch, nodes, 3)")
@@ -123,11 +123,16 @@ def neighbour_edges(x, cutoff, box, capacity, out=None):
                        row_ptr=torch.empty(B * N + 1, dtype=torch.int32, device=dev),
                        edge_counts=torch.empty(B, dtype=torch.int32, device=dev),
                        stats=torch.empty(4, dtype=torch.int32, device=dev),
-                       src=torch.empty(int(capacity), dtype=torch.int32, device=dev),
-                       dst=torch.empty(int(capacity), dtype=torch.int32, device=dev))
+                       # zeros: entries past the edge count are never written by the search and must stay valid
+                       # node indices for kernels that run over the whole capacity
+                       src=torch.zeros(int(capacity), dtype=torch.int32, device=dev),
+                       dst=torch.zeros(int(capacity), dtype=torch.int32, device=dev),
+                       order=torch.empty(B * N, dtype=torch.int32, device=dev))
         L.check(_lib.mg_neighbour_edges(_p(x), B, N, float(cutoff), *box, _p(out["workspace"]), out["workspace"].numel(),
                                         _p(out["row_ptr"]), _p(out["edge_counts"]), _p(out["stats"]),
                                         int(out["src"].numel()), _p(out["src"]), _p(out["dst"]), _stream()))
+        L.check(_lib.mg_neighbour_cell_order(_p(out["workspace"]), out["workspace"].numel(), B, N, float(cutoff), *box,
+                                             _p(out["order"]), _stream()))
     return out
 
 

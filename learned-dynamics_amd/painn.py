@@ -259,6 +259,11 @@ class Message(nn.Module):
                 out_a, out_v = ops.painn_table_message(graph.row_ptr, graph.dst32, r_ij, self.filter_table(rows),
                                                        2.0 * self.r0, actv, flat_v, self.epsilon, res_a, res_v)
                 return out_a.reshape(B, N, n), out_v.reshape(B, N, n, 3)
+        if getattr(graph, "padded", False):
+            # the edge arrays are longer than the graph: only the kernels above, which reach the edges through
+            # row_ptr, are valid; the per-edge GEMMs below would also process the rows past the edge count
+            raise RuntimeError("Message.forward on a capacity-sized graph needs the filter-grid path "
+                               "(n a multiple of 16, a grid accepted for these weights, edge capacity >= 4 x grid rows)")
         if actv is None:
             actv = self.mlp_actv(flat_a)
         if ops.painn_filter_message_supported(n, 4 * n, r_ij.shape[0]):
