@@ -261,9 +261,12 @@ int mg_tensor_linear_f16x2_rowmax_parts(long rows, int dim_in, int dim_out);   /
 int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts,
                            long x_rowmax_stride, long x_rows_per_bound, long rows, int dim_in, int dim_out, const float* bias, int act, int accumulate,
                            int out_comps, float* y, float* y_rowmax, mg_stream_t stream);
-/* dW[o,i] = sum_{r,t} dy[r,o,t] x[r,i,t]  (tensor_ops_kern.cu:45-71), dW dense (dim_out,dim_in). */
+/* dW[o,i] = sum_{r,t} dy[r,o,t] x[r,i,t]  (tensor_ops_kern.cu:45-71), dW dense (dim_out,dim_in).  The rows are
+ * reduced in slices whose partial results go to `workspace` (mg_tensor_linear_wgrad_workspace_bytes) and are added
+ * in slice order: no atomics, the same bits on every run. */
+int mg_tensor_linear_wgrad_workspace_bytes(long rows, int dim_in, int dim_out, size_t* bytes /* host */);
 int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows, int dim_in, int dim_out,
-                           float* dW, mg_stream_t stream);
+                           void* workspace, float* dW, mg_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Ant16 (managan/codegen_tensor_products.py:19-34; ant16_o0_cuda / ant16_o1_cuda / ant16_o2_cuda /

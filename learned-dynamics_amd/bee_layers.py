@@ -19,6 +19,7 @@ ill-conditioned: alternating coefficients up to ~1e5).
 import torch
 import torch.nn as nn
 
+from . import differentiable as diff
 from . import ops
 from .codegen_tensor_products import Bee
 from .graph_layers import Graph
@@ -95,6 +96,9 @@ class TensGroupNorm(nn.Module):
 
     def forward(self, x, res=None):
         """gamma * x / sqrt(eps + second moment of the group) (+ res)."""
+        if diff.wants_grad(self, x, res):
+            y = diff.tens_group_norm(self, x)
+            return y if res is None else y + res
         return ops.group_norm(ops.GN_TENSOR, x.contiguous(), self.groups, self.gamma.reshape(-1).contiguous(), None,
                               self.epsilon, res=res)
 
@@ -117,6 +121,9 @@ class SelfTensProds(nn.Module):
 
     def forward(self, x_a, x_v, x_d, residual=False):
         """Returns the three normalised product features, or x + them with residual=True."""
+        if diff.wants_grad(self, x_a, x_v, x_d):
+            y = diff.self_tens_prods(self, x_a, x_v, x_d)
+            return tuple(x + t for x, t in zip((x_a, x_v, x_d), y)) if residual else y
         in_a, in_v, in_d = x_a, x_v, x_d
         *rest, dim_a = x_a.shape
         dim_v, dim_d = x_v.shape[-2], x_d.shape[-3]
@@ -182,6 +189,9 @@ class MLP(nn.Module):
     def forward(self, x, plus_identity=False, bound=None):
         """Returns mlp(x), or x + mlp(x) with plus_identity=True.  bound: upper bounds of the row
         maxima of |x| ((rows, 1) or (1, 1)) if the caller has them."""
+        if diff.wants_grad(self, x):
+            y = diff.mlp_leaky(self, x)
+            return x + y if plus_identity else y
         lead = x.shape[:-1]
         x2 = x.reshape(-1, x.shape[-1]).contiguous()
         Wd = self.lin_direct.weight
@@ -246,6 +256,8 @@ class DisplacementTensors(nn.Module):
 
     def forward(self, graph: Graph, r_ij):
         """r_ij (edges, 3) -> A_a (batch, nodes, dim_a), A_v (batch, nodes, dim_v, 3), A_d (batch, nodes, dim_d, 3, 3)."""
+        if diff.wants_grad(self, r_ij):
+            raise RuntimeError("DisplacementTensors has no differentiable path: call it under torch.no_grad()")
         r_ij = r_ij.contiguous()
         enc, _ = ops.bee_edge_geometry(r_ij, self.r0)                            # radial_encode_8: (edges, 8)
         first = self.mlp_radial[0]
@@ -278,6 +290,8 @@ class Messages(nn.Module):
         Returns 0.1 * sum over edges of the messages: (B_a, B_v, B_d) with the input shapes.
         node_order: row processing order of the edge kernel ("cell": the graph's cell order when it has
         one, None: index order, or an int32 tensor); it does not change the results."""
+        if diff.wants_grad(self, r_ij, x_a, x_v, x_d):
+            return diff.bee_messages(self, graph, r_ij, x_a, x_v, x_d)
         if isinstance(node_order, str):
             node_order = getattr(graph, "cell_order", None)
         B, N = x_a.shape[:2]

@@ -54,18 +54,55 @@ class Ant16(torch.autograd.Function):
 
 
 class Bee(torch.autograd.Function):
+    """The 13 products y = P(l, r) (managan/codegen_tensor_products.py:64-75).  P is bilinear, so the three kernels
+    (forward, gradient for l, gradient for r) are each other's derivatives:
+        <g, BWL(r, dy)> = <P(g, r), dy>,   <g, BWR(l, dy)> = <P(l, g), dy>.
+    The backward passes are written with the autograd functions below, which makes Bee differentiable any number of
+    times (the meanflow loss takes a Jacobian-vector product with create_graph=True)."""
+
     @staticmethod
     def forward(ctx, l_0, l_1, l_2, r_0, r_1, r_2):
         ctx.save_for_backward(l_0, l_1, l_2, r_0, r_1, r_2)
-        return tuple(ops.bee_fwd(l_0, l_1, l_2, r_0, r_1, r_2))
+        return tuple(ops.bee_fwd(*_c((l_0, l_1, l_2, r_0, r_1, r_2))))
 
     @staticmethod
     def backward(ctx, *dys):
         l_0, l_1, l_2, r_0, r_1, r_2 = ctx.saved_tensors
-        dys = _c(dys)
-        dl = ops.bee_bwl(r_0, r_1, r_2, *dys)
-        dr = ops.bee_bwr(l_0, l_1, l_2, *dys)
+        dl = _BeeGradLeft.apply(r_0, r_1, r_2, *dys) if any(ctx.needs_input_grad[:3]) else (None, None, None)
+        dr = _BeeGradRight.apply(l_0, l_1, l_2, *dys) if any(ctx.needs_input_grad[3:]) else (None, None, None)
         return (*dl, *dr)
+
+
+class _BeeGradLeft(torch.autograd.Function):
+    """(r, dy) -> dl = BWL(r, dy) (bee_bwl_cuda)."""
+
+    @staticmethod
+    def forward(ctx, r_0, r_1, r_2, *dys):
+        ctx.save_for_backward(r_0, r_1, r_2, *dys)
+        return tuple(ops.bee_bwl(*_c((r_0, r_1, r_2)), *_c(dys)))
+
+    @staticmethod
+    def backward(ctx, g_0, g_1, g_2):
+        r_0, r_1, r_2, *dys = ctx.saved_tensors
+        d_r = _BeeGradRight.apply(g_0, g_1, g_2, *dys) if any(ctx.needs_input_grad[:3]) else (None, None, None)
+        d_dy = Bee.apply(g_0, g_1, g_2, r_0, r_1, r_2) if any(ctx.needs_input_grad[3:]) else (None,) * 13
+        return (*d_r, *d_dy)
+
+
+class _BeeGradRight(torch.autograd.Function):
+    """(l, dy) -> dr = BWR(l, dy) (bee_bwr_cuda)."""
+
+    @staticmethod
+    def forward(ctx, l_0, l_1, l_2, *dys):
+        ctx.save_for_backward(l_0, l_1, l_2, *dys)
+        return tuple(ops.bee_bwr(*_c((l_0, l_1, l_2)), *_c(dys)))
+
+    @staticmethod
+    def backward(ctx, g_0, g_1, g_2):
+        l_0, l_1, l_2, *dys = ctx.saved_tensors
+        d_l = _BeeGradLeft.apply(g_0, g_1, g_2, *dys) if any(ctx.needs_input_grad[:3]) else (None, None, None)
+        d_dy = Bee.apply(l_0, l_1, l_2, g_0, g_1, g_2) if any(ctx.needs_input_grad[3:]) else (None,) * 13
+        return (*d_l, *d_dy)
 
 
 class Cow0(torch.autograd.Function):

@@ -14,9 +14,10 @@ assembly of reference parts; every part is parity-checked on its own.
 import torch
 import torch.nn as nn
 
+from . import differentiable as diff
 from . import ops
 from .bee_layers import Messages, SelfTensProds
-from .graph_layers import graph_setup
+from .painn import graph_setup
 from .tensor_products import TensLinear
 
 
@@ -36,6 +37,8 @@ class TimeEmbedding(nn.Module):
 
     def forward(self, st):
         emb = self.raw_t_embed(st).contiguous()
+        if diff.wants_grad(self, emb):
+            return diff.linear(self.lin1, emb)
         return ops.tensor_linear_fwd(0, self.lin1.weight, emb, bias=self.lin1.bias)
 
 
@@ -62,7 +65,10 @@ class Denoiser(nn.Module):
         s, t = st
         B, N = x1.shape[:2]
         dim_a, dim_v, dim_d = self.dims
-        x_a = ops.tensor_linear_fwd(0, self.embed.weight, one_hot.contiguous(), bias=self.embed.bias)
+        if diff.wants_grad(self, x0, x1):
+            x_a = diff.linear(self.embed, one_hot)
+        else:
+            x_a = ops.tensor_linear_fwd(0, self.embed.weight, one_hot.contiguous(), bias=self.embed.bias)
         x_a = x_a + self.t_embed(st)[:, None]
         x_v = self.v_readin((x1 - x0)[..., None, :].contiguous())
         x_d = torch.zeros(B, N, dim_d, 3, 3, device=x1.device)

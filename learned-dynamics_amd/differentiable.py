@@ -1,0 +1,178 @@
+"""The layers as the reference writes them, out of differentiable pieces: what the modules run when a gradient is
+asked for (training, or the Jacobian-vector product of the meanflow loss, archs/meanflow_painn8.py:274-282).
+
+The fused inference kernels have no backward pass.  Every heavy operation here is an autograd function of this
+package whose forward AND backward passes are HIP kernels (tensor_linear with its weight / input gradients, the 13
+products with their two gradient kernels, gather and segment sum, which are each other's adjoints) and whose
+backward is itself differentiable; the elementwise glue in between (activations, norms, the radial encodings, the
+cross product, the periodic wrap) is plain torch arithmetic on the device, which autograd differentiates as it does
+for the reference.  Results equal the fused path up to fp32 summation order (tests/test_gpu_autograd.py).
+"""
+import math
+
+import torch
+import torch.nn.functional as F
+
+from . import graph_layers as gl
+from .codegen_tensor_products import Bee
+from .tensor_products import tensor_linear
+
+
+def wants_grad(module, *tensors):
+    """True when autograd is recording and a gradient could flow to an input or a parameter."""
+    if not torch.is_grad_enabled():
+        return False
+    if any(t is not None and t.requires_grad for t in tensors):
+        return True
+    return any(p.requires_grad for p in module.parameters())
+
+
+def linear(lin, x):
+    """nn.Linear through the tensor_linear kernels (weight and input gradients are kernels too)."""
+    lead = x.shape[:-1]
+    y = tensor_linear(0, lin.weight, x.reshape(-1, x.shape[-1]).contiguous())
+    if lin.bias is not None:
+        y = y + lin.bias
+    return y.reshape(*lead, -1)
+
+
+def mlp_silu(mlp, x):
+    """painn.MLP: Linear, SiLU, Linear, SiLU, Linear (archs/meanflow_painn8.py:38-51)."""
+    L = mlp.layers
+    return linear(L[4], F.silu(linear(L[2], F.silu(linear(L[0], x)))))
+
+
+def mlp_leaky(mlp, x):
+    """bee_layers.MLP: lin_direct(x) + layers(x) with LeakyReLU(0.1) (archs/diffuser_atoms15.py:98-110)."""
+    L = mlp.layers
+    h = F.leaky_relu(linear(L[2], F.leaky_relu(linear(L[0], x), 0.1)), 0.1)
+    return linear(mlp.lin_direct, x) + linear(L[4], h)
+
+
+def radial_encode_painn(r, n, rmax):
+    """archs/meanflow_painn8.py:25-35"""
+    hn = (n + 1) // 2
+    coeffs = (math.pi / rmax) * (1 + torch.arange(0, hn, device=r.device) // 2)
+    phase = coeffs * torch.linalg.vector_norm(r, dim=-1)[..., None]
+    return torch.cat([torch.cos(phase), torch.sin(phase[..., :(n - hn)])], dim=-1)
+
+
+_JACOBI = {}
+
+
+def _jacobi_matrix(device):
+    """Coefficients of the shifted Jacobi polynomials P_i^(1,0)(2x - 1), i < 8 (managan/jacobi_radenc.py:8-22)."""
+    key = str(device)
+    if key not in _JACOBI:
+        A = torch.zeros(8, 9, dtype=torch.float64)
+        for n in range(8):
+            for s in range(n + 1):
+                w = math.comb(n + 1, n - s) * math.comb(n, s)
+                for k in range(s + 1):
+                    A[n, k + n - s] += w * math.comb(s, k) * (-1.0) ** (s - k)
+        _JACOBI[key] = A.to(device)
+    return _JACOBI[key]
+
+
+def radial_encode_8(r, rmax):
+    """managan/jacobi_radenc.py:24-37; the polynomials are evaluated in float64 (Horner) like the inference kernel:
+    their monomial form in fp32 loses three digits."""
+    z = (torch.linalg.vector_norm(r, dim=-1) / rmax)[..., None].double()
+    A = _jacobi_matrix(r.device)
+    acc = A[:, 8].expand(*z.shape[:-1], 8)
+    for k in range(7, -1, -1):
+        acc = acc * z + A[:, k]
+    return (acc * torch.relu(1.0 - z)).to(r.dtype)
+
+
+def tens_sigmoid(inds, x):
+    dims = tuple(-(1 + n) for n in range(inds))
+    xx = (x ** 2).sum(dims, keepdim=True) if inds > 0 else x ** 2
+    return x / torch.sqrt(1.0 + xx)
+
+
+def scal_group_norm(gn, x):
+    """managan/layers_common.py:201-223"""
+    B, N, chan = x.shape
+    xg = x.reshape(B, N, gn.groups, -1)
+    sh = xg - xg.mean([1, 3], keepdim=True)
+    var = (sh ** 2).mean([1, 3], keepdim=True)
+    return gn.beta + gn.gamma * (sh / torch.sqrt(gn.epsilon + var)).reshape(B, N, chan)
+
+
+def tens_group_norm(gn, x):
+    """managan/tensor_products.py:215-232"""
+    B, N, chan = x.shape[:3]
+    xg = x.reshape(B, N, gn.groups, -1, 3 ** gn.inds)
+    m2 = (xg ** 2).sum(-1, keepdim=True).mean([1, 3], keepdim=True)
+    return gn.gamma * (xg / torch.sqrt(gn.epsilon + m2)).reshape(x.shape)
+
+
+def edge_vectors(graph, pos, box):
+    """boxwrap(box, pos[dst] - pos[src]) with a gradient for pos (archs/meanflow_painn8.py:167-172)."""
+    pos_src, pos_dst = gl.edges_read(graph, pos)
+    tbox = torch.tensor(box, device=pos.device, dtype=pos.dtype)
+    return gl.boxwrap(tbox, pos_dst - pos_src)
+
+
+def painn_message(msg, graph, x_a, x_v, r_ij):
+    """archs/meanflow_painn8.py:85-100"""
+    n = msg.n
+    dist = mlp_silu(msg.mlp_dist, radial_encode_painn(r_ij, msg.n_rbf, msg.r0))
+    actv = mlp_silu(msg.mlp_actv, gl.edges_read_dst(graph, x_a))
+    prod = dist * actv
+    direction = r_ij / torch.sqrt(msg.epsilon + (r_ij ** 2).sum(-1, keepdim=True))
+    v = gl.edges_read_dst(graph, x_v)
+    cross = torch.linalg.cross(v, direction[:, None].expand_as(v))
+    m = v * prod[..., :n, None] + cross * prod[..., n:2 * n, None] + direction[:, None] * prod[..., 2 * n:3 * n, None]
+    return gl.edges_reduce_src(graph, prod[..., 3 * n:].contiguous()), gl.edges_reduce_src(graph, m)
+
+
+def painn_update(upd, x_a, x_v):
+    """archs/meanflow_painn8.py:63-75"""
+    n = upd.n
+    v_l, v_r = upd.lin_l(x_v), upd.lin_r(x_v)
+    ip = (v_l * v_r).sum(-1)
+    y = mlp_silu(upd.mlp, torch.cat([x_a, torch.linalg.vector_norm(v_r, dim=-1)], dim=-1))
+    v = upd.lin_v(x_v) * y[..., :n, None]
+    a = scal_group_norm(upd.gn, ip * y[..., n:2 * n]) + y[..., 2 * n:]
+    return a, v / torch.sqrt(1. + (v ** 2).sum(-1, keepdim=True))
+
+
+def apply_tens_prod_submodules(module, prods):
+    """archs/diffuser_atoms15.py:52-57"""
+    from .ops import BEE_ORDER
+    out = [None, None, None]
+    for lab, p in zip(BEE_ORDER, prods):
+        y = getattr(module, f"Y_{lab}")(p)
+        k = int(lab[2])
+        out[k] = y if out[k] is None else out[k] + y
+    return tuple(out)
+
+
+def bee_messages(msg, graph, r_ij, x_a, x_v, x_d):
+    """archs/diffuser_atoms15.py:238-253"""
+    enc = linear(msg.lin_enc, radial_encode_8(r_ij, msg.r0))
+    rh = tens_sigmoid(1, r_ij * (7. / msg.r0))
+    phi_a = enc
+    phi_v = enc[..., None] * rh[..., None, :]
+    phi_d = enc[..., None, None] * rh[..., None, None, :] * rh[..., None, :, None]
+    a_j = gl.edges_read_dst(graph, msg.L0(x_a))
+    v_j = gl.edges_read_dst(graph, msg.L1(x_v))
+    d_j = gl.edges_read_dst(graph, msg.L2(x_d))
+    prods = Bee.apply(a_j, v_j, d_j, phi_a.contiguous(), phi_v.contiguous(), phi_d.contiguous())
+    psi_a, psi_v, psi_d = apply_tens_prod_submodules(msg, prods)
+    psi_a = psi_a + mlp_leaky(msg.mlp_a, psi_a)
+    return (0.1 * gl.edges_reduce_src(graph, psi_a), 0.1 * gl.edges_reduce_src(graph, psi_v),
+            0.1 * gl.edges_reduce_src(graph, psi_d))
+
+
+def self_tens_prods(mod, x_a, x_v, x_d):
+    """archs/diffuser_atoms15.py:75-95"""
+    *rest, dim_a = x_a.shape
+    dim_v, dim_d = x_v.shape[-2], x_d.shape[-3]
+    a, v, d = x_a.reshape(-1, dim_a), x_v.reshape(-1, dim_v, 3), x_d.reshape(-1, dim_d, 3, 3)
+    prods = Bee.apply(mod.L0(a), mod.L1(v), mod.L2(d), mod.R0(a), mod.R1(v), mod.R2(d))
+    y_a, y_v, y_d = apply_tens_prod_submodules(mod, prods)
+    return (tens_group_norm(mod.gn_a, y_a.reshape(*rest, dim_a)), tens_group_norm(mod.gn_v, y_v.reshape(*rest, dim_v, 3)),
+            tens_group_norm(mod.gn_d, y_d.reshape(*rest, dim_d, 3, 3)))

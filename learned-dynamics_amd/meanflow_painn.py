@@ -7,6 +7,7 @@ one-hot type vectors, and the topology an OpenMMMetadata carries is passed as a 
 import torch
 import torch.nn as nn
 
+from . import differentiable as diff
 from . import ops
 from .denoiser import TimeEmbedding
 from .graph_layers import Graph
@@ -42,6 +43,8 @@ class OneHotAtomEmbed(nn.Module):
         self.lin = nn.Linear(atom_types, n)
 
     def forward(self, topology: Topology):
+        if diff.wants_grad(self):
+            return diff.linear(self.lin, topology.one_hot)
         return ops.tensor_linear_fwd(0, self.lin.weight, topology.one_hot.contiguous(), bias=self.lin.bias)
 
 

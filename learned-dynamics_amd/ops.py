@@ -839,7 +839,10 @@ def tensor_linear_wgrad(inds, dy, x):
         rows *= int(x.size(i))
     with torch.cuda.device(x.device):
         dW = torch.empty(dim_out, dim_in, dtype=torch.float32, device=x.device)
-        L.check(_lib.mg_tensor_linear_wgrad(inds, _p(dy), _p(x), rows, dim_in, dim_out, _p(dW), _stream()))
+        nbytes = ctypes.c_size_t(0)
+        L.check(_lib.mg_tensor_linear_wgrad_workspace_bytes(rows, dim_in, dim_out, ctypes.byref(nbytes)))
+        ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
+        L.check(_lib.mg_tensor_linear_wgrad(inds, _p(dy), _p(x), rows, dim_in, dim_out, _p(ws), _p(dW), _stream()))
     return dW
 
 

@@ -19,9 +19,19 @@ import math
 import torch
 import torch.nn as nn
 
+from . import differentiable as diff
 from . import ops
-from .graph_layers import Graph, graph_setup
+from .graph_layers import Graph
+from .graph_layers import graph_setup as _graph_setup
 from .tensor_products import TensLinear
+
+
+def graph_setup(r0, box, pos, neighbours_max=64, celllist_max=32):
+    """archs/meanflow_painn8.py:167-172; the edge vectors carry a gradient for pos when one is asked for."""
+    graph, r_ij = _graph_setup(r0, box, pos.detach(), neighbours_max=neighbours_max, celllist_max=celllist_max)
+    if torch.is_grad_enabled() and pos.requires_grad:
+        r_ij = diff.edge_vectors(graph, pos, box)
+    return graph, r_ij
 
 
 def radial_encode(r, n, rmax):
@@ -60,6 +70,8 @@ class MLP(nn.Module):
         )
 
     def forward(self, x_a, bound=None):
+        if diff.wants_grad(self, x_a):
+            return diff.mlp_silu(self, x_a)
         lead = x_a.shape[:-1]
         h = x_a.reshape(-1, x_a.shape[-1]).contiguous()
         h, bound = _linear(h, self.layers[0], ops.ACT_SILU, bound)
@@ -108,6 +120,9 @@ class Update(nn.Module):
 
     def forward(self, x_a, x_v, residual=False):
         """Returns (dx_a, dx_v), or (x_a + dx_a, x_v + dx_v) with residual=True."""
+        if diff.wants_grad(self, x_a, x_v):
+            da, dv = diff.painn_update(self, x_a, x_v)
+            return (x_a + da, x_v + dv) if residual else (da, dv)
         n = self.n
         B, N = x_a.shape[:2]
         rows = B * N
@@ -235,6 +250,9 @@ class Message(nn.Module):
     def forward(self, graph: Graph, x_a, x_v, r_ij, residual=False):
         """x_a: (batch, atoms, n), x_v: (batch, atoms, n, 3), r_ij: (edges, 3).
         Returns (dx_a, dx_v), or (x_a + dx_a, x_v + dx_v) with residual=True."""
+        if diff.wants_grad(self, x_a, x_v, r_ij):
+            da, dv = diff.painn_message(self, graph, x_a, x_v, r_ij)
+            return (x_a + da, x_v + dv) if residual else (da, dv)
         B, N, n = x_a.shape
         flat_a = x_a.reshape(B * N, n).contiguous()
         flat_v = x_v.reshape(B * N, n, 3).contiguous()

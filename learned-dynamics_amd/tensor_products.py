@@ -9,13 +9,16 @@ from . import ops
 
 
 class _TensorLinearFn(torch.autograd.Function):
-    """tensor_linear with gradients for W and x (extensions/tensor_ops/tensor_ops.cpp:31-169)."""
+    """tensor_linear with gradients for W and x (extensions/tensor_ops/tensor_ops.cpp:31-169).  The backward pass is
+    itself made of differentiable functions (this one and _WeightGradFn), so the operation can be differentiated any
+    number of times, as torch.autograd.functional.jvp(create_graph=True) of the meanflow loss needs
+    (archs/meanflow_painn8.py:274-282); the reference's C++ backward calls raw kernels and cannot."""
 
     @staticmethod
     def forward(ctx, inds, W, x):
         ctx.inds = inds
         ctx.save_for_backward(W, x)
-        return ops.tensor_linear_fwd(inds, W, x)
+        return ops.tensor_linear_fwd(inds, W, x.contiguous())
 
     @staticmethod
     def backward(ctx, dy):
@@ -23,10 +26,31 @@ class _TensorLinearFn(torch.autograd.Function):
         dy = dy.contiguous()
         dW = dx = None
         if ctx.needs_input_grad[1]:
-            dW = ops.tensor_linear_wgrad(ctx.inds, dy, x)
+            dW = _WeightGradFn.apply(ctx.inds, dy, x)
         if ctx.needs_input_grad[2]:
-            dx = ops.tensor_linear_fwd(ctx.inds, W.t(), dy)   # strides of W are honoured: no copy
+            dx = _TensorLinearFn.apply(ctx.inds, W.t(), dy)   # strides of W are honoured: no copy
         return None, dW, dx
+
+
+class _WeightGradFn(torch.autograd.Function):
+    """dW[o, i] = sum over rows and components of dy[.., o, :] x[.., i, :]: bilinear in (dy, x), and its own
+    gradients are two tensor_linear calls."""
+
+    @staticmethod
+    def forward(ctx, inds, dy, x):
+        ctx.inds = inds
+        ctx.save_for_backward(dy, x)
+        return ops.tensor_linear_wgrad(inds, dy.contiguous(), x.contiguous())
+
+    @staticmethod
+    def backward(ctx, ddW):
+        dy, x = ctx.saved_tensors
+        g_dy = g_x = None
+        if ctx.needs_input_grad[1]:
+            g_dy = _TensorLinearFn.apply(ctx.inds, ddW, x)            # (.., o, :) = ddW x
+        if ctx.needs_input_grad[2]:
+            g_x = _TensorLinearFn.apply(ctx.inds, ddW.t(), dy)        # (.., i, :) = ddW^T dy
+        return None, g_dy, g_x
 
 
 def tensor_linear(inds, W, x):

@@ -40,8 +40,14 @@ def radius_graph(pos, r0, box):
     The graph and the fp32 edge vectors come from the C oracle, as the device computes them."""
     p32 = pos.detach().to(torch.float32).numpy()
     ref = ON.edges(p32, r0, box)
+    src, dst = torch.from_numpy(ref["src"]).long(), torch.from_numpy(ref["dst"]).long()
+    if pos.requires_grad:
+        # a gradient for the positions is wanted: the same wrap as torch arithmetic (managan/graph_layers.py:62-66)
+        flat = pos.reshape(-1, 3)
+        tbox = torch.tensor(box, dtype=pos.dtype)
+        return src, dst, OL.boxwrap(tbox, flat[dst] - flat[src])
     r = ON.edge_vectors(p32, ref["src"], ref["dst"], box)
-    return torch.from_numpy(ref["src"]).long(), torch.from_numpy(ref["dst"]).long(), torch.from_numpy(r).to(pos.dtype)
+    return src, dst, torch.from_numpy(r).to(pos.dtype)
 
 
 def block(sd, prefix, tup, r0, n, dtype):

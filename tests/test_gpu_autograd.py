@@ -1,0 +1,236 @@
+"""Gradients of the layers on the GPU against the oracle's autograd (the same formulas on the CPU in float64):
+first derivatives with respect to inputs, edge vectors and weights for the PaiNN Message / Update and the rank-0/1/2
+Messages / SelfTensProds; the differentiable path against the fused inference path; second-order use as the meanflow
+loss makes it (torch.autograd.functional.jvp with create_graph=True followed by a backward pass,
+archs/meanflow_painn8.py:274-296) through TensLinear, the 13 products, gathers and segment sums and through the whole
+PaiNN meanflow denoiser; and the weight gradient's run-to-run reproducibility."""
+import importlib
+
+import pytest
+import torch
+
+from oracle import layers as OL
+from oracle import models as OM
+from oracle import products as OP
+
+pytestmark = pytest.mark.gpu
+F64 = torch.float64
+
+
+def _mlp_w(mlp, dt=F64):
+    L = mlp.layers
+    return {"W1": L[0].weight.detach().cpu().to(dt), "b1": L[0].bias.detach().cpu().to(dt),
+            "W2": L[2].weight.detach().cpu().to(dt), "b2": L[2].bias.detach().cpu().to(dt),
+            "W3": L[4].weight.detach().cpu().to(dt), "b3": L[4].bias.detach().cpu().to(dt)}
+
+
+def _close(got, ref, what, tol=2e-5):
+    got, ref = got.detach().cpu().double(), ref.detach().double()
+    scale = max(1.0, float(ref.abs().max()))
+    err = float((got - ref).abs().max())
+    assert err <= tol * scale, f"{what}: max err {err:.3g} at scale {scale:.3g}"
+
+
+def _ring(N, k, gen):
+    src = torch.arange(N).repeat_interleave(k)
+    dst = (src + torch.randint(1, N, (N * k,), generator=gen)) % N
+    return src, dst
+
+
+def test_painn_message_and_update_gradients(pkg):
+    painn = importlib.import_module("learned-dynamics_amd.painn")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    torch.manual_seed(3)
+    n, n_rbf, N, r0 = 16, 8, 40, 5.0
+    gen = torch.Generator().manual_seed(4)
+    src, dst = _ring(N, 6, gen)
+    msg, upd = painn.Message(r0, n, n_rbf).cuda(), painn.Update(n).cuda()
+    with torch.no_grad():
+        upd.gn.gamma.normal_(); upd.gn.beta.normal_()
+    x_a = torch.randn(1, N, n, generator=gen)
+    x_v = torch.randn(1, N, n, 3, generator=gen)
+    r = torch.randn(len(src), 3, generator=gen) * 2
+    ca, cv = torch.randn(1, N, n, generator=gen), torch.randn(1, N, n, 3, generator=gen)
+    graph = gl.Graph(src.cuda(), dst.cuda(), None, 1, N)
+    # device
+    xa_d, xv_d, r_d = (t.cuda().requires_grad_(True) for t in (x_a, x_v, r))
+    da, dv = msg(graph, xa_d, xv_d, r_d)
+    ua, uv = upd(xa_d + da, xv_d + dv)
+    loss = (ua * ca.cuda()).sum() + (uv * cv.cuda()).sum() + (da ** 2).sum()
+    loss.backward()
+    # oracle, float64
+    xa_o, xv_o, r_o = (t.double().requires_grad_(True) for t in (x_a, x_v, r))
+    wd, wa = _mlp_w(msg.mlp_dist), _mlp_w(msg.mlp_actv)
+    for w in (wd, wa):
+        for v in w.values():
+            v.requires_grad_(True)
+    wu = {"W_l": upd.lin_l.W.detach().cpu().double().requires_grad_(True), "W_r": upd.lin_r.W.detach().cpu().double().requires_grad_(True),
+          "W_v": upd.lin_v.W.detach().cpu().double().requires_grad_(True), "mlp": _mlp_w(upd.mlp),
+          "gn_gamma": upd.gn.gamma.detach().cpu().double().requires_grad_(True), "gn_beta": upd.gn.beta.detach().cpu().double().requires_grad_(True)}
+    for v in wu["mlp"].values():
+        v.requires_grad_(True)
+    oa, ov = OL.painn_message(src, dst, 1, N, xa_o, xv_o, r_o, wd, wa, r0, n, n_rbf)
+    qa, qv = OL.painn_update(xa_o + oa, xv_o + ov, wu, n)
+    ((qa * ca.double()).sum() + (qv * cv.double()).sum() + (oa ** 2).sum()).backward()
+    _close(da, oa, "forward dx_a"); _close(uv, qv, "forward update v")
+    _close(xa_d.grad, xa_o.grad, "d/dx_a"); _close(xv_d.grad, xv_o.grad, "d/dx_v"); _close(r_d.grad, r_o.grad, "d/dr_ij")
+    _close(msg.mlp_dist.layers[0].weight.grad, wd["W1"].grad, "d/dW1 of mlp_dist")
+    _close(msg.mlp_actv.layers[4].bias.grad, wa["b3"].grad, "d/db3 of mlp_actv")
+    _close(upd.lin_r.W.grad, wu["W_r"].grad, "d/dW_r"); _close(upd.gn.gamma.grad, wu["gn_gamma"].grad, "d/dgamma")
+    _close(upd.mlp.layers[2].weight.grad, wu["mlp"]["W2"].grad, "d/dW2 of the update MLP")
+    # and the differentiable path gives what the fused inference path gives
+    with torch.no_grad():
+        fa, fv = msg(graph, x_a.cuda(), x_v.cuda(), r.cuda())
+    _close(da, fa.cpu(), "differentiable vs fused dx_a", 5e-6); _close(dv, fv.cpu(), "differentiable vs fused dx_v", 5e-6)
+
+
+def test_bee_layers_gradients(pkg):
+    bee = importlib.import_module("learned-dynamics_amd.bee_layers")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    torch.manual_seed(5)
+    dims, chan, N, r0 = (12, 8, 4), 16, 30, 6.0
+    gen = torch.Generator().manual_seed(6)
+    src, dst = _ring(N, 5, gen)
+    msg, prod = bee.Messages(r0, *dims, chan).cuda(), bee.SelfTensProds(*dims, chan, groups=2).cuda()
+    xs = [torch.randn(1, N, dims[0], generator=gen), torch.randn(1, N, dims[1], 3, generator=gen),
+          torch.randn(1, N, dims[2], 3, 3, generator=gen)]
+    r = torch.randn(len(src), 3, generator=gen) * 2
+    cs = [torch.randn_like(t) for t in xs]
+    graph = gl.Graph(src.cuda(), dst.cuda(), None, 1, N)
+    xd = [t.cuda().requires_grad_(True) for t in xs]
+    r_d = r.cuda().requires_grad_(True)
+    B = msg(graph, r_d, *xd)
+    Y = prod(*[x + b for x, b in zip(xd, B)])
+    sum((y * c.cuda()).sum() for y, c in zip(Y, cs)).backward()
+    dd = lambda p: p.detach().cpu().double().requires_grad_(True)
+    Lm = msg.mlp_a.layers
+    w = {"L0": dd(msg.L0.W), "L1": dd(msg.L1.W), "L2": dd(msg.L2.W), "Y": {lab: dd(getattr(msg, f"Y_{lab}").W) for lab in OP.BEE_ORDER},
+         "enc_W": dd(msg.lin_enc.weight), "enc_b": dd(msg.lin_enc.bias),
+         "mlp_a": {"W_direct": dd(msg.mlp_a.lin_direct.weight), "W1": dd(Lm[0].weight), "b1": dd(Lm[0].bias), "W2": dd(Lm[2].weight),
+                   "b2": dd(Lm[2].bias), "W3": dd(Lm[4].weight), "b3": dd(Lm[4].bias)}}
+    ws = {k: dd(getattr(prod, k).W) for k in ("L0", "R0", "L1", "R1", "L2", "R2")}
+    ws["Y"] = {lab: dd(getattr(prod, f"Y_{lab}").W) for lab in OP.BEE_ORDER}
+    ws.update(gn_a=dd(prod.gn_a.gamma), gn_v=dd(prod.gn_v.gamma), gn_d=dd(prod.gn_d.gamma))
+    xo = [t.double().requires_grad_(True) for t in xs]
+    r_o = r.double().requires_grad_(True)
+    Bo = OL.bee_messages(src, dst, 1, N, r_o, *xo, w, r0)
+    Yo = OL.self_tens_prods(*[x + b for x, b in zip(xo, Bo)], ws, groups=2)
+    sum((y * c.double()).sum() for y, c in zip(Yo, cs)).backward()
+    for k in range(3):
+        _close(Y[k], Yo[k], f"forward rank {k}")
+        _close(xd[k].grad, xo[k].grad, f"d/dx rank {k}")
+    _close(r_d.grad, r_o.grad, "d/dr_ij")
+    _close(msg.Y_212.W.grad, w["Y"]["212"].grad, "d/dY_212 (Messages)")
+    _close(msg.lin_enc.weight.grad, w["enc_W"].grad, "d/d lin_enc")
+    _close(msg.mlp_a.layers[2].weight.grad, w["mlp_a"]["W2"].grad, "d/dW2 of mlp_a")
+    _close(prod.R1.W.grad, ws["R1"].grad, "d/dR1"); _close(prod.Y_111.W.grad, ws["Y"]["111"].grad, "d/dY_111 (SelfTensProds)")
+    _close(prod.gn_d.gamma.grad, ws["gn_d"].grad, "d/d gn_d.gamma")
+
+
+def test_second_order_through_linear_products_gather_and_scatter(pkg):
+    """jvp(create_graph=True) of f(x) = scatter(Y(Bee(L x, R gather(x)))) and a backward pass through the result,
+    against the same thing on the oracle's functions."""
+    tp = importlib.import_module("learned-dynamics_amd.tensor_products")
+    cg = importlib.import_module("learned-dynamics_amd.codegen_tensor_products")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    gen = torch.Generator().manual_seed(7)
+    N, C = 12, 8
+    src, dst = _ring(N, 3, gen)
+    graph = gl.Graph(src.cuda(), dst.cuda(), None, 1, N)
+    W = [torch.randn(C, C, generator=gen) * 0.4 for _ in range(7)]
+    xs = [torch.randn(1, N, C, generator=gen), torch.randn(1, N, C, 3, generator=gen), torch.randn(1, N, C, 3, 3, generator=gen)]
+    vs = [torch.randn_like(t) for t in xs]
+
+    def f_dev(Wd):
+        def f(a, v, d):
+            l = [tp.tensor_linear(k, Wd[k], t.reshape(N, C, *([3] * k))) for k, t in enumerate((a, v, d))]
+            r = [gl.edges_read_dst(graph, tp.tensor_linear(k, Wd[3 + k], t).contiguous()) for k, t in enumerate((a, v, d))]
+            l = [t[src.cuda()] for t in l]
+            prods = cg.Bee.apply(*l, *r)
+            y = tp.tensor_linear(1, Wd[6], prods[11]) + prods[5] + prods[3] + prods[4] + prods[6]   # 111 (chiral), 121, 011, 101, 211
+            return gl.edges_reduce_src(graph, y)
+        return f
+
+    def f_ref(Wr):
+        def f(a, v, d):
+            l = [OP.tensor_linear(k, Wr[k], t.reshape(N, C, *([3] * k)))[src] for k, t in enumerate((a, v, d))]
+            r = [OL.edges_read_dst(dst, OP.tensor_linear(k, Wr[3 + k], t), 1, N) for k, t in enumerate((a, v, d))]
+            prods = OP.bee(*l, *r)
+            y = OP.tensor_linear(1, Wr[6], prods[11]) + prods[5] + prods[3] + prods[4] + prods[6]
+            return OL.edges_reduce_src(src, y, 1, N)
+        return f
+
+    Wd = [w.cuda().requires_grad_(True) for w in W]
+    xd = tuple(t.cuda().requires_grad_(True) for t in xs)
+    out_d, jvp_d = torch.autograd.functional.jvp(f_dev(Wd), xd, tuple(v.cuda() for v in vs), create_graph=True)
+    (jvp_d ** 2).sum().backward()
+    Wr = [w.double().requires_grad_(True) for w in W]
+    xr = tuple(t.double().requires_grad_(True) for t in xs)
+    out_r, jvp_r = torch.autograd.functional.jvp(f_ref(Wr), xr, tuple(v.double() for v in vs), create_graph=True)
+    (jvp_r ** 2).sum().backward()
+    _close(out_d, out_r, "f"); _close(jvp_d, jvp_r, "jvp")
+    for k in range(3):
+        _close(xd[k].grad, xr[k].grad, f"d(jvp^2)/dx rank {k}", 1e-4)
+    for k in range(7):
+        _close(Wd[k].grad, Wr[k].grad, f"d(jvp^2)/dW[{k}]", 1e-4)
+
+
+def test_meanflow_loss_through_the_painn_denoiser(pkg):
+    """v_target = v - (t - s) jvp, loss = mean (v_pred - v_target)^2, loss.backward(): the reference's training step
+    (archs/meanflow_painn8.py:274-296) on a small PaiNN meanflow denoiser with positions that move, against the oracle."""
+    mp = importlib.import_module("learned-dynamics_amd.meanflow_painn")
+    torch.manual_seed(0x947 + 9)
+    B, N, n, r0, L = 1, 48, 8, 5.0, 30.0
+    box = (L, L, L)
+    model = mp.SE3ITO(r0, n, N, blks_0=1, blks_1=1, mutate_pos=True).cuda()
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if name.endswith("lin_push_pos.W"):
+                p.mul_(0.05)
+    sd = {k: v.detach().cpu().double().requires_grad_(True) for k, v in model.state_dict().items()}
+    gen = torch.Generator().manual_seed(2)
+    steps = torch.randn(B, N, 3, generator=gen)
+    x_prev = (2.0 * steps / steps.norm(dim=-1, keepdim=True)).cumsum(1) + 0.5 * L
+    z_0 = x_prev + 0.2 * torch.randn(B, N, 3, generator=gen)
+    z_1 = x_prev + 0.5 * torch.randn(B, N, 3, generator=gen)
+    t, s = torch.tensor([0.7]), torch.tensor([0.2])
+    one_hot = torch.nn.functional.one_hot(torch.randint(0, 20, (N,), generator=gen), 20).float()
+    i = torch.arange(N - 1)
+    bs, bd = torch.cat([i, i + 1]), torch.cat([i + 1, i])
+    topo = mp.Topology(one_hot.cuda(), bs.cuda(), bd.cuda())
+
+    def loss_of(dn, to):
+        z_t = to(t)[:, None, None] * to(z_1) + (1 - to(t)[:, None, None]) * to(z_0)
+        v = to(z_1) - to(z_0)
+        f = lambda zz, tt: dn((to(s), tt), to(x_prev), zz)
+        _, jvp = torch.autograd.functional.jvp(f, (z_t, to(t)), (v, torch.ones_like(to(t))), create_graph=True)
+        v_target = v - (to(t) - to(s))[:, None, None] * jvp
+        v_pred = dn((to(s), to(t)), to(x_prev), z_t)
+        return ((v_pred - v_target) ** 2).mean(), jvp
+
+    loss_d, jvp_d = loss_of(lambda st, x0, z: model(st, x0, z, box, topo), lambda a: a.cuda())
+    loss_d.backward()
+    loss_r, jvp_r = loss_of(lambda st, x0, z: OM.se3ito(sd, st, x0, z, box, one_hot.double(), bs, bd, r0, n, 1, 1, F64),
+                            lambda a: a.double())
+    loss_r.backward()
+    _close(jvp_d, jvp_r, "jvp of the denoiser", 1e-4)
+    assert abs(float(loss_d.detach()) - float(loss_r.detach())) <= 1e-4 * max(1.0, abs(float(loss_r.detach())))
+    checked = 0
+    for name, p in model.named_parameters():
+        if p.grad is None:
+            continue
+        ref = sd[name].grad
+        assert ref is not None, name
+        _close(p.grad, ref, f"d loss / d {name}", 5e-4)
+        checked += 1
+    assert checked >= 40
+
+
+def test_weight_gradient_is_reproducible(ops):
+    g = torch.Generator().manual_seed(8)
+    dy, x = torch.randn(30000, 96, 3, generator=g).cuda(), torch.randn(30000, 64, 3, generator=g).cuda()
+    a = ops.tensor_linear_wgrad(1, dy, x)
+    for _ in range(3):
+        assert torch.equal(ops.tensor_linear_wgrad(1, dy, x), a)
+    ref = torch.einsum("rot,rit->oi", dy.double().cpu(), x.double().cpu())
+    torch.testing.assert_close(a.cpu().double(), ref, rtol=1e-5, atol=2e-5 * float(ref.abs().max()))
