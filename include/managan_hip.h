@@ -272,7 +272,7 @@ int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows,
  * Ant16 (managan/codegen_tensor_products.py:19-34; ant16_o0_cuda / ant16_o1_cuda / ant16_o2_cuda /
  * ant16_oc_cuda, extensions/codegen_tensops/codegen_tensops.cpp:610-667,823-890,1072-1140,1327-1390):
  *   y[b,o,:] (+)= sum_t sum_{i<dim_l, j<dim_r} P_t[o,i,j] * (left_t[b,i,:] (x) x_r[b,j,:])
- * over n_terms <= 4 product types that share the output rank rank_o.  labels[t] indexes the order
+ * over n_terms <= 6 product types that share the output rank rank_o.  labels[t] indexes the order
  * 000 110 220 011 101 121 211 022 202 112 222 111 212; P_t (dim_o, dim_l, dim_r) and
  * left_t (rows, dim_l, (3,)^rank_l) dense; x_k (rows, dim_k, (3,)^k); y (rows, dim_o, (3,)^rank_o).
  * labels, P and left are HOST arrays of n_terms entries (device pointers inside).  accumulate != 0
@@ -281,6 +281,25 @@ int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows,
 int mg_ant16_fwd(int rank_o, int n_terms, const int* labels, const float* const* P, const float* const* left,
                  const float* x_0, const float* x_1, const float* x_2, long rows, int dim_0, int dim_1, int dim_2,
                  int dim_l, int accumulate, float* y, mg_stream_t stream);
+/* Gradient for x of rank rank_r (ant16_o{0,1,2,c}_backward_cuda, codegen_tensops.cpp:669-821 and the oc variant
+ * at 1374-1420): dx[b,j,:] (+)= sum_t sum_{o,i} P_t[o,i,j] * C(left_t[b,i,:], dy_o[b,o,:]) over n_terms <= 6 product
+ * types whose right operand has rank rank_r (they may differ in output rank: dy_k is the gradient of the rank-k
+ * output, null if no term needs it).  Tables as for mg_ant16_fwd.  dx (rows, dim_{rank_r}, (3,)^rank_r). */
+int mg_ant16_grad_x(int rank_r, int n_terms, const int* labels, const float* const* P, const float* const* left,
+                    const float* dy_0, const float* dy_1, const float* dy_2, long rows, int dim_0, int dim_1, int dim_2,
+                    int dim_l, int accumulate, float* dx, mg_stream_t stream);
+/* Gradient for the left operand of one product type (ant16_o*_backleft_cuda, codegen_tensops.cpp:892-1070,
+ * 1421-1470): dleft[b,i,:] = sum_{o,j} P[o,i,j] * C(x[b,j,:], dy[b,o,:]); x of the type's right rank, dy of its
+ * output rank; dleft (rows, dim_l, (3,)^rank_l). */
+int mg_ant16_grad_left(int label, const float* P, const float* x, const float* dy, long rows, int dim_0, int dim_1,
+                       int dim_2, int dim_l, float* dleft, mg_stream_t stream);
+/* Gradient for P of one product type (ant16_o*_wtsback_cuda, codegen_tensops.cpp:1142-1325, 1471-1517):
+ * dP[o,i,j] = sum_{b} <dy[b,o,:], left[b,i,:] (x) x[b,j,:]>.  The rows are reduced in slices whose partial results go
+ * to `workspace` (mg_ant16_grad_weight_workspace_bytes, with dim_o / dim_r the channel counts of the type's output /
+ * right rank) and are added in slice order: no atomics, the same bits on every run. */
+int mg_ant16_grad_weight_workspace_bytes(long rows, int dim_o, int dim_l, int dim_r, size_t* bytes /* host */);
+int mg_ant16_grad_weight(int label, const float* left, const float* x, const float* dy, long rows, int dim_0, int dim_1,
+                         int dim_2, int dim_l, void* workspace, float* dP, mg_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * PaiNN message passing (archs/meanflow_painn8.py:25-35,77-100).

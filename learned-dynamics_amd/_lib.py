@@ -64,6 +64,11 @@ _SIGNATURES = {
     "mg_tensor_linear_f16x2": [vp, vp, vp, i32, i64, i64, i64, i32, i32, vp, i32, i32, i32, vp, vp, vp],
     "mg_ant16_fwd": [i32, i32, ctypes.POINTER(i32), ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, vp, i64, i32, i32, i32,
                      i32, i32, vp, vp],
+    "mg_ant16_grad_x": [i32, i32, ctypes.POINTER(i32), ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, vp, i64, i32, i32, i32,
+                        i32, i32, vp, vp],
+    "mg_ant16_grad_left": [i32, vp, vp, vp, i64, i32, i32, i32, i32, vp, vp],
+    "mg_ant16_grad_weight_workspace_bytes": [i64, i32, i32, i32, ctypes.POINTER(ctypes.c_size_t)],
+    "mg_ant16_grad_weight": [i32, vp, vp, vp, i64, i32, i32, i32, i32, vp, vp, vp],
     "mg_set_linear_mode": [i32],
     "mg_get_linear_mode": [],
     "mg_group_norm_scratch_bytes": [i32, i32, ctypes.POINTER(ctypes.c_size_t)],

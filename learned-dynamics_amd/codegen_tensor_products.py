@@ -1,7 +1,6 @@
 """Ant16 / Bee / Cow0 / Cow1 autograd functions, mirroring
 managan/codegen_tensor_products.py:19-101 of the reference on top of the HIP
-kernels (Bee, Cow: forward and both backward passes; Ant16: forward kernel, backward as
-device-side contractions)."""
+kernels (forward and all backward passes of Bee, Cow and Ant16)."""
 import torch
 
 from . import ant16_backward as a16
@@ -35,19 +34,18 @@ class Ant16(torch.autograd.Function):
         return y_0, y_1 + y_1c, y_2 + y_2c
 
     @staticmethod
+    @torch.autograd.function.once_differentiable
     def backward(ctx, dy_0, dy_1, dy_2):
         xs = ctx.saved_tensors[:3]
         pairs = ctx.saved_tensors[3:]
-        dys = (dy_0, dy_1, dy_2)
-        dxs = [None, None, None]
+        dys = tuple(d.contiguous() for d in (dy_0, dy_1, dy_2))
+        needs = ctx.needs_input_grad
+        terms = [(lab, pairs[2 * k], pairs[2 * k + 1]) for k, lab in enumerate(_ANT16_LABELS)]
+        # one launch per rank of x, over every product type that reads that rank
+        dxs = a16.grad_x_all(dys, [t for t in terms if needs[int(t[0][1])]])
         grads = []
-        for k, lab in enumerate(_ANT16_LABELS):
-            P, left = pairs[2 * k], pairs[2 * k + 1]
-            dy, x, r = dys[int(lab[2])], xs[int(lab[1])], int(lab[1])
-            needs = ctx.needs_input_grad
-            if needs[r]:
-                d = a16.grad_x(lab, dy, P, left)
-                dxs[r] = d if dxs[r] is None else dxs[r] + d
+        for k, (lab, P, left) in enumerate(terms):
+            dy, x = dys[int(lab[2])], xs[int(lab[1])]
             grads.append(a16.grad_P(lab, dy, left, x) if needs[3 + 2 * k] else None)
             grads.append(a16.grad_left(lab, dy, P, x) if needs[4 + 2 * k] else None)
         return (*dxs, *grads)

@@ -504,6 +504,105 @@ def ant16_oc(x_1, x_2, P_111, left_111, P_212, left_212):
             _ant16(2, None, x_1, x_2, [("212", P_212, left_212)])]
 
 
+def _ant16_dims(pairs_P):
+    """(dim_0, dim_1, dim_2, dim_l) from the shapes of the P of some product types (label, P)."""
+    dims, dim_l = [0, 0, 0], 0
+    for lab, P in pairs_P:
+        if P.dim() != 3:
+            raise RuntimeError(f"P_{lab} has wrong number of axes")
+        for k, size in ((int(lab[2]), int(P.size(0))), (int(lab[1]), int(P.size(2)))):
+            if dims[k] not in (0, size):
+                raise RuntimeError(f"P_{lab}: channel counts of rank {k} disagree")
+            dims[k] = size
+        if dim_l not in (0, int(P.size(1))):
+            raise RuntimeError(f"P_{lab}: expected axis 1 to have size dim_l")
+        dim_l = int(P.size(1))
+    return dims, dim_l
+
+
+def ant16_grad_x(rank_r, dys, terms):
+    """Gradient for x_{rank_r} of the Ant16 contraction: sum over `terms` = [(label, P, left)] whose right operand
+    has that rank of  dx[b,j,X] = sum_{o,i} P[o,i,j] C_X(left[b,i,:], dy[b,o,:]); dys = (dy_0, dy_1, dy_2), entries
+    the terms do not use may be None (ant16_o*_backward_cuda, extensions/codegen_tensops/codegen_tensops.cpp:669-821)."""
+    terms = [(lab, P.contiguous(), left.contiguous()) for lab, P, left in terms]
+    dys = [None if d is None else d.contiguous() for d in dys]
+    dims, dim_l = _ant16_dims([(lab, P) for lab, P, _ in terms])
+    batch = int(terms[0][2].size(0))
+    dev = terms[0][1].device
+    n = len(terms)
+    for lab, P, left in terms:
+        if int(lab[1]) != rank_r:
+            raise RuntimeError(f"product {lab} has no right operand of rank {rank_r}")
+        dy = dys[int(lab[2])]
+        if dy is None or tuple(dy.shape) != _shape(batch, dims[int(lab[2])], int(lab[2])):
+            raise RuntimeError(f"dy_{lab[2]}: expected shape {_shape(batch, dims[int(lab[2])], int(lab[2]))}")
+        if tuple(left.shape) != _shape(batch, dim_l, int(lab[0])):
+            raise RuntimeError(f"left_{lab}: expected shape {_shape(batch, dim_l, int(lab[0]))}")
+    labels = (ctypes.c_int * n)(*[BEE_ORDER.index(lab) for lab, _, _ in terms])
+    Ps = (ctypes.c_void_p * n)(*[P.data_ptr() for _, P, _ in terms])
+    lefts = (ctypes.c_void_p * n)(*[left.data_ptr() for _, _, left in terms])
+    with torch.cuda.device(dev):
+        dx = torch.empty(_shape(batch, dims[rank_r], rank_r), dtype=torch.float32, device=dev)
+        if dx.numel() > 0:
+            L.check(_lib.mg_ant16_grad_x(rank_r, n, labels, Ps, lefts, _p(dys[0]), _p(dys[1]), _p(dys[2]), batch,
+                                         dims[0], dims[1], dims[2], dim_l, 0, _p(dx), _stream()))
+    return dx
+
+
+def _ant16_one(label, P, x, dy, left=None):
+    rl, rr, ro = (int(c) for c in label)
+    batch = int(dy.size(0))
+    dims = [0, 0, 0]
+    dims[ro] = int(dy.size(1))
+    if dims[rr] not in (0, int(x.size(1))):
+        raise RuntimeError(f"x_{rr} and dy_{ro} of product {label} disagree on the channel count of rank {rr}")
+    dims[rr] = int(x.size(1))
+    if tuple(x.shape) != _shape(batch, dims[rr], rr):
+        raise RuntimeError(f"x_{rr}: expected shape {_shape(batch, dims[rr], rr)}")
+    if tuple(dy.shape) != _shape(batch, dims[ro], ro):
+        raise RuntimeError(f"dy_{ro}: expected shape {_shape(batch, dims[ro], ro)}")
+    if P is not None:
+        dim_l = int(P.size(1))
+        if tuple(P.shape) != (dims[ro], dim_l, dims[rr]):
+            raise RuntimeError(f"P_{label}: expected shape {(dims[ro], dim_l, dims[rr])}")
+    else:
+        dim_l = int(left.size(1))
+        if tuple(left.shape) != _shape(batch, dim_l, rl):
+            raise RuntimeError(f"left_{label}: expected shape {_shape(batch, dim_l, rl)}")
+    return batch, dims, dim_l
+
+
+def ant16_grad_left(label, P, x, dy):
+    """dleft[b,i,L] = sum_{o,j} P[o,i,j] C_L(x[b,j,:], dy[b,o,:]) of one product type
+    (ant16_o*_backleft_cuda, extensions/codegen_tensops/codegen_tensops.cpp:892-1070)."""
+    P, x, dy = P.contiguous(), x.contiguous(), dy.contiguous()
+    batch, dims, dim_l = _ant16_one(label, P, x, dy)
+    with torch.cuda.device(P.device):
+        dleft = torch.empty(_shape(batch, dim_l, int(label[0])), dtype=torch.float32, device=P.device)
+        if dleft.numel() > 0:
+            L.check(_lib.mg_ant16_grad_left(BEE_ORDER.index(label), _p(P), _p(x), _p(dy), batch, dims[0], dims[1],
+                                            dims[2], dim_l, _p(dleft), _stream()))
+    return dleft
+
+
+def ant16_grad_weight(label, left, x, dy):
+    """dP[o,i,j] = sum_{b,O} dy[b,o,O] C_O(left[b,i,:], x[b,j,:]) of one product type; the rows are reduced in slices
+    that are added in order, so the result is the same on every run
+    (ant16_o*_wtsback_cuda, extensions/codegen_tensops/codegen_tensops.cpp:1142-1325)."""
+    left, x, dy = left.contiguous(), x.contiguous(), dy.contiguous()
+    batch, dims, dim_l = _ant16_one(label, None, x, dy, left=left)
+    dim_r, dim_o = dims[int(label[1])], dims[int(label[2])]
+    with torch.cuda.device(left.device):
+        dP = torch.empty(dim_o, dim_l, dim_r, dtype=torch.float32, device=left.device)
+        if dP.numel() > 0:
+            nbytes = ctypes.c_size_t(0)
+            L.check(_lib.mg_ant16_grad_weight_workspace_bytes(batch, dim_o, dim_l, dim_r, ctypes.byref(nbytes)))
+            ws = torch.empty(nbytes.value, dtype=torch.uint8, device=left.device)
+            L.check(_lib.mg_ant16_grad_weight(BEE_ORDER.index(label), _p(left), _p(x), _p(dy), batch, dims[0], dims[1],
+                                              dims[2], dim_l, _p(ws), _p(dP), _stream()))
+    return dP
+
+
 def tensor_prod_bare(inds_l, inds_r, inds_o, x_l, x_r):
     """TensorProdBare.forward for operands (..., chan, (3,)^inds); leading dims must agree."""
     _check_input(x_l, "x_l")

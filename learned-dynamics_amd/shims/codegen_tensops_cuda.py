@@ -1,7 +1,6 @@
 """Drop-in for the reference's `codegen_tensops_cuda` extension
-(extensions/codegen_tensops/codegen_tensops.cpp:1980-2011).  The Bee and Cow
-families and the Ant16 forward functions run on the HIP kernels; the Ant16 backward functions
-(training of the legacy architectures) are device-side contractions through the GEMM library."""
+(extensions/codegen_tensops/codegen_tensops.cpp:1980-2011): the Bee, Cow and Ant16
+families, forward and backward, on the HIP kernels."""
 import importlib
 
 _ops = importlib.import_module("learned-dynamics_amd.ops")

@@ -138,3 +138,27 @@ def test_ant16_backward_shim_families():
     close(dl111, rl["111"]); close(dl212, rl["212"]); close(dP111, rP["111"]); close(dP212, rP["212"])
     with pytest.raises(RuntimeError):
         shim.ant16_o0_backward_cuda(cot[0], *pl[:6])          # host tensor
+
+
+def test_ant16_weight_gradient_is_reproducible_and_handles_no_rows():
+    """The row slices of dP are added in a fixed order: two runs give the same bits (many more rows than one slice
+    holds); no rows give zeros; the gradients for x and left of an empty batch are empty."""
+    a16 = importlib.import_module("learned-dynamics_amd.ant16_backward")
+    g = torch.Generator().manual_seed(12)
+    batch, d1, d2, dl = 5000, 24, 40, 8
+    left = torch.randn(batch, dl, 3, 3, generator=g).cuda()
+    x = torch.randn(batch, d1, 3, generator=g).cuda()
+    dy = torch.randn(batch, d2, 3, 3, generator=g).cuda()
+    a = a16.grad_P("212", dy, left, x)
+    b = a16.grad_P("212", dy, left, x)
+    assert a.shape == (d2, dl, d1) and torch.equal(a, b)
+    ld, xd = left.cpu().double(), x.cpu().double()
+    q = OP.product("212", ld[:, :, None].expand(batch, dl, d1, 3, 3).reshape(batch, dl * d1, 3, 3),
+                   xd[:, None].expand(batch, dl, d1, 3).reshape(batch, dl * d1, 3)).reshape(batch, dl, d1, 3, 3)
+    want = torch.einsum("boxy,blixy->oli", dy.cpu().double(), q)
+    torch.testing.assert_close(a.cpu().double(), want, rtol=1e-5, atol=4e-6 * float(want.abs().max()))
+    z = a16.grad_P("212", dy[:0], left[:0], x[:0])
+    assert z.shape == (d2, dl, d1) and not bool(z.any())
+    Pz = torch.randn(d2, dl, d1, generator=g).cuda()
+    assert a16.grad_x("212", dy[:0], Pz, left[:0]).shape == (0, d1, 3)
+    assert a16.grad_left("212", dy[:0], Pz, x[:0]).shape == (0, dl, 3, 3)

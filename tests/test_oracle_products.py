@@ -5,6 +5,8 @@ and autograd consistency of the backward helper."""
 import itertools
 
 import pytest
+import os
+
 import torch
 
 from conftest import load_golden
@@ -192,25 +194,49 @@ def test_backward_helper_matches_finite_differences():
             assert abs(fd - dl[k].reshape(-1)[j]) < 1e-6
 
 
-def test_ant16_backward_contractions_against_autograd():
-    """The host-side contractions behind the Ant16 backward functions (a pure torch module, so it runs
-    here in float64 on the CPU) against autograd through the oracle's forward: every product type,
-    every operand, on sizes where all axes differ."""
-    import importlib
-    a16 = importlib.import_module("learned-dynamics_amd.ant16_backward")
-    g = torch.Generator().manual_seed(33)
-    batch, dims, dl = 3, (4, 5, 2), 6
-    x = [torch.randn(batch, dims[k], *([3] * k), generator=g, dtype=torch.float64, requires_grad=True) for k in range(3)]
-    for lab in OP.BEE_ORDER:
+def _coupling_generator():
+    import importlib.util
+    path = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "learned-dynamics_amd", "csrc",
+                        "gen_ant16_coupling.py")
+    spec = importlib.util.spec_from_file_location("gen_ant16_coupling", path)
+    mod = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(mod)
+    return mod, path
+
+
+def test_ant16_coupling_table_against_the_products_and_their_derivatives():
+    """The term lists the Ant16 kernels are generated from (forward, gradient for x, gradient for left), evaluated
+    here on random operands, against the oracle's product of each type and autograd through it; and the committed
+    table is what the generator writes."""
+    gen, path = _coupling_generator()
+    tab = gen.table()
+    assert gen.LABELS == tuple(OP.BEE_ORDER)
+
+    def apply(mode, k, n_out, a, b):
+        out = torch.zeros(n_out, dtype=torch.float64)
+        for c in range(n_out):
+            for e in tab[mode][k][c]:
+                out[c] += (-1.0 if e & 256 else 1.0) * a.reshape(-1)[e & 15] * b.reshape(-1)[(e >> 4) & 15]
+        return out
+
+    g = torch.Generator().manual_seed(5)
+    for k, lab in enumerate(OP.BEE_ORDER):
         rl, rr, ro = (int(c) for c in lab)
-        P = torch.randn(dims[ro], dl, dims[rr], generator=g, dtype=torch.float64, requires_grad=True)
-        left = torch.randn(batch, dl, *([3] * rl), generator=g, dtype=torch.float64, requires_grad=True)
-        zeros_P = {k: torch.zeros(dims[int(k[2])], dl, dims[int(k[1])], dtype=torch.float64) for k in OP.BEE_ORDER}
-        zeros_l = {k: torch.zeros(batch, dl, *([3] * int(k[0])), dtype=torch.float64) for k in OP.BEE_ORDER}
-        zeros_P[lab], zeros_l[lab] = P, left
-        y = OP.ant16(x[0], x[1], x[2], zeros_P, zeros_l)[ro]
+        l = torch.randn(1, 1, *([3] * rl), generator=g, dtype=torch.float64, requires_grad=True)
+        r = torch.randn(1, 1, *([3] * rr), generator=g, dtype=torch.float64, requires_grad=True)
+        y = OP.product(lab, l, r)
         dy = torch.randn(y.shape, generator=g, dtype=torch.float64)
-        gx, gP, gl = torch.autograd.grad((y * dy).sum(), (x[rr], P, left))
-        assert torch.allclose(a16.grad_x(lab, dy, P, left), gx, atol=1e-12)
-        assert torch.allclose(a16.grad_P(lab, dy, left, x[rr]), gP, atol=1e-12)
-        assert torch.allclose(a16.grad_left(lab, dy, P, x[rr]), gl, atol=1e-12)
+        gl, gr = torch.autograd.grad((y * dy).sum(), (l, r))
+        assert torch.allclose(apply(0, k, 3 ** ro, l.detach(), r.detach()), y.detach().reshape(-1), atol=1e-14)
+        assert torch.allclose(apply(1, k, 3 ** rr, l.detach(), dy), gr.reshape(-1), atol=1e-14)
+        assert torch.allclose(apply(2, k, 3 ** rl, r.detach(), dy), gl.reshape(-1), atol=1e-14)
+    committed = open(os.path.join(os.path.dirname(path), "ant16_coupling.inc")).read()
+    import tempfile, shutil
+    with tempfile.TemporaryDirectory() as tmp:
+        shutil.copy(path, tmp)
+        mod_path = os.path.join(tmp, "gen_ant16_coupling.py")
+        import importlib.util
+        spec = importlib.util.spec_from_file_location("gen_tmp", mod_path)
+        mod = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(mod)
+        assert open(mod.main()).read() == committed
