@@ -413,7 +413,7 @@ def bench_products(torch, args):
         flop = 2 * rows * 64 * 64 * ((3 + 3 + 1) + (1 + 3 + 3) + (3 + 3 + 9))
         out[f"rows_{rows}"]["with_linears"] = {"us": t * 1e6, "GFLOP": flop / 1e9, "TFLOP/s": flop / t / 1e12,
                                                "frac_of_fp32_mfma_peak": flop / t / 1e12 / PEAK_FP32_MFMA_TFLOPS,
-                                               "launches": 12}
+                                               "launches": 3}
     return {"metric": "fused tensor-product trio (v.v, x v, v(x)v), BASELINE configs[0]", "unit": "nodes/s",
             "value": out["rows_4096"]["nodes_per_s"], "detail": out,
             "note": "includes allocation of the three outputs; 4096 rows (17.8 MB) is launch-latency bound"}

@@ -190,6 +190,16 @@ int mg_cow_o1_bwd(int side, const float* o_0, const float* o_1, const float* dy_
  * (inds_l, inds_r, inds_o) with all ranks <= 2. */
 int mg_tensor_prod_bare(int inds_l, int inds_r, int inds_o, const float* x_l, const float* x_r,
                         long rows, int chan, float* y, mg_stream_t stream);
+/* TensorProds.forward in one launch (managan/tensor_products.py:109-121):
+ *   y = lin_o(prod(lin_l(x_l), lin_r(x_r))),  lin_l: W_l (rank, dim_l), lin_r: W_r (rank, dim_r), lin_o: W_o (dim_o, rank),
+ * weights with row strides ldl / ldr / ldo (unit stride along a row), x_l (rows, dim_l, (3,)^inds_l),
+ * x_r (rows, dim_r, (3,)^inds_r), y (rows, dim_o, (3,)^inds_o) dense and 16-byte aligned.  Needs channel counts that are
+ * multiples of 16 and weights that fit 64 KB of LDS: mg_tensor_prods_supported returns 1 if a problem qualifies
+ * (a yes/no answer, not a status); otherwise compose mg_tensor_linear and mg_tensor_prod_bare. */
+int mg_tensor_prods_supported(int inds_l, int inds_r, int inds_o, int dim_l, int dim_r, int rank, int dim_o);
+int mg_tensor_prods(int inds_l, int inds_r, int inds_o, const float* W_l, long ldl, const float* W_r, long ldr,
+                    const float* W_o, long ldo, const float* x_l, const float* x_r, long rows, int dim_l, int dim_r,
+                    int rank, int dim_o, float* y, mg_stream_t stream);
 /* The three products the vector/scalar pair of one TensorProds stack needs in one pass:
  * y_110 = v.v', y_011 = a v', y_112 = v (x) v' with v = left vector, v' = right vector,
  * a = scalar (managan/tensor_products.py:91-121 applied three times). */

@@ -48,6 +48,8 @@ _SIGNATURES = {
     "mg_cow_o1_bwd": [i32, vp, vp, vp, vp, vp, i64, i32, vp, vp, vp],
     "mg_tensor_prod_bare": [i32, i32, i32, vp, vp, i64, i32, vp, vp],
     "mg_tensor_prods_avd": [vp, vp, vp, i64, i32, vp, vp, vp, vp],
+    "mg_tensor_prods_supported": [i32, i32, i32, i32, i32, i32, i32],
+    "mg_tensor_prods": [i32, i32, i32, vp, i64, vp, i64, vp, i64, vp, vp, i64, i32, i32, i32, i32, vp, vp],
     "mg_tensor_linear": [i32, vp, i64, i64, vp, i64, i32, i32, vp, i32, i32, vp, vp],
     "mg_tensor_linear_wgrad_workspace_bytes": [i64, i32, i32, ctypes.POINTER(ctypes.c_size_t)],
     "mg_tensor_linear_wgrad": [i32, vp, vp, i64, i32, i32, vp, vp, vp],

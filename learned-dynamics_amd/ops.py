@@ -18,7 +18,14 @@ _lib = L.load()
 BEE_ORDER = ("000", "110", "220", "011", "101", "121", "211", "022", "202", "112", "222", "111", "212")
 
 
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_raw_device = getattr(torch._C, "_cuda_getDevice", None)
+
+
 def _stream():
+    """The current HIP stream of the current device as a pointer argument."""
+    if _raw_stream is not None and _raw_device is not None:     # same value as below, without building Stream objects
+        return ctypes.c_void_p(_raw_stream(_raw_device()))
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
@@ -619,6 +626,39 @@ def tensor_prod_bare(inds_l, inds_r, inds_o, x_l, x_r):
     with torch.cuda.device(x_l.device):
         y = torch.empty(lead_l + (3,) * inds_o, dtype=torch.float32, device=x_l.device)
         L.check(_lib.mg_tensor_prod_bare(inds_l, inds_r, inds_o, _p(x_l), _p(x_r), n, 1, _p(y), _stream()))
+    return y
+
+
+def tensor_prods_supported(inds_l, inds_r, inds_o, dim_l, dim_r, rank, dim_o):
+    """Whether tensor_prods (the one-launch TensorProds) takes this problem."""
+    return bool(_lib.mg_tensor_prods_supported(inds_l, inds_r, inds_o, dim_l, dim_r, rank, dim_o))
+
+
+def tensor_prods(inds_l, inds_r, inds_o, W_l, W_r, W_o, x_l, x_r):
+    """lin_o(prod(lin_l(x_l), lin_r(x_r))) in one launch (managan/tensor_products.py:109-121); x: (..., dim, (3,)^inds),
+    weights (out, in) with unit stride along a row."""
+    for t, nm in ((W_l, "W_l"), (W_r, "W_r"), (W_o, "W_o"), (x_l, "x_l"), (x_r, "x_r")):
+        if not t.is_cuda or t.dtype != torch.float32:
+            raise RuntimeError(f"{nm} must be a float32 CUDA tensor")
+    x_l, x_r = x_l.contiguous(), x_r.contiguous()
+    lead = tuple(x_l.shape[:x_l.dim() - inds_l - 1])
+    if lead != tuple(x_r.shape[:x_r.dim() - inds_r - 1]):
+        raise RuntimeError(f"operands do not broadcast: {tuple(x_l.shape)} vs {tuple(x_r.shape)}")
+    rank, dim_l = (int(v) for v in W_l.shape)
+    dim_o = int(W_o.shape[0])
+    dim_r = int(W_r.shape[1])
+    if tuple(x_l.shape[len(lead):]) != (dim_l,) + (3,) * inds_l or tuple(x_r.shape[len(lead):]) != (dim_r,) + (3,) * inds_r \
+            or int(W_r.shape[0]) != rank or int(W_o.shape[1]) != rank:
+        raise RuntimeError("shape mismatch between weights and operands")
+    Ws = [W if W.stride(1) == 1 and W.stride(0) % 4 == 0 and W.data_ptr() % 16 == 0 else W.contiguous() for W in (W_l, W_r, W_o)]
+    rows = 1
+    for d in lead:
+        rows *= int(d)
+    with torch.cuda.device(x_l.device):
+        y = torch.empty(lead + (dim_o,) + (3,) * inds_o, dtype=torch.float32, device=x_l.device)
+        L.check(_lib.mg_tensor_prods(inds_l, inds_r, inds_o, _p(Ws[0]), Ws[0].stride(0), _p(Ws[1]), Ws[1].stride(0),
+                                     _p(Ws[2]), Ws[2].stride(0), _p(x_l), _p(x_r), rows, dim_l, dim_r, rank, dim_o,
+                                     _p(y), _stream()))
     return y
 
 

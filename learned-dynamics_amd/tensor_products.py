@@ -100,4 +100,9 @@ class TensorProds(nn.Module):
         self.lin_o = TensLinear(inds_o, rank, dim_o)
 
     def forward(self, x_l, x_r):
+        W_l, W_r, W_o = self.lin_l.W, self.lin_r.W, self.lin_o.W
+        wants_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (x_l, x_r, W_l, W_r, W_o))
+        if not wants_grad and ops.tensor_prods_supported(*self.prod.inds, W_l.shape[1], W_r.shape[1], W_l.shape[0],
+                                                         W_o.shape[0]):
+            return ops.tensor_prods(*self.prod.inds, W_l, W_r, W_o, x_l, x_r)     # one launch, nothing stored between
         return self.lin_o(self.prod(self.lin_l(x_l), self.lin_r(x_r)))

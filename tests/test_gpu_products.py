@@ -115,3 +115,69 @@ def test_unaligned_views(ops):
     ys = ops.bee_fwd(*[shifted(t) for t in l], *[shifted(t) for t in r])
     for y, y_ref in zip(ys, OP.bee(*l, *r)):
         _close(y, y_ref)
+
+
+_TP_TYPES = [(0, 0, 0), (1, 1, 0), (2, 2, 0), (0, 1, 1), (1, 0, 1), (1, 2, 1), (2, 1, 1), (0, 2, 2), (2, 0, 2), (1, 1, 2),
+             (2, 2, 2)]
+
+
+def _tp_case(lro, rows, dims, seed):
+    il, ir, io = lro
+    dim_l, dim_r, rank, dim_o = dims
+    g = torch.Generator().manual_seed(seed)
+    x_l = torch.randn(rows, dim_l, *([3] * il), generator=g)
+    x_r = torch.randn(rows, dim_r, *([3] * ir), generator=g)
+    W_l = torch.randn(rank, dim_l, generator=g) * dim_l ** -0.5
+    W_r = torch.randn(rank, dim_r, generator=g) * dim_r ** -0.5
+    W_o = torch.randn(dim_o, rank, generator=g) * rank ** -0.5
+    return x_l, x_r, W_l, W_r, W_o
+
+
+@pytest.mark.parametrize("lro", _TP_TYPES)
+def test_tensor_prods_one_launch(ops, lro):
+    """lin_o(prod(lin_l, lin_r)) in one kernel (managan/tensor_products.py:109-121): every product type, channel
+    counts that all differ (80 output channels: two grid rows of output tiles), a row count that fills neither a
+    wave's 16 rows nor a workgroup's 64."""
+    from parity import assert_parity
+    dims = (32, 48, 64, 80)
+    x_l, x_r, W_l, W_r, W_o = _tp_case(lro, 150, dims, 100 + sum(lro))
+    assert ops.tensor_prods_supported(*lro, *dims)
+    y = ops.tensor_prods(*lro, W_l.cuda(), W_r.cuda(), W_o.cuda(), x_l.cuda(), x_r.cuda())
+    ref32 = OP.tensor_prods(*lro, W_l, W_r, W_o, x_l, x_r)
+    ref64 = OP.tensor_prods(*lro, W_l.double(), W_r.double(), W_o.double(), x_l.double(), x_r.double())
+    assert_parity(y, ref32, ref64, what=f"tensor_prods {lro}")
+
+
+def test_tensor_prods_module_routes_and_agrees(ops):
+    """TensorProds.forward takes the one-launch kernel when nothing asks for a gradient and the three-step path
+    otherwise; both agree with the oracle; strided weights (a transposed view) and leading batch axes are honoured;
+    unsupported channel counts fall back."""
+    from parity import assert_parity
+    tp = importlib.import_module("learned-dynamics_amd.tensor_products")
+    torch.manual_seed(5)
+    mod = tp.TensorProds(1, 1, 2, 64, 64, 64, 64).cuda()
+    g = torch.Generator().manual_seed(6)
+    v = torch.randn(3, 50, 64, 3, generator=g)
+    w = torch.randn(3, 50, 64, 3, generator=g)
+    W = [p.detach().cpu() for p in (mod.lin_l.W, mod.lin_r.W, mod.lin_o.W)]
+    ref32 = OP.tensor_prods(1, 1, 2, *W, v, w)
+    ref64 = OP.tensor_prods(1, 1, 2, *[t.double() for t in W], v.double(), w.double())
+    with torch.no_grad():
+        fused = mod(v.cuda(), w.cuda())
+    stepwise = mod(v.cuda(), w.cuda())                       # parameters require grad: three-step path
+    assert fused.shape == (3, 50, 64, 3, 3) and stepwise.requires_grad and not fused.requires_grad
+    assert_parity(fused, ref32, ref64, what="TensorProds fused")
+    assert_parity(stepwise, ref32, ref64, what="TensorProds stepwise")
+    Wt = W[0].t().contiguous().cuda().t()                    # same values, column-major storage
+    y = ops.tensor_prods(1, 1, 2, Wt, W[1].cuda(), W[2].cuda(), v.cuda(), w.cuda())
+    assert torch.equal(y, fused)
+    assert not ops.tensor_prods_supported(1, 1, 2, 64, 64, 40, 64)
+    assert not ops.tensor_prods_supported(1, 1, 1, 64, 64, 64, 64)
+    small = tp.TensorProds(0, 1, 1, 24, 24, 40, 24).cuda()   # not multiples of 16: composed path
+    with torch.no_grad():
+        ys = small(v[..., :24, 0].contiguous().cuda(), w[..., :24, :].contiguous().cuda())
+    Ws = [p.detach().cpu() for p in (small.lin_l.W, small.lin_r.W, small.lin_o.W)]
+    _close(ys, OP.tensor_prods(0, 1, 1, *Ws, v[..., :24, 0], w[..., :24, :]))
+    with pytest.raises(RuntimeError, match="multiples of 16"):
+        ops.tensor_prods(0, 1, 1, *[t.cuda() for t in Ws], v[..., :24, 0].contiguous().cuda(), w[..., :24, :].contiguous().cuda())
+    assert ops.tensor_prods(1, 1, 2, *[t.cuda() for t in W], v[:0].cuda(), w[:0].cuda()).shape == (0, 50, 64, 3, 3)
