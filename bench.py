@@ -47,7 +47,7 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="painn_layer",
-                    choices=["painn_layer", "neighbour", "products", "denoiser", "stress", "polymer"])
+                    choices=["painn_layer", "neighbour", "products", "denoiser", "stress", "polymer", "meanflow_painn"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-comparisons", action="store_true",
@@ -563,6 +563,42 @@ def bench_denoiser(torch, args, with_cpu=True):
     return out
 
 
+def bench_meanflow_painn(torch, args):
+    """The PaiNN meanflow denoiser (archs/meanflow_painn8.py:185-217 with a one-hot atom embedding): 2 + 5 blocks, each a
+    radius-graph message, a bond message and an update; 16384 atoms at the density of configs[2] (80 A box, n = 128)
+    on a jittered lattice with the cutoff at 5 A, which keeps every atom inside the reference's default caps (64
+    neighbours, 32 atoms per cell; the model calls graph_setup with them); bonds join lattice neighbours in chains of
+    1024; both radius graphs are rebuilt inside the forward."""
+    mf = importlib.import_module("learned-dynamics_amd.meanflow_painn")
+    n, r0, box_len, chains, atoms = 128, 5.0, 80.0, 16, 1024
+    box = (box_len,) * 3
+    seed = 0x947 + 7
+    torch.manual_seed(seed)
+    N = chains * atoms
+    g = torch.Generator().manual_seed(seed + 1)
+    side = 26                                                      # 26^3 >= 16384 lattice sites, 3.08 A apart
+    k = torch.arange(N)
+    sites = torch.stack([k % side, (k // side) % side, k // (side * side)], dim=1).float() * (box_len / side)
+    x1 = (sites + 0.5 * torch.randn(N, 3, generator=g)).reshape(1, N, 3).contiguous()
+    x0 = x1 + 0.3 * torch.randn(1, N, 3, generator=g)
+    one_hot = torch.nn.functional.one_hot(torch.randint(0, 20, (N,), generator=g), 20).float()
+    idx = torch.arange(N - 1)
+    idx = idx[(idx + 1) % atoms != 0]                              # bonds along each chain, both directions
+    topo = mf.Topology(one_hot.cuda(), torch.cat([idx, idx + 1]).cuda(), torch.cat([idx + 1, idx]).cuda())
+    model = mf.SE3ITO(r0, n, N).cuda().eval()
+    s, t = torch.zeros(1).cuda(), torch.rand(1, generator=g).cuda()
+    x0_d, x1_d = x0.cuda(), x1.cuda()
+    with torch.no_grad():
+        def step():
+            return model((s, t), x0_d, x1_d, box, topo)
+        step()
+        sec = timed_steps(torch, step, args.steps, args.warmup)
+    return {"metric": "PaiNN meanflow denoiser forward atoms/sec", "value": N / sec, "unit": "atoms/s",
+            "ms_per_step": sec * 1e3, "dtype": "f32 storage and accumulation",
+            "config": {"workload": "SE3ITO forward (2 + 5 PaiNN blocks with bond messages, n = 128), 16384 atoms on a jittered "
+                                   "lattice, box 80 A, cutoff 5 A, radius graphs rebuilt in the forward", "atoms": N}}
+
+
 def bench_stress(torch, args, with_cpu=True):
     """BASELINE configs[4]: 65536 atoms uniform in a periodic cube at 0.1 atoms/A^3, cutoff 6 A,
     4 x [Messages + SelfTensProds] with 128 channels per rank, features stored as bf16 with fp32
@@ -753,13 +789,16 @@ def main():
             st = bench_stress(torch, argparse.Namespace(steps=20, warmup=5, no_comparisons=False), with_cpu=not args.no_cpu)
             res["other_workloads"] = {"denoiser_forward_configs[3]": dn, "neighbour_search_configs[1]": nb,
                                       "tensor_products_configs[0]": bench_products(torch, small),
-                                      "stress_configs[4]": st}
+                                      "stress_configs[4]": st,
+                                      "meanflow_painn_forward": bench_meanflow_painn(torch, argparse.Namespace(steps=10, warmup=3))}
     elif args.workload == "neighbour":
         res = bench_neighbour(torch, args, with_cpu=not args.no_cpu)
     elif args.workload == "denoiser":
         res = bench_denoiser(torch, args, with_cpu=not args.no_cpu)
     elif args.workload == "stress":
         res = bench_stress(torch, args, with_cpu=not args.no_cpu)
+    elif args.workload == "meanflow_painn":
+        res = bench_meanflow_painn(torch, args)
     elif args.workload == "polymer":
         res = bench_polymer(torch, args, with_cpu=not args.no_cpu)
     else:
