@@ -86,7 +86,31 @@ class TensorProdBare(nn.Module):
         self.inds = (inds_l, inds_r, inds_o)
 
     def forward(self, x_l, x_r):
+        if torch.is_grad_enabled() and (x_l.requires_grad or x_r.requires_grad):
+            return _prod_with_grad(self.inds, x_l, x_r)
         return ops.tensor_prod_bare(*self.inds, x_l.contiguous(), x_r.contiguous())
+
+
+def _prod_with_grad(inds, x_l, x_r):
+    """The product through the 13-product autograd function (the reference relies on torch.einsum's autograd,
+    managan/tensor_products.py:104-106): the operands take their ranks' slots, the other slots are zeros, and the
+    output of type (inds_l inds_r inds_o) is picked.  Differentiable any number of times, like Bee."""
+    from .codegen_tensor_products import Bee
+    il, ir, io = inds
+    lead = x_l.shape[:x_l.dim() - il - 1]
+    chan = x_l.shape[len(lead)]
+    if tuple(x_r.shape[:x_r.dim() - ir]) != tuple(lead) + (chan,):
+        raise RuntimeError(f"operands do not broadcast: {tuple(x_l.shape)} vs {tuple(x_r.shape)}")
+    rows = 1
+    for d in lead:
+        rows *= int(d)
+    def slots(x, rank):
+        out = [torch.zeros(rows, chan, *([3] * k), dtype=torch.float32, device=x.device) for k in range(3)]
+        out[rank] = x.reshape(rows, chan, *([3] * rank))
+        return out
+    ys = Bee.apply(*slots(x_l, il), *slots(x_r, ir))
+    y = ys[ops.BEE_ORDER.index(f"{il}{ir}{io}")]
+    return y.reshape(*lead, chan, *([3] * io))
 
 
 class TensorProds(nn.Module):

@@ -234,3 +234,34 @@ def test_weight_gradient_is_reproducible(ops):
         assert torch.equal(ops.tensor_linear_wgrad(1, dy, x), a)
     ref = torch.einsum("rot,rit->oi", dy.double().cpu(), x.double().cpu())
     torch.testing.assert_close(a.cpu().double(), ref, rtol=1e-5, atol=2e-5 * float(ref.abs().max()))
+
+
+@pytest.mark.parametrize("lro", [(1, 1, 0), (0, 1, 1), (1, 1, 2), (1, 2, 1), (2, 2, 2)])
+def test_tensor_prods_module_trains(lro):
+    """TensorProds (managan/tensor_products.py:109-121) with gradients: first derivatives for both operands and the
+    three weights, and a second derivative (gradient of a gradient norm), against autograd through the oracle."""
+    tp = importlib.import_module("learned-dynamics_amd.tensor_products")
+    il, ir, io = lro
+    torch.manual_seed(11 + sum(lro))
+    mod = tp.TensorProds(il, ir, io, 24, 40, 16, 32).cuda()
+    g = torch.Generator().manual_seed(12)
+    x_l = torch.randn(7, 5, 24, *([3] * il), generator=g)
+    x_r = torch.randn(7, 5, 40, *([3] * ir), generator=g)
+    cot = torch.randn(7, 5, 16, *([3] * io), generator=g)
+
+    def run(W, xl, xr, c):
+        return (OP.tensor_prods(il, ir, io, *W, xl, xr) * c).sum()
+
+    Wd = [p.detach().cpu().double().requires_grad_() for p in (mod.lin_l.W, mod.lin_r.W, mod.lin_o.W)]
+    xl_d, xr_d = x_l.double().requires_grad_(), x_r.double().requires_grad_()
+    ref = torch.autograd.grad(run(Wd, xl_d, xr_d, cot.double()), [xl_d, xr_d, *Wd], create_graph=True)
+    ref2 = torch.autograd.grad(sum((r ** 2).sum() for r in ref[:2]), [xl_d, xr_d, *Wd])
+
+    xl_g, xr_g = x_l.cuda().requires_grad_(), x_r.cuda().requires_grad_()
+    params = [mod.lin_l.W, mod.lin_r.W, mod.lin_o.W]
+    y = mod(xl_g, xr_g)
+    assert y.requires_grad
+    got = torch.autograd.grad((y * cot.cuda()).sum(), [xl_g, xr_g, *params], create_graph=True)
+    got2 = torch.autograd.grad(sum((r ** 2).sum() for r in got[:2]), [xl_g, xr_g, *params])
+    for a, r in zip(list(got) + list(got2), list(ref) + list(ref2)):
+        torch.testing.assert_close(a.detach().cpu().double(), r.detach(), rtol=2e-4, atol=2e-5 * float(r.abs().max()) + 1e-9)

@@ -324,3 +324,40 @@ def test_plain_entry_point_through_ctypes(pkg, inds):
     L.check(lib.mg_tensor_linear(inds, Wd.data_ptr(), Wd.stride(1), Wd.stride(0), xd.data_ptr(), 0, 48, 96,
                                  None, 0, 0, yd.data_ptr(), st))
     assert torch.equal(yd, before)
+
+
+@pytest.mark.parametrize("span", [1e4, 1e6])
+def test_linear_f16x2_in_row_dynamic_range_meeting_zero_weights(ops, span):
+    """Inside ONE row: a few entries `span` times larger than the rest, and weights that are exactly zero on those
+    entries, so the result is made of the small entries alone.  The row scale puts the row maximum M at 2^14..2^15
+    and every entry is carried by two fp16 pieces with an absolute error of at most 2^-25 in scaled units, i.e.
+    2^-39 M per term whatever the term's own size: the error bound is relative to the ROW, not to the term.
+      span 1e4: the small terms still carry about 2^-26 relative error each: the rel 1e-5 / abs 1e-6 contract holds
+                on the result itself;
+      span 1e6: the bound 2^-39 M |w| sqrt(K) is about 1e-5 of a result of order one: the edge of the contract, and
+                what this test pins is that bound (rows of the models carry activations and products of order one,
+                their in-row spans stay far below 1e4)."""
+    g = torch.Generator().manual_seed(int(span) % 97)
+    rows, dim_in, dim_out = 4096, 512, 256
+    x = torch.randn(rows, dim_in, generator=g)
+    big = torch.zeros(dim_in, dtype=torch.bool)
+    big[::37] = True
+    x[:, big] *= span
+    W = torch.randn(dim_out, dim_in, generator=g) / dim_in ** 0.5
+    W[:, big] = 0.0
+    ref = x.double() @ W.double().t()
+    y = ops.tensor_linear_f16x2(W.cuda(), x.cuda())
+    small = x.clone()
+    small[:, big] = 0.0
+    ref32 = (small @ W.t()).double()                          # fp32 evaluation of the same sum (the zeros drop out exactly)
+    e_ref = float((ref32 - ref).abs().max())
+    err = (y.cpu().double() - ref).abs()
+    contract = 1e-6 + 1e-5 * ref.abs() + 2 * e_ref            # the tolerance on the result, as everywhere else
+    row_scale = (3 * 2.0 ** -39 * dim_in ** 0.5) * x.abs().amax(1, keepdim=True).double() * W.abs().amax(1).double()
+    print(f"[f16x2 in-row span {span:g}] max err {float(err.max()):.3g}  e_ref {e_ref:.3g}  max row-scale bound "
+          f"{float(row_scale.max()):.3g}  |ref| max {float(ref.abs().max()):.3g}")
+    if span <= 1e4:
+        assert bool((err <= contract).all()), (float(err.max()), e_ref)
+    else:
+        assert bool((err <= contract + row_scale).all()), (float(err.max()), e_ref)
+        assert float(err.max()) < 3e-5 * float(ref.abs().max())
