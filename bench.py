@@ -243,8 +243,14 @@ def bench_painn_layer(torch, args):
             sliced = msg.use_sliced and rows <= ops.PAINN_SLICED_MAX_ROWS and n % ops.PAINN_SLICE == 0
             if sliced:
                 actv_s = actv[:, ops.painn_slice_permutation(n, "cuda")].contiguous()
+                # the kernel alone, called as the layer calls it: rows in cell order, the per-edge records (grid row,
+                # interpolation weights, direction: 32 bytes per edge) written by their own small kernel
+                rec = ops.painn_edge_records(r_ij, rows, 2 * r0, 0.1)
+                t_rec = event_time(torch, lambda: ops.painn_edge_records(r_ij, rows, 2 * r0, 0.1), 20)
                 t_table = event_time(torch, lambda: ops.painn_table_message_sliced(
-                    graph.row_ptr, graph.dst32, r_ij, table, 2 * r0, actv_s, xv_flat, 0.1, xa_flat, xv_flat), 20)
+                    graph.row_ptr, graph.dst32, r_ij, table, 2 * r0, actv_s, xv_flat, 0.1, xa_flat, xv_flat,
+                    node_order=graph.cell_order, records=rec), 20)
+                breakdown["edge_records_ms"] = t_rec * 1e3
                 if comparisons:
                     msg.use_sliced = False
                     sec_cached_grid = timed_steps(torch, step, max(3, args.steps // 4), 2)
@@ -258,7 +264,7 @@ def bench_painn_layer(torch, args):
                 sec_exact = timed_steps(torch, step, max(3, args.steps // 4), 2)
                 msg.use_table = True
                 breakdown["layer_ms_with_filter_mlp_per_edge"] = sec_exact * 1e3
-            hbm_bytes = E * 16 + N * (16 * n + 12 * n) + 2 * N * 16 * n + rows * 16 * n
+            hbm_bytes = E * (36 if sliced else 16) + N * (16 * n + 12 * n) + 2 * N * 16 * n + rows * 16 * n
             gather_bytes = E * (16 * n + 12 * n + 16)
             grid_bytes = E * 4 * 16 * n
             cache_bytes = gather_bytes + (0 if sliced else grid_bytes)
