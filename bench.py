@@ -527,7 +527,7 @@ def single_system_latency(torch, model, dev, box, r0, atoms):
     return {"atoms": atoms, "edges": int(g1.src.numel()), "layers_eager_ms": t_eager * 1e3,
             "layers_hip_graph_replay_ms": t_graph * 1e3,
             "note": "8 blocks on a prebuilt neighbour graph, one system; the replay includes the copies into the "
-                    "capture's static inputs"}
+                    "capture's static inputs; inside a capture the independent pieces of a layer run on side streams"}
 
 
 def bench_denoiser(torch, args, with_cpu=True):

@@ -138,9 +138,11 @@ class SelfTensProds(nn.Module):
         # 5 chan, 5 chan instead of thirteen accumulating ones
         C = ops.LAYOUT_COMP_CHAN
         chan = self.L0.W.shape[0]
-        pairs = [ops.tensor_linear_fwd(k, lin.W, x, y_layout=C if k else ops.LAYOUT_CHAN_COMP, want_rowmax=True)
-                 for side in ((self.L0, self.L1, self.L2), (self.R0, self.R1, self.R2))
-                 for k, (lin, x) in enumerate(zip(side, (x_a, x_v, x_d)))]
+        def input_linear(k, lin, x):
+            return lambda: ops.tensor_linear_fwd(k, lin.W, x, y_layout=C if k else ops.LAYOUT_CHAN_COMP, want_rowmax=True)
+        pairs = ops.concurrent([input_linear(k, lin, x)
+                                for side in ((self.L0, self.L1, self.L2), (self.R0, self.R1, self.R2))
+                                for k, (lin, x) in enumerate(zip(side, (x_a, x_v, x_d)))], rows)
         ops_in = [p[0] for p in pairs]
         if ops.bee_products_linear_supported(rows, chan):
             # products and output linears in one kernel per output rank: the 13 products are never stored.
@@ -151,24 +153,27 @@ class SelfTensProds(nn.Module):
                         for t, m in side]
                 return torch.cat(cols, dim=1).amax(dim=1)
             bound = 9.0 * node_max(pairs[:3]) * node_max(pairs[3:])
-            y_a = ops.bee_products_linear(0, _cat_Y(self, LABELS_0), *ops_in, bound)
-            y_v = ops.bee_products_linear(1, _cat_Y(self, LABELS_1), *ops_in, bound)
-            y_d = ops.bee_products_linear(2, _cat_Y(self, LABELS_2), *ops_in, bound)
+            Ys = [_cat_Y(self, labels) for labels in (LABELS_0, LABELS_1, LABELS_2)]
+            y_a, y_v, y_d = ops.concurrent([(lambda k=k: ops.bee_products_linear(k, Ys[k], *ops_in, bound))
+                                            for k in range(3)], rows)
         else:
             P0, P1, P2, nmax = ops.bee_node_products(*ops_in, want_node_max=True)
             # nmax: per-node maxima of the products, the row bounds of the three GEMMs
-            y_a = ops.tensor_linear_fwd(0, _cat_Y(self, LABELS_0), P0.reshape(rows, 3 * chan), row_bound=nmax)
-            y_v = ops.tensor_linear_fwd(1, _cat_Y(self, LABELS_1), P1.reshape(rows, 3, 5 * chan), x_layout=C,
-                                        row_bound=nmax, rows_per_bound=3)
-            y_d = ops.tensor_linear_fwd(2, _cat_Y(self, LABELS_2), P2.reshape(rows, 9, 5 * chan), x_layout=C,
-                                        row_bound=nmax, rows_per_bound=9)
+            Ys = [_cat_Y(self, labels) for labels in (LABELS_0, LABELS_1, LABELS_2)]
+            y_a, y_v, y_d = ops.concurrent([
+                lambda: ops.tensor_linear_fwd(0, Ys[0], P0.reshape(rows, 3 * chan), row_bound=nmax),
+                lambda: ops.tensor_linear_fwd(1, Ys[1], P1.reshape(rows, 3, 5 * chan), x_layout=C, row_bound=nmax,
+                                              rows_per_bound=3),
+                lambda: ops.tensor_linear_fwd(2, Ys[2], P2.reshape(rows, 9, 5 * chan), x_layout=C, row_bound=nmax,
+                                              rows_per_bound=9)], rows)
         y_a = y_a.reshape(*rest, dim_a)
         y_v = y_v.reshape(*rest, dim_v, 3)
         y_d = y_d.reshape(*rest, dim_d, 3, 3)
         if residual:
-            return (self.gn_a(y_a, res=in_a.contiguous()), self.gn_v(y_v, res=in_v.contiguous()),
-                    self.gn_d(y_d, res=in_d.contiguous()))
-        return self.gn_a(y_a), self.gn_v(y_v), self.gn_d(y_d)
+            res = (in_a.contiguous(), in_v.contiguous(), in_d.contiguous())
+            return tuple(ops.concurrent([lambda: self.gn_a(y_a, res=res[0]), lambda: self.gn_v(y_v, res=res[1]),
+                                         lambda: self.gn_d(y_d, res=res[2])], rows))
+        return tuple(ops.concurrent([lambda: self.gn_a(y_a), lambda: self.gn_v(y_v), lambda: self.gn_d(y_d)], rows))
 
 
 class MLP(nn.Module):
@@ -297,29 +302,36 @@ class Messages(nn.Module):
         B, N = x_a.shape[:2]
         rows = B * N
         C = ops.LAYOUT_COMP_CHAN
-        La = ops.tensor_linear_fwd(0, self.L0.W, x_a.reshape(rows, -1).contiguous())
-        Lv = ops.tensor_linear_fwd(1, self.L1.W, x_v.reshape(rows, -1, 3).contiguous(), y_layout=C)
-        Ld = ops.tensor_linear_fwd(2, self.L2.W, x_d.reshape(rows, -1, 3, 3).contiguous(), y_layout=C)
-        enc, rhat = ops.bee_edge_geometry(r_ij.contiguous(), self.r0)
+        La, Lv, Ld, (enc, rhat) = ops.concurrent([
+            lambda: ops.tensor_linear_fwd(0, self.L0.W, x_a.reshape(rows, -1).contiguous()),
+            lambda: ops.tensor_linear_fwd(1, self.L1.W, x_v.reshape(rows, -1, 3).contiguous(), y_layout=C),
+            lambda: ops.tensor_linear_fwd(2, self.L2.W, x_d.reshape(rows, -1, 3, 3).contiguous(), y_layout=C),
+            lambda: ops.bee_edge_geometry(r_ij.contiguous(), self.r0)], rows)
         P0, S1, S2, nmax, emax = ops.bee_message(graph.row_ptr, graph.dst32, rhat, enc, La, Lv, Ld, self.lin_enc.weight,
                                            self.lin_enc.bias, node_order=node_order, want_node_max=True)
         E, chan = P0.shape[0], P0.shape[2]
         # scalar channel: per-edge linear + MLP, then the edge sum
         P0 = P0.reshape(E, 3 * chan)
         bound = emax if ops.get_linear_mode() == ops.LINEAR_F16X2 else None     # row maxima of P0 from the edge kernel
-        Y0 = self._cat_Y(LABELS_0)
-        if bound is not None and ops.f16x2_rowsum_supported(E, 3 * chan, Y0.shape[0], P0):
-            # psi_a and its sum over the edges of each node from one kernel
-            s_psi, psi_a = ops.tensor_linear_f16x2_rowsum(Y0, P0, bound, graph.row_ptr, graph.src32, rows, want_rows=True)
-            bound = ops.linear_out_bound(Y0, None, bound)
-        else:
-            psi_a, bound = _linear(P0, Y0, None, ops.ACT_NONE, bound)
-            s_psi = None
-        B_a = self.mlp_a.summed_over_rows(psi_a, graph.row_ptr, rows, plus_identity=True, bound=bound, scale=0.1,
-                                          seg=graph.src32, s_x=s_psi)
-        # vector and rank-2 channels: output linears after the edge sum, on node rows
-        B_v = ops.tensor_linear_fwd(1, self._cat_Y(LABELS_1, 0.1), S1.reshape(rows, 3, 5 * chan), x_layout=C,
-                                    row_bound=nmax, rows_per_bound=3)
-        B_d = ops.tensor_linear_fwd(2, self._cat_Y(LABELS_2, 0.1), S2.reshape(rows, 9, 5 * chan), x_layout=C,
-                                    row_bound=nmax, rows_per_bound=9)
+        Y0, Y1, Y2 = self._cat_Y(LABELS_0), self._cat_Y(LABELS_1, 0.1), self._cat_Y(LABELS_2, 0.1)
+
+        def scalar_channel(bound=bound):
+            if bound is not None and ops.f16x2_rowsum_supported(E, 3 * chan, Y0.shape[0], P0):
+                # psi_a and its sum over the edges of each node from one kernel
+                s_psi, psi_a = ops.tensor_linear_f16x2_rowsum(Y0, P0, bound, graph.row_ptr, graph.src32, rows,
+                                                              want_rows=True)
+                bound = ops.linear_out_bound(Y0, None, bound)
+            else:
+                psi_a, bound = _linear(P0, Y0, None, ops.ACT_NONE, bound)
+                s_psi = None
+            return self.mlp_a.summed_over_rows(psi_a, graph.row_ptr, rows, plus_identity=True, bound=bound, scale=0.1,
+                                               seg=graph.src32, s_x=s_psi)
+        # vector and rank-2 channels: output linears after the edge sum, on node rows (beside the per-edge MLP of the
+        # scalar channel when the system is small)
+        B_a, B_v, B_d = ops.concurrent([
+            scalar_channel,
+            lambda: ops.tensor_linear_fwd(1, Y1, S1.reshape(rows, 3, 5 * chan), x_layout=C, row_bound=nmax,
+                                          rows_per_bound=3),
+            lambda: ops.tensor_linear_fwd(2, Y2, S2.reshape(rows, 9, 5 * chan), x_layout=C, row_bound=nmax,
+                                          rows_per_bound=9)], rows)
         return (B_a.reshape(B, N, -1), B_v.reshape(B, N, -1, 3), B_d.reshape(B, N, -1, 3, 3))

@@ -309,8 +309,9 @@ static int launch_bee_message(const char* what, const int* row_ptr, const int* d
     long blocks = ceil_div(items, 4);
     if (blocks > 256L * 16) blocks = 256L * 16;
     blocks = ceil_div(blocks, 8) * 8;
-    // rows of a few edges do not repay the pipeline's start-up (one extra set of loads per row)
-    if (n_edges >= 32L * n_nodes)
+    // rows of a few edges do not repay the pipeline's start-up (one extra set of loads per row), unless the system
+    // is so small that the chip is not filled and a row's chain of load latencies is all there is to the time
+    if (n_edges >= 32L * n_nodes || items <= 16384)
         hipLaunchKernelGGL((bee_message_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                            row_ptr, dst, node_order, (long)n_nodes, rhat, enc, La, Lv, Ld, chan, enc_W, enc_b, P0, S1, S2,
                            node_max, edge_max);

@@ -433,8 +433,14 @@ int launch(const _Float16* planes, const float* w_inv, const Operands& ops, cons
 template <int T>
 int dispatch(const _Float16* planes, const float* w_inv, const Operands& ops, const float* bound, long n_nodes,
              int chan, int O, int O_pad, float* y, hipStream_t st) {
-    if (O <= 32) return launch<4, 1, T>(planes, w_inv, ops, bound, n_nodes, chan, O, O_pad, y, st);
-    if (O <= 64) return launch<4, 2, T>(planes, w_inv, ops, bound, n_nodes, chan, O, O_pad, y, st);
+    // few rows: narrow column tiles, so that the chip sees a hundred workgroups and more instead of a handful (a
+    // workgroup walks the whole reduction dimension: with 2048 nodes and 256 outputs the 256-column tile gave 8
+    // workgroups 24 chunks each and took 270 us; the operands re-read by the column tiles come from L2)
+    const long rows = n_nodes * T;
+    if (O <= 32 || (O % 32 == 0 && ceil_div(rows, 128) * ceil_div(O, 64) < 256))
+        return launch<4, 1, T>(planes, w_inv, ops, bound, n_nodes, chan, O, O_pad, y, st);
+    if (O <= 64 || (O % 64 == 0 && ceil_div(rows, 256) * ceil_div(O, 128) < 256))
+        return launch<4, 2, T>(planes, w_inv, ops, bound, n_nodes, chan, O, O_pad, y, st);
     if (O <= 128) return launch<8, 4, T>(planes, w_inv, ops, bound, n_nodes, chan, O, O_pad, y, st);
     return launch<8, 8, T>(planes, w_inv, ops, bound, n_nodes, chan, O, O_pad, y, st);
 }

@@ -35,6 +35,7 @@
 // B[k][n] likewise; D[m][n]: n = lane%32, m = 8*(q/4) + 4*(lane/32) + q%4 for register q.
 #include "common.hpp"
 #include "f16x2.hpp"
+#include <cstdlib>
 #include <type_traits>
 
 namespace mg {
@@ -365,18 +366,32 @@ struct Shape {
     int ni;      // 32-column blocks per tile
     int waves;   // waves per workgroup (32 rows each)
 };
-inline Shape choose_shape(long R, int O) {
+inline Shape choose_shape(long R, int I, int O) {
     Shape s;
     s.ni = O <= 32 ? 1 : (O <= 64 ? 2 : (O <= 128 ? 4 : 8));
     // column tiles that divide O: a partly filled tile takes the slow, bounds-checked epilogue (O = 384 with
     // 256-column tiles ran 4 times slower than with 128-column tiles)
     if (O % 32 == 0)
         while (s.ni > 1 && O % (32 * s.ni) != 0 && ceil_div(O, 16 * s.ni) <= 64) s.ni >>= 1;
-    // few rows: narrower column tiles until the 256 CUs have two workgroups each (at most 64 column tiles: the
-    // row maxima are emitted per column tile)
-    while (s.ni > 1 && ceil_div(R, 128) * ceil_div(O, 32 * s.ni) < 512 && ceil_div(O, 16 * s.ni) <= 64) s.ni >>= 1;
-    const long tiles = ceil_div(R, 256) * ceil_div(O, 32 * s.ni);
-    s.waves = tiles >= 512 ? 8 : 4;
+    const long tiles_m = ceil_div(R, 256);
+    if (tiles_m * ceil_div(O, 32 * s.ni) >= 1024 || O % 32 != 0) {
+        s.waves = 8;                                       // many tiles: the widest tile, one 8-wave workgroup per CU
+        return s;
+    }
+    // Few tiles (node-sized problems, the edges of one small system).  The chip takes 256 workgroups of 8 waves at
+    // a time, and a workgroup's time was measured (33 392 rows, K = 256 .. 768, all tile widths) as about
+    // 5 us + chunks x (1 + ni / 4) us: among the column tiles that divide O take the one with the least
+    // (rounds of 256 workgroups) x (time per workgroup); ties go to the wider tile, which re-reads x less often.
+    const long chunks = ceil_div(I, 32);
+    long best = -1;
+    for (int ni = s.ni; ni >= 1; ni >>= 1) {
+        if (O % (32 * ni) != 0 || ceil_div(O, 32 * ni) > 64) continue;   // at most 64 column tiles (row maxima per tile)
+        const long cost = ceil_div(tiles_m * (O / (32 * ni)), 256) * (20 + chunks * (4 + ni));
+        if (best < 0 || cost < best) { best = cost; s.ni = ni; }
+    }
+    // fewer than two chips' worth of 8-wave workgroups: 4-wave workgroups (128 rows) double their number; not with
+    // 256-column tiles, whose 4-wave variant keeps one wave per SIMD
+    s.waves = (tiles_m * ceil_div(O, 32 * s.ni) >= 512 || (s.ni == 8 && tiles_m >= 32)) ? 8 : 4;
     return s;
 }
 
@@ -448,8 +463,7 @@ int mg_components_to_rows(const float* x, long rows, int dim, int comps, int dim
 }
 
 int mg_tensor_linear_f16x2_rowmax_parts(long rows, int dim_in, int dim_out) {
-    (void)dim_in;
-    return (int)ceil_div(dim_out, 32 * choose_shape(rows, dim_out).ni);
+    return (int)ceil_div(dim_out, 32 * choose_shape(rows, dim_in, dim_out).ni);
 }
 
 int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts,
@@ -472,7 +486,7 @@ int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_
     const _Float16* planes = static_cast<const _Float16*>(packed_W);
     const float* w_inv = reinterpret_cast<const float*>(planes + 2L * O_pad * dim_in);
     hipStream_t st = (hipStream_t)stream;
-    const Shape sh = choose_shape(rows, dim_out);
+    const Shape sh = choose_shape(rows, dim_in, dim_out);
 #define MG_F16X2_LAUNCH(WV, N)                                                                                       \
     return launch<WV, N>(planes, w_inv, x, x_rowmax, x_rowmax_parts, x_rowmax_stride, x_rows_per_bound, rows, dim_in, \
                          dim_out, O_pad, bias, act, accumulate, y, y_rowmax, out_comps, st)

@@ -29,6 +29,47 @@ def _stream():
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
+CONCURRENT_MAX_ROWS = 16384      # above this many rows a kernel fills the chip by itself
+_side_streams = {}
+
+
+def concurrent(fns, rows=0):
+    """Results of independent callables.  With few rows (a single small system) each kernel of a layer occupies a
+    fraction of the chip for a few microseconds, so independent pieces of a layer (the input linears of the three
+    ranks, the three output kernels, the norms) are enqueued on side streams between a fork event and join events and
+    overlap on the GPU when the launches are being captured into a HIP graph; with many rows, one callable or eager
+    execution they simply run in turn.  Every side stream starts after
+    everything enqueued so far on the current stream and the current stream continues after all of them, so sections
+    are totally ordered among each other, memory handed between them needs no extra bookkeeping, and a HIP graph
+    capture records the fork and join as dependencies.  Default stream priority throughout."""
+    fns = list(fns)
+    # eager launches of such small kernels are bound by the host, which the events would only slow down further: the
+    # overlap is for captured graphs
+    if len(fns) < 2 or rows > CONCURRENT_MAX_ROWS or not torch.cuda.is_current_stream_capturing():
+        return [f() for f in fns]
+    main = torch.cuda.current_stream()
+    key = main.device.index
+    pool = _side_streams.setdefault(key, [])
+    while len(pool) < len(fns) - 1:
+        pool.append(torch.cuda.Stream(device=main.device))
+    fork = torch.cuda.Event()
+    fork.record(main)
+    outs = [None] * len(fns)
+    joins = []
+    for k in range(1, len(fns)):
+        side = pool[k - 1]
+        side.wait_event(fork)
+        with torch.cuda.stream(side):
+            outs[k] = fns[k]()
+            done = torch.cuda.Event()
+            done.record(side)
+        joins.append(done)
+    outs[0] = fns[0]()
+    for done in joins:
+        main.wait_event(done)
+    return outs
+
+
 def _p(t):
     return ctypes.c_void_p(t.data_ptr()) if t is not None else ctypes.c_void_p(0)
 
@@ -1379,7 +1420,9 @@ def painn_table_message_sliced(row_ptr, dst, r_ij, table, period, actv_sliced, x
 
 
 def bee_products_linear_supported(n_nodes, chan):
-    return get_linear_mode() == LINEAR_F16X2 and chan % 32 == 0 and chan >= 32 and n_nodes >= 1024
+    # below a few thousand nodes the fused kernels (a workgroup walks the whole reduction dimension, building its
+    # operand from cache reads) are bound by that chain's latency: products kernel + three plain GEMMs are faster
+    return get_linear_mode() == LINEAR_F16X2 and chan % 32 == 0 and chan >= 32 and n_nodes >= 8192
 
 
 def bee_products_linear(rank_o, W, l0, l1, l2, r0, r1, r2, node_bound):

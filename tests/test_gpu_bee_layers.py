@@ -305,7 +305,7 @@ def test_products_and_output_linears_in_one_kernel(pkg, chan, dims, N):
 
 
 def test_self_tens_prods_module_fused_path(pkg):
-    """SelfTensProds at a size that takes the products + linears kernel (chan % 32 == 0, >= 1024 nodes)."""
+    """SelfTensProds at a size that takes the products + linears kernel (chan % 32 == 0, >= 8192 nodes)."""
     bee = importlib.import_module("learned-dynamics_amd.bee_layers")
     torch.manual_seed(8)
     dim_a, dim_v, dim_d, chan = 64, 32, 16, 64
@@ -313,7 +313,7 @@ def test_self_tens_prods_module_fused_path(pkg):
     with torch.no_grad():
         for gn in (mod.gn_a, mod.gn_v, mod.gn_d):
             gn.gamma.copy_(torch.randn_like(gn.gamma))
-    x_a, x_v, x_d = torch.randn(2, 700, dim_a), torch.randn(2, 700, dim_v, 3), torch.randn(2, 700, dim_d, 3, 3)
+    x_a, x_v, x_d = torch.randn(2, 4200, dim_a), torch.randn(2, 4200, dim_v, 3), torch.randn(2, 4200, dim_d, 3, 3)
     with torch.no_grad():
         y_a, y_v, y_d = mod(x_a.cuda(), x_v.cuda(), x_d.cuda(), residual=True)
     dd = lambda t: t.detach().cpu()
