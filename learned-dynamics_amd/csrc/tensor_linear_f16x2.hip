@@ -35,7 +35,6 @@
 // B[k][n] likewise; D[m][n]: n = lane%32, m = 8*(q/4) + 4*(lane/32) + q%4 for register q.
 #include "common.hpp"
 #include "f16x2.hpp"
-#include <cstdlib>
 #include <type_traits>
 
 namespace mg {
