@@ -231,9 +231,10 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
 
             if (active) {
                 T* p = P0 + (e * 3) * chan;
-                p[lane_off] = (T)pl0;                       // 000
-                (p + chan)[lane_off] = (T)pd1;              // 110
-                (p + 2 * chan)[lane_off] = (T)(phi * quad); // 220
+                // outputs are written once and not read back here: streaming stores leave the L2 to the gathered rows
+                __builtin_nontemporal_store((T)pl0, p + lane_off);                       // 000
+                __builtin_nontemporal_store((T)pd1, p + chan + lane_off);                // 110
+                __builtin_nontemporal_store((T)(phi * quad), p + 2 * chan + lane_off);   // 220
             }
             if (edge_max) {
                 // largest |P0| entry of this (edge, 64-channel chunk): a row bound for the per-edge GEMM
@@ -272,9 +273,9 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
             T* o1 = S1 + node * 15 * chan;
             T* o2 = S2 + node * 45 * chan;
 #pragma unroll
-            for (int k = 0; k < 15; k++) (o1 + k * chan)[lane_off] = (T)s1[k];
+            for (int k = 0; k < 15; k++) __builtin_nontemporal_store((T)s1[k], o1 + k * chan + lane_off);
 #pragma unroll
-            for (int k = 0; k < 45; k++) (o2 + k * chan)[lane_off] = (T)s2[k];
+            for (int k = 0; k < 45; k++) __builtin_nontemporal_store((T)s2[k], o2 + k * chan + lane_off);
         }
         if (node_max) {
             // largest |sum| of this (node, 64-channel chunk): a row bound for the GEMMs that read S1 / S2
