@@ -2,17 +2,21 @@
 //
 // Pipeline (all on the caller's stream, no allocation, no host sync):
 //   bin      wrap each atom into the box, cell id
-//   sort     one workgroup per box: counting sort by cell in LDS (histogram, scan,
-//            placement, rank by atom id inside the cell, so that the cell-ordered
-//            array, and with it every output row, is deterministic) -> cell_start.
+//   sort     up to 16 workgroups per box, each sorting a slab of the box's cells:
+//            counting sort by cell in LDS (histogram, scan, placement, rank by
+//            atom id inside the cell, so that the cell-ordered array, and with it
+//            every output row, is deterministic) -> cell_start.
 //            Boxes of more than 16384 atoms or 4096 cells take four kernels instead
 //            (histogram with global atomics, scan, place, order)
 //   count    one workgroup per home cell: the 27 window cells are staged in LDS
 //            once, each wave takes home atoms and sweeps the staged candidates
-//            64 at a time, counting hits with ballot/popcount -> degree, hit masks
+//            64 at a time, counting hits with ballot/popcount -> degree; the hits
+//            themselves go, in window order, into the atom's row of a scratch
+//            array (hit rows of a fixed capacity)
 //   scan     degrees -> CSR row_ptr (+ per-box edge counts, statistics)
-//   fill     replays the hit masks, compacts a row's hits in LDS and writes them
-//            at row_ptr[i] (exact-size rows, no atomics per edge)
+//   fill     copies the hit rows to row_ptr[i] (exact-size rows, no atomics per
+//            edge, no geometry); a row with more hits than a hit row holds is
+//            swept again by one wave
 //
 // fp32 recipe (this file is compiled with -ffp-contract=off):
 //   w    = remainderf(x - box/2, box) + box/2                 (IEEE remainder)
@@ -83,14 +87,14 @@ struct Workspace {
     int* deg_sums;      // sums / maxima of the degrees per tile of kScanTile rows
     int* deg_max;
     int* box_max;       // batch: largest cell occupancy of each box (per-box sort)
-    unsigned long long* masks;   // A x mask_words: hit bits of the count pass, reused by the fill pass
-    int mask_words;     // 64-candidate groups kept per atom (= LDS tile size / 64)
+    int* hits;          // A x hit_cap: neighbours found by the count pass (global atom ids, window order)
+    int hit_cap;        // entries per hit row; rows with more hits are recomputed by the fill pass
     size_t bytes;
 };
 
 inline size_t align_up(size_t v) { return (v + 255) & ~size_t(255); }
 
-Workspace carve(void* base, long A, long C, int mask_words) {
+Workspace carve(void* base, long A, long C, int hit_cap) {
     Workspace w{};
     size_t off = 0;
     auto take = [&](size_t bytes) {
@@ -112,8 +116,8 @@ Workspace carve(void* base, long A, long C, int mask_words) {
     w.deg_sums = static_cast<int*>(take(sizeof(int) * scan_blocks));
     w.deg_max = static_cast<int*>(take(sizeof(int) * scan_blocks));
     w.box_max = static_cast<int*>(take(sizeof(int) * (A > 0 ? A : 1)));   // (batch <= A)
-    w.masks = static_cast<unsigned long long*>(take(sizeof(unsigned long long) * A * mask_words));
-    w.mask_words = mask_words;
+    w.hits = static_cast<int*>(take(sizeof(int) * A * hit_cap));
+    w.hit_cap = hit_cap;
     w.bytes = off;
     return w;
 }
@@ -191,40 +195,61 @@ __global__ void __launch_bounds__(256) bin_kernel(const float* __restrict__ x, G
     if (HIST) w.slot[a] = atomicAdd(&w.cell_count[cell], 1);
 }
 
-// Counting sort of one box by cell, entirely in LDS: histogram (LDS atomics), scan, placement, rank by atom id
-// inside the cell.  One workgroup per box; replaces the histogram / scan / place / order kernels for boxes of at
-// most kSortNodes atoms and kSortCells cells.  Writes cell_start (global positions), sorted, box_max[b].
+// Counting sort of a box by cell, entirely in LDS: histogram (LDS atomics), scan, placement, rank by atom id inside
+// the cell.  A box is shared by gridDim.x workgroups: each takes a contiguous range of the box's cells (a slab),
+// reads the cell of every atom of the box, counts the atoms of the slabs before its own (its place in the
+// cell-ordered array) and sorts the atoms of its own slab.  Replaces the histogram / scan / place / order kernels
+// for boxes of at most kSortNodes atoms and kSortCells cells.  Writes cell_start (global positions), sorted,
+// box_max[b * slabs + slab].
 constexpr int kSortThreads = 1024, kSortNodes = 16384, kSortCells = 4096;   // 2^14 atoms: 14 key bits
+constexpr int kSortSlabsMax = 16;
 __global__ void __launch_bounds__(kSortThreads) sort_box_kernel(Grid g, Workspace w) {
     constexpr int kPer = kSortNodes / kSortThreads, kCellsPer = kSortCells / kSortThreads;
-    __shared__ int start[kSortCells + 1];     // cell sizes, then exclusive starts (start[ncells] = nodes)
+    // cell sizes, then exclusive starts (start[cells of the slab] = its atoms), then a spare bin per lane
+    __shared__ int start[kSortCells + 1 + kWave];
     // keys (cell << 14 | atom) in cell order: a key of a later cell compares greater than any key of this cell, so the
     // rank loop may read past the end of its cell without a bounds check (the array ends in 8 keys of INT_MAX)
-    __shared__ int placed[kSortNodes + 8];
-    __shared__ int wave_sum[kSortThreads / kWave], wave_max[kSortThreads / kWave];
-    const int b = blockIdx.x, tid = threadIdx.x;
+    __shared__ int placed[kSortNodes + 8 + 1];   // (+ a spare word that takes the writes for atoms of other slabs)
+    __shared__ int wave_sum[kSortThreads / kWave], wave_max[kSortThreads / kWave], wave_before[kSortThreads / kWave];
+    const int slab = blockIdx.x, slabs = gridDim.x;
+    const int b = blockIdx.y, tid = threadIdx.x;
     const int lane = tid & (kWave - 1), wave = tid / kWave;
     const long base = (long)b * g.nodes;
     const int cell_base = b * g.ncells;
-    for (int c = tid; c <= g.ncells; c += kSortThreads) start[c] = 0;
+    const int c_lo = (int)((long)slab * g.ncells / slabs), c_hi = (int)((long)(slab + 1) * g.ncells / slabs);
+    const int ncs = c_hi - c_lo;              // cells of this slab
+    for (int c = tid; c <= ncs + kWave; c += kSortThreads) start[c] = 0;
     __syncthreads();
-    int cl[kPer], sl[kPer];
+    int cl[kPer], sl[kPer];                   // cell within the slab (-1: another slab's atom), slot within the cell
+    int n_before = 0;
+    // Straight-line code, so that the 16 loads (and then the 16 LDS atomics) of a thread are in flight together:
+    // an index past the box reads the box's last atom and is discarded, an atom of another slab counts into a
+    // spare bin of its lane.
+    const int* cells = w.cell_of + base;
+    const int last = g.nodes - 1;
 #pragma unroll
     for (int j = 0; j < kPer; j++) {
         const int i = tid + kSortThreads * j;
-        cl[j] = 0; sl[j] = 0;
-        if (i < g.nodes) {
-            cl[j] = w.cell_of[base + i] - cell_base;
-            sl[j] = atomicAdd(&start[cl[j]], 1);
-        }
+        const int c = cells[i < g.nodes ? i : last] - cell_base;
+        cl[j] = i < g.nodes ? c : g.ncells;
     }
+#pragma unroll
+    for (int j = 0; j < kPer; j++) {
+        const int c = cl[j];
+        n_before += c < c_lo ? 1 : 0;
+        const bool own = c >= c_lo && c < c_hi;
+        cl[j] = own ? c - c_lo : -1;
+        sl[j] = atomicAdd(&start[own ? c - c_lo : ncs + 1 + lane], 1);
+    }
+    for (int d = kWave / 2; d > 0; d >>= 1) n_before += __shfl_xor(n_before, d);
+    if (lane == 0) wave_before[wave] = n_before;
     __syncthreads();
     // exclusive scan of the cell sizes: a thread owns kCellsPer consecutive cells
     int cnt[kCellsPer], sum = 0, mx = 0;
 #pragma unroll
     for (int k = 0; k < kCellsPer; k++) {
         const int c = tid * kCellsPer + k;
-        cnt[k] = c < g.ncells ? start[c] : 0;
+        cnt[k] = c < ncs ? start[c] : 0;
         sum += cnt[k];
         mx = cnt[k] > mx ? cnt[k] : mx;
     }
@@ -232,49 +257,56 @@ __global__ void __launch_bounds__(kSortThreads) sort_box_kernel(Grid g, Workspac
     for (int d = kWave / 2; d > 0; d >>= 1) { const int t = __shfl_xor(mx, d); mx = t > mx ? t : mx; }
     if (lane == kWave - 1) wave_sum[wave] = incl;
     if (lane == 0) wave_max[wave] = mx;
+    int before = 0;                           // atoms of this box in the slabs before this one
+    for (int k = 0; k < kSortThreads / kWave; k++) before += wave_before[k];
     __syncthreads();
     int run = incl - sum;
     for (int k = 0; k < wave; k++) run += wave_sum[k];
+    int mine = 0;                             // atoms of this slab
+    for (int k = 0; k < kSortThreads / kWave; k++) mine += wave_sum[k];
 #pragma unroll
     for (int k = 0; k < kCellsPer; k++) {
         const int c = tid * kCellsPer + k;
-        if (c < g.ncells) {
+        if (c < ncs) {
             start[c] = run;
-            w.cell_start[cell_base + c] = (int)base + run;
+            w.cell_start[cell_base + c_lo + c] = (int)base + before + run;
         }
         run += cnt[k];
     }
     if (tid == 0) {
-        start[g.ncells] = g.nodes;
+        start[ncs] = mine;
         int m = 0;
         for (int k = 0; k < kSortThreads / kWave; k++) m = wave_max[k] > m ? wave_max[k] : m;
-        w.box_max[b] = m;
-        if (b == g.batch - 1) w.cell_start[(long)g.batch * g.ncells] = g.batch * g.nodes;
+        w.box_max[b * slabs + slab] = m;
+        if (b == g.batch - 1 && slab == slabs - 1) w.cell_start[(long)g.batch * g.ncells] = g.batch * g.nodes;
     }
     __syncthreads();
 #pragma unroll
     for (int j = 0; j < kPer; j++) {
         const int i = tid + kSortThreads * j;
-        if (i < g.nodes) placed[start[cl[j]] + sl[j]] = (cl[j] << 14) | i;
+        const bool own = cl[j] >= 0;
+        const int first = start[own ? cl[j] : 0];
+        placed[own ? first + sl[j] : kSortNodes + 8] = (cl[j] << 14) | i;
     }
-    if (tid < 8) placed[g.nodes + tid] = 0x7fffffff;
+    if (tid < 8) placed[mine + tid] = 0x7fffffff;
     __syncthreads();
+    // position p of the slab holds atom (key & 16383) of cell (key >> 14); its final place is its rank by atom id
+    // inside the cell.  Going by position keeps every lane busy (a slab has about gridDim.x times fewer atoms than
+    // the box), and the atom's record is requested before the ranking, not after it.
+    for (int p = tid; p < mine; p += kSortThreads) {
+        const int key = placed[p];
+        const int c = key >> 14;
+        const float4 rec = w.wrapped[base + (key & (kSortNodes - 1))];
+        const int lo = start[c], hi = start[c + 1];
+        int rank = 0;
+        for (int q0 = lo; q0 < hi; q0 += 8) {          // 8 independent LDS reads per trip, one wait
+            int v[8];
 #pragma unroll
-    for (int j = 0; j < kPer; j++) {
-        const int i = tid + kSortThreads * j;
-        if (i < g.nodes) {
-            const int lo = start[cl[j]], hi = start[cl[j] + 1];
-            const int key = (cl[j] << 14) | i;
-            int rank = 0;
-            for (int q0 = lo; q0 < hi; q0 += 8) {          // 8 independent LDS reads per trip, one wait
-                int v[8];
+            for (int u = 0; u < 8; u++) v[u] = placed[q0 + u];
 #pragma unroll
-                for (int u = 0; u < 8; u++) v[u] = placed[q0 + u];
-#pragma unroll
-                for (int u = 0; u < 8; u++) rank += v[u] < key ? 1 : 0;
-            }
-            w.sorted[base + lo + rank] = w.wrapped[base + i];
+            for (int u = 0; u < 8; u++) rank += v[u] < key ? 1 : 0;
         }
+        w.sorted[base + before + lo + rank] = rec;
     }
 }
 
@@ -454,19 +486,19 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(const int* __r
 }
 
 
-// One workgroup per home cell, two passes.  The count pass stages the 27 window cells in LDS once
-// (wrapped positions + atom ids), each wave takes home atoms and sweeps the staged candidates 64 at a
-// time; it keeps, per home atom, one 64-bit ballot per group of 64 candidates.  The fill pass replays
-// those masks and never touches the geometry again (it stages only the candidates' atom ids).
-// Windows larger than the LDS tile (kCandCap candidates) take a slow path that reads the tail from
-// global memory and recomputes the geometry in the fill pass.
+// One workgroup per home cell.  The count pass stages the 27 window cells in LDS once (wrapped positions
+// + atom ids), each wave takes home atoms and sweeps the staged candidates 64 at a time; the hits of a
+// group go straight into the atom's hit row, behind the hits of the groups before it, so a hit row lists
+// the neighbours in window order.  The fill pass is a copy of the hit rows to their places in the edge
+// list and never touches the geometry again.  Windows larger than the LDS tile (kCandCap candidates) read
+// their tail from global memory.
 //
-// The hot loops are straight-line code:
+// The hot loop is straight-line code:
 //   * the tile is padded to a multiple of 64 with candidates at +infinity (their distance test fails),
 //     so no lane checks whether its candidate exists;
-//   * the home atom is itself a candidate (the centre cell is part of the window, its place there is
-//     known) and passes the distance test: its bit is cleared once after the sweep instead of
-//     comparing ids on every pair;
+//   * a hit row is addressed through a buffer descriptor that covers exactly that row: entries past its
+//     capacity are dropped by the bounds check of the store, the count goes on, and the fill pass finds
+//     such rows by their degree;
 //   * minimum image without compares: remainder(t, box) = t - rint(t / box) box, evaluated as
 //     fma(-rint(t * (1 / box)), box, t).  For |t| <= box the multiple is -1, 0 or 1 and the fma is
 //     exact, so the result is the IEEE remainder bit for bit unless t / box is within rounding of
@@ -478,10 +510,6 @@ __global__ void __launch_bounds__(kScanThreads) scan_apply_kernel(const int* __r
 //     and such an atom sits in cell 0 because the cell index is taken modulo ndiv.  Only a home cell
 //     whose window holds neither cell 0 nor cell ndiv - 1 on any axis (coordinates 2 .. ndiv - 3,
 //     ndiv >= 5) skips the minimum image altogether: there |w_i - w_j| < 2/5 box.
-//   * the fill pass compacts the hits of a row into a per-wave LDS buffer with mbcnt prefix counts and
-//     writes them as whole runs, a few full-width stores per row instead of a dozen partial ones.
-constexpr int kRowBuf = 256;              // fill pass: hits buffered per wave before they are written (ints)
-
 struct Window {
     int M;            // candidates in the 27 cells
     int self_base;    // the home cell's atoms are candidates self_base .. self_base + home_n - 1
@@ -545,9 +573,14 @@ __device__ __forceinline__ bool within_cutoff(const float4& self, const float4& 
     return d2 <= g.r0sq;
 }
 
+// hits below this lane in a ballot, plus `add`
+__device__ __forceinline__ int hits_below(unsigned long long mask, int add) {
+    return (int)__builtin_amdgcn_mbcnt_hi((unsigned)(mask >> 32),
+                                          __builtin_amdgcn_mbcnt_lo((unsigned)(mask & 0xffffffffull), (unsigned)add));
+}
+
 template <int kCandCap>
 __global__ void __launch_bounds__(256) count_kernel(Grid g, Workspace w) {
-    constexpr int kWords = kCandCap / kWave;
     __shared__ float4 cand[kCandCap];
     __shared__ int range_start[27];
     __shared__ int range_prefix[28];
@@ -573,20 +606,28 @@ __global__ void __launch_bounds__(256) count_kernel(Grid g, Workspace w) {
                      ((g.nz < 5 || cz < 2 || cz > g.nz - 3) ? 4 : 0);
     const float ibx = 1.0f / g.bx, iby = 1.0f / g.by, ibz = 1.0f / g.bz;
     const int node_base = b * g.nodes;
+    const int row_bytes = w.hit_cap * (int)sizeof(int);
 
     for (int h = wave; h < win.home_n; h += nwaves) {
         const int k_self = win.self_base + h;
         float4 self;
         if (k_self < kCandCap) self = cand[k_self];
         else self = w.sorted[win.home_lo + h];
-        const int row = node_base + __float_as_int(self.w);
+        const int row = node_base + __builtin_amdgcn_readfirstlane(__float_as_int(self.w));
+        // descriptor of this atom's hit row alone: a store past the row's capacity is dropped
+        const __amdgpu_buffer_rsrc_t hit_row =
+            __builtin_amdgcn_make_buffer_rsrc(w.hits + (long)row * w.hit_cap, 0, row_bytes, 0x00020000);
+        const int k_self_lane = k_self - lane;         // this lane's candidate is the home atom when k0 == k_self_lane
         int running = 0;
-        unsigned long long keep = 0;                   // lane i keeps the ballot of candidate group i
         auto sweep = [&](auto wrap_tag) {
             constexpr int kWrap = decltype(wrap_tag)::value;
             for (int k0 = 0; k0 < padded; k0 += kWave) {
-                const unsigned long long mask = __ballot(within_cutoff<kWrap>(self, cand[k0 + lane], g, ibx, iby, ibz));
-                if (lane == k0 / kWave) keep = mask;
+                const float4 o = cand[k0 + lane];
+                const bool hit = within_cutoff<kWrap>(self, o, g, ibx, iby, ibz) && k0 != k_self_lane;
+                const unsigned long long mask = __ballot(hit);
+                if (hit)
+                    __builtin_amdgcn_raw_buffer_store_b32(node_base + __float_as_int(o.w), hit_row,
+                                                          hits_below(mask, running) * (int)sizeof(int), 0, 0);
                 running += __popcll(mask);
             }
         };
@@ -600,131 +641,111 @@ __global__ void __launch_bounds__(256) count_kernel(Grid g, Workspace w) {
             case 6: sweep(std::integral_constant<int, 6>{}); break;
             default: sweep(std::integral_constant<int, 7>{}); break;
         }
-        if (k_self < kCandCap) {
-            // the atom found itself: take its bit out of the kept ballot and of the count
-            const int g_self = k_self / kWave;
-            const unsigned long long bit = 1ull << (k_self & (kWave - 1));
-            const int found = lane == g_self ? (int)((keep & bit) != 0ull) : 0;
-            if (lane == g_self) keep &= ~bit;
-            running -= __shfl(found, g_self);
-        }
-        // candidates beyond the tile: from global memory, ids compared
+        // candidates beyond the tile: from global memory
         for (int k0 = kCandCap; k0 < M; k0 += kWave) {
             const int k = k0 + lane;
             bool hit = false;
+            int other = 0;
             if (k < M) {
                 const float4 o = w.sorted[locate(range_start, range_prefix, k)];
+                other = __float_as_int(o.w);
                 hit = k != k_self && within_cutoff<7>(self, o, g, ibx, iby, ibz);
             }
-            running += __popcll(__ballot(hit));
+            const unsigned long long mask = __ballot(hit);
+            if (hit)
+                __builtin_amdgcn_raw_buffer_store_b32(node_base + other, hit_row,
+                                                      hits_below(mask, running) * (int)sizeof(int), 0, 0);
+            running += __popcll(mask);
         }
-        // masks are kept by position in the cell-ordered array: the home atoms of a cell write one contiguous block
-        if (M <= kCandCap && lane < padded / kWave) w.masks[(long)(win.home_lo + h) * kWords + lane] = keep;
         if (lane == 0) w.degree[row] = running;
     }
 }
 
-template <int kCandCap>
+// Fill pass, slow path: one wave sweeps the window of atom `row` again (candidates from global memory, all axes with
+// the minimum image) and writes its hits at out_pos, in window order.  For rows whose hit row was too short.
+__device__ void refill_row(const Grid& g, const Workspace& w, int row, int out_pos, int capacity,
+                           int* __restrict__ src, int* __restrict__ dst) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int b = row / g.nodes;
+    const int id_self = row - b * g.nodes;
+    const int node_base = b * g.nodes;
+    const float4 self = w.wrapped[row];
+    int c = w.cell_of[row] - b * g.ncells;
+    const int cz = c % g.nz;
+    c /= g.nz;
+    const int cy = c % g.ny, cx = c / g.ny;
+    const int t = lane < 27 ? lane : 26;
+    const int dx = t / 9 - 1, dy = (t / 3) % 3 - 1, dz = t % 3 - 1;
+    int nx = cx + dx, ny = cy + dy, nz = cz + dz;
+    nx = nx < 0 ? nx + g.nx : (nx >= g.nx ? nx - g.nx : nx);
+    ny = ny < 0 ? ny + g.ny : (ny >= g.ny ? ny - g.ny : ny);
+    nz = nz < 0 ? nz + g.nz : (nz >= g.nz ? nz - g.nz : nz);
+    const int nc = ((b * g.nx + nx) * g.ny + ny) * g.nz + nz;
+    const int start = w.cell_start[nc];
+    const int len = lane < 27 ? w.cell_start[nc + 1] - start : 0;
+    const int incl = wave_incl_scan(len, lane);
+    const int excl = incl - len;                       // lane t < 27: candidates before cell t of the window
+    const int M = __shfl(incl, 26);
+    const float ibx = 1.0f / g.bx, iby = 1.0f / g.by, ibz = 1.0f / g.bz;
+    int cnt = 0;
+    for (int k0 = 0; k0 < M; k0 += kWave) {
+        const int k = k0 + lane;
+        int lo = 0, hi = 26;                           // last cell of the window with excl <= k (5 halvings of 27)
+#pragma unroll
+        for (int it = 0; it < 5; it++) {
+            const int mid = (lo + hi + 1) >> 1;
+            const int pm = __shfl(excl, mid);
+            if (pm <= k) lo = mid; else hi = mid - 1;
+        }
+        const int st = __shfl(start, lo), ex = __shfl(excl, lo);
+        bool hit = false;
+        int other = 0;
+        if (k < M) {
+            const float4 o = w.sorted[st + (k - ex)];
+            other = __float_as_int(o.w);
+            hit = other != id_self && within_cutoff<7>(self, o, g, ibx, iby, ibz);
+        }
+        const unsigned long long mask = __ballot(hit);
+        const int pos = out_pos + hits_below(mask, cnt);
+        if (hit && pos >= 0 && pos < capacity) {
+            src[pos] = row;
+            dst[pos] = node_base + other;
+        }
+        cnt += __popcll(mask);
+    }
+}
+
+// Fill pass: a workgroup takes kFillRows consecutive rows, whose edges are one contiguous range of the edge list; a
+// thread takes every 256th edge of the range, finds its row among the staged row starts and copies one entry of
+// that row's hits.  Edges beyond the capacity are dropped.
+constexpr int kFillRows = 64;
 __global__ void __launch_bounds__(256) fill_kernel(Grid g, Workspace w, const int* __restrict__ row_ptr,
                                                    int* __restrict__ src, int* __restrict__ dst, int capacity) {
-    constexpr int kWords = kCandCap / kWave;
-    constexpr int kMaxWaves = 4;
-    __shared__ int cand_idx[kCandCap];
-    __shared__ int row_buf[kMaxWaves * kRowBuf];
-    __shared__ int range_start[27];
-    __shared__ int range_prefix[28];
-
-    // grid (nz, ny, nx * batch): the cell coordinates come from the workgroup id without a division chain
-    const int cz = blockIdx.x, cy = blockIdx.y;
-    const int b = blockIdx.z / g.nx, cx = blockIdx.z - b * g.nx;
-    Window win;
-    if (!window_ranges(g, w, b, cx, cy, cz, range_start, range_prefix, &win)) return;
-    const int M = win.M;
-    const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave, nwaves = blockDim.x / kWave;
-    const int staged = M < kCandCap ? M : kCandCap;
-    const int padded = (staged + kWave - 1) & ~(kWave - 1);
-    for (int k = threadIdx.x; k < padded; k += blockDim.x)
-        cand_idx[k] = k < staged ? __float_as_int(w.sorted[locate(range_start, range_prefix, k)].w) : 0;
+    __shared__ int rp[kFillRows + 1];
+    const long A = (long)g.batch * g.nodes;
+    const long r0 = (long)blockIdx.x * kFillRows;
+    const int nrows = A - r0 < kFillRows ? (int)(A - r0) : kFillRows;
+    if ((int)threadIdx.x <= nrows) rp[threadIdx.x] = row_ptr[r0 + threadIdx.x];
     __syncthreads();
-
-    const int node_base = b * g.nodes;
-    const float ibx = 1.0f / g.bx, iby = 1.0f / g.by, ibz = 1.0f / g.bz;
-    int* buf = row_buf + wave * kRowBuf;
-
-    // leave the buffered hits of row `row` at out_pos .. out_pos + cnt - 1 (edges beyond the capacity are dropped)
-    auto flush = [&](int row, int out_pos, int cnt) {
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        for (int i = lane; i < cnt; i += kWave) {
-            const int pos = out_pos + i;
-            if (pos < capacity) {
-                src[pos] = row;
-                dst[pos] = buf[i];
-            }
+    const int cap = w.hit_cap;
+    const int e_hi = rp[nrows];
+    for (int e = rp[0] + (int)threadIdx.x; e < e_hi; e += 256) {
+        int lo = 0, hi = nrows - 1;                    // last row with rp <= e (6 halvings of 64)
+#pragma unroll
+        for (int it = 0; it < 6; it++) {
+            const int mid = (lo + hi + 1) >> 1;
+            if (rp[mid] <= e) lo = mid; else hi = mid - 1;
         }
-        __builtin_amdgcn_wave_barrier();
-    };
-
-    // the fast path keeps one home atom's row start and masks in flight while the previous atom's hits are written
-    int next_row = 0, next_pos = 0;
-    unsigned long long next_keep = 0;
-    auto fetch = [&](int h) {
-        next_row = node_base + cand_idx[win.self_base + h];
-        next_pos = row_ptr[next_row];
-        next_keep = lane < padded / kWave ? w.masks[(long)(win.home_lo + h) * kWords + lane] : 0ull;
-    };
-    if (M <= kCandCap && wave < win.home_n) fetch(wave);
-    for (int h = wave; h < win.home_n; h += nwaves) {
-        const int k_self = win.self_base + h;
-        if (M <= kCandCap) {
-            const int row = next_row;
-            int out_pos = next_pos;
-            int cnt = 0;
-            const unsigned long long keep = next_keep;
-            if (h + nwaves < win.home_n) fetch(h + nwaves);
-            const unsigned keep_lo = (unsigned)(keep & 0xffffffffull), keep_hi = (unsigned)(keep >> 32);
-            for (int k0 = 0; k0 < padded; k0 += kWave) {
-                const int it = k0 / kWave;
-                const unsigned lo = __builtin_amdgcn_readlane(keep_lo, it), hi = __builtin_amdgcn_readlane(keep_hi, it);
-                const unsigned below = __builtin_amdgcn_mbcnt_hi(hi, __builtin_amdgcn_mbcnt_lo(lo, 0u));   // hits in lower lanes
-                const unsigned mine = lane < 32 ? (lo >> lane) & 1u : (hi >> (lane - 32)) & 1u;
-                if (mine) buf[cnt + below] = node_base + cand_idx[k0 + lane];
-                cnt += __popc(lo) + __popc(hi);
-                if (cnt > kRowBuf - kWave) {             // uniform: the next group might not fit
-                    flush(row, out_pos, cnt);
-                    out_pos += cnt;
-                    cnt = 0;
-                }
-            }
-            flush(row, out_pos, cnt);
-        } else {
-            // window larger than the tile: no masks were kept, recompute (ids compared, candidates from global memory)
-            const float4 self = w.sorted[win.home_lo + h];
-            const int row = node_base + __float_as_int(self.w);
-            int out_pos = row_ptr[row];
-            int cnt = 0;
-            for (int k0 = 0; k0 < M; k0 += kWave) {
-                const int k = k0 + lane;
-                bool hit = false;
-                int other_idx = 0;
-                if (k < M) {
-                    const float4 o = w.sorted[locate(range_start, range_prefix, k)];
-                    other_idx = __float_as_int(o.w);
-                    hit = k != k_self && within_cutoff<7>(self, o, g, ibx, iby, ibz);
-                }
-                const unsigned long long mask = __ballot(hit);
-                if (hit) buf[cnt + __popcll(mask & ((1ull << lane) - 1ull))] = node_base + other_idx;
-                cnt += __popcll(mask);
-                if (cnt > kRowBuf - kWave) {
-                    flush(row, out_pos, cnt);
-                    out_pos += cnt;
-                    cnt = 0;
-                }
-            }
-            flush(row, out_pos, cnt);
+        const int idx = e - rp[lo], deg = rp[lo + 1] - rp[lo];
+        if (deg <= cap && idx >= 0 && idx < deg && e >= 0 && e < capacity) {
+            src[e] = (int)(r0 + lo);
+            dst[e] = w.hits[(r0 + lo) * cap + idx];
         }
     }
+    // rows with more hits than a hit row holds: a wave each
+    const int wave = threadIdx.x / kWave;
+    for (int r = wave; r < nrows; r += 256 / kWave)
+        if (rp[r + 1] - rp[r] > cap) refill_row(g, w, (int)(r0 + r), rp[r], capacity, src, dst);
 }
 
 // order[k] = global id of the k-th atom in cell order (cells x-major, atoms by id inside a cell)
@@ -834,9 +855,20 @@ int run_scan(const int* in, long n, int* out, Workspace& w, int* out_total, int*
 }
 
 int pairs_block_size(const Grid& g);
+// workgroups that share the sort of one box: one per 1024 atoms (box_max has batch * nodes entries, so slabs <= nodes)
+int sort_slabs(const Grid& g) {
+    const int s = g.nodes / 1024;
+    return s < 1 ? 1 : (s > kSortSlabsMax ? kSortSlabsMax : s);
+}
 // one workgroup per cell, laid out so that the kernels read the cell coordinates off the workgroup id
 dim3 cell_grid(const Grid& g) { return dim3((unsigned)g.nz, (unsigned)g.ny, (unsigned)(g.nx * g.batch)); }
-int mask_words(const Grid& g) { return (pairs_block_size(g) == 64 ? kCandCapSparse : kCandCapDense) / kWave; }
+// Entries per hit row: twice the number of neighbours a uniform density would give (a sphere of the cutoff radius
+// holds 0.155 of what the 27-cell window holds), in steps of 32, between 32 and 256.
+int hit_cap(const Grid& g) {
+    const double expected = 0.155 * 27.0 * (double)g.nodes / (double)g.ncells;
+    const long cap = ((long)(2.0 * expected) + 31) / 32 * 32;
+    return (int)(cap < 32 ? 32 : (cap > 256 ? 256 : cap));
+}
 
 int pairs_block_size(const Grid& g) {
     // sparse boxes: one wave per cell is plenty
@@ -864,7 +896,7 @@ int mg_neighbour_workspace_bytes(int batch, int nodes, float cutoff, float box_x
     Grid g;
     if (int s = make_grid(cutoff, box_x, box_y, box_z, batch, nodes, &g)) return s;
     const long A = (long)batch * nodes, C = (long)batch * g.ncells;
-    *bytes = carve(nullptr, A, C, mask_words(g)).bytes + 256;
+    *bytes = carve(nullptr, A, C, hit_cap(g)).bytes + 256;
     return MG_OK;
 }
 
@@ -877,7 +909,7 @@ int mg_neighbour_count(const float* x, int batch, int nodes, float cutoff, float
     MG_REQUIRE(batch == 0 || edge_counts, "mg_neighbour_count: edge_counts is null");
     const long A = (long)batch * nodes, C = (long)batch * g.ncells;
     void* base = reinterpret_cast<void*>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~uintptr_t(255));
-    Workspace w = carve(base, A, C, mask_words(g));
+    Workspace w = carve(base, A, C, hit_cap(g));
     if (w.bytes + 256 > workspace_bytes)
         return fail(MG_ERR_WORKSPACE, "mg_neighbour_count: workspace has %zu bytes, %zu needed", workspace_bytes,
                     w.bytes + 256);
@@ -893,7 +925,7 @@ int mg_neighbour_count(const float* x, int batch, int nodes, float cutoff, float
     if (per_box_sort) {
         // six launches in all: bin, per-box sort, count, two for the scan of the degrees, fill
         hipLaunchKernelGGL(bin_kernel<false>, dim3(ablocks), dim3(256), 0, st, x, g, w);
-        hipLaunchKernelGGL(sort_box_kernel, dim3((unsigned)batch), dim3(kSortThreads), 0, st, g, w);
+        hipLaunchKernelGGL(sort_box_kernel, dim3((unsigned)sort_slabs(g), (unsigned)batch), dim3(kSortThreads), 0, st, g, w);
     } else {
         hipLaunchKernelGGL(zero3_kernel, dim3((unsigned)(ceil_div(C, 256) < 1024 ? ceil_div(C, 256) : 1024)), dim3(256),
                            0, st, stats, 4L, row_ptr, 1L, w.cell_count, C);
@@ -910,7 +942,7 @@ int mg_neighbour_count(const float* x, int batch, int nodes, float cutoff, float
                        w.deg_sums, w.deg_max);
     hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)deg_tiles), dim3(kScanThreads), 0, st, (const int*)w.degree, A,
                        (const int*)w.deg_sums, (const int*)w.deg_max, deg_tiles, row_ptr, nodes, edge_counts, stats + 0,
-                       stats + 2, stats + 3, per_box_sort ? (const int*)w.box_max : (const int*)nullptr, batch, stats + 1);
+                       stats + 2, stats + 3, per_box_sort ? (const int*)w.box_max : (const int*)nullptr, batch * sort_slabs(g), stats + 1);
     return check_launch("mg_neighbour_count");
 }
 
@@ -924,16 +956,12 @@ int mg_neighbour_fill(const void* workspace, size_t workspace_bytes, int batch, 
     if (A == 0 || n_edges == 0) return MG_OK;
     MG_REQUIRE(workspace && row_ptr && src && dst, "mg_neighbour_fill: null pointer");
     void* base = reinterpret_cast<void*>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~uintptr_t(255));
-    Workspace w = carve(base, A, C, mask_words(g));
+    Workspace w = carve(base, A, C, hit_cap(g));
     if (w.bytes + 256 > workspace_bytes)
         return fail(MG_ERR_WORKSPACE, "mg_neighbour_fill: workspace has %zu bytes, %zu needed", workspace_bytes,
                     w.bytes + 256);
-    if (pairs_block_size(g) == 64)
-        hipLaunchKernelGGL((fill_kernel<kCandCapSparse>), cell_grid(g), dim3(64), 0, (hipStream_t)stream,
-                           g, w, row_ptr, src, dst, n_edges);
-    else
-        hipLaunchKernelGGL((fill_kernel<kCandCapDense>), cell_grid(g), dim3(256), 0, (hipStream_t)stream,
-                           g, w, row_ptr, src, dst, n_edges);
+    hipLaunchKernelGGL(fill_kernel, dim3((unsigned)ceil_div(A, kFillRows)), dim3(256), 0, (hipStream_t)stream, g, w,
+                       row_ptr, src, dst, n_edges);
     return check_launch("mg_neighbour_fill");
 }
 
@@ -975,7 +1003,7 @@ int mg_neighbour_cell_order(const void* workspace, size_t workspace_bytes, int b
     if (A == 0) return MG_OK;
     MG_REQUIRE(workspace && order, "mg_neighbour_cell_order: null pointer");
     void* base = reinterpret_cast<void*>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~uintptr_t(255));
-    Workspace w = carve(base, A, C, mask_words(g));
+    Workspace w = carve(base, A, C, hit_cap(g));
     if (w.bytes + 256 > workspace_bytes)
         return fail(MG_ERR_WORKSPACE, "mg_neighbour_cell_order: workspace has %zu bytes, %zu needed", workspace_bytes,
                     w.bytes + 256);
