@@ -984,9 +984,10 @@ int mg_neighbour_edges_static(const float* x, int batch, int nodes, float cutoff
     if (int s = mg_neighbour_workspace_bytes(batch, nodes, cutoff, box_x, box_y, box_z, &need)) return s;
     if (need > kScratchBytes)
         return fail(MG_ERR_WORKSPACE,
-                    "mg_neighbour_edges_static: this search needs %zu bytes of workspace, the built-in one holds %zu "
-                    "(about %ld atoms in total); use mg_neighbour_edges with a workspace of your own",
-                    need, kScratchBytes, (long)(kScratchBytes / 180));
+                    "mg_neighbour_edges_static: this search needs %zu bytes of workspace (%zu per atom, most of it the "
+                    "rows that collect each atom's neighbours), the built-in one holds %zu; use mg_neighbour_edges with "
+                    "a workspace of your own",
+                    need, need / (size_t)((long)batch * nodes > 0 ? (long)batch * nodes : 1), kScratchBytes);
     void* ws = nullptr;
     if (int s = scratch_of_current_device(&ws)) return s;
     // every array of the workspace that must start at zero (the cell histogram) is cleared by a kernel inside
