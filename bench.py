@@ -390,7 +390,7 @@ def bench_neighbour(torch, args, with_cpu=True):
     out = {"metric": "neighbour search edges/sec", "value": E / sec, "unit": "edges/s", "ms_per_step": sec * 1e3,
            "dtype": "f32+int32",
            "config": {"workload": "BASELINE configs[1]: 8 boxes x 16384 atoms, box 55 A, cutoff 5 A", "edges": E},
-           "roofline": {"kernel": "whole search (bin, scan, place, order, pairs<count>, scan, pairs<fill>)",
+           "roofline": {"kernel": "whole search (bin, sort, count, scan_sums, scan_apply, fill)",
                         "bound": "hbm", "achieved": alg_bytes / sec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
                         "frac": alg_bytes / sec / 1e9 / PEAK_HBM_GBS, "traffic": None},
            "breakdown": {"count_phase_ms": t_count * 1e3, "fill_phase_ms": t_fill * 1e3,

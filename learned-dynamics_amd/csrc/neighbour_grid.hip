@@ -87,7 +87,7 @@ struct Workspace {
     int* deg_sums;      // sums / maxima of the degrees per tile of kScanTile rows
     int* deg_max;
     int* box_max;       // batch: largest cell occupancy of each box (per-box sort)
-    int* hits;          // A x hit_cap: neighbours found by the count pass (global atom ids, window order)
+    int* hits;          // A x hit_cap: neighbours found by the count pass (box-local atom ids, window order)
     int hit_cap;        // entries per hit row; rows with more hits are recomputed by the fill pass
     size_t bytes;
 };
@@ -592,7 +592,7 @@ __global__ void __launch_bounds__(256) count_kernel(Grid g, Workspace w) {
     if (!window_ranges(g, w, b, cx, cy, cz, range_start, range_prefix, &win)) return;   // uniform
     const int M = win.M;
     const int lane = threadIdx.x & (kWave - 1);
-    const int wave = threadIdx.x / kWave, nwaves = blockDim.x / kWave;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), nwaves = blockDim.x / kWave;   // (scalar)
 
     const int staged = M < kCandCap ? M : kCandCap;
     const int padded = (staged + kWave - 1) & ~(kWave - 1);        // <= kCandCap (a multiple of 64)
@@ -608,8 +608,9 @@ __global__ void __launch_bounds__(256) count_kernel(Grid g, Workspace w) {
     const int node_base = b * g.nodes;
     const int row_bytes = w.hit_cap * (int)sizeof(int);
 
-    for (int h = wave; h < win.home_n; h += nwaves) {
-        const int k_self = win.self_base + h;
+    const int self_base = __builtin_amdgcn_readfirstlane(win.self_base), home_n = __builtin_amdgcn_readfirstlane(win.home_n);
+    for (int h = wave; h < home_n; h += nwaves) {
+        const int k_self = self_base + h;              // uniform
         float4 self;
         if (k_self < kCandCap) self = cand[k_self];
         else self = w.sorted[win.home_lo + h];
@@ -617,17 +618,21 @@ __global__ void __launch_bounds__(256) count_kernel(Grid g, Workspace w) {
         // descriptor of this atom's hit row alone: a store past the row's capacity is dropped
         const __amdgpu_buffer_rsrc_t hit_row =
             __builtin_amdgcn_make_buffer_rsrc(w.hits + (long)row * w.hit_cap, 0, row_bytes, 0x00020000);
-        const int k_self_lane = k_self - lane;         // this lane's candidate is the home atom when k0 == k_self_lane
+        // the home atom is itself a candidate and passes the distance test: its bit is taken out of the ballot of
+        // its group with scalar instructions (no lane compares ids)
+        const int self_group = k_self & ~(kWave - 1);
+        const unsigned long long self_clear = ~(1ull << (k_self & (kWave - 1)));
         int running = 0;
         auto sweep = [&](auto wrap_tag) {
             constexpr int kWrap = decltype(wrap_tag)::value;
             for (int k0 = 0; k0 < padded; k0 += kWave) {
                 const float4 o = cand[k0 + lane];
-                const bool hit = within_cutoff<kWrap>(self, o, g, ibx, iby, ibz) && k0 != k_self_lane;
-                const unsigned long long mask = __ballot(hit);
-                if (hit)
-                    __builtin_amdgcn_raw_buffer_store_b32(node_base + __float_as_int(o.w), hit_row,
-                                                          hits_below(mask, running) * (int)sizeof(int), 0, 0);
+                unsigned long long mask = __ballot(within_cutoff<kWrap>(self, o, g, ibx, iby, ibz));
+                if (k0 == self_group) mask &= self_clear;
+                // (box-local atom ids: the fill pass adds the box's first row)
+                if (__builtin_amdgcn_inverse_ballot_w64(mask))
+                    __builtin_amdgcn_raw_buffer_store_b32(__float_as_int(o.w), hit_row,
+                                                          (hits_below(mask, 0) << 2) + 4 * running, 0, 0);
                 running += __popcll(mask);
             }
         };
@@ -653,8 +658,7 @@ __global__ void __launch_bounds__(256) count_kernel(Grid g, Workspace w) {
             }
             const unsigned long long mask = __ballot(hit);
             if (hit)
-                __builtin_amdgcn_raw_buffer_store_b32(node_base + other, hit_row,
-                                                      hits_below(mask, running) * (int)sizeof(int), 0, 0);
+                __builtin_amdgcn_raw_buffer_store_b32(other, hit_row, hits_below(mask, running) * (int)sizeof(int), 0, 0);
             running += __popcll(mask);
         }
         if (lane == 0) w.degree[row] = running;
@@ -722,10 +726,12 @@ constexpr int kFillRows = 64;
 __global__ void __launch_bounds__(256) fill_kernel(Grid g, Workspace w, const int* __restrict__ row_ptr,
                                                    int* __restrict__ src, int* __restrict__ dst, int capacity) {
     __shared__ int rp[kFillRows + 1];
+    __shared__ int first_row[kFillRows];      // first row of the box that the row belongs to
     const long A = (long)g.batch * g.nodes;
     const long r0 = (long)blockIdx.x * kFillRows;
     const int nrows = A - r0 < kFillRows ? (int)(A - r0) : kFillRows;
     if ((int)threadIdx.x <= nrows) rp[threadIdx.x] = row_ptr[r0 + threadIdx.x];
+    if ((int)threadIdx.x < nrows) first_row[threadIdx.x] = (int)((r0 + threadIdx.x) / g.nodes) * g.nodes;
     __syncthreads();
     const int cap = w.hit_cap;
     const int e_hi = rp[nrows];
@@ -739,7 +745,7 @@ __global__ void __launch_bounds__(256) fill_kernel(Grid g, Workspace w, const in
         const int idx = e - rp[lo], deg = rp[lo + 1] - rp[lo];
         if (deg <= cap && idx >= 0 && idx < deg && e >= 0 && e < capacity) {
             src[e] = (int)(r0 + lo);
-            dst[e] = w.hits[(r0 + lo) * cap + idx];
+            dst[e] = first_row[lo] + w.hits[(r0 + lo) * cap + idx];
         }
     }
     // rows with more hits than a hit row holds: a wave each
