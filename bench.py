@@ -47,7 +47,8 @@ def parse():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="painn_layer",
-                    choices=["painn_layer", "neighbour", "products", "denoiser", "stress", "polymer", "meanflow_painn"])
+                    choices=["painn_layer", "neighbour", "products", "denoiser", "stress", "polymer", "meanflow_painn",
+                             "gemm_power"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-comparisons", action="store_true",
@@ -407,6 +408,88 @@ def bench_neighbour(torch, args, with_cpu=True):
         out["cpu_baseline"] = {"value": len(ref["src"]) / dt, "unit": "edges/s", "cores": 1, "kind": "port",
                                "sample": "1 of the 8 boxes, C cell list (oracle/neighbour_oracle.c), count+fill passes"}
     return out
+
+
+def _board_sample():
+    """(socket power in W, shader clock in MHz) as amd-smi / rocm-smi report them right now; None where unavailable."""
+    import subprocess
+    power = clock = None
+    try:
+        out = subprocess.run(["amd-smi", "metric", "-p", "--json"], capture_output=True, text=True, timeout=10).stdout
+        data = json.loads(out)
+        gpu = (data.get("gpu_data") or data)[0] if isinstance(data, dict) else data[0]
+        power = float(gpu["power"]["socket_power"]["value"])
+    except Exception:
+        pass
+    try:
+        out = subprocess.run(["rocm-smi", "--showclocks", "--json"], capture_output=True, text=True, timeout=10).stdout
+        card = next(iter(json.loads(out).values()))
+        text = next(v for k, v in card.items() if k.startswith("sclk clock speed"))
+        clock = float("".join(ch for ch in text if ch.isdigit() or ch == "."))
+    except Exception:
+        pass
+    return power, clock
+
+
+def bench_gemm_power(torch, args):
+    """The split-fp16 row GEMM at E x 512 x 512 on random and on all-zero operands, with the board's socket power and
+    shader clock sampled while it runs: what limits the kernel is the 1400 W socket power, which the chip holds by
+    lowering its clock."""
+    import statistics
+    import threading
+    ops = importlib.import_module("learned-dynamics_amd.ops")
+    E, K, N = 1046456, 512, 512
+    g = torch.Generator(device="cuda").manual_seed(0x947 + 9)
+    W = torch.randn(N, K, device="cuda", generator=g) * K ** -0.5
+    b = torch.randn(N, device="cuda", generator=g)
+    y = torch.empty(E, N, device="cuda")
+    out = {}
+    for name in ("random", "zeros"):
+        x = torch.randn(E, K, device="cuda", generator=g) if name == "random" else torch.zeros(E, K, device="cuda")
+        xm = ops.row_absmax(x).reshape(E, 1) if name == "random" else torch.ones(E, 1, device="cuda")
+        call = lambda: ops.tensor_linear_f16x2(W, x, xm, bias=b, act=ops.ACT_NONE, out=y)
+        samples, stop = [], threading.Event()
+
+        def sampler():
+            while not stop.is_set():
+                samples.append(_board_sample())
+                time.sleep(0.1)
+
+        th = threading.Thread(target=sampler, daemon=True)
+        for _ in range(20):
+            call()
+        torch.cuda.synchronize()
+        th.start()
+        s, e = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        n, t0 = 0, time.perf_counter()
+        try:
+            s.record()
+            while time.perf_counter() - t0 < 5.0:
+                for _ in range(50):
+                    call()
+                n += 50
+                torch.cuda.synchronize()
+            e.record()
+            torch.cuda.synchronize()
+        finally:
+            stop.set()
+            th.join()
+        ms = s.elapsed_time(e) / n
+        steady = samples[len(samples) // 3:]               # the first samples see the ramp
+        pw = [p for p, _ in steady if p is not None]
+        ck = [c for _, c in steady if c is not None]
+        out[name] = {"ms": ms, "executed_TFLOP/s": 3 * 2 * E * K * N / ms / 1e9, "logical_TFLOP/s": 2 * E * K * N / ms / 1e9,
+                     "socket_power_W_median": statistics.median(pw) if pw else None,
+                     "socket_power_W_max": max(pw) if pw else None,
+                     "shader_clock_MHz_median": statistics.median(ck) if ck else None, "samples": len(steady)}
+        del x, xm
+    r = out["random"]
+    return {"metric": "split-fp16 row GEMM, E x 512 x 512, executed fp16 matrix FLOP/s", "unit": "TFLOP/s",
+            "value": r["executed_TFLOP/s"], "ms_per_step": r["ms"], "dtype": "f32 storage/accumulate, split-fp16 MFMA products",
+            "config": {"workload": "E = 1046456 rows, K = 512, N = 512, bias, no activation; 5 s of back-to-back calls per case"},
+            "detail": out,
+            "note": "socket power from `amd-smi metric -p`, shader clock from `rocm-smi --showclocks`, sampled every 0.1 s "
+                    "by a thread of this process while the GPU runs the loop; the published board power of MI355X is 1400 W"}
 
 
 def bench_products(torch, args):
@@ -822,6 +905,8 @@ def main():
         res = bench_meanflow_painn(torch, args)
     elif args.workload == "polymer":
         res = bench_polymer(torch, args, with_cpu=not args.no_cpu)
+    elif args.workload == "gemm_power":
+        res = bench_gemm_power(torch, args)
     else:
         res = bench_products(torch, args)
         res.setdefault("ms_per_step", res["detail"]["rows_4096"]["us"] * 1e-3)
