@@ -129,6 +129,10 @@ def bench_painn_layer(torch, args):
         xv_flat, xa_flat = x_v_d.reshape(N, n, 3), x_a_d.reshape(N, n)
         t_graph = event_time(torch, lambda: gl.graph_setup(r0, box, pos_d, neighbours_max=512, celllist_max=128), 5)
         breakdown = {"graph_build_ms_not_in_step": t_graph * 1e3}
+        # the same step recorded into a HIP graph and replayed (every launch of the layer, nothing cached between replays)
+        ro = importlib.import_module("learned-dynamics_amd.rollout")
+        graphed = ro.GraphedCall(lambda xa, xv: block((pos_d, graph, r_ij, None, None, xa, xv, box))[5:7], x_a_d, x_v_d)
+        breakdown["layer_ms_replayed_from_a_hip_graph"] = event_time(torch, graphed.graph.replay, 20) * 1e3
         roofline, roofline_hbm = None, None
         comparisons = not getattr(args, "no_comparisons", False)
         if comparisons:
