@@ -48,7 +48,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="painn_layer",
                     choices=["painn_layer", "neighbour", "products", "denoiser", "stress", "polymer", "meanflow_painn",
-                             "gemm_power"])
+                             "gemm_power", "painn_train"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-comparisons", action="store_true",
@@ -496,6 +496,48 @@ def bench_gemm_power(torch, args):
                     "by a thread of this process while the GPU runs the loop; the published board power of MI355X is 1400 W"}
 
 
+def bench_painn_train(torch, args):
+    """Forward + backward of one PaiNN block (Message + Update) at BASELINE configs[2] through the differentiable path
+    (every adjoint a kernel of this library: tensor_linear input / weight gradients, gather / segment-sum adjoints,
+    the elementwise autograd functions); gradients for all parameters and both inputs."""
+    painn = importlib.import_module("learned-dynamics_amd.painn")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    n, n_rbf, r0, box_len = 128, 16, 8.0, 80.0
+    box = (box_len,) * 3
+    seed = 0x947 + 3
+    torch.manual_seed(seed)
+    pos_d = polymer_positions(torch, 16, 1024, box_len, seed).cuda()
+    block = painn.Block(r0, n, n_rbf=n_rbf).cuda().train()
+    g = torch.Generator().manual_seed(seed + 1)
+    x_a = torch.randn(1, 16384, n, generator=g).cuda().requires_grad_(True)
+    x_v = (torch.randn(1, 16384, n, 3, generator=g) / 3 ** 0.5).cuda().requires_grad_(True)
+    with torch.no_grad():
+        graph, r_ij = gl.graph_setup(r0, box, pos_d, neighbours_max=512, celllist_max=128)
+    E = int(graph.src.numel())
+    params = [p for p in block.parameters() if p.requires_grad]
+
+    def step():
+        out = block((pos_d, graph, r_ij, None, None, x_a, x_v, box))
+        loss = out[5].square().mean() + out[6].square().mean()
+        grads = torch.autograd.grad(loss, [x_a, x_v] + params, allow_unused=True)
+        return loss, grads
+
+    loss, grads = step()
+    finite = all(bool(torch.isfinite(gr).all()) for gr in grads if gr is not None)
+    sec = timed_steps(torch, step, args.steps, args.warmup)
+    with torch.no_grad():
+        t_fwd = event_time(torch, lambda: block((pos_d, graph, r_ij, None, None, x_a, x_v, box)), 10)
+    return {"metric": "PaiNN block training step (forward + backward) edges/sec", "unit": "edges/s", "value": E / sec,
+            "ms_per_step": sec * 1e3, "dtype": "f32",
+            "config": {"workload": "BASELINE configs[2]: 16384 atoms, n = 128, 16 radial functions; gradients for the "
+                                   "parameters, x_a and x_v", "edges": E},
+            "detail": {"loss": float(loss), "gradients_finite": finite,
+                       "parameters_with_gradient": sum(gr is not None for gr in grads[2:]),
+                       "inference_forward_ms_same_inputs": t_fwd * 1e3},
+            "note": "the differentiable path evaluates the filter MLP on every edge and stores what the backward pass "
+                    "needs; it is composed of the library's unfused kernels and their adjoints"}
+
+
 def bench_products(torch, args):
     ops = importlib.import_module("learned-dynamics_amd.ops")
     out = {}
@@ -911,6 +953,8 @@ def main():
         res = bench_polymer(torch, args, with_cpu=not args.no_cpu)
     elif args.workload == "gemm_power":
         res = bench_gemm_power(torch, args)
+    elif args.workload == "painn_train":
+        res = bench_painn_train(torch, args)
     else:
         res = bench_products(torch, args)
         res.setdefault("ms_per_step", res["detail"]["rows_4096"]["us"] * 1e-3)

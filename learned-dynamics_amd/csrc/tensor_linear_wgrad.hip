@@ -5,7 +5,10 @@
 // for one 64x64 tile of dW in registers and writes it to its own plane of a
 // workspace; a second kernel adds the planes in slice order.  No atomics: the
 // result does not depend on the order in which workgroups finish.
-// Training-side helper: not on the inference hot path and not tuned.
+// Plain rows (no tensor components) go through the fp32 matrix cores: v_mfma_f32_32x32x2_f32 takes dy and x exactly
+// as they lie in memory (for the reduction index r, lanes 0..31 supply 32 consecutive columns of row r and lanes
+// 32..63 those of row r + 1), products and sums are fp32, nothing is rounded to a shorter format.
+// Training-side helper: not on the inference hot path.
 #include "common.hpp"
 
 namespace mg {
@@ -57,6 +60,190 @@ __global__ void __launch_bounds__(256) wgrad_kernel(const float* __restrict__ dy
         }
 }
 
+// Plain rows on the matrix cores.  A workgroup of 4 waves owns a 128 x 128 tile of dW over its slice of the rows;
+// wave w owns the 64 x 64 quarter (w / 2, w % 2) as 2 x 2 accumulators of 32 x 32.  Columns past the matrix and rows
+// past the slice are read from a clamped address and replaced by zero.
+constexpr int kMTile = 128;
+constexpr int kMRows = 8;       // rows per trip of the loop: 4 matrix steps of 2 rows
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+__global__ void __launch_bounds__(256) wgrad_mfma_kernel(const float* __restrict__ dy, const float* __restrict__ x,
+                                                         long R, int I, int O, long rows_per_block,
+                                                         float* __restrict__ part) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int m = lane & 31, kk = lane >> 5;
+    const int o_base = blockIdx.x * kMTile + (wave >> 1) * 64, i_base = blockIdx.y * kMTile + (wave & 1) * 64;
+    const long r_lo = (long)blockIdx.z * rows_per_block;
+    const long r_hi = r_lo + rows_per_block < R ? r_lo + rows_per_block : R;
+    // this lane's two columns of dy and of x (clamped; `live` says whether the column exists)
+    int oc[2], ic[2];
+    bool o_live[2], i_live[2];
+#pragma unroll
+    for (int p = 0; p < 2; p++) {
+        const int o = o_base + 32 * p + m, i = i_base + 32 * p + m;
+        o_live[p] = o < O; i_live[p] = i < I;
+        oc[p] = o_live[p] ? o : O - 1;
+        ic[p] = i_live[p] ? i : I - 1;
+    }
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int p = 0; p < 2; p++)
+#pragma unroll
+        for (int q = 0; q < 2; q++)
+#pragma unroll
+            for (int k = 0; k < 16; k++) acc[p][q][k] = 0.f;
+
+    // the operands of the next trip are requested before the matrix instructions of this one
+    float a[2][kMRows / 2][2], b[2][kMRows / 2][2];
+    auto fetch = [&](float (&aa)[kMRows / 2][2], float (&bb)[kMRows / 2][2], long r) {
+#pragma unroll
+        for (int s = 0; s < kMRows / 2; s++) {
+            const long row = r + 2 * s + kk;
+            const bool row_live = row < r_hi;
+            const long rc = row_live ? row : r_hi - 1;
+#pragma unroll
+            for (int p = 0; p < 2; p++) {
+                const float va = dy[rc * O + oc[p]], vb = x[rc * I + ic[p]];
+                aa[s][p] = (row_live && o_live[p]) ? va : 0.f;
+                bb[s][p] = (row_live && i_live[p]) ? vb : 0.f;
+            }
+        }
+    };
+    auto multiply = [&](const float (&aa)[kMRows / 2][2], const float (&bb)[kMRows / 2][2]) {
+#pragma unroll
+        for (int s = 0; s < kMRows / 2; s++)
+#pragma unroll
+            for (int p = 0; p < 2; p++)
+#pragma unroll
+                for (int q = 0; q < 2; q++)
+                    acc[p][q] = __builtin_amdgcn_mfma_f32_32x32x2f32(aa[s][p], bb[s][q], acc[p][q], 0, 0, 0);
+    };
+    fetch(a[0], b[0], r_lo);
+    for (long r = r_lo; r < r_hi; r += 2 * kMRows) {
+        fetch(a[1], b[1], r + kMRows);                 // (past the slice: clamped addresses, zeros)
+        multiply(a[0], b[0]);
+        fetch(a[0], b[0], r + 2 * kMRows);
+        multiply(a[1], b[1]);
+    }
+    // D[o][i]: i = lane % 32, o = 8 (k / 4) + 4 (lane / 32) + k % 4 for register k
+    float* plane = part + (long)blockIdx.z * O * I;
+#pragma unroll
+    for (int p = 0; p < 2; p++)
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            const int i = i_base + 32 * q + m;
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                const int o = o_base + 32 * p + 8 * (k / 4) + 4 * kk + (k % 4);
+                if (o < O && i < I) plane[(long)o * I + i] = acc[p][q][k];
+            }
+        }
+}
+
+// The same with the operands staged through LDS, for dimensions that are multiples of 4: a lane of the kernel above
+// loads one float per matrix operand, and the vector memory front end spends as long on such a load as on a 16-byte
+// one (about a cycle per lane), four times the matrix time of the tile.  Here the workgroup loads 16 rows x 128
+// columns of dy and of x with 16-byte loads into LDS (rows padded to 160 floats: the two rows that the two halves of a
+// wave read lie 32 banks apart) and the lanes pick their operands out of LDS; the next 16 rows are on their way while
+// the current ones are multiplied.
+constexpr int kSRows = 16, kSPitch = 160;
+__global__ void __launch_bounds__(256) wgrad_mfma_lds_kernel(const float* __restrict__ dy, const float* __restrict__ x,
+                                                             long R, int I, int O, long rows_per_block,
+                                                             float* __restrict__ part) {
+    __shared__ __attribute__((aligned(16))) float dys[2][kSRows * kSPitch];
+    __shared__ __attribute__((aligned(16))) float xs[2][kSRows * kSPitch];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int m = lane & 31, kk = lane >> 5;
+    const int o_tile = blockIdx.x * kMTile, i_tile = blockIdx.y * kMTile;
+    const int o_wave = (wave >> 1) * 64, i_wave = (wave & 1) * 64;
+    const long r_lo = (long)blockIdx.z * rows_per_block;
+    const long r_hi = r_lo + rows_per_block < R ? r_lo + rows_per_block : R;
+
+    // staging: thread -> two 16-byte pieces per operand (piece = row * 32 + column quad)
+    int st_row[2], st_col[2];
+    bool o_ok[2], i_ok[2];
+    const float* dy_src[2];
+    const float* x_src[2];
+#pragma unroll
+    for (int u = 0; u < 2; u++) {
+        const int piece = threadIdx.x + 256 * u;
+        st_row[u] = piece >> 5;
+        st_col[u] = (piece & 31) * 4;
+        o_ok[u] = o_tile + st_col[u] < O;
+        i_ok[u] = i_tile + st_col[u] < I;
+        dy_src[u] = dy + (o_ok[u] ? o_tile + st_col[u] : 0);
+        x_src[u] = x + (i_ok[u] ? i_tile + st_col[u] : 0);
+    }
+    float4 ra[2], rb[2];
+    auto fetch = [&](long r) {
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const long row = r + st_row[u];
+            const long rc = row < r_hi ? row : r_hi - 1;            // (clamped: replaced by zeros when stored)
+            ra[u] = *reinterpret_cast<const float4*>(dy_src[u] + rc * O);
+            rb[u] = *reinterpret_cast<const float4*>(x_src[u] + rc * I);
+        }
+    };
+    auto store = [&](long r, int buf) {
+        const float4 zero = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int u = 0; u < 2; u++) {
+            const bool row_ok = r + st_row[u] < r_hi;
+            *reinterpret_cast<float4*>(&dys[buf][st_row[u] * kSPitch + st_col[u]]) = (row_ok && o_ok[u]) ? ra[u] : zero;
+            *reinterpret_cast<float4*>(&xs[buf][st_row[u] * kSPitch + st_col[u]]) = (row_ok && i_ok[u]) ? rb[u] : zero;
+        }
+    };
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int p = 0; p < 2; p++)
+#pragma unroll
+        for (int q = 0; q < 2; q++)
+#pragma unroll
+            for (int k = 0; k < 16; k++) acc[p][q][k] = 0.f;
+
+    fetch(r_lo);
+    store(r_lo, 0);
+    __syncthreads();
+    int buf = 0;
+    for (long r = r_lo; r < r_hi; r += kSRows) {
+        const bool more = r + kSRows < r_hi;                          // uniform
+        if (more) fetch(r + kSRows);
+        const float* a_lds = &dys[buf][kk * kSPitch + o_wave + m];
+        const float* b_lds = &xs[buf][kk * kSPitch + i_wave + m];
+#pragma unroll
+        for (int s = 0; s < kSRows / 2; s++) {
+            float a[2], b[2];
+#pragma unroll
+            for (int p = 0; p < 2; p++) {
+                a[p] = a_lds[2 * s * kSPitch + 32 * p];
+                b[p] = b_lds[2 * s * kSPitch + 32 * p];
+            }
+#pragma unroll
+            for (int p = 0; p < 2; p++)
+#pragma unroll
+                for (int q = 0; q < 2; q++)
+                    acc[p][q] = __builtin_amdgcn_mfma_f32_32x32x2f32(a[p], b[q], acc[p][q], 0, 0, 0);
+        }
+        if (more) store(r + kSRows, buf ^ 1);
+        __syncthreads();
+        buf ^= 1;
+    }
+    // D[o][i]: i = lane % 32, o = 8 (k / 4) + 4 (lane / 32) + k % 4 for register k
+    float* plane = part + (long)blockIdx.z * O * I;
+#pragma unroll
+    for (int p = 0; p < 2; p++)
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            const int i = i_tile + i_wave + 32 * q + m;
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                const int o = o_tile + o_wave + 32 * p + 8 * (k / 4) + 4 * kk + (k % 4);
+                if (o < O && i < I) plane[(long)o * I + i] = acc[p][q][k];
+            }
+        }
+}
+
 // dW[k] = part[0][k] + part[1][k] + ... in this order
 __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restrict__ part, long n, int splits,
                                                            float* __restrict__ dW) {
@@ -68,18 +255,20 @@ __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restri
 }
 
 // rows per slice and number of slices for a problem (the same on the sizing and the launching side)
-void wgrad_split(long rows, int dim_in, int dim_out, long* rows_per_block, long* splits) {
-    const int gx = (int)ceil_div(dim_out, kTile), gy = (int)ceil_div(dim_in, kTile);
+void wgrad_split(long rows, int dim_in, int dim_out, int tile, long* rows_per_block, long* splits) {
+    const int gx = (int)ceil_div(dim_out, tile), gy = (int)ceil_div(dim_in, tile);
     long s = ceil_div(1024, (long)gx * gy);             // aim at ~4 workgroups per CU
     const long max_splits = ceil_div(rows, 64);
     if (s > max_splits) s = max_splits;
     if (s < 1) s = 1;
     if (s > 65535) s = 65535;
     long rpb = ceil_div(rows, s);
-    rpb = ceil_div(rpb, kRowsPerStep) * kRowsPerStep;
+    rpb = ceil_div(rpb, kSRows) * kSRows;              // (a multiple of every kernel's rows per trip)
     *rows_per_block = rpb;
     *splits = rows > 0 ? ceil_div(rows, rpb) : 0;
 }
+// plain rows take the matrix-core kernel and its 128 x 128 tiles
+inline int wgrad_tile(int inds) { return inds == 0 ? kMTile : kTile; }
 
 }  // namespace
 }  // namespace mg
@@ -90,8 +279,11 @@ extern "C" {
 
 int mg_tensor_linear_wgrad_workspace_bytes(long rows, int dim_in, int dim_out, size_t* bytes) {
     MG_REQUIRE(bytes != nullptr && rows >= 0 && dim_in >= 0 && dim_out >= 0, "mg_tensor_linear_wgrad_workspace_bytes: bad argument");
-    long rpb, splits;
-    wgrad_split(rows, dim_in, dim_out, &rpb, &splits);
+    // (the number of tensor indices is not known here: room for either kernel's slices)
+    long rpb, s_plain, s_comp;
+    wgrad_split(rows, dim_in, dim_out, kMTile, &rpb, &s_plain);
+    wgrad_split(rows, dim_in, dim_out, kTile, &rpb, &s_comp);
+    const long splits = s_plain > s_comp ? s_plain : s_comp;
     *bytes = (size_t)splits * (size_t)dim_in * (size_t)dim_out * sizeof(float) + 16;
     return MG_OK;
 }
@@ -112,12 +304,18 @@ int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows,
     }
     MG_REQUIRE(dy && x && workspace, "mg_tensor_linear_wgrad: null pointer");
     long rpb, splits;
-    wgrad_split(rows, dim_in, dim_out, &rpb, &splits);
+    const int tile = wgrad_tile(inds);
+    wgrad_split(rows, dim_in, dim_out, tile, &rpb, &splits);
     float* part = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(workspace) + 15) & ~uintptr_t(15));
-    const int gx = (int)ceil_div(dim_out, kTile), gy = (int)ceil_div(dim_in, kTile);
+    const int gx = (int)ceil_div(dim_out, tile), gy = (int)ceil_div(dim_in, tile);
     dim3 grid(gx, gy, (unsigned)splits), block(256);
     switch (inds) {
-        case 0: hipLaunchKernelGGL(wgrad_kernel<1>, grid, block, 0, st, dy, x, rows, dim_in, dim_out, rpb, part); break;
+        case 0:
+            if (dim_in % 4 == 0 && dim_out % 4 == 0 && aligned16(dy) && aligned16(x))
+                hipLaunchKernelGGL(wgrad_mfma_lds_kernel, grid, block, 0, st, dy, x, rows, dim_in, dim_out, rpb, part);
+            else
+                hipLaunchKernelGGL(wgrad_mfma_kernel, grid, block, 0, st, dy, x, rows, dim_in, dim_out, rpb, part);
+            break;
         case 1: hipLaunchKernelGGL(wgrad_kernel<3>, grid, block, 0, st, dy, x, rows, dim_in, dim_out, rpb, part); break;
         default: hipLaunchKernelGGL(wgrad_kernel<9>, grid, block, 0, st, dy, x, rows, dim_in, dim_out, rpb, part); break;
     }

@@ -361,3 +361,22 @@ def test_linear_f16x2_in_row_dynamic_range_meeting_zero_weights(ops, span):
     else:
         assert bool((err <= contract + row_scale).all()), (float(err.max()), e_ref)
         assert float(err.max()) < 3e-5 * float(ref.abs().max())
+
+
+@pytest.mark.parametrize("inds,rows,dim_in,dim_out", [(0, 5000, 117, 210), (0, 70, 16, 512), (0, 1, 33, 31),
+                                                      (0, 100003, 512, 384), (1, 3000, 48, 70), (2, 900, 20, 130)])
+def test_weight_gradient_against_float64(ops, inds, rows, dim_in, dim_out):
+    """dW[o, i] = sum over rows and components of dy[r, o, t] x[r, i, t]: plain rows through the fp32 matrix cores
+    (tiles of 128 x 128 with ragged edges, row slices that do not divide the rows), tensor components through the
+    vector kernel; slices are summed in a fixed order, so two runs agree bit for bit."""
+    g = torch.Generator().manual_seed(rows + dim_in)
+    comps = (3,) * inds
+    x = torch.randn(rows, dim_in, *comps, generator=g).cuda()
+    dy = torch.randn(rows, dim_out, *comps, generator=g).cuda()
+    got = ops.tensor_linear_wgrad(inds, dy, x)
+    want = torch.einsum("ro...,ri...->oi", dy.double(), x.double())
+    fp32 = torch.einsum("ro...,ri...->oi", dy, x).double()
+    scale = float(want.abs().max())
+    err, err_ref = float((got.double() - want).abs().max()), float((fp32 - want).abs().max())
+    assert err <= 1e-6 + 1e-5 * scale + 2 * err_ref, (err, err_ref, scale)
+    assert torch.equal(ops.tensor_linear_wgrad(inds, dy, x), got)
