@@ -119,7 +119,8 @@ def painn_message(msg, graph, x_a, x_v, r_ij):
     """archs/meanflow_painn8.py:85-100"""
     n = msg.n
     dist = mlp_silu(msg.mlp_dist, radial_encode_painn(r_ij, msg.n_rbf, msg.r0))
-    actv = mlp_silu(msg.mlp_actv, gl.edges_read_dst(graph, x_a))
+    # the MLP acts on rows, so it commutes with the gather: N rows go through it, not E (the reference gathers first)
+    actv = gl.edges_read_dst(graph, mlp_silu(msg.mlp_actv, x_a))
     prod = dist * actv
     direction = r_ij / torch.sqrt(msg.epsilon + (r_ij ** 2).sum(-1, keepdim=True))
     v = gl.edges_read_dst(graph, x_v)
