@@ -940,7 +940,8 @@ def main():
             res["other_workloads"] = {"denoiser_forward_configs[3]": dn, "neighbour_search_configs[1]": nb,
                                       "tensor_products_configs[0]": bench_products(torch, small),
                                       "stress_configs[4]": st,
-                                      "meanflow_painn_forward": bench_meanflow_painn(torch, argparse.Namespace(steps=10, warmup=3))}
+                                      "meanflow_painn_forward": bench_meanflow_painn(torch, argparse.Namespace(steps=10, warmup=3)),
+                                      "painn_block_training_step": bench_painn_train(torch, argparse.Namespace(steps=5, warmup=2))}
     elif args.workload == "neighbour":
         res = bench_neighbour(torch, args, with_cpu=not args.no_cpu)
     elif args.workload == "denoiser":

@@ -162,10 +162,21 @@ def bee_messages(msg, graph, r_ij, x_a, x_v, x_d):
     v_j = gl.edges_read_dst(graph, msg.L1(x_v))
     d_j = gl.edges_read_dst(graph, msg.L2(x_d))
     prods = Bee.apply(a_j, v_j, d_j, phi_a.contiguous(), phi_v.contiguous(), phi_d.contiguous())
-    psi_a, psi_v, psi_d = apply_tens_prod_submodules(msg, prods)
+    # The output linears of the vector and rank-2 channels have no bias and nothing nonlinear follows them before the
+    # sum over edges, so they commute with it: the products are summed per node first and the ten linears run on N
+    # rows, not E (the reference applies them per edge).  The scalar channel goes through an MLP per edge.
+    from .ops import BEE_ORDER
+    psi_a, sums = None, [None, None, None]
+    for lab, p in zip(BEE_ORDER, prods):
+        k = int(lab[2])
+        if k == 0:
+            y = getattr(msg, f"Y_{lab}")(p)
+            psi_a = y if psi_a is None else psi_a + y
+        else:
+            y = getattr(msg, f"Y_{lab}")(gl.edges_reduce_src(graph, p.contiguous()))
+            sums[k] = y if sums[k] is None else sums[k] + y
     psi_a = psi_a + mlp_leaky(msg.mlp_a, psi_a)
-    return (0.1 * gl.edges_reduce_src(graph, psi_a), 0.1 * gl.edges_reduce_src(graph, psi_v),
-            0.1 * gl.edges_reduce_src(graph, psi_d))
+    return 0.1 * gl.edges_reduce_src(graph, psi_a), 0.1 * sums[1], 0.1 * sums[2]
 
 
 def self_tens_prods(mod, x_a, x_v, x_d):
