@@ -48,7 +48,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="painn_layer",
                     choices=["painn_layer", "neighbour", "products", "denoiser", "stress", "polymer", "meanflow_painn",
-                             "gemm_power", "painn_train"])
+                             "gemm_power", "painn_train", "denoiser_train"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-comparisons", action="store_true",
@@ -531,11 +531,48 @@ def bench_painn_train(torch, args):
             "ms_per_step": sec * 1e3, "dtype": "f32",
             "config": {"workload": "BASELINE configs[2]: 16384 atoms, n = 128, 16 radial functions; gradients for the "
                                    "parameters, x_a and x_v", "edges": E},
-            "detail": {"loss": float(loss), "gradients_finite": finite,
+            "detail": {"loss": float(loss.detach()), "gradients_finite": finite,
                        "parameters_with_gradient": sum(gr is not None for gr in grads[2:]),
                        "inference_forward_ms_same_inputs": t_fwd * 1e3},
             "note": "the differentiable path evaluates the filter MLP on every edge and stores what the backward pass "
                     "needs; it is composed of the library's unfused kernels and their adjoints"}
+
+
+def bench_denoiser_train(torch, args):
+    """Forward + backward of a 2-block rank-0/1/2 denoiser (Messages + SelfTensProds per block) on 4 systems of 2048
+    atoms through the differentiable path: gradients for every parameter and for the noised positions."""
+    den = importlib.import_module("learned-dynamics_amd.denoiser")
+    seed = 0x947 + 4
+    torch.manual_seed(seed)
+    B, N, box_len, r0 = 4, 2048, 70.0, 6.0
+    dims = dict(dim_a=256, dim_v=64, dim_d=16, chan=256, blocks=2)
+    box = (box_len,) * 3
+    x1 = chain_positions(torch, B, N, box_len, seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    x0 = (x1 + torch.randn(B, N, 3, generator=g)).cuda().requires_grad_(True)
+    one_hot = torch.nn.functional.one_hot(torch.randint(0, 20, (B, N), generator=g), 20).float().cuda()
+    s, t = torch.zeros(B).cuda(), torch.rand(B, generator=g).cuda()
+    x1 = x1.cuda()
+    model = den.Denoiser(r0, **dims).cuda().train()
+    params = [p for p in model.parameters() if p.requires_grad]
+
+    def step():
+        out = model((s, t), x0, x1, one_hot, box)
+        loss = out.square().mean()
+        return loss, torch.autograd.grad(loss, [x0] + params, allow_unused=True)
+
+    loss, grads = step()
+    finite = all(bool(torch.isfinite(gr).all()) for gr in grads if gr is not None)
+    sec = timed_steps(torch, step, args.steps, args.warmup)
+    with torch.no_grad():
+        t_fwd = event_time(torch, lambda: model((s, t), x0, x1, one_hot, box), 5)
+    return {"metric": "rank-0/1/2 denoiser training step (forward + backward) atoms/sec", "unit": "atoms/s",
+            "value": B * N / sec, "ms_per_step": sec * 1e3, "dtype": "f32",
+            "config": {"workload": "2 x [Messages + SelfTensProds], 4 systems x 2048 atoms, box 70 A, cutoff 6 A, 256 scalar "
+                                   "+ 64 vector + 16 rank-2 channels, chan 256; gradients for the parameters and x0"},
+            "detail": {"loss": float(loss.detach()), "gradients_finite": finite,
+                       "parameters_with_gradient": sum(gr is not None for gr in grads[1:]), "parameters": len(params),
+                       "inference_forward_ms_same_inputs": t_fwd * 1e3}}
 
 
 def bench_products(torch, args):
@@ -956,6 +993,8 @@ def main():
         res = bench_gemm_power(torch, args)
     elif args.workload == "painn_train":
         res = bench_painn_train(torch, args)
+    elif args.workload == "denoiser_train":
+        res = bench_denoiser_train(torch, args)
     else:
         res = bench_products(torch, args)
         res.setdefault("ms_per_step", res["detail"]["rows_4096"]["us"] * 1e-3)
