@@ -159,10 +159,10 @@ def test_sparse_box_uses_single_wave_blocks(ops):
     _compare(ops, x, 6.0, box)
 
 
-@pytest.mark.parametrize("nodes,clump", [(600, 80), (5000, 300)])
+@pytest.mark.parametrize("nodes,clump", [(400, 80), (5000, 300)])
 def test_rows_longer_than_a_hit_row_next_to_short_ones(ops, nodes, clump):
     """The count pass leaves each atom's neighbours in a row of fixed capacity (twice the degree a uniform density
-    gives, here 32 and 224 entries) and the fill pass copies the rows; atoms of a clump have more neighbours than
+    gives, here 64 and 224 entries) and the fill pass copies the rows; atoms of a clump have more neighbours than
     that and are swept again by the fill pass.  Both kinds of rows sit in one workgroup's range here, in the
     one-wave (sparse) and in the four-wave variant of the count pass, and the clump straddles a box face."""
     rng = np.random.default_rng(nodes)
