@@ -92,10 +92,9 @@ int mg_neighbour_edges(const float* x /* (batch,nodes,3) */, int batch, int node
 
 /* mg_neighbour_edges without a workspace argument, for callers that cannot allocate one (code under HIP graph
  * capture, tight serving loops, harnesses that forbid allocation).  No counterpart in the reference.  The workspace
- * is a 32 MiB buffer built into the library (one per GPU, held until the process ends); a search that needs more
- * (52 bytes per atom plus 4 bytes per entry of the row that collects an atom's neighbours, 64 to 256 entries
- * depending on the density: roughly 100 000 atoms over all boxes at up to 30 neighbours each, 57 000 at 50) is
- * refused with MG_ERR_WORKSPACE and a message.  The call allocates and frees nothing and synchronises nothing;
+ * is a 64 MiB buffer built into the library (one per GPU, held until the process ends); a search that needs more
+ * (about 1.1 KB per atom, most of it the 256-entry row that collects an atom's neighbours, plus 8 bytes per cell:
+ * roughly 60 000 atoms over all boxes) is refused with MG_ERR_WORKSPACE and a message.  The call allocates and frees nothing and synchronises nothing;
  * inputs and outputs are the caller's.
  * All calls on one GPU share the buffer: calls that overlap in time on the same GPU (two streams, two threads)
  * race, calls ordered on one stream do not.  The first call on a device looks the buffer's address up

@@ -38,7 +38,7 @@ namespace {
 // Built-in workspace of mg_neighbour_edges_static, for callers that cannot allocate one.  One copy per GPU, held
 // from the moment the library is loaded until the process ends.  Host code never passes `scratch` itself anywhere:
 // the name is a host-side handle, the device address comes from hipGetSymbolAddress (scratch_of_current_device).
-constexpr size_t kScratchBytes = size_t(32) << 20;
+constexpr size_t kScratchBytes = size_t(64) << 20;
 static __device__ __align__(256) unsigned char scratch[kScratchBytes];
 constexpr int kMaxDevices = 64;
 void* g_scratch_ptr[kMaxDevices] = {nullptr};
@@ -868,14 +868,10 @@ int sort_slabs(const Grid& g) {
 }
 // one workgroup per cell, laid out so that the kernels read the cell coordinates off the workgroup id
 dim3 cell_grid(const Grid& g) { return dim3((unsigned)g.nz, (unsigned)g.ny, (unsigned)(g.nx * g.batch)); }
-// Entries per hit row: twice the number of neighbours a uniform density would give (a sphere of the cutoff radius
-// holds 0.155 of what the 27-cell window holds), in steps of 32, between 64 and 256.  Atoms with more neighbours than
-// that (clumps in an otherwise empty box) cost the fill pass a second sweep of their window, nothing else.
-int hit_cap(const Grid& g) {
-    const double expected = 0.155 * 27.0 * (double)g.nodes / (double)g.ncells;
-    const long cap = ((long)(2.0 * expected) + 31) / 32 * 32;
-    return (int)(cap < 64 ? 64 : (cap > 256 ? 256 : cap));
-}
+// Entries per hit row.  The host knows the mean density only, and a row that is too short costs a second sweep of the
+// atom's window in the fill pass, so the rows are long enough for any density short of a dense liquid with a long
+// cutoff: 1 KB per atom of address space, of which a search touches what its neighbour counts need.
+int hit_cap(const Grid&) { return 256; }
 
 int pairs_block_size(const Grid& g) {
     // sparse boxes: one wave per cell and a tile of 256 candidates are plenty (10 % faster than four waves at 1.2

@@ -159,19 +159,19 @@ def test_sparse_box_uses_single_wave_blocks(ops):
     _compare(ops, x, 6.0, box)
 
 
-@pytest.mark.parametrize("nodes,clump", [(400, 80), (5000, 300)])
+@pytest.mark.parametrize("nodes,clump", [(400, 300), (5000, 300)])
 def test_rows_longer_than_a_hit_row_next_to_short_ones(ops, nodes, clump):
-    """The count pass leaves each atom's neighbours in a row of fixed capacity (twice the degree a uniform density
-    gives, here 64 and 224 entries) and the fill pass copies the rows; atoms of a clump have more neighbours than
-    that and are swept again by the fill pass.  Both kinds of rows sit in one workgroup's range here, in the
-    one-wave (sparse) and in the four-wave variant of the count pass, and the clump straddles a box face."""
+    """The count pass leaves each atom's neighbours in a row of 256 entries and the fill pass copies the rows; atoms of
+    a clump of 300 have more neighbours than that and are swept again by the fill pass.  Both kinds of rows sit in one
+    workgroup's range here, in the one-wave (sparse, with a window larger than its tile) and in the four-wave variant
+    of the count pass, and the clump straddles a box face."""
     rng = np.random.default_rng(nodes)
     box = (30., 30., 30.)
     x = (rng.random((2, nodes, 3)) * 30).astype(np.float32)
     x[0, ::nodes // clump][:clump] = (rng.standard_normal((clump, 3)) * 0.8 + np.array([29.5, 14., 0.2])).astype(np.float32)
     ref = _compare(ops, x, 5.0, box)
     degrees = ref["counts"].reshape(-1)
-    assert degrees.max() >= clump - 1 and np.median(degrees) < 150
+    assert degrees.max() >= clump - 1 and degrees.min() < 150
 
 
 @pytest.mark.parametrize("seed", range(12))

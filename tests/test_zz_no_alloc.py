@@ -68,7 +68,7 @@ def test_built_in_workspace_gives_the_same_graph_twice_in_a_row():
 def test_search_larger_than_the_built_in_workspace_is_refused():
     L = importlib.import_module("learned-dynamics_amd._lib")
     lib = L.load()
-    B, N = 4, 65536                                                   # 262144 atoms: about 46 MB of workspace
+    B, N = 4, 65536                                                   # 262144 atoms: about 280 MB of workspace
     x = torch.rand(B, N, 3, device="cuda") * 100
     out = _buffers(B, N, 16)
     status = lib.mg_neighbour_edges_static(_ptr(x), B, N, 5.0, 100., 100., 100., _ptr(out["row_ptr"]),
