@@ -61,7 +61,7 @@ int scratch_of_current_device(void** out) {
 }
 
 constexpr int kCandCapDense = 1024;   // candidates staged in LDS per home cell (16 KB), 4-wave workgroups
-constexpr int kCandCapSparse = 256;   // sparse boxes: 1-wave workgroups, 4 KB
+constexpr int kCandCapSparse = 512;   // sparse boxes: 1-wave workgroups, 8 KB
 constexpr int kScanThreads = 256;
 constexpr int kScanItems = 8;       // per thread
 constexpr int kScanTile = kScanThreads * kScanItems;
