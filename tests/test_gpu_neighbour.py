@@ -174,6 +174,26 @@ def test_rows_longer_than_a_hit_row_next_to_short_ones(ops, nodes, clump, box_le
     assert degrees.max() >= clump - 1 and degrees.min() < 150
 
 
+@pytest.mark.parametrize("seed", range(12))
+def test_random_shapes_and_densities(ops, seed):
+    """Boxes, atom counts and densities drawn at random (1 to 4 boxes of 1 to 6000 atoms, 3 to 14 cells per axis,
+    anisotropic, a third of them with a clump and a tenth of the coordinates outside the box): every variant of the
+    sort (1 to 5 slabs per box), of the count pass (one and four waves per cell) and of the fill pass (copied and
+    re-swept rows) against the oracle."""
+    rng = np.random.default_rng(1000 + seed)
+    batch = int(rng.integers(1, 5))
+    nodes = int(rng.choice([1, 2, 63, 64, 65, 300, 1023, 1025, 2500, 6000]))
+    cutoff = float(rng.uniform(2.0, 7.0))
+    box = tuple(float(cutoff * rng.uniform(3.05, 14.0)) for _ in range(3))
+    x = (rng.random((batch, nodes, 3)) * np.array(box)).astype(np.float32)
+    if seed % 3 == 0 and nodes >= 64:
+        k = nodes // 4
+        x[0, :k] = (rng.standard_normal((k, 3)) * 0.5 * cutoff + np.array(box) * rng.random(3)).astype(np.float32)
+    far = rng.random((batch, nodes)) < 0.1
+    x[far] += (rng.integers(-3, 4, size=(int(far.sum()), 3)) * np.array(box)).astype(np.float32)
+    _compare(ops, np.ascontiguousarray(x), cutoff, box)
+
+
 def test_many_candidates_exceed_lds_tile(ops):
     """More candidates in a 27-cell window than the LDS tile holds (1024): the tail is read from global
     memory, and every row is longer than a hit row, so the fill pass sweeps every window again."""
