@@ -278,6 +278,17 @@ int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_
 int mg_tensor_linear_wgrad_workspace_bytes(long rows, int dim_in, int dim_out, size_t* bytes /* host */);
 int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows, int dim_in, int dim_out,
                            void* workspace, float* dW, mg_stream_t stream);
+/* The same for plain rows (inds = 0) on the fp16 matrix cores with two-piece operands: dy and x are each scaled by one
+ * power of two and split into hi + lo fp16 pieces, three matrix instructions per step, fp32 accumulation; the error
+ * is a few fp32 ulps of sum |dy| |x|, as for mg_tensor_linear_f16x2.  dy_bound / x_bound: device arrays of
+ * n_dy_bound / n_x_bound floats whose largest magnitude is an upper bound of |dy| / |x| (for instance the row maxima
+ * from mg_row_absmax; how tight does not matter within a factor 2^14), or NULL: the operand itself is scanned first.
+ * Needs mg_tensor_linear_wgrad_f16x2_supported(rows, dim_in, dim_out) != 0 and 16-byte aligned dy, x; workspace as for
+ * mg_tensor_linear_wgrad.  Same sum as tensor_ops_kern.cu:45-71; scales and bounds have no counterpart there. */
+int mg_tensor_linear_wgrad_f16x2_supported(long rows, int dim_in, int dim_out);   /* returns 0 / 1, not a status */
+int mg_tensor_linear_wgrad_f16x2(const float* dy, const float* x, const float* dy_bound, long n_dy_bound,
+                                 const float* x_bound, long n_x_bound, long rows, int dim_in, int dim_out,
+                                 void* workspace, float* dW, mg_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Ant16 (managan/codegen_tensor_products.py:19-34; ant16_o0_cuda / ant16_o1_cuda / ant16_o2_cuda /

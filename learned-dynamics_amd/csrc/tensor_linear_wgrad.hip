@@ -10,6 +10,7 @@
 // 32..63 those of row r + 1), products and sums are fp32, nothing is rounded to a shorter format.
 // Training-side helper: not on the inference hot path.
 #include "common.hpp"
+#include "f16x2.hpp"
 
 namespace mg {
 namespace {
@@ -65,7 +66,6 @@ __global__ void __launch_bounds__(256) wgrad_kernel(const float* __restrict__ dy
 // past the slice are read from a clamped address and replaced by zero.
 constexpr int kMTile = 128;
 constexpr int kMRows = 8;       // rows per trip of the loop: 4 matrix steps of 2 rows
-typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 __global__ void __launch_bounds__(256) wgrad_mfma_kernel(const float* __restrict__ dy, const float* __restrict__ x,
                                                          long R, int I, int O, long rows_per_block,
@@ -244,6 +244,175 @@ __global__ void __launch_bounds__(256) wgrad_mfma_lds_kernel(const float* __rest
         }
 }
 
+// Plain rows on the fp16 matrix cores with two-piece operands: dy and x are scaled by one power of two each (taken
+// from an upper bound of their magnitudes, so that nothing overflows fp16; an entry 2^17 times smaller than the bound
+// still keeps 22 bits) and split into hi + lo fp16 pieces; dy^T x takes three v_mfma_f32_32x32x16_f16 per step
+// (lo hi, hi lo, hi hi; the lo lo term is below fp32 rounding), accumulated in fp32 and unscaled on the way out.
+//
+// The matrix instruction wants, per lane, 8 consecutive values along the reduction index, which here is the row
+// index: both operands are transposed on their way into LDS.  A stage is 32 rows x 128 columns of each operand.
+// Waves 0-1 stage dy, waves 2-3 stage x: a thread loads 8 rows x 4 columns (eight 16-byte loads), splits the 32
+// values and writes, for each of its 4 columns, the 8 row-consecutive halves of each piece with one 16-byte store.
+// Column c of the tile lives in LDS row 32 (c % 4) + c / 4, so that the 32 column quads of a wave write 32
+// consecutive LDS rows (pitch 80 bytes: conflict free for 16-byte accesses, as for the reads of 32 consecutive rows
+// by the matrix lanes); the epilogue undoes the permutation.  The loads of the next stage are in flight while the
+// current one is multiplied.
+constexpr int kFTile = 128;                        // dW tile edge
+constexpr int kFRows = 32;                         // rows per stage: two matrix steps of 16
+constexpr int kFPlane = kFTile * kRowW;            // bytes of one piece of one operand
+constexpr int kFParts = 1024;                      // partial maxima per operand
+
+// parts[b] = max |x| over the b-th share of n floats (n % 4 == 0, x 16-byte aligned)
+__global__ void __launch_bounds__(256) absmax_parts_kernel(const float* __restrict__ x, long n,
+                                                           float* __restrict__ parts) {
+    float m = 0.f;
+    const long n4 = n >> 2, stride = (long)gridDim.x * 256;
+    const float4* x4 = reinterpret_cast<const float4*>(x);
+    long k = (long)blockIdx.x * 256 + threadIdx.x;
+    for (; k + 3 * stride < n4; k += 4 * stride) {
+        const float4 a = x4[k], b = x4[k + stride], c = x4[k + 2 * stride], d = x4[k + 3 * stride];
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(b.x), fabsf(b.y)), fmaxf(fabsf(b.z), fabsf(b.w))));
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(c.x), fabsf(c.y)), fmaxf(fabsf(c.z), fabsf(c.w))));
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(d.x), fabsf(d.y)), fmaxf(fabsf(d.z), fabsf(d.w))));
+    }
+    for (; k < n4; k += stride) {
+        const float4 a = x4[k];
+        m = fmaxf(m, fmaxf(fmaxf(fabsf(a.x), fabsf(a.y)), fmaxf(fabsf(a.z), fabsf(a.w))));
+    }
+    for (int d = 1; d < 64; d <<= 1) m = fmaxf(m, __shfl_xor(m, d));
+    __shared__ float wave_max[4];
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) parts[blockIdx.x] = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+}
+// the same for an array of any length and alignment (bounds handed in by the caller)
+__global__ void __launch_bounds__(256) absmax_parts_scalar_kernel(const float* __restrict__ x, long n,
+                                                                  float* __restrict__ parts) {
+    float m = 0.f;
+    for (long k = (long)blockIdx.x * 256 + threadIdx.x; k < n; k += (long)gridDim.x * 256) m = fmaxf(m, fabsf(x[k]));
+    for (int d = 1; d < 64; d <<= 1) m = fmaxf(m, __shfl_xor(m, d));
+    __shared__ float wave_max[4];
+    if ((threadIdx.x & 63) == 0) wave_max[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) parts[blockIdx.x] = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+}
+
+__global__ void __launch_bounds__(256) wgrad_f16x2_kernel(const float* __restrict__ dy, const float* __restrict__ x,
+                                                          const float* __restrict__ dy_parts, int n_dy_parts,
+                                                          const float* __restrict__ x_parts, int n_x_parts,
+                                                          long R, int I, int O, long rows_per_block,
+                                                          float* __restrict__ part) {
+    // [operand: dy, x][piece: hi, lo][LDS row][80 bytes]
+    __shared__ __attribute__((aligned(16))) unsigned char lds[4 * kFPlane];
+    __shared__ float wave_max[2][4];
+    const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int m = lane & 31, g = lane >> 5;
+    const int o_tile = blockIdx.x * kFTile, i_tile = blockIdx.y * kFTile;
+    const long r_lo = (long)blockIdx.z * rows_per_block;
+    const long r_hi = r_lo + rows_per_block < R ? r_lo + rows_per_block : R;
+
+    // the two scales, from the partial maxima
+    float ma = 0.f, mb = 0.f;
+    for (int k = threadIdx.x; k < n_dy_parts; k += 256) ma = fmaxf(ma, dy_parts[k]);
+    for (int k = threadIdx.x; k < n_x_parts; k += 256) mb = fmaxf(mb, x_parts[k]);
+    for (int d = 1; d < 64; d <<= 1) { ma = fmaxf(ma, __shfl_xor(ma, d)); mb = fmaxf(mb, __shfl_xor(mb, d)); }
+    if (lane == 0) { wave_max[0][wave] = ma; wave_max[1][wave] = mb; }
+    __syncthreads();
+    ma = fmaxf(fmaxf(wave_max[0][0], wave_max[0][1]), fmaxf(wave_max[0][2], wave_max[0][3]));
+    mb = fmaxf(fmaxf(wave_max[1][0], wave_max[1][1]), fmaxf(wave_max[1][2], wave_max[1][3]));
+    float inv_a, inv_b;
+    const float scale_a = pow2_scale(ma, &inv_a), scale_b = pow2_scale(mb, &inv_b);
+
+    // staging role of this thread: operand (wave-uniform), 8 rows from row 8 * octet, columns 4 cq .. 4 cq + 3
+    const bool stage_x = wave >= 2;
+    const int st = threadIdx.x & 127, octet = st >> 5, cq = st & 31;
+    const int dim = stage_x ? I : O, tile0 = stage_x ? i_tile : o_tile;
+    const bool col_ok = tile0 + 4 * cq < dim;
+    const float* src = (stage_x ? x : dy) + (col_ok ? tile0 + 4 * cq : 0);
+    const float scale = stage_x ? scale_b : scale_a;
+    unsigned char* st_dst = lds + (stage_x ? 2 * kFPlane : 0) + cq * kRowW + octet * 16;
+    float4 v[8];
+    auto fetch = [&](long r) {
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const long row = r + 8 * octet + u;
+            const long rc = row < r_hi ? row : r_hi - 1;            // (clamped: replaced by zeros when stored)
+            v[u] = *reinterpret_cast<const float4*>(src + rc * dim);
+        }
+    };
+    auto store = [&](long r) {
+        halfx8 hi[4], lo[4];
+#pragma unroll
+        for (int u = 0; u < 8; u++) {
+            const bool ok = col_ok && r + 8 * octet + u < r_hi;
+            const HalfSplit4 p = split(ok ? v[u] : make_float4(0.f, 0.f, 0.f, 0.f), scale);
+#pragma unroll
+            for (int j = 0; j < 4; j++) { hi[j][u] = p.hi[j]; lo[j][u] = p.lo[j]; }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            *reinterpret_cast<halfx8*>(st_dst + 32 * j * kRowW) = hi[j];
+            *reinterpret_cast<halfx8*>(st_dst + kFPlane + 32 * j * kRowW) = lo[j];
+        }
+    };
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int p = 0; p < 2; p++)
+#pragma unroll
+        for (int q = 0; q < 2; q++)
+#pragma unroll
+            for (int k = 0; k < 16; k++) acc[p][q][k] = 0.f;
+
+    // matrix lanes: LDS rows 64 (wave / 2) + 32 p + m of dy, 64 (wave % 2) + 32 q + m of x; 16 bytes at (2 step + g)
+    const unsigned char* a_lds = lds + ((wave >> 1) * 64 + m) * kRowW + 16 * g;
+    const unsigned char* b_lds = lds + 2 * kFPlane + ((wave & 1) * 64 + m) * kRowW + 16 * g;
+
+    fetch(r_lo);
+    for (long r = r_lo; r < r_hi; r += kFRows) {
+        __syncthreads();                                   // the matrix lanes are done with the previous stage
+        store(r);
+        __syncthreads();
+        if (r + kFRows < r_hi) fetch(r + kFRows);          // (uniform)
+#pragma unroll
+        for (int s = 0; s < 2; s++) {
+            halfx8 ah[2], al[2], bh[2], bl[2];
+#pragma unroll
+            for (int p = 0; p < 2; p++) {
+                ah[p] = *reinterpret_cast<const halfx8*>(a_lds + 32 * p * kRowW + 32 * s);
+                al[p] = *reinterpret_cast<const halfx8*>(a_lds + kFPlane + 32 * p * kRowW + 32 * s);
+                bh[p] = *reinterpret_cast<const halfx8*>(b_lds + 32 * p * kRowW + 32 * s);
+                bl[p] = *reinterpret_cast<const halfx8*>(b_lds + kFPlane + 32 * p * kRowW + 32 * s);
+            }
+#pragma unroll
+            for (int p = 0; p < 2; p++)
+#pragma unroll
+                for (int q = 0; q < 2; q++) {
+                    // small terms first
+                    acc[p][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al[p], bh[q], acc[p][q], 0, 0, 0);
+                    acc[p][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[p], bl[q], acc[p][q], 0, 0, 0);
+                    acc[p][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[p], bh[q], acc[p][q], 0, 0, 0);
+                }
+        }
+    }
+    // D[row][col]: col = lane % 32, row = 8 (k / 4) + 4 (lane / 32) + k % 4 for register k; LDS row 32 j + c / 4 of
+    // an operand is column 4 (c / 4) + j of the tile
+    const float unscale = inv_a * inv_b;
+    float* plane = part + (long)blockIdx.z * O * I;
+#pragma unroll
+    for (int p = 0; p < 2; p++)
+#pragma unroll
+        for (int q = 0; q < 2; q++) {
+            const int i = i_tile + 4 * m + 2 * (wave & 1) + q;
+#pragma unroll
+            for (int k = 0; k < 16; k++) {
+                const int o = o_tile + 4 * (8 * (k / 4) + 4 * g + (k % 4)) + 2 * (wave >> 1) + p;
+                if (o < O && i < I) plane[(long)o * I + i] = acc[p][q][k] * unscale;
+            }
+        }
+}
+
 // dW[k] = part[0][k] + part[1][k] + ... in this order
 __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restrict__ part, long n, int splits,
                                                            float* __restrict__ dW) {
@@ -284,8 +453,49 @@ int mg_tensor_linear_wgrad_workspace_bytes(long rows, int dim_in, int dim_out, s
     wgrad_split(rows, dim_in, dim_out, kMTile, &rpb, &s_plain);
     wgrad_split(rows, dim_in, dim_out, kTile, &rpb, &s_comp);
     const long splits = s_plain > s_comp ? s_plain : s_comp;
-    *bytes = (size_t)splits * (size_t)dim_in * (size_t)dim_out * sizeof(float) + 16;
+    // (+ the partial maxima of the split-fp16 variant)
+    *bytes = (size_t)splits * (size_t)dim_in * (size_t)dim_out * sizeof(float) + 16 + 2 * kFParts * sizeof(float);
     return MG_OK;
+}
+
+int mg_tensor_linear_wgrad_f16x2_supported(long rows, int dim_in, int dim_out) {
+    return rows >= 4096 && dim_in >= 64 && dim_out >= 64 && dim_in % 4 == 0 && dim_out % 4 == 0;
+}
+
+int mg_tensor_linear_wgrad_f16x2(const float* dy, const float* x, const float* dy_bound, long n_dy_bound,
+                                 const float* x_bound, long n_x_bound, long rows, int dim_in, int dim_out,
+                                 void* workspace, float* dW, mg_stream_t stream) {
+    MG_REQUIRE(mg_tensor_linear_wgrad_f16x2_supported(rows, dim_in, dim_out),
+               "mg_tensor_linear_wgrad_f16x2: needs rows >= 4096 and dims >= 64 that are multiples of 4");
+    MG_REQUIRE(dy && x && workspace && dW, "mg_tensor_linear_wgrad_f16x2: null pointer");
+    MG_REQUIRE(aligned16(dy) && aligned16(x), "mg_tensor_linear_wgrad_f16x2: dy and x must be 16-byte aligned");
+    MG_REQUIRE((dy_bound == nullptr || n_dy_bound > 0) && (x_bound == nullptr || n_x_bound > 0),
+               "mg_tensor_linear_wgrad_f16x2: empty bound array");
+    hipStream_t st = (hipStream_t)stream;
+    const long n = (long)dim_in * dim_out;
+    long rpb, splits;
+    wgrad_split(rows, dim_in, dim_out, kFTile, &rpb, &splits);
+    float* part = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(workspace) + 15) & ~uintptr_t(15));
+    float* maxima = part + splits * n;                       // [dy: kFParts][x: kFParts]
+    auto bound_parts = [&](const float* data, long count, const float* bound, long n_bound, float* parts) -> int {
+        // partial maxima of the caller's bounds, or of the data itself
+        const float* from = bound ? bound : data;
+        const long len = bound ? n_bound : count;
+        const int blocks = (int)(ceil_div(len, 4096) < kFParts ? ceil_div(len, 4096) : kFParts);
+        if (bound)
+            hipLaunchKernelGGL(absmax_parts_scalar_kernel, dim3(blocks), dim3(256), 0, st, from, len, parts);
+        else
+            hipLaunchKernelGGL(absmax_parts_kernel, dim3(blocks), dim3(256), 0, st, from, len, parts);
+        return blocks;
+    };
+    const int na = bound_parts(dy, rows * dim_out, dy_bound, n_dy_bound, maxima);
+    const int nb = bound_parts(x, rows * dim_in, x_bound, n_x_bound, maxima + kFParts);
+    dim3 grid((unsigned)ceil_div(dim_out, kFTile), (unsigned)ceil_div(dim_in, kFTile), (unsigned)splits), block(256);
+    hipLaunchKernelGGL(wgrad_f16x2_kernel, grid, block, 0, st, dy, x, (const float*)maxima, na,
+                       (const float*)(maxima + kFParts), nb, rows, dim_in, dim_out, rpb, part);
+    const unsigned nblocks = (unsigned)(ceil_div(n, 256) < 1024 ? ceil_div(n, 256) : 1024);
+    hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(nblocks), dim3(256), 0, st, (const float*)part, n, (int)splits, dW);
+    return check_launch("mg_tensor_linear_wgrad_f16x2");
 }
 
 int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows, int dim_in, int dim_out,

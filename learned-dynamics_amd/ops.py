@@ -1009,7 +1009,11 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
     return (y, ymax) if want_rowmax else y
 
 
-def tensor_linear_wgrad(inds, dy, x):
+def tensor_linear_wgrad(inds, dy, x, dy_bound=None, x_bound=None):
+    """dW[o, i] = sum over rows and components of dy[.., o, :] x[.., i, :].  Plain rows (inds = 0) of the sizes
+    mg_tensor_linear_wgrad_f16x2 takes go through it while the linear mode is the split-fp16 one; dy_bound / x_bound
+    (float tensors of any shape whose largest magnitude bounds |dy| / |x|, e.g. row maxima that the caller already
+    holds) save it a pass over the operand."""
     _check_input(dy, "dy")
     _check_input(x, "x")
     batch_dims = x.dim() - (1 + inds)
@@ -1022,7 +1026,16 @@ def tensor_linear_wgrad(inds, dy, x):
         nbytes = ctypes.c_size_t(0)
         L.check(_lib.mg_tensor_linear_wgrad_workspace_bytes(rows, dim_in, dim_out, ctypes.byref(nbytes)))
         ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
-        L.check(_lib.mg_tensor_linear_wgrad(inds, _p(dy), _p(x), rows, dim_in, dim_out, _p(ws), _p(dW), _stream()))
+        if (inds == 0 and get_linear_mode() == LINEAR_F16X2 and x.data_ptr() % 16 == 0 and dy.data_ptr() % 16 == 0
+                and _lib.mg_tensor_linear_wgrad_f16x2_supported(rows, dim_in, dim_out)):
+            for b, name in ((dy_bound, "dy_bound"), (x_bound, "x_bound")):
+                if b is not None:
+                    _check_input(b, name)
+            L.check(_lib.mg_tensor_linear_wgrad_f16x2(
+                _p(dy), _p(x), _p(dy_bound), 0 if dy_bound is None else dy_bound.numel(),
+                _p(x_bound), 0 if x_bound is None else x_bound.numel(), rows, dim_in, dim_out, _p(ws), _p(dW), _stream()))
+        else:
+            L.check(_lib.mg_tensor_linear_wgrad(inds, _p(dy), _p(x), rows, dim_in, dim_out, _p(ws), _p(dW), _stream()))
     return dW
 
 

@@ -380,3 +380,38 @@ def test_weight_gradient_against_float64(ops, inds, rows, dim_in, dim_out):
     err, err_ref = float((got.double() - want).abs().max()), float((fp32 - want).abs().max())
     assert err <= 1e-6 + 1e-5 * scale + 2 * err_ref, (err, err_ref, scale)
     assert torch.equal(ops.tensor_linear_wgrad(inds, dy, x), got)
+
+
+@pytest.mark.parametrize("rows,dim_in,dim_out", [(4096, 64, 64), (5000, 68, 132), (40001, 512, 512), (33333, 128, 512),
+                                                 (9000, 260, 64)])
+@pytest.mark.parametrize("bounds", ["scanned", "row maxima", "loose"])
+def test_weight_gradient_split_fp16(ops, rows, dim_in, dim_out, bounds):
+    """Plain rows on the fp16 matrix cores with hi + lo operands: tiles with ragged edges, row slices that do not
+    divide the rows, rows whose magnitudes span 2^12, the scales taken from the operands themselves, from row maxima
+    or from a bound 1000 times too large; to the tolerance of the fp32 kernels, and the same bits on every run."""
+    g = torch.Generator().manual_seed(rows + 3 * dim_in + dim_out)
+    spread = torch.exp2(torch.randint(-12, 1, (rows, 1), generator=g).float())
+    x = (torch.randn(rows, dim_in, generator=g) * spread).cuda()
+    dy = (torch.randn(rows, dim_out, generator=g) * spread.flip(0) * 37.0).cuda()
+    assert ops.get_linear_mode() == ops.LINEAR_F16X2
+    kw = {}
+    if bounds == "row maxima":
+        kw = dict(dy_bound=ops.row_absmax(dy), x_bound=ops.row_absmax(x))
+    elif bounds == "loose":
+        kw = dict(dy_bound=dy.abs().max().reshape(1) * 1000.0, x_bound=x.abs().max().reshape(1) * 1000.0)
+    got = ops.tensor_linear_wgrad(0, dy, x, **kw)
+    want = dy.double().t() @ x.double()
+    fp32 = (dy.t() @ x).double()
+    scale = float(want.abs().max())
+    err, err_ref = float((got.double() - want).abs().max()), float((fp32 - want).abs().max())
+    print(f"[wgrad f16x2 {rows}x{dim_in}x{dim_out} {bounds}] err {err:.3g} fp32 err {err_ref:.3g} scale {scale:.3g}")
+    assert err <= 1e-6 + 1e-5 * scale + 2 * err_ref, (err, err_ref, scale)
+    assert torch.equal(ops.tensor_linear_wgrad(0, dy, x, **kw), got)
+    # the fp32 matrix-core kernel on the same operands
+    ops.set_linear_mode(ops.LINEAR_FP32_MFMA)
+    try:
+        plain = ops.tensor_linear_wgrad(0, dy, x)
+    finally:
+        ops.set_linear_mode(ops.LINEAR_F16X2)
+    assert float((plain.double() - want).abs().max()) <= 1e-6 + 1e-5 * scale + 2 * err_ref
+    assert not torch.equal(plain, got)          # (another kernel, another summation order)
