@@ -254,12 +254,16 @@ __global__ void __launch_bounds__(256) wgrad_mfma_lds_kernel(const float* __rest
 // Waves 0-1 stage dy, waves 2-3 stage x: a thread loads 8 rows x 4 columns (eight 16-byte loads), splits the 32
 // values and writes, for each of its 4 columns, the 8 row-consecutive halves of each piece with one 16-byte store.
 // Column c of the tile lives in LDS row 32 (c % 4) + c / 4, so that the 32 column quads of a wave write 32
-// consecutive LDS rows (pitch 80 bytes: conflict free for 16-byte accesses, as for the reads of 32 consecutive rows
-// by the matrix lanes); the epilogue undoes the permutation.  The loads of the next stage are in flight while the
-// current one is multiplied.
+// consecutive LDS rows (as the matrix lanes read 32 consecutive rows); the epilogue undoes the permutation.  Two
+// stage buffers: while one is multiplied the next stage is split into the other and the loads of the one after are
+// in flight.
 constexpr int kFTile = 128;                        // dW tile edge
 constexpr int kFRows = 32;                         // rows per stage: two matrix steps of 16
-constexpr int kFPlane = kFTile * kRowW;            // bytes of one piece of one operand
+constexpr int kFRowW = 64;                         // bytes per LDS row: 32 halves in four 16-byte pieces, piece k of
+                                                   // row R at position k ^ ((R >> 2) & 3): 16 consecutive rows
+                                                   // touch every bank once, in writes and in reads
+constexpr int kFPlane = kFTile * kFRowW;           // bytes of one piece of one operand
+constexpr int kFBuf = 4 * kFPlane;                 // one stage: two operands x two pieces
 constexpr int kFParts = 1024;                      // partial maxima per operand
 
 // parts[b] = max |x| over the b-th share of n floats (n % 4 == 0, x 16-byte aligned)
@@ -298,14 +302,13 @@ __global__ void __launch_bounds__(256) absmax_parts_scalar_kernel(const float* _
     if (threadIdx.x == 0) parts[blockIdx.x] = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
 }
 
-__global__ void __launch_bounds__(256) wgrad_f16x2_kernel(const float* __restrict__ dy, const float* __restrict__ x,
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) wgrad_f16x2_kernel(const float* __restrict__ dy, const float* __restrict__ x,
                                                           const float* __restrict__ dy_parts, int n_dy_parts,
                                                           const float* __restrict__ x_parts, int n_x_parts,
                                                           long R, int I, int O, long rows_per_block,
                                                           float* __restrict__ part) {
-    // [operand: dy, x][piece: hi, lo][LDS row][80 bytes]
-    __shared__ __attribute__((aligned(16))) unsigned char lds[4 * kFPlane];
-    __shared__ float wave_max[2][4];
+    // [stage buffer][operand: dy, x][piece: hi, lo][LDS row][64 bytes]
+    __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kFBuf];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     const int m = lane & 31, g = lane >> 5;
     const int o_tile = blockIdx.x * kFTile, i_tile = blockIdx.y * kFTile;
@@ -317,43 +320,49 @@ __global__ void __launch_bounds__(256) wgrad_f16x2_kernel(const float* __restric
     for (int k = threadIdx.x; k < n_dy_parts; k += 256) ma = fmaxf(ma, dy_parts[k]);
     for (int k = threadIdx.x; k < n_x_parts; k += 256) mb = fmaxf(mb, x_parts[k]);
     for (int d = 1; d < 64; d <<= 1) { ma = fmaxf(ma, __shfl_xor(ma, d)); mb = fmaxf(mb, __shfl_xor(mb, d)); }
-    if (lane == 0) { wave_max[0][wave] = ma; wave_max[1][wave] = mb; }
+    float* wave_max = reinterpret_cast<float*>(lds);
+    if (lane == 0) { wave_max[wave] = ma; wave_max[4 + wave] = mb; }
     __syncthreads();
-    ma = fmaxf(fmaxf(wave_max[0][0], wave_max[0][1]), fmaxf(wave_max[0][2], wave_max[0][3]));
-    mb = fmaxf(fmaxf(wave_max[1][0], wave_max[1][1]), fmaxf(wave_max[1][2], wave_max[1][3]));
+    ma = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+    mb = fmaxf(fmaxf(wave_max[4], wave_max[5]), fmaxf(wave_max[6], wave_max[7]));
+    __syncthreads();
     float inv_a, inv_b;
     const float scale_a = pow2_scale(ma, &inv_a), scale_b = pow2_scale(mb, &inv_b);
 
-    // staging role of this thread: operand (wave-uniform), 8 rows from row 8 * octet, columns 4 cq .. 4 cq + 3
+    // staging role of this thread: operand (wave-uniform), 8 rows from row 8 * octet, columns 4 cq .. 4 cq + 3.
+    // A stage is the 32 rows from `first`; the last stage of a slice starts at r_hi - 32, inside the matrix
+    // (rows >= 32), and the rows it shares with the stage before, or with the slice before, are scaled by zero, as
+    // are the columns past the matrix (read from column 0): every load is unconditional and in bounds, and its
+    // address is a uniform row address plus a constant lane offset.
     const bool stage_x = wave >= 2;
     const int st = threadIdx.x & 127, octet = st >> 5, cq = st & 31;
     const int dim = stage_x ? I : O, tile0 = stage_x ? i_tile : o_tile;
     const bool col_ok = tile0 + 4 * cq < dim;
-    const float* src = (stage_x ? x : dy) + (col_ok ? tile0 + 4 * cq : 0);
-    const float scale = stage_x ? scale_b : scale_a;
-    unsigned char* st_dst = lds + (stage_x ? 2 * kFPlane : 0) + cq * kRowW + octet * 16;
+    const float* operand = stage_x ? x : dy;                                       // (uniform)
+    const unsigned lane_off = (unsigned)(8 * octet * dim + (col_ok ? tile0 + 4 * cq : 0));
+    const float scale = col_ok ? (stage_x ? scale_b : scale_a) : 0.f;
+    // LDS rows cq + 32 j: their swizzle term ((row >> 2) & 3) does not depend on j
+    unsigned char* st_dst = lds + (stage_x ? 2 * kFPlane : 0) + cq * kFRowW + 16 * (octet ^ ((cq >> 2) & 3));
     float4 v[8];
+    auto first_row = [&](long r) { return r + kFRows <= r_hi ? r : r_hi - kFRows; };
     auto fetch = [&](long r) {
+        const float* rows = operand + first_row(r) * dim;                          // (uniform)
 #pragma unroll
-        for (int u = 0; u < 8; u++) {
-            const long row = r + 8 * octet + u;
-            const long rc = row < r_hi ? row : r_hi - 1;            // (clamped: replaced by zeros when stored)
-            v[u] = *reinterpret_cast<const float4*>(src + rc * dim);
-        }
+        for (int u = 0; u < 8; u++) v[u] = *reinterpret_cast<const float4*>(rows + u * dim + lane_off);
     };
-    auto store = [&](long r) {
+    auto store = [&](long r, int buf_off) {
+        const int first_live = (int)(r - first_row(r)) - 8 * octet;                // rows u >= first_live count
         halfx8 hi[4], lo[4];
 #pragma unroll
         for (int u = 0; u < 8; u++) {
-            const bool ok = col_ok && r + 8 * octet + u < r_hi;
-            const HalfSplit4 p = split(ok ? v[u] : make_float4(0.f, 0.f, 0.f, 0.f), scale);
+            const HalfSplit4 p = split(v[u], u >= first_live ? scale : 0.f);
 #pragma unroll
             for (int j = 0; j < 4; j++) { hi[j][u] = p.hi[j]; lo[j][u] = p.lo[j]; }
         }
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            *reinterpret_cast<halfx8*>(st_dst + 32 * j * kRowW) = hi[j];
-            *reinterpret_cast<halfx8*>(st_dst + kFPlane + 32 * j * kRowW) = lo[j];
+            *reinterpret_cast<halfx8*>(st_dst + buf_off + 32 * j * kFRowW) = hi[j];
+            *reinterpret_cast<halfx8*>(st_dst + buf_off + kFPlane + 32 * j * kFRowW) = lo[j];
         }
     };
 
@@ -365,25 +374,22 @@ __global__ void __launch_bounds__(256) wgrad_f16x2_kernel(const float* __restric
 #pragma unroll
             for (int k = 0; k < 16; k++) acc[p][q][k] = 0.f;
 
-    // matrix lanes: LDS rows 64 (wave / 2) + 32 p + m of dy, 64 (wave % 2) + 32 q + m of x; 16 bytes at (2 step + g)
-    const unsigned char* a_lds = lds + ((wave >> 1) * 64 + m) * kRowW + 16 * g;
-    const unsigned char* b_lds = lds + 2 * kFPlane + ((wave & 1) * 64 + m) * kRowW + 16 * g;
-
-    fetch(r_lo);
-    for (long r = r_lo; r < r_hi; r += kFRows) {
-        __syncthreads();                                   // the matrix lanes are done with the previous stage
-        store(r);
-        __syncthreads();
-        if (r + kFRows < r_hi) fetch(r + kFRows);          // (uniform)
+    // matrix lanes: LDS rows 64 (wave / 2) + 32 p + m of dy, 64 (wave % 2) + 32 q + m of x; 16-byte piece 2 step + g,
+    // swizzled with (row >> 2) & 3 = (m >> 2) & 3
+    const int sw = (m >> 2) & 3;
+    const unsigned char* a_lds = lds + ((wave >> 1) * 64 + m) * kFRowW;
+    const unsigned char* b_lds = lds + 2 * kFPlane + ((wave & 1) * 64 + m) * kFRowW;
+    auto multiply = [&](int buf_off) {
 #pragma unroll
         for (int s = 0; s < 2; s++) {
+            const int piece = buf_off + 16 * ((2 * s + g) ^ sw);
             halfx8 ah[2], al[2], bh[2], bl[2];
 #pragma unroll
             for (int p = 0; p < 2; p++) {
-                ah[p] = *reinterpret_cast<const halfx8*>(a_lds + 32 * p * kRowW + 32 * s);
-                al[p] = *reinterpret_cast<const halfx8*>(a_lds + kFPlane + 32 * p * kRowW + 32 * s);
-                bh[p] = *reinterpret_cast<const halfx8*>(b_lds + 32 * p * kRowW + 32 * s);
-                bl[p] = *reinterpret_cast<const halfx8*>(b_lds + kFPlane + 32 * p * kRowW + 32 * s);
+                ah[p] = *reinterpret_cast<const halfx8*>(a_lds + piece + 32 * p * kFRowW);
+                al[p] = *reinterpret_cast<const halfx8*>(a_lds + piece + kFPlane + 32 * p * kFRowW);
+                bh[p] = *reinterpret_cast<const halfx8*>(b_lds + piece + 32 * p * kFRowW);
+                bl[p] = *reinterpret_cast<const halfx8*>(b_lds + piece + kFPlane + 32 * p * kFRowW);
             }
 #pragma unroll
             for (int p = 0; p < 2; p++)
@@ -395,6 +401,28 @@ __global__ void __launch_bounds__(256) wgrad_f16x2_kernel(const float* __restric
                     acc[p][q] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah[p], bh[q], acc[p][q], 0, 0, 0);
                 }
         }
+    };
+
+    // a stage is multiplied out of one buffer while the next one is split into the other and the loads of the one
+    // after that are on their way
+    // (stages past the slice are fetched and stored like the others, scaled by zero and never multiplied: the loop
+    // body has no branch, and the splitting of one stage can be issued between the matrix instructions of another)
+    fetch(r_lo);
+    store(r_lo, 0);
+    fetch(r_lo + kFRows);
+    __syncthreads();
+    int buf_off = 0;
+    for (long r = r_lo; r < r_hi; r += kFRows) {
+        multiply(buf_off);
+        buf_off ^= kFBuf;
+        store(r + kFRows, buf_off);
+        fetch(r + 2 * kFRows);
+#pragma unroll
+        for (int k = 0; k < 24; k++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // one matrix instruction,
+            __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);     // seven vector instructions in its shadow
+        }
+        __syncthreads();
     }
     // D[row][col]: col = lane % 32, row = 8 (k / 4) + 4 (lane / 32) + k % 4 for register k; LDS row 32 j + c / 4 of
     // an operand is column 4 (c / 4) + j of the tile

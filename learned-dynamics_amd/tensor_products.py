@@ -8,28 +8,45 @@ import torch.nn as nn
 from . import ops
 
 
+def _row_bound(inds, x):
+    """Row maxima of |x| for plain rows that the split-fp16 kernels would otherwise scan themselves (the forward
+    GEMM and the weight gradient both scale by them): computed once per tensor and handed to both."""
+    if inds != 0 or ops.get_linear_mode() != ops.LINEAR_F16X2 or x.dim() < 2:
+        return None
+    x2 = x.reshape(-1, x.shape[-1])
+    if x2.size(0) < 4096 or x2.size(1) < 64 or x2.data_ptr() % 16 != 0:
+        return None
+    return ops.row_absmax(x2)
+
+
 class _TensorLinearFn(torch.autograd.Function):
     """tensor_linear with gradients for W and x (extensions/tensor_ops/tensor_ops.cpp:31-169).  The backward pass is
     itself made of differentiable functions (this one and _WeightGradFn), so the operation can be differentiated any
     number of times, as torch.autograd.functional.jvp(create_graph=True) of the meanflow loss needs
-    (archs/meanflow_painn8.py:274-282); the reference's C++ backward calls raw kernels and cannot."""
+    (archs/meanflow_painn8.py:274-282); the reference's C++ backward calls raw kernels and cannot.
+    x_bound: row maxima of |x| when the caller already holds them (a scaling hint, not differentiated)."""
 
     @staticmethod
-    def forward(ctx, inds, W, x):
+    def forward(ctx, inds, W, x, x_bound=None):
         ctx.inds = inds
+        x = x.contiguous()
+        if x_bound is None:
+            x_bound = _row_bound(inds, x)
+        ctx.x_bound = x_bound
         ctx.save_for_backward(W, x)
-        return ops.tensor_linear_fwd(inds, W, x.contiguous())
+        return ops.tensor_linear_fwd(inds, W, x, row_bound=x_bound)
 
     @staticmethod
     def backward(ctx, dy):
         W, x = ctx.saved_tensors
         dy = dy.contiguous()
         dW = dx = None
+        dy_bound = _row_bound(ctx.inds, dy)
         if ctx.needs_input_grad[1]:
-            dW = _WeightGradFn.apply(ctx.inds, dy, x)
+            dW = _WeightGradFn.apply(ctx.inds, dy, x, dy_bound, ctx.x_bound)
         if ctx.needs_input_grad[2]:
-            dx = _TensorLinearFn.apply(ctx.inds, W.t(), dy)   # strides of W are honoured: no copy
-        return None, dW, dx
+            dx = _TensorLinearFn.apply(ctx.inds, W.t(), dy, dy_bound)   # strides of W are honoured: no copy
+        return None, dW, dx, None
 
 
 class _WeightGradFn(torch.autograd.Function):
@@ -37,20 +54,22 @@ class _WeightGradFn(torch.autograd.Function):
     gradients are two tensor_linear calls."""
 
     @staticmethod
-    def forward(ctx, inds, dy, x):
+    def forward(ctx, inds, dy, x, dy_bound=None, x_bound=None):
         ctx.inds = inds
+        ctx.bounds = (dy_bound, x_bound)
         ctx.save_for_backward(dy, x)
-        return ops.tensor_linear_wgrad(inds, dy.contiguous(), x.contiguous())
+        return ops.tensor_linear_wgrad(inds, dy.contiguous(), x.contiguous(), dy_bound=dy_bound, x_bound=x_bound)
 
     @staticmethod
     def backward(ctx, ddW):
         dy, x = ctx.saved_tensors
+        dy_bound, x_bound = ctx.bounds
         g_dy = g_x = None
         if ctx.needs_input_grad[1]:
-            g_dy = _TensorLinearFn.apply(ctx.inds, ddW, x)            # (.., o, :) = ddW x
+            g_dy = _TensorLinearFn.apply(ctx.inds, ddW, x, x_bound)            # (.., o, :) = ddW x
         if ctx.needs_input_grad[2]:
-            g_x = _TensorLinearFn.apply(ctx.inds, ddW.t(), dy)        # (.., i, :) = ddW^T dy
-        return None, g_dy, g_x
+            g_x = _TensorLinearFn.apply(ctx.inds, ddW.t(), dy, dy_bound)       # (.., i, :) = ddW^T dy
+        return None, g_dy, g_x, None, None
 
 
 def tensor_linear(inds, W, x):
