@@ -14,6 +14,7 @@ import torch
 import torch.nn.functional as F
 
 from . import graph_layers as gl
+from . import ops
 from .codegen_tensor_products import Bee
 from .tensor_products import tensor_linear
 
@@ -115,18 +116,54 @@ def edge_vectors(graph, pos, box):
     return gl.boxwrap(tbox, pos_dst - pos_src)
 
 
+def _painn_combine_plain(dist, actv, v, direction):
+    """archs/meanflow_painn8.py:94-100, as the reference writes it"""
+    n = v.size(1)
+    prod = dist * actv
+    cross = torch.linalg.cross(v, direction[:, None].expand_as(v))
+    m = v * prod[..., :n, None] + cross * prod[..., n:2 * n, None] + direction[:, None] * prod[..., 2 * n:3 * n, None]
+    return m, prod[..., 3 * n:]
+
+
+class _PainnCombine(torch.autograd.Function):
+    """The same lines as one kernel, and their gradient as another.  When the backward pass itself is recorded
+    (create_graph=True, as the Jacobian-vector product of the meanflow loss does), it is evaluated as the gradient of
+    the plain tensor arithmetic instead, which autograd can differentiate again."""
+
+    @staticmethod
+    def forward(ctx, dist, actv, v, direction):
+        ctx.save_for_backward(dist, actv, v, direction)
+        return ops.painn_combine_fwd(dist, actv, v, direction)
+
+    @staticmethod
+    def backward(ctx, dm, da):
+        saved = ctx.saved_tensors
+        if torch.is_grad_enabled():
+            with torch.enable_grad():
+                leaves = [t if t.requires_grad else t.detach().requires_grad_() for t in saved]
+                out = _painn_combine_plain(*leaves)
+                grads = torch.autograd.grad(out, leaves, (dm, da), create_graph=True)
+            return tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad))
+        grads = ops.painn_combine_bwd(*saved, dm.contiguous(), da.contiguous())
+        return tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad))
+
+
+def painn_combine(dist, actv, v, direction):
+    if (ops.painn_combine_supported(v.size(1)) and all(t.is_contiguous() and t.data_ptr() % 16 == 0
+                                                       for t in (dist, actv, v, direction))):
+        return _PainnCombine.apply(dist, actv, v, direction)
+    return _painn_combine_plain(dist, actv, v, direction)
+
+
 def painn_message(msg, graph, x_a, x_v, r_ij):
     """archs/meanflow_painn8.py:85-100"""
-    n = msg.n
     dist = mlp_silu(msg.mlp_dist, radial_encode_painn(r_ij, msg.n_rbf, msg.r0))
     # the MLP acts on rows, so it commutes with the gather: N rows go through it, not E (the reference gathers first)
     actv = gl.edges_read_dst(graph, mlp_silu(msg.mlp_actv, x_a))
-    prod = dist * actv
     direction = r_ij / torch.sqrt(msg.epsilon + (r_ij ** 2).sum(-1, keepdim=True))
     v = gl.edges_read_dst(graph, x_v)
-    cross = torch.linalg.cross(v, direction[:, None].expand_as(v))
-    m = v * prod[..., :n, None] + cross * prod[..., n:2 * n, None] + direction[:, None] * prod[..., 2 * n:3 * n, None]
-    return gl.edges_reduce_src(graph, prod[..., 3 * n:].contiguous()), gl.edges_reduce_src(graph, m)
+    m, a = painn_combine(dist, actv, v, direction)
+    return gl.edges_reduce_src(graph, a.contiguous()), gl.edges_reduce_src(graph, m)
 
 
 def painn_update(upd, x_a, x_v):

@@ -1283,6 +1283,46 @@ def painn_radial_linear(r_ij, n, rmax, W, bias=None, act=ACT_NONE):
     return y
 
 
+def painn_combine_supported(n):
+    return bool(_lib.mg_painn_combine_supported(int(n)))
+
+
+def _combine_inputs(dist, actv, v, direction):
+    for t, name in ((dist, "dist"), (actv, "actv"), (v, "v"), (direction, "direction")):
+        _check_input(t, name)
+    E, n = int(v.size(0)), int(v.size(1))
+    if v.dim() != 3 or v.size(2) != 3 or tuple(dist.shape) != (E, 4 * n) or tuple(actv.shape) != (E, 4 * n) \
+            or tuple(direction.shape) != (E, 3):
+        raise RuntimeError("expected dist, actv (E, 4n), v (E, n, 3), direction (E, 3)")
+    return E, n
+
+
+def painn_combine_fwd(dist, actv, v, direction):
+    """m = v p[:, :n] + (v x direction) p[:, n:2n] + direction p[:, 2n:3n], a = p[:, 3n:] with p = dist * actv
+    (archs/meanflow_painn8.py:94-100), in one pass."""
+    E, n = _combine_inputs(dist, actv, v, direction)
+    with torch.cuda.device(v.device):
+        m = torch.empty(E, n, 3, dtype=torch.float32, device=v.device)
+        a = torch.empty(E, n, dtype=torch.float32, device=v.device)
+        L.check(_lib.mg_painn_combine_fwd(_p(dist), _p(actv), _p(v), _p(direction), E, n, _p(m), _p(a), _stream()))
+    return m, a
+
+
+def painn_combine_bwd(dist, actv, v, direction, dm, da):
+    """Gradients of painn_combine_fwd's four inputs from those of its outputs."""
+    E, n = _combine_inputs(dist, actv, v, direction)
+    _check_input(dm, "dm")
+    _check_input(da, "da")
+    if tuple(dm.shape) != (E, n, 3) or tuple(da.shape) != (E, n):
+        raise RuntimeError("expected dm (E, n, 3) and da (E, n)")
+    with torch.cuda.device(v.device):
+        d_dist, d_actv = torch.empty_like(dist), torch.empty_like(actv)
+        dv, d_dir = torch.empty_like(v), torch.empty_like(direction)
+        L.check(_lib.mg_painn_combine_bwd(_p(dist), _p(actv), _p(v), _p(direction), _p(dm), _p(da), E, n,
+                                          _p(d_dist), _p(d_actv), _p(dv), _p(d_dir), _stream()))
+    return d_dist, d_actv, dv, d_dir
+
+
 def painn_message(row_ptr, dst, r_ij, filt, actv, x_v, epsilon, res_a=None, res_v=None, node_order=None):
     """Fused gather-product-scatter of the PaiNN message (archs/meanflow_painn8.py:91-100).
     filt (E,4n), actv (nodes,4n), x_v (nodes,n,3) -> out_a (nodes,n), out_v (nodes,n,3).

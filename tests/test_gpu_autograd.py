@@ -265,3 +265,36 @@ def test_tensor_prods_module_trains(lro):
     got2 = torch.autograd.grad(sum((r ** 2).sum() for r in got[:2]), [xl_g, xr_g, *params])
     for a, r in zip(list(got) + list(got2), list(ref) + list(ref2)):
         torch.testing.assert_close(a.detach().cpu().double(), r.detach(), rtol=2e-4, atol=2e-5 * float(r.abs().max()) + 1e-9)
+
+
+@pytest.mark.parametrize("E,n", [(1000, 128), (257, 4), (3001, 32), (130, 256)])
+def test_painn_combine_against_plain_arithmetic(pkg, E, n):
+    """The fused elementwise middle of the PaiNN message (archs/meanflow_painn8.py:94-100) and its fused gradient
+    against the same lines in float64 tensor arithmetic; and the gradient of a gradient (which takes the plain
+    arithmetic path) against float64 as well."""
+    diff = importlib.import_module("learned-dynamics_amd.differentiable")
+    g = torch.Generator().manual_seed(E + n)
+    shapes = [(E, 4 * n), (E, 4 * n), (E, n, 3), (E, 3)]
+    cpu = [torch.randn(*s, generator=g, dtype=F64).requires_grad_() for s in shapes]
+    gpu = [t.detach().float().cuda().requires_grad_() for t in cpu]
+    wm, wa = torch.randn(E, n, 3, generator=g, dtype=F64), torch.randn(E, n, generator=g, dtype=F64)
+
+    ref = diff._painn_combine_plain(*cpu)
+    got = diff.painn_combine(*gpu)
+    assert got[0].grad_fn is not None and type(got[0].grad_fn).__name__.startswith("_PainnCombine")
+    _close(got[0], ref[0], "m")
+    _close(got[1], ref[1], "a")
+
+    loss_ref = (ref[0] * wm).sum() + (ref[1] * wa).sum()
+    loss_got = (got[0] * wm.float().cuda()).sum() + (got[1] * wa.float().cuda()).sum()
+    g_ref = torch.autograd.grad(loss_ref, cpu, create_graph=True)
+    g_fused = torch.autograd.grad(loss_got, gpu, retain_graph=True)               # the fused gradient kernel
+    g_got = torch.autograd.grad(loss_got, gpu, create_graph=True)                 # recorded: plain arithmetic
+    for a, b, c, name in zip(g_fused, g_got, g_ref, ("dist", "actv", "v", "direction")):
+        _close(a, c, f"fused gradient of {name}")
+        _close(b, c, f"recorded gradient of {name}")
+    # second order: gradient of |gradient|^2
+    s_ref = sum((t ** 2).sum() for t in g_ref)
+    s_got = sum((t ** 2).sum() for t in g_got)
+    for a, c, name in zip(torch.autograd.grad(s_got, gpu), torch.autograd.grad(s_ref, cpu), ("dist", "actv", "v", "direction")):
+        _close(a, c, f"second-order gradient of {name}", tol=1e-4)
