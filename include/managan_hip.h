@@ -283,12 +283,13 @@ int mg_tensor_linear_wgrad(int inds, const float* dy, const float* x, long rows,
  * is a few fp32 ulps of sum |dy| |x|, as for mg_tensor_linear_f16x2.  dy_bound / x_bound: device arrays of
  * n_dy_bound / n_x_bound floats whose largest magnitude is an upper bound of |dy| / |x| (for instance the row maxima
  * from mg_row_absmax; how tight does not matter within a factor 2^14), or NULL: the operand itself is scanned first.
- * Needs mg_tensor_linear_wgrad_f16x2_supported(rows, dim_in, dim_out) != 0 and 16-byte aligned dy, x; workspace as for
- * mg_tensor_linear_wgrad.  Same sum as tensor_ops_kern.cu:45-71; scales and bounds have no counterpart there. */
+ * db, if not NULL, receives the bias gradient db[o] = sum_r dy[r,o] (plain fp32 sums, slices added in order) from the
+ * same pass.  Needs mg_tensor_linear_wgrad_f16x2_supported(rows, dim_in, dim_out) != 0 and 16-byte aligned dy, x;
+ * workspace as for mg_tensor_linear_wgrad.  Same sum as tensor_ops_kern.cu:45-71; scales and bounds have no counterpart there. */
 int mg_tensor_linear_wgrad_f16x2_supported(long rows, int dim_in, int dim_out);   /* returns 0 / 1, not a status */
 int mg_tensor_linear_wgrad_f16x2(const float* dy, const float* x, const float* dy_bound, long n_dy_bound,
                                  const float* x_bound, long n_x_bound, long rows, int dim_in, int dim_out,
-                                 void* workspace, float* dW, mg_stream_t stream);
+                                 void* workspace, float* dW, float* db /* (dim_out) or NULL */, mg_stream_t stream);
 
 /* ------------------------------------------------------------------------
  * Ant16 (managan/codegen_tensor_products.py:19-34; ant16_o0_cuda / ant16_o1_cuda / ant16_o2_cuda /

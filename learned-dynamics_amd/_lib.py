@@ -54,7 +54,7 @@ _SIGNATURES = {
     "mg_tensor_linear_wgrad_workspace_bytes": [i64, i32, i32, ctypes.POINTER(ctypes.c_size_t)],
     "mg_tensor_linear_wgrad": [i32, vp, vp, i64, i32, i32, vp, vp, vp],
     "mg_tensor_linear_wgrad_f16x2_supported": [i64, i32, i32],
-    "mg_tensor_linear_wgrad_f16x2": [vp, vp, vp, i64, vp, i64, i64, i32, i32, vp, vp, vp],
+    "mg_tensor_linear_wgrad_f16x2": [vp, vp, vp, i64, vp, i64, i64, i32, i32, vp, vp, vp, vp],
     "mg_tensor_linear_layout": [i32, vp, i64, i64, vp, i64, i32, i32, vp, i32, i32, i32, i32, vp, vp],
     "mg_bee_edge_geometry": [vp, i64, f32, vp, vp, vp],
     "mg_bee_message": [vp, vp, vp, i32, i64, vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp],

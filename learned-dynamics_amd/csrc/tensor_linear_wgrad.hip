@@ -306,7 +306,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
                                                           const float* __restrict__ dy_parts, int n_dy_parts,
                                                           const float* __restrict__ x_parts, int n_x_parts,
                                                           long R, int I, int O, long rows_per_block,
-                                                          float* __restrict__ part) {
+                                                          float* __restrict__ part, float* __restrict__ colsum_part) {
     // [stage buffer][operand: dy, x][piece: hi, lo][LDS row][64 bytes]
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kFBuf];
     const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -350,9 +350,19 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
         for (int u = 0; u < 8; u++) v[u] = *reinterpret_cast<const float4*>(rows + u * dim + lane_off);
     };
+    // column sums of dy over the slice (the bias gradient), by the workgroups of the first column of tiles
+    const bool sum_cols = colsum_part != nullptr && blockIdx.y == 0 && !stage_x;   // (uniform)
+    float4 colsum = make_float4(0.f, 0.f, 0.f, 0.f);
     auto store = [&](long r, int buf_off) {
         const int first_live = (int)(r - first_row(r)) - 8 * octet;                // rows u >= first_live count
         halfx8 hi[4], lo[4];
+        if (sum_cols) {
+#pragma unroll
+            for (int u = 0; u < 8; u++) {
+                const float w = (u >= first_live && r < r_hi) ? 1.f : 0.f;
+                colsum.x += w * v[u].x; colsum.y += w * v[u].y; colsum.z += w * v[u].z; colsum.w += w * v[u].w;
+            }
+        }
 #pragma unroll
         for (int u = 0; u < 8; u++) {
             const HalfSplit4 p = split(v[u], u >= first_live ? scale : 0.f);
@@ -424,6 +434,20 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
         }
         __syncthreads();
     }
+    if (colsum_part != nullptr && blockIdx.y == 0) {                              // (uniform)
+        // the four row groups of a column quad, added in a fixed order
+        float4* sums = reinterpret_cast<float4*>(lds);                             // [octet][cq]; the stage buffers are done with
+        if (!stage_x) sums[octet * 32 + cq] = colsum;
+        __syncthreads();
+        if (threadIdx.x < 32) {
+            const float4 s0 = sums[cq], s1 = sums[32 + cq], s2 = sums[64 + cq], s3 = sums[96 + cq];
+            const int o = o_tile + 4 * cq;
+            if (o < O)
+                *reinterpret_cast<float4*>(colsum_part + (long)blockIdx.z * O + o) =
+                    make_float4((s0.x + s1.x) + (s2.x + s3.x), (s0.y + s1.y) + (s2.y + s3.y),
+                                (s0.z + s1.z) + (s2.z + s3.z), (s0.w + s1.w) + (s2.w + s3.w));
+        }
+    }
     // D[row][col]: col = lane % 32, row = 8 (k / 4) + 4 (lane / 32) + k % 4 for register k; LDS row 32 j + c / 4 of
     // an operand is column 4 (c / 4) + j of the tile
     const float unscale = inv_a * inv_b;
@@ -481,20 +505,20 @@ int mg_tensor_linear_wgrad_workspace_bytes(long rows, int dim_in, int dim_out, s
     wgrad_split(rows, dim_in, dim_out, kMTile, &rpb, &s_plain);
     wgrad_split(rows, dim_in, dim_out, kTile, &rpb, &s_comp);
     const long splits = s_plain > s_comp ? s_plain : s_comp;
-    // (+ the partial maxima of the split-fp16 variant)
-    *bytes = (size_t)splits * (size_t)dim_in * (size_t)dim_out * sizeof(float) + 16 + 2 * kFParts * sizeof(float);
+    // (+ the partial maxima and the column sums of the split-fp16 variant)
+    *bytes = (size_t)splits * ((size_t)dim_in + 1) * (size_t)dim_out * sizeof(float) + 16 + 2 * kFParts * sizeof(float);
     return MG_OK;
 }
 
 int mg_tensor_linear_wgrad_f16x2_supported(long rows, int dim_in, int dim_out) {
-    return rows >= 4096 && dim_in >= 64 && dim_out >= 64 && dim_in % 4 == 0 && dim_out % 4 == 0;
+    return rows >= 4096 && dim_in >= 4 && dim_out >= 4 && dim_in % 4 == 0 && dim_out % 4 == 0;
 }
 
 int mg_tensor_linear_wgrad_f16x2(const float* dy, const float* x, const float* dy_bound, long n_dy_bound,
                                  const float* x_bound, long n_x_bound, long rows, int dim_in, int dim_out,
-                                 void* workspace, float* dW, mg_stream_t stream) {
+                                 void* workspace, float* dW, float* db, mg_stream_t stream) {
     MG_REQUIRE(mg_tensor_linear_wgrad_f16x2_supported(rows, dim_in, dim_out),
-               "mg_tensor_linear_wgrad_f16x2: needs rows >= 4096 and dims >= 64 that are multiples of 4");
+               "mg_tensor_linear_wgrad_f16x2: needs rows >= 4096 and dims that are multiples of 4");
     MG_REQUIRE(dy && x && workspace && dW, "mg_tensor_linear_wgrad_f16x2: null pointer");
     MG_REQUIRE(aligned16(dy) && aligned16(x), "mg_tensor_linear_wgrad_f16x2: dy and x must be 16-byte aligned");
     MG_REQUIRE((dy_bound == nullptr || n_dy_bound > 0) && (x_bound == nullptr || n_x_bound > 0),
@@ -505,6 +529,7 @@ int mg_tensor_linear_wgrad_f16x2(const float* dy, const float* x, const float* d
     wgrad_split(rows, dim_in, dim_out, kFTile, &rpb, &splits);
     float* part = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(workspace) + 15) & ~uintptr_t(15));
     float* maxima = part + splits * n;                       // [dy: kFParts][x: kFParts]
+    float* colsum_part = db ? maxima + 2 * kFParts : nullptr; // [slice][dim_out]
     auto bound_parts = [&](const float* data, long count, const float* bound, long n_bound, float* parts) -> int {
         // partial maxima of the caller's bounds, or of the data itself
         const float* from = bound ? bound : data;
@@ -520,9 +545,12 @@ int mg_tensor_linear_wgrad_f16x2(const float* dy, const float* x, const float* d
     const int nb = bound_parts(x, rows * dim_in, x_bound, n_x_bound, maxima + kFParts);
     dim3 grid((unsigned)ceil_div(dim_out, kFTile), (unsigned)ceil_div(dim_in, kFTile), (unsigned)splits), block(256);
     hipLaunchKernelGGL(wgrad_f16x2_kernel, grid, block, 0, st, dy, x, (const float*)maxima, na,
-                       (const float*)(maxima + kFParts), nb, rows, dim_in, dim_out, rpb, part);
+                       (const float*)(maxima + kFParts), nb, rows, dim_in, dim_out, rpb, part, colsum_part);
     const unsigned nblocks = (unsigned)(ceil_div(n, 256) < 1024 ? ceil_div(n, 256) : 1024);
     hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(nblocks), dim3(256), 0, st, (const float*)part, n, (int)splits, dW);
+    if (db)
+        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)ceil_div(dim_out, 256)), dim3(256), 0, st,
+                           (const float*)colsum_part, (long)dim_out, (int)splits, db);
     return check_launch("mg_tensor_linear_wgrad_f16x2");
 }
 

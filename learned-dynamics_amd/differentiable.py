@@ -31,9 +31,7 @@ def wants_grad(module, *tensors):
 def linear(lin, x):
     """nn.Linear through the tensor_linear kernels (weight and input gradients are kernels too)."""
     lead = x.shape[:-1]
-    y = tensor_linear(0, lin.weight, x.reshape(-1, x.shape[-1]).contiguous())
-    if lin.bias is not None:
-        y = y + lin.bias
+    y = tensor_linear(0, lin.weight, x.reshape(-1, x.shape[-1]).contiguous(), bias=lin.bias)
     return y.reshape(*lead, -1)
 
 

@@ -1009,13 +1009,16 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
     return (y, ymax) if want_rowmax else y
 
 
-def tensor_linear_wgrad(inds, dy, x, dy_bound=None, x_bound=None):
+def tensor_linear_wgrad(inds, dy, x, dy_bound=None, x_bound=None, want_bias=False):
     """dW[o, i] = sum over rows and components of dy[.., o, :] x[.., i, :].  Plain rows (inds = 0) of the sizes
     mg_tensor_linear_wgrad_f16x2 takes go through it while the linear mode is the split-fp16 one; dy_bound / x_bound
     (float tensors of any shape whose largest magnitude bounds |dy| / |x|, e.g. row maxima that the caller already
-    holds) save it a pass over the operand."""
+    holds) save it a pass over the operand.  want_bias (inds = 0): returns (dW, db) with db[o] = sum over rows of
+    dy[.., o], from the same pass where the kernel offers it."""
     _check_input(dy, "dy")
     _check_input(x, "x")
+    if want_bias and inds != 0:
+        raise RuntimeError("the bias gradient is defined for plain rows only")
     batch_dims = x.dim() - (1 + inds)
     dim_in, dim_out = int(x.size(batch_dims)), int(dy.size(batch_dims))
     rows = 1
@@ -1023,6 +1026,7 @@ def tensor_linear_wgrad(inds, dy, x, dy_bound=None, x_bound=None):
         rows *= int(x.size(i))
     with torch.cuda.device(x.device):
         dW = torch.empty(dim_out, dim_in, dtype=torch.float32, device=x.device)
+        db = None
         nbytes = ctypes.c_size_t(0)
         L.check(_lib.mg_tensor_linear_wgrad_workspace_bytes(rows, dim_in, dim_out, ctypes.byref(nbytes)))
         ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
@@ -1031,12 +1035,17 @@ def tensor_linear_wgrad(inds, dy, x, dy_bound=None, x_bound=None):
             for b, name in ((dy_bound, "dy_bound"), (x_bound, "x_bound")):
                 if b is not None:
                     _check_input(b, name)
+            if want_bias:
+                db = torch.empty(dim_out, dtype=torch.float32, device=x.device)
             L.check(_lib.mg_tensor_linear_wgrad_f16x2(
                 _p(dy), _p(x), _p(dy_bound), 0 if dy_bound is None else dy_bound.numel(),
-                _p(x_bound), 0 if x_bound is None else x_bound.numel(), rows, dim_in, dim_out, _p(ws), _p(dW), _stream()))
+                _p(x_bound), 0 if x_bound is None else x_bound.numel(), rows, dim_in, dim_out, _p(ws), _p(dW), _p(db),
+                _stream()))
         else:
             L.check(_lib.mg_tensor_linear_wgrad(inds, _p(dy), _p(x), rows, dim_in, dim_out, _p(ws), _p(dW), _stream()))
-    return dW
+            if want_bias:
+                db = dy.reshape(-1, dim_out).sum(0)
+    return (dW, db) if want_bias else dW
 
 
 # ------------------------------------------------- bf16-storage configuration

@@ -24,56 +24,73 @@ class _TensorLinearFn(torch.autograd.Function):
     itself made of differentiable functions (this one and _WeightGradFn), so the operation can be differentiated any
     number of times, as torch.autograd.functional.jvp(create_graph=True) of the meanflow loss needs
     (archs/meanflow_painn8.py:274-282); the reference's C++ backward calls raw kernels and cannot.
-    x_bound: row maxima of |x| when the caller already holds them (a scaling hint, not differentiated)."""
+    x_bound: row maxima of |x| when the caller already holds them (a scaling hint, not differentiated).
+    bias (plain rows only): added in the kernel's epilogue; its gradient comes out of the weight-gradient pass."""
 
     @staticmethod
-    def forward(ctx, inds, W, x, x_bound=None):
+    def forward(ctx, inds, W, x, x_bound=None, bias=None):
         ctx.inds = inds
         x = x.contiguous()
         if x_bound is None:
             x_bound = _row_bound(inds, x)
         ctx.x_bound = x_bound
+        ctx.has_bias = bias is not None
         ctx.save_for_backward(W, x)
-        return ops.tensor_linear_fwd(inds, W, x, row_bound=x_bound)
+        return ops.tensor_linear_fwd(inds, W, x, bias=None if bias is None else bias.contiguous(), row_bound=x_bound)
 
     @staticmethod
     def backward(ctx, dy):
         W, x = ctx.saved_tensors
         dy = dy.contiguous()
-        dW = dx = None
+        dW = dx = db = None
         dy_bound = _row_bound(ctx.inds, dy)
-        if ctx.needs_input_grad[1]:
-            dW = _WeightGradFn.apply(ctx.inds, dy, x, dy_bound, ctx.x_bound)
+        want_bias = ctx.has_bias and ctx.needs_input_grad[4]
+        if ctx.needs_input_grad[1] or want_bias:
+            dW, db = _WeightGradFn.apply(ctx.inds, dy, x, dy_bound, ctx.x_bound, want_bias)
+            if not want_bias:
+                db = None
         if ctx.needs_input_grad[2]:
             dx = _TensorLinearFn.apply(ctx.inds, W.t(), dy, dy_bound)   # strides of W are honoured: no copy
-        return None, dW, dx, None
+        return None, dW, dx, None, db
 
 
 class _WeightGradFn(torch.autograd.Function):
-    """dW[o, i] = sum over rows and components of dy[.., o, :] x[.., i, :]: bilinear in (dy, x), and its own
-    gradients are two tensor_linear calls."""
+    """dW[o, i] = sum over rows and components of dy[.., o, :] x[.., i, :], and with want_bias db[o] = sum over rows of
+    dy[.., o] (else an empty tensor): bilinear / linear in (dy, x), and their own gradients are two tensor_linear
+    calls."""
 
     @staticmethod
-    def forward(ctx, inds, dy, x, dy_bound=None, x_bound=None):
+    def forward(ctx, inds, dy, x, dy_bound=None, x_bound=None, want_bias=False):
         ctx.inds = inds
         ctx.bounds = (dy_bound, x_bound)
+        ctx.want_bias = want_bias
         ctx.save_for_backward(dy, x)
-        return ops.tensor_linear_wgrad(inds, dy.contiguous(), x.contiguous(), dy_bound=dy_bound, x_bound=x_bound)
+        out = ops.tensor_linear_wgrad(inds, dy.contiguous(), x.contiguous(), dy_bound=dy_bound, x_bound=x_bound,
+                                      want_bias=want_bias)
+        if want_bias:
+            return out
+        db = dy.new_empty(0)
+        ctx.mark_non_differentiable(db)
+        return out, db
 
     @staticmethod
-    def backward(ctx, ddW):
+    def backward(ctx, ddW, ddb):
         dy, x = ctx.saved_tensors
         dy_bound, x_bound = ctx.bounds
         g_dy = g_x = None
         if ctx.needs_input_grad[1]:
-            g_dy = _TensorLinearFn.apply(ctx.inds, ddW, x, x_bound)            # (.., o, :) = ddW x
+            # (.., o, :) = ddW x (+ ddb)
+            g_dy = _TensorLinearFn.apply(ctx.inds, ddW, x, x_bound, ddb if ctx.want_bias else None)
         if ctx.needs_input_grad[2]:
             g_x = _TensorLinearFn.apply(ctx.inds, ddW.t(), dy, dy_bound)       # (.., i, :) = ddW^T dy
-        return None, g_dy, g_x, None, None
+        return None, g_dy, g_x, None, None, None
 
 
-def tensor_linear(inds, W, x):
-    return _TensorLinearFn.apply(inds, W, x)
+def tensor_linear(inds, W, x, bias=None):
+    """bias (inds = 0 only): y = x W^T + bias in one kernel."""
+    if bias is not None and inds != 0:
+        raise RuntimeError("a bias is defined for plain rows only")
+    return _TensorLinearFn.apply(inds, W, x, None, bias)
 
 
 class TensLinear(nn.Module):

@@ -383,7 +383,7 @@ def test_weight_gradient_against_float64(ops, inds, rows, dim_in, dim_out):
 
 
 @pytest.mark.parametrize("rows,dim_in,dim_out", [(4096, 64, 64), (5000, 68, 132), (40001, 512, 512), (33333, 128, 512),
-                                                 (9000, 260, 64)])
+                                                 (9000, 260, 64), (20011, 16, 512), (4100, 4, 8)])
 @pytest.mark.parametrize("bounds", ["scanned", "row maxima", "loose"])
 def test_weight_gradient_split_fp16(ops, rows, dim_in, dim_out, bounds):
     """Plain rows on the fp16 matrix cores with hi + lo operands: tiles with ragged edges, row slices that do not
@@ -399,7 +399,10 @@ def test_weight_gradient_split_fp16(ops, rows, dim_in, dim_out, bounds):
         kw = dict(dy_bound=ops.row_absmax(dy), x_bound=ops.row_absmax(x))
     elif bounds == "loose":
         kw = dict(dy_bound=dy.abs().max().reshape(1) * 1000.0, x_bound=x.abs().max().reshape(1) * 1000.0)
-    got = ops.tensor_linear_wgrad(0, dy, x, **kw)
+    got, got_b = ops.tensor_linear_wgrad(0, dy, x, want_bias=True, **kw)
+    want_b = dy.double().sum(0)
+    err_b, ref_b = float((got_b.double() - want_b).abs().max()), float((dy.sum(0).double() - want_b).abs().max())
+    assert err_b <= 1e-6 + 1e-5 * float(want_b.abs().max()) + 2 * ref_b, (err_b, ref_b)
     want = dy.double().t() @ x.double()
     fp32 = (dy.t() @ x).double()
     scale = float(want.abs().max())
