@@ -48,7 +48,7 @@ def parse():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="painn_layer",
                     choices=["painn_layer", "neighbour", "products", "denoiser", "stress", "polymer", "meanflow_painn",
-                             "gemm_power", "painn_train", "denoiser_train"])
+                             "gemm_power", "painn_train", "denoiser_train", "meanflow_train"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the cpu_baseline leg")
     ap.add_argument("--no-extras", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-comparisons", action="store_true",
@@ -786,6 +786,59 @@ def bench_meanflow_painn(torch, args):
                                    "lattice, box 80 A, cutoff 5 A, radius graphs rebuilt in the forward", "atoms": N}}
 
 
+def bench_meanflow_train(torch, args):
+    """The reference's training step for the PaiNN meanflow denoiser (archs/meanflow_painn8.py:274-296): the
+    Jacobian-vector product of the model along (v, 1) with create_graph=True, the target v - (t - s) jvp, a second
+    evaluation of the model, the squared error, and its gradient for every parameter: three nested differentiations
+    through the library's autograd functions.  4 systems of 1024 atoms (jittered lattice, cutoff 5 A), n = 128, 1 + 2
+    blocks, positions that move."""
+    mf = importlib.import_module("learned-dynamics_amd.meanflow_painn")
+    n, r0, box_len, B, N = 128, 5.0, 32.0, 4, 1024
+    box = (box_len,) * 3
+    seed = 0x947 + 11
+    torch.manual_seed(seed)
+    g = torch.Generator().manual_seed(seed + 1)
+    side = 11                                                      # 11^3 >= 1024 lattice sites, 2.9 A apart
+    k = torch.arange(N)
+    sites = torch.stack([k % side, (k // side) % side, k // (side * side)], dim=1).float() * (box_len / side)
+    x_prev = (sites[None] + 0.4 * torch.randn(B, N, 3, generator=g)).contiguous().cuda()
+    z_0 = (x_prev.cpu() + 0.2 * torch.randn(B, N, 3, generator=g)).cuda()
+    z_1 = (x_prev.cpu() + 0.5 * torch.randn(B, N, 3, generator=g)).cuda()
+    one_hot = torch.nn.functional.one_hot(torch.randint(0, 20, (N,), generator=g), 20).float()
+    idx = torch.arange(N - 1)
+    topo = mf.Topology(one_hot.cuda(), torch.cat([idx, idx + 1]).cuda(), torch.cat([idx + 1, idx]).cuda())
+    model = mf.SE3ITO(r0, n, N, blks_0=1, blks_1=2, mutate_pos=True).cuda().train()
+    with torch.no_grad():
+        for name, p in model.named_parameters():
+            if name.endswith("lin_push_pos.W"):
+                p.mul_(0.05)
+    params = [p for p in model.parameters() if p.requires_grad]
+    t, s_ = torch.rand(B, generator=g).cuda(), torch.zeros(B).cuda()
+
+    def step():
+        z_t = t[:, None, None] * z_1 + (1 - t[:, None, None]) * z_0
+        v = z_1 - z_0
+        f = lambda zz, tt: model((s_, tt), x_prev, zz, box, topo)
+        _, jvp = torch.autograd.functional.jvp(f, (z_t, t), (v, torch.ones_like(t)), create_graph=True)
+        v_target = v - (t - s_)[:, None, None] * jvp
+        v_pred = model((s_, t), x_prev, z_t, box, topo)
+        loss = ((v_pred - v_target) ** 2).mean()
+        return loss, torch.autograd.grad(loss, params, allow_unused=True)
+
+    loss, grads = step()
+    finite = all(bool(torch.isfinite(gr).all()) for gr in grads if gr is not None)
+    sec = timed_steps(torch, step, args.steps, args.warmup)
+    with torch.no_grad():
+        t_fwd = event_time(torch, lambda: model((s_, t), x_prev, z_1, box, topo), 5)
+    return {"metric": "PaiNN meanflow training step (jvp + loss gradient) atoms/sec", "unit": "atoms/s",
+            "value": B * N / sec, "ms_per_step": sec * 1e3, "dtype": "f32",
+            "config": {"workload": "SE3ITO, 1 + 2 blocks with bond messages, n = 128, positions that move; 4 systems x 1024 "
+                                   "atoms, box 32 A, cutoff 5 A; torch.autograd.functional.jvp(create_graph=True) + backward"},
+            "detail": {"loss": float(loss.detach()), "gradients_finite": finite,
+                       "parameters_with_gradient": sum(gr is not None for gr in grads), "parameters": len(params),
+                       "inference_forward_ms_same_inputs": t_fwd * 1e3}}
+
+
 def bench_stress(torch, args, with_cpu=True):
     """BASELINE configs[4]: 65536 atoms uniform in a periodic cube at 0.1 atoms/A^3, cutoff 6 A,
     4 x [Messages + SelfTensProds] with 128 channels per rank, features stored as bf16 with fp32
@@ -995,6 +1048,8 @@ def main():
         res = bench_painn_train(torch, args)
     elif args.workload == "denoiser_train":
         res = bench_denoiser_train(torch, args)
+    elif args.workload == "meanflow_train":
+        res = bench_meanflow_train(torch, args)
     else:
         res = bench_products(torch, args)
         res.setdefault("ms_per_step", res["detail"]["rows_4096"]["us"] * 1e-3)

@@ -317,8 +317,8 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 
     // the two scales, from the partial maxima
     float ma = 0.f, mb = 0.f;
-    for (int k = threadIdx.x; k < n_dy_parts; k += 256) ma = fmaxf(ma, dy_parts[k]);
-    for (int k = threadIdx.x; k < n_x_parts; k += 256) mb = fmaxf(mb, x_parts[k]);
+    for (int k = threadIdx.x; k < n_dy_parts; k += 256) ma = fmaxf(ma, fabsf(dy_parts[k]));
+    for (int k = threadIdx.x; k < n_x_parts; k += 256) mb = fmaxf(mb, fabsf(x_parts[k]));
     for (int d = 1; d < 64; d <<= 1) { ma = fmaxf(ma, __shfl_xor(ma, d)); mb = fmaxf(mb, __shfl_xor(mb, d)); }
     float* wave_max = reinterpret_cast<float*>(lds);
     if (lane == 0) { wave_max[wave] = ma; wave_max[4 + wave] = mb; }
@@ -475,6 +475,21 @@ __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restri
     }
 }
 
+// the same for two sets of planes in one launch (the weight gradient and the column sums)
+__global__ void __launch_bounds__(256) wgrad_reduce2_kernel(const float* __restrict__ part_a, long n_a,
+                                                            float* __restrict__ out_a,
+                                                            const float* __restrict__ part_b, long n_b,
+                                                            float* __restrict__ out_b, int splits) {
+    for (long k = (long)blockIdx.x * blockDim.x + threadIdx.x; k < n_a + n_b; k += (long)gridDim.x * blockDim.x) {
+        const bool first = k < n_a;
+        const float* src = first ? part_a + k : part_b + (k - n_a);
+        const long stride = first ? n_a : n_b;
+        float s = 0.f;
+        for (int z = 0; z < splits; z++) s += src[(long)z * stride];
+        if (first) out_a[k] = s; else out_b[k - n_a] = s;
+    }
+}
+
 // rows per slice and number of slices for a problem (the same on the sizing and the launching side)
 void wgrad_split(long rows, int dim_in, int dim_out, int tile, long* rows_per_block, long* splits) {
     const int gx = (int)ceil_div(dim_out, tile), gy = (int)ceil_div(dim_in, tile);
@@ -530,8 +545,10 @@ int mg_tensor_linear_wgrad_f16x2(const float* dy, const float* x, const float* d
     float* part = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(workspace) + 15) & ~uintptr_t(15));
     float* maxima = part + splits * n;                       // [dy: kFParts][x: kFParts]
     float* colsum_part = db ? maxima + 2 * kFParts : nullptr; // [slice][dim_out]
+    constexpr long kDirectBounds = 16384;                    // a bound array this short is read by every workgroup itself
     auto bound_parts = [&](const float* data, long count, const float* bound, long n_bound, float* parts) -> int {
         // partial maxima of the caller's bounds, or of the data itself
+        if (bound && n_bound <= kDirectBounds) return (int)n_bound;
         const float* from = bound ? bound : data;
         const long len = bound ? n_bound : count;
         const int blocks = (int)(ceil_div(len, 4096) < kFParts ? ceil_div(len, 4096) : kFParts);
@@ -543,14 +560,15 @@ int mg_tensor_linear_wgrad_f16x2(const float* dy, const float* x, const float* d
     };
     const int na = bound_parts(dy, rows * dim_out, dy_bound, n_dy_bound, maxima);
     const int nb = bound_parts(x, rows * dim_in, x_bound, n_x_bound, maxima + kFParts);
+    const float* dy_parts = (dy_bound && n_dy_bound <= kDirectBounds) ? dy_bound : maxima;
+    const float* x_parts = (x_bound && n_x_bound <= kDirectBounds) ? x_bound : maxima + kFParts;
     dim3 grid((unsigned)ceil_div(dim_out, kFTile), (unsigned)ceil_div(dim_in, kFTile), (unsigned)splits), block(256);
-    hipLaunchKernelGGL(wgrad_f16x2_kernel, grid, block, 0, st, dy, x, (const float*)maxima, na,
-                       (const float*)(maxima + kFParts), nb, rows, dim_in, dim_out, rpb, part, colsum_part);
-    const unsigned nblocks = (unsigned)(ceil_div(n, 256) < 1024 ? ceil_div(n, 256) : 1024);
-    hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(nblocks), dim3(256), 0, st, (const float*)part, n, (int)splits, dW);
-    if (db)
-        hipLaunchKernelGGL(wgrad_reduce_kernel, dim3((unsigned)ceil_div(dim_out, 256)), dim3(256), 0, st,
-                           (const float*)colsum_part, (long)dim_out, (int)splits, db);
+    hipLaunchKernelGGL(wgrad_f16x2_kernel, grid, block, 0, st, dy, x, dy_parts, na, x_parts, nb, rows, dim_in, dim_out,
+                       rpb, part, colsum_part);
+    const long n_sum = n + (db ? dim_out : 0);
+    const unsigned nblocks = (unsigned)(ceil_div(n_sum, 256) < 1024 ? ceil_div(n_sum, 256) : 1024);
+    hipLaunchKernelGGL(wgrad_reduce2_kernel, dim3(nblocks), dim3(256), 0, st, (const float*)part, n, dW,
+                       (const float*)colsum_part, (long)(db ? dim_out : 0), db, (int)splits);
     return check_launch("mg_tensor_linear_wgrad_f16x2");
 }
 
