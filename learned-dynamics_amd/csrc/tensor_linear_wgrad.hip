@@ -470,7 +470,15 @@ __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float* __restri
                                                            float* __restrict__ dW) {
     for (long k = (long)blockIdx.x * blockDim.x + threadIdx.x; k < n; k += (long)gridDim.x * blockDim.x) {
         float s = 0.f;
-        for (int z = 0; z < splits; z++) s += part[(long)z * n + k];
+        int z = 0;
+        for (; z + 8 <= splits; z += 8) {                  // eight loads in flight, added in slice order
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = part[(long)(z + u) * n + k];
+#pragma unroll
+            for (int u = 0; u < 8; u++) s += v[u];
+        }
+        for (; z < splits; z++) s += part[(long)z * n + k];
         dW[k] = s;
     }
 }
@@ -485,7 +493,15 @@ __global__ void __launch_bounds__(256) wgrad_reduce2_kernel(const float* __restr
         const float* src = first ? part_a + k : part_b + (k - n_a);
         const long stride = first ? n_a : n_b;
         float s = 0.f;
-        for (int z = 0; z < splits; z++) s += src[(long)z * stride];
+        int z = 0;
+        for (; z + 8 <= splits; z += 8) {                  // eight loads in flight, added in slice order
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = src[(long)(z + u) * stride];
+#pragma unroll
+            for (int u = 0; u < 8; u++) s += v[u];
+        }
+        for (; z < splits; z++) s += src[(long)z * stride];
         if (first) out_a[k] = s; else out_b[k - n_a] = s;
     }
 }
