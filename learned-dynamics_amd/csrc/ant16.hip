@@ -342,7 +342,15 @@ __global__ void __launch_bounds__(256) planes_sum_kernel(const float* __restrict
                                                          float* __restrict__ out) {
     for (long k = (long)blockIdx.x * blockDim.x + threadIdx.x; k < n; k += (long)gridDim.x * blockDim.x) {
         float s = 0.f;
-        for (int z = 0; z < splits; z++) s += part[(long)z * n + k];
+        int z = 0;
+        for (; z + 8 <= splits; z += 8) {                  // eight loads in flight, added in slice order
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = part[(long)(z + u) * n + k];
+#pragma unroll
+            for (int u = 0; u < 8; u++) s += v[u];
+        }
+        for (; z < splits; z++) s += part[(long)z * n + k];
         out[k] = s;
     }
 }

@@ -315,20 +315,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     const long r_lo = (long)blockIdx.z * rows_per_block;
     const long r_hi = r_lo + rows_per_block < R ? r_lo + rows_per_block : R;
 
-    // the two scales, from the partial maxima
-    float ma = 0.f, mb = 0.f;
-    for (int k = threadIdx.x; k < n_dy_parts; k += 256) ma = fmaxf(ma, fabsf(dy_parts[k]));
-    for (int k = threadIdx.x; k < n_x_parts; k += 256) mb = fmaxf(mb, fabsf(x_parts[k]));
-    for (int d = 1; d < 64; d <<= 1) { ma = fmaxf(ma, __shfl_xor(ma, d)); mb = fmaxf(mb, __shfl_xor(mb, d)); }
-    float* wave_max = reinterpret_cast<float*>(lds);
-    if (lane == 0) { wave_max[wave] = ma; wave_max[4 + wave] = mb; }
-    __syncthreads();
-    ma = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
-    mb = fmaxf(fmaxf(wave_max[4], wave_max[5]), fmaxf(wave_max[6], wave_max[7]));
-    __syncthreads();
-    float inv_a, inv_b;
-    const float scale_a = pow2_scale(ma, &inv_a), scale_b = pow2_scale(mb, &inv_b);
-
+    float scale = 0.f, unscale = 0.f;                      // (set by set_scales below)
     // staging role of this thread: operand (wave-uniform), 8 rows from row 8 * octet, columns 4 cq .. 4 cq + 3.
     // A stage is the 32 rows from `first`; the last stage of a slice starts at r_hi - 32, inside the matrix
     // (rows >= 32), and the rows it shares with the stage before, or with the slice before, are scaled by zero, as
@@ -340,7 +327,6 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     const bool col_ok = tile0 + 4 * cq < dim;
     const float* operand = stage_x ? x : dy;                                       // (uniform)
     const unsigned lane_off = (unsigned)(8 * octet * dim + (col_ok ? tile0 + 4 * cq : 0));
-    const float scale = col_ok ? (stage_x ? scale_b : scale_a) : 0.f;
     // LDS rows cq + 32 j: their swizzle term ((row >> 2) & 3) does not depend on j
     unsigned char* st_dst = lds + (stage_x ? 2 * kFPlane : 0) + cq * kFRowW + 16 * (octet ^ ((cq >> 2) & 3));
     float4 v[8];
@@ -374,6 +360,24 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
             *reinterpret_cast<halfx8*>(st_dst + buf_off + 32 * j * kFRowW) = hi[j];
             *reinterpret_cast<halfx8*>(st_dst + buf_off + kFPlane + 32 * j * kFRowW) = lo[j];
         }
+    };
+
+    // the two scales, from the partial maxima
+    auto set_scales = [&]() {
+    float ma = 0.f, mb = 0.f;
+    for (int k = threadIdx.x; k < n_dy_parts; k += 256) ma = fmaxf(ma, fabsf(dy_parts[k]));
+    for (int k = threadIdx.x; k < n_x_parts; k += 256) mb = fmaxf(mb, fabsf(x_parts[k]));
+    for (int d = 1; d < 64; d <<= 1) { ma = fmaxf(ma, __shfl_xor(ma, d)); mb = fmaxf(mb, __shfl_xor(mb, d)); }
+    float* wave_max = reinterpret_cast<float*>(lds);
+    if (lane == 0) { wave_max[wave] = ma; wave_max[4 + wave] = mb; }
+    __syncthreads();
+    ma = fmaxf(fmaxf(wave_max[0], wave_max[1]), fmaxf(wave_max[2], wave_max[3]));
+    mb = fmaxf(fmaxf(wave_max[4], wave_max[5]), fmaxf(wave_max[6], wave_max[7]));
+    __syncthreads();
+    float inv_a, inv_b;
+    const float scale_a = pow2_scale(ma, &inv_a), scale_b = pow2_scale(mb, &inv_b);
+    scale = col_ok ? (stage_x ? scale_b : scale_a) : 0.f;
+    unscale = inv_a * inv_b;
     };
 
     floatx16 acc[2][2];
@@ -418,6 +422,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     // (stages past the slice are fetched and stored like the others, scaled by zero and never multiplied: the loop
     // body has no branch, and the splitting of one stage can be issued between the matrix instructions of another)
     fetch(r_lo);
+    set_scales();                                          // (the first stage is on its way meanwhile)
     store(r_lo, 0);
     fetch(r_lo + kFRows);
     __syncthreads();
@@ -450,7 +455,6 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     }
     // D[row][col]: col = lane % 32, row = 8 (k / 4) + 4 (lane / 32) + k % 4 for register k; LDS row 32 j + c / 4 of
     // an operand is column 4 (c / 4) + j of the tile
-    const float unscale = inv_a * inv_b;
     float* plane = part + (long)blockIdx.z * O * I;
 #pragma unroll
     for (int p = 0; p < 2; p++)
@@ -507,15 +511,16 @@ __global__ void __launch_bounds__(256) wgrad_reduce2_kernel(const float* __restr
 }
 
 // rows per slice and number of slices for a problem (the same on the sizing and the launching side)
-void wgrad_split(long rows, int dim_in, int dim_out, int tile, long* rows_per_block, long* splits) {
+void wgrad_split(long rows, int dim_in, int dim_out, int tile, long* rows_per_block, long* splits,
+                 long min_rows_per_slice = 64) {
     const int gx = (int)ceil_div(dim_out, tile), gy = (int)ceil_div(dim_in, tile);
     long s = ceil_div(1024, (long)gx * gy);             // aim at ~4 workgroups per CU
-    const long max_splits = ceil_div(rows, 64);
+    const long max_splits = ceil_div(rows, min_rows_per_slice);
     if (s > max_splits) s = max_splits;
     if (s < 1) s = 1;
     if (s > 65535) s = 65535;
     long rpb = ceil_div(rows, s);
-    rpb = ceil_div(rpb, kSRows) * kSRows;              // (a multiple of every kernel's rows per trip)
+    rpb = ceil_div(rpb, 32) * 32;                      // (a multiple of every kernel's rows per trip)
     *rows_per_block = rpb;
     *splits = rows > 0 ? ceil_div(rows, rpb) : 0;
 }
@@ -557,7 +562,8 @@ int mg_tensor_linear_wgrad_f16x2(const float* dy, const float* x, const float* d
     hipStream_t st = (hipStream_t)stream;
     const long n = (long)dim_in * dim_out;
     long rpb, splits;
-    wgrad_split(rows, dim_in, dim_out, kFTile, &rpb, &splits);
+    // (slices of at least 512 rows: with few rows, writing and adding the planes costs more than the products)
+    wgrad_split(rows, dim_in, dim_out, kFTile, &rpb, &splits, 512);
     float* part = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(workspace) + 15) & ~uintptr_t(15));
     float* maxima = part + splits * n;                       // [dy: kFParts][x: kFParts]
     float* colsum_part = db ? maxima + 2 * kFParts : nullptr; // [slice][dim_out]
