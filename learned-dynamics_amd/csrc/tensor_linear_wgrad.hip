@@ -511,11 +511,13 @@ __global__ void __launch_bounds__(256) wgrad_reduce2_kernel(const float* __restr
 }
 
 // rows per slice and number of slices for a problem (the same on the sizing and the launching side)
+// resident_groups = 0: aim at ~4 workgroups per CU; otherwise the number of workgroups the chip holds at once, which
+// the grid then does not exceed (a second, partly filled round would cost a whole slice's time)
 void wgrad_split(long rows, int dim_in, int dim_out, int tile, long* rows_per_block, long* splits,
-                 long min_rows_per_slice = 64) {
+                 long resident_groups = 0) {
     const int gx = (int)ceil_div(dim_out, tile), gy = (int)ceil_div(dim_in, tile);
-    long s = ceil_div(1024, (long)gx * gy);             // aim at ~4 workgroups per CU
-    const long max_splits = ceil_div(rows, min_rows_per_slice);
+    long s = resident_groups > 0 ? resident_groups / ((long)gx * gy) : ceil_div(1024, (long)gx * gy);
+    const long max_splits = ceil_div(rows, 64);
     if (s > max_splits) s = max_splits;
     if (s < 1) s = 1;
     if (s > 65535) s = 65535;
@@ -562,8 +564,7 @@ int mg_tensor_linear_wgrad_f16x2(const float* dy, const float* x, const float* d
     hipStream_t st = (hipStream_t)stream;
     const long n = (long)dim_in * dim_out;
     long rpb, splits;
-    // (slices of at least 512 rows: with few rows, writing and adding the planes costs more than the products)
-    wgrad_split(rows, dim_in, dim_out, kFTile, &rpb, &splits, 512);
+    wgrad_split(rows, dim_in, dim_out, kFTile, &rpb, &splits, 512);      // two workgroups per CU fit
     float* part = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(workspace) + 15) & ~uintptr_t(15));
     float* maxima = part + splits * n;                       // [dy: kFParts][x: kFParts]
     float* colsum_part = db ? maxima + 2 * kFParts : nullptr; // [slice][dim_out]
