@@ -1041,6 +1041,29 @@ def tensor_linear_wgrad(inds, dy, x, dy_bound=None, x_bound=None, want_bias=Fals
                 _p(dy), _p(x), _p(dy_bound), 0 if dy_bound is None else dy_bound.numel(),
                 _p(x_bound), 0 if x_bound is None else x_bound.numel(), rows, dim_in, dim_out, _p(ws), _p(dW), _p(db),
                 _stream()))
+        elif (inds > 0 and get_linear_mode() == LINEAR_F16X2 and rows * 3 ** inds >= 4096
+              and max(dim_in, dim_out) <= 256):
+            # (row, chan, comp) -> one plain row per (row, comp), channels zero-padded to a power of two: the sum over
+            # rows and components is then the plain-row weight gradient, on the matrix cores; the transposition
+            # also yields the row maxima the kernel scales by
+            T = 3 ** inds
+
+            def as_rows(t, dim):
+                pad = max(32, 1 << (dim - 1).bit_length())
+                out = torch.empty(rows * T, pad, dtype=torch.float32, device=t.device)
+                bound = torch.empty(rows * T, 1, dtype=torch.float32, device=t.device)
+                L.check(_lib.mg_components_to_rows(_p(t), rows, dim, T, pad, _p(out), _p(bound), _stream()))
+                return out, bound, pad
+            dy2, dy2_bound, o_pad = as_rows(dy, dim_out)
+            x2, x2_bound, i_pad = as_rows(x, dim_in)
+            L.check(_lib.mg_tensor_linear_wgrad_workspace_bytes(rows * T, i_pad, o_pad, ctypes.byref(nbytes)))
+            ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
+            dW_pad = dW if (o_pad, i_pad) == (dim_out, dim_in) else torch.empty(o_pad, i_pad, dtype=torch.float32,
+                                                                                device=x.device)
+            L.check(_lib.mg_tensor_linear_wgrad_f16x2(_p(dy2), _p(x2), _p(dy2_bound), rows * T, _p(x2_bound), rows * T,
+                                                      rows * T, i_pad, o_pad, _p(ws), _p(dW_pad), None, _stream()))
+            if dW_pad is not dW:
+                dW = dW_pad[:dim_out, :dim_in].contiguous()
         else:
             L.check(_lib.mg_tensor_linear_wgrad(inds, _p(dy), _p(x), rows, dim_in, dim_out, _p(ws), _p(dW), _stream()))
             if want_bias:

@@ -364,11 +364,15 @@ def test_linear_f16x2_in_row_dynamic_range_meeting_zero_weights(ops, span):
 
 
 @pytest.mark.parametrize("inds,rows,dim_in,dim_out", [(0, 5000, 117, 210), (0, 70, 16, 512), (0, 1, 33, 31),
-                                                      (0, 100003, 512, 384), (1, 3000, 48, 70), (2, 900, 20, 130)])
+                                                      (0, 100003, 512, 384), (1, 3000, 48, 70), (2, 900, 20, 130),
+                                                      (1, 300, 48, 70), (2, 100, 20, 130), (1, 8192, 64, 256),
+                                                      (2, 4001, 16, 16), (1, 2000, 300, 64)])
 def test_weight_gradient_against_float64(ops, inds, rows, dim_in, dim_out):
-    """dW[o, i] = sum over rows and components of dy[r, o, t] x[r, i, t]: plain rows through the fp32 matrix cores
-    (tiles of 128 x 128 with ragged edges, row slices that do not divide the rows), tensor components through the
-    vector kernel; slices are summed in a fixed order, so two runs agree bit for bit."""
+    """dW[o, i] = sum over rows and components of dy[r, o, t] x[r, i, t]: plain rows through the matrix cores (fp32
+    ones where a dimension is not a multiple of 4 or the rows are few, else split fp16; tiles of 128 x 128 with ragged
+    edges, row slices that do not divide the rows), tensor components transposed to plain rows for the matrix cores
+    when there are at least 4096 of them and the channels fit 256, else through the vector kernel; slices are summed
+    in a fixed order, so two runs agree bit for bit."""
     g = torch.Generator().manual_seed(rows + dim_in)
     comps = (3,) * inds
     x = torch.randn(rows, dim_in, *comps, generator=g).cuda()
