@@ -5,9 +5,11 @@
 // for one 64x64 tile of dW in registers and writes it to its own plane of a
 // workspace; a second kernel adds the planes in slice order.  No atomics: the
 // result does not depend on the order in which workgroups finish.
-// Plain rows (no tensor components) go through the fp32 matrix cores: v_mfma_f32_32x32x2_f32 takes dy and x exactly
-// as they lie in memory (for the reduction index r, lanes 0..31 supply 32 consecutive columns of row r and lanes
-// 32..63 those of row r + 1), products and sums are fp32, nothing is rounded to a shorter format.
+// Plain rows (no tensor components) go through the matrix cores.  mg_tensor_linear_wgrad uses the fp32 ones:
+// v_mfma_f32_32x32x2_f32 takes dy and x exactly as they lie in memory (for the reduction index r, lanes 0..31 supply
+// 32 consecutive columns of row r and lanes 32..63 those of row r + 1), products and sums are fp32, nothing is
+// rounded to a shorter format.  mg_tensor_linear_wgrad_f16x2 uses the fp16 ones with two-piece operands (three times
+// the rate at an error of a few fp32 ulps of sum |dy| |x|) and also sums the columns of dy, the bias gradient.
 // Training-side helper: not on the inference hot path.
 #include "common.hpp"
 #include "f16x2.hpp"
