@@ -421,13 +421,23 @@ int mg_tensor_linear_layout(int inds, const float* W, long w_stride_o, long w_st
         return launch_cfg<1, 2, 2, 2, 2>(W, so, si, x, R, dim_in, dim_out, b, act, accumulate, y, st, false, out_T);
     }
     const bool soa = y_layout == 1;
+    // column tile of 128, 64 or 32: the widest one that still gives the chip two workgroups per CU (a node-sized problem
+    // on 128-column tiles runs on a quarter of the CUs and takes twice as long)
+    auto tile_cols = [&](int rows_per_group) {
+        const long row_groups = ceil_div(rows, rows_per_group);
+        int cols = dim_out <= 32 ? 32 : (dim_out <= 64 ? 64 : 128);
+        while (cols > 32 && row_groups * ceil_div(dim_out, cols) < 512) cols >>= 1;
+        return cols;
+    };
     if (inds == 1) {
-        if (dim_out <= 32) return launch_cfg<3, 2, 1, 3, 1>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
-        if (dim_out <= 64) return launch_cfg<3, 2, 2, 3, 1>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
+        const int cols = tile_cols(64);
+        if (cols == 32) return launch_cfg<3, 2, 1, 3, 1>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
+        if (cols == 64) return launch_cfg<3, 2, 2, 3, 1>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
         return launch_cfg<3, 2, 2, 3, 2>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
     }
-    if (dim_out <= 32) return launch_cfg<9, 3, 1, 3, 1>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
-    if (dim_out <= 64) return launch_cfg<9, 3, 1, 3, 2>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
+    const int cols = tile_cols(32);
+    if (cols == 32) return launch_cfg<9, 3, 1, 3, 1>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
+    if (cols == 64) return launch_cfg<9, 3, 1, 3, 2>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
     return launch_cfg<9, 3, 2, 3, 2>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, y, st, soa);
 }
 
