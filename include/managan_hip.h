@@ -156,6 +156,12 @@ int mg_segment_row_ptr(const void* index, int index_is_int64, long n_edges, int 
 /* out[r, :] = sum over e in [row_ptr[r], row_ptr[r+1]) of x_edge[e, :], in edge order. */
 int mg_segment_sum_csr(const float* x_edge /* (E,feat) */, const int* row_ptr, int n_rows, int feat,
                        float* out /* (n_rows,feat) */, mg_stream_t stream);
+/* The same for an index that is not sorted: perm (E ints) lists the rows of x_edge in the sorted order of the index
+ * (a stable sort), row_ptr is that of the sorted index, and out[r, :] = sum over e in [row_ptr[r], row_ptr[r+1]) of
+ * x_edge[perm[e], :]: the adjoint of a gather by an unsorted index (torch's index backward under
+ * managan/graph_layers.py:37-52), without a permuted copy of x_edge.  perm == NULL: mg_segment_sum_csr. */
+int mg_segment_sum_csr_perm(const float* x_edge /* (E,feat) */, const int* perm, const int* row_ptr, int n_rows,
+                            int feat, float* out /* (n_rows,feat) */, mg_stream_t stream);
 /* out[e, :] = x[index[e], :] */
 int mg_gather_rows(const float* x /* (n_rows,feat) */, const void* index, int index_is_int64,
                    long n_edges, int n_rows, int feat, float* out /* (E,feat) */, mg_stream_t stream);

@@ -39,6 +39,7 @@ _SIGNATURES = {
     "mg_edge_vectors": [vp, vp, vp, i64, f32, f32, f32, vp, vp, vp],
     "mg_segment_row_ptr": [vp, i32, i64, i32, vp, vp],
     "mg_segment_sum_csr": [vp, vp, i32, i32, vp, vp],
+    "mg_segment_sum_csr_perm": [vp, vp, vp, i32, i32, vp, vp],
     "mg_gather_rows": [vp, vp, i32, i64, i32, i32, vp, vp],
     "mg_bee_fwd": [vp, vp, vp, vp, vp, vp, i64, i32, ctypes.POINTER(PtrArray13), vp],
     "mg_bee_bwd": [i32, vp, vp, vp, ctypes.POINTER(PtrArray13), i64, i32, vp, vp, vp, vp],

@@ -65,8 +65,11 @@ struct Acc<1> {
     __device__ void store(float* p) const { *p = v; }
 };
 
-template <int VEC>
-__global__ void __launch_bounds__(256) segment_sum_kernel(const float* __restrict__ x, const int* __restrict__ row_ptr,
+// PERM: edge e of the CSR order is row perm[e] of x (an index that is not sorted, summed in its sorted order without
+// first copying the rows into that order)
+template <int VEC, bool PERM>
+__global__ void __launch_bounds__(256) segment_sum_kernel(const float* __restrict__ x, const int* __restrict__ perm,
+                                                          const int* __restrict__ row_ptr,
                                                           long n_rows, int feat, Chunks ch, float* __restrict__ out) {
     const int lane = threadIdx.x & (kWave - 1);
     const long wave_global = ((long)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
@@ -84,10 +87,11 @@ __global__ void __launch_bounds__(256) segment_sum_kernel(const float* __restric
         a1.zero();
         long e = lo + sub;
         for (; e + per_iter < hi; e += 2 * per_iter) {   // two independent loads in flight
-            a0.add(x + e * feat + col);
-            a1.add(x + (e + per_iter) * feat + col);
+            const long r0 = PERM ? perm[e] : e, r1 = PERM ? perm[e + per_iter] : e + per_iter;
+            a0.add(x + r0 * feat + col);
+            a1.add(x + r1 * feat + col);
         }
-        if (e < hi) a0.add(x + e * feat + col);
+        if (e < hi) a0.add(x + (PERM ? (long)perm[e] : e) * feat + col);
         a0.merge(a1);
         for (int d = L; d < kWave; d <<= 1) a0.fold(d);
         if (sub == 0) a0.store(out + row * feat + col);
@@ -193,6 +197,11 @@ int mg_segment_row_ptr(const void* index, int index_is_int64, long n_edges, int 
 
 int mg_segment_sum_csr(const float* x_edge, const int* row_ptr, int n_rows, int feat, float* out,
                        mg_stream_t stream) {
+    return mg_segment_sum_csr_perm(x_edge, nullptr, row_ptr, n_rows, feat, out, stream);
+}
+
+int mg_segment_sum_csr_perm(const float* x_edge, const int* perm, const int* row_ptr, int n_rows, int feat, float* out,
+                            mg_stream_t stream) {
     MG_REQUIRE(n_rows >= 0 && feat >= 0, "mg_segment_sum_csr: negative size");
     if (n_rows == 0 || feat == 0) return MG_OK;
     MG_REQUIRE(row_ptr && out, "mg_segment_sum_csr: null pointer");
@@ -204,12 +213,16 @@ int mg_segment_sum_csr(const float* x_edge, const int* row_ptr, int n_rows, int 
     const long items = (long)n_rows * ch.n;
     long blocks = ceil_div(items, 4);
     if (blocks > 256L * 64) blocks = 256L * 64;   // grid-stride beyond 64 workgroups per CU
-    if (vec)
-        hipLaunchKernelGGL(segment_sum_kernel<4>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, x_edge,
-                           row_ptr, (long)n_rows, feat, ch, out);
+    const dim3 grid((unsigned)blocks), block(256);
+    hipStream_t st = (hipStream_t)stream;
+    if (vec && perm)
+        hipLaunchKernelGGL((segment_sum_kernel<4, true>), grid, block, 0, st, x_edge, perm, row_ptr, (long)n_rows, feat, ch, out);
+    else if (vec)
+        hipLaunchKernelGGL((segment_sum_kernel<4, false>), grid, block, 0, st, x_edge, perm, row_ptr, (long)n_rows, feat, ch, out);
+    else if (perm)
+        hipLaunchKernelGGL((segment_sum_kernel<1, true>), grid, block, 0, st, x_edge, perm, row_ptr, (long)n_rows, feat, ch, out);
     else
-        hipLaunchKernelGGL(segment_sum_kernel<1>, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, x_edge,
-                           row_ptr, (long)n_rows, feat, ch, out);
+        hipLaunchKernelGGL((segment_sum_kernel<1, false>), grid, block, 0, st, x_edge, perm, row_ptr, (long)n_rows, feat, ch, out);
     return check_launch("mg_segment_sum_csr");
 }
 

@@ -118,10 +118,8 @@ class _ScatterSum(torch.autograd.Function):
     @staticmethod
     def forward(ctx, x_edge, sidx):
         ctx.sidx = sidx
-        x_edge = x_edge.contiguous()
-        if not sidx.is_sorted:
-            x_edge = ops.gather_rows(x_edge, sidx.perm)       # rows in index order
-        return ops.segment_sum_csr(x_edge, sidx.row_ptr, sidx.n_rows)
+        # (an unsorted index: the rows are read in its sorted order through the permutation)
+        return ops.segment_sum_csr(x_edge.contiguous(), sidx.row_ptr, sidx.n_rows, perm=sidx.perm)
 
     @staticmethod
     def backward(ctx, dy):

@@ -307,17 +307,22 @@ def segment_row_ptr(index, n_rows):
     return row_ptr
 
 
-def segment_sum_csr(x_edge, row_ptr, n_rows):
-    """out[r] = sum of x_edge[row_ptr[r]:row_ptr[r+1]]; trailing dims kept."""
+def segment_sum_csr(x_edge, row_ptr, n_rows, perm=None):
+    """out[r] = sum of x_edge[row_ptr[r]:row_ptr[r+1]]; trailing dims kept.  perm (int32, one entry per edge): the rows
+    are taken in the order x_edge[perm] without copying them into it."""
     _check_input(x_edge, "x_edge")
     _check_input(row_ptr, "row_ptr", torch.int32)
+    if perm is not None:
+        _check_input(perm, "perm", torch.int32)
+        if perm.numel() != x_edge.size(0):
+            raise RuntimeError("perm must have one entry per edge")
     rest = tuple(x_edge.shape[1:])
     feat = 1
     for d in rest:
         feat *= int(d)
     with torch.cuda.device(x_edge.device):
         out = torch.empty((n_rows,) + rest, dtype=torch.float32, device=x_edge.device)
-        L.check(_lib.mg_segment_sum_csr(_p(x_edge), _p(row_ptr), int(n_rows), feat, _p(out), _stream()))
+        L.check(_lib.mg_segment_sum_csr_perm(_p(x_edge), _p(perm), _p(row_ptr), int(n_rows), feat, _p(out), _stream()))
     return out
 
 

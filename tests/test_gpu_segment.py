@@ -44,6 +44,24 @@ def test_segment_sum_long_rows(ops):
     torch.testing.assert_close(out.cpu(), ref, rtol=1e-5, atol=2e-4)
 
 
+@pytest.mark.parametrize("feat_shape", [(), (4,), (3,), (128, 3), (5,), (512,)])
+def test_segment_sum_through_a_permutation(ops, feat_shape):
+    """An unsorted index: rows summed in its stable sorted order through the permutation, bit for bit what gathering
+    the rows into that order and summing them gives (the adjoint of edges_read_dst)."""
+    n_rows, n_edges = 300, 5000
+    g = torch.Generator().manual_seed(11)
+    idx = torch.randint(0, n_rows, (n_edges,), generator=g)
+    idx[idx == 7] = 8
+    x = torch.randn(n_edges, *feat_shape, generator=g).cuda()
+    perm = torch.sort(idx, stable=True).indices
+    row_ptr = ops.segment_row_ptr(idx[perm].cuda(), n_rows)
+    out = ops.segment_sum_csr(x, row_ptr, n_rows, perm=perm.to(torch.int32).cuda())
+    two_step = ops.segment_sum_csr(ops.gather_rows(x, perm.cuda()), row_ptr, n_rows)
+    assert torch.equal(out, two_step)
+    ref = torch.zeros(n_rows, *feat_shape, dtype=torch.float64).index_add_(0, idx, x.cpu().double())
+    torch.testing.assert_close(out.cpu().double(), ref, rtol=1e-5, atol=1e-5)
+
+
 def test_segment_edge_cases(ops):
     row_ptr = ops.segment_row_ptr(torch.empty(0, dtype=torch.int64).cuda(), 7)
     assert row_ptr.tolist() == [0] * 8
