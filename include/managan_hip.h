@@ -388,15 +388,18 @@ int mg_painn_message(const int* row_ptr /* n_nodes+1 */, const int* dst /* E */,
  * edges (archs/meanflow_painn8.py:94-100), as one pass, and the adjoint of that pass.  dist, actv (E, 4n); v (E, n, 3)
  * the gathered vectors; dir (E, 3) = r_ij / sqrt(epsilon + |r_ij|^2):
  *   p = dist * actv;  m[e,c,:] = v[e,c,:] p[e,c] + (v[e,c,:] x dir[e]) p[e,n+c] + dir[e] p[e,2n+c];  a[e,c] = p[e,3n+c]
- * mg_painn_combine_bwd takes the gradients dm (E, n, 3), da (E, n) and writes those of the four inputs.  n: a power of
- * two in 4..256 (mg_painn_combine_supported); arrays contiguous and 16-byte aligned.  The reference evaluates these
- * lines as separate tensor operations. */
+ * node (E ints) or NULL: with an index, actv is (n_rows, 4n) and v (n_rows, n, 3) and edge e reads row node[e] of both
+ * (the gather by destination folded into the pass; an index outside 0..n_rows-1 is clamped); NULL: row e.
+ * mg_painn_combine_bwd takes the gradients dm (E, n, 3), da (E, n) and writes those of the four inputs, all per edge
+ * (d_actv (E, 4n), dv (E, n, 3): with an index the caller sums them over the edges of a row).  n: a power of two in
+ * 4..256 (mg_painn_combine_supported); arrays contiguous and 16-byte aligned.  The reference evaluates these lines as
+ * separate tensor operations. */
 int mg_painn_combine_supported(int n);   /* returns 0 / 1, not a status */
-int mg_painn_combine_fwd(const float* dist, const float* actv, const float* v, const float* dir, long E, int n,
-                         float* m, float* a, mg_stream_t stream);
-int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, const float* dir, const float* dm,
-                         const float* da, long E, int n, float* d_dist, float* d_actv, float* dv, float* d_dir,
-                         mg_stream_t stream);
+int mg_painn_combine_fwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
+                         long n_rows, long E, int n, float* m, float* a, mg_stream_t stream);
+int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
+                         long n_rows, const float* dm, const float* da, long E, int n, float* d_dist, float* d_actv,
+                         float* dv, float* d_dir, mg_stream_t stream);
 
 /* The first two layers of the radial MLP from the edge vectors (archs/meanflow_painn8.py:25-35 feeding :38-51):
  *   y[e] = SiLU(b2 + W2 SiLU(b1 + W1 radial_encode(r_ij[e], 16, rmax))),   y (E, hidden)

@@ -7,6 +7,9 @@
 // HBM, and twice as many in the backward pass; here every input is read once and every output written once.
 // A thread owns 4 consecutive channels of one edge (16-byte loads and stores throughout); the n / 4 threads of an
 // edge are neighbours in a wave, which is what the gradient of d, a sum over channels, is reduced over.
+// actv and v may be given per node with an index (`node`, the edge's destination): the rows are then read through the
+// caches instead of from a gathered per-edge copy; their gradients are still written per edge (the caller sums them
+// over the edges of a node).
 // Not on the inference hot path (that one never materialises dist, actv or v per edge).
 #include "common.hpp"
 
@@ -47,18 +50,21 @@ __device__ __forceinline__ float at(const float4& v, int j) { return j == 0 ? v.
 __global__ void __launch_bounds__(256) painn_combine_fwd_kernel(const float* __restrict__ dist,
                                                                 const float* __restrict__ actv,
                                                                 const float* __restrict__ v,
-                                                                const float* __restrict__ dir, long E, int n,
-                                                                float* __restrict__ m, float* __restrict__ a) {
+                                                                const float* __restrict__ dir,
+                                                                const int* __restrict__ node, long n_rows, long E,
+                                                                int n, float* __restrict__ m, float* __restrict__ a) {
     const int tpe = n >> 2;                                       // threads per edge
     const long t = (long)blockIdx.x * 256 + threadIdx.x;
     const long e = t / tpe;
     if (e >= E) return;
     const int c = (int)(t - e * tpe) * 4;
+    // row of actv and v that this edge reads (an index outside the rows is clamped: never an access out of bounds)
+    const long en = node ? min(max((long)node[e], 0L), n_rows - 1) : e;
     const float* de = dist + e * 4 * n + c;
-    const float* ae = actv + e * 4 * n + c;
+    const float* ae = actv + en * 4 * n + c;
     const float4 p0 = mul4(ld4(de), ld4(ae)), p1 = mul4(ld4(de + n), ld4(ae + n));
     const float4 p2 = mul4(ld4(de + 2 * n), ld4(ae + 2 * n)), p3 = mul4(ld4(de + 3 * n), ld4(ae + 3 * n));
-    const Vec3x4 vv = ld12(v + (e * n + c) * 3);
+    const Vec3x4 vv = ld12(v + (en * n + c) * 3);
     const Vec3 d = {dir[3 * e], dir[3 * e + 1], dir[3 * e + 2]};
     Vec3x4 out;
 #pragma unroll
@@ -77,7 +83,8 @@ __global__ void __launch_bounds__(256) painn_combine_fwd_kernel(const float* __r
 //   d_dir = sum_c (dm[c] x v[c]) p[n + c] + dm[c] p[2n + c]
 __global__ void __launch_bounds__(256) painn_combine_bwd_kernel(
     const float* __restrict__ dist, const float* __restrict__ actv, const float* __restrict__ v,
-    const float* __restrict__ dir, const float* __restrict__ dm, const float* __restrict__ da, long E, int n,
+    const float* __restrict__ dir, const int* __restrict__ node, long n_rows, const float* __restrict__ dm,
+    const float* __restrict__ da, long E, int n,
     float* __restrict__ d_dist, float* __restrict__ d_actv, float* __restrict__ dv, float* __restrict__ d_dir) {
     const int tpe = n >> 2;                                       // a power of two <= 64
     const long t = (long)blockIdx.x * 256 + threadIdx.x;
@@ -85,12 +92,14 @@ __global__ void __launch_bounds__(256) painn_combine_bwd_kernel(
     const bool live = e_raw < E;                                  // (dead threads still take part in the shuffles)
     const long e = live ? e_raw : E - 1;
     const int c = (int)(t - e_raw * tpe) * 4;
+    // row of actv and v that this edge reads (an index outside the rows is clamped: never an access out of bounds)
+    const long en = node ? min(max((long)node[e], 0L), n_rows - 1) : e;
     const float* de = dist + e * 4 * n + c;
-    const float* ae = actv + e * 4 * n + c;
+    const float* ae = actv + en * 4 * n + c;
     float4 dk[4], ak[4];
 #pragma unroll
     for (int k = 0; k < 4; k++) { dk[k] = ld4(de + k * n); ak[k] = ld4(ae + k * n); }
-    const Vec3x4 vv = ld12(v + (e * n + c) * 3), g = ld12(dm + (e * n + c) * 3);
+    const Vec3x4 vv = ld12(v + (en * n + c) * 3), g = ld12(dm + (e * n + c) * 3);
     const float4 ga = ld4(da + e * n + c);
     const Vec3 d = {dir[3 * e], dir[3 * e + 1], dir[3 * e + 2]};
     float dp[3][4];
@@ -140,34 +149,36 @@ extern "C" {
 
 int mg_painn_combine_supported(int n) { return combine_shape_ok(n) ? 1 : 0; }
 
-int mg_painn_combine_fwd(const float* dist, const float* actv, const float* v, const float* dir, long E, int n,
-                         float* m, float* a, mg_stream_t stream) {
+int mg_painn_combine_fwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
+                         long n_rows, long E, int n, float* m, float* a, mg_stream_t stream) {
     MG_REQUIRE(E >= 0 && combine_shape_ok(n), "mg_painn_combine_fwd: n must be a power of two in 4..256");
     if (E == 0) return MG_OK;
     MG_REQUIRE(dist && actv && v && dir && m && a, "mg_painn_combine_fwd: null pointer");
+    MG_REQUIRE(node == nullptr || n_rows > 0, "mg_painn_combine_fwd: an index needs n_rows > 0");
     MG_REQUIRE(aligned16(dist) && aligned16(actv) && aligned16(v) && aligned16(m) && aligned16(a),
                "mg_painn_combine_fwd: arrays must be 16-byte aligned");
     const long threads = E * (n / 4);
     MG_REQUIRE(ceil_div(threads, 256) < (1L << 31), "mg_painn_combine_fwd: too many edges");
     hipLaunchKernelGGL(painn_combine_fwd_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
-                       (hipStream_t)stream, dist, actv, v, dir, E, n, m, a);
+                       (hipStream_t)stream, dist, actv, v, dir, node, n_rows, E, n, m, a);
     return check_launch("mg_painn_combine_fwd");
 }
 
-int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, const float* dir, const float* dm,
-                         const float* da, long E, int n, float* d_dist, float* d_actv, float* dv, float* d_dir,
-                         mg_stream_t stream) {
+int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
+                         long n_rows, const float* dm, const float* da, long E, int n, float* d_dist, float* d_actv,
+                         float* dv, float* d_dir, mg_stream_t stream) {
     MG_REQUIRE(E >= 0 && combine_shape_ok(n), "mg_painn_combine_bwd: n must be a power of two in 4..256");
     if (E == 0) return MG_OK;
     MG_REQUIRE(dist && actv && v && dir && dm && da && d_dist && d_actv && dv && d_dir,
                "mg_painn_combine_bwd: null pointer");
+    MG_REQUIRE(node == nullptr || n_rows > 0, "mg_painn_combine_bwd: an index needs n_rows > 0");
     MG_REQUIRE(aligned16(dist) && aligned16(actv) && aligned16(v) && aligned16(dm) && aligned16(da) &&
                    aligned16(d_dist) && aligned16(d_actv) && aligned16(dv),
                "mg_painn_combine_bwd: arrays must be 16-byte aligned");
     const long threads = E * (n / 4);
     MG_REQUIRE(ceil_div(threads, 256) < (1L << 31), "mg_painn_combine_bwd: too many edges");
     hipLaunchKernelGGL(painn_combine_bwd_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
-                       (hipStream_t)stream, dist, actv, v, dir, dm, da, E, n, d_dist, d_actv, dv, d_dir);
+                       (hipStream_t)stream, dist, actv, v, dir, node, n_rows, dm, da, E, n, d_dist, d_actv, dv, d_dir);
     return check_launch("mg_painn_combine_bwd");
 }
 

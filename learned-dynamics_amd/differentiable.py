@@ -124,43 +124,54 @@ def _painn_combine_plain(dist, actv, v, direction):
 
 
 class _PainnCombine(torch.autograd.Function):
-    """The same lines as one kernel, and their gradient as another.  When the backward pass itself is recorded
-    (create_graph=True, as the Jacobian-vector product of the meanflow loss does), it is evaluated as the gradient of
-    the plain tensor arithmetic instead, which autograd can differentiate again."""
+    """The same lines as one kernel, and their gradient as another, with the gather by destination folded in: actv and
+    v come per node and the kernels read the destination's row (sidx: graph.by_dst); their gradients are summed over
+    the edges of a node here.  When the backward pass itself is recorded (create_graph=True, as the Jacobian-vector
+    product of the meanflow loss does), it is evaluated as the gradient of the plain tensor arithmetic instead, which
+    autograd can differentiate again."""
 
     @staticmethod
-    def forward(ctx, dist, actv, v, direction):
-        ctx.save_for_backward(dist, actv, v, direction)
-        return ops.painn_combine_fwd(dist, actv, v, direction)
+    def forward(ctx, dist, actv_node, v_node, direction, sidx):
+        ctx.sidx = sidx
+        ctx.save_for_backward(dist, actv_node, v_node, direction)
+        return ops.painn_combine_fwd(dist, actv_node, v_node, direction, node=sidx.index)
 
     @staticmethod
     def backward(ctx, dm, da):
-        saved = ctx.saved_tensors
+        saved, sidx = ctx.saved_tensors, ctx.sidx
         if torch.is_grad_enabled():
             with torch.enable_grad():
                 leaves = [t if t.requires_grad else t.detach().requires_grad_() for t in saved]
-                out = _painn_combine_plain(*leaves)
+                out = _painn_combine_plain(leaves[0], gl._Gather.apply(leaves[1], sidx), gl._Gather.apply(leaves[2], sidx),
+                                           leaves[3])
                 grads = torch.autograd.grad(out, leaves, (dm, da), create_graph=True)
-            return tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad))
-        grads = ops.painn_combine_bwd(*saved, dm.contiguous(), da.contiguous())
-        return tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad))
+            return tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad)) + (None,)
+        d_dist, d_actv, dv, d_dir = ops.painn_combine_bwd(*saved, dm.contiguous(), da.contiguous(), node=sidx.index)
+        need = ctx.needs_input_grad
+        return (d_dist if need[0] else None,
+                ops.segment_sum_csr(d_actv, sidx.row_ptr, sidx.n_rows, perm=sidx.perm) if need[1] else None,
+                ops.segment_sum_csr(dv, sidx.row_ptr, sidx.n_rows, perm=sidx.perm) if need[2] else None,
+                d_dir if need[3] else None, None)
 
 
-def painn_combine(dist, actv, v, direction):
-    if (ops.painn_combine_supported(v.size(1)) and all(t.is_contiguous() and t.data_ptr() % 16 == 0
-                                                       for t in (dist, actv, v, direction))):
-        return _PainnCombine.apply(dist, actv, v, direction)
-    return _painn_combine_plain(dist, actv, v, direction)
+def painn_combine(graph, dist, actv_node, v_node, direction):
+    """dist (E, 4n), direction (E, 3) per edge; actv_node (batch, nodes, 4n), v_node (batch, nodes, n, 3) per node, read
+    at each edge's destination.  Returns m (E, n, 3), a (E, n)."""
+    actv_flat, v_flat = gl._flat_nodes(graph, actv_node), gl._flat_nodes(graph, v_node)
+    if (ops.painn_combine_supported(v_flat.size(1)) and all(t.is_contiguous() and t.data_ptr() % 16 == 0
+                                                            for t in (dist, actv_flat, v_flat, direction))):
+        return _PainnCombine.apply(dist, actv_flat, v_flat, direction, graph.by_dst)
+    return _painn_combine_plain(dist, gl._Gather.apply(actv_flat, graph.by_dst), gl._Gather.apply(v_flat, graph.by_dst),
+                                direction)
 
 
 def painn_message(msg, graph, x_a, x_v, r_ij):
     """archs/meanflow_painn8.py:85-100"""
     dist = mlp_silu(msg.mlp_dist, radial_encode_painn(r_ij, msg.n_rbf, msg.r0))
-    # the MLP acts on rows, so it commutes with the gather: N rows go through it, not E (the reference gathers first)
-    actv = gl.edges_read_dst(graph, mlp_silu(msg.mlp_actv, x_a))
+    # the MLP acts on rows, so it commutes with the gather: N rows go through it, not E (the reference gathers first),
+    # and the gathers themselves are folded into the combining kernel
     direction = r_ij / torch.sqrt(msg.epsilon + (r_ij ** 2).sum(-1, keepdim=True))
-    v = gl.edges_read_dst(graph, x_v)
-    m, a = painn_combine(dist, actv, v, direction)
+    m, a = painn_combine(graph, dist, mlp_silu(msg.mlp_actv, x_a), x_v, direction)
     return gl.edges_reduce_src(graph, a.contiguous()), gl.edges_reduce_src(graph, m)
 
 

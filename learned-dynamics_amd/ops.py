@@ -1324,38 +1324,51 @@ def painn_combine_supported(n):
     return bool(_lib.mg_painn_combine_supported(int(n)))
 
 
-def _combine_inputs(dist, actv, v, direction):
+def _combine_inputs(dist, actv, v, direction, node):
     for t, name in ((dist, "dist"), (actv, "actv"), (v, "v"), (direction, "direction")):
         _check_input(t, name)
-    E, n = int(v.size(0)), int(v.size(1))
-    if v.dim() != 3 or v.size(2) != 3 or tuple(dist.shape) != (E, 4 * n) or tuple(actv.shape) != (E, 4 * n) \
+    E, n = int(dist.size(0)), int(v.size(1))
+    rows = int(v.size(0))
+    if node is None:
+        if rows != E:
+            raise RuntimeError("without an index v needs one row per edge")
+    else:
+        _check_input(node, "node", torch.int32)
+        if node.numel() != E:
+            raise RuntimeError("node must have one entry per edge")
+    if v.dim() != 3 or v.size(2) != 3 or tuple(dist.shape) != (E, 4 * n) or tuple(actv.shape) != (rows, 4 * n) \
             or tuple(direction.shape) != (E, 3):
-        raise RuntimeError("expected dist, actv (E, 4n), v (E, n, 3), direction (E, 3)")
-    return E, n
+        raise RuntimeError("expected dist (E, 4n), actv (rows, 4n), v (rows, n, 3), direction (E, 3)")
+    return E, n, rows
 
 
-def painn_combine_fwd(dist, actv, v, direction):
+def painn_combine_fwd(dist, actv, v, direction, node=None):
     """m = v p[:, :n] + (v x direction) p[:, n:2n] + direction p[:, 2n:3n], a = p[:, 3n:] with p = dist * actv
-    (archs/meanflow_painn8.py:94-100), in one pass."""
-    E, n = _combine_inputs(dist, actv, v, direction)
+    (archs/meanflow_painn8.py:94-100), in one pass.  node (int32, one per edge): actv and v hold one row per node and
+    edge e reads row node[e] (the reference's edges_read_dst folded in)."""
+    E, n, rows = _combine_inputs(dist, actv, v, direction, node)
     with torch.cuda.device(v.device):
         m = torch.empty(E, n, 3, dtype=torch.float32, device=v.device)
         a = torch.empty(E, n, dtype=torch.float32, device=v.device)
-        L.check(_lib.mg_painn_combine_fwd(_p(dist), _p(actv), _p(v), _p(direction), E, n, _p(m), _p(a), _stream()))
+        L.check(_lib.mg_painn_combine_fwd(_p(dist), _p(actv), _p(v), _p(direction), _p(node), rows, E, n, _p(m), _p(a),
+                                          _stream()))
     return m, a
 
 
-def painn_combine_bwd(dist, actv, v, direction, dm, da):
-    """Gradients of painn_combine_fwd's four inputs from those of its outputs."""
-    E, n = _combine_inputs(dist, actv, v, direction)
+def painn_combine_bwd(dist, actv, v, direction, dm, da, node=None):
+    """Gradients of painn_combine_fwd's four inputs from those of its outputs; those of actv and v per edge
+    ((E, 4n), (E, n, 3)) also when the inputs are per node."""
+    E, n, rows = _combine_inputs(dist, actv, v, direction, node)
     _check_input(dm, "dm")
     _check_input(da, "da")
     if tuple(dm.shape) != (E, n, 3) or tuple(da.shape) != (E, n):
         raise RuntimeError("expected dm (E, n, 3) and da (E, n)")
     with torch.cuda.device(v.device):
-        d_dist, d_actv = torch.empty_like(dist), torch.empty_like(actv)
-        dv, d_dir = torch.empty_like(v), torch.empty_like(direction)
-        L.check(_lib.mg_painn_combine_bwd(_p(dist), _p(actv), _p(v), _p(direction), _p(dm), _p(da), E, n,
+        d_dist = torch.empty_like(dist)
+        d_actv = torch.empty(E, 4 * n, dtype=torch.float32, device=v.device)
+        dv = torch.empty(E, n, 3, dtype=torch.float32, device=v.device)
+        d_dir = torch.empty_like(direction)
+        L.check(_lib.mg_painn_combine_bwd(_p(dist), _p(actv), _p(v), _p(direction), _p(node), rows, _p(dm), _p(da), E, n,
                                           _p(d_dist), _p(d_actv), _p(dv), _p(d_dir), _stream()))
     return d_dist, d_actv, dv, d_dir
 

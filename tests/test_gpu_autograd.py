@@ -269,18 +269,23 @@ def test_tensor_prods_module_trains(lro):
 
 @pytest.mark.parametrize("E,n", [(1000, 128), (257, 4), (3001, 32), (130, 256)])
 def test_painn_combine_against_plain_arithmetic(pkg, E, n):
-    """The fused elementwise middle of the PaiNN message (archs/meanflow_painn8.py:94-100) and its fused gradient
-    against the same lines in float64 tensor arithmetic; and the gradient of a gradient (which takes the plain
-    arithmetic path) against float64 as well."""
+    """The fused elementwise middle of the PaiNN message (archs/meanflow_painn8.py:94-100, the gathers by destination
+    included) and its fused gradient against the same lines in float64 tensor arithmetic; and the gradient of a
+    gradient (which takes the plain arithmetic path) against float64 as well."""
     diff = importlib.import_module("learned-dynamics_amd.differentiable")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
     g = torch.Generator().manual_seed(E + n)
-    shapes = [(E, 4 * n), (E, 4 * n), (E, n, 3), (E, 3)]
+    N = max(3, E // 7)
+    src = torch.sort(torch.randint(0, N, (E,), generator=g)).values
+    dst = torch.randint(0, N, (E,), generator=g)
+    graph = gl.Graph(src.cuda(), dst.cuda(), None, 1, N)
+    shapes = [(E, 4 * n), (1, N, 4 * n), (1, N, n, 3), (E, 3)]
     cpu = [torch.randn(*s, generator=g, dtype=F64).requires_grad_() for s in shapes]
     gpu = [t.detach().float().cuda().requires_grad_() for t in cpu]
     wm, wa = torch.randn(E, n, 3, generator=g, dtype=F64), torch.randn(E, n, generator=g, dtype=F64)
 
-    ref = diff._painn_combine_plain(*cpu)
-    got = diff.painn_combine(*gpu)
+    ref = diff._painn_combine_plain(cpu[0], cpu[1][0, dst], cpu[2][0, dst], cpu[3])
+    got = diff.painn_combine(graph, *gpu)
     assert got[0].grad_fn is not None and type(got[0].grad_fn).__name__.startswith("_PainnCombine")
     _close(got[0], ref[0], "m")
     _close(got[1], ref[1], "a")
