@@ -28,24 +28,32 @@ def wants_grad(module, *tensors):
     return any(p.requires_grad for p in module.parameters())
 
 
-def linear(lin, x):
-    """nn.Linear through the tensor_linear kernels (weight and input gradients are kernels too)."""
+def linear(lin, x, x_bound=None, want_bound=False):
+    """nn.Linear through the tensor_linear kernels (weight and input gradients are kernels too).  x_bound / want_bound:
+    row maxima handed from one layer to the next (tensor_products.tensor_linear)."""
     lead = x.shape[:-1]
-    y = tensor_linear(0, lin.weight, x.reshape(-1, x.shape[-1]).contiguous(), bias=lin.bias)
-    return y.reshape(*lead, -1)
+    out = tensor_linear(0, lin.weight, x.reshape(-1, x.shape[-1]).contiguous(), bias=lin.bias, x_bound=x_bound,
+                        want_bound=want_bound)
+    if want_bound:
+        return out[0].reshape(*lead, -1), out[1]
+    return out.reshape(*lead, -1)
 
 
 def mlp_silu(mlp, x):
-    """painn.MLP: Linear, SiLU, Linear, SiLU, Linear (archs/meanflow_painn8.py:38-51)."""
+    """painn.MLP: Linear, SiLU, Linear, SiLU, Linear (archs/meanflow_painn8.py:38-51).  |SiLU(z)| <= |z|: the row
+    maxima that a layer's kernel emits for z bound the next layer's input."""
     L = mlp.layers
-    return linear(L[4], F.silu(linear(L[2], F.silu(linear(L[0], x)))))
+    z, b = linear(L[0], x, want_bound=True)
+    z, b = linear(L[2], F.silu(z), x_bound=b, want_bound=True)
+    return linear(L[4], F.silu(z), x_bound=b)
 
 
 def mlp_leaky(mlp, x):
     """bee_layers.MLP: lin_direct(x) + layers(x) with LeakyReLU(0.1) (archs/diffuser_atoms15.py:98-110)."""
     L = mlp.layers
-    h = F.leaky_relu(linear(L[2], F.leaky_relu(linear(L[0], x), 0.1)), 0.1)
-    return linear(mlp.lin_direct, x) + linear(L[4], h)
+    z, b = linear(L[0], x, want_bound=True)
+    z, b = linear(L[2], F.leaky_relu(z, 0.1), x_bound=b, want_bound=True)
+    return linear(mlp.lin_direct, x) + linear(L[4], F.leaky_relu(z, 0.1), x_bound=b)
 
 
 def radial_encode_painn(r, n, rmax):

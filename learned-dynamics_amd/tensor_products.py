@@ -28,7 +28,7 @@ class _TensorLinearFn(torch.autograd.Function):
     bias (plain rows only): added in the kernel's epilogue; its gradient comes out of the weight-gradient pass."""
 
     @staticmethod
-    def forward(ctx, inds, W, x, x_bound=None, bias=None):
+    def forward(ctx, inds, W, x, x_bound=None, bias=None, want_bound=False):
         ctx.inds = inds
         x = x.contiguous()
         if x_bound is None:
@@ -36,10 +36,18 @@ class _TensorLinearFn(torch.autograd.Function):
         ctx.x_bound = x_bound
         ctx.has_bias = bias is not None
         ctx.save_for_backward(W, x)
-        return ops.tensor_linear_fwd(inds, W, x, bias=None if bias is None else bias.contiguous(), row_bound=x_bound)
+        bias = None if bias is None else bias.contiguous()
+        if not want_bound:
+            return ops.tensor_linear_fwd(inds, W, x, bias=bias, row_bound=x_bound)
+        # the kernel's partial row maxima of |y| (an empty tensor when the kernel that ran does not produce them)
+        y, y_bound = ops.tensor_linear_fwd(inds, W, x, bias=bias, row_bound=x_bound, want_rowmax=True)
+        if y_bound is None:
+            y_bound = y.new_empty(0)
+        ctx.mark_non_differentiable(y_bound)
+        return y, y_bound
 
     @staticmethod
-    def backward(ctx, dy):
+    def backward(ctx, dy, *_):
         W, x = ctx.saved_tensors
         dy = dy.contiguous()
         dW = dx = db = None
@@ -51,7 +59,7 @@ class _TensorLinearFn(torch.autograd.Function):
                 db = None
         if ctx.needs_input_grad[2]:
             dx = _TensorLinearFn.apply(ctx.inds, W.t(), dy, dy_bound)   # strides of W are honoured: no copy
-        return None, dW, dx, None, db
+        return None, dW, dx, None, db, None
 
 
 class _WeightGradFn(torch.autograd.Function):
@@ -86,11 +94,17 @@ class _WeightGradFn(torch.autograd.Function):
         return None, g_dy, g_x, None, None, None
 
 
-def tensor_linear(inds, W, x, bias=None):
-    """bias (inds = 0 only): y = x W^T + bias in one kernel."""
+def tensor_linear(inds, W, x, bias=None, x_bound=None, want_bound=False):
+    """bias (inds = 0 only): y = x W^T + bias in one kernel.  x_bound: upper bounds of the row maxima of |x|
+    ((rows, parts)) when the caller holds them.  want_bound: returns (y, bound) with the kernel's partial row maxima
+    of |y|, or None where the kernel that ran does not produce them: they bound |f(y)| for any f with |f(z)| <= |z|
+    (SiLU, LeakyReLU) and save the next layer its pass over the rows."""
     if bias is not None and inds != 0:
         raise RuntimeError("a bias is defined for plain rows only")
-    return _TensorLinearFn.apply(inds, W, x, None, bias)
+    if not want_bound:
+        return _TensorLinearFn.apply(inds, W, x, x_bound, bias)
+    y, y_bound = _TensorLinearFn.apply(inds, W, x, x_bound, bias, True)
+    return y, (y_bound if y_bound.numel() else None)
 
 
 class TensLinear(nn.Module):
