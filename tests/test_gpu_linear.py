@@ -422,3 +422,29 @@ def test_weight_gradient_split_fp16(ops, rows, dim_in, dim_out, bounds):
         ops.set_linear_mode(ops.LINEAR_F16X2)
     assert float((plain.double() - want).abs().max()) <= 1e-6 + 1e-5 * scale + 2 * err_ref
     assert not torch.equal(plain, got)          # (another kernel, another summation order)
+
+
+def test_weight_gradient_at_the_edge_count_of_configs2(ops):
+    """The split-fp16 weight gradient at the size training runs it at (1592454 edge rows, 512 x 512): against float64
+    accumulated over row chunks on the device, with the error of torch's own fp32 product of the same operands as
+    the yardstick; the bias gradient from the same pass; and the same bits on a second run."""
+    rows, dim = 1592454, 512
+    g = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(rows, dim, device="cuda", generator=g)
+    dy = torch.randn(rows, dim, device="cuda", generator=g) * torch.rand(rows, 1, device="cuda", generator=g)
+    got, got_b = ops.tensor_linear_wgrad(0, dy, x, want_bias=True)
+    want = torch.zeros(dim, dim, dtype=torch.float64, device="cuda")
+    want_b = torch.zeros(dim, dtype=torch.float64, device="cuda")
+    fp32 = torch.zeros(dim, dim, dtype=torch.float64, device="cuda")
+    for lo in range(0, rows, 65536):
+        a, b = dy[lo:lo + 65536], x[lo:lo + 65536]
+        want += a.double().t() @ b.double()
+        want_b += a.double().sum(0)
+        fp32 += (a.t() @ b).double()
+    scale = float(want.abs().max())
+    err, err_ref = float((got.double() - want).abs().max()), float((fp32 - want).abs().max())
+    print(f"[wgrad f16x2 {rows}x{dim}x{dim}] err {err:.3g}  chunked fp32 err {err_ref:.3g}  scale {scale:.3g}")
+    assert err <= 1e-6 + 1e-5 * scale + 2 * err_ref, (err, err_ref, scale)
+    assert float((got_b.double() - want_b).abs().max()) <= 1e-6 + 1e-5 * float(want_b.abs().max())
+    again, again_b = ops.tensor_linear_wgrad(0, dy, x, want_bias=True)
+    assert torch.equal(again, got) and torch.equal(again_b, got_b)
