@@ -499,7 +499,8 @@ def bench_gemm_power(torch, args):
 def bench_painn_train(torch, args):
     """Forward + backward of one PaiNN block (Message + Update) at BASELINE configs[2] through the differentiable path
     (every adjoint a kernel of this library: tensor_linear input / weight gradients, gather / segment-sum adjoints,
-    the elementwise autograd functions); gradients for all parameters and both inputs."""
+    the filter's grid interpolation and the message's elementwise middle with their adjoints); gradients for all
+    parameters and both inputs."""
     painn = importlib.import_module("learned-dynamics_amd.painn")
     gl = importlib.import_module("learned-dynamics_amd.graph_layers")
     n, n_rbf, r0, box_len = 128, 16, 8.0, 80.0
@@ -534,8 +535,10 @@ def bench_painn_train(torch, args):
             "detail": {"loss": float(loss.detach()), "gradients_finite": finite,
                        "parameters_with_gradient": sum(gr is not None for gr in grads[2:]),
                        "inference_forward_ms_same_inputs": t_fwd * 1e3},
-            "note": "the differentiable path evaluates the filter MLP on every edge and stores what the backward pass "
-                    "needs; it is composed of the library's unfused kernels and their adjoints"}
+            "note": "the differentiable path: the filter through its 512-row grid (the MLP is differentiated on the grid's "
+                    "rows, each edge interpolates; per-edge evaluation when the grid test rejects the weights), the "
+                    "elementwise middle of the message and the gathers as one kernel each way, split-fp16 GEMMs and "
+                    "weight gradients for the node-sized MLPs"}
 
 
 def bench_denoiser_train(torch, args):

@@ -401,6 +401,25 @@ int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, c
                          long n_rows, const float* dm, const float* da, long E, int n, float* d_dist, float* d_actv,
                          float* dv, float* d_dir, mg_stream_t stream);
 
+/* The filter from its grid, for training (the grid itself: mg_painn_table_message above).  table (table_rows, cols):
+ * the filter at d = k period / table_rows; table_rows and cols powers of two, cols <= 1024.
+ *   mg_painn_table_interp_fwd:  out[e, :] = the 4-point Lagrange interpolation of the grid at d[e] (as the inference kernels do).
+ *   mg_painn_table_buckets:     bucket[e] = the grid row floor(d[e] table_rows / period) mod table_rows.
+ *   mg_painn_table_interp_bwd:  d_table = the adjoint of that interpolation applied to g (E, cols); perm (E ints) lists the
+ *     edges in the order of a stable sort by bucket and bucket_ptr (table_rows + 1 ints) is the row pointer of the sorted
+ *     buckets: the sums run in that order, in pieces added in a fixed order (same bits on every run; workspace from the
+ *     _bytes call).  dd (E) or NULL: the gradient for the lengths, sum_c g[e, c] d out[e, c] / d d[e].
+ * The reference evaluates the filter MLP on every edge (archs/meanflow_painn8.py:92); differentiating through the grid
+ * moves the MLP's backward pass from E rows to table_rows rows. */
+int mg_painn_table_interp_supported(int table_rows, int cols);   /* returns 0 / 1, not a status */
+int mg_painn_table_interp_fwd(const float* table, int table_rows, int cols, float period, const float* d, long E,
+                              float* out, mg_stream_t stream);
+int mg_painn_table_buckets(const float* d, long E, int table_rows, float period, int* bucket, mg_stream_t stream);
+int mg_painn_table_interp_bwd_workspace_bytes(int table_rows, int cols, size_t* bytes /* host */);
+int mg_painn_table_interp_bwd(const float* g, const float* table, int table_rows, int cols, float period, const float* d,
+                              const int* perm, const int* bucket_ptr, long E, void* workspace, float* d_table,
+                              float* dd, mg_stream_t stream);
+
 /* The first two layers of the radial MLP from the edge vectors (archs/meanflow_painn8.py:25-35 feeding :38-51):
  *   y[e] = SiLU(b2 + W2 SiLU(b1 + W1 radial_encode(r_ij[e], 16, rmax))),   y (E, hidden)
  * in one kernel; the first layer's output is produced chunk by chunk on the matrix cores and never stored.

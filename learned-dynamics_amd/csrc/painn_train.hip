@@ -138,6 +138,155 @@ __global__ void __launch_bounds__(256) painn_combine_bwd_kernel(
     if (c == 0) { d_dir[3 * e] = gd.x; d_dir[3 * e + 1] = gd.y; d_dir[3 * e + 2] = gd.z; }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The filter from its grid, for training.  The filter MLP sees an edge only through its length d, so inference
+// evaluates it on a grid over one period of d and interpolates (painn.hip); training can do the same: the forward
+// pass interpolates the (rows, cols) grid at every edge, and the backward pass sends each edge's gradient row to the
+// four grid rows it read, after which the MLP is differentiated on the grid's few hundred rows instead of on every
+// edge.  Interpolation as in painn.hip: u = d * inv_h, i = floor(u), t = u - i, 4-point Lagrange weights on the rows
+// i - 1 .. i + 2 (mod rows; rows is a power of two).
+//
+// The sum over edges has to come out the same on every run: the edges are taken in the order of a stable sort by
+// grid row (perm, bucket_ptr from the host side), each grid row's edges are cut into `splits` consecutive pieces,
+// a workgroup sums one piece (its thread groups take the piece's edges round robin, each in order, and are added in
+// group order), and the pieces and the four taps are added in a fixed order by a second kernel.
+__device__ __forceinline__ void lagrange4(float t, float (&w)[4]) {
+    const float tp = t + 1.0f, tm = t - 1.0f, tq = t - 2.0f;
+    w[0] = -(1.0f / 6.0f) * t * tm * tq;
+    w[1] = 0.5f * tp * tm * tq;
+    w[2] = -0.5f * tp * t * tq;
+    w[3] = (1.0f / 6.0f) * tp * t * tm;
+}
+__device__ __forceinline__ void lagrange4_derivative(float t, float (&w)[4]) {
+    const float tp = t + 1.0f, tm = t - 1.0f, tq = t - 2.0f;
+    w[0] = -(1.0f / 6.0f) * (tm * tq + t * tq + t * tm);
+    w[1] = 0.5f * (tm * tq + tp * tq + tp * tm);
+    w[2] = -0.5f * (t * tq + tp * tq + tp * t);
+    w[3] = (1.0f / 6.0f) * (t * tm + tp * tm + tp * t);
+}
+__device__ __forceinline__ float4 fma4(float w, float4 a, float4 acc) {
+    return make_float4(fmaf(w, a.x, acc.x), fmaf(w, a.y, acc.y), fmaf(w, a.z, acc.z), fmaf(w, a.w, acc.w));
+}
+
+// bucket[e] = i_e & mask, the grid row an edge is sorted by (computed here so that it is the kernels' own i_e)
+__global__ void __launch_bounds__(256) table_bucket_kernel(const float* __restrict__ d, long E, int mask, float inv_h,
+                                                           int* __restrict__ bucket) {
+    const long e = (long)blockIdx.x * 256 + threadIdx.x;
+    if (e < E) bucket[e] = (int)floorf(d[e] * inv_h) & mask;
+}
+
+// out[e, :] = sum_j w_j(t_e) table[(i_e - 1 + j) & mask, :]; a thread owns 4 columns of one edge
+__global__ void __launch_bounds__(256) table_interp_kernel(const float* __restrict__ table, const float* __restrict__ d,
+                                                           long E, int cols, int mask, float inv_h,
+                                                           float* __restrict__ out) {
+    const int tpe = cols >> 2;
+    const long t = (long)blockIdx.x * 256 + threadIdx.x;
+    const long e = t / tpe;
+    if (e >= E) return;
+    const int c = (int)(t - e * tpe) * 4;
+    const float u = d[e] * inv_h, fl = floorf(u);
+    float w[4];
+    lagrange4(u - fl, w);
+    const int i = (int)fl;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc = fma4(w[j], ld4(table + (long)((i - 1 + j) & mask) * cols + c), acc);
+    st4(out + e * cols + c, acc);
+}
+
+// part[((row * splits + s) * 4 + j) * cols + c] = sum over the edges e of piece s of grid row `row` of w_j(t_e) g[e, c]
+__global__ void __launch_bounds__(256) table_scatter_kernel(const float* __restrict__ g, const float* __restrict__ d,
+                                                            const int* __restrict__ perm,
+                                                            const int* __restrict__ bucket_ptr, int cols, float inv_h,
+                                                            int splits, float* __restrict__ part) {
+    __shared__ float4 fold[256 * 4];
+    const int tpe = cols >> 2;                                    // threads per edge: a power of two <= 256
+    const int groups = 256 / tpe, group = threadIdx.x / tpe;
+    const int c = (threadIdx.x - group * tpe) * 4;
+    const int row = blockIdx.x, s = blockIdx.y;
+    const long lo = bucket_ptr[row], hi = bucket_ptr[row + 1];
+    const long len = hi - lo;
+    const long p_lo = lo + len * s / splits, p_hi = lo + len * (s + 1) / splits;
+    float4 acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) acc[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (long p = p_lo + group; p < p_hi; p += groups) {
+        const long e = perm[p];
+        const float u = d[e] * inv_h;
+        float w[4];
+        lagrange4(u - floorf(u), w);
+        const float4 ge = ld4(g + e * cols + c);
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[j] = fma4(w[j], ge, acc[j]);
+    }
+    // thread groups added in group order
+#pragma unroll
+    for (int j = 0; j < 4; j++) fold[threadIdx.x * 4 + j] = acc[j];
+    __syncthreads();
+    if (group == 0) {
+        for (int k = 1; k < groups; k++)
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float4 o = fold[(k * tpe + threadIdx.x) * 4 + j];
+                acc[j].x += o.x; acc[j].y += o.y; acc[j].z += o.z; acc[j].w += o.w;
+            }
+        float* dst = part + ((long)(row * splits + s) * 4) * cols + c;
+#pragma unroll
+        for (int j = 0; j < 4; j++) st4(dst + (long)j * cols, acc[j]);
+    }
+}
+
+// d_table[m, :] = sum_j sum_s part[(m + 1 - j) & mask][s][j][:], taps and pieces in this order
+__global__ void __launch_bounds__(256) table_scatter_finish_kernel(const float* __restrict__ part, int rows, int cols,
+                                                                   int splits, float* __restrict__ d_table) {
+    const int tpe = cols >> 2;
+    const long t = (long)blockIdx.x * 256 + threadIdx.x;
+    const long m = t / tpe;
+    if (m >= rows) return;
+    const int c = (int)(t - m * tpe) * 4;
+    const int mask = rows - 1;
+    float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
+    for (int j = 0; j < 4; j++) {
+        const long row = (m + 1 - j) & mask;
+        const float* src = part + ((row * splits) * 4 + j) * (long)cols + c;
+        for (int s = 0; s < splits; s++) {
+            const float4 v = ld4(src + (long)s * 4 * cols);
+            acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+        }
+    }
+    st4(d_table + m * cols + c, acc);
+}
+
+// dd[e] = inv_h * sum_c g[e, c] sum_j w_j'(t_e) table[(i_e - 1 + j) & mask, c]: a wave per edge
+__global__ void __launch_bounds__(256) table_interp_grad_length_kernel(const float* __restrict__ g,
+                                                                       const float* __restrict__ table,
+                                                                       const float* __restrict__ d, long E, int cols,
+                                                                       int mask, float inv_h, float* __restrict__ dd) {
+    const int lane = threadIdx.x & 63;
+    const long wave = ((long)blockIdx.x * 256 + threadIdx.x) >> 6, n_waves = ((long)gridDim.x * 256) >> 6;
+    for (long e = wave; e < E; e += n_waves) {
+        const float u = d[e] * inv_h, fl = floorf(u);
+        float w[4];
+        lagrange4_derivative(u - fl, w);
+        const int i = (int)fl;
+        float s = 0.f;
+        for (int c = lane * 4; c < cols; c += 256) {
+            float4 tv = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int j = 0; j < 4; j++) tv = fma4(w[j], ld4(table + (long)((i - 1 + j) & mask) * cols + c), tv);
+            const float4 ge = ld4(g + e * cols + c);
+            s += ge.x * tv.x + ge.y * tv.y + ge.z * tv.z + ge.w * tv.w;
+        }
+        for (int k = 1; k < 64; k <<= 1) s += __shfl_xor(s, k);
+        if (lane == 0) dd[e] = s * inv_h;
+    }
+}
+
+constexpr int kTableSplits = 16;
+inline bool table_shape_ok(int rows, int cols) {
+    return rows >= 4 && (rows & (rows - 1)) == 0 && cols >= 4 && cols <= 1024 && (cols & (cols - 1)) == 0;
+}
+
 inline bool combine_shape_ok(int n) { return n >= 4 && n <= 256 && (n & (n - 1)) == 0; }
 
 }  // namespace
@@ -180,6 +329,62 @@ int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, c
     hipLaunchKernelGGL(painn_combine_bwd_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
                        (hipStream_t)stream, dist, actv, v, dir, node, n_rows, dm, da, E, n, d_dist, d_actv, dv, d_dir);
     return check_launch("mg_painn_combine_bwd");
+}
+
+int mg_painn_table_interp_supported(int table_rows, int cols) { return table_shape_ok(table_rows, cols) ? 1 : 0; }
+
+int mg_painn_table_interp_fwd(const float* table, int table_rows, int cols, float period, const float* d, long E,
+                              float* out, mg_stream_t stream) {
+    MG_REQUIRE(E >= 0 && table_shape_ok(table_rows, cols) && period > 0.f,
+               "mg_painn_table_interp_fwd: rows and cols must be powers of two (cols <= 1024), period positive");
+    if (E == 0) return MG_OK;
+    MG_REQUIRE(table && d && out && aligned16(table) && aligned16(out), "mg_painn_table_interp_fwd: null or unaligned pointer");
+    const long threads = E * (cols / 4);
+    MG_REQUIRE(ceil_div(threads, 256) < (1L << 31), "mg_painn_table_interp_fwd: too many edges");
+    hipLaunchKernelGGL(table_interp_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, (hipStream_t)stream,
+                       table, d, E, cols, table_rows - 1, (float)table_rows / period, out);
+    return check_launch("mg_painn_table_interp_fwd");
+}
+
+int mg_painn_table_buckets(const float* d, long E, int table_rows, float period, int* bucket, mg_stream_t stream) {
+    MG_REQUIRE(E >= 0 && table_rows >= 4 && (table_rows & (table_rows - 1)) == 0 && period > 0.f,
+               "mg_painn_table_buckets: rows must be a power of two, period positive");
+    if (E == 0) return MG_OK;
+    MG_REQUIRE(d && bucket, "mg_painn_table_buckets: null pointer");
+    hipLaunchKernelGGL(table_bucket_kernel, dim3((unsigned)ceil_div(E, 256)), dim3(256), 0, (hipStream_t)stream, d, E,
+                       table_rows - 1, (float)table_rows / period, bucket);
+    return check_launch("mg_painn_table_buckets");
+}
+
+int mg_painn_table_interp_bwd_workspace_bytes(int table_rows, int cols, size_t* bytes) {
+    MG_REQUIRE(bytes != nullptr && table_shape_ok(table_rows, cols), "mg_painn_table_interp_bwd_workspace_bytes: bad argument");
+    *bytes = (size_t)table_rows * kTableSplits * 4 * (size_t)cols * sizeof(float) + 16;
+    return MG_OK;
+}
+
+int mg_painn_table_interp_bwd(const float* g, const float* table, int table_rows, int cols, float period, const float* d,
+                              const int* perm, const int* bucket_ptr, long E, void* workspace, float* d_table,
+                              float* dd, mg_stream_t stream) {
+    MG_REQUIRE(E >= 0 && table_shape_ok(table_rows, cols) && period > 0.f,
+               "mg_painn_table_interp_bwd: rows and cols must be powers of two (cols <= 1024), period positive");
+    MG_REQUIRE(d_table && workspace && bucket_ptr && aligned16(d_table), "mg_painn_table_interp_bwd: null or unaligned pointer");
+    MG_REQUIRE(E == 0 || (g && d && perm && aligned16(g)), "mg_painn_table_interp_bwd: null or unaligned pointer");
+    hipStream_t st = (hipStream_t)stream;
+    const float inv_h = (float)table_rows / period;
+    float* part = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(workspace) + 15) & ~uintptr_t(15));
+    hipLaunchKernelGGL(table_scatter_kernel, dim3((unsigned)table_rows, kTableSplits), dim3(256), 0, st, g, d, perm,
+                       bucket_ptr, cols, inv_h, kTableSplits, part);
+    const long threads = (long)table_rows * (cols / 4);
+    hipLaunchKernelGGL(table_scatter_finish_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, st,
+                       (const float*)part, table_rows, cols, kTableSplits, d_table);
+    if (dd && E > 0) {
+        MG_REQUIRE(table && aligned16(table), "mg_painn_table_interp_bwd: the length gradient needs the table");
+        long blocks = ceil_div(E, 4);
+        if (blocks > 256L * 32) blocks = 256L * 32;
+        hipLaunchKernelGGL(table_interp_grad_length_kernel, dim3((unsigned)blocks), dim3(256), 0, st, g, table, d, E, cols,
+                           table_rows - 1, inv_h, dd);
+    }
+    return check_launch("mg_painn_table_interp_bwd");
 }
 
 }  // extern "C"

@@ -173,9 +173,60 @@ def painn_combine(graph, dist, actv_node, v_node, direction):
                                 direction)
 
 
+def _table_interp_plain(table, d, period):
+    """4-point Lagrange interpolation of a periodic grid in tensor arithmetic (differentiable in the grid and in d)."""
+    rows = table.size(0)
+    u = d * (float(rows) / period)
+    fl = torch.floor(u).detach()
+    t = (u - fl)[:, None]
+    i = fl.long()
+    tp, tm, tq = t + 1.0, t - 1.0, t - 2.0
+    w = (-(1.0 / 6.0) * t * tm * tq, 0.5 * tp * tm * tq, -0.5 * tp * t * tq, (1.0 / 6.0) * tp * t * tm)
+    return sum(w[j] * table[(i - 1 + j) % rows] for j in range(4))
+
+
+class _TableInterp(torch.autograd.Function):
+    """The filter of every edge from its grid (forward), and the gradients for the grid and the edge lengths
+    (backward): one kernel each way; the backward sums in the order of a sort by grid row, the same on every run.
+    When the backward pass itself is recorded it is the gradient of the plain tensor arithmetic."""
+
+    @staticmethod
+    def forward(ctx, table, d, period):
+        ctx.period = period
+        ctx.save_for_backward(table, d)
+        return ops.painn_table_interp_fwd(table, d, period)
+
+    @staticmethod
+    def backward(ctx, g):
+        table, d = ctx.saved_tensors
+        if torch.is_grad_enabled():
+            with torch.enable_grad():
+                leaves = [t if t.requires_grad else t.detach().requires_grad_() for t in (table, d)]
+                grads = torch.autograd.grad(_table_interp_plain(*leaves, ctx.period), leaves, g, create_graph=True)
+            return tuple(gr if need else None for gr, need in zip(grads, ctx.needs_input_grad)) + (None,)
+        perm, bucket_ptr = ops.painn_table_sorted_edges(d, table.size(0), ctx.period)
+        d_table, dd = ops.painn_table_interp_bwd(g.contiguous(), table, d, ctx.period, perm, bucket_ptr,
+                                                 want_length_grad=ctx.needs_input_grad[1])
+        return (d_table if ctx.needs_input_grad[0] else None), dd, None
+
+
+def painn_filter(msg, r_ij):
+    """mlp_dist(radial_encode(r_ij)) (archs/meanflow_painn8.py:92), (edges, 4n).  The filter is a smooth periodic
+    function of the edge length: when the module's grid test accepts a grid for the current weights (the test the
+    inference path uses, Message.table_rows) the MLP runs on the grid's rows and every edge interpolates, so that the
+    backward pass differentiates the MLP on a few hundred rows instead of on every edge."""
+    E = r_ij.shape[0]
+    rows = msg.table_rows() if (getattr(msg, "use_table", False) and E >= 4 * msg.TABLE_ROWS[0]) else 0
+    if rows and E >= 4 * rows and ops.painn_table_interp_supported(rows, 4 * msg.n):
+        table = mlp_silu(msg.mlp_dist, msg._grid_encoding(rows, 0.0, r_ij.device))
+        d = torch.linalg.vector_norm(r_ij, dim=-1).contiguous()
+        return _TableInterp.apply(table.contiguous(), d, 2.0 * msg.r0)
+    return mlp_silu(msg.mlp_dist, radial_encode_painn(r_ij, msg.n_rbf, msg.r0))
+
+
 def painn_message(msg, graph, x_a, x_v, r_ij):
     """archs/meanflow_painn8.py:85-100"""
-    dist = mlp_silu(msg.mlp_dist, radial_encode_painn(r_ij, msg.n_rbf, msg.r0))
+    dist = painn_filter(msg, r_ij)
     # the MLP acts on rows, so it commutes with the gather: N rows go through it, not E (the reference gathers first),
     # and the gathers themselves are folded into the combining kernel
     direction = r_ij / torch.sqrt(msg.epsilon + (r_ij ** 2).sum(-1, keepdim=True))

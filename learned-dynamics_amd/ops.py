@@ -1373,6 +1373,59 @@ def painn_combine_bwd(dist, actv, v, direction, dm, da, node=None):
     return d_dist, d_actv, dv, d_dir
 
 
+def painn_table_interp_supported(table_rows, cols):
+    return bool(_lib.mg_painn_table_interp_supported(int(table_rows), int(cols)))
+
+
+def _table_inputs(table, d):
+    _check_input(table, "table")
+    _check_input(d, "d")
+    if table.dim() != 2 or d.dim() != 1:
+        raise RuntimeError("expected table (rows, cols) and d (edges)")
+    return int(table.size(0)), int(table.size(1)), int(d.numel())
+
+
+def painn_table_interp_fwd(table, d, period):
+    """(edges, cols): the grid `table` of a function of period `period`, interpolated at the lengths d (4-point
+    Lagrange, as the inference kernels do)."""
+    rows, cols, E = _table_inputs(table, d)
+    with torch.cuda.device(d.device):
+        out = torch.empty(E, cols, dtype=torch.float32, device=d.device)
+        L.check(_lib.mg_painn_table_interp_fwd(_p(table), rows, cols, float(period), _p(d), E, _p(out), _stream()))
+    return out
+
+
+def painn_table_sorted_edges(d, table_rows, period):
+    """(perm, bucket_ptr): the edges in the order of a stable sort by the grid row below their length, and the row
+    pointer of the sorted rows: what painn_table_interp_bwd sums by."""
+    _check_input(d, "d")
+    E = int(d.numel())
+    with torch.cuda.device(d.device):
+        bucket = torch.empty(E, dtype=torch.int32, device=d.device)
+        L.check(_lib.mg_painn_table_buckets(_p(d), E, int(table_rows), float(period), _p(bucket), _stream()))
+        ordered, perm = torch.sort(bucket, stable=True)
+    return perm.to(torch.int32).contiguous(), segment_row_ptr(ordered.contiguous(), int(table_rows))
+
+
+def painn_table_interp_bwd(g, table, d, period, perm, bucket_ptr, want_length_grad=True):
+    """(d_table, dd): the gradients of painn_table_interp_fwd's table and lengths for the output gradient g."""
+    rows, cols, E = _table_inputs(table, d)
+    _check_input(g, "g")
+    _check_input(perm, "perm", torch.int32)
+    _check_input(bucket_ptr, "bucket_ptr", torch.int32)
+    if tuple(g.shape) != (E, cols) or perm.numel() != E or bucket_ptr.numel() != rows + 1:
+        raise RuntimeError("expected g (edges, cols), perm (edges), bucket_ptr (rows + 1)")
+    with torch.cuda.device(d.device):
+        nbytes = ctypes.c_size_t(0)
+        L.check(_lib.mg_painn_table_interp_bwd_workspace_bytes(rows, cols, ctypes.byref(nbytes)))
+        ws = torch.empty(nbytes.value, dtype=torch.uint8, device=d.device)
+        d_table = torch.empty_like(table)
+        dd = torch.empty_like(d) if want_length_grad else None
+        L.check(_lib.mg_painn_table_interp_bwd(_p(g), _p(table), rows, cols, float(period), _p(d), _p(perm),
+                                               _p(bucket_ptr), E, _p(ws), _p(d_table), _p(dd), _stream()))
+    return d_table, dd
+
+
 def painn_message(row_ptr, dst, r_ij, filt, actv, x_v, epsilon, res_a=None, res_v=None, node_order=None):
     """Fused gather-product-scatter of the PaiNN message (archs/meanflow_painn8.py:91-100).
     filt (E,4n), actv (nodes,4n), x_v (nodes,n,3) -> out_a (nodes,n), out_v (nodes,n,3).
