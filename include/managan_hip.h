@@ -390,7 +390,9 @@ int mg_painn_message(const int* row_ptr /* n_nodes+1 */, const int* dst /* E */,
  *   p = dist * actv;  m[e,c,:] = v[e,c,:] p[e,c] + (v[e,c,:] x dir[e]) p[e,n+c] + dir[e] p[e,2n+c];  a[e,c] = p[e,3n+c]
  * node (E ints) or NULL: with an index, actv is (n_rows, 4n) and v (n_rows, n, 3) and edge e reads row node[e] of both
  * (the gather by destination folded into the pass; an index outside 0..n_rows-1 is clamped); NULL: row e.
- * mg_painn_combine_bwd takes the gradients dm (E, n, 3), da (E, n) and writes those of the four inputs, all per edge
+ * mg_painn_combine_bwd takes the gradients dm (E, n, 3), da (E, n), or with grad_row (E ints) dm (n_grad_rows, n, 3),
+ * da (n_grad_rows, n) read at row grad_row[e] (m and a were summed over the edges of a source node: the gradient of an
+ * edge is its node's), and writes those of the four inputs, all per edge
  * (d_actv (E, 4n), dv (E, n, 3): with an index the caller sums them over the edges of a row).  n: a power of two in
  * 4..256 (mg_painn_combine_supported); arrays contiguous and 16-byte aligned.  The reference evaluates these lines as
  * separate tensor operations. */
@@ -398,8 +400,8 @@ int mg_painn_combine_supported(int n);   /* returns 0 / 1, not a status */
 int mg_painn_combine_fwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
                          long n_rows, long E, int n, float* m, float* a, mg_stream_t stream);
 int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
-                         long n_rows, const float* dm, const float* da, long E, int n, float* d_dist, float* d_actv,
-                         float* dv, float* d_dir, mg_stream_t stream);
+                         long n_rows, const float* dm, const float* da, const int* grad_row, long n_grad_rows, long E,
+                         int n, float* d_dist, float* d_actv, float* dv, float* d_dir, mg_stream_t stream);
 
 /* The filter from its grid, for training (the grid itself: mg_painn_table_message above).  table (table_rows, cols):
  * the filter at d = k period / table_rows; table_rows and cols powers of two, cols <= 1024.

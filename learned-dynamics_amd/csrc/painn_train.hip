@@ -84,7 +84,7 @@ __global__ void __launch_bounds__(256) painn_combine_fwd_kernel(const float* __r
 __global__ void __launch_bounds__(256) painn_combine_bwd_kernel(
     const float* __restrict__ dist, const float* __restrict__ actv, const float* __restrict__ v,
     const float* __restrict__ dir, const int* __restrict__ node, long n_rows, const float* __restrict__ dm,
-    const float* __restrict__ da, long E, int n,
+    const float* __restrict__ da, const int* __restrict__ grad_row, long n_grad_rows, long E, int n,
     float* __restrict__ d_dist, float* __restrict__ d_actv, float* __restrict__ dv, float* __restrict__ d_dir) {
     const int tpe = n >> 2;                                       // a power of two <= 64
     const long t = (long)blockIdx.x * 256 + threadIdx.x;
@@ -99,8 +99,10 @@ __global__ void __launch_bounds__(256) painn_combine_bwd_kernel(
     float4 dk[4], ak[4];
 #pragma unroll
     for (int k = 0; k < 4; k++) { dk[k] = ld4(de + k * n); ak[k] = ld4(ae + k * n); }
-    const Vec3x4 vv = ld12(v + (en * n + c) * 3), g = ld12(dm + (e * n + c) * 3);
-    const float4 ga = ld4(da + e * n + c);
+    // row of dm and da: the edge itself, or (the outputs were summed over the edges of a source node) that node
+    const long eg = grad_row ? min(max((long)grad_row[e], 0L), n_grad_rows - 1) : e;
+    const Vec3x4 vv = ld12(v + (en * n + c) * 3), g = ld12(dm + (eg * n + c) * 3);
+    const float4 ga = ld4(da + eg * n + c);
     const Vec3 d = {dir[3 * e], dir[3 * e + 1], dir[3 * e + 2]};
     float dp[3][4];
     Vec3x4 gv;
@@ -210,7 +212,24 @@ __global__ void __launch_bounds__(256) table_scatter_kernel(const float* __restr
     float4 acc[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) acc[j] = make_float4(0.f, 0.f, 0.f, 0.f);
-    for (long p = p_lo + group; p < p_hi; p += groups) {
+    long p = p_lo + group;
+    for (; p + 3 * groups < p_hi; p += 4 * groups) {              // four edges in flight, added in order
+        long e[4];
+        float u[4];
+        float4 ge[4];
+#pragma unroll
+        for (int q = 0; q < 4; q++) e[q] = perm[p + q * groups];
+#pragma unroll
+        for (int q = 0; q < 4; q++) { u[q] = d[e[q]] * inv_h; ge[q] = ld4(g + e[q] * cols + c); }
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            float w[4];
+            lagrange4(u[q] - floorf(u[q]), w);
+#pragma unroll
+            for (int j = 0; j < 4; j++) acc[j] = fma4(w[j], ge[q], acc[j]);
+        }
+    }
+    for (; p < p_hi; p += groups) {
         const long e = perm[p];
         const float u = d[e] * inv_h;
         float w[4];
@@ -314,20 +333,22 @@ int mg_painn_combine_fwd(const float* dist, const float* actv, const float* v, c
 }
 
 int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
-                         long n_rows, const float* dm, const float* da, long E, int n, float* d_dist, float* d_actv,
-                         float* dv, float* d_dir, mg_stream_t stream) {
+                         long n_rows, const float* dm, const float* da, const int* grad_row, long n_grad_rows, long E,
+                         int n, float* d_dist, float* d_actv, float* dv, float* d_dir, mg_stream_t stream) {
     MG_REQUIRE(E >= 0 && combine_shape_ok(n), "mg_painn_combine_bwd: n must be a power of two in 4..256");
     if (E == 0) return MG_OK;
     MG_REQUIRE(dist && actv && v && dir && dm && da && d_dist && d_actv && dv && d_dir,
                "mg_painn_combine_bwd: null pointer");
-    MG_REQUIRE(node == nullptr || n_rows > 0, "mg_painn_combine_bwd: an index needs n_rows > 0");
+    MG_REQUIRE((node == nullptr || n_rows > 0) && (grad_row == nullptr || n_grad_rows > 0),
+               "mg_painn_combine_bwd: an index needs a positive row count");
     MG_REQUIRE(aligned16(dist) && aligned16(actv) && aligned16(v) && aligned16(dm) && aligned16(da) &&
                    aligned16(d_dist) && aligned16(d_actv) && aligned16(dv),
                "mg_painn_combine_bwd: arrays must be 16-byte aligned");
     const long threads = E * (n / 4);
     MG_REQUIRE(ceil_div(threads, 256) < (1L << 31), "mg_painn_combine_bwd: too many edges");
     hipLaunchKernelGGL(painn_combine_bwd_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
-                       (hipStream_t)stream, dist, actv, v, dir, node, n_rows, dm, da, E, n, d_dist, d_actv, dv, d_dir);
+                       (hipStream_t)stream, dist, actv, v, dir, node, n_rows, dm, da, grad_row, n_grad_rows, E, n, d_dist, d_actv, dv,
+                       d_dir);
     return check_launch("mg_painn_combine_bwd");
 }
 

@@ -132,45 +132,54 @@ def _painn_combine_plain(dist, actv, v, direction):
 
 
 class _PainnCombine(torch.autograd.Function):
-    """The same lines as one kernel, and their gradient as another, with the gather by destination folded in: actv and
-    v come per node and the kernels read the destination's row (sidx: graph.by_dst); their gradients are summed over
-    the edges of a node here.  When the backward pass itself is recorded (create_graph=True, as the Jacobian-vector
-    product of the meanflow loss does), it is evaluated as the gradient of the plain tensor arithmetic instead, which
-    autograd can differentiate again."""
+    """The same lines as one kernel, and their gradient as another, with the graph operations on either side folded
+    in: actv and v come per node and the kernels read the destination's row (by_dst); m and a are summed over the
+    edges of their source node (by_src) and the gradient kernel reads the node's gradient row through the source
+    index; the gradients of actv and v are summed over the edges of a destination here.  When the backward pass
+    itself is recorded (create_graph=True, as the Jacobian-vector product of the meanflow loss does), it is evaluated
+    as the gradient of the plain tensor arithmetic instead, which autograd can differentiate again."""
 
     @staticmethod
-    def forward(ctx, dist, actv_node, v_node, direction, sidx):
-        ctx.sidx = sidx
+    def forward(ctx, dist, actv_node, v_node, direction, by_dst, by_src):
+        ctx.by_dst, ctx.by_src = by_dst, by_src
         ctx.save_for_backward(dist, actv_node, v_node, direction)
-        return ops.painn_combine_fwd(dist, actv_node, v_node, direction, node=sidx.index)
+        m, a = ops.painn_combine_fwd(dist, actv_node, v_node, direction, node=by_dst.index)
+        return (ops.segment_sum_csr(m, by_src.row_ptr, by_src.n_rows), ops.segment_sum_csr(a, by_src.row_ptr, by_src.n_rows))
 
     @staticmethod
-    def backward(ctx, dm, da):
-        saved, sidx = ctx.saved_tensors, ctx.sidx
+    def backward(ctx, d_out_v, d_out_a):
+        saved, by_dst, by_src = ctx.saved_tensors, ctx.by_dst, ctx.by_src
         if torch.is_grad_enabled():
             with torch.enable_grad():
                 leaves = [t if t.requires_grad else t.detach().requires_grad_() for t in saved]
-                out = _painn_combine_plain(leaves[0], gl._Gather.apply(leaves[1], sidx), gl._Gather.apply(leaves[2], sidx),
-                                           leaves[3])
-                grads = torch.autograd.grad(out, leaves, (dm, da), create_graph=True)
-            return tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad)) + (None,)
-        d_dist, d_actv, dv, d_dir = ops.painn_combine_bwd(*saved, dm.contiguous(), da.contiguous(), node=sidx.index)
+                m, a = _painn_combine_plain(leaves[0], gl._Gather.apply(leaves[1], by_dst),
+                                            gl._Gather.apply(leaves[2], by_dst), leaves[3])
+                out = (gl._ScatterSum.apply(m, by_src), gl._ScatterSum.apply(a.contiguous(), by_src))
+                grads = torch.autograd.grad(out, leaves, (d_out_v, d_out_a), create_graph=True)
+            return tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad)) + (None, None)
+        d_dist, d_actv, dv, d_dir = ops.painn_combine_bwd(*saved, d_out_v.contiguous(), d_out_a.contiguous(),
+                                                          node=by_dst.index, grad_row=by_src.index)
         need = ctx.needs_input_grad
         return (d_dist if need[0] else None,
-                ops.segment_sum_csr(d_actv, sidx.row_ptr, sidx.n_rows, perm=sidx.perm) if need[1] else None,
-                ops.segment_sum_csr(dv, sidx.row_ptr, sidx.n_rows, perm=sidx.perm) if need[2] else None,
-                d_dir if need[3] else None, None)
+                ops.segment_sum_csr(d_actv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm) if need[1] else None,
+                ops.segment_sum_csr(dv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm) if need[2] else None,
+                d_dir if need[3] else None, None, None)
 
 
 def painn_combine(graph, dist, actv_node, v_node, direction):
     """dist (E, 4n), direction (E, 3) per edge; actv_node (batch, nodes, 4n), v_node (batch, nodes, n, 3) per node, read
-    at each edge's destination.  Returns m (E, n, 3), a (E, n)."""
+    at each edge's destination.  Returns the sums over the edges of each source node: (out_v (batch, nodes, n, 3),
+    out_a (batch, nodes, n))."""
     actv_flat, v_flat = gl._flat_nodes(graph, actv_node), gl._flat_nodes(graph, v_node)
     if (ops.painn_combine_supported(v_flat.size(1)) and all(t.is_contiguous() and t.data_ptr() % 16 == 0
                                                             for t in (dist, actv_flat, v_flat, direction))):
-        return _PainnCombine.apply(dist, actv_flat, v_flat, direction, graph.by_dst)
-    return _painn_combine_plain(dist, gl._Gather.apply(actv_flat, graph.by_dst), gl._Gather.apply(v_flat, graph.by_dst),
-                                direction)
+        out_v, out_a = _PainnCombine.apply(dist, actv_flat, v_flat, direction, graph.by_dst, graph.by_src)
+    else:
+        m, a = _painn_combine_plain(dist, gl._Gather.apply(actv_flat, graph.by_dst),
+                                    gl._Gather.apply(v_flat, graph.by_dst), direction)
+        out_v, out_a = gl._ScatterSum.apply(m, graph.by_src), gl._ScatterSum.apply(a.contiguous(), graph.by_src)
+    return (out_v.reshape(graph.batch, graph.nodes, *out_v.shape[1:]),
+            out_a.reshape(graph.batch, graph.nodes, *out_a.shape[1:]))
 
 
 def _table_interp_plain(table, d, period):
@@ -230,8 +239,8 @@ def painn_message(msg, graph, x_a, x_v, r_ij):
     # the MLP acts on rows, so it commutes with the gather: N rows go through it, not E (the reference gathers first),
     # and the gathers themselves are folded into the combining kernel
     direction = r_ij / torch.sqrt(msg.epsilon + (r_ij ** 2).sum(-1, keepdim=True))
-    m, a = painn_combine(graph, dist, mlp_silu(msg.mlp_actv, x_a), x_v, direction)
-    return gl.edges_reduce_src(graph, a.contiguous()), gl.edges_reduce_src(graph, m)
+    out_v, out_a = painn_combine(graph, dist, mlp_silu(msg.mlp_actv, x_a), x_v, direction)
+    return out_a, out_v
 
 
 def painn_update(upd, x_a, x_v):

@@ -1355,21 +1355,29 @@ def painn_combine_fwd(dist, actv, v, direction, node=None):
     return m, a
 
 
-def painn_combine_bwd(dist, actv, v, direction, dm, da, node=None):
+def painn_combine_bwd(dist, actv, v, direction, dm, da, node=None, grad_row=None):
     """Gradients of painn_combine_fwd's four inputs from those of its outputs; those of actv and v per edge
-    ((E, 4n), (E, n, 3)) also when the inputs are per node."""
+    ((E, 4n), (E, n, 3)) also when the inputs are per node.  grad_row (int32, one per edge): dm and da hold one row per
+    node and edge e takes row grad_row[e] (the adjoint of summing m and a over the edges of a source node)."""
     E, n, rows = _combine_inputs(dist, actv, v, direction, node)
     _check_input(dm, "dm")
     _check_input(da, "da")
-    if tuple(dm.shape) != (E, n, 3) or tuple(da.shape) != (E, n):
-        raise RuntimeError("expected dm (E, n, 3) and da (E, n)")
+    g_rows = E
+    if grad_row is not None:
+        _check_input(grad_row, "grad_row", torch.int32)
+        g_rows = int(dm.size(0))
+        if grad_row.numel() != E:
+            raise RuntimeError("grad_row must have one entry per edge")
+    if tuple(dm.shape) != (g_rows, n, 3) or tuple(da.shape) != (g_rows, n):
+        raise RuntimeError("expected dm (rows, n, 3) and da (rows, n)")
     with torch.cuda.device(v.device):
         d_dist = torch.empty_like(dist)
         d_actv = torch.empty(E, 4 * n, dtype=torch.float32, device=v.device)
         dv = torch.empty(E, n, 3, dtype=torch.float32, device=v.device)
         d_dir = torch.empty_like(direction)
-        L.check(_lib.mg_painn_combine_bwd(_p(dist), _p(actv), _p(v), _p(direction), _p(node), rows, _p(dm), _p(da), E, n,
-                                          _p(d_dist), _p(d_actv), _p(dv), _p(d_dir), _stream()))
+        L.check(_lib.mg_painn_combine_bwd(_p(dist), _p(actv), _p(v), _p(direction), _p(node), rows, _p(dm), _p(da),
+                                          _p(grad_row), g_rows, E, n, _p(d_dist), _p(d_actv), _p(dv), _p(d_dir),
+                                          _stream()))
     return d_dist, d_actv, dv, d_dir
 
 
