@@ -411,16 +411,19 @@ int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, c
  *     edges in the order of a stable sort by bucket and bucket_ptr (table_rows + 1 ints) is the row pointer of the sorted
  *     buckets: the sums run in that order, in pieces added in a fixed order (same bits on every run; workspace from the
  *     _bytes call).  dd (E) or NULL: the gradient for the lengths, sum_c g[e, c] d out[e, c] / d d[e].
+ * order (0 .. 3): the interpolant's order-th derivative with respect to d in place of the interpolant (its weights are
+ * cubics in d): the derivatives of these operations are the same operations at other orders, which is what makes them
+ * differentiable any number of times.
  * The reference evaluates the filter MLP on every edge (archs/meanflow_painn8.py:92); differentiating through the grid
  * moves the MLP's backward pass from E rows to table_rows rows. */
 int mg_painn_table_interp_supported(int table_rows, int cols);   /* returns 0 / 1, not a status */
 int mg_painn_table_interp_fwd(const float* table, int table_rows, int cols, float period, const float* d, long E,
-                              float* out, mg_stream_t stream);
+                              int order, float* out, mg_stream_t stream);
 int mg_painn_table_buckets(const float* d, long E, int table_rows, float period, int* bucket, mg_stream_t stream);
 int mg_painn_table_interp_bwd_workspace_bytes(int table_rows, int cols, size_t* bytes /* host */);
 int mg_painn_table_interp_bwd(const float* g, const float* table, int table_rows, int cols, float period, const float* d,
-                              const int* perm, const int* bucket_ptr, long E, void* workspace, float* d_table,
-                              float* dd, mg_stream_t stream);
+                              const int* perm, const int* bucket_ptr, long E, int order, void* workspace,
+                              float* d_table, float* dd, mg_stream_t stream);
 
 /* The first two layers of the radial MLP from the edge vectors (archs/meanflow_painn8.py:25-35 feeding :38-51):
  *   y[e] = SiLU(b2 + W2 SiLU(b1 + W1 radial_encode(r_ij[e], 16, rmax))),   y (E, hidden)

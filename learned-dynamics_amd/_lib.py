@@ -94,10 +94,10 @@ _SIGNATURES = {
     "mg_painn_table_message_sliced": [vp, vp, vp, i32, i64, vp, vp, i32, vp, vp, i32, vp, vp, vp, vp, vp],
     "mg_painn_combine_supported": [i32],
     "mg_painn_table_interp_supported": [i32, i32],
-    "mg_painn_table_interp_fwd": [vp, i32, i32, f32, vp, i64, vp, vp],
+    "mg_painn_table_interp_fwd": [vp, i32, i32, f32, vp, i64, i32, vp, vp],
     "mg_painn_table_buckets": [vp, i64, i32, f32, vp, vp],
     "mg_painn_table_interp_bwd_workspace_bytes": [i32, i32, ctypes.POINTER(ctypes.c_size_t)],
-    "mg_painn_table_interp_bwd": [vp, vp, i32, i32, f32, vp, vp, vp, i64, vp, vp, vp, vp],
+    "mg_painn_table_interp_bwd": [vp, vp, i32, i32, f32, vp, vp, vp, i64, i32, vp, vp, vp, vp],
     "mg_painn_combine_fwd": [vp, vp, vp, vp, vp, i64, i64, i32, vp, vp, vp],
     "mg_painn_combine_bwd": [vp, vp, vp, vp, vp, i64, vp, vp, vp, i64, i64, i32, vp, vp, vp, vp, vp],
     "mg_painn_message": [vp, vp, vp, i32, i64, vp, vp, vp, vp, i32, f32, vp, vp, vp, vp, vp],

@@ -166,6 +166,16 @@ __device__ __forceinline__ void lagrange4_derivative(float t, float (&w)[4]) {
     w[2] = -0.5f * (t * tq + tp * tq + tp * t);
     w[3] = (1.0f / 6.0f) * (t * tm + tp * tm + tp * t);
 }
+// the order-th derivative of the four weights with respect to t (order 0 .. 3; the weights are cubics)
+__device__ __forceinline__ void lagrange4_order(float t, int order, float (&w)[4]) {
+    if (order == 0) { lagrange4(t, w); return; }
+    if (order == 1) { lagrange4_derivative(t, w); return; }
+    if (order == 2) {
+        w[0] = 1.0f - t; w[1] = 3.0f * t - 2.0f; w[2] = 1.0f - 3.0f * t; w[3] = t;
+        return;
+    }
+    w[0] = -1.0f; w[1] = 3.0f; w[2] = -3.0f; w[3] = 1.0f;
+}
 __device__ __forceinline__ float4 fma4(float w, float4 a, float4 acc) {
     return make_float4(fmaf(w, a.x, acc.x), fmaf(w, a.y, acc.y), fmaf(w, a.z, acc.z), fmaf(w, a.w, acc.w));
 }
@@ -178,9 +188,10 @@ __global__ void __launch_bounds__(256) table_bucket_kernel(const float* __restri
 }
 
 // out[e, :] = sum_j w_j(t_e) table[(i_e - 1 + j) & mask, :]; a thread owns 4 columns of one edge
+// (order > 0: the order-th derivative with respect to d, weights differentiated and scaled by inv_h^order)
 __global__ void __launch_bounds__(256) table_interp_kernel(const float* __restrict__ table, const float* __restrict__ d,
-                                                           long E, int cols, int mask, float inv_h,
-                                                           float* __restrict__ out) {
+                                                           long E, int cols, int mask, float inv_h, int order,
+                                                           float scale, float* __restrict__ out) {
     const int tpe = cols >> 2;
     const long t = (long)blockIdx.x * 256 + threadIdx.x;
     const long e = t / tpe;
@@ -188,11 +199,11 @@ __global__ void __launch_bounds__(256) table_interp_kernel(const float* __restri
     const int c = (int)(t - e * tpe) * 4;
     const float u = d[e] * inv_h, fl = floorf(u);
     float w[4];
-    lagrange4(u - fl, w);
+    lagrange4_order(u - fl, order, w);
     const int i = (int)fl;
     float4 acc = make_float4(0.f, 0.f, 0.f, 0.f);
 #pragma unroll
-    for (int j = 0; j < 4; j++) acc = fma4(w[j], ld4(table + (long)((i - 1 + j) & mask) * cols + c), acc);
+    for (int j = 0; j < 4; j++) acc = fma4(w[j] * scale, ld4(table + (long)((i - 1 + j) & mask) * cols + c), acc);
     st4(out + e * cols + c, acc);
 }
 
@@ -200,7 +211,8 @@ __global__ void __launch_bounds__(256) table_interp_kernel(const float* __restri
 __global__ void __launch_bounds__(256) table_scatter_kernel(const float* __restrict__ g, const float* __restrict__ d,
                                                             const int* __restrict__ perm,
                                                             const int* __restrict__ bucket_ptr, int cols, float inv_h,
-                                                            int splits, float* __restrict__ part) {
+                                                            int order, float scale, int splits,
+                                                            float* __restrict__ part) {
     __shared__ float4 fold[256 * 4];
     const int tpe = cols >> 2;                                    // threads per edge: a power of two <= 256
     const int groups = 256 / tpe, group = threadIdx.x / tpe;
@@ -224,19 +236,19 @@ __global__ void __launch_bounds__(256) table_scatter_kernel(const float* __restr
 #pragma unroll
         for (int q = 0; q < 4; q++) {
             float w[4];
-            lagrange4(u[q] - floorf(u[q]), w);
+            lagrange4_order(u[q] - floorf(u[q]), order, w);
 #pragma unroll
-            for (int j = 0; j < 4; j++) acc[j] = fma4(w[j], ge[q], acc[j]);
+            for (int j = 0; j < 4; j++) acc[j] = fma4(w[j] * scale, ge[q], acc[j]);
         }
     }
     for (; p < p_hi; p += groups) {
         const long e = perm[p];
         const float u = d[e] * inv_h;
         float w[4];
-        lagrange4(u - floorf(u), w);
+        lagrange4_order(u - floorf(u), order, w);
         const float4 ge = ld4(g + e * cols + c);
 #pragma unroll
-        for (int j = 0; j < 4; j++) acc[j] = fma4(w[j], ge, acc[j]);
+        for (int j = 0; j < 4; j++) acc[j] = fma4(w[j] * scale, ge, acc[j]);
     }
     // thread groups added in group order
 #pragma unroll
@@ -280,13 +292,14 @@ __global__ void __launch_bounds__(256) table_scatter_finish_kernel(const float* 
 __global__ void __launch_bounds__(256) table_interp_grad_length_kernel(const float* __restrict__ g,
                                                                        const float* __restrict__ table,
                                                                        const float* __restrict__ d, long E, int cols,
-                                                                       int mask, float inv_h, float* __restrict__ dd) {
+                                                                       int mask, float inv_h, int order, float scale,
+                                                                       float* __restrict__ dd) {
     const int lane = threadIdx.x & 63;
     const long wave = ((long)blockIdx.x * 256 + threadIdx.x) >> 6, n_waves = ((long)gridDim.x * 256) >> 6;
     for (long e = wave; e < E; e += n_waves) {
         const float u = d[e] * inv_h, fl = floorf(u);
         float w[4];
-        lagrange4_derivative(u - fl, w);
+        lagrange4_order(u - fl, order + 1, w);
         const int i = (int)fl;
         float s = 0.f;
         for (int c = lane * 4; c < cols; c += 256) {
@@ -297,7 +310,7 @@ __global__ void __launch_bounds__(256) table_interp_grad_length_kernel(const flo
             s += ge.x * tv.x + ge.y * tv.y + ge.z * tv.z + ge.w * tv.w;
         }
         for (int k = 1; k < 64; k <<= 1) s += __shfl_xor(s, k);
-        if (lane == 0) dd[e] = s * inv_h;
+        if (lane == 0) dd[e] = s * scale * inv_h;
     }
 }
 
@@ -354,16 +367,19 @@ int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, c
 
 int mg_painn_table_interp_supported(int table_rows, int cols) { return table_shape_ok(table_rows, cols) ? 1 : 0; }
 
+inline float int_power(float x, int k) { float p = 1.f; for (int i = 0; i < k; i++) p *= x; return p; }
+
 int mg_painn_table_interp_fwd(const float* table, int table_rows, int cols, float period, const float* d, long E,
-                              float* out, mg_stream_t stream) {
-    MG_REQUIRE(E >= 0 && table_shape_ok(table_rows, cols) && period > 0.f,
-               "mg_painn_table_interp_fwd: rows and cols must be powers of two (cols <= 1024), period positive");
+                              int order, float* out, mg_stream_t stream) {
+    MG_REQUIRE(E >= 0 && table_shape_ok(table_rows, cols) && period > 0.f && order >= 0 && order <= 3,
+               "mg_painn_table_interp_fwd: rows and cols must be powers of two (cols <= 1024), period positive, order 0..3");
     if (E == 0) return MG_OK;
     MG_REQUIRE(table && d && out && aligned16(table) && aligned16(out), "mg_painn_table_interp_fwd: null or unaligned pointer");
     const long threads = E * (cols / 4);
     MG_REQUIRE(ceil_div(threads, 256) < (1L << 31), "mg_painn_table_interp_fwd: too many edges");
     hipLaunchKernelGGL(table_interp_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, (hipStream_t)stream,
-                       table, d, E, cols, table_rows - 1, (float)table_rows / period, out);
+                       table, d, E, cols, table_rows - 1, (float)table_rows / period, order,
+                       int_power((float)table_rows / period, order), out);
     return check_launch("mg_painn_table_interp_fwd");
 }
 
@@ -384,17 +400,19 @@ int mg_painn_table_interp_bwd_workspace_bytes(int table_rows, int cols, size_t* 
 }
 
 int mg_painn_table_interp_bwd(const float* g, const float* table, int table_rows, int cols, float period, const float* d,
-                              const int* perm, const int* bucket_ptr, long E, void* workspace, float* d_table,
-                              float* dd, mg_stream_t stream) {
-    MG_REQUIRE(E >= 0 && table_shape_ok(table_rows, cols) && period > 0.f,
-               "mg_painn_table_interp_bwd: rows and cols must be powers of two (cols <= 1024), period positive");
+                              const int* perm, const int* bucket_ptr, long E, int order, void* workspace,
+                              float* d_table, float* dd, mg_stream_t stream) {
+    MG_REQUIRE(E >= 0 && table_shape_ok(table_rows, cols) && period > 0.f && order >= 0 && order <= 3,
+               "mg_painn_table_interp_bwd: rows and cols must be powers of two (cols <= 1024), period positive, order 0..3");
+    MG_REQUIRE(dd == nullptr || order < 3, "mg_painn_table_interp_bwd: the third derivative has no length gradient");
     MG_REQUIRE(d_table && workspace && bucket_ptr && aligned16(d_table), "mg_painn_table_interp_bwd: null or unaligned pointer");
     MG_REQUIRE(E == 0 || (g && d && perm && aligned16(g)), "mg_painn_table_interp_bwd: null or unaligned pointer");
     hipStream_t st = (hipStream_t)stream;
     const float inv_h = (float)table_rows / period;
     float* part = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(workspace) + 15) & ~uintptr_t(15));
+    const float scale = int_power(inv_h, order);
     hipLaunchKernelGGL(table_scatter_kernel, dim3((unsigned)table_rows, kTableSplits), dim3(256), 0, st, g, d, perm,
-                       bucket_ptr, cols, inv_h, kTableSplits, part);
+                       bucket_ptr, cols, inv_h, order, scale, kTableSplits, part);
     const long threads = (long)table_rows * (cols / 4);
     hipLaunchKernelGGL(table_scatter_finish_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, st,
                        (const float*)part, table_rows, cols, kTableSplits, d_table);
@@ -403,7 +421,7 @@ int mg_painn_table_interp_bwd(const float* g, const float* table, int table_rows
         long blocks = ceil_div(E, 4);
         if (blocks > 256L * 32) blocks = 256L * 32;
         hipLaunchKernelGGL(table_interp_grad_length_kernel, dim3((unsigned)blocks), dim3(256), 0, st, g, table, d, E, cols,
-                           table_rows - 1, inv_h, dd);
+                           table_rows - 1, inv_h, order, scale, dd);
     }
     return check_launch("mg_painn_table_interp_bwd");
 }

@@ -194,29 +194,81 @@ def _table_interp_plain(table, d, period):
     return sum(w[j] * table[(i - 1 + j) % rows] for j in range(4))
 
 
+class _SortedLengths:
+    """The edges sorted by the grid row below their length: what the sums into the grid run by; computed on first
+    use and shared by every pass over the same lengths."""
+
+    def __init__(self, d, rows, period):
+        self.d, self.rows, self.period = d, rows, period
+        self._sorted = None
+
+    def get(self):
+        if self._sorted is None:
+            self._sorted = ops.painn_table_sorted_edges(self.d.detach(), self.rows, self.period)
+        return self._sorted
+
+
 class _TableInterp(torch.autograd.Function):
-    """The filter of every edge from its grid (forward), and the gradients for the grid and the edge lengths
-    (backward): one kernel each way; the backward sums in the order of a sort by grid row, the same on every run.
-    When the backward pass itself is recorded it is the gradient of the plain tensor arithmetic."""
+    """order 0: the filter of every edge interpolated from its grid; order k: the interpolant's k-th derivative in
+    the edge length (its weights are cubics: orders 0 .. 3 exist, the fourth derivative is zero).  The gradient for
+    the grid is _TableScatter of the same order, the gradient for the lengths a row-wise product with _TableInterp of
+    the next order: the family is closed under differentiation, so any number of nested derivatives run on these
+    kernels.  Outside a recorded backward pass both gradients come from one fused call."""
 
     @staticmethod
-    def forward(ctx, table, d, period):
-        ctx.period = period
+    def forward(ctx, table, d, period, order, order_by):
+        ctx.period, ctx.order, ctx.order_by = period, order, order_by
         ctx.save_for_backward(table, d)
-        return ops.painn_table_interp_fwd(table, d, period)
+        return ops.painn_table_interp_fwd(table, d, period, order)
 
     @staticmethod
     def backward(ctx, g):
         table, d = ctx.saved_tensors
-        if torch.is_grad_enabled():
-            with torch.enable_grad():
-                leaves = [t if t.requires_grad else t.detach().requires_grad_() for t in (table, d)]
-                grads = torch.autograd.grad(_table_interp_plain(*leaves, ctx.period), leaves, g, create_graph=True)
-            return tuple(gr if need else None for gr, need in zip(grads, ctx.needs_input_grad)) + (None,)
-        perm, bucket_ptr = ops.painn_table_sorted_edges(d, table.size(0), ctx.period)
-        d_table, dd = ops.painn_table_interp_bwd(g.contiguous(), table, d, ctx.period, perm, bucket_ptr,
-                                                 want_length_grad=ctx.needs_input_grad[1])
-        return (d_table if ctx.needs_input_grad[0] else None), dd, None
+        g = g.contiguous()
+        need_t, need_d = ctx.needs_input_grad[0], ctx.needs_input_grad[1] and ctx.order < 3
+        if not torch.is_grad_enabled():
+            perm, bucket_ptr = ctx.order_by.get()
+            d_table, dd = ops.painn_table_interp_bwd(g, table, d, ctx.period, perm, bucket_ptr, want_length_grad=need_d,
+                                                     order=ctx.order)
+            return (d_table if need_t else None), dd, None, None, None
+        d_table = dd = None
+        if need_t:
+            d_table = _TableScatter.apply(g, d, ctx.period, ctx.order, table.size(0), ctx.order_by)
+        if need_d:
+            dd = (g * _TableInterp.apply(table, d, ctx.period, ctx.order + 1, ctx.order_by)).sum(-1)
+        return d_table, dd, None, None, None
+
+
+class _TableScatter(torch.autograd.Function):
+    """The adjoint of _TableInterp in the grid: every edge's row g[e] added to the four grid rows around its length
+    with the (order-th derivative) weights, in the order of a sort by grid row.  Linear in g; its gradients are
+    _TableInterp calls."""
+
+    @staticmethod
+    def forward(ctx, g, d, period, order, rows, order_by):
+        ctx.period, ctx.order, ctx.order_by = period, order, order_by
+        ctx.save_for_backward(g, d)
+        perm, bucket_ptr = order_by.get()
+        return ops.painn_table_interp_bwd(g.contiguous(), None, d, period, perm, bucket_ptr, want_length_grad=False,
+                                          order=order, table_rows=rows)[0]
+
+    @staticmethod
+    def backward(ctx, dd_table):
+        g, d = ctx.saved_tensors
+        dd_table = dd_table.contiguous()
+        d_g = dd = None
+        if ctx.needs_input_grad[0]:
+            d_g = _TableInterp.apply(dd_table, d, ctx.period, ctx.order, ctx.order_by)
+        if ctx.needs_input_grad[1] and ctx.order < 3:
+            dd = (g * _TableInterp.apply(dd_table, d, ctx.period, ctx.order + 1, ctx.order_by)).sum(-1)
+        return d_g, dd, None, None, None, None
+
+
+def table_interp(table, d, period):
+    """The grid `table` (rows, cols) of a function of period `period` interpolated at the lengths d (edges):
+    (edges, cols), differentiable in both any number of times."""
+    table, d = table.contiguous(), d.contiguous()
+    return _TableInterp.apply(table, d, period, 0, _SortedLengths(d, table.size(0), period))
 
 
 def painn_filter(msg, r_ij):
@@ -229,7 +281,7 @@ def painn_filter(msg, r_ij):
     if rows and E >= 4 * rows and ops.painn_table_interp_supported(rows, 4 * msg.n):
         table = mlp_silu(msg.mlp_dist, msg._grid_encoding(rows, 0.0, r_ij.device))
         d = torch.linalg.vector_norm(r_ij, dim=-1).contiguous()
-        return _TableInterp.apply(table.contiguous(), d, 2.0 * msg.r0)
+        return table_interp(table, d, 2.0 * msg.r0)
     return mlp_silu(msg.mlp_dist, radial_encode_painn(r_ij, msg.n_rbf, msg.r0))
 
 

@@ -1393,13 +1393,14 @@ def _table_inputs(table, d):
     return int(table.size(0)), int(table.size(1)), int(d.numel())
 
 
-def painn_table_interp_fwd(table, d, period):
+def painn_table_interp_fwd(table, d, period, order=0):
     """(edges, cols): the grid `table` of a function of period `period`, interpolated at the lengths d (4-point
-    Lagrange, as the inference kernels do)."""
+    Lagrange, as the inference kernels do); order 1 .. 3: the interpolant's derivative of that order in d."""
     rows, cols, E = _table_inputs(table, d)
     with torch.cuda.device(d.device):
         out = torch.empty(E, cols, dtype=torch.float32, device=d.device)
-        L.check(_lib.mg_painn_table_interp_fwd(_p(table), rows, cols, float(period), _p(d), E, _p(out), _stream()))
+        L.check(_lib.mg_painn_table_interp_fwd(_p(table), rows, cols, float(period), _p(d), E, int(order), _p(out),
+                                               _stream()))
     return out
 
 
@@ -1415,10 +1416,17 @@ def painn_table_sorted_edges(d, table_rows, period):
     return perm.to(torch.int32).contiguous(), segment_row_ptr(ordered.contiguous(), int(table_rows))
 
 
-def painn_table_interp_bwd(g, table, d, period, perm, bucket_ptr, want_length_grad=True):
-    """(d_table, dd): the gradients of painn_table_interp_fwd's table and lengths for the output gradient g."""
-    rows, cols, E = _table_inputs(table, d)
+def painn_table_interp_bwd(g, table, d, period, perm, bucket_ptr, want_length_grad=True, order=0, table_rows=None):
+    """(d_table, dd): the gradients of painn_table_interp_fwd's table and lengths for the output gradient g.
+    table may be None when only d_table is wanted (table_rows then gives the grid's size)."""
+    _check_input(d, "d")
     _check_input(g, "g")
+    if table is not None:
+        rows, cols, E = _table_inputs(table, d)
+    else:
+        rows, cols, E = int(table_rows), int(g.size(1)), int(d.numel())
+        if want_length_grad:
+            raise RuntimeError("the length gradient needs the table")
     _check_input(perm, "perm", torch.int32)
     _check_input(bucket_ptr, "bucket_ptr", torch.int32)
     if tuple(g.shape) != (E, cols) or perm.numel() != E or bucket_ptr.numel() != rows + 1:
@@ -1427,10 +1435,10 @@ def painn_table_interp_bwd(g, table, d, period, perm, bucket_ptr, want_length_gr
         nbytes = ctypes.c_size_t(0)
         L.check(_lib.mg_painn_table_interp_bwd_workspace_bytes(rows, cols, ctypes.byref(nbytes)))
         ws = torch.empty(nbytes.value, dtype=torch.uint8, device=d.device)
-        d_table = torch.empty_like(table)
+        d_table = torch.empty(rows, cols, dtype=torch.float32, device=d.device)
         dd = torch.empty_like(d) if want_length_grad else None
         L.check(_lib.mg_painn_table_interp_bwd(_p(g), _p(table), rows, cols, float(period), _p(d), _p(perm),
-                                               _p(bucket_ptr), E, _p(ws), _p(d_table), _p(dd), _stream()))
+                                               _p(bucket_ptr), E, int(order), _p(ws), _p(d_table), _p(dd), _stream()))
     return d_table, dd
 
 

@@ -334,6 +334,22 @@ def test_table_interpolation_kernels_against_float64(pkg, ops, rows, cols, E):
     again, _ = ops.painn_table_interp_bwd(w32, tab32, d32, period, perm, bucket_ptr, want_length_grad=False)
     assert torch.equal(again, d_table)
 
+    # the autograd functions over these kernels, recorded: first derivatives again, and a second-order gradient
+    # (derivative orders 1 and 2 of the interpolation weights) against float64
+    tab_g, d_g = tab32.clone().requires_grad_(), d32.clone().requires_grad_()
+    out_g = diff.table_interp(tab_g, d_g, period)
+    g1 = torch.autograd.grad((out_g * w32).sum(), (tab_g, d_g), create_graph=True)
+    _close(g1[0], ref_t, "recorded grid gradient", 2e-5)
+    _close(g1[1], ref_d, "recorded length gradient", 1e-4)
+    ref = diff._table_interp_plain(table, d, period)
+    r1 = torch.autograd.grad((ref * w).sum(), (table, d), create_graph=True)
+    v_t, v_d = torch.randn(rows, cols, generator=g, dtype=F64), torch.randn(E, generator=g, dtype=F64)
+    s_ref = (r1[0] * v_t).sum() + (r1[1] * v_d).sum() + (r1[1] ** 2).sum()
+    s_got = (g1[0] * v_t.float().cuda()).sum() + (g1[1] * v_d.float().cuda()).sum() + (g1[1] ** 2).sum()
+    for a, c, name in zip(torch.autograd.grad(s_got, (tab_g, d_g)), torch.autograd.grad(s_ref, (table, d)),
+                          ("grid", "lengths")):
+        _close(a, c, f"second-order gradient for the {name}", 2e-4)
+
 
 def test_painn_filter_from_its_grid(pkg):
     """The differentiable filter through the grid (Message.table_rows accepts 512 rows for these weights) against the
