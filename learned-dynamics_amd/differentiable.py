@@ -183,7 +183,8 @@ def painn_combine(graph, dist, actv_node, v_node, direction):
 
 
 def _table_interp_plain(table, d, period):
-    """4-point Lagrange interpolation of a periodic grid in tensor arithmetic (differentiable in the grid and in d)."""
+    """4-point Lagrange interpolation of a periodic grid in tensor arithmetic (differentiable in the grid and in d):
+    the formula table_interp's kernels implement, kept as the yardstick its tests differentiate in float64."""
     rows = table.size(0)
     u = d * (float(rows) / period)
     fl = torch.floor(u).detach()
