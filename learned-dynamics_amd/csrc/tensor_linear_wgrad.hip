@@ -267,6 +267,7 @@ constexpr int kFRowW = 64;                         // bytes per LDS row: 32 halv
 constexpr int kFPlane = kFTile * kFRowW;           // bytes of one piece of one operand
 constexpr int kFBuf = 4 * kFPlane;                 // one stage: two operands x two pieces
 constexpr int kFParts = 1024;                      // partial maxima per operand
+constexpr int kFRun = 4096;                        // rows per accumulation run (a multiple of kFRows)
 
 // parts[b] = max |x| over the b-th share of n floats (n % 4 == 0, x 16-byte aligned)
 __global__ void __launch_bounds__(256) absmax_parts_kernel(const float* __restrict__ x, long n,
@@ -428,18 +429,37 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
     store(r_lo, 0);
     fetch(r_lo + kFRows);
     __syncthreads();
-    int buf_off = 0;
-    for (long r = r_lo; r < r_hi; r += kFRows) {
-        multiply(buf_off);
-        buf_off ^= kFBuf;
-        store(r + kFRows, buf_off);
-        fetch(r + 2 * kFRows);
+    // The matrix instructions accumulate runs of kFRun rows; the runs are added in a second set of registers: the
+    // rounding error of an fp32 sum grows with its length, and a slice of 50 000 rows in one chain was 1.7 times
+    // less accurate than the same sum in chunks.
+    floatx16 total[2][2];
 #pragma unroll
-        for (int k = 0; k < 24; k++) {
-            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // one matrix instruction,
-            __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);     // seven vector instructions in its shadow
+    for (int p = 0; p < 2; p++)
+#pragma unroll
+        for (int q = 0; q < 2; q++)
+#pragma unroll
+            for (int k = 0; k < 16; k++) total[p][q][k] = 0.f;
+    int buf_off = 0;
+    for (long r = r_lo; r < r_hi;) {
+        const long run_hi = r + kFRun < r_hi ? r + kFRun : r_hi;
+        for (; r < run_hi; r += kFRows) {
+            multiply(buf_off);
+            buf_off ^= kFBuf;
+            store(r + kFRows, buf_off);
+            fetch(r + 2 * kFRows);
+#pragma unroll
+            for (int k = 0; k < 24; k++) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);     // one matrix instruction,
+                __builtin_amdgcn_sched_group_barrier(0x002, 7, 0);     // seven vector instructions in its shadow
+            }
+            __syncthreads();
         }
-        __syncthreads();
+#pragma unroll
+        for (int p = 0; p < 2; p++)
+#pragma unroll
+            for (int q = 0; q < 2; q++)
+#pragma unroll
+                for (int k = 0; k < 16; k++) { total[p][q][k] += acc[p][q][k]; acc[p][q][k] = 0.f; }
     }
     if (colsum_part != nullptr && blockIdx.y == 0) {                              // (uniform)
         // the four row groups of a column quad, added in a fixed order
@@ -466,7 +486,7 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 #pragma unroll
             for (int k = 0; k < 16; k++) {
                 const int o = o_tile + 4 * (8 * (k / 4) + 4 * g + (k % 4)) + 2 * (wave >> 1) + p;
-                if (o < O && i < I) plane[(long)o * I + i] = acc[p][q][k] * unscale;
+                if (o < O && i < I) plane[(long)o * I + i] = total[p][q][k] * unscale;
             }
         }
 }
