@@ -82,17 +82,25 @@ __global__ void __launch_bounds__(256) segment_sum_kernel(const float* __restric
         const int col = ch.start[c] + (lane & (L - 1)) * VEC;
         const int sub = lane / L, per_iter = kWave / L;
         const long lo = row_ptr[row], hi = row_ptr[row + 1];
-        Acc<VEC> a0, a1;
+        Acc<VEC> a0, a1, a2, a3;
         a0.zero();
         a1.zero();
+        a2.zero();
+        a3.zero();
         long e = lo + sub;
-        for (; e + per_iter < hi; e += 2 * per_iter) {   // two independent loads in flight
+        for (; e + 3 * per_iter < hi; e += 4 * per_iter) {   // four independent loads in flight
             const long r0 = PERM ? perm[e] : e, r1 = PERM ? perm[e + per_iter] : e + per_iter;
+            const long r2 = PERM ? perm[e + 2 * per_iter] : e + 2 * per_iter;
+            const long r3 = PERM ? perm[e + 3 * per_iter] : e + 3 * per_iter;
             a0.add(x + r0 * feat + col);
             a1.add(x + r1 * feat + col);
+            a2.add(x + r2 * feat + col);
+            a3.add(x + r3 * feat + col);
         }
-        if (e < hi) a0.add(x + (PERM ? (long)perm[e] : e) * feat + col);
+        for (; e < hi; e += per_iter) a0.add(x + (PERM ? (long)perm[e] : e) * feat + col);
         a0.merge(a1);
+        a2.merge(a3);
+        a0.merge(a2);
         for (int d = L; d < kWave; d <<= 1) a0.fold(d);
         if (sub == 0) a0.store(out + row * feat + col);
     }
