@@ -395,13 +395,17 @@ int mg_painn_message(const int* row_ptr /* n_nodes+1 */, const int* dst /* E */,
  * edge is its node's), and writes those of the four inputs, all per edge
  * (d_actv (E, 4n), dv (E, n, 3): with an index the caller sums them over the edges of a row).  n: a power of two in
  * 4..256 (mg_painn_combine_supported); arrays contiguous and 16-byte aligned.  The reference evaluates these lines as
- * separate tensor operations. */
+ * separate tensor operations.
+ * terms: 15 for the message.  Bit k keeps the term that contains p[e, k n + c] (bits 0, 1: the terms with v; bits 1, 2:
+ * those with dir).  sum (dm . m + da . a) is linear in dm / da, dist and actv, and in v and dir once restricted to
+ * their terms, so a gradient of a gradient is the same pair of kernels with a cotangent in one argument's place and
+ * that argument's mask: the operations are differentiable any number of times on these two kernels. */
 int mg_painn_combine_supported(int n);   /* returns 0 / 1, not a status */
 int mg_painn_combine_fwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
-                         long n_rows, long E, int n, float* m, float* a, mg_stream_t stream);
+                         long n_rows, long E, int n, int terms, float* m, float* a, mg_stream_t stream);
 int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
                          long n_rows, const float* dm, const float* da, const int* grad_row, long n_grad_rows, long E,
-                         int n, float* d_dist, float* d_actv, float* dv, float* d_dir, mg_stream_t stream);
+                         int n, int terms, float* d_dist, float* d_actv, float* dv, float* d_dir, mg_stream_t stream);
 
 /* The filter from its grid, for training (the grid itself: mg_painn_table_message above).  table (table_rows, cols):
  * the filter at d = k period / table_rows; table_rows and cols powers of two, cols <= 1024.

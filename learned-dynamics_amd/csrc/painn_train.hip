@@ -52,7 +52,8 @@ __global__ void __launch_bounds__(256) painn_combine_fwd_kernel(const float* __r
                                                                 const float* __restrict__ v,
                                                                 const float* __restrict__ dir,
                                                                 const int* __restrict__ node, long n_rows, long E,
-                                                                int n, float* __restrict__ m, float* __restrict__ a) {
+                                                                int n, int terms, float* __restrict__ m,
+                                                                float* __restrict__ a) {
     const int tpe = n >> 2;                                       // threads per edge
     const long t = (long)blockIdx.x * 256 + threadIdx.x;
     const long e = t / tpe;
@@ -66,15 +67,19 @@ __global__ void __launch_bounds__(256) painn_combine_fwd_kernel(const float* __r
     const float4 p2 = mul4(ld4(de + 2 * n), ld4(ae + 2 * n)), p3 = mul4(ld4(de + 3 * n), ld4(ae + 3 * n));
     const Vec3x4 vv = ld12(v + (en * n + c) * 3);
     const Vec3 d = {dir[3 * e], dir[3 * e + 1], dir[3 * e + 2]};
+    // terms (bit k: the term with p[k n + c] takes part): all four for the message itself; subsets when a gradient of
+    // a gradient puts another tensor in the place of v (bits 0, 1: the terms that contain v) or of d (bits 1, 2)
+    const float k0 = (terms & 1) ? 1.f : 0.f, k1 = (terms & 2) ? 1.f : 0.f, k2 = (terms & 4) ? 1.f : 0.f;
+    const float k3 = (terms & 8) ? 1.f : 0.f;
     Vec3x4 out;
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const Vec3 x = vv.get(j), xd = cross(x, d);
-        const float s0 = at(p0, j), s1 = at(p1, j), s2 = at(p2, j);
+        const float s0 = at(p0, j) * k0, s1 = at(p1, j) * k1, s2 = at(p2, j) * k2;
         out.set(j, {x.x * s0 + xd.x * s1 + d.x * s2, x.y * s0 + xd.y * s1 + d.y * s2, x.z * s0 + xd.z * s1 + d.z * s2});
     }
     st12(m + (e * n + c) * 3, out);
-    st4(a + e * n + c, p3);
+    st4(a + e * n + c, make_float4(p3.x * k3, p3.y * k3, p3.z * k3, p3.w * k3));
 }
 
 // Adjoint: with p = dist actv and dp its gradient,
@@ -84,7 +89,7 @@ __global__ void __launch_bounds__(256) painn_combine_fwd_kernel(const float* __r
 __global__ void __launch_bounds__(256) painn_combine_bwd_kernel(
     const float* __restrict__ dist, const float* __restrict__ actv, const float* __restrict__ v,
     const float* __restrict__ dir, const int* __restrict__ node, long n_rows, const float* __restrict__ dm,
-    const float* __restrict__ da, const int* __restrict__ grad_row, long n_grad_rows, long E, int n,
+    const float* __restrict__ da, const int* __restrict__ grad_row, long n_grad_rows, long E, int n, int terms,
     float* __restrict__ d_dist, float* __restrict__ d_actv, float* __restrict__ dv, float* __restrict__ d_dir) {
     const int tpe = n >> 2;                                       // a power of two <= 64
     const long t = (long)blockIdx.x * 256 + threadIdx.x;
@@ -104,16 +109,19 @@ __global__ void __launch_bounds__(256) painn_combine_bwd_kernel(
     const Vec3x4 vv = ld12(v + (en * n + c) * 3), g = ld12(dm + (eg * n + c) * 3);
     const float4 ga = ld4(da + eg * n + c);
     const Vec3 d = {dir[3 * e], dir[3 * e + 1], dir[3 * e + 2]};
+    const float k0 = (terms & 1) ? 1.f : 0.f, k1 = (terms & 2) ? 1.f : 0.f, k2 = (terms & 4) ? 1.f : 0.f;
+    const float k3 = (terms & 8) ? 1.f : 0.f;
     float dp[3][4];
     Vec3x4 gv;
     Vec3 gd = {0.f, 0.f, 0.f};
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const Vec3 x = vv.get(j), gm = g.get(j);
-        const float p0 = at(dk[0], j) * at(ak[0], j), p1 = at(dk[1], j) * at(ak[1], j), p2 = at(dk[2], j) * at(ak[2], j);
-        dp[0][j] = dot(gm, x);
-        dp[1][j] = dot(gm, cross(x, d));
-        dp[2][j] = dot(gm, d);
+        const float p0 = at(dk[0], j) * at(ak[0], j) * k0, p1 = at(dk[1], j) * at(ak[1], j) * k1;
+        const float p2 = at(dk[2], j) * at(ak[2], j) * k2;
+        dp[0][j] = dot(gm, x) * k0;
+        dp[1][j] = dot(gm, cross(x, d)) * k1;
+        dp[2][j] = dot(gm, d) * k2;
         const Vec3 dg = cross(d, gm), gx = cross(gm, x);
         gv.set(j, {gm.x * p0 + dg.x * p1, gm.y * p0 + dg.y * p1, gm.z * p0 + dg.z * p1});
         gd.x += gx.x * p1 + gm.x * p2;
@@ -134,8 +142,9 @@ __global__ void __launch_bounds__(256) painn_combine_bwd_kernel(
         st4(dde + k * n, mul4(gp, ak[k]));
         st4(dae + k * n, mul4(gp, dk[k]));
     }
-    st4(dde + 3 * n, mul4(ga, ak[3]));
-    st4(dae + 3 * n, mul4(ga, dk[3]));
+    const float4 ga3 = make_float4(ga.x * k3, ga.y * k3, ga.z * k3, ga.w * k3);
+    st4(dde + 3 * n, mul4(ga3, ak[3]));
+    st4(dae + 3 * n, mul4(ga3, dk[3]));
     st12(dv + (e * n + c) * 3, gv);
     if (c == 0) { d_dir[3 * e] = gd.x; d_dir[3 * e + 1] = gd.y; d_dir[3 * e + 2] = gd.z; }
 }
@@ -339,8 +348,9 @@ extern "C" {
 int mg_painn_combine_supported(int n) { return combine_shape_ok(n) ? 1 : 0; }
 
 int mg_painn_combine_fwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
-                         long n_rows, long E, int n, float* m, float* a, mg_stream_t stream) {
+                         long n_rows, long E, int n, int terms, float* m, float* a, mg_stream_t stream) {
     MG_REQUIRE(E >= 0 && combine_shape_ok(n), "mg_painn_combine_fwd: n must be a power of two in 4..256");
+    MG_REQUIRE(terms >= 0 && terms <= 15, "mg_painn_combine_fwd: terms is a mask of four bits");
     if (E == 0) return MG_OK;
     MG_REQUIRE(dist && actv && v && dir && m && a, "mg_painn_combine_fwd: null pointer");
     MG_REQUIRE(node == nullptr || n_rows > 0, "mg_painn_combine_fwd: an index needs n_rows > 0");
@@ -349,14 +359,15 @@ int mg_painn_combine_fwd(const float* dist, const float* actv, const float* v, c
     const long threads = E * (n / 4);
     MG_REQUIRE(ceil_div(threads, 256) < (1L << 31), "mg_painn_combine_fwd: too many edges");
     hipLaunchKernelGGL(painn_combine_fwd_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
-                       (hipStream_t)stream, dist, actv, v, dir, node, n_rows, E, n, m, a);
+                       (hipStream_t)stream, dist, actv, v, dir, node, n_rows, E, n, terms, m, a);
     return check_launch("mg_painn_combine_fwd");
 }
 
 int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
                          long n_rows, const float* dm, const float* da, const int* grad_row, long n_grad_rows, long E,
-                         int n, float* d_dist, float* d_actv, float* dv, float* d_dir, mg_stream_t stream) {
+                         int n, int terms, float* d_dist, float* d_actv, float* dv, float* d_dir, mg_stream_t stream) {
     MG_REQUIRE(E >= 0 && combine_shape_ok(n), "mg_painn_combine_bwd: n must be a power of two in 4..256");
+    MG_REQUIRE(terms >= 0 && terms <= 15, "mg_painn_combine_bwd: terms is a mask of four bits");
     if (E == 0) return MG_OK;
     MG_REQUIRE(dist && actv && v && dir && dm && da && d_dist && d_actv && dv && d_dir,
                "mg_painn_combine_bwd: null pointer");
@@ -368,8 +379,8 @@ int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, c
     const long threads = E * (n / 4);
     MG_REQUIRE(ceil_div(threads, 256) < (1L << 31), "mg_painn_combine_bwd: too many edges");
     hipLaunchKernelGGL(painn_combine_bwd_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
-                       (hipStream_t)stream, dist, actv, v, dir, node, n_rows, dm, da, grad_row, n_grad_rows, E, n, d_dist, d_actv, dv,
-                       d_dir);
+                       (hipStream_t)stream, dist, actv, v, dir, node, n_rows, dm, da, grad_row, n_grad_rows, E, n, terms, d_dist,
+                       d_actv, dv, d_dir);
     return check_launch("mg_painn_combine_bwd");
 }
 

@@ -131,39 +131,73 @@ def _painn_combine_plain(dist, actv, v, direction):
     return m, prod[..., 3 * n:]
 
 
+_TERMS_ALL, _TERMS_V, _TERMS_DIR = 15, 3, 6      # the four terms of the message; those that contain v; those with the direction
+
+
+def _sum_opt(parts):
+    parts = [p for p in parts if p is not None]
+    return sum(parts[1:], parts[0]) if parts else None
+
+
 class _PainnCombine(torch.autograd.Function):
-    """The same lines as one kernel, and their gradient as another, with the graph operations on either side folded
-    in: actv and v come per node and the kernels read the destination's row (by_dst); m and a are summed over the
-    edges of their source node (by_src) and the gradient kernel reads the node's gradient row through the source
-    index; the gradients of actv and v are summed over the edges of a destination here.  When the backward pass
-    itself is recorded (create_graph=True, as the Jacobian-vector product of the meanflow loss does), it is evaluated
-    as the gradient of the plain tensor arithmetic instead, which autograd can differentiate again."""
+    """Lines 94-100 of archs/meanflow_painn8.py as one kernel with the graph operations on either side folded in:
+    actv and v come per node and the kernel reads the destination's row (by_dst); m and a are summed over the edges
+    of their source node (by_src).  Returns (out_v (nodes, n, 3), out_a (nodes, n)).  `terms` masks the four terms of
+    the message.  The pairing sum (G_v . out_v + G_a . out_a) is linear in (G_v, G_a), in dist and in actv, and in v
+    and the direction once restricted to the terms that contain them: every derivative of this function and of
+    _PainnCombineGrad is one of the two with a cotangent in one argument's place and that argument's mask, so the
+    pair is closed under differentiation and recorded backward passes run on the same two kernels."""
 
     @staticmethod
-    def forward(ctx, dist, actv_node, v_node, direction, by_dst, by_src):
-        ctx.by_dst, ctx.by_src = by_dst, by_src
+    def forward(ctx, dist, actv_node, v_node, direction, by_dst, by_src, terms):
+        ctx.by_dst, ctx.by_src, ctx.terms = by_dst, by_src, terms
         ctx.save_for_backward(dist, actv_node, v_node, direction)
-        m, a = ops.painn_combine_fwd(dist, actv_node, v_node, direction, node=by_dst.index)
+        m, a = ops.painn_combine_fwd(dist.contiguous(), actv_node.contiguous(), v_node.contiguous(),
+                                     direction.contiguous(), node=by_dst.index, terms=terms)
         return (ops.segment_sum_csr(m, by_src.row_ptr, by_src.n_rows), ops.segment_sum_csr(a, by_src.row_ptr, by_src.n_rows))
 
     @staticmethod
-    def backward(ctx, d_out_v, d_out_a):
-        saved, by_dst, by_src = ctx.saved_tensors, ctx.by_dst, ctx.by_src
-        if torch.is_grad_enabled():
-            with torch.enable_grad():
-                leaves = [t if t.requires_grad else t.detach().requires_grad_() for t in saved]
-                m, a = _painn_combine_plain(leaves[0], gl._Gather.apply(leaves[1], by_dst),
-                                            gl._Gather.apply(leaves[2], by_dst), leaves[3])
-                out = (gl._ScatterSum.apply(m, by_src), gl._ScatterSum.apply(a.contiguous(), by_src))
-                grads = torch.autograd.grad(out, leaves, (d_out_v, d_out_a), create_graph=True)
-            return tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad)) + (None, None)
-        d_dist, d_actv, dv, d_dir = ops.painn_combine_bwd(*saved, d_out_v.contiguous(), d_out_a.contiguous(),
-                                                          node=by_dst.index, grad_row=by_src.index)
+    def backward(ctx, g_v, g_a):
+        grads = _PainnCombineGrad.apply(g_v, g_a, *ctx.saved_tensors, ctx.by_dst, ctx.by_src, ctx.terms)
+        return tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad)) + (None, None, None)
+
+
+class _PainnCombineGrad(torch.autograd.Function):
+    """(g_v, g_a, dist, actv, v, direction) -> the gradients of _PainnCombine's four inputs: d_dist (edges, 4n),
+    d_actv (nodes, 4n), dv (nodes, n, 3), d_direction (edges, 3): one kernel; the gradient rows of an edge's source
+    node are read through the source index, the gradients of actv and v are summed over the edges of a destination."""
+
+    @staticmethod
+    def forward(ctx, g_v, g_a, dist, actv_node, v_node, direction, by_dst, by_src, terms):
+        ctx.by_dst, ctx.by_src, ctx.terms = by_dst, by_src, terms
+        ctx.save_for_backward(g_v, g_a, dist, actv_node, v_node, direction)
+        d_dist, d_actv, dv, d_dir = ops.painn_combine_bwd(
+            dist.contiguous(), actv_node.contiguous(), v_node.contiguous(), direction.contiguous(), g_v.contiguous(),
+            g_a.contiguous(), node=by_dst.index, grad_row=by_src.index, terms=terms)
+        return (d_dist, ops.segment_sum_csr(d_actv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm),
+                ops.segment_sum_csr(dv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm), d_dir)
+
+    @staticmethod
+    def backward(ctx, h_dist, h_actv, h_v, h_dir):
+        g_v, g_a, dist, actv, v, direction = ctx.saved_tensors
+        idx, t = (ctx.by_dst, ctx.by_src), ctx.terms
         need = ctx.needs_input_grad
-        return (d_dist if need[0] else None,
-                ops.segment_sum_csr(d_actv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm) if need[1] else None,
-                ops.segment_sum_csr(dv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm) if need[2] else None,
-                d_dir if need[3] else None, None, None)
+        # one entry per cotangent: the four arguments with the cotangent in its own argument's place, and the mask
+        slots = [(h_dist, (h_dist, actv, v, direction), t), (h_actv, (dist, h_actv, v, direction), t),
+                 (h_v, (dist, actv, h_v, direction), t & _TERMS_V), (h_dir, (dist, actv, v, h_dir), t & _TERMS_DIR)]
+        slots = [(k, args, mask) for k, (h, args, mask) in enumerate(slots) if h is not None]
+        out_g_v = out_g_a = None
+        if need[0] or need[1]:
+            pairs = [_PainnCombine.apply(*args, *idx, mask) for _, args, mask in slots]
+            out_g_v, out_g_a = _sum_opt([p[0] for p in pairs]), _sum_opt([p[1] for p in pairs])
+        grads = [[], [], [], []]
+        if any(need[2:6]):
+            for k, args, mask in slots:
+                outs = _PainnCombineGrad.apply(g_v, g_a, *args, *idx, mask)
+                for j in range(4):
+                    if j != k:                      # (output k of this call is the derivative in the cotangent itself)
+                        grads[j].append(outs[j])
+        return (out_g_v, out_g_a) + tuple(_sum_opt(g) if nd else None for g, nd in zip(grads, need[2:6])) + (None, None, None)
 
 
 def painn_combine(graph, dist, actv_node, v_node, direction):
@@ -173,7 +207,7 @@ def painn_combine(graph, dist, actv_node, v_node, direction):
     actv_flat, v_flat = gl._flat_nodes(graph, actv_node), gl._flat_nodes(graph, v_node)
     if (ops.painn_combine_supported(v_flat.size(1)) and all(t.is_contiguous() and t.data_ptr() % 16 == 0
                                                             for t in (dist, actv_flat, v_flat, direction))):
-        out_v, out_a = _PainnCombine.apply(dist, actv_flat, v_flat, direction, graph.by_dst, graph.by_src)
+        out_v, out_a = _PainnCombine.apply(dist, actv_flat, v_flat, direction, graph.by_dst, graph.by_src, _TERMS_ALL)
     else:
         m, a = _painn_combine_plain(dist, gl._Gather.apply(actv_flat, graph.by_dst),
                                     gl._Gather.apply(v_flat, graph.by_dst), direction)

@@ -1342,20 +1342,21 @@ def _combine_inputs(dist, actv, v, direction, node):
     return E, n, rows
 
 
-def painn_combine_fwd(dist, actv, v, direction, node=None):
+def painn_combine_fwd(dist, actv, v, direction, node=None, terms=15):
     """m = v p[:, :n] + (v x direction) p[:, n:2n] + direction p[:, 2n:3n], a = p[:, 3n:] with p = dist * actv
     (archs/meanflow_painn8.py:94-100), in one pass.  node (int32, one per edge): actv and v hold one row per node and
-    edge e reads row node[e] (the reference's edges_read_dst folded in)."""
+    edge e reads row node[e] (the reference's edges_read_dst folded in).  terms: mask of the four terms that take part
+    (15: all; include/managan_hip.h)."""
     E, n, rows = _combine_inputs(dist, actv, v, direction, node)
     with torch.cuda.device(v.device):
         m = torch.empty(E, n, 3, dtype=torch.float32, device=v.device)
         a = torch.empty(E, n, dtype=torch.float32, device=v.device)
-        L.check(_lib.mg_painn_combine_fwd(_p(dist), _p(actv), _p(v), _p(direction), _p(node), rows, E, n, _p(m), _p(a),
-                                          _stream()))
+        L.check(_lib.mg_painn_combine_fwd(_p(dist), _p(actv), _p(v), _p(direction), _p(node), rows, E, n, int(terms),
+                                          _p(m), _p(a), _stream()))
     return m, a
 
 
-def painn_combine_bwd(dist, actv, v, direction, dm, da, node=None, grad_row=None):
+def painn_combine_bwd(dist, actv, v, direction, dm, da, node=None, grad_row=None, terms=15):
     """Gradients of painn_combine_fwd's four inputs from those of its outputs; those of actv and v per edge
     ((E, 4n), (E, n, 3)) also when the inputs are per node.  grad_row (int32, one per edge): dm and da hold one row per
     node and edge e takes row grad_row[e] (the adjoint of summing m and a over the edges of a source node)."""
@@ -1376,8 +1377,8 @@ def painn_combine_bwd(dist, actv, v, direction, dm, da, node=None, grad_row=None
         dv = torch.empty(E, n, 3, dtype=torch.float32, device=v.device)
         d_dir = torch.empty_like(direction)
         L.check(_lib.mg_painn_combine_bwd(_p(dist), _p(actv), _p(v), _p(direction), _p(node), rows, _p(dm), _p(da),
-                                          _p(grad_row), g_rows, E, n, _p(d_dist), _p(d_actv), _p(dv), _p(d_dir),
-                                          _stream()))
+                                          _p(grad_row), g_rows, E, n, int(terms), _p(d_dist), _p(d_actv), _p(dv),
+                                          _p(d_dir), _stream()))
     return d_dist, d_actv, dv, d_dir
 
 
