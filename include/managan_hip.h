@@ -392,7 +392,7 @@ int mg_painn_message(const int* row_ptr /* n_nodes+1 */, const int* dst /* E */,
  * (the gather by destination folded into the pass; an index outside 0..n_rows-1 is clamped); NULL: row e.
  * mg_painn_combine_bwd takes the gradients dm (E, n, 3), da (E, n), or with grad_row (E ints) dm (n_grad_rows, n, 3),
  * da (n_grad_rows, n) read at row grad_row[e] (m and a were summed over the edges of a source node: the gradient of an
- * edge is its node's), and writes those of the four inputs, all per edge
+ * edge is its node's), and writes those of the four inputs (any of the four output pointers may be NULL), all per edge
  * (d_actv (E, 4n), dv (E, n, 3): with an index the caller sums them over the edges of a row).  n: a power of two in
  * 4..256 (mg_painn_combine_supported); arrays contiguous and 16-byte aligned.  The reference evaluates these lines as
  * separate tensor operations.

@@ -134,19 +134,22 @@ __global__ void __launch_bounds__(256) painn_combine_bwd_kernel(
         gd.z += __shfl_xor(gd.z, s);
     }
     if (!live) return;
-    float* dde = d_dist + e * 4 * n + c;
-    float* dae = d_actv + e * 4 * n + c;
-#pragma unroll
-    for (int k = 0; k < 3; k++) {
-        const float4 gp = make_float4(dp[k][0], dp[k][1], dp[k][2], dp[k][3]);
-        st4(dde + k * n, mul4(gp, ak[k]));
-        st4(dae + k * n, mul4(gp, dk[k]));
-    }
+    // (an output that the caller does not want is a null pointer: uniform branches)
     const float4 ga3 = make_float4(ga.x * k3, ga.y * k3, ga.z * k3, ga.w * k3);
-    st4(dde + 3 * n, mul4(ga3, ak[3]));
-    st4(dae + 3 * n, mul4(ga3, dk[3]));
-    st12(dv + (e * n + c) * 3, gv);
-    if (c == 0) { d_dir[3 * e] = gd.x; d_dir[3 * e + 1] = gd.y; d_dir[3 * e + 2] = gd.z; }
+    if (d_dist) {
+        float* dde = d_dist + e * 4 * n + c;
+#pragma unroll
+        for (int k = 0; k < 3; k++) st4(dde + k * n, mul4(make_float4(dp[k][0], dp[k][1], dp[k][2], dp[k][3]), ak[k]));
+        st4(dde + 3 * n, mul4(ga3, ak[3]));
+    }
+    if (d_actv) {
+        float* dae = d_actv + e * 4 * n + c;
+#pragma unroll
+        for (int k = 0; k < 3; k++) st4(dae + k * n, mul4(make_float4(dp[k][0], dp[k][1], dp[k][2], dp[k][3]), dk[k]));
+        st4(dae + 3 * n, mul4(ga3, dk[3]));
+    }
+    if (dv) st12(dv + (e * n + c) * 3, gv);
+    if (d_dir && c == 0) { d_dir[3 * e] = gd.x; d_dir[3 * e + 1] = gd.y; d_dir[3 * e + 2] = gd.z; }
 }
 
 // ---------------------------------------------------------------------------------------------------------------
@@ -369,13 +372,13 @@ int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, c
     MG_REQUIRE(E >= 0 && combine_shape_ok(n), "mg_painn_combine_bwd: n must be a power of two in 4..256");
     MG_REQUIRE(terms >= 0 && terms <= 15, "mg_painn_combine_bwd: terms is a mask of four bits");
     if (E == 0) return MG_OK;
-    MG_REQUIRE(dist && actv && v && dir && dm && da && d_dist && d_actv && dv && d_dir,
-               "mg_painn_combine_bwd: null pointer");
+    MG_REQUIRE(dist && actv && v && dir && dm && da, "mg_painn_combine_bwd: null pointer");
+    if (!d_dist && !d_actv && !dv && !d_dir) return MG_OK;       // (any of the four outputs may be left out)
     MG_REQUIRE((node == nullptr || n_rows > 0) && (grad_row == nullptr || n_grad_rows > 0),
                "mg_painn_combine_bwd: an index needs a positive row count");
     MG_REQUIRE(aligned16(dist) && aligned16(actv) && aligned16(v) && aligned16(dm) && aligned16(da) &&
                    aligned16(d_dist) && aligned16(d_actv) && aligned16(dv),
-               "mg_painn_combine_bwd: arrays must be 16-byte aligned");
+               "mg_painn_combine_bwd: arrays must be 16-byte aligned");     // (a null pointer counts as aligned)
     const long threads = E * (n / 4);
     MG_REQUIRE(ceil_div(threads, 256) < (1L << 31), "mg_painn_combine_bwd: too many edges");
     hipLaunchKernelGGL(painn_combine_bwd_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,

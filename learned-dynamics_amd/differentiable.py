@@ -158,8 +158,9 @@ class _PainnCombine(torch.autograd.Function):
 
     @staticmethod
     def backward(ctx, g_v, g_a):
-        grads = _PainnCombineGrad.apply(g_v, g_a, *ctx.saved_tensors, ctx.by_dst, ctx.by_src, ctx.terms)
-        return tuple(g if need else None for g, need in zip(grads, ctx.needs_input_grad)) + (None, None, None)
+        want = tuple(ctx.needs_input_grad[:4])
+        grads = _PainnCombineGrad.apply(g_v, g_a, *ctx.saved_tensors, ctx.by_dst, ctx.by_src, ctx.terms, want)
+        return tuple(g if need else None for g, need in zip(grads, want)) + (None, None, None)
 
 
 class _PainnCombineGrad(torch.autograd.Function):
@@ -168,14 +169,23 @@ class _PainnCombineGrad(torch.autograd.Function):
     node are read through the source index, the gradients of actv and v are summed over the edges of a destination."""
 
     @staticmethod
-    def forward(ctx, g_v, g_a, dist, actv_node, v_node, direction, by_dst, by_src, terms):
-        ctx.by_dst, ctx.by_src, ctx.terms = by_dst, by_src, terms
+    def forward(ctx, g_v, g_a, dist, actv_node, v_node, direction, by_dst, by_src, terms, want):
+        """want: which of the four gradients to compute (the others come back as empty tensors)."""
+        ctx.by_dst, ctx.by_src, ctx.terms, ctx.want = by_dst, by_src, terms, want
         ctx.save_for_backward(g_v, g_a, dist, actv_node, v_node, direction)
         d_dist, d_actv, dv, d_dir = ops.painn_combine_bwd(
             dist.contiguous(), actv_node.contiguous(), v_node.contiguous(), direction.contiguous(), g_v.contiguous(),
-            g_a.contiguous(), node=by_dst.index, grad_row=by_src.index, terms=terms)
-        return (d_dist, ops.segment_sum_csr(d_actv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm),
-                ops.segment_sum_csr(dv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm), d_dir)
+            g_a.contiguous(), node=by_dst.index, grad_row=by_src.index, terms=terms, want=want)
+        if want[1]:
+            d_actv = ops.segment_sum_csr(d_actv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm)
+        if want[2]:
+            dv = ops.segment_sum_csr(dv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm)
+        outs = [d_dist, d_actv, dv, d_dir]
+        for k in range(4):
+            if outs[k] is None:
+                outs[k] = dist.new_empty(0)
+                ctx.mark_non_differentiable(outs[k])
+        return tuple(outs)
 
     @staticmethod
     def backward(ctx, h_dist, h_actv, h_v, h_dir):
@@ -185,19 +195,22 @@ class _PainnCombineGrad(torch.autograd.Function):
         # one entry per cotangent: the four arguments with the cotangent in its own argument's place, and the mask
         slots = [(h_dist, (h_dist, actv, v, direction), t), (h_actv, (dist, h_actv, v, direction), t),
                  (h_v, (dist, actv, h_v, direction), t & _TERMS_V), (h_dir, (dist, actv, v, h_dir), t & _TERMS_DIR)]
-        slots = [(k, args, mask) for k, (h, args, mask) in enumerate(slots) if h is not None]
+        slots = [(k, args, mask) for k, (h, args, mask) in enumerate(slots) if h is not None and ctx.want[k]]
         out_g_v = out_g_a = None
         if need[0] or need[1]:
             pairs = [_PainnCombine.apply(*args, *idx, mask) for _, args, mask in slots]
             out_g_v, out_g_a = _sum_opt([p[0] for p in pairs]), _sum_opt([p[1] for p in pairs])
         grads = [[], [], [], []]
-        if any(need[2:6]):
-            for k, args, mask in slots:
-                outs = _PainnCombineGrad.apply(g_v, g_a, *args, *idx, mask)
+        for k, args, mask in slots:
+            # (output k of such a call would be the derivative in the cotangent itself: not wanted)
+            want = tuple(bool(need[2 + j]) and j != k for j in range(4))
+            if any(want):
+                outs = _PainnCombineGrad.apply(g_v, g_a, *args, *idx, mask, want)
                 for j in range(4):
-                    if j != k:                      # (output k of this call is the derivative in the cotangent itself)
+                    if want[j]:
                         grads[j].append(outs[j])
-        return (out_g_v, out_g_a) + tuple(_sum_opt(g) if nd else None for g, nd in zip(grads, need[2:6])) + (None, None, None)
+        return ((out_g_v, out_g_a) + tuple(_sum_opt(g) if nd else None for g, nd in zip(grads, need[2:6]))
+                + (None, None, None, None))
 
 
 def painn_combine(graph, dist, actv_node, v_node, direction):

@@ -1356,7 +1356,7 @@ def painn_combine_fwd(dist, actv, v, direction, node=None, terms=15):
     return m, a
 
 
-def painn_combine_bwd(dist, actv, v, direction, dm, da, node=None, grad_row=None, terms=15):
+def painn_combine_bwd(dist, actv, v, direction, dm, da, node=None, grad_row=None, terms=15, want=(True, True, True, True)):
     """Gradients of painn_combine_fwd's four inputs from those of its outputs; those of actv and v per edge
     ((E, 4n), (E, n, 3)) also when the inputs are per node.  grad_row (int32, one per edge): dm and da hold one row per
     node and edge e takes row grad_row[e] (the adjoint of summing m and a over the edges of a source node)."""
@@ -1372,10 +1372,11 @@ def painn_combine_bwd(dist, actv, v, direction, dm, da, node=None, grad_row=None
     if tuple(dm.shape) != (g_rows, n, 3) or tuple(da.shape) != (g_rows, n):
         raise RuntimeError("expected dm (rows, n, 3) and da (rows, n)")
     with torch.cuda.device(v.device):
-        d_dist = torch.empty_like(dist)
-        d_actv = torch.empty(E, 4 * n, dtype=torch.float32, device=v.device)
-        dv = torch.empty(E, n, 3, dtype=torch.float32, device=v.device)
-        d_dir = torch.empty_like(direction)
+        # (want: which of the four gradients to compute; the others come back as None)
+        d_dist = torch.empty_like(dist) if want[0] else None
+        d_actv = torch.empty(E, 4 * n, dtype=torch.float32, device=v.device) if want[1] else None
+        dv = torch.empty(E, n, 3, dtype=torch.float32, device=v.device) if want[2] else None
+        d_dir = torch.empty_like(direction) if want[3] else None
         L.check(_lib.mg_painn_combine_bwd(_p(dist), _p(actv), _p(v), _p(direction), _p(node), rows, _p(dm), _p(da),
                                           _p(grad_row), g_rows, E, n, int(terms), _p(d_dist), _p(d_actv), _p(dv),
                                           _p(d_dir), _stream()))
