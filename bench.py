@@ -1034,7 +1034,8 @@ def main():
                                       "tensor_products_configs[0]": bench_products(torch, small),
                                       "stress_configs[4]": st,
                                       "meanflow_painn_forward": bench_meanflow_painn(torch, argparse.Namespace(steps=10, warmup=3)),
-                                      "painn_block_training_step": bench_painn_train(torch, argparse.Namespace(steps=5, warmup=2))}
+                                      "painn_block_training_step": bench_painn_train(torch, argparse.Namespace(steps=5, warmup=2)),
+                                      "painn_meanflow_training_step": bench_meanflow_train(torch, argparse.Namespace(steps=3, warmup=1))}
     elif args.workload == "neighbour":
         res = bench_neighbour(torch, args, with_cpu=not args.no_cpu)
     elif args.workload == "denoiser":
