@@ -1033,8 +1033,10 @@ def tensor_linear_wgrad(inds, dy, x, dy_bound=None, x_bound=None, want_bias=Fals
         dW = torch.empty(dim_out, dim_in, dtype=torch.float32, device=x.device)
         db = None
         nbytes = ctypes.c_size_t(0)
-        L.check(_lib.mg_tensor_linear_wgrad_workspace_bytes(rows, dim_in, dim_out, ctypes.byref(nbytes)))
-        ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
+
+        def workspace(n_rows, n_in, n_out):
+            L.check(_lib.mg_tensor_linear_wgrad_workspace_bytes(n_rows, n_in, n_out, ctypes.byref(nbytes)))
+            return torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
         if (inds == 0 and get_linear_mode() == LINEAR_F16X2 and x.data_ptr() % 16 == 0 and dy.data_ptr() % 16 == 0
                 and _lib.mg_tensor_linear_wgrad_f16x2_supported(rows, dim_in, dim_out)):
             for b, name in ((dy_bound, "dy_bound"), (x_bound, "x_bound")):
@@ -1042,6 +1044,7 @@ def tensor_linear_wgrad(inds, dy, x, dy_bound=None, x_bound=None, want_bias=Fals
                     _check_input(b, name)
             if want_bias:
                 db = torch.empty(dim_out, dtype=torch.float32, device=x.device)
+            ws = workspace(rows, dim_in, dim_out)
             L.check(_lib.mg_tensor_linear_wgrad_f16x2(
                 _p(dy), _p(x), _p(dy_bound), 0 if dy_bound is None else dy_bound.numel(),
                 _p(x_bound), 0 if x_bound is None else x_bound.numel(), rows, dim_in, dim_out, _p(ws), _p(dW), _p(db),
@@ -1061,8 +1064,7 @@ def tensor_linear_wgrad(inds, dy, x, dy_bound=None, x_bound=None, want_bias=Fals
                 return out, bound, pad
             dy2, dy2_bound, o_pad = as_rows(dy, dim_out)
             x2, x2_bound, i_pad = as_rows(x, dim_in)
-            L.check(_lib.mg_tensor_linear_wgrad_workspace_bytes(rows * T, i_pad, o_pad, ctypes.byref(nbytes)))
-            ws = torch.empty(nbytes.value, dtype=torch.uint8, device=x.device)
+            ws = workspace(rows * T, i_pad, o_pad)
             dW_pad = dW if (o_pad, i_pad) == (dim_out, dim_in) else torch.empty(o_pad, i_pad, dtype=torch.float32,
                                                                                 device=x.device)
             L.check(_lib.mg_tensor_linear_wgrad_f16x2(_p(dy2), _p(x2), _p(dy2_bound), rows * T, _p(x2_bound), rows * T,
@@ -1070,6 +1072,7 @@ def tensor_linear_wgrad(inds, dy, x, dy_bound=None, x_bound=None, want_bias=Fals
             if dW_pad is not dW:
                 dW = dW_pad[:dim_out, :dim_in].contiguous()
         else:
+            ws = workspace(rows, dim_in, dim_out)
             L.check(_lib.mg_tensor_linear_wgrad(inds, _p(dy), _p(x), rows, dim_in, dim_out, _p(ws), _p(dW), _stream()))
             if want_bias:
                 db = dy.reshape(-1, dim_out).sum(0)
