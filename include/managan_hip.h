@@ -182,6 +182,21 @@ int mg_bee_fwd(const float* l_0, const float* l_1, const float* l_2,
 int mg_bee_bwd(int side, const float* o_0, const float* o_1, const float* o_2,
                const float* const dy[13] /* host array */, long rows, int chan,
                float* d_0, float* d_1, float* d_2, mg_stream_t stream);
+/* The same with operands given per node and read through an index (a gather folded into the kernel; chan a multiple
+ * of 256: mg_bee_indexed_supported).  mg_bee_fwd_indexed: l_* hold l_rows rows and product row e reads row l_index[e]
+ * (Messages: the destination's L0 x_a, L1 x_v, L2 x_d, archs/diffuser_atoms15.py:244-247).  mg_bee_bwd_indexed: the
+ * other side's operands through o_index (or NULL), and the output gradients dy[k] with bit k of dy_indexed set hold
+ * dy_rows rows and are read at row dy_index[e] (products that were summed over the edges of a node: the gradient of an
+ * edge's row is its node's).  Indices outside the operand are clamped.  The reference gathers first
+ * (managan/graph_layers.py:37-52). */
+int mg_bee_indexed_supported(int chan);   /* returns 0 / 1, not a status */
+int mg_bee_fwd_indexed(const float* l_0, const float* l_1, const float* l_2, const int* l_index, long l_rows,
+                       const float* r_0, const float* r_1, const float* r_2, long rows, int chan,
+                       float* const y[13] /* host array */, mg_stream_t stream);
+int mg_bee_bwd_indexed(int side, const float* o_0, const float* o_1, const float* o_2, const int* o_index, long o_rows,
+                       const float* const dy[13] /* host array */, const int* dy_index, long dy_rows,
+                       unsigned dy_indexed, long rows, int chan, float* d_0, float* d_1, float* d_2,
+                       mg_stream_t stream);
 /* cow_o0_fwd_cuda: products 000,110 (codegen_tensops.cpp:1771-1802). */
 int mg_cow_o0_fwd(const float* l_0, const float* l_1, const float* r_0, const float* r_1,
                   long rows, int chan, float* y_000, float* y_110, mg_stream_t stream);

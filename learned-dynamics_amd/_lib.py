@@ -43,6 +43,10 @@ _SIGNATURES = {
     "mg_gather_rows": [vp, vp, i32, i64, i32, i32, vp, vp],
     "mg_bee_fwd": [vp, vp, vp, vp, vp, vp, i64, i32, ctypes.POINTER(PtrArray13), vp],
     "mg_bee_bwd": [i32, vp, vp, vp, ctypes.POINTER(PtrArray13), i64, i32, vp, vp, vp, vp],
+    "mg_bee_indexed_supported": [i32],
+    "mg_bee_fwd_indexed": [vp, vp, vp, vp, i64, vp, vp, vp, i64, i32, ctypes.POINTER(PtrArray13), vp],
+    "mg_bee_bwd_indexed": [i32, vp, vp, vp, vp, i64, ctypes.POINTER(PtrArray13), vp, i64, ctypes.c_uint, i64, i32, vp, vp,
+                           vp, vp],
     "mg_cow_o0_fwd": [vp, vp, vp, vp, i64, i32, vp, vp, vp],
     "mg_cow_o1_fwd": [vp, vp, vp, vp, i64, i32, vp, vp, vp, vp],
     "mg_cow_o0_bwd": [i32, vp, vp, vp, vp, i64, i32, vp, vp, vp],

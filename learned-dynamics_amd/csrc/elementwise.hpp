@@ -66,6 +66,13 @@ struct Args {
     float* out[NOUT];
     unsigned in_vec;   // bit k: operand k is 16-byte aligned
     unsigned out_vec;
+    // Row indirection of inputs (all null / zero: none).  The elements are (row, channel) pairs, `chan` channels per
+    // row, chan a multiple of kTile, so that a workgroup's elements lie in one row; input k with in_index[k] != null
+    // holds in_rows[k] rows and the workgroup's row r reads its row in_index[k][r] (clamped into the operand): a gather
+    // folded into the kernel.
+    const int* in_index[NIN];
+    long in_rows[NIN];
+    int chan;
 };
 
 // span copy HBM -> LDS, `count` floats, both sides unit stride
@@ -116,9 +123,19 @@ __global__ void __launch_bounds__(kTile) kernel(Args<F::NIN, F::NOUT> a, long n)
     float in[pin.off[F::NIN]];
     float out[pout.off[F::NOUT]];
 
+    // first element of this workgroup in input k (another row of the operand when the input is indexed)
+    const long tile_row = a.chan > 0 ? base / a.chan : 0;
+    const long tile_col = a.chan > 0 ? base - tile_row * a.chan : 0;
+    auto in_base = [&](int k) -> long {
+        if (a.in_index[k] == nullptr) return base;
+        long r = a.in_index[k][tile_row];
+        r = r < 0 ? 0 : (r >= a.in_rows[k] ? a.in_rows[k] - 1 : r);
+        return r * a.chan + tile_col;
+    };
+
     static_for<0, F::NIN>([&](auto K) {
         constexpr int k = decltype(K)::value;
-        if constexpr (pin.grp[k] < 0) in[pin.off[k]] = active ? a.in[k][base + tid] : 0.0f;
+        if constexpr (pin.grp[k] < 0) in[pin.off[k]] = active ? a.in[k][in_base(k) + tid] : 0.0f;
     });
     static_for<0, pin.ngroups>([&](auto G) {
         constexpr int g = decltype(G)::value;
@@ -127,7 +144,7 @@ __global__ void __launch_bounds__(kTile) kernel(Args<F::NIN, F::NOUT> a, long n)
             constexpr int k = decltype(K)::value;
             if constexpr (pin.grp[k] == g) {
                 constexpr int T = F::in_T[k];
-                span_to_lds(a.in[k] + base * T, lds + pin.lds_off[k] * kTile, nvalid * T,
+                span_to_lds(a.in[k] + in_base(k) * T, lds + pin.lds_off[k] * kTile, nvalid * T,
                             full && ((a.in_vec >> k) & 1u), tid);
             }
         });

@@ -261,15 +261,26 @@ struct AvdTrio {
     }
 };
 
+// in_index / in_rows (or null): row indirection per input (ew::Args), for `chan` channels per row
 template <class F>
-int launch(const float* const* in, float* const* out, long n, hipStream_t stream, const char* name) {
+int launch(const float* const* in, float* const* out, long n, hipStream_t stream, const char* name,
+           const int* const* in_index = nullptr, const long* in_rows = nullptr, int chan = 0) {
     ew::Args<F::NIN, F::NOUT> a;
     a.in_vec = 0;
     a.out_vec = 0;
+    a.chan = 0;
     for (int k = 0; k < F::NIN; k++) {
         MG_REQUIRE(in[k] != nullptr, "%s: input %d is null", name, k);
         a.in[k] = in[k];
         if (aligned16(in[k])) a.in_vec |= 1u << k;
+        a.in_index[k] = in_index ? in_index[k] : nullptr;
+        a.in_rows[k] = in_index && in_index[k] ? in_rows[k] : 0;
+        if (a.in_index[k]) {
+            MG_REQUIRE(chan > 0 && chan % ew::kTile == 0, "%s: indexed operands need a channel count that is a multiple of %d",
+                       name, ew::kTile);
+            MG_REQUIRE(a.in_rows[k] > 0, "%s: indexed input %d has no rows", name, k);
+            a.chan = chan;
+        }
     }
     for (int k = 0; k < F::NOUT; k++) {
         MG_REQUIRE(out[k] != nullptr, "%s: output %d is null", name, k);
@@ -316,6 +327,43 @@ int mg_bee_bwd(int side, const float* o_0, const float* o_1, const float* o_2,
     float* out[3] = {d_0, d_1, d_2};
     if (side == 0) return launch<BeeBwd<0>>(in, out, rows * chan, (hipStream_t)stream, "mg_bee_bwd(left)");
     return launch<BeeBwd<1>>(in, out, rows * chan, (hipStream_t)stream, "mg_bee_bwd(right)");
+}
+
+int mg_bee_indexed_supported(int chan) { return chan > 0 && chan % ew::kTile == 0; }
+
+int mg_bee_fwd_indexed(const float* l_0, const float* l_1, const float* l_2, const int* l_index, long l_rows,
+                       const float* r_0, const float* r_1, const float* r_2, long rows, int chan, float* const y[13],
+                       mg_stream_t stream) {
+    if (int s = check_sizes(rows, chan, "mg_bee_fwd_indexed")) return s;
+    if (rows == 0 || chan == 0) return MG_OK;
+    MG_REQUIRE(y != nullptr && l_index != nullptr, "mg_bee_fwd_indexed: null pointer");
+    const float* in[6] = {l_0, l_1, l_2, r_0, r_1, r_2};
+    const int* index[6] = {l_index, l_index, l_index, nullptr, nullptr, nullptr};
+    const long n_rows[6] = {l_rows, l_rows, l_rows, 0, 0, 0};
+    return launch<BeeFwd>(in, y, rows * chan, (hipStream_t)stream, "mg_bee_fwd_indexed", index, n_rows, chan);
+}
+
+int mg_bee_bwd_indexed(int side, const float* o_0, const float* o_1, const float* o_2, const int* o_index, long o_rows,
+                       const float* const dy[13], const int* dy_index, long dy_rows, unsigned dy_indexed, long rows,
+                       int chan, float* d_0, float* d_1, float* d_2, mg_stream_t stream) {
+    if (int s = check_sizes(rows, chan, "mg_bee_bwd_indexed")) return s;
+    MG_REQUIRE(side == 0 || side == 1, "mg_bee_bwd_indexed: side must be 0 (left) or 1 (right)");
+    if (rows == 0 || chan == 0) return MG_OK;
+    MG_REQUIRE(dy != nullptr, "mg_bee_bwd_indexed: dy is null");
+    MG_REQUIRE(dy_indexed == 0 || dy_index != nullptr, "mg_bee_bwd_indexed: dy_indexed without an index");
+    const float* in[16] = {o_0, o_1, o_2};
+    const int* index[16] = {o_index, o_index, o_index};
+    long n_rows[16] = {o_rows, o_rows, o_rows};
+    for (int k = 0; k < 13; k++) {
+        in[3 + k] = dy[k];
+        const bool indexed = (dy_indexed >> k) & 1u;
+        index[3 + k] = indexed ? dy_index : nullptr;
+        n_rows[3 + k] = indexed ? dy_rows : 0;
+    }
+    float* out[3] = {d_0, d_1, d_2};
+    hipStream_t st = (hipStream_t)stream;
+    if (side == 0) return launch<BeeBwd<0>>(in, out, rows * chan, st, "mg_bee_bwd_indexed(left)", index, n_rows, chan);
+    return launch<BeeBwd<1>>(in, out, rows * chan, st, "mg_bee_bwd_indexed(right)", index, n_rows, chan);
 }
 
 int mg_cow_o0_fwd(const float* l_0, const float* l_1, const float* r_0, const float* r_1, long rows,

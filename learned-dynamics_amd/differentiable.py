@@ -365,6 +365,64 @@ def apply_tens_prod_submodules(module, prods):
     return tuple(out)
 
 
+def _message_products_plain(a_node, v_node, d_node, phi_a, phi_v, phi_d, by_dst, by_src):
+    """The 13 products of the gathered node operands with the edge filters; those of rank 1 and 2 summed over the
+    edges of their source node (archs/diffuser_atoms15.py:244-252 with the sum moved before the output linears)."""
+    from .ops import BEE_ORDER
+    prods = Bee.apply(gl._Gather.apply(a_node, by_dst), gl._Gather.apply(v_node, by_dst), gl._Gather.apply(d_node, by_dst),
+                      phi_a, phi_v, phi_d)
+    return tuple(p if lab[2] == "0" else gl._ScatterSum.apply(p.contiguous(), by_src) for lab, p in zip(BEE_ORDER, prods))
+
+
+class _MessageProducts(torch.autograd.Function):
+    """The same with the graph operations folded into the product kernels: the node operands are read at the edge's
+    destination through the index, and in the backward pass the gradients of the summed products at the edge's source.
+    Nothing node-sized is copied to the edges.  A recorded backward pass (create_graph=True) differentiates the plain
+    formulation instead."""
+
+    @staticmethod
+    def forward(ctx, a_node, v_node, d_node, phi_a, phi_v, phi_d, by_dst, by_src):
+        from .ops import BEE_ORDER
+        ctx.by_dst, ctx.by_src = by_dst, by_src
+        ctx.save_for_backward(a_node, v_node, d_node, phi_a, phi_v, phi_d)
+        prods = ops.bee_fwd_indexed(a_node, v_node, d_node, by_dst.index, phi_a, phi_v, phi_d)
+        return tuple(p if lab[2] == "0" else ops.segment_sum_csr(p, by_src.row_ptr, by_src.n_rows)
+                     for lab, p in zip(BEE_ORDER, prods))
+
+    @staticmethod
+    def backward(ctx, *dys):
+        saved, by_dst, by_src = ctx.saved_tensors, ctx.by_dst, ctx.by_src
+        need = ctx.needs_input_grad
+        if torch.is_grad_enabled():
+            with torch.enable_grad():
+                leaves = [t if t.requires_grad else t.detach().requires_grad_() for t in saved]
+                out = _message_products_plain(*leaves, by_dst, by_src)
+                grads = torch.autograd.grad(out, leaves, dys, create_graph=True)
+            return tuple(g if nd else None for g, nd in zip(grads, need)) + (None, None)
+        a_node, v_node, d_node, phi_a, phi_v, phi_d = saved
+        dys = [dy.contiguous() for dy in dys]
+        E = phi_a.size(0)
+        d_l = d_r = (None, None, None)
+        if any(need[:3]):
+            per_edge = ops.bee_bwd_indexed(0, phi_a, phi_v, phi_d, None, dys, by_src.index, E)
+            d_l = tuple(ops.segment_sum_csr(t, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm) if nd else None
+                        for t, nd in zip(per_edge, need[:3]))
+        if any(need[3:6]):
+            d_r = tuple(ops.bee_bwd_indexed(1, a_node, v_node, d_node, by_dst.index, dys, by_src.index, E))
+        return (*d_l, *d_r, None, None)
+
+
+def message_products(graph, a_node, v_node, d_node, phi_a, phi_v, phi_d):
+    """a_node (batch, nodes, chan), v_node (.., chan, 3), d_node (.., chan, 3, 3): the node operands, read at each
+    edge's destination; phi_*: the edge filters (edges, chan, ...).  Returns the 13 products in ops.BEE_ORDER: those of
+    rank 0 per edge, those of rank 1 and 2 summed over the edges of their source node ((batch * nodes, chan, ...))."""
+    flat = [gl._flat_nodes(graph, t) for t in (a_node, v_node, d_node)]
+    phis = [t.contiguous() for t in (phi_a, phi_v, phi_d)]
+    if ops.bee_indexed_supported(phi_a.size(1)) and all(t.data_ptr() % 16 == 0 for t in flat + phis):
+        return _MessageProducts.apply(*flat, *phis, graph.by_dst, graph.by_src)
+    return _message_products_plain(*flat, *phis, graph.by_dst, graph.by_src)
+
+
 def bee_messages(msg, graph, r_ij, x_a, x_v, x_d):
     """archs/diffuser_atoms15.py:238-253"""
     enc = linear(msg.lin_enc, radial_encode_8(r_ij, msg.r0))
@@ -372,22 +430,18 @@ def bee_messages(msg, graph, r_ij, x_a, x_v, x_d):
     phi_a = enc
     phi_v = enc[..., None] * rh[..., None, :]
     phi_d = enc[..., None, None] * rh[..., None, None, :] * rh[..., None, :, None]
-    a_j = gl.edges_read_dst(graph, msg.L0(x_a))
-    v_j = gl.edges_read_dst(graph, msg.L1(x_v))
-    d_j = gl.edges_read_dst(graph, msg.L2(x_d))
-    prods = Bee.apply(a_j, v_j, d_j, phi_a.contiguous(), phi_v.contiguous(), phi_d.contiguous())
     # The output linears of the vector and rank-2 channels have no bias and nothing nonlinear follows them before the
     # sum over edges, so they commute with it: the products are summed per node first and the ten linears run on N
     # rows, not E (the reference applies them per edge).  The scalar channel goes through an MLP per edge.
+    prods = message_products(graph, msg.L0(x_a), msg.L1(x_v), msg.L2(x_d), phi_a, phi_v, phi_d)
     from .ops import BEE_ORDER
     psi_a, sums = None, [None, None, None]
     for lab, p in zip(BEE_ORDER, prods):
         k = int(lab[2])
+        y = getattr(msg, f"Y_{lab}")(p if k == 0 else p.reshape(graph.batch, graph.nodes, *p.shape[1:]))
         if k == 0:
-            y = getattr(msg, f"Y_{lab}")(p)
             psi_a = y if psi_a is None else psi_a + y
         else:
-            y = getattr(msg, f"Y_{lab}")(gl.edges_reduce_src(graph, p.contiguous()))
             sums[k] = y if sums[k] is None else sums[k] + y
     psi_a = psi_a + mlp_leaky(msg.mlp_a, psi_a)
     return 0.1 * gl.edges_reduce_src(graph, psi_a), 0.1 * sums[1], 0.1 * sums[2]

@@ -399,6 +399,60 @@ def _bee_bwd(side, o_0, o_1, o_2, dys):
     return d
 
 
+def bee_indexed_supported(chan):
+    return bool(_lib.mg_bee_indexed_supported(int(chan)))
+
+
+def bee_fwd_indexed(l_0, l_1, l_2, l_index, r_0, r_1, r_2):
+    """bee_fwd with the left operands given per node: product row e reads row l_index[e] (int32) of l_*."""
+    n_l, chan = _rows_chan((l_0, l_1, l_2), ("l_0", "l_1", "l_2"))
+    rows, chan2 = _rows_chan((r_0, r_1, r_2), ("r_0", "r_1", "r_2"))
+    _check_input(l_index, "l_index", torch.int32)
+    if chan2 != chan or l_index.numel() != rows:
+        raise RuntimeError("operands must agree on the channel size and l_index must have one entry per row")
+    dev = r_0.device
+    with torch.cuda.device(dev):
+        ys = [torch.empty(_shape(rows, chan, int(lab[2])), dtype=torch.float32, device=dev) for lab in BEE_ORDER]
+        arr = L.PtrArray13(*[y.data_ptr() for y in ys])
+        L.check(_lib.mg_bee_fwd_indexed(_p(l_0), _p(l_1), _p(l_2), _p(l_index), n_l, _p(r_0), _p(r_1), _p(r_2), rows,
+                                        chan, ctypes.byref(arr), _stream()))
+    return ys
+
+
+def bee_bwd_indexed(side, o_0, o_1, o_2, o_index, dys, dy_index, rows):
+    """bee_bwl (side 0) / bee_bwr (side 1) for `rows` product rows, with the other side's operands read through
+    o_index (or None: one row per product row) and every output gradient that does not have `rows` rows read through
+    dy_index (gradients of products that were summed over the edges of a node)."""
+    n_o, chan = _rows_chan((o_0, o_1, o_2), ("x_0", "x_1", "x_2"))
+    if len(dys) != 13:
+        raise RuntimeError("expected 13 output gradients")
+    if o_index is None and n_o != rows:
+        raise RuntimeError("operands without an index need one row per product row")
+    mask, dy_rows = 0, 0
+    for k, (dy, lab) in enumerate(zip(dys, BEE_ORDER)):
+        _check_input(dy, f"dy_{lab}")
+        if tuple(dy.shape[1:]) != _shape(rows, chan, int(lab[2]))[1:]:
+            raise RuntimeError(f"dy_{lab} has wrong shape")
+        if dy.size(0) != rows:
+            if dy_index is None or (dy_rows and dy.size(0) != dy_rows):
+                raise RuntimeError(f"dy_{lab} has {dy.size(0)} rows for {rows} product rows")
+            mask |= 1 << k
+            dy_rows = int(dy.size(0))
+    for idx, name in ((o_index, "o_index"), (dy_index, "dy_index")):
+        if idx is not None:
+            _check_input(idx, name, torch.int32)
+            if idx.numel() != rows:
+                raise RuntimeError(f"{name} must have one entry per product row")
+    dev = o_0.device
+    with torch.cuda.device(dev):
+        d = [torch.empty(_shape(rows, chan, k), dtype=torch.float32, device=dev) for k in range(3)]
+        arr = L.PtrArray13(*[dy.data_ptr() for dy in dys])
+        L.check(_lib.mg_bee_bwd_indexed(side, _p(o_0), _p(o_1), _p(o_2), _p(o_index), n_o, ctypes.byref(arr),
+                                        _p(dy_index), dy_rows, mask, int(rows), chan, _p(d[0]), _p(d[1]), _p(d[2]),
+                                        _stream()))
+    return d
+
+
 def bee_bwl(r_0, r_1, r_2, *dys):
     return _bee_bwd(0, r_0, r_1, r_2, dys)
 
