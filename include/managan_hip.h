@@ -444,6 +444,15 @@ int mg_painn_table_interp_bwd(const float* g, const float* table, int table_rows
                               const int* perm, const int* bucket_ptr, long E, int order, void* workspace,
                               float* d_table, float* dd, mg_stream_t stream);
 
+/* The edge filters of Messages for its training path (archs/diffuser_atoms15.py:240-243): from enc (E, chan) and
+ * rh (E, 3), phi_v[e,c,i] = enc[e,c] rh[e,i] (E, chan, 3) and phi_d[e,c,i,j] = (enc[e,c] rh[e,j]) rh[e,i] (E, chan, 3, 3), and
+ * the adjoint: d_enc (E, chan) and d_rh (E, 3) from the gradients g_v, g_d of the two (sums over channels in a fixed
+ * order).  The reference writes them as broadcasting products. */
+int mg_bee_edge_filters_fwd(const float* enc, const float* rh, long E, int chan, float* phi_v, float* phi_d,
+                            mg_stream_t stream);
+int mg_bee_edge_filters_bwd(const float* enc, const float* rh, const float* g_v, const float* g_d, long E, int chan,
+                            float* d_enc, float* d_rh, mg_stream_t stream);
+
 /* The first two layers of the radial MLP from the edge vectors (archs/meanflow_painn8.py:25-35 feeding :38-51):
  *   y[e] = SiLU(b2 + W2 SiLU(b1 + W1 radial_encode(r_ij[e], 16, rmax))),   y (E, hidden)
  * in one kernel; the first layer's output is produced chunk by chunk on the matrix cores and never stored.

@@ -339,6 +339,68 @@ inline bool table_shape_ok(int rows, int cols) {
     return rows >= 4 && (rows & (rows - 1)) == 0 && cols >= 4 && cols <= 1024 && (cols & (cols - 1)) == 0;
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// The edge filters of the rank-0/1/2 Messages layer (archs/diffuser_atoms15.py:240-243) for its training path:
+//   phi_v[e, c, i] = enc[e, c] rh[e, i],   phi_d[e, c, i, j] = (enc[e, c] rh[e, j]) rh[e, i]
+// and the adjoint: d_enc[e, c] = sum_i g_v[e,c,i] rh[e,i] + sum_ij g_d[e,c,i,j] rh[e,i] rh[e,j],
+//   d_rh[e, k] = sum_c enc[e,c] (g_v[e,c,k] + sum_j (g_d[e,c,k,j] + g_d[e,c,j,k]) rh[e,j]).
+// As broadcasting tensor arithmetic these are two passes forward and a dozen (products and reductions over the
+// broadcast axes) backward over (E, C, 9) arrays.  One workgroup per edge; the channel sum of d_rh is reduced in LDS
+// in a fixed order.
+__global__ void __launch_bounds__(256) edge_filters_fwd_kernel(const float* __restrict__ enc, const float* __restrict__ rh,
+                                                               int C, float* __restrict__ phi_v, float* __restrict__ phi_d) {
+    const long e = blockIdx.x;
+    const float r[3] = {rh[3 * e], rh[3 * e + 1], rh[3 * e + 2]};
+    for (int c = threadIdx.x; c < C; c += 256) {
+        const float v = enc[e * C + c];
+        float* pv = phi_v + (e * C + c) * 3;
+        float* pd = phi_d + (e * C + c) * 9;
+#pragma unroll
+        for (int i = 0; i < 3; i++) pv[i] = v * r[i];
+#pragma unroll
+        for (int i = 0; i < 3; i++)
+#pragma unroll
+            for (int j = 0; j < 3; j++) pd[3 * i + j] = (v * r[j]) * r[i];
+    }
+}
+
+__global__ void __launch_bounds__(256) edge_filters_bwd_kernel(const float* __restrict__ enc, const float* __restrict__ rh,
+                                                               const float* __restrict__ g_v, const float* __restrict__ g_d,
+                                                               int C, float* __restrict__ d_enc, float* __restrict__ d_rh) {
+    __shared__ float part[4][3];
+    const long e = blockIdx.x;
+    const float r[3] = {rh[3 * e], rh[3 * e + 1], rh[3 * e + 2]};
+    float acc[3] = {0.f, 0.f, 0.f};
+    for (int c = threadIdx.x; c < C; c += 256) {
+        const float v = enc[e * C + c];
+        const float* gv = g_v + (e * C + c) * 3;
+        const float* gd = g_d + (e * C + c) * 9;
+        float g9[9], g3[3];
+#pragma unroll
+        for (int k = 0; k < 9; k++) g9[k] = gd[k];
+#pragma unroll
+        for (int k = 0; k < 3; k++) g3[k] = gv[k];
+        float de = 0.f;
+#pragma unroll
+        for (int i = 0; i < 3; i++) {
+            de += g3[i] * r[i];
+            float row = 0.f, sym = 0.f;
+#pragma unroll
+            for (int j = 0; j < 3; j++) { row += g9[3 * i + j] * r[j]; sym += (g9[3 * i + j] + g9[3 * j + i]) * r[j]; }
+            de += row * r[i];
+            acc[i] += v * (g3[i] + sym);
+        }
+        d_enc[e * C + c] = de;
+    }
+#pragma unroll
+    for (int k = 0; k < 3; k++)
+        for (int s = 1; s < 64; s <<= 1) acc[k] += __shfl_xor(acc[k], s);
+    if ((threadIdx.x & 63) == 0)
+        for (int k = 0; k < 3; k++) part[threadIdx.x >> 6][k] = acc[k];
+    __syncthreads();
+    if (threadIdx.x < 3) d_rh[3 * e + threadIdx.x] = (part[0][threadIdx.x] + part[1][threadIdx.x]) + (part[2][threadIdx.x] + part[3][threadIdx.x]);
+}
+
 inline bool combine_shape_ok(int n) { return n >= 4 && n <= 256 && (n & (n - 1)) == 0; }
 
 }  // namespace
@@ -446,6 +508,26 @@ int mg_painn_table_interp_bwd(const float* g, const float* table, int table_rows
                            table_rows - 1, inv_h, order, scale, dd);
     }
     return check_launch("mg_painn_table_interp_bwd");
+}
+
+int mg_bee_edge_filters_fwd(const float* enc, const float* rh, long E, int chan, float* phi_v, float* phi_d,
+                            mg_stream_t stream) {
+    MG_REQUIRE(E >= 0 && chan >= 0 && E < (1L << 31), "mg_bee_edge_filters_fwd: bad size");
+    if (E == 0 || chan == 0) return MG_OK;
+    MG_REQUIRE(enc && rh && phi_v && phi_d, "mg_bee_edge_filters_fwd: null pointer");
+    hipLaunchKernelGGL(edge_filters_fwd_kernel, dim3((unsigned)E), dim3(256), 0, (hipStream_t)stream, enc, rh, chan, phi_v,
+                       phi_d);
+    return check_launch("mg_bee_edge_filters_fwd");
+}
+
+int mg_bee_edge_filters_bwd(const float* enc, const float* rh, const float* g_v, const float* g_d, long E, int chan,
+                            float* d_enc, float* d_rh, mg_stream_t stream) {
+    MG_REQUIRE(E >= 0 && chan >= 0 && E < (1L << 31), "mg_bee_edge_filters_bwd: bad size");
+    if (E == 0) return MG_OK;
+    MG_REQUIRE(rh && d_rh && (chan == 0 || (enc && g_v && g_d && d_enc)), "mg_bee_edge_filters_bwd: null pointer");
+    hipLaunchKernelGGL(edge_filters_bwd_kernel, dim3((unsigned)E), dim3(256), 0, (hipStream_t)stream, enc, rh, g_v, g_d,
+                       chan, d_enc, d_rh);
+    return check_launch("mg_bee_edge_filters_bwd");
 }
 
 }  // extern "C"

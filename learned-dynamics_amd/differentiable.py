@@ -423,13 +423,38 @@ def message_products(graph, a_node, v_node, d_node, phi_a, phi_v, phi_d):
     return _message_products_plain(*flat, *phis, graph.by_dst, graph.by_src)
 
 
+def _edge_filters_plain(enc, rh):
+    """archs/diffuser_atoms15.py:241-243"""
+    return enc[..., None] * rh[..., None, :], enc[..., None, None] * rh[..., None, None, :] * rh[..., None, :, None]
+
+
+class _EdgeFilters(torch.autograd.Function):
+    """phi_v = enc (x) rh and phi_d = enc (x) rh (x) rh as one kernel, and their adjoint as another; a recorded
+    backward pass differentiates the broadcasting arithmetic instead."""
+
+    @staticmethod
+    def forward(ctx, enc, rh):
+        ctx.save_for_backward(enc, rh)
+        return ops.bee_edge_filters_fwd(enc.contiguous(), rh.contiguous())
+
+    @staticmethod
+    def backward(ctx, g_v, g_d):
+        enc, rh = ctx.saved_tensors
+        if torch.is_grad_enabled():
+            with torch.enable_grad():
+                leaves = [t if t.requires_grad else t.detach().requires_grad_() for t in (enc, rh)]
+                grads = torch.autograd.grad(_edge_filters_plain(*leaves), leaves, (g_v, g_d), create_graph=True)
+            return tuple(g if nd else None for g, nd in zip(grads, ctx.needs_input_grad))
+        d_enc, d_rh = ops.bee_edge_filters_bwd(enc.contiguous(), rh.contiguous(), g_v.contiguous(), g_d.contiguous())
+        return (d_enc if ctx.needs_input_grad[0] else None), (d_rh if ctx.needs_input_grad[1] else None)
+
+
 def bee_messages(msg, graph, r_ij, x_a, x_v, x_d):
     """archs/diffuser_atoms15.py:238-253"""
     enc = linear(msg.lin_enc, radial_encode_8(r_ij, msg.r0))
     rh = tens_sigmoid(1, r_ij * (7. / msg.r0))
     phi_a = enc
-    phi_v = enc[..., None] * rh[..., None, :]
-    phi_d = enc[..., None, None] * rh[..., None, None, :] * rh[..., None, :, None]
+    phi_v, phi_d = _EdgeFilters.apply(enc, rh)
     # The output linears of the vector and rank-2 channels have no bias and nothing nonlinear follows them before the
     # sum over edges, so they commute with it: the products are summed per node first and the ten linears run on N
     # rows, not E (the reference applies them per edge).  The scalar channel goes through an MLP per edge.

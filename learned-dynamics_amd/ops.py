@@ -399,6 +399,34 @@ def _bee_bwd(side, o_0, o_1, o_2, dys):
     return d
 
 
+def bee_edge_filters_fwd(enc, rh):
+    """(phi_v, phi_d) = (enc[..., None] * rh[:, None, :], enc[..., None, None] * rh[:, None, None, :] * rh[:, None, :, None])
+    for enc (E, chan) and rh (E, 3) (archs/diffuser_atoms15.py:240-243), one kernel."""
+    _check_input(enc, "enc")
+    _check_input(rh, "rh")
+    E, chan = int(enc.size(0)), int(enc.size(1))
+    if enc.dim() != 2 or tuple(rh.shape) != (E, 3):
+        raise RuntimeError("expected enc (E, chan) and rh (E, 3)")
+    with torch.cuda.device(enc.device):
+        phi_v = torch.empty(E, chan, 3, dtype=torch.float32, device=enc.device)
+        phi_d = torch.empty(E, chan, 3, 3, dtype=torch.float32, device=enc.device)
+        L.check(_lib.mg_bee_edge_filters_fwd(_p(enc), _p(rh), E, chan, _p(phi_v), _p(phi_d), _stream()))
+    return phi_v, phi_d
+
+
+def bee_edge_filters_bwd(enc, rh, g_v, g_d):
+    """(d_enc, d_rh): the adjoint of bee_edge_filters_fwd."""
+    for t, name in ((enc, "enc"), (rh, "rh"), (g_v, "g_v"), (g_d, "g_d")):
+        _check_input(t, name)
+    E, chan = int(enc.size(0)), int(enc.size(1))
+    if tuple(rh.shape) != (E, 3) or tuple(g_v.shape) != (E, chan, 3) or tuple(g_d.shape) != (E, chan, 3, 3):
+        raise RuntimeError("expected rh (E, 3), g_v (E, chan, 3), g_d (E, chan, 3, 3)")
+    with torch.cuda.device(enc.device):
+        d_enc, d_rh = torch.empty_like(enc), torch.empty_like(rh)
+        L.check(_lib.mg_bee_edge_filters_bwd(_p(enc), _p(rh), _p(g_v), _p(g_d), E, chan, _p(d_enc), _p(d_rh), _stream()))
+    return d_enc, d_rh
+
+
 def bee_indexed_supported(chan):
     return bool(_lib.mg_bee_indexed_supported(int(chan)))
 
