@@ -451,3 +451,24 @@ def test_edge_filters_against_broadcasting_arithmetic(pkg, E, C):
         _close(a, c, f"gradient of {name}")
         _close(b, c, f"recorded gradient of {name}")
     assert all(bool(torch.isfinite(t).all()) for t in torch.autograd.grad(sum((t ** 2).sum() for t in g_rec), (enc, rh)))
+
+
+def test_fused_training_functions_on_a_graph_without_edges(pkg):
+    """No edges at all: the folded functions return zero sums and zero gradients for the node operands."""
+    diff = importlib.import_module("learned-dynamics_amd.differentiable")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    N, n, C = 5, 8, 256
+    empty = torch.empty(0, dtype=torch.long).cuda()
+    graph = gl.Graph(empty, empty, None, 1, N)
+    actv = torch.randn(1, N, 4 * n).cuda().requires_grad_()
+    v = torch.randn(1, N, n, 3).cuda().requires_grad_()
+    out_v, out_a = diff.painn_combine(graph, torch.empty(0, 4 * n).cuda(), actv, v, torch.empty(0, 3).cuda())
+    assert tuple(out_v.shape) == (1, N, n, 3) and float(out_v.abs().max()) == 0.0 and float(out_a.abs().max()) == 0.0
+    ga, gv = torch.autograd.grad(out_v.sum() + out_a.sum(), (actv, v))
+    assert float(ga.abs().max()) == 0.0 and float(gv.abs().max()) == 0.0
+    nodes = [torch.randn(1, N, C, *([3] * k)).cuda().requires_grad_() for k in range(3)]
+    phis = [torch.empty(0, C, *([3] * k)).cuda() for k in range(3)]
+    prods = diff.message_products(graph, *nodes, *phis)
+    assert len(prods) == 13 and all(float(p.abs().sum()) == 0.0 for p in prods)
+    grads = torch.autograd.grad(sum(p.sum() for p in prods), nodes, allow_unused=True)
+    assert all(g is None or float(g.abs().max()) == 0.0 for g in grads)
