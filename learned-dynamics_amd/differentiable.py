@@ -365,27 +365,52 @@ def apply_tens_prod_submodules(module, prods):
     return tuple(out)
 
 
-def _message_products_plain(a_node, v_node, d_node, phi_a, phi_v, phi_d, by_dst, by_src):
-    """The 13 products of the gathered node operands with the edge filters; those of rank 1 and 2 summed over the
-    edges of their source node (archs/diffuser_atoms15.py:244-252 with the sum moved before the output linears)."""
+def _message_products_plain(a_node, v_node, d_node, enc, rh, by_dst, by_src):
+    """The 13 products of the gathered node operands with the edge filters (enc, enc (x) rh, enc (x) rh (x) rh); those
+    of rank 1 and 2 summed over the edges of their source node (archs/diffuser_atoms15.py:241-252 with the sum moved
+    before the output linears).  Built from functions that are differentiable any number of times."""
     from .ops import BEE_ORDER
+    phi_v, phi_d = _EdgeFilters.apply(enc, rh)
     prods = Bee.apply(gl._Gather.apply(a_node, by_dst), gl._Gather.apply(v_node, by_dst), gl._Gather.apply(d_node, by_dst),
-                      phi_a, phi_v, phi_d)
+                      enc.contiguous(), phi_v, phi_d)
     return tuple(p if lab[2] == "0" else gl._ScatterSum.apply(p.contiguous(), by_src) for lab, p in zip(BEE_ORDER, prods))
 
 
+_S1_LABELS, _S2_LABELS = ("011", "101", "121", "211", "111"), ("022", "202", "112", "222", "212")
+
+
 class _MessageProducts(torch.autograd.Function):
-    """The same with the graph operations folded into the product kernels: the node operands are read at the edge's
-    destination through the index, and in the backward pass the gradients of the summed products at the edge's source.
-    Nothing node-sized is copied to the edges.  A recorded backward pass (create_graph=True) differentiates the plain
-    formulation instead."""
+    """The same with everything between the node operands and the per-node sums folded into kernels.  Forward: the
+    inference kernel of the layer (mg_bee_message: filters formed in registers, node rows gathered at the destination,
+    products summed over the edges of a node; only the three scalar products are stored per edge) when `enc_source`
+    = (the 8 radial functions, weight and bias of the encoding linear) is given, else the indexed product kernel and
+    segment sums.  Backward: the filters are recomputed, the two gradient kernels read the node operands at the
+    destination and the gradients of the summed products at the source through the indices, and the filters' adjoint
+    folds the three filter gradients into those of enc and rh.  A recorded backward pass (create_graph=True)
+    differentiates the plain formulation instead."""
 
     @staticmethod
-    def forward(ctx, a_node, v_node, d_node, phi_a, phi_v, phi_d, by_dst, by_src):
+    def forward(ctx, a_node, v_node, d_node, enc, rh, by_dst, by_src, enc_source):
         from .ops import BEE_ORDER
         ctx.by_dst, ctx.by_src = by_dst, by_src
-        ctx.save_for_backward(a_node, v_node, d_node, phi_a, phi_v, phi_d)
-        prods = ops.bee_fwd_indexed(a_node, v_node, d_node, by_dst.index, phi_a, phi_v, phi_d)
+        a_node, v_node, d_node, enc, rh = (t.contiguous() for t in (a_node, v_node, d_node, enc, rh))
+        ctx.save_for_backward(a_node, v_node, d_node, enc, rh)
+        N, C = a_node.shape
+        if enc_source is not None:
+            enc8, W, b = enc_source
+            b = b if b is not None else torch.zeros(C, dtype=torch.float32, device=enc.device)
+            P0, S1, S2 = ops.bee_message(by_src.row_ptr, by_dst.index, rh, enc8.contiguous(), a_node,
+                                         v_node.transpose(1, 2).contiguous(),
+                                         d_node.reshape(N, C, 9).transpose(1, 2).contiguous(),
+                                         W.detach().contiguous(), b.detach().contiguous())
+            by_label = {lab: P0[:, k].contiguous() for k, lab in enumerate(("000", "110", "220"))}
+            for k, lab in enumerate(_S1_LABELS):
+                by_label[lab] = S1[:, :, k].transpose(1, 2).contiguous()
+            for k, lab in enumerate(_S2_LABELS):
+                by_label[lab] = S2[:, :, k].transpose(1, 2).contiguous().reshape(N, C, 3, 3)
+            return tuple(by_label[lab] for lab in BEE_ORDER)
+        phi_v, phi_d = ops.bee_edge_filters_fwd(enc, rh)
+        prods = ops.bee_fwd_indexed(a_node, v_node, d_node, by_dst.index, enc, phi_v, phi_d)
         return tuple(p if lab[2] == "0" else ops.segment_sum_csr(p, by_src.row_ptr, by_src.n_rows)
                      for lab, p in zip(BEE_ORDER, prods))
 
@@ -398,29 +423,34 @@ class _MessageProducts(torch.autograd.Function):
                 leaves = [t if t.requires_grad else t.detach().requires_grad_() for t in saved]
                 out = _message_products_plain(*leaves, by_dst, by_src)
                 grads = torch.autograd.grad(out, leaves, dys, create_graph=True)
-            return tuple(g if nd else None for g, nd in zip(grads, need)) + (None, None)
-        a_node, v_node, d_node, phi_a, phi_v, phi_d = saved
+            return tuple(g if nd else None for g, nd in zip(grads, need)) + (None, None, None)
+        a_node, v_node, d_node, enc, rh = saved
         dys = [dy.contiguous() for dy in dys]
-        E = phi_a.size(0)
-        d_l = d_r = (None, None, None)
+        E = enc.size(0)
+        phi_v, phi_d = ops.bee_edge_filters_fwd(enc, rh)
+        d_l = (None, None, None)
+        d_enc = d_rh = None
         if any(need[:3]):
-            per_edge = ops.bee_bwd_indexed(0, phi_a, phi_v, phi_d, None, dys, by_src.index, E)
+            per_edge = ops.bee_bwd_indexed(0, enc, phi_v, phi_d, None, dys, by_src.index, E)
             d_l = tuple(ops.segment_sum_csr(t, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm) if nd else None
                         for t, nd in zip(per_edge, need[:3]))
-        if any(need[3:6]):
-            d_r = tuple(ops.bee_bwd_indexed(1, a_node, v_node, d_node, by_dst.index, dys, by_src.index, E))
-        return (*d_l, *d_r, None, None)
+        if need[3] or need[4]:
+            dr_0, dr_1, dr_2 = ops.bee_bwd_indexed(1, a_node, v_node, d_node, by_dst.index, dys, by_src.index, E)
+            d_enc, d_rh = ops.bee_edge_filters_bwd(enc, rh, dr_1, dr_2)
+            d_enc = d_enc + dr_0
+        return (*d_l, d_enc if need[3] else None, d_rh if need[4] else None, None, None, None)
 
 
-def message_products(graph, a_node, v_node, d_node, phi_a, phi_v, phi_d):
+def message_products(graph, a_node, v_node, d_node, enc, rh, enc_source=None):
     """a_node (batch, nodes, chan), v_node (.., chan, 3), d_node (.., chan, 3, 3): the node operands, read at each
-    edge's destination; phi_*: the edge filters (edges, chan, ...).  Returns the 13 products in ops.BEE_ORDER: those of
-    rank 0 per edge, those of rank 1 and 2 summed over the edges of their source node ((batch * nodes, chan, ...))."""
+    edge's destination; enc (edges, chan), rh (edges, 3): what the edge filters are made of.  Returns the 13 products
+    in ops.BEE_ORDER: those of rank 0 per edge, those of rank 1 and 2 summed over the edges of their source node
+    ((batch * nodes, chan, ...)).  enc_source: see _MessageProducts."""
     flat = [gl._flat_nodes(graph, t) for t in (a_node, v_node, d_node)]
-    phis = [t.contiguous() for t in (phi_a, phi_v, phi_d)]
-    if ops.bee_indexed_supported(phi_a.size(1)) and all(t.data_ptr() % 16 == 0 for t in flat + phis):
-        return _MessageProducts.apply(*flat, *phis, graph.by_dst, graph.by_src)
-    return _message_products_plain(*flat, *phis, graph.by_dst, graph.by_src)
+    enc, rh = enc.contiguous(), rh.contiguous()
+    if ops.bee_indexed_supported(enc.size(1)) and all(t.data_ptr() % 16 == 0 for t in flat + [enc]):
+        return _MessageProducts.apply(*flat, enc, rh, graph.by_dst, graph.by_src, enc_source)
+    return _message_products_plain(*flat, enc, rh, graph.by_dst, graph.by_src)
 
 
 def _edge_filters_plain(enc, rh):
@@ -451,14 +481,14 @@ class _EdgeFilters(torch.autograd.Function):
 
 def bee_messages(msg, graph, r_ij, x_a, x_v, x_d):
     """archs/diffuser_atoms15.py:238-253"""
-    enc = linear(msg.lin_enc, radial_encode_8(r_ij, msg.r0))
+    enc8 = radial_encode_8(r_ij, msg.r0)
+    enc = linear(msg.lin_enc, enc8)
     rh = tens_sigmoid(1, r_ij * (7. / msg.r0))
-    phi_a = enc
-    phi_v, phi_d = _EdgeFilters.apply(enc, rh)
     # The output linears of the vector and rank-2 channels have no bias and nothing nonlinear follows them before the
     # sum over edges, so they commute with it: the products are summed per node first and the ten linears run on N
     # rows, not E (the reference applies them per edge).  The scalar channel goes through an MLP per edge.
-    prods = message_products(graph, msg.L0(x_a), msg.L1(x_v), msg.L2(x_d), phi_a, phi_v, phi_d)
+    prods = message_products(graph, msg.L0(x_a), msg.L1(x_v), msg.L2(x_d), enc, rh,
+                             enc_source=(enc8.detach(), msg.lin_enc.weight, msg.lin_enc.bias))
     from .ops import BEE_ORDER
     psi_a, sums = None, [None, None, None]
     for lab, p in zip(BEE_ORDER, prods):
