@@ -334,7 +334,9 @@ __global__ void __launch_bounds__(256) table_interp_grad_length_kernel(const flo
     }
 }
 
-constexpr int kTableSplits = 16;
+// pieces per grid row: 16 for 512 rows, fewer for finer grids (whose rows hold fewer edges): the partial sums stay
+// within 64 MB for 512 columns
+inline int table_splits(int rows) { const int s = 8192 / rows; return s < 1 ? 1 : (s > 16 ? 16 : s); }
 inline bool table_shape_ok(int rows, int cols) {
     return rows >= 4 && (rows & (rows - 1)) == 0 && cols >= 4 && cols <= 1024 && (cols & (cols - 1)) == 0;
 }
@@ -479,7 +481,7 @@ int mg_painn_table_buckets(const float* d, long E, int table_rows, float period,
 
 int mg_painn_table_interp_bwd_workspace_bytes(int table_rows, int cols, size_t* bytes) {
     MG_REQUIRE(bytes != nullptr && table_shape_ok(table_rows, cols), "mg_painn_table_interp_bwd_workspace_bytes: bad argument");
-    *bytes = (size_t)table_rows * kTableSplits * 4 * (size_t)cols * sizeof(float) + 16;
+    *bytes = (size_t)table_rows * table_splits(table_rows) * 4 * (size_t)cols * sizeof(float) + 16;
     return MG_OK;
 }
 
@@ -495,11 +497,12 @@ int mg_painn_table_interp_bwd(const float* g, const float* table, int table_rows
     const float inv_h = (float)table_rows / period;
     float* part = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(workspace) + 15) & ~uintptr_t(15));
     const float scale = int_power(inv_h, order);
-    hipLaunchKernelGGL(table_scatter_kernel, dim3((unsigned)table_rows, kTableSplits), dim3(256), 0, st, g, d, perm,
-                       bucket_ptr, cols, inv_h, order, scale, kTableSplits, part);
+    const int splits = table_splits(table_rows);
+    hipLaunchKernelGGL(table_scatter_kernel, dim3((unsigned)table_rows, (unsigned)splits), dim3(256), 0, st, g, d, perm,
+                       bucket_ptr, cols, inv_h, order, scale, splits, part);
     const long threads = (long)table_rows * (cols / 4);
     hipLaunchKernelGGL(table_scatter_finish_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0, st,
-                       (const float*)part, table_rows, cols, kTableSplits, d_table);
+                       (const float*)part, table_rows, cols, splits, d_table);
     if (dd && E > 0) {
         MG_REQUIRE(table && aligned16(table), "mg_painn_table_interp_bwd: the length gradient needs the table");
         long blocks = ceil_div(E, 4);

@@ -323,9 +323,17 @@ def painn_filter(msg, r_ij):
     """mlp_dist(radial_encode(r_ij)) (archs/meanflow_painn8.py:92), (edges, 4n).  The filter is a smooth periodic
     function of the edge length: when the module's grid test accepts a grid for the current weights (the test the
     inference path uses, Message.table_rows) the MLP runs on the grid's rows and every edge interpolates, so that the
-    backward pass differentiates the MLP on a few hundred rows instead of on every edge."""
+    backward pass differentiates the MLP on a few hundred rows instead of on every edge.  Only when the edge vectors
+    need no gradient (see below)."""
     E = r_ij.shape[0]
     rows = msg.table_rows() if (getattr(msg, "use_table", False) and E >= 4 * msg.TABLE_ROWS[0]) else 0
+    if r_ij.requires_grad:
+        # The gradient for the edge vectors would go through the interpolant's derivative: differences of neighbouring
+        # grid rows divided by the spacing, which amplifies the fp32-level noise of the grid values (1e-6 of their size
+        # from the GEMMs that evaluate them) by rows / period: 4e-5 of the largest gradient entry at 2048 rows, 2e-4 at
+        # 512 (where the interpolation error of the derivative dominates), against 7e-7 for the MLP on every edge.
+        # Positions that are differentiated (the meanflow loss, blocks that move them) keep the per-edge MLP.
+        rows = 0
     if rows and E >= 4 * rows and ops.painn_table_interp_supported(rows, 4 * msg.n):
         table = mlp_silu(msg.mlp_dist, msg._grid_encoding(rows, 0.0, r_ij.device))
         d = torch.linalg.vector_norm(r_ij, dim=-1).contiguous()

@@ -353,8 +353,10 @@ def test_table_interpolation_kernels_against_float64(pkg, ops, rows, cols, E):
 
 def test_painn_filter_from_its_grid(pkg):
     """The differentiable filter through the grid (Message.table_rows accepts 512 rows for these weights) against the
-    filter MLP on every edge (archs/meanflow_painn8.py:92): values, gradients for the MLP's parameters and for the
-    edge vectors, the recorded backward pass, and a second-order gradient."""
+    filter MLP on every edge (archs/meanflow_painn8.py:92): values, gradients for the MLP's parameters, the recorded
+    backward pass and a second-order gradient.  Edge vectors that require a gradient keep the MLP on every edge (the
+    interpolant's derivative amplifies the rounding noise of the grid values); the grid functions' own length
+    gradient is tested against float64 in test_table_interpolation_kernels_against_float64."""
     diff = importlib.import_module("learned-dynamics_amd.differentiable")
     painn = importlib.import_module("learned-dynamics_amd.painn")
     torch.manual_seed(0x947 + 12)
@@ -362,29 +364,31 @@ def test_painn_filter_from_its_grid(pkg):
     g = torch.Generator().manual_seed(3)
     E = 6000
     u = torch.randn(E, 3, generator=g)
-    r_ij = (u / u.norm(dim=-1, keepdim=True) * (0.4 + 4.6 * torch.rand(E, 1, generator=g))).cuda().requires_grad_()
+    r_ij = (u / u.norm(dim=-1, keepdim=True) * (0.4 + 4.6 * torch.rand(E, 1, generator=g))).cuda()
     w = torch.randn(E, 4 * msg.n, generator=g).cuda()
     params = list(msg.mlp_dist.parameters())
     assert msg.table_rows() == 512
 
+    f_moving = diff.painn_filter(msg, r_ij.clone().requires_grad_())
+    assert not type(f_moving.grad_fn).__name__.startswith("_TableInterp")
     f_grid = diff.painn_filter(msg, r_ij)
     assert type(f_grid.grad_fn).__name__.startswith("_TableInterp")
     msg.use_table = False
     try:
         f_edge = diff.painn_filter(msg, r_ij)
-        g_edge = torch.autograd.grad((f_edge * w).sum(), params + [r_ij])
+        g_edge = torch.autograd.grad((f_edge * w).sum(), params)
     finally:
         msg.use_table = True
     scale = float(f_edge.abs().max())
     assert float((f_grid - f_edge).abs().max()) <= 1e-5 * scale
-    g_grid = torch.autograd.grad((f_grid * w).sum(), params + [r_ij], retain_graph=True)
-    g_rec = torch.autograd.grad((f_grid * w).sum(), params + [r_ij], create_graph=True)
-    for a, b, c, p in zip(g_grid, g_rec, g_edge, params + [r_ij]):
+    assert torch.equal(f_moving.detach(), f_edge.detach())
+    g_grid = torch.autograd.grad((f_grid * w).sum(), params, retain_graph=True)
+    g_rec = torch.autograd.grad((f_grid * w).sum(), params, create_graph=True)
+    for a, b, c, p in zip(g_grid, g_rec, g_edge, params):
         s = float(c.abs().max())
-        tol = 2e-4 if p is r_ij else 2e-5          # (the interpolant's derivative is one order less accurate)
-        assert float((a - c).abs().max()) <= tol * s, (tuple(p.shape), float((a - c).abs().max()), s)
+        assert float((a - c).abs().max()) <= 2e-5 * s, (tuple(p.shape), float((a - c).abs().max()), s)
         assert float((b - a).abs().max()) <= 2e-5 * s
-    second = torch.autograd.grad(sum((t ** 2).sum() for t in g_rec), params + [r_ij], allow_unused=True)
+    second = torch.autograd.grad(sum((t ** 2).sum() for t in g_rec), params, allow_unused=True)
     assert all(t is None or bool(torch.isfinite(t).all()) for t in second)
 
 
