@@ -332,7 +332,9 @@ def painn_filter(msg, r_ij):
         # grid rows divided by the spacing, which amplifies the fp32-level noise of the grid values (1e-6 of their size
         # from the GEMMs that evaluate them) by rows / period: 4e-5 of the largest gradient entry at 2048 rows, 2e-4 at
         # 512 (where the interpolation error of the derivative dominates), against 7e-7 for the MLP on every edge.
-        # Positions that are differentiated (the meanflow loss, blocks that move them) keep the per-edge MLP.
+        # A grid evaluated in float64 does not help (3e-5 at 2048 rows): the float32 differences themselves cancel
+        # that many digits.  Positions that are differentiated (the meanflow loss, blocks that move them) keep the
+        # per-edge MLP.
         rows = 0
     if rows and E >= 4 * rows and ops.painn_table_interp_supported(rows, 4 * msg.n):
         table = mlp_silu(msg.mlp_dist, msg._grid_encoding(rows, 0.0, r_ij.device))
