@@ -827,10 +827,13 @@ _packed_cache = {}
 def _packed(W, kind):
     """Pre-split planes of W for the packed GEMM entry points.  Cached per tensor OBJECT (weak
     reference) and version counter, so parameters are packed once and re-packed after an in-place
-    update; a new tensor that happens to reuse a freed address never hits a stale entry."""
-    key = (id(W), kind)
+    update; a new tensor that happens to reuse a freed address never hits a stale entry.  A view
+    (the transposed weight of every input-gradient GEMM is a fresh view object of the parameter) is
+    cached under the tensor it is a view of, with its offset, shape and strides."""
+    owner = W._base if W._base is not None else W
+    key = (id(owner), kind, int(W.storage_offset()), tuple(W.shape), tuple(W.stride()))
     hit = _packed_cache.get(key)
-    if hit is not None and hit[0]() is W and hit[1] == W._version and hit[2] == (W.data_ptr(), tuple(W.stride())):
+    if hit is not None and hit[0]() is owner and hit[1] == owner._version and hit[2] == owner.data_ptr():
         return hit[3]
     dim_out, dim_in = int(W.size(0)), int(W.size(1))
     nbytes = ctypes.c_size_t(0)
@@ -840,12 +843,12 @@ def _packed(W, kind):
     with torch.cuda.device(W.device):
         packed = torch.empty(nbytes.value, dtype=torch.uint8, device=W.device)
         L.check(pack_fn(_p(W), int(W.stride(0)), int(W.stride(1)), dim_in, dim_out, _p(packed), _stream()))
-    if len(_packed_cache) > 512:
+    if len(_packed_cache) > 4096:
         for k in [k for k, v in _packed_cache.items() if v[0]() is None]:
             del _packed_cache[k]
-        if len(_packed_cache) > 512:
+        if len(_packed_cache) > 4096:
             _packed_cache.clear()
-    _packed_cache[key] = (weakref.ref(W), W._version, (W.data_ptr(), tuple(W.stride())), packed)
+    _packed_cache[key] = (weakref.ref(owner), owner._version, owner.data_ptr(), packed)
     return packed
 
 
