@@ -72,17 +72,17 @@ def _cat_Y(module, labels, scale=None):
     return _derived(module, ("cat_Y", labels, scale), params, make)
 
 
-def _linear(x, W, bias, act, bound, out=None, accumulate=False):
+def _linear(x, W, bias, act, bound, out=None, accumulate=False, want_bound=True):
     """Plain-row linear with fused bias / activation.  With the split-fp16 matrix path active and
     a row bound of |x| at hand, the bound is used (no pass over x) and the bound of the output rows
-    is returned with y; otherwise (y, None)."""
+    is returned with y; otherwise (y, None).  want_bound=False: the output feeds no GEMM, no bound is formed."""
     rows, dim_in, dim_out = x.shape[0], W.shape[1], W.shape[0]
     if (bound is not None and ops.get_linear_mode() == ops.LINEAR_F16X2
             and ops.f16x2_supported(rows, dim_in, dim_out, x)):
         y = ops.tensor_linear_f16x2(W, x, bound, bias=bias, act=act, out=out, accumulate=accumulate)
     else:
         y = ops.tensor_linear_fwd(0, W, x, bias=bias, act=act, out=out, accumulate=accumulate)
-    return y, (ops.linear_out_bound(W, bias, bound) if bound is not None and not accumulate else None)
+    return y, (ops.linear_out_bound(W, bias, bound) if bound is not None and want_bound and not accumulate else None)
 
 
 class TensGroupNorm(nn.Module):
@@ -206,7 +206,7 @@ class MLP(nn.Module):
         L = self.layers
         if bound is None and ops.get_linear_mode() == ops.LINEAR_F16X2:
             bound = ops.row_absmax(x2)
-        out, _ = _linear(x2, Wd, None, ops.ACT_NONE, bound)
+        out, _ = _linear(x2, Wd, None, ops.ACT_NONE, bound, want_bound=False)
         h, b1 = _linear(x2, L[0].weight, L[0].bias, ops.ACT_LEAKY, bound)
         h, b2 = _linear(h, L[2].weight, L[2].bias, ops.ACT_LEAKY, b1)
         _linear(h, L[4].weight, L[4].bias, ops.ACT_NONE, b2, out=out, accumulate=True)
@@ -234,7 +234,7 @@ class MLP(nn.Module):
             s_h, _ = ops.tensor_linear_f16x2_rowsum(L[2].weight, h, b1, row_ptr, seg, n_out, bias=L[2].bias,
                                                     act=ops.ACT_LEAKY)
         else:
-            h, _ = _linear(h, L[2].weight, L[2].bias, ops.ACT_LEAKY, b1)
+            h, _ = _linear(h, L[2].weight, L[2].bias, ops.ACT_LEAKY, b1, want_bound=False)
             s_h = ops.segment_sum_csr(h, row_ptr, n_out)
         del h
         if s_x is None:

@@ -844,18 +844,17 @@ def _packed(W, kind):
         packed = torch.empty(nbytes.value, dtype=torch.uint8, device=W.device)
         L.check(pack_fn(_p(W), int(W.stride(0)), int(W.stride(1)), dim_in, dim_out, _p(packed), _stream()))
     if len(_packed_cache) > 4096:
-        for k in [k for k, v in _packed_cache.items() if v[0]() is None]:
-            del _packed_cache[k]
-        if len(_packed_cache) > 4096:
-            _packed_cache.clear()
-    _packed_cache[key] = (weakref.ref(owner), owner._version, owner.data_ptr(), packed)
+        _packed_cache.clear()
+    # the entry (and the device memory of its planes) goes when the tensor it was packed from does
+    _packed_cache[key] = (weakref.ref(owner, lambda _, key=key: _packed_cache.pop(key, None)),
+                          owner._version, owner.data_ptr(), packed)
     return packed
 
 
 _padded_cache = {}
 
 
-def _zero_padded_columns(W, k_pad):
+def zero_padded_columns(W, k_pad):
     """W (dim_out, dim_in) with zero columns appended up to k_pad; cached per parameter object and version."""
     if int(W.size(1)) == k_pad:
         return W
@@ -1072,7 +1071,7 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
                 xt = torch.nn.functional.pad(xt, (0, k_pad - dim_in)) if k_pad != dim_in else xt.contiguous()
                 x2 = xt.reshape(rows * T, k_pad)
                 x2max = row_absmax(x2)
-            Wp = _zero_padded_columns(W, k_pad)
+            Wp = zero_padded_columns(W, k_pad)
             ymax = rowmax_buffer(k_pad)
             L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(Wp)), _p(x2), _p(x2max), 1, 1, 1,
                                                 rows * T, k_pad, dim_out, _p(bias), int(act), int(bool(accumulate)),

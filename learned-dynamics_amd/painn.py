@@ -40,9 +40,10 @@ def radial_encode(r, n, rmax):
     return ops.painn_radial_encode(r.reshape(-1, 3).contiguous(), n, rmax).reshape(*lead, n)
 
 
-def _linear(x, lin, act, bound=None):
+def _linear(x, lin, act, bound=None, want_bound=True):
     """One nn.Linear with fused bias and activation.  bound: upper bounds of the row maxima of |x|
-    ((rows, 1) or (1, 1)) if the caller knows them.  Returns (y, bound of the rows of |y| or None)."""
+    ((rows, 1) or (1, 1)) if the caller knows them.  Returns (y, bound of the rows of |y| or None);
+    want_bound=False leaves the second out (a last layer, whose output feeds no GEMM)."""
     rows = x.shape[0]
     if ops.get_linear_mode() == ops.LINEAR_F16X2 and ops.f16x2_supported(rows, lin.in_features, lin.out_features, x):
         if bound is None:
@@ -50,7 +51,7 @@ def _linear(x, lin, act, bound=None):
         y = ops.tensor_linear_f16x2(lin.weight, x, bound, bias=lin.bias, act=act)
     else:
         y = ops.tensor_linear_fwd(0, lin.weight, x, bias=lin.bias, act=act)
-    return y, (ops.linear_out_bound(lin.weight, lin.bias, bound) if bound is not None else None)
+    return y, (ops.linear_out_bound(lin.weight, lin.bias, bound) if bound is not None and want_bound else None)
 
 
 class MLP(nn.Module):
@@ -85,7 +86,7 @@ class MLP(nn.Module):
     def after_first(self, h, bound=None):
         """Layers 2 and 3 on the (rows, dim_out) output of the first layer + SiLU."""
         h, bound = _linear(h, self.layers[2], ops.ACT_SILU, bound)
-        return _linear(h, self.layers[4], ops.ACT_NONE, bound)[0]
+        return _linear(h, self.layers[4], ops.ACT_NONE, bound, want_bound=False)[0]
 
 
 class ScalGroupNorm(nn.Module):
@@ -158,6 +159,8 @@ class Message(nn.Module):
         self.mlp_dist = MLP(self.n_rbf, 4 * n)
         self.mlp_actv = MLP(n, 4 * n)
 
+    GRID_K = 64          # reduction dimension of the grid's first layer after padding
+
     def _hidden(self, r_ij):
         """Radial encoding + first layer + SiLU of the filter MLP: (edges, 4n) and the bound of its rows."""
         first = self.mlp_dist.layers[0]
@@ -209,10 +212,17 @@ class Message(nn.Module):
     TABLE_TOL = 3e-6            # of max |filter|: the level of the split-fp16 GEMMs that evaluate the filter itself
     use_table = True
 
-    def _grid_encoding(self, rows, shift, device):
+    def _grid_encoding(self, rows, shift, device, width=None):
         """radial_encode at the lengths (k + shift) 2 r0 / rows, k = 0 .. rows - 1: (rows, n_rbf).  The lengths are
-        known exactly, so the phases are formed in float64 and only the encodings are rounded to float32."""
+        known exactly, so the phases are formed in float64 and only the encodings are rounded to float32.
+        width: zero columns appended up to this many (a reduction dimension the matrix path accepts)."""
         cache = self.__dict__.setdefault("_grid_cache", {})
+        if width is not None and width > self.n_rbf:
+            key = (rows, shift, str(device), width)
+            if key not in cache:
+                enc = self._grid_encoding(rows, shift, device)
+                cache[key] = torch.nn.functional.pad(enc, (0, width - self.n_rbf)).contiguous()
+            return cache[key]
         key = (rows, shift, str(device))
         if key not in cache:
             n = self.n_rbf
@@ -225,8 +235,18 @@ class Message(nn.Module):
 
     def filter_table(self, rows, shift=0.0):
         """The filter at d = (k + shift) 2 r0 / rows, k = 0 .. rows - 1: (rows, 4n)."""
-        enc = self._grid_encoding(rows, shift, self.mlp_dist.layers[0].weight.device)
-        return self.mlp_dist(enc, ops.linear_in_unit_bound(enc.device))
+        first = self.mlp_dist.layers[0]
+        device = first.weight.device
+        unit = ops.linear_in_unit_bound(device)
+        if (self.n_rbf < self.GRID_K and ops.get_linear_mode() == ops.LINEAR_F16X2 and not diff.wants_grad(self.mlp_dist)
+                and ops.f16x2_supported(rows, self.GRID_K, first.out_features, first.weight)):
+            # a reduction dimension of n_rbf is below what the matrix path takes: the encodings (constants of the
+            # grid) and the weight's columns are padded with zeros, which leaves every product as it was
+            enc = self._grid_encoding(rows, shift, device, self.GRID_K)
+            h = ops.tensor_linear_f16x2(ops.zero_padded_columns(first.weight, self.GRID_K), enc, unit,
+                                        bias=first.bias, act=ops.ACT_SILU)
+            return self.mlp_dist.after_first(h, ops.linear_out_bound(first.weight, first.bias, unit))
+        return self.mlp_dist(self._grid_encoding(rows, shift, device), unit)
 
     def table_rows(self):
         """Rows of the grid whose interpolation error is below TABLE_TOL for the current weights, or 0 if none of
@@ -264,7 +284,7 @@ class Message(nn.Module):
             if rows and rows <= ops.PAINN_SLICED_MAX_ROWS and n % ops.PAINN_SLICE == 0 and self.use_sliced:
                 # the grid fits in LDS: actv comes out of its MLP with the columns regrouped slice by slice
                 h_a, b_a = self.mlp_actv.hidden(flat_a)
-                actv_s = _linear(h_a, self._sliced_actv_last(), ops.ACT_NONE, b_a)[0]
+                actv_s = _linear(h_a, self._sliced_actv_last(), ops.ACT_NONE, b_a, want_bound=False)[0]
                 # rows in cell order when the graph has one: consecutive rows then gather the same neighbours
                 order = getattr(graph, "cell_order", None) if self.use_cell_order else None
                 out_a, out_v = ops.painn_table_message_sliced(graph.row_ptr, graph.dst32, r_ij, self.filter_table(rows),
