@@ -45,15 +45,28 @@ __global__ void __launch_bounds__(256) group_stats_kernel(const float* __restric
     const float* mul_g = mul ? mul + (long)g * cg * T : nullptr;
     const long x_row = x_stride * T, m_row = mul_stride * T;
     double s = 0.0, ss = 0.0;
+    // four trips' loads are requested before the first is used (a trip alone waits out the memory latency); a trip
+    // past the end re-reads the chunk's last node and counts as zero
+    constexpr int kAhead = 4;
     while (i < n_hi) {
-        const long row = (long)b * N + i;
-        float v = xg[row * x_row + r];
-        if (mul_g) v *= mul_g[row * m_row + r];
-        s += v;
-        ss += (double)v * v;
-        i += step_i;
-        r += step_r;
-        if (r >= run) { r -= run; i++; }
+        float v[kAhead], m[kAhead];
+#pragma unroll
+        for (int u = 0; u < kAhead; u++) {
+            const bool live = i < n_hi;
+            const long row = (long)b * N + (live ? i : n_hi - 1);
+            v[u] = xg[row * x_row + r];
+            m[u] = mul_g ? mul_g[row * m_row + r] : 1.0f;
+            if (!live) m[u] = 0.f;
+            i += step_i;
+            r += step_r;
+            if (r >= run) { r -= run; i++; }
+        }
+#pragma unroll
+        for (int u = 0; u < kAhead; u++) {
+            const float w = v[u] * m[u];
+            s += w;
+            ss += (double)w * w;
+        }
     }
     const double ts = block_sum(s, lds);
     const double tss = block_sum(ss, lds);
