@@ -367,9 +367,24 @@ __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))
 
     // the two scales, from the partial maxima
     auto set_scales = [&]() {
-    float ma = 0.f, mb = 0.f;
-    for (int k = threadIdx.x; k < n_dy_parts; k += 256) ma = fmaxf(ma, fabsf(dy_parts[k]));
-    for (int k = threadIdx.x; k < n_x_parts; k += 256) mb = fmaxf(mb, fabsf(x_parts[k]));
+    // (16-byte loads, four of them requested before the first is used: up to 64 values per thread and array)
+    auto absmax_of = [&](const float* __restrict__ p, int n) {
+        float mx = 0.f;
+        const int n4 = (reinterpret_cast<uintptr_t>(p) & 15) == 0 ? n / 4 : 0;
+        const float4* p4 = reinterpret_cast<const float4*>(p);
+        auto fold = [&](const float4 t) {
+            mx = fmaxf(fmaxf(mx, fmaxf(fabsf(t.x), fabsf(t.y))), fmaxf(fabsf(t.z), fabsf(t.w)));
+        };
+        int k = threadIdx.x;
+        for (; k + 3 * 256 < n4; k += 4 * 256) {
+            const float4 t0 = p4[k], t1 = p4[k + 256], t2 = p4[k + 512], t3 = p4[k + 768];
+            fold(t0); fold(t1); fold(t2); fold(t3);
+        }
+        for (; k < n4; k += 256) fold(p4[k]);
+        for (int j = 4 * n4 + threadIdx.x; j < n; j += 256) mx = fmaxf(mx, fabsf(p[j]));
+        return mx;
+    };
+    float ma = absmax_of(dy_parts, n_dy_parts), mb = absmax_of(x_parts, n_x_parts);
     for (int d = 1; d < 64; d <<= 1) { ma = fmaxf(ma, __shfl_xor(ma, d)); mb = fmaxf(mb, __shfl_xor(mb, d)); }
     float* wave_max = reinterpret_cast<float*>(lds);
     if (lane == 0) { wave_max[wave] = ma; wave_max[4 + wave] = mb; }
@@ -586,7 +601,10 @@ int mg_tensor_linear_wgrad_f16x2(const float* dy, const float* x, const float* d
     hipStream_t st = (hipStream_t)stream;
     const long n = (long)dim_in * dim_out;
     long rpb, splits;
-    wgrad_split(rows, dim_in, dim_out, kFTile, &rpb, &splits, 512);      // two workgroups per CU fit
+    // two workgroups per CU fit; with node-sized operands one per CU is faster (longer slices, half the partial
+    // results to write and add up: 4096 x 512 x 512 29 against 35 us, 12288 x 128 x 384 26 against 30 us;
+    // 101000 x 512 x 512 281 against 238 us)
+    wgrad_split(rows, dim_in, dim_out, kFTile, &rpb, &splits, rows < 65536 ? 256 : 512);
     float* part = reinterpret_cast<float*>((reinterpret_cast<uintptr_t>(workspace) + 15) & ~uintptr_t(15));
     float* maxima = part + splits * n;                       // [dy: kFParts][x: kFParts]
     float* colsum_part = db ? maxima + 2 * kFParts : nullptr; // [slice][dim_out]
