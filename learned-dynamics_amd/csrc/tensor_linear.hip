@@ -384,6 +384,86 @@ int launch_rows(const float* W, long so, long si, const float* X, long R, int I,
     return check_launch("mg_tensor_linear");
 }
 
+
+// A handful of output channels (readouts: n -> 1 vectors).  The matrix tiles above are 32 columns wide, so a one-column
+// output uses 1/32 of them, and the launch is bound by the latency of its few workgroups' loop over dim_in.  Here a
+// group of lanes takes one row of x, (dim_in, T) with T = 1, 3 or 9 components per channel: a lane reads 4 channels
+// = T 16-byte pieces at a time, so which component and channel an element belongs to is fixed at compile time, forms
+// OC x T partial sums and the group adds them up with lane shuffles.  y_comp_major: y (row, comp, chan) instead of
+// (row, chan, comp).
+template <int T, int OC>
+__global__ void __launch_bounds__(256) linear_few_outputs_kernel(const float* __restrict__ W, long so, long si,
+                                                                 const float* __restrict__ X, long R, int I, int O,
+                                                                 const float* __restrict__ bias, int act, int accumulate,
+                                                                 int y_comp_major, int lanes_per_row,
+                                                                 float* __restrict__ Y) {
+    const int lane = threadIdx.x & 63;
+    const long wave = ((long)blockIdx.x * blockDim.x + threadIdx.x) >> 6;
+    const int rows_per_wave = 64 / lanes_per_row;
+    const int sub = lane & (lanes_per_row - 1);
+    const long row = wave * rows_per_wave + lane / lanes_per_row;
+    const long ld_row = row < R ? row : R - 1;                  // (surplus groups repeat the last row and store nothing)
+    const float* xrow = X + ld_row * (long)I * T;
+    float sum[OC][T];
+#pragma unroll
+    for (int o = 0; o < OC; o++)
+#pragma unroll
+        for (int t = 0; t < T; t++) sum[o][t] = 0.f;
+    for (int p = sub; p < I / 4; p += lanes_per_row) {
+        float4 v[T];
+#pragma unroll
+        for (int k = 0; k < T; k++) v[k] = *reinterpret_cast<const float4*>(xrow + 4L * T * p + 4 * k);
+        float e[4 * T];
+#pragma unroll
+        for (int k = 0; k < T; k++) { e[4 * k] = v[k].x; e[4 * k + 1] = v[k].y; e[4 * k + 2] = v[k].z; e[4 * k + 3] = v[k].w; }
+#pragma unroll
+        for (int o = 0; o < OC; o++) {
+            const float* wrow = W + (long)(o < O ? o : 0) * so + 4L * p * si;
+#pragma unroll
+            for (int c = 0; c < 4; c++) {
+                const float w = wrow[c * si];
+#pragma unroll
+                for (int t = 0; t < T; t++) sum[o][t] = fmaf(w, e[c * T + t], sum[o][t]);
+            }
+        }
+    }
+#pragma unroll
+    for (int o = 0; o < OC; o++)
+#pragma unroll
+        for (int t = 0; t < T; t++)
+            for (int d = 1; d < lanes_per_row; d <<= 1) sum[o][t] += __shfl_xor(sum[o][t], d);
+    if (sub != 0 || row >= R) return;
+#pragma unroll
+    for (int o = 0; o < OC; o++) {
+        if (o >= O) break;
+        const float bv = bias ? bias[o] : 0.f;
+#pragma unroll
+        for (int t = 0; t < T; t++) {
+            float* dst = Y + (y_comp_major ? (row * T + t) * O + o : (row * O + o) * T + t);
+            float v = activate(sum[o][t] + bv, act);
+            if (accumulate) v += *dst;
+            *dst = v;
+        }
+    }
+}
+
+template <int T>
+int launch_few_outputs(const float* W, long so, long si, const float* X, long R, int I, int O, const float* bias, int act,
+                       int accumulate, int y_comp_major, float* Y, hipStream_t st) {
+    int lanes = 1;
+    while (lanes < 64 && lanes < I / 4) lanes <<= 1;
+    const long waves = ceil_div(R, 64 / lanes);
+    const long grid = ceil_div(waves, 4);
+    MG_REQUIRE(grid <= 0x7fffffffL, "mg_tensor_linear: grid too large (rows=%ld)", R);
+    if (O == 1)
+        hipLaunchKernelGGL((linear_few_outputs_kernel<T, 1>), dim3((unsigned)grid), dim3(256), 0, st, W, so, si, X, R, I, O,
+                           bias, act, accumulate, y_comp_major, lanes, Y);
+    else
+        hipLaunchKernelGGL((linear_few_outputs_kernel<T, 4>), dim3((unsigned)grid), dim3(256), 0, st, W, so, si, X, R, I, O,
+                           bias, act, accumulate, y_comp_major, lanes, Y);
+    return check_launch("mg_tensor_linear");
+}
+
 }  // namespace
 }  // namespace mg
 
@@ -407,6 +487,13 @@ int mg_tensor_linear_layout(int inds, const float* W, long w_stride_o, long w_st
     const float* b = bias;
     const long so = w_stride_o, si = w_stride_i;
     const int T = inds == 0 ? 1 : (inds == 1 ? 3 : 9);
+    if (dim_out <= 4 && dim_in >= 16 && dim_in % 4 == 0 && aligned16(x) && (x_layout == 0 || inds == 0)) {
+        // a readout: too few output channels for a 32-column matrix tile
+        const int ycm = (inds > 0 && y_layout == 1) ? 1 : 0;
+        if (inds == 0) return launch_few_outputs<1>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, ycm, y, st);
+        if (inds == 1) return launch_few_outputs<3>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, ycm, y, st);
+        return launch_few_outputs<9>(W, so, si, x, rows, dim_in, dim_out, b, act, accumulate, ycm, y, st);
+    }
     if (inds == 0 || x_layout == 1) {
         // component-major input: every (row, comp) pair is an independent row of a plain GEMM
         const long R = rows * T;

@@ -58,6 +58,38 @@ def test_tensor_linear_accumulate(ops):
     _check(out, base + OP.tensor_linear(1, W, x), 24)
 
 
+@pytest.mark.parametrize("inds", [0, 1, 2])
+@pytest.mark.parametrize("rows,dim_in,dim_out", [(4096, 128, 1), (77, 16, 3), (1001, 132, 4), (5, 1280, 2), (1, 64, 1)])
+def test_tensor_linear_with_a_few_output_channels(ops, inds, rows, dim_in, dim_out):
+    """Readout shapes (at most four output channels) have a kernel of their own: every layout, weight stride,
+    bias / activation and the accumulating form against float64."""
+    g = torch.Generator().manual_seed(300 + 10 * inds + dim_out)
+    T = 3 ** inds
+    W = torch.randn(dim_out, dim_in, generator=g) * dim_in ** -0.5
+    x = torch.randn(rows, dim_in, *([3] * inds), generator=g)
+    ref = torch.einsum("oi,ri...->ro...", W.double(), x.double())
+    y = ops.tensor_linear_fwd(inds, W.cuda(), x.cuda())
+    assert tuple(y.shape) == (rows, dim_out) + (3,) * inds
+    _check(y, ref.float(), dim_in)
+    # a weight with strides (the transposed view the input gradient of an n -> few linear would pass is the other
+    # shape; this is the forward of a layer whose weight is stored transposed)
+    Wt = W.t().contiguous().cuda().t()
+    assert dim_out == 1 or Wt.stride() == (1, dim_out)
+    _check(ops.tensor_linear_fwd(inds, Wt, x.cuda()), ref.float(), dim_in)
+    # component-major output
+    ycm = ops.tensor_linear_fwd(inds, W.cuda(), x.cuda(), y_layout=ops.LAYOUT_COMP_CHAN)
+    _check(ycm.reshape(rows, T, dim_out), ref.reshape(rows, dim_out, T).transpose(1, 2).float(), dim_in)
+    # accumulate
+    base = torch.randn(rows, dim_out, *([3] * inds), generator=g)
+    out = base.cuda().clone()
+    ops.tensor_linear_fwd(inds, W.cuda(), x.cuda(), out=out, accumulate=True)
+    _check(out, (base.double() + ref).float(), dim_in)
+    if inds == 0:
+        b = torch.randn(dim_out, generator=g)
+        yb = ops.tensor_linear_fwd(0, W.cuda(), x.cuda(), bias=b.cuda(), act=ops.ACT_SILU)
+        _check(yb, torch.nn.functional.silu(ref + b.double()).float(), dim_in)
+
+
 def test_tensor_linear_empty_and_errors(ops):
     W = torch.randn(8, 4).cuda()
     y = ops.tensor_linear_fwd(1, W, torch.empty(0, 4, 3).cuda())
