@@ -453,6 +453,11 @@ int mg_bee_edge_filters_fwd(const float* enc, const float* rh, long E, int chan,
 int mg_bee_edge_filters_bwd(const float* enc, const float* rh, const float* g_v, const float* g_d, long E, int chan,
                             float* d_enc, float* d_rh, mg_stream_t stream);
 
+/* SiLU and its derivatives for the MLPs' training path (nn.SiLU in archs/meanflow_painn8.py:38-51, differentiated up
+ * to three times by the meanflow loss, :274-296): out[k] = SiLU^(order)(z[k]) (* mul[k] if mul is not null), order 0..4,
+ * n floats, 16-byte aligned.  The reference leaves these derivatives to autograd's elementwise formulas. */
+int mg_silu_order(const float* z, const float* mul, long n, int order, float* out, mg_stream_t stream);
+
 /* The first two layers of the radial MLP from the edge vectors (archs/meanflow_painn8.py:25-35 feeding :38-51):
  *   y[e] = SiLU(b2 + W2 SiLU(b1 + W1 radial_encode(r_ij[e], 16, rmax))),   y (E, hidden)
  * in one kernel; the first layer's output is produced chunk by chunk on the matrix cores and never stored.

@@ -97,6 +97,7 @@ _SIGNATURES = {
     "mg_painn_edge_records": [vp, i64, i32, f32, f32, vp, vp],
     "mg_painn_table_message_sliced": [vp, vp, vp, i32, i64, vp, vp, i32, vp, vp, i32, vp, vp, vp, vp, vp],
     "mg_painn_combine_supported": [i32],
+    "mg_silu_order": [vp, vp, i64, i32, vp, vp],
     "mg_bee_edge_filters_fwd": [vp, vp, i64, i32, vp, vp, vp],
     "mg_bee_edge_filters_bwd": [vp, vp, vp, vp, i64, i32, vp, vp, vp],
     "mg_painn_table_interp_supported": [i32, i32],

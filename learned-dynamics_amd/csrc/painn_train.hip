@@ -405,6 +405,41 @@ __global__ void __launch_bounds__(256) edge_filters_bwd_kernel(const float* __re
 
 inline bool combine_shape_ok(int n) { return n >= 4 && n <= 256 && (n & (n - 1)) == 0; }
 
+
+// k-th derivative of SiLU(z) = z sigma(z), k = 0..4, times an optional factor.  With s = sigma(z), p = s (1 - s) and
+// u = 1 - 2 s the derivatives of sigma are d1 = p, d2 = p u, d3 = p (u^2 - 2 p), d4 = p u (u^2 - 8 p), and
+// SiLU^(k) = k d(k-1) + z d(k).  Differentiating an MLP k times needs SiLU^(k) of the same pre-activations;
+// autograd's own formula for the derivative of SiLU's derivative is a chain of seven elementwise launches.
+__device__ __forceinline__ float silu_derivative(float z, int order) {
+    const float s = 1.0f / (1.0f + expf(-z));
+    if (order == 0) return z * s;
+    const float p = s * (1.0f - s), u = 1.0f - 2.0f * s;
+    if (order == 1) return s + z * p;
+    if (order == 2) return p * (2.0f + z * u);
+    const float q = u * u - 2.0f * p;
+    if (order == 3) return p * (3.0f * u + z * q);
+    return p * (4.0f * q + z * u * (u * u - 8.0f * p));
+}
+
+__global__ void __launch_bounds__(256) silu_order_kernel(const float* __restrict__ z, const float* __restrict__ mul,
+                                                         long n, int order, float* __restrict__ out) {
+    const long n4 = n / 4;
+    for (long k = (long)blockIdx.x * blockDim.x + threadIdx.x; k < n4; k += (long)gridDim.x * blockDim.x) {
+        const float4 v = reinterpret_cast<const float4*>(z)[k];
+        float4 r = make_float4(silu_derivative(v.x, order), silu_derivative(v.y, order), silu_derivative(v.z, order),
+                               silu_derivative(v.w, order));
+        if (mul) {
+            const float4 m = reinterpret_cast<const float4*>(mul)[k];
+            r.x *= m.x; r.y *= m.y; r.z *= m.z; r.w *= m.w;
+        }
+        reinterpret_cast<float4*>(out)[k] = r;
+    }
+    if (blockIdx.x == 0 && threadIdx.x < n - 4 * n4) {
+        const long k = 4 * n4 + threadIdx.x;
+        out[k] = silu_derivative(z[k], order) * (mul ? mul[k] : 1.0f);
+    }
+}
+
 }  // namespace
 }  // namespace mg
 
@@ -531,6 +566,18 @@ int mg_bee_edge_filters_bwd(const float* enc, const float* rh, const float* g_v,
     hipLaunchKernelGGL(edge_filters_bwd_kernel, dim3((unsigned)E), dim3(256), 0, (hipStream_t)stream, enc, rh, g_v, g_d,
                        chan, d_enc, d_rh);
     return check_launch("mg_bee_edge_filters_bwd");
+}
+
+int mg_silu_order(const float* z, const float* mul, long n, int order, float* out, mg_stream_t stream) {
+    MG_REQUIRE(n >= 0 && order >= 0 && order <= 4, "mg_silu_order: order must be in 0..4 (got %d)", order);
+    if (n == 0) return MG_OK;
+    MG_REQUIRE(z && out && aligned16(z) && aligned16(out) && (mul == nullptr || aligned16(mul)),
+               "mg_silu_order: null or unaligned pointer");
+    long blocks = ceil_div(ceil_div(n, 4), 256);
+    if (blocks > 256L * 16) blocks = 256L * 16;
+    if (blocks < 1) blocks = 1;
+    hipLaunchKernelGGL(silu_order_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, z, mul, n, order, out);
+    return check_launch("mg_silu_order");
 }
 
 }  // extern "C"

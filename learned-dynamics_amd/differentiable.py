@@ -39,13 +39,46 @@ def linear(lin, x, x_bound=None, want_bound=False):
     return out.reshape(*lead, -1)
 
 
+class _SiluOrder(torch.autograd.Function):
+    """SiLU^(order)(z).  Its derivative is the next member of the same family times the incoming gradient, so the
+    family is closed under differentiation: every derivative order of an MLP costs one kernel per activation (plus one
+    product while a higher derivative is still being recorded) instead of autograd's chain of elementwise formulas for
+    the derivative of SiLU's derivative."""
+
+    @staticmethod
+    def forward(ctx, z, order):
+        ctx.save_for_backward(z)
+        ctx.order = order
+        return ops.silu_order(z.contiguous(), order)
+
+    @staticmethod
+    def backward(ctx, g):
+        z, = ctx.saved_tensors
+        if not torch.is_grad_enabled():
+            return ops.silu_order(z.contiguous(), ctx.order + 1, mul=g.contiguous()), None
+        return g * _silu_order(z, ctx.order + 1), None
+
+
+def _silu_order(z, order):
+    if order > ops.SILU_MAX_ORDER:
+        raise RuntimeError(f"SiLU is differentiable {ops.SILU_MAX_ORDER} times here")
+    return _SiluOrder.apply(z, order)
+
+
+def silu(z):
+    """nn.SiLU on a CUDA float32 tensor, differentiable up to ops.SILU_MAX_ORDER times."""
+    if z.is_cuda and z.dtype == torch.float32:
+        return _silu_order(z, 0)
+    return F.silu(z)
+
+
 def mlp_silu(mlp, x):
     """painn.MLP: Linear, SiLU, Linear, SiLU, Linear (archs/meanflow_painn8.py:38-51).  |SiLU(z)| <= |z|: the row
     maxima that a layer's kernel emits for z bound the next layer's input."""
     L = mlp.layers
     z, b = linear(L[0], x, want_bound=True)
-    z, b = linear(L[2], F.silu(z), x_bound=b, want_bound=True)
-    return linear(L[4], F.silu(z), x_bound=b)
+    z, b = linear(L[2], silu(z), x_bound=b, want_bound=True)
+    return linear(L[4], silu(z), x_bound=b)
 
 
 def mlp_leaky(mlp, x):

@@ -427,6 +427,24 @@ def bee_edge_filters_bwd(enc, rh, g_v, g_d):
     return d_enc, d_rh
 
 
+SILU_MAX_ORDER = 4
+
+
+def silu_order(z, order, mul=None):
+    """SiLU^(order)(z), elementwise, times mul if given (same shape); order 0 .. SILU_MAX_ORDER."""
+    _check_input(z, "z")
+    if mul is not None:
+        _check_input(mul, "mul")
+        if mul.shape != z.shape:
+            raise RuntimeError("mul must have the shape of z")
+    if not 0 <= int(order) <= SILU_MAX_ORDER:
+        raise RuntimeError(f"silu_order: order must be in 0..{SILU_MAX_ORDER}")
+    with torch.cuda.device(z.device):
+        out = torch.empty_like(z)
+        L.check(_lib.mg_silu_order(_p(z), _p(mul) if mul is not None else None, z.numel(), int(order), _p(out), _stream()))
+    return out
+
+
 def bee_indexed_supported(chan):
     return bool(_lib.mg_bee_indexed_supported(int(chan)))
 

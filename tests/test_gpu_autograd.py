@@ -456,6 +456,39 @@ def test_edge_filters_against_broadcasting_arithmetic(pkg, E, C):
     assert all(bool(torch.isfinite(t).all()) for t in torch.autograd.grad(sum((t ** 2).sum() for t in g_rec), (enc, rh)))
 
 
+def test_silu_family_against_float64_derivatives(pkg, ops):
+    """SiLU and its first four derivatives (one kernel each) against autograd in float64 through F.silu, as values
+    (ops.silu_order, with and without the fused factor) and through the closed autograd family: the plain backward
+    pass and three recorded ones."""
+    diff = importlib.import_module("learned-dynamics_amd.differentiable")
+    g = torch.Generator().manual_seed(77)
+    z64 = torch.cat([torch.linspace(-30, 30, 1203, dtype=F64), 4 * torch.randn(5000, generator=g, dtype=F64)]).requires_grad_()
+    ders = [torch.nn.functional.silu(z64)]
+    for _ in range(4):
+        ders.append(torch.autograd.grad(ders[-1].sum(), z64, create_graph=True)[0])
+    z = z64.detach().float().cuda()
+    m = torch.randn(z.shape, generator=g).cuda()
+    for k in range(5):
+        _close(ops.silu_order(z, k), ders[k], f"SiLU derivative {k}", tol=2e-6)
+        _close(ops.silu_order(z, k, mul=m), ders[k] * m.cpu().double(), f"SiLU derivative {k} times a factor", tol=2e-6)
+    with pytest.raises(RuntimeError):
+        ops.silu_order(z, 5)
+    # through autograd: w . silu(z), its gradient without recording, and the chain of recorded gradients
+    zg = z.clone().requires_grad_()
+    w = torch.randn(z.shape, generator=g, dtype=F64)
+    w32 = w.float().cuda()
+    y = diff.silu(zg)
+    _close(y, ders[0], "silu")
+    _close(torch.autograd.grad((y * w32).sum(), zg, retain_graph=True)[0], ders[1] * w, "gradient")
+    cur = (y * w32).sum()
+    for k in range(1, 4):
+        grad, = torch.autograd.grad(cur, zg, create_graph=True)
+        _close(grad, ders[k] * w, f"recorded gradient {k}", tol=2e-5)
+        cur = grad.sum()
+    # an odd length takes the scalar tail
+    _close(ops.silu_order(z[:1001].contiguous(), 2), ders[2][:1001], "tail", tol=2e-6)
+
+
 def test_fused_training_functions_on_a_graph_without_edges(pkg):
     """No edges at all: the folded functions return zero sums and zero gradients for the node operands."""
     diff = importlib.import_module("learned-dynamics_amd.differentiable")
