@@ -54,10 +54,10 @@ def _derived(module, key, params, make):
     one of the parameters changes (object or version), so that pre-split weight planes and norms
     keyed on the tensor object stay valid from one forward to the next."""
     cache = module.__dict__.setdefault("_derived_cache", {})
-    stamp = tuple((id(p), p._version, p.data_ptr()) for p in params)
+    stamp = ops.stamp(params)
     hit = cache.get(key)
     if hit is None or hit[0] != stamp:
-        with torch.no_grad():
+        with ops.derived_tensors():
             hit = cache[key] = (stamp, make())
     return hit[1]
 

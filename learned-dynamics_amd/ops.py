@@ -6,6 +6,7 @@ the outputs with torch, and enqueues the HIP kernels on the current torch
 stream through libmanagan_hip.so.  Nothing here computes on the CPU or with
 torch kernels: if the library is missing, importing this module fails.
 """
+import contextlib
 import ctypes
 import weakref
 
@@ -839,6 +840,26 @@ def get_linear_mode():
     return int(_lib.mg_get_linear_mode())
 
 
+def tensor_version(t):
+    """t's version counter, or -1 for an inference tensor, which has none: a result cached for -1 is never reused."""
+    return -1 if t.is_inference() else t._version
+
+
+def stamp(tensors):
+    """What a cache of something computed from these tensors compares: objects, versions, addresses.  With an inference
+    tensor among them (no version counter) the stamp equals no other, so the cached value is rebuilt."""
+    st = tuple((id(t), tensor_version(t), t.data_ptr()) for t in tensors)
+    return st if all(v[1] >= 0 for v in st) else (object(),)
+
+
+@contextlib.contextmanager
+def derived_tensors():
+    """For tensors computed from parameters and kept across calls: nothing recorded for autograd, and ordinary tensors
+    (with the version counter the caches check) also when the caller runs under torch.inference_mode()."""
+    with torch.inference_mode(False), torch.no_grad():
+        yield
+
+
 _packed_cache = {}
 
 
@@ -851,7 +872,8 @@ def _packed(W, kind):
     owner = W._base if W._base is not None else W
     key = (id(owner), kind, int(W.storage_offset()), tuple(W.shape), tuple(W.stride()))
     hit = _packed_cache.get(key)
-    if hit is not None and hit[0]() is owner and hit[1] == owner._version and hit[2] == owner.data_ptr():
+    version = tensor_version(owner)
+    if hit is not None and version >= 0 and hit[0]() is owner and hit[1] == version and hit[2] == owner.data_ptr():
         return hit[3]
     dim_out, dim_in = int(W.size(0)), int(W.size(1))
     nbytes = ctypes.c_size_t(0)
@@ -865,7 +887,7 @@ def _packed(W, kind):
         _packed_cache.clear()
     # the entry (and the device memory of its planes) goes when the tensor it was packed from does
     _packed_cache[key] = (weakref.ref(owner, lambda _, key=key: _packed_cache.pop(key, None)),
-                          owner._version, owner.data_ptr(), packed)
+                          version, owner.data_ptr(), packed)
     return packed
 
 
@@ -878,13 +900,13 @@ def zero_padded_columns(W, k_pad):
         return W
     key = (id(W), k_pad)
     hit = _padded_cache.get(key)
-    if hit is not None and hit[0]() is W and hit[1] == W._version and hit[2] == W.data_ptr():
+    if hit is not None and hit[0]() is W and hit[1] == tensor_version(W) >= 0 and hit[2] == W.data_ptr():
         return hit[3]
-    with torch.no_grad():
+    with derived_tensors():
         Wp = torch.nn.functional.pad(W.detach(), (0, k_pad - int(W.size(1)))).contiguous()
     if len(_padded_cache) > 256:
         _padded_cache.clear()
-    _padded_cache[key] = (weakref.ref(W), W._version, W.data_ptr(), Wp)
+    _padded_cache[key] = (weakref.ref(W), tensor_version(W), W.data_ptr(), Wp)
     return Wp
 
 
@@ -932,13 +954,13 @@ def linear_out_bound(W, bias, in_bound):
         in_bound = linear_in_unit_bound(W.device)
     key = ("norms", id(W), id(bias))
     hit = _bound_cache.get(key)
-    if (hit is None or hit[0]() is not W or hit[1] != W._version
-            or (bias is not None and (hit[2]() is not bias or hit[3] != bias._version))):
-        with torch.no_grad():
+    w_ver, b_ver = tensor_version(W), (tensor_version(bias) if bias is not None else 0)
+    if (hit is None or min(w_ver, b_ver) < 0 or hit[0]() is not W or hit[1] != w_ver
+            or (bias is not None and (hit[2]() is not bias or hit[3] != b_ver))):
+        with derived_tensors():
             l1 = W.detach().abs().sum(dim=1).amax().reshape(1, 1)
             bmax = bias.detach().abs().amax().reshape(1, 1) if bias is not None else torch.zeros_like(l1)
-        hit = (weakref.ref(W), W._version, weakref.ref(bias) if bias is not None else None,
-               bias._version if bias is not None else 0, l1, bmax, {})
+        hit = (weakref.ref(W), w_ver, weakref.ref(bias) if bias is not None else None, b_ver, l1, bmax, {})
         if len(_bound_cache) > 1024:
             _bound_cache.clear()
         _bound_cache[key] = hit
@@ -1739,14 +1761,14 @@ def _channel_block_major_columns(W, n_types, chan):
     channel in block); cached per tensor object and version."""
     key = (id(W), n_types, chan)
     hit = _reordered_cache.get(key)
-    if hit is not None and hit[0]() is W and hit[1] == W._version and hit[2] == W.data_ptr():
+    if hit is not None and hit[0]() is W and hit[1] == tensor_version(W) >= 0 and hit[2] == W.data_ptr():
         return hit[3]
-    with torch.no_grad():
+    with derived_tensors():
         Wr = (W.detach().reshape(W.shape[0], n_types, chan // 32, 32).permute(0, 2, 1, 3)
               .reshape(W.shape[0], n_types * chan).contiguous())
     if len(_reordered_cache) > 256:
         _reordered_cache.clear()
-    _reordered_cache[key] = (weakref.ref(W), W._version, W.data_ptr(), Wr)
+    _reordered_cache[key] = (weakref.ref(W), tensor_version(W), W.data_ptr(), Wr)
     return Wr
 
 
@@ -1802,17 +1824,17 @@ def _operand_order_columns(W):
     matrix core (position 16 g + p holds channel 8 (p / 4) + 4 g + p % 4); cached per tensor object and version."""
     key = id(W)
     hit = _chunk_perm_cache.get(key)
-    if hit is not None and hit[0]() is W and hit[1] == W._version and hit[2] == W.data_ptr():
+    if hit is not None and hit[0]() is W and hit[1] == tensor_version(W) >= 0 and hit[2] == W.data_ptr():
         return hit[3]
     pos = torch.arange(32, device=W.device)
     g, p = pos // 16, pos % 16
     src = 8 * (p // 4) + 4 * g + p % 4
     cols = (torch.arange(0, W.shape[1], 32, device=W.device)[:, None] + src[None, :]).reshape(-1)
-    with torch.no_grad():
+    with derived_tensors():
         Wr = W.detach()[:, cols].contiguous()
     if len(_chunk_perm_cache) > 256:
         _chunk_perm_cache.clear()
-    _chunk_perm_cache[key] = (weakref.ref(W), W._version, W.data_ptr(), Wr)
+    _chunk_perm_cache[key] = (weakref.ref(W), tensor_version(W), W.data_ptr(), Wr)
     return Wr
 
 

@@ -131,9 +131,9 @@ class Update(nn.Module):
         flat_v = x_v.reshape(rows, n, 3).contiguous()
         params = (self.lin_l.W, self.lin_r.W, self.lin_v.W)
         cache = self.__dict__.setdefault("_lrv_cache", {})
-        stamp = tuple((id(p), p._version, p.data_ptr()) for p in params)
+        stamp = ops.stamp(params)
         if cache.get("stamp") != stamp:                                         # (3n, n): one GEMM for l, r, v; kept
-            with torch.no_grad():                                               # while the weights are unchanged, so
+            with ops.derived_tensors():                                         # while the weights are unchanged, so
                 cache.update(stamp=stamp, W=torch.cat(params, dim=0))           # its packed planes stay valid too
         W = cache["W"]
         # component-major (rows, 3, 3n): the GEMM stores whole rows, the two kernels below read with unit stride
@@ -182,9 +182,9 @@ class Message(nn.Module):
         """Last layer of mlp_actv with its rows in the slice-major column order of painn_table_message_sliced."""
         last = self.mlp_actv.layers[4]
         cache = self.__dict__.setdefault("_slice_cache", {})
-        stamp = tuple((id(p), p._version, p.data_ptr()) for p in (last.weight, last.bias))
+        stamp = ops.stamp((last.weight, last.bias))
         if cache.get("stamp") != stamp:
-            with torch.no_grad():
+            with ops.derived_tensors():
                 perm = ops.painn_slice_permutation(self.n, last.weight.device)
                 lin = nn.Linear(last.in_features, last.out_features, device=last.weight.device)
                 lin.weight.copy_(last.weight[perm])
@@ -196,9 +196,9 @@ class Message(nn.Module):
         """Last layer of the filter MLP with its rows in the column order of the fused kernel."""
         last = self.mlp_dist.layers[4]
         cache = self.__dict__.setdefault("_perm_cache", {})
-        stamp = tuple((id(p), p._version, p.data_ptr()) for p in (last.weight, last.bias))
+        stamp = ops.stamp((last.weight, last.bias))
         if cache.get("stamp") != stamp:
-            with torch.no_grad():
+            with ops.derived_tensors():
                 perm = ops.painn_filter_permutation(self.n, last.weight.device)
                 cache.update(stamp=stamp, W=last.weight[perm].contiguous(), b=last.bias[perm].contiguous())
         return cache["W"], cache["b"]
@@ -252,7 +252,7 @@ class Message(nn.Module):
         """Rows of the grid whose interpolation error is below TABLE_TOL for the current weights, or 0 if none of
         TABLE_ROWS is fine enough (then the filter is evaluated per edge).  Decided once per set of weights."""
         params = list(self.mlp_dist.parameters())
-        stamp = tuple((id(p), p._version, p.data_ptr()) for p in params)
+        stamp = ops.stamp(params)
         cache = self.__dict__.setdefault("_table_cache", {})
         if cache.get("stamp") != stamp:
             chosen = 0

@@ -198,3 +198,40 @@ def test_concurrent_sections_inside_a_capture(pkg):
         big = ops.CONCURRENT_MAX_ROWS + 1
         ops.concurrent([lambda: order.append(0), lambda: order.append(1), lambda: order.append(2)], big)
         assert order == [0, 1, 2]
+
+
+def test_forward_under_inference_mode_equals_no_grad(pkg):
+    """torch.inference_mode(), the usual wrapper of a serving loop: tensors made there have no version counter, and the
+    layers keep tensors derived from their weights (concatenations, permuted and padded copies, pre-split planes).  Both
+    denoisers give bit for bit the no_grad result, on the first call (caches filled inside inference mode) and later."""
+    den = importlib.import_module("learned-dynamics_amd.denoiser")
+    mf = importlib.import_module("learned-dynamics_amd.meanflow_painn")
+    torch.manual_seed(0x947 + 5)
+    B, N, L_box, r0 = 2, 384, 36.0, 6.0
+    box = (L_box,) * 3
+    x1 = _chain(B, N, L_box, 21)
+    x0 = x1 + 0.1 * torch.randn_like(x1)
+    s, t = torch.zeros(B).cuda(), torch.rand(B).cuda()
+    one_hot = torch.nn.functional.one_hot(torch.randint(0, 20, (B, N)), 20).float().cuda()
+    idx = torch.arange(N - 1)
+    topo = mf.Topology(one_hot[0], torch.cat([idx, idx + 1]).cuda(), torch.cat([idx + 1, idx]).cuda())
+    calls = []
+    for make, call in ((lambda: den.Denoiser(r0, dim_a=64, dim_v=32, dim_d=16, chan=64, blocks=2),
+                        lambda m: m((s, t), x0, x1, one_hot, box)),
+                       (lambda: mf.SE3ITO(r0, 64, N, blks_0=1, blks_1=1, mutate_pos=True),
+                        lambda m: m((s, t), x1, x0, box, topo))):
+        torch.manual_seed(7)
+        fresh = make().cuda().eval()
+        with torch.inference_mode():
+            first = call(fresh).clone()
+            second = call(fresh).clone()
+        torch.manual_seed(7)
+        model = make().cuda().eval()
+        with torch.no_grad():
+            ref = call(model)
+        with torch.inference_mode():
+            third = call(model)                 # caches filled under no_grad, read under inference mode
+        for got in (first, second, third):
+            torch.testing.assert_close(got, ref, rtol=0, atol=0)
+        calls.append(ref)
+    assert all(bool(torch.isfinite(r).all()) for r in calls)
