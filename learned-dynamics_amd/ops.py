@@ -840,9 +840,21 @@ def get_linear_mode():
     return int(_lib.mg_get_linear_mode())
 
 
+_cache_epoch = 0
+
+
+def invalidate_weight_caches():
+    """Forget everything kept per weight tensor (pre-split planes, norms, permuted / padded / concatenated copies, here
+    and in the layers).  The caches notice a new tensor object and an in-place update through the tensor itself (its
+    version counter); a write that bypasses the counter (`param.data.mul_(...)`, a raw pointer) needs this call."""
+    global _cache_epoch
+    _cache_epoch += 1
+
+
 def tensor_version(t):
-    """t's version counter, or -1 for an inference tensor, which has none: a result cached for -1 is never reused."""
-    return -1 if t.is_inference() else t._version
+    """t's version counter (with the epoch of invalidate_weight_caches in the high bits), or -1 for an inference
+    tensor, which has none: a result cached for -1 is never reused."""
+    return -1 if t.is_inference() else (_cache_epoch << 40) | t._version
 
 
 def stamp(tensors):

@@ -245,6 +245,26 @@ def test_packed_weight_cache_tracks_in_place_updates(ops):
         ops.set_linear_mode(prev)
 
 
+def test_weight_written_behind_the_version_counter(pkg, ops):
+    """`param.data.mul_()` changes a weight without touching its version counter: the caches cannot see it, and
+    ops.invalidate_weight_caches() is the documented remedy (layer caches included)."""
+    painn = importlib.import_module("learned-dynamics_amd.painn")
+    torch.manual_seed(5)
+    upd = painn.Update(64).cuda().eval()
+    x_a, x_v = torch.randn(1, 700, 64).cuda(), torch.randn(1, 700, 64, 3).cuda()
+    with torch.no_grad():
+        upd(x_a, x_v)                                            # fills the caches
+        for p in upd.parameters():
+            p.data.mul_(1.25)
+        ops.invalidate_weight_caches()
+        got = upd(x_a, x_v)
+        fresh = painn.Update(64).cuda().eval()
+        fresh.load_state_dict(upd.state_dict())
+        ref = fresh(x_a, x_v)
+    for a, b in zip(got, ref):
+        torch.testing.assert_close(a, b, rtol=0, atol=0)
+
+
 def _segment_lengths(kind, n, g):
     if kind == "long":
         return torch.randint(40, 140, (n,), generator=g)
