@@ -53,7 +53,7 @@ int mg_abi_version(void);
  *   count: bins atoms, walks the 3x3x3 cell window, writes the CSR row_ptr
  *          (batch*nodes+1, exclusive prefix), edge_counts (batch, inclusive
  *          prefix per box, as the reference's edgeCounts) and stats[4] =
- *          {E, max atoms in a cell, max degree, 1 if E overflowed int32};
+ *          {E, max atoms in a cell, max degree, flags: bit 0 = E overflowed int32};
  *   fill:  writes src[e] = b*nodes+i and dst[e] = b*nodes+j, rows ordered by
  *          (b,i); order inside a row is deterministic.  n_edges is the CAPACITY of
  *          src and dst in edges: an edge whose position row_ptr[row] + k is not
@@ -83,7 +83,11 @@ int mg_neighbour_fill(const void* workspace, size_t workspace_bytes, int batch, 
 
 /* Both phases in one call for a caller that sizes src / dst itself (`capacity` edges each) and does not want to read
  * the edge count back in between: get_edges (extensions/neighbour_grid/neighbour_grid.cpp:170-195) without its
- * device->host copies.  Edges beyond the capacity are dropped as in mg_neighbour_fill; stats[0] holds the true count.
+ * device->host copies.  What the caller gets is the graph truncated at `capacity` edges: edges beyond the capacity
+ * are dropped as in mg_neighbour_fill, and row_ptr / edge_counts entries above the capacity are lowered to it, so a
+ * kernel that walks the edges through row_ptr never leaves the edge arrays (the rows that did not fit are short or
+ * empty).  stats[0] holds the true count and stats[3] has bit 1 (value 2) set when edges were dropped: read them
+ * after the work that used the graph to know whether its result is that of the whole graph.
  * Nothing in it synchronises or allocates, so the call can be recorded into a HIP graph. */
 int mg_neighbour_edges(const float* x /* (batch,nodes,3) */, int batch, int nodes, float cutoff,
                        float box_x, float box_y, float box_z, void* workspace, size_t workspace_bytes,
@@ -293,6 +297,13 @@ int mg_tensor_linear_f16x2_rowmax_parts(long rows, int dim_in, int dim_out);   /
 int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts,
                            long x_rowmax_stride, long x_rows_per_bound, long rows, int dim_in, int dim_out, const float* bias, int act, int accumulate,
                            int out_comps, float* y, float* y_rowmax, mg_stream_t stream);
+/* y = act(x W^T + bias) in float64 arithmetic: W (dim_out, dim_in) and bias are the float32 parameters, widened
+ * exactly; x (rows, dim_in), every product and sum, the activation and y (rows, dim_out) are double.  The same
+ * contraction as nn.Linear inside the reference's MLPs (archs/meanflow_painn8.py:38-51); float64 has no counterpart
+ * in the reference.  It exists to measure approximations of a float32 MLP against exact arithmetic on the device
+ * (the acceptance test of the PaiNN filter grid), not as a compute path. */
+int mg_linear_f64(const float* W, const float* bias /* may be NULL */, const double* x, long rows, int dim_in,
+                  int dim_out, int act, double* y, mg_stream_t stream);
 /* dW[o,i] = sum_{r,t} dy[r,o,t] x[r,i,t]  (tensor_ops_kern.cu:45-71), dW dense (dim_out,dim_in).  The rows are
  * reduced in slices whose partial results go to `workspace` (mg_tensor_linear_wgrad_workspace_bytes) and are added
  * in slice order: no atomics, the same bits on every run. */

@@ -69,6 +69,7 @@ _SIGNATURES = {
     "mg_linear_f16x2_packed_weight_bytes": [i32, i32, ctypes.POINTER(ctypes.c_size_t)],
     "mg_linear_f16x2_pack_weight": [vp, i64, i64, i32, i32, vp, vp],
     "mg_row_absmax": [vp, i64, i32, vp, vp],
+    "mg_linear_f64": [vp, vp, vp, i64, i32, i32, i32, vp, vp],
     "mg_tensor_linear_f16x2_rowmax_parts": [i64, i32, i32],
     "mg_tensor_linear_f16x2": [vp, vp, vp, i32, i64, i64, i64, i32, i32, vp, i32, i32, i32, vp, vp, vp],
     "mg_ant16_fwd": [i32, i32, ctypes.POINTER(i32), ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, vp, i64, i32, i32, i32,

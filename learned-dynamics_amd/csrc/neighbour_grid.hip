@@ -860,6 +860,18 @@ int run_scan(const int* in, long n, int* out, Workspace& w, int* out_total, int*
     return check_launch("neighbour scan");
 }
 
+// The graph truncated at `capacity` edges: row pointers and per-box counts above the capacity are lowered to it, so
+// that every kernel that walks the edges through row_ptr stays inside edge arrays of that many entries.  stats[0]
+// keeps the true count; bit 1 of stats[3] says that edges were dropped.
+__global__ void __launch_bounds__(256) clamp_row_ptr_kernel(int* __restrict__ row_ptr, long n_ptr,
+                                                            int* __restrict__ edge_counts, int batch, int capacity,
+                                                            int* __restrict__ stats) {
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n_ptr && row_ptr[i] > capacity) row_ptr[i] = capacity;
+    if (i < batch && edge_counts[i] > capacity) edge_counts[i] = capacity;
+    if (i == 0 && stats[0] > capacity) stats[3] |= 2;
+}
+
 int pairs_block_size(const Grid& g);
 // workgroups that share the sort of one box: one per 1024 atoms (box_max has batch * nodes entries, so slabs <= nodes)
 int sort_slabs(const Grid& g) {
@@ -979,8 +991,15 @@ int mg_neighbour_edges(const float* x, int batch, int nodes, float cutoff, float
     if (int s = mg_neighbour_count(x, batch, nodes, cutoff, box_x, box_y, box_z, workspace, workspace_bytes, row_ptr,
                                    edge_counts, stats, stream))
         return s;
-    return mg_neighbour_fill(workspace, workspace_bytes, batch, nodes, cutoff, box_x, box_y, box_z, row_ptr, capacity,
-                             src, dst, stream);
+    if (int s = mg_neighbour_fill(workspace, workspace_bytes, batch, nodes, cutoff, box_x, box_y, box_z, row_ptr,
+                                  capacity, src, dst, stream))
+        return s;
+    const long n_ptr = (long)batch * nodes + 1;
+    if (n_ptr == 1) return MG_OK;
+    // after the fill pass (which places edges by the exact row_ptr): the caller's view is the graph cut at capacity
+    hipLaunchKernelGGL(clamp_row_ptr_kernel, dim3((unsigned)ceil_div(n_ptr, 256)), dim3(256), 0, (hipStream_t)stream,
+                       row_ptr, n_ptr, edge_counts, batch, capacity, stats);
+    return check_launch("mg_neighbour_edges");
 }
 
 int mg_neighbour_edges_static(const float* x, int batch, int nodes, float cutoff, float box_x, float box_y,

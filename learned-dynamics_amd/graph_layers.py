@@ -181,7 +181,11 @@ def graph_setup_capacity(r0, box, pos, capacity, buffers=None):
     call can be recorded into a HIP graph together with the layers (pass the `buffers` of an earlier call,
     graph.buffers, so that a replay writes into the same memory).  Entries of src / dst past E are valid but
     meaningless node indices: only kernels that walk the edges through row_ptr may be used on such a graph
-    (graph.padded is True); per-edge tensors such as r_ij have `capacity` rows."""
+    (graph.padded is True); per-edge tensors such as r_ij have `capacity` rows.
+    When the graph has more than `capacity` edges the result is the graph cut at `capacity` edges: the edges that do
+    not fit are dropped and row_ptr / edge counts are lowered to the capacity on the device, so nothing reads past
+    the arrays; graph.stats[0] keeps the true count and graph.stats[3] has bit 1 set.  The count stays on the device
+    inside a capture, so read graph.stats after the replay to know whether a result is that of the whole graph."""
     out = ops.neighbour_edges(pos.contiguous(), r0, box, capacity, out=buffers)
     batch, nodes = int(pos.shape[0]), int(pos.shape[1])
     graph = Graph(out["src"], out["dst"], out["edge_counts"], batch, nodes, row_ptr=out["row_ptr"],

@@ -857,11 +857,15 @@ def tensor_version(t):
     return -1 if t.is_inference() else (_cache_epoch << 40) | t._version
 
 
-def stamp(tensors):
+def stamp(tensors, keep_unversioned=False):
     """What a cache of something computed from these tensors compares: objects, versions, addresses.  With an inference
-    tensor among them (no version counter) the stamp equals no other, so the cached value is rebuilt."""
+    tensor among them (no version counter) the stamp equals no other, so the cached value is rebuilt; with
+    keep_unversioned such a tensor is stamped by object, address and the epoch of invalidate_weight_caches instead
+    (for decisions that are expensive to re-make and that a caller who writes such tensors in place can reset)."""
     st = tuple((id(t), tensor_version(t), t.data_ptr()) for t in tensors)
-    return st if all(v[1] >= 0 for v in st) else (object(),)
+    if all(v[1] >= 0 for v in st):
+        return st
+    return tuple((i, v if v >= 0 else -1 - _cache_epoch, p) for i, v, p in st) if keep_unversioned else (object(),)
 
 
 @contextlib.contextmanager
@@ -941,6 +945,22 @@ def row_absmax(x):
         out = torch.empty(x.size(0), 1, dtype=torch.float32, device=x.device)
         L.check(_lib.mg_row_absmax(_p(x), int(x.size(0)), int(x.size(1)), _p(out), _stream()))
     return out
+
+
+def linear_f64(W, bias, x, act=ACT_NONE):
+    """act(x W^T + bias) in float64 arithmetic: W (dim_out, dim_in) and bias float32 parameters, x (rows, dim_in) and
+    the result float64.  For measuring approximations of a float32 MLP against exact arithmetic, not a compute path."""
+    _check_input(W, "W")
+    _check_input(x, "x", torch.float64)
+    if bias is not None:
+        _check_input(bias, "bias")
+    if x.dim() != 2 or W.dim() != 2 or W.size(1) != x.size(1) or (bias is not None and bias.numel() != W.size(0)):
+        raise RuntimeError("linear_f64: x (rows, dim_in), W (dim_out, dim_in), bias (dim_out)")
+    with torch.cuda.device(x.device):
+        y = torch.empty(x.size(0), W.size(0), dtype=torch.float64, device=x.device)
+        L.check(_lib.mg_linear_f64(_p(W), _p(bias) if bias is not None else None, _p(x), int(x.size(0)),
+                                   int(W.size(1)), int(W.size(0)), int(act), _p(y), _stream()))
+    return y
 
 
 _bound_cache = {}

@@ -206,10 +206,17 @@ class Message(nn.Module):
     # The filter sees an edge only through its length d, and radial_encode is made of cos / sin (k pi d / r0) with
     # integer k: the filter is a smooth function of d with period 2 r0.  It is evaluated on a grid over one period
     # (a few thousand rows through the same kernels as the exact path) and every edge interpolates between the four
-    # grid rows around its d.  The grid is accepted per set of weights by comparing the interpolation with the exact
-    # filter at the grid's midpoints, where the 4-point Lagrange error is largest.
+    # grid rows around its d.  A grid is accepted per set of weights, element by element: at the grid's midpoints,
+    # where the 4-point Lagrange error peaks, |interpolated - exact| must stay below TABLE_ATOL + TABLE_RTOL |exact|
+    # for every one of the 4n filter columns.  Both sides of that comparison are evaluated in float64
+    # (ops.linear_f64), because the quantity bounded is the interpolation error alone: the float32 GEMMs that
+    # evaluate the grid at run time round exactly as they do when they evaluate the filter of every edge, and that
+    # rounding (1e-6 of a row's scale) would drown an error of this size.  The bound is a tenth of the layer
+    # tolerance (abs 1e-6, rel 1e-5), so an accepted grid uses a tenth of the error a filter element may have.
     TABLE_ROWS = (512, 2048, 4096, 8192)      # 512 rows fit in LDS beside a slice of 16 channels
-    TABLE_TOL = 3e-6            # of max |filter|: the level of the split-fp16 GEMMs that evaluate the filter itself
+    TABLE_ATOL = 1e-7
+    TABLE_RTOL = 1e-6
+    TABLE_RECHECK = 64          # while training, the decision is re-made every this many changes of the weights
     use_table = True
 
     def _grid_encoding(self, rows, shift, device, width=None):
@@ -225,12 +232,7 @@ class Message(nn.Module):
             return cache[key]
         key = (rows, shift, str(device))
         if key not in cache:
-            n = self.n_rbf
-            hn = (n + 1) // 2
-            d = (torch.arange(rows, dtype=torch.float64) + shift) * (2.0 * self.r0 / rows)
-            phase = (math.pi / self.r0) * (1 + torch.arange(hn) // 2).to(torch.float64)[None, :] * d[:, None]
-            enc = torch.cat([torch.cos(phase), torch.sin(phase[:, :n - hn])], dim=-1)
-            cache[key] = enc.to(torch.float32).to(device).contiguous()
+            cache[key] = self._grid_phases(rows, shift).to(torch.float32).to(device).contiguous()
         return cache[key]
 
     def filter_table(self, rows, shift=0.0):
@@ -248,23 +250,58 @@ class Message(nn.Module):
             return self.mlp_dist.after_first(h, ops.linear_out_bound(first.weight, first.bias, unit))
         return self.mlp_dist(self._grid_encoding(rows, shift, device), unit)
 
+    def _grid_phases(self, rows, shift):
+        """The float64 encodings at d = (k + shift) 2 r0 / rows (host tensor)."""
+        n = self.n_rbf
+        hn = (n + 1) // 2
+        d = (torch.arange(rows, dtype=torch.float64) + shift) * (2.0 * self.r0 / rows)
+        phase = (math.pi / self.r0) * (1 + torch.arange(hn) // 2).to(torch.float64)[None, :] * d[:, None]
+        return torch.cat([torch.cos(phase), torch.sin(phase[:, :n - hn])], dim=-1)
+
+    def filter_table_f64(self, rows, shift=0.0):
+        """filter_table in float64 arithmetic (the float32 parameters widened exactly): (rows, 4n) double."""
+        L = self.mlp_dist.layers
+        device = L[0].weight.device
+        cache = self.__dict__.setdefault("_grid_cache", {})
+        key = (rows, shift, str(device), "f64")
+        if key not in cache:
+            cache[key] = self._grid_phases(rows, shift).to(device).contiguous()
+        with ops.derived_tensors():
+            h = ops.linear_f64(L[0].weight.detach(), L[0].bias.detach(), cache[key], ops.ACT_SILU)
+            h = ops.linear_f64(L[2].weight.detach(), L[2].bias.detach(), h, ops.ACT_SILU)
+            return ops.linear_f64(L[4].weight.detach(), L[4].bias.detach(), h, ops.ACT_NONE)
+
+    def table_error(self, rows):
+        """max over the grid's midpoints and the 4n filter columns of
+        |4-point interpolation - exact| / (TABLE_ATOL + TABLE_RTOL |exact|), both in float64: a device scalar.
+        A grid of this many rows is accepted when the value is at most 1."""
+        tab = self.filter_table_f64(rows)
+        mid = self.filter_table_f64(rows, 0.5)
+        interp = (9.0 / 16.0) * (tab + tab.roll(-1, 0)) - (1.0 / 16.0) * (tab.roll(1, 0) + tab.roll(-2, 0))
+        return ((interp - mid).abs() / (self.TABLE_ATOL + self.TABLE_RTOL * mid.abs())).amax()
+
     def table_rows(self):
-        """Rows of the grid whose interpolation error is below TABLE_TOL for the current weights, or 0 if none of
-        TABLE_ROWS is fine enough (then the filter is evaluated per edge).  Decided once per set of weights."""
+        """Rows of the smallest grid of TABLE_ROWS that table_error accepts for the current weights, or 0 if none
+        does (then the filter is evaluated per edge).  Decided once per set of weights (one host read-back per
+        candidate grid).  While the weights are being trained (autograd is recording for them) the decision is kept
+        for TABLE_RECHECK changes of the weights before it is made again: one optimizer step moves the
+        interpolation error by far less than the factor ten between TABLE_ATOL / TABLE_RTOL and the layer
+        tolerance, and the check costs host synchronisations that a training step should not pay every time."""
         params = list(self.mlp_dist.parameters())
-        stamp = ops.stamp(params)
+        stamp = ops.stamp(params, keep_unversioned=True)
         cache = self.__dict__.setdefault("_table_cache", {})
         if cache.get("stamp") != stamp:
-            chosen = 0
-            with torch.no_grad():
-                for rows in self.TABLE_ROWS:
-                    tab = self.filter_table(rows)
-                    mid = self.filter_table(rows, 0.5)
-                    interp = (9.0 / 16.0) * (tab + tab.roll(-1, 0)) - (1.0 / 16.0) * (tab.roll(1, 0) + tab.roll(-2, 0))
-                    if float((interp - mid).abs().max()) <= self.TABLE_TOL * float(tab.abs().max()):
-                        chosen = rows
-                        break
-            cache.update(stamp=stamp, rows=chosen)
+            training = diff.wants_grad(self.mlp_dist)
+            cache["changes"] = cache.get("changes", 0) + 1
+            if not ("rows" in cache and training and cache.get("trained") and cache["changes"] % self.TABLE_RECHECK):
+                chosen = 0
+                with torch.no_grad():
+                    for rows in self.TABLE_ROWS:
+                        if float(self.table_error(rows)) <= 1.0:
+                            chosen = rows
+                            break
+                cache["rows"] = chosen
+            cache.update(stamp=stamp, trained=training)
         return cache["rows"]
 
     def forward(self, graph: Graph, x_a, x_v, r_ij, residual=False):

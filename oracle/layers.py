@@ -10,6 +10,8 @@ Follows (relative to the reference checkout):
   archs/meanflow_painn8.py:53-75           Update
   archs/meanflow_painn8.py:77-100          Message
   managan/jacobi_radenc.py:8-37            radial_encode_8 (shifted Jacobi(1,0) x relu(1-z))
+  archs/diffuser_atoms14.py:32-48          normed_sq_dist, sq_radial_encode, radial_encode (hyperbolic distance)
+  archs/diffuser_atoms5.py:25-30           radial_encode_edge (cosines x relu(1 - |r|^2 / rmax))
   managan/tensor_products.py:167-182       tens_sigmoid
   managan/tensor_products.py:215-232       TensGroupNorm
   managan/layers_common.py:201-223         ScalGroupNorm
@@ -82,6 +84,24 @@ def radial_encode_8(r, rmax):
     z = (torch.linalg.vector_norm(r, dim=-1) / rmax)[..., None]
     pows = z ** torch.arange(A.shape[1])
     return F.linear(pows, A) * torch.relu(1.0 - z)
+
+
+def sq_radial_encode(r, n, rmax):
+    """archs/diffuser_atoms14.py:32-48 (radial_encode = sq_radial_encode o normed_sq_dist): with q = |r|^2 / rmax^2 and
+    h = sqrt(1 + q), column m is sin(c_m h) (sqrt(1/2) - h), c_m = (pi / sqrt 2) exp(m n^-0.7).  r: (..., 3) -> (..., n)."""
+    sq_dist = (r ** 2).sum(-1, keepdim=True) / rmax ** 2
+    coeffs = (math.pi * 2 ** -0.5) * torch.exp(n ** -0.7 * torch.arange(0, n, dtype=r.dtype))
+    hyperdist = torch.sqrt(1 + sq_dist)
+    return torch.sin(coeffs * hyperdist) * (0.5 ** 0.5 - hyperdist)
+
+
+def radial_encode_edge(r, n, rmax):
+    """archs/diffuser_atoms5.py:25-30: column m is cos(m pi sqrt(x)) relu(1 - x) with x = |r|^2 / rmax.  The squared
+    length is divided by rmax, not by rmax^2: the envelope reaches zero at |r| = sqrt(rmax), as in the reference.
+    r: (..., 3) -> (..., n)."""
+    npi = math.pi * torch.arange(0, n, dtype=r.dtype)
+    x_sq = (r ** 2).sum(-1) / rmax
+    return torch.cos(npi * torch.sqrt(x_sq)[..., None]) * torch.relu(1. - x_sq)[..., None]
 
 
 # ---------------------------------------------------------- norms and squashes

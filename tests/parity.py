@@ -28,3 +28,13 @@ def assert_parity(got, ref32, ref64, what="", rtol=1e-5, atol=1e-6, slack=2.0):
     assert not bool(bad.any()), (f"{what}: {int(bad.sum())} of {bad.numel()} elements outside rel {rtol} / abs {atol} "
                                  f"+ {slack} x e_ref ({e_ref:.3g}); max |hip - f64| = {e_hip:.3g}")
     return e_ref, e_hip
+
+
+def assert_parity_of(got, reference, what="", **kw):
+    """assert_parity for a kernel whose reference is a formula: reference(dtype) evaluates it on the CPU in that
+    dtype (a tensor or a tuple of tensors matching got), once in float32 and once in float64."""
+    r32, r64 = reference(torch.float32), reference(torch.float64)
+    if isinstance(got, (tuple, list)):
+        assert len(got) == len(r32) == len(r64)
+        return [assert_parity(g, a, b, f"{what}[{i}]", **kw) for i, (g, a, b) in enumerate(zip(got, r32, r64))]
+    return assert_parity(got, r32, r64, what, **kw)

@@ -10,7 +10,7 @@ import torch
 from oracle import layers as OL
 from oracle import neighbour as ON
 from oracle import products as OP
-from parity import assert_parity
+from parity import assert_parity, assert_parity_of
 
 pytestmark = pytest.mark.gpu
 
@@ -21,19 +21,17 @@ def _to(tree, dtype):
     return tree.to(dtype)
 
 
-def _close(a, ref, rtol=1e-5, atol_scale=2e-6):
-    ref = ref.to(torch.float32)
-    scale = max(1.0, float(ref.abs().max()))
-    torch.testing.assert_close(a.cpu(), ref, rtol=rtol, atol=atol_scale * scale)
-
-
 def test_edge_geometry(ops):
     g = torch.Generator().manual_seed(1)
     r = torch.randn(4000, 3, generator=g) * 3
     enc, rhat = ops.bee_edge_geometry(r.cuda(), 6.0)
+    # radial_encode_8: the kernel evaluates the polynomial in float64 and rounds once (the reference's float32
+    # monomial form is ill-conditioned, tests/test_oracle_layers.py), so the bar is the float64 oracle with no e_ref.
+    # z = |r| / rmax itself is formed in float32, as in the reference: half an ulp of z (at most 3e-8) passes through
+    # the polynomial's slope (up to about 30 where z is large enough to have such an ulp), which is the second 1e-6
     ref = OL.radial_encode_8(r.double(), 6.0)
     torch.testing.assert_close(enc.cpu().double(), ref, rtol=1e-5, atol=2e-6)
-    torch.testing.assert_close(rhat.cpu(), OL.tens_sigmoid(1, r * (7.0 / 6.0)), rtol=1e-5, atol=1e-6)
+    assert_parity_of(rhat, lambda dt: OL.tens_sigmoid(1, r.to(dt) * (7.0 / 6.0)), "edge direction")
 
 
 @pytest.mark.parametrize("lin_layout", [(0, 64, 40), (1, 64, 40), (2, 32, 72), (1, 20, 7), (2, 8, 130)])
@@ -43,16 +41,18 @@ def test_linear_layouts(ops, lin_layout):
     g = torch.Generator().manual_seed(2)
     W = torch.randn(dim_out, dim_in, generator=g)
     x = torch.randn(50, dim_in, *([3] * inds), generator=g)
-    ref = OP.tensor_linear(inds, W, x)                                   # (50, O, 3..)
-    ref_cm = ref.reshape(50, dim_out, T).transpose(1, 2).contiguous()    # (50, T, O)
+    def ref(dt):                                                         # (50, O, 3..)
+        return OP.tensor_linear(inds, W.to(dt), x.to(dt))
+
+    ref_cm = lambda dt: ref(dt).reshape(50, dim_out, T).transpose(1, 2).contiguous()     # (50, T, O)
     x_cm = x.reshape(50, dim_in, T).transpose(1, 2).contiguous()         # (50, T, I)
     C = ops.LAYOUT_COMP_CHAN
     y = ops.tensor_linear_fwd(inds, W.cuda(), x.cuda(), y_layout=C)
-    torch.testing.assert_close(y.cpu(), ref_cm, rtol=1e-5, atol=1e-5)
+    assert_parity_of(y, ref_cm, f"tensor_linear rank {inds}, component-major output")
     y = ops.tensor_linear_fwd(inds, W.cuda(), x_cm.cuda(), x_layout=C)
-    torch.testing.assert_close(y.cpu(), ref, rtol=1e-5, atol=1e-5)
+    assert_parity_of(y, ref, f"tensor_linear rank {inds}, component-major input")
     y = ops.tensor_linear_fwd(inds, W.cuda(), x_cm.cuda(), x_layout=C, y_layout=C)
-    torch.testing.assert_close(y.cpu(), ref_cm, rtol=1e-5, atol=1e-5)
+    assert_parity_of(y, ref_cm, f"tensor_linear rank {inds}, component-major both")
 
 
 @pytest.mark.parametrize("chan,E", [(64, 3000), (8, 3000), (100, 3000), (64, 9000), (40, 7000)])
@@ -79,19 +79,21 @@ def test_bee_message_kernel(ops, chan, E):
         assert torch.equal(nmax.amax(1), torch.maximum(S1.abs().amax(dim=(1, 2, 3)), S2.abs().amax(dim=(1, 2, 3))))
         assert emax.shape == (E, (chan + 63) // 64) and torch.equal(emax.amax(1), P0.abs().amax(dim=(1, 2)))
         # oracle on the device's own enc / rhat (they are checked separately)
-        phi_a = torch.nn.functional.linear(enc.cpu(), encW, encb)
-        rh = rhat.cpu()
-        phi_v = phi_a[..., None] * rh[:, None, :]
-        phi_d = phi_a[..., None, None] * rh[:, None, None, :] * rh[:, None, :, None]
-        prods = dict(zip(OP.BEE_ORDER, OP.bee(La[dst], Lv[dst], Ld[dst], phi_a, phi_v, phi_d)))
+        def products(dt):
+            phi_a = torch.nn.functional.linear(enc.cpu().to(dt), encW.to(dt), encb.to(dt))
+            rh = rhat.cpu().to(dt)
+            phi_v = phi_a[..., None] * rh[:, None, :]
+            phi_d = phi_a[..., None, None] * rh[:, None, None, :] * rh[:, None, :, None]
+            return dict(zip(OP.BEE_ORDER, OP.bee(La.to(dt)[dst], Lv.to(dt)[dst], Ld.to(dt)[dst], phi_a, phi_v, phi_d)))
+
         for k, lab in enumerate(("000", "110", "220")):
-            _close(P0[:, k], prods[lab])
+            assert_parity_of(P0[:, k], lambda dt: products(dt)[lab], f"bee_message P0 {lab} chan={chan}")
         for k, lab in enumerate(("011", "101", "121", "211", "111")):
-            ref = torch.zeros(N, chan, 3).index_add_(0, src, prods[lab])
-            _close(S1[:, :, k], ref.transpose(1, 2), atol_scale=4e-6)
+            assert_parity_of(S1[:, :, k], lambda dt: torch.zeros(N, chan, 3, dtype=dt).index_add_(
+                0, src, products(dt)[lab]).transpose(1, 2), f"bee_message S1 {lab} chan={chan}")
         for k, lab in enumerate(("022", "202", "112", "222", "212")):
-            ref = torch.zeros(N, chan, 3, 3).index_add_(0, src, prods[lab]).reshape(N, chan, 9)
-            _close(S2[:, :, k], ref.transpose(1, 2), atol_scale=4e-6)
+            assert_parity_of(S2[:, :, k], lambda dt: torch.zeros(N, chan, 3, 3, dtype=dt).index_add_(
+                0, src, products(dt)[lab]).reshape(N, chan, 9).transpose(1, 2), f"bee_message S2 {lab} chan={chan}")
 
 
 def test_node_products_emit_node_maxima(ops):
@@ -247,18 +249,20 @@ def test_mlp_summed_over_rows_equals_sum_of_rows(pkg, plus_identity):
     with torch.no_grad():
         got = mlp.summed_over_rows(x, row_ptr, N, plus_identity=plus_identity, scale=0.1)
         per_row = mlp(x, plus_identity=plus_identity)
-        # float64 reference of the same thing from plain torch modules
-        xd = x.double().cpu()
-        L = mlp.layers
-        f = torch.nn.functional
-        h = f.leaky_relu(f.linear(xd, L[0].weight.double().cpu(), L[0].bias.double().cpu()), 0.1)
-        h = f.leaky_relu(f.linear(h, L[2].weight.double().cpu(), L[2].bias.double().cpu()), 0.1)
-        y = f.linear(h, L[4].weight.double().cpu(), L[4].bias.double().cpu()) + f.linear(xd, mlp.lin_direct.weight.double().cpu())
-        if plus_identity:
-            y = y + xd
-        ref = 0.1 * torch.zeros(N, d, dtype=torch.float64).index_add_(0, src, y)
-    torch.testing.assert_close(per_row.cpu().double(), y, rtol=1e-5, atol=2e-6 * float(y.abs().max()))
-    torch.testing.assert_close(got.cpu().double(), ref, rtol=1e-5, atol=3e-6 * float(ref.abs().max()))
+    f = torch.nn.functional
+    L = mlp.layers
+
+    def rows(dt):
+        """The per-row MLP from plain torch modules in dt."""
+        w = lambda t: t.detach().cpu().to(dt)
+        xd = x.cpu().to(dt)
+        h = f.leaky_relu(f.linear(xd, w(L[0].weight), w(L[0].bias)), 0.1)
+        h = f.leaky_relu(f.linear(h, w(L[2].weight), w(L[2].bias)), 0.1)
+        y = f.linear(h, w(L[4].weight), w(L[4].bias)) + f.linear(xd, w(mlp.lin_direct.weight))
+        return y + xd if plus_identity else y
+
+    assert_parity_of(per_row, rows, "MLP per row")
+    assert_parity_of(got, lambda dt: 0.1 * torch.zeros(N, d, dtype=dt).index_add_(0, src, rows(dt)), "MLP summed over rows")
     assert not bool(got[deg.cuda() == 0].any())
 
 
@@ -280,8 +284,6 @@ def test_products_and_output_linears_in_one_kernel(pkg, chan, dims, N):
     P0, P1, P2, nmax = ops.bee_node_products(*dev, want_node_max=True)
     # the oracle's products in the reference layout (rows, chan, 3..)
     to_ref = lambda t, k: t if k == 0 else t.reshape(N, 3 ** k, chan).transpose(1, 2).reshape(N, chan, *([3] * k))
-    prods = dict(zip(OP.BEE_ORDER, OP.bee(*[to_ref(t.double(), k) for k, t in enumerate(l)],
-                                          *[to_ref(t.double(), k) for k, t in enumerate(r)])))
     groups = (("000", "110", "220"), ("011", "101", "121", "211", "111"), ("022", "202", "112", "222", "212"))
     for rank, (labs, P, dim_out) in enumerate(zip(groups, (P0, P1, P2), dims)):
         W = (torch.randn(dim_out, len(labs) * chan, generator=g) / (len(labs) * chan) ** 0.5).cuda()
@@ -292,16 +294,19 @@ def test_products_and_output_linears_in_one_kernel(pkg, chan, dims, N):
             stored = ops.tensor_linear_fwd(0, W, P.reshape(N, 3 * chan))
         else:
             stored = ops.tensor_linear_fwd(rank, W, P.reshape(N, T, len(labs) * chan), x_layout=ops.LAYOUT_COMP_CHAN)
-        ref = sum(torch.einsum("oc,nc...->no...", W[:, k * chan:(k + 1) * chan].double().cpu(), prods[lab])
-                  for k, lab in enumerate(labs))
-        scale = float(ref.abs().max())
-        torch.testing.assert_close(y, stored, rtol=1e-5, atol=3e-6 * scale)
-        torch.testing.assert_close(y.cpu().double(), ref, rtol=1e-5, atol=3e-6 * scale)
-        # rows of small nodes keep their relative accuracy (per-node scales)
+        def ref(dt):
+            pr = dict(zip(OP.BEE_ORDER, OP.bee(*[to_ref(t.to(dt), k) for k, t in enumerate(l)],
+                                               *[to_ref(t.to(dt), k) for k, t in enumerate(r)])))
+            return sum(torch.einsum("oc,nc...->no...", W[:, k * chan:(k + 1) * chan].cpu().to(dt), pr[lab])
+                       for k, lab in enumerate(labs))
+
+        assert_parity_of(y, ref, f"bee_products_linear rank {rank} chan={chan}")
+        assert_parity_of(stored, ref, f"stored products + GEMM rank {rank} chan={chan}")
+        # rows of small nodes keep their relative accuracy (per-node scales): the same bar on those rows alone,
+        # where e_ref is the float32 formula's error on rows of that size
         small = (size[:, 0] < 0.1)
         if bool(small.any()):
-            rs = ref[small]
-            torch.testing.assert_close(y.cpu().double()[small], rs, rtol=1e-5, atol=3e-6 * float(rs.abs().max()))
+            assert_parity_of(y[small.cuda()], lambda dt: ref(dt)[small], f"bee_products_linear rank {rank}, small rows")
 
 
 def test_self_tens_prods_module_fused_path(pkg):
@@ -342,15 +347,14 @@ def test_displacement_sums_kernel(ops, chan, kind):
     row_ptr = ops.segment_row_ptr(src.int().cuda(), N)
     s = 7.0 / 6.0
     A_a, A_v, A_d = ops.displacement_sums(row_ptr, r.cuda(), phi.cuda(), s)
-    u = OL.tens_sigmoid(1, r.double() * s)
-    p = phi.double()
-    ref_a = torch.zeros(N, chan, dtype=torch.float64).index_add_(0, src, p)
-    ref_v = torch.zeros(N, chan, 3, dtype=torch.float64).index_add_(0, src, p[..., None] * u[:, None, :])
-    ref_d = torch.zeros(N, chan, 3, 3, dtype=torch.float64).index_add_(
-        0, src, p[..., None, None] * u[:, None, :, None] * u[:, None, None, :])
-    _close(A_a, ref_a.float(), atol_scale=2e-6)
-    _close(A_v, ref_v.float(), atol_scale=2e-6)
-    _close(A_d, ref_d.float(), atol_scale=2e-6)
+    def sums(dt):
+        u = OL.tens_sigmoid(1, r.to(dt) * s)
+        p = phi.to(dt)
+        return (torch.zeros(N, chan, dtype=dt).index_add_(0, src, p),
+                torch.zeros(N, chan, 3, dtype=dt).index_add_(0, src, p[..., None] * u[:, None, :]),
+                torch.zeros(N, chan, 3, 3, dtype=dt).index_add_(0, src, p[..., None, None] * u[:, None, :, None] * u[:, None, None, :]))
+
+    assert_parity_of((A_a, A_v, A_d), sums, f"displacement_sums chan={chan} {kind}")
     assert not bool(A_a[(deg == 0).cuda()].any()) and not bool(A_d[(deg == 0).cuda()].any())
 
 

@@ -1,18 +1,19 @@
-"""MFMA tensor_linear against the oracle (plain matmul), rel 1e-5 / abs 1e-6
-scaled by the reduction length (fp32 accumulation order differs)."""
+"""MFMA tensor_linear against the oracle (plain matmul): rel 1e-5 / abs 1e-6 against the float64 evaluation, widened
+only by twice the distance of the float32 evaluation of the same formula from it (tests/parity.py)."""
 import importlib
 
 import pytest
 import torch
 
 from oracle import products as OP
+from parity import assert_parity_of
 
 pytestmark = pytest.mark.gpu
 
 
-def _check(y, ref, dim_in):
-    # accumulation-order noise grows like sqrt(K) * eps * |terms|
-    torch.testing.assert_close(y.cpu(), ref, rtol=1e-5, atol=1e-6 * max(1.0, dim_in ** 0.5))
+def _check(y, formula, what="tensor_linear"):
+    """formula(dtype): the reference on the CPU in that dtype."""
+    assert_parity_of(y, formula, what)
 
 
 @pytest.mark.parametrize("inds", [0, 1, 2])
@@ -24,7 +25,7 @@ def test_tensor_linear(ops, inds, dims):
     x = torch.randn(10, 37, dim_in, *([3] * inds), generator=g)
     y = ops.tensor_linear_fwd(inds, W.cuda(), x.cuda())
     assert tuple(y.shape) == (10, 37, dim_out) + (3,) * inds
-    _check(y, OP.tensor_linear(inds, W, x), dim_in)
+    _check(y, lambda dt: OP.tensor_linear(inds, W.to(dt), x.to(dt)))
 
 
 @pytest.mark.parametrize("inds", [0, 1, 2])
@@ -33,7 +34,7 @@ def test_tensor_linear_transposed_weight(ops, inds):
     W = torch.randn(96, 48, generator=g)
     x = torch.randn(50, 96, *([3] * inds), generator=g)
     y = ops.tensor_linear_fwd(inds, W.cuda().t(), x.cuda())
-    _check(y, OP.tensor_linear(inds, W.t(), x), 96)
+    _check(y, lambda dt: OP.tensor_linear(inds, W.t().to(dt), x.to(dt)))
 
 
 def test_tensor_linear_large_rows(ops):
@@ -42,10 +43,10 @@ def test_tensor_linear_large_rows(ops):
     x = torch.randn(3000, 512, generator=g)
     b = torch.randn(512, generator=g)
     y = ops.tensor_linear_fwd(0, W.cuda(), x.cuda(), bias=b.cuda(), act=ops.ACT_SILU)
-    ref = torch.nn.functional.silu(torch.nn.functional.linear(x, W, b))
-    _check(y, ref, 512)
+    lin = lambda dt: torch.nn.functional.linear(x.to(dt), W.to(dt), b.to(dt))
+    _check(y, lambda dt: torch.nn.functional.silu(lin(dt)))
     y2 = ops.tensor_linear_fwd(0, W.cuda(), x.cuda(), bias=b.cuda(), act=ops.ACT_LEAKY)
-    _check(y2, torch.nn.functional.leaky_relu(torch.nn.functional.linear(x, W, b), 0.1), 512)
+    _check(y2, lambda dt: torch.nn.functional.leaky_relu(lin(dt), 0.1))
 
 
 def test_tensor_linear_accumulate(ops):
@@ -55,7 +56,7 @@ def test_tensor_linear_accumulate(ops):
     base = torch.randn(33, 40, 3, generator=g)
     out = base.cuda().clone()
     ops.tensor_linear_fwd(1, W.cuda(), x.cuda(), out=out, accumulate=True)
-    _check(out, base + OP.tensor_linear(1, W, x), 24)
+    _check(out, lambda dt: base.to(dt) + OP.tensor_linear(1, W.to(dt), x.to(dt)))
 
 
 @pytest.mark.parametrize("inds", [0, 1, 2])
@@ -67,27 +68,27 @@ def test_tensor_linear_with_a_few_output_channels(ops, inds, rows, dim_in, dim_o
     T = 3 ** inds
     W = torch.randn(dim_out, dim_in, generator=g) * dim_in ** -0.5
     x = torch.randn(rows, dim_in, *([3] * inds), generator=g)
-    ref = torch.einsum("oi,ri...->ro...", W.double(), x.double())
+    ref = lambda dt: torch.einsum("oi,ri...->ro...", W.to(dt), x.to(dt))
     y = ops.tensor_linear_fwd(inds, W.cuda(), x.cuda())
     assert tuple(y.shape) == (rows, dim_out) + (3,) * inds
-    _check(y, ref.float(), dim_in)
+    _check(y, ref)
     # a weight with strides (the transposed view the input gradient of an n -> few linear would pass is the other
     # shape; this is the forward of a layer whose weight is stored transposed)
     Wt = W.t().contiguous().cuda().t()
     assert dim_out == 1 or Wt.stride() == (1, dim_out)
-    _check(ops.tensor_linear_fwd(inds, Wt, x.cuda()), ref.float(), dim_in)
+    _check(ops.tensor_linear_fwd(inds, Wt, x.cuda()), ref)
     # component-major output
     ycm = ops.tensor_linear_fwd(inds, W.cuda(), x.cuda(), y_layout=ops.LAYOUT_COMP_CHAN)
-    _check(ycm.reshape(rows, T, dim_out), ref.reshape(rows, dim_out, T).transpose(1, 2).float(), dim_in)
+    _check(ycm.reshape(rows, T, dim_out), lambda dt: ref(dt).reshape(rows, dim_out, T).transpose(1, 2))
     # accumulate
     base = torch.randn(rows, dim_out, *([3] * inds), generator=g)
     out = base.cuda().clone()
     ops.tensor_linear_fwd(inds, W.cuda(), x.cuda(), out=out, accumulate=True)
-    _check(out, (base.double() + ref).float(), dim_in)
+    _check(out, lambda dt: base.to(dt) + ref(dt))
     if inds == 0:
         b = torch.randn(dim_out, generator=g)
         yb = ops.tensor_linear_fwd(0, W.cuda(), x.cuda(), bias=b.cuda(), act=ops.ACT_SILU)
-        _check(yb, torch.nn.functional.silu(ref + b.double()).float(), dim_in)
+        _check(yb, lambda dt: torch.nn.functional.silu(ref(dt) + b.to(dt)))
 
 
 def test_tensor_linear_empty_and_errors(ops):
@@ -134,9 +135,10 @@ def test_linear_modes_agree_with_float64(ops, mode, shape):
     W = torch.randn(dim_out, dim_in, generator=g) / dim_in ** 0.5
     b = torch.randn(dim_out, generator=g)
     x_cm = torch.randn(rows, T, dim_in, generator=g)                   # component-major rows
-    ref = (x_cm.double() @ W.double().t() + b.double())
-    ref = torch.nn.functional.silu(ref)                                # (rows, T, O)
-    ref_aos = ref.transpose(1, 2).reshape(rows, dim_out, *([3] * inds))
+    def ref_aos(dt):
+        ref = torch.nn.functional.silu(x_cm.to(dt) @ W.to(dt).t() + b.to(dt))            # (rows, T, O)
+        return ref.transpose(1, 2).reshape(rows, dim_out, *([3] * inds))
+
     prev = ops.get_linear_mode()
     try:
         ops.set_linear_mode(mode)
@@ -145,9 +147,7 @@ def test_linear_modes_agree_with_float64(ops, mode, shape):
                                   bias=b.cuda(), act=ops.ACT_SILU, x_layout=C if inds else 0)
     finally:
         ops.set_linear_mode(prev)
-    err = (y.cpu().double() - ref_aos).abs().max().item()
-    assert err < 2e-6 * max(1.0, dim_in ** 0.5), err
-    torch.testing.assert_close(y.cpu(), ref_aos.float(), rtol=1e-5, atol=1e-6 * dim_in ** 0.5)
+    _check(y, ref_aos, f"tensor_linear mode {mode} {shape}")
 
 
 @pytest.mark.parametrize("shape", [(70000, 512, 512, 1), (3001, 256, 192, 0), (1500, 96, 16, 2), (2048, 1280, 64, 0),
@@ -201,14 +201,14 @@ def test_linear_f16x2_component_outputs_and_node_bounds(ops):
     bound = x.abs().amax(dim=(1, 2)).reshape(nodes, 1)
     y = ops.tensor_linear_f16x2(W.cuda(), x.reshape(nodes * T, dim_in).cuda(), bound.cuda(), out_comps=T,
                                 rows_per_bound=T)
-    ref = (x.double() @ W.double().t()).transpose(1, 2)
+    ref = lambda dt: (x.to(dt) @ W.to(dt).t()).transpose(1, 2)
     assert y.shape == (nodes, dim_out, T)
-    torch.testing.assert_close(y.cpu().double(), ref, rtol=1e-5, atol=2e-6 * dim_in ** 0.5)
+    _check(y, ref, "f16x2, component outputs, one bound per node")
     base = torch.randn(nodes, dim_out, T, generator=g)
     out = base.cuda().clone()
     ops.tensor_linear_f16x2(W.cuda(), x.reshape(nodes * T, dim_in).cuda(), bound.cuda(), out=out, accumulate=True,
                             out_comps=T, rows_per_bound=T)
-    torch.testing.assert_close(out.cpu().double(), base.double() + ref, rtol=1e-5, atol=2e-6 * dim_in ** 0.5)
+    _check(out, lambda dt: base.to(dt) + ref(dt), "f16x2, component outputs, accumulate")
 
 
 def test_linear_out_bound_is_an_upper_bound(ops):
@@ -299,12 +299,13 @@ def test_linear_with_row_sums_in_the_epilogue(ops, dim_in, dim_out, act, kind, w
     else:
         assert y is None
     two_step = 0.5 * ops.segment_sum_csr(y_ref, row_ptr, n_seg)
-    z = x.double().cpu() @ W.double().cpu().T + b.double().cpu()
-    z = torch.nn.functional.silu(z) if act == 1 else (torch.nn.functional.leaky_relu(z, 0.1) if act == 2 else z)
-    ref = 0.5 * torch.zeros(n_seg, dim_out, dtype=torch.float64).index_add_(0, seg, z)
-    scale = float(ref.abs().max())
-    torch.testing.assert_close(out, two_step, rtol=1e-5, atol=2e-6 * scale)
-    torch.testing.assert_close(out.cpu().double(), ref, rtol=1e-5, atol=3e-6 * scale)
+    def ref(dt):
+        z = x.cpu().to(dt) @ W.cpu().to(dt).T + b.cpu().to(dt)
+        z = torch.nn.functional.silu(z) if act == 1 else (torch.nn.functional.leaky_relu(z, 0.1) if act == 2 else z)
+        return 0.5 * torch.zeros(n_seg, dim_out, dtype=dt).index_add_(0, seg, z)
+
+    _check(out, ref, f"row sums in the epilogue {dim_in}->{dim_out} {kind}")
+    _check(two_step, ref, f"GEMM then segment sum {dim_in}->{dim_out} {kind}")
     assert not bool(out[(lengths == 0).cuda()].any())
 
 
@@ -319,14 +320,14 @@ def test_component_major_output_from_reference_layout_at_many_rows(ops, inds, ro
     x = torch.randn(rows, dim_in, *([3] * inds), generator=g).cuda()
     W = (torch.randn(dim_out, dim_in, generator=g) / dim_in ** 0.5).cuda()
     y = ops.tensor_linear_fwd(inds, W, x, y_layout=ops.LAYOUT_COMP_CHAN)
-    ref = torch.einsum("oi,bit->bto", W.double().cpu(), x.double().cpu().reshape(rows, dim_in, T))
+    ref = lambda dt: torch.einsum("oi,bit->bto", W.cpu().to(dt), x.cpu().to(dt).reshape(rows, dim_in, T))
     assert y.shape == (rows, T, dim_out)
-    torch.testing.assert_close(y.cpu().double(), ref, rtol=1e-5, atol=2e-6 * float(ref.abs().max()))
+    _check(y, ref, f"component-major output, {rows} rows")
     y2 = ops.tensor_linear_fwd(inds, W, x, y_layout=ops.LAYOUT_COMP_CHAN, out=y.clone(), accumulate=True)
-    torch.testing.assert_close(y2.cpu().double(), 2 * ref, rtol=1e-5, atol=4e-6 * float(ref.abs().max()))
-    # the same numbers as the generic kernel gives at fewer rows (first rows only)
+    _check(y2, lambda dt: y.cpu().to(dt) + ref(dt), f"component-major output, accumulate, {rows} rows")
+    # the generic kernel, which serves fewer rows, on the first rows
     small = ops.tensor_linear_fwd(inds, W, x[:500].contiguous(), y_layout=ops.LAYOUT_COMP_CHAN)
-    torch.testing.assert_close(y[:500], small, rtol=1e-5, atol=2e-6 * float(ref.abs().max()))
+    _check(small, lambda dt: ref(dt)[:500], "component-major output, generic kernel")
 
 
 def test_linear_with_row_sums_edge_cases(ops):
@@ -341,8 +342,7 @@ def test_linear_with_row_sums_edge_cases(ops):
     seg = torch.zeros(77, dtype=torch.int32, device="cuda")
     row_ptr = torch.tensor([0, 77], dtype=torch.int32, device="cuda")
     out, _ = ops.tensor_linear_f16x2_rowsum(W, x, ops.row_absmax(x), row_ptr, seg, 1)
-    ref = (x.double() @ W.double().T).sum(0, keepdim=True)
-    torch.testing.assert_close(out.double(), ref, rtol=1e-5, atol=3e-6 * float(ref.abs().max()))
+    _check(out, lambda dt: (x.cpu().to(dt) @ W.cpu().to(dt).T).sum(0, keepdim=True), "one segment of 77 rows")
     with pytest.raises(RuntimeError, match="multiple of 256"):
         ops.tensor_linear_f16x2_rowsum(W[:128].contiguous(), x, ops.row_absmax(x), row_ptr, seg, 1)
 
@@ -365,13 +365,14 @@ def test_plain_entry_point_through_ctypes(pkg, inds):
     act = 1 if inds == 0 else 0
     L.check(lib.mg_tensor_linear(inds, Wd.data_ptr(), Wd.stride(1), Wd.stride(0), xd.data_ptr(), 33, 48, 96,
                                  bd.data_ptr() if bd is not None else None, act, 0, yd.data_ptr(), st))
-    ref = OP.tensor_linear(inds, Wt.t(), x)
-    if inds == 0:
-        ref = torch.nn.functional.silu(ref + bias)
-    _check(yd, ref, 48)
+    def ref(dt):
+        lin = OP.tensor_linear(inds, Wt.t().to(dt), x.to(dt))
+        return torch.nn.functional.silu(lin + bias.to(dt)) if inds == 0 else lin
+
+    _check(yd, ref)
     L.check(lib.mg_tensor_linear(inds, Wd.data_ptr(), Wd.stride(1), Wd.stride(0), xd.data_ptr(), 33, 48, 96,
                                  None, 0, 1, yd.data_ptr(), st))
-    _check(yd, ref + OP.tensor_linear(inds, Wt.t(), x), 48)
+    _check(yd, lambda dt: ref(dt) + OP.tensor_linear(inds, Wt.t().to(dt), x.to(dt)))
     before = yd.clone()
     L.check(lib.mg_tensor_linear(inds, Wd.data_ptr(), Wd.stride(1), Wd.stride(0), xd.data_ptr(), 0, 48, 96,
                                  None, 0, 0, yd.data_ptr(), st))

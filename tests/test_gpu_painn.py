@@ -1,8 +1,8 @@
 """PaiNN radial encoding, fused message kernel and Message/Update/Block modules
 against the oracle's restatement of archs/meanflow_painn8.py.
 
-Tolerance: rel 1e-5 / abs 1e-6 per unit of output scale (the sums over ~30-90
-edges and K=512 reductions are evaluated in a different fp32 order)."""
+Tolerance (tests/parity.py): rel 1e-5 / abs 1e-6 against the formula in float64, widened only by twice the distance of
+the same formula evaluated in float32 from it."""
 import importlib
 
 import numpy as np
@@ -11,7 +11,7 @@ import torch
 
 from oracle import layers as OL
 from oracle import neighbour as ON
-from parity import assert_parity
+from parity import assert_parity, assert_parity_of
 
 pytestmark = pytest.mark.gpu
 
@@ -23,9 +23,22 @@ def _to(tree, dtype):
     return tree.to(dtype)
 
 
-def _close(a, ref, rtol=1e-5, atol_scale=1e-6):
-    scale = max(1.0, float(ref.abs().max()))
-    torch.testing.assert_close(a.cpu(), ref, rtol=rtol, atol=atol_scale * scale)
+def _message_formula(src, dst, N, n, r, filt, actv, x_a, x_v, with_res, epsilon=0.1):
+    """The elementwise middle and the two edge sums of Message.forward (archs/meanflow_painn8.py:93-100) for a given
+    per-edge filter (a tensor, or dtype -> tensor), as a function of the dtype it is evaluated in:
+    dtype -> (out_a, out_v)."""
+    def formula(dt):
+        f = filt(dt) if callable(filt) else filt.to(dt)
+        a, xa, xv, rr = (t.to(dt) for t in (actv, x_a, x_v, r))
+        p = f * a[dst]
+        u = rr / torch.sqrt(epsilon + (rr ** 2).sum(-1, keepdim=True))
+        v = xv[dst]
+        m_v = v * p[:, :n, None] + torch.linalg.cross(v, u[:, None].expand_as(v)) * p[:, n:2 * n, None] \
+            + u[:, None] * p[:, 2 * n:3 * n, None]
+        out_v = torch.zeros(N, n, 3, dtype=dt).index_add_(0, src, m_v)
+        out_a = torch.zeros(N, n, dtype=dt).index_add_(0, src, p[:, 3 * n:])
+        return (out_a + xa, out_v + xv) if with_res else (out_a, out_v)
+    return formula
 
 
 def _mlp_weights(mlp):
@@ -103,17 +116,8 @@ def test_fused_message_kernel(ops, n, with_res):
     row_ptr = ops.segment_row_ptr(src.int().cuda(), N)
     out_a, out_v = ops.painn_message(row_ptr, dst.int().cuda(), r.cuda(), filt.cuda(), actv.cuda(), x_v.cuda(), 0.1,
                                      x_a.cuda() if with_res else None, x_v.cuda() if with_res else None)
-    p = filt * actv[dst]
-    u = r / torch.sqrt(0.1 + (r ** 2).sum(-1, keepdim=True))
-    v = x_v[dst]
-    m_v = v * p[:, :n, None] + torch.linalg.cross(v, u[:, None].expand_as(v)) * p[:, n:2 * n, None] \
-        + u[:, None] * p[:, 2 * n:3 * n, None]
-    ref_v = torch.zeros(N, n, 3).index_add_(0, src, m_v)
-    ref_a = torch.zeros(N, n).index_add_(0, src, p[:, 3 * n:])
-    if with_res:
-        ref_v, ref_a = ref_v + x_v, ref_a + x_a
-    _close(out_a, ref_a, atol_scale=2e-6)
-    _close(out_v, ref_v, atol_scale=2e-6)
+    assert_parity_of((out_a, out_v), _message_formula(src, dst, N, n, r, filt, actv, x_a, x_v, with_res),
+                     f"painn_message n={n}")
 
 
 def _degrees(kind, N, g):
@@ -158,27 +162,18 @@ def test_filter_message_fused_with_last_linear(ops, n, hidden, kind, with_res):
     # the same numbers through the stored filter
     filt = ops.tensor_linear_f16x2(dev(W3), dev(h), bound, bias=dev(b3))
     two_a, two_v = ops.painn_message(row_ptr, dev(dst.int()), dev(r), filt, dev(actv), dev(x_v), 0.1, *res)
-    _close(out_a, two_a.cpu(), atol_scale=2e-6)
-    _close(out_v, two_v.cpu(), atol_scale=2e-6)
-    # and plain arithmetic
-    d = lambda t: t.double()
-    p = (d(h) @ d(W3).T + d(b3)) * d(actv)[dst]
-    u = d(r) / torch.sqrt(0.1 + (d(r) ** 2).sum(-1, keepdim=True))
-    v = d(x_v)[dst]
-    m_v = v * p[:, :n, None] + torch.linalg.cross(v, u[:, None].expand_as(v)) * p[:, n:2 * n, None] \
-        + u[:, None] * p[:, 2 * n:3 * n, None]
-    ref_v = torch.zeros(N, n, 3, dtype=torch.float64).index_add_(0, src, m_v)
-    ref_a = torch.zeros(N, n, dtype=torch.float64).index_add_(0, src, p[:, 3 * n:])
-    if with_res:
-        ref_v, ref_a = ref_v + x_v, ref_a + x_a
-    _close(out_a, ref_a.float(), atol_scale=3e-6)
-    _close(out_v, ref_v.float(), atol_scale=3e-6)
+    # all against plain arithmetic: the filter is h W3^T + b3 in the dtype of the evaluation
+    def formula(dt):
+        filt_dt = h.to(dt) @ W3.to(dt).T + b3.to(dt)
+        return _message_formula(src, dst, N, n, r, filt_dt, actv, x_a, x_v, with_res)(dt)
+
+    assert_parity_of((out_a, out_v), formula, f"painn_filter_message n={n} hidden={hidden} {kind}")
+    assert_parity_of((two_a, two_v), formula, f"stored filter + painn_message n={n} hidden={hidden} {kind}")
     # a shared bound for all rows (one row of parts) is accepted as well
     shared = bound.amax().reshape(1, 1)
     sh_a, sh_v = ops.painn_filter_message(W3p, b3p, dev(h), shared, row_ptr, dev(src.int()), dev(dst.int()), dev(r),
                                           dev(actv), dev(x_v), 0.1, *res)
-    _close(sh_a, ref_a.float(), atol_scale=3e-6)
-    _close(sh_v, ref_v.float(), atol_scale=3e-6)
+    assert_parity_of((sh_a, sh_v), formula, f"painn_filter_message, one bound for all rows, n={n}")
 
 
 @pytest.mark.parametrize("n,n_rbf", [(32, None), (128, 16)])
@@ -262,37 +257,36 @@ def test_norm_and_squash_kernels(ops):
     yc = y.cuda()
     out = ops.group_norm(ops.GN_SCALAR, ip.cuda(), 4, gamma.cuda(), beta.cuda(), 1.0, mul=yc[..., chan:2 * chan],
                          add=yc[..., 2 * chan:], res=res.cuda())
-    ref = OL.scal_group_norm(ip * y[..., chan:2 * chan], 4, gamma, beta, 1.0) + y[..., 2 * chan:] + res
-    _close(out, ref, atol_scale=2e-6)
+    assert_parity_of(out, lambda dt: OL.scal_group_norm(ip.to(dt) * y.to(dt)[..., chan:2 * chan], 4, gamma.to(dt),
+                                                        beta.to(dt), 1.0) + y.to(dt)[..., 2 * chan:] + res.to(dt),
+                     "ScalGroupNorm with multiplier, add and residual")
     for inds in (0, 1, 2):
         x = torch.randn(B, N, chan, *([3] * inds)) * 2 + 0.3
         g = torch.randn(chan, *([1] * inds))
         out = ops.group_norm(ops.GN_TENSOR, x.cuda(), 8, g.reshape(-1).cuda(), None, 1e-5)
-        _close(out, OL.tens_group_norm(inds, x, 8, g), atol_scale=2e-6)
-        _close(ops.tens_sigmoid(inds, x.cuda()), OL.tens_sigmoid(inds, x), atol_scale=1e-6)
+        assert_parity_of(out, lambda dt: OL.tens_group_norm(inds, x.to(dt), 8, g.to(dt)), f"TensGroupNorm rank {inds}")
+        assert_parity_of(ops.tens_sigmoid(inds, x.cuda()), lambda dt: OL.tens_sigmoid(inds, x.to(dt)),
+                         f"tens_sigmoid rank {inds}")
 
 
 @pytest.mark.parametrize("kind", [1, 2])
 def test_other_radial_encodings(ops, kind):
-    """sq_radial_encode (archs/diffuser_atoms14.py:32-48) and radial_encode_edge (archs/diffuser_atoms5.py:25-30),
-    restated here in float64 as the check."""
+    """sq_radial_encode (archs/diffuser_atoms14.py:32-48) and radial_encode_edge (archs/diffuser_atoms5.py:25-30)
+    against the oracle's versions (pinned on the CPU by their zeros, special values and a scalar loop)."""
     g = torch.Generator().manual_seed(3)
     r = torch.randn(3000, 3, generator=g) * 3
-    n, rmax = 12, 7.0
+    # rmax = 6 = 2^2 + 1 + 1: lengths whose square is exactly rmax, 6 rmax and rmax / 4 in float32
+    r[:4] = torch.tensor([[0.0, 0.0, 0.0], [2.0, 1.0, 1.0], [0.0, 6.0, 0.0], [1.0, 0.5, 0.5]])
+    n, rmax = 12, 6.0
     out = ops.radial_encode(kind, r.cuda(), n, rmax)
-    rd = r.double()
-    if kind == 1:
-        q = (rd ** 2).sum(-1, keepdim=True) / rmax ** 2
-        coeffs = (torch.pi * 2 ** -0.5) * torch.exp(n ** -0.7 * torch.arange(0, n).double())
-        h = torch.sqrt(1 + q)
-        ref = torch.sin(coeffs * h) * (0.5 ** 0.5 - h)
-        tol = 4 * float((coeffs.max() * h.max())) * 2.0 ** -24 + 2e-6
-    else:
-        npi = torch.pi * torch.arange(0, n).double()
-        x_sq = (rd ** 2).sum(-1) / rmax
-        ref = torch.cos(npi * torch.sqrt(x_sq)[..., None]) * torch.relu(1. - x_sq)[..., None]
-        tol = 4 * float(npi.max() * torch.sqrt(x_sq).max()) * 2.0 ** -24 + 2e-6
-    torch.testing.assert_close(out.cpu().double(), ref, rtol=1e-5, atol=tol)
+    oracle = OL.sq_radial_encode if kind == 1 else OL.radial_encode_edge
+    # the float32 evaluation of the oracle rounds its phases as the kernel does: e_ref is that rounding
+    assert_parity_of(out, lambda dt: oracle(r.to(dt), n, rmax), f"radial_encode kind {kind}")
+    if kind == 2:
+        assert torch.equal(out[0].cpu(), torch.ones(n))              # r = 0
+        assert not bool(out[1].any()) and not bool(out[2].any())     # |r|^2 = rmax and beyond: the envelope's zero
+        want = torch.tensor([1.0, 0.0, -1.0, 0.0] * 3) * 0.75        # |r|^2 = rmax / 4: cos(m pi / 2) 3/4
+        torch.testing.assert_close(out[3].cpu(), want, rtol=0, atol=2e-6)
 
 
 def test_filter_message_without_edges_returns_the_residual(ops):
@@ -327,20 +321,26 @@ def test_first_two_filter_layers_from_edge_vectors(ops, hidden, E):
     y = ops.painn_filter_hidden(r, 8.0, W1, b1, W2, b2, bound1)
     h1 = ops.painn_radial_linear(r, 16, 8.0, W1, b1, ops.ACT_SILU)
     two = ops.tensor_linear_f16x2(W2, h1, bound1, bias=b2, act=ops.ACT_SILU)
-    enc = OL.radial_encode_painn(r.cpu().double(), 16, 8.0)
     f = torch.nn.functional
-    ref = f.silu(f.linear(f.silu(f.linear(enc, W1.double().cpu(), b1.double().cpu())), W2.double().cpu(), b2.double().cpu()))
-    scale = float(ref.abs().max())
-    torch.testing.assert_close(y, two, rtol=1e-5, atol=3e-6 * scale)
-    torch.testing.assert_close(y.cpu().double(), ref, rtol=1e-5, atol=4e-6 * scale)
+
+    def formula(dt):
+        # in float32 the encoding carries the rounding of its phase, as the reference's does: part of e_ref
+        enc = OL.radial_encode_painn(r.cpu().to(dt), 16, 8.0)
+        w = [t.cpu().to(dt) for t in (W1, b1, W2, b2)]
+        return f.silu(f.linear(f.silu(f.linear(enc, w[0], w[1])), w[2], w[3]))
+
+    assert_parity_of(y, formula, f"painn_filter_hidden {hidden} x {E}")
+    assert_parity_of(two, formula, f"radial_linear + GEMM {hidden} x {E}")
 
 
 @pytest.mark.parametrize("n,rows", [(128, 256), (32, 512), (20, 256)])
 def test_table_message_kernel_interpolates_a_known_periodic_filter(ops, n, rows):
-    """mg_painn_table_message with a table of an analytic filter, cos(m pi d / r0 + phase) per column with m <= 3,
-    against mg_painn_message fed with that filter evaluated per edge in float64.  Edge lengths run from 0 to beyond
-    two periods, so the wrap of the row index and the interval [rows - 1, rows) are covered.  4-point Lagrange error
-    bound: 0.0234 h^4 (3 pi / r0)^4 = 7e-7 at h = 2 r0 / 256, r0 = 4."""
+    """mg_painn_table_message with a table of an analytic filter, amp cos(m pi d / r0 + phase) per column, against
+    the layer's formula fed with that filter evaluated at every edge's length.  m is at most 1 for 256 rows and at
+    most 2 for 512, so that the 4-point Lagrange error, at most 0.0234 h^4 (m pi / r0)^4 = 9e-9 per unit of
+    amplitude at h = 2 r0 / rows, r0 = 4, is below the float32 rounding of the filter itself (a 2-point
+    interpolation would err by h^2 / 8 (m pi / r0)^2 = 8e-5 and fail).  Edge lengths run from 0 to beyond two periods,
+    so the wrap of the row index and the interval [rows - 1, rows) are covered."""
     g = torch.Generator().manual_seed(n + rows)
     r0, N = 4.0, 300
     deg = torch.randint(0, 40, (N,), generator=g)
@@ -351,21 +351,23 @@ def test_table_message_kernel_interpolates_a_known_periodic_filter(ops, n, rows)
     length[:4] = torch.tensor([0.0, 2 * r0, 2 * r0 * (1 - 1e-7), 2 * r0 * (rows - 0.5) / rows])
     direction = torch.randn(E, 3, generator=g).double()
     r = (direction / direction.norm(dim=-1, keepdim=True) * length[:, None]).float()
-    m = torch.randint(0, 4, (4 * n,), generator=g).double()
+    m = torch.randint(0, 2 if rows == 256 else 3, (4 * n,), generator=g).double()
     phase = torch.rand(4 * n, generator=g).double() * 6.28
     amp = torch.randn(4 * n, generator=g).double()
-    f = lambda d: amp * torch.cos(m * (torch.pi / r0) * d[:, None] + phase)
+    f = lambda d: amp.to(d.dtype) * torch.cos(m.to(d.dtype) * (torch.pi / r0) * d[:, None] + phase.to(d.dtype))
     table = f(torch.arange(rows).double() * (2 * r0 / rows)).float()
-    filt = f(r.double().norm(dim=-1)).float()                # at the float32 edge vectors the kernel sees
+    # the filter of every edge, evaluated in the dtype of the check from the float32 edge vectors the kernel sees
+    # (in float32 it carries the rounding of its phase, as any float32 evaluation of a filter does)
+    exact = lambda dt: f(r.to(dt).norm(dim=-1))
     actv = torch.randn(N, 4 * n, generator=g)
     x_a, x_v = torch.randn(N, n, generator=g), torch.randn(N, n, 3, generator=g)
     dev = lambda t: t.cuda()
     row_ptr = ops.segment_row_ptr(dev(src.int()), N)
     got_a, got_v = ops.painn_table_message(row_ptr, dev(dst.int()), dev(r), dev(table), 2 * r0, dev(actv), dev(x_v), 0.1,
                                            dev(x_a), dev(x_v))
-    ref_a, ref_v = ops.painn_message(row_ptr, dev(dst.int()), dev(r), dev(filt), dev(actv), dev(x_v), 0.1, dev(x_a), dev(x_v))
-    _close(got_a, ref_a.cpu(), atol_scale=3e-6)
-    _close(got_v, ref_v.cpu(), atol_scale=3e-6)
+    with_res = _message_formula(src, dst, N, n, r, exact, actv, x_a, x_v, True)
+    without = _message_formula(src, dst, N, n, r, exact, actv, x_a, x_v, False)
+    assert_parity_of((got_a, got_v), with_res, f"painn_table_message n={n} rows={rows}")
     with pytest.raises(RuntimeError, match="power of two"):
         ops.painn_table_message(row_ptr, dev(dst.int()), dev(r), dev(table[:rows - 1].contiguous()), 2 * r0, dev(actv),
                                 dev(x_v), 0.1)
@@ -375,12 +377,10 @@ def test_table_message_kernel_interpolates_a_known_periodic_filter(ops, n, rows)
         assert torch.equal(torch.sort(perm).values, torch.arange(4 * n, device="cuda"))
         sl_a, sl_v = ops.painn_table_message_sliced(row_ptr, dev(dst.int()), dev(r), dev(table), 2 * r0,
                                                     dev(actv)[:, perm].contiguous(), dev(x_v), 0.1, dev(x_a), dev(x_v))
-        _close(sl_a, ref_a.cpu(), atol_scale=3e-6)
-        _close(sl_v, ref_v.cpu(), atol_scale=3e-6)
+        assert_parity_of((sl_a, sl_v), with_res, f"painn_table_message_sliced n={n} rows={rows}")
         no_a, no_v = ops.painn_table_message_sliced(row_ptr, dev(dst.int()), dev(r), dev(table), 2 * r0,
                                                     dev(actv)[:, perm].contiguous(), dev(x_v), 0.1)
-        _close(no_a, (ref_a - dev(x_a)).cpu(), atol_scale=3e-6)
-        _close(no_v, (ref_v - dev(x_v)).cpu(), atol_scale=3e-6)
+        assert_parity_of((no_a, no_v), without, f"painn_table_message_sliced without residual n={n} rows={rows}")
         # rows processed in another order, records passed in by the caller: same bits
         order = torch.randperm(N, generator=g).int().cuda()
         records = ops.painn_edge_records(dev(r), rows, 2 * r0, 0.1)
@@ -393,10 +393,20 @@ def test_table_message_kernel_interpolates_a_known_periodic_filter(ops, n, rows)
                                            dev(actv), dev(x_v), 0.1)
 
 
+def _message_oracle(msg, src, dst, N, x_a, x_v, r, residual):
+    """dtype -> OL.painn_message for the module's weights (+ the residual), inputs on the CPU."""
+    def formula(dt):
+        da, dv = OL.painn_message(src, dst, 1, N, x_a.to(dt), x_v.to(dt), r.to(dt), _to(_mlp_weights(msg.mlp_dist), dt),
+                                  _to(_mlp_weights(msg.mlp_actv), dt), msg.r0, msg.n, msg.n_rbf)
+        return (x_a.to(dt) + da, x_v.to(dt) + dv) if residual else (da, dv)
+    return formula
+
+
 @pytest.mark.parametrize("n_rbf", [16, None])
-def test_message_with_filter_table_equals_filter_mlp_per_edge(pkg, n_rbf):
-    """Message.forward through the grid of the filter against the same module evaluating the filter MLP on every
-    edge, on edge vectors of any length (the filter has period 2 r0 in the length)."""
+def test_message_with_filter_table_and_with_filter_mlp_per_edge_against_the_oracle(pkg, n_rbf):
+    """Message.forward through the grid of the filter (held in LDS, read through the caches) and with the filter MLP
+    on every edge, each against the oracle in float64 at the layer tolerance, on edge vectors of any length (the
+    filter has period 2 r0 in the length)."""
     painn = importlib.import_module("learned-dynamics_amd.painn")
     torch.manual_seed(7)
     n, N, r0 = 64, 512, 6.0
@@ -410,19 +420,74 @@ def test_message_with_filter_table_equals_filter_mlp_per_edge(pkg, n_rbf):
     r[0] = 0.0
     gl = importlib.import_module("learned-dynamics_amd.graph_layers")
     graph = gl.Graph(src.cuda(), dst.cuda(), None, 1, N)
-    x_a, x_v = torch.randn(1, N, n).cuda(), torch.randn(1, N, n, 3).cuda()
+    x_a, x_v = torch.randn(1, N, n), torch.randn(1, N, n, 3)
     with torch.no_grad():
         rows = msg.table_rows()
         assert rows in msg.TABLE_ROWS and E >= 4 * rows
-        a1, v1 = msg(graph, x_a, x_v, r.cuda(), residual=True)       # grid in LDS when 512 rows are enough
+        a1, v1 = msg(graph, x_a.cuda(), x_v.cuda(), r.cuda(), residual=True)       # grid in LDS when 512 rows are enough
         msg.use_sliced = False
-        a2, v2 = msg(graph, x_a, x_v, r.cuda(), residual=True)       # grid read through the caches
+        a2, v2 = msg(graph, x_a.cuda(), x_v.cuda(), r.cuda(), residual=True)       # grid read through the caches
         msg.use_table = False
-        a0, v0 = msg(graph, x_a, x_v, r.cuda(), residual=True)
+        a0, v0 = msg(graph, x_a.cuda(), x_v.cuda(), r.cuda(), residual=True)
     assert float(r.norm(dim=-1).max()) > 2 * r0
-    for a, v in ((a1, v1), (a2, v2)):
-        _close(a, a0.cpu(), atol_scale=3e-6)
-        _close(v, v0.cpu(), atol_scale=3e-6)
+    oracle = _message_oracle(msg, src, dst, N, x_a, x_v, r, True)
+    for name, pair in (("grid in LDS", (a1, v1)), ("grid through the caches", (a2, v2)), ("MLP per edge", (a0, v0))):
+        assert_parity_of(pair, oracle, f"Message n_rbf={n_rbf}, {rows} rows, {name}")
+
+
+def _scale_first_filter_layer(msg, factor):
+    with torch.no_grad():
+        msg.mlp_dist.layers[0].weight.mul_(factor)
+        msg.mlp_dist.layers[0].bias.mul_(factor)
+
+
+@pytest.mark.parametrize("rows,side", [(512, "below"), (512, "above"), (2048, "below"), (2048, "above")])
+def test_filter_grid_acceptance_at_its_threshold(pkg, rows, side):
+    """The first layer of the filter MLP is scaled up (a rougher filter) until the interpolation error of the grid of
+    `rows` rows sits at the acceptance threshold (bisection on Message.table_error), then 3 % below or above it.
+    Below, the grid of `rows` rows is accepted; above, it is refused and the next size is taken.  Either way the
+    layer is held to the layer tolerance against the float64 oracle, with nothing added for the grid."""
+    painn = importlib.import_module("learned-dynamics_amd.painn")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    torch.manual_seed(0x947 + rows)
+    n, r0, box = 64, 8.0, (40., 40., 40.)
+    msg = painn.Message(r0, n, 16).cuda()
+    first = msg.mlp_dist.layers[0]
+    W0, b0 = first.weight.detach().clone(), first.bias.detach().clone()
+
+    def error_at(factor):
+        with torch.no_grad():
+            first.weight.copy_(W0 * factor)
+            first.bias.copy_(b0 * factor)
+            return float(msg.table_error(rows))
+
+    lo, hi = 1.0, 1.0
+    assert error_at(lo) < 1.0
+    while error_at(hi) < 1.0:
+        hi *= 2.0
+        assert hi < 1e4
+    for _ in range(30):
+        mid = (lo * hi) ** 0.5
+        lo, hi = (mid, hi) if error_at(mid) < 1.0 else (lo, mid)
+    factor = lo * (0.97 if side == "below" else 1.03)
+    err = error_at(factor)
+    print(f"[grid threshold] rows {rows} {side}: first layer x {factor:.3f}, table_error {err:.3f}")
+    assert (0.5 < err < 1.0) if side == "below" else (1.0 < err < 2.0)
+    chosen = msg.table_rows()
+    bigger = msg.TABLE_ROWS[msg.TABLE_ROWS.index(rows) + 1]
+    assert chosen == (rows if side == "below" else bigger)
+    pos = _polymer(4, 256, 40., 0x947 + 5)
+    N = 1024
+    x_a, x_v = torch.randn(1, N, n), torch.randn(1, N, n, 3) / 3 ** 0.5
+    with torch.no_grad():
+        graph, r_ij = gl.graph_setup(r0, box, pos.cuda(), neighbours_max=256, celllist_max=64)
+        assert r_ij.shape[0] >= 4 * chosen                  # so that the grid path is the one that runs
+        got = msg(graph, x_a.cuda(), x_v.cuda(), r_ij)
+        msg.use_table = False
+        per_edge = msg(graph, x_a.cuda(), x_v.cuda(), r_ij)
+    oracle = _message_oracle(msg, graph.src.cpu(), graph.dst.cpu(), N, x_a, x_v, r_ij.cpu(), False)
+    assert_parity_of(got, oracle, f"Message at the grid threshold, {chosen} rows ({side} the threshold of {rows})")
+    assert_parity_of(per_edge, oracle, f"Message at the same weights, filter MLP on every edge")
 
 
 def test_table_message_kernels_without_edges_return_the_residual(ops):
@@ -472,7 +537,7 @@ def test_update_elementwise_kernels_in_both_layouts(ops, rows, n):
     for lay in (lrv.cuda(), lrv.permute(0, 2, 1).contiguous().cuda()):
         ip, cat = ops.painn_update_pre(lay, x_a.cuda())
         out_v = ops.painn_update_vec(lay, y.cuda(), res.cuda())
-        torch.testing.assert_close(ip.cpu().double(), want_ip, rtol=1e-5, atol=1e-5)
+        torch.testing.assert_close(ip.cpu().double(), want_ip, rtol=1e-5, atol=2e-6)
         torch.testing.assert_close(cat.cpu().double(), want_cat, rtol=1e-5, atol=1e-6)
         torch.testing.assert_close(out_v.cpu().double(), want_v, rtol=1e-5, atol=1e-6)
         outs.append((ip, cat, out_v))

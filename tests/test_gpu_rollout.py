@@ -161,6 +161,46 @@ def test_captured_forward_including_the_neighbour_search(pkg):
     assert len(counts) == 4
 
 
+def test_capacity_below_the_edge_count_gives_the_truncated_graph(pkg, ops):
+    """Edge arrays smaller than the graph: the search drops the edges that do not fit AND lowers the row pointers to
+    the capacity, so the layers (which walk the edges through row_ptr) see exactly the graph cut at `capacity` edges
+    and never read past the arrays; stats keeps the true count and flags the loss."""
+    painn = importlib.import_module("learned-dynamics_amd.painn")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    torch.manual_seed(0x947 + 6)
+    B, N, L_box, r0, n = 2, 1024, 40.0, 8.0, 64
+    box = (L_box,) * 3
+    x = _chain(B, N, L_box, 17)
+    msg = painn.Message(r0, n, 16).cuda().eval()
+    x_a, x_v = torch.randn(B, N, n, device="cuda"), torch.randn(B, N, n, 3, device="cuda") / 3 ** 0.5
+    with torch.no_grad():
+        exact, r_exact = gl.graph_setup(r0, box, x, neighbours_max=512, celllist_max=128)
+    E0 = int(exact.src.numel())
+    for capacity in (E0 - 1, (2 * E0) // 3, 4 * msg.TABLE_ROWS[0]):
+        assert 4 * msg.TABLE_ROWS[0] <= capacity < E0
+        with torch.no_grad():
+            graph, r_ij = gl.graph_setup_capacity(r0, box, x, capacity)
+            got_a, got_v = msg(graph, x_a, x_v, r_ij)
+        stats = graph.stats.cpu()
+        assert int(stats[0]) == E0 and int(stats[3]) & 2
+        row_ptr = graph.row_ptr.cpu()
+        assert torch.equal(row_ptr, exact.row_ptr.cpu().clamp(max=capacity))
+        assert int(row_ptr[-1]) == capacity and int(row_ptr.max()) == capacity
+        assert torch.equal(graph.src32[:capacity], exact.src32[:capacity])
+        assert torch.equal(graph.dst32[:capacity], exact.dst32[:capacity])
+        assert torch.equal(graph.edge_indices, exact.edge_indices.clamp(max=capacity))
+        # the same layer on a graph built from the first `capacity` edges
+        cut = gl.Graph(exact.src[:capacity].contiguous(), exact.dst[:capacity].contiguous(), None, B, N)
+        cut.cell_order = graph.cell_order
+        with torch.no_grad():
+            ref_a, ref_v = msg(cut, x_a, x_v, r_exact[:capacity].contiguous())
+        assert torch.equal(got_a, ref_a) and torch.equal(got_v, ref_v)
+    # enough room: nothing flagged, nothing lowered
+    with torch.no_grad():
+        graph, _ = gl.graph_setup_capacity(r0, box, x, E0)
+    assert int(graph.stats[3]) == 0 and torch.equal(graph.row_ptr, exact.row_ptr)
+
+
 def test_concurrent_sections_inside_a_capture(pkg):
     """ops.concurrent: independent pieces of a layer on side streams while a HIP graph is being captured (fork and join
     events become dependencies of the graph), in turn otherwise.  Two sections in a row that hand tensors to each other,

@@ -54,6 +54,74 @@ def test_radial_encode_painn_closed_form():
     assert torch.allclose(enc, expect)
 
 
+def test_sq_radial_encode_zeros_special_values_and_scalar_loop():
+    """archs/diffuser_atoms14.py:32-48.  Column m is sin(c_m h)(sqrt(1/2) - h) with h = sqrt(1 + |r|^2 / rmax^2) and
+    c_m = (pi / sqrt 2) exp(m n^-0.7): it vanishes where c_m h is a multiple of pi, which pins c_m and the
+    normalisation of the length without restating the product."""
+    n, rmax = 4, 7.0
+    D = torch.float64
+    # r = 0: h = 1, value sin(c_m) (sqrt(1/2) - 1)
+    at0 = OL.sq_radial_encode(torch.zeros(1, 3, dtype=D), n, rmax)[0]
+    for m in range(n):
+        c = math.pi / math.sqrt(2.0) * math.exp(m * n ** -0.7)
+        assert abs(float(at0[m]) - math.sin(c) * (math.sqrt(0.5) - 1.0)) < 1e-14
+    # |r| = rmax: h = sqrt 2, c_0 h = pi, so column 0 vanishes; |r| = sqrt(7) rmax: h = 2 sqrt 2, c_0 h = 2 pi
+    for length in (rmax, math.sqrt(7.0) * rmax):
+        e = OL.sq_radial_encode(torch.tensor([[0.0, length, 0.0]], dtype=D), n, rmax)[0]
+        assert abs(float(e[0])) < 1e-13
+        assert abs(float(e[1])) > 1e-2                       # the other columns do not vanish there
+    # column m vanishes at h = k sqrt(2) exp(-m n^-0.7) for integer k (taken where h >= 1)
+    for m, k in ((1, 2), (2, 2), (3, 3), (3, 4)):
+        h = k * math.sqrt(2.0) * math.exp(-m * n ** -0.7)
+        assert h > 1.0
+        length = rmax * math.sqrt(h * h - 1.0)
+        e = OL.sq_radial_encode(torch.tensor([[length, 0.0, 0.0]], dtype=D), n, rmax)[0]
+        assert abs(float(e[m])) < 1e-12, (m, k, float(e[m]))
+    # the envelope alone: where sin(c_m h) = +-1 the value is +-(sqrt(1/2) - h); c_0 h = pi / 2 needs h < 1, so take
+    # c_0 h = 3 pi / 2: h = 3 / sqrt 2
+    h = 3.0 / math.sqrt(2.0)
+    e = OL.sq_radial_encode(torch.tensor([[0.0, 0.0, rmax * math.sqrt(h * h - 1.0)]], dtype=D), n, rmax)[0]
+    assert abs(float(e[0]) - (-1.0) * (math.sqrt(0.5) - h)) < 1e-13
+    # a scalar loop over (edge, column) on leading dims of different sizes
+    g = torch.Generator().manual_seed(5)
+    r = torch.randn(3, 5, 3, generator=g, dtype=D) * 4
+    enc = OL.sq_radial_encode(r, 6, 5.5)
+    assert enc.shape == (3, 5, 6)
+    for a in range(3):
+        for b in range(5):
+            x, y, z = (float(v) for v in r[a, b])
+            h = math.sqrt(1.0 + (x * x + y * y + z * z) / (5.5 * 5.5))
+            for m in range(6):
+                c = math.pi / math.sqrt(2.0) * math.exp(m * 6 ** -0.7)
+                assert abs(float(enc[a, b, m]) - math.sin(c * h) * (math.sqrt(0.5) - h)) < 1e-12
+
+
+def test_radial_encode_edge_special_values_and_scalar_loop():
+    """archs/diffuser_atoms5.py:25-30.  x = |r|^2 / rmax (the reference divides the squared length by rmax, not by
+    rmax^2): all columns are 1 at r = 0, 0 from |r|^2 = rmax on, and cos(m pi / 2) 3/4 at |r|^2 = rmax / 4."""
+    n, rmax = 6, 7.0
+    D = torch.float64
+    assert torch.equal(OL.radial_encode_edge(torch.zeros(2, 3, dtype=D), n, rmax), torch.ones(2, n, dtype=D))
+    edge = torch.tensor([[math.sqrt(rmax), 0.0, 0.0], [0.0, 1.5 * math.sqrt(rmax), 0.0], [0.0, 0.0, rmax]], dtype=D)
+    at_zero = OL.radial_encode_edge(edge, n, rmax)
+    assert float(at_zero.abs().max()) < 1e-15              # |r|^2 >= rmax; with rmax^2 in the quotient none would vanish
+    inside = OL.radial_encode_edge(torch.tensor([[0.0, 0.99 * math.sqrt(rmax), 0.0]], dtype=D), n, rmax)
+    assert float(inside[0, 0]) > 1e-3                      # cos(0) (1 - 0.98): open just inside the envelope's zero
+    quarter = OL.radial_encode_edge(torch.tensor([[0.0, 0.0, 0.5 * math.sqrt(rmax)]], dtype=D), n, rmax)[0]
+    want = torch.tensor([1.0, 0.0, -1.0, 0.0, 1.0, 0.0], dtype=D) * 0.75
+    assert float((quarter - want).abs().max()) < 1e-15
+    g = torch.Generator().manual_seed(6)
+    r = torch.randn(4, 3, 3, generator=g, dtype=D)
+    enc = OL.radial_encode_edge(r, 5, 3.0)
+    assert enc.shape == (4, 3, 5)
+    for a in range(4):
+        for b in range(3):
+            x, y, z = (float(v) for v in r[a, b])
+            xs = (x * x + y * y + z * z) / 3.0
+            for m in range(5):
+                assert abs(float(enc[a, b, m]) - math.cos(m * math.pi * math.sqrt(xs)) * max(0.0, 1.0 - xs)) < 1e-13
+
+
 def test_tens_sigmoid_norm_and_direction():
     x = torch.randn(5, 4, 3, 3, dtype=torch.float64)
     y = OL.tens_sigmoid(2, x)
