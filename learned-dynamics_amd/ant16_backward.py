@@ -8,7 +8,12 @@ types) the forward is  y[b,o,O] = sum_{l,i,L,X} P[o,l,i] T[L,X,O] left[b,l,L] x[
     dleft[b,l,L] = sum_{o,i,X,O} P[o,l,i] T[L,X,O] x[b,i,X] dy[b,o,O]          ("backleft")
     dP[o,l,i]    = sum_{b,L,X,O} T[L,X,O] left[b,l,L] x[b,i,X] dy[b,o,O]       ("wtsback")
 The first two run on the forward kernel with the roles of the channel axes of P permuted, the third is a
-contraction over rows with an ordered (deterministic) reduction."""
+contraction over rows with an ordered (deterministic) reduction.
+
+These are raw kernels, not autograd functions: Ant16 is differentiable ONCE, as the reference's is (its backward
+also calls kernels); codegen_tensor_products.Ant16.backward is marked once_differentiable, so a second derivative
+(a double backward, or jvp(create_graph=True) followed by backward) raises instead of silently treating these
+gradients as constants.  Bee, the linears and the PaiNN layers are differentiable to any order."""
 import torch
 
 from . import ops
@@ -77,3 +82,33 @@ def oc_backleft(x_1, x_2, dy_1, dy_2, P_111, P_212):
 
 def oc_wtsback(x_1, x_2, dy_1, dy_2, left_111, left_212):
     return [grad_P("111", dy_1, left_111, x_1), grad_P("212", dy_2, left_212, x_1)]
+
+
+# The reference's generated example with nine product types of mixed output rank (fused_tensor_prods_example{,_backward,
+# _backleft,_wtsback}_cuda: extensions/codegen_tensops/do_codegen.py:4-7, codegen_tensops.cpp:158-608, bound at
+# :1981-1984; exercised by extensions/codegen_tensops/test.py:29-39).  Same contraction as Ant16, so the same kernels:
+# one forward launch per output rank, one gradient launch per rank of x, one per left / P.
+EXAMPLE = ("000", "011", "101", "110", "220", "222", "211", "111", "212")
+
+
+def example_forward(x_0, x_1, x_2, *P_left):
+    """fused_tensor_prods_example_cuda(x_0, x_1, x_2, P_000, left_000, P_011, left_011, ...) -> [y_0, y_1, y_2]."""
+    terms = [(lab, P_left[2 * k], P_left[2 * k + 1]) for k, lab in enumerate(EXAMPLE)]
+    return [ops._ant16(rank, x_0, x_1, x_2, [t for t in terms if int(t[0][2]) == rank]) for rank in range(3)]
+
+
+def example_backward(dy_0, dy_1, dy_2, *P_left):
+    """fused_tensor_prods_example_backward_cuda(dy_0, dy_1, dy_2, P_000, left_000, ...) -> [dx_0, dx_1, dx_2]."""
+    return grad_x_all([dy_0, dy_1, dy_2], [(lab, P_left[2 * k], P_left[2 * k + 1]) for k, lab in enumerate(EXAMPLE)])
+
+
+def example_backleft(x_0, x_1, x_2, dy_0, dy_1, dy_2, *Ps):
+    """fused_tensor_prods_example_backleft_cuda(x_0, x_1, x_2, dy_0, dy_1, dy_2, P_000, P_011, ...) -> nine dleft."""
+    xs, dys = (x_0, x_1, x_2), (dy_0, dy_1, dy_2)
+    return [grad_left(lab, dys[int(lab[2])], P, xs[int(lab[1])]) for lab, P in zip(EXAMPLE, Ps)]
+
+
+def example_wtsback(x_0, x_1, x_2, dy_0, dy_1, dy_2, *lefts):
+    """fused_tensor_prods_example_wtsback_cuda(x_0, x_1, x_2, dy_0, dy_1, dy_2, left_000, left_011, ...) -> nine dP."""
+    xs, dys = (x_0, x_1, x_2), (dy_0, dy_1, dy_2)
+    return [grad_P(lab, dys[int(lab[2])], left, xs[int(lab[1])]) for lab, left in zip(EXAMPLE, lefts)]

@@ -22,13 +22,6 @@ def set_kern_attributes():
     return None
 
 
-def _unavailable(name):
-    def fn(*args, **kwargs):
-        raise NotImplementedError(f"{name}: the reference's worked example kernel is not part of this library")
-    fn.__name__ = name
-    return fn
-
-
 ant16_o0_cuda = _ops.ant16_o0
 ant16_o1_cuda = _ops.ant16_o1
 ant16_o2_cuda = _ops.ant16_o2
@@ -51,6 +44,8 @@ for _o in ("o0", "o1", "o2"):
 ant16_oc_backward_cuda = _checked("ant16_oc_backward_cuda", _a16.oc_backward)
 ant16_oc_backleft_cuda = _checked("ant16_oc_backleft_cuda", _a16.oc_backleft)
 ant16_oc_wtsback_cuda = _checked("ant16_oc_wtsback_cuda", _a16.oc_wtsback)
-for _suffix in ("", "_backward", "_backleft", "_wtsback"):
-    _name = f"fused_tensor_prods_example{_suffix}_cuda"
-    globals()[_name] = _unavailable(_name)
+# the generated example with nine product types of mixed output rank (codegen_tensops.cpp:1981-1984)
+fused_tensor_prods_example_cuda = _checked("fused_tensor_prods_example_cuda", _a16.example_forward)
+fused_tensor_prods_example_backward_cuda = _checked("fused_tensor_prods_example_backward_cuda", _a16.example_backward)
+fused_tensor_prods_example_backleft_cuda = _checked("fused_tensor_prods_example_backleft_cuda", _a16.example_backleft)
+fused_tensor_prods_example_wtsback_cuda = _checked("fused_tensor_prods_example_wtsback_cuda", _a16.example_wtsback)

@@ -137,14 +137,48 @@ class TensorProdBare(nn.Module):
 
     def forward(self, x_l, x_r):
         if torch.is_grad_enabled() and (x_l.requires_grad or x_r.requires_grad):
-            return _prod_with_grad(self.inds, x_l, x_r)
+            return _ProdBareFn.apply(*self.inds, x_l, x_r)
         return ops.tensor_prod_bare(*self.inds, x_l.contiguous(), x_r.contiguous())
 
 
+def _swap_index_groups(x, first, second):
+    """x (..., chan, (3,)^(first + second)) with its trailing indices in two groups: the groups exchanged.  With
+    ranks up to 2 that is a transposition when both groups hold one index, and nothing otherwise."""
+    return x.transpose(-1, -2).contiguous() if first == 1 and second == 1 else x
+
+
+class _ProdBareFn(torch.autograd.Function):
+    """One product y[keep_l, keep_r] = sum_con l[keep_l, con] r[keep_r, con] (the reference relies on
+    torch.einsum's autograd, managan/tensor_products.py:104-106).  Both gradients are products of the same family
+    with index groups exchanged,
+        dl[keep_l, con] = sum_keep_r dy[keep_l, keep_r] r[keep_r, con]     type (inds_o, inds_r, inds_l)
+        dr[keep_r, con] = sum_keep_l dy[keep_l, keep_r] l[keep_l, con]     type (inds_o, inds_l, inds_r)
+    and they are taken through this function again, so the product is differentiable any number of times at the
+    cost of one product kernel per gradient."""
+
+    @staticmethod
+    def forward(ctx, il, ir, io, x_l, x_r):
+        ctx.inds = (il, ir, io)
+        ctx.save_for_backward(x_l, x_r)
+        return ops.tensor_prod_bare(il, ir, io, x_l.contiguous(), x_r.contiguous())
+
+    @staticmethod
+    def backward(ctx, dy):
+        il, ir, io = ctx.inds
+        k = (il + ir - io) // 2                       # contracted indices; il - k and ir - k are kept
+        x_l, x_r = ctx.saved_tensors
+        dl = dr = None
+        if ctx.needs_input_grad[3]:
+            dl = _ProdBareFn.apply(io, ir, il, dy, _swap_index_groups(x_r, ir - k, k))
+        if ctx.needs_input_grad[4]:
+            dr = _ProdBareFn.apply(io, il, ir, _swap_index_groups(dy, il - k, ir - k), _swap_index_groups(x_l, il - k, k))
+        return None, None, None, dl, dr
+
+
 def _prod_with_grad(inds, x_l, x_r):
-    """The product through the 13-product autograd function (the reference relies on torch.einsum's autograd,
-    managan/tensor_products.py:104-106): the operands take their ranks' slots, the other slots are zeros, and the
-    output of type (inds_l inds_r inds_o) is picked.  Differentiable any number of times, like Bee."""
+    """The product through the 13-product autograd function: the operands take their ranks' slots, the other slots
+    are zeros, and the output of type (inds_l inds_r inds_o) is picked.  Ten times the arithmetic of _ProdBareFn;
+    kept as an independent route that the tests compare it with."""
     from .codegen_tensor_products import Bee
     il, ir, io = inds
     lead = x_l.shape[:x_l.dim() - il - 1]

@@ -267,6 +267,34 @@ def test_tensor_prods_module_trains(lro):
         torch.testing.assert_close(a.detach().cpu().double(), r.detach(), rtol=2e-4, atol=2e-5 * float(r.abs().max()) + 1e-9)
 
 
+@pytest.mark.parametrize("lro", [(0, 0, 0), (1, 1, 0), (2, 2, 0), (0, 1, 1), (1, 0, 1), (1, 2, 1), (2, 1, 1),
+                                 (0, 2, 2), (2, 0, 2), (1, 1, 2), (2, 2, 2)])
+def test_one_product_autograd_function(lro):
+    """TensorProdBare with gradients (one product kernel per gradient, tensor_products._ProdBareFn): first derivatives
+    for both operands and the gradient of a gradient norm, against autograd through the oracle's einsum in float64 and
+    against the route through the 13-product function."""
+    tp = importlib.import_module("learned-dynamics_amd.tensor_products")
+    il, ir, io = lro
+    g = torch.Generator().manual_seed(40 + 9 * il + 3 * ir + io)
+    x_l = torch.randn(5, 6, 24, *([3] * il), generator=g)
+    x_r = torch.randn(5, 6, 24, *([3] * ir), generator=g)
+    cot = torch.randn(5, 6, 24, *([3] * io), generator=g)
+    ld, rd = x_l.double().requires_grad_(), x_r.double().requires_grad_()
+    ref = torch.autograd.grad((OP.tensor_prod_bare(il, ir, io, ld, rd) * cot.double()).sum(), [ld, rd], create_graph=True)
+    ref2 = torch.autograd.grad(sum((r ** 2).sum() for r in ref), [ld, rd])
+    outs = []
+    for route in (tp.TensorProdBare(il, ir, io), lambda a, b: tp._prod_with_grad((il, ir, io), a, b)):
+        lg, rg = x_l.cuda().requires_grad_(), x_r.cuda().requires_grad_()
+        y = route(lg, rg)
+        got = torch.autograd.grad((y * cot.cuda()).sum(), [lg, rg], create_graph=True)
+        got2 = torch.autograd.grad(sum((t ** 2).sum() for t in got), [lg, rg])
+        outs.append([y, *got, *got2])
+        for a, r in zip(list(got) + list(got2), list(ref) + list(ref2)):
+            torch.testing.assert_close(a.detach().cpu().double(), r.detach(), rtol=1e-5, atol=2e-6 * float(r.abs().max()) + 1e-9)
+    for a, b in zip(*outs):
+        torch.testing.assert_close(a, b, rtol=1e-5, atol=2e-6 * float(b.abs().max()) + 1e-9)
+
+
 @pytest.mark.parametrize("E,n", [(1000, 128), (257, 4), (3001, 32), (130, 256)])
 def test_painn_combine_against_plain_arithmetic(pkg, E, n):
     """The fused elementwise middle of the PaiNN message (archs/meanflow_painn8.py:91-100: the gathers by destination

@@ -23,9 +23,9 @@ def _buffers(B, N, capacity):
                 dst=torch.full((capacity,), -1, **i32))
 
 
-def _call(lib, L, static, x, cutoff, box, capacity):
+def _call(lib, L, static, x, cutoff, box, capacity, out=None):
     B, N = x.shape[:2]
-    out = _buffers(B, N, capacity)
+    out = _buffers(B, N, capacity) if out is None else out
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
     tail = (_ptr(out["row_ptr"]), _ptr(out["edge_counts"]), _ptr(out["stats"]), capacity, _ptr(out["src"]),
             _ptr(out["dst"]), stream)
@@ -46,23 +46,32 @@ def test_built_in_workspace_gives_the_same_graph_twice_in_a_row():
     rng = np.random.default_rng(0x947)
     cases = [((4, 9000, 3), 5.0, (40., 40., 40.), 3_000_000),        # dense cells, ~120 neighbours per atom
              ((2, 700, 3), 6.0, (70., 70., 70.), 40_000),            # smaller, sparse cells (one-wave workgroups)
-             ((1, 3000, 3), 4.0, (12., 12., 12.), 100_000)]           # windows larger than the LDS tile; capacity < E
+             ((1, 3000, 3), 4.0, (12., 12., 12.), 100_000),           # windows larger than the LDS tile; capacity < E
+             # more atoms in one box than the per-box sort in LDS takes: the histogram / scan / place path, on a
+             # workspace that the calls before left dirty
+             ((1, 20000, 3), 5.0, (60., 60., 60.), 1_500_000)]
     for shape, cutoff, box, capacity in cases:
         x = torch.from_numpy((rng.random(shape) * 3 - 1).astype(np.float32) * box[0]).cuda()
         print("case", shape, cutoff, box, capacity, flush=True)
         want = _call(lib, L, False, x, cutoff, box, capacity)
-        before = torch.cuda.memory_allocated()
-        got = _call(lib, L, True, x, cutoff, box, capacity)
+        # outputs allocated before the window; the driver's own count of free device memory (hipMemGetInfo) must
+        # not move across the call: it sees any allocation, through torch or not
+        got = _buffers(shape[0], shape[1], capacity)
+        torch.cuda.synchronize()
+        free_before = torch.cuda.mem_get_info()[0]
+        torch_before = torch.cuda.memory_allocated()
+        _call(lib, L, True, x, cutoff, box, capacity, out=got)
+        assert torch.cuda.mem_get_info()[0] == free_before
+        assert torch.cuda.memory_allocated() == torch_before
         E = int(want["stats"][0])
         assert E > 0 and int(got["stats"][0]) == E
         for key in ("row_ptr", "edge_counts", "stats", "src", "dst"):
             assert torch.equal(got[key], want[key]), key
         if capacity < E:
             assert shape == (1, 3000, 3) and bool((got["src"] >= 0).all())
+            assert int(got["row_ptr"].max()) == capacity and int(got["stats"][3]) & 2
         else:
             assert bool((got["src"][E:] == -1).all()) and bool((got["dst"][E:] == -1).all())
-        del got
-        assert torch.cuda.memory_allocated() <= before + 64          # nothing allocated through torch by the call
 
 
 def test_search_larger_than_the_built_in_workspace_is_refused():
