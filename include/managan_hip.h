@@ -53,7 +53,9 @@ int mg_abi_version(void);
  *   count: bins atoms, walks the 3x3x3 cell window, writes the CSR row_ptr
  *          (batch*nodes+1, exclusive prefix), edge_counts (batch, inclusive
  *          prefix per box, as the reference's edgeCounts) and stats[4] =
- *          {E, max atoms in a cell, max degree, flags: bit 0 = E overflowed int32};
+ *          {E, max atoms in a cell, max degree, flags: bit 0 = E overflowed int32},
+ *          each word stored exactly once per call (a caller may point stats at
+ *          device-visible pinned host memory preset to -1 and poll it);
  *   fill:  writes src[e] = b*nodes+i and dst[e] = b*nodes+j, rows ordered by
  *          (b,i); order inside a row is deterministic.  n_edges is the CAPACITY of
  *          src and dst in edges: an edge whose position row_ptr[row] + k is not
@@ -68,6 +70,12 @@ int mg_abi_version(void);
  * ---------------------------------------------------------------------- */
 int mg_neighbour_ndiv(float cutoff, float box_x, float box_y, float box_z, int ndiv[3] /* host */);
 
+/* The workspace holds the wrapped and cell-sorted atoms, the cell table and one row per atom that collects the
+ * atom's neighbours between the two phases (box-local ids: 16 bits each when a box has at most 65536 atoms, else
+ * 32).  mg_neighbour_workspace_bytes reports the preferred size: rows of 256 entries.  The count, fill and
+ * cell-order calls also accept a smaller workspace (the same pointer and size in all of them) and then use the
+ * longest rows that fit, down to 32 entries; an atom with more neighbours than a row holds costs a second sweep
+ * of its window in the fill pass, nothing else.  Below that the calls return MG_ERR_WORKSPACE. */
 int mg_neighbour_workspace_bytes(int batch, int nodes, float cutoff,
                                  float box_x, float box_y, float box_z, size_t* bytes /* host */);
 
@@ -96,9 +104,11 @@ int mg_neighbour_edges(const float* x /* (batch,nodes,3) */, int batch, int node
 
 /* mg_neighbour_edges without a workspace argument, for callers that cannot allocate one (code under HIP graph
  * capture, tight serving loops, harnesses that forbid allocation).  No counterpart in the reference.  The workspace
- * is a 64 MiB buffer built into the library (one per GPU, held until the process ends); a search that needs more
- * (about 1.1 KB per atom, most of it the 256-entry row that collects an atom's neighbours, plus 8 bytes per cell:
- * roughly 60 000 atoms over all boxes) is refused with MG_ERR_WORKSPACE and a message.  The call allocates and frees nothing and synchronises nothing;
+ * is a 64 MiB buffer built into the library (one per GPU, held until the process ends), used with the longest
+ * neighbour rows that fit (see mg_neighbour_workspace_bytes: 8 boxes of 16384 atoms get rows of 224 entries); a
+ * search that does not fit with rows of 32 entries (116 bytes per atom plus 8 per cell: beyond about 500 000 atoms
+ * over all boxes) is refused with MG_ERR_WORKSPACE and a message.  The call allocates and frees nothing and
+ * synchronises nothing;
  * inputs and outputs are the caller's.
  * All calls on one GPU share the buffer: calls that overlap in time on the same GPU (two streams, two threads)
  * race, calls ordered on one stream do not.  The first call on a device looks the buffer's address up

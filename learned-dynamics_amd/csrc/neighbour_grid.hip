@@ -87,14 +87,16 @@ struct Workspace {
     int* deg_sums;      // sums / maxima of the degrees per tile of kScanTile rows
     int* deg_max;
     int* box_max;       // batch: largest cell occupancy of each box (per-box sort)
-    int* hits;          // A x hit_cap: neighbours found by the count pass (box-local atom ids, window order)
+    void* hits;         // A x hit_cap: neighbours found by the count pass (box-local atom ids, window order);
+                        // 16-bit entries when a box has at most 65536 atoms, else 32-bit
     int hit_cap;        // entries per hit row; rows with more hits are recomputed by the fill pass
+    int hit_bytes;      // 2 or 4
     size_t bytes;
 };
 
 inline size_t align_up(size_t v) { return (v + 255) & ~size_t(255); }
 
-Workspace carve(void* base, long A, long C, int hit_cap) {
+Workspace carve(void* base, long A, long C, int hit_cap, int hit_bytes) {
     Workspace w{};
     size_t off = 0;
     auto take = [&](size_t bytes) {
@@ -116,8 +118,9 @@ Workspace carve(void* base, long A, long C, int hit_cap) {
     w.deg_sums = static_cast<int*>(take(sizeof(int) * scan_blocks));
     w.deg_max = static_cast<int*>(take(sizeof(int) * scan_blocks));
     w.box_max = static_cast<int*>(take(sizeof(int) * (A > 0 ? A : 1)));   // (batch <= A)
-    w.hits = static_cast<int*>(take(sizeof(int) * A * hit_cap));
+    w.hits = take((size_t)hit_bytes * A * hit_cap);
     w.hit_cap = hit_cap;
+    w.hit_bytes = hit_bytes;
     w.bytes = off;
     return w;
 }
@@ -579,7 +582,15 @@ __device__ __forceinline__ int hits_below(unsigned long long mask, int add) {
                                           __builtin_amdgcn_mbcnt_lo((unsigned)(mask & 0xffffffffull), (unsigned)add));
 }
 
-template <int kCandCap>
+// HitT: unsigned short (boxes of at most 65536 atoms) or int
+__device__ __forceinline__ void store_hit(__amdgpu_buffer_rsrc_t row, int id, int entry, unsigned short) {
+    __builtin_amdgcn_raw_buffer_store_b16((short)id, row, entry << 1, 0, 0);
+}
+__device__ __forceinline__ void store_hit(__amdgpu_buffer_rsrc_t row, int id, int entry, int) {
+    __builtin_amdgcn_raw_buffer_store_b32(id, row, entry << 2, 0, 0);
+}
+
+template <int kCandCap, typename HitT>
 __global__ void __launch_bounds__(256) count_kernel(Grid g, Workspace w) {
     __shared__ float4 cand[kCandCap];
     __shared__ int range_start[27];
@@ -606,7 +617,8 @@ __global__ void __launch_bounds__(256) count_kernel(Grid g, Workspace w) {
                      ((g.nz < 5 || cz < 2 || cz > g.nz - 3) ? 4 : 0);
     const float ibx = 1.0f / g.bx, iby = 1.0f / g.by, ibz = 1.0f / g.bz;
     const int node_base = b * g.nodes;
-    const int row_bytes = w.hit_cap * (int)sizeof(int);
+    const int row_bytes = w.hit_cap * (int)sizeof(HitT);
+    HitT* const hits = static_cast<HitT*>(w.hits);
 
     const int self_base = __builtin_amdgcn_readfirstlane(win.self_base), home_n = __builtin_amdgcn_readfirstlane(win.home_n);
     for (int h = wave; h < home_n; h += nwaves) {
@@ -617,7 +629,7 @@ __global__ void __launch_bounds__(256) count_kernel(Grid g, Workspace w) {
         const int row = node_base + __builtin_amdgcn_readfirstlane(__float_as_int(self.w));
         // descriptor of this atom's hit row alone: a store past the row's capacity is dropped
         const __amdgpu_buffer_rsrc_t hit_row =
-            __builtin_amdgcn_make_buffer_rsrc(w.hits + (long)row * w.hit_cap, 0, row_bytes, 0x00020000);
+            __builtin_amdgcn_make_buffer_rsrc(hits + (long)row * w.hit_cap, 0, row_bytes, 0x00020000);
         // the home atom is itself a candidate and passes the distance test: its bit is taken out of the ballot of
         // its group with scalar instructions (no lane compares ids)
         const int self_group = k_self & ~(kWave - 1);
@@ -631,8 +643,7 @@ __global__ void __launch_bounds__(256) count_kernel(Grid g, Workspace w) {
                 if (k0 == self_group) mask &= self_clear;
                 // (box-local atom ids: the fill pass adds the box's first row)
                 if (__builtin_amdgcn_inverse_ballot_w64(mask))
-                    __builtin_amdgcn_raw_buffer_store_b32(__float_as_int(o.w), hit_row,
-                                                          (hits_below(mask, 0) << 2) + 4 * running, 0, 0);
+                    store_hit(hit_row, __float_as_int(o.w), hits_below(mask, running), HitT{});
                 running += __popcll(mask);
             }
         };
@@ -657,8 +668,7 @@ __global__ void __launch_bounds__(256) count_kernel(Grid g, Workspace w) {
                 hit = k != k_self && within_cutoff<7>(self, o, g, ibx, iby, ibz);
             }
             const unsigned long long mask = __ballot(hit);
-            if (hit)
-                __builtin_amdgcn_raw_buffer_store_b32(other, hit_row, hits_below(mask, running) * (int)sizeof(int), 0, 0);
+            if (hit) store_hit(hit_row, other, hits_below(mask, running), HitT{});
             running += __popcll(mask);
         }
         if (lane == 0) w.degree[row] = running;
@@ -723,6 +733,7 @@ __device__ void refill_row(const Grid& g, const Workspace& w, int row, int out_p
 // thread takes every 256th edge of the range, finds its row among the staged row starts and copies one entry of
 // that row's hits.  Edges beyond the capacity are dropped.
 constexpr int kFillRows = 64;
+template <typename HitT>
 __global__ void __launch_bounds__(256) fill_kernel(Grid g, Workspace w, const int* __restrict__ row_ptr,
                                                    int* __restrict__ src, int* __restrict__ dst, int capacity) {
     __shared__ int rp[kFillRows + 1];
@@ -734,6 +745,7 @@ __global__ void __launch_bounds__(256) fill_kernel(Grid g, Workspace w, const in
     if ((int)threadIdx.x < nrows) first_row[threadIdx.x] = (int)((r0 + threadIdx.x) / g.nodes) * g.nodes;
     __syncthreads();
     const int cap = w.hit_cap;
+    const HitT* __restrict__ hits = static_cast<const HitT*>(w.hits);
     const int e_hi = rp[nrows];
     for (int e = rp[0] + (int)threadIdx.x; e < e_hi; e += 256) {
         int lo = 0, hi = nrows - 1;                    // last row with rp <= e (6 halvings of 64)
@@ -745,7 +757,7 @@ __global__ void __launch_bounds__(256) fill_kernel(Grid g, Workspace w, const in
         const int idx = e - rp[lo], deg = rp[lo + 1] - rp[lo];
         if (deg <= cap && idx >= 0 && idx < deg && e >= 0 && e < capacity) {
             src[e] = (int)(r0 + lo);
-            dst[e] = first_row[lo] + w.hits[(r0 + lo) * cap + idx];
+            dst[e] = first_row[lo] + (int)hits[(r0 + lo) * cap + idx];
         }
     }
     // rows with more hits than a hit row holds: a wave each
@@ -880,10 +892,40 @@ int sort_slabs(const Grid& g) {
 }
 // one workgroup per cell, laid out so that the kernels read the cell coordinates off the workgroup id
 dim3 cell_grid(const Grid& g) { return dim3((unsigned)g.nz, (unsigned)g.ny, (unsigned)(g.nx * g.batch)); }
-// Entries per hit row.  The host knows the mean density only, and a row that is too short costs a second sweep of the
-// atom's window in the fill pass, so the rows are long enough for any density short of a dense liquid with a long
-// cutoff: 1 KB per atom of address space, of which a search touches what its neighbour counts need.
-int hit_cap(const Grid&) { return 256; }
+// Hit rows.  An entry is a box-local atom id: 16 bits when a box has at most 65536 atoms.  The host knows the mean
+// density only, and a row that is too short costs a second sweep of the atom's window in the fill pass, so a row has
+// kHitCapMax entries (enough for any density short of a dense liquid with a long cutoff: 512 bytes of address space
+// per atom, of which a search touches what its neighbour counts need) whenever the workspace is as large as
+// mg_neighbour_workspace_bytes says; a smaller workspace (the library's built-in one) gets the longest rows that
+// fit, down to kHitCapMin entries.  Count, fill and cell-order calls derive the same layout from the same
+// (batch, nodes, box, workspace size).
+constexpr int kHitCapMax = 256, kHitCapMin = 32;
+int hit_entry_bytes(const Grid& g) { return g.nodes <= 65536 ? 2 : 4; }
+
+// Workspace layout for a buffer of `workspace_bytes` (0: the preferred size).  Returns false when not even the
+// shortest rows fit; *needed is then the smallest size that works.
+bool layout(const Grid& g, void* base, size_t workspace_bytes, Workspace* w, size_t* needed) {
+    const long A = (long)g.batch * g.nodes, C = (long)g.batch * g.ncells;
+    const int eb = hit_entry_bytes(g);
+    int cap = kHitCapMax;
+    if (workspace_bytes != 0 && A > 0) {
+        const size_t fixed = carve(nullptr, A, C, 0, eb).bytes + 512;      // alignment of the base and of the rows
+        const size_t room = workspace_bytes > fixed ? workspace_bytes - fixed : 0;
+        long fit = (long)(room / ((size_t)eb * (size_t)A));
+        fit &= ~7L;                                     // rows stay 16-byte aligned
+        if (fit < kHitCapMin) {
+            if (needed) *needed = carve(nullptr, A, C, kHitCapMin, eb).bytes + 256;
+            return false;
+        }
+        cap = fit < kHitCapMax ? (int)fit : kHitCapMax;
+    }
+    *w = carve(base, A, C, cap, eb);
+    if (workspace_bytes != 0 && w->bytes + 256 > workspace_bytes) {     // (A == 0: the fixed arrays alone)
+        if (needed) *needed = w->bytes + 256;
+        return false;
+    }
+    return true;
+}
 
 int pairs_block_size(const Grid& g) {
     // sparse boxes: one wave per cell and a tile of 256 candidates are plenty (10 % faster than four waves at 1.2
@@ -913,8 +955,9 @@ int mg_neighbour_workspace_bytes(int batch, int nodes, float cutoff, float box_x
     MG_REQUIRE(bytes != nullptr, "bytes is null");
     Grid g;
     if (int s = make_grid(cutoff, box_x, box_y, box_z, batch, nodes, &g)) return s;
-    const long A = (long)batch * nodes, C = (long)batch * g.ncells;
-    *bytes = carve(nullptr, A, C, hit_cap(g)).bytes + 256;
+    Workspace w;
+    layout(g, nullptr, 0, &w, nullptr);
+    *bytes = w.bytes + 256;
     return MG_OK;
 }
 
@@ -927,10 +970,11 @@ int mg_neighbour_count(const float* x, int batch, int nodes, float cutoff, float
     MG_REQUIRE(batch == 0 || edge_counts, "mg_neighbour_count: edge_counts is null");
     const long A = (long)batch * nodes, C = (long)batch * g.ncells;
     void* base = reinterpret_cast<void*>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~uintptr_t(255));
-    Workspace w = carve(base, A, C, hit_cap(g));
-    if (w.bytes + 256 > workspace_bytes)
-        return fail(MG_ERR_WORKSPACE, "mg_neighbour_count: workspace has %zu bytes, %zu needed", workspace_bytes,
-                    w.bytes + 256);
+    Workspace w;
+    size_t needed = 0;
+    if (workspace_bytes == 0 || !layout(g, base, workspace_bytes, &w, &needed))
+        return fail(MG_ERR_WORKSPACE, "mg_neighbour_count: workspace has %zu bytes, at least %zu needed", workspace_bytes,
+                    needed);
     hipStream_t st = (hipStream_t)stream;
     if (A == 0) {
         hipLaunchKernelGGL(zero3_kernel, dim3(1), dim3(256), 0, st, stats, 4L, row_ptr, 1L, edge_counts, (long)batch);
@@ -946,16 +990,20 @@ int mg_neighbour_count(const float* x, int batch, int nodes, float cutoff, float
         hipLaunchKernelGGL(sort_box_kernel, dim3((unsigned)sort_slabs(g), (unsigned)batch), dim3(kSortThreads), 0, st, g, w);
     } else {
         hipLaunchKernelGGL(zero3_kernel, dim3((unsigned)(ceil_div(C, 256) < 1024 ? ceil_div(C, 256) : 1024)), dim3(256),
-                           0, st, stats, 4L, row_ptr, 1L, w.cell_count, C);
+                           0, st, (int*)nullptr, 0L, row_ptr, 1L, w.cell_count, C);    // (every word of stats is stored below)
         hipLaunchKernelGGL(bin_kernel<true>, dim3(ablocks), dim3(256), 0, st, x, g, w);
         if (int s = run_scan(w.cell_count, C, w.cell_start, w, nullptr, stats + 1, nullptr, st)) return s;
         hipLaunchKernelGGL(place_kernel, dim3(ablocks), dim3(256), 0, st, g, w);
         hipLaunchKernelGGL(order_kernel, dim3(ablocks), dim3(256), 0, st, g, w);
     }
-    if (pairs_block_size(g) == 64)
-        hipLaunchKernelGGL((count_kernel<kCandCapSparse>), cell_grid(g), dim3(64), 0, st, g, w);
-    else
-        hipLaunchKernelGGL((count_kernel<kCandCapDense>), cell_grid(g), dim3(256), 0, st, g, w);
+    const bool narrow = w.hit_bytes == 2;
+    if (pairs_block_size(g) == 64) {
+        if (narrow) hipLaunchKernelGGL((count_kernel<kCandCapSparse, unsigned short>), cell_grid(g), dim3(64), 0, st, g, w);
+        else hipLaunchKernelGGL((count_kernel<kCandCapSparse, int>), cell_grid(g), dim3(64), 0, st, g, w);
+    } else {
+        if (narrow) hipLaunchKernelGGL((count_kernel<kCandCapDense, unsigned short>), cell_grid(g), dim3(256), 0, st, g, w);
+        else hipLaunchKernelGGL((count_kernel<kCandCapDense, int>), cell_grid(g), dim3(256), 0, st, g, w);
+    }
     hipLaunchKernelGGL(scan_sums_kernel, dim3((unsigned)deg_tiles), dim3(kScanThreads), 0, st, (const int*)w.degree, A,
                        w.deg_sums, w.deg_max);
     hipLaunchKernelGGL(scan_apply_kernel, dim3((unsigned)deg_tiles), dim3(kScanThreads), 0, st, (const int*)w.degree, A,
@@ -970,16 +1018,21 @@ int mg_neighbour_fill(const void* workspace, size_t workspace_bytes, int batch, 
     Grid g;
     if (int s = make_grid(cutoff, box_x, box_y, box_z, batch, nodes, &g)) return s;
     MG_REQUIRE(n_edges >= 0, "mg_neighbour_fill: negative n_edges");
-    const long A = (long)batch * nodes, C = (long)batch * g.ncells;
+    const long A = (long)batch * nodes;
     if (A == 0 || n_edges == 0) return MG_OK;
     MG_REQUIRE(workspace && row_ptr && src && dst, "mg_neighbour_fill: null pointer");
     void* base = reinterpret_cast<void*>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~uintptr_t(255));
-    Workspace w = carve(base, A, C, hit_cap(g));
-    if (w.bytes + 256 > workspace_bytes)
-        return fail(MG_ERR_WORKSPACE, "mg_neighbour_fill: workspace has %zu bytes, %zu needed", workspace_bytes,
-                    w.bytes + 256);
-    hipLaunchKernelGGL(fill_kernel, dim3((unsigned)ceil_div(A, kFillRows)), dim3(256), 0, (hipStream_t)stream, g, w,
-                       row_ptr, src, dst, n_edges);
+    Workspace w;
+    size_t needed = 0;
+    if (workspace_bytes == 0 || !layout(g, base, workspace_bytes, &w, &needed))
+        return fail(MG_ERR_WORKSPACE, "mg_neighbour_fill: workspace has %zu bytes, at least %zu needed", workspace_bytes,
+                    needed);
+    if (w.hit_bytes == 2)
+        hipLaunchKernelGGL(fill_kernel<unsigned short>, dim3((unsigned)ceil_div(A, kFillRows)), dim3(256), 0,
+                           (hipStream_t)stream, g, w, row_ptr, src, dst, n_edges);
+    else
+        hipLaunchKernelGGL(fill_kernel<int>, dim3((unsigned)ceil_div(A, kFillRows)), dim3(256), 0, (hipStream_t)stream, g,
+                           w, row_ptr, src, dst, n_edges);
     return check_launch("mg_neighbour_fill");
 }
 
@@ -1005,13 +1058,14 @@ int mg_neighbour_edges(const float* x, int batch, int nodes, float cutoff, float
 int mg_neighbour_edges_static(const float* x, int batch, int nodes, float cutoff, float box_x, float box_y,
                               float box_z, int* row_ptr, int* edge_counts, int* stats, int capacity, int* src,
                               int* dst, mg_stream_t stream) {
+    Grid g;
+    if (int s = make_grid(cutoff, box_x, box_y, box_z, batch, nodes, &g)) return s;
+    Workspace probe;
     size_t need = 0;
-    if (int s = mg_neighbour_workspace_bytes(batch, nodes, cutoff, box_x, box_y, box_z, &need)) return s;
-    if (need > kScratchBytes)
+    if (!layout(g, nullptr, kScratchBytes, &probe, &need))
         return fail(MG_ERR_WORKSPACE,
-                    "mg_neighbour_edges_static: this search needs %zu bytes of workspace (%zu per atom, most of it the "
-                    "rows that collect each atom's neighbours), the built-in one holds %zu; use mg_neighbour_edges with "
-                    "a workspace of your own",
+                    "mg_neighbour_edges_static: this search needs at least %zu bytes of workspace (%zu per atom), the "
+                    "built-in one holds %zu; use mg_neighbour_edges with a workspace of your own",
                     need, need / (size_t)((long)batch * nodes > 0 ? (long)batch * nodes : 1), kScratchBytes);
     void* ws = nullptr;
     if (int s = scratch_of_current_device(&ws)) return s;
@@ -1025,14 +1079,15 @@ int mg_neighbour_cell_order(const void* workspace, size_t workspace_bytes, int b
                             float box_x, float box_y, float box_z, int* order, mg_stream_t stream) {
     Grid g;
     if (int s = make_grid(cutoff, box_x, box_y, box_z, batch, nodes, &g)) return s;
-    const long A = (long)batch * nodes, C = (long)batch * g.ncells;
+    const long A = (long)batch * nodes;
     if (A == 0) return MG_OK;
     MG_REQUIRE(workspace && order, "mg_neighbour_cell_order: null pointer");
     void* base = reinterpret_cast<void*>((reinterpret_cast<uintptr_t>(workspace) + 255) & ~uintptr_t(255));
-    Workspace w = carve(base, A, C, hit_cap(g));
-    if (w.bytes + 256 > workspace_bytes)
-        return fail(MG_ERR_WORKSPACE, "mg_neighbour_cell_order: workspace has %zu bytes, %zu needed", workspace_bytes,
-                    w.bytes + 256);
+    Workspace w;
+    size_t needed = 0;
+    if (workspace_bytes == 0 || !layout(g, base, workspace_bytes, &w, &needed))
+        return fail(MG_ERR_WORKSPACE, "mg_neighbour_cell_order: workspace has %zu bytes, at least %zu needed",
+                    workspace_bytes, needed);
     hipLaunchKernelGGL(cell_order_kernel, dim3((unsigned)ceil_div(A, 256)), dim3(256), 0, (hipStream_t)stream, g, w,
                        order);
     return check_launch("mg_neighbour_cell_order");

@@ -86,6 +86,21 @@ def _check_input(t, name, dtype=torch.float32):
 
 
 # --------------------------------------------------------------------- stage A
+_pinned_pool = []          # statistics words free for the next search
+_pinned_abandoned = []     # words of searches that were dropped unread: a kernel may still be about to write them
+
+
+def _pinned_stats():
+    """Four int32 words of pinned host memory (device-visible at the same address), reused between searches.  The
+    words are never handed back to the allocator: a search that is dropped before its statistics were read leaves
+    them on a list that is recycled after a device synchronisation."""
+    if not _pinned_pool and len(_pinned_abandoned) >= 64:
+        torch.cuda.synchronize()
+        _pinned_pool.extend(_pinned_abandoned)
+        del _pinned_abandoned[:]
+    return _pinned_pool.pop() if _pinned_pool else torch.empty(4, dtype=torch.int32, pin_memory=True)
+
+
 class NeighbourSearch:
     """Result of the count phase; `fill()` writes the edges."""
 
@@ -105,19 +120,40 @@ class NeighbourSearch:
             self.workspace = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
             self.row_ptr = torch.empty(self.batch * self.nodes + 1, dtype=torch.int32, device=dev)
             self.edge_counts = torch.empty(self.batch, dtype=torch.int32, device=dev)
-            self.stats = torch.empty(4, dtype=torch.int32, device=dev)
+            # The four statistics go to pinned host memory, which the GPU writes directly: the host needs the edge
+            # count to size src / dst, and polling four words that the scan kernel stores as soon as it knows them
+            # costs a few microseconds where a device->host copy with its synchronisation costs about twenty.
+            self.stats = _pinned_stats()
+            self._stats_np = self.stats.numpy()
+            self._stats_np[:] = -1                     # (never a valid value: the kernels store counts and flags)
             L.check(_lib.mg_neighbour_count(_p(x), self.batch, self.nodes, self.cutoff, *self.box,
                                             _p(self.workspace), self.workspace.numel(), _p(self.row_ptr),
                                             _p(self.edge_counts), _p(self.stats), _stream()))
         self._host_stats = None
 
     def host_stats(self):
-        """(E, max atoms per cell, max degree, overflow flag) — one device->host copy."""
+        """(E, max atoms per cell, max degree, overflow flag), read from the pinned words the kernels write; falls
+        back to a stream synchronisation if they have not all arrived after a bounded number of polls."""
         if self._host_stats is None:
-            self._host_stats = tuple(int(v) for v in self.stats.tolist())
+            st = self._stats_np
+            for _ in range(20000):
+                if st.min() >= 0:
+                    break
+            else:
+                torch.cuda.current_stream(self.x.device).synchronize()
+            self._host_stats = tuple(int(v) for v in st)
+            _pinned_pool.append(self.stats)            # every word has arrived: nothing will write them again
+            self.stats = torch.tensor(self._host_stats, dtype=torch.int32)
+            self._stats_np = None
+            if min(self._host_stats) < 0:
+                raise RuntimeError("the neighbour search did not report its statistics")
             if self._host_stats[3]:
                 raise RuntimeError("edge count does not fit int32")
         return self._host_stats
+
+    def __del__(self):
+        if getattr(self, "_stats_np", None) is not None:
+            _pinned_abandoned.append(self.stats)
 
     def fill(self, n_edges=None):
         """src, dst of exactly E edges (E read back from the device unless the caller passes the capacity to use:

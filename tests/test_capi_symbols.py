@@ -36,8 +36,11 @@ def test_host_only_entry_points():
     assert list(nd) == [12, 12, 12]
     nbytes = ctypes.c_size_t(0)
     assert lib.mg_neighbour_workspace_bytes(8, 16384, 5.0, 55.0, 55.0, 55.0, ctypes.byref(nbytes)) == 0
-    # 256 hit entries of 4 bytes per atom (134 MB for 131072 atoms) plus the sorted records and cell tables
-    assert 8 * 16384 * 256 * 4 < nbytes.value < 8 * 16384 * 256 * 4 + 16_000_000
+    # preferred size: 256 neighbour entries of 2 bytes per atom (boxes of at most 65536 atoms: 67 MB for 131072 atoms)
+    # plus the sorted records and cell tables; 4-byte entries for larger boxes
+    assert 8 * 16384 * 256 * 2 < nbytes.value < 8 * 16384 * 256 * 2 + 8_000_000
+    assert lib.mg_neighbour_workspace_bytes(1, 70000, 5.0, 90.0, 90.0, 90.0, ctypes.byref(nbytes)) == 0
+    assert 70000 * 256 * 4 < nbytes.value < 70000 * 256 * 4 + 5_000_000
     # box smaller than 3 cells: the reference's error, as a status code
     assert lib.mg_neighbour_workspace_bytes(1, 10, 5.5, 10.0, 10.0, 10.0, ctypes.byref(nbytes)) == L.MG_ERR_BOX_TOO_SMALL
     assert b"3*cutoff" in lib.mg_status_string(L.MG_ERR_BOX_TOO_SMALL)

@@ -244,6 +244,13 @@ def test_ant16_is_differentiable_once():
     x, P, left = _inputs(5, 16, 8, 8, 4, seed=9)
     args = [t.requires_grad_() for t in _args(x, P, left, "cuda")]
     ys = cg.Ant16.apply(*args)
-    g, = torch.autograd.grad(sum(y.sum() for y in ys), args[0], create_graph=True)
+    # a plain second derivative: the first derivative comes back detached from the graph
+    g, = torch.autograd.grad(sum(y.sum() for y in ys), args[0], create_graph=True, retain_graph=True)
+    assert not g.requires_grad
+    with pytest.raises(RuntimeError, match="does not require grad"):
+        g.sum().backward()
+    # the double-backward construction of a Jacobian-vector product (cotangents that require a gradient)
+    cot = [torch.ones_like(y).requires_grad_() for y in ys]
+    g, = torch.autograd.grad(ys, args[0], cot, create_graph=True)
     with pytest.raises(RuntimeError, match="once_differentiable|differentiate twice"):
         g.sum().backward()

@@ -275,3 +275,54 @@ def test_cell_order_is_a_permutation_sorted_by_cell(ops):
     assert np.all(np.diff(keys) >= 0)
     same = np.diff(keys) == 0
     assert np.all(np.diff(order)[same] > 0)                                   # atom id ascending inside a cell
+
+
+@pytest.mark.parametrize("nodes,box_len,cutoff", [(3000, 40.0, 5.0), (70000, 80.0, 4.0)])
+def test_workspace_smaller_than_the_preferred_size(nodes, box_len, cutoff):
+    """The count / fill / cell-order calls take any workspace down to neighbour rows of 32 entries: the edge list is
+    the same bit for bit, whether the rows are 256 entries long or so short that most atoms overflow theirs and are
+    swept again by the fill pass; one byte less than the minimum is refused.  Boxes of at most 65536 atoms keep
+    16-bit neighbour ids between the passes, larger ones 32-bit ids."""
+    import ctypes
+    L = importlib.import_module("learned-dynamics_amd._lib")
+    lib = L.load()
+    rng = np.random.default_rng(nodes)
+    B = 2 if nodes < 65536 else 1
+    x = torch.from_numpy((rng.random((B, nodes, 3)) * box_len).astype(np.float32)).cuda()
+    box = (box_len,) * 3
+    ndiv = int(np.ceil(box_len / cutoff))
+    A, C = B * nodes, B * ndiv ** 3
+    entry = 2 if nodes <= 65536 else 4
+    pref = ctypes.c_size_t(0)
+    L.check(lib.mg_neighbour_workspace_bytes(B, nodes, cutoff, *box, ctypes.byref(pref)))
+    assert A * 256 * entry < pref.value < A * (256 * entry + 60) + 8 * C + 8192
+    p = lambda t: ctypes.c_void_p(t.data_ptr())
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def search(ws_bytes):
+        ws = torch.empty(ws_bytes, dtype=torch.uint8, device="cuda")
+        row_ptr = torch.empty(A + 1, dtype=torch.int32, device="cuda")
+        ec = torch.empty(B, dtype=torch.int32, device="cuda")
+        stats = torch.empty(4, dtype=torch.int32, device="cuda")
+        status = lib.mg_neighbour_count(p(x), B, nodes, cutoff, *box, p(ws), ws_bytes, p(row_ptr), p(ec), p(stats), st)
+        if status != 0:
+            return status, None
+        E = int(stats[0])
+        src = torch.empty(E, dtype=torch.int32, device="cuda")
+        dst = torch.empty(E, dtype=torch.int32, device="cuda")
+        L.check(lib.mg_neighbour_fill(p(ws), ws_bytes, B, nodes, cutoff, *box, p(row_ptr), E, p(src), p(dst), st))
+        order = torch.empty(A, dtype=torch.int32, device="cuda")
+        L.check(lib.mg_neighbour_cell_order(p(ws), ws_bytes, B, nodes, cutoff, *box, p(order), st))
+        return 0, (row_ptr, ec, stats, src, dst, order)
+
+    status, want = search(pref.value)
+    assert status == 0
+    assert int(want[2][2]) > 40                                   # degrees above the shortest rows
+    fixed = pref.value - A * 256 * entry
+    for ws_bytes in (fixed + A * 100 * entry, fixed + A * 32 * entry + 4096):
+        status, got = search(ws_bytes)
+        assert status == 0, ws_bytes
+        for a, b in zip(got, want):
+            assert torch.equal(a, b)
+    status, _ = search(fixed + A * 31 * entry)
+    assert status == L.MG_ERR_WORKSPACE and b"at least" in lib.mg_last_error()

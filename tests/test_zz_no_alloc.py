@@ -49,7 +49,10 @@ def test_built_in_workspace_gives_the_same_graph_twice_in_a_row():
              ((1, 3000, 3), 4.0, (12., 12., 12.), 100_000),           # windows larger than the LDS tile; capacity < E
              # more atoms in one box than the per-box sort in LDS takes: the histogram / scan / place path, on a
              # workspace that the calls before left dirty
-             ((1, 20000, 3), 5.0, (60., 60., 60.), 1_500_000)]
+             ((1, 20000, 3), 5.0, (60., 60., 60.), 1_500_000),
+             # 8 boxes x 16384 atoms at 0.098 atoms / A^3: the built-in workspace takes it with neighbour rows of 224
+             # entries where the caller's workspace of the preferred size has 256; the graph is the same
+             ((8, 16384, 3), 5.0, (55., 55., 55.), 7_200_000)]
     for shape, cutoff, box, capacity in cases:
         x = torch.from_numpy((rng.random(shape) * 3 - 1).astype(np.float32) * box[0]).cuda()
         print("case", shape, cutoff, box, capacity, flush=True)
@@ -77,7 +80,7 @@ def test_built_in_workspace_gives_the_same_graph_twice_in_a_row():
 def test_search_larger_than_the_built_in_workspace_is_refused():
     L = importlib.import_module("learned-dynamics_amd._lib")
     lib = L.load()
-    B, N = 4, 65536                                                   # 262144 atoms: about 280 MB of workspace
+    B, N = 16, 65536                                                  # 1048576 atoms: 122 MB even with the shortest rows
     x = torch.rand(B, N, 3, device="cuda") * 100
     out = _buffers(B, N, 16)
     status = lib.mg_neighbour_edges_static(_ptr(x), B, N, 5.0, 100., 100., 100., _ptr(out["row_ptr"]),
