@@ -31,9 +31,9 @@ PEAK_FP32_MFMA_TFLOPS = 157.3  # MI355X dense fp32 matrix
 PEAK_BF16_MFMA_TFLOPS = 2500.0  # MI355X dense bf16 matrix
 
 
-def measured_traffic(kernel):
-    """HBM bytes per launch from the committed rocprofv3 --pmc summary (None if absent)."""
-    path = os.path.join(ROOT, "profiles", "painn_layer_configs2_traffic.json")
+def measured_traffic(kernel, summary="painn_layer_configs2_traffic.json"):
+    """HBM bytes per launch of a kernel from a committed rocprofv3 --pmc summary under profiles/ (None if absent)."""
+    path = os.path.join(ROOT, "profiles", summary)
     try:
         with open(path) as f:
             return json.load(f).get(kernel, {}).get("traffic_bytes")
@@ -267,8 +267,16 @@ def bench_painn_layer(torch, args):
             if comparisons:
                 msg.use_table = False
                 sec_exact = timed_steps(torch, step, max(3, args.steps // 4), 2)
-                msg.use_table = True
                 breakdown["layer_ms_with_filter_mlp_per_edge"] = sec_exact * 1e3
+                # and with every linear of the layer in true fp32 matrix arithmetic (v_mfma_f32_32x32x2_f32)
+                prev_mode = ops.get_linear_mode()
+                ops.set_linear_mode(ops.LINEAR_FP32_MFMA)
+                try:
+                    sec_fp32 = timed_steps(torch, step, 3, 1)
+                finally:
+                    ops.set_linear_mode(prev_mode)
+                breakdown["layer_ms_with_filter_mlp_per_edge_fp32_mfma"] = sec_fp32 * 1e3
+                msg.use_table = True
             hbm_bytes = E * (36 if sliced else 16) + N * (16 * n + 12 * n) + 2 * N * 16 * n + rows * 16 * n
             gather_bytes = E * (16 * n + 12 * n + 16)
             grid_bytes = E * 4 * 16 * n
@@ -299,6 +307,38 @@ def bench_painn_layer(torch, args):
                                 "the kernel is bound by vector arithmetic and by the gathers of node rows from L2 "
                                 "(cache_to_cu, against 64 B per clock per CU), not by HBM (hbm)",
                         "filter_mlp_per_edge_path": roofline}
+            # The three ways the layer can run, side by side.  The filter MLP's FLOPs (2 E (16 x 512 + 2 x 512^2)) are
+            # only executed when the MLP runs on every edge; with the grid they are replaced by 512 rows of the same MLP.
+            mlp_flops = 2.0 * E * (n_rbf * 4 * n + 2 * (4 * n) * (4 * n))
+            variants = {"filter_grid": {"value": E / sec, "unit": "edges/s", "ms_per_step": sec * 1e3,
+                                        "dominant_kernel": "painn_table_message_lds_kernel" if sliced else "painn_message_kernel<true>",
+                                        "bound": "fp32_vector", "frac": roofline["frac"], "traffic": roofline["traffic"],
+                                        "grid_rows": rows}}
+            if comparisons:
+                per_edge = breakdown["layer_ms_with_filter_mlp_per_edge"] * 1e-3
+                fused = roofline["filter_mlp_per_edge_path"]
+                variants["filter_mlp_per_edge"] = {
+                    "value": E / per_edge, "unit": "edges/s", "ms_per_step": per_edge * 1e3,
+                    "dominant_kernel": "painn_filter_message_kernel + painn_filter_hidden_kernel",
+                    "bound": "mfma", "peak": PEAK_BF16_MFMA_TFLOPS, "unit_roofline": "TFLOP/s",
+                    # executed fp16 matrix work of the whole layer step (3 per fp32 multiply-add) against the fp16 peak
+                    "achieved": 3 * mlp_flops / per_edge / 1e12, "frac": 3 * mlp_flops / per_edge / 1e12 / PEAK_BF16_MFMA_TFLOPS,
+                    "fp32_equivalent_tflops": mlp_flops / per_edge / 1e12,
+                    "fp32_equivalent_over_fp32_mfma_peak": mlp_flops / per_edge / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+                    "kernel_frac": None if fused is None else fused.get("frac"),
+                    "traffic": None if fused is None else fused.get("traffic"),
+                    "note": "the path every set of weights takes whose grid is refused, and every forward whose "
+                            "positions are differentiated"}
+                fp32 = breakdown["layer_ms_with_filter_mlp_per_edge_fp32_mfma"] * 1e-3
+                variants["filter_mlp_per_edge_fp32_mfma"] = {
+                    "value": E / fp32, "unit": "edges/s", "ms_per_step": fp32 * 1e3,
+                    "dominant_kernel": "linear_rows_kernel (v_mfma_f32_32x32x2_f32) + painn_message_kernel",
+                    "bound": "mfma", "peak": PEAK_FP32_MFMA_TFLOPS, "unit_roofline": "TFLOP/s",
+                    "achieved": mlp_flops / fp32 / 1e12, "frac": mlp_flops / fp32 / 1e12 / PEAK_FP32_MFMA_TFLOPS,
+                    "traffic": None,
+                    "note": "mg_set_linear_mode(0): 24-bit significand products on the fp32 matrix cores in every linear "
+                            "of the layer; the price of strict fp32 arithmetic (the filter is stored, E x 4n floats)"}
+            roofline["layer_variants"] = variants
         del actv
 
     cpu = None
@@ -310,8 +350,10 @@ def bench_painn_layer(torch, args):
         "ms_per_step": sec * 1e3,
         "dtype": "f32 storage and accumulation; products of the wide linears as split-fp16 MFMA (2 x 11 significand bits)",
         "value_note": "the filter MLP of the layer is evaluated on a 512-point grid over the edge length and "
-                      "interpolated per edge (accepted per set of weights at 3e-6 of max |filter|); "
-                      "value_filter_mlp_per_edge is the same layer with the MLP evaluated on every edge",
+                      "interpolated per edge (a grid is accepted per set of weights when its interpolation error, "
+                      "measured in float64, is below 1e-7 + 1e-6 |filter| for every filter element); "
+                      "roofline.layer_variants holds the same layer with the MLP evaluated on every edge, in "
+                      "split-fp16 and in true fp32 matrix arithmetic",
         "value_filter_mlp_per_edge": None if per_edge_ms is None else E / (per_edge_ms * 1e-3),
         "ms_per_step_filter_mlp_per_edge": per_edge_ms,
         "config": {"workload": "BASELINE configs[2]: one PaiNN layer (Message + Update, residuals), 16 chains x 1024 "
@@ -397,7 +439,8 @@ def bench_neighbour(torch, args, with_cpu=True):
            "config": {"workload": "BASELINE configs[1]: 8 boxes x 16384 atoms, box 55 A, cutoff 5 A", "edges": E},
            "roofline": {"kernel": "whole search (bin, sort, count, scan_sums, scan_apply, fill)",
                         "bound": "hbm", "achieved": alg_bytes / sec / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                        "frac": alg_bytes / sec / 1e9 / PEAK_HBM_GBS, "traffic": None},
+                        "frac": alg_bytes / sec / 1e9 / PEAK_HBM_GBS,
+                        "traffic": measured_traffic("whole_search", "neighbour_search_configs1_traffic.json")},
            "breakdown": {"count_phase_ms": t_count * 1e3, "fill_phase_ms": t_fill * 1e3,
                          "capacity_mode_ms": t_capacity * 1e3, "capacity_mode_replayed_ms": t_replay * 1e3,
                          "note": "ms_per_step is the exact-size search (edge count read back by the host between "
@@ -684,7 +727,9 @@ def edge_kernel_roofline(torch, msg, graph, r_ij, rows, bf16=False):
     p0_bytes = E * 3 * chan * w
     return {"kernel": "bee_message_kernel (gathers, 13 products, edge sums; one Messages layer)", "bound": "hbm",
             "achieved": nbytes / t / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": nbytes / t / 1e9 / PEAK_HBM_GBS,
-            "traffic": None, "bytes_per_launch": nbytes, "ms": t * 1e3,
+            "traffic": measured_traffic("bee_message_kernel", "stress_configs4_traffic.json" if bf16
+                                        else "denoiser_configs3_traffic.json"),
+            "bytes_per_launch": nbytes, "ms": t * 1e3,
             "per_edge_scalar_products_stored_bytes": p0_bytes,
             "frac_counting_the_stored_scalar_products": (nbytes + p0_bytes) / t / 1e9 / PEAK_HBM_GBS,
             # the 13 products are 167 flop per (edge, channel), the 60 running sums another 60

@@ -86,6 +86,7 @@ def _check_input(t, name, dtype=torch.float32):
 
 
 # --------------------------------------------------------------------- stage A
+_edge_count_hint = {}      # (batch, nodes, cutoff, box) -> edge count of the last search of that shape
 _pinned_pool = []          # statistics words free for the next search
 _pinned_abandoned = []     # words of searches that were dropped unread: a kernel may still be about to write them
 
@@ -156,14 +157,35 @@ class NeighbourSearch:
             _pinned_abandoned.append(self.stats)
 
     def fill(self, n_edges=None):
-        """src, dst of exactly E edges (E read back from the device unless the caller passes the capacity to use:
-        edges beyond a capacity below E are dropped, never written)."""
-        E = self.host_stats()[0] if n_edges is None else int(n_edges)
+        """src, dst of exactly E edges.  With n_edges the caller fixes the capacity (edges beyond a capacity below E
+        are dropped, never written).  Otherwise the edge count comes from the device, and the wait for it is taken off
+        the critical path: the fill pass is queued at once into arrays sized from an estimate (the edge count of the
+        last search of this shape, else the mean density, plus a margin), the count is read afterwards, and the
+        first E entries are returned; only when the estimate was too small is the pass run again at the exact size."""
         dev = self.x.device
+        if n_edges is not None or self._host_stats is not None:
+            E = self.host_stats()[0] if n_edges is None else int(n_edges)
+            with torch.cuda.device(dev):
+                src = torch.empty(E, dtype=torch.int32, device=dev)
+                dst = torch.empty(E, dtype=torch.int32, device=dev)
+            return self.fill_into(src, dst)
+        key = (self.batch, self.nodes, self.cutoff, self.box)
+        hint = _edge_count_hint.get(key)
+        if hint is None:
+            volume = self.box[0] * self.box[1] * self.box[2]
+            hint = 1.5 * self.batch * self.nodes * (self.nodes / volume) * 4.18879 * self.cutoff ** 3
+        capacity = min(int(1.125 * hint) + 4096, 2 ** 31 - 1)
         with torch.cuda.device(dev):
-            src = torch.empty(E, dtype=torch.int32, device=dev)
-            dst = torch.empty(E, dtype=torch.int32, device=dev)
-        return self.fill_into(src, dst)
+            src = torch.empty(capacity, dtype=torch.int32, device=dev)
+            dst = torch.empty(capacity, dtype=torch.int32, device=dev)
+        self.fill_into(src, dst)
+        E = self.host_stats()[0]
+        if len(_edge_count_hint) > 256:
+            _edge_count_hint.clear()
+        _edge_count_hint[key] = E
+        if E <= capacity:
+            return src[:E], dst[:E]
+        return self.fill(E)
 
     def fill_into(self, src, dst):
         """Write the edges into caller-owned int32 arrays whose common length is the capacity; no host
@@ -236,8 +258,8 @@ def _check_caps(search, listmax, neighboursmax):
 def get_edges(listmax, neighboursmax, cutoff, box_x, box_y, box_z, x, return_row_ptr=False, return_order=False):
     """(src int32[E], dst int32[E], edgeCounts int32[B]); extensions/neighbour_grid/neighbour_grid.cpp:170-195."""
     search = NeighbourSearch(x, cutoff, (box_x, box_y, box_z))
+    src, dst = search.fill()                       # queued before the statistics are read (see fill)
     _check_caps(search, listmax, neighboursmax)
-    src, dst = search.fill()
     out = (src, dst, search.edge_counts)
     if return_row_ptr:
         out = out + (search.row_ptr,)
