@@ -8,6 +8,7 @@ import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libmanagan_hip.so")
+EXT_PATH = os.path.join(_HERE, "managan_torch_ext.so")
 
 c_float_p = ctypes.c_void_p   # device pointers travel as integers
 c_int_p = ctypes.c_void_p
@@ -151,6 +152,27 @@ def load():
     lib.mg_abi_version.argtypes = []
     _lib = lib
     return lib
+
+
+_ext = None
+
+
+def load_torch_ext():
+    """The PyTorch C++ binding of the library (csrc/torch_binding.cpp): the reference's extension functions with
+    at::Tensor arguments.  Raises if it has not been built."""
+    global _ext
+    if _ext is None:
+        load()                                              # the library it links to, by its path
+        if not os.path.exists(EXT_PATH):
+            raise ImportError(f"{EXT_PATH} is missing: build it with `python learned-dynamics_amd/build.py`")
+        import importlib.util
+
+        import torch  # noqa: F401  (the binding links to torch's libraries)
+        spec = importlib.util.spec_from_file_location("managan_torch_ext", EXT_PATH)
+        module = importlib.util.module_from_spec(spec)
+        spec.loader.exec_module(module)
+        _ext = module
+    return _ext
 
 
 def check(status):

@@ -6,15 +6,17 @@ import importlib
 _ops = importlib.import_module("learned-dynamics_amd.ops")
 _a16 = importlib.import_module("learned-dynamics_amd.ant16_backward")
 
-bee_fwd_cuda = _ops.bee_fwd
-bee_bwl_cuda = _ops.bee_bwl
-bee_bwr_cuda = _ops.bee_bwr
-cow_o0_fwd_cuda = _ops.cow_o0_fwd
-cow_o0_bwl_cuda = _ops.cow_o0_bwl
-cow_o0_bwr_cuda = _ops.cow_o0_bwr
-cow_o1_fwd_cuda = _ops.cow_o1_fwd
-cow_o1_bwl_cuda = _ops.cow_o1_bwl
-cow_o1_bwr_cuda = _ops.cow_o1_bwr
+# Bee and Cow: the package's PyTorch C++ binding (csrc/torch_binding.cpp)
+_ext = importlib.import_module("learned-dynamics_amd._lib").load_torch_ext()
+bee_fwd_cuda = _ext.bee_fwd_cuda
+bee_bwl_cuda = _ext.bee_bwl_cuda
+bee_bwr_cuda = _ext.bee_bwr_cuda
+cow_o0_fwd_cuda = _ext.cow_o0_fwd_cuda
+cow_o0_bwl_cuda = _ext.cow_o0_bwl_cuda
+cow_o0_bwr_cuda = _ext.cow_o0_bwr_cuda
+cow_o1_fwd_cuda = _ext.cow_o1_fwd_cuda
+cow_o1_bwl_cuda = _ext.cow_o1_bwl_cuda
+cow_o1_bwr_cuda = _ext.cow_o1_bwr_cuda
 
 
 def set_kern_attributes():

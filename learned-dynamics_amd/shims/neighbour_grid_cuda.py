@@ -1,25 +1,11 @@
 """Drop-in for the reference's `neighbour_grid_cuda` extension
-(extensions/neighbour_grid/neighbour_grid.cpp:198-203), backed by HIP kernels."""
+(extensions/neighbour_grid/neighbour_grid.cpp:198-203): the same four functions, exported by the
+package's PyTorch C++ binding (csrc/torch_binding.cpp) over the HIP kernels."""
 import importlib
 
-_ops = importlib.import_module("learned-dynamics_amd.ops")
+_ext = importlib.import_module("learned-dynamics_amd._lib").load_torch_ext()
 
-
-def get_edges(listmax, neighboursmax, cutoff, box_x, box_y, box_z, x):
-    """Like get_neighbours, except it returns lists of edge tensors."""
-    return _ops.get_edges(listmax, neighboursmax, cutoff, box_x, box_y, box_z, x)
-
-
-def get_neighbours(listmax, neighboursmax, cutoff, box_x, box_y, box_z, x):
-    """Define neighbours based on cutoff radius using a grid method."""
-    return _ops.get_neighbours(listmax, neighboursmax, cutoff, box_x, box_y, box_z, x)
-
-
-def edges_read(neighbourCounts, neighbours, x):
-    """Read data from nodes to edges."""
-    return _ops.padded_edges_read(neighbourCounts, neighbours, x)
-
-
-def edges_reduce(neighbourCounts, neighbours, x):
-    """Reduce data from edges to nodes."""
-    return _ops.padded_edges_reduce(neighbourCounts, neighbours, x)
+get_edges = _ext.get_edges                # "Like get_neighbours, except it returns lists of edge tensors."
+get_neighbours = _ext.get_neighbours      # "Define neighbours based on cutoff radius using a grid method."
+edges_read = _ext.edges_read              # "Read data from nodes to edges."
+edges_reduce = _ext.edges_reduce          # "Reduce data from edges to nodes."
