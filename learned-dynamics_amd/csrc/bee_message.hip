@@ -320,7 +320,7 @@ static int launch_bee_message(const char* what, const int* row_ptr, const int* d
     MG_REQUIRE(blocks < (1L << 31), "%s: too many (node, channel chunk) items for one launch", what);
     // rows of a few edges do not repay the pipeline's start-up (one extra set of loads per row), unless the system
     // is so small that the chip is not filled and a row's chain of load latencies is all there is to the time
-    if (n_edges >= 32L * n_nodes || items <= 16384)
+    if (n_edges >= 8L * n_nodes || items <= 16384)
         hipLaunchKernelGGL((bee_message_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
                            row_ptr, dst, node_order, (long)n_nodes, rhat, enc, La, Lv, Ld, chan, enc_W, enc_b, P0, S1, S2,
                            node_max, edge_max);
