@@ -6,7 +6,8 @@ The directory name contains a hyphen, so import it with
     importlib.import_module("learned-dynamics_amd")
 
 Layout
-  csrc/                      HIP kernels and the extern "C" entry points (libmanagan_hip.so)
+  csrc/                      HIP kernels and the extern "C" entry points (libmanagan_hip.so);
+                             torch_binding.cpp: the PyTorch C++ binding (managan_torch_ext.so)
   _lib.py, ops.py            ctypes binding and torch-facing operators
   graph_layers.py            Graph, radius_graph, edges_read*, edges_reduce_src, boxwrap
   tensor_products.py         TensLinear, TensorProdBare, TensorProds, norms, tens_sigmoid
