@@ -212,34 +212,94 @@ def test_configs3_denoiser_is_equivariant_at_full_size(pkg):
     torch.testing.assert_close(v_r, _quarter_turn(v), rtol=1e-4, atol=1e-4 * float(v.abs().max()))
 
 
+def _configs4(seed_offset=5):
+    N, r0, C = 65536, 6.0, 128
+    L = (N / 0.1) ** (1.0 / 3.0)
+    g = torch.Generator().manual_seed(SEED + seed_offset)
+    pos = torch.rand(1, N, 3, generator=g) * L
+    x_a = torch.randn(1, N, C, generator=g)
+    x_v = torch.randn(1, N, C, 3, generator=g) / 3 ** 0.5
+    x_d = torch.randn(1, N, C, 3, 3, generator=g) / 3.0
+    return N, r0, C, L, pos, x_a, x_v, x_d
+
+
 def test_configs4_bf16_storage_within_one_percent_at_full_size(pkg):
-    """65536 atoms at 0.1 / A^3, cutoff 6, 128 channels per rank: bf16 storage against fp32 storage, one of
-    the four layers (each layer ends in group norms, so the deviation does not grow with depth)."""
+    """65536 atoms at 0.1 / A^3, cutoff 6, 128 channels per rank, all four layers of the stack: bf16 storage against
+    fp32 storage after every layer (each layer ends in group norms, so the deviation does not grow with depth), and
+    the rank-2 equivariance of the fp32 layer at this size."""
     bee = importlib.import_module("learned-dynamics_amd.bee_layers")
     b16 = importlib.import_module("learned-dynamics_amd.bee_layers_bf16")
     gl = importlib.import_module("learned-dynamics_amd.graph_layers")
-    N, r0, C = 65536, 6.0, 128
-    L = (N / 0.1) ** (1.0 / 3.0)
-    g = torch.Generator().manual_seed(SEED + 5)
-    pos = (torch.rand(1, N, 3, generator=g) * L).cuda()
-    x_a = torch.randn(1, N, C, generator=g).cuda()
-    x_v = (torch.randn(1, N, C, 3, generator=g) / 3 ** 0.5).cuda()
-    x_d = (torch.randn(1, N, C, 3, 3, generator=g) / 3.0).cuda()
+    N, r0, C, L, pos, x_a, x_v, x_d = _configs4()
+    pos, x_a, x_v, x_d = pos.cuda(), x_a.cuda(), x_v.cuda(), x_d.cuda()
     torch.manual_seed(SEED + 5)
-    msg = bee.Messages(r0, C, C, C, C).cuda().eval()
-    prod = bee.SelfTensProds(C, C, C, C).cuda().eval()
+    msgs = [bee.Messages(r0, C, C, C, C).cuda().eval() for _ in range(4)]
+    prods = [bee.SelfTensProds(C, C, C, C).cuda().eval() for _ in range(4)]
     with torch.no_grad():
         graph, r_ij = gl.graph_setup(r0, (L, L, L), pos, neighbours_max=256, celllist_max=64)
         assert 5_500_000 < int(graph.src.numel()) < 6_400_000
-        da, dv, dd = msg(graph, r_ij, x_a, x_v, x_d)
-        ref = prod(x_a + da, x_v + dv, x_d + dd, residual=True)
-        out = b16.stack_forward([msg], [prod], graph, r_ij, x_a, x_v, x_d)
-        # rank-2 equivariance of the fp32 layer at this size
-        ref_r = prod(*[f(t) for f, t in zip((lambda t: t, _quarter_turn, _quarter_turn_rank2),
-                                           (x_a + da, x_v + dv, x_d + dd))], residual=True)
-    for o, r in zip(out, ref):
-        assert float((o - r).abs().max() / r.abs().max()) < 1e-2
-    torch.testing.assert_close(ref_r[2], _quarter_turn_rank2(ref[2]), rtol=1e-5, atol=1e-5 * float(ref[2].abs().max()))
+        ref = (x_a, x_v, x_d)
+        for depth, (msg, prod) in enumerate(zip(msgs, prods), 1):
+            da, dv, dd = msg(graph, r_ij, *ref)
+            mid = (ref[0] + da, ref[1] + dv, ref[2] + dd)
+            ref = prod(*mid, residual=True)
+            out = b16.stack_forward(msgs[:depth], prods[:depth], graph, r_ij, x_a, x_v, x_d)
+            dev = [float((o - r).abs().max() / r.abs().max()) for o, r in zip(out, ref)]
+            print(f"[configs4] bf16 against fp32 storage after {depth} layers: {dev}")
+            assert max(dev) < 1e-2
+            if depth == 1:
+                # rank-2 equivariance of the fp32 layer at this size
+                ref_r = prod(*[f(t) for f, t in zip((lambda t: t, _quarter_turn, _quarter_turn_rank2), mid)], residual=True)
+                torch.testing.assert_close(ref_r[2], _quarter_turn_rank2(ref[2]), rtol=1e-5,
+                                           atol=1e-5 * float(ref[2].abs().max()))
+            del da, dv, dd, mid, out
+
+
+def test_configs4_messages_on_sampled_atoms_against_the_oracle(pkg):
+    """The rank-0/1/2 Messages layer of configs[4] at full size (65536 atoms, about 90 neighbours each, 128 channels per
+    rank): 48 sampled atoms of the fp32-storage path against the oracle's Messages (archs/diffuser_atoms15.py:238-253)
+    evaluated in float32 and float64 on exactly those atoms' edges at the layer tolerance, and the same atoms of the
+    bf16-storage path against the float64 oracle within 1e-2 of the output scale."""
+    bee = importlib.import_module("learned-dynamics_amd.bee_layers")
+    b16 = importlib.import_module("learned-dynamics_amd.bee_layers_bf16")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    from oracle import products as OP
+    from test_gpu_bee_layers import _mlp_leaky_weights
+    N, r0, C, L, pos, x_a, x_v, x_d = _configs4(seed_offset=6)
+    box = (L, L, L)
+    torch.manual_seed(SEED + 6)
+    msg = bee.Messages(r0, C, C, C, C).cuda().eval()
+    with torch.no_grad():
+        graph, r_ij = gl.graph_setup(r0, box, pos.cuda(), neighbours_max=256, celllist_max=64)
+        got = msg(graph, r_ij, x_a.cuda(), x_v.cuda(), x_d.cuda())
+        s = b16.to_storage(x_a.cuda(), x_v.cuda(), x_d.cuda())
+        got16 = b16.from_storage(*b16.messages_forward(msg, graph, r_ij, *s), 1)
+    g = torch.Generator().manual_seed(SEED + 7)
+    sample = torch.randint(0, N, (48,), generator=g).sort().values.unique()
+    row_ptr = graph.row_ptr.cpu().long()
+    pick = torch.cat([torch.arange(int(row_ptr[i]), int(row_ptr[i + 1])) for i in sample.tolist()])
+    assert pick.numel() > 3000
+    src, dst = graph.src.cpu()[pick], graph.dst.cpu()[pick]
+    r_ref = torch.from_numpy(ON.edge_vectors(pos.numpy(), src.numpy(), dst.numpy(), box))
+    assert torch.equal(r_ij.cpu()[pick], r_ref)
+    dd = lambda t, dt: t.detach().cpu().to(dt)
+    refs = {}
+    for dt in (torch.float32, torch.float64):
+        w = {"L0": dd(msg.L0.W, dt), "L1": dd(msg.L1.W, dt), "L2": dd(msg.L2.W, dt),
+             "Y": {lab: dd(getattr(msg, f"Y_{lab}").W, dt) for lab in OP.BEE_ORDER},
+             "enc_W": dd(msg.lin_enc.weight, dt), "enc_b": dd(msg.lin_enc.bias, dt),
+             "mlp_a": {k: v.to(dt) for k, v in _mlp_leaky_weights(msg.mlp_a).items()}}
+        out = OL.bee_messages(src, dst, 1, N, r_ref.to(dt), x_a.to(dt), x_v.to(dt), x_d.to(dt), w, r0,
+                              radial_dtype=torch.float64)
+        refs[dt] = [t[0, sample] for t in out]
+        del out, w
+    for k, name in enumerate("avd"):
+        assert_parity(got[k][0, sample.cuda()], refs[torch.float32][k], refs[torch.float64][k],
+                      f"configs[4] Messages, fp32 storage, B_{name}")
+        r64 = refs[torch.float64][k]
+        dev = float((got16[k][0, sample.cuda()].cpu().double() - r64).abs().max() / r64.abs().max())
+        print(f"[configs4] Messages, bf16 storage against the float64 oracle, B_{name}: {dev:.3g} of the output scale")
+        assert dev < 1e-2
 
 
 def test_configs2_training_step_through_the_filter_grid(pkg):
