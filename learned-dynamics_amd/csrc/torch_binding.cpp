@@ -15,6 +15,7 @@
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 
 #include <array>
+#include <cstdint>
 #include <string>
 #include <tuple>
 #include <vector>
@@ -287,6 +288,48 @@ torch::autograd::variable_list TensorLinearFn::backward(torch::autograd::Autogra
 
 at::Tensor tensor_linear(int64_t inds, const at::Tensor& W, const at::Tensor& x) { return TensorLinearFn::apply(inds, W, x); }
 
+// ------------------------------------------------------------------ TensorProds in one launch
+// y = lin_o(prod(lin_l(x_l), lin_r(x_r))) (managan/tensor_products.py:109-121), for problems mg_tensor_prods_supported
+// accepts; x: (..., dim, (3,)^inds), weights (out, in).  The module's forward is three such calls per a / v / d trio,
+// node-sized: the host time of a call is what the caller sees.
+bool tensor_prods_supported(int inds_l, int inds_r, int inds_o, int dim_l, int dim_r, int rank, int dim_o) {
+    return mg_tensor_prods_supported(inds_l, inds_r, inds_o, dim_l, dim_r, rank, dim_o) != 0;
+}
+
+at::Tensor tensor_prods(int inds_l, int inds_r, int inds_o, const at::Tensor& W_l, const at::Tensor& W_r, const at::Tensor& W_o,
+                        const at::Tensor& x_l_in, const at::Tensor& x_r_in) {
+    const char* names[5] = {"W_l", "W_r", "W_o", "x_l", "x_r"};
+    const at::Tensor* all[5] = {&W_l, &W_r, &W_o, &x_l_in, &x_r_in};
+    for (int k = 0; k < 5; k++)
+        TORCH_CHECK(all[k]->is_cuda() && all[k]->scalar_type() == at::kFloat, names[k], " must be a float32 CUDA tensor");
+    TORCH_CHECK(W_l.dim() == 2 && W_r.dim() == 2 && W_o.dim() == 2, "weights must be matrices");
+    TORCH_CHECK(inds_l >= 0 && inds_l <= 2 && inds_r >= 0 && inds_r <= 2 && inds_o >= 0 && inds_o <= 2, "ranks up to 2");
+    const at::Tensor x_l = x_l_in.contiguous(), x_r = x_r_in.contiguous();
+    const int64_t lead_l = x_l.dim() - inds_l - 1, lead_r = x_r.dim() - inds_r - 1;
+    TORCH_CHECK(lead_l >= 0 && lead_l == lead_r && x_l.sizes().slice(0, lead_l) == x_r.sizes().slice(0, lead_r),
+                "operands do not broadcast: ", x_l.sizes(), " vs ", x_r.sizes());
+    const int64_t rank = W_l.size(0), dim_l = W_l.size(1), dim_r = W_r.size(1), dim_o = W_o.size(0);
+    bool ok = x_l.size(lead_l) == dim_l && x_r.size(lead_r) == dim_r && W_r.size(0) == rank && W_o.size(1) == rank;
+    for (int64_t k = lead_l + 1; k < x_l.dim(); k++) ok = ok && x_l.size(k) == 3;
+    for (int64_t k = lead_r + 1; k < x_r.dim(); k++) ok = ok && x_r.size(k) == 3;
+    TORCH_CHECK(ok, "shape mismatch between weights and operands");
+    auto usable = [](const at::Tensor& W) {          // unit stride along a row, rows 16-byte aligned
+        return (W.stride(1) == 1 && W.stride(0) % 4 == 0 && reinterpret_cast<uintptr_t>(W.data_ptr()) % 16 == 0) ? W
+                                                                                                                 : W.contiguous();
+    };
+    const at::Tensor Wl = usable(W_l), Wr = usable(W_r), Wo = usable(W_o);
+    int64_t rows = 1;
+    std::vector<int64_t> y_shape;
+    for (int64_t k = 0; k < lead_l; k++) { rows *= x_l.size(k); y_shape.push_back(x_l.size(k)); }
+    y_shape.push_back(dim_o);
+    for (int k = 0; k < inds_o; k++) y_shape.push_back(3);
+    c10::hip::HIPGuardMasqueradingAsCUDA guard(x_l.device());
+    at::Tensor y = torch::empty(y_shape, x_l.options());
+    check(mg_tensor_prods(inds_l, inds_r, inds_o, fp(Wl), Wl.stride(0), fp(Wr), Wr.stride(0), fp(Wo), Wo.stride(0), fp(x_l),
+                          fp(x_r), rows, (int)dim_l, (int)dim_r, (int)rank, (int)dim_o, fp(y), stream_of(x_l)));
+    return y;
+}
+
 // ------------------------------------------------------------------ codegen_tensops_cuda: Bee and Cow
 std::vector<at::Tensor> bee_fwd(const at::Tensor& l_0, const at::Tensor& l_1, const at::Tensor& l_2, const at::Tensor& r_0,
                                 const at::Tensor& r_1, const at::Tensor& r_2) {
@@ -379,6 +422,9 @@ PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
     m.def("get_edges", &get_edges, "Like get_neighbours, except it returns lists of edge tensors.");
     // tensor_ops_cuda (tensor_ops.cpp:180-182)
     m.def("tensor_linear", &tensor_linear, "tensor_linear(inds, W, x)");
+    // TensorProds.forward (managan/tensor_products.py:109-121) as one launch
+    m.def("tensor_prods_supported", &tensor_prods_supported);
+    m.def("tensor_prods", &tensor_prods, "lin_o(prod(lin_l(x_l), lin_r(x_r)))");
     // codegen_tensops_cuda (codegen_tensops.cpp:2001-2010): the gradients arrive as positional arguments
     m.def("bee_fwd_cuda", &bee_fwd);
     m.def("bee_bwl_cuda", [](const at::Tensor& r_0, const at::Tensor& r_1, const at::Tensor& r_2, const py::args& dys) {

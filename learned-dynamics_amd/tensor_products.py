@@ -197,6 +197,11 @@ def _prod_with_grad(inds, x_l, x_r):
     return y.reshape(*lead, chan, *([3] * io))
 
 
+def _torch_ext():
+    from . import _lib
+    return _lib.load_torch_ext()
+
+
 class TensorProds(nn.Module):
     """Tensor product sandwiched by linear maps (managan/tensor_products.py:109-121)."""
 
@@ -210,7 +215,9 @@ class TensorProds(nn.Module):
     def forward(self, x_l, x_r):
         W_l, W_r, W_o = self.lin_l.W, self.lin_r.W, self.lin_o.W
         wants_grad = torch.is_grad_enabled() and any(t.requires_grad for t in (x_l, x_r, W_l, W_r, W_o))
-        if not wants_grad and ops.tensor_prods_supported(*self.prod.inds, W_l.shape[1], W_r.shape[1], W_l.shape[0],
-                                                         W_o.shape[0]):
-            return ops.tensor_prods(*self.prod.inds, W_l, W_r, W_o, x_l, x_r)     # one launch, nothing stored between
+        if not wants_grad:
+            # one launch, nothing stored between; through the C++ binding (a node-sized call is host time)
+            ext = _torch_ext()
+            if ext.tensor_prods_supported(*self.prod.inds, W_l.shape[1], W_r.shape[1], W_l.shape[0], W_o.shape[0]):
+                return ext.tensor_prods(*self.prod.inds, W_l, W_r, W_o, x_l, x_r)
         return self.lin_o(self.prod(self.lin_l(x_l), self.lin_r(x_r)))

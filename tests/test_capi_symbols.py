@@ -72,9 +72,9 @@ def test_torch_binding_loads_and_exports_the_reference_names():
     compiled extensions export (neighbour_grid.cpp:198-203, tensor_ops.cpp:180-182, codegen_tensops.cpp:2001-2010)."""
     L = importlib.import_module("learned-dynamics_amd._lib")
     ext = L.load_torch_ext()
-    for name in ("get_neighbours", "edges_read", "edges_reduce", "get_edges", "tensor_linear", "bee_fwd_cuda",
-                 "bee_bwl_cuda", "bee_bwr_cuda", "cow_o0_fwd_cuda", "cow_o0_bwl_cuda", "cow_o0_bwr_cuda", "cow_o1_fwd_cuda",
-                 "cow_o1_bwl_cuda", "cow_o1_bwr_cuda"):
+    for name in ("get_neighbours", "edges_read", "edges_reduce", "get_edges", "tensor_linear", "tensor_prods",
+                 "tensor_prods_supported", "bee_fwd_cuda", "bee_bwl_cuda", "bee_bwr_cuda", "cow_o0_fwd_cuda", "cow_o0_bwl_cuda",
+                 "cow_o0_bwr_cuda", "cow_o1_fwd_cuda", "cow_o1_bwl_cuda", "cow_o1_bwr_cuda"):
         assert callable(getattr(ext, name)), name
     import torch
     try:

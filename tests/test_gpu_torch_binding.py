@@ -137,3 +137,33 @@ def test_shims_are_the_binding_and_its_calls_cost_less_host_time(ext, pkg, ops):
         t_py = host_us(lambda: ops.tensor_linear_fwd(0, W, x))
     print(f"[host time per call] tensor_linear 256 x 64 -> 64: binding {t_ext:.1f} us, ctypes route {t_py:.1f} us")
     assert t_ext < t_py
+
+
+@pytest.mark.parametrize("inds", [(1, 1, 0), (0, 1, 1), (1, 1, 2), (2, 1, 1), (2, 2, 0)])
+def test_tensor_prods_equals_the_ctypes_route_and_the_module_uses_it(ext, ops, inds):
+    tp = importlib.import_module("learned-dynamics_amd.tensor_products")
+    g = torch.Generator().manual_seed(77)
+    mod = tp.TensorProds(*inds, 64, 64, 64, 64).cuda()
+    lead = (3, 37)
+    x_l = torch.randn(*lead, 64, *([3] * inds[0]), generator=g).cuda()
+    x_r = torch.randn(*lead, 64, *([3] * inds[1]), generator=g).cuda()
+    W_l, W_r, W_o = mod.lin_l.W.detach(), mod.lin_r.W.detach(), mod.lin_o.W.detach()
+    assert ext.tensor_prods_supported(*inds, 64, 64, 64, 64) == ops.tensor_prods_supported(*inds, 64, 64, 64, 64)
+    if not ext.tensor_prods_supported(*inds, 64, 64, 64, 64):
+        pytest.skip("not a one-launch problem")
+    y = ext.tensor_prods(*inds, W_l, W_r, W_o, x_l, x_r)
+    assert y.shape == (*lead, 64, *([3] * inds[2]))
+    assert torch.equal(y, ops.tensor_prods(*inds, W_l, W_r, W_o, x_l, x_r))
+    with torch.no_grad():
+        assert torch.equal(mod(x_l, x_r), y)
+    # a weight that is a view with padded rows goes in as it is; one with a non-unit inner stride is copied
+    wide = torch.zeros(64, 68, device="cuda")
+    wide[:, :64] = W_l
+    assert torch.equal(ext.tensor_prods(*inds, wide[:, :64], W_r, W_o, x_l, x_r), y)
+    assert torch.equal(ext.tensor_prods(*inds, W_l.t().contiguous().t(), W_r, W_o, x_l, x_r), y)
+    with pytest.raises(RuntimeError, match="shape mismatch"):
+        ext.tensor_prods(*inds, W_l[:, :32], W_r, W_o, x_l, x_r)
+    with pytest.raises(RuntimeError, match="do not broadcast"):
+        ext.tensor_prods(*inds, W_l, W_r, W_o, x_l[:2], x_r)
+    with pytest.raises(RuntimeError, match="float32 CUDA"):
+        ext.tensor_prods(*inds, W_l, W_r, W_o, x_l.cpu(), x_r)
