@@ -359,7 +359,145 @@ linear_rows_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restric
     }
 }
 
+// Few rows, few columns, long K (the output linears of one small system: 18 432 rows, K = 1280, 16 columns): the
+// row-streaming kernel above gives such a problem a handful of workgroups that each walk 40 chunks one barrier at a
+// time, about 1.3 us per chunk of load and LDS latency with nothing to overlap it.  Here a workgroup owns a tile of
+// 32 rows x 32 NI columns and its WAVES waves split K: wave w takes chunks w, w + WAVES, ... with private
+// accumulators, reads its W fragments straight from the packed planes (L2 resident; no LDS, no barrier in the loop),
+// and the partial tiles are summed through LDS in wave order, so the result does not depend on timing.
+template <int WAVES, int NI>
+__global__ void __launch_bounds__(64 * WAVES)
+linear_rows_splitk_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restrict__ w_inv,
+                                const float* __restrict__ X, const float* __restrict__ xmax, int xmax_parts,
+                                long xmax_stride, long xmax_div, long R, int I, int O, int O_pad,
+                                const float* __restrict__ bias, int act, int accumulate, float* __restrict__ Y,
+                                float* __restrict__ ymax, int tiles_n, int out_T) {
+    constexpr int TN = 32 * NI, THREADS = 64 * WAVES;
+    constexpr int kPitch = TN + 1;                            // floats per row of a partial tile
+    __shared__ float partial[WAVES][32 * kPitch];
+    __shared__ float inv_sx[32];
+
+    const long tile_m = blockIdx.x / tiles_n;
+    const int tile_n = (int)(blockIdx.x - tile_m * tiles_n);
+    const int tid = threadIdx.x;
+    const int lane = tid & 63, wave = tid >> 6;
+    const int m = lane & 31, g = lane >> 5;
+    const long r0 = tile_m * 32;
+    const int n0 = tile_n * TN;
+    const long plane_elems = (long)O_pad * I;
+
+    const long my_row = r0 + m;
+    const long ld_row = my_row < R ? my_row : R - 1;
+    const float* xrow = X + ld_row * I + 16 * g;
+    float sx;
+    {
+        float amax = 0.f;
+        const float* xm = xmax + (ld_row / xmax_div) * xmax_stride;
+        for (int p = 0; p < xmax_parts; p++) amax = fmaxf(amax, xm[p]);
+        float inv;
+        sx = pow2_scale(amax, &inv);
+        if (wave == 0 && g == 0) inv_sx[m] = inv;
+    }
+    // lane's fragment of W for MFMA step s, column block ni: row n0 + 32 ni + m, k = k0 + 16 g + 8 s .. + 8
+    const _Float16* wrow = Wp + (long)(n0 + m) * I + 16 * g;
+
+    floatx16 acc[NI];
+#pragma unroll
+    for (int ni = 0; ni < NI; ni++)
+#pragma unroll
+        for (int q = 0; q < 16; q++) acc[ni][q] = 0.f;
+
+    struct Chunk {
+        float4 a[4];
+        halfx8 wh[NI][2], wl[NI][2];
+    };
+    auto load = [&](Chunk& c, int k0) {
+#pragma unroll
+        for (int ni = 0; ni < NI; ni++)
+#pragma unroll
+            for (int s2 = 0; s2 < 2; s2++) {
+                c.wh[ni][s2] = *reinterpret_cast<const halfx8*>(wrow + (long)ni * 32 * I + k0 + 8 * s2);
+                c.wl[ni][s2] = *reinterpret_cast<const halfx8*>(wrow + plane_elems + (long)ni * 32 * I + k0 + 8 * s2);
+            }
+#pragma unroll
+        for (int j = 0; j < 4; j++) c.a[j] = *reinterpret_cast<const float4*>(xrow + k0 + 4 * j);
+    };
+    auto compute = [&](const Chunk& c) {
+#pragma unroll
+        for (int s2 = 0; s2 < 2; s2++) {
+            const HalfSplit4 p0 = split(c.a[2 * s2], sx), p1 = split(c.a[2 * s2 + 1], sx);
+            halfx8 ah, al;
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                ah[i] = p0.hi[i]; ah[4 + i] = p1.hi[i];
+                al[i] = p0.lo[i]; al[4 + i] = p1.lo[i];
+            }
+#pragma unroll
+            for (int ni = 0; ni < NI; ni++) {
+                acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(al, c.wh[ni][s2], acc[ni], 0, 0, 0);
+                acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, c.wl[ni][s2], acc[ni], 0, 0, 0);
+                acc[ni] = __builtin_amdgcn_mfma_f32_32x32x16_f16(ah, c.wh[ni][s2], acc[ni], 0, 0, 0);
+            }
+        }
+    };
+    // this wave's chunks, the next one requested before the current one is consumed
+    const int chunks = I / kCK;
+    Chunk cur, nxt;
+    if (wave < chunks) load(cur, wave * kCK);
+    for (int c = wave; c < chunks; c += WAVES) {
+        const bool more = c + WAVES < chunks;
+        if (more) load(nxt, (c + WAVES) * kCK);
+        compute(cur);
+        if (more) cur = nxt;
+    }
+    // partial tiles -> LDS; accumulator register q of block ni is row 8 (q / 4) + 4 g + q % 4, column 32 ni + m
+#pragma unroll
+    for (int ni = 0; ni < NI; ni++)
+#pragma unroll
+        for (int q = 0; q < 16; q++)
+            partial[wave][(8 * (q / 4) + 4 * g + (q % 4)) * kPitch + 32 * ni + m] = acc[ni][q];
+    __syncthreads();
+    // a thread finishes the elements e = tid, tid + THREADS, ...: row e / TN, column e % TN (the TN / 1 lanes of a
+    // row are neighbours, so its maximum is a shuffle away)
+    constexpr int kPer = 32 * TN / THREADS;
+    static_assert(32 * TN % THREADS == 0 && THREADS % TN == 0, "whole rows per pass");
+#pragma unroll
+    for (int j = 0; j < kPer; j++) {
+        const int e = tid + THREADS * j;
+        const int rl = e / TN, col = e - rl * TN;
+        float sum = 0.f;
+#pragma unroll
+        for (int w = 0; w < WAVES; w++) sum += partial[w][rl * kPitch + col];
+        const long r = r0 + rl;
+        const int n = n0 + col;
+        float v = 0.f;
+        if (r < R && n < O) {
+            const long row = r / out_T;
+            const long addr = (row * O + n) * out_T + (r - row * out_T);
+            v = activate(sum * inv_sx[rl] * w_inv[n] + (bias ? bias[n] : 0.f), act);
+            if (accumulate) v += Y[addr];
+            Y[addr] = v;
+        }
+        if (ymax) {
+            float mx = fabsf(v);
+#pragma unroll
+            for (int d = 1; d < TN; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+            if (col == 0 && r < R) ymax[r * tiles_n + tile_n] = mx;
+        }
+    }
+}
+
 inline int o_pad_of(int dim_out) { return (dim_out + 255) / 256 * 256; }
+
+// the split-K kernel's domain: one column tile of at most 64 columns (the packed planes are zero filled up to a
+// multiple of 256 rows, so a partly used tile reads zeros), at least 16 chunks of K, and few rows.  Measured
+// against the row-streaming kernel for K = 512 .. 2048: 11 - 19 us against 13 - 67 us up to 6144 rows; from
+// about 12 000 rows on the row-streaming kernel (which reads W once per 256 rows and keeps more of x in flight)
+// is level or ahead, except at 16 columns or fewer, where its 32-column tile is half empty (31 against 48 us at
+// 18 432 rows, K = 1280).
+inline bool use_splitk(long R, int I, int O) {
+    return O <= 64 && I >= 512 && (R <= 8192 || (O <= 16 && R <= 32768));
+}
 
 struct Shape {
     int ni;      // 32-column blocks per tile
@@ -462,6 +600,7 @@ int mg_components_to_rows(const float* x, long rows, int dim, int comps, int dim
 }
 
 int mg_tensor_linear_f16x2_rowmax_parts(long rows, int dim_in, int dim_out) {
+    if (use_splitk(rows, dim_in, dim_out)) return 1;
     return (int)ceil_div(dim_out, 32 * choose_shape(rows, dim_in, dim_out).ni);
 }
 
@@ -485,6 +624,19 @@ int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_
     const _Float16* planes = static_cast<const _Float16*>(packed_W);
     const float* w_inv = reinterpret_cast<const float*>(planes + 2L * O_pad * dim_in);
     hipStream_t st = (hipStream_t)stream;
+    if (use_splitk(rows, dim_in, dim_out)) {
+        const long tiles = ceil_div(rows, 32);
+        MG_REQUIRE(tiles <= 0x7fffffffL, "mg_tensor_linear_f16x2: grid too large (rows=%ld)", rows);
+        if (dim_out <= 32)
+            hipLaunchKernelGGL((linear_rows_splitk_f16x2_kernel<8, 1>), dim3((unsigned)tiles), dim3(512), 0, st, planes,
+                               w_inv, x, x_rowmax, x_rowmax_parts, x_rowmax_stride, x_rows_per_bound, rows, dim_in,
+                               dim_out, O_pad, bias, act, accumulate, y, y_rowmax, 1, out_comps);
+        else
+            hipLaunchKernelGGL((linear_rows_splitk_f16x2_kernel<8, 2>), dim3((unsigned)tiles), dim3(512), 0, st, planes,
+                               w_inv, x, x_rowmax, x_rowmax_parts, x_rowmax_stride, x_rows_per_bound, rows, dim_in,
+                               dim_out, O_pad, bias, act, accumulate, y, y_rowmax, 1, out_comps);
+        return check_launch("mg_tensor_linear_f16x2");
+    }
     const Shape sh = choose_shape(rows, dim_in, dim_out);
 #define MG_F16X2_LAUNCH(WV, N)                                                                                       \
     return launch<WV, N>(planes, w_inv, x, x_rowmax, x_rowmax_parts, x_rowmax_stride, x_rows_per_bound, rows, dim_in, \

@@ -154,7 +154,10 @@ def test_linear_modes_agree_with_float64(ops, mode, shape):
                                    (1024, 64, 8, 0), (40000, 160, 130, 1), (140001, 64, 256, 2),
                                    # column tiles chosen to divide the width and narrowed for few rows
                                    (49152, 128, 384, 1), (16384, 256, 384, 0), (512, 512, 512, 1), (300, 64, 96, 2),
-                                   (700, 64, 2080, 0), (2048, 64, 1056, 0)])
+                                   (700, 64, 2080, 0), (2048, 64, 1056, 0),
+                                   # few rows, at most 64 columns, long K: the waves of a workgroup split K
+                                   (18432, 1280, 16, 0), (6144, 1280, 64, 2), (33, 512, 32, 1), (1000, 544, 40, 0),
+                                   (8192, 768, 64, 1), (32768, 768, 16, 1), (1, 2048, 3, 0)])
 def test_linear_f16x2_rows_of_very_different_size(ops, shape):
     """mg_tensor_linear_f16x2 through the C ABI.  Rows spanning twelve orders of magnitude: the per-row
     power-of-two scales keep the error relative to EACH row's own scale at fp32 rounding level (a single
@@ -192,10 +195,12 @@ def test_linear_f16x2_rows_of_very_different_size(ops, shape):
         assert bool(((out.cpu().double() - ref2).abs() <= budget2).all())
 
 
-def test_linear_f16x2_component_outputs_and_node_bounds(ops):
-    """Rows that are (node, comp) pairs with one bound per node, output stored (node, chan, comp)."""
+@pytest.mark.parametrize("nodes,T,dim_in,dim_out", [(700, 9, 320, 16), (2048, 9, 1280, 16), (2048, 3, 1280, 64),
+                                                    (37, 3, 640, 24)])
+def test_linear_f16x2_component_outputs_and_node_bounds(ops, nodes, T, dim_in, dim_out):
+    """Rows that are (node, comp) pairs with one bound per node, output stored (node, chan, comp); the shapes with
+    K >= 512 take the kernel whose waves split K."""
     g = torch.Generator().manual_seed(4)
-    nodes, T, dim_in, dim_out = 700, 9, 320, 16
     W = torch.randn(dim_out, dim_in, generator=g) / dim_in ** 0.5
     x = torch.randn(nodes, T, dim_in, generator=g)
     bound = x.abs().amax(dim=(1, 2)).reshape(nodes, 1)
