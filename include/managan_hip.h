@@ -644,6 +644,18 @@ int mg_bee_message(const int* row_ptr, const int* dst, const int* node_order, in
                    const float* rhat, const float* enc, const float* La, const float* Lv, const float* Ld,
                    int chan, const float* enc_W /* (chan,8) */, const float* enc_b /* (chan) */,
                    float* P0, float* S1, float* S2, float* node_max, float* edge_max, mg_stream_t stream);
+/* mg_bee_message with the bias-free rank-2 output linear of Messages.forward (the Y_022 .. Y_212 of line 245,
+ * which commute with the edge sum of line 252) applied inside the kernel: Y2 (dim_d, 5 chan) = the five Y_lab.W side
+ * by side in the label order of S2, packed by mg_bee_pack_rank2_weight into mg_bee_rank2_weight_bytes(chan) bytes;
+ * out_d (N, dim_d, 9) = Y2 S2 replaces S2, which is never stored.  For chan = 64, 128 or 256 and dim_d <= 16
+ * (mg_bee_message_rank2_supported); the packing has no counterpart in the reference. */
+int mg_bee_message_rank2_supported(int chan, int dim_d);
+int mg_bee_rank2_weight_bytes(int chan, size_t* bytes);
+int mg_bee_pack_rank2_weight(const float* Y2, long row_stride, int chan, int dim_d, float* packed, mg_stream_t stream);
+int mg_bee_message_rank2(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
+                         const float* rhat, const float* enc, const float* La, const float* Lv, const float* Ld,
+                         int chan, const float* enc_W, const float* enc_b, const float* packed_Y2, int dim_d,
+                         float* P0, float* S1, float* out_d, float* node_max, float* edge_max, mg_stream_t stream);
 /* node_max (above and below; may be NULL): (N, ceil(chan/64)) partial maxima of |S1|, |S2| (of |P0|,
  * |P1|, |P2| below) per node, which mg_tensor_linear_f16x2 accepts as row bounds of those tensors
  * (x_rows_per_bound = 3 or 9); edge_max (may be NULL): (E, ceil(chan/64)) partial maxima of the rows

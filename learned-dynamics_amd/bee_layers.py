@@ -307,13 +307,16 @@ class Messages(nn.Module):
             lambda: ops.tensor_linear_fwd(1, self.L1.W, x_v.reshape(rows, -1, 3).contiguous(), y_layout=C),
             lambda: ops.tensor_linear_fwd(2, self.L2.W, x_d.reshape(rows, -1, 3, 3).contiguous(), y_layout=C),
             lambda: ops.bee_edge_geometry(r_ij.contiguous(), self.r0)], rows)
+        Y0, Y1, Y2 = self._cat_Y(LABELS_0), self._cat_Y(LABELS_1, 0.1), self._cat_Y(LABELS_2, 0.1)
+        # few rank-2 output channels: the edge kernel applies Y2 to its sums itself and S2 (nodes, 9, 5 chan) never exists
+        fused_d = ops.bee_rank2_supported(La.shape[1], Y2.shape[0])
         P0, S1, S2, nmax, emax = ops.bee_message(graph.row_ptr, graph.dst32, rhat, enc, La, Lv, Ld, self.lin_enc.weight,
-                                           self.lin_enc.bias, node_order=node_order, want_node_max=True)
+                                                 self.lin_enc.bias, node_order=node_order, want_node_max=True,
+                                                 Y2=Y2 if fused_d else None)
         E, chan = P0.shape[0], P0.shape[2]
         # scalar channel: per-edge linear + MLP, then the edge sum
         P0 = P0.reshape(E, 3 * chan)
         bound = emax if ops.get_linear_mode() == ops.LINEAR_F16X2 else None     # row maxima of P0 from the edge kernel
-        Y0, Y1, Y2 = self._cat_Y(LABELS_0), self._cat_Y(LABELS_1, 0.1), self._cat_Y(LABELS_2, 0.1)
 
         def scalar_channel(bound=bound):
             if bound is not None and ops.f16x2_rowsum_supported(E, 3 * chan, Y0.shape[0], P0):
@@ -328,10 +331,12 @@ class Messages(nn.Module):
                                                seg=graph.src32, s_x=s_psi)
         # vector and rank-2 channels: output linears after the edge sum, on node rows (beside the per-edge MLP of the
         # scalar channel when the system is small)
-        B_a, B_v, B_d = ops.concurrent([
-            scalar_channel,
-            lambda: ops.tensor_linear_fwd(1, Y1, S1.reshape(rows, 3, 5 * chan), x_layout=C, row_bound=nmax,
-                                          rows_per_bound=3),
-            lambda: ops.tensor_linear_fwd(2, Y2, S2.reshape(rows, 9, 5 * chan), x_layout=C, row_bound=nmax,
-                                          rows_per_bound=9)], rows)
+        jobs = [scalar_channel,
+                lambda: ops.tensor_linear_fwd(1, Y1, S1.reshape(rows, 3, 5 * chan), x_layout=C, row_bound=nmax,
+                                              rows_per_bound=3)]
+        if not fused_d:
+            jobs.append(lambda: ops.tensor_linear_fwd(2, Y2, S2.reshape(rows, 9, 5 * chan), x_layout=C, row_bound=nmax,
+                                                      rows_per_bound=9))
+        outs = ops.concurrent(jobs, rows)
+        B_a, B_v, B_d = outs[0], outs[1], (S2 if fused_d else outs[2])
         return (B_a.reshape(B, N, -1), B_v.reshape(B, N, -1, 3), B_d.reshape(B, N, -1, 3, 3))

@@ -17,6 +17,12 @@
 // applied to S1/S2 on N rows afterwards; the (comp, label, chan) order makes
 // each of those one plain GEMM with K = 5*chan.
 //
+// With Y2F the rank-2 sums do not leave the kernel either: the four waves of a workgroup hold the sums of
+// 4 / chunks whole nodes, the bias-free output linear of the rank-2 channel (K = 5 chan, dim_d <= 16 outputs) is
+// applied to them on the fp32 matrix cores (v_mfma_f32_16x16x4_f32: rows = the 9 components, 80 steps per wave),
+// the waves' partial results are summed through LDS, and (node, dim_d, 9) is stored instead of (node, 9, 5, chan):
+// 45 chan floats per node less to write, the same again less to read, and one GEMM launch less.
+//
 // Node features are read in component-major layout (node, comp, chan): the 13
 // gathers of a wave are 13 unit-stride 256-byte reads.  A lane owns one channel
 // and keeps its 60 running sums in registers; rows are summed in edge order.
@@ -123,14 +129,21 @@ __device__ __forceinline__ __bf16 gather_row(__amdgpu_buffer_rsrc_t r, unsigned 
 
 // T: storage type of the node features and of the outputs (float, or __bf16 with fp32 arithmetic)
 // PIPE: keep one edge of operands in flight ahead of the one being consumed (pays on long rows)
-template <typename T, bool PIPE>
+// Y2F: the rank-2 output linear is applied here (float storage, chan % 64 == 0, 1, 2 or 4 chunks, dim_d <= 16):
+// y2_packed as written by pack_rank2_weight_kernel, out_d (nodes, dim_d, 9); S2 is not touched
+constexpr int kTrPitch = 68;   // floats per LDS row of a wave's transposition buffer (16-byte aligned rows)
+typedef float floatx4 __attribute__((ext_vector_type(4)));
+
+template <typename T, bool PIPE, bool Y2F>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4)))
 bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst, const int* __restrict__ order,
                    long n_nodes, const float* __restrict__ rhat, const float* __restrict__ enc,
                    const T* __restrict__ La, const T* __restrict__ Lv, const T* __restrict__ Ld, int chan,
                    const float* __restrict__ enc_W, const float* __restrict__ enc_b, T* __restrict__ P0,
                    T* __restrict__ S1, T* __restrict__ S2, float* __restrict__ node_max,
-                   float* __restrict__ edge_max) {
+                   float* __restrict__ edge_max, const float* __restrict__ y2_packed, int dim_d,
+                   float* __restrict__ out_d) {
+    static_assert(!Y2F || std::is_same<T, float>::value, "the fused output linear is for float storage");
     const int lane = threadIdx.x & (kWave - 1);
     const int chunks = (chan + kWave - 1) / kWave;
     const long items = n_nodes * chunks;
@@ -144,21 +157,27 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
     // system's nodes into flight at every trip: 2.66 ms against 2.37 ms at 32 x 2048 atoms, 256 channels, and 5.26
     // against 4.44 ms at 65536 atoms with 90 neighbours, 128 channels.  (Giving each XCD one 64-channel chunk, so
     // that its L2 sees a quarter of each row, was measured with both grids and is slower by 5 %.)
-    const long per_xcd = (items + 7) / 8;
+    // Y2F: a workgroup's four items must be whole nodes, and its four waves must make the same trips (barriers)
+    const long per_xcd = Y2F ? (((items + 7) / 8 + 3) & ~3L) : (items + 7) / 8;
     const int xcd = blockIdx.x & 7;
     const long waves_per_xcd = (long)(gridDim.x >> 3) * (blockDim.x / kWave);
     const long wave_local = (long)(blockIdx.x >> 3) * (blockDim.x / kWave) + threadIdx.x / kWave;
 
     for (long item_local = wave_local; item_local < per_xcd; item_local += waves_per_xcd) {
-        const long item = uniform(xcd * per_xcd + item_local);
-        if (item >= items) break;
+        long item = uniform(xcd * per_xcd + item_local);
+        const bool valid = item < items;                       // uniform over the wave
+        if constexpr (Y2F) {
+            item = valid ? item : items - 1;                   // a wave without an item still meets the barriers
+        } else {
+            if (!valid) break;
+        }
         const long k_node = item / chunks;
         const int chunk = (int)(item - k_node * chunks);
         const int c = chunk * kWave + lane;
         const bool active = c < chan;
         const int cc = active ? c : chan - 1;   // inactive lanes shadow a valid channel, stores are masked
         const long node = order ? (long)order[k_node] : k_node;
-        const long lo = row_ptr[node], hi = row_ptr[node + 1];
+        const long lo = valid ? row_ptr[node] : 0, hi = valid ? row_ptr[node + 1] : 0;
 
         float w[8];
 #pragma unroll
@@ -277,13 +296,15 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
                 }
             }
         }
-        if (active) {
+        if (active && valid) {
             T* o1 = S1 + node * 15 * chan;
-            T* o2 = S2 + node * 45 * chan;
 #pragma unroll
             for (int k = 0; k < 15; k++) __builtin_nontemporal_store((T)s1[k], o1 + k * chan + lane_off);
+            if constexpr (!Y2F) {
+                T* o2 = S2 + node * 45 * chan;
 #pragma unroll
-            for (int k = 0; k < 45; k++) __builtin_nontemporal_store((T)s2[k], o2 + k * chan + lane_off);
+                for (int k = 0; k < 45; k++) __builtin_nontemporal_store((T)s2[k], o2 + k * chan + lane_off);
+            }
         }
         if (node_max) {
             // largest |sum| of this (node, 64-channel chunk): a row bound for the GEMMs that read S1 / S2
@@ -293,9 +314,87 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
 #pragma unroll
             for (int k = 0; k < 45; k++) mx = fmaxf(mx, fabsf(s2[k]));
             mx = wave_max_nonneg_last_lane(active ? mx : 0.f);
-            if (lane == kWave - 1) node_max[node * chunks + chunk] = mx;
+            if (lane == kWave - 1 && valid) node_max[node * chunks + chunk] = mx;
+        }
+        if constexpr (Y2F) {
+            // out[comp i][o] = sum over (label, channel) of s2[i][label][channel] Y2[o][label chan + channel].
+            // A lane holds one channel of all (comp, label); the matrix core wants lane (i, kk) to hold comp i at
+            // k = kk: one label at a time the wave's 9 x 64 values go through its own LDS rows, and step t of the
+            // label multiplies channels 16 kk + t (read four steps at a time).
+            __shared__ __attribute__((aligned(16))) float tr_buf[4][9 * kTrPitch];
+            __shared__ float part[4][16 * 16];
+            const int wave = threadIdx.x / kWave;
+            float* tr = tr_buf[wave];
+            const int ci = lane & 15, kk = lane >> 4;
+            const float* a_src = tr + (ci < 9 ? ci : 0) * kTrPitch + 16 * kk;
+            const float4* yb = reinterpret_cast<const float4*>(y2_packed) + (long)chunk * 5 * 4 * 64 + lane;
+            floatx4 d = {0.f, 0.f, 0.f, 0.f};
+            float4 b[4];
+#pragma unroll
+            for (int tq = 0; tq < 4; tq++) b[tq] = yb[tq * 64];
+#pragma unroll
+            for (int lab = 0; lab < 5; lab++) {
+#pragma unroll
+                for (int k = 0; k < 9; k++) tr[k * kTrPitch + lane] = (active && valid) ? s2[k * 5 + lab] : 0.f;
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+                float4 a[4];
+#pragma unroll
+                for (int tq = 0; tq < 4; tq++) {
+                    a[tq] = *reinterpret_cast<const float4*>(a_src + 4 * tq);
+                    if (ci >= 9) a[tq] = make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+                float4 bn[4];
+                if (lab < 4) {
+#pragma unroll
+                    for (int tq = 0; tq < 4; tq++) bn[tq] = yb[((lab + 1) * 4 + tq) * 64];
+                }
+#pragma unroll
+                for (int tq = 0; tq < 4; tq++) {
+                    d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[tq].x, b[tq].x, d, 0, 0, 0);
+                    d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[tq].y, b[tq].y, d, 0, 0, 0);
+                    d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[tq].z, b[tq].z, d, 0, 0, 0);
+                    d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[tq].w, b[tq].w, d, 0, 0, 0);
+                }
+                if (lab < 4) {
+#pragma unroll
+                    for (int tq = 0; tq < 4; tq++) b[tq] = bn[tq];
+                }
+                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+                __builtin_amdgcn_wave_barrier();                // the rows are rewritten by the next label
+                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+            }
+            // accumulator register q of lane l: comp 4 (l / 16) + q, output l % 16
+#pragma unroll
+            for (int q = 0; q < 4; q++) part[wave][(4 * kk + q) * 16 + ci] = d[q];
+            __syncthreads();
+            if (chunk == 0 && valid) {                          // the first wave of a node adds up its chunks
+                float* o = out_d + node * (long)dim_d * 9;
+                for (int idx = lane; idx < dim_d * 9; idx += kWave) {
+                    const int j = idx / 9, i = idx - 9 * j;
+                    float sum = 0.f;
+                    for (int wv = 0; wv < chunks; wv++) sum += part[wave + wv][i * 16 + j];
+                    o[idx] = sum;
+                }
+            }
+            __syncthreads();                                    // before a further trip writes part again
         }
     }
+}
+
+// Y2 (dim_d, 5 chan), row stride ld -> [chunk][label][tq][lane = 16 kk + j][tr] = Y2[j][label chan + 64 chunk + 16 kk + 4 tq + tr]
+// (zero for j >= dim_d): what lane (kk, j) of the fused kernel multiplies in steps 4 tq .. 4 tq + 3 of a label
+__global__ void __launch_bounds__(256) pack_rank2_weight_kernel(const float* __restrict__ Y2, long ld, int chan,
+                                                                int dim_d, float* __restrict__ packed) {
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long total = (long)(chan / 64) * 5 * 4 * 64 * 4;
+    if (idx >= total) return;
+    const int tr = (int)(idx & 3), lane = (int)((idx >> 2) & 63), tq = (int)((idx >> 8) & 3);
+    const long rest = idx >> 10;                              // chunk * 5 + label
+    const int label = (int)(rest % 5), chunk = (int)(rest / 5);
+    const int j = lane & 15, kk = lane >> 4;
+    packed[idx] = j < dim_d ? Y2[j * ld + (long)label * chan + 64 * chunk + 16 * kk + 4 * tq + tr] : 0.f;
 }
 
 }  // namespace
@@ -303,14 +402,22 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
 
 using namespace mg;
 
+static bool rank2_fusable(int chan, int dim_d) {
+    const int chunks = chan / 64;
+    return chan > 0 && chan % 64 == 0 && (chunks == 1 || chunks == 2 || chunks == 4) && dim_d >= 1 && dim_d <= 16;
+}
+
 template <typename T>
 static int launch_bee_message(const char* what, const int* row_ptr, const int* dst, const int* node_order, int n_nodes,
                               long n_edges, const float* rhat, const float* enc, const T* La, const T* Lv, const T* Ld,
                               int chan, const float* enc_W, const float* enc_b, T* P0, T* S1, T* S2,
-                              float* node_max, float* edge_max, mg_stream_t stream) {
+                              float* node_max, float* edge_max, mg_stream_t stream, const float* y2_packed = nullptr,
+                              int dim_d = 0, float* out_d = nullptr) {
     MG_REQUIRE(n_nodes >= 0 && n_edges >= 0 && chan >= 0, "%s: negative size", what);
     if (n_nodes == 0 || chan == 0) return MG_OK;
-    MG_REQUIRE(row_ptr && La && Lv && Ld && enc_W && enc_b && S1 && S2, "%s: null pointer", what);
+    const bool fused = y2_packed != nullptr;
+    MG_REQUIRE(row_ptr && La && Lv && Ld && enc_W && enc_b && S1 && (fused ? out_d != nullptr : S2 != nullptr),
+               "%s: null pointer", what);
     MG_REQUIRE(n_edges == 0 || (dst && rhat && enc && P0), "%s: null edge operand", what);
     MG_REQUIRE((long)n_nodes * 9 * chan * (long)sizeof(T) < (1L << 32),
                "%s: the rank-2 node rows must stay below 4 GiB (32-bit row offsets)", what);
@@ -320,14 +427,23 @@ static int launch_bee_message(const char* what, const int* row_ptr, const int* d
     MG_REQUIRE(blocks < (1L << 31), "%s: too many (node, channel chunk) items for one launch", what);
     // rows of a few edges do not repay the pipeline's start-up (one extra set of loads per row), unless the system
     // is so small that the chip is not filled and a row's chain of load latencies is all there is to the time
-    if (n_edges >= 8L * n_nodes || items <= 16384)
-        hipLaunchKernelGGL((bee_message_kernel<T, true>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                           row_ptr, dst, node_order, (long)n_nodes, rhat, enc, La, Lv, Ld, chan, enc_W, enc_b, P0, S1, S2,
-                           node_max, edge_max);
-    else
-        hipLaunchKernelGGL((bee_message_kernel<T, false>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream,
-                           row_ptr, dst, node_order, (long)n_nodes, rhat, enc, La, Lv, Ld, chan, enc_W, enc_b, P0, S1, S2,
-                           node_max, edge_max);
+    const bool pipe = n_edges >= 8L * n_nodes || items <= 16384;
+#define MG_BEE_LAUNCH(PIPE, Y2F)                                                                                      \
+    hipLaunchKernelGGL((bee_message_kernel<T, PIPE, Y2F>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, \
+                       row_ptr, dst, node_order, (long)n_nodes, rhat, enc, La, Lv, Ld, chan, enc_W, enc_b, P0, S1, S2, \
+                       node_max, edge_max, y2_packed, dim_d, out_d)
+    if constexpr (std::is_same<T, float>::value) {
+        if (fused) {
+            MG_REQUIRE(rank2_fusable(chan, dim_d), "%s: the fused rank-2 linear needs chan = 64, 128 or 256 and dim_d <= 16", what);
+            MG_REQUIRE(aligned16(y2_packed), "%s: packed weight must be 16-byte aligned", what);
+            if (pipe) MG_BEE_LAUNCH(true, true);
+            else MG_BEE_LAUNCH(false, true);
+            return check_launch(what);
+        }
+    }
+    if (pipe) MG_BEE_LAUNCH(true, false);
+    else MG_BEE_LAUNCH(false, false);
+#undef MG_BEE_LAUNCH
     return check_launch(what);
 }
 
@@ -351,6 +467,33 @@ int mg_bee_message(const int* row_ptr, const int* dst, const int* node_order, in
                    float* edge_max, mg_stream_t stream) {
     return launch_bee_message<float>("mg_bee_message", row_ptr, dst, node_order, n_nodes, n_edges, rhat, enc, La, Lv,
                                      Ld, chan, enc_W, enc_b, P0, S1, S2, node_max, edge_max, stream);
+}
+
+int mg_bee_message_rank2_supported(int chan, int dim_d) { return rank2_fusable(chan, dim_d) ? 1 : 0; }
+
+int mg_bee_rank2_weight_bytes(int chan, size_t* bytes) {
+    MG_REQUIRE(bytes != nullptr && chan >= 0, "mg_bee_rank2_weight_bytes: bad argument");
+    *bytes = (size_t)ceil_div(chan, 64) * 5 * 4 * 64 * 4 * sizeof(float);
+    return MG_OK;
+}
+
+int mg_bee_pack_rank2_weight(const float* Y2, long ld, int chan, int dim_d, float* packed, mg_stream_t stream) {
+    MG_REQUIRE(rank2_fusable(chan, dim_d), "mg_bee_pack_rank2_weight: needs chan = 64, 128 or 256 and dim_d <= 16");
+    MG_REQUIRE(Y2 && packed && ld >= 5L * chan, "mg_bee_pack_rank2_weight: null pointer or short rows");
+    const long total = (long)(chan / 64) * 5 * 4 * 64 * 4;
+    hipLaunchKernelGGL(pack_rank2_weight_kernel, dim3((unsigned)ceil_div(total, 256)), dim3(256), 0, (hipStream_t)stream,
+                       Y2, ld, chan, dim_d, packed);
+    return check_launch("mg_bee_pack_rank2_weight");
+}
+
+int mg_bee_message_rank2(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
+                         const float* rhat, const float* enc, const float* La, const float* Lv, const float* Ld, int chan,
+                         const float* enc_W, const float* enc_b, const float* packed_Y2, int dim_d, float* P0, float* S1,
+                         float* out_d, float* node_max, float* edge_max, mg_stream_t stream) {
+    MG_REQUIRE(packed_Y2 != nullptr, "mg_bee_message_rank2: null weight");
+    return launch_bee_message<float>("mg_bee_message_rank2", row_ptr, dst, node_order, n_nodes, n_edges, rhat, enc, La,
+                                     Lv, Ld, chan, enc_W, enc_b, P0, S1, nullptr, node_max, edge_max, stream, packed_Y2,
+                                     dim_d, out_d);
 }
 
 int mg_bee_message_bf16(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,

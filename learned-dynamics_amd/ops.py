@@ -2025,11 +2025,39 @@ def bee_edge_geometry(r_ij, r0):
     return enc, rhat
 
 
-def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=None, want_node_max=False):
+_rank2_cache = {}
+
+
+def bee_rank2_supported(chan, dim_d):
+    """Can the edge kernel apply the rank-2 output linear (dim_d, 5 chan) itself?"""
+    return bool(_lib.mg_bee_message_rank2_supported(int(chan), int(dim_d)))
+
+
+def _packed_rank2_weight(Y2, chan):
+    """Y2 (dim_d, 5 chan) in the lane order of the fused edge kernel; cached per tensor object and version."""
+    key = id(Y2)
+    hit = _rank2_cache.get(key)
+    version = tensor_version(Y2)
+    if hit is not None and version >= 0 and hit[0]() is Y2 and hit[1] == version and hit[2] == Y2.data_ptr():
+        return hit[3]
+    nbytes = ctypes.c_size_t(0)
+    L.check(_lib.mg_bee_rank2_weight_bytes(chan, ctypes.byref(nbytes)))
+    with torch.cuda.device(Y2.device):
+        packed = torch.empty(nbytes.value // 4, dtype=torch.float32, device=Y2.device)
+        L.check(_lib.mg_bee_pack_rank2_weight(_p(Y2), int(Y2.stride(0)), chan, int(Y2.size(0)), _p(packed), _stream()))
+    if len(_rank2_cache) > 256:
+        _rank2_cache.clear()
+    _rank2_cache[key] = (weakref.ref(Y2, lambda _, key=key: _rank2_cache.pop(key, None)), version, Y2.data_ptr(), packed)
+    return packed
+
+
+def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=None, want_node_max=False, Y2=None):
     """Fused products + edge sums of the rank-0/1/2 message (see mg_bee_message).
     La (N,chan), Lv (N,3,chan), Ld (N,9,chan) -> P0 (E,3,chan), S1 (N,3,5,chan), S2 (N,9,5,chan)
     (+ node_max (N, ceil(chan/64)) and edge_max (E, ceil(chan/64)): partial maxima of |S1|, |S2| per node
-    and of |P0| per edge, with want_node_max)."""
+    and of |P0| per edge, with want_node_max).
+    Y2 (dim_d, 5 chan), bee_rank2_supported(chan, dim_d): the rank-2 output linear is applied inside the kernel and
+    the third result is Y2 S2 as (N, dim_d, 9) instead of S2 (mg_bee_message_rank2)."""
     _check_input(row_ptr, "row_ptr", torch.int32)
     _check_input(dst, "dst", torch.int32)
     for t, nm in ((rhat, "rhat"), (enc, "enc"), (La, "La"), (Lv, "Lv"), (Ld, "Ld"), (enc_W, "enc_W"),
@@ -2050,15 +2078,30 @@ def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=No
         if node_order.numel() != N:
             raise RuntimeError("node_order must have one entry per node")
     dev = La.device
+    if Y2 is not None:
+        if not Y2.is_cuda or Y2.dtype != torch.float32:
+            raise RuntimeError("Y2 must be a float32 CUDA tensor")
+        if Y2.dim() != 2 or int(Y2.size(1)) != 5 * chan or Y2.stride(1) != 1:
+            raise RuntimeError("Y2 must be (dim_d, 5 chan) with unit stride along a row")
+        if not bee_rank2_supported(chan, Y2.size(0)):
+            raise RuntimeError("the fused rank-2 linear needs chan = 64, 128 or 256 and dim_d <= 16")
     with torch.cuda.device(dev):
         P0 = torch.empty(E, 3, chan, dtype=torch.float32, device=dev)
         S1 = torch.empty(N, 3, 5, chan, dtype=torch.float32, device=dev)
-        S2 = torch.empty(N, 9, 5, chan, dtype=torch.float32, device=dev)
         node_max = torch.empty(N, (chan + 63) // 64, dtype=torch.float32, device=dev) if want_node_max else None
         edge_max = torch.empty(E, (chan + 63) // 64, dtype=torch.float32, device=dev) if want_node_max else None
-        L.check(_lib.mg_bee_message(_p(row_ptr), _p(dst), _p(node_order), N, E, _p(rhat), _p(enc), _p(La), _p(Lv),
-                                    _p(Ld), chan, _p(enc_W), _p(enc_b), _p(P0), _p(S1), _p(S2), _p(node_max),
-                                    _p(edge_max), _stream()))
+        if Y2 is not None:
+            dim_d = int(Y2.size(0))
+            S2 = torch.empty(N, dim_d, 9, dtype=torch.float32, device=dev)
+            L.check(_lib.mg_bee_message_rank2(_p(row_ptr), _p(dst), _p(node_order), N, E, _p(rhat), _p(enc), _p(La),
+                                              _p(Lv), _p(Ld), chan, _p(enc_W), _p(enc_b),
+                                              _p(_packed_rank2_weight(Y2, chan)), dim_d, _p(P0), _p(S1), _p(S2),
+                                              _p(node_max), _p(edge_max), _stream()))
+        else:
+            S2 = torch.empty(N, 9, 5, chan, dtype=torch.float32, device=dev)
+            L.check(_lib.mg_bee_message(_p(row_ptr), _p(dst), _p(node_order), N, E, _p(rhat), _p(enc), _p(La), _p(Lv),
+                                        _p(Ld), chan, _p(enc_W), _p(enc_b), _p(P0), _p(S1), _p(S2), _p(node_max),
+                                        _p(edge_max), _stream()))
     return (P0, S1, S2, node_max, edge_max) if want_node_max else (P0, S1, S2)
 
 

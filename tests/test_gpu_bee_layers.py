@@ -96,6 +96,43 @@ def test_bee_message_kernel(ops, chan, E):
                 0, src, products(dt)[lab]).reshape(N, chan, 9).transpose(1, 2), f"bee_message S2 {lab} chan={chan}")
 
 
+@pytest.mark.parametrize("chan,dim_d,N,E", [(256, 16, 203, 3000), (128, 7, 101, 2500), (64, 16, 37, 900), (256, 1, 50, 30)])
+def test_bee_message_with_the_rank2_linear_inside(ops, chan, dim_d, N, E):
+    """mg_bee_message_rank2: Y2 S2 from the edge kernel against Y2 applied to the S2 of mg_bee_message by the oracle's
+    matmul; everything else the two entry points write is bit-equal.  Node counts that leave the last workgroup partly
+    filled (chan 128: two nodes per workgroup, odd node count), nodes without edges, and an uneven row stride of Y2."""
+    torch.manual_seed(chan + dim_d)
+    src = torch.sort(torch.randint(0, N, (E,))).values
+    src[src == 5] = 6
+    dst = torch.randint(0, N, (E,))
+    r = torch.randn(E, 3) * 2.5
+    La, Lv, Ld = torch.randn(N, chan).cuda(), torch.randn(N, 3, chan).cuda(), torch.randn(N, 9, chan).cuda()
+    encW, encb = (torch.randn(chan, 8) * 0.3).cuda(), torch.randn(chan).cuda()
+    wide = (torch.randn(dim_d, 5 * chan + 4) / (5 * chan) ** 0.5).cuda()
+    Y2 = wide[:, :5 * chan]
+    enc, rhat = ops.bee_edge_geometry(r.cuda(), 6.0)
+    row_ptr = ops.segment_row_ptr(src.int().cuda(), N)
+    assert ops.bee_rank2_supported(chan, dim_d) and not ops.bee_rank2_supported(chan, 17) and not ops.bee_rank2_supported(100, 8)
+    for node_order in (None, torch.randperm(N).int().cuda()):
+        args = (row_ptr, dst.int().cuda(), rhat, enc, La, Lv, Ld, encW, encb)
+        P0, S1, S2, nmax, emax = ops.bee_message(*args, node_order=node_order, want_node_max=True)
+        Q0, T1, out, nmax2, emax2 = ops.bee_message(*args, node_order=node_order, want_node_max=True, Y2=Y2)
+        assert torch.equal(Q0, P0) and torch.equal(T1, S1) and torch.equal(nmax2, nmax) and torch.equal(emax2, emax)
+        assert out.shape == (N, dim_d, 9)
+        s2 = S2.cpu().reshape(N, 9, 5 * chan)
+        assert_parity_of(out, lambda dt: (s2.to(dt) @ Y2.cpu().to(dt).t()).transpose(1, 2),
+                         f"rank-2 linear inside the edge kernel, chan={chan}, dim_d={dim_d}")
+    with pytest.raises(RuntimeError, match="dim_d <= 16"):
+        ops.bee_message(*args, Y2=torch.zeros(17, 5 * chan, device="cuda"))
+    with pytest.raises(RuntimeError, match="5 chan"):
+        ops.bee_message(*args, Y2=torch.zeros(8, 4 * chan, device="cuda"))
+    # the packed weight follows an in-place update of Y2's storage
+    with torch.no_grad():
+        wide.mul_(2.0)
+    out2 = ops.bee_message(*args, Y2=Y2)[2]
+    assert_parity_of(out2, lambda dt: (s2.to(dt) @ Y2.cpu().to(dt).t()).transpose(1, 2), "after the weight changed")
+
+
 def test_node_products_emit_node_maxima(ops):
     g = torch.Generator().manual_seed(3)
     N, chan = 50, 128
