@@ -715,8 +715,13 @@ def edge_kernel_roofline(torch, msg, graph, r_ij, rows, bf16=False):
         fn = lambda: ops.bee_message_bf16(graph.row_ptr, graph.dst32, rhat, enc, La, Lv, Ld, msg.lin_enc.weight,
                                           msg.lin_enc.bias, node_order=order)
     else:
+        # as the layer calls it: with few rank-2 output channels the kernel applies that output linear to its node
+        # sums itself (and then does not store them)
+        bl = importlib.import_module("learned-dynamics_amd.bee_layers")
+        Y2 = msg._cat_Y(bl.LABELS_2, 0.1)
+        fused = ops.bee_rank2_supported(chan, Y2.shape[0])
         fn = lambda: ops.bee_message(graph.row_ptr, graph.dst32, rhat, enc, La, Lv, Ld, msg.lin_enc.weight,
-                                     msg.lin_enc.bias, node_order=order, want_node_max=True)
+                                     msg.lin_enc.bias, node_order=order, want_node_max=True, Y2=Y2 if fused else None)
     t = event_time(torch, fn, 10)
     E = int(graph.src.numel())
     w = 2 if bf16 else 4
@@ -725,7 +730,9 @@ def edge_kernel_roofline(torch, msg, graph, r_ij, rows, bf16=False):
     # per-edge MLP) are not compulsory traffic and are listed on their own.
     nbytes = rows * (13 + 63) * chan * w + E * 16
     p0_bytes = E * 3 * chan * w
-    return {"kernel": "bee_message_kernel (gathers, 13 products, edge sums; one Messages layer)", "bound": "hbm",
+    return {"kernel": "bee_message_kernel (gathers, 13 products, edge sums; one Messages layer"
+                      + ("; the rank-2 output linear applied to the node sums in the kernel)" if not bf16 and fused else ")"),
+            "bound": "hbm",
             "achieved": nbytes / t / 1e9, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": nbytes / t / 1e9 / PEAK_HBM_GBS,
             "traffic": measured_traffic("bee_message_kernel", "stress_configs4_traffic.json" if bf16
                                         else "denoiser_configs3_traffic.json"),
