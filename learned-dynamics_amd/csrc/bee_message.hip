@@ -321,12 +321,15 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
             // A lane holds one channel of all (comp, label); the matrix core wants lane (i, kk) to hold comp i at
             // k = kk: one label at a time the wave's 9 x 64 values go through its own LDS rows, and step t of the
             // label multiplies channels 16 kk + t (read four steps at a time).
-            __shared__ __attribute__((aligned(16))) float tr_buf[4][9 * kTrPitch];
+            // (rows 9 .. 15 of the matrix operand are rows of zeros that are written once and never again)
+            __shared__ __attribute__((aligned(16))) float tr_buf[4][16 * kTrPitch];
             __shared__ float part[4][16 * 16];
             const int wave = threadIdx.x / kWave;
             float* tr = tr_buf[wave];
             const int ci = lane & 15, kk = lane >> 4;
-            const float* a_src = tr + (ci < 9 ? ci : 0) * kTrPitch + 16 * kk;
+#pragma unroll
+            for (int k = 9; k < 16; k++) tr[k * kTrPitch + lane] = 0.f;
+            const float* a_src = tr + ci * kTrPitch + 16 * kk;
             const float4* yb = reinterpret_cast<const float4*>(y2_packed) + (long)chunk * 5 * 4 * 64 + lane;
             floatx4 d = {0.f, 0.f, 0.f, 0.f};
             float4 b[4];
@@ -335,16 +338,13 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
 #pragma unroll
             for (int lab = 0; lab < 5; lab++) {
 #pragma unroll
-                for (int k = 0; k < 9; k++) tr[k * kTrPitch + lane] = (active && valid) ? s2[k * 5 + lab] : 0.f;
+                for (int k = 0; k < 9; k++) tr[k * kTrPitch + lane] = s2[k * 5 + lab];   // zeros in a wave without an item
                 __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
                 __builtin_amdgcn_wave_barrier();
                 __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
                 float4 a[4];
 #pragma unroll
-                for (int tq = 0; tq < 4; tq++) {
-                    a[tq] = *reinterpret_cast<const float4*>(a_src + 4 * tq);
-                    if (ci >= 9) a[tq] = make_float4(0.f, 0.f, 0.f, 0.f);
-                }
+                for (int tq = 0; tq < 4; tq++) a[tq] = *reinterpret_cast<const float4*>(a_src + 4 * tq);
                 float4 bn[4];
                 if (lab < 4) {
 #pragma unroll
