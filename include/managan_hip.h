@@ -656,6 +656,12 @@ int mg_bee_message_rank2(const int* row_ptr, const int* dst, const int* node_ord
                          const float* rhat, const float* enc, const float* La, const float* Lv, const float* Ld,
                          int chan, const float* enc_W, const float* enc_b, const float* packed_Y2, int dim_d,
                          float* P0, float* S1, float* out_d, float* node_max, float* edge_max, mg_stream_t stream);
+/* The rank-2 part of SelfTensProds.forward (archs/diffuser_atoms15.py:82-94) in one pass over the nodes: the five
+ * rank-2 products of l = L_k x_k and r = R_k x_k (component-major operands as for mg_bee_node_products) and their
+ * output linears Y_022 .. Y_212, packed as for mg_bee_message_rank2; out_d (N, dim_d, 9).  Same domain. */
+int mg_bee_node_products_rank2(long n_nodes, int chan, const float* l0, const float* l1, const float* l2,
+                               const float* r0, const float* r1, const float* r2, const float* packed_Y2, int dim_d,
+                               float* out_d, mg_stream_t stream);
 /* node_max (above and below; may be NULL): (N, ceil(chan/64)) partial maxima of |S1|, |S2| (of |P0|,
  * |P1|, |P2| below) per node, which mg_tensor_linear_f16x2 accepts as row bounds of those tensors
  * (x_rows_per_bound = 3 or 9); edge_max (may be NULL): (E, ceil(chan/64)) partial maxima of the rows

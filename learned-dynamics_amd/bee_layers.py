@@ -154,8 +154,13 @@ class SelfTensProds(nn.Module):
                 return torch.cat(cols, dim=1).amax(dim=1)
             bound = 9.0 * node_max(pairs[:3]) * node_max(pairs[3:])
             Ys = [_cat_Y(self, labels) for labels in (LABELS_0, LABELS_1, LABELS_2)]
-            y_a, y_v, y_d = ops.concurrent([(lambda k=k: ops.bee_products_linear(k, Ys[k], *ops_in, bound))
-                                            for k in range(3)], rows)
+            jobs = [(lambda k=k: ops.bee_products_linear(k, Ys[k], *ops_in, bound)) for k in range(2)]
+            if ops.bee_rank2_supported(chan, Ys[2].shape[0]):
+                # few rank-2 output channels: fp32 matrix cores on the products of one node at a time
+                jobs.append(lambda: ops.bee_node_products_rank2(*ops_in, Ys[2]))
+            else:
+                jobs.append(lambda: ops.bee_products_linear(2, Ys[2], *ops_in, bound))
+            y_a, y_v, y_d = ops.concurrent(jobs, rows)
         else:
             P0, P1, P2, nmax = ops.bee_node_products(*ops_in, want_node_max=True)
             # nmax: per-node maxima of the products, the row bounds of the three GEMMs

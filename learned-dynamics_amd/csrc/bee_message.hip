@@ -27,6 +27,7 @@
 // gathers of a wave are 13 unit-stride 256-byte reads.  A lane owns one channel
 // and keeps its 60 running sums in registers; rows are summed in edge order.
 #include "common.hpp"
+#include "rank2_linear.hpp"
 #include <type_traits>
 
 namespace mg {
@@ -131,9 +132,6 @@ __device__ __forceinline__ __bf16 gather_row(__amdgpu_buffer_rsrc_t r, unsigned 
 // PIPE: keep one edge of operands in flight ahead of the one being consumed (pays on long rows)
 // Y2F: the rank-2 output linear is applied here (float storage, chan % 64 == 0, 1, 2 or 4 chunks, dim_d <= 16):
 // y2_packed as written by pack_rank2_weight_kernel, out_d (nodes, dim_d, 9); S2 is not touched
-constexpr int kTrPitch = 68;   // floats per LDS row of a wave's transposition buffer (16-byte aligned rows)
-typedef float floatx4 __attribute__((ext_vector_type(4)));
-
 template <typename T, bool PIPE, bool Y2F>
 __global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 4)))
 bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst, const int* __restrict__ order,
@@ -317,68 +315,10 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
             if (lane == kWave - 1 && valid) node_max[node * chunks + chunk] = mx;
         }
         if constexpr (Y2F) {
-            // out[comp i][o] = sum over (label, channel) of s2[i][label][channel] Y2[o][label chan + channel].
-            // A lane holds one channel of all (comp, label); the matrix core wants lane (i, kk) to hold comp i at
-            // k = kk: one label at a time the wave's 9 x 64 values go through its own LDS rows, and step t of the
-            // label multiplies channels 16 kk + t (read four steps at a time).
-            // (rows 9 .. 15 of the matrix operand are rows of zeros that are written once and never again)
             __shared__ __attribute__((aligned(16))) float tr_buf[4][16 * kTrPitch];
             __shared__ float part[4][16 * 16];
-            const int wave = threadIdx.x / kWave;
-            float* tr = tr_buf[wave];
-            const int ci = lane & 15, kk = lane >> 4;
-#pragma unroll
-            for (int k = 9; k < 16; k++) tr[k * kTrPitch + lane] = 0.f;
-            const float* a_src = tr + ci * kTrPitch + 16 * kk;
-            const float4* yb = reinterpret_cast<const float4*>(y2_packed) + (long)chunk * 5 * 4 * 64 + lane;
-            floatx4 d = {0.f, 0.f, 0.f, 0.f};
-            float4 b[4];
-#pragma unroll
-            for (int tq = 0; tq < 4; tq++) b[tq] = yb[tq * 64];
-#pragma unroll
-            for (int lab = 0; lab < 5; lab++) {
-#pragma unroll
-                for (int k = 0; k < 9; k++) tr[k * kTrPitch + lane] = s2[k * 5 + lab];   // zeros in a wave without an item
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                __builtin_amdgcn_wave_barrier();
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-                float4 a[4];
-#pragma unroll
-                for (int tq = 0; tq < 4; tq++) a[tq] = *reinterpret_cast<const float4*>(a_src + 4 * tq);
-                float4 bn[4];
-                if (lab < 4) {
-#pragma unroll
-                    for (int tq = 0; tq < 4; tq++) bn[tq] = yb[((lab + 1) * 4 + tq) * 64];
-                }
-#pragma unroll
-                for (int tq = 0; tq < 4; tq++) {
-                    d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[tq].x, b[tq].x, d, 0, 0, 0);
-                    d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[tq].y, b[tq].y, d, 0, 0, 0);
-                    d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[tq].z, b[tq].z, d, 0, 0, 0);
-                    d = __builtin_amdgcn_mfma_f32_16x16x4f32(a[tq].w, b[tq].w, d, 0, 0, 0);
-                }
-                if (lab < 4) {
-#pragma unroll
-                    for (int tq = 0; tq < 4; tq++) b[tq] = bn[tq];
-                }
-                __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-                __builtin_amdgcn_wave_barrier();                // the rows are rewritten by the next label
-                __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-            }
-            // accumulator register q of lane l: comp 4 (l / 16) + q, output l % 16
-#pragma unroll
-            for (int q = 0; q < 4; q++) part[wave][(4 * kk + q) * 16 + ci] = d[q];
-            __syncthreads();
-            if (chunk == 0 && valid) {                          // the first wave of a node adds up its chunks
-                float* o = out_d + node * (long)dim_d * 9;
-                for (int idx = lane; idx < dim_d * 9; idx += kWave) {
-                    const int j = idx / 9, i = idx - 9 * j;
-                    float sum = 0.f;
-                    for (int wv = 0; wv < chunks; wv++) sum += part[wave + wv][i * 16 + j];
-                    o[idx] = sum;
-                }
-            }
-            __syncthreads();                                    // before a further trip writes part again
+            rank2_linear_of_node_sums(s2, tr_buf, part, chunk, chunks, valid, y2_packed, dim_d,
+                                      out_d + node * (long)dim_d * 9);
         }
     }
 }
@@ -401,11 +341,6 @@ __global__ void __launch_bounds__(256) pack_rank2_weight_kernel(const float* __r
 }  // namespace mg
 
 using namespace mg;
-
-static bool rank2_fusable(int chan, int dim_d) {
-    const int chunks = chan / 64;
-    return chan > 0 && chan % 64 == 0 && (chunks == 1 || chunks == 2 || chunks == 4) && dim_d >= 1 && dim_d <= 16;
-}
 
 template <typename T>
 static int launch_bee_message(const char* what, const int* row_ptr, const int* dst, const int* node_order, int n_nodes,

@@ -2051,6 +2051,28 @@ def _packed_rank2_weight(Y2, chan):
     return packed
 
 
+def bee_node_products_rank2(l0, l1, l2, r0, r1, r2, Y2):
+    """The rank-2 output of SelfTensProds from its six operands in one kernel: Y2 (dim_d, 5 chan) applied to the five
+    rank-2 products of l0/r0 (N, chan), l1/r1 (N, 3, chan), l2/r2 (N, 9, chan) -> (N, dim_d, 9); the products are
+    never stored.  For bee_rank2_supported(chan, dim_d)."""
+    for t, nm in ((l0, "l0"), (l1, "l1"), (l2, "l2"), (r0, "r0"), (r1, "r1"), (r2, "r2")):
+        _check_input(t, nm)
+    N, chan = int(l0.size(0)), int(l0.size(1))
+    for t, comps in ((l0, None), (r0, None), (l1, 3), (r1, 3), (l2, 9), (r2, 9)):
+        if tuple(t.shape) != ((N, chan) if comps is None else (N, comps, chan)):
+            raise RuntimeError("operands must be (nodes, chan), (nodes, 3, chan), (nodes, 9, chan)")
+    if not Y2.is_cuda or Y2.dtype != torch.float32 or Y2.dim() != 2 or int(Y2.size(1)) != 5 * chan or Y2.stride(1) != 1:
+        raise RuntimeError("Y2 must be a float32 CUDA tensor (dim_d, 5 chan) with unit stride along a row")
+    if not bee_rank2_supported(chan, Y2.size(0)):
+        raise RuntimeError("the fused rank-2 linear needs chan = 64, 128 or 256 and dim_d <= 16")
+    dim_d = int(Y2.size(0))
+    with torch.cuda.device(l0.device):
+        out = torch.empty(N, dim_d, 9, dtype=torch.float32, device=l0.device)
+        L.check(_lib.mg_bee_node_products_rank2(N, chan, _p(l0), _p(l1), _p(l2), _p(r0), _p(r1), _p(r2),
+                                                _p(_packed_rank2_weight(Y2, chan)), dim_d, _p(out), _stream()))
+    return out
+
+
 def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=None, want_node_max=False, Y2=None):
     """Fused products + edge sums of the rank-0/1/2 message (see mg_bee_message).
     La (N,chan), Lv (N,3,chan), Ld (N,9,chan) -> P0 (E,3,chan), S1 (N,3,5,chan), S2 (N,9,5,chan)

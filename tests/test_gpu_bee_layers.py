@@ -346,6 +346,43 @@ def test_products_and_output_linears_in_one_kernel(pkg, chan, dims, N):
             assert_parity_of(y[small.cuda()], lambda dt: ref(dt)[small], f"bee_products_linear rank {rank}, small rows")
 
 
+@pytest.mark.parametrize("chan,dim_d,N", [(256, 16, 1001), (128, 5, 333), (64, 16, 70), (256, 1, 2)])
+def test_rank2_products_and_their_output_linear_in_one_kernel(pkg, chan, dim_d, N):
+    """mg_bee_node_products_rank2 against float64 einsums of the oracle's rank-2 products; node counts that leave the
+    last workgroup partly filled, nodes of very different size, a weight with an uneven row stride."""
+    ops = importlib.import_module("learned-dynamics_amd.ops")
+    g = torch.Generator().manual_seed(chan + N)
+    size = torch.rand(N, 1, generator=g) * 3 + 0.01
+    l = [torch.randn(N, chan, generator=g) * size, torch.randn(N, 3, chan, generator=g) * size[:, None],
+         torch.randn(N, 9, chan, generator=g) * size[:, None]]
+    r = [torch.randn(N, chan, generator=g), torch.randn(N, 3, chan, generator=g), torch.randn(N, 9, chan, generator=g)]
+    dev = [t.cuda() for t in l + r]
+    wide = (torch.randn(dim_d, 5 * chan + 8, generator=g) / (5 * chan) ** 0.5).cuda()
+    W = wide[:, :5 * chan]
+    y = ops.bee_node_products_rank2(*dev, W)
+    assert y.shape == (N, dim_d, 9)
+    to_ref = lambda t, k: t if k == 0 else t.reshape(N, 3 ** k, chan).transpose(1, 2).reshape(N, chan, *([3] * k))
+    labs = ("022", "202", "112", "222", "212")
+
+    def ref(dt):
+        pr = dict(zip(OP.BEE_ORDER, OP.bee(*[to_ref(t.to(dt), k) for k, t in enumerate(l)],
+                                           *[to_ref(t.to(dt), k) for k, t in enumerate(r)])))
+        return sum(torch.einsum("oc,ncxy->noxy", W[:, k * chan:(k + 1) * chan].cpu().to(dt), pr[lab])
+                   for k, lab in enumerate(labs)).reshape(N, dim_d, 9)
+
+    assert_parity_of(y, ref, f"rank-2 products + linear, chan={chan}, dim_d={dim_d}")
+    small = (size[:, 0] < 0.1)
+    if bool(small.any()):
+        assert_parity_of(y[small.cuda()], lambda dt: ref(dt)[small], "rank-2 products + linear, small nodes")
+    # the stored-products route gives the same within the same bar
+    P2 = ops.bee_node_products(*dev)[2]
+    stored = ops.tensor_linear_fwd(2, W, P2.reshape(N, 9, 5 * chan), x_layout=ops.LAYOUT_COMP_CHAN)
+    assert_parity_of(stored.reshape(N, dim_d, 9), ref, "stored products + GEMM")
+    with pytest.raises(RuntimeError, match="dim_d <= 16"):
+        ops.bee_node_products_rank2(*dev, torch.zeros(32, 5 * chan, device="cuda"))
+    assert ops.bee_node_products_rank2(*[t[:0] for t in dev], W).shape == (0, dim_d, 9)
+
+
 def test_self_tens_prods_module_fused_path(pkg):
     """SelfTensProds at a size that takes the products + linears kernel (chan % 32 == 0, >= 8192 nodes)."""
     bee = importlib.import_module("learned-dynamics_amd.bee_layers")
