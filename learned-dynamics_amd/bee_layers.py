@@ -218,18 +218,22 @@ class MLP(nn.Module):
         return out.reshape(*lead, out.shape[-1])
 
 
-    def summed_over_rows(self, x, row_ptr, n_out, plus_identity=False, bound=None, scale=1.0, seg=None, s_x=None):
+    def summed_over_rows(self, x, row_ptr, n_out, plus_identity=False, bound=None, scale=1.0, seg=None, s_x=None,
+                         count=None):
         """scale * (sum over the rows of each CSR segment of forward(x, plus_identity)), x (rows, d) ->
         (n_out, d).  Only the first two layers are nonlinear: the direct linear and the last layer commute
         with the sum, so they run on the n_out summed rows instead of on every row:
             sum_e mlp(x_e) = (W_direct [+ I]) sum_e x_e + W_last sum_e h_e + (rows in the segment) b_last
         with h = act(W_2 act(W_1 x + b_1) + b_2).  seg (rows,) int32: the segment of every row; with it the
         second layer sums its output rows in its own epilogue and h is never stored.  s_x: sum_e x_e if the
-        caller already has it."""
-        Wd = self.lin_direct.weight
-        if plus_identity:
-            Wd = _derived(self, "direct_plus_identity", (Wd,),
-                          lambda: Wd + torch.eye(Wd.shape[0], device=Wd.device, dtype=Wd.dtype))
+        caller already has it; count (n_out, 1) float32: the rows per segment, if the caller has them.
+        The scale is carried by the two node-level matrices and the bias (scaled copies cached with the weights)."""
+        Wd0, W_last0, b_last0 = self.lin_direct.weight, self.layers[4].weight, self.layers[4].bias
+        Wd = _derived(self, ("direct_scaled", plus_identity, scale), (Wd0,),
+                      lambda: scale * (Wd0 + torch.eye(Wd0.shape[0], device=Wd0.device, dtype=Wd0.dtype)
+                                       if plus_identity else Wd0))
+        W_last = W_last0 if scale == 1.0 else _derived(self, ("last_scaled", scale), (W_last0,), lambda: scale * W_last0)
+        b_last = b_last0 if scale == 1.0 else _derived(self, ("last_bias_scaled", scale), (b_last0,), lambda: scale * b_last0)
         L = self.layers
         if bound is None and ops.get_linear_mode() == ops.LINEAR_F16X2:
             bound = ops.row_absmax(x)
@@ -245,10 +249,10 @@ class MLP(nn.Module):
         if s_x is None:
             s_x = ops.segment_sum_csr(x, row_ptr, n_out)
         out = ops.tensor_linear_fwd(0, Wd, s_x)
-        ops.tensor_linear_fwd(0, L[4].weight, s_h, out=out, accumulate=True)
-        count = (row_ptr[1:] - row_ptr[:-1]).to(out.dtype)[:, None]
-        out = torch.addcmul(out, count, L[4].bias[None, :])
-        return out.mul_(scale) if scale != 1.0 else out
+        ops.tensor_linear_fwd(0, W_last, s_h, out=out, accumulate=True)
+        if count is None:
+            count = (row_ptr[1:] - row_ptr[:-1]).to(out.dtype)[:, None]
+        return out.addcmul_(count, b_last[None, :])
 
 
 class DisplacementTensors(nn.Module):
@@ -333,7 +337,7 @@ class Messages(nn.Module):
                 psi_a, bound = _linear(P0, Y0, None, ops.ACT_NONE, bound)
                 s_psi = None
             return self.mlp_a.summed_over_rows(psi_a, graph.row_ptr, rows, plus_identity=True, bound=bound, scale=0.1,
-                                               seg=graph.src32, s_x=s_psi)
+                                               seg=graph.src32, s_x=s_psi, count=graph.degree)
         # vector and rank-2 channels: output linears after the edge sum, on node rows (beside the per-edge MLP of the
         # scalar channel when the system is small)
         jobs = [scalar_channel,

@@ -52,6 +52,17 @@ class Graph:
             self._row_ptr = ops.segment_row_ptr(self.src32, self.batch * self.nodes)
         return self._row_ptr
 
+    @property
+    def degree(self):
+        """Edges per node as a float32 column (nodes, 1): what a per-edge bias sums to.  Formed once per graph, except
+        for a capacity-sized graph, whose row pointer is rewritten in place by every search of a captured rollout."""
+        rp = self.row_ptr
+        if getattr(self, "padded", False):
+            return (rp[1:] - rp[:-1]).to(torch.float32)[:, None]
+        if getattr(self, "_degree", None) is None:
+            self._degree = (rp[1:] - rp[:-1]).to(torch.float32)[:, None]
+        return self._degree
+
     @staticmethod
     def radius_graph(r0, box, pos, celllist_max=32, neighbours_max=64):
         """Nodes are connected if they are within r0 of each other under periodic
