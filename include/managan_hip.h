@@ -655,7 +655,8 @@ int mg_bee_pack_rank2_weight(const float* Y2, long row_stride, int chan, int dim
 int mg_bee_message_rank2(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
                          const float* rhat, const float* enc, const float* La, const float* Lv, const float* Ld,
                          int chan, const float* enc_W, const float* enc_b, const float* packed_Y2, int dim_d,
-                         float* P0, float* S1, float* out_d, float* node_max, float* edge_max, mg_stream_t stream);
+                         float* P0, float* S1, float* out_d, int accumulate /* out_d += Y2 S2 instead of = */,
+                         float* node_max, float* edge_max, mg_stream_t stream);
 /* The rank-2 part of SelfTensProds.forward (archs/diffuser_atoms15.py:82-94) in one pass over the nodes: the five
  * rank-2 products of l = L_k x_k and r = R_k x_k (component-major operands as for mg_bee_node_products) and their
  * output linears Y_022 .. Y_212, packed as for mg_bee_message_rank2; out_d (N, dim_d, 9).  Same domain. */

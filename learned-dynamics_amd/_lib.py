@@ -68,7 +68,7 @@ _SIGNATURES = {
     "mg_bee_message_rank2_supported": [i32, i32],
     "mg_bee_rank2_weight_bytes": [i32, vp],
     "mg_bee_pack_rank2_weight": [vp, i64, i32, i32, vp, vp],
-    "mg_bee_message_rank2": [vp, vp, vp, i32, i64, vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, vp, vp, vp, vp, vp],
+    "mg_bee_message_rank2": [vp, vp, vp, i32, i64, vp, vp, vp, vp, vp, i32, vp, vp, vp, i32, vp, vp, vp, i32, vp, vp, vp],
     "mg_linear_packed_weight_bytes": [i32, i32, ctypes.POINTER(ctypes.c_size_t)],
     "mg_linear_pack_weight": [vp, i64, i64, i32, i32, vp, vp],
     "mg_tensor_linear_packed": [vp, vp, i64, i32, i32, vp, i32, i32, i32, vp, vp],

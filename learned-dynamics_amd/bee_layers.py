@@ -219,7 +219,7 @@ class MLP(nn.Module):
 
 
     def summed_over_rows(self, x, row_ptr, n_out, plus_identity=False, bound=None, scale=1.0, seg=None, s_x=None,
-                         count=None):
+                         count=None, add_to=None):
         """scale * (sum over the rows of each CSR segment of forward(x, plus_identity)), x (rows, d) ->
         (n_out, d).  Only the first two layers are nonlinear: the direct linear and the last layer commute
         with the sum, so they run on the n_out summed rows instead of on every row:
@@ -227,7 +227,8 @@ class MLP(nn.Module):
         with h = act(W_2 act(W_1 x + b_1) + b_2).  seg (rows,) int32: the segment of every row; with it the
         second layer sums its output rows in its own epilogue and h is never stored.  s_x: sum_e x_e if the
         caller already has it; count (n_out, 1) float32: the rows per segment, if the caller has them.
-        The scale is carried by the two node-level matrices and the bias (scaled copies cached with the weights)."""
+        The scale is carried by the two node-level matrices and the bias (scaled copies cached with the weights).
+        add_to (n_out, d) contiguous: the result is added to it in place (and it is returned)."""
         Wd0, W_last0, b_last0 = self.lin_direct.weight, self.layers[4].weight, self.layers[4].bias
         Wd = _derived(self, ("direct_scaled", plus_identity, scale), (Wd0,),
                       lambda: scale * (Wd0 + torch.eye(Wd0.shape[0], device=Wd0.device, dtype=Wd0.dtype)
@@ -248,7 +249,10 @@ class MLP(nn.Module):
         del h
         if s_x is None:
             s_x = ops.segment_sum_csr(x, row_ptr, n_out)
-        out = ops.tensor_linear_fwd(0, Wd, s_x)
+        if add_to is None:
+            out = ops.tensor_linear_fwd(0, Wd, s_x)
+        else:
+            out = ops.tensor_linear_fwd(0, Wd, s_x, out=add_to, accumulate=True)
         ops.tensor_linear_fwd(0, W_last, s_h, out=out, accumulate=True)
         if count is None:
             count = (row_ptr[1:] - row_ptr[:-1]).to(out.dtype)[:, None]
@@ -299,13 +303,19 @@ class Messages(nn.Module):
     def _cat_Y(self, labels, scale=None):
         return _cat_Y(self, labels, scale)
 
-    def forward(self, graph: Graph, r_ij, x_a, x_v, x_d, node_order="cell"):
+    def forward(self, graph: Graph, r_ij, x_a, x_v, x_d, node_order="cell", add_to_inputs=False):
         """x_a (batch, nodes, dim_a), x_v (..., dim_v, 3), x_d (..., dim_d, 3, 3), r_ij (edges, 3).
         Returns 0.1 * sum over edges of the messages: (B_a, B_v, B_d) with the input shapes.
         node_order: row processing order of the edge kernel ("cell": the graph's cell order when it has
-        one, None: index order, or an int32 tensor); it does not change the results."""
+        one, None: index order, or an int32 tensor); it does not change the results.
+        add_to_inputs: returns (x_a + B_a, x_v + B_v, x_d + B_d) instead, the residual step of the denoiser's
+        block (archs/diffuser_atoms15.py:276-279).  Without autograd and with contiguous inputs the sums are formed
+        IN the inputs' memory by the kernels that produce the messages (their last use as inputs is over by then), so
+        the caller must own x_a, x_v, x_d; three full-size additions per block are not launched."""
         if diff.wants_grad(self, r_ij, x_a, x_v, x_d):
-            return diff.bee_messages(self, graph, r_ij, x_a, x_v, x_d)
+            out = diff.bee_messages(self, graph, r_ij, x_a, x_v, x_d)
+            return tuple(x + d for x, d in zip((x_a, x_v, x_d), out)) if add_to_inputs else out
+        in_place = add_to_inputs and x_a.is_contiguous() and x_v.is_contiguous() and x_d.is_contiguous()
         if isinstance(node_order, str):
             node_order = getattr(graph, "cell_order", None)
         B, N = x_a.shape[:2]
@@ -321,7 +331,8 @@ class Messages(nn.Module):
         fused_d = ops.bee_rank2_supported(La.shape[1], Y2.shape[0])
         P0, S1, S2, nmax, emax = ops.bee_message(graph.row_ptr, graph.dst32, rhat, enc, La, Lv, Ld, self.lin_enc.weight,
                                                  self.lin_enc.bias, node_order=node_order, want_node_max=True,
-                                                 Y2=Y2 if fused_d else None)
+                                                 Y2=Y2 if fused_d else None,
+                                                 out_d=x_d.reshape(rows, -1, 9) if (fused_d and in_place) else None)
         E, chan = P0.shape[0], P0.shape[2]
         # scalar channel: per-edge linear + MLP, then the edge sum
         P0 = P0.reshape(E, 3 * chan)
@@ -337,15 +348,21 @@ class Messages(nn.Module):
                 psi_a, bound = _linear(P0, Y0, None, ops.ACT_NONE, bound)
                 s_psi = None
             return self.mlp_a.summed_over_rows(psi_a, graph.row_ptr, rows, plus_identity=True, bound=bound, scale=0.1,
-                                               seg=graph.src32, s_x=s_psi, count=graph.degree)
+                                               seg=graph.src32, s_x=s_psi, count=graph.degree,
+                                               add_to=x_a.reshape(rows, -1) if in_place else None)
         # vector and rank-2 channels: output linears after the edge sum, on node rows (beside the per-edge MLP of the
         # scalar channel when the system is small)
+        into_v = dict(out=x_v.reshape(rows, -1, 3), accumulate=True) if in_place else {}
+        into_d = dict(out=x_d.reshape(rows, -1, 3, 3), accumulate=True) if in_place else {}
         jobs = [scalar_channel,
                 lambda: ops.tensor_linear_fwd(1, Y1, S1.reshape(rows, 3, 5 * chan), x_layout=C, row_bound=nmax,
-                                              rows_per_bound=3)]
+                                              rows_per_bound=3, **into_v)]
         if not fused_d:
             jobs.append(lambda: ops.tensor_linear_fwd(2, Y2, S2.reshape(rows, 9, 5 * chan), x_layout=C, row_bound=nmax,
-                                                      rows_per_bound=9))
+                                                      rows_per_bound=9, **into_d))
         outs = ops.concurrent(jobs, rows)
         B_a, B_v, B_d = outs[0], outs[1], (S2 if fused_d else outs[2])
-        return (B_a.reshape(B, N, -1), B_v.reshape(B, N, -1, 3), B_d.reshape(B, N, -1, 3, 3))
+        shapes = ((B, N, -1), (B, N, -1, 3), (B, N, -1, 3, 3))
+        if add_to_inputs and not in_place:
+            B_a, B_v, B_d = (x + d.reshape(x.shape) for x, d in zip((x_a, x_v, x_d), (B_a, B_v, B_d)))
+        return tuple(t.reshape(sh) for t, sh in zip((B_a, B_v, B_d), shapes))

@@ -140,7 +140,7 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
                    const float* __restrict__ enc_W, const float* __restrict__ enc_b, T* __restrict__ P0,
                    T* __restrict__ S1, T* __restrict__ S2, float* __restrict__ node_max,
                    float* __restrict__ edge_max, const float* __restrict__ y2_packed, int dim_d,
-                   float* __restrict__ out_d) {
+                   float* __restrict__ out_d, int out_d_accumulate) {
     static_assert(!Y2F || std::is_same<T, float>::value, "the fused output linear is for float storage");
     const int lane = threadIdx.x & (kWave - 1);
     const int chunks = (chan + kWave - 1) / kWave;
@@ -318,7 +318,7 @@ bee_message_kernel(const int* __restrict__ row_ptr, const int* __restrict__ dst,
             __shared__ __attribute__((aligned(16))) float tr_buf[4][16 * kTrPitch];
             __shared__ float part[4][16 * 16];
             rank2_linear_of_node_sums(s2, tr_buf, part, chunk, chunks, valid, y2_packed, dim_d,
-                                      out_d + node * (long)dim_d * 9);
+                                      out_d + node * (long)dim_d * 9, out_d_accumulate != 0);
         }
     }
 }
@@ -347,7 +347,7 @@ static int launch_bee_message(const char* what, const int* row_ptr, const int* d
                               long n_edges, const float* rhat, const float* enc, const T* La, const T* Lv, const T* Ld,
                               int chan, const float* enc_W, const float* enc_b, T* P0, T* S1, T* S2,
                               float* node_max, float* edge_max, mg_stream_t stream, const float* y2_packed = nullptr,
-                              int dim_d = 0, float* out_d = nullptr) {
+                              int dim_d = 0, float* out_d = nullptr, int out_d_accumulate = 0) {
     MG_REQUIRE(n_nodes >= 0 && n_edges >= 0 && chan >= 0, "%s: negative size", what);
     if (n_nodes == 0 || chan == 0) return MG_OK;
     const bool fused = y2_packed != nullptr;
@@ -366,7 +366,7 @@ static int launch_bee_message(const char* what, const int* row_ptr, const int* d
 #define MG_BEE_LAUNCH(PIPE, Y2F)                                                                                      \
     hipLaunchKernelGGL((bee_message_kernel<T, PIPE, Y2F>), dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, \
                        row_ptr, dst, node_order, (long)n_nodes, rhat, enc, La, Lv, Ld, chan, enc_W, enc_b, P0, S1, S2, \
-                       node_max, edge_max, y2_packed, dim_d, out_d)
+                       node_max, edge_max, y2_packed, dim_d, out_d, out_d_accumulate)
     if constexpr (std::is_same<T, float>::value) {
         if (fused) {
             MG_REQUIRE(rank2_fusable(chan, dim_d), "%s: the fused rank-2 linear needs chan = 64, 128 or 256 and dim_d <= 16", what);
@@ -424,11 +424,11 @@ int mg_bee_pack_rank2_weight(const float* Y2, long ld, int chan, int dim_d, floa
 int mg_bee_message_rank2(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,
                          const float* rhat, const float* enc, const float* La, const float* Lv, const float* Ld, int chan,
                          const float* enc_W, const float* enc_b, const float* packed_Y2, int dim_d, float* P0, float* S1,
-                         float* out_d, float* node_max, float* edge_max, mg_stream_t stream) {
+                         float* out_d, int accumulate, float* node_max, float* edge_max, mg_stream_t stream) {
     MG_REQUIRE(packed_Y2 != nullptr, "mg_bee_message_rank2: null weight");
     return launch_bee_message<float>("mg_bee_message_rank2", row_ptr, dst, node_order, n_nodes, n_edges, rhat, enc, La,
                                      Lv, Ld, chan, enc_W, enc_b, P0, S1, nullptr, node_max, edge_max, stream, packed_Y2,
-                                     dim_d, out_d);
+                                     dim_d, out_d, accumulate);
 }
 
 int mg_bee_message_bf16(const int* row_ptr, const int* dst, const int* node_order, int n_nodes, long n_edges,

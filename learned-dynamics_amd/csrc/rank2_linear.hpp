@@ -18,11 +18,11 @@ constexpr int kTrPitch = 68;   // floats per LDS row of a wave's transposition b
 typedef float floatx4 __attribute__((ext_vector_type(4)));
 
 // Called by all four waves of the workgroup (it holds two barriers); valid = false: a wave without an item, whose s2
-// must be zeros.  out: this wave's node, (dim_d, 9).
+// must be zeros.  out: this wave's node, (dim_d, 9); accumulate: the result is added to what out holds.
 __device__ __forceinline__ void rank2_linear_of_node_sums(const float (&s2)[45], float (&tr_buf)[4][16 * kTrPitch],
                                                           float (&part)[4][16 * 16], int chunk, int chunks, bool valid,
                                                           const float* __restrict__ y2_packed, int dim_d,
-                                                          float* __restrict__ out) {
+                                                          float* __restrict__ out, bool accumulate = false) {
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     float* tr = tr_buf[wave];
     const int ci = lane & 15, kk = lane >> 4;
@@ -74,7 +74,7 @@ __device__ __forceinline__ void rank2_linear_of_node_sums(const float (&s2)[45],
             const int j = idx / 9, i = idx - 9 * j;
             float sum = 0.f;
             for (int wv = 0; wv < chunks; wv++) sum += part[wave + wv][i * 16 + j];
-            out[idx] = sum;
+            out[idx] = accumulate ? out[idx] + sum : sum;
         }
     }
     __syncthreads();                                            // before the workgroup's next use of part

@@ -73,8 +73,8 @@ class Denoiser(nn.Module):
         x_v = self.v_readin((x1 - x0)[..., None, :].contiguous())
         x_d = torch.zeros(B, N, dim_d, 3, 3, device=x1.device)
         for msg, prod in zip(self.messages, self.prods):
-            d_a, d_v, d_d = msg(graph, r_ij, x_a, x_v, x_d, node_order=node_order)
-            x_a, x_v, x_d = x_a + d_a, x_v + d_v, x_d + d_d
+            # x_a, x_v, x_d are this function's own tensors: the messages are added in their memory
+            x_a, x_v, x_d = msg(graph, r_ij, x_a, x_v, x_d, node_order=node_order, add_to_inputs=True)
             x_a, x_v, x_d = prod(x_a, x_v, x_d, residual=True)
         v_pred = self.readout(x_v).squeeze(-2)
         return (1. - (t - s)[:, None, None]) * v_pred

@@ -2073,13 +2073,15 @@ def bee_node_products_rank2(l0, l1, l2, r0, r1, r2, Y2):
     return out
 
 
-def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=None, want_node_max=False, Y2=None):
+def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=None, want_node_max=False, Y2=None,
+                out_d=None):
     """Fused products + edge sums of the rank-0/1/2 message (see mg_bee_message).
     La (N,chan), Lv (N,3,chan), Ld (N,9,chan) -> P0 (E,3,chan), S1 (N,3,5,chan), S2 (N,9,5,chan)
     (+ node_max (N, ceil(chan/64)) and edge_max (E, ceil(chan/64)): partial maxima of |S1|, |S2| per node
     and of |P0| per edge, with want_node_max).
     Y2 (dim_d, 5 chan), bee_rank2_supported(chan, dim_d): the rank-2 output linear is applied inside the kernel and
-    the third result is Y2 S2 as (N, dim_d, 9) instead of S2 (mg_bee_message_rank2)."""
+    the third result is Y2 S2 as (N, dim_d, 9) instead of S2 (mg_bee_message_rank2); with out_d (N dim_d 9 floats,
+    contiguous) Y2 S2 is added to out_d in place, which is then the third result."""
     _check_input(row_ptr, "row_ptr", torch.int32)
     _check_input(dst, "dst", torch.int32)
     for t, nm in ((rhat, "rhat"), (enc, "enc"), (La, "La"), (Lv, "Lv"), (Ld, "Ld"), (enc_W, "enc_W"),
@@ -2114,11 +2116,15 @@ def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=No
         edge_max = torch.empty(E, (chan + 63) // 64, dtype=torch.float32, device=dev) if want_node_max else None
         if Y2 is not None:
             dim_d = int(Y2.size(0))
-            S2 = torch.empty(N, dim_d, 9, dtype=torch.float32, device=dev)
+            if out_d is not None:
+                _check_input(out_d, "out_d")
+                if out_d.numel() != N * dim_d * 9:
+                    raise RuntimeError("out_d must hold nodes x dim_d x 9 floats")
+            S2 = out_d if out_d is not None else torch.empty(N, dim_d, 9, dtype=torch.float32, device=dev)
             L.check(_lib.mg_bee_message_rank2(_p(row_ptr), _p(dst), _p(node_order), N, E, _p(rhat), _p(enc), _p(La),
                                               _p(Lv), _p(Ld), chan, _p(enc_W), _p(enc_b),
                                               _p(_packed_rank2_weight(Y2, chan)), dim_d, _p(P0), _p(S1), _p(S2),
-                                              _p(node_max), _p(edge_max), _stream()))
+                                              int(out_d is not None), _p(node_max), _p(edge_max), _stream()))
         else:
             S2 = torch.empty(N, 9, 5, chan, dtype=torch.float32, device=dev)
             L.check(_lib.mg_bee_message(_p(row_ptr), _p(dst), _p(node_order), N, E, _p(rhat), _p(enc), _p(La), _p(Lv),

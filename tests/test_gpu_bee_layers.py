@@ -180,6 +180,21 @@ def test_messages_module(pkg, dims):
     r32 = OL.bee_messages(src, dst, 2, 500, r_ref, x_a, x_v, x_d, _to(w, torch.float32), r0, radial_dtype=torch.float64)
     for k, (got, name) in enumerate(zip((B_a, B_v, B_d), "avd")):
         assert_parity(got, r32[k], r64[k], f"Messages {dims} B_{name}")
+    # the residual step formed in the inputs' memory: x + messages against the same oracle, the inputs overwritten,
+    # and a non-contiguous input taking the out-of-place route
+    own = [x_a.cuda(), x_v.cuda(), x_d.cuda()]
+    with torch.no_grad():
+        y = msg(graph, r_ij, *own, add_to_inputs=True)
+    for k, (got, x, name) in enumerate(zip(y, (x_a, x_v, x_d), "avd")):
+        assert got.data_ptr() == own[k].data_ptr() and got.shape == x.shape
+        assert_parity(got, x + r32[k], x.double() + r64[k], f"Messages {dims} x_{name} + B_{name} in place")
+    wide = torch.randn(2, 500, dim_a + 3).cuda()
+    wide[..., :dim_a] = x_a.cuda()
+    with torch.no_grad():
+        y2 = msg(graph, r_ij, wide[..., :dim_a], x_v.cuda(), x_d.cuda(), add_to_inputs=True)
+    assert torch.equal(wide[..., :dim_a], x_a.cuda())
+    for k, (got, x, name) in enumerate(zip(y2, (x_a, x_v, x_d), "avd")):
+        assert_parity(got, x + r32[k], x.double() + r64[k], f"Messages {dims} x_{name} + B_{name} out of place")
 
 
 def test_self_tens_prods_module(pkg):
