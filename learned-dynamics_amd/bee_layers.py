@@ -138,8 +138,11 @@ class SelfTensProds(nn.Module):
         # 5 chan, 5 chan instead of thirteen accumulating ones
         C = ops.LAYOUT_COMP_CHAN
         chan = self.L0.W.shape[0]
+        # L_k and R_k act on the same x_k: its rows per component are formed once for both
+        as_rows = [None, ops.components_as_rows(1, x_v), ops.components_as_rows(2, x_d)]
         def input_linear(k, lin, x):
-            return lambda: ops.tensor_linear_fwd(k, lin.W, x, y_layout=C if k else ops.LAYOUT_CHAN_COMP, want_rowmax=True)
+            return lambda: ops.tensor_linear_fwd(k, lin.W, x, y_layout=C if k else ops.LAYOUT_CHAN_COMP, want_rowmax=True,
+                                                 x_rows=as_rows[k])
         pairs = ops.concurrent([input_linear(k, lin, x)
                                 for side in ((self.L0, self.L1, self.L2), (self.R0, self.R1, self.R2))
                                 for k, (lin, x) in enumerate(zip(side, (x_a, x_v, x_d)))], rows)

@@ -1119,16 +1119,38 @@ def tensor_linear_f16x2(W, x, x_rowmax=None, bias=None, act=ACT_NONE, out=None, 
 LAYOUT_CHAN_COMP, LAYOUT_COMP_CHAN = 0, 1
 
 
+def components_as_rows(inds, x):
+    """x (..., dim_in, (3,)^inds) in the reference's layout -> (x2, x2max): one plain GEMM row per (row, component)
+    with the channels zero-padded to a power of two, and the row maxima of |x2| -- what tensor_linear_fwd forms for
+    itself when it sends such an input through the split-fp16 path, for callers that apply several weights to the same
+    x (x_rows= of tensor_linear_fwd).  None when that path would not be taken for this input."""
+    _check_input(x, "x")
+    if inds < 1 or inds > 2 or x.dim() < 1 + inds:
+        return None
+    T = 3 ** inds
+    dim_in = int(x.size(x.dim() - 1 - inds))
+    rows = x.numel() // (dim_in * T) if dim_in else 0
+    k_pad = (dim_in + 31) // 32 * 32
+    if get_linear_mode() != LINEAR_F16X2 or rows * T < 32768 or k_pad > 256 or k_pad & (k_pad - 1):
+        return None
+    with torch.cuda.device(x.device):
+        x2 = torch.empty(rows * T, k_pad, dtype=torch.float32, device=x.device)
+        x2max = torch.empty(rows * T, 1, dtype=torch.float32, device=x.device)
+        L.check(_lib.mg_components_to_rows(_p(x), rows, dim_in, T, k_pad, _p(x2), _p(x2max), _stream()))
+    return x2, x2max
+
+
 def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=False,
                       x_layout=LAYOUT_CHAN_COMP, y_layout=LAYOUT_CHAN_COMP, row_bound=None, rows_per_bound=1,
-                      want_rowmax=False):
+                      want_rowmax=False, x_rows=None):
     """y[..., o, t] = act(sum_i W[o, i] x[..., i, t] + bias[o]); W may have any strides.
     Layout 0 stores a tensor as (..., chan, (3,)^inds) like the reference; layout 1 is
     component-major (..., 3^inds, chan), the layout the fused edge kernels read and write.
     row_bound ((rows of the GEMM) / rows_per_bound, parts): upper bounds of the row maxima of |x| from
     the kernel that produced x, used by the split-fp16 matrix path instead of a pass over x.
     want_rowmax: return (y, rowmax) with rowmax ((GEMM rows), parts) partial row maxima of |y| when the kernel
-    that ran can emit them (plain-row output through the split-fp16 path), else (y, None)."""
+    that ran can emit them (plain-row output through the split-fp16 path), else (y, None).
+    x_rows: components_as_rows(inds, x) of this same x, if the caller has it (None is allowed)."""
     if not W.is_cuda:
         raise RuntimeError("W must be a CUDA tensor")
     _check_input(x, "x")
@@ -1191,7 +1213,9 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
             # kernel's layout mapping is not; with the reference's output layout its component epilogue still
             # beats the generic kernel (61 against 104 us for 16384 x 128 x 3 -> 384)
             k_pad = (dim_in + 31) // 32 * 32
-            if k_pad <= 256 and k_pad & (k_pad - 1) == 0:
+            if x_rows is not None and tuple(x_rows[0].shape) == (rows * T, k_pad):
+                x2, x2max = x_rows
+            elif k_pad <= 256 and k_pad & (k_pad - 1) == 0:
                 # transposition, padding and the row maxima in one pass
                 x2 = torch.empty(rows * T, k_pad, dtype=torch.float32, device=x.device)
                 x2max = torch.empty(rows * T, 1, dtype=torch.float32, device=x.device)
