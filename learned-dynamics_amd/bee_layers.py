@@ -140,14 +140,27 @@ class SelfTensProds(nn.Module):
         chan = self.L0.W.shape[0]
         # L_k and R_k act on the same x_k: its rows per component are formed once for both
         as_rows = [None, ops.components_as_rows(1, x_v), ops.components_as_rows(2, x_d)]
+        fused_products = ops.bee_products_linear_supported(rows, chan)
+        # few rank-2 output channels: see below; the row maxima of the six operands are then not needed
+        node_pass = ops.bee_rank2_supported(chan, dim_d)
         def input_linear(k, lin, x):
-            return lambda: ops.tensor_linear_fwd(k, lin.W, x, y_layout=C if k else ops.LAYOUT_CHAN_COMP, want_rowmax=True,
-                                                 x_rows=as_rows[k])
+            return lambda: ops.tensor_linear_fwd(k, lin.W, x, y_layout=C if k else ops.LAYOUT_CHAN_COMP,
+                                                 want_rowmax=not node_pass, x_rows=as_rows[k])
         pairs = ops.concurrent([input_linear(k, lin, x)
                                 for side in ((self.L0, self.L1, self.L2), (self.R0, self.R1, self.R2))
                                 for k, (lin, x) in enumerate(zip(side, (x_a, x_v, x_d)))], rows)
-        ops_in = [p[0] for p in pairs]
-        if ops.bee_products_linear_supported(rows, chan):
+        ops_in = [p[0] for p in pairs] if not node_pass else list(pairs)
+        if node_pass:
+            # one pass over the nodes applies the rank-2 output linear to the products of a node on the fp32 matrix
+            # cores and stores the scalar and vector products (18 chan floats per node) for two plain GEMMs, whose row
+            # bounds it emits
+            Ys = [_cat_Y(self, labels) for labels in (LABELS_0, LABELS_1, LABELS_2)]
+            y_d, P0, P1, nmax = ops.bee_node_products_rank2(*ops_in, Ys[2], want_lower_ranks=True)
+            y_a, y_v = ops.concurrent([
+                lambda: ops.tensor_linear_fwd(0, Ys[0], P0.reshape(rows, 3 * chan), row_bound=nmax),
+                lambda: ops.tensor_linear_fwd(1, Ys[1], P1.reshape(rows, 3, 5 * chan), x_layout=C, row_bound=nmax,
+                                              rows_per_bound=3)], rows)
+        elif fused_products:
             # products and output linears in one kernel per output rank: the 13 products are never stored.
             # Its row scales need a bound of the products per node: 9 max|l| max|r| (at most 9 terms per
             # component), from the row maxima the six GEMMs above emit
@@ -157,13 +170,8 @@ class SelfTensProds(nn.Module):
                 return torch.cat(cols, dim=1).amax(dim=1)
             bound = 9.0 * node_max(pairs[:3]) * node_max(pairs[3:])
             Ys = [_cat_Y(self, labels) for labels in (LABELS_0, LABELS_1, LABELS_2)]
-            jobs = [(lambda k=k: ops.bee_products_linear(k, Ys[k], *ops_in, bound)) for k in range(2)]
-            if ops.bee_rank2_supported(chan, Ys[2].shape[0]):
-                # few rank-2 output channels: fp32 matrix cores on the products of one node at a time
-                jobs.append(lambda: ops.bee_node_products_rank2(*ops_in, Ys[2]))
-            else:
-                jobs.append(lambda: ops.bee_products_linear(2, Ys[2], *ops_in, bound))
-            y_a, y_v, y_d = ops.concurrent(jobs, rows)
+            y_a, y_v, y_d = ops.concurrent([(lambda k=k: ops.bee_products_linear(k, Ys[k], *ops_in, bound))
+                                            for k in range(3)], rows)
         else:
             P0, P1, P2, nmax = ops.bee_node_products(*ops_in, want_node_max=True)
             # nmax: per-node maxima of the products, the row bounds of the three GEMMs

@@ -100,7 +100,8 @@ __global__ void __launch_bounds__(256) node_rank2_linear_kernel(long n_nodes, in
                                                                 const float* __restrict__ r0, const float* __restrict__ r1,
                                                                 const float* __restrict__ r2,
                                                                 const float* __restrict__ y2_packed, int dim_d,
-                                                                float* __restrict__ out) {
+                                                                float* __restrict__ out, float* __restrict__ P0,
+                                                                float* __restrict__ P1, float* __restrict__ node_max) {
     __shared__ __attribute__((aligned(16))) float tr_buf[4][16 * kTrPitch];
     __shared__ float part[4][16 * 16];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
@@ -125,6 +126,37 @@ __global__ void __launch_bounds__(256) node_rank2_linear_kernel(long n_nodes, in
         for (int k = 0; k < 9; k++) {
             L[k] = l2[(node * 9 + k) * chan + c];
             R[k] = r2[(node * 9 + k) * chan + c];
+        }
+        if (P0) {
+            // the scalar and vector products as well, stored in the layout of mg_bee_node_products with their
+            // maximum per (node, chunk): the operands are in registers once, and the two GEMMs that follow read
+            // 18 chan floats per node instead of gathering 26 chan through their operand loads
+            float dot = 0.f, ddot = 0.f;
+#pragma unroll
+            for (int x = 0; x < 3; x++) dot += u[x] * v[x];
+#pragma unroll
+            for (int k = 0; k < 9; k++) ddot += L[k] * R[k];
+            float* p0 = P0 + (node * 3) * chan + c;
+            __builtin_nontemporal_store(a * b, p0);
+            __builtin_nontemporal_store(dot, p0 + chan);
+            __builtin_nontemporal_store(ddot, p0 + 2 * chan);
+            float mx = fmaxf(fabsf(a * b), fmaxf(fabsf(dot), fabsf(ddot)));
+            const float cr[3] = {u[1] * v[2] - u[2] * v[1], u[2] * v[0] - u[0] * v[2], u[0] * v[1] - u[1] * v[0]};
+#pragma unroll
+            for (int x = 0; x < 3; x++) {
+                float* p1 = P1 + ((node * 3 + x) * 5) * chan + c;
+                const float q[5] = {a * v[x], u[x] * b, u[0] * R[3 * x] + u[1] * R[3 * x + 1] + u[2] * R[3 * x + 2],
+                                    L[3 * x] * v[0] + L[3 * x + 1] * v[1] + L[3 * x + 2] * v[2], cr[x]};   // 011 101 121 211 111
+#pragma unroll
+                for (int t = 0; t < 5; t++) {
+                    __builtin_nontemporal_store(q[t], p1 + t * chan);
+                    mx = fmaxf(mx, fabsf(q[t]));
+                }
+            }
+            if (node_max) {
+                for (int d = 1; d < kWave; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+                if (lane == 0) node_max[node * chunks + chunk] = mx;
+            }
         }
 #pragma unroll
         for (int x = 0; x < 3; x++) {
@@ -179,7 +211,9 @@ int mg_bee_node_products(long n_nodes, int chan, const float* l0, const float* l
 
 int mg_bee_node_products_rank2(long n_nodes, int chan, const float* l0, const float* l1, const float* l2,
                                const float* r0, const float* r1, const float* r2, const float* packed_Y2, int dim_d,
-                               float* out_d, mg_stream_t stream) {
+                               float* out_d, float* P0, float* P1, float* node_max, mg_stream_t stream) {
+    MG_REQUIRE((P0 == nullptr) == (P1 == nullptr) && (node_max == nullptr || P0 != nullptr),
+               "mg_bee_node_products_rank2: P0 and P1 go together, node_max with them");
     MG_REQUIRE(n_nodes >= 0, "mg_bee_node_products_rank2: negative size");
     MG_REQUIRE(rank2_fusable(chan, dim_d), "mg_bee_node_products_rank2: needs chan = 64, 128 or 256 and dim_d <= 16");
     if (n_nodes == 0) return MG_OK;
@@ -188,7 +222,7 @@ int mg_bee_node_products_rank2(long n_nodes, int chan, const float* l0, const fl
     const long blocks = ceil_div(n_nodes * (chan / kWave), 4);
     MG_REQUIRE(blocks < (1L << 31), "mg_bee_node_products_rank2: too many nodes for one launch");
     hipLaunchKernelGGL(node_rank2_linear_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, n_nodes,
-                       chan, l0, l1, l2, r0, r1, r2, packed_Y2, dim_d, out_d);
+                       chan, l0, l1, l2, r0, r1, r2, packed_Y2, dim_d, out_d, P0, P1, node_max);
     return check_launch("mg_bee_node_products_rank2");
 }
 

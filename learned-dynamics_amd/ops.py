@@ -2075,10 +2075,12 @@ def _packed_rank2_weight(Y2, chan):
     return packed
 
 
-def bee_node_products_rank2(l0, l1, l2, r0, r1, r2, Y2):
+def bee_node_products_rank2(l0, l1, l2, r0, r1, r2, Y2, want_lower_ranks=False):
     """The rank-2 output of SelfTensProds from its six operands in one kernel: Y2 (dim_d, 5 chan) applied to the five
-    rank-2 products of l0/r0 (N, chan), l1/r1 (N, 3, chan), l2/r2 (N, 9, chan) -> (N, dim_d, 9); the products are
-    never stored.  For bee_rank2_supported(chan, dim_d)."""
+    rank-2 products of l0/r0 (N, chan), l1/r1 (N, 3, chan), l2/r2 (N, 9, chan) -> (N, dim_d, 9); the rank-2 products
+    are never stored.  For bee_rank2_supported(chan, dim_d).
+    want_lower_ranks: returns (out_d, P0 (N,3,chan), P1 (N,3,5,chan), node_max (N, chan/64)) with the scalar and
+    vector products of bee_node_products and their partial maxima per node, written in the same pass."""
     for t, nm in ((l0, "l0"), (l1, "l1"), (l2, "l2"), (r0, "r0"), (r1, "r1"), (r2, "r2")):
         _check_input(t, nm)
     N, chan = int(l0.size(0)), int(l0.size(1))
@@ -2092,9 +2094,15 @@ def bee_node_products_rank2(l0, l1, l2, r0, r1, r2, Y2):
     dim_d = int(Y2.size(0))
     with torch.cuda.device(l0.device):
         out = torch.empty(N, dim_d, 9, dtype=torch.float32, device=l0.device)
+        P0 = P1 = nmax = None
+        if want_lower_ranks:
+            P0 = torch.empty(N, 3, chan, dtype=torch.float32, device=l0.device)
+            P1 = torch.empty(N, 3, 5, chan, dtype=torch.float32, device=l0.device)
+            nmax = torch.empty(N, chan // 64, dtype=torch.float32, device=l0.device)
         L.check(_lib.mg_bee_node_products_rank2(N, chan, _p(l0), _p(l1), _p(l2), _p(r0), _p(r1), _p(r2),
-                                                _p(_packed_rank2_weight(Y2, chan)), dim_d, _p(out), _stream()))
-    return out
+                                                _p(_packed_rank2_weight(Y2, chan)), dim_d, _p(out), _p(P0), _p(P1),
+                                                _p(nmax), _stream()))
+    return (out, P0, P1, nmax) if want_lower_ranks else out
 
 
 def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=None, want_node_max=False, Y2=None,

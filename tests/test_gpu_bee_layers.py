@@ -389,13 +389,28 @@ def test_rank2_products_and_their_output_linear_in_one_kernel(pkg, chan, dim_d, 
     small = (size[:, 0] < 0.1)
     if bool(small.any()):
         assert_parity_of(y[small.cuda()], lambda dt: ref(dt)[small], "rank-2 products + linear, small nodes")
-    # the stored-products route gives the same within the same bar
+    # the scalar and vector products written in the same pass, against the oracle's, and the emitted maxima are
+    # exactly the maxima of what was written
+    y3, Q0, Q1, nmax = ops.bee_node_products_rank2(*dev, W, want_lower_ranks=True)
+    assert torch.equal(y3, y)
+
+    def products(dt):
+        return dict(zip(OP.BEE_ORDER, OP.bee(*[to_ref(t.to(dt), k) for k, t in enumerate(l)],
+                                             *[to_ref(t.to(dt), k) for k, t in enumerate(r)])))
+    for k, lab in enumerate(("000", "110", "220")):
+        assert_parity_of(Q0[:, k], lambda dt: products(dt)[lab], f"scalar product {lab} from the node pass")
+    for k, lab in enumerate(("011", "101", "121", "211", "111")):
+        assert_parity_of(Q1[:, :, k], lambda dt: products(dt)[lab].transpose(1, 2), f"vector product {lab} from the node pass")
+    assert nmax.shape == (N, chan // 64)
+    assert torch.equal(nmax.amax(1), torch.maximum(Q0.abs().amax(dim=(1, 2)), Q1.abs().amax(dim=(1, 2, 3))))
     P2 = ops.bee_node_products(*dev)[2]
+    # the stored-products route gives the same within the same bar
     stored = ops.tensor_linear_fwd(2, W, P2.reshape(N, 9, 5 * chan), x_layout=ops.LAYOUT_COMP_CHAN)
     assert_parity_of(stored.reshape(N, dim_d, 9), ref, "stored products + GEMM")
     with pytest.raises(RuntimeError, match="dim_d <= 16"):
         ops.bee_node_products_rank2(*dev, torch.zeros(32, 5 * chan, device="cuda"))
     assert ops.bee_node_products_rank2(*[t[:0] for t in dev], W).shape == (0, dim_d, 9)
+    assert ops.bee_node_products_rank2(*[t[:0] for t in dev], W, want_lower_ranks=True)[2].shape == (0, 3, 5, chan)
 
 
 def test_self_tens_prods_module_fused_path(pkg):
