@@ -662,10 +662,13 @@ int mg_bee_message_rank2(const int* row_ptr, const int* dst, const int* node_ord
  * output linears Y_022 .. Y_212, packed as for mg_bee_message_rank2; out_d (N, dim_d, 9).  Same domain.
  * P0 (N,3,chan), P1 (N,3,5,chan) (both or neither; may be NULL): the scalar and vector products as
  * mg_bee_node_products stores them, written in the same pass; node_max (N, chan/64; may be NULL): their partial
- * maxima per node. */
+ * maxima per node.
+ * x_d (N, dim_in2, 9) with L2t, R2t (dim_in2, chan) = the transposed weights of L2 and R2, dim_in2 <= 16 (or all
+ * NULL / 0): l2 = L2 x_d and r2 = R2 x_d are formed inside the kernel and the arguments l2, r2 are not read. */
 int mg_bee_node_products_rank2(long n_nodes, int chan, const float* l0, const float* l1, const float* l2,
                                const float* r0, const float* r1, const float* r2, const float* packed_Y2, int dim_d,
-                               float* out_d, float* P0, float* P1, float* node_max, mg_stream_t stream);
+                               float* out_d, float* P0, float* P1, float* node_max, const float* x_d,
+                               const float* L2t, const float* R2t, int dim_in2, mg_stream_t stream);
 /* node_max (above and below; may be NULL): (N, ceil(chan/64)) partial maxima of |S1|, |S2| (of |P0|,
  * |P1|, |P2| below) per node, which mg_tensor_linear_f16x2 accepts as row bounds of those tensors
  * (x_rows_per_bound = 3 or 9); edge_max (may be NULL): (E, ceil(chan/64)) partial maxima of the rows

@@ -64,7 +64,7 @@ _SIGNATURES = {
     "mg_tensor_linear_layout": [i32, vp, i64, i64, vp, i64, i32, i32, vp, i32, i32, i32, i32, vp, vp],
     "mg_bee_edge_geometry": [vp, i64, f32, vp, vp, vp],
     "mg_bee_message": [vp, vp, vp, i32, i64, vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, vp, vp, vp, vp],
-    "mg_bee_node_products_rank2": [i64, i32, vp, vp, vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, vp],
+    "mg_bee_node_products_rank2": [i64, i32, vp, vp, vp, vp, vp, vp, vp, i32, vp, vp, vp, vp, vp, vp, vp, i32, vp],
     "mg_bee_message_rank2_supported": [i32, i32],
     "mg_bee_rank2_weight_bytes": [i32, vp],
     "mg_bee_pack_rank2_weight": [vp, i64, i32, i32, vp, vp],

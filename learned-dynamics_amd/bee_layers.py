@@ -139,11 +139,16 @@ class SelfTensProds(nn.Module):
         C = ops.LAYOUT_COMP_CHAN
         chan = self.L0.W.shape[0]
         # L_k and R_k act on the same x_k: its rows per component are formed once for both
-        as_rows = [None, ops.components_as_rows(1, x_v), ops.components_as_rows(2, x_d)]
         fused_products = ops.bee_products_linear_supported(rows, chan)
         # few rank-2 output channels: see below; the row maxima of the six operands are then not needed
         node_pass = ops.bee_rank2_supported(chan, dim_d)
+        as_rows = [None, ops.components_as_rows(1, x_v),
+                   None if (node_pass and dim_d <= 16) else ops.components_as_rows(2, x_d)]
+        # ... and with at most 16 rank-2 input channels it also forms L2 x_d and R2 x_d itself
+        inside2 = node_pass and dim_d <= 16
         def input_linear(k, lin, x):
+            if k == 2 and inside2:
+                return lambda: None
             return lambda: ops.tensor_linear_fwd(k, lin.W, x, y_layout=C if k else ops.LAYOUT_CHAN_COMP,
                                                  want_rowmax=not node_pass, x_rows=as_rows[k])
         pairs = ops.concurrent([input_linear(k, lin, x)
@@ -155,7 +160,11 @@ class SelfTensProds(nn.Module):
             # cores and stores the scalar and vector products (18 chan floats per node) for two plain GEMMs, whose row
             # bounds it emits
             Ys = [_cat_Y(self, labels) for labels in (LABELS_0, LABELS_1, LABELS_2)]
-            y_d, P0, P1, nmax = ops.bee_node_products_rank2(*ops_in, Ys[2], want_lower_ranks=True)
+            extra = {}
+            if inside2:
+                extra = dict(x_d=x_d, L2t=_derived(self, "L2_transposed", (self.L2.W,), lambda: self.L2.W.t().contiguous()),
+                             R2t=_derived(self, "R2_transposed", (self.R2.W,), lambda: self.R2.W.t().contiguous()))
+            y_d, P0, P1, nmax = ops.bee_node_products_rank2(*ops_in, Ys[2], want_lower_ranks=True, **extra)
             y_a, y_v = ops.concurrent([
                 lambda: ops.tensor_linear_fwd(0, Ys[0], P0.reshape(rows, 3 * chan), row_bound=nmax),
                 lambda: ops.tensor_linear_fwd(1, Ys[1], P1.reshape(rows, 3, 5 * chan), x_layout=C, row_bound=nmax,

@@ -101,9 +101,13 @@ __global__ void __launch_bounds__(256) node_rank2_linear_kernel(long n_nodes, in
                                                                 const float* __restrict__ r2,
                                                                 const float* __restrict__ y2_packed, int dim_d,
                                                                 float* __restrict__ out, float* __restrict__ P0,
-                                                                float* __restrict__ P1, float* __restrict__ node_max) {
+                                                                float* __restrict__ P1, float* __restrict__ node_max,
+                                                                const float* __restrict__ x_d,
+                                                                const float* __restrict__ L2t,
+                                                                const float* __restrict__ R2t, int dim_in2) {
     __shared__ __attribute__((aligned(16))) float tr_buf[4][16 * kTrPitch];
     __shared__ float part[4][16 * 16];
+    __shared__ float xd_buf[4][16 * 9];
     const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
     const int chunks = chan / kWave;
     const long items = n_nodes * chunks;
@@ -122,10 +126,34 @@ __global__ void __launch_bounds__(256) node_rank2_linear_kernel(long n_nodes, in
             u[x] = l1[(node * 3 + x) * chan + c];
             v[x] = r1[(node * 3 + x) * chan + c];
         }
+        if (x_d) {
+            // the rank-2 operands are formed here: l2[k] = sum_i L2[c, i] x_d[node, i, k] (dim_in2 <= 16 input
+            // channels; the node's 9 dim_in2 values go through LDS and are read back as broadcasts, the weights come
+            // transposed, (dim_in2, chan), one coalesced row per input channel).  Two GEMMs that would each write
+            // (node, 9, chan) and this kernel's read of both are not needed.
+            float* xd = xd_buf[wave];
+            const float* src = x_d + node * (long)(dim_in2 * 9);
+            for (int t = lane; t < dim_in2 * 9; t += kWave) xd[t] = src[t];
+            __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+            __builtin_amdgcn_wave_barrier();
+            __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 #pragma unroll
-        for (int k = 0; k < 9; k++) {
-            L[k] = l2[(node * 9 + k) * chan + c];
-            R[k] = r2[(node * 9 + k) * chan + c];
+            for (int k = 0; k < 9; k++) { L[k] = 0.f; R[k] = 0.f; }
+            for (int i = 0; i < dim_in2; i++) {
+                const float wl = L2t[(long)i * chan + c], wr = R2t[(long)i * chan + c];
+#pragma unroll
+                for (int k = 0; k < 9; k++) {
+                    const float xv = xd[i * 9 + k];
+                    L[k] = fmaf(wl, xv, L[k]);
+                    R[k] = fmaf(wr, xv, R[k]);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int k = 0; k < 9; k++) {
+                L[k] = l2[(node * 9 + k) * chan + c];
+                R[k] = r2[(node * 9 + k) * chan + c];
+            }
         }
         if (P0) {
             // the scalar and vector products as well, stored in the layout of mg_bee_node_products with their
@@ -211,18 +239,23 @@ int mg_bee_node_products(long n_nodes, int chan, const float* l0, const float* l
 
 int mg_bee_node_products_rank2(long n_nodes, int chan, const float* l0, const float* l1, const float* l2,
                                const float* r0, const float* r1, const float* r2, const float* packed_Y2, int dim_d,
-                               float* out_d, float* P0, float* P1, float* node_max, mg_stream_t stream) {
+                               float* out_d, float* P0, float* P1, float* node_max, const float* x_d,
+                               const float* L2t, const float* R2t, int dim_in2, mg_stream_t stream) {
     MG_REQUIRE((P0 == nullptr) == (P1 == nullptr) && (node_max == nullptr || P0 != nullptr),
                "mg_bee_node_products_rank2: P0 and P1 go together, node_max with them");
+    MG_REQUIRE(x_d == nullptr || (L2t && R2t && dim_in2 >= 1 && dim_in2 <= 16),
+               "mg_bee_node_products_rank2: x_d needs both transposed weights and 1 .. 16 input channels");
+
     MG_REQUIRE(n_nodes >= 0, "mg_bee_node_products_rank2: negative size");
     MG_REQUIRE(rank2_fusable(chan, dim_d), "mg_bee_node_products_rank2: needs chan = 64, 128 or 256 and dim_d <= 16");
     if (n_nodes == 0) return MG_OK;
-    MG_REQUIRE(l0 && l1 && l2 && r0 && r1 && r2 && packed_Y2 && out_d && aligned16(packed_Y2),
+    MG_REQUIRE(l0 && l1 && r0 && r1 && packed_Y2 && out_d && aligned16(packed_Y2),
                "mg_bee_node_products_rank2: null or unaligned pointer");
+    MG_REQUIRE(x_d != nullptr || (l2 && r2), "mg_bee_node_products_rank2: l2 and r2, or x_d and the weights");
     const long blocks = ceil_div(n_nodes * (chan / kWave), 4);
     MG_REQUIRE(blocks < (1L << 31), "mg_bee_node_products_rank2: too many nodes for one launch");
     hipLaunchKernelGGL(node_rank2_linear_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, n_nodes,
-                       chan, l0, l1, l2, r0, r1, r2, packed_Y2, dim_d, out_d, P0, P1, node_max);
+                       chan, l0, l1, l2, r0, r1, r2, packed_Y2, dim_d, out_d, P0, P1, node_max, x_d, L2t, R2t, dim_in2);
     return check_launch("mg_bee_node_products_rank2");
 }
 

@@ -2075,18 +2075,30 @@ def _packed_rank2_weight(Y2, chan):
     return packed
 
 
-def bee_node_products_rank2(l0, l1, l2, r0, r1, r2, Y2, want_lower_ranks=False):
+def bee_node_products_rank2(l0, l1, l2, r0, r1, r2, Y2, want_lower_ranks=False, x_d=None, L2t=None, R2t=None):
     """The rank-2 output of SelfTensProds from its six operands in one kernel: Y2 (dim_d, 5 chan) applied to the five
     rank-2 products of l0/r0 (N, chan), l1/r1 (N, 3, chan), l2/r2 (N, 9, chan) -> (N, dim_d, 9); the rank-2 products
     are never stored.  For bee_rank2_supported(chan, dim_d).
     want_lower_ranks: returns (out_d, P0 (N,3,chan), P1 (N,3,5,chan), node_max (N, chan/64)) with the scalar and
-    vector products of bee_node_products and their partial maxima per node, written in the same pass."""
-    for t, nm in ((l0, "l0"), (l1, "l1"), (l2, "l2"), (r0, "r0"), (r1, "r1"), (r2, "r2")):
+    vector products of bee_node_products and their partial maxima per node, written in the same pass.
+    x_d (N, dim_in, 3, 3) with L2t, R2t (dim_in, chan), dim_in <= 16, in place of l2 and r2 (then None): the rank-2
+    operands l2 = L2 x_d, r2 = R2 x_d (L2t = L2.W.t() contiguous) are formed inside the kernel."""
+    inside = x_d is not None
+    named = [(l0, "l0"), (l1, "l1"), (r0, "r0"), (r1, "r1")] + ([(x_d, "x_d"), (L2t, "L2t"), (R2t, "R2t")] if inside
+                                                                 else [(l2, "l2"), (r2, "r2")])
+    for t, nm in named:
         _check_input(t, nm)
     N, chan = int(l0.size(0)), int(l0.size(1))
-    for t, comps in ((l0, None), (r0, None), (l1, 3), (r1, 3), (l2, 9), (r2, 9)):
+    shaped = [(l0, None), (r0, None), (l1, 3), (r1, 3)] + ([] if inside else [(l2, 9), (r2, 9)])
+    for t, comps in shaped:
         if tuple(t.shape) != ((N, chan) if comps is None else (N, comps, chan)):
             raise RuntimeError("operands must be (nodes, chan), (nodes, 3, chan), (nodes, 9, chan)")
+    dim_in2 = 0
+    if inside:
+        dim_in2 = int(L2t.size(0))
+        if (tuple(L2t.shape) != (dim_in2, chan) or tuple(R2t.shape) != (dim_in2, chan) or dim_in2 > 16
+                or x_d.numel() != N * dim_in2 * 9):
+            raise RuntimeError("x_d must hold nodes x dim_in x 9 floats and L2t, R2t be (dim_in, chan), dim_in <= 16")
     if not Y2.is_cuda or Y2.dtype != torch.float32 or Y2.dim() != 2 or int(Y2.size(1)) != 5 * chan or Y2.stride(1) != 1:
         raise RuntimeError("Y2 must be a float32 CUDA tensor (dim_d, 5 chan) with unit stride along a row")
     if not bee_rank2_supported(chan, Y2.size(0)):
@@ -2101,7 +2113,7 @@ def bee_node_products_rank2(l0, l1, l2, r0, r1, r2, Y2, want_lower_ranks=False):
             nmax = torch.empty(N, chan // 64, dtype=torch.float32, device=l0.device)
         L.check(_lib.mg_bee_node_products_rank2(N, chan, _p(l0), _p(l1), _p(l2), _p(r0), _p(r1), _p(r2),
                                                 _p(_packed_rank2_weight(Y2, chan)), dim_d, _p(out), _p(P0), _p(P1),
-                                                _p(nmax), _stream()))
+                                                _p(nmax), _p(x_d), _p(L2t), _p(R2t), dim_in2, _stream()))
     return (out, P0, P1, nmax) if want_lower_ranks else out
 
 

@@ -404,6 +404,28 @@ def test_rank2_products_and_their_output_linear_in_one_kernel(pkg, chan, dim_d, 
     assert nmax.shape == (N, chan // 64)
     assert torch.equal(nmax.amax(1), torch.maximum(Q0.abs().amax(dim=(1, 2)), Q1.abs().amax(dim=(1, 2, 3))))
     P2 = ops.bee_node_products(*dev)[2]
+    # the rank-2 operands formed inside the kernel from x_d and the two weights: against the oracle fed with the
+    # float64 (float32) operands L2 x_d, R2 x_d
+    dim_in = 16 if chan == 256 else 5
+    x_d = torch.randn(N, dim_in, 3, 3, generator=g) * size[:, None, None]
+    W_L2, W_R2 = torch.randn(chan, dim_in, generator=g) / dim_in ** 0.5, torch.randn(chan, dim_in, generator=g) / dim_in ** 0.5
+    y4, R0, R1, nmax4 = ops.bee_node_products_rank2(dev[0], dev[1], None, dev[3], dev[4], None, W, want_lower_ranks=True,
+                                                     x_d=x_d.cuda(), L2t=W_L2.t().contiguous().cuda(),
+                                                     R2t=W_R2.t().contiguous().cuda())
+
+    def products_inside(dt):
+        l2 = torch.einsum("ci,nixy->ncxy", W_L2.to(dt), x_d.to(dt))
+        r2 = torch.einsum("ci,nixy->ncxy", W_R2.to(dt), x_d.to(dt))
+        return dict(zip(OP.BEE_ORDER, OP.bee(to_ref(l[0].to(dt), 0), to_ref(l[1].to(dt), 1), l2,
+                                             to_ref(r[0].to(dt), 0), to_ref(r[1].to(dt), 1), r2)))
+    assert_parity_of(y4, lambda dt: sum(torch.einsum("oc,ncxy->noxy", W[:, k * chan:(k + 1) * chan].cpu().to(dt),
+                                                      products_inside(dt)[lab])
+                                        for k, lab in enumerate(labs)).reshape(N, dim_d, 9),
+                     "rank-2 output with the rank-2 operands formed inside")
+    assert_parity_of(R0[:, 2], lambda dt: products_inside(dt)["220"], "220 with the rank-2 operands formed inside")
+    for k, lab in ((2, "121"), (3, "211")):
+        assert_parity_of(R1[:, :, k], lambda dt: products_inside(dt)[lab].transpose(1, 2), f"{lab} with operands formed inside")
+    assert torch.equal(nmax4.amax(1), torch.maximum(R0.abs().amax(dim=(1, 2)), R1.abs().amax(dim=(1, 2, 3))))
     # the stored-products route gives the same within the same bar
     stored = ops.tensor_linear_fwd(2, W, P2.reshape(N, 9, 5 * chan), x_layout=ops.LAYOUT_COMP_CHAN)
     assert_parity_of(stored.reshape(N, dim_d, 9), ref, "stored products + GEMM")
