@@ -95,7 +95,8 @@ __global__ void __launch_bounds__(256) node_products_kernel(long n_nodes, int ch
 // (A persistent variant whose workgroups walk over the nodes with the next node's operands already requested was
 // measured at 65 536 nodes, 256 channels: 0.61 ms against 0.57 ms; the kernel is bound by the matrix instructions,
 // 0.31 ms of pipe time at 9 of 16 rows used, and what each wave does around them, not by the latency of its loads.)
-__global__ void __launch_bounds__(256) node_rank2_linear_kernel(long n_nodes, int chan, const float* __restrict__ l0,
+__global__ void __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(5, 8)))
+node_rank2_linear_kernel(long n_nodes, int chan, const float* __restrict__ l0,
                                                                 const float* __restrict__ l1, const float* __restrict__ l2,
                                                                 const float* __restrict__ r0, const float* __restrict__ r1,
                                                                 const float* __restrict__ r2,
