@@ -146,11 +146,14 @@ class SelfTensProds(nn.Module):
                    None if (node_pass and dim_d <= 16) else ops.components_as_rows(2, x_d)]
         # ... and with at most 16 rank-2 input channels it also forms L2 x_d and R2 x_d itself
         inside2 = node_pass and dim_d <= 16
+        # (and the row maxima of x_a, which the split-fp16 path scales by)
+        bound_a = ops.row_absmax(x_a) if ops.get_linear_mode() == ops.LINEAR_F16X2 else None
         def input_linear(k, lin, x):
             if k == 2 and inside2:
                 return lambda: None
             return lambda: ops.tensor_linear_fwd(k, lin.W, x, y_layout=C if k else ops.LAYOUT_CHAN_COMP,
-                                                 want_rowmax=not node_pass, x_rows=as_rows[k])
+                                                 want_rowmax=not node_pass, x_rows=as_rows[k],
+                                                 row_bound=bound_a if k == 0 else None)
         pairs = ops.concurrent([input_linear(k, lin, x)
                                 for side in ((self.L0, self.L1, self.L2), (self.R0, self.R1, self.R2))
                                 for k, (lin, x) in enumerate(zip(side, (x_a, x_v, x_d)))], rows)
