@@ -216,6 +216,25 @@ def test_linear_f16x2_component_outputs_and_node_bounds(ops, nodes, T, dim_in, d
     _check(out, lambda dt: base.to(dt) + ref(dt), "f16x2, component outputs, accumulate")
 
 
+@pytest.mark.parametrize("inds,rows,dim_in,dim_out", [(1, 12000, 64, 256), (2, 4000, 16, 128), (1, 11000, 40, 64)])
+def test_rows_per_component_formed_once_for_several_weights(ops, inds, rows, dim_in, dim_out):
+    """components_as_rows + x_rows=: two weights applied to the same x give, bit for bit, what two plain calls give;
+    None (and the plain route) when the input would not take that path."""
+    g = torch.Generator().manual_seed(inds + rows)
+    x = torch.randn(rows, dim_in, *([3] * inds), generator=g).cuda()
+    shared = ops.components_as_rows(inds, x)
+    assert shared is not None and shared[0].shape[0] == rows * 3 ** inds and shared[0].shape[1] % 32 == 0
+    for k in range(2):
+        W = (torch.randn(dim_out, dim_in, generator=g) / dim_in ** 0.5).cuda()
+        y0 = ops.tensor_linear_fwd(inds, W, x, y_layout=ops.LAYOUT_COMP_CHAN)
+        y1 = ops.tensor_linear_fwd(inds, W, x, y_layout=ops.LAYOUT_COMP_CHAN, x_rows=shared)
+        assert torch.equal(y0, y1)
+        _check(y1, lambda dt: OP.tensor_linear(inds, W.cpu().to(dt), x.cpu().to(dt)).reshape(
+            rows, dim_out, 3 ** inds).transpose(1, 2), "shared rows per component")
+    assert ops.components_as_rows(inds, x[:100].contiguous()) is None
+    assert ops.components_as_rows(0, x) is None
+
+
 def test_linear_out_bound_is_an_upper_bound(ops):
     g = torch.Generator().manual_seed(5)
     W = torch.randn(96, 64, generator=g).cuda()
