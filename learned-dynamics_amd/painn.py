@@ -235,8 +235,22 @@ class Message(nn.Module):
             cache[key] = self._grid_phases(rows, shift).to(torch.float32).to(device).contiguous()
         return cache[key]
 
+    keep_table = False        # opt-in: the grid of one set of weights is kept from one forward to the next
+
     def filter_table(self, rows, shift=0.0):
-        """The filter at d = (k + shift) 2 r0 / rows, k = 0 .. rows - 1: (rows, 4n)."""
+        """The filter at d = (k + shift) 2 r0 / rows, k = 0 .. rows - 1: (rows, 4n).  Evaluated in every call unless
+        keep_table is set: then the grid (a function of the weights alone, like their packed planes) is kept per
+        version of the weights, which saves the forward its 512-row MLP."""
+        if not (self.keep_table and shift == 0.0) or diff.wants_grad(self.mlp_dist):
+            return self._evaluate_filter_table(rows, shift)
+        key = (ops.stamp(list(self.mlp_dist.parameters())), rows, ops.get_linear_mode())
+        kept = self.__dict__.get("_kept_table")
+        if kept is None or kept[0] != key:
+            with ops.derived_tensors():
+                kept = self.__dict__["_kept_table"] = (key, self._evaluate_filter_table(rows, shift))
+        return kept[1]
+
+    def _evaluate_filter_table(self, rows, shift=0.0):
         first = self.mlp_dist.layers[0]
         device = first.weight.device
         unit = ops.linear_in_unit_bound(device)

@@ -435,6 +435,37 @@ def test_message_with_filter_table_and_with_filter_mlp_per_edge_against_the_orac
         assert_parity_of(pair, oracle, f"Message n_rbf={n_rbf}, {rows} rows, {name}")
 
 
+def test_kept_filter_grid_follows_the_weights(pkg):
+    """Message.keep_table: the grid is evaluated once per version of the weights (the same tensor comes back), the
+    forward gives bit for bit what it gives with the grid evaluated in the call, and an in-place update of a weight
+    makes the next call evaluate it again."""
+    painn = importlib.import_module("learned-dynamics_amd.painn")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    torch.manual_seed(11)
+    n, N, r0 = 64, 300, 6.0
+    msg = painn.Message(r0, n, 16).cuda()
+    g = torch.Generator().manual_seed(12)
+    src = torch.repeat_interleave(torch.arange(N), torch.randint(20, 40, (N,), generator=g))
+    E = int(src.numel())
+    graph = gl.Graph(src.cuda(), torch.randint(0, N, (E,), generator=g).cuda(), None, 1, N)
+    r = (torch.randn(E, 3, generator=g) * 3.0).cuda()
+    x_a, x_v = torch.randn(1, N, n, generator=g).cuda(), torch.randn(1, N, n, 3, generator=g).cuda()
+    with torch.no_grad():
+        rows = msg.table_rows()
+        assert rows and E >= 4 * rows
+        ref = msg(graph, x_a, x_v, r)
+        msg.keep_table = True
+        t1 = msg.filter_table(rows)
+        assert msg.filter_table(rows) is t1
+        got = msg(graph, x_a, x_v, r)
+        assert torch.equal(got[0], ref[0]) and torch.equal(got[1], ref[1])
+        msg.mlp_dist.layers[4].bias.add_(0.25)
+        t2 = msg.filter_table(rows)
+        assert t2 is not t1 and not torch.equal(t2, t1)
+        msg.keep_table = False
+        assert torch.equal(msg.filter_table(rows), t2) and msg.filter_table(rows) is not t2
+
+
 def _scale_first_filter_layer(msg, factor):
     with torch.no_grad():
         msg.mlp_dist.layers[0].weight.mul_(factor)
