@@ -307,6 +307,13 @@ int mg_tensor_linear_f16x2_rowmax_parts(long rows, int dim_in, int dim_out);   /
 int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts,
                            long x_rowmax_stride, long x_rows_per_bound, long rows, int dim_in, int dim_out, const float* bias, int act, int accumulate,
                            int out_comps, float* y, float* y_rowmax, mg_stream_t stream);
+/* The same with the bound of row r given as bound_mul * x_rowmax[r] + bound_add (both >= 0): lets a caller carry one
+ * array of row maxima through a chain of layers, |act(x W^T + b)| <= |x|max * max_o sum_i |W[o,i]| + max|b|, without a
+ * launch per layer to update it.  No counterpart in the reference. */
+int mg_tensor_linear_f16x2_scaled_bound(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts,
+                                        long x_rowmax_stride, long x_rows_per_bound, long rows, int dim_in, int dim_out,
+                                        const float* bias, int act, int accumulate, int out_comps, float* y,
+                                        float* y_rowmax, float bound_mul, float bound_add, mg_stream_t stream);
 /* y = act(x W^T + bias) in float64 arithmetic: W (dim_out, dim_in) and bias are the float32 parameters, widened
  * exactly; x (rows, dim_in), every product and sum, the activation and y (rows, dim_out) are double.  The same
  * contraction as nn.Linear inside the reference's MLPs (archs/meanflow_painn8.py:38-51); float64 has no counterpart

@@ -78,6 +78,8 @@ _SIGNATURES = {
     "mg_linear_f64": [vp, vp, vp, i64, i32, i32, i32, vp, vp],
     "mg_tensor_linear_f16x2_rowmax_parts": [i64, i32, i32],
     "mg_tensor_linear_f16x2": [vp, vp, vp, i32, i64, i64, i64, i32, i32, vp, i32, i32, i32, vp, vp, vp],
+    "mg_tensor_linear_f16x2_scaled_bound": [vp, vp, vp, i32, i64, i64, i64, i32, i32, vp, i32, i32, i32, vp, vp,
+                                            ctypes.c_float, ctypes.c_float, vp],
     "mg_ant16_fwd": [i32, i32, ctypes.POINTER(i32), ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, vp, i64, i32, i32, i32,
                      i32, i32, vp, vp],
     "mg_ant16_grad_x": [i32, i32, ctypes.POINTER(i32), ctypes.POINTER(vp), ctypes.POINTER(vp), vp, vp, vp, i64, i32, i32, i32,

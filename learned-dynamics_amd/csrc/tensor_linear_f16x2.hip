@@ -127,7 +127,8 @@ __global__ void __launch_bounds__(64 * WAVES)
 linear_rows_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restrict__ w_inv, const float* __restrict__ X,
                          const float* __restrict__ xmax, int xmax_parts, long xmax_stride, long xmax_div, long R, int I,
                          int O, int O_pad, const float* __restrict__ bias, int act, int accumulate,
-                         float* __restrict__ Y, float* __restrict__ ymax, int tiles_n, long tiles_total, int out_T) {
+                         float* __restrict__ Y, float* __restrict__ ymax, int tiles_n, long tiles_total, int out_T,
+                         float bound_mul, float bound_add) {
     constexpr int TM = 32 * WAVES, TN = 32 * NI, THREADS = 64 * WAVES;
     constexpr int kPlaneW = TN * kRowW, kBufW = 2 * kPlaneW;
     constexpr int kPieces = 8 * TN;                          // 16-byte pieces of W per chunk (2 planes x TN rows x 4)
@@ -164,6 +165,7 @@ linear_rows_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restric
         float amax = 0.f;
         const float* xm = xmax + (ld_row / xmax_div) * xmax_stride;
         for (int p = 0; p < xmax_parts; p++) amax = fmaxf(amax, xm[p]);
+        amax = fmaf(amax, bound_mul, bound_add);             // the caller's bound of |x| is bound_mul * xmax + bound_add
         float inv;
         sx = pow2_scale(amax, &inv);
         if (g == 0) inv_sx[wave * 32 + m] = inv;
@@ -371,7 +373,7 @@ linear_rows_splitk_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __
                                 const float* __restrict__ X, const float* __restrict__ xmax, int xmax_parts,
                                 long xmax_stride, long xmax_div, long R, int I, int O, int O_pad,
                                 const float* __restrict__ bias, int act, int accumulate, float* __restrict__ Y,
-                                float* __restrict__ ymax, int tiles_n, int out_T) {
+                                float* __restrict__ ymax, int tiles_n, int out_T, float bound_mul, float bound_add) {
     constexpr int TN = 32 * NI, THREADS = 64 * WAVES;
     constexpr int kPitch = TN + 1;                            // floats per row of a partial tile
     __shared__ float partial[WAVES][32 * kPitch];
@@ -394,6 +396,7 @@ linear_rows_splitk_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __
         float amax = 0.f;
         const float* xm = xmax + (ld_row / xmax_div) * xmax_stride;
         for (int p = 0; p < xmax_parts; p++) amax = fmaxf(amax, xm[p]);
+        amax = fmaf(amax, bound_mul, bound_add);
         float inv;
         sx = pow2_scale(amax, &inv);
         if (wave == 0 && g == 0) inv_sx[m] = inv;
@@ -535,7 +538,7 @@ inline Shape choose_shape(long R, int I, int O) {
 template <int WAVES, int NI>
 int launch(const _Float16* planes, const float* w_inv, const float* x, const float* xmax, int parts, long stride,
            long div, long rows, int I, int O, int O_pad, const float* bias, int act, int accumulate, float* y,
-           float* ymax, int out_T, hipStream_t st) {
+           float* ymax, int out_T, float bound_mul, float bound_add, hipStream_t st) {
     const long tiles_m = ceil_div(rows, 32 * WAVES);
     const int tiles_n = (int)ceil_div(O, 32 * NI);
     const long total = tiles_m * tiles_n;
@@ -543,7 +546,7 @@ int launch(const _Float16* planes, const float* w_inv, const float* x, const flo
     MG_REQUIRE(grid <= 0x7fffffffL, "mg_tensor_linear_f16x2: grid too large (rows=%ld dim_out=%d)", rows, O);
     hipLaunchKernelGGL((linear_rows_f16x2_kernel<WAVES, NI>), dim3((unsigned)grid), dim3(64 * WAVES), 0, st, planes,
                        w_inv, x, xmax, parts, stride, div, rows, I, O, O_pad, bias, act, accumulate, y, ymax, tiles_n,
-                       total, out_T);
+                       total, out_T, bound_mul, bound_add);
     return check_launch("mg_tensor_linear_f16x2");
 }
 
@@ -608,6 +611,17 @@ int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_
                            long x_rowmax_stride, long x_rows_per_bound, long rows, int dim_in, int dim_out,
                            const float* bias, int act, int accumulate, int out_comps, float* y, float* y_rowmax,
                            mg_stream_t stream) {
+    return mg_tensor_linear_f16x2_scaled_bound(packed_W, x, x_rowmax, x_rowmax_parts, x_rowmax_stride, x_rows_per_bound,
+                                               rows, dim_in, dim_out, bias, act, accumulate, out_comps, y, y_rowmax, 1.0f,
+                                               0.0f, stream);
+}
+
+int mg_tensor_linear_f16x2_scaled_bound(const void* packed_W, const float* x, const float* x_rowmax, int x_rowmax_parts,
+                                        long x_rowmax_stride, long x_rows_per_bound, long rows, int dim_in, int dim_out,
+                                        const float* bias, int act, int accumulate, int out_comps, float* y,
+                                        float* y_rowmax, float bound_mul, float bound_add, mg_stream_t stream) {
+    MG_REQUIRE(bound_mul >= 0.f && bound_add >= 0.f && bound_mul == bound_mul && bound_add == bound_add,
+               "mg_tensor_linear_f16x2: the bound's factor and offset must be non-negative numbers");
     MG_REQUIRE(rows >= 0 && dim_in > 0 && dim_out >= 0, "mg_tensor_linear_f16x2: bad size");
     MG_REQUIRE(dim_in % 32 == 0, "mg_tensor_linear_f16x2: dim_in must be a multiple of 32");
     MG_REQUIRE(act >= 0 && act <= 2, "mg_tensor_linear_f16x2: unknown activation %d", act);
@@ -630,17 +644,17 @@ int mg_tensor_linear_f16x2(const void* packed_W, const float* x, const float* x_
         if (dim_out <= 32)
             hipLaunchKernelGGL((linear_rows_splitk_f16x2_kernel<8, 1>), dim3((unsigned)tiles), dim3(512), 0, st, planes,
                                w_inv, x, x_rowmax, x_rowmax_parts, x_rowmax_stride, x_rows_per_bound, rows, dim_in,
-                               dim_out, O_pad, bias, act, accumulate, y, y_rowmax, 1, out_comps);
+                               dim_out, O_pad, bias, act, accumulate, y, y_rowmax, 1, out_comps, bound_mul, bound_add);
         else
             hipLaunchKernelGGL((linear_rows_splitk_f16x2_kernel<8, 2>), dim3((unsigned)tiles), dim3(512), 0, st, planes,
                                w_inv, x, x_rowmax, x_rowmax_parts, x_rowmax_stride, x_rows_per_bound, rows, dim_in,
-                               dim_out, O_pad, bias, act, accumulate, y, y_rowmax, 1, out_comps);
+                               dim_out, O_pad, bias, act, accumulate, y, y_rowmax, 1, out_comps, bound_mul, bound_add);
         return check_launch("mg_tensor_linear_f16x2");
     }
     const Shape sh = choose_shape(rows, dim_in, dim_out);
 #define MG_F16X2_LAUNCH(WV, N)                                                                                       \
     return launch<WV, N>(planes, w_inv, x, x_rowmax, x_rowmax_parts, x_rowmax_stride, x_rows_per_bound, rows, dim_in, \
-                         dim_out, O_pad, bias, act, accumulate, y, y_rowmax, out_comps, st)
+                         dim_out, O_pad, bias, act, accumulate, y, y_rowmax, out_comps, bound_mul, bound_add, st)
     if (sh.waves == 8) {
         if (sh.ni == 1) MG_F16X2_LAUNCH(8, 1);
         if (sh.ni == 2) MG_F16X2_LAUNCH(8, 2);

@@ -1070,15 +1070,60 @@ def linear_out_bound(W, bias, in_bound):
     return torch.addcmul(bmax, in_bound.reshape(-1, 1), l1)
 
 
+_factor_cache = {}
+
+
+def linear_out_bound_factors(W, bias):
+    """(max_o sum_i |W[o, i]|, max_o |bias[o]|) as host floats: |act(x W^T + bias)| <= |x|max * first + second.
+    Read back once per version of the parameters (one host synchronisation then, none afterwards)."""
+    key = (id(W), id(bias))
+    hit = _factor_cache.get(key)
+    w_ver, b_ver = tensor_version(W), (tensor_version(bias) if bias is not None else 0)
+    if (hit is None or min(w_ver, b_ver) < 0 or hit[0]() is not W or hit[1] != w_ver
+            or (bias is not None and (hit[2]() is not bias or hit[3] != b_ver))):
+        with derived_tensors():
+            both = torch.stack([W.detach().abs().sum(dim=1).amax(),
+                                bias.detach().abs().amax() if bias is not None else W.new_zeros(())]).tolist()
+        # a little above the float32 value: the product with a row maximum must not round below the true bound
+        hit = (weakref.ref(W), w_ver, weakref.ref(bias) if bias is not None else None, b_ver,
+               both[0] * (1.0 + 1e-6), both[1] * (1.0 + 1e-6))
+        if len(_factor_cache) > 1024:
+            _factor_cache.clear()
+        _factor_cache[key] = hit
+    return hit[4], hit[5]
+
+
 def f16x2_supported(rows, dim_in, dim_out, x):
     return dim_in % 32 == 0 and dim_in >= 64 and dim_out >= 8 and rows >= 256 and x.data_ptr() % 16 == 0
+
+
+class ScaledBound:
+    """Row bounds given as mul * base + add: base (rows, parts) row maxima as some kernel emitted them, mul and add host
+    floats.  A chain of layers whose bounds follow from the weight norms (linear_out_bound_factors) carries one array
+    this way, without a launch per layer to update it; tensor() forms the array for a consumer that wants one."""
+    __slots__ = ("base", "mul", "add")
+
+    def __init__(self, base, mul=1.0, add=0.0):
+        self.base, self.mul, self.add = base, float(mul), float(add)
+
+    def through(self, l1, bmax):
+        """The bound after a linear layer with these norms (and any act with |act(z)| <= |z|)."""
+        return ScaledBound(self.base, self.mul * l1, self.add * l1 + bmax)
+
+    def tensor(self):
+        b = self.base if self.base.size(1) == 1 else self.base.amax(dim=1, keepdim=True)
+        return b * self.mul + self.add
 
 
 def tensor_linear_f16x2(W, x, x_rowmax=None, bias=None, act=ACT_NONE, out=None, accumulate=False, out_comps=1,
                         want_rowmax=False, rows_per_bound=1):
     """y = act(x W^T + bias) for plain rows x (rows, dim_in) through the two-piece fp16 split.
     x_rowmax (rows, parts), or (1, parts) for one bound shared by all rows: upper bounds of the
-    row maxima of |x| (None: computed here).  Returns y, or (y, y_rowmax) with want_rowmax=True."""
+    row maxima of |x| (None: computed here), or a ScaledBound of such an array.
+    Returns y, or (y, y_rowmax) with want_rowmax=True."""
+    bound_mul, bound_add = 1.0, 0.0
+    if isinstance(x_rowmax, ScaledBound):
+        x_rowmax, bound_mul, bound_add = x_rowmax.base, x_rowmax.mul, x_rowmax.add
     _check_input(x, "x")
     if x.dim() != 2 or W.dim() != 2 or x.size(1) != W.size(1):
         raise RuntimeError("expected x (rows, dim_in) and W (dim_out, dim_in)")
@@ -1110,9 +1155,10 @@ def tensor_linear_f16x2(W, x, x_rowmax=None, bias=None, act=ACT_NONE, out=None, 
                 raise RuntimeError("row maxima are only produced for out_comps == 1")
             parts = int(_lib.mg_tensor_linear_f16x2_rowmax_parts(rows, dim_in, dim_out))
             ymax = torch.empty(rows, parts, dtype=torch.float32, device=x.device)
-        L.check(_lib.mg_tensor_linear_f16x2(_p(packed_weight_f16x2(W)), _p(x), _p(x_rowmax), int(x_rowmax.size(1)),
-                                            rowmax_stride, int(rows_per_bound), rows, dim_in, dim_out, _p(bias), int(act), int(bool(accumulate)),
-                                            int(out_comps), _p(y), _p(ymax), _stream()))
+        L.check(_lib.mg_tensor_linear_f16x2_scaled_bound(
+            _p(packed_weight_f16x2(W)), _p(x), _p(x_rowmax), int(x_rowmax.size(1)), rowmax_stride, int(rows_per_bound),
+            rows, dim_in, dim_out, _p(bias), int(act), int(bool(accumulate)), int(out_comps), _p(y), _p(ymax),
+            bound_mul, bound_add, _stream()))
     return (y, ymax) if want_rowmax else y
 
 

@@ -51,7 +51,15 @@ def _linear(x, lin, act, bound=None, want_bound=True):
         y = ops.tensor_linear_f16x2(lin.weight, x, bound, bias=lin.bias, act=act)
     else:
         y = ops.tensor_linear_fwd(0, lin.weight, x, bias=lin.bias, act=act)
-    return y, (ops.linear_out_bound(lin.weight, lin.bias, bound) if bound is not None and want_bound else None)
+    if bound is None or not want_bound:
+        return y, None
+    if isinstance(bound, ops.ScaledBound) or bound.size(0) > 1:
+        # one bound per row: the array stays as it is and the layer's norms go into a factor and an offset that the
+        # next kernel applies (a constant bound, below, is a cached tensor and costs no launch either)
+        if not isinstance(bound, ops.ScaledBound):
+            bound = ops.ScaledBound(bound)
+        return y, bound.through(*ops.linear_out_bound_factors(lin.weight, lin.bias))
+    return y, ops.linear_out_bound(lin.weight, lin.bias, bound)
 
 
 class MLP(nn.Module):

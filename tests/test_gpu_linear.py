@@ -235,6 +235,39 @@ def test_rows_per_component_formed_once_for_several_weights(ops, inds, rows, dim
     assert ops.components_as_rows(0, x) is None
 
 
+def test_row_bounds_carried_as_factor_and_offset(ops):
+    """ScaledBound: a chain of three layers that hands the first layer's row maxima on as (array, factor, offset)
+    gives the float64 chain at the layer tolerance, the factors are upper bounds of what they stand for, and a
+    negative factor is refused by the library."""
+    g = torch.Generator().manual_seed(21)
+    x = (torch.randn(3000, 128, generator=g) * 10.0 ** torch.randint(-3, 4, (3000, 1), generator=g).float()).cuda()
+    Ws = [(torch.randn(256, 128, generator=g) / 128 ** 0.5).cuda(), (torch.randn(256, 256, generator=g) / 16).cuda(),
+          (torch.randn(192, 256, generator=g) / 16).cuda()]
+    bs = [torch.randn(256, generator=g).cuda() * 0.1, torch.randn(256, generator=g).cuda() * 0.1, None]
+    bound = ops.ScaledBound(ops.row_absmax(x))
+    h = x
+    for k, (W, b) in enumerate(zip(Ws, bs)):
+        l1, bmax = ops.linear_out_bound_factors(W, b)
+        assert l1 >= float(W.abs().sum(1).amax()) and bmax >= (float(b.abs().amax()) if b is not None else 0.0)
+        h_next = ops.tensor_linear_f16x2(W, h, bound, bias=b, act=ops.ACT_SILU if k < 2 else ops.ACT_NONE)
+        assert bool((h_next.abs().amax(1, keepdim=True) <= bound.through(l1, bmax).tensor() * (1 + 1e-6)).all())
+        h, bound = h_next, bound.through(l1, bmax)
+
+    def chain(dt):
+        t = x.cpu().to(dt)
+        for k, (W, b) in enumerate(zip(Ws, bs)):
+            t = torch.nn.functional.linear(t, W.cpu().to(dt), None if b is None else b.cpu().to(dt))
+            t = torch.nn.functional.silu(t) if k < 2 else t
+        return t
+    _check(h, chain, "three layers on one array of row maxima")
+    assert ops.linear_out_bound_factors(Ws[0], bs[0]) == ops.linear_out_bound_factors(Ws[0], bs[0])
+    with torch.no_grad():
+        Ws[0].mul_(3.0)
+    assert ops.linear_out_bound_factors(Ws[0], bs[0])[0] > 2.9 * l1 * 0 + float(Ws[0].abs().sum(1).amax()) * 0.999
+    with pytest.raises(RuntimeError, match="non-negative"):
+        ops.tensor_linear_f16x2(Ws[1], h.new_zeros(300, 256), ops.ScaledBound(h.new_ones(300, 1), -1.0, 0.0))
+
+
 def test_linear_out_bound_is_an_upper_bound(ops):
     g = torch.Generator().manual_seed(5)
     W = torch.randn(96, 64, generator=g).cuda()
