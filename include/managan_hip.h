@@ -594,6 +594,12 @@ int mg_tensor_linear_f16x2_rowsum(const void* packed_W, const float* x, const fl
                                   long x_rowmax_stride, long rows, int dim_in, int dim_out, const float* bias, int act,
                                   const int* row_ptr, const int* seg, long n_out, float scale, void* workspace,
                                   float* y, float* out, mg_stream_t stream);
+/* The same with the bound of row r given as bound_mul * x_rowmax[r] + bound_add (see mg_tensor_linear_f16x2_scaled_bound). */
+int mg_tensor_linear_f16x2_rowsum_scaled_bound(const void* packed_W, const float* x, const float* x_rowmax,
+                                               int x_rowmax_parts, long x_rowmax_stride, long rows, int dim_in,
+                                               int dim_out, const float* bias, int act, const int* row_ptr,
+                                               const int* seg, long n_out, float scale, void* workspace, float* y,
+                                               float* out, float bound_mul, float bound_add, mg_stream_t stream);
 
 /* Update.forward (archs/meanflow_painn8.py:63-75), elementwise parts around its GEMMs.
  * lrv = [lin_l | lin_r | lin_v] applied to x_v (one stacked tensor_linear), stored (rows, 3n, 3) as the reference

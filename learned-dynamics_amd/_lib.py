@@ -129,6 +129,8 @@ _SIGNATURES = {
     "mg_bee_products_linear": [i32, vp, vp, vp, vp, vp, vp, vp, i64, i32, vp, i32, i32, vp, vp],
     "mg_tensor_linear_f16x2_rowsum_workspace_bytes": [i64, i32, ctypes.POINTER(ctypes.c_size_t)],
     "mg_tensor_linear_f16x2_rowsum": [vp, vp, vp, i32, i64, i64, i32, i32, vp, i32, vp, vp, i64, f32, vp, vp, vp, vp],
+    "mg_tensor_linear_f16x2_rowsum_scaled_bound": [vp, vp, vp, i32, i64, i64, i32, i32, vp, i32, vp, vp, i64, f32, vp, vp,
+                                                   vp, f32, f32, vp],
     "mg_painn_filter_hidden": [vp, i64, f32, vp, i64, i64, vp, vp, vp, i32, vp, vp, vp],
     "mg_painn_filter_message_workspace_bytes": [i64, i32, ctypes.POINTER(ctypes.c_size_t)],
     "mg_painn_filter_message": [vp, vp, vp, vp, i32, i64, i32, vp, vp, vp, vp, vp, vp, i64, i64, i32, f32, vp, vp, vp, vp, vp, vp],

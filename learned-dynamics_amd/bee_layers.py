@@ -366,7 +366,8 @@ class Messages(nn.Module):
                 # psi_a and its sum over the edges of each node from one kernel
                 s_psi, psi_a = ops.tensor_linear_f16x2_rowsum(Y0, P0, bound, graph.row_ptr, graph.src32, rows,
                                                               want_rows=True)
-                bound = ops.linear_out_bound(Y0, None, bound)
+                # from here on the edge kernel's row maxima travel with a factor and an offset (the layers' norms)
+                bound = ops.linear_out_bound(Y0, None, ops.ScaledBound(bound))
             else:
                 psi_a, bound = _linear(P0, Y0, None, ops.ACT_NONE, bound)
                 s_psi = None

@@ -373,7 +373,8 @@ linear_rowsum_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restr
                            const float* __restrict__ bias, const float* __restrict__ X,
                            const float* __restrict__ xmax, int xmax_parts, long xmax_stride, long R, int I, int O,
                            const int* __restrict__ seg, float* __restrict__ slots, long n_blocks, float scale,
-                           float* __restrict__ Y, float* __restrict__ out, int tiles_n, long tiles_total) {
+                           float* __restrict__ Y, float* __restrict__ out, int tiles_n, long tiles_total,
+                           float bound_mul, float bound_add) {
     constexpr int kSlice = kFSlice, kRed = kFRed;
     __shared__ __attribute__((aligned(16))) unsigned char lds[2 * kFBufW];
     __shared__ __attribute__((aligned(16))) float wb[2 * kFTN];   // the tile's 1 / weight scale, then its bias
@@ -405,6 +406,7 @@ linear_rowsum_f16x2_kernel(const _Float16* __restrict__ Wp, const float* __restr
         float amax = 0.f;
         const float* xm = xmax + ld_row * xmax_stride;
         for (int p = 0; p < xmax_parts; p++) amax = fmaxf(amax, xm[p]);
+        amax = fmaf(amax, bound_mul, bound_add);             // the caller's bound of |x| is bound_mul * xmax + bound_add
         sx = pow2_scale(amax, &isx);
     }
     const int my_seg = seg[ld_row];
@@ -747,6 +749,18 @@ int mg_tensor_linear_f16x2_rowsum(const void* packed_W, const float* x, const fl
                                   long x_rowmax_stride, long rows, int dim_in, int dim_out, const float* bias, int act,
                                   const int* row_ptr, const int* seg, long n_out, float scale, void* workspace,
                                   float* y, float* out, mg_stream_t stream) {
+    return mg_tensor_linear_f16x2_rowsum_scaled_bound(packed_W, x, x_rowmax, x_rowmax_parts, x_rowmax_stride, rows, dim_in,
+                                                      dim_out, bias, act, row_ptr, seg, n_out, scale, workspace, y, out,
+                                                      1.0f, 0.0f, stream);
+}
+
+int mg_tensor_linear_f16x2_rowsum_scaled_bound(const void* packed_W, const float* x, const float* x_rowmax,
+                                               int x_rowmax_parts, long x_rowmax_stride, long rows, int dim_in,
+                                               int dim_out, const float* bias, int act, const int* row_ptr,
+                                               const int* seg, long n_out, float scale, void* workspace, float* y,
+                                               float* out, float bound_mul, float bound_add, mg_stream_t stream) {
+    MG_REQUIRE(bound_mul >= 0.f && bound_add >= 0.f && bound_mul == bound_mul && bound_add == bound_add,
+               "mg_tensor_linear_f16x2_rowsum: the bound's factor and offset must be non-negative numbers");
     MG_REQUIRE(dim_out >= 256 && dim_out % 256 == 0, "mg_tensor_linear_f16x2_rowsum: dim_out must be a multiple of 256 (got %d)", dim_out);
     MG_REQUIRE(dim_in >= 64 && dim_in % 32 == 0, "mg_tensor_linear_f16x2_rowsum: dim_in must be a multiple of 32, at least 64 (got %d)", dim_in);
     MG_REQUIRE(rows >= 0 && n_out >= 0 && rows < (1L << 31) && n_out < (1L << 31), "mg_tensor_linear_f16x2_rowsum: bad size");
@@ -770,7 +784,7 @@ int mg_tensor_linear_f16x2_rowsum(const void* packed_W, const float* x, const fl
 #define MG_ROWSUM_LAUNCH(A, S)                                                                                       \
     linear_rowsum_f16x2_kernel<A, S><<<dim3((unsigned)grid), dim3(64 * kFW), 0, s>>>(                                \
         planes, w_inv, bias, x, x_rowmax, x_rowmax_parts, x_rowmax_stride, rows, dim_in, dim_out, seg, slots, n_blocks, \
-        scale, y, out, tiles_n, tiles_total)
+        scale, y, out, tiles_n, tiles_total, bound_mul, bound_add)
         if (y) {
             if (act == 1) MG_ROWSUM_LAUNCH(1, true);
             else if (act == 2) MG_ROWSUM_LAUNCH(2, true);

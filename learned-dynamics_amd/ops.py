@@ -1040,6 +1040,8 @@ def linear_out_bound(W, bias, in_bound):
     The two weight norms are cached per parameter object and version (device tensors; no host
     synchronisation).  These bounds feed mg_tensor_linear_f16x2, whose accuracy does not depend on
     how tight they are as long as they stay within a factor 2^14 of the true row maxima."""
+    if isinstance(in_bound, ScaledBound):
+        return in_bound.through(*linear_out_bound_factors(W, bias))
     if in_bound is None:
         in_bound = linear_in_unit_bound(W.device)
     key = ("norms", id(W), id(bias))
@@ -1941,7 +1943,11 @@ def f16x2_rowsum_supported(rows, dim_in, dim_out, x):
 def tensor_linear_f16x2_rowsum(W, x, x_bound, row_ptr, seg, n_out, bias=None, act=ACT_NONE, scale=1.0, want_rows=False):
     """(out, y): out[s] = scale * sum over the rows r of segment s of act(bias + W x[r]) (n_out, dim_out); y is the
     per-row result (rows, dim_out) when want_rows is set, else None.  Rows are sorted by segment: seg (rows,) int32
-    ascending, row_ptr its CSR form.  x_bound: (rows, parts) or (1, parts) upper bounds of the row maxima of |x|."""
+    ascending, row_ptr its CSR form.  x_bound: (rows, parts) or (1, parts) upper bounds of the row maxima of |x|, or
+    a ScaledBound of such an array."""
+    bound_mul, bound_add = 1.0, 0.0
+    if isinstance(x_bound, ScaledBound):
+        x_bound, bound_mul, bound_add = x_bound.base, x_bound.mul, x_bound.add
     for t, nm in ((W, "W"), (x, "x"), (x_bound, "x_bound")):
         _check_input(t, nm)
     for t, nm in ((row_ptr, "row_ptr"), (seg, "seg")):
@@ -1965,9 +1971,10 @@ def tensor_linear_f16x2_rowsum(W, x, x_bound, row_ptr, seg, n_out, bias=None, ac
         y = torch.empty(rows, dim_out, dtype=torch.float32, device=dev) if want_rows else None
         work = torch.empty(nbytes.value // 4, dtype=torch.float32, device=dev)
         stride = 0 if x_bound.size(0) == 1 else int(x_bound.size(1))
-        L.check(_lib.mg_tensor_linear_f16x2_rowsum(
+        L.check(_lib.mg_tensor_linear_f16x2_rowsum_scaled_bound(
             _p(packed_weight_f16x2(W)), _p(x), _p(x_bound), int(x_bound.size(1)), stride, rows, dim_in, dim_out,
-            _p(bias), int(act), _p(row_ptr), _p(seg), int(n_out), float(scale), _p(work), _p(y), _p(out), _stream()))
+            _p(bias), int(act), _p(row_ptr), _p(seg), int(n_out), float(scale), _p(work), _p(y), _p(out),
+            bound_mul, bound_add, _stream()))
     return out, y
 
 
