@@ -608,7 +608,7 @@ int mg_tensor_linear_f16x2_rowsum_scaled_bound(const void* packed_W, const float
  *   vec:  v = lin_v(x_v) * y[:, 0:n];  out_v (rows, n, 3) = res_v + v / sqrt(1 + |v|^2)   (y: (rows, 3n) MLP output)
  * The scalar output is mg_group_norm(mode 1) of ip * y[:, n:2n] plus y[:, 2n:3n]. */
 int mg_painn_update_pre(const float* lrv, int lrv_comp_major, const float* x_a, long rows, int n, float* ip, float* cat,
-                        mg_stream_t stream);
+                        float* cat_rowmax /* (rows) max |cat[r,:]|, or NULL; n <= 256 */, mg_stream_t stream);
 int mg_painn_update_vec(const float* lrv, int lrv_comp_major, const float* y, const float* res_v /* or NULL */, long rows, int n,
                         float* out_v, mg_stream_t stream);
 

@@ -92,7 +92,7 @@ _SIGNATURES = {
     "mg_group_norm_scratch_bytes": [i32, i32, ctypes.POINTER(ctypes.c_size_t)],
     "mg_group_norm": [i32, vp, i64, vp, i64, i32, i32, i32, i32, i32, f32, vp, vp, vp, i64, vp, vp, vp, vp],
     "mg_tens_sigmoid": [i32, vp, i64, vp, vp],
-    "mg_painn_update_pre": [vp, i32, vp, i64, i32, vp, vp, vp],
+    "mg_painn_update_pre": [vp, i32, vp, i64, i32, vp, vp, vp, vp],
     "mg_painn_update_vec": [vp, i32, vp, vp, i64, i32, vp, vp],
     "mg_radial_encode": [i32, vp, i64, i32, f32, vp, vp],
     "mg_bee_node_products": [i64, i32, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp, vp],

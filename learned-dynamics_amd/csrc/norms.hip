@@ -152,19 +152,36 @@ __device__ __forceinline__ float lrv_at(const float* __restrict__ row, int n, in
     return COMP_MAJOR ? row[x * 3 * n + j] : row[j * 3 + x];
 }
 
+// cat_rowmax (rows; or null): max |cat[r, :]|, the row bound of the MLP that reads cat; written when one workgroup
+// covers a row (n <= 256: gridDim.y == 1)
 template <bool COMP_MAJOR>
 __global__ void __launch_bounds__(256) painn_update_pre_kernel(const float* __restrict__ lrv, const float* __restrict__ x_a,
-                                                               int n, float* __restrict__ ip, float* __restrict__ cat) {
+                                                               int n, float* __restrict__ ip, float* __restrict__ cat,
+                                                               float* __restrict__ cat_rowmax) {
+    __shared__ float wave_max[4];
     const long r = blockIdx.x;
     const int c = blockIdx.y * blockDim.x + threadIdx.x;
-    if (c >= n) return;
-    const float* row = lrv + r * 9 * n;
-    float l[3], rr[3];
+    float mx = 0.f;
+    if (c < n) {
+        const float* row = lrv + r * 9 * n;
+        float l[3], rr[3];
 #pragma unroll
-    for (int x = 0; x < 3; x++) { l[x] = lrv_at<COMP_MAJOR>(row, n, c, x); rr[x] = lrv_at<COMP_MAJOR>(row, n, n + c, x); }
-    ip[r * n + c] = l[0] * rr[0] + l[1] * rr[1] + l[2] * rr[2];
-    cat[r * 2 * n + c] = x_a[r * n + c];
-    cat[r * 2 * n + n + c] = sqrtf(rr[0] * rr[0] + rr[1] * rr[1] + rr[2] * rr[2]);
+        for (int x = 0; x < 3; x++) { l[x] = lrv_at<COMP_MAJOR>(row, n, c, x); rr[x] = lrv_at<COMP_MAJOR>(row, n, n + c, x); }
+        ip[r * n + c] = l[0] * rr[0] + l[1] * rr[1] + l[2] * rr[2];
+        const float a = x_a[r * n + c], nr = sqrtf(rr[0] * rr[0] + rr[1] * rr[1] + rr[2] * rr[2]);
+        cat[r * 2 * n + c] = a;
+        cat[r * 2 * n + n + c] = nr;
+        mx = fmaxf(fabsf(a), nr);
+    }
+    if (cat_rowmax) {                                         // uniform over the workgroup
+        for (int d = 1; d < kWave; d <<= 1) mx = fmaxf(mx, __shfl_xor(mx, d));
+        if ((threadIdx.x & (kWave - 1)) == 0) wave_max[threadIdx.x / kWave] = mx;
+        __syncthreads();
+        if (threadIdx.x == 0) {
+            for (int w = 1; w < (int)(blockDim.x / kWave); w++) mx = fmaxf(mx, wave_max[w]);
+            cat_rowmax[r] = mx;
+        }
+    }
 }
 
 // PaiNN Update, vector output: v = lin_v(x_v) * y[0:n]; out = res_v + v / sqrt(1 + |v|^2), out (rows, n, 3)
@@ -265,7 +282,8 @@ int mg_tens_sigmoid(int inds, const float* x, long rows_times_chan, float* out, 
 }
 
 int mg_painn_update_pre(const float* lrv, int lrv_comp_major, const float* x_a, long rows, int n, float* ip, float* cat,
-                        mg_stream_t stream) {
+                        float* cat_rowmax, mg_stream_t stream) {
+    MG_REQUIRE(cat_rowmax == nullptr || n <= 256, "mg_painn_update_pre: row maxima are emitted for n <= 256");
     MG_REQUIRE(rows >= 0 && n >= 0, "mg_painn_update_pre: negative size");
     if (rows * n == 0) return MG_OK;
     MG_REQUIRE(lrv && x_a && ip && cat, "mg_painn_update_pre: null pointer");
@@ -273,9 +291,11 @@ int mg_painn_update_pre(const float* lrv, int lrv_comp_major, const float* x_a, 
     const int threads = n >= 256 ? 256 : (int)ceil_div(n, kWave) * kWave;
     const dim3 grid((unsigned)rows, (unsigned)ceil_div(n, threads));
     if (lrv_comp_major)
-        hipLaunchKernelGGL(painn_update_pre_kernel<true>, grid, dim3(threads), 0, (hipStream_t)stream, lrv, x_a, n, ip, cat);
+        hipLaunchKernelGGL(painn_update_pre_kernel<true>, grid, dim3(threads), 0, (hipStream_t)stream, lrv, x_a, n, ip, cat,
+                           cat_rowmax);
     else
-        hipLaunchKernelGGL(painn_update_pre_kernel<false>, grid, dim3(threads), 0, (hipStream_t)stream, lrv, x_a, n, ip, cat);
+        hipLaunchKernelGGL(painn_update_pre_kernel<false>, grid, dim3(threads), 0, (hipStream_t)stream, lrv, x_a, n, ip, cat,
+                           cat_rowmax);
     return check_launch("mg_painn_update_pre");
 }
 

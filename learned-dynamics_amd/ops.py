@@ -2308,8 +2308,9 @@ def _lrv_layout(lrv, rows, n):
     raise RuntimeError("lrv must have shape (rows, 3n, 3) or, component-major, (rows, 3, 3n)")
 
 
-def painn_update_pre(lrv, x_a):
-    """lrv (rows, 3n, 3) or component-major (rows, 3, 3n), x_a (rows, n) -> ip (rows, n), cat (rows, 2n)."""
+def painn_update_pre(lrv, x_a, want_rowmax=False):
+    """lrv (rows, 3n, 3) or component-major (rows, 3, 3n), x_a (rows, n) -> ip (rows, n), cat (rows, 2n);
+    want_rowmax: (ip, cat, rowmax) with rowmax (rows, 1) = max |cat[r, :]| from the same pass (None for n > 256)."""
     _check_input(lrv, "lrv")
     _check_input(x_a, "x_a")
     rows, n = int(x_a.shape[0]), int(x_a.shape[1])
@@ -2317,8 +2318,9 @@ def painn_update_pre(lrv, x_a):
     with torch.cuda.device(x_a.device):
         ip = torch.empty(rows, n, dtype=torch.float32, device=x_a.device)
         cat = torch.empty(rows, 2 * n, dtype=torch.float32, device=x_a.device)
-        L.check(_lib.mg_painn_update_pre(_p(lrv), layout, _p(x_a), rows, n, _p(ip), _p(cat), _stream()))
-    return ip, cat
+        rowmax = torch.empty(rows, 1, dtype=torch.float32, device=x_a.device) if want_rowmax and n <= 256 else None
+        L.check(_lib.mg_painn_update_pre(_p(lrv), layout, _p(x_a), rows, n, _p(ip), _p(cat), _p(rowmax), _stream()))
+    return (ip, cat, rowmax) if want_rowmax else (ip, cat)
 
 
 def painn_update_vec(lrv, y, res_v=None):

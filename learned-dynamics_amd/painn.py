@@ -146,8 +146,8 @@ class Update(nn.Module):
         W = cache["W"]
         # component-major (rows, 3, 3n): the GEMM stores whole rows, the two kernels below read with unit stride
         lrv = ops.tensor_linear_fwd(1, W, flat_v, y_layout=ops.LAYOUT_COMP_CHAN)
-        ip, cat = ops.painn_update_pre(lrv, flat_a)                             # l.r and [x_a | |r|]
-        y = self.mlp(cat)                                                       # (rows, 3n)
+        ip, cat, cat_max = ops.painn_update_pre(lrv, flat_a, want_rowmax=True)  # l.r, [x_a | |r|] and its row maxima
+        y = self.mlp(cat, cat_max)                                              # (rows, 3n)
         y3 = y.reshape(B, N, 3 * n)
         out_a = self.gn(ip.reshape(B, N, n), mul=y3[..., n:2 * n], add=y3[..., 2 * n:],
                         res=flat_a.reshape(B, N, n) if residual else None)

@@ -567,6 +567,12 @@ def test_update_elementwise_kernels_in_both_layouts(ops, rows, n):
     outs = []
     for lay in (lrv.cuda(), lrv.permute(0, 2, 1).contiguous().cuda()):
         ip, cat = ops.painn_update_pre(lay, x_a.cuda())
+        ip2, cat2, cat_max = ops.painn_update_pre(lay, x_a.cuda(), want_rowmax=True)
+        assert torch.equal(ip2, ip) and torch.equal(cat2, cat)
+        if n <= 256:                                         # the row maxima of cat from the same pass, exactly
+            assert torch.equal(cat_max, cat.abs().amax(dim=1, keepdim=True))
+        else:
+            assert cat_max is None
         out_v = ops.painn_update_vec(lay, y.cuda(), res.cuda())
         torch.testing.assert_close(ip.cpu().double(), want_ip, rtol=1e-5, atol=2e-6)
         torch.testing.assert_close(cat.cpu().double(), want_cat, rtol=1e-5, atol=1e-6)
