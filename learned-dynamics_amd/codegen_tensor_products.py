@@ -61,7 +61,15 @@ class Bee(torch.autograd.Function):
     @staticmethod
     def forward(ctx, l_0, l_1, l_2, r_0, r_1, r_2):
         ctx.save_for_backward(l_0, l_1, l_2, r_0, r_1, r_2)
+        ctx.save_for_forward(l_0, l_1, l_2, r_0, r_1, r_2)
         return tuple(ops.bee_fwd(*_c((l_0, l_1, l_2, r_0, r_1, r_2))))
+
+    @staticmethod
+    def jvp(ctx, *tangents):
+        """Forward mode: P(l_t, r) + P(l, r_t) (an operand without a tangent arrives as zeros)."""
+        l_0, l_1, l_2, r_0, r_1, r_2 = ctx.saved_tensors
+        left, right = Bee.apply(*tangents[:3], r_0, r_1, r_2), Bee.apply(l_0, l_1, l_2, *tangents[3:])
+        return tuple(a + b for a, b in zip(left, right))
 
     @staticmethod
     def backward(ctx, *dys):

@@ -11,6 +11,7 @@ for the reference.  Results equal the fused path up to fp32 summation order (tes
 import math
 
 import torch
+import torch.autograd.forward_ad as fwAD
 import torch.nn.functional as F
 
 from . import graph_layers as gl
@@ -19,13 +20,42 @@ from .codegen_tensor_products import Bee
 from .tensor_products import tensor_linear
 
 
+def has_tangent(t):
+    """True for a tensor that carries a forward-mode tangent (inside jvp below)."""
+    return t is not None and fwAD.unpack_dual(t).tangent is not None
+
+
+def differentiated(t):
+    """True when a derivative with respect to t is being taken, in either mode."""
+    return t is not None and ((torch.is_grad_enabled() and t.requires_grad) or has_tangent(t))
+
+
 def wants_grad(module, *tensors):
-    """True when autograd is recording and a gradient could flow to an input or a parameter."""
+    """True when a gradient could flow to an input or a parameter (autograd is recording), or an input carries a
+    forward-mode tangent: the cases the fused inference kernels do not serve."""
+    if any(has_tangent(t) for t in tensors):
+        return True
     if not torch.is_grad_enabled():
         return False
     if any(t is not None and t.requires_grad for t in tensors):
         return True
     return any(p.requires_grad for p in module.parameters())
+
+
+def jvp(f, primals, tangents):
+    """(f(*primals), the derivative of f at primals along tangents) in forward mode: every autograd function of this
+    package that a forward pass runs has a jvp rule made of the package's differentiable functions, so the pair costs
+    about two forward passes and both results can be differentiated afterwards (loss.backward()).
+    torch.autograd.functional.jvp(f, primals, tangents, create_graph=True), which the reference's meanflow loss calls
+    (archs/meanflow_painn8.py:274-282), gets the same derivative out of two nested backward passes, and the loss then
+    differentiates all three; its first result is the same f(*primals) that the loss evaluates again as v_pred
+    (archs/meanflow_painn8.py:291-292), so one call here stands for both."""
+    with fwAD.dual_level():
+        out = f(*(fwAD.make_dual(p, t) for p, t in zip(primals, tangents)))
+        value, tangent = fwAD.unpack_dual(out)
+        if tangent is None:
+            tangent = torch.zeros_like(value)
+    return value, tangent
 
 
 def linear(lin, x, x_bound=None, want_bound=False):
@@ -48,8 +78,14 @@ class _SiluOrder(torch.autograd.Function):
     @staticmethod
     def forward(ctx, z, order):
         ctx.save_for_backward(z)
+        ctx.save_for_forward(z)
         ctx.order = order
         return ops.silu_order(z.contiguous(), order)
+
+    @staticmethod
+    def jvp(ctx, z_t, _):
+        z, = ctx.saved_tensors
+        return z_t * _silu_order(z, ctx.order + 1)
 
     @staticmethod
     def backward(ctx, g):
@@ -185,12 +221,30 @@ class _PainnCombine(torch.autograd.Function):
     def forward(ctx, dist, actv_node, v_node, direction, by_dst, by_src, terms):
         ctx.by_dst, ctx.by_src, ctx.terms = by_dst, by_src, terms
         ctx.save_for_backward(dist, actv_node, v_node, direction)
+        ctx.save_for_forward(dist, actv_node, v_node, direction)
+        ctx.set_materialize_grads(False)
         m, a = ops.painn_combine_fwd(dist.contiguous(), actv_node.contiguous(), v_node.contiguous(),
                                      direction.contiguous(), node=by_dst.index, terms=terms)
         return (ops.segment_sum_csr(m, by_src.row_ptr, by_src.n_rows), ops.segment_sum_csr(a, by_src.row_ptr, by_src.n_rows))
 
     @staticmethod
+    def jvp(ctx, dist_t, actv_t, v_t, dir_t, *_):
+        """The function is linear in each argument within the terms that contain it: the tangent is the sum of the
+        function itself with one argument's tangent in that argument's place."""
+        dist, actv, v, direction = ctx.saved_tensors
+        idx, t = (ctx.by_dst, ctx.by_src), ctx.terms
+        slots = [(dist_t, (dist_t, actv, v, direction), t), (actv_t, (dist, actv_t, v, direction), t),
+                 (v_t, (dist, actv, v_t, direction), t & _TERMS_V), (dir_t, (dist, actv, v, dir_t), t & _TERMS_DIR)]
+        pairs = [_PainnCombine.apply(*args, *idx, mask) for x_t, args, mask in slots if x_t is not None and mask]
+        return _sum_opt([p[0] for p in pairs]), _sum_opt([p[1] for p in pairs])
+
+    @staticmethod
     def backward(ctx, g_v, g_a):
+        if g_v is None or g_a is None:
+            ref_v, ref_a = ctx.saved_tensors[2], ctx.saved_tensors[1]
+            nodes = ctx.by_src.n_rows
+            g_v = g_v if g_v is not None else ref_v.new_zeros(nodes, ref_v.size(1), 3)
+            g_a = g_a if g_a is not None else ref_a.new_zeros(nodes, ref_v.size(1))
         want = tuple(ctx.needs_input_grad[:4])
         grads = _PainnCombineGrad.apply(g_v, g_a, *ctx.saved_tensors, ctx.by_dst, ctx.by_src, ctx.terms, want)
         return tuple(g if need else None for g, need in zip(grads, want)) + (None, None, None)
@@ -360,7 +414,7 @@ def painn_filter(msg, r_ij):
     need no gradient (see below)."""
     E = r_ij.shape[0]
     rows = msg.table_rows() if (getattr(msg, "use_table", False) and E >= 4 * msg.TABLE_ROWS[0]) else 0
-    if r_ij.requires_grad:
+    if r_ij.requires_grad or has_tangent(r_ij):
         # The gradient for the edge vectors would go through the interpolant's derivative: differences of neighbouring
         # grid rows divided by the spacing, which amplifies the fp32-level noise of the grid values (1e-6 of their size
         # from the GEMMs that evaluate them) by rows / period: 4e-5 of the largest gradient entry at 2048 rows, 2e-4 at
@@ -438,6 +492,7 @@ class _MessageProducts(torch.autograd.Function):
         ctx.by_dst, ctx.by_src = by_dst, by_src
         a_node, v_node, d_node, enc, rh = (t.contiguous() for t in (a_node, v_node, d_node, enc, rh))
         ctx.save_for_backward(a_node, v_node, d_node, enc, rh)
+        ctx.save_for_forward(a_node, v_node, d_node, enc, rh)
         N, C = a_node.shape
         if enc_source is not None:
             enc8, W, b = enc_source
@@ -456,6 +511,22 @@ class _MessageProducts(torch.autograd.Function):
         prods = ops.bee_fwd_indexed(a_node, v_node, d_node, by_dst.index, enc, phi_v, phi_d)
         return tuple(p if lab[2] == "0" else ops.segment_sum_csr(p, by_src.row_ptr, by_src.n_rows)
                      for lab, p in zip(BEE_ORDER, prods))
+
+    @staticmethod
+    def jvp(ctx, a_t, v_t, d_t, enc_t, rh_t, *_):
+        """Forward mode through the plain formulation: the products are bilinear in (node operands, edge filters), so
+        the tangent is P(gathered tangents, filters) + P(gathered operands, the filters' tangent), summed per node
+        like the products themselves (an operand without a tangent arrives as zeros)."""
+        from .ops import BEE_ORDER
+        a_node, v_node, d_node, enc, rh = ctx.saved_tensors
+        by_dst, by_src = ctx.by_dst, ctx.by_src
+        gather = lambda ts: [gl._Gather.apply(t, by_dst) for t in ts]
+        phi_v, phi_d = _EdgeFilters.apply(enc, rh)
+        phi_v_t, phi_d_t = _edge_filters_tangent(enc, rh, enc_t, rh_t)
+        left = Bee.apply(*gather((a_t, v_t, d_t)), enc, phi_v, phi_d)
+        right = Bee.apply(*gather((a_node, v_node, d_node)), enc_t.contiguous(), phi_v_t.contiguous(), phi_d_t.contiguous())
+        prods = [a + b for a, b in zip(left, right)]
+        return tuple(p if lab[2] == "0" else gl._ScatterSum.apply(p.contiguous(), by_src) for lab, p in zip(BEE_ORDER, prods))
 
     @staticmethod
     def backward(ctx, *dys):
@@ -501,6 +572,14 @@ def _edge_filters_plain(enc, rh):
     return enc[..., None] * rh[..., None, :], enc[..., None, None] * rh[..., None, None, :] * rh[..., None, :, None]
 
 
+def _edge_filters_tangent(enc, rh, enc_t, rh_t):
+    """The derivative of _edge_filters_plain along (enc_t, rh_t): the product rule on its two and three factors."""
+    phi_v_t = enc_t[..., None] * rh[..., None, :] + enc[..., None] * rh_t[..., None, :]
+    rr = rh[..., None, None, :] * rh[..., None, :, None]
+    rr_t = rh_t[..., None, None, :] * rh[..., None, :, None] + rh[..., None, None, :] * rh_t[..., None, :, None]
+    return phi_v_t, enc_t[..., None, None] * rr + enc[..., None, None] * rr_t
+
+
 class _EdgeFilters(torch.autograd.Function):
     """phi_v = enc (x) rh and phi_d = enc (x) rh (x) rh as one kernel, and their adjoint as another; a recorded
     backward pass differentiates the broadcasting arithmetic instead."""
@@ -508,7 +587,12 @@ class _EdgeFilters(torch.autograd.Function):
     @staticmethod
     def forward(ctx, enc, rh):
         ctx.save_for_backward(enc, rh)
+        ctx.save_for_forward(enc, rh)
         return ops.bee_edge_filters_fwd(enc.contiguous(), rh.contiguous())
+
+    @staticmethod
+    def jvp(ctx, enc_t, rh_t):
+        return _edge_filters_tangent(*ctx.saved_tensors, enc_t, rh_t)
 
     @staticmethod
     def backward(ctx, g_v, g_d):

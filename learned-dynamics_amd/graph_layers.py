@@ -118,6 +118,10 @@ class _Gather(torch.autograd.Function):
         return ops.gather_rows(x.contiguous(), sidx.index)
 
     @staticmethod
+    def jvp(ctx, x_t, _):
+        return _Gather.apply(x_t, ctx.sidx)
+
+    @staticmethod
     def backward(ctx, dy):
         return _ScatterSum.apply(dy, ctx.sidx), None
 
@@ -131,6 +135,10 @@ class _ScatterSum(torch.autograd.Function):
         ctx.sidx = sidx
         # (an unsorted index: the rows are read in its sorted order through the permutation)
         return ops.segment_sum_csr(x_edge.contiguous(), sidx.row_ptr, sidx.n_rows, perm=sidx.perm)
+
+    @staticmethod
+    def jvp(ctx, x_t, _):
+        return _ScatterSum.apply(x_t, ctx.sidx)
 
     @staticmethod
     def backward(ctx, dy):

@@ -29,7 +29,7 @@ from .tensor_products import TensLinear
 def graph_setup(r0, box, pos, neighbours_max=64, celllist_max=32):
     """archs/meanflow_painn8.py:167-172; the edge vectors carry a gradient for pos when one is asked for."""
     graph, r_ij = _graph_setup(r0, box, pos.detach(), neighbours_max=neighbours_max, celllist_max=celllist_max)
-    if torch.is_grad_enabled() and pos.requires_grad:
+    if diff.differentiated(pos):
         r_ij = diff.edge_vectors(graph, pos, box)
     return graph, r_ij
 

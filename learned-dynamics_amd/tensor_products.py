@@ -35,7 +35,10 @@ class _TensorLinearFn(torch.autograd.Function):
             x_bound = _row_bound(inds, x)
         ctx.x_bound = x_bound
         ctx.has_bias = bias is not None
+        ctx.want_bound = want_bound
         ctx.save_for_backward(W, x)
+        ctx.save_for_forward(W, x)
+        ctx.set_materialize_grads(False)
         bias = None if bias is None else bias.contiguous()
         if not want_bound:
             return ops.tensor_linear_fwd(inds, W, x, bias=bias, row_bound=x_bound)
@@ -47,8 +50,26 @@ class _TensorLinearFn(torch.autograd.Function):
         return y, y_bound
 
     @staticmethod
+    def jvp(ctx, _inds, W_t, x_t, *rest):
+        """Forward-mode derivative: y_t = x_t W^T + x W_t^T + bias_t, each piece this same function, so that a
+        backward pass through the tangent runs on the same kernels.  (One tangent per argument that apply was given.)"""
+        W, x = ctx.saved_tensors
+        bias_t = rest[1] if len(rest) > 1 else None
+        parts = []
+        if x_t is not None:
+            parts.append(_TensorLinearFn.apply(ctx.inds, W, x_t))
+        if W_t is not None:
+            parts.append(_TensorLinearFn.apply(ctx.inds, W_t, x, ctx.x_bound))
+        if bias_t is not None:
+            parts.append(bias_t.expand_as(parts[0]) if parts else bias_t)
+        y_t = sum(parts[1:], parts[0]) if parts else None
+        return (y_t, None) if ctx.want_bound else y_t
+
+    @staticmethod
     def backward(ctx, dy, *_):
         W, x = ctx.saved_tensors
+        if dy is None:
+            return None, None, None, None, None, None
         dy = dy.contiguous()
         dW = dx = db = None
         dy_bound = _row_bound(ctx.inds, dy)
@@ -101,6 +122,7 @@ def tensor_linear(inds, W, x, bias=None, x_bound=None, want_bound=False):
     (SiLU, LeakyReLU) and save the next layer its pass over the rows."""
     if bias is not None and inds != 0:
         raise RuntimeError("a bias is defined for plain rows only")
+    x = x.contiguous()          # (here, where autograd records the copy: the function saves x for later derivatives)
     if not want_bound:
         return _TensorLinearFn.apply(inds, W, x, x_bound, bias)
     y, y_bound = _TensorLinearFn.apply(inds, W, x, x_bound, bias, True)
@@ -160,10 +182,21 @@ class _ProdBareFn(torch.autograd.Function):
     def forward(ctx, il, ir, io, x_l, x_r):
         ctx.inds = (il, ir, io)
         ctx.save_for_backward(x_l, x_r)
+        ctx.save_for_forward(x_l, x_r)
+        ctx.set_materialize_grads(False)
         return ops.tensor_prod_bare(il, ir, io, x_l.contiguous(), x_r.contiguous())
 
     @staticmethod
+    def jvp(ctx, _il, _ir, _io, l_t, r_t):
+        """Bilinear: the product with one operand's tangent in its place, summed over the operands that have one."""
+        x_l, x_r = ctx.saved_tensors
+        parts = [_ProdBareFn.apply(*ctx.inds, a, b) for a, b in ((l_t, x_r), (x_l, r_t)) if a is not None and b is not None]
+        return sum(parts[1:], parts[0])
+
+    @staticmethod
     def backward(ctx, dy):
+        if dy is None:
+            return None, None, None, None, None
         il, ir, io = ctx.inds
         k = (il + ir - io) // 2                       # contracted indices; il - k and ir - k are kept
         x_l, x_r = ctx.saved_tensors

@@ -175,9 +175,8 @@ def test_second_order_through_linear_products_gather_and_scatter(pkg):
         _close(Wd[k].grad, Wr[k].grad, f"d(jvp^2)/dW[{k}]", 1e-4)
 
 
-def test_meanflow_loss_through_the_painn_denoiser(pkg):
-    """v_target = v - (t - s) jvp, loss = mean (v_pred - v_target)^2, loss.backward(): the reference's training step
-    (archs/meanflow_painn8.py:274-296) on a small PaiNN meanflow denoiser with positions that move, against the oracle."""
+def _meanflow_case():
+    """A small PaiNN meanflow denoiser with positions that move, its float64 copy for the oracle, and one batch."""
     mp = importlib.import_module("learned-dynamics_amd.meanflow_painn")
     torch.manual_seed(0x947 + 9)
     B, N, n, r0, L = 1, 48, 8, 5.0, 30.0
@@ -198,21 +197,30 @@ def test_meanflow_loss_through_the_painn_denoiser(pkg):
     i = torch.arange(N - 1)
     bs, bd = torch.cat([i, i + 1]), torch.cat([i + 1, i])
     topo = mp.Topology(one_hot.cuda(), bs.cuda(), bd.cuda())
+    on_device = lambda st, x0, z: model(st, x0, z, box, topo)
+    oracle = lambda st, x0, z: OM.se3ito(sd, st, x0, z, box, one_hot.double(), bs, bd, r0, n, 1, 1, F64)
+    return model, sd, on_device, oracle, (x_prev, z_0, z_1, t, s)
 
-    def loss_of(dn, to):
-        z_t = to(t)[:, None, None] * to(z_1) + (1 - to(t)[:, None, None]) * to(z_0)
-        v = to(z_1) - to(z_0)
-        f = lambda zz, tt: dn((to(s), tt), to(x_prev), zz)
-        _, jvp = torch.autograd.functional.jvp(f, (z_t, to(t)), (v, torch.ones_like(to(t))), create_graph=True)
-        v_target = v - (to(t) - to(s))[:, None, None] * jvp
+
+def _meanflow_loss(dn, to, batch, jvp_of):
+    """archs/meanflow_painn8.py:283-296 up to the mean over the batch.  jvp_of(f, primals, tangents) -> (f(primals)
+    or None, jvp); when the first is None the model is evaluated again for v_pred, as the reference does."""
+    x_prev, z_0, z_1, t, s = batch
+    z_t = to(t)[:, None, None] * to(z_1) + (1 - to(t)[:, None, None]) * to(z_0)
+    v = to(z_1) - to(z_0)
+    f = lambda zz, tt: dn((to(s), tt), to(x_prev), zz)
+    v_pred, jvp = jvp_of(f, (z_t, to(t)), (v, torch.ones_like(to(t))))
+    v_target = v - (to(t) - to(s))[:, None, None] * jvp
+    if v_pred is None:
         v_pred = dn((to(s), to(t)), to(x_prev), z_t)
-        return ((v_pred - v_target) ** 2).mean(), jvp
+    return ((v_pred - v_target) ** 2).mean(), jvp
 
-    loss_d, jvp_d = loss_of(lambda st, x0, z: model(st, x0, z, box, topo), lambda a: a.cuda())
-    loss_d.backward()
-    loss_r, jvp_r = loss_of(lambda st, x0, z: OM.se3ito(sd, st, x0, z, box, one_hot.double(), bs, bd, r0, n, 1, 1, F64),
-                            lambda a: a.double())
-    loss_r.backward()
+
+def _nested_backward_jvp(f, primals, tangents):
+    return None, torch.autograd.functional.jvp(f, primals, tangents, create_graph=True)[1]
+
+
+def _check_meanflow_gradients(model, sd, loss_d, jvp_d, loss_r, jvp_r):
     _close(jvp_d, jvp_r, "jvp of the denoiser", 1e-4)
     assert abs(float(loss_d.detach()) - float(loss_r.detach())) <= 1e-4 * max(1.0, abs(float(loss_r.detach())))
     checked = 0
@@ -224,6 +232,96 @@ def test_meanflow_loss_through_the_painn_denoiser(pkg):
         _close(p.grad, ref, f"d loss / d {name}", 5e-4)
         checked += 1
     assert checked >= 40
+
+
+def test_meanflow_loss_through_the_painn_denoiser(pkg):
+    """v_target = v - (t - s) jvp, loss = mean (v_pred - v_target)^2, loss.backward(): the reference's training step
+    (archs/meanflow_painn8.py:274-296) on a small PaiNN meanflow denoiser with positions that move, against the oracle."""
+    model, sd, on_device, oracle, batch = _meanflow_case()
+    loss_d, jvp_d = _meanflow_loss(on_device, lambda a: a.cuda(), batch, _nested_backward_jvp)
+    loss_d.backward()
+    loss_r, jvp_r = _meanflow_loss(oracle, lambda a: a.double(), batch, _nested_backward_jvp)
+    loss_r.backward()
+    _check_meanflow_gradients(model, sd, loss_d, jvp_d, loss_r, jvp_r)
+
+
+def test_meanflow_loss_with_the_jvp_in_forward_mode(pkg):
+    """The same loss and gradients with the Jacobian-vector product taken in forward mode (differentiable.jvp: one
+    pass gives v_pred and the jvp) against the oracle, which keeps the reference's nested backward passes."""
+    diff = importlib.import_module("learned-dynamics_amd.differentiable")
+    model, sd, on_device, oracle, batch = _meanflow_case()
+    loss_d, jvp_d = _meanflow_loss(on_device, lambda a: a.cuda(), batch, diff.jvp)
+    assert jvp_d.grad_fn is not None
+    loss_d.backward()
+    loss_r, jvp_r = _meanflow_loss(oracle, lambda a: a.double(), batch, _nested_backward_jvp)
+    loss_r.backward()
+    _check_meanflow_gradients(model, sd, loss_d, jvp_d, loss_r, jvp_r)
+    # forward mode leaves nothing behind on the inputs or the parameters
+    assert all(not diff.has_tangent(p) for p in model.parameters())
+
+
+def test_forward_mode_rules_agree_with_nested_backward(pkg, ops):
+    """differentiable.jvp against torch.autograd.functional.jvp on each autograd function that has a forward-mode
+    rule (linear with and without bias and with emitted row bounds, SiLU, gather, segment sum, the PaiNN combine, the
+    13 products alone and with the edge filters and gathers folded in, one bare product),
+    and a backward pass through the tangent against one through the nested-backward result."""
+    diff = importlib.import_module("learned-dynamics_amd.differentiable")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    tp = importlib.import_module("learned-dynamics_amd.tensor_products")
+    g = torch.Generator().manual_seed(0x947 + 31)
+    rnd = lambda *shape: torch.randn(*shape, generator=g).cuda()
+    nodes, n = 40, 16
+    src = torch.sort(torch.randint(0, nodes, (300,), generator=g)).values
+    dst = torch.randint(0, nodes, (300,), generator=g)
+    graph = gl.Graph(src.cuda(), dst.cuda(), None, 1, nodes)
+    W, W1, b = rnd(24, n).requires_grad_(), rnd(8, n).requires_grad_(), rnd(24).requires_grad_()
+    torch.manual_seed(5)
+    lin, lin2 = torch.nn.Linear(n, 24).cuda(), torch.nn.Linear(24, 24).cuda()
+
+    def linear_chain(x, xv):
+        y, bound = diff.linear(lin, x, want_bound=True)
+        z = diff.linear(lin2, diff.silu(y), x_bound=bound)
+        return z.sum(-1, keepdim=True) * tp.tensor_linear(1, W1, xv)[..., 0, :] + tp.tensor_linear(0, W, x, bias=b)[:, :3]
+
+    def graph_ops(x):
+        x_src, x_dst = gl.edges_read(graph, x[None])
+        return gl.edges_reduce_src(graph, diff.silu(x_src) * x_dst)
+
+    def combine(dist, actv, v, r):
+        direction = r / torch.sqrt(0.01 + (r ** 2).sum(-1, keepdim=True))
+        out_v, out_a = diff.painn_combine(graph, dist, actv[None], v[None], direction)
+        return out_v.sum(-2) * out_a[..., :3]
+
+    bee = importlib.import_module("learned-dynamics_amd.bee_layers")
+    dims = (12, 8, 4)
+    msg, prod = bee.Messages(6.0, *dims, 16).cuda(), bee.SelfTensProds(*dims, 16, groups=2).cuda()
+    bare = tp.TensorProdBare(1, 2, 1)
+
+    def rank012_block(r, a, v, d):
+        B = msg(graph, r, a[None], v[None], d[None])
+        ya, yv, yd = prod(a[None] + B[0], v[None] + B[1], d[None] + B[2])
+        return ya.sum(-1)[..., None] + bare(yv.sum(-2, keepdim=True), yd.sum(-3, keepdim=True))[..., 0, :]
+
+    cases = [("linear chain", linear_chain, (rnd(50, n), rnd(50, n, 3)),
+              [W, W1, b] + list(lin.parameters()) + list(lin2.parameters())),
+             ("gather / segment sum", graph_ops, (rnd(nodes, 12),), []),
+             ("painn combine", combine, (rnd(300, 4 * n), rnd(nodes, 4 * n), rnd(nodes, n, 3), rnd(300, 3)), []),
+             ("Messages, SelfTensProds and one bare product", rank012_block,
+              (2.0 * rnd(300, 3), rnd(nodes, dims[0]), rnd(nodes, dims[1], 3), rnd(nodes, dims[2], 3, 3)),
+              list(msg.parameters()) + list(prod.parameters()))]
+    for name, f, primals, params in cases:
+        tangents = tuple(rnd(*p.shape) for p in primals)
+        leaves = [p.requires_grad_() for p in primals] + params
+        value, tangent = diff.jvp(f, primals, tangents)
+        grads = torch.autograd.grad((tangent ** 2).sum() + value.sum(), leaves, allow_unused=True)
+        value_n, tangent_n = torch.autograd.functional.jvp(f, primals, tangents, create_graph=True)
+        grads_n = torch.autograd.grad((tangent_n ** 2).sum() + value_n.sum(), leaves, allow_unused=True)
+        _close(value, value_n.double().cpu(), f"{name}: value", 1e-5)
+        _close(tangent, tangent_n.double().cpu(), f"{name}: tangent", 1e-4)
+        for k, (a, r) in enumerate(zip(grads, grads_n)):
+            assert (a is None) == (r is None), (name, k)
+            if a is not None:
+                _close(a, r.double().cpu(), f"{name}: gradient {k}", 1e-4)
 
 
 def test_weight_gradient_is_reproducible(ops):
