@@ -22,7 +22,9 @@ from .tensor_products import tensor_linear
 
 def has_tangent(t):
     """True for a tensor that carries a forward-mode tangent (inside jvp below)."""
-    return t is not None and fwAD.unpack_dual(t).tangent is not None
+    if t is None or getattr(fwAD, "_current_level", 0) < 0:       # (no dual level is open: nothing to unpack)
+        return False
+    return fwAD.unpack_dual(t).tangent is not None
 
 
 def differentiated(t):
