@@ -32,7 +32,7 @@ class TimeEmbedding(nn.Module):
     def raw_t_embed(self, st):
         s, t = st
         ang_freqs = torch.exp(-torch.arange(self.freqs, device=s.device) / (self.freqs - 1))
-        phases = torch.cat([t[:, None] * ang_freqs[None, :], (t - s)[:, None] * ang_freqs[None, :]], dim=1)
+        phases = torch.cat([diff.mul(t[:, None], ang_freqs[None, :]), diff.mul(diff.sub(t, s)[:, None], ang_freqs[None, :])], dim=1)
         return torch.cat([torch.sin(phases), torch.cos(phases)], dim=1)
 
     def forward(self, st):

@@ -44,6 +44,46 @@ def wants_grad(module, *tensors):
     return any(p.requires_grad for p in module.parameters())
 
 
+def _one_sided(a, b):
+    """(the operand with a tangent, the other, whether they were exchanged) when exactly one of a, b carries a
+    forward-mode tangent, else None."""
+    ta, tb = torch.is_tensor(a) and has_tangent(a), torch.is_tensor(b) and has_tangent(b)
+    if ta == tb:
+        return None
+    return (b, a, True) if tb else (a, b, False)
+
+
+def add(a, b):
+    """a + b.  When only one operand carries a forward-mode tangent the tangent passes through unchanged: torch's own
+    rule forms a symbolic zero for the other operand (a number or a parameter has none) and adds it through a slow
+    path (Python meta kernels, 0.15 ms of host time per call).  Outside forward mode this is a + b."""
+    one = _one_sided(a, b)
+    if one is None:
+        return a + b
+    p, t = fwAD.unpack_dual(one[0])
+    out = p + one[1]
+    return fwAD.make_dual(out, t if t.shape == out.shape else t.expand(out.shape))
+
+
+def sub(a, b):
+    """a - b, in forward mode as add."""
+    one = _one_sided(a, b)
+    if one is None:
+        return a - b
+    p, t = fwAD.unpack_dual(one[0])
+    out, t = (one[1] - p, -t) if one[2] else (p - one[1], t)
+    return fwAD.make_dual(out, t if t.shape == out.shape else t.expand(out.shape))
+
+
+def mul(a, b):
+    """a * b, in forward mode as add: the tangent is the one operand's tangent times the other operand."""
+    one = _one_sided(a, b)
+    if one is None:
+        return a * b
+    p, t = fwAD.unpack_dual(one[0])
+    return fwAD.make_dual(p * one[1], t * one[1])
+
+
 def jvp(f, primals, tangents):
     """(f(*primals), the derivative of f at primals along tangents) in forward mode: every autograd function of this
     package that a forward pass runs has a jvp rule made of the package's differentiable functions, so the pair costs
@@ -131,7 +171,7 @@ def radial_encode_painn(r, n, rmax):
     """archs/meanflow_painn8.py:25-35"""
     hn = (n + 1) // 2
     coeffs = (math.pi / rmax) * (1 + torch.arange(0, hn, device=r.device) // 2)
-    phase = coeffs * torch.linalg.vector_norm(r, dim=-1)[..., None]
+    phase = mul(torch.linalg.vector_norm(r, dim=-1)[..., None], coeffs)
     return torch.cat([torch.cos(phase), torch.sin(phase[..., :(n - hn)])], dim=-1)
 
 
@@ -166,7 +206,7 @@ def radial_encode_8(r, rmax):
 def tens_sigmoid(inds, x):
     dims = tuple(-(1 + n) for n in range(inds))
     xx = (x ** 2).sum(dims, keepdim=True) if inds > 0 else x ** 2
-    return x / torch.sqrt(1.0 + xx)
+    return x / torch.sqrt(add(xx, 1.0))
 
 
 def scal_group_norm(gn, x):
@@ -175,7 +215,7 @@ def scal_group_norm(gn, x):
     xg = x.reshape(B, N, gn.groups, -1)
     sh = xg - xg.mean([1, 3], keepdim=True)
     var = (sh ** 2).mean([1, 3], keepdim=True)
-    return gn.beta + gn.gamma * (sh / torch.sqrt(gn.epsilon + var)).reshape(B, N, chan)
+    return add(mul((sh / torch.sqrt(add(var, gn.epsilon))).reshape(B, N, chan), gn.gamma), gn.beta)
 
 
 def tens_group_norm(gn, x):
@@ -183,14 +223,19 @@ def tens_group_norm(gn, x):
     B, N, chan = x.shape[:3]
     xg = x.reshape(B, N, gn.groups, -1, 3 ** gn.inds)
     m2 = (xg ** 2).sum(-1, keepdim=True).mean([1, 3], keepdim=True)
-    return gn.gamma * (xg / torch.sqrt(gn.epsilon + m2)).reshape(x.shape)
+    return mul((xg / torch.sqrt(add(m2, gn.epsilon))).reshape(x.shape), gn.gamma)
 
 
 def edge_vectors(graph, pos, box):
     """boxwrap(box, pos[dst] - pos[src]) with a gradient for pos (archs/meanflow_painn8.py:167-172)."""
     pos_src, pos_dst = gl.edges_read(graph, pos)
     tbox = torch.tensor(box, device=pos.device, dtype=pos.dtype)
-    return gl.boxwrap(tbox, pos_dst - pos_src)
+    delta = pos_dst - pos_src
+    if has_tangent(delta):
+        # the wrap shifts by a locally constant multiple of the box: its Jacobian is the identity
+        p, t = fwAD.unpack_dual(delta)
+        return fwAD.make_dual(gl.boxwrap(tbox, p), t)
+    return gl.boxwrap(tbox, delta)
 
 
 def _painn_combine_plain(dist, actv, v, direction):
@@ -437,7 +482,7 @@ def painn_message(msg, graph, x_a, x_v, r_ij):
     dist = painn_filter(msg, r_ij)
     # the MLP acts on rows, so it commutes with the gather: N rows go through it, not E (the reference gathers first),
     # and the gathers themselves are folded into the combining kernel
-    direction = r_ij / torch.sqrt(msg.epsilon + (r_ij ** 2).sum(-1, keepdim=True))
+    direction = r_ij / torch.sqrt(add((r_ij ** 2).sum(-1, keepdim=True), msg.epsilon))
     out_v, out_a = painn_combine(graph, dist, mlp_silu(msg.mlp_actv, x_a), x_v, direction)
     return out_a, out_v
 
@@ -450,7 +495,7 @@ def painn_update(upd, x_a, x_v):
     y = mlp_silu(upd.mlp, torch.cat([x_a, torch.linalg.vector_norm(v_r, dim=-1)], dim=-1))
     v = upd.lin_v(x_v) * y[..., :n, None]
     a = scal_group_norm(upd.gn, ip * y[..., n:2 * n]) + y[..., 2 * n:]
-    return a, v / torch.sqrt(1. + (v ** 2).sum(-1, keepdim=True))
+    return a, v / torch.sqrt(add((v ** 2).sum(-1, keepdim=True), 1.))
 
 
 def apply_tens_prod_submodules(module, prods):

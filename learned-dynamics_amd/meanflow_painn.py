@@ -57,7 +57,7 @@ class CPaiNN(nn.Module):
         self.blocks = nn.Sequential(*[Block(r0, n, pos_mutable=mutate_pos) for _ in range(blks)])
 
     def forward(self, pos, graph_bond, r_ij_bond, x_a, x_v, box, topology):
-        x_a = x_a + self.atom_embed(topology)[None]
+        x_a = diff.add(x_a, self.atom_embed(topology)[None])
         pos, _, _, _, _, x_a, x_v, _ = self.blocks((pos, None, None, graph_bond, r_ij_bond, x_a, x_v, box))
         return pos, x_a, x_v
 
@@ -70,7 +70,7 @@ class PosEmbed(nn.Module):
         self.lin_v = TensLinear(1, 1, dim_v)
 
     def forward(self, pos_0, pos_1):
-        return self.lin_v((0.1 * (pos_1 - pos_0))[:, :, None].contiguous())
+        return self.lin_v(diff.mul(diff.sub(pos_1, pos_0), 0.1)[:, :, None].contiguous())
 
 
 class SE3ITO(nn.Module):
@@ -94,7 +94,8 @@ class SE3ITO(nn.Module):
 
     def get_v_pred(self, st, v_pred, x1_s_pred, x1_t):
         s, t = st
-        return (1. - (t - s)[:, None, None]) * v_pred + x1_t - x1_s_pred
+        span = diff.sub(1., diff.sub(t, s)[:, None, None])
+        return diff.sub(diff.add(diff.mul(span, v_pred), x1_t), x1_s_pred)
 
     def forward(self, st, x0, x1, box, topology: Topology):
         """st: ((batch), (batch)); x0, x1: (batch, atoms, 3)."""
@@ -106,10 +107,10 @@ class SE3ITO(nn.Module):
         r_ij_bond_0 = (x0.reshape(-1, 3)[graph_bond.dst] - x0.reshape(-1, 3)[graph_bond.src]).contiguous()
         r_ij_bond_1 = (x1.reshape(-1, 3)[graph_bond.dst] - x1.reshape(-1, 3)[graph_bond.src]).contiguous()
         x_a = self.atom_embeddings[None].expand(batch, -1, -1)
-        x_v = self.v_readin((x1 - x0)[..., None, :].contiguous())
+        x_v = self.v_readin(diff.sub(x1, x0)[..., None, :].contiguous())
         x_a = self.mlp_embed(x_a.contiguous())
         x0, x_a, x_v = self.cpainn_0(x0, graph_bond, r_ij_bond_0, x_a, x_v, box, topology)
-        x_a = self.mlp_denoise(x_a + self.t_embed(st)[:, None])
-        x_v = x_v + self.pos_emb(x0, x1)
+        x_a = self.mlp_denoise(diff.add(x_a, self.t_embed(st)[:, None]))
+        x_v = diff.add(x_v, self.pos_emb(x0, x1))
         x1, x_a, x_v = self.cpainn_1(x1, graph_bond, r_ij_bond_1, x_a, x_v, box, topology)
         return self.get_v_pred(st, self.readout(x_v).squeeze(-2), x1, x1_t)

@@ -131,7 +131,7 @@ class Update(nn.Module):
         """Returns (dx_a, dx_v), or (x_a + dx_a, x_v + dx_v) with residual=True."""
         if diff.wants_grad(self, x_a, x_v):
             da, dv = diff.painn_update(self, x_a, x_v)
-            return (x_a + da, x_v + dv) if residual else (da, dv)
+            return (diff.add(x_a, da), diff.add(x_v, dv)) if residual else (da, dv)
         n = self.n
         B, N = x_a.shape[:2]
         rows = B * N
@@ -331,7 +331,7 @@ class Message(nn.Module):
         Returns (dx_a, dx_v), or (x_a + dx_a, x_v + dx_v) with residual=True."""
         if diff.wants_grad(self, x_a, x_v, r_ij):
             da, dv = diff.painn_message(self, graph, x_a, x_v, r_ij)
-            return (x_a + da, x_v + dv) if residual else (da, dv)
+            return (diff.add(x_a, da), diff.add(x_v, dv)) if residual else (da, dv)
         B, N, n = x_a.shape
         flat_a = x_a.reshape(B * N, n).contiguous()
         flat_v = x_v.reshape(B * N, n, 3).contiguous()
@@ -406,6 +406,6 @@ class Block(nn.Module):
         x_a, x_v = self.message(graph, x_a, x_v, r_ij, residual=True)
         x_a, x_v = self.update(x_a, x_v, residual=True)
         if self.pos_mutable:
-            pos = pos + self.lin_push_pos(x_v).squeeze(-2)
+            pos = diff.add(pos, self.lin_push_pos(x_v).squeeze(-2))
             graph, r_ij = None, None
         return pos, graph, r_ij, graph_bond, r_ij_bond, x_a, x_v, box
