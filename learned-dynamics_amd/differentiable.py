@@ -453,12 +453,8 @@ def table_interp(table, d, period):
     return _TableInterp.apply(table, d, period, 0, _SortedLengths(d, table.size(0), period))
 
 
-def painn_filter(msg, r_ij):
-    """mlp_dist(radial_encode(r_ij)) (archs/meanflow_painn8.py:92), (edges, 4n).  The filter is a smooth periodic
-    function of the edge length: when the module's grid test accepts a grid for the current weights (the test the
-    inference path uses, Message.table_rows) the MLP runs on the grid's rows and every edge interpolates, so that the
-    backward pass differentiates the MLP on a few hundred rows instead of on every edge.  Only when the edge vectors
-    need no gradient (see below)."""
+def _filter_grid_rows(msg, r_ij):
+    """Rows of the grid the differentiable filter interpolates from, or 0 for the MLP on every edge."""
     E = r_ij.shape[0]
     rows = msg.table_rows() if (getattr(msg, "use_table", False) and E >= 4 * msg.TABLE_ROWS[0]) else 0
     if r_ij.requires_grad or has_tangent(r_ij):
@@ -469,21 +465,113 @@ def painn_filter(msg, r_ij):
         # A grid evaluated in float64 does not help (3e-5 at 2048 rows): the float32 differences themselves cancel
         # that many digits.  Positions that are differentiated (the meanflow loss, blocks that move them) keep the
         # per-edge MLP.
-        rows = 0
-    if rows and E >= 4 * rows and ops.painn_table_interp_supported(rows, 4 * msg.n):
+        return 0
+    return rows if rows and E >= 4 * rows and ops.painn_table_interp_supported(rows, 4 * msg.n) else 0
+
+
+def painn_filter(msg, r_ij):
+    """mlp_dist(radial_encode(r_ij)) (archs/meanflow_painn8.py:92), (edges, 4n).  The filter is a smooth periodic
+    function of the edge length: when the module's grid test accepts a grid for the current weights (the test the
+    inference path uses, Message.table_rows) the MLP runs on the grid's rows and every edge interpolates, so that the
+    backward pass differentiates the MLP on a few hundred rows instead of on every edge.  Only when the edge vectors
+    need no gradient (_filter_grid_rows)."""
+    rows = _filter_grid_rows(msg, r_ij)
+    if rows:
         table = mlp_silu(msg.mlp_dist, msg._grid_encoding(rows, 0.0, r_ij.device))
         d = torch.linalg.vector_norm(r_ij, dim=-1).contiguous()
         return table_interp(table, d, 2.0 * msg.r0)
     return mlp_silu(msg.mlp_dist, radial_encode_painn(r_ij, msg.n_rbf, msg.r0))
 
 
+def _unit_vectors(r_ij, epsilon):
+    return r_ij / torch.sqrt(add((r_ij ** 2).sum(-1, keepdim=True), epsilon))
+
+
+_SLICE_PERMUTATIONS = {}
+
+
+def _slice_permutation(n, device):
+    key = (n, str(device))
+    if key not in _SLICE_PERMUTATIONS:
+        _SLICE_PERMUTATIONS[key] = ops.painn_slice_permutation(n, device)
+    return _SLICE_PERMUTATIONS[key]
+
+
+class _PainnGridMessage(torch.autograd.Function):
+    """(grid (rows, 4n), actv (nodes, 4n), v (nodes, n, 3)) -> (out_v, out_a) of the message for edge vectors that are
+    not differentiated, with the filter interpolated from the grid.  Forward: the inference kernel of the layer
+    (mg_painn_table_message: lengths, directions, interpolation, the lines 94-100 of archs/meanflow_painn8.py and the
+    sum over the edges of a node in one pass; no per-edge filter is stored).  Backward: the filter of every edge is
+    interpolated again and the gradient kernels of the unfused formulation run (painn_combine_bwd, the segment sums,
+    the scatter into the grid).  A recorded backward pass differentiates the unfused formulation instead."""
+
+    @staticmethod
+    def forward(ctx, table, actv, v, r_ij, graph, period, epsilon):
+        ctx.graph, ctx.period, ctx.epsilon = graph, period, epsilon
+        table, actv, v = table.contiguous(), actv.contiguous(), v.contiguous()
+        ctx.save_for_backward(table, actv, v, r_ij)
+        n = v.size(1)
+        if table.size(0) <= ops.PAINN_SLICED_MAX_ROWS and n % ops.PAINN_SLICE == 0:
+            # the grid fits in LDS: the kernel that holds it there takes actv with its columns grouped slice by slice
+            actv_s = actv[:, _slice_permutation(n, actv.device)].contiguous()
+            out_a, out_v = ops.painn_table_message_sliced(graph.row_ptr, graph.dst32, r_ij, table, period, actv_s, v, epsilon,
+                                                          node_order=getattr(graph, "cell_order", None))
+        else:
+            out_a, out_v = ops.painn_table_message(graph.row_ptr, graph.dst32, r_ij, table, period, actv, v, epsilon)
+        return out_v, out_a
+
+    @staticmethod
+    def backward(ctx, g_v, g_a):
+        table, actv, v, r_ij = ctx.saved_tensors
+        graph, need = ctx.graph, ctx.needs_input_grad
+        if torch.is_grad_enabled():
+            with torch.enable_grad():
+                leaves = [t if t.requires_grad else t.detach().requires_grad_() for t in (table, actv, v)]
+                out = _grid_message_unfused(*leaves, r_ij, graph, ctx.period, ctx.epsilon)
+                grads = torch.autograd.grad(out, leaves, (g_v, g_a), create_graph=True, allow_unused=True)
+            return tuple(g if nd else None for g, nd in zip(grads, need)) + (None, None, None, None)
+        by_dst, by_src = graph.by_dst, graph.by_src
+        d = torch.linalg.vector_norm(r_ij, dim=-1).contiguous()
+        dist = ops.painn_table_interp_fwd(table, d, ctx.period, 0)
+        want = (bool(need[0]), bool(need[1]), bool(need[2]), False)
+        d_dist, d_actv, dv, _ = ops.painn_combine_bwd(dist, actv, v, _unit_vectors(r_ij, ctx.epsilon).contiguous(),
+                                                      g_v.contiguous(), g_a.contiguous(), node=by_dst.index,
+                                                      grad_row=by_src.index, terms=_TERMS_ALL, want=want)
+        d_table = None
+        if need[0]:
+            rows = table.size(0)
+            perm, bucket_ptr = ops.painn_table_sorted_edges(d, rows, ctx.period)
+            d_table = ops.painn_table_interp_bwd(d_dist, None, d, ctx.period, perm, bucket_ptr, want_length_grad=False,
+                                                 order=0, table_rows=rows)[0]
+        if need[1]:
+            d_actv = ops.segment_sum_csr(d_actv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm)
+        if need[2]:
+            dv = ops.segment_sum_csr(dv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm)
+        return (d_table, d_actv if need[1] else None, dv if need[2] else None, None, None, None, None)
+
+
+def _grid_message_unfused(table, actv, v, r_ij, graph, period, epsilon):
+    d = torch.linalg.vector_norm(r_ij, dim=-1).contiguous()
+    return _PainnCombine.apply(table_interp(table, d, period), actv, v, _unit_vectors(r_ij, epsilon).contiguous(),
+                               graph.by_dst, graph.by_src, _TERMS_ALL)
+
+
 def painn_message(msg, graph, x_a, x_v, r_ij):
     """archs/meanflow_painn8.py:85-100"""
-    dist = painn_filter(msg, r_ij)
     # the MLP acts on rows, so it commutes with the gather: N rows go through it, not E (the reference gathers first),
     # and the gathers themselves are folded into the combining kernel
-    direction = r_ij / torch.sqrt(add((r_ij ** 2).sum(-1, keepdim=True), msg.epsilon))
-    out_v, out_a = painn_combine(graph, dist, mlp_silu(msg.mlp_actv, x_a), x_v, direction)
+    actv = mlp_silu(msg.mlp_actv, x_a)
+    rows = _filter_grid_rows(msg, r_ij)
+    n = x_v.size(-2)
+    if (rows and n % 4 == 0 and ops.painn_combine_supported(n) and not any(has_tangent(t) for t in (x_a, x_v))
+            and r_ij.is_contiguous() and not getattr(graph, "padded", False)):
+        table = mlp_silu(msg.mlp_dist, msg._grid_encoding(rows, 0.0, r_ij.device))
+        out_v, out_a = _PainnGridMessage.apply(table, gl._flat_nodes(graph, actv), gl._flat_nodes(graph, x_v), r_ij, graph,
+                                               2.0 * msg.r0, msg.epsilon)
+        return (out_a.reshape(graph.batch, graph.nodes, *out_a.shape[1:]),
+                out_v.reshape(graph.batch, graph.nodes, *out_v.shape[1:]))
+    dist = painn_filter(msg, r_ij)
+    out_v, out_a = painn_combine(graph, dist, actv, x_v, _unit_vectors(r_ij, msg.epsilon))
     return out_a, out_v
 
 

@@ -518,6 +518,73 @@ def test_painn_filter_from_its_grid(pkg):
     assert all(t is None or bool(torch.isfinite(t).all()) for t in second)
 
 
+def test_painn_message_through_its_grid_in_one_forward_kernel(pkg):
+    """Message under autograd with edge vectors that are not differentiated: the forward pass is the inference kernel
+    on the grid (differentiable._PainnGridMessage) and the backward pass interpolates the filter again.  Values and
+    every gradient against the unfused formulation (interpolated filter stored, painn_combine), the recorded backward
+    pass and a second-order gradient likewise; the unfused formulation has its own tests against float64."""
+    diff = importlib.import_module("learned-dynamics_amd.differentiable")
+    painn = importlib.import_module("learned-dynamics_amd.painn")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    torch.manual_seed(0x947 + 41)
+    n, N = 32, 400
+    msg = painn.Message(5.0, n, n_rbf=16).cuda()
+    g = torch.Generator().manual_seed(5)
+    src, dst = _ring(N, 16, g)
+    E = len(src)
+    u = torch.randn(E, 3, generator=g)
+    r_ij = (u / u.norm(dim=-1, keepdim=True) * (0.4 + 4.6 * torch.rand(E, 1, generator=g))).cuda()
+    graph = gl.Graph(src.cuda(), dst.cuda(), None, 1, N)
+    x_a = torch.randn(1, N, n, generator=g).cuda().requires_grad_()
+    x_v = torch.randn(1, N, n, 3, generator=g).cuda().requires_grad_()
+    c_a, c_v = torch.randn(1, N, n, generator=g).cuda(), torch.randn(1, N, n, 3, generator=g).cuda()
+    params = list(msg.parameters())
+    assert msg.table_rows() == 512 and E >= 4 * 512
+
+    def unfused():
+        dist = diff.painn_filter(msg, r_ij)
+        out_v, out_a = diff.painn_combine(graph, dist, diff.mlp_silu(msg.mlp_actv, x_a), x_v,
+                                          diff._unit_vectors(r_ij, msg.epsilon))
+        return out_a, out_v
+
+    ops = importlib.import_module("learned-dynamics_amd.ops")
+    calls, kernels = [], (ops.painn_table_message, ops.painn_table_message_sliced)
+    ops.painn_table_message = lambda *a, **k: (calls.append("caches"), kernels[0](*a, **k))[1]
+    ops.painn_table_message_sliced = lambda *a, **k: (calls.append("lds"), kernels[1](*a, **k))[1]
+    try:
+        da, dv = msg(graph, x_a, x_v, r_ij)
+    finally:
+        ops.painn_table_message, ops.painn_table_message_sliced = kernels
+    assert calls == ["lds"]                              # the forward pass was the inference kernel (grid in LDS)
+    ra, rv = unfused()
+    _close(da, ra.double().cpu(), "out_a"); _close(dv, rv.double().cpu(), "out_v")
+    leaves = [x_a, x_v] + params
+    loss = lambda a, v: (a * c_a).sum() + (v * c_v).sum()
+    got = torch.autograd.grad(loss(da, dv), leaves, allow_unused=True)
+    ref = torch.autograd.grad(loss(ra, rv), leaves, allow_unused=True)
+    for k, (a, r) in enumerate(zip(got, ref)):
+        assert (a is None) == (r is None), k
+        if a is not None:
+            _close(a, r.double().cpu(), f"gradient {k}", 3e-5)
+    # the recorded backward pass and a gradient of its result
+    da, dv = msg(graph, x_a, x_v, r_ij)
+    ra, rv = unfused()
+    g1 = torch.autograd.grad(loss(da, dv), [x_a, x_v], create_graph=True)
+    r1 = torch.autograd.grad(loss(ra, rv), [x_a, x_v], create_graph=True)
+    second = lambda gs: sum((t ** 2).sum() for t in gs)
+    got2 = torch.autograd.grad(second(g1), leaves, allow_unused=True)
+    ref2 = torch.autograd.grad(second(r1), leaves, allow_unused=True)
+    for k, (a, r) in enumerate(zip(got2, ref2)):
+        assert (a is None) == (r is None), k
+        if a is not None:
+            _close(a, r.double().cpu(), f"second-order gradient {k}", 1e-4)
+    # inputs with a forward-mode tangent take the unfused formulation
+    value, tangent = diff.jvp(lambda a, v: msg(graph, a, v, r_ij)[0], (x_a.detach(), x_v.detach()),
+                              (torch.randn_like(x_a), torch.randn_like(x_v)))
+    _close(value, ra.double().cpu(), "value in forward mode")
+    assert bool(torch.isfinite(tangent).all())
+
+
 def test_message_products_with_folded_gathers(pkg):
     """The 13 products of Messages with the node operands read through the destination index and the gradients of the
     summed products through the source index (chan = 256, the width the folded kernels take), against the plain
