@@ -449,6 +449,14 @@ int mg_painn_combine_fwd(const float* dist, const float* actv, const float* v, c
 int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
                          long n_rows, const float* dm, const float* da, const int* grad_row, long n_grad_rows, long E,
                          int n, int terms, float* d_dist, float* d_actv, float* dv, float* d_dir, mg_stream_t stream);
+/* mg_painn_combine_bwd with dist given by its grid: table (table_rows, 4n) is the filter at d = k period / table_rows
+ * and edge e takes the 4-point Lagrange interpolation at len[e] (mg_painn_table_interp_fwd's arithmetic), so the
+ * (E, 4n) filter is not stored between the forward and the backward pass (the forward pass being
+ * mg_painn_table_message).  d_dist is still per edge, (E, 4n): mg_painn_table_interp_bwd sums it into the grid. */
+int mg_painn_combine_bwd_grid(const float* table, int table_rows, float period, const float* len /* (E) */,
+                              const float* actv, const float* v, const float* dir, const int* node, long n_rows,
+                              const float* dm, const float* da, const int* grad_row, long n_grad_rows, long E, int n,
+                              int terms, float* d_dist, float* d_actv, float* dv, float* d_dir, mg_stream_t stream);
 
 /* The filter from its grid, for training (the grid itself: mg_painn_table_message above).  table (table_rows, cols):
  * the filter at d = k period / table_rows; table_rows and cols powers of two, cols <= 1024.

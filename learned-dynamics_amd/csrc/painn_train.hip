@@ -86,11 +86,27 @@ __global__ void __launch_bounds__(256) painn_combine_fwd_kernel(const float* __r
 //   dp[c] = dm[c] . v[c],  dp[n + c] = dm[c] . (v[c] x d),  dp[2n + c] = dm[c] . d,  dp[3n + c] = da[c]
 //   d_dist = dp actv,  d_actv = dp dist,  dv[c] = dm[c] p[c] + (d x dm[c]) p[n + c]
 //   d_dir = sum_c (dm[c] x v[c]) p[n + c] + dm[c] p[2n + c]
+// 4-point Lagrange weights on the grid rows i - 1 .. i + 2 at the fraction t (the grid kernels further down use them too)
+__device__ __forceinline__ void lagrange4(float t, float (&w)[4]) {
+    const float tp = t + 1.0f, tm = t - 1.0f, tq = t - 2.0f;
+    w[0] = -(1.0f / 6.0f) * t * tm * tq;
+    w[1] = 0.5f * tp * tm * tq;
+    w[2] = -0.5f * tp * t * tq;
+    w[3] = (1.0f / 6.0f) * tp * t * tm;
+}
+__device__ __forceinline__ float4 fma4(float w, float4 a, float4 acc) {
+    return make_float4(fmaf(w, a.x, acc.x), fmaf(w, a.y, acc.y), fmaf(w, a.z, acc.z), fmaf(w, a.w, acc.w));
+}
+
+// GRID: dist is a (mask + 1, 4n) grid of the filter over one period of the edge length and edge e interpolates its row
+// at len[e] (the arithmetic of table_interp_kernel, order 0): the per-edge filter is never stored.
+template <bool GRID>
 __global__ void __launch_bounds__(256) painn_combine_bwd_kernel(
     const float* __restrict__ dist, const float* __restrict__ actv, const float* __restrict__ v,
     const float* __restrict__ dir, const int* __restrict__ node, long n_rows, const float* __restrict__ dm,
     const float* __restrict__ da, const int* __restrict__ grad_row, long n_grad_rows, long E, int n, int terms,
-    float* __restrict__ d_dist, float* __restrict__ d_actv, float* __restrict__ dv, float* __restrict__ d_dir) {
+    float* __restrict__ d_dist, float* __restrict__ d_actv, float* __restrict__ dv, float* __restrict__ d_dir,
+    const float* __restrict__ len, int mask, float inv_h) {
     const int tpe = n >> 2;                                       // a power of two <= 64
     const long t = (long)blockIdx.x * 256 + threadIdx.x;
     const long e_raw = t / tpe;
@@ -99,11 +115,28 @@ __global__ void __launch_bounds__(256) painn_combine_bwd_kernel(
     const int c = (int)(t - e_raw * tpe) * 4;
     // row of actv and v that this edge reads (an index outside the rows is clamped: never an access out of bounds)
     const long en = node ? min(max((long)node[e], 0L), n_rows - 1) : e;
-    const float* de = dist + e * 4 * n + c;
     const float* ae = actv + en * 4 * n + c;
     float4 dk[4], ak[4];
 #pragma unroll
-    for (int k = 0; k < 4; k++) { dk[k] = ld4(de + k * n); ak[k] = ld4(ae + k * n); }
+    for (int k = 0; k < 4; k++) ak[k] = ld4(ae + k * n);
+    if constexpr (GRID) {
+        const float u = len[e] * inv_h, fl = floorf(u);
+        float w[4];
+        lagrange4(u - fl, w);
+        const int i = (int)fl;
+#pragma unroll
+        for (int k = 0; k < 4; k++) dk[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const float* row = dist + (long)((i - 1 + j) & mask) * 4 * n + c;
+#pragma unroll
+            for (int k = 0; k < 4; k++) dk[k] = fma4(w[j], ld4(row + k * n), dk[k]);
+        }
+    } else {
+        const float* de = dist + e * 4 * n + c;
+#pragma unroll
+        for (int k = 0; k < 4; k++) dk[k] = ld4(de + k * n);
+    }
     // row of dm and da: the edge itself, or (the outputs were summed over the edges of a source node) that node
     const long eg = grad_row ? min(max((long)grad_row[e], 0L), n_grad_rows - 1) : e;
     const Vec3x4 vv = ld12(v + (en * n + c) * 3), g = ld12(dm + (eg * n + c) * 3);
@@ -164,13 +197,6 @@ __global__ void __launch_bounds__(256) painn_combine_bwd_kernel(
 // grid row (perm, bucket_ptr from the host side), each grid row's edges are cut into `splits` consecutive pieces,
 // a workgroup sums one piece (its thread groups take the piece's edges round robin, each in order, and are added in
 // group order), and the pieces and the four taps are added in a fixed order by a second kernel.
-__device__ __forceinline__ void lagrange4(float t, float (&w)[4]) {
-    const float tp = t + 1.0f, tm = t - 1.0f, tq = t - 2.0f;
-    w[0] = -(1.0f / 6.0f) * t * tm * tq;
-    w[1] = 0.5f * tp * tm * tq;
-    w[2] = -0.5f * tp * t * tq;
-    w[3] = (1.0f / 6.0f) * tp * t * tm;
-}
 __device__ __forceinline__ void lagrange4_derivative(float t, float (&w)[4]) {
     const float tp = t + 1.0f, tm = t - 1.0f, tq = t - 2.0f;
     w[0] = -(1.0f / 6.0f) * (tm * tq + t * tq + t * tm);
@@ -187,9 +213,6 @@ __device__ __forceinline__ void lagrange4_order(float t, int order, float (&w)[4
         return;
     }
     w[0] = -1.0f; w[1] = 3.0f; w[2] = -3.0f; w[3] = 1.0f;
-}
-__device__ __forceinline__ float4 fma4(float w, float4 a, float4 acc) {
-    return make_float4(fmaf(w, a.x, acc.x), fmaf(w, a.y, acc.y), fmaf(w, a.z, acc.z), fmaf(w, a.w, acc.w));
 }
 
 // bucket[e] = i_e & mask, the grid row an edge is sorted by (computed here so that it is the kernels' own i_e)
@@ -480,10 +503,34 @@ int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, c
                "mg_painn_combine_bwd: arrays must be 16-byte aligned");     // (a null pointer counts as aligned)
     const long threads = E * (n / 4);
     MG_REQUIRE(ceil_div(threads, 256) < (1L << 31), "mg_painn_combine_bwd: too many edges");
-    hipLaunchKernelGGL(painn_combine_bwd_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
+    hipLaunchKernelGGL(painn_combine_bwd_kernel<false>, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
                        (hipStream_t)stream, dist, actv, v, dir, node, n_rows, dm, da, grad_row, n_grad_rows, E, n, terms, d_dist,
-                       d_actv, dv, d_dir);
+                       d_actv, dv, d_dir, nullptr, 0, 0.f);
     return check_launch("mg_painn_combine_bwd");
+}
+
+int mg_painn_combine_bwd_grid(const float* table, int table_rows, float period, const float* len, const float* actv,
+                              const float* v, const float* dir, const int* node, long n_rows, const float* dm,
+                              const float* da, const int* grad_row, long n_grad_rows, long E, int n, int terms,
+                              float* d_dist, float* d_actv, float* dv, float* d_dir, mg_stream_t stream) {
+    MG_REQUIRE(E >= 0 && combine_shape_ok(n), "mg_painn_combine_bwd_grid: n must be a power of two in 4..256");
+    MG_REQUIRE(table_shape_ok(table_rows, 4 * n) && period > 0.f,
+               "mg_painn_combine_bwd_grid: grid rows must be a power of two, period positive");
+    MG_REQUIRE(terms >= 0 && terms <= 15, "mg_painn_combine_bwd_grid: terms is a mask of four bits");
+    if (E == 0) return MG_OK;
+    MG_REQUIRE(table && len && actv && v && dir && dm && da, "mg_painn_combine_bwd_grid: null pointer");
+    if (!d_dist && !d_actv && !dv && !d_dir) return MG_OK;       // (any of the four outputs may be left out)
+    MG_REQUIRE((node == nullptr || n_rows > 0) && (grad_row == nullptr || n_grad_rows > 0),
+               "mg_painn_combine_bwd_grid: an index needs a positive row count");
+    MG_REQUIRE(aligned16(table) && aligned16(actv) && aligned16(v) && aligned16(dm) && aligned16(da) &&
+                   aligned16(d_dist) && aligned16(d_actv) && aligned16(dv),
+               "mg_painn_combine_bwd_grid: arrays must be 16-byte aligned");
+    const long threads = E * (n / 4);
+    MG_REQUIRE(ceil_div(threads, 256) < (1L << 31), "mg_painn_combine_bwd_grid: too many edges");
+    hipLaunchKernelGGL(painn_combine_bwd_kernel<true>, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
+                       (hipStream_t)stream, table, actv, v, dir, node, n_rows, dm, da, grad_row, n_grad_rows, E, n, terms,
+                       d_dist, d_actv, dv, d_dir, len, table_rows - 1, (float)table_rows / period);
+    return check_launch("mg_painn_combine_bwd_grid");
 }
 
 int mg_painn_table_interp_supported(int table_rows, int cols) { return table_shape_ok(table_rows, cols) ? 1 : 0; }

@@ -501,9 +501,9 @@ class _PainnGridMessage(torch.autograd.Function):
     """(grid (rows, 4n), actv (nodes, 4n), v (nodes, n, 3)) -> (out_v, out_a) of the message for edge vectors that are
     not differentiated, with the filter interpolated from the grid.  Forward: the inference kernel of the layer
     (mg_painn_table_message: lengths, directions, interpolation, the lines 94-100 of archs/meanflow_painn8.py and the
-    sum over the edges of a node in one pass; no per-edge filter is stored).  Backward: the filter of every edge is
-    interpolated again and the gradient kernels of the unfused formulation run (painn_combine_bwd, the segment sums,
-    the scatter into the grid).  A recorded backward pass differentiates the unfused formulation instead."""
+    sum over the edges of a node in one pass; no per-edge filter is stored).  Backward: the gradient kernel of the
+    unfused formulation with the filter of every edge interpolated again inside it (mg_painn_combine_bwd_grid), the
+    segment sums, the scatter into the grid.  A recorded backward pass differentiates the unfused formulation instead."""
 
     @staticmethod
     def forward(ctx, table, actv, v, r_ij, graph, period, epsilon):
@@ -532,11 +532,11 @@ class _PainnGridMessage(torch.autograd.Function):
             return tuple(g if nd else None for g, nd in zip(grads, need)) + (None, None, None, None)
         by_dst, by_src = graph.by_dst, graph.by_src
         d = torch.linalg.vector_norm(r_ij, dim=-1).contiguous()
-        dist = ops.painn_table_interp_fwd(table, d, ctx.period, 0)
         want = (bool(need[0]), bool(need[1]), bool(need[2]), False)
-        d_dist, d_actv, dv, _ = ops.painn_combine_bwd(dist, actv, v, _unit_vectors(r_ij, ctx.epsilon).contiguous(),
-                                                      g_v.contiguous(), g_a.contiguous(), node=by_dst.index,
-                                                      grad_row=by_src.index, terms=_TERMS_ALL, want=want)
+        d_dist, d_actv, dv, _ = ops.painn_combine_bwd_grid(table, ctx.period, d, actv, v,
+                                                           _unit_vectors(r_ij, ctx.epsilon).contiguous(), g_v.contiguous(),
+                                                           g_a.contiguous(), by_dst.index, by_src.index, terms=_TERMS_ALL,
+                                                           want=want)
         d_table = None
         if need[0]:
             rows = table.size(0)

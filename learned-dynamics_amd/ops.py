@@ -1672,6 +1672,34 @@ def painn_combine_bwd(dist, actv, v, direction, dm, da, node=None, grad_row=None
     return d_dist, d_actv, dv, d_dir
 
 
+def painn_combine_bwd_grid(table, period, d, actv, v, direction, dm, da, node, grad_row, terms=15,
+                           want=(True, True, True, True)):
+    """painn_combine_bwd with the filter of edge e interpolated from `table` (rows, 4n) at the length d[e] inside the
+    kernel (the backward pass of a message whose forward pass was painn_table_message: no (E, 4n) filter is kept).
+    actv (nodes, 4n) and v (nodes, n, 3) are read at node[e], dm and da at grad_row[e]."""
+    for t, name in ((table, "table"), (d, "d"), (actv, "actv"), (v, "v"), (direction, "direction"), (dm, "dm"), (da, "da")):
+        _check_input(t, name)
+    _check_input(node, "node", torch.int32)
+    _check_input(grad_row, "grad_row", torch.int32)
+    E, n, rows = int(d.numel()), int(v.size(1)), int(v.size(0))
+    if tuple(table.shape[1:]) != (4 * n,) or tuple(actv.shape) != (rows, 4 * n) or tuple(v.shape) != (rows, n, 3):
+        raise RuntimeError("expected table (grid rows, 4n), actv (rows, 4n), v (rows, n, 3)")
+    if tuple(direction.shape) != (E, 3) or node.numel() != E or grad_row.numel() != E:
+        raise RuntimeError("expected direction (edges, 3) and one index entry per edge")
+    g_rows = int(dm.size(0))
+    if tuple(dm.shape) != (g_rows, n, 3) or tuple(da.shape) != (g_rows, n):
+        raise RuntimeError("expected dm (rows, n, 3) and da (rows, n)")
+    with torch.cuda.device(v.device):
+        d_dist = torch.empty(E, 4 * n, dtype=torch.float32, device=v.device) if want[0] else None
+        d_actv = torch.empty(E, 4 * n, dtype=torch.float32, device=v.device) if want[1] else None
+        dv = torch.empty(E, n, 3, dtype=torch.float32, device=v.device) if want[2] else None
+        d_dir = torch.empty_like(direction) if want[3] else None
+        L.check(_lib.mg_painn_combine_bwd_grid(_p(table), int(table.size(0)), float(period), _p(d), _p(actv), _p(v),
+                                               _p(direction), _p(node), rows, _p(dm), _p(da), _p(grad_row), g_rows, E, n,
+                                               int(terms), _p(d_dist), _p(d_actv), _p(dv), _p(d_dir), _stream()))
+    return d_dist, d_actv, dv, d_dir
+
+
 def painn_table_interp_supported(table_rows, cols):
     return bool(_lib.mg_painn_table_interp_supported(int(table_rows), int(cols)))
 

@@ -518,6 +518,32 @@ def test_painn_filter_from_its_grid(pkg):
     assert all(t is None or bool(torch.isfinite(t).all()) for t in second)
 
 
+@pytest.mark.parametrize("n, rows", [(32, 512), (128, 512), (8, 2048)])
+def test_combine_gradient_with_the_filter_interpolated_inside(ops, n, rows):
+    """mg_painn_combine_bwd_grid against mg_painn_table_interp_fwd followed by mg_painn_combine_bwd on a smooth grid
+    (the two kernels may round the position inside a grid cell differently, by an ulp of length x rows / period: the
+    compiler is free to contract the subtraction of the floor into the product), with outputs left out as well."""
+    g = torch.Generator().manual_seed(0x947 + 43 + n)
+    E, nodes, period = 3000, 200, 10.0
+    phase = 2 * torch.pi * torch.arange(rows)[:, None] / rows
+    table = (torch.sin(phase * torch.randint(1, 4, (1, 4 * n), generator=g) + torch.rand(1, 4 * n, generator=g))
+             * torch.randn(1, 4 * n, generator=g)).cuda()
+    d = (torch.rand(E, generator=g) * period * 0.999).cuda()
+    actv, v = torch.randn(nodes, 4 * n, generator=g).cuda(), torch.randn(nodes, n, 3, generator=g).cuda()
+    direction = torch.nn.functional.normalize(torch.randn(E, 3, generator=g), dim=-1).cuda()
+    dm, da = torch.randn(nodes, n, 3, generator=g).cuda(), torch.randn(nodes, n, generator=g).cuda()
+    node = torch.randint(0, nodes, (E,), generator=g).int().cuda()
+    grad_row = torch.randint(0, nodes, (E,), generator=g).int().cuda()
+    dist = ops.painn_table_interp_fwd(table, d, period, 0)
+    for want in ((True, True, True, True), (True, False, True, False), (False, True, False, False)):
+        ref = ops.painn_combine_bwd(dist, actv, v, direction, dm, da, node=node, grad_row=grad_row, want=want)
+        got = ops.painn_combine_bwd_grid(table, period, d, actv, v, direction, dm, da, node, grad_row, want=want)
+        for k in range(4):
+            assert (got[k] is None) == (not want[k]) and (ref[k] is None) == (not want[k])
+            if want[k]:
+                _close(got[k], ref[k].double().cpu(), f"gradient {k} with outputs {want}", 2e-6)
+
+
 def test_painn_message_through_its_grid_in_one_forward_kernel(pkg):
     """Message under autograd with edge vectors that are not differentiated: the forward pass is the inference kernel
     on the grid (differentiable._PainnGridMessage) and the backward pass interpolates the filter again.  Values and
