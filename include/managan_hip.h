@@ -458,6 +458,19 @@ int mg_painn_combine_bwd_grid(const float* table, int table_rows, float period, 
                               const float* dm, const float* da, const int* grad_row, long n_grad_rows, long E, int n,
                               int terms, float* d_dist, float* d_actv, float* dv, float* d_dir, mg_stream_t stream);
 
+/* The same gradients with those of actv and v summed inside the kernel, for actv (n_rows, 4n) and v (n_rows, n, 3) read
+ * by every edge at one row (its destination): row r is read by the edges order[row_ptr[r]] .. order[row_ptr[r + 1] - 1]
+ * (order NULL: by the edge positions themselves, edges sorted by that row), the caller's CSR of the index that
+ * mg_painn_combine_bwd takes as `node`.  d_actv (n_rows, 4n) and dv (n_rows, n, 3) come out per row, summed in the
+ * order of `order` (the same on every run); d_dist (E, 4n) and d_dir (E, 3) stay per edge; any of the four may be NULL.
+ * The filter is dist (E, 4n), or (dist NULL) table (table_rows, 4n) interpolated at len[e] as in
+ * mg_painn_combine_bwd_grid.  Replaces mg_painn_combine_bwd followed by two segment sums over (E, 4n) and (E, n, 3). */
+int mg_painn_combine_bwd_rows(const float* dist, const float* table, int table_rows, float period, const float* len,
+                              const float* actv, const float* v, const float* dir, const int* row_ptr, const int* order,
+                              long n_rows, const float* dm, const float* da, const int* grad_row, long n_grad_rows,
+                              long E, int n, int terms, float* d_dist, float* d_actv, float* dv, float* d_dir,
+                              mg_stream_t stream);
+
 /* The filter from its grid, for training (the grid itself: mg_painn_table_message above).  table (table_rows, cols):
  * the filter at d = k period / table_rows; table_rows and cols powers of two, cols <= 1024.
  *   mg_painn_table_interp_fwd:  out[e, :] = the 4-point Lagrange interpolation of the grid at d[e] (as the inference kernels do).

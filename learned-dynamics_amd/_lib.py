@@ -116,6 +116,8 @@ _SIGNATURES = {
     "mg_painn_table_interp_bwd": [vp, vp, i32, i32, f32, vp, vp, vp, i64, i32, vp, vp, vp, vp],
     "mg_painn_combine_fwd": [vp, vp, vp, vp, vp, i64, i64, i32, i32, vp, vp, vp],
     "mg_painn_combine_bwd": [vp, vp, vp, vp, vp, i64, vp, vp, vp, i64, i64, i32, i32, vp, vp, vp, vp, vp],
+    "mg_painn_combine_bwd_rows": [vp, vp, i32, f32, vp, vp, vp, vp, vp, vp, i64, vp, vp, vp, i64, i64, i32, i32, vp, vp, vp,
+                                  vp, vp],
     "mg_painn_combine_bwd_grid": [vp, i32, f32, vp, vp, vp, vp, vp, i64, vp, vp, vp, i64, i64, i32, i32, vp, vp, vp, vp, vp],
     "mg_painn_message": [vp, vp, vp, i32, i64, vp, vp, vp, vp, i32, f32, vp, vp, vp, vp, vp],
     "mg_tensor_linear_bf16_rowsum_workspace_bytes": [i64, i32, ctypes.POINTER(ctypes.c_size_t)],

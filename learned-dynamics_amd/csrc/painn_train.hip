@@ -185,6 +185,116 @@ __global__ void __launch_bounds__(256) painn_combine_bwd_kernel(
     if (d_dir && c == 0) { d_dir[3 * e] = gd.x; d_dir[3 * e + 1] = gd.y; d_dir[3 * e + 2] = gd.z; }
 }
 
+// The same adjoint with the gradients of actv and v summed inside the kernel.  actv and v hold one row per node and
+// every edge reads the row of its destination; a group of n / 4 threads owns one such row r and walks the edges that
+// read it (edge ids order[row_ptr[r]] .. order[row_ptr[r + 1] - 1], or the positions themselves when order is null:
+// edges sorted by that row), keeps the row's actv and v in registers, adds the edges' contributions to d_actv[r] and
+// dv[r] in that order (the same on every run) and writes them once: no per-edge copies of the two gradients and no
+// segment sums after the kernel.  d_dist and d_dir stay per edge.  GRID as above.
+template <bool GRID>
+__global__ void __launch_bounds__(256) painn_combine_bwd_rows_kernel(
+    const float* __restrict__ dist, const float* __restrict__ actv, const float* __restrict__ v,
+    const float* __restrict__ dir, const int* __restrict__ row_ptr, const int* __restrict__ order, long n_rows,
+    const float* __restrict__ dm, const float* __restrict__ da, const int* __restrict__ grad_row, long n_grad_rows,
+    long E, int n, int terms, float* __restrict__ d_dist, float* __restrict__ d_actv, float* __restrict__ dv,
+    float* __restrict__ d_dir, const float* __restrict__ len, int mask, float inv_h) {
+    const int tpe = n >> 2;                                       // a power of two <= 64: a group never straddles waves
+    const long t = (long)blockIdx.x * 256 + threadIdx.x;
+    const long r_raw = t / tpe;
+    const bool live = r_raw < n_rows;
+    const long r = live ? r_raw : n_rows - 1;
+    const int c = (int)(t - r_raw * tpe) * 4;
+    const float* ae = actv + r * 4 * n + c;
+    float4 ak[4], acc_a[4];
+#pragma unroll
+    for (int k = 0; k < 4; k++) { ak[k] = ld4(ae + k * n); acc_a[k] = make_float4(0.f, 0.f, 0.f, 0.f); }
+    const Vec3x4 vv = ld12(v + (r * n + c) * 3);
+    Vec3x4 acc_v;
+#pragma unroll
+    for (int q = 0; q < 12; q++) acc_v.f[q] = 0.f;
+    const float k0 = (terms & 1) ? 1.f : 0.f, k1 = (terms & 2) ? 1.f : 0.f, k2 = (terms & 4) ? 1.f : 0.f;
+    const float k3 = (terms & 8) ? 1.f : 0.f;
+    // (the threads of a group share r, so they make the same trips and the shuffles below stay inside live lanes)
+    const int lo = max(row_ptr[r], 0), hi = live ? min(row_ptr[r + 1], (int)min(E, 0x7fffffffL)) : lo;
+    for (int pos = lo; pos < hi; pos++) {
+        long e = order ? (long)order[pos] : (long)pos;
+        e = min(max(e, 0L), E - 1);                               // (never an access out of bounds)
+        float4 dk[4];
+        if constexpr (GRID) {
+            const float u = len[e] * inv_h, fl = floorf(u);
+            float w[4];
+            lagrange4(u - fl, w);
+            const int i = (int)fl;
+#pragma unroll
+            for (int k = 0; k < 4; k++) dk[k] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int j = 0; j < 4; j++) {
+                const float* row = dist + (long)((i - 1 + j) & mask) * 4 * n + c;
+#pragma unroll
+                for (int k = 0; k < 4; k++) dk[k] = fma4(w[j], ld4(row + k * n), dk[k]);
+            }
+        } else {
+            const float* de = dist + e * 4 * n + c;
+#pragma unroll
+            for (int k = 0; k < 4; k++) dk[k] = ld4(de + k * n);
+        }
+        const long eg = grad_row ? min(max((long)grad_row[e], 0L), n_grad_rows - 1) : e;
+        const Vec3x4 g = ld12(dm + (eg * n + c) * 3);
+        const float4 ga = ld4(da + eg * n + c);
+        const Vec3 d = {dir[3 * e], dir[3 * e + 1], dir[3 * e + 2]};
+        float dp[3][4];
+        Vec3 gd = {0.f, 0.f, 0.f};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const Vec3 x = vv.get(j), gm = g.get(j);
+            const float p0 = at(dk[0], j) * at(ak[0], j) * k0, p1 = at(dk[1], j) * at(ak[1], j) * k1;
+            const float p2 = at(dk[2], j) * at(ak[2], j) * k2;
+            dp[0][j] = dot(gm, x) * k0;
+            dp[1][j] = dot(gm, cross(x, d)) * k1;
+            dp[2][j] = dot(gm, d) * k2;
+            const Vec3 dg = cross(d, gm), gx = cross(gm, x);
+            acc_v.f[3 * j] += gm.x * p0 + dg.x * p1;
+            acc_v.f[3 * j + 1] += gm.y * p0 + dg.y * p1;
+            acc_v.f[3 * j + 2] += gm.z * p0 + dg.z * p1;
+            gd.x += gx.x * p1 + gm.x * p2;
+            gd.y += gx.y * p1 + gm.y * p2;
+            gd.z += gx.z * p1 + gm.z * p2;
+        }
+        const float4 ga3 = make_float4(ga.x * k3, ga.y * k3, ga.z * k3, ga.w * k3);
+        float4 dpk[4];
+#pragma unroll
+        for (int k = 0; k < 3; k++) dpk[k] = make_float4(dp[k][0], dp[k][1], dp[k][2], dp[k][3]);
+        dpk[3] = ga3;
+        if (d_dist) {
+            float* dde = d_dist + e * 4 * n + c;
+#pragma unroll
+            for (int k = 0; k < 4; k++) st4(dde + k * n, mul4(dpk[k], ak[k]));
+        }
+#pragma unroll
+        for (int k = 0; k < 4; k++) {
+            acc_a[k].x = fmaf(dpk[k].x, dk[k].x, acc_a[k].x);
+            acc_a[k].y = fmaf(dpk[k].y, dk[k].y, acc_a[k].y);
+            acc_a[k].z = fmaf(dpk[k].z, dk[k].z, acc_a[k].z);
+            acc_a[k].w = fmaf(dpk[k].w, dk[k].w, acc_a[k].w);
+        }
+        if (d_dir) {                                              // (uniform)
+            for (int sh = 1; sh < tpe; sh <<= 1) {
+                gd.x += __shfl_xor(gd.x, sh);
+                gd.y += __shfl_xor(gd.y, sh);
+                gd.z += __shfl_xor(gd.z, sh);
+            }
+            if (c == 0) { d_dir[3 * e] = gd.x; d_dir[3 * e + 1] = gd.y; d_dir[3 * e + 2] = gd.z; }
+        }
+    }
+    if (!live) return;
+    if (d_actv) {
+        float* dae = d_actv + r * 4 * n + c;
+#pragma unroll
+        for (int k = 0; k < 4; k++) st4(dae + k * n, acc_a[k]);
+    }
+    if (dv) st12(dv + (r * n + c) * 3, acc_v);
+}
+
 // ---------------------------------------------------------------------------------------------------------------
 // The filter from its grid, for training.  The filter MLP sees an edge only through its length d, so inference
 // evaluates it on a grid over one period of d and interpolates (painn.hip); training can do the same: the forward
@@ -531,6 +641,38 @@ int mg_painn_combine_bwd_grid(const float* table, int table_rows, float period, 
                        (hipStream_t)stream, table, actv, v, dir, node, n_rows, dm, da, grad_row, n_grad_rows, E, n, terms,
                        d_dist, d_actv, dv, d_dir, len, table_rows - 1, (float)table_rows / period);
     return check_launch("mg_painn_combine_bwd_grid");
+}
+
+int mg_painn_combine_bwd_rows(const float* dist, const float* table, int table_rows, float period, const float* len,
+                              const float* actv, const float* v, const float* dir, const int* row_ptr, const int* order,
+                              long n_rows, const float* dm, const float* da, const int* grad_row, long n_grad_rows,
+                              long E, int n, int terms, float* d_dist, float* d_actv, float* dv, float* d_dir,
+                              mg_stream_t stream) {
+    MG_REQUIRE(E >= 0 && n_rows >= 0 && combine_shape_ok(n), "mg_painn_combine_bwd_rows: n must be a power of two in 4..256");
+    MG_REQUIRE(terms >= 0 && terms <= 15, "mg_painn_combine_bwd_rows: terms is a mask of four bits");
+    MG_REQUIRE(E == 0 || (dist != nullptr) != (table != nullptr),       // (without edges neither is read)
+               "mg_painn_combine_bwd_rows: give dist or table, not both");
+    MG_REQUIRE(table == nullptr || (table_shape_ok(table_rows, 4 * n) && period > 0.f && (len != nullptr || E == 0)),
+               "mg_painn_combine_bwd_rows: grid rows must be a power of two, period positive, len given");
+    if (n_rows == 0) return MG_OK;
+    if (!d_dist && !d_actv && !dv && !d_dir) return MG_OK;       // (any of the four outputs may be left out)
+    MG_REQUIRE(actv && v && row_ptr && (E == 0 || (dir && dm && da)), "mg_painn_combine_bwd_rows: null pointer");
+    MG_REQUIRE(grad_row == nullptr || n_grad_rows > 0, "mg_painn_combine_bwd_rows: an index needs a positive row count");
+    MG_REQUIRE(aligned16(dist) && aligned16(table) && aligned16(actv) && aligned16(v) && aligned16(dm) && aligned16(da) &&
+                   aligned16(d_dist) && aligned16(d_actv) && aligned16(dv),
+               "mg_painn_combine_bwd_rows: arrays must be 16-byte aligned");
+    const long threads = n_rows * (n / 4);
+    MG_REQUIRE(ceil_div(threads, 256) < (1L << 31), "mg_painn_combine_bwd_rows: too many rows");
+    const dim3 grid((unsigned)ceil_div(threads, 256)), block(256);
+    if (table)
+        hipLaunchKernelGGL(painn_combine_bwd_rows_kernel<true>, grid, block, 0, (hipStream_t)stream, table, actv, v, dir,
+                           row_ptr, order, n_rows, dm, da, grad_row, n_grad_rows, E, n, terms, d_dist, d_actv, dv, d_dir, len,
+                           table_rows - 1, (float)table_rows / period);
+    else
+        hipLaunchKernelGGL(painn_combine_bwd_rows_kernel<false>, grid, block, 0, (hipStream_t)stream, dist, actv, v, dir,
+                           row_ptr, order, n_rows, dm, da, grad_row, n_grad_rows, E, n, terms, d_dist, d_actv, dv, d_dir,
+                           nullptr, 0, 0.f);
+    return check_launch("mg_painn_combine_bwd_rows");
 }
 
 int mg_painn_table_interp_supported(int table_rows, int cols) { return table_shape_ok(table_rows, cols) ? 1 : 0; }

@@ -300,20 +300,23 @@ class _PainnCombine(torch.autograd.Function):
 class _PainnCombineGrad(torch.autograd.Function):
     """(g_v, g_a, dist, actv, v, direction) -> the gradients of _PainnCombine's four inputs: d_dist (edges, 4n),
     d_actv (nodes, 4n), dv (nodes, n, 3), d_direction (edges, 3): one kernel; the gradient rows of an edge's source
-    node are read through the source index, the gradients of actv and v are summed over the edges of a destination."""
+    node are read through the source index, the gradients of actv and v are summed over the edges of a destination
+    inside it (mg_painn_combine_bwd_rows)."""
 
     @staticmethod
     def forward(ctx, g_v, g_a, dist, actv_node, v_node, direction, by_dst, by_src, terms, want):
         """want: which of the four gradients to compute (the others come back as empty tensors)."""
         ctx.by_dst, ctx.by_src, ctx.terms, ctx.want = by_dst, by_src, terms, want
         ctx.save_for_backward(g_v, g_a, dist, actv_node, v_node, direction)
-        d_dist, d_actv, dv, d_dir = ops.painn_combine_bwd(
-            dist.contiguous(), actv_node.contiguous(), v_node.contiguous(), direction.contiguous(), g_v.contiguous(),
-            g_a.contiguous(), node=by_dst.index, grad_row=by_src.index, terms=terms, want=want)
-        if want[1]:
-            d_actv = ops.segment_sum_csr(d_actv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm)
-        if want[2]:
-            dv = ops.segment_sum_csr(dv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm)
+        args = (dist.contiguous(), actv_node.contiguous(), v_node.contiguous(), direction.contiguous(), g_v.contiguous(),
+                g_a.contiguous())
+        if want[1] or want[2]:
+            # the gradients of actv and v are summed over the edges of a destination inside the kernel
+            d_dist, d_actv, dv, d_dir = ops.painn_combine_bwd_rows(*args, by_dst.row_ptr, by_dst.perm, by_src.index,
+                                                                   terms=terms, want=want)
+        else:
+            d_dist, d_actv, dv, d_dir = ops.painn_combine_bwd(*args, node=by_dst.index, grad_row=by_src.index,
+                                                              terms=terms, want=want)
         outs = [d_dist, d_actv, dv, d_dir]
         for k in range(4):
             if outs[k] is None:
@@ -502,8 +505,8 @@ class _PainnGridMessage(torch.autograd.Function):
     not differentiated, with the filter interpolated from the grid.  Forward: the inference kernel of the layer
     (mg_painn_table_message: lengths, directions, interpolation, the lines 94-100 of archs/meanflow_painn8.py and the
     sum over the edges of a node in one pass; no per-edge filter is stored).  Backward: the gradient kernel of the
-    unfused formulation with the filter of every edge interpolated again inside it (mg_painn_combine_bwd_grid), the
-    segment sums, the scatter into the grid.  A recorded backward pass differentiates the unfused formulation instead."""
+    unfused formulation with the filter of every edge interpolated again inside it and the gradients of actv and v
+    summed per destination inside it (mg_painn_combine_bwd_rows), then the scatter into the grid.  A recorded backward pass differentiates the unfused formulation instead."""
 
     @staticmethod
     def forward(ctx, table, actv, v, r_ij, graph, period, epsilon):
@@ -533,20 +536,17 @@ class _PainnGridMessage(torch.autograd.Function):
         by_dst, by_src = graph.by_dst, graph.by_src
         d = torch.linalg.vector_norm(r_ij, dim=-1).contiguous()
         want = (bool(need[0]), bool(need[1]), bool(need[2]), False)
-        d_dist, d_actv, dv, _ = ops.painn_combine_bwd_grid(table, ctx.period, d, actv, v,
-                                                           _unit_vectors(r_ij, ctx.epsilon).contiguous(), g_v.contiguous(),
-                                                           g_a.contiguous(), by_dst.index, by_src.index, terms=_TERMS_ALL,
-                                                           want=want)
+        # (actv and v are read at an edge's destination: their gradients are summed over a destination's edges inside)
+        d_dist, d_actv, dv, _ = ops.painn_combine_bwd_rows(None, actv, v, _unit_vectors(r_ij, ctx.epsilon).contiguous(),
+                                                           g_v.contiguous(), g_a.contiguous(), by_dst.row_ptr, by_dst.perm,
+                                                           by_src.index, terms=_TERMS_ALL, want=want, table=table,
+                                                           period=ctx.period, d=d)
         d_table = None
         if need[0]:
             rows = table.size(0)
             perm, bucket_ptr = ops.painn_table_sorted_edges(d, rows, ctx.period)
             d_table = ops.painn_table_interp_bwd(d_dist, None, d, ctx.period, perm, bucket_ptr, want_length_grad=False,
                                                  order=0, table_rows=rows)[0]
-        if need[1]:
-            d_actv = ops.segment_sum_csr(d_actv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm)
-        if need[2]:
-            dv = ops.segment_sum_csr(dv, by_dst.row_ptr, by_dst.n_rows, perm=by_dst.perm)
         return (d_table, d_actv if need[1] else None, dv if need[2] else None, None, None, None, None)
 
 

@@ -1700,6 +1700,51 @@ def painn_combine_bwd_grid(table, period, d, actv, v, direction, dm, da, node, g
     return d_dist, d_actv, dv, d_dir
 
 
+def painn_combine_bwd_rows(dist, actv, v, direction, dm, da, row_ptr, order, grad_row, terms=15,
+                           want=(True, True, True, True), table=None, period=None, d=None):
+    """The gradients of painn_combine_fwd's inputs for actv (rows, 4n) and v (rows, n, 3) read per edge at one row,
+    with those two gradients summed per row inside the kernel: (d_dist (E, 4n), d_actv (rows, 4n), dv (rows, n, 3),
+    d_dir (E, 3)).  (row_ptr, order): the CSR of the edges by the row they read (order None: edges sorted by it).
+    dm, da are read at grad_row[e] (None: at e).  The filter: dist (E, 4n), or dist None and table (grid rows, 4n),
+    period, d (E): interpolated inside the kernel."""
+    grid = dist is None
+    for t, name in ((actv, "actv"), (v, "v"), (direction, "direction"), (dm, "dm"), (da, "da")):
+        _check_input(t, name)
+    _check_input(row_ptr, "row_ptr", torch.int32)
+    if order is not None:
+        _check_input(order, "order", torch.int32)
+    if grad_row is not None:
+        _check_input(grad_row, "grad_row", torch.int32)
+    E, n, rows = int(direction.size(0)), int(v.size(1)), int(v.size(0))
+    if grid:
+        _check_input(table, "table")
+        _check_input(d, "d")
+        if table.dim() != 2 or table.size(1) != 4 * n or d.numel() != E:
+            raise RuntimeError("expected table (grid rows, 4n) and d (edges)")
+    else:
+        _check_input(dist, "dist")
+        if tuple(dist.shape) != (E, 4 * n):
+            raise RuntimeError("expected dist (edges, 4n)")
+    if tuple(actv.shape) != (rows, 4 * n) or tuple(v.shape) != (rows, n, 3) or tuple(direction.shape) != (E, 3):
+        raise RuntimeError("expected actv (rows, 4n), v (rows, n, 3), direction (edges, 3)")
+    if row_ptr.numel() != rows + 1 or (order is not None and order.numel() != E) or \
+            (grad_row is not None and grad_row.numel() != E):
+        raise RuntimeError("expected row_ptr (rows + 1) and one entry per edge in order / grad_row")
+    g_rows = int(dm.size(0))
+    if tuple(dm.shape) != (g_rows, n, 3) or tuple(da.shape) != (g_rows, n) or (grad_row is None and g_rows != E):
+        raise RuntimeError("expected dm (rows, n, 3) and da (rows, n)")
+    with torch.cuda.device(v.device):
+        d_dist = torch.empty(E, 4 * n, dtype=torch.float32, device=v.device) if want[0] else None
+        d_actv = torch.empty(rows, 4 * n, dtype=torch.float32, device=v.device) if want[1] else None
+        dv = torch.empty(rows, n, 3, dtype=torch.float32, device=v.device) if want[2] else None
+        d_dir = torch.empty_like(direction) if want[3] else None
+        L.check(_lib.mg_painn_combine_bwd_rows(_p(dist), _p(table) if grid else None, int(table.size(0)) if grid else 0,
+                                               float(period) if grid else 0.0, _p(d) if grid else None, _p(actv), _p(v),
+                                               _p(direction), _p(row_ptr), _p(order), rows, _p(dm), _p(da), _p(grad_row),
+                                               g_rows, E, n, int(terms), _p(d_dist), _p(d_actv), _p(dv), _p(d_dir), _stream()))
+    return d_dist, d_actv, dv, d_dir
+
+
 def painn_table_interp_supported(table_rows, cols):
     return bool(_lib.mg_painn_table_interp_supported(int(table_rows), int(cols)))
 

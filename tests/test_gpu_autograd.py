@@ -544,6 +544,49 @@ def test_combine_gradient_with_the_filter_interpolated_inside(ops, n, rows):
                 _close(got[k], ref[k].double().cpu(), f"gradient {k} with outputs {want}", 2e-6)
 
 
+@pytest.mark.parametrize("n, E, nodes", [(32, 3000, 200), (128, 5000, 64), (4, 700, 900)])
+def test_combine_gradient_summed_per_row_inside_the_kernel(ops, n, E, nodes):
+    """mg_painn_combine_bwd_rows (the gradients of actv and v summed over the edges that read a row, inside the kernel)
+    against mg_painn_combine_bwd followed by segment sums, with the filter stored and with the filter interpolated
+    from its grid; rows that no edge reads; a subset of the outputs; and float64 for the sums."""
+    g = torch.Generator().manual_seed(0x947 + 47 + n)
+    rows, period = 512, 10.0
+    phase = 2 * torch.pi * torch.arange(rows)[:, None] / rows
+    table = (torch.sin(phase * torch.randint(1, 4, (1, 4 * n), generator=g) + torch.rand(1, 4 * n, generator=g))
+             * torch.randn(1, 4 * n, generator=g)).cuda()
+    d = (torch.rand(E, generator=g) * period * 0.999).cuda()
+    actv, v = torch.randn(nodes, 4 * n, generator=g).cuda(), torch.randn(nodes, n, 3, generator=g).cuda()
+    direction = torch.nn.functional.normalize(torch.randn(E, 3, generator=g), dim=-1).cuda()
+    dm, da = torch.randn(nodes, n, 3, generator=g).cuda(), torch.randn(nodes, n, generator=g).cuda()
+    node = torch.randint(0, nodes, (E,), generator=g).int().cuda()
+    grad_row = torch.randint(0, nodes, (E,), generator=g).int().cuda()
+    order = torch.sort(node.long(), stable=True).indices.int().contiguous()
+    row_ptr = ops.segment_row_ptr(node[order.long()].contiguous(), nodes)
+    dist = ops.painn_table_interp_fwd(table, d, period, 0)
+    ref = ops.painn_combine_bwd(dist, actv, v, direction, dm, da, node=node, grad_row=grad_row)
+    sums = [torch.zeros(nodes, *t.shape[1:], dtype=F64).index_add_(0, node.long().cpu(), t.double().cpu()) for t in ref[1:3]]
+    for name, kw in (("stored filter", dict(dist=dist)), ("grid", dict(dist=None, table=table, period=period, d=d))):
+        filt = kw.pop("dist")
+        for want in ((True, True, True, True), (False, True, True, False), (True, False, True, False)):
+            got = ops.painn_combine_bwd_rows(filt, actv, v, direction, dm, da, row_ptr, order, grad_row, want=want, **kw)
+            for k in range(4):
+                assert (got[k] is None) == (not want[k])
+            if want[0]:
+                _close(got[0], ref[0].double().cpu(), f"{name}: d_dist", 2e-6)
+            if want[3]:
+                _close(got[3], ref[3].double().cpu(), f"{name}: d_dir", 2e-6)
+            if want[1]:
+                _close(got[1], sums[0], f"{name}: d_actv per row", 4e-6)
+            _close(got[2], sums[1], f"{name}: dv per row", 4e-6)
+    # edges already sorted by the row they read: no order array
+    node_sorted = node[order.long()].contiguous()
+    pick = lambda t: t[order.long()].contiguous()
+    got = ops.painn_combine_bwd_rows(pick(dist), actv, v, pick(direction), dm, da, row_ptr, None, pick(grad_row))
+    _close(got[1], sums[0], "sorted edges: d_actv per row", 4e-6)
+    _close(got[0], pick(ref[0]).double().cpu(), "sorted edges: d_dist", 2e-6)
+    assert int(node_sorted[0]) <= int(node_sorted[-1])
+
+
 def test_painn_message_through_its_grid_in_one_forward_kernel(pkg):
     """Message under autograd with edge vectors that are not differentiated: the forward pass is the inference kernel
     on the grid (differentiable._PainnGridMessage) and the backward pass interpolates the filter again.  Values and
