@@ -7,6 +7,10 @@ products with their two gradient kernels, gather and segment sum, which are each
 backward is itself differentiable; the elementwise glue in between (activations, norms, the radial encodings, the
 cross product, the periodic wrap) is plain torch arithmetic on the device, which autograd differentiates as it does
 for the reference.  Results equal the fused path up to fp32 summation order (tests/test_gpu_autograd.py).
+
+Forward mode: the functions that a forward pass runs also carry jvp rules, written with the same functions, so `jvp`
+below returns a value and its derivative along a direction from one pass on dual tensors, both differentiable
+afterwards; add / sub / mul are the arithmetic to use where only one operand can carry a tangent.
 """
 import math
 
