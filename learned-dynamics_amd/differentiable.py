@@ -96,12 +96,16 @@ def jvp(f, primals, tangents):
     (archs/meanflow_painn8.py:274-282), gets the same derivative out of two nested backward passes, and the loss then
     differentiates all three; its first result is the same f(*primals) that the loss evaluates again as v_pred
     (archs/meanflow_painn8.py:291-292), so one call here stands for both."""
+    def unpack(out):
+        value, tangent = fwAD.unpack_dual(out)
+        return value, (tangent if tangent is not None else torch.zeros_like(value))
+
     with fwAD.dual_level():
         out = f(*(fwAD.make_dual(p, t) for p, t in zip(primals, tangents)))
-        value, tangent = fwAD.unpack_dual(out)
-        if tangent is None:
-            tangent = torch.zeros_like(value)
-    return value, tangent
+        if isinstance(out, (tuple, list)):               # several results: (values, tangents), like functional.jvp
+            pairs = [unpack(o) for o in out]
+            return tuple(v for v, _ in pairs), tuple(t for _, t in pairs)
+        return unpack(out)
 
 
 def linear(lin, x, x_bound=None, want_bound=False):

@@ -54,3 +54,11 @@ def test_jvp_of_a_function_without_dependence_gives_zeros():
     diff = _diff()
     value, tangent = diff.jvp(lambda x: torch.ones(2), (torch.randn(2),), (torch.randn(2),))
     assert torch.equal(value, torch.ones(2)) and torch.equal(tangent, torch.zeros(2))
+
+
+def test_jvp_of_a_function_with_several_results():
+    diff = _diff()
+    x, u = torch.randn(3, dtype=torch.float64), torch.randn(3, dtype=torch.float64)
+    values, tangents = diff.jvp(lambda t: (t.sin(), t * t), (x,), (u,))
+    torch.testing.assert_close(values[0], x.sin()); torch.testing.assert_close(values[1], x * x)
+    torch.testing.assert_close(tangents[0], x.cos() * u); torch.testing.assert_close(tangents[1], 2 * x * u)
