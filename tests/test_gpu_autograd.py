@@ -544,7 +544,7 @@ def test_combine_gradient_with_the_filter_interpolated_inside(ops, n, rows):
                 _close(got[k], ref[k].double().cpu(), f"gradient {k} with outputs {want}", 2e-6)
 
 
-@pytest.mark.parametrize("n, E, nodes", [(32, 3000, 200), (128, 5000, 64), (4, 700, 900)])
+@pytest.mark.parametrize("n, E, nodes", [(32, 3000, 200), (128, 5000, 64), (4, 700, 900), (256, 2500, 7), (64, 1, 300)])
 def test_combine_gradient_summed_per_row_inside_the_kernel(ops, n, E, nodes):
     """mg_painn_combine_bwd_rows (the gradients of actv and v summed over the edges that read a row, inside the kernel)
     against mg_painn_combine_bwd followed by segment sums, with the filter stored and with the filter interpolated
