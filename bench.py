@@ -591,9 +591,10 @@ def bench_painn_train(torch, args):
                        "parameters_with_gradient": sum(gr is not None for gr in grads[2:]),
                        "inference_forward_ms_same_inputs": t_fwd * 1e3},
             "note": "the differentiable path: the filter through its 512-row grid (the MLP is differentiated on the grid's "
-                    "rows, each edge interpolates; per-edge evaluation when the grid test rejects the weights), the "
-                    "elementwise middle of the message and the gathers as one kernel each way, split-fp16 GEMMs and "
-                    "weight gradients for the node-sized MLPs"}
+                    "rows, each edge interpolates; per-edge evaluation when the grid test rejects the weights); the "
+                    "message's forward pass is the inference kernel, its backward pass one kernel that interpolates the "
+                    "filter again and sums the gradients of the node operands per destination, plus the scatter into "
+                    "the grid; split-fp16 GEMMs and weight gradients for the node-sized MLPs"}
 
 
 def bench_denoiser_train(torch, args):
