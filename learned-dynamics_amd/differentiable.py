@@ -88,14 +88,19 @@ def mul(a, b):
     return fwAD.make_dual(p * one[1], t * one[1])
 
 
-def jvp(f, primals, tangents):
+def jvp(f, primals, tangents, create_graph=True, strict=False):
     """(f(*primals), the derivative of f at primals along tangents) in forward mode: every autograd function of this
     package that a forward pass runs has a jvp rule made of the package's differentiable functions, so the pair costs
     about two forward passes and both results can be differentiated afterwards (loss.backward()).
     torch.autograd.functional.jvp(f, primals, tangents, create_graph=True), which the reference's meanflow loss calls
     (archs/meanflow_painn8.py:274-282), gets the same derivative out of two nested backward passes, and the loss then
     differentiates all three; its first result is the same f(*primals) that the loss evaluates again as v_pred
-    (archs/meanflow_painn8.py:291-292), so one call here stands for both."""
+    (archs/meanflow_painn8.py:291-292), so one call here stands for both.  The signature and the order of the results
+    are functional.jvp's, so the name is the only change at a call site; create_graph and strict are accepted for that
+    and change nothing (both results are always recorded when autograd is recording; without it, under no_grad, neither
+    is).  primals and tangents may be single tensors."""
+    if torch.is_tensor(primals):
+        primals, tangents = (primals,), (tangents,)
     def unpack(out):
         value, tangent = fwAD.unpack_dual(out)
         return value, (tangent if tangent is not None else torch.zeros_like(value))

@@ -62,3 +62,12 @@ def test_jvp_of_a_function_with_several_results():
     values, tangents = diff.jvp(lambda t: (t.sin(), t * t), (x,), (u,))
     torch.testing.assert_close(values[0], x.sin()); torch.testing.assert_close(values[1], x * x)
     torch.testing.assert_close(tangents[0], x.cos() * u); torch.testing.assert_close(tangents[1], 2 * x * u)
+
+
+def test_jvp_takes_the_arguments_of_functional_jvp():
+    diff = _diff()
+    x, u = torch.randn(3, dtype=torch.float64), torch.randn(3, dtype=torch.float64)
+    f = lambda t: t.exp() * t
+    ours = diff.jvp(f, x, u, create_graph=True)
+    theirs = torch.autograd.functional.jvp(f, x, u, create_graph=True)
+    torch.testing.assert_close(ours[0], theirs[0]); torch.testing.assert_close(ours[1], theirs[1])
