@@ -123,7 +123,7 @@ class SelfTensProds(nn.Module):
         """Returns the three normalised product features, or x + them with residual=True."""
         if diff.wants_grad(self, x_a, x_v, x_d):
             y = diff.self_tens_prods(self, x_a, x_v, x_d)
-            return tuple(x + t for x, t in zip((x_a, x_v, x_d), y)) if residual else y
+            return tuple(diff.add(x, t) for x, t in zip((x_a, x_v, x_d), y)) if residual else y
         in_a, in_v, in_d = x_a, x_v, x_d
         *rest, dim_a = x_a.shape
         dim_v, dim_d = x_v.shape[-2], x_d.shape[-3]
@@ -337,7 +337,7 @@ class Messages(nn.Module):
         the caller must own x_a, x_v, x_d; three full-size additions per block are not launched."""
         if diff.wants_grad(self, r_ij, x_a, x_v, x_d):
             out = diff.bee_messages(self, graph, r_ij, x_a, x_v, x_d)
-            return tuple(x + d for x, d in zip((x_a, x_v, x_d), out)) if add_to_inputs else out
+            return tuple(diff.add(x, d) for x, d in zip((x_a, x_v, x_d), out)) if add_to_inputs else out
         in_place = add_to_inputs and x_a.is_contiguous() and x_v.is_contiguous() and x_d.is_contiguous()
         if isinstance(node_order, str):
             node_order = getattr(graph, "cell_order", None)

@@ -69,12 +69,12 @@ class Denoiser(nn.Module):
             x_a = diff.linear(self.embed, one_hot)
         else:
             x_a = ops.tensor_linear_fwd(0, self.embed.weight, one_hot.contiguous(), bias=self.embed.bias)
-        x_a = x_a + self.t_embed(st)[:, None]
-        x_v = self.v_readin((x1 - x0)[..., None, :].contiguous())
+        x_a = diff.add(x_a, self.t_embed(st)[:, None])
+        x_v = self.v_readin(diff.sub(x1, x0)[..., None, :].contiguous())
         x_d = torch.zeros(B, N, dim_d, 3, 3, device=x1.device)
         for msg, prod in zip(self.messages, self.prods):
             # x_a, x_v, x_d are this function's own tensors: the messages are added in their memory
             x_a, x_v, x_d = msg(graph, r_ij, x_a, x_v, x_d, node_order=node_order, add_to_inputs=True)
             x_a, x_v, x_d = prod(x_a, x_v, x_d, residual=True)
         v_pred = self.readout(x_v).squeeze(-2)
-        return (1. - (t - s)[:, None, None]) * v_pred
+        return diff.mul(diff.sub(1., diff.sub(t, s)[:, None, None]), v_pred)

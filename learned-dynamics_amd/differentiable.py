@@ -88,6 +88,14 @@ def mul(a, b):
     return fwAD.make_dual(p * one[1], t * one[1])
 
 
+def div(a, b):
+    """a / b for a b without a tangent, in forward mode as add."""
+    if not (torch.is_tensor(a) and has_tangent(a)) or (torch.is_tensor(b) and has_tangent(b)):
+        return a / b
+    p, t = fwAD.unpack_dual(a)
+    return fwAD.make_dual(p / b, t / b)
+
+
 def jvp(f, primals, tangents, create_graph=True, strict=False):
     """(f(*primals), the derivative of f at primals along tangents) in forward mode: every autograd function of this
     package that a forward pass runs has a jvp rule made of the package's differentiable functions, so the pair costs
@@ -208,12 +216,12 @@ def _jacobi_matrix(device):
 def radial_encode_8(r, rmax):
     """managan/jacobi_radenc.py:24-37; the polynomials are evaluated in float64 (Horner) like the inference kernel:
     their monomial form in fp32 loses three digits."""
-    z = (torch.linalg.vector_norm(r, dim=-1) / rmax)[..., None].double()
+    z = div(torch.linalg.vector_norm(r, dim=-1), rmax)[..., None].double()
     A = _jacobi_matrix(r.device)
     acc = A[:, 8].expand(*z.shape[:-1], 8)
     for k in range(7, -1, -1):
-        acc = acc * z + A[:, k]
-    return (acc * torch.relu(1.0 - z)).to(r.dtype)
+        acc = add(mul(acc, z), A[:, k])
+    return (acc * torch.relu(sub(1.0, z))).to(r.dtype)
 
 
 def tens_sigmoid(inds, x):
@@ -758,7 +766,7 @@ def bee_messages(msg, graph, r_ij, x_a, x_v, x_d):
     """archs/diffuser_atoms15.py:238-253"""
     enc8 = radial_encode_8(r_ij, msg.r0)
     enc = linear(msg.lin_enc, enc8)
-    rh = tens_sigmoid(1, r_ij * (7. / msg.r0))
+    rh = tens_sigmoid(1, mul(r_ij, 7. / msg.r0))
     # The output linears of the vector and rank-2 channels have no bias and nothing nonlinear follows them before the
     # sum over edges, so they commute with it: the products are summed per node first and the ten linears run on N
     # rows, not E (the reference applies them per edge).  The scalar channel goes through an MLP per edge.
@@ -774,7 +782,7 @@ def bee_messages(msg, graph, r_ij, x_a, x_v, x_d):
         else:
             sums[k] = y if sums[k] is None else sums[k] + y
     psi_a = psi_a + mlp_leaky(msg.mlp_a, psi_a)
-    return 0.1 * gl.edges_reduce_src(graph, psi_a), 0.1 * sums[1], 0.1 * sums[2]
+    return mul(gl.edges_reduce_src(graph, psi_a), 0.1), mul(sums[1], 0.1), mul(sums[2], 0.1)
 
 
 def self_tens_prods(mod, x_a, x_v, x_d):

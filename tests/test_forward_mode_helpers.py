@@ -18,10 +18,11 @@ def test_one_sided_arithmetic_equals_torchs_rules():
     c = torch.randn(5, 3, dtype=torch.float64, requires_grad=True)
 
     def with_helpers(xx):
-        return diff.mul(diff.sub(2.0, diff.add(diff.mul(xx, c), c)), diff.sub(xx, 0.5)) + diff.sub(c, xx)
+        return diff.mul(diff.sub(2.0, diff.add(diff.mul(xx, c), c)), diff.sub(xx, 0.5)) + diff.sub(c, xx) + diff.div(xx, 3.0) \
+            + diff.div(xx, c.exp())
 
     def plain(xx):
-        return (2.0 - (xx * c + c)) * (xx - 0.5) + (c - xx)
+        return (2.0 - (xx * c + c)) * (xx - 0.5) + (c - xx) + xx / 3.0 + xx / c.exp()
 
     assert torch.equal(with_helpers(x), plain(x))                       # outside forward mode: plain arithmetic
     value, tangent = diff.jvp(with_helpers, (x,), (u,))

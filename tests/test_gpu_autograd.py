@@ -324,6 +324,38 @@ def test_forward_mode_rules_agree_with_nested_backward(pkg, ops):
                 _close(a, r.double().cpu(), f"{name}: gradient {k}", 1e-4)
 
 
+def test_rank012_denoiser_in_forward_mode(pkg):
+    """The whole rank-0/1/2 denoiser (neighbour search, time embedding, two blocks of Messages + SelfTensProds, readout)
+    under differentiable.jvp against torch.autograd.functional.jvp(create_graph=True) on the device: value, tangent and
+    the gradients of a function of both for every parameter."""
+    den = importlib.import_module("learned-dynamics_amd.denoiser")
+    diff = importlib.import_module("learned-dynamics_amd.differentiable")
+    torch.manual_seed(0x947 + 51)
+    B, N, box = 2, 200, (30.0, 30.0, 30.0)
+    model = den.Denoiser(6.0, dim_a=32, dim_v=16, dim_d=8, chan=32, blocks=2).cuda()
+    g = torch.Generator().manual_seed(1)
+    x1 = (torch.rand(B, N, 3, generator=g) * 30).cuda()
+    x0 = x1 + 0.3 * torch.randn(B, N, 3, generator=g).cuda()
+    one_hot = torch.nn.functional.one_hot(torch.randint(0, 20, (B, N), generator=g), 20).float().cuda()
+    s, t = torch.zeros(B).cuda(), torch.rand(B, generator=g).cuda()
+    v = torch.randn(B, N, 3, generator=g).cuda()
+    f = lambda xx, tt: model((s, tt), x0, xx, one_hot, box)
+    params = list(model.parameters())
+    value, tangent = diff.jvp(f, (x1, t), (v, torch.ones_like(t)))
+    got = torch.autograd.grad((tangent ** 2).sum() + value.sum(), params, allow_unused=True)
+    value_n, tangent_n = torch.autograd.functional.jvp(f, (x1, t), (v, torch.ones_like(t)), create_graph=True)
+    ref = torch.autograd.grad((tangent_n ** 2).sum() + f(x1, t).sum(), params, allow_unused=True)
+    _close(value, value_n.double().cpu(), "value", 1e-5)
+    _close(tangent, tangent_n.double().cpu(), "tangent", 1e-5)
+    checked = 0
+    for (name, _), a, r in zip(model.named_parameters(), got, ref):
+        assert (a is None) == (r is None), name
+        if a is not None:
+            _close(a, r.double().cpu(), f"gradient for {name}", 1e-4)
+            checked += 1
+    assert checked >= 80
+
+
 def test_weight_gradient_is_reproducible(ops):
     g = torch.Generator().manual_seed(8)
     dy, x = torch.randn(30000, 96, 3, generator=g).cuda(), torch.randn(30000, 64, 3, generator=g).cuda()
