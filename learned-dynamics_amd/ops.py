@@ -23,6 +23,27 @@ _raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
 _raw_device = getattr(torch._C, "_cuda_getDevice", None)
 
 
+class _AlreadyCurrent:
+    """A context that does nothing: the device asked for is the current one."""
+
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_ALREADY_CURRENT = _AlreadyCurrent()
+
+
+def _on(device):
+    """`with _on(t.device):` makes t's device current for the allocations and launches inside, like torch.cuda.device,
+    without that context manager's bookkeeping when the device is current already (every call on a one-GPU host)."""
+    if _raw_device is not None and (device.index is None or device.index == _raw_device()):
+        return _ALREADY_CURRENT
+    return torch.cuda.device(device)
+
+
 def _stream():
     """The current HIP stream of the current device as a pointer argument."""
     if _raw_stream is not None and _raw_device is not None:     # same value as below, without building Stream objects
@@ -117,7 +138,7 @@ class NeighbourSearch:
         L.check(_lib.mg_neighbour_workspace_bytes(self.batch, self.nodes, self.cutoff, *self.box,
                                                   ctypes.byref(nbytes)))
         dev = x.device
-        with torch.cuda.device(dev):
+        with _on(dev):
             self.workspace = torch.empty(nbytes.value, dtype=torch.uint8, device=dev)
             self.row_ptr = torch.empty(self.batch * self.nodes + 1, dtype=torch.int32, device=dev)
             self.edge_counts = torch.empty(self.batch, dtype=torch.int32, device=dev)
@@ -165,7 +186,7 @@ class NeighbourSearch:
         dev = self.x.device
         if n_edges is not None or self._host_stats is not None:
             E = self.host_stats()[0] if n_edges is None else int(n_edges)
-            with torch.cuda.device(dev):
+            with _on(dev):
                 src = torch.empty(E, dtype=torch.int32, device=dev)
                 dst = torch.empty(E, dtype=torch.int32, device=dev)
             return self.fill_into(src, dst)
@@ -175,7 +196,7 @@ class NeighbourSearch:
             volume = self.box[0] * self.box[1] * self.box[2]
             hint = 1.5 * self.batch * self.nodes * (self.nodes / volume) * 4.18879 * self.cutoff ** 3
         capacity = min(int(1.125 * hint) + 4096, 2 ** 31 - 1)
-        with torch.cuda.device(dev):
+        with _on(dev):
             src = torch.empty(capacity, dtype=torch.int32, device=dev)
             dst = torch.empty(capacity, dtype=torch.int32, device=dev)
         self.fill_into(src, dst)
@@ -194,7 +215,7 @@ class NeighbourSearch:
         _check_input(dst, "dst", torch.int32)
         if src.numel() != dst.numel():
             raise RuntimeError("src and dst must have the same length")
-        with torch.cuda.device(self.x.device):
+        with _on(self.x.device):
             L.check(_lib.mg_neighbour_fill(_p(self.workspace), self.workspace.numel(), self.batch, self.nodes,
                                            self.cutoff, *self.box, _p(self.row_ptr), int(src.numel()), _p(src),
                                            _p(dst), _stream()))
@@ -204,7 +225,7 @@ class NeighbourSearch:
     def cell_order(self):
         """int32 (batch*nodes): atom ids in cell order (a cache-friendly row order for the edge kernels)."""
         dev = self.x.device
-        with torch.cuda.device(dev):
+        with _on(dev):
             order = torch.empty(self.batch * self.nodes, dtype=torch.int32, device=dev)
             L.check(_lib.mg_neighbour_cell_order(_p(self.workspace), self.workspace.numel(), self.batch, self.nodes,
                                                  self.cutoff, *self.box, _p(order), _stream()))
@@ -222,7 +243,7 @@ def neighbour_edges(x, cutoff, box, capacity, out=None):
     B, N = int(x.size(0)), int(x.size(1))
     box = tuple(float(b) for b in box)
     dev = x.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         if out is None:
             nbytes = ctypes.c_size_t(0)
             L.check(_lib.mg_neighbour_workspace_bytes(B, N, float(cutoff), *box, ctypes.byref(nbytes)))
@@ -274,7 +295,7 @@ def get_neighbours(listmax, neighboursmax, cutoff, box_x, box_y, box_z, x):
     _check_caps(search, listmax, neighboursmax)
     _, dst = search.fill()
     B, N = search.batch, search.nodes
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         neighbours = torch.empty(B, N, neighboursmax, dtype=torch.int32, device=x.device)
         counts = torch.empty(B, N, dtype=torch.int32, device=x.device)
         L.check(_lib.mg_neighbour_pad(_p(search.row_ptr), _p(dst), B, N, neighboursmax, _p(neighbours),
@@ -285,7 +306,7 @@ def get_neighbours(listmax, neighboursmax, cutoff, box_x, box_y, box_z, x):
 def wrap_cells(cutoff, box, x):
     _check_input(x, "x")
     B, N = int(x.size(0)), int(x.size(1))
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         w = torch.empty_like(x)
         cell = torch.empty(B, N, dtype=torch.int32, device=x.device)
         L.check(_lib.mg_neighbour_wrap_cells(_p(x), B, N, float(cutoff), *[float(b) for b in box], _p(w),
@@ -309,7 +330,7 @@ def padded_edges_read(counts, neighbours, x):
     if not (N == neighbours.size(1) == x.size(1)):
         raise RuntimeError("node dimension of all tensors must match")
     nmax, chan = int(neighbours.size(2)), int(x.size(2))
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         out = torch.empty(B, N, nmax, chan, dtype=torch.float32, device=x.device)
         L.check(_lib.mg_padded_edges_read(_p(counts), _p(neighbours), _p(x), B, N, nmax, chan, _p(out), _stream()))
     return out
@@ -334,7 +355,7 @@ def padded_edges_reduce(counts, neighbours, x):
     if nmax != x.size(2):
         raise RuntimeError("neighboursmax dimension must match between neighbours and x")
     chan = int(x.size(3))
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         out = torch.empty(B, N, chan, dtype=torch.float32, device=x.device)
         L.check(_lib.mg_padded_edges_reduce(_p(counts), _p(x), B, N, nmax, chan, _p(out), _stream()))
     return out
@@ -346,7 +367,7 @@ def edge_vectors(pos, src, dst, box, want_shift=False):
     _check_input(src, "src", torch.int32)
     _check_input(dst, "dst", torch.int32)
     E = int(src.numel())
-    with torch.cuda.device(pos.device):
+    with _on(pos.device):
         r = torch.empty(E, 3, dtype=torch.float32, device=pos.device)
         shift = torch.empty(E, 3, dtype=torch.int8, device=pos.device) if want_shift else None
         L.check(_lib.mg_edge_vectors(_p(pos), _p(src), _p(dst), E, *[float(b) for b in box], _p(r), _p(shift),
@@ -359,7 +380,7 @@ def segment_row_ptr(index, n_rows):
     if index.dtype not in (torch.int32, torch.int64):
         raise RuntimeError("index must be int32 or int64")
     _check_input(index, "index", index.dtype)
-    with torch.cuda.device(index.device):
+    with _on(index.device):
         row_ptr = torch.empty(n_rows + 1, dtype=torch.int32, device=index.device)
         L.check(_lib.mg_segment_row_ptr(_p(index), int(index.dtype == torch.int64), int(index.numel()), int(n_rows),
                                         _p(row_ptr), _stream()))
@@ -379,7 +400,7 @@ def segment_sum_csr(x_edge, row_ptr, n_rows, perm=None):
     feat = 1
     for d in rest:
         feat *= int(d)
-    with torch.cuda.device(x_edge.device):
+    with _on(x_edge.device):
         out = torch.empty((n_rows,) + rest, dtype=torch.float32, device=x_edge.device)
         L.check(_lib.mg_segment_sum_csr_perm(_p(x_edge), _p(perm), _p(row_ptr), int(n_rows), feat, _p(out), _stream()))
     return out
@@ -396,7 +417,7 @@ def gather_rows(x, index):
     for d in rest:
         feat *= int(d)
     E = int(index.numel())
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         out = torch.empty((E,) + rest, dtype=torch.float32, device=x.device)
         L.check(_lib.mg_gather_rows(_p(x), _p(index), int(index.dtype == torch.int64), E, int(x.size(0)), feat,
                                     _p(out), _stream()))
@@ -433,7 +454,7 @@ def bee_fwd(l_0, l_1, l_2, r_0, r_1, r_2):
     if rows2 != rows or chan2 != chan:
         raise RuntimeError("left and right operands must agree on batch and channel sizes")
     dev = l_0.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         ys = [torch.empty(_shape(rows, chan, int(lab[2])), dtype=torch.float32, device=dev) for lab in BEE_ORDER]
         arr = L.PtrArray13(*[y.data_ptr() for y in ys])
         L.check(_lib.mg_bee_fwd(_p(l_0), _p(l_1), _p(l_2), _p(r_0), _p(r_1), _p(r_2), rows, chan,
@@ -450,7 +471,7 @@ def _bee_bwd(side, o_0, o_1, o_2, dys):
         if tuple(dy.shape) != _shape(rows, chan, int(lab[2])):
             raise RuntimeError(f"dy_{lab} has wrong shape")
     dev = o_0.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         d = [torch.empty(_shape(rows, chan, k), dtype=torch.float32, device=dev) for k in range(3)]
         arr = L.PtrArray13(*[dy.data_ptr() for dy in dys])
         L.check(_lib.mg_bee_bwd(side, _p(o_0), _p(o_1), _p(o_2), ctypes.byref(arr), rows, chan, _p(d[0]),
@@ -466,7 +487,7 @@ def bee_edge_filters_fwd(enc, rh):
     E, chan = int(enc.size(0)), int(enc.size(1))
     if enc.dim() != 2 or tuple(rh.shape) != (E, 3):
         raise RuntimeError("expected enc (E, chan) and rh (E, 3)")
-    with torch.cuda.device(enc.device):
+    with _on(enc.device):
         phi_v = torch.empty(E, chan, 3, dtype=torch.float32, device=enc.device)
         phi_d = torch.empty(E, chan, 3, 3, dtype=torch.float32, device=enc.device)
         L.check(_lib.mg_bee_edge_filters_fwd(_p(enc), _p(rh), E, chan, _p(phi_v), _p(phi_d), _stream()))
@@ -480,7 +501,7 @@ def bee_edge_filters_bwd(enc, rh, g_v, g_d):
     E, chan = int(enc.size(0)), int(enc.size(1))
     if tuple(rh.shape) != (E, 3) or tuple(g_v.shape) != (E, chan, 3) or tuple(g_d.shape) != (E, chan, 3, 3):
         raise RuntimeError("expected rh (E, 3), g_v (E, chan, 3), g_d (E, chan, 3, 3)")
-    with torch.cuda.device(enc.device):
+    with _on(enc.device):
         d_enc, d_rh = torch.empty_like(enc), torch.empty_like(rh)
         L.check(_lib.mg_bee_edge_filters_bwd(_p(enc), _p(rh), _p(g_v), _p(g_d), E, chan, _p(d_enc), _p(d_rh), _stream()))
     return d_enc, d_rh
@@ -498,7 +519,7 @@ def silu_order(z, order, mul=None):
             raise RuntimeError("mul must have the shape of z")
     if not 0 <= int(order) <= SILU_MAX_ORDER:
         raise RuntimeError(f"silu_order: order must be in 0..{SILU_MAX_ORDER}")
-    with torch.cuda.device(z.device):
+    with _on(z.device):
         out = torch.empty_like(z)
         L.check(_lib.mg_silu_order(_p(z), _p(mul) if mul is not None else None, z.numel(), int(order), _p(out), _stream()))
     return out
@@ -516,7 +537,7 @@ def bee_fwd_indexed(l_0, l_1, l_2, l_index, r_0, r_1, r_2):
     if chan2 != chan or l_index.numel() != rows:
         raise RuntimeError("operands must agree on the channel size and l_index must have one entry per row")
     dev = r_0.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         ys = [torch.empty(_shape(rows, chan, int(lab[2])), dtype=torch.float32, device=dev) for lab in BEE_ORDER]
         arr = L.PtrArray13(*[y.data_ptr() for y in ys])
         L.check(_lib.mg_bee_fwd_indexed(_p(l_0), _p(l_1), _p(l_2), _p(l_index), n_l, _p(r_0), _p(r_1), _p(r_2), rows,
@@ -549,7 +570,7 @@ def bee_bwd_indexed(side, o_0, o_1, o_2, o_index, dys, dy_index, rows):
             if idx.numel() != rows:
                 raise RuntimeError(f"{name} must have one entry per product row")
     dev = o_0.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         d = [torch.empty(_shape(rows, chan, k), dtype=torch.float32, device=dev) for k in range(3)]
         arr = L.PtrArray13(*[dy.data_ptr() for dy in dys])
         L.check(_lib.mg_bee_bwd_indexed(side, _p(o_0), _p(o_1), _p(o_2), _p(o_index), n_o, ctypes.byref(arr),
@@ -577,7 +598,7 @@ def _cow_inputs(l_0, l_1, r_0, r_1):
 def cow_o0_fwd(l_0, l_1, r_0, r_1):
     rows, chan = _cow_inputs(l_0, l_1, r_0, r_1)
     dev = l_0.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         y0 = torch.empty(rows, chan, dtype=torch.float32, device=dev)
         y1 = torch.empty(rows, chan, dtype=torch.float32, device=dev)
         L.check(_lib.mg_cow_o0_fwd(_p(l_0), _p(l_1), _p(r_0), _p(r_1), rows, chan, _p(y0), _p(y1), _stream()))
@@ -587,7 +608,7 @@ def cow_o0_fwd(l_0, l_1, r_0, r_1):
 def cow_o1_fwd(l_0, l_1, r_0, r_1):
     rows, chan = _cow_inputs(l_0, l_1, r_0, r_1)
     dev = l_0.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         ys = [torch.empty(rows, chan, 3, dtype=torch.float32, device=dev) for _ in range(3)]
         L.check(_lib.mg_cow_o1_fwd(_p(l_0), _p(l_1), _p(r_0), _p(r_1), rows, chan, _p(ys[0]), _p(ys[1]),
                                    _p(ys[2]), _stream()))
@@ -604,7 +625,7 @@ def _cow_bwd(which, side, o_0, o_1, dys):
         if tuple(dy.shape) != _shape(rows, chan, rk):
             raise RuntimeError(f"dy[{k}] has wrong shape")
     dev = o_0.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         d0 = torch.empty(rows, chan, dtype=torch.float32, device=dev)
         d1 = torch.empty(rows, chan, 3, dtype=torch.float32, device=dev)
         if which == 0:
@@ -688,7 +709,7 @@ def _ant16(rank_o, x_0, x_1, x_2, pairs):
     labels = (ctypes.c_int * n)(*[BEE_ORDER.index(lab) for lab, _, _ in pairs])
     Ps = (ctypes.c_void_p * n)(*[P.data_ptr() for _, P, _ in pairs])
     lefts = (ctypes.c_void_p * n)(*[left.data_ptr() for _, _, left in pairs])
-    with torch.cuda.device(dev):
+    with _on(dev):
         y = torch.empty(_shape(batch, dims[rank_o], rank_o), dtype=torch.float32, device=dev)
         if batch > 0:
             L.check(_lib.mg_ant16_fwd(rank_o, n, labels, Ps, lefts, _p(x_0), _p(x_1), _p(x_2), batch,
@@ -753,7 +774,7 @@ def ant16_grad_x(rank_r, dys, terms):
     labels = (ctypes.c_int * n)(*[BEE_ORDER.index(lab) for lab, _, _ in terms])
     Ps = (ctypes.c_void_p * n)(*[P.data_ptr() for _, P, _ in terms])
     lefts = (ctypes.c_void_p * n)(*[left.data_ptr() for _, _, left in terms])
-    with torch.cuda.device(dev):
+    with _on(dev):
         dx = torch.empty(_shape(batch, dims[rank_r], rank_r), dtype=torch.float32, device=dev)
         if dx.numel() > 0:
             L.check(_lib.mg_ant16_grad_x(rank_r, n, labels, Ps, lefts, _p(dys[0]), _p(dys[1]), _p(dys[2]), batch,
@@ -789,7 +810,7 @@ def ant16_grad_left(label, P, x, dy):
     (ant16_o*_backleft_cuda, extensions/codegen_tensops/codegen_tensops.cpp:892-1070)."""
     P, x, dy = P.contiguous(), x.contiguous(), dy.contiguous()
     batch, dims, dim_l = _ant16_one(label, P, x, dy)
-    with torch.cuda.device(P.device):
+    with _on(P.device):
         dleft = torch.empty(_shape(batch, dim_l, int(label[0])), dtype=torch.float32, device=P.device)
         if dleft.numel() > 0:
             L.check(_lib.mg_ant16_grad_left(BEE_ORDER.index(label), _p(P), _p(x), _p(dy), batch, dims[0], dims[1],
@@ -804,7 +825,7 @@ def ant16_grad_weight(label, left, x, dy):
     left, x, dy = left.contiguous(), x.contiguous(), dy.contiguous()
     batch, dims, dim_l = _ant16_one(label, None, x, dy, left=left)
     dim_r, dim_o = dims[int(label[1])], dims[int(label[2])]
-    with torch.cuda.device(left.device):
+    with _on(left.device):
         dP = torch.empty(dim_o, dim_l, dim_r, dtype=torch.float32, device=left.device)
         if dP.numel() > 0:
             nbytes = ctypes.c_size_t(0)
@@ -828,7 +849,7 @@ def tensor_prod_bare(inds_l, inds_r, inds_o, x_l, x_r):
     n = 1
     for d in lead_l:
         n *= int(d)
-    with torch.cuda.device(x_l.device):
+    with _on(x_l.device):
         y = torch.empty(lead_l + (3,) * inds_o, dtype=torch.float32, device=x_l.device)
         L.check(_lib.mg_tensor_prod_bare(inds_l, inds_r, inds_o, _p(x_l), _p(x_r), n, 1, _p(y), _stream()))
     return y
@@ -859,7 +880,7 @@ def tensor_prods(inds_l, inds_r, inds_o, W_l, W_r, W_o, x_l, x_r):
     rows = 1
     for d in lead:
         rows *= int(d)
-    with torch.cuda.device(x_l.device):
+    with _on(x_l.device):
         y = torch.empty(lead + (dim_o,) + (3,) * inds_o, dtype=torch.float32, device=x_l.device)
         L.check(_lib.mg_tensor_prods(inds_l, inds_r, inds_o, _p(Ws[0]), Ws[0].stride(0), _p(Ws[1]), Ws[1].stride(0),
                                      _p(Ws[2]), Ws[2].stride(0), _p(x_l), _p(x_r), rows, dim_l, dim_r, rank, dim_o,
@@ -875,7 +896,7 @@ def tensor_prods_avd(a, v_l, v_r):
         raise RuntimeError("shape mismatch")
     n = int(a.numel())
     dev = a.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         y0 = torch.empty_like(a)
         y1 = torch.empty_like(v_l)
         y2 = torch.empty(tuple(v_l.shape) + (3,), dtype=torch.float32, device=dev)
@@ -954,7 +975,7 @@ def _packed(W, kind):
     size_fn, pack_fn = ((_lib.mg_linear_packed_weight_bytes, _lib.mg_linear_pack_weight) if kind == "bf16x3" else
                         (_lib.mg_linear_f16x2_packed_weight_bytes, _lib.mg_linear_f16x2_pack_weight))
     L.check(size_fn(dim_in, dim_out, ctypes.byref(nbytes)))
-    with torch.cuda.device(W.device):
+    with _on(W.device):
         packed = torch.empty(nbytes.value, dtype=torch.uint8, device=W.device)
         L.check(pack_fn(_p(W), int(W.stride(0)), int(W.stride(1)), dim_in, dim_out, _p(packed), _stream()))
     if len(_packed_cache) > 4096:
@@ -999,7 +1020,7 @@ def row_absmax(x):
     _check_input(x, "x")
     if x.dim() != 2:
         raise RuntimeError("x must have two dims")
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         out = torch.empty(x.size(0), 1, dtype=torch.float32, device=x.device)
         L.check(_lib.mg_row_absmax(_p(x), int(x.size(0)), int(x.size(1)), _p(out), _stream()))
     return out
@@ -1014,7 +1035,7 @@ def linear_f64(W, bias, x, act=ACT_NONE):
         _check_input(bias, "bias")
     if x.dim() != 2 or W.dim() != 2 or W.size(1) != x.size(1) or (bias is not None and bias.numel() != W.size(0)):
         raise RuntimeError("linear_f64: x (rows, dim_in), W (dim_out, dim_in), bias (dim_out)")
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         y = torch.empty(x.size(0), W.size(0), dtype=torch.float64, device=x.device)
         L.check(_lib.mg_linear_f64(_p(W), _p(bias) if bias is not None else None, _p(x), int(x.size(0)),
                                    int(W.size(1)), int(W.size(0)), int(act), _p(y), _stream()))
@@ -1143,7 +1164,7 @@ def tensor_linear_f16x2(W, x, x_rowmax=None, bias=None, act=ACT_NONE, out=None, 
     if rows % out_comps != 0:
         raise RuntimeError("rows must be a multiple of out_comps")
     y_shape = [rows, dim_out] if out_comps == 1 else [rows // out_comps, dim_out, out_comps]
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         if out is None:
             y = torch.empty(y_shape, dtype=torch.float32, device=x.device)
         else:
@@ -1181,7 +1202,7 @@ def components_as_rows(inds, x):
     k_pad = (dim_in + 31) // 32 * 32
     if get_linear_mode() != LINEAR_F16X2 or rows * T < 32768 or k_pad > 256 or k_pad & (k_pad - 1):
         return None
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         x2 = torch.empty(rows * T, k_pad, dtype=torch.float32, device=x.device)
         x2max = torch.empty(rows * T, 1, dtype=torch.float32, device=x.device)
         L.check(_lib.mg_components_to_rows(_p(x), rows, dim_in, T, k_pad, _p(x2), _p(x2max), _stream()))
@@ -1233,7 +1254,7 @@ def tensor_linear_fwd(inds, W, x, bias=None, act=ACT_NONE, out=None, accumulate=
         _check_input(bias, "bias")
         if bias.numel() != dim_out:
             raise RuntimeError("bias size mismatch")
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         if out is None:
             y = torch.empty(y_shape, dtype=torch.float32, device=x.device)
         else:
@@ -1315,7 +1336,7 @@ def tensor_linear_wgrad(inds, dy, x, dy_bound=None, x_bound=None, want_bias=Fals
     rows = 1
     for i in range(batch_dims):
         rows *= int(x.size(i))
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         dW = torch.empty(dim_out, dim_in, dtype=torch.float32, device=x.device)
         db = None
         nbytes = ctypes.c_size_t(0)
@@ -1394,7 +1415,7 @@ def tensor_linear_bf16(W, x, bias=None, act=ACT_NONE, out=None, accumulate=False
     if bias is not None and (bias.dtype != torch.float32 or not bias.is_contiguous() or bias.numel() != dim_out):
         raise RuntimeError("bias must be a contiguous float32 tensor of dim_out elements")
     shape = (rows, dim_out) if out_comps == 1 else (rows // out_comps, dim_out, out_comps)
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         if out is None:
             if accumulate:
                 raise RuntimeError("accumulate needs out")
@@ -1424,7 +1445,7 @@ def bee_message_bf16(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_ord
         raise RuntimeError("row_ptr (nodes+1) and dst must be int32")
     if node_order is not None and (node_order.dtype != torch.int32 or node_order.numel() != N):
         raise RuntimeError("node_order must be int32 with one entry per node")
-    with torch.cuda.device(La.device):
+    with _on(La.device):
         P0 = torch.empty(E, 3, chan, dtype=torch.bfloat16, device=La.device)
         S1 = torch.empty(N, 3, 5, chan, dtype=torch.bfloat16, device=La.device)
         S2 = torch.empty(N, 9, 5, chan, dtype=torch.bfloat16, device=La.device)
@@ -1447,7 +1468,7 @@ def bee_node_products(l0, l1, l2, r0, r1, r2, want_node_max=False):
         want = (N, chan) if comps is None else (N, comps, chan)
         if tuple(t.shape) != want:
             raise RuntimeError("operands must be (nodes, chan), (nodes, 3, chan), (nodes, 9, chan)")
-    with torch.cuda.device(l0.device):
+    with _on(l0.device):
         P0 = torch.empty(N, 3, chan, dtype=l0.dtype, device=l0.device)
         P1 = torch.empty(N, 3, 5, chan, dtype=l0.dtype, device=l0.device)
         P2 = torch.empty(N, 9, 5, chan, dtype=l0.dtype, device=l0.device)
@@ -1484,7 +1505,7 @@ def tensor_linear_bf16_rowsum(W, x, row_ptr, seg, n_out, bias=None, act=ACT_NONE
         raise RuntimeError("bias must be a contiguous float32 tensor of dim_out elements")
     nbytes = ctypes.c_size_t(0)
     L.check(_lib.mg_tensor_linear_bf16_rowsum_workspace_bytes(rows, dim_out, ctypes.byref(nbytes)))
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         out = torch.empty(n_out, dim_out, dtype=torch.float32, device=x.device)
         y = torch.empty(rows, dim_out, dtype=torch.bfloat16, device=x.device) if want_rows else None
         work = torch.empty(nbytes.value // 4, dtype=torch.float32, device=x.device)
@@ -1516,7 +1537,7 @@ def mlp_chain_bf16(Y, x, W1, b1, W2, b2, row_ptr, seg, n_out, act=ACT_LEAKY):
         raise RuntimeError("seg must have one entry per row and row_ptr n_out + 1 entries")
     nbytes = ctypes.c_size_t(0)
     L.check(_lib.mg_mlp_chain_bf16_workspace_bytes(rows, ctypes.byref(nbytes)))
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         s_psi = torch.empty(n_out, 128, dtype=torch.float32, device=x.device)
         s_h = torch.empty(n_out, 256, dtype=torch.float32, device=x.device)
         work = torch.empty(nbytes.value // 4, dtype=torch.float32, device=x.device)
@@ -1546,7 +1567,7 @@ def tens_group_norm_bf16(y, batch, groups, gamma, eps, res=None):
         raise RuntimeError("rows must be a multiple of batch and gamma must have chan entries")
     nbytes = ctypes.c_size_t(0)
     L.check(_lib.mg_tens_group_norm_bf16_scratch_bytes(int(batch), int(groups), ctypes.byref(nbytes)))
-    with torch.cuda.device(y.device):
+    with _on(y.device):
         out = torch.empty_like(y)
         scratch = torch.empty((nbytes.value + 7) // 8, dtype=torch.float64, device=y.device)
         L.check(_lib.mg_tens_group_norm_bf16(_p(y), _p(res), int(batch), rows // batch, comps, chan, int(groups), float(eps),
@@ -1562,7 +1583,7 @@ def segment_sum_csr_bf16(x_edge, row_ptr, n_rows, scale=1.0):
     if row_ptr.dtype != torch.int32 or row_ptr.numel() != n_rows + 1:
         raise RuntimeError("row_ptr must be int32 with n_rows + 1 entries")
     feat = int(x_edge.size(1))
-    with torch.cuda.device(x_edge.device):
+    with _on(x_edge.device):
         out = torch.empty(n_rows, feat, dtype=torch.bfloat16, device=x_edge.device)
         L.check(_lib.mg_segment_sum_csr_bf16(_p(x_edge), _p(row_ptr), int(n_rows), feat, float(scale), _p(out),
                                              _stream()))
@@ -1576,7 +1597,7 @@ def painn_radial_encode(r_ij, n, rmax):
     if r_ij.dim() != 2 or r_ij.size(1) != 3:
         raise RuntimeError("r_ij must have shape (edges, 3)")
     E = int(r_ij.size(0))
-    with torch.cuda.device(r_ij.device):
+    with _on(r_ij.device):
         out = torch.empty(E, n, dtype=torch.float32, device=r_ij.device)
         L.check(_lib.mg_painn_radial_encode(_p(r_ij), E, int(n), float(rmax), _p(out), _stream()))
     return out
@@ -1602,7 +1623,7 @@ def painn_radial_linear(r_ij, n, rmax, W, bias=None, act=ACT_NONE):
                              or bias.numel() != W.size(0)):
         raise RuntimeError("bias must be a contiguous float32 CUDA tensor of dim_out elements")
     E, O = int(r_ij.size(0)), int(W.size(0))
-    with torch.cuda.device(r_ij.device):
+    with _on(r_ij.device):
         y = torch.empty(E, O, dtype=torch.float32, device=r_ij.device)
         L.check(_lib.mg_painn_radial_linear(_p(r_ij), E, int(n), float(rmax), _p(W), W.stride(0), W.stride(1),
                                             _p(bias) if bias is not None else None, O, int(act), _p(y), _stream()))
@@ -1637,7 +1658,7 @@ def painn_combine_fwd(dist, actv, v, direction, node=None, terms=15):
     edge e reads row node[e] (the reference's edges_read_dst folded in).  terms: mask of the four terms that take part
     (15: all; include/managan_hip.h)."""
     E, n, rows = _combine_inputs(dist, actv, v, direction, node)
-    with torch.cuda.device(v.device):
+    with _on(v.device):
         m = torch.empty(E, n, 3, dtype=torch.float32, device=v.device)
         a = torch.empty(E, n, dtype=torch.float32, device=v.device)
         L.check(_lib.mg_painn_combine_fwd(_p(dist), _p(actv), _p(v), _p(direction), _p(node), rows, E, n, int(terms),
@@ -1660,7 +1681,7 @@ def painn_combine_bwd(dist, actv, v, direction, dm, da, node=None, grad_row=None
             raise RuntimeError("grad_row must have one entry per edge")
     if tuple(dm.shape) != (g_rows, n, 3) or tuple(da.shape) != (g_rows, n):
         raise RuntimeError("expected dm (rows, n, 3) and da (rows, n)")
-    with torch.cuda.device(v.device):
+    with _on(v.device):
         # (want: which of the four gradients to compute; the others come back as None)
         d_dist = torch.empty_like(dist) if want[0] else None
         d_actv = torch.empty(E, 4 * n, dtype=torch.float32, device=v.device) if want[1] else None
@@ -1689,7 +1710,7 @@ def painn_combine_bwd_grid(table, period, d, actv, v, direction, dm, da, node, g
     g_rows = int(dm.size(0))
     if tuple(dm.shape) != (g_rows, n, 3) or tuple(da.shape) != (g_rows, n):
         raise RuntimeError("expected dm (rows, n, 3) and da (rows, n)")
-    with torch.cuda.device(v.device):
+    with _on(v.device):
         d_dist = torch.empty(E, 4 * n, dtype=torch.float32, device=v.device) if want[0] else None
         d_actv = torch.empty(E, 4 * n, dtype=torch.float32, device=v.device) if want[1] else None
         dv = torch.empty(E, n, 3, dtype=torch.float32, device=v.device) if want[2] else None
@@ -1733,7 +1754,7 @@ def painn_combine_bwd_rows(dist, actv, v, direction, dm, da, row_ptr, order, gra
     g_rows = int(dm.size(0))
     if tuple(dm.shape) != (g_rows, n, 3) or tuple(da.shape) != (g_rows, n) or (grad_row is None and g_rows != E):
         raise RuntimeError("expected dm (rows, n, 3) and da (rows, n)")
-    with torch.cuda.device(v.device):
+    with _on(v.device):
         d_dist = torch.empty(E, 4 * n, dtype=torch.float32, device=v.device) if want[0] else None
         d_actv = torch.empty(rows, 4 * n, dtype=torch.float32, device=v.device) if want[1] else None
         dv = torch.empty(rows, n, 3, dtype=torch.float32, device=v.device) if want[2] else None
@@ -1761,7 +1782,7 @@ def painn_table_interp_fwd(table, d, period, order=0):
     """(edges, cols): the grid `table` of a function of period `period`, interpolated at the lengths d (4-point
     Lagrange, as the inference kernels do); order 1 .. 3: the interpolant's derivative of that order in d."""
     rows, cols, E = _table_inputs(table, d)
-    with torch.cuda.device(d.device):
+    with _on(d.device):
         out = torch.empty(E, cols, dtype=torch.float32, device=d.device)
         L.check(_lib.mg_painn_table_interp_fwd(_p(table), rows, cols, float(period), _p(d), E, int(order), _p(out),
                                                _stream()))
@@ -1773,7 +1794,7 @@ def painn_table_sorted_edges(d, table_rows, period):
     pointer of the sorted rows: what painn_table_interp_bwd sums by."""
     _check_input(d, "d")
     E = int(d.numel())
-    with torch.cuda.device(d.device):
+    with _on(d.device):
         bucket = torch.empty(E, dtype=torch.int32, device=d.device)
         L.check(_lib.mg_painn_table_buckets(_p(d), E, int(table_rows), float(period), _p(bucket), _stream()))
         ordered, perm = torch.sort(bucket, stable=True)
@@ -1795,7 +1816,7 @@ def painn_table_interp_bwd(g, table, d, period, perm, bucket_ptr, want_length_gr
     _check_input(bucket_ptr, "bucket_ptr", torch.int32)
     if tuple(g.shape) != (E, cols) or perm.numel() != E or bucket_ptr.numel() != rows + 1:
         raise RuntimeError("expected g (edges, cols), perm (edges), bucket_ptr (rows + 1)")
-    with torch.cuda.device(d.device):
+    with _on(d.device):
         nbytes = ctypes.c_size_t(0)
         L.check(_lib.mg_painn_table_interp_bwd_workspace_bytes(rows, cols, ctypes.byref(nbytes)))
         ws = torch.empty(nbytes.value, dtype=torch.uint8, device=d.device)
@@ -1836,7 +1857,7 @@ def painn_message(row_ptr, dst, r_ij, filt, actv, x_v, epsilon, res_a=None, res_
         if node_order.numel() != n_nodes:
             raise RuntimeError("node_order must have one entry per node")
     dev = x_v.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         out_a = torch.empty(n_nodes, n, dtype=torch.float32, device=dev)
         out_v = torch.empty(n_nodes, n, 3, dtype=torch.float32, device=dev)
         L.check(_lib.mg_painn_message(_p(row_ptr), _p(dst), _p(node_order), n_nodes, E, _p(r_ij), _p(filt), _p(actv), _p(x_v), n,
@@ -1873,7 +1894,7 @@ def painn_table_message(row_ptr, dst, r_ij, table, period, actv, x_v, epsilon, r
         if node_order.numel() != n_nodes:
             raise RuntimeError("node_order must have one entry per node")
     dev = x_v.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         out_a = torch.empty(n_nodes, n, dtype=torch.float32, device=dev)
         out_v = torch.empty(n_nodes, n, 3, dtype=torch.float32, device=dev)
         L.check(_lib.mg_painn_table_message(_p(row_ptr), _p(dst), _p(node_order), n_nodes, E, _p(r_ij), _p(table),
@@ -1900,7 +1921,7 @@ def painn_edge_records(r_ij, table_rows, period, epsilon):
     E = int(r_ij.size(0))
     if tuple(r_ij.shape) != (E, 3):
         raise RuntimeError("r_ij must have shape (edges, 3)")
-    with torch.cuda.device(r_ij.device):
+    with _on(r_ij.device):
         rec = torch.empty(E, 8, dtype=torch.float32, device=r_ij.device)
         L.check(_lib.mg_painn_edge_records(_p(r_ij), E, int(table_rows), float(period), float(epsilon), _p(rec), _stream()))
     return rec
@@ -1946,7 +1967,7 @@ def painn_table_message_sliced(row_ptr, dst, r_ij, table, period, actv_sliced, x
         if tuple(records.shape) != (E, 8):
             raise RuntimeError("records must have shape (edges, 8)")
     dev = x_v.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         out_a = torch.empty(n_nodes, n, dtype=torch.float32, device=dev)
         out_v = torch.empty(n_nodes, n, 3, dtype=torch.float32, device=dev)
         L.check(_lib.mg_painn_table_message_sliced(_p(row_ptr), _p(dst), _p(node_order), n_nodes, E, _p(records),
@@ -1981,7 +2002,7 @@ def bee_products_linear(rank_o, W, l0, l1, l2, r0, r1, r2, node_bound):
     k_order = 1 if (rank_o == 2 and dim_out <= 64) else 0
     if k_order:
         W = _channel_block_major_columns(W, n_types, chan)
-    with torch.cuda.device(l0.device):
+    with _on(l0.device):
         y = torch.empty((N, dim_out) + (3,) * rank_o, dtype=torch.float32, device=l0.device)
         L.check(_lib.mg_bee_products_linear(int(rank_o), _p(l0), _p(l1), _p(l2), _p(r0), _p(r1), _p(r2), _p(node_bound),
                                             N, chan, _p(packed_weight_f16x2(W)), k_order, dim_out, _p(y), _stream()))
@@ -2039,7 +2060,7 @@ def tensor_linear_f16x2_rowsum(W, x, x_bound, row_ptr, seg, n_out, bias=None, ac
     dev = x.device
     nbytes = ctypes.c_size_t(0)
     L.check(_lib.mg_tensor_linear_f16x2_rowsum_workspace_bytes(rows, dim_out, ctypes.byref(nbytes)))
-    with torch.cuda.device(dev):
+    with _on(dev):
         out = torch.empty(n_out, dim_out, dtype=torch.float32, device=dev)
         y = torch.empty(rows, dim_out, dtype=torch.float32, device=dev) if want_rows else None
         work = torch.empty(nbytes.value // 4, dtype=torch.float32, device=dev)
@@ -2093,7 +2114,7 @@ def painn_filter_hidden(r_ij, rmax, W1, b1, W2, b2, h1_bound):
     if b1 is not None:
         _check_input(b1, "b1")
     E = int(r_ij.size(0))
-    with torch.cuda.device(r_ij.device):
+    with _on(r_ij.device):
         y = torch.empty(E, hidden, dtype=torch.float32, device=r_ij.device)
         L.check(_lib.mg_painn_filter_hidden(_p(r_ij), E, float(rmax), _p(W1), int(W1.stride(0)), int(W1.stride(1)),
                                             _p(b1), _p(packed_weight_f16x2(_operand_order_columns(W2))), _p(b2), hidden,
@@ -2149,7 +2170,7 @@ def painn_filter_message(W3_perm, bias3_perm, h, h_bound, row_ptr, src, dst, r_i
     dev = x_v.device
     nbytes = ctypes.c_size_t(0)
     L.check(_lib.mg_painn_filter_message_workspace_bytes(E, n, ctypes.byref(nbytes)))
-    with torch.cuda.device(dev):
+    with _on(dev):
         out_a = torch.empty(n_nodes, n, dtype=torch.float32, device=dev)
         out_v = torch.empty(n_nodes, n, 3, dtype=torch.float32, device=dev)
         work = torch.empty(nbytes.value // 4, dtype=torch.float32, device=dev)
@@ -2168,7 +2189,7 @@ def bee_edge_geometry(r_ij, r0):
     if r_ij.dim() != 2 or r_ij.size(1) != 3:
         raise RuntimeError("r_ij must have shape (edges, 3)")
     E = int(r_ij.size(0))
-    with torch.cuda.device(r_ij.device):
+    with _on(r_ij.device):
         enc = torch.empty(E, 8, dtype=torch.float32, device=r_ij.device)
         rhat = torch.empty(E, 3, dtype=torch.float32, device=r_ij.device)
         L.check(_lib.mg_bee_edge_geometry(_p(r_ij), E, float(r0), _p(enc), _p(rhat), _stream()))
@@ -2192,7 +2213,7 @@ def _packed_rank2_weight(Y2, chan):
         return hit[3]
     nbytes = ctypes.c_size_t(0)
     L.check(_lib.mg_bee_rank2_weight_bytes(chan, ctypes.byref(nbytes)))
-    with torch.cuda.device(Y2.device):
+    with _on(Y2.device):
         packed = torch.empty(nbytes.value // 4, dtype=torch.float32, device=Y2.device)
         L.check(_lib.mg_bee_pack_rank2_weight(_p(Y2), int(Y2.stride(0)), chan, int(Y2.size(0)), _p(packed), _stream()))
     if len(_rank2_cache) > 256:
@@ -2230,7 +2251,7 @@ def bee_node_products_rank2(l0, l1, l2, r0, r1, r2, Y2, want_lower_ranks=False, 
     if not bee_rank2_supported(chan, Y2.size(0)):
         raise RuntimeError("the fused rank-2 linear needs chan = 64, 128 or 256 and dim_d <= 16")
     dim_d = int(Y2.size(0))
-    with torch.cuda.device(l0.device):
+    with _on(l0.device):
         out = torch.empty(N, dim_d, 9, dtype=torch.float32, device=l0.device)
         P0 = P1 = nmax = None
         if want_lower_ranks:
@@ -2279,7 +2300,7 @@ def bee_message(row_ptr, dst, rhat, enc, La, Lv, Ld, enc_W, enc_b, node_order=No
             raise RuntimeError("Y2 must be (dim_d, 5 chan) with unit stride along a row")
         if not bee_rank2_supported(chan, Y2.size(0)):
             raise RuntimeError("the fused rank-2 linear needs chan = 64, 128 or 256 and dim_d <= 16")
-    with torch.cuda.device(dev):
+    with _on(dev):
         P0 = torch.empty(E, 3, chan, dtype=torch.float32, device=dev)
         S1 = torch.empty(N, 3, 5, chan, dtype=torch.float32, device=dev)
         node_max = torch.empty(N, (chan + 63) // 64, dtype=torch.float32, device=dev) if want_node_max else None
@@ -2355,7 +2376,7 @@ def group_norm(mode, x, groups, gamma, beta=None, eps=1e-5, mul=None, add=None, 
             raise RuntimeError("res has wrong shape")
     nbytes = ctypes.c_size_t(0)
     L.check(_lib.mg_group_norm_scratch_bytes(B, int(groups), ctypes.byref(nbytes)))
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         scratch = torch.empty(max(nbytes.value, 8), dtype=torch.uint8, device=x.device)
         out = torch.empty(tuple(x.shape), dtype=torch.float32, device=x.device)
         L.check(_lib.mg_group_norm(int(mode), _p(x), xs, _p(mul), ms, B, N, chan, int(groups), comps, float(eps),
@@ -2366,7 +2387,7 @@ def group_norm(mode, x, groups, gamma, beta=None, eps=1e-5, mul=None, add=None, 
 def tens_sigmoid(inds, x):
     _check_input(x, "x")
     T = 3 ** inds
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         out = torch.empty_like(x)
         L.check(_lib.mg_tens_sigmoid(int(inds), _p(x), int(x.numel()) // T, _p(out), _stream()))
     return out
@@ -2388,7 +2409,7 @@ def painn_update_pre(lrv, x_a, want_rowmax=False):
     _check_input(x_a, "x_a")
     rows, n = int(x_a.shape[0]), int(x_a.shape[1])
     layout = _lrv_layout(lrv, rows, n)
-    with torch.cuda.device(x_a.device):
+    with _on(x_a.device):
         ip = torch.empty(rows, n, dtype=torch.float32, device=x_a.device)
         cat = torch.empty(rows, 2 * n, dtype=torch.float32, device=x_a.device)
         rowmax = torch.empty(rows, 1, dtype=torch.float32, device=x_a.device) if want_rowmax and n <= 256 else None
@@ -2404,7 +2425,7 @@ def painn_update_vec(lrv, y, res_v=None):
     layout = _lrv_layout(lrv, rows, n)
     if res_v is not None:
         _check_input(res_v, "res_v")
-    with torch.cuda.device(y.device):
+    with _on(y.device):
         out = torch.empty(rows, n, 3, dtype=torch.float32, device=y.device)
         L.check(_lib.mg_painn_update_vec(_p(lrv), layout, _p(y), _p(res_v), rows, n, _p(out), _stream()))
     return out
@@ -2422,7 +2443,7 @@ def radial_encode(kind, r_ij, n, rmax):
     E = 1
     for d in lead:
         E *= int(d)
-    with torch.cuda.device(r_ij.device):
+    with _on(r_ij.device):
         out = torch.empty(lead + (n,), dtype=torch.float32, device=r_ij.device)
         L.check(_lib.mg_radial_encode(int(kind), _p(r_ij), E, int(n), float(rmax), _p(out), _stream()))
     return out
@@ -2439,7 +2460,7 @@ def displacement_sums(row_ptr, r_ij, phi, scale):
         raise RuntimeError("r_ij (edges, 3) and phi (edges, chan) expected")
     n_nodes, C = int(row_ptr.numel()) - 1, int(phi.size(1))
     dev = phi.device
-    with torch.cuda.device(dev):
+    with _on(dev):
         out_a = torch.empty(n_nodes, C, dtype=torch.float32, device=dev)
         out_v = torch.empty(n_nodes, C, 3, dtype=torch.float32, device=dev)
         out_d = torch.empty(n_nodes, C, 3, 3, dtype=torch.float32, device=dev)
@@ -2463,7 +2484,7 @@ def repel5_sim(x, v, drag, T, dt, nsteps, seed, first_kick=0):
         raise RuntimeError("Number of particles must match")
     if x.size(2) != 3 or v.size(2) != 3:
         raise RuntimeError("Position and velocity must be 3D")
-    with torch.cuda.device(x.device):
+    with _on(x.device):
         L.check(_lib.mg_repel5_sim(_p(x), _p(v), _p(drag), float(T), float(dt), int(nsteps), int(x.size(0)),
                                    int(x.size(1)), int(seed) & 0xFFFFFFFFFFFFFFFF, int(first_kick), _stream()))
 
