@@ -446,6 +446,13 @@ int mg_painn_message(const int* row_ptr /* n_nodes+1 */, const int* dst /* E */,
 int mg_painn_combine_supported(int n);   /* returns 0 / 1, not a status */
 int mg_painn_combine_fwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
                          long n_rows, long E, int n, int terms, float* m, float* a, mg_stream_t stream);
+/* mg_painn_combine_fwd with the sums over the edges of a source node inside: the edge arrays are sorted by that node and
+ * row_ptr (n_out_rows + 1) is their CSR; out_v (n_out_rows, n, 3) and out_a (n_out_rows, n) are the sums of m and a over
+ * each row's edges, added in edge order (the same on every run).  Replaces mg_painn_combine_fwd followed by two
+ * segment sums (torch_scatter.segment_coo at managan/graph_layers.py:54-59). */
+int mg_painn_combine_fwd_rows(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
+                              long n_rows, const int* row_ptr, long n_out_rows, long E, int n, int terms, float* out_v,
+                              float* out_a, mg_stream_t stream);
 int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
                          long n_rows, const float* dm, const float* da, const int* grad_row, long n_grad_rows, long E,
                          int n, int terms, float* d_dist, float* d_actv, float* dv, float* d_dir, mg_stream_t stream);

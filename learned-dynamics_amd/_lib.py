@@ -115,6 +115,7 @@ _SIGNATURES = {
     "mg_painn_table_interp_bwd_workspace_bytes": [i32, i32, ctypes.POINTER(ctypes.c_size_t)],
     "mg_painn_table_interp_bwd": [vp, vp, i32, i32, f32, vp, vp, vp, i64, i32, vp, vp, vp, vp],
     "mg_painn_combine_fwd": [vp, vp, vp, vp, vp, i64, i64, i32, i32, vp, vp, vp],
+    "mg_painn_combine_fwd_rows": [vp, vp, vp, vp, vp, i64, vp, i64, i64, i32, i32, vp, vp, vp],
     "mg_painn_combine_bwd": [vp, vp, vp, vp, vp, i64, vp, vp, vp, i64, i64, i32, i32, vp, vp, vp, vp, vp],
     "mg_painn_combine_bwd_rows": [vp, vp, i32, f32, vp, vp, vp, vp, vp, vp, i64, vp, vp, vp, i64, i64, i32, i32, vp, vp, vp,
                                   vp, vp],

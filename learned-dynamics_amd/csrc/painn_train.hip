@@ -82,10 +82,6 @@ __global__ void __launch_bounds__(256) painn_combine_fwd_kernel(const float* __r
     st4(a + e * n + c, make_float4(p3.x * k3, p3.y * k3, p3.z * k3, p3.w * k3));
 }
 
-// Adjoint: with p = dist actv and dp its gradient,
-//   dp[c] = dm[c] . v[c],  dp[n + c] = dm[c] . (v[c] x d),  dp[2n + c] = dm[c] . d,  dp[3n + c] = da[c]
-//   d_dist = dp actv,  d_actv = dp dist,  dv[c] = dm[c] p[c] + (d x dm[c]) p[n + c]
-//   d_dir = sum_c (dm[c] x v[c]) p[n + c] + dm[c] p[2n + c]
 // 4-point Lagrange weights on the grid rows i - 1 .. i + 2 at the fraction t (the grid kernels further down use them too)
 __device__ __forceinline__ void lagrange4(float t, float (&w)[4]) {
     const float tp = t + 1.0f, tm = t - 1.0f, tq = t - 2.0f;
@@ -98,6 +94,51 @@ __device__ __forceinline__ float4 fma4(float w, float4 a, float4 acc) {
     return make_float4(fmaf(w, a.x, acc.x), fmaf(w, a.y, acc.y), fmaf(w, a.z, acc.z), fmaf(w, a.w, acc.w));
 }
 
+// The same pass with the sums over the edges of a source node inside: a group of n / 4 threads owns an output row r
+// and walks its edges (positions row_ptr[r] .. row_ptr[r + 1] - 1 of the edge arrays, which are sorted by that row),
+// adds their m and a in that order and writes out_v[r], out_a[r] once: no per-edge m and a and no segment sums after.
+__global__ void __launch_bounds__(256) painn_combine_fwd_rows_kernel(
+    const float* __restrict__ dist, const float* __restrict__ actv, const float* __restrict__ v,
+    const float* __restrict__ dir, const int* __restrict__ node, long n_rows, const int* __restrict__ row_ptr,
+    long n_out_rows, long E, int n, int terms, float* __restrict__ out_v, float* __restrict__ out_a) {
+    const int tpe = n >> 2;
+    const long t = (long)blockIdx.x * 256 + threadIdx.x;
+    const long r = t / tpe;
+    if (r >= n_out_rows) return;
+    const int c = (int)(t - r * tpe) * 4;
+    const float k0 = (terms & 1) ? 1.f : 0.f, k1 = (terms & 2) ? 1.f : 0.f, k2 = (terms & 4) ? 1.f : 0.f;
+    const float k3 = (terms & 8) ? 1.f : 0.f;
+    Vec3x4 acc_m;
+#pragma unroll
+    for (int q = 0; q < 12; q++) acc_m.f[q] = 0.f;
+    float4 acc_a = make_float4(0.f, 0.f, 0.f, 0.f);
+    const long lo = max((long)row_ptr[r], 0L), hi = min((long)row_ptr[r + 1], E);
+    for (long e = lo; e < hi; e++) {
+        const long en = node ? min(max((long)node[e], 0L), n_rows - 1) : e;
+        const float* de = dist + e * 4 * n + c;
+        const float* ae = actv + en * 4 * n + c;
+        const float4 p0 = mul4(ld4(de), ld4(ae)), p1 = mul4(ld4(de + n), ld4(ae + n));
+        const float4 p2 = mul4(ld4(de + 2 * n), ld4(ae + 2 * n)), p3 = mul4(ld4(de + 3 * n), ld4(ae + 3 * n));
+        const Vec3x4 vv = ld12(v + (en * n + c) * 3);
+        const Vec3 d = {dir[3 * e], dir[3 * e + 1], dir[3 * e + 2]};
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const Vec3 x = vv.get(j), xd = cross(x, d);
+            const float s0 = at(p0, j) * k0, s1 = at(p1, j) * k1, s2 = at(p2, j) * k2;
+            acc_m.f[3 * j] += x.x * s0 + xd.x * s1 + d.x * s2;
+            acc_m.f[3 * j + 1] += x.y * s0 + xd.y * s1 + d.y * s2;
+            acc_m.f[3 * j + 2] += x.z * s0 + xd.z * s1 + d.z * s2;
+        }
+        acc_a.x += p3.x * k3; acc_a.y += p3.y * k3; acc_a.z += p3.z * k3; acc_a.w += p3.w * k3;
+    }
+    st12(out_v + (r * n + c) * 3, acc_m);
+    st4(out_a + r * n + c, acc_a);
+}
+
+// Adjoint: with p = dist actv and dp its gradient,
+//   dp[c] = dm[c] . v[c],  dp[n + c] = dm[c] . (v[c] x d),  dp[2n + c] = dm[c] . d,  dp[3n + c] = da[c]
+//   d_dist = dp actv,  d_actv = dp dist,  dv[c] = dm[c] p[c] + (d x dm[c]) p[n + c]
+//   d_dir = sum_c (dm[c] x v[c]) p[n + c] + dm[c] p[2n + c]
 // GRID: dist is a (mask + 1, 4n) grid of the filter over one period of the edge length and edge e interpolates its row
 // at len[e] (the arithmetic of table_interp_kernel, order 0): the per-edge filter is never stored.
 template <bool GRID>
@@ -596,6 +637,23 @@ int mg_painn_combine_fwd(const float* dist, const float* actv, const float* v, c
     hipLaunchKernelGGL(painn_combine_fwd_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
                        (hipStream_t)stream, dist, actv, v, dir, node, n_rows, E, n, terms, m, a);
     return check_launch("mg_painn_combine_fwd");
+}
+
+int mg_painn_combine_fwd_rows(const float* dist, const float* actv, const float* v, const float* dir, const int* node,
+                              long n_rows, const int* row_ptr, long n_out_rows, long E, int n, int terms, float* out_v,
+                              float* out_a, mg_stream_t stream) {
+    MG_REQUIRE(E >= 0 && n_out_rows >= 0 && combine_shape_ok(n), "mg_painn_combine_fwd_rows: n must be a power of two in 4..256");
+    MG_REQUIRE(terms >= 0 && terms <= 15, "mg_painn_combine_fwd_rows: terms is a mask of four bits");
+    if (n_out_rows == 0) return MG_OK;
+    MG_REQUIRE(row_ptr && out_v && out_a && (E == 0 || (dist && actv && v && dir)), "mg_painn_combine_fwd_rows: null pointer");
+    MG_REQUIRE(node == nullptr || n_rows > 0, "mg_painn_combine_fwd_rows: an index needs n_rows > 0");
+    MG_REQUIRE(aligned16(dist) && aligned16(actv) && aligned16(v) && aligned16(out_v) && aligned16(out_a),
+               "mg_painn_combine_fwd_rows: arrays must be 16-byte aligned");
+    const long threads = n_out_rows * (n / 4);
+    MG_REQUIRE(ceil_div(threads, 256) < (1L << 31), "mg_painn_combine_fwd_rows: too many rows");
+    hipLaunchKernelGGL(painn_combine_fwd_rows_kernel, dim3((unsigned)ceil_div(threads, 256)), dim3(256), 0,
+                       (hipStream_t)stream, dist, actv, v, dir, node, n_rows, row_ptr, n_out_rows, E, n, terms, out_v, out_a);
+    return check_launch("mg_painn_combine_fwd_rows");
 }
 
 int mg_painn_combine_bwd(const float* dist, const float* actv, const float* v, const float* dir, const int* node,

@@ -291,9 +291,9 @@ class _PainnCombine(torch.autograd.Function):
         ctx.save_for_backward(dist, actv_node, v_node, direction)
         ctx.save_for_forward(dist, actv_node, v_node, direction)
         ctx.set_materialize_grads(False)
-        m, a = ops.painn_combine_fwd(dist.contiguous(), actv_node.contiguous(), v_node.contiguous(),
-                                     direction.contiguous(), node=by_dst.index, terms=terms)
-        return (ops.segment_sum_csr(m, by_src.row_ptr, by_src.n_rows), ops.segment_sum_csr(a, by_src.row_ptr, by_src.n_rows))
+        # (the edges are sorted by their source node: its CSR is the row pointer of the sums)
+        return ops.painn_combine_fwd_rows(dist.contiguous(), actv_node.contiguous(), v_node.contiguous(),
+                                          direction.contiguous(), by_dst.index, by_src.row_ptr, by_src.n_rows, terms=terms)
 
     @staticmethod
     def jvp(ctx, dist_t, actv_t, v_t, dir_t, *_):

@@ -1666,6 +1666,21 @@ def painn_combine_fwd(dist, actv, v, direction, node=None, terms=15):
     return m, a
 
 
+def painn_combine_fwd_rows(dist, actv, v, direction, node, row_ptr, n_out_rows, terms=15):
+    """painn_combine_fwd with m and a summed over the edges of each CSR row inside the kernel (edges sorted by the row,
+    row_ptr (n_out_rows + 1) int32): (out_v (n_out_rows, n, 3), out_a (n_out_rows, n))."""
+    E, n, rows = _combine_inputs(dist, actv, v, direction, node)
+    _check_input(row_ptr, "row_ptr", torch.int32)
+    if row_ptr.numel() != n_out_rows + 1:
+        raise RuntimeError("row_ptr must have n_out_rows + 1 entries")
+    with _on(v.device):
+        out_v = torch.empty(n_out_rows, n, 3, dtype=torch.float32, device=v.device)
+        out_a = torch.empty(n_out_rows, n, dtype=torch.float32, device=v.device)
+        L.check(_lib.mg_painn_combine_fwd_rows(_p(dist), _p(actv), _p(v), _p(direction), _p(node), rows, _p(row_ptr),
+                                               int(n_out_rows), E, n, int(terms), _p(out_v), _p(out_a), _stream()))
+    return out_v, out_a
+
+
 def painn_combine_bwd(dist, actv, v, direction, dm, da, node=None, grad_row=None, terms=15, want=(True, True, True, True)):
     """Gradients of painn_combine_fwd's four inputs from those of its outputs; those of actv and v per edge
     ((E, 4n), (E, n, 3)) also when the inputs are per node.  grad_row (int32, one per edge): dm and da hold one row per

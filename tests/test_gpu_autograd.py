@@ -619,6 +619,25 @@ def test_combine_gradient_summed_per_row_inside_the_kernel(ops, n, E, nodes):
     assert int(node_sorted[0]) <= int(node_sorted[-1])
 
 
+@pytest.mark.parametrize("n, E, nodes, terms", [(32, 3000, 200, 15), (128, 4000, 50, 15), (4, 500, 700, 6), (256, 900, 5, 3)])
+def test_combine_summed_per_source_row_inside_the_kernel(ops, n, E, nodes, terms):
+    """mg_painn_combine_fwd_rows against mg_painn_combine_fwd followed by sums over the edges of a source node in
+    float64 (edges sorted by source; rows without edges give zeros)."""
+    g = torch.Generator().manual_seed(0x947 + 53 + n)
+    src = torch.sort(torch.randint(0, nodes, (E,), generator=g)).values.int().cuda()
+    row_ptr = ops.segment_row_ptr(src, nodes)
+    dist, actv = torch.randn(E, 4 * n, generator=g).cuda(), torch.randn(nodes, 4 * n, generator=g).cuda()
+    v = torch.randn(nodes, n, 3, generator=g).cuda()
+    direction = torch.nn.functional.normalize(torch.randn(E, 3, generator=g), dim=-1).cuda()
+    node = torch.randint(0, nodes, (E,), generator=g).int().cuda()
+    m, a = ops.painn_combine_fwd(dist, actv, v, direction, node=node, terms=terms)
+    ref_v = torch.zeros(nodes, n, 3, dtype=F64).index_add_(0, src.long().cpu(), m.double().cpu())
+    ref_a = torch.zeros(nodes, n, dtype=F64).index_add_(0, src.long().cpu(), a.double().cpu())
+    out_v, out_a = ops.painn_combine_fwd_rows(dist, actv, v, direction, node, row_ptr, nodes, terms=terms)
+    _close(out_v, ref_v, "out_v", 4e-6)
+    _close(out_a, ref_a, "out_a", 4e-6)
+
+
 def test_painn_message_through_its_grid_in_one_forward_kernel(pkg):
     """Message under autograd with edge vectors that are not differentiated: the forward pass is the inference kernel
     on the grid (differentiable._PainnGridMessage) and the backward pass interpolates the filter again.  Values and
