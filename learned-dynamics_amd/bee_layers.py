@@ -298,7 +298,7 @@ class DisplacementTensors(nn.Module):
     def forward(self, graph: Graph, r_ij):
         """r_ij (edges, 3) -> A_a (batch, nodes, dim_a), A_v (batch, nodes, dim_v, 3), A_d (batch, nodes, dim_d, 3, 3)."""
         if diff.wants_grad(self, r_ij):
-            raise RuntimeError("DisplacementTensors has no differentiable path: call it under torch.no_grad()")
+            return diff.displacement_tensors(self, graph, r_ij)
         r_ij = r_ij.contiguous()
         enc, _ = ops.bee_edge_geometry(r_ij, self.r0)                            # radial_encode_8: (edges, 8)
         first = self.mlp_radial[0]

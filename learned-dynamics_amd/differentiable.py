@@ -785,6 +785,18 @@ def bee_messages(msg, graph, r_ij, x_a, x_v, x_d):
     return mul(gl.edges_reduce_src(graph, psi_a), 0.1), mul(sums[1], 0.1), mul(sums[2], 0.1)
 
 
+def displacement_tensors(mod, graph, r_ij):
+    """archs/diffuser_atoms15.py:216-225 out of differentiable pieces: the radial MLP per edge, the edge filters
+    rad (x) u and rad (x) u (x) u as one kernel (their adjoint another), sums over the edges of a source node, the two
+    readouts on node rows."""
+    first = mod.mlp_radial[0]
+    rad = mlp_leaky(mod.mlp_radial[1], linear(first, radial_encode_8(r_ij, mod.r0)))
+    u = tens_sigmoid(1, mul(r_ij, 7. / mod.r0))
+    phi_v, phi_d = _EdgeFilters.apply(rad.contiguous(), u.contiguous())
+    A_a, A_v, A_d = (gl.edges_reduce_src(graph, t) for t in (rad, phi_v, phi_d))
+    return A_a, mod.readout_v(A_v), mod.readout_d(A_d)
+
+
 def self_tens_prods(mod, x_a, x_v, x_d):
     """archs/diffuser_atoms15.py:75-95"""
     *rest, dim_a = x_a.shape

@@ -127,6 +127,49 @@ def test_bee_layers_gradients(pkg):
     _close(prod.gn_d.gamma.grad, ws["gn_d"].grad, "d/d gn_d.gamma")
 
 
+def test_displacement_tensors_gradients(pkg):
+    """DisplacementTensors under autograd (archs/diffuser_atoms15.py:206-225): outputs, the gradients for the edge
+    vectors and every parameter against the oracle's autograd in float64; the same tangent in forward mode as from
+    nested backward passes."""
+    bee = importlib.import_module("learned-dynamics_amd.bee_layers")
+    gl = importlib.import_module("learned-dynamics_amd.graph_layers")
+    diff = importlib.import_module("learned-dynamics_amd.differentiable")
+    torch.manual_seed(0x947 + 59)
+    dims, N, r0 = (24, 12, 6), 60, 6.0
+    gen = torch.Generator().manual_seed(7)
+    src, dst = _ring(N, 7, gen)
+    mod = bee.DisplacementTensors(r0, *dims).cuda()
+    r = torch.randn(len(src), 3, generator=gen) * 2.5
+    graph = gl.Graph(src.cuda(), dst.cuda(), None, 1, N)
+    cs = [torch.randn(1, N, dims[0], generator=gen), torch.randn(1, N, dims[1], 3, generator=gen),
+          torch.randn(1, N, dims[2], 3, 3, generator=gen)]
+    r_d = r.cuda().requires_grad_(True)
+    out = mod(graph, r_d)
+    sum((y * c.cuda()).sum() for y, c in zip(out, cs)).backward()
+    dd = lambda p: p.detach().cpu().double().requires_grad_(True)
+    L = mod.mlp_radial[1].layers
+    w = {"lin_W": dd(mod.mlp_radial[0].weight), "lin_b": dd(mod.mlp_radial[0].bias),
+         "mlp": {"W_direct": dd(mod.mlp_radial[1].lin_direct.weight), "W1": dd(L[0].weight), "b1": dd(L[0].bias),
+                 "W2": dd(L[2].weight), "b2": dd(L[2].bias), "W3": dd(L[4].weight), "b3": dd(L[4].bias)},
+         "readout_v": dd(mod.readout_v.W), "readout_d": dd(mod.readout_d.W)}
+    r_o = r.double().requires_grad_(True)
+    ref = OL.displacement_tensors(src, 1, N, r_o, w, r0)
+    sum((y * c.double()).sum() for y, c in zip(ref, cs)).backward()
+    for k in range(3):
+        _close(out[k], ref[k], f"A rank {k}")
+    _close(r_d.grad, r_o.grad, "d/dr_ij")
+    _close(mod.mlp_radial[0].weight.grad, w["lin_W"].grad, "d/d first linear")
+    _close(mod.mlp_radial[1].layers[2].weight.grad, w["mlp"]["W2"].grad, "d/dW2 of the radial MLP")
+    _close(mod.mlp_radial[1].lin_direct.weight.grad, w["mlp"]["W_direct"].grad, "d/d direct")
+    _close(mod.readout_v.W.grad, w["readout_v"].grad, "d/d readout_v")
+    _close(mod.readout_d.W.grad, w["readout_d"].grad, "d/d readout_d")
+    f = lambda rr: mod(graph, rr)[2]
+    u = torch.randn(len(src), 3, generator=gen).cuda()
+    _, t_fw = diff.jvp(f, (r.cuda(),), (u,))
+    _, t_bw = torch.autograd.functional.jvp(f, (r.cuda(),), (u,), create_graph=True)
+    _close(t_fw, t_bw.double().cpu(), "tangent of A_d", 1e-5)
+
+
 def test_second_order_through_linear_products_gather_and_scatter(pkg):
     """jvp(create_graph=True) of f(x) = scatter(Y(Bee(L x, R gather(x)))) and a backward pass through the result,
     against the same thing on the oracle's functions."""
