@@ -110,6 +110,11 @@ class ScalGroupNorm(nn.Module):
 
     def forward(self, x, mul=None, add=None, res=None):
         """beta + gamma * norm(x * mul) + add + res (the extra operands are optional fusions)."""
+        if diff.wants_grad(self, x, mul, add, res):
+            y = diff.scal_group_norm(self, x if mul is None else x * mul)
+            for extra in (add, res):
+                y = y if extra is None else y + extra
+            return y
         return ops.group_norm(ops.GN_SCALAR, x, self.groups, self.gamma, self.beta, self.epsilon, mul=mul, add=add,
                               res=res)
 

@@ -254,3 +254,30 @@ class TensorProds(nn.Module):
             if ext.tensor_prods_supported(*self.prod.inds, W_l.shape[1], W_r.shape[1], W_l.shape[0], W_o.shape[0]):
                 return ext.tensor_prods(*self.prod.inds, W_l, W_r, W_o, x_l, x_r)
         return self.lin_o(self.prod(self.lin_l(x_l), self.lin_r(x_r)))
+
+
+def tens_sigmoid(inds, x):
+    """x / sqrt(1 + |x|^2) over the trailing `inds` tensor indices (managan/tensor_products.py:167-182)."""
+    from . import differentiable as diff
+    if diff.differentiated(x):
+        return diff.tens_sigmoid(inds, x)
+    return ops.tens_sigmoid(inds, x.contiguous())
+
+
+class TensSigmoid(nn.Module):
+    """managan/tensor_products.py:184-189"""
+
+    def __init__(self, inds):
+        super().__init__()
+        self.inds = inds
+
+    def forward(self, x):
+        return tens_sigmoid(self.inds, x)
+
+
+def __getattr__(name):
+    # TensGroupNorm (managan/tensor_products.py:215-232) lives beside the layers that use it, which import this module
+    if name == "TensGroupNorm":
+        from .bee_layers import TensGroupNorm
+        return TensGroupNorm
+    raise AttributeError(f"module {__name__!r} has no attribute {name!r}")
